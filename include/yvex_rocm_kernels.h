@@ -1,0 +1,148 @@
+/*
+ * Launch-level C ABI of the gfx950 kernels: plain device pointers, sizes and a stream.
+ *
+ * This is the thin layer the C11 backend (include/yvex_rocm.h) sits on; every entry point
+ * enqueues work on `stream` (a hipStream_t passed as void *, NULL = the default stream) and
+ * returns without synchronising. Return value: 0 or a negative yvex_status
+ * (INVALID_ARG -10 / BOUNDS -7 / UNSUPPORTED -5 for a refused shape, BACKEND -6 when the launch
+ * itself fails). Numerical trouble is reported through the device `status` word the caller
+ * owns: 0 ok, 1 non-finite value met, 2 contract violation seen on device - the convention of
+ * the reference's kernels (src/backend/cuda/kernels.cu:555-564,623).
+ *
+ * All pointers are device pointers unless a comment says "host".
+ */
+#ifndef YVEX_ROCM_KERNELS_H
+#define YVEX_ROCM_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *yvex_hip_stream;
+
+/* Router scoring policies. 0 is the reference's only policy (include/yvex/internal/moe.h:35);
+ * 1 is the sigmoid scoring the benchmark configuration asks for. */
+#define YVEX_HIP_SCORING_SQRT_SOFTPLUS 0
+#define YVEX_HIP_SCORING_SIGMOID 1
+
+/* Replaces yvex_q8_quantize (src/backend/cuda/kernels.cu:436-489): F32 rows -> Q8_K blocks
+ * {f32 d; i8 q[256]; i16 bsums[16]}. width % 256 == 0, input_stride >= width (in floats).
+ * Among equal |x| the lowest index provides the sign of d. */
+int yvex_hip_q8k_quantize(const float *values, uint64_t rows, uint64_t width,
+                          uint64_t input_stride, uint8_t *encoded, int *status,
+                          yvex_hip_stream stream);
+
+/* Replaces yvex_qtype_matvec / yvex_qtype_tensorcore_rows (kernels.cu:529-626,
+ * tensorcore.cu:248-374): out[in * out_stride + row] = dot(encoded row, input row in)
+ * (+ additive[in * out_stride + row]) (optionally bf16-rounded).
+ * input is F32 rows of stride input_stride when input_q8 == 0, else Q8_K rows of
+ * (row_width / 256) * 292 bytes. */
+int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
+                    uint64_t row_width, uint64_t row_bytes, const void *input, int input_q8,
+                    uint64_t input_rows, uint64_t input_stride, const float *additive,
+                    float *out, uint64_t out_stride, int output_bf16, int *status,
+                    yvex_hip_stream stream);
+
+/* Verification twin of the integer hot loop (kernel_primitives.h:287-359): writes the int32
+ * block sums the Q8_K matvec accumulates, before any float scaling.
+ *   IQ2_XXS: sums[((in * row_count + row) * blocks + b) * 2 + 0] = T,            slot 1 = 0
+ *   Q4_K / Q2_K:                                       slot 0 = dot, slot 1 = min-sum
+ *   Q8_0:    sums[(in * row_count + row) * blocks * 8 + 8 * b + k] = D_k (eight per 256 block) */
+int yvex_hip_block_dots_i32(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
+                            uint64_t row_width, uint64_t row_bytes, const uint8_t *input_q8,
+                            uint64_t input_rows, int32_t *sums, int *status,
+                            yvex_hip_stream stream);
+
+/* Replaces yvex_qtype_gather / yvex_encoded_row_decode (kernels.cu:784-830): decode selected
+ * rows to F32. row_ids may be NULL (rows 0..selected-1). */
+int yvex_hip_gather(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
+                    uint64_t row_width, uint64_t row_bytes, const uint32_t *row_ids,
+                    uint64_t selected, float *out, int *status, yvex_hip_stream stream);
+
+/* Replaces yvex_moe_route_rows (src/backend/cuda/moe_kernels.cu:180-291): per row, scores in
+ * fp64 from the logits, top-k of score + bias with ties to the lowest expert, weights
+ * normalised over the selection and scaled. selected is [rows, topk] u64, weights [rows, topk]. */
+int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t rows,
+                            uint64_t experts, uint64_t topk, int scoring, int normalize,
+                            double scaling, uint64_t *selected, float *weights, int *status,
+                            yvex_hip_stream stream);
+
+/* Replaces yvex_expert_worklist_build_cuda (moe_kernels.cu:294-402): stable counting sort of
+ * the pairs = rows*topk (row, rank) pairs by expert; rows <= 4096 per call. Outputs, all
+ * device memory:
+ *   order[pairs]            source pair of each ordered position
+ *   expert_ids[experts], bucket_offsets[experts + 1], bucket_populations[experts]
+ *   counts[4]               {bucket_count, maximum_population, pair_count, 0} */
+int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
+                            uint64_t experts, uint64_t *order, uint64_t *expert_ids, uint64_t *bucket_offsets,
+                            uint64_t *bucket_populations, uint64_t *counts, int *status,
+                            yvex_hip_stream stream);
+
+/* Expert matrices of one MoE layer. routed_* are expert-major: expert e starts at
+ * base + e * expert_bytes and holds rows * row_bytes canonical GGUF bytes. */
+typedef struct {
+    const uint8_t *gate, *up, *down;
+    unsigned int gate_qtype, up_qtype, down_qtype;
+    uint64_t hidden, intermediate;
+    uint64_t gate_row_bytes, up_row_bytes, down_row_bytes;
+    uint64_t gate_expert_bytes, up_expert_bytes, down_expert_bytes;
+} yvex_hip_expert_weights;
+
+/* Replaces yvex_moe_grouped_up_rows (+ _up_tensorcore) (moe_kernels.cu:431-516,
+ * tensorcore.cu:527-626): for every ordered pair p of every bucket,
+ *   intermediate[p, i] = bf16(silu(min(g,L)) * clamp(u,+-L) * route_weight), g/u = gate/up row i
+ * dotted with the pair's source row. Each expert's bytes are read once per bucket.
+ * activations: Q8_K rows [rows][hidden/256 * 292] when act_q8, else F32 rows [rows][hidden].
+ * order == NULL means pair p is ordered position p and its expert is p / pairs_per_bucket...
+ * see yvex_hip_moe_shared below for the single-expert form. */
+int yvex_hip_moe_up(const yvex_hip_expert_weights *weights, const void *activations, int act_q8,
+                    const uint64_t *selected, const float *route_weights, const uint64_t *order,
+                    const uint64_t *expert_ids, const uint64_t *bucket_offsets,
+                    const uint64_t *bucket_populations, const uint64_t *counts,
+                    uint64_t pairs, uint64_t topk, uint64_t experts, double limit,
+                    float *intermediate, int *status, yvex_hip_stream stream);
+
+/* Replaces yvex_moe_grouped_down_rows (+ _down_tensorcore) (moe_kernels.cu:518-582,
+ * tensorcore.cu:628-702): pair_outputs[source_pair, c] = bf16(dot(down row c, intermediate of
+ * the ordered pair)). intermediate is Q8_K [pairs][intermediate/256*292] when act_q8 else F32. */
+int yvex_hip_moe_down(const yvex_hip_expert_weights *weights, const void *intermediate,
+                      int act_q8, const uint64_t *order, const uint64_t *expert_ids,
+                      const uint64_t *bucket_offsets, const uint64_t *bucket_populations,
+                      const uint64_t *counts, uint64_t pairs, uint64_t experts,
+                      float *pair_outputs, int *status, yvex_hip_stream stream);
+
+/* Replaces yvex_moe_reduce_rows + yvex_moe_combine_rows (moe_kernels.cu:584-616):
+ * routed[row, c] = sum over rank (in rank order, fp32) of pair_outputs[row*topk+rank, c];
+ * combined[row, c] = bf16(routed + shared) when shared != NULL and combined != NULL. */
+int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows, uint64_t topk,
+                                uint64_t hidden, const float *shared, float *routed,
+                                float *combined, int *status, yvex_hip_stream stream);
+
+/* Device-side fill, usable where a captured graph must not hold a memset node. */
+int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream stream);
+
+/* ---- plumbing for the C11 host layer (no HIP headers needed there) ---- */
+int yvex_hip_device_count(void);
+int yvex_hip_device_info(int device, char *name, unsigned long name_cap, char *arch,
+                         unsigned long arch_cap, uint64_t *total_bytes, uint64_t *free_bytes,
+                         int *compute_units);
+int yvex_hip_malloc(void **out, uint64_t bytes);
+int yvex_hip_free(void *ptr);
+int yvex_hip_host_alloc(void **out, uint64_t bytes);
+int yvex_hip_host_free(void *ptr);
+int yvex_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
+int yvex_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
+int yvex_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
+int yvex_hip_stream_create(yvex_hip_stream *out);
+int yvex_hip_stream_destroy(yvex_hip_stream stream);
+int yvex_hip_stream_sync(yvex_hip_stream stream);
+/* 1 when the gfx950 code object for the kernels is loadable on the current device. */
+int yvex_hip_kernels_loadable(void);
+const char *yvex_hip_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,347 @@
+"""ctypes binding of the CPU oracle (test infrastructure only).
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` import this
+package, and only to check or to time the CPU path. The shipped library never does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libyvex_oracle.so")
+REF_PATH = os.path.join(HERE, "_ref", "libyvex_ref.so")
+
+OK, ERR_FORMAT, ERR_UNSUPPORTED, ERR_BOUNDS, ERR_INVALID_ARG = 0, -4, -5, -7, -10
+F32, F16, Q8_0, Q2_K, Q4_K, Q8_K, IQ2_XXS, I32, BF16, MXFP4 = 0, 1, 8, 10, 12, 15, 16, 26, 30, 39
+SQRT_SOFTPLUS, SIGMOID = 0, 1
+
+u8p = C.POINTER(C.c_uint8)
+f32p = C.POINTER(C.c_float)
+u64p = C.POINTER(C.c_uint64)
+u32p = C.POINTER(C.c_uint32)
+i32p = C.POINTER(C.c_int32)
+
+
+def build(force: bool = False) -> None:
+    """Compile the restatement (and oracle/_ref when the reference tree is present)."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.run(["make", "-C", HERE, "oracle"], check=True, capture_output=True)
+    if os.path.isdir("/root/reference/src/gguf") and (force or not os.path.exists(REF_PATH)):
+        subprocess.run(["make", "-C", HERE, "ref"], check=True, capture_output=True)
+
+
+class MoeLayerArgs(C.Structure):
+    _fields_ = [
+        ("hidden", C.c_uint64), ("intermediate", C.c_uint64), ("experts", C.c_uint64),
+        ("topk", C.c_uint64), ("rows", C.c_uint64),
+        ("gate_qtype", C.c_uint), ("up_qtype", C.c_uint), ("down_qtype", C.c_uint),
+        ("routed_gate", C.c_void_p), ("routed_up", C.c_void_p), ("routed_down", C.c_void_p),
+        ("shared_gate", C.c_void_p), ("shared_up", C.c_void_p), ("shared_down", C.c_void_p),
+        ("router_bias", C.c_void_p),
+        ("scoring", C.c_int), ("normalize", C.c_int), ("act_q8", C.c_int),
+        ("scaling", C.c_double), ("activation_limit", C.c_double),
+        ("threads", C.c_uint),
+    ]
+
+
+class Rng(C.Structure):
+    _fields_ = [("s", C.c_uint64 * 4)]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = C.CDLL(LIB_PATH)
+        L.yvo_f16_decode.restype = C.c_float
+        L.yvo_f16_decode.argtypes = [C.c_uint16]
+        L.yvo_f16_encode.restype = C.c_uint16
+        L.yvo_f16_encode.argtypes = [C.c_float]
+        L.yvo_bf16_decode.restype = C.c_float
+        L.yvo_bf16_decode.argtypes = [C.c_uint16]
+        L.yvo_bf16_encode.restype = C.c_uint16
+        L.yvo_bf16_encode.argtypes = [C.c_float]
+        L.yvo_bf16_round.restype = C.c_float
+        L.yvo_bf16_round.argtypes = [C.c_float]
+        L.yvo_block_dot_iq2xxs_q8k.restype = C.c_int32
+        L.yvo_block_dot_float.restype = C.c_float
+        L.yvo_block_dot_float.argtypes = [C.c_uint, C.c_void_p, C.c_void_p]
+        L.yvo_rng_uniform.restype = C.c_double
+        L.yvo_rng_next.restype = C.c_uint64
+        for name in ("yvo_rng_normal_f32",):
+            getattr(L, name).argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_double]
+        L.yvo_fill_iq2xxs.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_double]
+        L.yvo_fill_q4k.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_double]
+        L.yvo_fill_q8_0_from_normal.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_double]
+        L.yvo_rng_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64]
+        L.yvo_rng_seed.argtypes = [C.c_void_p, C.c_uint64, C.c_char_p]
+        _lib = L
+    return _lib
+
+
+def ref_lib():
+    """The library compiled from the reference's own sources, or None where it cannot exist."""
+    if not os.path.exists(REF_PATH):
+        if os.path.isdir("/root/reference/src/gguf"):
+            build()
+        if not os.path.exists(REF_PATH):
+            return None
+    return C.CDLL(REF_PATH)
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def geometry(qtype: int):
+    b, n = C.c_uint(), C.c_uint()
+    if not lib().yvo_qtype_geometry(C.c_uint(qtype), C.byref(b), C.byref(n)):
+        return None
+    return b.value, n.value
+
+
+def row_bytes(qtype: int, width: int) -> int:
+    block, nbytes = geometry(qtype)
+    assert width % block == 0
+    return width // block * nbytes
+
+
+# ---- synthetic data -------------------------------------------------------------------------
+
+class Generator:
+    """splitmix64-seeded xoshiro256**; one sub-stream per tensor name."""
+
+    def __init__(self, seed: int, name: str):
+        self.state = Rng()
+        lib().yvo_rng_seed(C.byref(self.state), C.c_uint64(seed), name.encode())
+
+    def normal(self, count: int, sigma: float = 1.0) -> np.ndarray:
+        out = np.empty(count, np.float32)
+        lib().yvo_rng_normal_f32(C.byref(self.state), _p(out), count, sigma)
+        return out
+
+    def bytes(self, count: int) -> np.ndarray:
+        out = np.empty(count, np.uint8)
+        lib().yvo_rng_bytes(C.byref(self.state), _p(out), count)
+        return out
+
+    def iq2xxs(self, blocks: int, scale_sigma: float = 0.02) -> np.ndarray:
+        out = np.empty(blocks * 66, np.uint8)
+        lib().yvo_fill_iq2xxs(C.byref(self.state), _p(out), blocks, scale_sigma)
+        return out
+
+    def q4k(self, blocks: int, scale_sigma: float = 2.0 ** -8) -> np.ndarray:
+        out = np.empty(blocks * 144, np.uint8)
+        lib().yvo_fill_q4k(C.byref(self.state), _p(out), blocks, scale_sigma)
+        return out
+
+    def q8_0(self, blocks: int, sigma: float = 0.02) -> np.ndarray:
+        out = np.empty(blocks * 34, np.uint8)
+        lib().yvo_fill_q8_0_from_normal(C.byref(self.state), _p(out), blocks, sigma)
+        return out
+
+    def weights(self, qtype: int, rows: int, width: int) -> np.ndarray:
+        block, _ = geometry(qtype)
+        blocks = rows * width // block
+        if qtype == IQ2_XXS:
+            return self.iq2xxs(blocks)
+        if qtype == Q4_K:
+            return self.q4k(blocks)
+        if qtype == Q8_0:
+            return self.q8_0(blocks)
+        if qtype == F32:
+            return self.normal(rows * width, 0.02).view(np.uint8)
+        if qtype == Q2_K:
+            out = self.bytes(blocks * 84)
+            v = out.reshape(blocks, 84)
+            for b in range(blocks):
+                for off in (80, 82):
+                    bits = int(lib().yvo_f16_encode(C.c_float(0.004 + 0.002 * ((b + off) % 7))))
+                    v[b, off] = bits & 255
+                    v[b, off + 1] = bits >> 8
+            return out
+        raise ValueError(qtype)
+
+
+# ---- numerical entry points ------------------------------------------------------------------
+
+def decode_rows(qtype: int, encoded: np.ndarray, width: int, row_ids=None) -> np.ndarray:
+    rb = row_bytes(qtype, width)
+    if row_ids is None:
+        count = encoded.size // rb
+        ids = None
+    else:
+        ids = np.ascontiguousarray(row_ids, np.uint32)
+        count = ids.size
+    out = np.empty((count, width), np.float32)
+    rc = lib().yvo_decode_rows(C.c_uint(qtype), _p(encoded), C.c_uint64(width),
+                               _p(ids) if ids is not None else None, C.c_uint64(count), _p(out))
+    if rc:
+        raise RuntimeError(f"yvo_decode_rows rc={rc}")
+    return out
+
+
+def cpu_dot(qtype: int, encoded: np.ndarray, vector: np.ndarray):
+    out = C.c_float()
+    rc = lib().yvo_cpu_dot(C.c_uint(qtype), _p(encoded), C.c_size_t(encoded.size),
+                           _p(vector), C.c_uint64(vector.size), C.byref(out))
+    return rc, out.value
+
+
+def matvec(qtype: int, encoded: np.ndarray, rows: int, width: int, inputs: np.ndarray,
+           threads: int = 1) -> np.ndarray:
+    inputs = np.ascontiguousarray(inputs, np.float32).reshape(-1, width)
+    out = np.empty((inputs.shape[0], rows), np.float32)
+    rc = lib().yvo_matvec_threads(C.c_uint(qtype), _p(encoded), C.c_uint64(rows),
+                                  C.c_uint64(width), _p(inputs), C.c_uint64(inputs.shape[0]),
+                                  _p(out), C.c_uint(threads))
+    if rc:
+        raise RuntimeError(f"yvo_matvec rc={rc}")
+    return out
+
+
+def q8k_quantize(values: np.ndarray) -> np.ndarray:
+    values = np.ascontiguousarray(values, np.float32)
+    rows, width = (1, values.size) if values.ndim == 1 else values.shape
+    out = np.empty(rows * (width // 256) * 292, np.uint8)
+    rc = lib().yvo_q8k_quantize(_p(values), C.c_uint64(rows), C.c_uint64(width), _p(out))
+    if rc:
+        raise RuntimeError(f"yvo_q8k_quantize rc={rc}")
+    return out
+
+
+def q8k_dequantize(encoded: np.ndarray) -> np.ndarray:
+    blocks = encoded.size // 292
+    out = np.empty(blocks * 256, np.float32)
+    lib().yvo_q8k_dequantize(_p(encoded), C.c_uint64(blocks), _p(out))
+    return out
+
+
+def q8_matvec(qtype: int, encoded: np.ndarray, rows: int, width: int, act: np.ndarray,
+              input_rows: int) -> np.ndarray:
+    out = np.empty((input_rows, rows), np.float32)
+    rc = lib().yvo_q8_matvec(C.c_uint(qtype), _p(encoded), C.c_uint64(rows), C.c_uint64(width),
+                             _p(act), C.c_uint64(input_rows), _p(out))
+    if rc:
+        raise RuntimeError(f"yvo_q8_matvec rc={rc}")
+    return out
+
+
+def block_dots_i32(qtype: int, encoded: np.ndarray, rows: int, width: int, act: np.ndarray,
+                   input_rows: int) -> np.ndarray:
+    """int32 block sums [input_rows, rows, blocks, 2]; slot 1 is the min-sum (0 where unused).
+
+    For Q8_0 the eight 32-value sums of one 256 block are returned as [.., blocks*8] in slot 0
+    of an array with last dimension 1.
+    """
+    L = lib()
+    blocks = width // 256
+    wb = {IQ2_XXS: 66, Q4_K: 144, Q2_K: 84, Q8_0: 272}[qtype]
+    if qtype == Q8_0:
+        out = np.zeros((input_rows, rows, blocks * 8), np.int32)
+    else:
+        out = np.zeros((input_rows, rows, blocks, 2), np.int32)
+    base_w = encoded.ctypes.data
+    base_a = act.ctypes.data
+    for i in range(input_rows):
+        for r in range(rows):
+            for b in range(blocks):
+                w = C.c_void_p(base_w + (r * blocks + b) * wb)
+                a = C.c_void_p(base_a + (i * blocks + b) * 292)
+                if qtype == IQ2_XXS:
+                    out[i, r, b, 0] = L.yvo_block_dot_iq2xxs_q8k(w, a)
+                elif qtype == Q8_0:
+                    d = (C.c_int32 * 8)()
+                    L.yvo_block_dot_q8_0_q8k(w, a, d)
+                    out[i, r, 8 * b:8 * b + 8] = list(d)
+                else:
+                    d, m = C.c_int32(), C.c_int32()
+                    fn = L.yvo_block_dot_q4k_q8k if qtype == Q4_K else L.yvo_block_dot_q2k_q8k
+                    fn(w, a, C.byref(d), C.byref(m))
+                    out[i, r, b] = (d.value, m.value)
+    return out
+
+
+def moe_route(logits: np.ndarray, bias, topk: int, scoring: int, normalize: bool, scaling: float):
+    logits = np.ascontiguousarray(logits, np.float32)
+    experts = logits.size
+    sel = np.empty(topk, np.uint64)
+    w = np.empty(topk, np.float32)
+    scores = np.empty(experts, np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    rc = lib().yvo_moe_route(_p(logits), _p(b) if b is not None else None, C.c_uint64(experts),
+                             C.c_uint64(topk), C.c_int(scoring), C.c_int(int(normalize)),
+                             C.c_double(scaling), _p(scores), _p(sel), _p(w))
+    return rc, sel, w, scores
+
+
+def moe_expert(qtypes, gate, up, down, hidden, intermediate, x, route_weight, limit=10.0,
+               act_q8=False):
+    gq, uq, dq = qtypes
+    out = np.empty(hidden, np.float32)
+    mid = np.empty(intermediate, np.float32)
+    raw = np.empty(hidden, np.float32)
+    x = np.ascontiguousarray(x, np.float32)
+    rc = lib().yvo_moe_expert(C.c_uint(gq), _p(gate), C.c_uint(uq), _p(up), C.c_uint(dq), _p(down),
+                              C.c_uint64(hidden), C.c_uint64(intermediate), _p(x),
+                              C.c_float(route_weight), C.c_double(limit), C.c_int(int(act_q8)),
+                              _p(out), _p(mid), _p(raw))
+    return rc, out, mid, raw
+
+
+def worklist_build(selected: np.ndarray, weights: np.ndarray, topk: int, experts: int):
+    selected = np.ascontiguousarray(selected, np.uint64).ravel()
+    weights = np.ascontiguousarray(weights, np.float32).ravel()
+    pairs = selected.size
+    ids = np.zeros(experts, np.uint64)
+    off = np.zeros(experts + 1, np.uint64)
+    pop = np.zeros(experts, np.uint64)
+    sp = np.zeros(pairs, np.uint64)
+    sr = np.zeros(pairs, np.uint64)
+    dr = np.zeros(pairs, np.uint64)
+    ow = np.zeros(pairs, np.float32)
+    n = C.c_uint64()
+    rc = lib().yvo_worklist_build(_p(selected), _p(weights), C.c_uint64(pairs), C.c_uint64(topk),
+                                  C.c_uint64(experts), _p(ids), _p(off), _p(pop), _p(sp), _p(sr),
+                                  _p(dr), _p(ow), C.byref(n))
+    k = n.value
+    return rc, dict(expert_ids=ids[:k], bucket_offsets=off[:k + 1], bucket_populations=pop[:k],
+                    source_pairs=sp, source_rows=sr, destination_rows=dr, route_weights=ow)
+
+
+def moe_layer(*, hidden, intermediate, experts, topk, qtypes, routed, shared, inputs, logits,
+              bias=None, scoring=SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
+              act_q8=False, threads=1):
+    inputs = np.ascontiguousarray(inputs, np.float32).reshape(-1, hidden)
+    logits = np.ascontiguousarray(logits, np.float32).reshape(-1, experts)
+    rows = inputs.shape[0]
+    a = MoeLayerArgs()
+    a.hidden, a.intermediate, a.experts, a.topk, a.rows = hidden, intermediate, experts, topk, rows
+    a.gate_qtype, a.up_qtype, a.down_qtype = qtypes
+    keep = [np.ascontiguousarray(t, np.uint8) for t in routed]
+    a.routed_gate, a.routed_up, a.routed_down = (t.ctypes.data for t in keep)
+    if shared is not None:
+        keep_s = [np.ascontiguousarray(t, np.uint8) for t in shared]
+        a.shared_gate, a.shared_up, a.shared_down = (t.ctypes.data for t in keep_s)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    a.router_bias = b.ctypes.data if b is not None else None
+    a.scoring, a.normalize, a.act_q8 = scoring, int(normalize), int(act_q8)
+    a.scaling, a.activation_limit, a.threads = scaling, limit, threads
+    sel = np.empty((rows, topk), np.uint64)
+    w = np.empty((rows, topk), np.float32)
+    routed_out = np.empty((rows, hidden), np.float32)
+    shared_out = np.empty((rows, hidden), np.float32)
+    combined = np.empty((rows, hidden), np.float32)
+    rc = lib().yvo_moe_layer(C.byref(a), _p(inputs), _p(logits), _p(sel), _p(w), _p(routed_out),
+                             _p(shared_out), _p(combined))
+    if rc:
+        raise RuntimeError(f"yvo_moe_layer rc={rc}")
+    return dict(selected=sel, weights=w, routed=routed_out, shared=shared_out, combined=combined)

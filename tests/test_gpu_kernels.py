@@ -1,0 +1,189 @@
+"""Parity of the launch-level HIP kernels against the CPU oracle (through the C ABI)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-3, 1e-5   # the path's stated fp32 tolerance
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def assert_close(got, want, rel=REL, abs_=ABS):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bound = abs_ + rel * np.abs(want)
+    worst = np.argmax(err - bound)
+    assert np.all(err <= bound), (
+        f"max violation at {worst}: got {got.flat[worst]} want {want.flat[worst]}")
+
+
+def status_ok(status):
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+
+
+def test_q8k_quantize_bit_exact(gpu, oracle):
+    from yvex_amd import kernels as K
+    g = oracle.Generator(42, "q8k.rows")
+    x = g.normal(6 * 1024).reshape(6, 1024)
+    x[1, :256] = 0.0                       # all-zero block: d = 0, q = 0
+    x[2, 256:512] = 0.0
+    x[2, 300] = -3.5                       # single spike maps to -127 * sign
+    x[3, 10] = 7.25                        # exact |tie|, opposite signs: lowest index wins
+    x[3, 200] = -7.25
+    x[4] *= 1e-30
+    status = K.new_status(gpu)
+    got = K.q8k_quantize(dev(x, gpu), status).cpu().numpy()
+    status_ok(status)
+    want = oracle.q8k_quantize(x)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("IQ2_XXS", 37, 2048, 3), ("IQ2_XXS", 5, 7168, 1), ("Q4_K", 19, 1024, 2),
+    ("Q4_K", 6, 7168, 1), ("Q8_0", 23, 4096, 2), ("Q2_K", 11, 512, 3)])
+def test_integer_block_dots_bit_exact(gpu, oracle, qtype, rows, width, inputs):
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"blockdots.{qtype}.{rows}.{width}")
+    w = g.weights(qt, rows, width)
+    act = oracle.q8k_quantize(g.normal(inputs * width).reshape(inputs, width))
+    status = K.new_status(gpu)
+    got = K.block_dots_i32(dev(w, gpu), qt, rows, width, dev(act, gpu), inputs, status).cpu().numpy()
+    status_ok(status)
+    want = oracle.block_dots_i32(qt, w, rows, width, act, inputs)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("IQ2_XXS", 67, 2048, 1), ("IQ2_XXS", 9, 7168, 5), ("Q4_K", 33, 2048, 1),
+    ("Q4_K", 10, 7168, 16), ("Q8_0", 64, 4096, 1), ("Q8_0", 13, 96, 3), ("Q2_K", 21, 768, 2),
+    ("F32", 17, 100, 3)])
+def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec.{qtype}.{rows}.{width}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    got = K.matvec(dev(w, gpu), qt, rows, width, dev(x, gpu), status=status).cpu().numpy()
+    status_ok(status)
+    want = oracle.matvec(qt, w, rows, width, x)
+    assert_close(got, want)
+
+
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("IQ2_XXS", 67, 2048, 1), ("IQ2_XXS", 9, 7168, 6), ("Q4_K", 33, 7168, 1),
+    ("Q4_K", 12, 2048, 16), ("Q8_0", 40, 4096, 2), ("Q2_K", 21, 768, 3)])
+def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvecq8.{qtype}.{rows}.{width}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    assert np.array_equal(act.cpu().numpy(), act_host)
+    want = oracle.q8_matvec(qt, w, rows, width, act_host, inputs)
+    assert_close(got, want, rel=1e-5, abs_=1e-5)
+    # and against the reference CPU path fed the dequantised activations (its own test's form)
+    deq = oracle.q8k_dequantize(act_host).reshape(inputs, width)
+    assert_close(got, oracle.matvec(qt, w, rows, width, deq))
+
+
+def test_matvec_additive_and_bf16(gpu, oracle):
+    from yvex_amd import kernels as K
+    g = oracle.Generator(7, "matvec.additive")
+    rows, width = 33, 2048
+    w = g.weights(oracle.IQ2_XXS, rows, width)
+    x = g.normal(2 * width).reshape(2, width)
+    add = g.normal(2 * rows).reshape(2, rows)
+    status = K.new_status(gpu)
+    got = K.matvec(dev(w, gpu), oracle.IQ2_XXS, rows, width, dev(x, gpu), additive=dev(add, gpu),
+                   output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    base = oracle.matvec(oracle.IQ2_XXS, w, rows, width, x)
+    want = (base + add).astype(np.float32)
+    # a bf16 output differs from the unrounded sum by at most half a bf16 ulp
+    assert np.all((got.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 1e-5)
+
+
+@pytest.mark.parametrize("qtype,width", [("IQ2_XXS", 512), ("Q4_K", 512), ("Q8_0", 96),
+                                         ("Q2_K", 256), ("F32", 40)])
+def test_gather_bit_exact(gpu, oracle, qtype, width):
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(11, f"gather.{qtype}")
+    rows = 29
+    w = g.weights(qt, rows, width)
+    ids = np.array([28, 0, 3, 3, 17], np.uint32)
+    status = K.new_status(gpu)
+    got = K.gather(dev(w, gpu), qt, rows, width, dev(ids, gpu), status).cpu().numpy()
+    status_ok(status)
+    want = oracle.decode_rows(qt, w, width, ids)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("scoring", [0, 1])
+def test_route_rows(gpu, oracle, scoring):
+    from yvex_amd import kernels as K
+    g = oracle.Generator(42, f"route.{scoring}")
+    rows, experts, topk = 32, 256, 8
+    logits = g.normal(rows * experts).reshape(rows, experts)
+    logits[3, 10] = logits[3, 200]          # exact tie: lowest ordinal first
+    bias = (g.normal(experts) * 0.1).astype(np.float32)
+    status = K.new_status(gpu)
+    sel, w = K.moe_route_rows(dev(logits, gpu), dev(bias, gpu), topk, scoring, True, 2.5, status)
+    status_ok(status)
+    sel, w = sel.cpu().numpy(), w.cpu().numpy()
+    for r in range(rows):
+        rc, s, ww, _ = oracle.moe_route(logits[r], bias, topk, scoring, True, 2.5)
+        assert rc == 0
+        assert np.array_equal(sel[r].astype(np.uint64), s)
+        assert np.max(np.abs(w[r] - ww)) <= 1e-6
+
+
+@pytest.mark.parametrize("rows,topk,experts", [(32, 8, 256), (1, 6, 256), (61, 6, 256),
+                                               (2048, 8, 256), (5, 2, 4)])
+def test_worklist_matches_stable_sort(gpu, oracle, rows, topk, experts):
+    from yvex_amd import kernels as K
+    rng = np.random.default_rng(rows * 131 + topk)
+    # skewed popularity so some experts stay empty and some buckets are large
+    p = 1.0 / np.arange(1, experts + 1) ** 1.1
+    p /= p.sum()
+    sel = np.stack([rng.choice(experts, topk, replace=False, p=p) for _ in range(rows)])
+    w = rng.random((rows, topk), dtype=np.float32)
+    status = K.new_status(gpu)
+    wl = K.worklist_build(dev(sel.astype(np.int64), gpu), experts, status)
+    status_ok(status)
+    rc, want = oracle.worklist_build(sel, w, topk, experts)
+    assert rc == 0
+    n = int(wl.counts[0].item())
+    assert n == len(want["expert_ids"])
+    assert int(wl.counts[2].item()) == rows * topk
+    assert int(wl.counts[1].item()) == int(want["bucket_populations"].max())
+    assert np.array_equal(wl.expert_ids.cpu().numpy()[:n].astype(np.uint64), want["expert_ids"])
+    assert np.array_equal(wl.bucket_offsets.cpu().numpy()[:n + 1].astype(np.uint64),
+                          want["bucket_offsets"])
+    assert np.array_equal(wl.bucket_populations.cpu().numpy()[:n].astype(np.uint64),
+                          want["bucket_populations"])
+    assert np.array_equal(wl.order.cpu().numpy().astype(np.uint64), want["source_pairs"])
+
+
+def test_worklist_flags_duplicate_expert(gpu):
+    from yvex_amd import kernels as K
+    sel = np.array([[1, 2], [3, 3]], np.int64)
+    status = K.new_status(gpu)
+    K.worklist_build(dev(sel, gpu), 4, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 2

@@ -1,0 +1,235 @@
+// Device-side building blocks shared by every gfx950 kernel of the quantized matmul path:
+// scalar conversion rules, the IQ2_XXS lookup tables kept in LDS, and per-qtype "unit"
+// decoders that turn 32 packed weights into eight dwords of signed int8.
+//
+// Reference behaviour restated here: src/backend/cuda/kernel_primitives.h:49-142 (scalar
+// rules, sign parity), :274-359 (integer block dots). Wavefronts are 64 lanes wide.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../../include/yvex_iq2xxs_grid.h"
+
+namespace yvex {
+
+constexpr int kWave = 64;
+constexpr unsigned kQ8KBytes = 292u;
+
+enum QType : unsigned {
+    QT_F32 = 0, QT_F16 = 1, QT_Q8_0 = 8, QT_Q2_K = 10, QT_Q4_K = 12, QT_Q8_K = 15,
+    QT_IQ2_XXS = 16, QT_I32 = 26, QT_BF16 = 30, QT_MXFP4 = 39
+};
+
+// Kernel status word: 0 ok, 1 non-finite numerics, 2 contract violation
+// (same convention as src/backend/cuda/kernels.cu:555-564).
+__device__ __forceinline__ void raise_status(int *status, int code)
+{
+    atomicCAS(status, 0, code);
+}
+
+__device__ __forceinline__ float f16_bits_to_float(unsigned bits)
+{
+    // binary16 -> binary32 is exact for every finite code including subnormals.
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(unsigned bits)
+{
+    return __uint_as_float(bits << 16);
+}
+
+// Round-to-nearest-even binary32 -> bfloat16, returned widened (kernel_primitives.h:89-99).
+__device__ __forceinline__ float bf16_round(float value)
+{
+    unsigned bits = __float_as_uint(value);
+    unsigned upper = bits >> 16, lower = bits & 0xffffu;
+    if ((bits & 0x7f800000u) == 0x7f800000u && (bits & 0x007fffffu))
+        return __uint_as_float((upper | 0x40u) << 16);
+    if (lower > 0x8000u || (lower == 0x8000u && (upper & 1u))) upper++;
+    return __uint_as_float(upper << 16);
+}
+
+__device__ __forceinline__ bool finite_f32(float v)
+{
+    return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;
+}
+
+__device__ __forceinline__ unsigned load_u16(const unsigned char *p)
+{
+    unsigned short v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+__device__ __forceinline__ unsigned load_u32(const unsigned char *p)
+{
+    unsigned v;
+    __builtin_memcpy(&v, p, 4);   // global loads may be 2-byte aligned; the hardware allows it
+    return v;
+}
+__device__ __forceinline__ uint2 load_u32x2(const unsigned char *p)
+{
+    uint2 v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+
+__device__ __forceinline__ int dot4(unsigned a, unsigned b, int acc)
+{
+    return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
+}
+
+// ---- wave-wide reductions (64 lanes) -------------------------------------------------------
+
+template <int WIDTH>
+__device__ __forceinline__ float group_sum_f32(float v)
+{
+#pragma unroll
+    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    return v;
+}
+template <int WIDTH>
+__device__ __forceinline__ int group_sum_i32(int v)
+{
+#pragma unroll
+    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    return v;
+}
+
+// ---- IQ2_XXS lookup tables in LDS ----------------------------------------------------------
+//
+// magnitudes[idx] : eight bytes (8/25/43) for codebook entry idx, 2 KB.
+// signmask[s7]    : eight bytes 0xff/0x00 for the 7 stored sign bits plus the parity bit, 1 KB.
+// A signed int8x4 is (magnitude ^ mask) + (mask & 0x01010101): every magnitude is >= 8, so the
+// +1 never carries into the next byte.
+
+__constant__ unsigned short k_iq2_digits[256] = {YVEX_IQ2XXS_GRID_VALUES};
+
+struct Iq2Tables {
+    uint2 magnitudes[256];
+    uint2 signmask[128];
+};
+
+__device__ __forceinline__ void iq2_tables_fill(Iq2Tables &t)
+{
+    for (unsigned i = threadIdx.x; i < 256u; i += blockDim.x) {
+        unsigned digits = k_iq2_digits[i], lo = 0u, hi = 0u;
+#pragma unroll
+        for (unsigned l = 0; l < 4u; ++l) {
+            unsigned a = (digits >> (2u * l)) & 3u, b = (digits >> (2u * l + 8u)) & 3u;
+            lo |= (a == 0u ? 8u : a == 1u ? 25u : 43u) << (8u * l);
+            hi |= (b == 0u ? 8u : b == 1u ? 25u : 43u) << (8u * l);
+        }
+        t.magnitudes[i] = make_uint2(lo, hi);
+    }
+    for (unsigned i = threadIdx.x; i < 128u; i += blockDim.x) {
+        unsigned s = i | ((__popc(i) & 1u) << 7), lo = 0u, hi = 0u;
+#pragma unroll
+        for (unsigned l = 0; l < 4u; ++l) {
+            if ((s >> l) & 1u) lo |= 0xffu << (8u * l);
+            if ((s >> (l + 4u)) & 1u) hi |= 0xffu << (8u * l);
+        }
+        t.signmask[i] = make_uint2(lo, hi);
+    }
+}
+
+// 32 weights of one IQ2_XXS group -> eight int8x4 dwords; returns the odd factor 2s+1.
+__device__ __forceinline__ int iq2_unit(const Iq2Tables &t, unsigned grids, unsigned aux,
+                                        unsigned w[8])
+{
+#pragma unroll
+    for (unsigned j = 0; j < 4u; ++j) {
+        uint2 m = t.magnitudes[(grids >> (8u * j)) & 255u];
+        uint2 s = t.signmask[(aux >> (7u * j)) & 127u];
+        w[2 * j] = (m.x ^ s.x) + (s.x & 0x01010101u);
+        w[2 * j + 1] = (m.y ^ s.y) + (s.y & 0x01010101u);
+    }
+    return (int)(2u * (aux >> 28) + 1u);
+}
+
+// Same group decoded straight from the 2-bit digits, for kernels without the LDS tables.
+__device__ __forceinline__ int iq2_level(unsigned digits, unsigned signs, unsigned l)
+{
+    unsigned d = (digits >> (2u * l)) & 3u;
+    int level = d == 0u ? 8 : d == 1u ? 25 : 43;
+    return (signs >> l) & 1u ? -level : level;
+}
+__device__ __forceinline__ unsigned iq2_sign_byte(unsigned low7)
+{
+    return low7 | ((__popc(low7) & 1u) << 7);
+}
+
+// ---- Q4_K helpers (public ggml block_q4_K: f16 d, f16 dmin, 12 scale bytes, 128 nibble bytes)
+
+__device__ __forceinline__ void q4k_scale_min(const unsigned char *scales, unsigned j,
+                                              unsigned &sc, unsigned &mn)
+{
+    if (j < 4u) {
+        sc = scales[j] & 63u;
+        mn = scales[j + 4u] & 63u;
+    } else {
+        sc = (scales[j + 4u] & 15u) | ((scales[j - 4u] >> 6) << 4);
+        mn = (scales[j + 4u] >> 4) | ((scales[j] >> 6) << 4);
+    }
+}
+
+// ---- per-element decode, used by gather / row decode and as the slow exact path ------------
+// Mirrors qtype_value (kernel_primitives.h:143-217) for the admitted qtypes; NaN otherwise.
+__device__ inline float qtype_value(const unsigned char *row, unsigned long long index,
+                                    unsigned qtype)
+{
+    switch (qtype) {
+    case QT_F32: return __uint_as_float(load_u32(row + index * 4ull));
+    case QT_F16: return f16_bits_to_float(load_u16(row + index * 2ull));
+    case QT_BF16: return bf16_bits_to_float(load_u16(row + index * 2ull));
+    case QT_I32: return (float)(int)load_u32(row + index * 4ull);
+    case QT_Q8_0: {
+        const unsigned char *b = row + (index >> 5) * 34ull;
+        return f16_bits_to_float(load_u16(b)) * (float)(signed char)b[2u + (index & 31u)];
+    }
+    case QT_IQ2_XXS: {
+        const unsigned char *b = row + (index >> 8) * 66ull;
+        unsigned in = (unsigned)(index & 255u), g = in >> 5, j = (in >> 3) & 3u, l = in & 7u;
+        unsigned grids = load_u32(b + 2u + 8u * g), aux = load_u32(b + 6u + 8u * g);
+        float gs = f16_bits_to_float(load_u16(b)) * (0.5f + (float)(aux >> 28)) * 0.25f;
+        int level = iq2_level(k_iq2_digits[(grids >> (8u * j)) & 255u],
+                              iq2_sign_byte((aux >> (7u * j)) & 127u), l);
+        return gs * (float)(level < 0 ? -level : level) * (level < 0 ? -1.0f : 1.0f);
+    }
+    case QT_Q4_K: {
+        const unsigned char *b = row + (index >> 8) * 144ull;
+        unsigned in = (unsigned)(index & 255u), j = in >> 5, l = in & 31u, sc, mn;
+        unsigned byte = b[16u + 32u * (j >> 1) + l];
+        q4k_scale_min(b + 4u, j, sc, mn);
+        float d = f16_bits_to_float(load_u16(b)) * (float)sc;
+        float m = f16_bits_to_float(load_u16(b + 2u)) * (float)mn;
+        return d * (float)((j & 1u) ? byte >> 4 : byte & 15u) - m;
+    }
+    case QT_Q2_K: {
+        const unsigned char *b = row + (index >> 8) * 84ull;
+        unsigned in = (unsigned)(index & 255u), sub = in >> 4, lane = in & 15u;
+        unsigned shift = ((sub & 7u) >> 1) * 2u;
+        unsigned code = (b[16u + (sub >> 3) * 32u + (sub & 1u) * 16u + lane] >> shift) & 3u;
+        float scale = f16_bits_to_float(load_u16(b + 80u)) * (float)(b[sub] & 15u);
+        float minimum = f16_bits_to_float(load_u16(b + 82u)) * (float)(b[sub] >> 4);
+        return scale * (float)code - minimum;
+    }
+    default: return __uint_as_float(0x7fc00000u);
+    }
+}
+
+__host__ __device__ inline bool qtype_geometry(unsigned qtype, unsigned &block, unsigned &bytes)
+{
+    switch (qtype) {
+    case QT_F32: block = 1; bytes = 4; return true;
+    case QT_F16: case QT_BF16: block = 1; bytes = 2; return true;
+    case QT_I32: block = 1; bytes = 4; return true;
+    case QT_Q8_0: block = 32; bytes = 34; return true;
+    case QT_Q2_K: block = 256; bytes = 84; return true;
+    case QT_Q4_K: block = 256; bytes = 144; return true;
+    case QT_IQ2_XXS: block = 256; bytes = 66; return true;
+    default: block = 0; bytes = 0; return false;
+    }
+}
+
+}  // namespace yvex

@@ -1,0 +1,333 @@
+// Encoded matvec (dense projection / output head), gather and the int32 block-sum probe.
+//
+// One 64-lane wavefront owns one encoded weight row and up to T activation rows; lanes walk the
+// row in 32-weight units, so one unit's packed bytes are decoded once and reused for every
+// activation row of the tile. Q8_K activations go through v_dot4 integer dots whose exact sums
+// are reduced across the eight lanes of a superblock before the single float scaling; F32
+// activations use fused multiply-adds. Results are summed across the wave with shuffles.
+//
+// Behaviour restated from src/backend/cuda/kernels.cu:529-626 (matvec), :784-830 (gather) and
+// src/backend/cuda/kernel_primitives.h:218-255,566-596 (row dots).
+#include "common.hpp"
+#include "launch.hpp"
+#include "units.hpp"
+
+namespace yvex {
+
+struct MatvecArgs {
+    const unsigned char *encoded;
+    unsigned long long row_count, row_width, row_bytes;
+    const void *input;
+    unsigned long long input_rows, input_stride;
+    const float *additive;
+    float *out;
+    unsigned long long out_stride;
+    int output_bf16;
+    int *status;
+};
+
+__device__ __forceinline__ void matvec_publish(const MatvecArgs &a, unsigned long long in,
+                                               unsigned long long row, float sum)
+{
+    const unsigned long long at = in * a.out_stride + row;
+    float value = a.additive ? sum + a.additive[at] : sum;
+    if (!finite_f32(value)) raise_status(a.status, 1);
+    else a.out[at] = a.output_bf16 ? bf16_round(value) : value;
+}
+
+// Slow exact path for a row whose F32 sum overflowed before opposite terms cancelled
+// (kernels.cu:616-620): the whole wave recomputes it in double.
+__device__ float matvec_recover_f64(const unsigned char *row, const float *x,
+                                    unsigned long long width, unsigned qtype)
+{
+    double sum = 0.0;
+    for (unsigned long long i = threadIdx.x & 63u; i < width; i += 64u)
+        sum += (double)qtype_value(row, i, qtype) * (double)x[i];
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, kWave);
+    return (float)sum;
+}
+
+template <unsigned QT, bool Q8, int T>
+__global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
+{
+    __shared__ Iq2Tables tables;
+    if constexpr (QT == QT_IQ2_XXS) {
+        iq2_tables_fill(tables);
+        __syncthreads();
+    }
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
+    if (row >= a.row_count) return;
+    const unsigned char *wrow = a.encoded + row * a.row_bytes;
+    const unsigned units = (unsigned)(a.row_width >> 5);
+    const unsigned long long act_row_bytes = (a.row_width >> 8) * kQ8KBytes;
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+
+    // Every lane runs the same trip count so the superblock shuffles below stay converged.
+    for (unsigned base = 0; base < units; base += 64u) {
+        const unsigned u = base + lane;
+        const bool live = u < units;
+        const unsigned uu = live ? u : units - 1u;
+        Unit unit;
+        unit_load<QT>(tables, wrow, uu, unit);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            unsigned long long in = in0 + t;
+            if (in >= a.input_rows) in = a.input_rows - 1ull;   // clamped rows are never written
+            if constexpr (Q8) {
+                const unsigned char *act = (const unsigned char *)a.input + in * act_row_bytes +
+                                           (unsigned long long)(uu >> 3) * kQ8KBytes;
+                UnitSum s = unit_dot_q8<QT>(unit, act, uu & 7u);
+                const float act_scale = *reinterpret_cast<const float *>(act);
+                if constexpr (UnitTraits<QT>::kIntegerCombine) {
+                    if (!live) s.dot = s.min = 0;
+                    s.dot = group_sum_i32<8>(s.dot);
+                    if constexpr (QT != QT_IQ2_XXS) s.min = group_sum_i32<8>(s.min);
+                    if (live && (uu & 7u) == 0u)
+                        acc[t] += super_combine<QT>(wrow + (uu >> 3) * UnitTraits<QT>::kSuperBytes,
+                                                    act_scale, s);
+                } else {
+                    if (live) acc[t] += q8_0_unit_value(wrow, uu, act_scale, s.dot);
+                }
+            } else {
+                const float *x = (const float *)a.input + in * a.input_stride + 32ull * uu;
+                const float v = unit_dot_f32<QT>(unit, wrow, uu, x);
+                if (live) acc[t] += v;
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        float sum = group_sum_f32<64>(acc[t]);
+        const unsigned long long in = in0 + t;
+        if (in >= a.input_rows) continue;
+        if constexpr (!Q8) {
+            if (!finite_f32(sum) && *a.status == 0)
+                sum = matvec_recover_f64(wrow, (const float *)a.input + in * a.input_stride,
+                                         a.row_width, QT);
+        }
+        if (lane == 0u) matvec_publish(a, in, row, sum);
+    }
+}
+
+// F32 / F16 / BF16 weight rows: lanes stride the row element-wise.
+template <int T>
+__global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsigned qtype)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
+    if (row >= a.row_count) return;
+    const unsigned char *wrow = a.encoded + row * a.row_bytes;
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    for (unsigned long long i = lane; i < a.row_width; i += 64u) {
+        const float w = qtype_value(wrow, i, qtype);
+        if (!finite_f32(w)) raise_status(a.status, 1);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            unsigned long long in = in0 + t;
+            if (in >= a.input_rows) in = a.input_rows - 1ull;
+            acc[t] = fmaf(w, ((const float *)a.input)[in * a.input_stride + i], acc[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        float sum = group_sum_f32<64>(acc[t]);
+        const unsigned long long in = in0 + t;
+        if (in >= a.input_rows) continue;
+        if (!finite_f32(sum) && *a.status == 0)
+            sum = matvec_recover_f64(wrow, (const float *)a.input + in * a.input_stride,
+                                     a.row_width, qtype);
+        if (lane == 0u) matvec_publish(a, in, row, sum);
+    }
+}
+
+// int32 block sums of the Q8_K path, produced by the same unit code the matvec runs.
+template <unsigned QT>
+__global__ __launch_bounds__(256) void block_dots_kernel(
+    const unsigned char *encoded, unsigned long long row_count, unsigned long long row_width,
+    unsigned long long row_bytes, const unsigned char *input, unsigned long long input_rows,
+    int *sums)
+{
+    __shared__ Iq2Tables tables;
+    if constexpr (QT == QT_IQ2_XXS) {
+        iq2_tables_fill(tables);
+        __syncthreads();
+    }
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    const unsigned long long in = blockIdx.y;
+    if (row >= row_count || in >= input_rows) return;
+    const unsigned char *wrow = encoded + row * row_bytes;
+    const unsigned units = (unsigned)(row_width >> 5);
+    const unsigned long long blocks = row_width >> 8;
+    for (unsigned base = 0; base < units; base += 64u) {
+        const unsigned u = base + lane;
+        const bool live = u < units;
+        const unsigned uu = live ? u : units - 1u;
+        Unit unit;
+        unit_load<QT>(tables, wrow, uu, unit);
+        const unsigned char *act = input + (in * blocks + (uu >> 3)) * kQ8KBytes;
+        UnitSum s = unit_dot_q8<QT>(unit, act, uu & 7u);
+        if constexpr (UnitTraits<QT>::kIntegerCombine) {
+            if (!live) s.dot = s.min = 0;
+            s.dot = group_sum_i32<8>(s.dot);
+            s.min = group_sum_i32<8>(s.min);
+            if (live && (uu & 7u) == 0u) {
+                int *o = sums + ((in * row_count + row) * blocks + (uu >> 3)) * 2ull;
+                o[0] = s.dot;
+                o[1] = s.min;
+            }
+        } else if (live) {
+            sums[(in * row_count + row) * blocks * 8ull + uu] = s.dot;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void gather_kernel(
+    const unsigned char *encoded, unsigned qtype, unsigned long long row_count,
+    unsigned long long row_width, unsigned long long row_bytes, const unsigned *row_ids,
+    unsigned long long selected, float *out, int *status)
+{
+    const unsigned long long index = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    if (index >= selected * row_width) return;
+    const unsigned long long s = index / row_width, column = index % row_width;
+    const unsigned long long row = row_ids ? row_ids[s] : s;
+    if (row >= row_count) {
+        raise_status(status, 2);
+        return;
+    }
+    const float value = qtype_value(encoded + row * row_bytes, column, qtype);
+    if (!finite_f32(value)) raise_status(status, 1);
+    else out[index] = value;
+}
+
+template <unsigned QT, bool Q8>
+static int launch_block(const MatvecArgs &a, hipStream_t stream)
+{
+    const unsigned long long grid_x = (a.row_count + 3ull) / 4ull;
+    if (grid_x > 0x7fffffffull) return ST_BOUNDS;
+    if (a.input_rows == 1ull) {
+        matvec_block_kernel<QT, Q8, 1><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
+    } else {
+        const unsigned long long grid_y = (a.input_rows + 3ull) / 4ull;
+        if (grid_y > 65535ull) return ST_BOUNDS;
+        matvec_block_kernel<QT, Q8, 4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, stream>>>(a);
+    }
+    return check_launch("matvec");
+}
+
+template <unsigned QT>
+static int launch_block_q(const MatvecArgs &a, bool q8, hipStream_t stream)
+{
+    return q8 ? launch_block<QT, true>(a, stream) : launch_block<QT, false>(a, stream);
+}
+
+}  // namespace yvex
+
+using namespace yvex;
+
+extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
+                               uint64_t row_width, uint64_t row_bytes, const void *input,
+                               int input_q8, uint64_t input_rows, uint64_t input_stride,
+                               const float *additive, float *out, uint64_t out_stride,
+                               int output_bf16, int *status, yvex_hip_stream stream)
+{
+    unsigned block, bytes;
+    if (!encoded || !input || !out || !status || !row_count || !row_width || !input_rows ||
+        out_stride < row_count || (input_q8 != 0 && input_q8 != 1))
+        return ST_INVALID_ARG;
+    if (!qtype_geometry(qtype, block, bytes)) return ST_UNSUPPORTED;
+    if (row_width % block || row_width / block * bytes != row_bytes) return ST_BOUNDS;
+    if (row_width > 0xffffffffull * 32ull) return ST_BOUNDS;
+    if (((uintptr_t)input & 3u) || ((uintptr_t)out & 3u)) return ST_INVALID_ARG;
+    MatvecArgs a{encoded, row_count, row_width, row_bytes, input, input_rows, input_stride,
+                 additive, out, out_stride, output_bf16, status};
+    hipStream_t s = as_stream(stream);
+    const bool scalar = qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16 || qtype == QT_I32;
+    if (input_q8 && (scalar || row_width % 256u)) return ST_UNSUPPORTED;
+    if (!input_q8) {
+        if (input_stride < row_width) return ST_INVALID_ARG;
+        if (!scalar && (((uintptr_t)input & 15u) || (input_stride & 3u))) return ST_INVALID_ARG;
+    }
+    if (scalar) {
+        const unsigned long long grid_x = (row_count + 3ull) / 4ull;
+        if (grid_x > 0x7fffffffull) return ST_BOUNDS;
+        if (input_rows == 1ull) {
+            matvec_scalar_kernel<1><<<dim3((unsigned)grid_x, 1), 256, 0, s>>>(a, qtype);
+        } else {
+            const unsigned long long grid_y = (input_rows + 3ull) / 4ull;
+            if (grid_y > 65535ull) return ST_BOUNDS;
+            matvec_scalar_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a, qtype);
+        }
+        return check_launch("matvec_scalar");
+    }
+    switch (qtype) {
+    case QT_IQ2_XXS: return launch_block_q<QT_IQ2_XXS>(a, input_q8, s);
+    case QT_Q8_0: return launch_block_q<QT_Q8_0>(a, input_q8, s);
+    case QT_Q4_K: return launch_block_q<QT_Q4_K>(a, input_q8, s);
+    case QT_Q2_K: return launch_block_q<QT_Q2_K>(a, input_q8, s);
+    default: return ST_UNSUPPORTED;
+    }
+}
+
+extern "C" int yvex_hip_block_dots_i32(const uint8_t *encoded, unsigned int qtype,
+                                       uint64_t row_count, uint64_t row_width,
+                                       uint64_t row_bytes, const uint8_t *input_q8,
+                                       uint64_t input_rows, int32_t *sums, int *status,
+                                       yvex_hip_stream stream)
+{
+    unsigned block, bytes;
+    if (!encoded || !input_q8 || !sums || !status || !row_count || !row_width || !input_rows)
+        return ST_INVALID_ARG;
+    if (!qtype_geometry(qtype, block, bytes)) return ST_UNSUPPORTED;
+    if (row_width % 256u || row_width / block * bytes != row_bytes) return ST_BOUNDS;
+    if (((uintptr_t)input_q8 & 3u) || input_rows > 65535ull) return ST_INVALID_ARG;
+    const unsigned long long grid_x = (row_count + 3ull) / 4ull;
+    if (grid_x > 0x7fffffffull) return ST_BOUNDS;
+    dim3 grid((unsigned)grid_x, (unsigned)input_rows);
+    hipStream_t s = as_stream(stream);
+    switch (qtype) {
+    case QT_IQ2_XXS:
+        block_dots_kernel<QT_IQ2_XXS><<<grid, 256, 0, s>>>(encoded, row_count, row_width,
+                                                           row_bytes, input_q8, input_rows, sums);
+        break;
+    case QT_Q8_0:
+        block_dots_kernel<QT_Q8_0><<<grid, 256, 0, s>>>(encoded, row_count, row_width, row_bytes,
+                                                        input_q8, input_rows, sums);
+        break;
+    case QT_Q4_K:
+        block_dots_kernel<QT_Q4_K><<<grid, 256, 0, s>>>(encoded, row_count, row_width, row_bytes,
+                                                        input_q8, input_rows, sums);
+        break;
+    case QT_Q2_K:
+        block_dots_kernel<QT_Q2_K><<<grid, 256, 0, s>>>(encoded, row_count, row_width, row_bytes,
+                                                        input_q8, input_rows, sums);
+        break;
+    default: return ST_UNSUPPORTED;
+    }
+    return check_launch("block_dots");
+}
+
+extern "C" int yvex_hip_gather(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
+                               uint64_t row_width, uint64_t row_bytes, const uint32_t *row_ids,
+                               uint64_t selected, float *out, int *status,
+                               yvex_hip_stream stream)
+{
+    unsigned block, bytes;
+    if (!encoded || !out || !status || !row_count || !row_width || !selected) return ST_INVALID_ARG;
+    if (!qtype_geometry(qtype, block, bytes)) return ST_UNSUPPORTED;
+    if (row_width % block || row_width / block * bytes != row_bytes) return ST_BOUNDS;
+    if (selected > UINT64_MAX / row_width) return ST_BOUNDS;
+    const unsigned long long grid = (selected * row_width + 255ull) / 256ull;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    gather_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+        encoded, qtype, row_count, row_width, row_bytes, row_ids, selected, out, status);
+    return check_launch("gather");
+}

@@ -1,0 +1,650 @@
+// MoE routing, expert-major worklist, and the decode-width grouped expert kernels for gfx950.
+//
+// The grouped kernels walk buckets (one expert plus the ordered (row, rank) pairs routed to it)
+// so an expert's packed bytes are streamed from HBM once per bucket and reused for every pair in
+// it. Lanes own fixed column ranges of the activation rows and keep them in registers; weight
+// rows stream through with unaligned 16-byte loads; integer superblock sums are exact.
+//
+// Behaviour restated from src/backend/cuda/moe_kernels.cu:180-291 (routing), :294-402
+// (worklist), :431-616 (grouped up/down, reduce, combine) and src/graph/moe.c:497-622.
+#include "common.hpp"
+#include "launch.hpp"
+#include "units.hpp"
+
+namespace yvex {
+
+// ---- routing --------------------------------------------------------------------------------
+
+__device__ __forceinline__ double route_score(double v, int scoring)
+{
+    if (scoring == YVEX_HIP_SCORING_SIGMOID)
+        return v >= 0.0 ? 1.0 / (1.0 + exp(-v)) : exp(v) / (1.0 + exp(v));
+    const double softplus = v > 0.0 ? v + log1p(exp(-v)) : log1p(exp(v));
+    return sqrt(softplus);
+}
+
+// One wavefront per row; each lane scores four experts (experts <= 256).
+__global__ __launch_bounds__(256) void route_rows_kernel(
+    const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long rows,
+    unsigned experts, unsigned topk, int scoring, int normalize, double scaling,
+    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    float score[4];
+    unsigned long long key[4];
+#pragma unroll
+    for (unsigned i = 0; i < 4u; ++i) {
+        const unsigned e = lane * 4u + i;
+        score[i] = 0.0f;
+        key[i] = 0ull;
+        if (e < experts) {
+            const double s = route_score((double)logits[row * experts + e], scoring);
+            score[i] = (float)s;
+            float biased = (bias ? bias[e] : 0.0f) + score[i];
+            if (!(s == s) || !finite_f32(score[i]) || !finite_f32(biased)) raise_status(status, 1);
+            biased += 0.0f;   // -0 and +0 must compare equal
+            const unsigned bits = __float_as_uint(biased);
+            const unsigned sortable = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+            // larger score first, then the lower expert ordinal; +1 keeps live keys non-zero
+            key[i] = ((unsigned long long)sortable << 32) | (unsigned long long)(0xfffffffeu - e + 1u);
+        }
+    }
+    double total = 0.0;
+    float picked_score = 0.0f;   // lane r keeps the score of rank r
+    for (unsigned rank = 0; rank < topk; ++rank) {
+        unsigned long long best = key[0];
+#pragma unroll
+        for (unsigned i = 1; i < 4u; ++i) best = key[i] > best ? key[i] : best;
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) {
+            const unsigned long long other = __shfl_xor(best, offset, kWave);
+            best = other > best ? other : best;
+        }
+        const unsigned e = 0xffffffffu - (unsigned)(best & 0xffffffffull);
+        float s = 0.0f;
+#pragma unroll
+        for (unsigned i = 0; i < 4u; ++i)
+            if (lane * 4u + i == e) {
+                s = score[i];
+                key[i] = 0ull;
+            }
+        s = __shfl(s, (int)(e >> 2), kWave);
+        total += (double)s;                 // rank order, in double (src/graph/moe.c:566-574)
+        if (lane == rank) picked_score = s;
+        if (lane == 0u) selected[row * topk + rank] = e;
+    }
+    if (normalize && !(total > 0.0 && total < 1.0e300)) raise_status(status, 1);
+    if (lane < topk) {
+        double value = (double)picked_score;
+        if (normalize) value /= total;
+        value *= scaling;
+        const float w = (float)value;
+        if (!finite_f32(w)) raise_status(status, 1);
+        weights[row * topk + lane] = w;
+    }
+}
+
+// ---- worklist -------------------------------------------------------------------------------
+//
+// A row never routes to the same expert twice, so each expert's pairs are a set of rows: one bit
+// per (expert, row) in LDS. Bucket order is expert order, order inside a bucket is row order,
+// which is exactly the stable counting sort of pairs by expert (src/graph/worklist.c:380-393).
+
+constexpr unsigned kWorklistMaxRows = 4096u;
+
+__global__ __launch_bounds__(1024) void worklist_kernel(
+    const unsigned long long *__restrict__ selected, unsigned pairs, unsigned topk,
+    unsigned experts, unsigned long long *__restrict__ order,
+    unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
+    unsigned long long *__restrict__ bucket_populations, unsigned long long *__restrict__ counts,
+    int *status)
+{
+    extern __shared__ unsigned shared_words[];
+    const unsigned rows = pairs / topk;
+    const unsigned words = (rows + 31u) / 32u;            // bitmap words per expert
+    unsigned *bitmap = shared_words;                       // [experts][words]
+    unsigned *population = bitmap + experts * words;       // [experts]
+    unsigned *offset = population + experts;               // [experts + 1]
+    unsigned *slot = offset + experts + 1u;                // [experts] bucket index or ~0
+    __shared__ unsigned bad;
+    const unsigned tid = threadIdx.x;
+    for (unsigned i = tid; i < experts * words; i += blockDim.x) bitmap[i] = 0u;
+    if (tid == 0u) bad = 0u;
+    __syncthreads();
+    for (unsigned p = tid; p < pairs; p += blockDim.x) {
+        const unsigned long long e = selected[p];
+        if (e >= experts) {
+            bad = 1u;
+            continue;
+        }
+        const unsigned row = p / topk;
+        const unsigned old = atomicOr(&bitmap[(unsigned)e * words + (row >> 5)], 1u << (row & 31u));
+        if (old & (1u << (row & 31u))) bad = 1u;   // duplicate expert inside one row
+    }
+    __syncthreads();
+    for (unsigned e = tid; e < experts; e += blockDim.x) {
+        unsigned n = 0u;
+        for (unsigned w = 0; w < words; ++w) n += __popc(bitmap[e * words + w]);
+        population[e] = n;
+    }
+    __syncthreads();
+    if (tid == 0u) {
+        unsigned cursor = 0u, bucket = 0u, maximum = 0u;
+        for (unsigned e = 0; e < experts; ++e) {
+            const unsigned n = population[e];
+            offset[e] = cursor;
+            slot[e] = n ? bucket : 0xffffffffu;
+            if (n) {
+                expert_ids[bucket] = e;
+                bucket_offsets[bucket] = cursor;
+                bucket_populations[bucket] = n;
+                bucket++;
+                maximum = n > maximum ? n : maximum;
+            }
+            cursor += n;
+        }
+        offset[experts] = cursor;
+        bucket_offsets[bucket] = cursor;
+        for (unsigned b = bucket; b < experts; ++b) {
+            expert_ids[b] = 0ull;
+            bucket_populations[b] = 0ull;
+            if (b + 1u <= experts) bucket_offsets[b + 1u] = cursor;
+        }
+        counts[0] = bucket;
+        counts[1] = maximum;
+        counts[2] = cursor;
+        counts[3] = 0ull;
+        if (cursor != pairs) bad = 1u;
+    }
+    __syncthreads();
+    for (unsigned i = tid; i < experts * words; i += blockDim.x) {
+        const unsigned e = i / words, w = i % words;
+        unsigned bits = bitmap[i];
+        if (!bits) continue;
+        unsigned before = 0u;
+        for (unsigned k = 0; k < w; ++k) before += __popc(bitmap[e * words + k]);
+        while (bits) {
+            const unsigned bit = __ffs(bits) - 1u;
+            bits &= bits - 1u;
+            const unsigned row = w * 32u + bit;
+            unsigned rank = 0u;
+            for (unsigned r = 0; r < topk; ++r)
+                if (selected[row * topk + r] == e) rank = r;
+            order[offset[e] + before] = (unsigned long long)row * topk + rank;
+            before++;
+        }
+    }
+    __syncthreads();
+    if (tid == 0u && bad) raise_status(status, 2);
+}
+
+// ---- grouped expert projections ---------------------------------------------------------------
+
+constexpr int kPass = 4;   // pairs of one bucket handled per sweep over the expert's bytes
+constexpr int kUnitsPerLane = 4;
+
+struct GroupedArgs {
+    const unsigned char *gate, *up;          // up == nullptr: plain projection (down)
+    unsigned long long row_bytes, expert_bytes, up_row_bytes, up_expert_bytes;
+    unsigned width;                          // reduction width (activation row length)
+    unsigned out_rows;                       // rows of the weight matrix per expert
+    const void *activations;                 // Q8_K rows or F32 rows
+    unsigned long long act_stride;           // bytes between activation rows
+    int act_by_ordered_pair;                 // 1: activation row = ordered position (down)
+    const unsigned long long *selected, *order, *expert_ids, *bucket_offsets, *bucket_populations;
+    const unsigned long long *counts;
+    const float *route_weights;
+    unsigned pairs, topk, experts;
+    double limit;
+    float *out;                              // up: intermediate[ordered][out_rows]; down: pair_outputs[source][out_rows]
+    int out_by_source_pair;
+    int *status;
+    unsigned rows_per_block;                 // weight rows handled by one workgroup
+};
+
+// SiLU-gated product in double, as src/graph/moe.c:605-611 orders it.
+__device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weight, double limit)
+{
+    const double gv = fmin((double)g, limit);
+    const double uv = fmax(-limit, fmin((double)u, limit));
+    const double t = exp(-fabs(gv));
+    const double silu = gv >= 0.0 ? gv / (1.0 + t) : gv * t / (1.0 + t);
+    return bf16_round((float)(silu * uv * (double)route_weight));
+}
+
+// One workgroup = one (bucket, tile of weight rows). A lane owns half a superblock (four units,
+// 128 columns) of the reduction dimension; units/4 lanes span one weight row and, where that is
+// a power of two below 64, a wave covers several rows at once.
+template <unsigned QT, bool Q8, bool FUSED_UP>
+__global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
+{
+    __shared__ Iq2Tables tables;
+    __shared__ float gate_up[4][2][16][kPass];   // [wave][gate|up][row in wave tile][pair]
+    if constexpr (QT == QT_IQ2_XXS) iq2_tables_fill(tables);
+
+    const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
+    const unsigned bucket = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+    unsigned long long expert = 0ull, first = 0ull, population = a.pairs;
+    bool idle = false;
+    if (a.expert_ids) {
+        if (bucket >= (unsigned)a.counts[0]) idle = true;
+        else {
+            expert = a.expert_ids[bucket];
+            first = a.bucket_offsets[bucket];
+            population = a.bucket_populations[bucket];
+        }
+    } else if (bucket > 0u) {
+        idle = true;
+    }
+    if constexpr (QT == QT_IQ2_XXS) __syncthreads();
+    if (idle) return;
+    if (expert >= a.experts || first + population > a.pairs) {
+        if (threadIdx.x == 0u) raise_status(a.status, 2);
+        return;
+    }
+
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned units = a.width >> 5;                          // multiple of 8
+    const unsigned lanes_per_row = units / kUnitsPerLane;         // even, <= 64
+    const bool pow2 = (lanes_per_row & (lanes_per_row - 1u)) == 0u;
+    const unsigned rows_per_wave = pow2 ? 64u / lanes_per_row : 1u;
+    const unsigned reduce_width = pow2 ? lanes_per_row : 64u;
+    const unsigned sub = lane / lanes_per_row, seg = lane % lanes_per_row;
+    const bool lane_live = sub < rows_per_wave;
+    const unsigned unit0 = seg * kUnitsPerLane;                   // all four units share a superblock
+    const unsigned super = unit0 >> 3;
+
+    const unsigned char *gate_e = a.gate + expert * a.expert_bytes;
+    const unsigned char *up_e = FUSED_UP ? a.up + expert * a.up_expert_bytes : nullptr;
+    const unsigned row_begin = tile * a.rows_per_block;
+    const unsigned row_end = row_begin + a.rows_per_block < a.out_rows ? row_begin + a.rows_per_block
+                                                                       : a.out_rows;
+    const unsigned wave_rows = (a.rows_per_block + 3u) / 4u;      // rows per wave inside the tile
+    const unsigned wave_begin = row_begin + wave * wave_rows;
+    const unsigned wave_end = wave_begin + wave_rows < row_end ? wave_begin + wave_rows : row_end;
+
+    for (unsigned long long pass = 0; pass < population; pass += kPass) {
+        const int n = population - pass < (unsigned long long)kPass ? (int)(population - pass) : kPass;
+        // ---- the sweep's activation rows: this lane's 128 columns stay in registers (Q8_K) ----
+        unsigned act[kPass][kUnitsPerLane * 8];
+        float act_scale[kPass];
+        const unsigned char *act_row[kPass];
+        float route_weight[kPass];
+        unsigned long long out_index[kPass];
+#pragma unroll
+        for (int p = 0; p < kPass; ++p) {
+            const unsigned long long ordered = first + pass + (p < n ? p : 0);
+            const unsigned long long source = a.order ? a.order[ordered] : ordered;
+            const unsigned long long arow = a.act_by_ordered_pair ? ordered : source / a.topk;
+            act_row[p] = (const unsigned char *)a.activations + arow * a.act_stride;
+            route_weight[p] = a.route_weights ? a.route_weights[source] : 1.0f;
+            out_index[p] = a.out_by_source_pair ? source : ordered;
+            act_scale[p] = 0.0f;
+            if constexpr (Q8) {
+                const unsigned char *blk = act_row[p] + (unsigned long long)super * kQ8KBytes;
+                act_scale[p] = *reinterpret_cast<const float *>(blk);
+                const unsigned char *q = blk + 4u + 32u * (unit0 & 7u);   // 4-byte aligned payload
+#pragma unroll
+                for (int k = 0; k < kUnitsPerLane * 2; ++k) {
+                    uint4 v;
+                    __builtin_memcpy(&v, q + 16 * k, 16);
+                    act[p][4 * k] = v.x;
+                    act[p][4 * k + 1] = v.y;
+                    act[p][4 * k + 2] = v.z;
+                    act[p][4 * k + 3] = v.w;
+                }
+            }
+        }
+
+        for (unsigned base = wave_begin; base < wave_end; base += rows_per_wave) {
+            const unsigned row = base + sub;
+            const bool row_live = lane_live && row < wave_end;
+            const unsigned safe_row = row_live ? row : wave_begin;
+            float sum_gate[kPass], sum_up[kPass];
+#pragma unroll
+            for (int p = 0; p < kPass; ++p) sum_gate[p] = sum_up[p] = 0.0f;
+
+#pragma unroll
+            for (int which = 0; which < (FUSED_UP ? 2 : 1); ++which) {
+                const unsigned char *wrow =
+                    which == 0 ? gate_e + (unsigned long long)safe_row * a.row_bytes
+                               : up_e + (unsigned long long)safe_row * a.up_row_bytes;
+                float *sums = which == 0 ? sum_gate : sum_up;
+                UnitSum whole[kPass];
+#pragma unroll
+                for (int p = 0; p < kPass; ++p) whole[p].dot = whole[p].min = 0;
+#pragma unroll
+                for (int k = 0; k < kUnitsPerLane; ++k) {
+                    const unsigned u = unit0 + k;
+                    Unit unit;
+                    unit_load<QT>(tables, wrow, u, unit);
+#pragma unroll
+                    for (int p = 0; p < kPass; ++p) {
+                        if (p < n) {
+                            if constexpr (Q8) {
+                                const unsigned *av = &act[p][8 * k];
+                                int d = 0, d2 = 0;
+                                if constexpr (QT == QT_Q2_K) {
+#pragma unroll
+                                    for (int i = 0; i < 4; ++i) {
+                                        d = dot4(unit.w[i], av[i], d);
+                                        d2 = dot4(unit.w[4 + i], av[4 + i], d2);
+                                    }
+                                    d = unit.factor * d + unit.factor2 * d2;
+                                } else {
+#pragma unroll
+                                    for (int i = 0; i < 8; ++i) d = dot4(unit.w[i], av[i], d);
+                                    d *= unit.factor;
+                                }
+                                if constexpr (UnitTraits<QT>::kIntegerCombine) {
+                                    whole[p].dot += d;
+                                    if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) {
+                                        const short *bs = reinterpret_cast<const short *>(
+                                            act_row[p] + (unsigned long long)super * kQ8KBytes + 260u);
+                                        const unsigned g = u & 7u;
+                                        whole[p].min += unit.min1 * (int)bs[2u * g] +
+                                                        unit.min2 * (int)bs[2u * g + 1u];
+                                    }
+                                } else {
+                                    sums[p] += q8_0_unit_value(wrow, u, act_scale[p], d);
+                                }
+                            } else {
+                                const float *x = reinterpret_cast<const float *>(act_row[p]) + 32ull * u;
+                                sums[p] += unit_dot_f32<QT>(unit, wrow, u, x);
+                            }
+                        }
+                    }
+                }
+                if constexpr (Q8 && UnitTraits<QT>::kIntegerCombine) {
+                    // two neighbouring lanes hold the halves of one superblock: finish the exact
+                    // integer sum, then the even lane applies the single float scaling
+#pragma unroll
+                    for (int p = 0; p < kPass; ++p) {
+                        if (p < n) {
+                            UnitSum t = whole[p];
+                            t.dot += __shfl_xor(t.dot, 1, kWave);
+                            if constexpr (QT != QT_IQ2_XXS) t.min += __shfl_xor(t.min, 1, kWave);
+                            if ((seg & 1u) == 0u)
+                                sums[p] += super_combine<QT>(
+                                    wrow + (unsigned long long)super * UnitTraits<QT>::kSuperBytes,
+                                    act_scale[p], t);
+                        }
+                    }
+                }
+            }
+            // ---- sum across the lanes of each row ----
+#pragma unroll
+            for (int p = 0; p < kPass; ++p) {
+                if (p < n) {
+                    if (!row_live) sum_gate[p] = sum_up[p] = 0.0f;
+                    for (unsigned offset = reduce_width >> 1; offset > 0u; offset >>= 1) {
+                        sum_gate[p] += __shfl_xor(sum_gate[p], (int)offset, kWave);
+                        if constexpr (FUSED_UP) sum_up[p] += __shfl_xor(sum_up[p], (int)offset, kWave);
+                    }
+                }
+            }
+            if constexpr (FUSED_UP) {
+                // park (gate, up); the SwiGLU runs once per wave tile with every lane busy
+                const unsigned local = row - wave_begin;
+                if (row_live && seg == 0u && local < 16u) {
+#pragma unroll
+                    for (int p = 0; p < kPass; ++p) {
+                        gate_up[wave][0][local][p] = sum_gate[p];
+                        gate_up[wave][1][local][p] = sum_up[p];
+                    }
+                }
+            } else {
+                if (row_live && seg == 0u) {
+#pragma unroll
+                    for (int p = 0; p < kPass; ++p) {
+                        if (p < n) {
+                            const float value = bf16_round(sum_gate[p]);
+                            if (!finite_f32(value)) raise_status(a.status, 1);
+                            else a.out[out_index[p] * a.out_rows + row] = value;
+                        }
+                    }
+                }
+            }
+        }
+        if constexpr (FUSED_UP) {
+            // LDS operations of one wave complete in order: no barrier between park and read
+            const unsigned local = lane >> 2;
+            const int p = (int)(lane & 3u);
+            const unsigned row = wave_begin + local;
+            if (local < 16u && row < wave_end && p < n) {
+                float rw = route_weight[0];
+                unsigned long long oi = out_index[0];
+#pragma unroll
+                for (int q = 1; q < kPass; ++q) {
+                    if (p == q) {
+                        rw = route_weight[q];
+                        oi = out_index[q];
+                    }
+                }
+                const float value = swiglu_bf16(gate_up[wave][0][local][p], gate_up[wave][1][local][p],
+                                                rw, a.limit);
+                if (!finite_f32(value)) raise_status(a.status, 1);
+                else a.out[oi * a.out_rows + row] = value;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void reduce_combine_kernel(
+    const float *__restrict__ pair_outputs, unsigned long long rows, unsigned topk,
+    unsigned long long hidden, const float *__restrict__ shared, float *__restrict__ routed,
+    float *__restrict__ combined, int *status)
+{
+    const unsigned long long index = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    if (index >= rows * hidden) return;
+    const unsigned long long row = index / hidden, column = index % hidden;
+    float total = 0.0f;
+    for (unsigned rank = 0; rank < topk; ++rank)
+        total += pair_outputs[(row * topk + rank) * hidden + column];   // rank order, fp32
+    if (!finite_f32(total)) {
+        raise_status(status, 1);
+        return;
+    }
+    if (routed) routed[index] = total;
+    if (combined && shared) {
+        const float value = bf16_round(total + shared[index]);
+        if (!finite_f32(value)) raise_status(status, 1);
+        else combined[index] = value;
+    }
+}
+
+template <unsigned QT>
+static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, unsigned buckets,
+                          hipStream_t stream)
+{
+    const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
+    const unsigned long long grid = (unsigned long long)buckets * tiles;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    if (fused) {
+        if (q8) grouped_kernel<QT, true, true><<<(unsigned)grid, 256, 0, stream>>>(a);
+        else grouped_kernel<QT, false, true><<<(unsigned)grid, 256, 0, stream>>>(a);
+    } else {
+        if (q8) grouped_kernel<QT, true, false><<<(unsigned)grid, 256, 0, stream>>>(a);
+        else grouped_kernel<QT, false, false><<<(unsigned)grid, 256, 0, stream>>>(a);
+    }
+    return check_launch("moe_grouped");
+}
+
+static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool fused,
+                            unsigned buckets, hipStream_t stream)
+{
+    switch (qtype) {
+    case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, buckets, stream);
+    case QT_Q4_K: return launch_grouped<QT_Q4_K>(a, q8, fused, buckets, stream);
+    case QT_Q8_0: return launch_grouped<QT_Q8_0>(a, q8, fused, buckets, stream);
+    case QT_Q2_K: return launch_grouped<QT_Q2_K>(a, q8, fused, buckets, stream);
+    default: return ST_UNSUPPORTED;
+    }
+}
+
+static int check_matrix(unsigned qtype, uint64_t width, uint64_t row_bytes)
+{
+    unsigned block, bytes;
+    if (!qtype_geometry(qtype, block, bytes) || block < 32u) return ST_UNSUPPORTED;
+    if (!width || width % 256u || width / block * bytes != row_bytes) return ST_BOUNDS;
+    if (width / 32u > 64u * kUnitsPerLane) return ST_UNSUPPORTED;   // one wave spans a row
+    return ST_OK;
+}
+
+}  // namespace yvex
+
+using namespace yvex;
+
+extern "C" int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t rows,
+                                       uint64_t experts, uint64_t topk, int scoring,
+                                       int normalize, double scaling, uint64_t *selected,
+                                       float *weights, int *status, yvex_hip_stream stream)
+{
+    if (!logits || !selected || !weights || !status || !rows || !experts || experts > 256u ||
+        !topk || topk > 16u || topk > experts ||
+        (scoring != YVEX_HIP_SCORING_SQRT_SOFTPLUS && scoring != YVEX_HIP_SCORING_SIGMOID))
+        return ST_INVALID_ARG;
+    const uint64_t grid = (rows + 3u) / 4u;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    route_rows_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+        logits, bias, rows, (unsigned)experts, (unsigned)topk, scoring, normalize, scaling,
+        (unsigned long long *)selected, weights, status);
+    return check_launch("moe_route_rows");
+}
+
+extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
+                                       uint64_t experts, uint64_t *order, uint64_t *expert_ids,
+                                       uint64_t *bucket_offsets, uint64_t *bucket_populations,
+                                       uint64_t *counts, int *status, yvex_hip_stream stream)
+{
+    if (!selected || !order || !expert_ids || !bucket_offsets || !bucket_populations || !counts ||
+        !status || !pairs || !topk || !experts || experts > 256u || pairs % topk)
+        return ST_INVALID_ARG;
+    const uint64_t rows = pairs / topk;
+    if (rows > kWorklistMaxRows) return ST_BOUNDS;
+    const uint64_t words = (rows + 31u) / 32u;
+    const size_t lds = (size_t)(experts * words + 3u * experts + 1u) * sizeof(unsigned);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void *)worklist_kernel,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) !=
+            hipSuccess)
+            (void)hipGetLastError();
+        configured = true;
+    }
+    if (lds > 160u * 1024u - 64u) return ST_BOUNDS;
+    worklist_kernel<<<1, 1024, lds, as_stream(stream)>>>(
+        (const unsigned long long *)selected, (unsigned)pairs, (unsigned)topk, (unsigned)experts,
+        (unsigned long long *)order, (unsigned long long *)expert_ids,
+        (unsigned long long *)bucket_offsets, (unsigned long long *)bucket_populations,
+        (unsigned long long *)counts, status);
+    return check_launch("worklist_build");
+}
+
+extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *activations,
+                               int act_q8, const uint64_t *selected, const float *route_weights,
+                               const uint64_t *order, const uint64_t *expert_ids,
+                               const uint64_t *bucket_offsets, const uint64_t *bucket_populations,
+                               const uint64_t *counts, uint64_t pairs, uint64_t topk,
+                               uint64_t experts, double limit, float *intermediate, int *status,
+                               yvex_hip_stream stream)
+{
+    if (!w || !w->gate || !w->up || !activations || !intermediate || !status || !pairs || !topk ||
+        !experts || !(limit > 0.0) || (act_q8 != 0 && act_q8 != 1) ||
+        (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        return ST_INVALID_ARG;
+    if (w->gate_qtype != w->up_qtype) return ST_UNSUPPORTED;
+    int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
+    if (rc) return rc;
+    if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
+    if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull) return ST_BOUNDS;
+    GroupedArgs a{};
+    a.gate = w->gate;
+    a.up = w->up;
+    a.row_bytes = w->gate_row_bytes;
+    a.expert_bytes = w->gate_expert_bytes;
+    a.up_row_bytes = w->up_row_bytes;
+    a.up_expert_bytes = w->up_expert_bytes;
+    a.width = (unsigned)w->hidden;
+    a.out_rows = (unsigned)w->intermediate;
+    a.activations = activations;
+    a.act_stride = act_q8 ? w->hidden / 256u * kQ8KBytes : w->hidden * sizeof(float);
+    a.act_by_ordered_pair = 0;
+    a.selected = (const unsigned long long *)selected;
+    a.order = (const unsigned long long *)order;
+    a.expert_ids = (const unsigned long long *)expert_ids;
+    a.bucket_offsets = (const unsigned long long *)bucket_offsets;
+    a.bucket_populations = (const unsigned long long *)bucket_populations;
+    a.counts = (const unsigned long long *)counts;
+    a.route_weights = route_weights;
+    a.pairs = (unsigned)pairs;
+    a.topk = (unsigned)topk;
+    a.experts = (unsigned)experts;
+    a.limit = limit;
+    a.out = intermediate;
+    a.out_by_source_pair = 0;
+    a.status = status;
+    a.rows_per_block = 64u;
+    const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
+    return dispatch_grouped(w->gate_qtype, a, act_q8 != 0, true, buckets, as_stream(stream));
+}
+
+extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *intermediate,
+                                 int act_q8, const uint64_t *order, const uint64_t *expert_ids,
+                                 const uint64_t *bucket_offsets,
+                                 const uint64_t *bucket_populations, const uint64_t *counts,
+                                 uint64_t pairs, uint64_t experts, float *pair_outputs,
+                                 int *status, yvex_hip_stream stream)
+{
+    if (!w || !w->down || !intermediate || !pair_outputs || !status || !pairs || !experts ||
+        (act_q8 != 0 && act_q8 != 1) ||
+        (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        return ST_INVALID_ARG;
+    int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
+    if (rc) return rc;
+    if (pairs > 0xffffffffull || w->hidden > 0xffffffffull) return ST_BOUNDS;
+    GroupedArgs a{};
+    a.gate = w->down;
+    a.up = nullptr;
+    a.row_bytes = w->down_row_bytes;
+    a.expert_bytes = w->down_expert_bytes;
+    a.width = (unsigned)w->intermediate;
+    a.out_rows = (unsigned)w->hidden;
+    a.activations = intermediate;
+    a.act_stride = act_q8 ? w->intermediate / 256u * kQ8KBytes : w->intermediate * sizeof(float);
+    a.act_by_ordered_pair = 1;
+    a.order = (const unsigned long long *)order;
+    a.expert_ids = (const unsigned long long *)expert_ids;
+    a.bucket_offsets = (const unsigned long long *)bucket_offsets;
+    a.bucket_populations = (const unsigned long long *)bucket_populations;
+    a.counts = (const unsigned long long *)counts;
+    a.route_weights = nullptr;
+    a.pairs = (unsigned)pairs;
+    a.topk = 1u;
+    a.experts = (unsigned)experts;
+    a.limit = 1.0;
+    a.out = pair_outputs;
+    a.out_by_source_pair = 1;
+    a.status = status;
+    a.rows_per_block = 256u;
+    const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
+    return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, buckets, as_stream(stream));
+}
+
+extern "C" int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows,
+                                           uint64_t topk, uint64_t hidden, const float *shared,
+                                           float *routed, float *combined, int *status,
+                                           yvex_hip_stream stream)
+{
+    if (!pair_outputs || !status || !rows || !topk || !hidden || (!routed && !combined) ||
+        (combined && !shared) || topk > 0xffffffffull)
+        return ST_INVALID_ARG;
+    if (rows > UINT64_MAX / hidden) return ST_BOUNDS;
+    const uint64_t grid = (rows * hidden + 255u) / 256u;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    reduce_combine_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+        pair_outputs, rows, (unsigned)topk, hidden, shared, routed, combined, status);
+    return check_launch("moe_reduce_combine");
+}

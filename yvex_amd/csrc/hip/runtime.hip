@@ -1,0 +1,160 @@
+// Plumbing the C11 host layer needs from the HIP runtime: memory, copies, streams, device facts.
+// Kept behind plain C entry points so the host sources compile with a C11 compiler alone.
+#include <stdio.h>
+#include <string.h>
+
+#include "launch.hpp"
+
+namespace yvex {
+
+static thread_local char g_last_error[256] = "";
+
+void set_last_error(const char *where, hipError_t code)
+{
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s", where, hipGetErrorString(code));
+}
+void set_last_error_text(const char *text)
+{
+    snprintf(g_last_error, sizeof(g_last_error), "%s", text);
+}
+
+static int wrap(const char *where, hipError_t code)
+{
+    if (code == hipSuccess) return ST_OK;
+    set_last_error(where, code);
+    (void)hipGetLastError();
+    return code == hipErrorOutOfMemory ? ST_NOMEM : ST_BACKEND;
+}
+
+__global__ void fill_u32_kernel(uint32_t *dst, uint32_t value, uint64_t count)
+{
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) dst[i] = value;
+}
+
+__global__ void probe_kernel(int *out)
+{
+    if (out) *out = 950;
+}
+
+}  // namespace yvex
+
+using namespace yvex;
+
+extern "C" {
+
+const char *yvex_hip_last_error(void) { return g_last_error; }
+
+int yvex_hip_device_count(void)
+{
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return count;
+}
+
+int yvex_hip_device_info(int device, char *name, unsigned long name_cap, char *arch,
+                         unsigned long arch_cap, uint64_t *total_bytes, uint64_t *free_bytes,
+                         int *compute_units)
+{
+    hipDeviceProp_t prop;
+    size_t free_b = 0, total_b = 0;
+    int rc = wrap("hipGetDeviceProperties", hipGetDeviceProperties(&prop, device));
+    if (rc) return rc;
+    if (name && name_cap) snprintf(name, name_cap, "%s", prop.name);
+    if (arch && arch_cap) snprintf(arch, arch_cap, "%s", prop.gcnArchName);
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    rc = wrap("hipSetDevice", hipSetDevice(device));
+    if (rc) return rc;
+    rc = wrap("hipMemGetInfo", hipMemGetInfo(&free_b, &total_b));
+    if (rc) return rc;
+    if (total_bytes) *total_bytes = total_b;
+    if (free_bytes) *free_bytes = free_b;
+    return ST_OK;
+}
+
+int yvex_hip_kernels_loadable(void)
+{
+    // Fail closed: the code object counts as present only if a kernel from it really launches.
+    int *flag = nullptr, host = 0;
+    if (yvex_hip_device_count() <= 0) return 0;
+    if (hipMalloc(&flag, sizeof(int)) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    (void)hipMemset(flag, 0, sizeof(int));
+    probe_kernel<<<1, 1>>>(flag);
+    bool ok = hipGetLastError() == hipSuccess && hipDeviceSynchronize() == hipSuccess &&
+              hipMemcpy(&host, flag, sizeof(int), hipMemcpyDeviceToHost) == hipSuccess;
+    (void)hipFree(flag);
+    (void)hipGetLastError();
+    return ok && host == 950;
+}
+
+int yvex_hip_malloc(void **out, uint64_t bytes)
+{
+    if (!out) return ST_INVALID_ARG;
+    *out = nullptr;
+    return wrap("hipMalloc", hipMalloc(out, bytes ? bytes : 1));
+}
+int yvex_hip_free(void *ptr) { return ptr ? wrap("hipFree", hipFree(ptr)) : ST_OK; }
+
+int yvex_hip_host_alloc(void **out, uint64_t bytes)
+{
+    if (!out) return ST_INVALID_ARG;
+    *out = nullptr;
+    return wrap("hipHostMalloc", hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+}
+int yvex_hip_host_free(void *ptr) { return ptr ? wrap("hipHostFree", hipHostFree(ptr)) : ST_OK; }
+
+int yvex_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream)
+{
+    if (!bytes) return ST_OK;
+    int rc = wrap("hipMemcpyAsync(h2d)",
+                  hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return rc ? rc : wrap("hipStreamSynchronize", hipStreamSynchronize(as_stream(stream)));
+}
+int yvex_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream)
+{
+    if (!bytes) return ST_OK;
+    int rc = wrap("hipMemcpyAsync(d2h)",
+                  hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return rc ? rc : wrap("hipStreamSynchronize", hipStreamSynchronize(as_stream(stream)));
+}
+int yvex_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream)
+{
+    if (!bytes) return ST_OK;
+    return wrap("hipMemcpyAsync(d2d)",
+                hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+}
+
+int yvex_hip_stream_create(yvex_hip_stream *out)
+{
+    hipStream_t s = nullptr;
+    if (!out) return ST_INVALID_ARG;
+    int rc = wrap("hipStreamCreate", hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = rc ? nullptr : reinterpret_cast<yvex_hip_stream>(s);
+    return rc;
+}
+int yvex_hip_stream_destroy(yvex_hip_stream stream)
+{
+    return stream ? wrap("hipStreamDestroy", hipStreamDestroy(as_stream(stream))) : ST_OK;
+}
+int yvex_hip_stream_sync(yvex_hip_stream stream)
+{
+    return wrap("hipStreamSynchronize", hipStreamSynchronize(as_stream(stream)));
+}
+
+int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream stream)
+{
+    if (!count) return ST_OK;
+    if (!dst || ((uintptr_t)dst & 3u)) return ST_INVALID_ARG;
+    uint64_t blocks = (count + 255u) / 256u;
+    if (blocks > 0x7fffffffull) return ST_BOUNDS;
+    fill_u32_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>((uint32_t *)dst, value, count);
+    return check_launch("fill_u32");
+}
+
+}  // extern "C"

@@ -1,0 +1,179 @@
+"""Python-side callers of the launch-level C ABI (include/yvex_rocm_kernels.h).
+
+torch is used for device memory and the current stream only; every computation goes through
+``libyvex_rocm.so``. Tensors must live on the GPU and be contiguous.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import load_library
+
+F32, F16, Q8_0, Q2_K, Q4_K, Q8_K, IQ2_XXS, I32, BF16 = 0, 1, 8, 10, 12, 15, 16, 26, 30
+SQRT_SOFTPLUS, SIGMOID = 0, 1
+
+_GEOMETRY = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), I32: (1, 4), Q8_0: (32, 34), Q2_K: (256, 84),
+             Q4_K: (256, 144), IQ2_XXS: (256, 66), Q8_K: (256, 292)}
+
+
+class KernelError(RuntimeError):
+    def __init__(self, name: str, rc: int):
+        lib = load_library()
+        lib.yvex_hip_last_error.restype = C.c_char_p
+        text = lib.yvex_hip_last_error().decode(errors="replace")
+        super().__init__(f"{name} returned {rc} {text}")
+        self.rc = rc
+
+
+class ExpertWeights(C.Structure):
+    _fields_ = [("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
+                ("gate_qtype", C.c_uint), ("up_qtype", C.c_uint), ("down_qtype", C.c_uint),
+                ("hidden", C.c_uint64), ("intermediate", C.c_uint64),
+                ("gate_row_bytes", C.c_uint64), ("up_row_bytes", C.c_uint64),
+                ("down_row_bytes", C.c_uint64),
+                ("gate_expert_bytes", C.c_uint64), ("up_expert_bytes", C.c_uint64),
+                ("down_expert_bytes", C.c_uint64)]
+
+
+def row_bytes(qtype: int, width: int) -> int:
+    block, nbytes = _GEOMETRY[qtype]
+    if width % block:
+        raise ValueError("row width is not block divisible")
+    return width // block * nbytes
+
+
+def _ptr(t):
+    if t is None:
+        return C.c_void_p(0)
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError("device, contiguous tensors only")
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _call(name, *args):
+    fn = getattr(load_library(), name)
+    fn.restype = C.c_int
+    rc = fn(*args)
+    if rc != 0:
+        raise KernelError(name, rc)
+
+
+def new_status(device="cuda"):
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def q8k_quantize(values: torch.Tensor, status: torch.Tensor, out: torch.Tensor | None = None):
+    rows, width = values.shape
+    if out is None:
+        out = torch.empty(rows * (width // 256) * 292, dtype=torch.uint8, device=values.device)
+    _call("yvex_hip_q8k_quantize", _ptr(values), C.c_uint64(rows), C.c_uint64(width),
+          C.c_uint64(values.stride(0)), _ptr(out), _ptr(status), _stream())
+    return out
+
+
+def matvec(encoded, qtype, row_count, row_width, inputs, *, input_q8=False, input_rows=None,
+           additive=None, output_bf16=False, status=None, out=None):
+    if input_rows is None:
+        input_rows = inputs.shape[0]
+    if out is None:
+        out = torch.empty((input_rows, row_count), dtype=torch.float32, device=encoded.device)
+    stride = row_width if input_q8 else inputs.stride(0)
+    _call("yvex_hip_matvec", _ptr(encoded), C.c_uint(qtype), C.c_uint64(row_count),
+          C.c_uint64(row_width), C.c_uint64(row_bytes(qtype, row_width)), _ptr(inputs),
+          C.c_int(int(input_q8)), C.c_uint64(input_rows), C.c_uint64(stride), _ptr(additive),
+          _ptr(out), C.c_uint64(row_count), C.c_int(int(output_bf16)), _ptr(status), _stream())
+    return out
+
+
+def block_dots_i32(encoded, qtype, row_count, row_width, act_q8, input_rows, status):
+    blocks = row_width // 256
+    shape = (input_rows, row_count, blocks * 8) if qtype == Q8_0 else (input_rows, row_count, blocks, 2)
+    sums = torch.zeros(shape, dtype=torch.int32, device=encoded.device)
+    _call("yvex_hip_block_dots_i32", _ptr(encoded), C.c_uint(qtype), C.c_uint64(row_count),
+          C.c_uint64(row_width), C.c_uint64(row_bytes(qtype, row_width)), _ptr(act_q8),
+          C.c_uint64(input_rows), _ptr(sums), _ptr(status), _stream())
+    return sums
+
+
+def gather(encoded, qtype, row_count, row_width, row_ids, status):
+    selected = row_count if row_ids is None else row_ids.numel()
+    out = torch.empty((selected, row_width), dtype=torch.float32, device=encoded.device)
+    _call("yvex_hip_gather", _ptr(encoded), C.c_uint(qtype), C.c_uint64(row_count),
+          C.c_uint64(row_width), C.c_uint64(row_bytes(qtype, row_width)), _ptr(row_ids),
+          C.c_uint64(selected), _ptr(out), _ptr(status), _stream())
+    return out
+
+
+def moe_route_rows(logits, bias, topk, scoring, normalize, scaling, status):
+    rows, experts = logits.shape
+    selected = torch.empty((rows, topk), dtype=torch.int64, device=logits.device)
+    weights = torch.empty((rows, topk), dtype=torch.float32, device=logits.device)
+    _call("yvex_hip_moe_route_rows", _ptr(logits), _ptr(bias), C.c_uint64(rows),
+          C.c_uint64(experts), C.c_uint64(topk), C.c_int(scoring), C.c_int(int(normalize)),
+          C.c_double(scaling), _ptr(selected), _ptr(weights), _ptr(status), _stream())
+    return selected, weights
+
+
+class Worklist:
+    """Device-resident expert-major worklist (all int64 tensors hold unsigned 64-bit values)."""
+
+    def __init__(self, pairs: int, experts: int, device):
+        self.order = torch.empty(pairs, dtype=torch.int64, device=device)
+        self.expert_ids = torch.empty(experts, dtype=torch.int64, device=device)
+        self.bucket_offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
+        self.bucket_populations = torch.empty(experts, dtype=torch.int64, device=device)
+        self.counts = torch.empty(4, dtype=torch.int64, device=device)
+
+
+def worklist_build(selected, experts, status, worklist: Worklist | None = None) -> Worklist:
+    rows, topk = selected.shape
+    pairs = rows * topk
+    wl = worklist or Worklist(pairs, experts, selected.device)
+    _call("yvex_hip_worklist_build", _ptr(selected), C.c_uint64(pairs), C.c_uint64(topk),
+          C.c_uint64(experts), _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
+          _ptr(wl.bucket_populations), _ptr(wl.counts), _ptr(status), _stream())
+    return wl
+
+
+def expert_weights(gate, up, down, qtypes, hidden, intermediate) -> ExpertWeights:
+    w = ExpertWeights()
+    w.gate, w.up, w.down = gate.data_ptr(), up.data_ptr(), down.data_ptr()
+    w.gate_qtype, w.up_qtype, w.down_qtype = qtypes
+    w.hidden, w.intermediate = hidden, intermediate
+    w.gate_row_bytes = row_bytes(qtypes[0], hidden)
+    w.up_row_bytes = row_bytes(qtypes[1], hidden)
+    w.down_row_bytes = row_bytes(qtypes[2], intermediate)
+    w.gate_expert_bytes = w.gate_row_bytes * intermediate
+    w.up_expert_bytes = w.up_row_bytes * intermediate
+    w.down_expert_bytes = w.down_row_bytes * hidden
+    w._keep = (gate, up, down)
+    return w
+
+
+def moe_up(w: ExpertWeights, activations, act_q8, selected, route_weights, wl, pairs, topk,
+           experts, limit, intermediate, status):
+    _call("yvex_hip_moe_up", C.byref(w), _ptr(activations), C.c_int(int(act_q8)), _ptr(selected),
+          _ptr(route_weights), _ptr(wl.order if wl else None),
+          _ptr(wl.expert_ids if wl else None), _ptr(wl.bucket_offsets if wl else None),
+          _ptr(wl.bucket_populations if wl else None), _ptr(wl.counts if wl else None),
+          C.c_uint64(pairs), C.c_uint64(topk), C.c_uint64(experts), C.c_double(limit),
+          _ptr(intermediate), _ptr(status), _stream())
+
+
+def moe_down(w: ExpertWeights, intermediate, act_q8, wl, pairs, experts, pair_outputs, status):
+    _call("yvex_hip_moe_down", C.byref(w), _ptr(intermediate), C.c_int(int(act_q8)),
+          _ptr(wl.order if wl else None), _ptr(wl.expert_ids if wl else None),
+          _ptr(wl.bucket_offsets if wl else None), _ptr(wl.bucket_populations if wl else None),
+          _ptr(wl.counts if wl else None), C.c_uint64(pairs), C.c_uint64(experts),
+          _ptr(pair_outputs), _ptr(status), _stream())
+
+
+def moe_reduce_combine(pair_outputs, rows, topk, hidden, shared, routed, combined, status):
+    _call("yvex_hip_moe_reduce_combine", _ptr(pair_outputs), C.c_uint64(rows), C.c_uint64(topk),
+          C.c_uint64(hidden), _ptr(shared), _ptr(routed), _ptr(combined), _ptr(status), _stream())

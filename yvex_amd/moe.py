@@ -1,0 +1,79 @@
+"""Launch sequence of one MoE layer over a row batch, driven from Python through the C ABI.
+
+This is the same sequence the C11 host layer's ``execute_rows`` enqueues
+(src/backend/cuda/moe.c:1619 in the reference): quantize activations -> route -> worklist ->
+grouped up (+SwiGLU) -> quantize intermediate -> grouped down -> rank-ordered reduce -> shared
+expert -> combine. It exists so tests and the benchmark can reach each stage's buffers; it does
+no arithmetic itself.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import kernels as K
+
+
+class MoeLayer:
+    def __init__(self, *, hidden, intermediate, experts, topk, qtypes, routed, shared=None,
+                 bias=None, scoring=K.SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
+                 act_q8=True, max_rows=64, device="cuda"):
+        self.hidden, self.intermediate, self.experts, self.topk = hidden, intermediate, experts, topk
+        self.qtypes, self.scoring, self.normalize = qtypes, scoring, normalize
+        self.scaling, self.limit, self.act_q8 = scaling, limit, act_q8
+        self.device = device
+        self.routed = K.expert_weights(*routed, qtypes, hidden, intermediate)
+        self.shared = K.expert_weights(*shared, qtypes, hidden, intermediate) if shared else None
+        self.bias = bias
+        self.max_rows = max_rows
+        pairs = max_rows * topk
+        f32 = dict(dtype=torch.float32, device=device)
+        u8 = dict(dtype=torch.uint8, device=device)
+        self.status = K.new_status(device)
+        self.act_q8_rows = torch.empty(max_rows * (hidden // 256) * 292, **u8)
+        self.worklist = K.Worklist(pairs, experts, device)
+        self.intermediate_f32 = torch.empty((pairs, intermediate), **f32)
+        self.intermediate_q8 = torch.empty(pairs * (intermediate // 256) * 292, **u8)
+        self.pair_outputs = torch.empty((pairs, hidden), **f32)
+        self.shared_mid = torch.empty((max_rows, intermediate), **f32)
+        self.shared_mid_q8 = torch.empty(max_rows * (intermediate // 256) * 292, **u8)
+        self.shared_out = torch.zeros((max_rows, hidden), **f32)
+        self.routed_out = torch.empty((max_rows, hidden), **f32)
+        self.combined = torch.empty((max_rows, hidden), **f32)
+        self.selected = None
+        self.weights = None
+
+    def run(self, rows_f32: torch.Tensor, logits: torch.Tensor):
+        """Enqueue one batch; returns the combined rows (device tensor, not synchronised)."""
+        rows = rows_f32.shape[0]
+        assert rows <= self.max_rows
+        pairs = rows * self.topk
+        st = self.status
+        if self.act_q8:
+            K.q8k_quantize(rows_f32, st, self.act_q8_rows)
+            acts = self.act_q8_rows
+        else:
+            acts = rows_f32
+        self.selected, self.weights = K.moe_route_rows(
+            logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st)
+        K.worklist_build(self.selected, self.experts, st, self.worklist)
+        K.moe_up(self.routed, acts, self.act_q8, self.selected, self.weights, self.worklist, pairs,
+                 self.topk, self.experts, self.limit, self.intermediate_f32, st)
+        if self.act_q8:
+            K.q8k_quantize(self.intermediate_f32[:pairs], st, self.intermediate_q8)
+            mid = self.intermediate_q8
+        else:
+            mid = self.intermediate_f32
+        K.moe_down(self.routed, mid, self.act_q8, self.worklist, pairs, self.experts,
+                   self.pair_outputs, st)
+        if self.shared is not None:
+            K.moe_up(self.shared, acts, self.act_q8, None, None, None, rows, 1, 1, self.limit,
+                     self.shared_mid, st)
+            if self.act_q8:
+                K.q8k_quantize(self.shared_mid[:rows], st, self.shared_mid_q8)
+                smid = self.shared_mid_q8
+            else:
+                smid = self.shared_mid
+            K.moe_down(self.shared, smid, self.act_q8, None, rows, 1, self.shared_out, st)
+        K.moe_reduce_combine(self.pair_outputs, rows, self.topk, self.hidden, self.shared_out,
+                             self.routed_out, self.combined, st)
+        return self.combined[:rows]
