@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight matmul path on one MI355X.
+
+A "step" is one pass of the decode MoE layer (BASELINE.json config 3: hidden 7168, 256 routed
+experts + 1 shared, top-8 sigmoid routing, expert width 2048, IQ2_XXS weights, 32 concurrent
+single-token rows, Q8_K device activations) over synthetic inputs already resident in HBM.
+`value` is the algorithmic expert-weight bytes the step must read, (U + 1) * 11 354 112 with U
+the distinct routed experts hit, divided by the step time.
+
+Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up sweep), timed
+with events on the launch stream; `cpu_baseline` is the CPU oracle timed on the host cores over
+a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_INT8_PEAK_TOPS = 5000.0
+HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
+EXPERT_BYTES = 3 * 3_784_704   # gate + up + down of one IQ2_XXS expert
+
+
+def synth_iq2xxs(torch, blocks: int, device, seed: int):
+    """Random IQ2_XXS superblocks: uniform grid/sign/scale bytes, positive fp16 block scale."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 66), dtype=torch.uint8, device=device, generator=gen)
+    d = (torch.rand(blocks, device=device, generator=gen) * 3.5e-4 + 1.0e-4).to(torch.float16)
+    raw[:, :2] = d.view(torch.uint8).reshape(blocks, 2)
+    return raw.reshape(-1)
+
+
+def event_ms(torch, fn, repeats: int) -> float:
+    """Average duration of fn() in ms, measured with events on the current (launch) stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(repeats):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / repeats
+
+
+def cpu_baseline(sample_rows: int, threads: int):
+    """Time the CPU oracle (reference algorithm: decode to float, double accumulate) on
+    `sample_rows` rows of the same layer shape; weights for the experts those rows hit only."""
+    import numpy as np
+    import oracle
+    g = oracle.Generator(42, "bench.cpu")
+    experts = 16   # the rows below route among 16 experts: enough for top-8, small enough to build
+    gate = g.iq2xxs(experts * INTERMEDIATE * HIDDEN // 256)
+    up = g.iq2xxs(experts * INTERMEDIATE * HIDDEN // 256)
+    down = g.iq2xxs(experts * HIDDEN * INTERMEDIATE // 256)
+    shared = tuple(g.iq2xxs(INTERMEDIATE * HIDDEN // 256) for _ in range(3))
+    x = g.normal(sample_rows * HIDDEN).reshape(sample_rows, HIDDEN)
+    logits = g.normal(sample_rows * experts).reshape(sample_rows, experts)
+    t0 = time.perf_counter()
+    oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=experts, topk=TOPK,
+                     qtypes=(oracle.IQ2_XXS,) * 3, routed=(gate, up, down), shared=shared,
+                     inputs=x, logits=logits, scoring=oracle.SIGMOID, normalize=True, scaling=1.0,
+                     act_q8=False, threads=threads)
+    seconds = time.perf_counter() - t0
+    touched = sample_rows * (TOPK + 1) * EXPERT_BYTES   # the CPU path re-reads an expert per row
+    return {"value": touched / seconds / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{sample_rows} rows x (top-8 + shared) expert FFNs of the same layer shape, "
+                      f"scalar C restatement of yvex_quant_cpu_dot/yvex_moe_expert_cpu",
+            "tokens_per_s": sample_rows / seconds, "seconds": seconds}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--act", choices=["q8k", "f32"], default="q8k")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from yvex_amd import kernels as K
+    from yvex_amd.moe import MoeLayer
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    qt = K.IQ2_XXS
+    up_blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
+    gate = synth_iq2xxs(torch, up_blocks, dev, 1)
+    up = synth_iq2xxs(torch, up_blocks, dev, 2)
+    down = synth_iq2xxs(torch, up_blocks, dev, 3)
+    shared = tuple(synth_iq2xxs(torch, INTERMEDIATE * HIDDEN // 256, dev, 10 + i) for i in range(3))
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(42)
+    x = torch.randn((ROWS, HIDDEN), device=dev, generator=gen)
+    logits = torch.randn((ROWS, EXPERTS), device=dev, generator=gen)
+    layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                     qtypes=(qt, qt, qt), routed=(gate, up, down), shared=shared, bias=None,
+                     scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
+                     act_q8=args.act == "q8k", max_rows=ROWS, device=dev)
+
+    for _ in range(args.warmup):
+        layer.run(x, logits)
+    torch.cuda.synchronize()
+    if int(layer.status.item()) != 0:
+        print(f"device status {int(layer.status.item())}", file=sys.stderr)
+        return 1
+    unique = int(layer.worklist.counts[0].item())
+    max_pop = int(layer.worklist.counts[1].item())
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step_ms_events = event_ms(torch, lambda: layer.run(x, logits), args.steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    step_ms = max(step_ms_events, wall_ms)
+    weight_bytes = (unique + 1) * EXPERT_BYTES
+    value = weight_bytes / (step_ms * 1e-3) / 1e9
+
+    # dominant kernel alone: the routed gate/up sweep (2/3 of the routed bytes)
+    pairs = ROWS * TOPK
+    acts = layer.act_q8_rows if layer.act_q8 else x
+
+    def up_only():
+        K.moe_up(layer.routed, acts, layer.act_q8, layer.selected, layer.weights, layer.worklist,
+                 pairs, TOPK, EXPERTS, layer.limit, layer.intermediate_f32, layer.status)
+
+    def down_only():
+        mid = layer.intermediate_q8 if layer.act_q8 else layer.intermediate_f32
+        K.moe_down(layer.routed, mid, layer.act_q8, layer.worklist, pairs, EXPERTS,
+                   layer.pair_outputs, layer.status)
+
+    up_ms = event_ms(torch, up_only, max(10, args.steps))
+    down_ms = event_ms(torch, down_only, max(10, args.steps))
+    up_bytes = unique * 2 * 3_784_704
+    achieved = up_bytes / (up_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "IQ2_XXS MoE decode weight GB/s", "value": round(value, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 dot / f32 scale" if layer.act_q8 else "f32",
+        "data": "synthetic",
+        "config": {"workload": "moe_decode_iq2xxs: hidden 7168, 256 routed + 1 shared experts, "
+                               "top-8 sigmoid, expert width 2048, 32 rows",
+                   "activations": args.act, "distinct_routed_experts": unique,
+                   "max_bucket_population": max_pop, "weight_bytes_per_step": weight_bytes},
+        "hbm_peak_frac": round(value / HBM_PEAK_GBS, 4),
+        "tokens_per_s": round(ROWS / (step_ms * 1e-3), 1),
+        "roofline": {"bound": "hbm", "kernel": "grouped_kernel<IQ2_XXS> gate/up sweep",
+                     "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "launch_ms": round(up_ms, 4), "algorithmic_bytes": up_bytes},
+        "kernels_ms": {"routed_up": round(up_ms, 4), "routed_down": round(down_ms, 4)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_rows, 1)
+        out["cpu_baseline_all_cores"] = cpu_baseline(max(args.cpu_rows, 8), min(16, os.cpu_count() or 1))
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

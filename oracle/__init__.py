@@ -133,12 +133,12 @@ class Generator:
         lib().yvo_rng_bytes(C.byref(self.state), _p(out), count)
         return out
 
-    def iq2xxs(self, blocks: int, scale_sigma: float = 0.02) -> np.ndarray:
+    def iq2xxs(self, blocks: int, scale_sigma: float = 3.5e-4) -> np.ndarray:
         out = np.empty(blocks * 66, np.uint8)
         lib().yvo_fill_iq2xxs(C.byref(self.state), _p(out), blocks, scale_sigma)
         return out
 
-    def q4k(self, blocks: int, scale_sigma: float = 2.0 ** -8) -> np.ndarray:
+    def q4k(self, blocks: int, scale_sigma: float = 1.0e-4) -> np.ndarray:
         out = np.empty(blocks * 144, np.uint8)
         lib().yvo_fill_q4k(C.byref(self.state), _p(out), blocks, scale_sigma)
         return out
@@ -164,7 +164,7 @@ class Generator:
             v = out.reshape(blocks, 84)
             for b in range(blocks):
                 for off in (80, 82):
-                    bits = int(lib().yvo_f16_encode(C.c_float(0.004 + 0.002 * ((b + off) % 7))))
+                    bits = int(lib().yvo_f16_encode(C.c_float((0.004 + 0.002 * ((b + off) % 7)) * (1.0 if off == 80 else 1.5))))
                     v[b, off] = bits & 255
                     v[b, off + 1] = bits >> 8
             return out

@@ -974,7 +974,7 @@ void yvo_fill_q4k(yvo_rng *rng, uint8_t *encoded, uint64_t blocks, double scale_
     yvo_rng_bytes(rng, encoded, blocks * 144u);
     for (b = 0; b < blocks; ++b) {
         uint16_t d = positive_scale_f16(rng, scale_sigma);
-        uint16_t dmin = positive_scale_f16(rng, scale_sigma);
+        uint16_t dmin = positive_scale_f16(rng, scale_sigma * 8.0);
         encoded[144u * b] = (uint8_t)(d & 0xffu);
         encoded[144u * b + 1u] = (uint8_t)(d >> 8);
         encoded[144u * b + 2u] = (uint8_t)(dmin & 0xffu);

@@ -13,15 +13,17 @@ def dev(a, device):
 
 
 def bf16_flip_report(got, want):
-    """Elements that differ must differ by one bf16 step; returns their fraction."""
+    """Elements that differ are either inside the path's fp32 tolerance (1e-3 rel / 1e-5 abs:
+    sums that cancel to almost nothing) or exactly one bf16 step away, which happens when the
+    unrounded value sits on a rounding boundary. Returns the fraction of one-step elements."""
     got = np.asarray(got, np.float32)
     want = np.asarray(want, np.float32)
-    diff = got != want
-    if diff.any():
-        step = np.abs(got[diff].astype(np.float64) - want[diff]) / np.maximum(
-            np.abs(want[diff]).astype(np.float64), 1e-30)
+    err = np.abs(got.astype(np.float64) - want)
+    outside = err > 1e-5 + 1e-3 * np.abs(want)
+    if outside.any():
+        step = err[outside] / np.abs(want[outside]).astype(np.float64)
         assert np.all(step <= BF16_ULP * 1.001), f"worst relative step {step.max()}"
-    return diff.mean()
+    return outside.mean()
 
 
 def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype, act_q8, scoring,
