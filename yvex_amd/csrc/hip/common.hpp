@@ -80,20 +80,77 @@ __device__ __forceinline__ int dot4(unsigned a, unsigned b, int acc)
 }
 
 // ---- wave-wide reductions (64 lanes) -------------------------------------------------------
+//
+// Sums over aligned groups of WIDTH lanes, returned in every lane of the group. Steps inside a
+// row of 16 lanes are data-parallel-primitive moves that run at ALU rate (no LDS crossbar);
+// the two steps that cross rows use the row broadcasts and a scalar read-back.
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_move(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+
+template <int WIDTH>
+__device__ __forceinline__ int group_sum_i32(int v)
+{
+    static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 ||
+                  WIDTH == 32 || WIDTH == 64, "power of two up to the wave");
+    if constexpr (WIDTH >= 2) v += dpp_move<0xb1, 0xf>(v);    // quad_perm [1,0,3,2]
+    if constexpr (WIDTH >= 4) v += dpp_move<0x4e, 0xf>(v);    // quad_perm [2,3,0,1]
+    if constexpr (WIDTH >= 8) v += dpp_move<0x141, 0xf>(v);   // row_half_mirror
+    if constexpr (WIDTH >= 16) v += dpp_move<0x140, 0xf>(v);  // row_mirror
+    if constexpr (WIDTH >= 32) v += dpp_move<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
+    if constexpr (WIDTH == 64) {
+        v += dpp_move<0x143, 0xc>(v);                          // row_bcast31 into rows 2 and 3
+        v = __builtin_amdgcn_readlane(v, 63);
+    } else if constexpr (WIDTH == 32) {
+        const int low = __builtin_amdgcn_readlane(v, 31), high = __builtin_amdgcn_readlane(v, 63);
+        v = (threadIdx.x & 32u) ? high : low;
+    }
+    return v;
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move_f32(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf,
+                                                      false));
+}
 
 template <int WIDTH>
 __device__ __forceinline__ float group_sum_f32(float v)
 {
-#pragma unroll
-    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 ||
+                  WIDTH == 32 || WIDTH == 64, "power of two up to the wave");
+    if constexpr (WIDTH >= 2) v += dpp_move_f32<0xb1, 0xf>(v);
+    if constexpr (WIDTH >= 4) v += dpp_move_f32<0x4e, 0xf>(v);
+    if constexpr (WIDTH >= 8) v += dpp_move_f32<0x141, 0xf>(v);
+    if constexpr (WIDTH >= 16) v += dpp_move_f32<0x140, 0xf>(v);
+    if constexpr (WIDTH >= 32) v += dpp_move_f32<0x142, 0xa>(v);
+    if constexpr (WIDTH == 64) {
+        v += dpp_move_f32<0x143, 0xc>(v);
+        v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+    } else if constexpr (WIDTH == 32) {
+        const int low = __builtin_amdgcn_readlane(__float_as_int(v), 31);
+        const int high = __builtin_amdgcn_readlane(__float_as_int(v), 63);
+        v = __int_as_float((threadIdx.x & 32u) ? high : low);
+    }
     return v;
 }
-template <int WIDTH>
-__device__ __forceinline__ int group_sum_i32(int v)
+
+// Same with the width known only at run time (wave-uniform).
+__device__ __forceinline__ float group_sum_f32_dynamic(float v, unsigned width)
 {
-#pragma unroll
-    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
-    return v;
+    switch (width) {
+    case 2: return group_sum_f32<2>(v);
+    case 4: return group_sum_f32<4>(v);
+    case 8: return group_sum_f32<8>(v);
+    case 16: return group_sum_f32<16>(v);
+    case 32: return group_sum_f32<32>(v);
+    case 64: return group_sum_f32<64>(v);
+    default: return v;
+    }
 }
 
 // ---- IQ2_XXS lookup tables in LDS ----------------------------------------------------------

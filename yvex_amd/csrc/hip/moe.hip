@@ -182,8 +182,9 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
 
 // ---- grouped expert projections ---------------------------------------------------------------
 
-constexpr int kPass = 4;   // pairs of one bucket handled per sweep over the expert's bytes
-constexpr int kUnitsPerLane = 4;
+constexpr int kPass = 2;          // pairs of one bucket handled per sweep over the expert's bytes
+constexpr int kUnitsPerLane = 4;  // a lane owns half a superblock: 128 columns
+constexpr int kRowsInFlight = 2;  // weight rows a wave decodes back to back before reducing
 
 struct GroupedArgs {
     const unsigned char *gate, *up;          // up == nullptr: plain projection (down)
@@ -202,6 +203,7 @@ struct GroupedArgs {
     int out_by_source_pair;
     int *status;
     unsigned rows_per_block;                 // weight rows handled by one workgroup
+    unsigned pass_slots;                     // workgroups that share one (bucket, tile), one sweep each
 };
 
 // SiLU-gated product in double, as src/graph/moe.c:605-611 orders it.
@@ -214,9 +216,189 @@ __device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weigh
     return bf16_round((float)(silu * uv * (double)route_weight));
 }
 
-// One workgroup = one (bucket, tile of weight rows). A lane owns half a superblock (four units,
-// 128 columns) of the reduction dimension; units/4 lanes span one weight row and, where that is
-// a power of two below 64, a wave covers several rows at once.
+struct LaneGeometry {
+    unsigned rows_per_wave, reduce_width, sub, seg, unit0, super;
+    bool lane_live;
+    unsigned wave, wave_begin, wave_end;
+};
+
+// One sweep of a wave over its weight rows with N live pairs of the bucket.
+template <unsigned QT, bool Q8, bool FUSED_UP, int N>
+__device__ __forceinline__ void grouped_sweep(
+    const GroupedArgs &a, const Iq2Tables &tables, const LaneGeometry &g,
+    const unsigned char *gate_e, const unsigned char *up_e, unsigned long long first_ordered,
+    float (&gate_up)[4][2][16][kPass])
+{
+    // ---- the sweep's activation rows: this lane's 128 columns stay in registers (Q8_K) ----
+    unsigned act[N][kUnitsPerLane * 8];
+    float act_scale[N];
+    const unsigned char *act_row[N];
+    float route_weight[N];
+    unsigned long long out_index[N];
+#pragma unroll
+    for (int p = 0; p < N; ++p) {
+        const unsigned long long ordered = first_ordered + p;
+        const unsigned long long source = a.order ? a.order[ordered] : ordered;
+        const unsigned long long arow = a.act_by_ordered_pair ? ordered : source / a.topk;
+        act_row[p] = (const unsigned char *)a.activations + arow * a.act_stride;
+        route_weight[p] = a.route_weights ? a.route_weights[source] : 1.0f;
+        out_index[p] = a.out_by_source_pair ? source : ordered;
+        act_scale[p] = 0.0f;
+        if constexpr (Q8) {
+            const unsigned char *blk = act_row[p] + (unsigned long long)g.super * kQ8KBytes;
+            act_scale[p] = *reinterpret_cast<const float *>(blk);
+            const unsigned char *q = blk + 4u + 32u * (g.unit0 & 7u);   // 4-byte aligned payload
+#pragma unroll
+            for (int k = 0; k < kUnitsPerLane * 2; ++k) {
+                uint4 v;
+                __builtin_memcpy(&v, q + 16 * k, 16);
+                act[p][4 * k] = v.x;
+                act[p][4 * k + 1] = v.y;
+                act[p][4 * k + 2] = v.z;
+                act[p][4 * k + 3] = v.w;
+            }
+        }
+    }
+
+    const unsigned stride = kRowsInFlight * g.rows_per_wave;
+    for (unsigned base = g.wave_begin; base < g.wave_end; base += stride) {
+        float sum_gate[kRowsInFlight][N], sum_up[kRowsInFlight][N];
+        unsigned row[kRowsInFlight];
+        bool row_live[kRowsInFlight];
+#pragma unroll
+        for (int r = 0; r < kRowsInFlight; ++r) {
+            row[r] = base + r * g.rows_per_wave + g.sub;
+            row_live[r] = g.lane_live && row[r] < g.wave_end;
+#pragma unroll
+            for (int p = 0; p < N; ++p) sum_gate[r][p] = sum_up[r][p] = 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < kRowsInFlight; ++r) {
+            const unsigned safe_row = row_live[r] ? row[r] : g.wave_begin;
+#pragma unroll
+            for (int which = 0; which < (FUSED_UP ? 2 : 1); ++which) {
+                const unsigned char *wrow =
+                    which == 0 ? gate_e + (unsigned long long)safe_row * a.row_bytes
+                               : up_e + (unsigned long long)safe_row * a.up_row_bytes;
+                float *sums = which == 0 ? sum_gate[r] : sum_up[r];
+                int whole_dot[N], whole_min[N];
+#pragma unroll
+                for (int p = 0; p < N; ++p) whole_dot[p] = whole_min[p] = 0;
+#pragma unroll
+                for (int k = 0; k < kUnitsPerLane; ++k) {
+                    const unsigned u = g.unit0 + k;
+                    Unit unit;
+                    unit_load<QT>(tables, wrow, u, unit);
+#pragma unroll
+                    for (int p = 0; p < N; ++p) {
+                        if constexpr (Q8) {
+                            const unsigned *av = &act[p][8 * k];
+                            int d = 0, d2 = 0;
+                            if constexpr (QT == QT_Q2_K) {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) {
+                                    d = dot4(unit.w[i], av[i], d);
+                                    d2 = dot4(unit.w[4 + i], av[4 + i], d2);
+                                }
+                                d = unit.factor * d + unit.factor2 * d2;
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < 8; ++i) d = dot4(unit.w[i], av[i], d);
+                                d *= unit.factor;
+                            }
+                            if constexpr (UnitTraits<QT>::kIntegerCombine) {
+                                whole_dot[p] += d;
+                                if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) {
+                                    const short *bs = reinterpret_cast<const short *>(
+                                        act_row[p] + (unsigned long long)g.super * kQ8KBytes + 260u);
+                                    const unsigned gi = u & 7u;
+                                    whole_min[p] += unit.min1 * (int)bs[2u * gi] +
+                                                    unit.min2 * (int)bs[2u * gi + 1u];
+                                }
+                            } else {
+                                sums[p] += q8_0_unit_value(wrow, u, act_scale[p], d);
+                            }
+                        } else {
+                            const float *x = reinterpret_cast<const float *>(act_row[p]) + 32ull * u;
+                            sums[p] += unit_dot_f32<QT>(unit, wrow, u, x);
+                        }
+                    }
+                }
+                if constexpr (Q8 && UnitTraits<QT>::kIntegerCombine) {
+                    // two neighbouring lanes hold the halves of one superblock: finish the exact
+                    // integer sum, then the even lane applies the single float scaling
+#pragma unroll
+                    for (int p = 0; p < N; ++p) {
+                        UnitSum t;
+                        t.dot = group_sum_i32<2>(whole_dot[p]);
+                        t.min = 0;
+                        if constexpr (QT != QT_IQ2_XXS) t.min = group_sum_i32<2>(whole_min[p]);
+                        if ((g.seg & 1u) == 0u)
+                            sums[p] += super_combine<QT>(
+                                wrow + (unsigned long long)g.super * UnitTraits<QT>::kSuperBytes,
+                                act_scale[p], t);
+                    }
+                }
+            }
+        }
+        // ---- sum across the lanes of each row, then publish ----
+#pragma unroll
+        for (int r = 0; r < kRowsInFlight; ++r) {
+#pragma unroll
+            for (int p = 0; p < N; ++p) {
+                sum_gate[r][p] = group_sum_f32_dynamic(row_live[r] ? sum_gate[r][p] : 0.0f,
+                                                       g.reduce_width);
+                if constexpr (FUSED_UP)
+                    sum_up[r][p] = group_sum_f32_dynamic(row_live[r] ? sum_up[r][p] : 0.0f,
+                                                         g.reduce_width);
+            }
+            if constexpr (FUSED_UP) {
+                // park (gate, up); the SwiGLU runs once per wave tile with every lane busy
+                const unsigned local = row[r] - g.wave_begin;
+                if (row_live[r] && g.seg == 0u && local < 16u) {
+#pragma unroll
+                    for (int p = 0; p < N; ++p) {
+                        gate_up[g.wave][0][local][p] = sum_gate[r][p];
+                        gate_up[g.wave][1][local][p] = sum_up[r][p];
+                    }
+                }
+            } else if (row_live[r] && g.seg == 0u) {
+#pragma unroll
+                for (int p = 0; p < N; ++p) {
+                    const float value = bf16_round(sum_gate[r][p]);
+                    if (!finite_f32(value)) raise_status(a.status, 1);
+                    else a.out[out_index[p] * a.out_rows + row[r]] = value;
+                }
+            }
+        }
+    }
+    if constexpr (FUSED_UP) {
+        // LDS operations of one wave complete in order: no barrier between park and read
+        const unsigned lane = threadIdx.x & 63u;
+        const unsigned local = lane >> 2;
+        const int p = (int)(lane & 3u);
+        const unsigned out_row = g.wave_begin + local;
+        if (local < 16u && out_row < g.wave_end && p < N) {
+            float rw = route_weight[0];
+            unsigned long long oi = out_index[0];
+#pragma unroll
+            for (int q = 1; q < N; ++q) {
+                if (p == q) {
+                    rw = route_weight[q];
+                    oi = out_index[q];
+                }
+            }
+            const float value = swiglu_bf16(gate_up[g.wave][0][local][p], gate_up[g.wave][1][local][p],
+                                            rw, a.limit);
+            if (!finite_f32(value)) raise_status(a.status, 1);
+            else a.out[oi * a.out_rows + out_row] = value;
+        }
+    }
+}
+
+// One workgroup = one (bucket, tile of weight rows, pass slot). A lane owns half a superblock
+// (four units, 128 columns) of the reduction dimension; units/4 lanes span one weight row and,
+// where that is a power of two below 64, a wave covers several rows at once.
 template <unsigned QT, bool Q8, bool FUSED_UP>
 __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
 {
@@ -225,7 +407,9 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
     if constexpr (QT == QT_IQ2_XXS) iq2_tables_fill(tables);
 
     const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
-    const unsigned bucket = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+    const unsigned slot = blockIdx.x % a.pass_slots;
+    const unsigned work = blockIdx.x / a.pass_slots;
+    const unsigned bucket = work / tiles, tile = work % tiles;
     unsigned long long expert = 0ull, first = 0ull, population = a.pairs;
     bool idle = false;
     if (a.expert_ids) {
@@ -238,6 +422,7 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
     } else if (bucket > 0u) {
         idle = true;
     }
+    if ((unsigned long long)slot * kPass >= population) idle = true;
     if constexpr (QT == QT_IQ2_XXS) __syncthreads();
     if (idle) return;
     if (expert >= a.experts || first + population > a.pairs) {
@@ -245,16 +430,19 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
         return;
     }
 
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned lane = threadIdx.x & 63u;
     const unsigned units = a.width >> 5;                          // multiple of 8
     const unsigned lanes_per_row = units / kUnitsPerLane;         // even, <= 64
     const bool pow2 = (lanes_per_row & (lanes_per_row - 1u)) == 0u;
-    const unsigned rows_per_wave = pow2 ? 64u / lanes_per_row : 1u;
-    const unsigned reduce_width = pow2 ? lanes_per_row : 64u;
-    const unsigned sub = lane / lanes_per_row, seg = lane % lanes_per_row;
-    const bool lane_live = sub < rows_per_wave;
-    const unsigned unit0 = seg * kUnitsPerLane;                   // all four units share a superblock
-    const unsigned super = unit0 >> 3;
+    LaneGeometry g;
+    g.rows_per_wave = pow2 ? 64u / lanes_per_row : 1u;
+    g.reduce_width = pow2 ? lanes_per_row : 64u;
+    g.sub = lane / lanes_per_row;
+    g.seg = lane % lanes_per_row;
+    g.lane_live = g.sub < g.rows_per_wave;
+    g.unit0 = g.seg * kUnitsPerLane;                              // four units, one superblock
+    g.super = g.unit0 >> 3;
+    g.wave = threadIdx.x >> 6;
 
     const unsigned char *gate_e = a.gate + expert * a.expert_bytes;
     const unsigned char *up_e = FUSED_UP ? a.up + expert * a.up_expert_bytes : nullptr;
@@ -262,173 +450,16 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
     const unsigned row_end = row_begin + a.rows_per_block < a.out_rows ? row_begin + a.rows_per_block
                                                                        : a.out_rows;
     const unsigned wave_rows = (a.rows_per_block + 3u) / 4u;      // rows per wave inside the tile
-    const unsigned wave_begin = row_begin + wave * wave_rows;
-    const unsigned wave_end = wave_begin + wave_rows < row_end ? wave_begin + wave_rows : row_end;
+    g.wave_begin = row_begin + g.wave * wave_rows;
+    g.wave_end = g.wave_begin + wave_rows < row_end ? g.wave_begin + wave_rows : row_end;
 
-    for (unsigned long long pass = 0; pass < population; pass += kPass) {
-        const int n = population - pass < (unsigned long long)kPass ? (int)(population - pass) : kPass;
-        // ---- the sweep's activation rows: this lane's 128 columns stay in registers (Q8_K) ----
-        unsigned act[kPass][kUnitsPerLane * 8];
-        float act_scale[kPass];
-        const unsigned char *act_row[kPass];
-        float route_weight[kPass];
-        unsigned long long out_index[kPass];
-#pragma unroll
-        for (int p = 0; p < kPass; ++p) {
-            const unsigned long long ordered = first + pass + (p < n ? p : 0);
-            const unsigned long long source = a.order ? a.order[ordered] : ordered;
-            const unsigned long long arow = a.act_by_ordered_pair ? ordered : source / a.topk;
-            act_row[p] = (const unsigned char *)a.activations + arow * a.act_stride;
-            route_weight[p] = a.route_weights ? a.route_weights[source] : 1.0f;
-            out_index[p] = a.out_by_source_pair ? source : ordered;
-            act_scale[p] = 0.0f;
-            if constexpr (Q8) {
-                const unsigned char *blk = act_row[p] + (unsigned long long)super * kQ8KBytes;
-                act_scale[p] = *reinterpret_cast<const float *>(blk);
-                const unsigned char *q = blk + 4u + 32u * (unit0 & 7u);   // 4-byte aligned payload
-#pragma unroll
-                for (int k = 0; k < kUnitsPerLane * 2; ++k) {
-                    uint4 v;
-                    __builtin_memcpy(&v, q + 16 * k, 16);
-                    act[p][4 * k] = v.x;
-                    act[p][4 * k + 1] = v.y;
-                    act[p][4 * k + 2] = v.z;
-                    act[p][4 * k + 3] = v.w;
-                }
-            }
-        }
-
-        for (unsigned base = wave_begin; base < wave_end; base += rows_per_wave) {
-            const unsigned row = base + sub;
-            const bool row_live = lane_live && row < wave_end;
-            const unsigned safe_row = row_live ? row : wave_begin;
-            float sum_gate[kPass], sum_up[kPass];
-#pragma unroll
-            for (int p = 0; p < kPass; ++p) sum_gate[p] = sum_up[p] = 0.0f;
-
-#pragma unroll
-            for (int which = 0; which < (FUSED_UP ? 2 : 1); ++which) {
-                const unsigned char *wrow =
-                    which == 0 ? gate_e + (unsigned long long)safe_row * a.row_bytes
-                               : up_e + (unsigned long long)safe_row * a.up_row_bytes;
-                float *sums = which == 0 ? sum_gate : sum_up;
-                UnitSum whole[kPass];
-#pragma unroll
-                for (int p = 0; p < kPass; ++p) whole[p].dot = whole[p].min = 0;
-#pragma unroll
-                for (int k = 0; k < kUnitsPerLane; ++k) {
-                    const unsigned u = unit0 + k;
-                    Unit unit;
-                    unit_load<QT>(tables, wrow, u, unit);
-#pragma unroll
-                    for (int p = 0; p < kPass; ++p) {
-                        if (p < n) {
-                            if constexpr (Q8) {
-                                const unsigned *av = &act[p][8 * k];
-                                int d = 0, d2 = 0;
-                                if constexpr (QT == QT_Q2_K) {
-#pragma unroll
-                                    for (int i = 0; i < 4; ++i) {
-                                        d = dot4(unit.w[i], av[i], d);
-                                        d2 = dot4(unit.w[4 + i], av[4 + i], d2);
-                                    }
-                                    d = unit.factor * d + unit.factor2 * d2;
-                                } else {
-#pragma unroll
-                                    for (int i = 0; i < 8; ++i) d = dot4(unit.w[i], av[i], d);
-                                    d *= unit.factor;
-                                }
-                                if constexpr (UnitTraits<QT>::kIntegerCombine) {
-                                    whole[p].dot += d;
-                                    if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) {
-                                        const short *bs = reinterpret_cast<const short *>(
-                                            act_row[p] + (unsigned long long)super * kQ8KBytes + 260u);
-                                        const unsigned g = u & 7u;
-                                        whole[p].min += unit.min1 * (int)bs[2u * g] +
-                                                        unit.min2 * (int)bs[2u * g + 1u];
-                                    }
-                                } else {
-                                    sums[p] += q8_0_unit_value(wrow, u, act_scale[p], d);
-                                }
-                            } else {
-                                const float *x = reinterpret_cast<const float *>(act_row[p]) + 32ull * u;
-                                sums[p] += unit_dot_f32<QT>(unit, wrow, u, x);
-                            }
-                        }
-                    }
-                }
-                if constexpr (Q8 && UnitTraits<QT>::kIntegerCombine) {
-                    // two neighbouring lanes hold the halves of one superblock: finish the exact
-                    // integer sum, then the even lane applies the single float scaling
-#pragma unroll
-                    for (int p = 0; p < kPass; ++p) {
-                        if (p < n) {
-                            UnitSum t = whole[p];
-                            t.dot += __shfl_xor(t.dot, 1, kWave);
-                            if constexpr (QT != QT_IQ2_XXS) t.min += __shfl_xor(t.min, 1, kWave);
-                            if ((seg & 1u) == 0u)
-                                sums[p] += super_combine<QT>(
-                                    wrow + (unsigned long long)super * UnitTraits<QT>::kSuperBytes,
-                                    act_scale[p], t);
-                        }
-                    }
-                }
-            }
-            // ---- sum across the lanes of each row ----
-#pragma unroll
-            for (int p = 0; p < kPass; ++p) {
-                if (p < n) {
-                    if (!row_live) sum_gate[p] = sum_up[p] = 0.0f;
-                    for (unsigned offset = reduce_width >> 1; offset > 0u; offset >>= 1) {
-                        sum_gate[p] += __shfl_xor(sum_gate[p], (int)offset, kWave);
-                        if constexpr (FUSED_UP) sum_up[p] += __shfl_xor(sum_up[p], (int)offset, kWave);
-                    }
-                }
-            }
-            if constexpr (FUSED_UP) {
-                // park (gate, up); the SwiGLU runs once per wave tile with every lane busy
-                const unsigned local = row - wave_begin;
-                if (row_live && seg == 0u && local < 16u) {
-#pragma unroll
-                    for (int p = 0; p < kPass; ++p) {
-                        gate_up[wave][0][local][p] = sum_gate[p];
-                        gate_up[wave][1][local][p] = sum_up[p];
-                    }
-                }
-            } else {
-                if (row_live && seg == 0u) {
-#pragma unroll
-                    for (int p = 0; p < kPass; ++p) {
-                        if (p < n) {
-                            const float value = bf16_round(sum_gate[p]);
-                            if (!finite_f32(value)) raise_status(a.status, 1);
-                            else a.out[out_index[p] * a.out_rows + row] = value;
-                        }
-                    }
-                }
-            }
-        }
-        if constexpr (FUSED_UP) {
-            // LDS operations of one wave complete in order: no barrier between park and read
-            const unsigned local = lane >> 2;
-            const int p = (int)(lane & 3u);
-            const unsigned row = wave_begin + local;
-            if (local < 16u && row < wave_end && p < n) {
-                float rw = route_weight[0];
-                unsigned long long oi = out_index[0];
-#pragma unroll
-                for (int q = 1; q < kPass; ++q) {
-                    if (p == q) {
-                        rw = route_weight[q];
-                        oi = out_index[q];
-                    }
-                }
-                const float value = swiglu_bf16(gate_up[wave][0][local][p], gate_up[wave][1][local][p],
-                                                rw, a.limit);
-                if (!finite_f32(value)) raise_status(a.status, 1);
-                else a.out[oi * a.out_rows + row] = value;
-            }
-        }
+    for (unsigned long long pass = (unsigned long long)slot * kPass; pass < population;
+         pass += (unsigned long long)a.pass_slots * kPass) {
+        const unsigned long long left = population - pass;
+        if (left >= 2ull)
+            grouped_sweep<QT, Q8, FUSED_UP, 2>(a, tables, g, gate_e, up_e, first + pass, gate_up);
+        else
+            grouped_sweep<QT, Q8, FUSED_UP, 1>(a, tables, g, gate_e, up_e, first + pass, gate_up);
     }
 }
 
@@ -460,7 +491,7 @@ static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, unsigned bu
                           hipStream_t stream)
 {
     const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
-    const unsigned long long grid = (unsigned long long)buckets * tiles;
+    const unsigned long long grid = (unsigned long long)buckets * tiles * a.pass_slots;
     if (grid > 0x7fffffffull) return ST_BOUNDS;
     if (fused) {
         if (q8) grouped_kernel<QT, true, true><<<(unsigned)grid, 256, 0, stream>>>(a);
@@ -588,6 +619,8 @@ extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *act
     a.status = status;
     a.rows_per_block = 64u;
     const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
+    // a single known bucket (shared expert): its sweeps run side by side instead of in a loop
+    a.pass_slots = expert_ids ? 1u : (unsigned)((pairs + kPass - 1u) / kPass);
     return dispatch_grouped(w->gate_qtype, a, act_q8 != 0, true, buckets, as_stream(stream));
 }
 
@@ -630,6 +663,7 @@ extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *i
     a.status = status;
     a.rows_per_block = 256u;
     const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
+    a.pass_slots = expert_ids ? 1u : (unsigned)((pairs + kPass - 1u) / kPass);
     return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, buckets, as_stream(stream));
 }
 
