@@ -223,15 +223,20 @@ struct LaneGeometry {
 };
 
 // One sweep of a wave over its weight rows with N live pairs of the bucket.
+// Each iteration handles kRowsInFlight row groups; the packed bytes of the next iteration are
+// requested before the current one is decoded, so HBM latency hides behind the decode.
 template <unsigned QT, bool Q8, bool FUSED_UP, int N>
 __device__ __forceinline__ void grouped_sweep(
     const GroupedArgs &a, const Iq2Tables &tables, const LaneGeometry &g,
     const unsigned char *gate_e, const unsigned char *up_e, unsigned long long first_ordered,
     float (&gate_up)[4][2][16][kPass])
 {
+    constexpr int kStreams = FUSED_UP ? 2 : 1;
+    constexpr int kRows = Q8 ? kRowsInFlight : 1;
     // ---- the sweep's activation rows: this lane's 128 columns stay in registers (Q8_K) ----
-    unsigned act[N][kUnitsPerLane * 8];
+    unsigned act[N][Q8 ? kUnitsPerLane * 8 : 1];
     float act_scale[N];
+    int act_bsum[N][(QT == QT_Q4_K || QT == QT_Q2_K) ? 8 : 1];
     const unsigned char *act_row[N];
     float route_weight[N];
     unsigned long long out_index[N];
@@ -257,38 +262,56 @@ __device__ __forceinline__ void grouped_sweep(
                 act[p][4 * k + 2] = v.z;
                 act[p][4 * k + 3] = v.w;
             }
+            if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) {
+                const short *bs = reinterpret_cast<const short *>(blk + 260u) + 2u * (g.unit0 & 7u);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) act_bsum[p][i] = bs[i];
+            }
         }
     }
 
-    const unsigned stride = kRowsInFlight * g.rows_per_wave;
-    for (unsigned base = g.wave_begin; base < g.wave_end; base += stride) {
-        float sum_gate[kRowsInFlight][N], sum_up[kRowsInFlight][N];
-        unsigned row[kRowsInFlight];
-        bool row_live[kRowsInFlight];
+    const unsigned stride = kRows * g.rows_per_wave;
+    LaneChunk<QT> next[kRows][kStreams];
+    auto request = [&](unsigned base) {
 #pragma unroll
-        for (int r = 0; r < kRowsInFlight; ++r) {
+        for (int r = 0; r < kRows; ++r) {
+            const unsigned want = base + r * g.rows_per_wave + g.sub;
+            const unsigned safe_row = (g.lane_live && want < g.wave_end) ? want : g.wave_begin;
+            next[r][0].load(gate_e + (unsigned long long)safe_row * a.row_bytes, g.unit0);
+            if constexpr (FUSED_UP)
+                next[r][1].load(up_e + (unsigned long long)safe_row * a.up_row_bytes, g.unit0);
+        }
+    };
+    if (g.wave_begin < g.wave_end) request(g.wave_begin);
+
+    for (unsigned base = g.wave_begin; base < g.wave_end; base += stride) {
+        LaneChunk<QT> chunk[kRows][kStreams];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int w = 0; w < kStreams; ++w) chunk[r][w] = next[r][w];
+        if (base + stride < g.wave_end) request(base + stride);
+
+        float sums[kRows][kStreams][N];
+        unsigned row[kRows];
+        bool row_live[kRows];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
             row[r] = base + r * g.rows_per_wave + g.sub;
             row_live[r] = g.lane_live && row[r] < g.wave_end;
 #pragma unroll
-            for (int p = 0; p < N; ++p) sum_gate[r][p] = sum_up[r][p] = 0.0f;
-        }
-#pragma unroll
-        for (int r = 0; r < kRowsInFlight; ++r) {
-            const unsigned safe_row = row_live[r] ? row[r] : g.wave_begin;
-#pragma unroll
-            for (int which = 0; which < (FUSED_UP ? 2 : 1); ++which) {
-                const unsigned char *wrow =
-                    which == 0 ? gate_e + (unsigned long long)safe_row * a.row_bytes
-                               : up_e + (unsigned long long)safe_row * a.up_row_bytes;
-                float *sums = which == 0 ? sum_gate[r] : sum_up[r];
+            for (int w = 0; w < kStreams; ++w) {
+                const LaneChunk<QT> &c = chunk[r][w];
                 int whole_dot[N], whole_min[N];
 #pragma unroll
-                for (int p = 0; p < N; ++p) whole_dot[p] = whole_min[p] = 0;
+                for (int p = 0; p < N; ++p) {
+                    whole_dot[p] = whole_min[p] = 0;
+                    sums[r][w][p] = 0.0f;
+                }
 #pragma unroll
                 for (int k = 0; k < kUnitsPerLane; ++k) {
-                    const unsigned u = g.unit0 + k;
                     Unit unit;
-                    unit_load<QT>(tables, wrow, u, unit);
+                    c.decode(tables, k, g.unit0, unit);
 #pragma unroll
                     for (int p = 0; p < N; ++p) {
                         if constexpr (Q8) {
@@ -300,72 +323,65 @@ __device__ __forceinline__ void grouped_sweep(
                                     d = dot4(unit.w[i], av[i], d);
                                     d2 = dot4(unit.w[4 + i], av[4 + i], d2);
                                 }
-                                d = unit.factor * d + unit.factor2 * d2;
+                                d = __mul24(unit.factor, d) + __mul24(unit.factor2, d2);
                             } else {
 #pragma unroll
                                 for (int i = 0; i < 8; ++i) d = dot4(unit.w[i], av[i], d);
-                                d *= unit.factor;
+                                if constexpr (QT != QT_Q8_0) d = __mul24(d, unit.factor);
                             }
                             if constexpr (UnitTraits<QT>::kIntegerCombine) {
                                 whole_dot[p] += d;
-                                if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) {
-                                    const short *bs = reinterpret_cast<const short *>(
-                                        act_row[p] + (unsigned long long)g.super * kQ8KBytes + 260u);
-                                    const unsigned gi = u & 7u;
-                                    whole_min[p] += unit.min1 * (int)bs[2u * gi] +
-                                                    unit.min2 * (int)bs[2u * gi + 1u];
-                                }
+                                if constexpr (QT == QT_Q4_K || QT == QT_Q2_K)
+                                    whole_min[p] += unit.min1 * act_bsum[p][2 * k] +
+                                                    unit.min2 * act_bsum[p][2 * k + 1];
                             } else {
-                                sums[p] += q8_0_unit_value(wrow, u, act_scale[p], d);
+                                sums[r][w][p] += c.unit_value(k, act_scale[p], d);
                             }
                         } else {
-                            const float *x = reinterpret_cast<const float *>(act_row[p]) + 32ull * u;
-                            sums[p] += unit_dot_f32<QT>(unit, wrow, u, x);
+                            const float *x = reinterpret_cast<const float *>(act_row[p]) +
+                                             32ull * (g.unit0 + k);
+                            sums[r][w][p] += chunk_unit_dot_f32<QT>(c, k, unit, x);
                         }
                     }
                 }
                 if constexpr (Q8 && UnitTraits<QT>::kIntegerCombine) {
                     // two neighbouring lanes hold the halves of one superblock: finish the exact
-                    // integer sum, then the even lane applies the single float scaling
+                    // integer sum; both compute the float value, the odd lane contributes zero
 #pragma unroll
                     for (int p = 0; p < N; ++p) {
                         UnitSum t;
                         t.dot = group_sum_i32<2>(whole_dot[p]);
                         t.min = 0;
                         if constexpr (QT != QT_IQ2_XXS) t.min = group_sum_i32<2>(whole_min[p]);
-                        if ((g.seg & 1u) == 0u)
-                            sums[p] += super_combine<QT>(
-                                wrow + (unsigned long long)g.super * UnitTraits<QT>::kSuperBytes,
-                                act_scale[p], t);
+                        const float v = c.combine(act_scale[p], t);
+                        sums[r][w][p] = (g.seg & 1u) ? 0.0f : v;
                     }
                 }
             }
         }
         // ---- sum across the lanes of each row, then publish ----
 #pragma unroll
-        for (int r = 0; r < kRowsInFlight; ++r) {
+        for (int r = 0; r < kRows; ++r) {
 #pragma unroll
-            for (int p = 0; p < N; ++p) {
-                sum_gate[r][p] = group_sum_f32_dynamic(row_live[r] ? sum_gate[r][p] : 0.0f,
-                                                       g.reduce_width);
-                if constexpr (FUSED_UP)
-                    sum_up[r][p] = group_sum_f32_dynamic(row_live[r] ? sum_up[r][p] : 0.0f,
-                                                         g.reduce_width);
-            }
+            for (int w = 0; w < kStreams; ++w)
+#pragma unroll
+                for (int p = 0; p < N; ++p)
+                    sums[r][w][p] = group_sum_f32_dynamic(row_live[r] ? sums[r][w][p] : 0.0f,
+                                                          g.reduce_width);
             if constexpr (FUSED_UP) {
                 // park (gate, up); the SwiGLU runs once per wave tile with every lane busy
                 const unsigned local = row[r] - g.wave_begin;
                 if (row_live[r] && g.seg == 0u && local < 16u) {
 #pragma unroll
                     for (int p = 0; p < N; ++p) {
-                        gate_up[g.wave][0][local][p] = sum_gate[r][p];
-                        gate_up[g.wave][1][local][p] = sum_up[r][p];
+                        gate_up[g.wave][0][local][p] = sums[r][0][p];
+                        gate_up[g.wave][1][local][p] = sums[r][1][p];
                     }
                 }
             } else if (row_live[r] && g.seg == 0u) {
 #pragma unroll
                 for (int p = 0; p < N; ++p) {
-                    const float value = bf16_round(sum_gate[r][p]);
+                    const float value = bf16_round(sums[r][0][p]);
                     if (!finite_f32(value)) raise_status(a.status, 1);
                     else a.out[out_index[p] * a.out_rows + row[r]] = value;
                 }

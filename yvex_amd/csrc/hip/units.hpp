@@ -93,6 +93,152 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
     }
 }
 
+// ---- a lane's share of one weight row, loaded first and decoded later -----------------------
+//
+// The grouped kernels give every lane four consecutive units (half a superblock) of each weight
+// row. LaneChunk keeps those packed bytes in registers so all loads of an iteration can be in
+// flight before the first decode starts.
+
+template <unsigned QT>
+struct LaneChunk;
+
+template <>
+struct LaneChunk<QT_IQ2_XXS> {
+    unsigned q[8];
+    unsigned d16;
+    __device__ __forceinline__ void load(const unsigned char *row, unsigned unit0)
+    {
+        const unsigned char *b = row + (unit0 >> 3) * 66u;
+        uint4 lo, hi;
+        d16 = load_u16(b);
+        __builtin_memcpy(&lo, b + 2u + 8u * (unit0 & 7u), 16);
+        __builtin_memcpy(&hi, b + 18u + 8u * (unit0 & 7u), 16);
+        q[0] = lo.x; q[1] = lo.y; q[2] = lo.z; q[3] = lo.w;
+        q[4] = hi.x; q[5] = hi.y; q[6] = hi.z; q[7] = hi.w;
+    }
+    __device__ __forceinline__ void decode(const Iq2Tables &t, int k, unsigned, Unit &unit) const
+    {
+        unit.factor = unit.factor2 = iq2_unit(t, q[2 * k], q[2 * k + 1], unit.w);
+        unit.min1 = unit.min2 = 0;
+    }
+    __device__ __forceinline__ float combine(float act_scale, UnitSum sum) const
+    {
+        return 0.125f * f16_bits_to_float(d16) * act_scale * (float)sum.dot;
+    }
+};
+
+template <>
+struct LaneChunk<QT_Q4_K> {
+    unsigned q[16];     // two 32-byte nibble chunks
+    unsigned head[4];   // f16 d, f16 dmin, 12 scale bytes
+    __device__ __forceinline__ void load(const unsigned char *row, unsigned unit0)
+    {
+        const unsigned char *b = row + (unit0 >> 3) * 144u;
+        uint4 v;
+        __builtin_memcpy(&v, b, 16);
+        head[0] = v.x; head[1] = v.y; head[2] = v.z; head[3] = v.w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_memcpy(&v, b + 16u + 32u * ((unit0 & 7u) >> 1) + 16u * i, 16);
+            q[4 * i] = v.x; q[4 * i + 1] = v.y; q[4 * i + 2] = v.z; q[4 * i + 3] = v.w;
+        }
+    }
+    __device__ __forceinline__ unsigned scale_byte(unsigned i) const
+    {
+        return (head[1u + (i >> 2)] >> (8u * (i & 3u))) & 255u;
+    }
+    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned unit0, Unit &unit) const
+    {
+        const unsigned g = (unit0 & 7u) + (unsigned)k, shift = (g & 1u) * 4u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) unit.w[i] = (q[8 * (k >> 1) + i] >> shift) & 0x0f0f0f0fu;
+        unsigned sc, mn;
+        if (g < 4u) {
+            sc = scale_byte(g) & 63u;
+            mn = scale_byte(g + 4u) & 63u;
+        } else {
+            sc = (scale_byte(g + 4u) & 15u) | ((scale_byte(g - 4u) >> 6) << 4);
+            mn = (scale_byte(g + 4u) >> 4) | ((scale_byte(g) >> 6) << 4);
+        }
+        unit.factor = unit.factor2 = (int)sc;
+        unit.min1 = unit.min2 = (int)mn;
+    }
+    __device__ __forceinline__ float combine(float act_scale, UnitSum sum) const
+    {
+        const float left = act_scale * f16_bits_to_float(head[0] & 0xffffu) * (float)sum.dot;
+        const float right = act_scale * f16_bits_to_float(head[0] >> 16) * (float)sum.min;
+        return left - right;
+    }
+};
+
+template <>
+struct LaneChunk<QT_Q2_K> {
+    unsigned q[8];       // one 32-byte plane chunk shared by the lane's four units
+    unsigned scales[2];  // eight scale/min bytes
+    unsigned dd;         // f16 d, f16 dmin
+    __device__ __forceinline__ void load(const unsigned char *row, unsigned unit0)
+    {
+        const unsigned char *b = row + (unit0 >> 3) * 84u;
+        uint4 lo, hi;
+        __builtin_memcpy(&lo, b + 16u + ((unit0 & 7u) >> 2) * 32u, 16);
+        __builtin_memcpy(&hi, b + 32u + ((unit0 & 7u) >> 2) * 32u, 16);
+        q[0] = lo.x; q[1] = lo.y; q[2] = lo.z; q[3] = lo.w;
+        q[4] = hi.x; q[5] = hi.y; q[6] = hi.z; q[7] = hi.w;
+        uint2 sc = load_u32x2(b + 2u * (unit0 & 7u));
+        scales[0] = sc.x;
+        scales[1] = sc.y;
+        dd = load_u32(b + 80u);
+    }
+    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned, Unit &unit) const
+    {
+        const unsigned shift = 2u * (unsigned)k;   // unit0 & 3 == 0
+#pragma unroll
+        for (int i = 0; i < 8; ++i) unit.w[i] = (q[i] >> shift) & 0x03030303u;
+        const unsigned pair = (scales[k >> 1] >> (16u * (k & 1))) & 0xffffu;
+        unit.factor = pair & 15u;
+        unit.min1 = (pair >> 4) & 15u;
+        unit.factor2 = (pair >> 8) & 15u;
+        unit.min2 = pair >> 12;
+    }
+    __device__ __forceinline__ float combine(float act_scale, UnitSum sum) const
+    {
+        const float left = act_scale * f16_bits_to_float(dd & 0xffffu) * (float)sum.dot;
+        const float right = act_scale * f16_bits_to_float(dd >> 16) * (float)sum.min;
+        return left - right;
+    }
+};
+
+template <>
+struct LaneChunk<QT_Q8_0> {
+    unsigned q[32];
+    unsigned d16[4];
+    __device__ __forceinline__ void load(const unsigned char *row, unsigned unit0)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const unsigned char *b = row + (unit0 + k) * 34u;
+            uint4 lo, hi;
+            d16[k] = load_u16(b);
+            __builtin_memcpy(&lo, b + 2u, 16);
+            __builtin_memcpy(&hi, b + 18u, 16);
+            q[8 * k] = lo.x; q[8 * k + 1] = lo.y; q[8 * k + 2] = lo.z; q[8 * k + 3] = lo.w;
+            q[8 * k + 4] = hi.x; q[8 * k + 5] = hi.y; q[8 * k + 6] = hi.z; q[8 * k + 7] = hi.w;
+        }
+    }
+    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned, Unit &unit) const
+    {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) unit.w[i] = q[8 * k + i];
+        unit.factor = unit.factor2 = 1;
+        unit.min1 = unit.min2 = 0;
+    }
+    __device__ __forceinline__ float unit_value(int k, float act_scale, int dot) const
+    {
+        return f16_bits_to_float(d16[k]) * act_scale * (float)dot;
+    }
+    __device__ __forceinline__ float combine(float, UnitSum) const { return 0.0f; }
+};
+
 // Unit against Q8_K block `act` (292 bytes, 4-byte aligned); g = unit index inside the block.
 template <unsigned QT>
 __device__ __forceinline__ UnitSum unit_dot_q8(const Unit &unit, const unsigned char *act,
@@ -191,6 +337,56 @@ __device__ __forceinline__ float unit_dot_f32(const Unit &unit, const unsigned c
         float d = f16_bits_to_float(load_u16(b + 80u)), dm = f16_bits_to_float(load_u16(b + 82u));
         return (d * (float)unit.factor * s1 - dm * (float)unit.min1 * xs1) +
                (d * (float)unit.factor2 * s2 - dm * (float)unit.min2 * xs2);
+    }
+}
+
+// Partial sums of one decoded unit against 32 F32 activations: halves of 16 values each, and
+// (for the affine qtypes) the matching sums of the activations themselves.
+struct UnitF32 {
+    float s1, s2, xs1, xs2;
+};
+
+template <bool AFFINE>
+__device__ __forceinline__ UnitF32 unit_dot_f32_core(const Unit &unit, const float *x)
+{
+    UnitF32 r{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + 4 * i);
+        const unsigned w = unit.w[i];
+        float p = 0.0f;
+        p = fmaf((float)(signed char)(w & 255u), v.x, p);
+        p = fmaf((float)(signed char)((w >> 8) & 255u), v.y, p);
+        p = fmaf((float)(signed char)((w >> 16) & 255u), v.z, p);
+        p = fmaf((float)(signed char)(w >> 24), v.w, p);
+        if (i < 4) r.s1 += p; else r.s2 += p;
+        if constexpr (AFFINE) {
+            const float xs = (v.x + v.y) + (v.z + v.w);
+            if (i < 4) r.xs1 += xs; else r.xs2 += xs;
+        }
+    }
+    return r;
+}
+
+// Contribution of unit k of a LaneChunk to the row dot with F32 activations x (32 floats).
+template <unsigned QT>
+__device__ __forceinline__ float chunk_unit_dot_f32(const LaneChunk<QT> &c, int k, const Unit &unit,
+                                                    const float *x)
+{
+    const UnitF32 r = unit_dot_f32_core<QT == QT_Q4_K || QT == QT_Q2_K>(unit, x);
+    if constexpr (QT == QT_IQ2_XXS) {
+        const float gs = f16_bits_to_float(c.d16) * (0.5f + (float)((unit.factor - 1) >> 1)) * 0.25f;
+        return gs * (r.s1 + r.s2);
+    } else if constexpr (QT == QT_Q8_0) {
+        return f16_bits_to_float(c.d16[k]) * (r.s1 + r.s2);
+    } else if constexpr (QT == QT_Q4_K) {
+        const float d = f16_bits_to_float(c.head[0] & 0xffffu) * (float)unit.factor;
+        const float m = f16_bits_to_float(c.head[0] >> 16) * (float)unit.min1;
+        return d * (r.s1 + r.s2) - m * (r.xs1 + r.xs2);
+    } else {
+        const float d = f16_bits_to_float(c.dd & 0xffffu), dm = f16_bits_to_float(c.dd >> 16);
+        return (d * (float)unit.factor * r.s1 - dm * (float)unit.min1 * r.xs1) +
+               (d * (float)unit.factor2 * r.s2 - dm * (float)unit.min2 * r.xs2);
     }
 }
 
