@@ -136,8 +136,8 @@ def main() -> int:
     acts = layer.act_q8_rows if layer.act_q8 else x
 
     def up_only():
-        K.moe_up(layer.routed, acts, layer.act_q8, layer.selected, layer.weights, layer.worklist,
-                 pairs, TOPK, EXPERTS, layer.limit, layer.intermediate_f32, layer.status)
+        K.moe_up(layer.routed, acts, layer.act_q8, layer.weights, layer.worklist, pairs, TOPK,
+                 EXPERTS, layer.limit, layer.intermediate_f32, layer.status)
 
     def down_only():
         mid = layer.intermediate_q8 if layer.act_q8 else layer.intermediate_f32

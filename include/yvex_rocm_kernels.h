@@ -74,10 +74,13 @@ int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t row
  * device memory:
  *   order[pairs]            source pair of each ordered position
  *   expert_ids[experts], bucket_offsets[experts + 1], bucket_populations[experts]
- *   counts[4]               {bucket_count, maximum_population, pair_count, 0} */
+ *   sweep_offsets[experts + 1]  running count of weight sweeps (two pairs per sweep) before each
+ *                           bucket: the grouped kernels spread sweeps, not buckets, over the chip
+ *   counts[4]               {bucket_count, maximum_population, pair_count, sweep_count} */
 int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
-                            uint64_t experts, uint64_t *order, uint64_t *expert_ids, uint64_t *bucket_offsets,
-                            uint64_t *bucket_populations, uint64_t *counts, int *status,
+                            uint64_t experts, uint64_t *order, uint64_t *expert_ids,
+                            uint64_t *bucket_offsets, uint64_t *bucket_populations,
+                            uint64_t *sweep_offsets, uint64_t *counts, int *status,
                             yvex_hip_stream stream);
 
 /* Expert matrices of one MoE layer. routed_* are expert-major: expert e starts at
@@ -93,25 +96,38 @@ typedef struct {
 /* Replaces yvex_moe_grouped_up_rows (+ _up_tensorcore) (moe_kernels.cu:431-516,
  * tensorcore.cu:527-626): for every ordered pair p of every bucket,
  *   intermediate[p, i] = bf16(silu(min(g,L)) * clamp(u,+-L) * route_weight), g/u = gate/up row i
- * dotted with the pair's source row. Each expert's bytes are read once per bucket.
+ * dotted with the pair's source row (source pair / topk). An expert's bytes are read once per
+ * two pairs of its bucket.
  * activations: Q8_K rows [rows][hidden/256 * 292] when act_q8, else F32 rows [rows][hidden].
- * order == NULL means pair p is ordered position p and its expert is p / pairs_per_bucket...
- * see yvex_hip_moe_shared below for the single-expert form. */
+ * With expert_ids == NULL the call is the single-expert form: one bucket holding pairs
+ * 0..pairs-1 of expert 0, pair p reading activation row p / topk, weight 1 when
+ * route_weights == NULL.
+ * shared != NULL folds the layer's shared expert into the same launch: it must have the same
+ * qtypes and shapes as the routed experts (else UNSUPPORTED: launch it separately), is applied
+ * to activation rows 0..shared_rows-1 with weight 1 and writes shared_intermediate[row, i]. */
 int yvex_hip_moe_up(const yvex_hip_expert_weights *weights, const void *activations, int act_q8,
-                    const uint64_t *selected, const float *route_weights, const uint64_t *order,
+                    const float *route_weights, const uint64_t *order,
                     const uint64_t *expert_ids, const uint64_t *bucket_offsets,
-                    const uint64_t *bucket_populations, const uint64_t *counts,
-                    uint64_t pairs, uint64_t topk, uint64_t experts, double limit,
-                    float *intermediate, int *status, yvex_hip_stream stream);
+                    const uint64_t *bucket_populations, const uint64_t *sweep_offsets,
+                    const uint64_t *counts, uint64_t pairs, uint64_t topk, uint64_t experts,
+                    double limit,
+                    float *intermediate, const yvex_hip_expert_weights *shared,
+                    uint64_t shared_rows, float *shared_intermediate, int *status,
+                    yvex_hip_stream stream);
 
 /* Replaces yvex_moe_grouped_down_rows (+ _down_tensorcore) (moe_kernels.cu:518-582,
  * tensorcore.cu:628-702): pair_outputs[source_pair, c] = bf16(dot(down row c, intermediate of
- * the ordered pair)). intermediate is Q8_K [pairs][intermediate/256*292] when act_q8 else F32. */
+ * the ordered pair)). intermediate is Q8_K [pairs][intermediate/256*292] when act_q8 else F32,
+ * indexed by ordered position. shared != NULL folds the shared expert in as for the up sweep:
+ * shared_outputs[row, c] = bf16(dot(shared down row c, shared_intermediate row)). */
 int yvex_hip_moe_down(const yvex_hip_expert_weights *weights, const void *intermediate,
                       int act_q8, const uint64_t *order, const uint64_t *expert_ids,
                       const uint64_t *bucket_offsets, const uint64_t *bucket_populations,
-                      const uint64_t *counts, uint64_t pairs, uint64_t experts,
-                      float *pair_outputs, int *status, yvex_hip_stream stream);
+                      const uint64_t *sweep_offsets, const uint64_t *counts, uint64_t pairs,
+                      uint64_t experts,
+                      float *pair_outputs, const yvex_hip_expert_weights *shared,
+                      uint64_t shared_rows, const void *shared_intermediate,
+                      float *shared_outputs, int *status, yvex_hip_stream stream);
 
 /* Replaces yvex_moe_reduce_rows + yvex_moe_combine_rows (moe_kernels.cu:584-616):
  * routed[row, c] = sum over rank (in rank order, fp32) of pair_outputs[row*topk+rank, c];
@@ -119,6 +135,11 @@ int yvex_hip_moe_down(const yvex_hip_expert_weights *weights, const void *interm
 int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows, uint64_t topk,
                                 uint64_t hidden, const float *shared, float *routed,
                                 float *combined, int *status, yvex_hip_stream stream);
+
+/* Bandwidth probe (the reference publishes the same fact at backend start,
+ * src/backend/cuda/backend.c:1550): streams `bytes` of device memory through 16-byte loads.
+ * Time it with events; `sink` is a 4-byte device word that is practically never written. */
+int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_hip_stream stream);
 
 /* Device-side fill, usable where a captured graph must not hold a memset node. */
 int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream stream);

@@ -165,41 +165,132 @@ __constant__ unsigned short k_iq2_digits[256] = {YVEX_IQ2XXS_GRID_VALUES};
 struct Iq2Tables {
     uint2 magnitudes[256];
     uint2 signmask[128];
+    // magnitudes, byte masks and the +1 bytes of subgroup j of one 32-weight group
+    __device__ __forceinline__ void lookup(unsigned grids, unsigned aux, unsigned j, uint2 &m,
+                                           uint2 &mask, uint2 &one) const
+    {
+        m = magnitudes[(grids >> (8u * j)) & 255u];
+        mask = signmask[(aux >> (7u * j)) & 127u];
+        one = make_uint2(mask.x & 0x01010101u, mask.y & 0x01010101u);
+    }
 };
+
+__device__ __forceinline__ uint2 iq2_magnitude_entry(unsigned i)
+{
+    const unsigned digits = k_iq2_digits[i];
+    unsigned lo = 0u, hi = 0u;
+#pragma unroll
+    for (unsigned l = 0; l < 4u; ++l) {
+        const unsigned a = (digits >> (2u * l)) & 3u, b = (digits >> (2u * l + 8u)) & 3u;
+        lo |= (a == 0u ? 8u : a == 1u ? 25u : 43u) << (8u * l);
+        hi |= (b == 0u ? 8u : b == 1u ? 25u : 43u) << (8u * l);
+    }
+    return make_uint2(lo, hi);
+}
+
+__device__ __forceinline__ uint2 iq2_signmask_entry(unsigned i)
+{
+    const unsigned s = i | ((__popc(i) & 1u) << 7);
+    unsigned lo = 0u, hi = 0u;
+#pragma unroll
+    for (unsigned l = 0; l < 4u; ++l) {
+        if ((s >> l) & 1u) lo |= 0xffu << (8u * l);
+        if ((s >> (l + 4u)) & 1u) hi |= 0xffu << (8u * l);
+    }
+    return make_uint2(lo, hi);
+}
 
 __device__ __forceinline__ void iq2_tables_fill(Iq2Tables &t)
 {
-    for (unsigned i = threadIdx.x; i < 256u; i += blockDim.x) {
-        unsigned digits = k_iq2_digits[i], lo = 0u, hi = 0u;
-#pragma unroll
-        for (unsigned l = 0; l < 4u; ++l) {
-            unsigned a = (digits >> (2u * l)) & 3u, b = (digits >> (2u * l + 8u)) & 3u;
-            lo |= (a == 0u ? 8u : a == 1u ? 25u : 43u) << (8u * l);
-            hi |= (b == 0u ? 8u : b == 1u ? 25u : 43u) << (8u * l);
-        }
-        t.magnitudes[i] = make_uint2(lo, hi);
+    for (unsigned i = threadIdx.x; i < 256u; i += blockDim.x) t.magnitudes[i] = iq2_magnitude_entry(i);
+    for (unsigned i = threadIdx.x; i < 128u; i += blockDim.x) t.signmask[i] = iq2_signmask_entry(i);
+}
+
+// The same tables replicated 32 times for the persistent kernels. Replica r of entry e sits at
+// [e * 32 + r] and a lane always reads replica (lane % 32), so the 32 lanes of a half-wave hit
+// 32 different bank groups whatever entries they ask for: random lookups never conflict.
+// Layout in LDS (128 KB of the CU's 160 KB):
+//   [0, 64 KB)      magnitudes: 256 entries x 32 replicas x 8 bytes
+//   [64 KB, 128 KB) signs:      128 entries x 32 replicas x 16 bytes {mask.x, mask.y, one.x, one.y}
+// Byte addresses are assembled with one byte-permute (magnitudes) or one shift-or (signs).
+constexpr unsigned kIq2Replicas = 32u;
+constexpr unsigned kIq2SignBase = 256u * kIq2Replicas * 8u;
+constexpr unsigned kIq2WideBytes = kIq2SignBase + 128u * kIq2Replicas * 16u;
+
+// LDS reads by byte address. The host pass of the compiler never executes these.
+__device__ __forceinline__ uint2 lds_read_uint2(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const uint2 *>(address);
+#else
+    (void)address;
+    return make_uint2(0u, 0u);
+#endif
+}
+__device__ __forceinline__ uint4 lds_read_uint4(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const uint4 *>(address);
+#else
+    (void)address;
+    return make_uint4(0u, 0u, 0u, 0u);
+#endif
+}
+__device__ __forceinline__ unsigned lds_address_of(const void *shared_pointer)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const void *)shared_pointer;
+#else
+    (void)shared_pointer;
+    return 0u;
+#endif
+}
+
+struct Iq2TablesWide {
+    unsigned lane_magnitude;   // (lane % 32) * 8
+    unsigned lane_sign;        // kIq2SignBase + (lane % 32) * 16
+    __device__ __forceinline__ void lookup(unsigned grids, unsigned aux, unsigned j, uint2 &m,
+                                           uint2 &mask, uint2 &one) const
+    {
+        // The tables start at LDS address 0, so these byte offsets are LDS addresses.
+        // magnitude address = (index byte j) << 8 | lane offset: bytes {lane, index, 0, 0}
+        const unsigned ma = __builtin_amdgcn_perm(grids, lane_magnitude, 0x0c0c0400u + (j << 8));
+        // sign address = field j (7 bits at bit 7j) moved to bit 9, or-ed with the lane offset
+        const unsigned moved = 7u * j >= 9u ? aux >> (7u * j - 9u) : aux << (9u - 7u * j);
+        const unsigned sa = (moved & 0xfe00u) | lane_sign;
+        m = lds_read_uint2(ma);
+        const uint4 s = lds_read_uint4(sa);
+        mask = make_uint2(s.x, s.y);
+        one = make_uint2(s.z, s.w);
     }
-    for (unsigned i = threadIdx.x; i < 128u; i += blockDim.x) {
-        unsigned s = i | ((__popc(i) & 1u) << 7), lo = 0u, hi = 0u;
-#pragma unroll
-        for (unsigned l = 0; l < 4u; ++l) {
-            if ((s >> l) & 1u) lo |= 0xffu << (8u * l);
-            if ((s >> (l + 4u)) & 1u) hi |= 0xffu << (8u * l);
-        }
-        t.signmask[i] = make_uint2(lo, hi);
+};
+
+__device__ __forceinline__ Iq2TablesWide iq2_tables_wide_fill(unsigned char *lds)
+{
+    uint2 *mag = reinterpret_cast<uint2 *>(lds);
+    uint4 *sgn = reinterpret_cast<uint4 *>(lds + kIq2SignBase);
+    for (unsigned i = threadIdx.x; i < 256u * kIq2Replicas; i += blockDim.x)
+        mag[i] = iq2_magnitude_entry(i / kIq2Replicas);
+    for (unsigned i = threadIdx.x; i < 128u * kIq2Replicas; i += blockDim.x) {
+        const uint2 m = iq2_signmask_entry(i / kIq2Replicas);
+        sgn[i] = make_uint4(m.x, m.y, m.x & 0x01010101u, m.y & 0x01010101u);
     }
+    const unsigned replica = threadIdx.x & (kIq2Replicas - 1u);
+    return Iq2TablesWide{replica * 8u, kIq2SignBase + replica * 16u};
 }
 
 // 32 weights of one IQ2_XXS group -> eight int8x4 dwords; returns the odd factor 2s+1.
-__device__ __forceinline__ int iq2_unit(const Iq2Tables &t, unsigned grids, unsigned aux,
+// A signed byte is (magnitude ^ mask) + one: magnitudes are >= 8 so the +1 never carries.
+template <typename Tables>
+__device__ __forceinline__ int iq2_unit(const Tables &t, unsigned grids, unsigned aux,
                                         unsigned w[8])
 {
 #pragma unroll
     for (unsigned j = 0; j < 4u; ++j) {
-        uint2 m = t.magnitudes[(grids >> (8u * j)) & 255u];
-        uint2 s = t.signmask[(aux >> (7u * j)) & 127u];
-        w[2 * j] = (m.x ^ s.x) + (s.x & 0x01010101u);
-        w[2 * j + 1] = (m.y ^ s.y) + (s.y & 0x01010101u);
+        uint2 m, mask, one;
+        t.lookup(grids, aux, j, m, mask, one);
+        w[2 * j] = (m.x ^ mask.x) + one.x;
+        w[2 * j + 1] = (m.y ^ mask.y) + one.y;
     }
     return (int)(2u * (aux >> 28) + 1u);
 }

@@ -93,12 +93,14 @@ __global__ __launch_bounds__(256) void route_rows_kernel(
 // which is exactly the stable counting sort of pairs by expert (src/graph/worklist.c:380-393).
 
 constexpr unsigned kWorklistMaxRows = 4096u;
+constexpr int kPass = 2;          // pairs of one bucket handled per sweep over the expert's bytes
 
 __global__ __launch_bounds__(1024) void worklist_kernel(
     const unsigned long long *__restrict__ selected, unsigned pairs, unsigned topk,
     unsigned experts, unsigned long long *__restrict__ order,
     unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
-    unsigned long long *__restrict__ bucket_populations, unsigned long long *__restrict__ counts,
+    unsigned long long *__restrict__ bucket_populations,
+    unsigned long long *__restrict__ sweep_offsets, unsigned long long *__restrict__ counts,
     int *status)
 {
     extern __shared__ unsigned shared_words[];
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
     }
     __syncthreads();
     if (tid == 0u) {
-        unsigned cursor = 0u, bucket = 0u, maximum = 0u;
+        unsigned cursor = 0u, bucket = 0u, maximum = 0u, sweeps = 0u;
         for (unsigned e = 0; e < experts; ++e) {
             const unsigned n = population[e];
             offset[e] = cursor;
@@ -140,6 +142,8 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
                 expert_ids[bucket] = e;
                 bucket_offsets[bucket] = cursor;
                 bucket_populations[bucket] = n;
+                sweep_offsets[bucket] = sweeps;
+                sweeps += (n + (unsigned)kPass - 1u) / (unsigned)kPass;
                 bucket++;
                 maximum = n > maximum ? n : maximum;
             }
@@ -147,15 +151,17 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
         }
         offset[experts] = cursor;
         bucket_offsets[bucket] = cursor;
+        sweep_offsets[bucket] = sweeps;
         for (unsigned b = bucket; b < experts; ++b) {
             expert_ids[b] = 0ull;
             bucket_populations[b] = 0ull;
-            if (b + 1u <= experts) bucket_offsets[b + 1u] = cursor;
+            bucket_offsets[b + 1u] = cursor;
+            sweep_offsets[b + 1u] = sweeps;
         }
         counts[0] = bucket;
         counts[1] = maximum;
         counts[2] = cursor;
-        counts[3] = 0ull;
+        counts[3] = sweeps;
         if (cursor != pairs) bad = 1u;
     }
     __syncthreads();
@@ -181,29 +187,42 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
 }
 
 // ---- grouped expert projections ---------------------------------------------------------------
+//
+// Persistent kernel: one 512-thread workgroup per compute unit builds the conflict-free lookup
+// tables once, then each of its waves walks a strided list of work items. An item is
+// (bucket, tile of weight rows, sweep): a bucket's expert bytes stream from HBM once per sweep
+// and every sweep serves up to kPass pairs of the bucket.
 
-constexpr int kPass = 2;          // pairs of one bucket handled per sweep over the expert's bytes
 constexpr int kUnitsPerLane = 4;  // a lane owns half a superblock: 128 columns
-constexpr int kRowsInFlight = 2;  // weight rows a wave decodes back to back before reducing
+constexpr int kRowsInFlight = 1;  // weight-row groups a wave decodes back to back
+constexpr int kGroupedThreads = 768;
+constexpr int kGroupedWaves = kGroupedThreads / 64;
+constexpr unsigned kItemRowsMax = 16u;   // gate/up row pairs per item when the SwiGLU is fused
 
-struct GroupedArgs {
+// One set of expert matrices plus the pairs that use it.
+struct GroupedProblem {
     const unsigned char *gate, *up;          // up == nullptr: plain projection (down)
     unsigned long long row_bytes, expert_bytes, up_row_bytes, up_expert_bytes;
-    unsigned width;                          // reduction width (activation row length)
-    unsigned out_rows;                       // rows of the weight matrix per expert
     const void *activations;                 // Q8_K rows or F32 rows
     unsigned long long act_stride;           // bytes between activation rows
     int act_by_ordered_pair;                 // 1: activation row = ordered position (down)
-    const unsigned long long *selected, *order, *expert_ids, *bucket_offsets, *bucket_populations;
-    const unsigned long long *counts;
+    const unsigned long long *order, *expert_ids, *bucket_offsets, *bucket_populations;
+    const unsigned long long *sweep_offsets, *counts;
     const float *route_weights;
     unsigned pairs, topk, experts;
-    double limit;
-    float *out;                              // up: intermediate[ordered][out_rows]; down: pair_outputs[source][out_rows]
+    float *out;                              // [ordered or source pair][out_rows]
     int out_by_source_pair;
+    unsigned sweeps;                         // single known bucket: ceil(pairs / kPass), else 0
+};
+
+struct GroupedArgs {
+    GroupedProblem problem[2];               // [0] routed experts, [1] optional shared expert
+    unsigned problems;
+    unsigned width;                          // reduction width (activation row length)
+    unsigned out_rows;                       // rows of the weight matrix per expert
+    unsigned item_rows;                      // weight rows (row pairs when fused) per work item
+    double limit;
     int *status;
-    unsigned rows_per_block;                 // weight rows handled by one workgroup
-    unsigned pass_slots;                     // workgroups that share one (bucket, tile), one sweep each
 };
 
 // SiLU-gated product in double, as src/graph/moe.c:605-611 orders it.
@@ -219,17 +238,17 @@ __device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weigh
 struct LaneGeometry {
     unsigned rows_per_wave, reduce_width, sub, seg, unit0, super;
     bool lane_live;
-    unsigned wave, wave_begin, wave_end;
+    unsigned wave;
 };
 
-// One sweep of a wave over its weight rows with N live pairs of the bucket.
-// Each iteration handles kRowsInFlight row groups; the packed bytes of the next iteration are
-// requested before the current one is decoded, so HBM latency hides behind the decode.
-template <unsigned QT, bool Q8, bool FUSED_UP, int N>
+// One sweep of a wave over the item's weight rows [row_begin, row_end) with N live pairs.
+// Each iteration handles kRows row groups; the packed bytes of the next iteration are requested
+// before the current one is decoded, so HBM latency hides behind the decode.
+template <unsigned QT, bool Q8, bool FUSED_UP, int N, typename Tables>
 __device__ __forceinline__ void grouped_sweep(
-    const GroupedArgs &a, const Iq2Tables &tables, const LaneGeometry &g,
+    const GroupedArgs &a, const GroupedProblem &pr, const Tables &tables, const LaneGeometry &g,
     const unsigned char *gate_e, const unsigned char *up_e, unsigned long long first_ordered,
-    float (&gate_up)[4][2][16][kPass])
+    unsigned row_begin, unsigned row_end, float *park)
 {
     constexpr int kStreams = FUSED_UP ? 2 : 1;
     constexpr int kRows = Q8 ? kRowsInFlight : 1;
@@ -243,11 +262,11 @@ __device__ __forceinline__ void grouped_sweep(
 #pragma unroll
     for (int p = 0; p < N; ++p) {
         const unsigned long long ordered = first_ordered + p;
-        const unsigned long long source = a.order ? a.order[ordered] : ordered;
-        const unsigned long long arow = a.act_by_ordered_pair ? ordered : source / a.topk;
-        act_row[p] = (const unsigned char *)a.activations + arow * a.act_stride;
-        route_weight[p] = a.route_weights ? a.route_weights[source] : 1.0f;
-        out_index[p] = a.out_by_source_pair ? source : ordered;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
+        act_row[p] = (const unsigned char *)pr.activations + arow * pr.act_stride;
+        route_weight[p] = pr.route_weights ? pr.route_weights[source] : 1.0f;
+        out_index[p] = pr.out_by_source_pair ? source : ordered;
         act_scale[p] = 0.0f;
         if constexpr (Q8) {
             const unsigned char *blk = act_row[p] + (unsigned long long)g.super * kQ8KBytes;
@@ -276,21 +295,21 @@ __device__ __forceinline__ void grouped_sweep(
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
             const unsigned want = base + r * g.rows_per_wave + g.sub;
-            const unsigned safe_row = (g.lane_live && want < g.wave_end) ? want : g.wave_begin;
-            next[r][0].load(gate_e + (unsigned long long)safe_row * a.row_bytes, g.unit0);
+            const unsigned safe_row = (g.lane_live && want < row_end) ? want : row_begin;
+            next[r][0].load(gate_e + (unsigned long long)safe_row * pr.row_bytes, g.unit0);
             if constexpr (FUSED_UP)
-                next[r][1].load(up_e + (unsigned long long)safe_row * a.up_row_bytes, g.unit0);
+                next[r][1].load(up_e + (unsigned long long)safe_row * pr.up_row_bytes, g.unit0);
         }
     };
-    if (g.wave_begin < g.wave_end) request(g.wave_begin);
+    request(row_begin);
 
-    for (unsigned base = g.wave_begin; base < g.wave_end; base += stride) {
+    for (unsigned base = row_begin; base < row_end; base += stride) {
         LaneChunk<QT> chunk[kRows][kStreams];
 #pragma unroll
         for (int r = 0; r < kRows; ++r)
 #pragma unroll
             for (int w = 0; w < kStreams; ++w) chunk[r][w] = next[r][w];
-        if (base + stride < g.wave_end) request(base + stride);
+        if (base + stride < row_end) request(base + stride);
 
         float sums[kRows][kStreams][N];
         unsigned row[kRows];
@@ -298,7 +317,7 @@ __device__ __forceinline__ void grouped_sweep(
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
             row[r] = base + r * g.rows_per_wave + g.sub;
-            row_live[r] = g.lane_live && row[r] < g.wave_end;
+            row_live[r] = g.lane_live && row[r] < row_end;
 #pragma unroll
             for (int w = 0; w < kStreams; ++w) {
                 const LaneChunk<QT> &c = chunk[r][w];
@@ -369,13 +388,13 @@ __device__ __forceinline__ void grouped_sweep(
                     sums[r][w][p] = group_sum_f32_dynamic(row_live[r] ? sums[r][w][p] : 0.0f,
                                                           g.reduce_width);
             if constexpr (FUSED_UP) {
-                // park (gate, up); the SwiGLU runs once per wave tile with every lane busy
-                const unsigned local = row[r] - g.wave_begin;
-                if (row_live[r] && g.seg == 0u && local < 16u) {
+                // park (gate, up); the SwiGLU runs once per item with every lane busy
+                const unsigned local = row[r] - row_begin;
+                if (row_live[r] && g.seg == 0u && local < kItemRowsMax) {
 #pragma unroll
                     for (int p = 0; p < N; ++p) {
-                        gate_up[g.wave][0][local][p] = sums[r][0][p];
-                        gate_up[g.wave][1][local][p] = sums[r][1][p];
+                        park[(0u * kItemRowsMax + local) * kPass + p] = sums[r][0][p];
+                        park[(1u * kItemRowsMax + local) * kPass + p] = sums[r][1][p];
                     }
                 }
             } else if (row_live[r] && g.seg == 0u) {
@@ -383,7 +402,7 @@ __device__ __forceinline__ void grouped_sweep(
                 for (int p = 0; p < N; ++p) {
                     const float value = bf16_round(sums[r][0][p]);
                     if (!finite_f32(value)) raise_status(a.status, 1);
-                    else a.out[out_index[p] * a.out_rows + row[r]] = value;
+                    else pr.out[out_index[p] * a.out_rows + row[r]] = value;
                 }
             }
         }
@@ -393,8 +412,8 @@ __device__ __forceinline__ void grouped_sweep(
         const unsigned lane = threadIdx.x & 63u;
         const unsigned local = lane >> 2;
         const int p = (int)(lane & 3u);
-        const unsigned out_row = g.wave_begin + local;
-        if (local < 16u && out_row < g.wave_end && p < N) {
+        const unsigned out_row = row_begin + local;
+        if (local < kItemRowsMax && out_row < row_end && p < N) {
             float rw = route_weight[0];
             unsigned long long oi = out_index[0];
 #pragma unroll
@@ -404,49 +423,42 @@ __device__ __forceinline__ void grouped_sweep(
                     oi = out_index[q];
                 }
             }
-            const float value = swiglu_bf16(gate_up[g.wave][0][local][p], gate_up[g.wave][1][local][p],
-                                            rw, a.limit);
+            const float value = swiglu_bf16(park[(0u * kItemRowsMax + local) * kPass + p],
+                                            park[(1u * kItemRowsMax + local) * kPass + p], rw, a.limit);
             if (!finite_f32(value)) raise_status(a.status, 1);
-            else a.out[oi * a.out_rows + out_row] = value;
+            else pr.out[oi * a.out_rows + out_row] = value;
         }
     }
 }
 
-// One workgroup = one (bucket, tile of weight rows, pass slot). A lane owns half a superblock
-// (four units, 128 columns) of the reduction dimension; units/4 lanes span one weight row and,
-// where that is a power of two below 64, a wave covers several rows at once.
+template <unsigned QT>
+struct GroupedTables {
+    using type = Iq2Tables;   // unused placeholder for qtypes without lookup tables
+};
+template <>
+struct GroupedTables<QT_IQ2_XXS> {
+    using type = Iq2TablesWide;
+};
+
 template <unsigned QT, bool Q8, bool FUSED_UP>
-__global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
+__global__ __launch_bounds__(kGroupedThreads) void grouped_kernel(GroupedArgs a)
 {
-    __shared__ Iq2Tables tables;
-    __shared__ float gate_up[4][2][16][kPass];   // [wave][gate|up][row in wave tile][pair]
-    if constexpr (QT == QT_IQ2_XXS) iq2_tables_fill(tables);
-
-    const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
-    const unsigned slot = blockIdx.x % a.pass_slots;
-    const unsigned work = blockIdx.x / a.pass_slots;
-    const unsigned bucket = work / tiles, tile = work % tiles;
-    unsigned long long expert = 0ull, first = 0ull, population = a.pairs;
-    bool idle = false;
-    if (a.expert_ids) {
-        if (bucket >= (unsigned)a.counts[0]) idle = true;
-        else {
-            expert = a.expert_ids[bucket];
-            first = a.bucket_offsets[bucket];
-            population = a.bucket_populations[bucket];
+    extern __shared__ __align__(16) unsigned char grouped_lds[];
+    typename GroupedTables<QT>::type tables;
+    unsigned char *after_tables = grouped_lds;
+    if constexpr (QT == QT_IQ2_XXS) {
+        // the lookups address LDS directly: the dynamic block must start at LDS address 0
+        if (lds_address_of(grouped_lds) != 0u) {
+            if (threadIdx.x == 0u) raise_status(a.status, 2);
+            return;
         }
-    } else if (bucket > 0u) {
-        idle = true;
+        tables = iq2_tables_wide_fill(grouped_lds);
+        after_tables = grouped_lds + kIq2WideBytes;
+        __syncthreads();
     }
-    if ((unsigned long long)slot * kPass >= population) idle = true;
-    if constexpr (QT == QT_IQ2_XXS) __syncthreads();
-    if (idle) return;
-    if (expert >= a.experts || first + population > a.pairs) {
-        if (threadIdx.x == 0u) raise_status(a.status, 2);
-        return;
-    }
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    float *park = reinterpret_cast<float *>(after_tables) + wave * (2u * kItemRowsMax * kPass);
 
-    const unsigned lane = threadIdx.x & 63u;
     const unsigned units = a.width >> 5;                          // multiple of 8
     const unsigned lanes_per_row = units / kUnitsPerLane;         // even, <= 64
     const bool pow2 = (lanes_per_row & (lanes_per_row - 1u)) == 0u;
@@ -458,24 +470,58 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a)
     g.lane_live = g.sub < g.rows_per_wave;
     g.unit0 = g.seg * kUnitsPerLane;                              // four units, one superblock
     g.super = g.unit0 >> 3;
-    g.wave = threadIdx.x >> 6;
+    g.wave = wave;
 
-    const unsigned char *gate_e = a.gate + expert * a.expert_bytes;
-    const unsigned char *up_e = FUSED_UP ? a.up + expert * a.up_expert_bytes : nullptr;
-    const unsigned row_begin = tile * a.rows_per_block;
-    const unsigned row_end = row_begin + a.rows_per_block < a.out_rows ? row_begin + a.rows_per_block
-                                                                       : a.out_rows;
-    const unsigned wave_rows = (a.rows_per_block + 3u) / 4u;      // rows per wave inside the tile
-    g.wave_begin = row_begin + g.wave * wave_rows;
-    g.wave_end = g.wave_begin + wave_rows < row_end ? g.wave_begin + wave_rows : row_end;
+    const unsigned tiles = (a.out_rows + a.item_rows - 1u) / a.item_rows;
+    const unsigned long long wave_id = (unsigned long long)blockIdx.x * kGroupedWaves + wave;
+    const unsigned long long wave_count = (unsigned long long)gridDim.x * kGroupedWaves;
 
-    for (unsigned long long pass = (unsigned long long)slot * kPass; pass < population;
-         pass += (unsigned long long)a.pass_slots * kPass) {
-        const unsigned long long left = population - pass;
-        if (left >= 2ull)
-            grouped_sweep<QT, Q8, FUSED_UP, 2>(a, tables, g, gate_e, up_e, first + pass, gate_up);
-        else
-            grouped_sweep<QT, Q8, FUSED_UP, 1>(a, tables, g, gate_e, up_e, first + pass, gate_up);
+    // The shared expert's items come first (their number is known at launch), then the routed
+    // buckets the device-built worklist reports.
+    for (int which = (int)a.problems - 1; which >= 0; --which) {
+        const GroupedProblem &pr = a.problem[which];
+        const bool fixed = pr.expert_ids == nullptr;
+        // a work item is one sweep over one tile; sweeps are numbered across all buckets
+        const unsigned long long buckets = fixed ? 1ull : pr.counts[0];
+        const unsigned long long sweeps = fixed ? pr.sweeps : pr.counts[3];
+        const unsigned long long items = sweeps * tiles;
+        // stagger the second list so the waves that ran short on the first start it
+        const unsigned long long shift = which == 0 && a.problems > 1
+            ? ((unsigned long long)tiles * a.problem[1].sweeps) % wave_count : 0ull;
+        unsigned long long item = (wave_id + wave_count - shift) % wave_count;
+        for (; item < items; item += wave_count) {
+            const unsigned long long sweep = item / tiles;
+            const unsigned tile = (unsigned)(item % tiles);
+            unsigned long long expert = 0ull, first = 0ull, population = pr.pairs, pass = sweep * kPass;
+            if (!fixed) {
+                // last bucket whose first sweep is <= sweep
+                unsigned long long low = 0ull, high = buckets;
+                while (low + 1ull < high) {
+                    const unsigned long long middle = (low + high) >> 1;
+                    if (pr.sweep_offsets[middle] <= sweep) low = middle;
+                    else high = middle;
+                }
+                expert = pr.expert_ids[low];
+                first = pr.bucket_offsets[low];
+                population = pr.bucket_populations[low];
+                pass = (sweep - pr.sweep_offsets[low]) * kPass;
+            }
+            if (expert >= pr.experts || first + population > pr.pairs || pass >= population) {
+                if (lane == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            const unsigned char *gate_e = pr.gate + expert * pr.expert_bytes;
+            const unsigned char *up_e = FUSED_UP ? pr.up + expert * pr.up_expert_bytes : nullptr;
+            const unsigned row_begin = tile * a.item_rows;
+            const unsigned row_end = row_begin + a.item_rows < a.out_rows ? row_begin + a.item_rows
+                                                                          : a.out_rows;
+            if (population - pass >= 2ull)
+                grouped_sweep<QT, Q8, FUSED_UP, 2>(a, pr, tables, g, gate_e, up_e, first + pass,
+                                                   row_begin, row_end, park);
+            else
+                grouped_sweep<QT, Q8, FUSED_UP, 1>(a, pr, tables, g, gate_e, up_e, first + pass,
+                                                   row_begin, row_end, park);
+        }
     }
 }
 
@@ -502,31 +548,54 @@ __global__ __launch_bounds__(256) void reduce_combine_kernel(
     }
 }
 
-template <unsigned QT>
-static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, unsigned buckets,
-                          hipStream_t stream)
+static int grouped_grid()
 {
-    const unsigned tiles = (a.out_rows + a.rows_per_block - 1u) / a.rows_per_block;
-    const unsigned long long grid = (unsigned long long)buckets * tiles * a.pass_slots;
-    if (grid > 0x7fffffffull) return ST_BOUNDS;
-    if (fused) {
-        if (q8) grouped_kernel<QT, true, true><<<(unsigned)grid, 256, 0, stream>>>(a);
-        else grouped_kernel<QT, false, true><<<(unsigned)grid, 256, 0, stream>>>(a);
-    } else {
-        if (q8) grouped_kernel<QT, true, false><<<(unsigned)grid, 256, 0, stream>>>(a);
-        else grouped_kernel<QT, false, false><<<(unsigned)grid, 256, 0, stream>>>(a);
+    static int units = 0;
+    if (!units) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
+    return units;
+}
+
+template <unsigned QT, bool Q8, bool FUSED>
+static int launch_grouped_variant(const GroupedArgs &a, hipStream_t stream)
+{
+    const size_t lds = (QT == QT_IQ2_XXS ? kIq2WideBytes : 0u) +
+                       (size_t)kGroupedWaves * 2u * kItemRowsMax * kPass * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void *)grouped_kernel<QT, Q8, FUSED>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            (void)hipGetLastError();
+        configured = true;
+    }
+    grouped_kernel<QT, Q8, FUSED><<<grouped_grid(), kGroupedThreads, lds, stream>>>(a);
     return check_launch("moe_grouped");
 }
 
+template <unsigned QT>
+static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, hipStream_t stream)
+{
+    if (fused) return q8 ? launch_grouped_variant<QT, true, true>(a, stream)
+                         : launch_grouped_variant<QT, false, true>(a, stream);
+    return q8 ? launch_grouped_variant<QT, true, false>(a, stream)
+              : launch_grouped_variant<QT, false, false>(a, stream);
+}
+
 static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool fused,
-                            unsigned buckets, hipStream_t stream)
+                            hipStream_t stream)
 {
     switch (qtype) {
-    case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, buckets, stream);
-    case QT_Q4_K: return launch_grouped<QT_Q4_K>(a, q8, fused, buckets, stream);
-    case QT_Q8_0: return launch_grouped<QT_Q8_0>(a, q8, fused, buckets, stream);
-    case QT_Q2_K: return launch_grouped<QT_Q2_K>(a, q8, fused, buckets, stream);
+    case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);
+    case QT_Q4_K: return launch_grouped<QT_Q4_K>(a, q8, fused, stream);
+    case QT_Q8_0: return launch_grouped<QT_Q8_0>(a, q8, fused, stream);
+    case QT_Q2_K: return launch_grouped<QT_Q2_K>(a, q8, fused, stream);
     default: return ST_UNSUPPORTED;
     }
 }
@@ -538,6 +607,66 @@ static int check_matrix(unsigned qtype, uint64_t width, uint64_t row_bytes)
     if (!width || width % 256u || width / block * bytes != row_bytes) return ST_BOUNDS;
     if (width / 32u > 64u * kUnitsPerLane) return ST_UNSUPPORTED;   // one wave spans a row
     return ST_OK;
+}
+
+struct WorklistView {
+    const uint64_t *order, *expert_ids, *bucket_offsets, *bucket_populations, *sweep_offsets, *counts;
+};
+
+static void fill_up_problem(GroupedProblem &p, const yvex_hip_expert_weights *w,
+                            const void *activations, int act_q8, const float *route_weights,
+                            const WorklistView &wl, uint64_t pairs, uint64_t topk, uint64_t experts,
+                            float *out)
+{
+    p.gate = w->gate;
+    p.up = w->up;
+    p.row_bytes = w->gate_row_bytes;
+    p.expert_bytes = w->gate_expert_bytes;
+    p.up_row_bytes = w->up_row_bytes;
+    p.up_expert_bytes = w->up_expert_bytes;
+    p.activations = activations;
+    p.act_stride = act_q8 ? w->hidden / 256u * kQ8KBytes : w->hidden * sizeof(float);
+    p.act_by_ordered_pair = 0;
+    p.order = (const unsigned long long *)wl.order;
+    p.expert_ids = (const unsigned long long *)wl.expert_ids;
+    p.bucket_offsets = (const unsigned long long *)wl.bucket_offsets;
+    p.bucket_populations = (const unsigned long long *)wl.bucket_populations;
+    p.sweep_offsets = (const unsigned long long *)wl.sweep_offsets;
+    p.counts = (const unsigned long long *)wl.counts;
+    p.route_weights = route_weights;
+    p.pairs = (unsigned)pairs;
+    p.topk = (unsigned)topk;
+    p.experts = (unsigned)experts;
+    p.out = out;
+    p.out_by_source_pair = 0;
+    p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
+}
+
+static void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_weights *w,
+                              const void *intermediate, int act_q8, const WorklistView &wl,
+                              uint64_t pairs, uint64_t experts, float *out)
+{
+    p.gate = w->down;
+    p.up = nullptr;
+    p.row_bytes = w->down_row_bytes;
+    p.expert_bytes = w->down_expert_bytes;
+    p.up_row_bytes = p.up_expert_bytes = 0;
+    p.activations = intermediate;
+    p.act_stride = act_q8 ? w->intermediate / 256u * kQ8KBytes : w->intermediate * sizeof(float);
+    p.act_by_ordered_pair = 1;
+    p.order = (const unsigned long long *)wl.order;
+    p.expert_ids = (const unsigned long long *)wl.expert_ids;
+    p.bucket_offsets = (const unsigned long long *)wl.bucket_offsets;
+    p.bucket_populations = (const unsigned long long *)wl.bucket_populations;
+    p.sweep_offsets = (const unsigned long long *)wl.sweep_offsets;
+    p.counts = (const unsigned long long *)wl.counts;
+    p.route_weights = nullptr;
+    p.pairs = (unsigned)pairs;
+    p.topk = 1u;
+    p.experts = (unsigned)experts;
+    p.out = out;
+    p.out_by_source_pair = 1;
+    p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
 }
 
 }  // namespace yvex
@@ -564,9 +693,11 @@ extern "C" int yvex_hip_moe_route_rows(const float *logits, const float *bias, u
 extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
                                        uint64_t experts, uint64_t *order, uint64_t *expert_ids,
                                        uint64_t *bucket_offsets, uint64_t *bucket_populations,
-                                       uint64_t *counts, int *status, yvex_hip_stream stream)
+                                       uint64_t *sweep_offsets, uint64_t *counts, int *status,
+                                       yvex_hip_stream stream)
 {
-    if (!selected || !order || !expert_ids || !bucket_offsets || !bucket_populations || !counts ||
+    if (!selected || !order || !expert_ids || !bucket_offsets || !bucket_populations ||
+        !sweep_offsets || !counts ||
         !status || !pairs || !topk || !experts || experts > 256u || pairs % topk)
         return ST_INVALID_ARG;
     const uint64_t rows = pairs / topk;
@@ -586,101 +717,97 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
         (const unsigned long long *)selected, (unsigned)pairs, (unsigned)topk, (unsigned)experts,
         (unsigned long long *)order, (unsigned long long *)expert_ids,
         (unsigned long long *)bucket_offsets, (unsigned long long *)bucket_populations,
-        (unsigned long long *)counts, status);
+        (unsigned long long *)sweep_offsets, (unsigned long long *)counts, status);
     return check_launch("worklist_build");
 }
 
+static bool same_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)
+{
+    return a->gate_qtype == b->gate_qtype && a->up_qtype == b->up_qtype &&
+           a->down_qtype == b->down_qtype && a->hidden == b->hidden &&
+           a->intermediate == b->intermediate;
+}
+
 extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *activations,
-                               int act_q8, const uint64_t *selected, const float *route_weights,
-                               const uint64_t *order, const uint64_t *expert_ids,
-                               const uint64_t *bucket_offsets, const uint64_t *bucket_populations,
+                               int act_q8, const float *route_weights, const uint64_t *order,
+                               const uint64_t *expert_ids, const uint64_t *bucket_offsets,
+                               const uint64_t *bucket_populations, const uint64_t *sweep_offsets,
                                const uint64_t *counts, uint64_t pairs, uint64_t topk,
-                               uint64_t experts, double limit, float *intermediate, int *status,
+                               uint64_t experts, double limit,
+                               float *intermediate, const yvex_hip_expert_weights *shared,
+                               uint64_t shared_rows, float *shared_intermediate, int *status,
                                yvex_hip_stream stream)
 {
     if (!w || !w->gate || !w->up || !activations || !intermediate || !status || !pairs || !topk ||
         !experts || !(limit > 0.0) || (act_q8 != 0 && act_q8 != 1) ||
-        (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        (expert_ids && (!bucket_offsets || !bucket_populations || !sweep_offsets || !counts)) ||
+        (shared && (!shared->gate || !shared->up || !shared_rows || !shared_intermediate)))
         return ST_INVALID_ARG;
     if (w->gate_qtype != w->up_qtype) return ST_UNSUPPORTED;
     int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
     if (rc) return rc;
     if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
-    if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull) return ST_BOUNDS;
+    if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull || shared_rows > 0xffffffffull)
+        return ST_BOUNDS;
+    if (shared && (!same_shape(w, shared) || shared->gate_row_bytes != w->gate_row_bytes ||
+                   shared->up_row_bytes != w->up_row_bytes))
+        return ST_UNSUPPORTED;   // launch the shared expert on its own instead
     GroupedArgs a{};
-    a.gate = w->gate;
-    a.up = w->up;
-    a.row_bytes = w->gate_row_bytes;
-    a.expert_bytes = w->gate_expert_bytes;
-    a.up_row_bytes = w->up_row_bytes;
-    a.up_expert_bytes = w->up_expert_bytes;
+    const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts};
+    fill_up_problem(a.problem[0], w, activations, act_q8, route_weights, wl, pairs, topk, experts,
+                    intermediate);
+    a.problems = 1u;
+    if (shared) {
+        const WorklistView none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        fill_up_problem(a.problem[1], shared, activations, act_q8, nullptr, none, shared_rows, 1u,
+                        1u, shared_intermediate);
+        a.problems = 2u;
+    }
     a.width = (unsigned)w->hidden;
     a.out_rows = (unsigned)w->intermediate;
-    a.activations = activations;
-    a.act_stride = act_q8 ? w->hidden / 256u * kQ8KBytes : w->hidden * sizeof(float);
-    a.act_by_ordered_pair = 0;
-    a.selected = (const unsigned long long *)selected;
-    a.order = (const unsigned long long *)order;
-    a.expert_ids = (const unsigned long long *)expert_ids;
-    a.bucket_offsets = (const unsigned long long *)bucket_offsets;
-    a.bucket_populations = (const unsigned long long *)bucket_populations;
-    a.counts = (const unsigned long long *)counts;
-    a.route_weights = route_weights;
-    a.pairs = (unsigned)pairs;
-    a.topk = (unsigned)topk;
-    a.experts = (unsigned)experts;
+    a.item_rows = kItemRowsMax;
     a.limit = limit;
-    a.out = intermediate;
-    a.out_by_source_pair = 0;
     a.status = status;
-    a.rows_per_block = 64u;
-    const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
-    // a single known bucket (shared expert): its sweeps run side by side instead of in a loop
-    a.pass_slots = expert_ids ? 1u : (unsigned)((pairs + kPass - 1u) / kPass);
-    return dispatch_grouped(w->gate_qtype, a, act_q8 != 0, true, buckets, as_stream(stream));
+    return dispatch_grouped(w->gate_qtype, a, act_q8 != 0, true, as_stream(stream));
 }
 
 extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *intermediate,
                                  int act_q8, const uint64_t *order, const uint64_t *expert_ids,
                                  const uint64_t *bucket_offsets,
-                                 const uint64_t *bucket_populations, const uint64_t *counts,
-                                 uint64_t pairs, uint64_t experts, float *pair_outputs,
+                                 const uint64_t *bucket_populations, const uint64_t *sweep_offsets,
+                                 const uint64_t *counts, uint64_t pairs, uint64_t experts,
+                                 float *pair_outputs,
+                                 const yvex_hip_expert_weights *shared, uint64_t shared_rows,
+                                 const void *shared_intermediate, float *shared_outputs,
                                  int *status, yvex_hip_stream stream)
 {
     if (!w || !w->down || !intermediate || !pair_outputs || !status || !pairs || !experts ||
         (act_q8 != 0 && act_q8 != 1) ||
-        (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        (expert_ids && (!bucket_offsets || !bucket_populations || !sweep_offsets || !counts)) ||
+        (shared && (!shared->down || !shared_rows || !shared_intermediate || !shared_outputs)))
         return ST_INVALID_ARG;
     int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
     if (rc) return rc;
-    if (pairs > 0xffffffffull || w->hidden > 0xffffffffull) return ST_BOUNDS;
+    if (pairs > 0xffffffffull || w->hidden > 0xffffffffull || shared_rows > 0xffffffffull)
+        return ST_BOUNDS;
+    if (shared && (!same_shape(w, shared) || shared->down_row_bytes != w->down_row_bytes))
+        return ST_UNSUPPORTED;
     GroupedArgs a{};
-    a.gate = w->down;
-    a.up = nullptr;
-    a.row_bytes = w->down_row_bytes;
-    a.expert_bytes = w->down_expert_bytes;
+    const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts};
+    fill_down_problem(a.problem[0], w, intermediate, act_q8, wl, pairs, experts, pair_outputs);
+    a.problems = 1u;
+    if (shared) {
+        const WorklistView none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        fill_down_problem(a.problem[1], shared, shared_intermediate, act_q8, none, shared_rows, 1u,
+                          shared_outputs);
+        a.problems = 2u;
+    }
     a.width = (unsigned)w->intermediate;
     a.out_rows = (unsigned)w->hidden;
-    a.activations = intermediate;
-    a.act_stride = act_q8 ? w->intermediate / 256u * kQ8KBytes : w->intermediate * sizeof(float);
-    a.act_by_ordered_pair = 1;
-    a.order = (const unsigned long long *)order;
-    a.expert_ids = (const unsigned long long *)expert_ids;
-    a.bucket_offsets = (const unsigned long long *)bucket_offsets;
-    a.bucket_populations = (const unsigned long long *)bucket_populations;
-    a.counts = (const unsigned long long *)counts;
-    a.route_weights = nullptr;
-    a.pairs = (unsigned)pairs;
-    a.topk = 1u;
-    a.experts = (unsigned)experts;
+    a.item_rows = 64u;
     a.limit = 1.0;
-    a.out = pair_outputs;
-    a.out_by_source_pair = 1;
     a.status = status;
-    a.rows_per_block = 256u;
-    const unsigned buckets = expert_ids ? (unsigned)(pairs < experts ? pairs : experts) : 1u;
-    a.pass_slots = expert_ids ? 1u : (unsigned)((pairs + kPass - 1u) / kPass);
-    return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, buckets, as_stream(stream));
+    return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, as_stream(stream));
 }
 
 extern "C" int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows,

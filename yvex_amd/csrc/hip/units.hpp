@@ -116,7 +116,8 @@ struct LaneChunk<QT_IQ2_XXS> {
         q[0] = lo.x; q[1] = lo.y; q[2] = lo.z; q[3] = lo.w;
         q[4] = hi.x; q[5] = hi.y; q[6] = hi.z; q[7] = hi.w;
     }
-    __device__ __forceinline__ void decode(const Iq2Tables &t, int k, unsigned, Unit &unit) const
+    template <typename Tables>
+    __device__ __forceinline__ void decode(const Tables &t, int k, unsigned, Unit &unit) const
     {
         unit.factor = unit.factor2 = iq2_unit(t, q[2 * k], q[2 * k + 1], unit.w);
         unit.min1 = unit.min2 = 0;
@@ -147,7 +148,8 @@ struct LaneChunk<QT_Q4_K> {
     {
         return (head[1u + (i >> 2)] >> (8u * (i & 3u))) & 255u;
     }
-    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned unit0, Unit &unit) const
+    template <typename Tables>
+    __device__ __forceinline__ void decode(const Tables &, int k, unsigned unit0, Unit &unit) const
     {
         const unsigned g = (unit0 & 7u) + (unsigned)k, shift = (g & 1u) * 4u;
 #pragma unroll
@@ -189,7 +191,8 @@ struct LaneChunk<QT_Q2_K> {
         scales[1] = sc.y;
         dd = load_u32(b + 80u);
     }
-    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned, Unit &unit) const
+    template <typename Tables>
+    __device__ __forceinline__ void decode(const Tables &, int k, unsigned, Unit &unit) const
     {
         const unsigned shift = 2u * (unsigned)k;   // unit0 & 3 == 0
 #pragma unroll
@@ -225,7 +228,8 @@ struct LaneChunk<QT_Q8_0> {
             q[8 * k + 4] = hi.x; q[8 * k + 5] = hi.y; q[8 * k + 6] = hi.z; q[8 * k + 7] = hi.w;
         }
     }
-    __device__ __forceinline__ void decode(const Iq2Tables &, int k, unsigned, Unit &unit) const
+    template <typename Tables>
+    __device__ __forceinline__ void decode(const Tables &, int k, unsigned, Unit &unit) const
     {
 #pragma unroll
         for (int i = 0; i < 8; ++i) unit.w[i] = q[8 * k + i];

@@ -128,6 +128,7 @@ class Worklist:
         self.expert_ids = torch.empty(experts, dtype=torch.int64, device=device)
         self.bucket_offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
         self.bucket_populations = torch.empty(experts, dtype=torch.int64, device=device)
+        self.sweep_offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
         self.counts = torch.empty(4, dtype=torch.int64, device=device)
 
 
@@ -137,7 +138,8 @@ def worklist_build(selected, experts, status, worklist: Worklist | None = None) 
     wl = worklist or Worklist(pairs, experts, selected.device)
     _call("yvex_hip_worklist_build", _ptr(selected), C.c_uint64(pairs), C.c_uint64(topk),
           C.c_uint64(experts), _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
-          _ptr(wl.bucket_populations), _ptr(wl.counts), _ptr(status), _stream())
+          _ptr(wl.bucket_populations), _ptr(wl.sweep_offsets), _ptr(wl.counts), _ptr(status),
+          _stream())
     return wl
 
 
@@ -156,22 +158,30 @@ def expert_weights(gate, up, down, qtypes, hidden, intermediate) -> ExpertWeight
     return w
 
 
-def moe_up(w: ExpertWeights, activations, act_q8, selected, route_weights, wl, pairs, topk,
-           experts, limit, intermediate, status):
-    _call("yvex_hip_moe_up", C.byref(w), _ptr(activations), C.c_int(int(act_q8)), _ptr(selected),
-          _ptr(route_weights), _ptr(wl.order if wl else None),
-          _ptr(wl.expert_ids if wl else None), _ptr(wl.bucket_offsets if wl else None),
-          _ptr(wl.bucket_populations if wl else None), _ptr(wl.counts if wl else None),
-          C.c_uint64(pairs), C.c_uint64(topk), C.c_uint64(experts), C.c_double(limit),
-          _ptr(intermediate), _ptr(status), _stream())
+def _wl_ptrs(wl):
+    if wl is None:
+        return [C.c_void_p(0)] * 6
+    return [_ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
+            _ptr(wl.bucket_populations), _ptr(wl.sweep_offsets), _ptr(wl.counts)]
 
 
-def moe_down(w: ExpertWeights, intermediate, act_q8, wl, pairs, experts, pair_outputs, status):
+def moe_up(w: ExpertWeights, activations, act_q8, route_weights, wl, pairs, topk, experts, limit,
+           intermediate, status, shared: ExpertWeights | None = None, shared_rows=0,
+           shared_intermediate=None):
+    _call("yvex_hip_moe_up", C.byref(w), _ptr(activations), C.c_int(int(act_q8)),
+          _ptr(route_weights), *_wl_ptrs(wl), C.c_uint64(pairs), C.c_uint64(topk),
+          C.c_uint64(experts), C.c_double(limit), _ptr(intermediate),
+          C.byref(shared) if shared is not None else C.c_void_p(0), C.c_uint64(shared_rows),
+          _ptr(shared_intermediate), _ptr(status), _stream())
+
+
+def moe_down(w: ExpertWeights, intermediate, act_q8, wl, pairs, experts, pair_outputs, status,
+             shared: ExpertWeights | None = None, shared_rows=0, shared_intermediate=None,
+             shared_outputs=None):
     _call("yvex_hip_moe_down", C.byref(w), _ptr(intermediate), C.c_int(int(act_q8)),
-          _ptr(wl.order if wl else None), _ptr(wl.expert_ids if wl else None),
-          _ptr(wl.bucket_offsets if wl else None), _ptr(wl.bucket_populations if wl else None),
-          _ptr(wl.counts if wl else None), C.c_uint64(pairs), C.c_uint64(experts),
-          _ptr(pair_outputs), _ptr(status), _stream())
+          *_wl_ptrs(wl), C.c_uint64(pairs), C.c_uint64(experts), _ptr(pair_outputs),
+          C.byref(shared) if shared is not None else C.c_void_p(0), C.c_uint64(shared_rows),
+          _ptr(shared_intermediate), _ptr(shared_outputs), _ptr(status), _stream())
 
 
 def moe_reduce_combine(pair_outputs, rows, topk, hidden, shared, routed, combined, status):

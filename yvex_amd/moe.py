@@ -41,6 +41,7 @@ class MoeLayer:
         self.combined = torch.empty((max_rows, hidden), **f32)
         self.selected = None
         self.weights = None
+        self.merge_shared = True
 
     def run(self, rows_f32: torch.Tensor, logits: torch.Tensor):
         """Enqueue one batch; returns the combined rows (device tensor, not synchronised)."""
@@ -56,23 +57,27 @@ class MoeLayer:
         self.selected, self.weights = K.moe_route_rows(
             logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st)
         K.worklist_build(self.selected, self.experts, st, self.worklist)
-        K.moe_up(self.routed, acts, self.act_q8, self.selected, self.weights, self.worklist, pairs,
-                 self.topk, self.experts, self.limit, self.intermediate_f32, st)
+        merged = self.shared is not None and self.merge_shared
+        K.moe_up(self.routed, acts, self.act_q8, self.weights, self.worklist, pairs, self.topk,
+                 self.experts, self.limit, self.intermediate_f32, st,
+                 shared=self.shared if merged else None, shared_rows=rows if merged else 0,
+                 shared_intermediate=self.shared_mid if merged else None)
+        if self.shared is not None and not merged:
+            K.moe_up(self.shared, acts, self.act_q8, None, None, rows, 1, 1, self.limit,
+                     self.shared_mid, st)
         if self.act_q8:
             K.q8k_quantize(self.intermediate_f32[:pairs], st, self.intermediate_q8)
             mid = self.intermediate_q8
-        else:
-            mid = self.intermediate_f32
-        K.moe_down(self.routed, mid, self.act_q8, self.worklist, pairs, self.experts,
-                   self.pair_outputs, st)
-        if self.shared is not None:
-            K.moe_up(self.shared, acts, self.act_q8, None, None, None, rows, 1, 1, self.limit,
-                     self.shared_mid, st)
-            if self.act_q8:
+            if self.shared is not None:
                 K.q8k_quantize(self.shared_mid[:rows], st, self.shared_mid_q8)
-                smid = self.shared_mid_q8
-            else:
-                smid = self.shared_mid
+            smid = self.shared_mid_q8
+        else:
+            mid, smid = self.intermediate_f32, self.shared_mid
+        K.moe_down(self.routed, mid, self.act_q8, self.worklist, pairs, self.experts,
+                   self.pair_outputs, st, shared=self.shared if merged else None,
+                   shared_rows=rows if merged else 0, shared_intermediate=smid if merged else None,
+                   shared_outputs=self.shared_out if merged else None)
+        if self.shared is not None and not merged:
             K.moe_down(self.shared, smid, self.act_q8, None, rows, 1, self.shared_out, st)
         K.moe_reduce_combine(self.pair_outputs, rows, self.topk, self.hidden, self.shared_out,
                              self.routed_out, self.combined, st)
