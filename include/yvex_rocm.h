@@ -1,0 +1,604 @@
+/*
+ * C ABI of the MI355X (gfx950) backend for YVEX's quantized-weight matmul path.
+ *
+ * This header is what a libyvex build binds instead of its CUDA backend for the operations on
+ * this path. Names, argument meaning, status codes and fail-closed behaviour follow the
+ * reference's backend contract; every declaration cites the reference interface it replaces.
+ * Structures that cross the boundary keep the reference's field names and order.
+ *
+ * Conventions (include/yvex/core.h:13-48, src/backend/cuda/qtype.c:246,299,391-392):
+ *   - every entry point returns a yvex_status (0 = OK, negative = refusal);
+ *   - the last parameter is a yvex_error that is cleared on success and may be NULL;
+ *   - output facts are zeroed on entry and published only on success;
+ *   - an output tensor is marked written only by a successful operation;
+ *   - nothing here ever falls back to another backend or to the CPU.
+ */
+#ifndef YVEX_ROCM_H
+#define YVEX_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status and error: include/yvex/core.h:13-48 ------------------------------------------ */
+
+typedef enum {
+    YVEX_OK = 0,
+    YVEX_ERR = -1,
+    YVEX_ERR_NOMEM = -2,
+    YVEX_ERR_IO = -3,
+    YVEX_ERR_FORMAT = -4,
+    YVEX_ERR_UNSUPPORTED = -5,
+    YVEX_ERR_BACKEND = -6,
+    YVEX_ERR_BOUNDS = -7,
+    YVEX_ERR_STATE = -8,
+    YVEX_ERR_CANCELLED = -9,
+    YVEX_ERR_INVALID_ARG = -10,
+    YVEX_ERR_TIMEOUT = -11
+} yvex_status;
+
+#define YVEX_ERROR_WHERE_CAP 96
+#define YVEX_ERROR_MESSAGE_CAP 256
+typedef struct {
+    yvex_status code;
+    char where[YVEX_ERROR_WHERE_CAP];
+    char message[YVEX_ERROR_MESSAGE_CAP];
+} yvex_error;
+
+const char *yvex_status_name(yvex_status status);
+void yvex_error_clear(yvex_error *err);
+void yvex_error_set(yvex_error *err, yvex_status code, const char *where, const char *message);
+int yvex_error_is_set(const yvex_error *err);
+yvex_status yvex_error_code(const yvex_error *err);
+
+/* ---- qtype identity, geometry and fail-closed admission ----------------------------------- */
+/* include/yvex/qtype.h:19-63, src/gguf/qtype.c:15-104, src/gguf/quant_registry.c:50-117 */
+
+enum {
+    YVEX_GGUF_QTYPE_F32 = 0, YVEX_GGUF_QTYPE_F16 = 1, YVEX_GGUF_QTYPE_Q8_0 = 8,
+    YVEX_GGUF_QTYPE_Q2_K = 10, YVEX_GGUF_QTYPE_Q4_K = 12, YVEX_GGUF_QTYPE_Q8_K = 15,
+    YVEX_GGUF_QTYPE_IQ2_XXS = 16, YVEX_GGUF_QTYPE_I32 = 26, YVEX_GGUF_QTYPE_BF16 = 30,
+    YVEX_GGUF_QTYPE_MXFP4 = 39, YVEX_GGUF_QTYPE_ABI_UPSTREAM_MAX_ID = 42
+};
+
+typedef enum {
+    YVEX_GGUF_QTYPE_IDENTITY_ADMITTED = 0,
+    YVEX_GGUF_QTYPE_IDENTITY_REMOVED = 1,
+    YVEX_GGUF_QTYPE_IDENTITY_RESERVED = 2,
+    YVEX_GGUF_QTYPE_IDENTITY_OUTSIDE_BASELINE = 3,
+    YVEX_GGUF_QTYPE_IDENTITY_UNKNOWN = 4
+} yvex_gguf_qtype_identity_status;
+
+typedef struct {
+    unsigned int qtype;
+    const char *name;
+    yvex_gguf_qtype_identity_status identity;
+    unsigned int block_size, bytes_per_block;
+} yvex_gguf_qtype_geometry;
+
+/* Replaces yvex_gguf_qtype_geometry_find (src/gguf/qtype.c:119-124): NULL above ID 42. */
+const yvex_gguf_qtype_geometry *yvex_gguf_qtype_geometry_find(unsigned int qtype);
+
+typedef enum {
+    YVEX_QUANT_REFUSAL_NONE = 0,
+    YVEX_QUANT_REFUSAL_ENCODER_UNAVAILABLE,
+    YVEX_QUANT_REFUSAL_REMOVED_IDENTITY,
+    YVEX_QUANT_REFUSAL_OUTSIDE_PINNED_BASELINE
+} yvex_quant_refusal;
+
+/* One row per qtype ID, index == ID (src/gguf/quant_registry.c:50-103). device_compute is the
+ * reference's dedicated_cuda_compute_available restated for this backend. Relative to the
+ * reference, exactly one row is extended: Q4_K is admitted with device compute; MXFP4 is
+ * admitted for storage but has no kernel in this backend yet (device_compute = 0). */
+typedef struct {
+    unsigned int qtype;
+    int known, storage_admitted, reference_decoder_available;
+    int dedicated_cpu_compute_available, device_compute_available;
+    int extension_of_reference;
+    yvex_quant_refusal refusal;
+} yvex_quant_numeric_capability;
+
+/* Replaces yvex_quant_numeric_capability_at (src/gguf/quant_registry.c:114-118). */
+const yvex_quant_numeric_capability *yvex_quant_numeric_capability_at(unsigned int qtype);
+
+/* ---- backend object: include/yvex/backend.h:13-152 ----------------------------------------- */
+
+typedef struct yvex_backend yvex_backend;
+typedef struct yvex_device_tensor yvex_device_tensor;
+
+typedef enum {
+    YVEX_BACKEND_KIND_CPU = 0,
+    YVEX_BACKEND_KIND_CUDA,
+    YVEX_BACKEND_KIND_METAL,
+    YVEX_BACKEND_KIND_ROCM
+} yvex_backend_kind;
+
+typedef enum {
+    YVEX_BACKEND_STATUS_READY = 0,
+    YVEX_BACKEND_STATUS_CONTEXT_READY,
+    YVEX_BACKEND_STATUS_UNSUPPORTED,
+    YVEX_BACKEND_STATUS_FAILED
+} yvex_backend_status;
+
+typedef struct {
+    yvex_backend_kind kind;
+    const char *device;                 /* NULL or "0".."N": device ordinal */
+    unsigned long long memory_limit_bytes;
+} yvex_backend_options;
+
+typedef struct {
+    unsigned long long allocated_bytes;
+    unsigned long long allocation_count, allocation_events, release_events;
+    unsigned long long h2d_bytes, d2h_bytes;
+    unsigned long long peak_allocated_bytes;
+    unsigned long long memory_limit_bytes;
+} yvex_backend_memory_stats;
+
+/* include/yvex/model.h:18-58, same values. Raw encoded bytes (resident arenas, workspaces)
+ * travel as I8 tensors. */
+typedef enum {
+    YVEX_DTYPE_UNKNOWN = 0,
+    YVEX_DTYPE_F32,
+    YVEX_DTYPE_F16,
+    YVEX_DTYPE_BF16,
+    YVEX_DTYPE_F64,
+    YVEX_DTYPE_I8,
+    YVEX_DTYPE_I16,
+    YVEX_DTYPE_I32,
+    YVEX_DTYPE_I64,
+    YVEX_DTYPE_Q4_0, YVEX_DTYPE_Q4_1, YVEX_DTYPE_Q5_0, YVEX_DTYPE_Q5_1, YVEX_DTYPE_Q8_0,
+    YVEX_DTYPE_Q8_1,
+    YVEX_DTYPE_Q2_K, YVEX_DTYPE_Q3_K, YVEX_DTYPE_Q4_K, YVEX_DTYPE_Q5_K, YVEX_DTYPE_Q6_K,
+    YVEX_DTYPE_Q8_K,
+    YVEX_DTYPE_IQ2_XXS, YVEX_DTYPE_IQ2_XS, YVEX_DTYPE_IQ3_XXS, YVEX_DTYPE_IQ1_S,
+    YVEX_DTYPE_IQ4_NL, YVEX_DTYPE_IQ3_S, YVEX_DTYPE_IQ2_S, YVEX_DTYPE_IQ4_XS, YVEX_DTYPE_IQ1_M,
+    YVEX_DTYPE_TQ1_0, YVEX_DTYPE_TQ2_0, YVEX_DTYPE_MXFP4
+} yvex_dtype;
+
+#define YVEX_TENSOR_MAX_DIMS 4
+typedef struct {
+    const char *name;
+    yvex_dtype dtype;
+    unsigned int rank;
+    unsigned long long dims[YVEX_TENSOR_MAX_DIMS];
+    unsigned long long bytes;
+} yvex_backend_tensor_desc;
+
+/* include/yvex/internal/backend.h:256-269, same fields in the same order. */
+struct yvex_device_tensor {
+    yvex_backend *owner;
+    unsigned long long owner_id;
+    char *name;
+    yvex_dtype dtype;
+    unsigned int rank;
+    unsigned long long dims[YVEX_TENSOR_MAX_DIMS];
+    unsigned long long bytes;
+    unsigned char *data, *host_data;    /* device address; host shadow of a resident tensor */
+    void *backend_allocation;
+    unsigned long long resident_bytes;
+    int virtual_reserved;
+    int is_written, host_accessible, borrowed_host;
+};
+
+typedef enum {
+    YVEX_BACKEND_VARIANT_TENSOR_ALLOC = 0,
+    YVEX_BACKEND_VARIANT_TENSOR_ZERO,
+    YVEX_BACKEND_VARIANT_TENSOR_WRITE,
+    YVEX_BACKEND_VARIANT_TENSOR_READ,
+    YVEX_BACKEND_VARIANT_TENSOR_COPY,
+    YVEX_BACKEND_VARIANT_QTYPE_ROW_DOT = 15,
+    YVEX_BACKEND_VARIANT_ATTENTION_ENCODED = 16,   /* the encoded matvec / MoE family */
+    YVEX_BACKEND_VARIANT_COUNT = 17
+} yvex_backend_operation_variant;
+
+typedef enum {
+    YVEX_BACKEND_CAPABILITY_UNSUPPORTED = 0,
+    YVEX_BACKEND_CAPABILITY_SUPPORTED,
+    YVEX_BACKEND_CAPABILITY_FAILED
+} yvex_backend_capability_state;
+
+typedef enum {
+    YVEX_BACKEND_CAPABILITY_REASON_NONE = 0,
+    YVEX_BACKEND_CAPABILITY_REASON_DRIVER_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_DEVICE_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_CONTEXT_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT,
+    YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_REJECTED,
+    YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING,
+    YVEX_BACKEND_CAPABILITY_REASON_VARIANT_UNSUPPORTED,
+    YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED,
+    YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED,
+    YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED
+} yvex_backend_capability_reason;
+
+typedef struct {
+    yvex_backend_kind backend_kind;
+    yvex_backend_operation_variant variant;
+    yvex_backend_capability_state state;
+    yvex_backend_capability_reason reason;
+    yvex_dtype input_dtype, weight_dtype, output_dtype;
+    int context_available, kernel_bundle_available, function_available;
+} yvex_backend_capability_result;
+
+/* Replaces yvex_backend_open (src/backend/core.c:176-205) for kind ROCM; every other kind
+ * answers UNSUPPORTED. Test seams, read from the environment like the reference's
+ * YVEX_TEST_CUDA_* (src/backend/cuda/capability.c:183, backend.c:275-453):
+ *   YVEX_TEST_ROCM_NO_DEVICE=1       open without a GPU: tensors live in host memory, every
+ *                                    kernel variant is unsupported (kernel-bundle-absent)
+ *   YVEX_TEST_ROCM_BUNDLE_FAILURE=1  a GPU is present but its kernels are treated as absent
+ *   YVEX_TEST_ROCM_LAUNCH_FAILURE=1 / _SYNC_FAILURE=1 / _CLEANUP_FAILURE=1
+ *                                    the next launch / synchronise / release reports failure */
+int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, yvex_error *err);
+/* include/yvex/backend.h:142-152: a cleanup failure keeps *backend non-NULL for a retry. */
+int yvex_backend_close_checked(yvex_backend **backend, yvex_error *err);
+yvex_backend_kind yvex_backend_kind_of(const yvex_backend *backend);
+yvex_backend_status yvex_backend_status_of(const yvex_backend *backend);
+int yvex_backend_get_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
+                                  yvex_error *err);
+int yvex_backend_sync(yvex_backend *backend, yvex_error *err);
+int yvex_backend_query_capability(const yvex_backend *backend,
+                                  yvex_backend_operation_variant variant,
+                                  yvex_backend_capability_result *out, yvex_error *err);
+
+/* include/yvex/backend.h:177-204 */
+int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                              yvex_device_tensor **out, yvex_error *err);
+int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor,
+                                yvex_error *err);
+int yvex_backend_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, const void *src,
+                              unsigned long long len, yvex_error *err);
+int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *tensor, void *dst,
+                             unsigned long long len, yvex_error *err);
+int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
+                             const yvex_device_tensor *src, yvex_error *err);
+int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_tensor *tensor);
+
+/* ---- resident weights: include/yvex/internal/backend.h:270-301, src/backend/residency.c ---- */
+/*
+ * The reference maps one pointer that the CPU writes and the GPU reads (unified memory). On a
+ * discrete-HBM MI355X the same calls are kept with these meanings: resident_alloc gives a device
+ * allocation in HBM plus a pinned host shadow returned through *host; resident_attach is the
+ * publication point that uploads [host_base, host_base + bytes) into HBM; later writes to the
+ * shadow become visible at the next attach or prefetch. resolve maps a borrowed pointer inside
+ * the shadow to device_base + offset exactly as src/backend/residency.c:89-112 does.
+ */
+typedef enum {
+    YVEX_BACKEND_RESIDENT_INVALID = -1,
+    YVEX_BACKEND_RESIDENT_MISS = 0,
+    YVEX_BACKEND_RESIDENT_HIT = 1
+} yvex_backend_resident_result;
+
+int yvex_backend_resident_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                                yvex_device_tensor **out, unsigned char **host, yvex_error *err);
+int yvex_backend_resident_prefetch(yvex_backend *backend, yvex_device_tensor *tensor,
+                                   unsigned long long *prefetched_bytes, yvex_error *err);
+int yvex_backend_resident_attach(yvex_backend *backend, const unsigned char *host_base,
+                                 unsigned long long bytes, const yvex_device_tensor *tensor,
+                                 unsigned long long generation, yvex_error *err);
+int yvex_backend_resident_detach(yvex_backend *backend, yvex_error *err);
+int yvex_backend_resident_resolve(const yvex_backend *backend, const unsigned char *host,
+                                  unsigned long long bytes, unsigned long long *device_address);
+
+/* include/yvex/internal/backend.h:350-354: bump-allocated device scratch, reset per operation. */
+int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *tensor,
+                                  unsigned long long bytes, yvex_error *err);
+void yvex_backend_workspace_detach(yvex_backend *backend);
+int yvex_backend_workspace_acquire(yvex_backend *backend, unsigned long long bytes,
+                                   unsigned long long alignment,
+                                   unsigned long long *device_address);
+
+/* ---- dense projection, output head, gather ------------------------------------------------- */
+
+/* include/yvex/internal/backend.h:325-331 (yvex_backend_cuda_operation_facts). */
+typedef struct yvex_backend_rocm_operation_facts {
+    unsigned long long h2d_bytes, d2h_bytes, d2d_bytes, kernel_launches, upload_count;
+    unsigned long long download_count, stream_synchronizations, device_synchronizations;
+    unsigned long long active_weight_bytes, state_bytes;
+    unsigned long long activation_bytes, temporary_bytes, tensor_core_launches;
+    int compulsory_memory_facts_available;
+} yvex_backend_rocm_operation_facts;
+
+/* Replaces yvex_backend_cuda_encoded_matvec (include/yvex/internal/backend.h:332-337,
+ * src/backend/cuda/qtype.c:220-405). output[in, row] = dot(encoded row, input row in)
+ * (+ additive). activation_q8 = 1 quantizes the F32 input rows to Q8_K on device first.
+ * Refusals: activation_q8 not 0/1 -> INVALID_ARG; qtype unknown, removed, outside the baseline
+ * or without device compute -> UNSUPPORTED (on the host, before any launch); geometry, byte
+ * count, ownership, unwritten input, additive aliasing output, resident MISS -> FORMAT; kernels
+ * absent -> UNSUPPORTED; non-finite numerics seen on device -> FORMAT. input_tail /
+ * input_head_width (the reference's split input for speculation) must be NULL / 0 here. */
+int yvex_backend_rocm_encoded_matvec(
+    yvex_backend *backend, const unsigned char *resident_encoded,
+    unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
+    unsigned long long row_width, unsigned long long row_bytes, unsigned long long input_rows,
+    const yvex_device_tensor *input, const yvex_device_tensor *input_tail,
+    unsigned long long input_head_width, const yvex_device_tensor *additive,
+    yvex_device_tensor *output, int activation_q8, yvex_backend_rocm_operation_facts *facts,
+    yvex_error *err);
+
+/* Replaces yvex_backend_cuda_encoded_gather (include/yvex/internal/backend.h:338-342,
+ * src/backend/cuda/qtype.c:411-521): decode selected rows to F32. row_ids is a host array. */
+int yvex_backend_rocm_encoded_gather(
+    yvex_backend *backend, const unsigned char *resident_encoded,
+    unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
+    unsigned long long row_width, unsigned long long row_bytes, const unsigned int *row_ids,
+    unsigned long long selected_rows, yvex_device_tensor *output,
+    yvex_backend_rocm_operation_facts *facts, yvex_error *err);
+
+/* ---- MoE row batch: include/yvex/internal/moe.h ------------------------------------------- */
+
+#define YVEX_SHA256_HEX_CAP 65u
+#define YVEX_MOE_MAX_SELECTED 16u
+#define YVEX_MOE_ROW_BATCH_SCHEMA_V1 1u
+#define YVEX_MOE_ROW_BATCH_RESULT_SCHEMA_V4 4u
+#define YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP 17u
+/* Kernel families this backend admits in a weight view (moe.h:20-23 list the CUDA ones). */
+#define YVEX_MOE_KERNEL_PORTABLE_ENCODED_ROW "portable-encoded-row"
+#define YVEX_MOE_KERNEL_PORTABLE_EXPERT_ROW "portable-expert-row"
+#define YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP "gfx950-int8-dot-expert-sweep"
+
+typedef enum {
+    YVEX_MOE_ROUTER_HASH_TOKEN_ID = 0,
+    YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE
+} yvex_moe_router_class;
+/* moe.h:35 has SQRT_SOFTPLUS only; SIGMOID is this build's addition for the benchmark layer. */
+typedef enum {
+    YVEX_MOE_SCORING_SQRT_SOFTPLUS = 0,
+    YVEX_MOE_SCORING_SIGMOID = 1
+} yvex_moe_scoring_policy;
+typedef enum { YVEX_MOE_TOPK_NOAUX_TC = 0 } yvex_moe_topk_policy;
+typedef enum { YVEX_MOE_ACTIVATION_SILU = 0 } yvex_moe_activation;
+
+typedef enum {
+    YVEX_MOE_WEIGHT_FFN_NORM = 0,
+    YVEX_MOE_WEIGHT_MHC_FUNCTION,
+    YVEX_MOE_WEIGHT_MHC_BASE,
+    YVEX_MOE_WEIGHT_MHC_SCALE,
+    YVEX_MOE_WEIGHT_ROUTER,
+    YVEX_MOE_WEIGHT_ROUTER_TABLE,
+    YVEX_MOE_WEIGHT_ROUTER_BIAS,
+    YVEX_MOE_WEIGHT_ROUTED_GATE,
+    YVEX_MOE_WEIGHT_ROUTED_UP,
+    YVEX_MOE_WEIGHT_ROUTED_DOWN,
+    YVEX_MOE_WEIGHT_SHARED_GATE,
+    YVEX_MOE_WEIGHT_SHARED_UP,
+    YVEX_MOE_WEIGHT_SHARED_DOWN,
+    YVEX_MOE_WEIGHT_COUNT
+} yvex_moe_weight_slot;
+
+typedef enum {
+    YVEX_EXECUTION_LAYOUT_CANONICAL_ROW = 0,
+    YVEX_EXECUTION_LAYOUT_CONTIGUOUS_DENSE,
+    YVEX_EXECUTION_LAYOUT_EXPERT_MAJOR,
+    YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND
+} yvex_execution_layout_class;
+
+typedef enum {
+    YVEX_EXECUTION_ACTIVATION_HOST_F32 = 0,
+    YVEX_EXECUTION_ACTIVATION_DEVICE_F32,
+    YVEX_EXECUTION_ACTIVATION_DEVICE_F16,
+    YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED
+} yvex_execution_activation_class;
+
+typedef enum {
+    YVEX_EXECUTION_CLASS_PORTABLE_REFERENCE = 0,
+    YVEX_EXECUTION_CLASS_DEVICE_NATIVE,
+    YVEX_EXECUTION_CLASS_FORENSIC_REFERENCE
+} yvex_execution_class;
+
+typedef enum {
+    YVEX_EXECUTION_BATCH_SINGLE_ROW = 0,
+    YVEX_EXECUTION_BATCH_SPECULATIVE_VERIFICATION,
+    YVEX_EXECUTION_BATCH_MULTI_SESSION,
+    YVEX_EXECUTION_BATCH_PREFILL,
+    YVEX_EXECUTION_BATCH_COMPILED_COMPATIBLE
+} yvex_execution_batch_provenance;
+
+/* moe.h:54-64 */
+typedef struct {
+    unsigned long long tensor_id, expert_index;
+    int role;
+    unsigned int qtype;
+    yvex_execution_layout_class layout;
+    yvex_execution_activation_class activation;
+    const char *kernel_family;
+    const unsigned char *encoded;        /* host pointer inside the attached resident arena */
+    size_t encoded_bytes, storage_bytes;
+    unsigned long long row_bytes, row_width, row_count, device_address;
+} yvex_moe_weight_view;
+
+/* moe.h:65-84 */
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long ordinal, layer_index, predictor_index;
+    int tensor_scope;
+    yvex_moe_router_class router_class;
+    yvex_moe_scoring_policy scoring;
+    yvex_moe_topk_policy topk_policy;
+    yvex_moe_activation activation;
+    unsigned long long hidden_width, residual_streams, expanded_width;
+    unsigned long long mhc_mixing_rows, mhc_sinkhorn_iterations;
+    unsigned long long routed_experts, shared_experts, experts_per_token;
+    unsigned long long expert_intermediate_width, shared_intermediate_width;
+    unsigned long long hash_table_rows, hash_table_columns, correction_bias_width;
+    double rms_epsilon, mhc_epsilon, mhc_post_multiplier;
+    double routed_scaling_factor, activation_limit;
+    int requires_token_ids, requires_correction_bias, normalize_topk_probabilities;
+    unsigned long long tensor_ids[YVEX_MOE_WEIGHT_COUNT];
+    unsigned int qtypes[YVEX_MOE_WEIGHT_COUNT];
+    char layer_identity[YVEX_SHA256_HEX_CAP];
+} yvex_moe_layer_plan;
+
+/* execution_batch.h:86-93 */
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long supported_width_mask;   /* bit n set: a batch of n rows is admitted */
+    unsigned long long tensor_core_minimum;
+    char narrow_kernel_family[64];
+    char tensor_core_kernel_family[64];
+    char identity[YVEX_SHA256_HEX_CAP];
+} yvex_expert_worklist_policy;
+
+/* execution_batch.h:128-137 */
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long worklist_count, pair_count, bucket_count;
+    unsigned long long maximum_bucket_population;
+    unsigned long long tensor_core_eligible_pairs, tensor_core_executed_pairs;
+    unsigned long long narrow_pairs, tail_rows;
+    unsigned long long width_histogram[YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP];
+    unsigned long long population_histogram[YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP];
+    unsigned long long provenance_counts[YVEX_EXECUTION_BATCH_COMPILED_COMPATIBLE + 1u];
+} yvex_expert_worklist_observation;
+
+/* execution.h:329-333 */
+typedef struct {
+    unsigned long long active_weight_bytes, state_bytes, activation_bytes, temporary_bytes;
+    unsigned long long measured_operations, missing_operations;
+    int complete;
+} yvex_execution_memory_facts;
+
+typedef struct {
+    int defer;
+    void *host;
+} yvex_moe_device_completion;
+
+/* moe.h:182-197. The plan-side identities the reference seals with SHA-256 (execution_batch,
+ * compiled profile) belong to its runtime, not to this path: execution_batch stays an opaque
+ * pointer whose presence must match worklist_policy's, as moe.c:1845 requires. */
+typedef struct {
+    const yvex_moe_layer_plan *layer;
+    yvex_moe_weight_view weights[YVEX_MOE_WEIGHT_COUNT];
+    const float *expanded_input;
+    const yvex_device_tensor *device_input;
+    yvex_device_tensor *device_output;
+    unsigned int token_id;
+    int token_id_present;
+    int (*cancel_requested)(void *context);
+    void *cancel_context;
+    int evidence_level;
+    int eager_execution;
+    const yvex_moe_device_completion *device_completion;
+    const void *execution_batch;
+    const yvex_expert_worklist_policy *worklist_policy;
+} yvex_moe_layer_job;
+
+/* moe.h:221-236 */
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long row_count, row_width, row_stride;
+    const float *expanded_rows;
+    const yvex_device_tensor *device_rows;
+    yvex_device_tensor *device_outputs;
+    const unsigned int *token_ids;
+    int token_ids_present;
+    yvex_execution_batch_provenance provenance;
+    unsigned int phase;
+    yvex_execution_class execution_class;
+    const char *execution_profile_identity;
+    const void *execution_sources;
+    const void *execution_rows;
+    unsigned long long execution_source_count;
+    int complete_after_operation;
+} yvex_moe_row_batch;
+
+/* moe.h:238-246: optional host copies; NULL pointers are skipped. */
+typedef struct {
+    float *combined_rows, *routed_rows, *shared_rows, *post_rows, *combination_rows;
+    unsigned long long combined_capacity, routed_capacity, shared_capacity;
+    unsigned long long post_capacity, combination_capacity;
+    unsigned long long *selected_experts;
+    float *selected_weights;
+    unsigned long long selection_capacity;
+} yvex_moe_row_batch_output;
+
+/* moe.h:248-271 */
+typedef struct {
+    unsigned int schema_version;
+    int completed, execution_profile_available, device_completion_pending;
+    yvex_execution_class execution_class;
+    unsigned long long row_count, row_expert_pairs, unique_experts;
+    yvex_expert_worklist_observation worklists;
+    unsigned long long grouped_expert_operations, shared_expert_operations;
+    unsigned long long expert_subviews_accessed, encoded_bytes_read;
+    unsigned long long h2d_bytes, d2h_bytes, d2d_bytes, kernel_launches;
+    unsigned long long tensor_core_launches;
+    unsigned long long graph_launches, graph_captures, graph_replays;
+    unsigned long long upload_count, download_count, cache_hits, cache_misses;
+    unsigned long long stream_synchronizations, device_synchronizations;
+    unsigned long long active_weight_base_bytes;
+    unsigned long long active_weight_per_unique_expert_bytes;
+    yvex_execution_memory_facts memory;
+    unsigned long long total_ns, synchronization_ns;
+    char execution_profile_identity[YVEX_SHA256_HEX_CAP];
+    char execution_batch_identity[YVEX_SHA256_HEX_CAP];
+    char worklist_policy_identity[YVEX_SHA256_HEX_CAP];
+    char expert_worklist_identity[YVEX_SHA256_HEX_CAP];
+    char routing_digest[YVEX_SHA256_HEX_CAP];
+    char execution_identity[YVEX_SHA256_HEX_CAP];
+} yvex_moe_row_batch_result;
+
+/* moe.h:277-297. derived_layout_plan/build take the reference's physical-execution decision;
+ * this backend streams canonical GGUF rows directly and needs no derived layout, so both
+ * answer UNSUPPORTED and callers keep layout CANONICAL_ROW / EXPERT_MAJOR. */
+typedef struct {
+    int (*derived_layout_plan)(const void *decision, unsigned long long *storage_bytes,
+                               yvex_error *err);
+    int (*derived_layout_build)(const void *decision, const unsigned char *canonical,
+                                unsigned long long canonical_bytes, unsigned char *derived,
+                                unsigned long long storage_bytes, yvex_error *err);
+    int (*workspace_required)(const yvex_moe_layer_plan *layer, unsigned long long row_count,
+                              unsigned long long *bytes, yvex_error *err);
+    /*
+     * One MoE layer over an ordered row batch (replaces moe_cuda_execute_rows,
+     * src/backend/cuda/moe.c:1826-1923): router projection, scoring and top-k, expert-major
+     * worklist, routed experts (gate/up -> clamped SwiGLU -> bf16 -> down -> bf16, summed in rank
+     * order), shared expert, combined = bf16(routed + shared) into batch->device_outputs.
+     * batch->device_rows holds the already normalised hidden rows [row_count, hidden_width]:
+     * the residual-mixing envelope around the experts is not part of this build, so a plan with
+     * expanded_width != hidden_width or mhc_mixing_rows != 0 is refused UNSUPPORTED, as is the
+     * hash-token router. Mandatory refusals kept from the reference: row count outside
+     * worklist_policy->supported_width_mask -> UNSUPPORTED before anything is touched
+     * (moe.c:1840-1862); gate/up activation or kernel family disagreement -> FORMAT
+     * (moe.c:923-928); unknown kernel family -> UNSUPPORTED (moe.c:961-969); workspace missing or
+     * too small -> NOMEM; cancellation -> CANCELLED; non-finite numerics -> FORMAT.
+     */
+    int (*execute_rows)(yvex_backend *backend, const yvex_moe_layer_job *job,
+                        const yvex_moe_row_batch *batch, const yvex_moe_row_batch_output *output,
+                        yvex_moe_row_batch_result *result, yvex_error *err);
+    int (*complete_rows)(yvex_backend *backend, int barrier_observed,
+                         yvex_moe_row_batch_result *result, yvex_error *err);
+} yvex_backend_moe_operations;
+
+/* moe.h:295-296: NULL unless the backend is ROCM and its kernels are loadable. */
+const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend);
+
+/* Largest row batch execute_rows accepts in one call. */
+#define YVEX_ROCM_MOE_MAX_ROWS 4096ull
+
+/* ---- expert worklist on the host: include/yvex/internal/execution_batch.h:95-169 ----------- */
+
+typedef struct {
+    unsigned long long *expert_ids, *bucket_offsets, *bucket_populations;
+    unsigned long long *source_pairs, *source_rows, *destination_rows;
+    float *route_weights;
+    unsigned long long bucket_capacity, pair_capacity;
+} yvex_expert_worklist_storage;
+
+/* Replaces the sorting core of yvex_expert_worklist_build (src/graph/worklist.c:369-441):
+ * stable counting sort of pairs by expert. bucket_offsets needs bucket_capacity + 1 entries.
+ * An expert ordinal >= expert_count or a non-finite weight -> FORMAT; storage too small or
+ * pair_count not a multiple of experts_per_row -> INVALID_ARG. */
+int yvex_expert_worklist_build(const unsigned long long *selected_experts,
+                               const float *route_weights, unsigned long long pair_count,
+                               unsigned long long experts_per_row,
+                               unsigned long long expert_count,
+                               const yvex_expert_worklist_storage *storage,
+                               yvex_expert_worklist_observation *observation, yvex_error *err);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,342 @@
+"""The drop-in boundary on a real MI355X: every call goes through include/yvex_rocm.h.
+
+Scenarios follow tests/unit/cuda/quant_qtype.c:273-517 (encoded matvec: F32 and Q8 activation
+paths, additive fusion, refusals, memory facts) and tests/unit/cuda/info.c:316-822 (width-N MoE:
+selection equal to the CPU router, weights <= 1e-6, refusal before mutation for an unsupported
+width, FORMAT for mixed gate/up activations).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from yvex_amd import abi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def backend(gpu):
+    from backend_helpers import Backend
+    b = Backend()
+    assert b.ok, b.err.message
+    assert b.lib.yvex_backend_status_of(b.handle) == abi.STATUS_READY
+    yield b
+    assert b.close() == 0
+
+
+def close_to(got, want, rel=1e-3, abs_=1e-5):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return np.all(np.abs(got - want) <= abs_ + rel * np.abs(want))
+
+
+def run_matvec(b, host, w, qt, rows, width, x_tensor, out, in_rows, q8, additive=None):
+    facts, err = abi.OperationFacts(), abi.Error()
+    rc = b.lib.yvex_backend_rocm_encoded_matvec(
+        b.handle, host, w.nbytes, qt, rows, width, w.nbytes // rows, in_rows, x_tensor, None, 0,
+        additive, out, q8, C.byref(facts), C.byref(err))
+    return rc, facts, err
+
+
+@pytest.mark.parametrize("qtype,rows,width,in_rows", [
+    ("Q8_0", 64, 4096, 1), ("IQ2_XXS", 96, 2048, 1), ("IQ2_XXS", 24, 7168, 3),
+    ("Q4_K", 40, 7168, 1), ("Q4_K", 16, 2048, 16), ("Q2_K", 20, 512, 2)])
+def test_encoded_matvec_both_activation_paths(backend, oracle, qtype, rows, width, in_rows):
+    b = backend
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"backend.matvec.{qtype}.{rows}.{width}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(in_rows * width).reshape(in_rows, width)
+    _, host = b.resident(w)
+    b.workspace(1 << 20)
+    xt, out = b.f32(x), b.empty_f32(in_rows * rows)
+    rc, facts, err = run_matvec(b, host, w, qt, rows, width, xt, out, in_rows, 0)
+    assert rc == 0, err.message
+    assert out.contents.is_written == 1
+    got = b.read_f32(out, in_rows * rows).reshape(in_rows, rows)
+    assert close_to(got, oracle.matvec(qt, w, rows, width, x))
+    assert facts.active_weight_bytes == w.nbytes and facts.compulsory_memory_facts_available == 1
+    assert facts.activation_bytes == x.nbytes + got.nbytes and facts.d2h_bytes == 4
+    # Q8_K activations: exact against the integer oracle path, and within the reference's own
+    # bound of the CPU path fed with the dequantised activations
+    rc, facts, err = run_matvec(b, host, w, qt, rows, width, xt, out, in_rows, 1)
+    assert rc == 0, err.message
+    got8 = b.read_f32(out, in_rows * rows).reshape(in_rows, rows)
+    act = oracle.q8k_quantize(x)
+    assert close_to(got8, oracle.q8_matvec(qt, w, rows, width, act, in_rows), rel=1e-5, abs_=1e-5)
+    deq = oracle.q8k_dequantize(act).reshape(in_rows, width)
+    want = oracle.matvec(qt, w, rows, width, deq)
+    assert np.all(np.abs(got8 - want) <= 1e-5 * (1 + np.abs(want)) * 10)
+    assert facts.temporary_bytes == 4 + in_rows * (width // 256) * 292
+
+
+def test_encoded_matvec_additive_and_refusals_on_device(backend, oracle):
+    b = backend
+    rows, width = 32, 2048
+    g = oracle.Generator(3, "backend.additive")
+    w = g.weights(oracle.IQ2_XXS, rows, width)
+    x, add = g.normal(width), g.normal(rows)
+    _, host = b.resident(w)
+    xt, at, out = b.f32(x), b.f32(add), b.empty_f32(rows)
+    rc, _, err = run_matvec(b, host, w, 16, rows, width, xt, out, 1, 0, additive=at)
+    assert rc == 0, err.message
+    want = oracle.matvec(16, w, rows, width, x)[0] + add
+    assert close_to(b.read_f32(out, rows), want)
+    # Q8 path without a workspace is refused, the output stays unpublished
+    rc, _, err = run_matvec(b, host, w, 16, rows, width, xt, out, 1, 1)
+    assert rc == abi.NOMEM and out.contents.is_written == 0
+    # aliasing and unwritten inputs
+    assert run_matvec(b, host, w, 16, rows, width, xt, out, 1, 0, additive=out)[0] == abi.FORMAT
+    assert run_matvec(b, host, w, 16, rows, width, b.empty_f32(width), out, 1, 0)[0] == abi.FORMAT
+    # non-finite activations surface as FORMAT through the device status word
+    bad = x.copy()
+    bad[5] = np.inf
+    rc, _, err = run_matvec(b, host, w, 16, rows, width, b.f32(bad), out, 1, 0)
+    assert rc == abi.FORMAT and b"invalid numerics" in err.message and out.contents.is_written == 0
+    # and the backend keeps working afterwards
+    assert run_matvec(b, host, w, 16, rows, width, xt, out, 1, 0)[0] == 0
+
+
+def test_launch_and_sync_failure_seams(backend, oracle, monkeypatch):
+    b = backend
+    rows, width = 8, 256
+    w = oracle.Generator(4, "backend.seams").weights(oracle.Q8_0, rows, width)
+    _, host = b.resident(w)
+    xt, out = b.f32(np.ones(width, np.float32)), b.empty_f32(rows)
+    monkeypatch.setenv("YVEX_TEST_ROCM_LAUNCH_FAILURE", "1")
+    rc, _, err = run_matvec(b, host, w, 8, rows, width, xt, out, 1, 0)
+    assert rc == abi.BACKEND and out.contents.is_written == 0
+    monkeypatch.delenv("YVEX_TEST_ROCM_LAUNCH_FAILURE")
+    monkeypatch.setenv("YVEX_TEST_ROCM_SYNC_FAILURE", "1")
+    rc, _, err = run_matvec(b, host, w, 8, rows, width, xt, out, 1, 0)
+    assert rc == abi.BACKEND and out.contents.is_written == 0
+    monkeypatch.delenv("YVEX_TEST_ROCM_SYNC_FAILURE")
+    assert run_matvec(b, host, w, 8, rows, width, xt, out, 1, 0)[0] == 0
+
+
+def test_bundle_failure_seam_is_fail_closed(gpu, monkeypatch):
+    monkeypatch.setenv("YVEX_TEST_ROCM_BUNDLE_FAILURE", "1")
+    from backend_helpers import Backend
+    b = Backend()
+    assert b.ok and b.lib.yvex_backend_status_of(b.handle) == abi.STATUS_CONTEXT_READY
+    t = b.f32(np.arange(4, dtype=np.float32))
+    assert np.array_equal(b.read_f32(t, 4), np.arange(4, dtype=np.float32))
+    cap = abi.CapabilityResult()
+    b.lib.yvex_backend_query_capability(b.handle, abi.VARIANT_ATTENTION_ENCODED, C.byref(cap), None)
+    assert cap.state == abi.CAP_UNSUPPORTED and cap.reason == abi.REASON_KERNEL_BUNDLE_ABSENT
+    assert not b.lib.yvex_backend_moe_operations_get(b.handle)
+    assert b.close() == 0
+
+
+def test_encoded_gather(backend, oracle):
+    b = backend
+    rows, width = 40, 512
+    w = oracle.Generator(6, "backend.gather").weights(oracle.IQ2_XXS, rows, width)
+    _, host = b.resident(w)
+    b.workspace(4096)
+    ids = np.array([39, 0, 7, 7], np.uint32)
+    out = b.empty_f32(ids.size * width)
+    facts, err = abi.OperationFacts(), abi.Error()
+    rc = b.lib.yvex_backend_rocm_encoded_gather(b.handle, host, w.nbytes, 16, rows, width, 132,
+                                                ids.ctypes.data, ids.size, out, C.byref(facts),
+                                                C.byref(err))
+    assert rc == 0, err.message
+    got = b.read_f32(out, ids.size * width).reshape(ids.size, width)
+    want = oracle.decode_rows(16, w, width, ids)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert facts.active_weight_bytes == ids.size * 132
+
+
+class MoeCase:
+    """One synthetic layer resident on the backend plus everything execute_rows needs."""
+
+    def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
+                 rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
+                 shared=True, family=abi.FAMILY_GFX950, seed=42):
+        self.b, self.oracle = b, oracle
+        qt = getattr(oracle, qtype)
+        self.qt, self.rows, self.hidden, self.experts, self.topk = qt, rows, hidden, experts, topk
+        self.intermediate, self.scoring = intermediate, scoring
+        g = oracle.Generator(seed, f"backend.moe.{qtype}.{hidden}.{experts}")
+        parts = {
+            "router": g.normal(experts * hidden, 0.05).view(np.uint8),
+            "bias": (g.normal(experts) * 0.05).astype(np.float32).view(np.uint8),
+            "gate": g.weights(qt, experts * intermediate, hidden),
+            "up": g.weights(qt, experts * intermediate, hidden),
+            "down": g.weights(qt, experts * hidden, intermediate),
+            "sgate": g.weights(qt, intermediate, hidden),
+            "sup": g.weights(qt, intermediate, hidden),
+            "sdown": g.weights(qt, hidden, intermediate),
+        }
+        self.parts = parts
+        offsets, cursor = {}, 0
+        for name, blob in parts.items():
+            offsets[name] = cursor
+            cursor += (blob.nbytes + 255) // 256 * 256
+        arena = np.zeros(cursor, np.uint8)
+        for name, blob in parts.items():
+            arena[offsets[name]:offsets[name] + blob.nbytes] = blob
+        _, host = b.resident(arena)
+        self.x = g.normal(rows * hidden).reshape(rows, hidden)
+        self.plan = abi.LayerPlan()
+        p = self.plan
+        p.schema_version, p.router_class, p.scoring = 1, abi.ROUTER_LEARNED, scoring
+        p.hidden_width = p.expanded_width = hidden
+        p.residual_streams = 1
+        p.routed_experts, p.shared_experts, p.experts_per_token = experts, int(shared), topk
+        p.expert_intermediate_width = p.shared_intermediate_width = intermediate
+        p.routed_scaling_factor, p.activation_limit = 1.5, 10.0
+        p.requires_correction_bias, p.normalize_topk_probabilities = int(bias), 1
+        self.job = abi.LayerJob()
+        self.job.layer = C.pointer(self.plan)
+        rb_h, rb_i = oracle.row_bytes(qt, hidden), oracle.row_bytes(qt, intermediate)
+
+        def view(slot, name, q, width, count, row_bytes, activation=act):
+            v = self.job.weights[slot]
+            v.qtype, v.layout, v.activation, v.kernel_family = q, abi.LAYOUT_EXPERT_MAJOR, activation, family
+            v.encoded, v.encoded_bytes = host + offsets[name], parts[name].nbytes
+            v.storage_bytes = parts[name].nbytes
+            v.row_bytes, v.row_width, v.row_count = row_bytes, width, count
+
+        view(abi.W_ROUTER, "router", 0, hidden, experts, hidden * 4, abi.ACT_DEVICE_F32)
+        view(abi.W_ROUTER_BIAS, "bias", 0, experts, 1, experts * 4, abi.ACT_DEVICE_F32)
+        view(abi.W_ROUTED_GATE, "gate", qt, hidden, experts * intermediate, rb_h)
+        view(abi.W_ROUTED_UP, "up", qt, hidden, experts * intermediate, rb_h)
+        view(abi.W_ROUTED_DOWN, "down", qt, intermediate, experts * hidden, rb_i)
+        view(abi.W_SHARED_GATE, "sgate", qt, hidden, intermediate, rb_h)
+        view(abi.W_SHARED_UP, "sup", qt, hidden, intermediate, rb_h)
+        view(abi.W_SHARED_DOWN, "sdown", qt, intermediate, hidden, rb_i)
+        self.ops = b.lib.yvex_backend_moe_operations_get(b.handle).contents
+        need, err = abi.ULL(), abi.Error()
+        assert self.ops.workspace_required(C.byref(self.plan), rows, C.byref(need), C.byref(err)) == 0
+        self.workspace_bytes = need.value
+        self.rows_in, self.rows_out = b.f32(self.x), b.empty_f32(rows * hidden)
+        self.batch = abi.RowBatch()
+        bt = self.batch
+        bt.schema_version, bt.row_count, bt.row_width, bt.row_stride = 1, rows, hidden, hidden
+        bt.device_rows, bt.device_outputs = self.rows_in, self.rows_out
+        bt.provenance, bt.execution_class = abi.BATCH_MULTI_SESSION, 1
+        self.sel = np.zeros(rows * topk, np.uint64)
+        self.wts = np.zeros(rows * topk, np.float32)
+        self.combined = np.zeros((rows, hidden), np.float32)
+        self.out = abi.RowBatchOutput()
+        self.out.combined_rows, self.out.combined_capacity = self.combined.ctypes.data, rows * hidden
+        self.out.selected_experts, self.out.selected_weights = self.sel.ctypes.data, self.wts.ctypes.data
+        self.out.selection_capacity = rows * topk
+        self.result, self.err = abi.RowBatchResult(), abi.Error()
+
+    def execute(self):
+        return self.ops.execute_rows(self.b.handle, C.byref(self.job), C.byref(self.batch),
+                                     C.byref(self.out), C.byref(self.result), C.byref(self.err))
+
+    def oracle_layer(self, act_q8):
+        o, p = self.oracle, self.parts
+        router = p["router"].view(np.float32).reshape(self.experts, self.hidden)
+        logits = o.matvec(o.F32, p["router"], self.experts, self.hidden, self.x)
+        assert np.allclose(logits, self.x @ router.T, rtol=1e-4, atol=1e-5)
+        bias = p["bias"].view(np.float32) if self.plan.requires_correction_bias else None
+        shared = (p["sgate"], p["sup"], p["sdown"]) if self.plan.shared_experts else None
+        return o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
+                           topk=self.topk, qtypes=(self.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
+                           shared=shared, inputs=self.x, logits=logits, bias=bias, scoring=self.scoring,
+                           normalize=True, scaling=1.5, act_q8=act_q8, threads=8)
+
+
+@pytest.mark.parametrize("qtype,act,scoring,shared", [
+    ("IQ2_XXS", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True),
+    ("IQ2_XXS", abi.ACT_DEVICE_F32, abi.SCORING_SIGMOID, True),
+    ("Q4_K", abi.ACT_DEVICE_ENCODED, abi.SCORING_SIGMOID, False),
+    ("Q8_0", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True)])
+def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, shared):
+    case = MoeCase(backend, oracle, qtype=qtype, act=act, scoring=scoring, shared=shared)
+    backend.workspace(case.workspace_bytes)
+    rc = case.execute()
+    assert rc == 0, case.err.message
+    res = case.result
+    want = case.oracle_layer(act_q8=act == abi.ACT_DEVICE_ENCODED)
+    assert np.array_equal(case.sel.reshape(case.rows, case.topk), want["selected"])     # identical routing
+    assert np.max(np.abs(case.wts.reshape(case.rows, case.topk) - want["weights"])) <= 1e-6
+    got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+    assert np.array_equal(got, case.combined) and case.rows_out.contents.is_written == 1
+    err = np.abs(got.astype(np.float64) - want["combined"])
+    outside = err > 1e-5 + 1e-3 * np.abs(want["combined"])
+    assert outside.mean() < 2e-2            # only bf16 rounding-boundary crossings may exceed it
+    assert np.all(err[outside] <= 2 * 2.0 ** -7 * np.abs(want["combined"][outside]) + 1e-4)
+    uniq = len(np.unique(want["selected"]))
+    assert res.completed == 1 and res.row_count == case.rows and res.unique_experts == uniq
+    assert res.row_expert_pairs == case.rows * case.topk and res.worklists.bucket_count == uniq
+    assert res.worklists.pair_count == case.rows * case.topk and res.stream_synchronizations == 1
+    per_expert = sum(case.parts[n].nbytes for n in ("gate", "up", "down")) // case.experts
+    assert res.active_weight_per_unique_expert_bytes == per_expert
+    assert res.encoded_bytes_read == res.active_weight_base_bytes + per_expert * uniq
+    assert res.kernel_launches >= 8 and res.memory.complete == 1
+
+
+def test_execute_rows_refusals(backend, oracle):
+    b = backend
+    case = MoeCase(b, oracle)
+    # workspace not preflighted
+    assert case.execute() == abi.NOMEM and case.rows_out.contents.is_written == 0
+    b.workspace(case.workspace_bytes)
+    # width outside the sealed mask: UNSUPPORTED before anything is touched
+    policy = abi.WorklistPolicy()
+    policy.schema_version, policy.supported_width_mask = 1, (1 << 1) | (1 << 4)
+    policy.narrow_kernel_family = abi.FAMILY_GFX950
+    case.job.worklist_policy = C.pointer(policy)
+    case.job.execution_batch = C.cast(C.pointer(policy), C.c_void_p)
+    sentinel = np.full(case.rows * case.hidden, 7.0, np.float32)
+    b.lib.yvex_backend_tensor_write(b.handle, case.rows_out, sentinel.ctypes.data, sentinel.nbytes, None)
+    assert case.execute() == abi.UNSUPPORTED
+    assert np.array_equal(b.read_f32(case.rows_out, sentinel.size), sentinel)
+    policy.supported_width_mask |= 1 << case.rows
+    assert case.execute() == 0, case.err.message
+    # execution batch and worklist policy must come together
+    case.job.execution_batch = None
+    assert case.execute() == abi.INVALID_ARG
+    case.job.worklist_policy = None
+    # mixed gate/up activation classes
+    case.job.weights[abi.W_ROUTED_UP].activation = abi.ACT_DEVICE_F32
+    assert case.execute() == abi.FORMAT
+    case.job.weights[abi.W_ROUTED_UP].activation = abi.ACT_DEVICE_ENCODED
+    # gate/up kernel families disagree
+    case.job.weights[abi.W_ROUTED_UP].kernel_family = abi.FAMILY_PORTABLE_EXPERT_ROW
+    assert case.execute() == abi.FORMAT
+    # unknown kernel family
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
+        case.job.weights[slot].kernel_family = b"sm121-int8-tensorcore-expert"
+    assert case.execute() == abi.UNSUPPORTED
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
+        case.job.weights[slot].kernel_family = abi.FAMILY_GFX950
+    # residual mixing envelope and the hash router are outside this backend
+    case.plan.mhc_mixing_rows = 24
+    assert case.execute() == abi.UNSUPPORTED
+    case.plan.mhc_mixing_rows = 0
+    case.plan.router_class = abi.ROUTER_HASH
+    assert case.execute() == abi.UNSUPPORTED
+    case.plan.router_class = abi.ROUTER_LEARNED
+    # cancellation is polled before launch
+    case.job.cancel_requested = abi.CANCEL_FN(lambda ctx: 1)
+    assert case.execute() == abi.CANCELLED
+    case.job.cancel_requested = abi.CANCEL_FN(0)
+    # a weight view outside the resident arena
+    saved = case.job.weights[abi.W_ROUTED_DOWN].encoded
+    case.job.weights[abi.W_ROUTED_DOWN].encoded = saved + (1 << 30)
+    assert case.execute() == abi.FORMAT
+    case.job.weights[abi.W_ROUTED_DOWN].encoded = saved
+    assert case.execute() == 0, case.err.message
+
+
+def test_execute_rows_deferred_completion(backend, oracle):
+    case = MoeCase(backend, oracle, rows=3)
+    backend.workspace(case.workspace_bytes)
+    completion = abi.DeviceCompletion(1, None)
+    case.job.device_completion = C.pointer(completion)
+    assert case.execute() == 0, case.err.message
+    assert case.result.device_completion_pending == 1 and case.result.completed == 0
+    done, err = abi.RowBatchResult(), abi.Error()
+    assert case.ops.complete_rows(backend.handle, 0, C.byref(done), C.byref(err)) == 0
+    assert done.completed == 1 and done.stream_synchronizations == 1
+    got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+    want = case.oracle_layer(act_q8=True)["combined"]
+    err_abs = np.abs(got.astype(np.float64) - want)
+    assert (err_abs > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2

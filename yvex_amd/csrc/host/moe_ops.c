@@ -1,0 +1,596 @@
+/*
+ * MoE row-batch operations of the ROCm backend (host side) and the host worklist builder.
+ * Restates the contract of src/backend/cuda/moe.c:113-183 (workspace), :905-990 (activation and
+ * kernel-family policy), :1826-1981 (execute / complete / operations table) and the sorting core
+ * of src/graph/worklist.c:369-441. All device work is enqueued on the backend's stream through
+ * the launch-level ABI; one synchronisation per layer publishes status, routing and worklist facts.
+ */
+#include <limits.h>
+#include <math.h>
+#include <string.h>
+#include <time.h>
+
+#include "private.h"
+
+#define ALIGN 256ull
+
+static unsigned long long align_up(unsigned long long v) { return (v + ALIGN - 1ull) & ~(ALIGN - 1ull); }
+
+static unsigned long long monotonic_ns(void)
+{
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (unsigned long long)ts.tv_sec * 1000000000ull + (unsigned long long)ts.tv_nsec;
+}
+
+/* Byte ranges bump-allocated from the attached workspace, in this order. */
+typedef struct {
+    unsigned long long input_q8, logits, bias, selected, weights;
+    unsigned long long order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts;
+    unsigned long long intermediate, intermediate_q8, pair_outputs;
+    unsigned long long shared_intermediate, shared_intermediate_q8, shared_outputs, routed;
+    unsigned long long total;
+} moe_ranges;
+
+static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows, moe_ranges *r)
+{
+    unsigned long long cursor = 0ull, pairs, hidden, routed_i, shared_i, experts;
+    if (!layer || !rows || rows > YVEX_ROCM_MOE_MAX_ROWS || !layer->hidden_width ||
+        !layer->routed_experts || layer->routed_experts > 256ull || !layer->experts_per_token ||
+        layer->experts_per_token > YVEX_MOE_MAX_SELECTED ||
+        layer->experts_per_token > layer->routed_experts || !layer->expert_intermediate_width ||
+        layer->hidden_width > (1ull << 20) || layer->expert_intermediate_width > (1ull << 20) ||
+        layer->shared_intermediate_width > (1ull << 20) || layer->shared_experts > 1ull)
+        return 0;
+    pairs = rows * layer->experts_per_token;
+    hidden = layer->hidden_width;
+    routed_i = layer->expert_intermediate_width;
+    shared_i = layer->shared_experts ? layer->shared_intermediate_width : 0ull;
+    experts = layer->routed_experts;
+#define TAKE(field, bytes) do { r->field = cursor; cursor = align_up(cursor + (bytes)); } while (0)
+    TAKE(input_q8, rows * ((hidden + 255ull) / 256ull) * 292ull);
+    TAKE(logits, rows * experts * sizeof(float));
+    TAKE(bias, experts * sizeof(float));
+    TAKE(selected, pairs * sizeof(unsigned long long));
+    TAKE(weights, pairs * sizeof(float));
+    TAKE(order, pairs * sizeof(unsigned long long));
+    TAKE(expert_ids, experts * sizeof(unsigned long long));
+    TAKE(bucket_offsets, (experts + 1ull) * sizeof(unsigned long long));
+    TAKE(bucket_populations, experts * sizeof(unsigned long long));
+    TAKE(sweep_offsets, (experts + 1ull) * sizeof(unsigned long long));
+    TAKE(counts, 4ull * sizeof(unsigned long long));
+    TAKE(intermediate, pairs * routed_i * sizeof(float));
+    TAKE(intermediate_q8, pairs * ((routed_i + 255ull) / 256ull) * 292ull);
+    TAKE(pair_outputs, pairs * hidden * sizeof(float));
+    TAKE(shared_intermediate, rows * shared_i * sizeof(float));
+    TAKE(shared_intermediate_q8, rows * ((shared_i + 255ull) / 256ull) * 292ull);
+    TAKE(shared_outputs, rows * hidden * sizeof(float));
+    TAKE(routed, rows * hidden * sizeof(float));
+#undef TAKE
+    r->total = cursor + ALIGN;   /* slack for aligning the workspace base itself */
+    return 1;
+}
+
+static int moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned long long row_count,
+                                  unsigned long long *bytes, yvex_error *err)
+{
+    moe_ranges ranges;
+    if (bytes) *bytes = 0ull;
+    if (!bytes || !moe_layout(layer, row_count, &ranges))
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.workspace",
+                                "MoE layer geometry or row count is outside this backend's bounds");
+    *bytes = ranges.total;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int layout_unsupported(const void *decision, unsigned long long *storage_bytes, yvex_error *err)
+{
+    (void)decision;
+    if (storage_bytes) *storage_bytes = 0ull;
+    return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.layout",
+                            "this backend streams canonical rows and defines no derived layout");
+}
+
+static int layout_build_unsupported(const void *decision, const unsigned char *canonical,
+                                    unsigned long long canonical_bytes, unsigned char *derived,
+                                    unsigned long long storage_bytes, yvex_error *err)
+{
+    (void)decision; (void)canonical; (void)canonical_bytes; (void)derived; (void)storage_bytes;
+    return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.layout",
+                            "this backend streams canonical rows and defines no derived layout");
+}
+
+static int q8_eligible(unsigned int qtype)
+{
+    return qtype == YVEX_GGUF_QTYPE_Q8_0 || qtype == YVEX_GGUF_QTYPE_Q2_K ||
+           qtype == YVEX_GGUF_QTYPE_Q4_K || qtype == YVEX_GGUF_QTYPE_IQ2_XXS;
+}
+
+static int family_admitted(const char *family)
+{
+    return family && (!strcmp(family, YVEX_MOE_KERNEL_PORTABLE_EXPERT_ROW) ||
+                      !strcmp(family, YVEX_MOE_KERNEL_PORTABLE_ENCODED_ROW) ||
+                      !strcmp(family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP));
+}
+
+/* Activation / kernel-family policy of one expert triple (moe.c:905-990). */
+static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight_view *up,
+                         const yvex_moe_weight_view *down, unsigned long long input_width,
+                         unsigned long long intermediate_width, int *act_q8, yvex_error *err)
+{
+    int gate_encoded, up_encoded, down_encoded;
+    if (gate->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED ||
+        up->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED ||
+        down->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.policy",
+                                "MoE activation policy is invalid");
+    gate_encoded = gate->activation == YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED;
+    up_encoded = up->activation == YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED;
+    down_encoded = down->activation == YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED;
+    if (gate_encoded != up_encoded)
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
+                                "MoE gate/up activations disagree");
+    if (gate_encoded && (!gate->kernel_family || !up->kernel_family ||
+                         strcmp(gate->kernel_family, up->kernel_family) != 0))
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
+                                "compiled MoE gate and up kernel-family decisions disagree");
+    if (gate->layout != up->layout || gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND ||
+        down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)
+        return yvex_rocm_refuse(err, gate->layout != up->layout ? YVEX_ERR_FORMAT : YVEX_ERR_UNSUPPORTED,
+                                "rocm.moe.policy", "compiled routed MoE layouts disagree or are derived");
+    if ((gate_encoded && !family_admitted(gate->kernel_family)) ||
+        (down_encoded && !family_admitted(down->kernel_family)))
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                "compiled MoE kernel family is not admitted by the rocm backend");
+    if (gate_encoded != down_encoded)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                "gate/up and down projections must share one activation class");
+    if (gate_encoded && (input_width % 256ull || intermediate_width % 256ull ||
+                         !q8_eligible(gate->qtype) || !q8_eligible(up->qtype) ||
+                         !q8_eligible(down->qtype)))
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                "compiled MoE activation is incompatible with its qtype geometry");
+    *act_q8 = gate_encoded;
+    return YVEX_OK;
+}
+
+/* Check one weight view against the geometry the plan implies and find its device address. */
+static int view_resolve(const yvex_backend *backend, const yvex_moe_weight_view *view,
+                        unsigned long long row_width, unsigned long long row_count,
+                        unsigned long long *device_address, yvex_error *err)
+{
+    const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(view->qtype);
+    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(view->qtype);
+    if (!capability || !geometry || !capability->device_compute_available)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.weights",
+                                "qtype has no device compute on this backend");
+    if (view->row_width != row_width || view->row_count != row_count || !geometry->block_size ||
+        row_width % geometry->block_size ||
+        row_width / geometry->block_size * geometry->bytes_per_block != view->row_bytes ||
+        view->row_bytes > ULLONG_MAX / (row_count ? row_count : 1ull) ||
+        view->row_bytes * row_count != view->encoded_bytes)
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                "MoE weight view geometry disagrees with the layer plan");
+    if (view->device_address) {
+        *device_address = view->device_address;
+        return YVEX_OK;
+    }
+    if (!view->encoded || !yvex_rocm_resolve(backend, view->encoded, view->encoded_bytes, device_address))
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                "MoE weight view is not inside the attached resident arena");
+    return YVEX_OK;
+}
+
+static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weight_view *gate,
+                                const yvex_moe_weight_view *up, const yvex_moe_weight_view *down,
+                                unsigned long long gate_address, unsigned long long up_address,
+                                unsigned long long down_address, unsigned long long hidden,
+                                unsigned long long intermediate)
+{
+    w->gate = (const uint8_t *)(uintptr_t)gate_address;
+    w->up = (const uint8_t *)(uintptr_t)up_address;
+    w->down = (const uint8_t *)(uintptr_t)down_address;
+    w->gate_qtype = gate->qtype;
+    w->up_qtype = up->qtype;
+    w->down_qtype = down->qtype;
+    w->hidden = hidden;
+    w->intermediate = intermediate;
+    w->gate_row_bytes = gate->row_bytes;
+    w->up_row_bytes = up->row_bytes;
+    w->down_row_bytes = down->row_bytes;
+    w->gate_expert_bytes = gate->row_bytes * intermediate;
+    w->up_expert_bytes = up->row_bytes * intermediate;
+    w->down_expert_bytes = down->row_bytes * hidden;
+}
+
+static int same_expert_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)
+{
+    return a->gate_qtype == b->gate_qtype && a->up_qtype == b->up_qtype &&
+           a->down_qtype == b->down_qtype && a->hidden == b->hidden &&
+           a->intermediate == b->intermediate;
+}
+
+static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job,
+                            const yvex_moe_row_batch *rows, const yvex_moe_row_batch_output *output,
+                            yvex_moe_row_batch_result *result, yvex_error *err)
+{
+    const yvex_moe_layer_plan *layer = job ? job->layer : NULL;
+    const yvex_moe_weight_view *views = job ? job->weights : NULL;
+    yvex_hip_expert_weights routed, shared;
+    moe_ranges ranges;
+    unsigned long long base, pairs, hidden, experts, topk, row_count, launches = 0ull;
+    unsigned long long router_address = 0ull, bias_address = 0ull, addresses[6] = {0};
+    unsigned long long d2h = 0ull, started, counts[4] = {0};
+    int unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, device_status = 0, rc, defer;
+    void *status;
+    yvex_hip_stream stream;
+    if (result) memset(result, 0, sizeof(*result));
+    unsupported_width = job && rows && job->worklist_policy &&
+                        (rows->row_count >= 64ull ||
+                         !(job->worklist_policy->supported_width_mask & (1ull << rows->row_count)));
+    if (unsupported_width)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
+                                "row count is outside the sealed supported width mask");
+    if (!backend || !job || !layer || !rows || !output || !result ||
+        backend->kind != YVEX_BACKEND_KIND_ROCM ||
+        ((job->execution_batch == NULL) != (job->worklist_policy == NULL)) ||
+        rows->schema_version != YVEX_MOE_ROW_BATCH_SCHEMA_V1 || !rows->row_count ||
+        rows->row_count > YVEX_ROCM_MOE_MAX_ROWS || rows->row_width != layer->hidden_width ||
+        rows->row_stride != rows->row_width ||
+        !yvex_rocm_tensor_owner_is(backend, rows->device_rows) ||
+        !yvex_rocm_tensor_owner_is(backend, rows->device_outputs) ||
+        rows->device_rows == rows->device_outputs || !rows->device_rows->is_written ||
+        rows->device_rows->dtype != YVEX_DTYPE_F32 || rows->device_outputs->dtype != YVEX_DTYPE_F32 ||
+        rows->device_rows->bytes < rows->row_count * rows->row_width * sizeof(float) ||
+        rows->device_outputs->bytes < rows->row_count * rows->row_width * sizeof(float))
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
+                                "width-N MoE owners, geometry or admitted width are invalid");
+    if (layer->expanded_width != layer->hidden_width || layer->mhc_mixing_rows ||
+        layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE ||
+        (layer->scoring != YVEX_MOE_SCORING_SQRT_SOFTPLUS && layer->scoring != YVEX_MOE_SCORING_SIGMOID))
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
+                                "residual mixing, hash routing and other scoring policies are outside this backend");
+    row_count = rows->row_count;
+    hidden = layer->hidden_width;
+    experts = layer->routed_experts;
+    topk = layer->experts_per_token;
+    if (!moe_layout(layer, row_count, &ranges))
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
+                                "MoE layer geometry is outside this backend's bounds");
+    pairs = row_count * topk;
+    if ((output->selected_experts || output->selected_weights) && output->selection_capacity < pairs)
+        return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows", "selection capacity is too small");
+    if ((output->combined_rows && output->combined_capacity < row_count * hidden) ||
+        (output->routed_rows && output->routed_capacity < row_count * hidden) ||
+        (output->shared_rows && output->shared_capacity < row_count * hidden))
+        return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows", "host output capacity is too small");
+    if (job->cancel_requested && job->cancel_requested(job->cancel_context))
+        return yvex_rocm_refuse(err, YVEX_ERR_CANCELLED, "rocm.moe.rows",
+                                "width-N MoE was cancelled before launch");
+    if (!backend->workspace_device_tensor || backend->workspace_bytes < ranges.total)
+        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.rows",
+                                "width-N MoE workspace was not preflighted");
+    has_shared = layer->shared_experts == 1ull;
+    rc = expert_policy(&views[YVEX_MOE_WEIGHT_ROUTED_GATE], &views[YVEX_MOE_WEIGHT_ROUTED_UP],
+                       &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], hidden, layer->expert_intermediate_width,
+                       &routed_q8, err);
+    if (rc == YVEX_OK && has_shared)
+        rc = expert_policy(&views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
+                           &views[YVEX_MOE_WEIGHT_SHARED_DOWN], hidden, layer->shared_intermediate_width,
+                           &shared_q8, err);
+    if (rc != YVEX_OK) return rc;
+    /* weights: router [experts x hidden], optional bias [1 x experts], expert-major matrices */
+    rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER], hidden, experts, &router_address, err);
+    if (rc == YVEX_OK && layer->requires_correction_bias)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER_BIAS], experts, 1ull, &bias_address, err);
+    if (rc == YVEX_OK)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], hidden,
+                          experts * layer->expert_intermediate_width, &addresses[0], err);
+    if (rc == YVEX_OK)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_UP], hidden,
+                          experts * layer->expert_intermediate_width, &addresses[1], err);
+    if (rc == YVEX_OK)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], layer->expert_intermediate_width,
+                          experts * hidden, &addresses[2], err);
+    if (rc == YVEX_OK && has_shared)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_GATE], hidden,
+                          layer->shared_intermediate_width, &addresses[3], err);
+    if (rc == YVEX_OK && has_shared)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_UP], hidden,
+                          layer->shared_intermediate_width, &addresses[4], err);
+    if (rc == YVEX_OK && has_shared)
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], layer->shared_intermediate_width,
+                          hidden, &addresses[5], err);
+    if (rc != YVEX_OK) return rc;
+    if (!(layer->activation_limit > 0.0) || !isfinite(layer->activation_limit) ||
+        !isfinite(layer->routed_scaling_factor))
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
+                                "activation limit and routed scaling must be finite");
+    rc = yvex_rocm_require_kernels(backend, "rocm.moe.rows", err);
+    if (rc != YVEX_OK) return rc;
+
+    rows->device_outputs->is_written = 0;
+    started = monotonic_ns();
+    yvex_rocm_workspace_reset(backend);
+    if (!yvex_backend_workspace_acquire(backend, ranges.total - ALIGN, ALIGN, &base))
+        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.rows", "workspace acquisition failed");
+    fill_expert_weights(&routed, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], &views[YVEX_MOE_WEIGHT_ROUTED_UP],
+                        &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], addresses[0], addresses[1], addresses[2],
+                        hidden, layer->expert_intermediate_width);
+    if (has_shared)
+        fill_expert_weights(&shared, &views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
+                            &views[YVEX_MOE_WEIGHT_SHARED_DOWN], addresses[3], addresses[4], addresses[5],
+                            hidden, layer->shared_intermediate_width);
+    merged = has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
+    if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
+        return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",
+                                "kernel launch failed (test seam)");
+    status = backend->device_status;
+    stream = backend->stream;
+#define AT(field) ((void *)(uintptr_t)(base + ranges.field))
+#define LAUNCH(call, where)                                             \
+    do {                                                                \
+        if (rc == YVEX_OK) {                                            \
+            rc = yvex_rocm_launch_result((call), (where), err);         \
+            if (rc == YVEX_OK) launches++;                              \
+        }                                                               \
+    } while (0)
+    LAUNCH(yvex_hip_fill_u32(status, 0u, 1u, stream), "rocm.moe.rows.status");
+    if (has_shared && !merged)
+        LAUNCH(yvex_hip_fill_u32(AT(shared_outputs), 0u, row_count * hidden, stream), "rocm.moe.rows.zero");
+    /* router: logits = router . row (F32 activations, as src/backend/cuda/moe.c:1259-1284) */
+    LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)router_address, views[YVEX_MOE_WEIGHT_ROUTER].qtype,
+                           experts, hidden, views[YVEX_MOE_WEIGHT_ROUTER].row_bytes,
+                           rows->device_rows->data, 0, row_count, hidden, NULL, (float *)AT(logits),
+                           experts, 0, (int *)status, stream), "rocm.moe.rows.router");
+    if (layer->requires_correction_bias)
+        LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)bias_address, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype,
+                               1ull, experts, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].row_bytes, NULL, 1ull,
+                               (float *)AT(bias), (int *)status, stream), "rocm.moe.rows.bias");
+    LAUNCH(yvex_hip_moe_route_rows((const float *)AT(logits),
+                                   layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                   row_count, experts, topk, (int)layer->scoring,
+                                   layer->normalize_topk_probabilities, layer->routed_scaling_factor,
+                                   (uint64_t *)AT(selected), (float *)AT(weights), (int *)status, stream),
+           "rocm.moe.rows.route");
+    LAUNCH(yvex_hip_worklist_build((const uint64_t *)AT(selected), pairs, topk, experts,
+                                   (uint64_t *)AT(order), (uint64_t *)AT(expert_ids),
+                                   (uint64_t *)AT(bucket_offsets), (uint64_t *)AT(bucket_populations),
+                                   (uint64_t *)AT(sweep_offsets), (uint64_t *)AT(counts), (int *)status,
+                                   stream), "rocm.moe.rows.worklist");
+    if (routed_q8 || (has_shared && shared_q8))
+        LAUNCH(yvex_hip_q8k_quantize((const float *)rows->device_rows->data, row_count, hidden, hidden,
+                                     (uint8_t *)AT(input_q8), (int *)status, stream), "rocm.moe.rows.q8");
+    LAUNCH(yvex_hip_moe_up(&routed, routed_q8 ? AT(input_q8) : (void *)rows->device_rows->data, routed_q8,
+                           (const float *)AT(weights), (const uint64_t *)AT(order),
+                           (const uint64_t *)AT(expert_ids), (const uint64_t *)AT(bucket_offsets),
+                           (const uint64_t *)AT(bucket_populations), (const uint64_t *)AT(sweep_offsets),
+                           (const uint64_t *)AT(counts), pairs, topk, experts, layer->activation_limit,
+                           (float *)AT(intermediate), merged ? &shared : NULL, merged ? row_count : 0ull,
+                           merged ? (float *)AT(shared_intermediate) : NULL, (int *)status, stream),
+           "rocm.moe.rows.up");
+    if (has_shared && !merged)
+        LAUNCH(yvex_hip_moe_up(&shared, shared_q8 ? AT(input_q8) : (void *)rows->device_rows->data,
+                               shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull, 1ull,
+                               layer->activation_limit, (float *)AT(shared_intermediate), NULL, 0ull, NULL,
+                               (int *)status, stream), "rocm.moe.rows.shared-up");
+    if (routed_q8)
+        LAUNCH(yvex_hip_q8k_quantize((const float *)AT(intermediate), pairs, layer->expert_intermediate_width,
+                                     layer->expert_intermediate_width, (uint8_t *)AT(intermediate_q8),
+                                     (int *)status, stream), "rocm.moe.rows.q8-mid");
+    if (has_shared && shared_q8)
+        LAUNCH(yvex_hip_q8k_quantize((const float *)AT(shared_intermediate), row_count,
+                                     layer->shared_intermediate_width, layer->shared_intermediate_width,
+                                     (uint8_t *)AT(shared_intermediate_q8), (int *)status, stream),
+               "rocm.moe.rows.q8-shared-mid");
+    LAUNCH(yvex_hip_moe_down(&routed, routed_q8 ? AT(intermediate_q8) : AT(intermediate), routed_q8,
+                             (const uint64_t *)AT(order), (const uint64_t *)AT(expert_ids),
+                             (const uint64_t *)AT(bucket_offsets), (const uint64_t *)AT(bucket_populations),
+                             (const uint64_t *)AT(sweep_offsets), (const uint64_t *)AT(counts), pairs,
+                             experts, (float *)AT(pair_outputs), merged ? &shared : NULL,
+                             merged ? row_count : 0ull,
+                             merged ? (shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate)) : NULL,
+                             merged ? (float *)AT(shared_outputs) : NULL, (int *)status, stream),
+           "rocm.moe.rows.down");
+    if (has_shared && !merged)
+        LAUNCH(yvex_hip_moe_down(&shared, shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate),
+                                 shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull,
+                                 (float *)AT(shared_outputs), NULL, 0ull, NULL, NULL, (int *)status, stream),
+               "rocm.moe.rows.shared-down");
+    if (!has_shared)
+        LAUNCH(yvex_hip_fill_u32(AT(shared_outputs), 0u, row_count * hidden, stream), "rocm.moe.rows.zero");
+    LAUNCH(yvex_hip_moe_reduce_combine((const float *)AT(pair_outputs), row_count, topk, hidden,
+                                       (const float *)AT(shared_outputs), (float *)AT(routed),
+                                       (float *)rows->device_outputs->data, (int *)status, stream),
+           "rocm.moe.rows.combine");
+    if (rc != YVEX_OK) return rc;
+
+    defer = job->device_completion && job->device_completion->defer;
+    result->schema_version = YVEX_MOE_ROW_BATCH_RESULT_SCHEMA_V4;
+    result->execution_class = YVEX_EXECUTION_CLASS_DEVICE_NATIVE;
+    result->row_count = row_count;
+    result->row_expert_pairs = pairs;
+    result->kernel_launches = launches;
+    result->shared_expert_operations = has_shared ? row_count : 0ull;
+    result->grouped_expert_operations = pairs;
+    result->active_weight_base_bytes = views[YVEX_MOE_WEIGHT_ROUTER].encoded_bytes +
+        (has_shared ? views[YVEX_MOE_WEIGHT_SHARED_GATE].encoded_bytes +
+                      views[YVEX_MOE_WEIGHT_SHARED_UP].encoded_bytes +
+                      views[YVEX_MOE_WEIGHT_SHARED_DOWN].encoded_bytes : 0ull);
+    result->active_weight_per_unique_expert_bytes =
+        routed.gate_expert_bytes + routed.up_expert_bytes + routed.down_expert_bytes;
+    result->memory.activation_bytes = 2ull * row_count * hidden * sizeof(float);
+    result->memory.temporary_bytes = ranges.total;
+    result->memory.measured_operations = 1ull;
+    if (defer) {
+        backend->pending_completion = 1;
+        result->device_completion_pending = 1;
+        rows->device_outputs->is_written = 1;   /* ordered on the backend stream */
+        result->total_ns = monotonic_ns() - started;
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    /* one synchronisation publishes status, worklist facts, routing and optional host copies */
+    {
+        unsigned long long sync_started = monotonic_ns();
+        rc = yvex_rocm_finish(backend, "rocm.moe.rows.sync", &device_status, err);
+        result->synchronization_ns = monotonic_ns() - sync_started;
+    }
+    d2h += sizeof(int);
+    if (rc == YVEX_OK && device_status)
+        rc = yvex_rocm_refuse(err, device_status == 1 ? YVEX_ERR_FORMAT : YVEX_ERR_BACKEND,
+                              "rocm.moe.rows", device_status == 1
+                                  ? "width-N MoE produced invalid numerics"
+                                  : "width-N MoE kernels met a contract violation");
+#define DOWNLOAD(dst, field, bytes)                                                          \
+    do {                                                                                     \
+        if (rc == YVEX_OK && (dst)) {                                                        \
+            if (yvex_hip_memcpy_d2h((dst), AT(field), (bytes), stream) != 0)                 \
+                rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.download",       \
+                                      yvex_hip_last_error());                                \
+            else { d2h += (bytes); result->download_count++; }                               \
+        }                                                                                    \
+    } while (0)
+    {
+        unsigned long long *counts_host = counts;
+        DOWNLOAD(counts_host, counts, sizeof(counts));
+    }
+    DOWNLOAD(output->selected_experts, selected, pairs * sizeof(unsigned long long));
+    DOWNLOAD(output->selected_weights, weights, pairs * sizeof(float));
+    DOWNLOAD(output->routed_rows, routed, row_count * hidden * sizeof(float));
+    DOWNLOAD(output->shared_rows, shared_outputs, row_count * hidden * sizeof(float));
+    if (rc == YVEX_OK && output->combined_rows) {
+        if (yvex_hip_memcpy_d2h(output->combined_rows, rows->device_outputs->data,
+                                row_count * hidden * sizeof(float), stream) != 0)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.download", yvex_hip_last_error());
+        else { d2h += row_count * hidden * sizeof(float); result->download_count++; }
+    }
+#undef DOWNLOAD
+#undef LAUNCH
+#undef AT
+    if (rc != YVEX_OK) {
+        memset(result, 0, sizeof(*result));
+        return rc;
+    }
+    backend->memory.d2h_bytes += d2h - sizeof(int);
+    result->completed = 1;
+    result->unique_experts = counts[0];
+    result->worklists.schema_version = 1u;
+    result->worklists.worklist_count = 1ull;
+    result->worklists.pair_count = counts[2];
+    result->worklists.bucket_count = counts[0];
+    result->worklists.maximum_bucket_population = counts[1];
+    result->worklists.narrow_pairs = counts[2];
+    result->worklists.width_histogram[row_count < YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP
+                                          ? row_count : YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP - 1u] = 1ull;
+    result->worklists.provenance_counts[rows->provenance <= YVEX_EXECUTION_BATCH_COMPILED_COMPATIBLE
+                                            ? rows->provenance : 0] = 1ull;
+    result->expert_subviews_accessed = 3ull * counts[0] + (has_shared ? 3ull : 0ull);
+    result->encoded_bytes_read = result->active_weight_base_bytes +
+                                 result->active_weight_per_unique_expert_bytes * counts[0];
+    result->memory.active_weight_bytes = result->encoded_bytes_read;
+    result->memory.complete = 1;
+    result->d2h_bytes = d2h;
+    result->stream_synchronizations = 1ull;
+    result->total_ns = monotonic_ns() - started;
+    rows->device_outputs->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int moe_complete_rows(yvex_backend *backend, int barrier_observed,
+                             yvex_moe_row_batch_result *result, yvex_error *err)
+{
+    unsigned long long started = 0ull;
+    int device_status = 0, rc = YVEX_OK;
+    if (result) memset(result, 0, sizeof(*result));
+    if (!backend || !result || (barrier_observed != 0 && barrier_observed != 1) ||
+        backend->kind != YVEX_BACKEND_KIND_ROCM)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.complete",
+                                "MoE completion owner is invalid");
+    if (!backend->host_only) {
+        started = monotonic_ns();
+        rc = yvex_rocm_finish(backend, "rocm.moe.rows.phase-sync", &device_status, err);
+        if (rc == YVEX_OK && device_status)
+            rc = yvex_rocm_refuse(err, device_status == 1 ? YVEX_ERR_FORMAT : YVEX_ERR_BACKEND,
+                                  "rocm.moe.complete", "deferred width-N MoE reported a device failure");
+    }
+    if (rc != YVEX_OK) return rc;
+    backend->pending_completion = 0;
+    result->schema_version = YVEX_MOE_ROW_BATCH_RESULT_SCHEMA_V4;
+    result->completed = 1;
+    result->execution_class = YVEX_EXECUTION_CLASS_DEVICE_NATIVE;
+    result->stream_synchronizations = barrier_observed ? 0ull : 1ull;
+    result->synchronization_ns = started ? monotonic_ns() - started : 0ull;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static const yvex_backend_moe_operations moe_operations = {
+    layout_unsupported, layout_build_unsupported, moe_workspace_required, moe_execute_rows,
+    moe_complete_rows};
+
+const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend)
+{
+    if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !backend->kernels_available ||
+        backend->status == YVEX_BACKEND_STATUS_FAILED)
+        return NULL;
+    return &moe_operations;
+}
+
+/* ---- host worklist: src/graph/worklist.c:369-441 ---------------------------------------------- */
+
+int yvex_expert_worklist_build(const unsigned long long *selected_experts,
+                               const float *route_weights, unsigned long long pair_count,
+                               unsigned long long experts_per_row, unsigned long long expert_count,
+                               const yvex_expert_worklist_storage *storage,
+                               yvex_expert_worklist_observation *observation, yvex_error *err)
+{
+    unsigned long long expert, pair, cursor = 0ull, bucket = 0ull, maximum = 0ull;
+    if (observation) memset(observation, 0, sizeof(*observation));
+    if (!selected_experts || !route_weights || !storage || !observation || !experts_per_row ||
+        !expert_count || expert_count > 256ull || experts_per_row > expert_count || !pair_count ||
+        pair_count % experts_per_row || !storage->expert_ids || !storage->bucket_offsets ||
+        !storage->bucket_populations || !storage->source_pairs || !storage->source_rows ||
+        !storage->destination_rows || !storage->route_weights ||
+        storage->bucket_capacity < expert_count || storage->pair_capacity < pair_count)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "worklist.build",
+                                "expert worklist request or storage is invalid");
+    for (pair = 0ull; pair < pair_count; ++pair)
+        if (selected_experts[pair] >= expert_count || !isfinite(route_weights[pair]))
+            return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "worklist.build",
+                                    "routed pair has an invalid expert or weight");
+    for (expert = 0ull; expert < expert_count; ++expert) {
+        unsigned long long start = cursor, population;
+        for (pair = 0ull; pair < pair_count; ++pair) {
+            if (selected_experts[pair] != expert) continue;
+            storage->source_pairs[cursor] = pair;
+            storage->source_rows[cursor] = pair / experts_per_row;
+            storage->destination_rows[cursor] = pair;
+            storage->route_weights[cursor] = route_weights[pair];
+            cursor++;
+        }
+        population = cursor - start;
+        if (!population) continue;
+        storage->expert_ids[bucket] = expert;
+        storage->bucket_offsets[bucket] = start;
+        storage->bucket_populations[bucket] = population;
+        if (population > maximum) maximum = population;
+        observation->population_histogram[population < YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP
+                                              ? population : YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP - 1u]++;
+        bucket++;
+    }
+    storage->bucket_offsets[bucket] = cursor;
+    if (cursor != pair_count)
+        return yvex_rocm_refuse(err, YVEX_ERR_STATE, "worklist.build",
+                                "expert worklist did not emit every routed pair");
+    observation->schema_version = 1u;
+    observation->worklist_count = 1ull;
+    observation->pair_count = pair_count;
+    observation->bucket_count = bucket;
+    observation->maximum_bucket_population = maximum;
+    observation->narrow_pairs = pair_count;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}

@@ -1,0 +1,51 @@
+/*
+ * Private state of the ROCm backend object. Mirrors the shape of the reference's backend owner
+ * (src/backend/private.h:66-162): status word, memory accounting, one attached resident arena,
+ * one attached device workspace with a bump cursor that every operation resets.
+ */
+#ifndef YVEX_ROCM_PRIVATE_H
+#define YVEX_ROCM_PRIVATE_H
+
+#include "yvex_rocm.h"
+#include "yvex_rocm_kernels.h"
+
+struct yvex_backend {
+    yvex_backend_kind kind;
+    yvex_backend_status status;
+    unsigned long long owner_id;
+    int device_index;
+    int host_only;             /* YVEX_TEST_ROCM_NO_DEVICE: tensors in host memory, no kernels */
+    int kernels_available;
+    yvex_hip_stream stream;
+    yvex_backend_memory_stats memory;
+    unsigned long long live_tensors;
+    /* resident arena: host shadow range -> device range */
+    const unsigned char *resident_host_base;
+    unsigned long long resident_host_bytes;
+    const yvex_device_tensor *resident_device_tensor;
+    unsigned long long resident_device_address;
+    unsigned long long resident_generation;
+    /* device workspace */
+    const yvex_device_tensor *workspace_device_tensor;
+    unsigned long long workspace_bytes, workspace_cursor;
+    /* device status word shared by the operations of this backend */
+    int *device_status;
+    int pending_completion;
+};
+
+int yvex_rocm_refuse(yvex_error *err, yvex_status code, const char *where, const char *message);
+int yvex_rocm_seam(const char *name);
+int yvex_rocm_tensor_owner_is(const yvex_backend *backend, const yvex_device_tensor *tensor);
+void yvex_rocm_workspace_reset(yvex_backend *backend);
+/* Kernels present and the backend healthy, else the typed refusal of a missing bundle. */
+int yvex_rocm_require_kernels(const yvex_backend *backend, const char *where, yvex_error *err);
+/* Map a launch-level return code (negative yvex_status) to an error. */
+int yvex_rocm_launch_result(int rc, const char *where, yvex_error *err);
+/* Stream synchronise + read the device status word (and clear it for the next operation). */
+int yvex_rocm_finish(yvex_backend *backend, const char *where, int *device_status, yvex_error *err);
+int yvex_rocm_status_reset(yvex_backend *backend, const char *where, yvex_error *err);
+/* Resolve a weight view: device_address if given, else the resident arena mapping. */
+int yvex_rocm_resolve(const yvex_backend *backend, const unsigned char *host,
+                      unsigned long long bytes, unsigned long long *device_address);
+
+#endif
