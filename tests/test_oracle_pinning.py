@@ -1,0 +1,405 @@
+"""What pins the CPU oracle: the reference's golden vectors and known-answer tests, fixtures
+written by the library compiled from the reference's own sources, that library itself where it
+can be built, and closed forms / brute force for what those leave open (Q4_K, sigmoid scoring,
+the Q8_K quantizer, the integer block dots).
+"""
+import ctypes as C
+import math
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def golden():
+    return np.load(GOLDEN)
+
+
+@pytest.fixture(scope="module")
+def L(oracle):
+    return oracle.lib()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+# ---- scalar rules: tests/unit/quant_numeric.c:188-259 ---------------------------------------
+
+def test_f16_exhaustive_round_trip(L):
+    for code in range(65536):
+        value = L.yvo_f16_decode(code)
+        exponent, mantissa = (code >> 10) & 31, code & 1023
+        encoded = L.yvo_f16_encode(value)
+        if exponent == 31 and mantissa:
+            assert math.isnan(value) and (encoded & 0x7c00) == 0x7c00 and (encoded & 0x3ff)
+        else:
+            assert encoded == code
+    # against numpy's IEEE binary16 (an independent implementation) for every finite code
+    codes = np.arange(65536, dtype=np.uint16)
+    want = codes.view(np.float16).astype(np.float32)
+    got = np.array([L.yvo_f16_decode(int(c)) for c in codes], np.float32)
+    finite = np.isfinite(want)
+    assert np.array_equal(bits(got[finite]), bits(want[finite]))
+    assert L.yvo_f16_encode(1.00048828125) == 0x3c00 and L.yvo_f16_encode(1.00146484375) == 0x3c02
+    assert L.yvo_f16_decode(0x0001) == 2.0 ** -24 and L.yvo_f16_decode(0x7bff) == 65504.0
+    assert math.copysign(1.0, L.yvo_f16_decode(0x8000)) == -1.0
+    assert math.isinf(L.yvo_f16_decode(0x7c00)) and L.yvo_f16_encode(3.4e38) == 0x7c00
+
+
+def test_bf16_exhaustive_round_trip(L):
+    for code in range(65536):
+        value = L.yvo_bf16_decode(code)
+        exponent, mantissa = (code >> 7) & 255, code & 127
+        encoded = L.yvo_bf16_encode(value)
+        if exponent == 255 and mantissa:
+            assert math.isnan(value) and (encoded & 0x7f80) == 0x7f80 and (encoded & 0x7f)
+        else:
+            assert encoded == code
+    halfway = np.array([0x3f808000, 0x3f818000], np.uint32).view(np.float32)
+    assert L.yvo_bf16_encode(float(halfway[0])) == 0x3f80 and L.yvo_bf16_encode(float(halfway[1])) == 0x3f82
+
+
+def test_scalar_rules_match_reference_fixture(L, golden):
+    got = np.array([L.yvo_f16_decode(int(c)) for c in golden["f16_codes"]], np.float32)
+    want = golden["f16_decode_bits"]
+    nan = np.isnan(got)
+    assert np.array_equal(bits(got)[~nan], want[~nan])
+    assert np.all(np.isnan(want[nan].view(np.float32)))
+    samples = golden["scalar_samples"]
+    assert np.array_equal(np.array([L.yvo_f16_encode(float(v)) for v in samples], np.uint16), golden["f16_encode"])
+    assert np.array_equal(np.array([L.yvo_bf16_encode(float(v)) for v in samples], np.uint16), golden["bf16_encode"])
+
+
+# ---- block codecs: tests/unit/quant_numeric.c:502-609 -----------------------------------------
+
+def test_golden_block_bytes(L, oracle):
+    src = np.zeros(32, np.float32)
+    src[:4] = [127.0, -127.0, 0.5, -0.5]
+    enc = np.zeros(34, np.uint8)
+    assert L.yvo_q8_0_encode_block(src.ctypes.data_as(C.c_void_p), enc.ctypes.data_as(C.c_void_p)) == 1
+    assert list(enc[:6]) == [0x00, 0x3c, 0x7f, 0x81, 0x01, 0xff]          # halfway codes round away
+    q2 = np.zeros(84, np.uint8)
+    q2[:16] = 0x01
+    q2[16:80] = 0xe4
+    q2[80:82] = [0x00, 0x3c]
+    dec = oracle.decode_rows(oracle.Q2_K, q2, 256)[0]
+    assert np.array_equal(dec, ((np.arange(256) % 128) // 32).astype(np.float32))
+    mx = np.zeros(17, np.uint8)
+    mx[0], mx[1:] = 127, 0x21
+    out = np.zeros(32, np.float32)
+    assert L.yvo_decode_block(oracle.MXFP4, mx.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p)) == 0
+    assert np.all(out[:16] == 0.5) and np.all(out[16:] == 1.0)
+    # refusals: non-finite or negative scales (quant_block.c:819-833, :856-881)
+    bad = np.zeros(34, np.uint8)
+    bad[1] = 0x7c
+    assert L.yvo_decode_block(oracle.Q8_0, bad.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p)) == oracle.ERR_FORMAT
+    bad2 = np.zeros(84, np.uint8)
+    bad2[81] = 0x7c
+    big = np.zeros(256, np.float32)
+    assert L.yvo_decode_block(oracle.Q2_K, bad2.ctypes.data_as(C.c_void_p), big.ctypes.data_as(C.c_void_p)) == oracle.ERR_FORMAT
+    neg = np.zeros(66, np.uint8)
+    neg[1] = 0xbc
+    assert L.yvo_decode_block(oracle.IQ2_XXS, neg.ctypes.data_as(C.c_void_p), big.ctypes.data_as(C.c_void_p)) == oracle.ERR_FORMAT
+
+
+@pytest.mark.parametrize("name,qtype", [("q8_0", 8), ("q2_k", 10), ("iq2_xxs", 16)])
+def test_decode_and_row_dot_match_reference_fixture(oracle, golden, name, qtype):
+    blob, x = golden[f"{name}_blob"], golden[f"{name}_x"]
+    block, nbytes = oracle.geometry(qtype)
+    decoded = oracle.decode_rows(qtype, blob, 512)
+    assert np.array_equal(bits(decoded).reshape(-1), golden[f"{name}_decoded_bits"].reshape(-1))
+    rb = 512 // block * nbytes
+    dots = [oracle.cpu_dot(qtype, blob[r * rb:(r + 1) * rb], x) for r in range(blob.size // rb)]
+    assert all(rc == 0 for rc, _ in dots)
+    assert np.array_equal(bits(np.array([v for _, v in dots], np.float32)), golden[f"{name}_dots_bits"])
+    # float64 brute force of the same definition
+    brute = (decoded.astype(np.float64) * x.astype(np.float64)).sum(axis=1)
+    assert np.allclose([v for _, v in dots], brute, rtol=1e-6, atol=1e-7)
+
+
+def test_iq2_grid_is_the_public_codebook(L, oracle):
+    # first and last entries of ggml's iq2xxs_grid and structural facts of the table
+    one = np.zeros(66, np.uint8)
+    one[0:2] = [0x00, 0x3c]                                     # d = 1
+    out = np.zeros(256, np.float32)
+
+    def magnitudes(index):
+        one[2:6] = [index, 0, 0, 0]
+        one[6:10] = [0, 0, 0, 0]
+        L.yvo_decode_block(oracle.IQ2_XXS, one.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+        return [int(round(v * 8)) for v in out[:8]]            # gs = 1 * 0.5 * 0.25
+
+    assert magnitudes(0) == [8] * 8
+    assert magnitudes(1) == [43, 8, 8, 8, 8, 8, 8, 8]           # 0x080808080808082b
+    assert magnitudes(2) == [25, 25, 8, 8, 8, 8, 8, 8]          # 0x0808080808081919
+    seen = {tuple(magnitudes(i)) for i in range(256)}
+    assert len(seen) == 256 and all(set(m) <= {8, 25, 43} for m in seen)
+    # sign rule: seven stored bits plus an even-parity eighth
+    one[2:6] = 0
+    one[6:10] = np.array([0b0000011], np.uint32).view(np.uint8)
+    L.yvo_decode_block(oracle.IQ2_XXS, one.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+    assert list(np.sign(out[:8])) == [-1, -1, 1, 1, 1, 1, 1, 1]
+    one[6:10] = np.array([0b0000001], np.uint32).view(np.uint8)
+    L.yvo_decode_block(oracle.IQ2_XXS, one.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+    assert list(np.sign(out[:8])) == [-1, 1, 1, 1, 1, 1, 1, -1]
+    # group scale (0.5 + s) / 4 from the top nibble
+    one[6:10] = np.array([7 << 28], np.uint32).view(np.uint8)
+    L.yvo_decode_block(oracle.IQ2_XXS, one.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+    assert out[0] == 8 * 7.5 * 0.25 and out[32] == 8 * 0.5 * 0.25
+
+
+def test_live_reference_library_agrees(oracle):
+    """Where oracle/_ref can be built, replay fresh random data through both."""
+    ref = oracle.ref_lib()
+    if ref is None:
+        pytest.skip("reference tree absent: the committed fixture stands in")
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import make_golden
+    for qtype in (oracle.Q8_0, oracle.Q2_K, oracle.IQ2_XXS, oracle.F32):
+        block, nbytes = oracle.geometry(qtype)
+        g = oracle.Generator(7, f"live.{qtype}")
+        width = 1024 if block > 1 else 96
+        blob, x = g.weights(qtype, 3, width), g.normal(width)
+        rb = width // block * nbytes
+        if block > 1:
+            want = make_golden.ref_decode(ref, qtype, blob, nbytes, block)
+            assert np.array_equal(bits(oracle.decode_rows(qtype, blob, width)).reshape(-1), bits(want).reshape(-1))
+        for r in range(3):
+            rc, got = oracle.cpu_dot(qtype, blob[r * rb:(r + 1) * rb], x)
+            assert rc == 0 and np.float32(got).view(np.uint32) == np.float32(
+                make_golden.ref_dot(ref, qtype, blob[r * rb:(r + 1) * rb], x)).view(np.uint32)
+    # the reference refuses Q4_K on its CPU path (src/gguf/quant_compute.c:131-136)
+    out, failure, err = C.c_float(), (C.c_ubyte * 512)(), (C.c_ubyte * 512)()
+    q4 = oracle.Generator(1, "live.q4k").weights(oracle.Q4_K, 1, 256)
+    x = np.ones(256, np.float32)
+    ref.yvex_quant_cpu_dot.argtypes = [C.c_uint, C.c_void_p, C.c_size_t, C.c_void_p, C.c_ulonglong,
+                                       C.c_void_p, C.c_void_p, C.c_void_p]
+    assert ref.yvex_quant_cpu_dot(12, q4.ctypes.data, q4.size, x.ctypes.data, 256, C.byref(out),
+                                  failure, err) == oracle.ERR_UNSUPPORTED
+
+
+def test_cpu_dot_refusals(oracle):
+    g = oracle.Generator(3, "refusals")
+    row, x = g.weights(oracle.IQ2_XXS, 1, 512), g.normal(512)
+    assert oracle.cpu_dot(oracle.IQ2_XXS, row, x[:511])[0] == oracle.ERR_BOUNDS       # not block divisible
+    assert oracle.cpu_dot(oracle.IQ2_XXS, row[:-2], x)[0] == oracle.ERR_BOUNDS        # byte count
+    assert oracle.cpu_dot(13, row, x)[0] == oracle.ERR_UNSUPPORTED                    # Q5_K: no codec
+    bad = x.copy()
+    bad[3] = np.inf
+    assert oracle.cpu_dot(oracle.IQ2_XXS, row, bad)[0] == oracle.ERR_FORMAT
+
+
+# ---- Q4_K: not in the reference, pinned by the public format's structure ---------------------
+
+def q4k_pack_scales(sc, mn):
+    """The public ggml packer (quantize_row_q4_K): the inverse direction of get_scale_min_k4."""
+    scales = np.zeros(12, np.uint8)
+    for j in range(8):
+        if j < 4:
+            scales[j] |= sc[j]
+            scales[j + 4] |= mn[j]
+        else:
+            scales[j + 4] = (sc[j] & 0xF) | ((mn[j] & 0xF) << 4)
+            scales[j - 4] |= (sc[j] >> 4) << 6
+            scales[j] |= (mn[j] >> 4) << 6
+    return scales
+
+
+def q4k_block(d, dmin, sc, mn, values):
+    """values[256] in 0..15, element order as the format stores them."""
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.array([d], np.float16).view(np.uint8)
+    blk[2:4] = np.array([dmin], np.float16).view(np.uint8)
+    blk[4:16] = q4k_pack_scales(sc, mn)
+    v = np.asarray(values, np.uint8).reshape(4, 2, 32)          # chunk, low/high nibble, lane
+    blk[16:] = (v[:, 0, :] | (v[:, 1, :] << 4)).reshape(-1)
+    return blk
+
+
+def test_q4k_closed_forms(oracle):
+    rng = np.random.default_rng(0)
+    values = rng.integers(0, 16, 256)
+    # equal scales, zero mins: a plain 4-bit affine code in element order
+    dec = oracle.decode_rows(oracle.Q4_K, q4k_block(0.5, 0.0, [3] * 8, [0] * 8, values), 256)[0]
+    assert np.array_equal(dec, (1.5 * values).astype(np.float32))
+    # all nibbles zero: every value is -dmin * m of its sub-block
+    mn = [1, 5, 9, 13, 17, 33, 49, 63]
+    dec = oracle.decode_rows(oracle.Q4_K, q4k_block(1.0, 0.25, [7] * 8, mn, np.zeros(256)), 256)[0]
+    assert np.array_equal(dec.reshape(8, 32), np.repeat(-0.25 * np.array(mn, np.float32), 32).reshape(8, 32))
+    # 6-bit scales above 15 exercise the split high bits; sub-block j scales only its 32 values
+    sc = [1, 17, 33, 63, 16, 31, 47, 62]
+    dec = oracle.decode_rows(oracle.Q4_K, q4k_block(1.0, 0.0, sc, [0] * 8, np.ones(256)), 256)[0]
+    assert np.array_equal(dec.reshape(8, 32)[:, 0], np.array(sc, np.float32))
+    # general case against float arithmetic spelt from the format description
+    sc, mn = rng.integers(0, 64, 8), rng.integers(0, 64, 8)
+    d, dmin = np.float32(np.float16(0.0123)), np.float32(np.float16(0.0071))
+    dec = oracle.decode_rows(oracle.Q4_K, q4k_block(d, dmin, sc, mn, values), 256)[0]
+    want = (d * sc.astype(np.float32)).repeat(32) * values.astype(np.float32) - \
+           (dmin * mn.astype(np.float32)).repeat(32)
+    assert np.array_equal(dec, want.astype(np.float32))
+    rc, dot = oracle.cpu_dot(oracle.Q4_K, q4k_block(d, dmin, sc, mn, values), np.ones(256, np.float32))
+    assert rc == 0 and abs(dot - want.astype(np.float64).sum()) < 1e-4
+
+
+# ---- Q8_K quantizer: closed forms (kernels.cu:436-489) ------------------------------------------
+
+def test_q8k_quantizer_closed_forms(oracle):
+    x = np.zeros((1, 512), np.float32)
+    x[0, 300] = -3.5
+    q = oracle.q8k_quantize(x).reshape(2, 292)
+    assert np.all(q[0] == 0)                                                # zero block: d = 0, q = 0
+    d = q[1, :4].view(np.float32)[0]
+    codes = q[1, 4:260].view(np.int8)
+    assert codes[300 - 256] == -127 and np.count_nonzero(codes) == 1       # the spike maps to -127
+    assert np.isclose(d * -127.0, -3.5, rtol=1e-6)
+    assert list(q[1, 260:].view(np.int16)) == [0, 0, -127] + [0] * 13
+    # exact |tie| with opposite signs: the first one sets the sign, d*q is the same either way
+    y = np.zeros((1, 256), np.float32)
+    y[0, 10], y[0, 200] = 7.25, -7.25
+    q = oracle.q8k_quantize(y)
+    assert q[4:260].view(np.int8)[10] == -127 and q[4:260].view(np.int8)[200] == 127
+    z = y.copy()
+    z[0, 10], z[0, 200] = -7.25, 7.25
+    assert np.array_equal(oracle.q8k_dequantize(q), -oracle.q8k_dequantize(oracle.q8k_quantize(z)))
+    # round to nearest even and the 16-wide sums on random data
+    g = oracle.Generator(9, "q8k")
+    r = g.normal(4 * 1024).reshape(4, 1024)
+    q = oracle.q8k_quantize(r).reshape(-1, 292)
+    for b, block in enumerate(r.reshape(-1, 256)):
+        d = q[b, :4].view(np.float32)[0]
+        m = block[np.argmax(np.abs(block))]
+        inv = np.float32(-127.0) / m
+        assert d == np.float32(1.0) / inv
+        want = np.clip(np.rint(inv * block), -128, 127).astype(np.int8)
+        assert np.array_equal(q[b, 4:260].view(np.int8), want)
+        assert np.array_equal(q[b, 260:].view(np.int16), want.reshape(16, 16).sum(axis=1, dtype=np.int16))
+    with pytest.raises(RuntimeError):
+        oracle.q8k_quantize(np.full((1, 256), np.nan, np.float32))
+
+
+# ---- integer block dots against the (reference-pinned) float decoders ---------------------------
+
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q8_0", "Q4_K", "Q2_K"])
+def test_integer_block_dots_from_decoded_values(oracle, qtype):
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(21, f"intdots.{qtype}")
+    rows, width = 3, 1024
+    w = g.weights(qt, rows, width)
+    act = oracle.q8k_quantize(g.normal(2 * width).reshape(2, width))
+    sums = oracle.block_dots_i32(qt, w, rows, width, act, 2)
+    a = act.reshape(2, -1, 292)[:, :, 4:260].view(np.int8).astype(np.int64)       # [in, block, 256]
+    da = act.reshape(2, -1, 292)[:, :, :4].copy().view(np.float32)[..., 0].astype(np.float64)
+    decoded = oracle.decode_rows(qt, w, width).astype(np.float64).reshape(rows, -1, 256)
+    if qtype == "IQ2_XXS":
+        d = np.array([oracle.lib().yvo_f16_decode(int(v)) for v in
+                      w.reshape(-1, 66)[:, :2].copy().view(np.uint16).ravel()]).reshape(rows, -1)
+        ints = np.rint(decoded / (0.125 * d[..., None])).astype(np.int64)   # (2s+1) * level * sign
+        want = np.einsum("rbk,ibk->irb", ints, a)
+        assert np.array_equal(sums[..., 0], want) and np.all(sums[..., 1] == 0)
+    elif qtype == "Q8_0":
+        q = w.reshape(rows, -1, 34)[:, :, 2:].view(np.int8).astype(np.int64)          # [rows, unit, 32]
+        want = np.einsum("ruk,iuk->iru", q, a.reshape(2, -1, 32))
+        assert np.array_equal(sums, want)
+    else:
+        # dot and min are not separable from one decode, but their float combination is
+        head = 0 if qtype == "Q4_K" else 80
+        nb = 144 if qtype == "Q4_K" else 84
+        dd = w.reshape(rows, -1, nb)[:, :, head:head + 4].copy().view(np.uint16)
+        f = np.vectorize(lambda v: oracle.lib().yvo_f16_decode(int(v)))
+        d, dmin = f(dd[..., 0]).astype(np.float64), f(dd[..., 1]).astype(np.float64)
+        got = da[:, None, :] * (d[None] * sums[..., 0] - dmin[None] * sums[..., 1])
+        want = np.einsum("rbk,ibk->irb", decoded, a * da[..., None])
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+# ---- routing and expert: tests/unit/runtime_moe.c:105-212 ----------------------------------------
+
+def score(v):
+    return math.sqrt(v + math.log1p(math.exp(-v)) if v > 0 else math.log1p(math.exp(v)))
+
+
+def test_router_reference_expectations(oracle):
+    logits = np.array([1.0, 2.0, 2.0, 0.0], np.float32)      # router rows dotted with input [1,0,0,0]
+    rc, sel, w, _ = oracle.moe_route(logits, [5.0, 0.0, 0.0, 0.0], 2, oracle.SQRT_SOFTPLUS, True, 1.5)
+    assert rc == 0 and list(sel) == [0, 1]                   # bias picks 0, the tie goes to ordinal 1
+    a, b = score(1.0), score(2.0)
+    assert abs(w[0] - a / (a + b) * 1.5) < 1e-6 and abs(w[1] - b / (a + b) * 1.5) < 1e-6
+    rc, sel, _, _ = oracle.moe_route(logits, [0.0] * 4, 2, oracle.SQRT_SOFTPLUS, True, 1.5)
+    assert list(sel) == [1, 2]
+
+
+def test_router_matches_reference_fixture(oracle, golden):
+    for r in range(golden["route_logits"].shape[0]):
+        rc, sel, w, _ = oracle.moe_route(golden["route_logits"][r], golden["route_bias"], 6,
+                                         oracle.SQRT_SOFTPLUS, True, 1.5)
+        assert rc == 0 and np.array_equal(sel, golden["route_selected"][r])
+        assert np.array_equal(bits(w), golden["route_weights_bits"][r])
+
+
+def test_sigmoid_scoring_closed_form(oracle):
+    g = oracle.Generator(5, "sigmoid")
+    logits = g.normal(256)
+    rc, sel, w, scores = oracle.moe_route(logits, None, 8, oracle.SIGMOID, True, 2.5)
+    assert rc == 0
+    assert np.allclose(scores, 1.0 / (1.0 + np.exp(-logits.astype(np.float64))), rtol=1e-6)
+    assert list(sel) == list(np.argsort(-logits, kind="stable")[:8])      # monotone: order of logits
+    assert abs(float(w.sum()) - 2.5) < 1e-6 and np.all(np.diff(w) <= 0)
+    rc, _, w, _ = oracle.moe_route(np.zeros(4, np.float32), None, 2, oracle.SIGMOID, False, 1.0)
+    assert list(w) == [0.5, 0.5]
+
+
+def bf16(oracle, v):
+    return oracle.lib().yvo_bf16_round(np.float32(v))
+
+
+def test_expert_exact_equality_case(oracle):
+    gate = np.array([1.0, 2.0, -1.0, 1.0], np.float32)
+    up = np.array([2.0, 0.0, 1.0, 3.0], np.float32)
+    down = np.array([1.0, 0.5, -0.25, 2.0], np.float32)
+    x = np.array([1.0, 2.0], np.float32)
+    mid = []
+    for r in range(2):
+        gv = float(gate[2 * r]) * 1.0 + float(gate[2 * r + 1]) * 2.0
+        uv = float(up[2 * r]) * 1.0 + float(up[2 * r + 1]) * 2.0
+        mid.append(bf16(oracle, np.float32((gv / (1.0 + math.exp(-gv))) * uv * 0.25)))
+    want = [bf16(oracle, down[0] * mid[0] + down[1] * mid[1]), bf16(oracle, down[2] * mid[0] + down[3] * mid[1])]
+    rc, out, got_mid, _ = oracle.moe_expert((0, 0, 0), gate.view(np.uint8), up.view(np.uint8),
+                                            down.view(np.uint8), 2, 2, x, 0.25)
+    assert rc == 0 and list(out) == want and list(got_mid) == mid
+
+
+@pytest.mark.parametrize("name,qtype,hidden,inter", [("iq2_xxs", 16, 256, 256), ("q8_0", 8, 128, 64)])
+def test_expert_matches_reference_fixture(oracle, golden, name, qtype, hidden, inter):
+    rc, out, mid, _ = oracle.moe_expert(
+        (qtype,) * 3, golden[f"expert_{name}_gate"], golden[f"expert_{name}_up"],
+        golden[f"expert_{name}_down"], hidden, inter, golden[f"expert_{name}_x"], 0.25)
+    assert rc == 0 and np.array_equal(bits(out), golden[f"expert_{name}_out_bits"])
+    if name == "iq2_xxs":
+        # the fixture drives gate/up beyond +-10: the clamp must have been active somewhere
+        g = oracle.matvec(qtype, golden[f"expert_{name}_gate"], inter, hidden, golden[f"expert_{name}_x"])[0]
+        assert np.any(np.abs(g) > 10.0)
+    assert np.all((bits(mid) & 0xffff) == 0) and np.all((bits(out) & 0xffff) == 0)
+
+
+def test_worklist_properties(oracle):
+    rng = np.random.default_rng(2)
+    rows, topk, experts = 40, 6, 64
+    sel = np.stack([rng.choice(experts, topk, replace=False) for _ in range(rows)])
+    w = rng.random((rows, topk), dtype=np.float32)
+    rc, wl = oracle.worklist_build(sel, w, topk, experts)
+    assert rc == 0
+    flat = sel.reshape(-1)
+    order = wl["source_pairs"].astype(np.int64)
+    assert np.array_equal(order, np.argsort(flat, kind="stable"))           # stable sort by expert
+    assert int(wl["bucket_populations"].sum()) == rows * topk
+    assert np.array_equal(wl["expert_ids"], np.unique(flat))
+    assert np.array_equal(wl["source_rows"], order // topk) and np.array_equal(wl["destination_rows"], order)
+    assert np.array_equal(wl["route_weights"], w.reshape(-1)[order])
+    bad = sel.copy()
+    bad[0, 0] = experts
+    assert oracle.worklist_build(bad, w, topk, experts)[0] == oracle.ERR_FORMAT
