@@ -83,6 +83,9 @@ def main() -> int:
     ap.add_argument("--act", choices=["q8k", "f32"], default="q8k")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=2)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain 1 GiB read kernel and a 256 MiB fill kernel, so a "
+                         "counter run of this command holds kernels of known HBM traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)",
@@ -121,6 +124,7 @@ def main() -> int:
         return 1
     unique = int(layer.worklist.counts[0].item())
     max_pop = int(layer.worklist.counts[1].item())
+    sweeps = int(layer.worklist.counts[3].item())
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -131,41 +135,58 @@ def main() -> int:
     weight_bytes = (unique + 1) * EXPERT_BYTES
     value = weight_bytes / (step_ms * 1e-3) / 1e9
 
-    # dominant kernel alone: the routed gate/up sweep (2/3 of the routed bytes)
+    # dominant kernel alone, launched exactly as in the step: the gate/up sweep over the routed
+    # experts hit plus the shared expert (2/3 of the step's weight bytes)
     pairs = ROWS * TOPK
     acts = layer.act_q8_rows if layer.act_q8 else x
 
     def up_only():
         K.moe_up(layer.routed, acts, layer.act_q8, layer.weights, layer.worklist, pairs, TOPK,
-                 EXPERTS, layer.limit, layer.intermediate_f32, layer.status)
+                 EXPERTS, layer.limit, layer.intermediate_f32, layer.status, shared=layer.shared,
+                 shared_rows=ROWS, shared_intermediate=layer.shared_mid)
 
     def down_only():
         mid = layer.intermediate_q8 if layer.act_q8 else layer.intermediate_f32
+        smid = layer.shared_mid_q8 if layer.act_q8 else layer.shared_mid
         K.moe_down(layer.routed, mid, layer.act_q8, layer.worklist, pairs, EXPERTS,
-                   layer.pair_outputs, layer.status)
+                   layer.pair_outputs, layer.status, shared=layer.shared, shared_rows=ROWS,
+                   shared_intermediate=smid, shared_outputs=layer.shared_out)
 
     up_ms = event_ms(torch, up_only, max(10, args.steps))
     down_ms = event_ms(torch, down_only, max(10, args.steps))
-    up_bytes = unique * 2 * 3_784_704
+    up_bytes = (unique + 1) * 2 * 3_784_704   # gate + up of every distinct routed expert and the shared one
     achieved = up_bytes / (up_ms * 1e-3) / 1e9
+
+    if args.calibrate:
+        import ctypes as C
+        span = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        from yvex_amd import load_library
+        lib = load_library()
+        for _ in range(3):
+            lib.yvex_hip_stream_read(C.c_void_p(span.data_ptr()), C.c_uint64(span.numel()),
+                                     C.c_void_p(sink.data_ptr()), stream)
+            lib.yvex_hip_fill_u32(C.c_void_p(span.data_ptr()), C.c_uint32(7), C.c_uint64(1 << 26), stream)
+        torch.cuda.synchronize()
 
     out = {
         "metric": "IQ2_XXS MoE decode weight GB/s", "value": round(value, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "int8 dot / f32 scale" if layer.act_q8 else "f32",
+        "vs_baseline": None, "dtype": "i8" if layer.act_q8 else "f32",
         "data": "synthetic",
         "config": {"workload": "moe_decode_iq2xxs: hidden 7168, 256 routed + 1 shared experts, "
                                "top-8 sigmoid, expert width 2048, 32 rows",
                    "activations": args.act, "distinct_routed_experts": unique,
-                   "max_bucket_population": max_pop, "weight_bytes_per_step": weight_bytes},
+                   "max_bucket_population": max_pop, "routed_sweeps": sweeps, "weight_bytes_per_step": weight_bytes},
         "hbm_peak_frac": round(value / HBM_PEAK_GBS, 4),
         "tokens_per_s": round(ROWS / (step_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "kernel": "grouped_kernel<IQ2_XXS> gate/up sweep",
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "launch_ms": round(up_ms, 4), "algorithmic_bytes": up_bytes},
-        "kernels_ms": {"routed_up": round(up_ms, 4), "routed_down": round(down_ms, 4)},
+        "kernels_ms": {"gate_up_sweep": round(up_ms, 4), "down_sweep": round(down_ms, 4)},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_rows, 1)

@@ -490,23 +490,33 @@ __global__ __launch_bounds__(kGroupedThreads) void grouped_kernel(GroupedArgs a)
             ? ((unsigned long long)tiles * a.problem[1].sweeps) % wave_count : 0ull;
         unsigned long long item = (wave_id + wave_count - shift) % wave_count;
         for (; item < items; item += wave_count) {
-            const unsigned long long sweep = item / tiles;
-            const unsigned tile = (unsigned)(item % tiles);
-            unsigned long long expert = 0ull, first = 0ull, population = pr.pairs, pass = sweep * kPass;
+            // Items of one bucket are contiguous and, inside a bucket, the sweeps over one tile
+            // are neighbours: neighbouring waves stream the same bytes at the same time, so only
+            // the first of them goes to HBM.
+            unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
+            unsigned long long local = item, bucket_sweeps = sweeps;
             if (!fixed) {
-                // last bucket whose first sweep is <= sweep
+                // last bucket whose first item is <= item
                 unsigned long long low = 0ull, high = buckets;
                 while (low + 1ull < high) {
                     const unsigned long long middle = (low + high) >> 1;
-                    if (pr.sweep_offsets[middle] <= sweep) low = middle;
+                    if (pr.sweep_offsets[middle] * tiles <= item) low = middle;
                     else high = middle;
                 }
                 expert = pr.expert_ids[low];
                 first = pr.bucket_offsets[low];
                 population = pr.bucket_populations[low];
-                pass = (sweep - pr.sweep_offsets[low]) * kPass;
+                local = item - pr.sweep_offsets[low] * tiles;
+                bucket_sweeps = pr.sweep_offsets[low + 1ull] - pr.sweep_offsets[low];
             }
-            if (expert >= pr.experts || first + population > pr.pairs || pass >= population) {
+            if (bucket_sweeps == 0ull) {
+                if (lane == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            const unsigned tile = (unsigned)(local / bucket_sweeps);
+            const unsigned long long pass = (local % bucket_sweeps) * kPass;
+            if (expert >= pr.experts || first + population > pr.pairs || pass >= population ||
+                tile >= tiles) {
                 if (lane == 0u) raise_status(a.status, 2);
                 continue;
             }
