@@ -75,6 +75,56 @@ def cpu_baseline(sample_rows: int, threads: int):
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
 
 
+def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: int):
+    """BASELINE config 4: the same layer over 2048 rows whose top-8 experts follow a Zipf(1.1)
+    popularity (Gumbel top-k over log-popularity logits), row-batch kernels on the int8 matrix
+    cores. Ops counted: 2 * (2*I*H + H*I) per (row, expert) pair, routed and shared."""
+    rows = 2048
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4242)
+    rank = torch.randperm(EXPERTS, device=dev, generator=gen).float() + 1.0
+    popularity = rank.pow(-1.1)
+    uniform = torch.rand((rows, EXPERTS), device=dev, generator=gen).clamp_(1e-9, 1.0 - 1e-9)
+    logits = popularity.log()[None, :] - (-uniform.log()).log()
+    x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
+    qt = K.IQ2_XXS
+    layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                     qtypes=(qt, qt, qt), routed=weights, shared=shared, bias=None,
+                     scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0, act_q8=True,
+                     max_rows=rows, device=dev, matrix_cores=True)
+    for _ in range(warmup):
+        layer.run(x, logits)
+    torch.cuda.synchronize()
+    if int(layer.status.item()) != 0:
+        return {"error": f"device status {int(layer.status.item())}"}
+    step_ms = event_ms(torch, lambda: layer.run(x, logits), steps)
+    pairs = rows * TOPK
+    acts = layer.act_q8_rows
+    up_ms = event_ms(torch, lambda: K.moe_up_rows(
+        layer.routed, acts, layer.weights, layer.worklist, pairs, TOPK, EXPERTS, layer.limit,
+        layer.intermediate_f32, layer.status), steps)
+    down_ms = event_ms(torch, lambda: K.moe_down_rows(
+        layer.routed, layer.intermediate_q8, layer.worklist, pairs, EXPERTS, layer.pair_outputs,
+        layer.status), steps)
+    pair_ops = 2 * (2 * INTERMEDIATE * HIDDEN + HIDDEN * INTERMEDIATE)
+    routed_ops, shared_ops = pair_ops * pairs, pair_ops * rows
+    up_ops = 2 * 2 * INTERMEDIATE * HIDDEN * pairs
+    populations = layer.worklist.bucket_populations[: int(layer.worklist.counts[0].item())]
+    return {
+        "workload": "moe_prefill_iq2xxs: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, Q8_K activations",
+        "ms_per_step": round(step_ms, 4), "tokens_per_s": round(rows / (step_ms * 1e-3), 1),
+        "int8_TOPs": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12, 2),
+        "mfma_peak_frac": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
+        "distinct_routed_experts": int(populations.numel()),
+        "max_bucket_population": int(populations.max().item()),
+        "roofline": {"bound": "mfma", "kernel": "mfma_iq2_kernel<fused gate/up>",
+                     "achieved": round(up_ops / (up_ms * 1e-3) / 1e12, 2), "peak": MFMA_INT8_PEAK_TOPS,
+                     "unit": "TOP/s", "frac": round(up_ops / (up_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
+                     "launch_ms": round(up_ms, 4)},
+        "kernels_ms": {"gate_up_rows": round(up_ms, 4), "down_rows": round(down_ms, 4)},
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,6 +133,7 @@ def main() -> int:
     ap.add_argument("--act", choices=["q8k", "f32"], default="q8k")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=2)
+    ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 1 GiB read kernel and a 256 MiB fill kernel, so a "
                          "counter run of this command holds kernels of known HBM traffic")
@@ -188,6 +239,9 @@ def main() -> int:
                      "launch_ms": round(up_ms, 4), "algorithmic_bytes": up_bytes},
         "kernels_ms": {"gate_up_sweep": round(up_ms, 4), "down_sweep": round(down_ms, 4)},
     }
+    if not args.no_prefill:
+        out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
+                                     max(3, args.steps // 10), 2)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_rows, 1)
         out["cpu_baseline_all_cores"] = cpu_baseline(max(args.cpu_rows, 8), min(16, os.cpu_count() or 1))

@@ -129,6 +129,24 @@ int yvex_hip_moe_down(const yvex_hip_expert_weights *weights, const void *interm
                       uint64_t shared_rows, const void *shared_intermediate,
                       float *shared_outputs, int *status, yvex_hip_stream stream);
 
+/* Row-batch (prefill-width) forms of the two sweeps above on the int8 matrix cores; they replace
+ * yvex_moe_grouped_up_tensorcore / _down_tensorcore (tensorcore.cu:378-702). Same inputs,
+ * outputs and rounding points as yvex_hip_moe_up / yvex_hip_moe_down with act_q8 = 1; weights
+ * must be IQ2_XXS. A work item is 128 ordered pairs of one bucket times a tile of weight rows,
+ * so buckets of any population are served; expert_ids == NULL is the single-bucket form
+ * (shared expert: every pair uses expert 0, order may be NULL for the identity). */
+int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *weights, const void *act_q8k,
+                         const float *route_weights, const uint64_t *order,
+                         const uint64_t *expert_ids, const uint64_t *bucket_offsets,
+                         const uint64_t *bucket_populations, const uint64_t *counts,
+                         uint64_t pairs, uint64_t topk, uint64_t experts, double limit,
+                         float *intermediate, int *status, yvex_hip_stream stream);
+int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *weights, const void *intermediate_q8k,
+                           const uint64_t *order, const uint64_t *expert_ids,
+                           const uint64_t *bucket_offsets, const uint64_t *bucket_populations,
+                           const uint64_t *counts, uint64_t pairs, uint64_t experts,
+                           float *pair_outputs, int *status, yvex_hip_stream stream);
+
 /* Replaces yvex_moe_reduce_rows + yvex_moe_combine_rows (moe_kernels.cu:584-616):
  * routed[row, c] = sum over rank (in rank order, fp32) of pair_outputs[row*topk+rank, c];
  * combined[row, c] = bf16(routed + shared) when shared != NULL and combined != NULL. */

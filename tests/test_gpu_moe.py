@@ -27,7 +27,7 @@ def bf16_flip_report(got, want):
 
 
 def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype, act_q8, scoring,
-               seed=42, shared=True):
+               seed=42, shared=True, matrix_cores=False):
     from yvex_amd.moe import MoeLayer
     qt = getattr(oracle, qtype)
     g = oracle.Generator(seed, f"moe.{qtype}.{hidden}.{intermediate}.{experts}")
@@ -45,23 +45,28 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
                      qtypes=(qt, qt, qt), routed=tuple(dev(t, gpu) for t in (gate, up, down)),
                      shared=tuple(dev(t, gpu) for t in sh) if sh else None, bias=dev(bias, gpu),
                      scoring=scoring, normalize=True, scaling=1.5, limit=10.0, act_q8=act_q8,
-                     max_rows=rows, device=gpu)
+                     max_rows=rows, device=gpu, matrix_cores=matrix_cores)
     host = dict(qt=qt, gate=gate, up=up, down=down, shared=sh, x=x, logits=logits, bias=bias)
     return layer, host
 
 
-@pytest.mark.parametrize("qtype,hidden,intermediate,experts,topk,rows,act_q8,scoring", [
-    ("IQ2_XXS", 512, 256, 8, 2, 7, True, 0),
-    ("IQ2_XXS", 1024, 512, 16, 4, 9, False, 1),
-    ("Q4_K", 512, 512, 8, 3, 6, True, 1),
-    ("Q8_0", 512, 256, 6, 2, 5, True, 0),
-    ("Q2_K", 768, 256, 6, 2, 5, True, 0),
-    ("IQ2_XXS", 7168, 2048, 12, 4, 6, True, 1),
+@pytest.mark.parametrize("qtype,hidden,intermediate,experts,topk,rows,act_q8,scoring,matrix_cores", [
+    ("IQ2_XXS", 512, 256, 8, 2, 7, True, 0, False),
+    ("IQ2_XXS", 1024, 512, 16, 4, 9, False, 1, False),
+    ("Q4_K", 512, 512, 8, 3, 6, True, 1, False),
+    ("Q8_0", 512, 256, 6, 2, 5, True, 0, False),
+    ("Q2_K", 768, 256, 6, 2, 5, True, 0, False),
+    ("IQ2_XXS", 7168, 2048, 12, 4, 6, True, 1, False),
+    # row-batch kernels on the matrix cores: tiny buckets, buckets past one 128-pair tile, real widths
+    ("IQ2_XXS", 512, 256, 8, 2, 7, True, 0, True),
+    ("IQ2_XXS", 768, 512, 4, 2, 300, True, 1, True),
+    ("IQ2_XXS", 7168, 2048, 12, 4, 10, True, 1, True),
 ])
 def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, topk, rows, act_q8,
-                             scoring):
+                             scoring, matrix_cores):
     layer, h = make_layer(oracle, gpu, hidden=hidden, intermediate=intermediate, experts=experts,
-                          topk=topk, rows=rows, qtype=qtype, act_q8=act_q8, scoring=scoring)
+                          topk=topk, rows=rows, qtype=qtype, act_q8=act_q8, scoring=scoring,
+                          matrix_cores=matrix_cores)
     qt = h["qt"]
     combined = layer.run(dev(h["x"], gpu), dev(h["logits"], gpu)).cpu().numpy()
     torch.cuda.synchronize()
@@ -121,6 +126,8 @@ def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, 
     err = np.abs(combined.astype(np.float64) - full["combined"])
     bound = 1e-5 + 1e-3 * np.abs(full["combined"])
     outside = err > bound
-    # beyond the stated tolerance only where a bf16 rounding boundary was crossed upstream
+    # beyond the stated tolerance only where a bf16 rounding boundary was crossed upstream: a
+    # one-step flip of any of the summed terms, measured against the terms' own magnitude
     assert outside.mean() < 2e-2
-    assert np.all(err[outside] <= 2 * BF16_ULP * np.abs(full["combined"][outside]) + 1e-4)
+    terms = np.abs(pair_out.reshape(rows, topk, hidden)).sum(axis=1) + np.abs(shared)
+    assert np.all(err[outside] <= 2 * BF16_ULP * terms[outside] + 1e-4)

@@ -1,0 +1,517 @@
+// Row-batch (prefill-width) grouped expert projections on the int8 matrix cores of gfx950.
+//
+// A work item is (bucket, tile of 128 ordered pairs, tile of weight rows). The workgroup's eight
+// waves split the weight rows, 16 each (four gate blocks and the four matching up blocks when the
+// SwiGLU is fused); every wave multiplies its rows by the item's 128 Q8_K activation rows with
+// V_MFMA_I32_16X16X64_I8. Two waves share a SIMD, so one wave's decode and scaling arithmetic
+// runs under the other's matrix instructions.
+//
+//   A operand (weights): each lane decodes the 16 weights it owns straight into registers. The
+//       IQ2_XXS value of one weight is level * sign * (2s+1), up to 43 * 31 = 1333, so it is
+//       split into two int8 limbs, value = 128 * hi + lo with hi in [1, 11] and lo in
+//       [-120, 63]; both limbs come from one 16-byte LDS lookup keyed by (grid index, s), signs
+//       from a second lookup. Neither limb is ever zero, so negating a byte as (x ^ 0xff) + 1
+//       cannot carry into its neighbour.
+//   B operand (activations): the 128 x 256 int8 block of the current superblock, staged in LDS
+//       (double buffered, 272-byte row pitch: conflict-free 16-byte reads).
+//   C: per superblock two int32 accumulators per 16 x 16 block; T = 128 * C_hi + C_lo is the
+//       exact integer superblock sum of the reference's primitive
+//       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
+//       ((0.125 * d_w) * d_a) * T and summed over superblocks.
+//
+// Same inputs, outputs and rounding points as the decode-width sweeps in moe.hip
+// (src/backend/cuda/tensorcore.cu:378-702 is the reference's counterpart, unused there).
+#include "common.hpp"
+#include "launch.hpp"
+#include "grouped.hpp"
+
+namespace yvex {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr unsigned kMfmaThreads = 512u;
+constexpr unsigned kMfmaWaves = kMfmaThreads / 64u;
+constexpr unsigned kTileTokens = 128u;
+constexpr unsigned kTokenBlocks = kTileTokens / 16u;
+constexpr unsigned kActPitch = 272u;                       // 256 activation bytes + 16 bytes pad
+constexpr unsigned kLimbBase = 0u;                          // 4096 entries x 16 bytes
+constexpr unsigned kSignBase = 65536u;                      // 128 entries x 8 replicas x 16 bytes
+constexpr unsigned kSignReplicas = 8u;
+constexpr unsigned kStageBase = kSignBase + 128u * kSignReplicas * 16u;
+constexpr unsigned kStageActs = kTileTokens * kActPitch;
+constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per token
+constexpr unsigned kTileStartBase = kStageBase + 2u * kStageBytes;
+constexpr unsigned kMfmaLdsBytes = kTileStartBase + 260u * 4u;
+
+struct MfmaArgs {
+    GroupedProblem pr;
+    unsigned width;          // reduction width
+    unsigned out_rows;       // weight rows per expert
+    double limit;
+    int *status;
+};
+
+__device__ __forceinline__ void lds_write_uint4(unsigned address, uint4 v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) uint4 *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ void lds_write_u32(unsigned address, unsigned v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) unsigned *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ unsigned lds_read_u32(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const unsigned *>(address);
+#else
+    (void)address;
+    return 0u;
+#endif
+}
+
+// Limb pair of one magnitude byte: low limb in bits 0-7, high limb in bits 8-15.
+__device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
+{
+    const unsigned magnitude = level * factor;
+    unsigned hi = (magnitude + 64u) >> 7;
+    if (hi == 0u) hi = 1u;
+    const int lo = (int)magnitude - 128 * (int)hi;
+    return ((unsigned)lo & 255u) | (hi << 8);
+}
+
+__device__ __forceinline__ void mfma_tables_fill()
+{
+    for (unsigned index = threadIdx.x; index < 4096u; index += blockDim.x) {
+        const unsigned factor = 2u * (index >> 8) + 1u;
+        const uint2 m = iq2_magnitude_entry(index & 255u);
+        uint4 entry = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (unsigned l = 0; l < 4u; ++l) {
+            const unsigned a = iq2_limbs((m.x >> (8u * l)) & 255u, factor);
+            const unsigned b = iq2_limbs((m.y >> (8u * l)) & 255u, factor);
+            entry.x |= (a & 255u) << (8u * l);
+            entry.y |= (b & 255u) << (8u * l);
+            entry.z |= (a >> 8) << (8u * l);
+            entry.w |= (b >> 8) << (8u * l);
+        }
+        lds_write_uint4(kLimbBase + index * 16u, entry);
+    }
+    // sign entries: replica r of entry e at (e * 8 + r) * 16, a lane reads replica lane % 8, so
+    // the 16 lanes served together spread over all bank groups whatever entries they ask for
+    for (unsigned index = threadIdx.x; index < 128u * kSignReplicas; index += blockDim.x) {
+        const uint2 m = iq2_signmask_entry(index / kSignReplicas);
+        lds_write_uint4(kSignBase + index * 16u,
+                        make_uint4(m.x, m.y, m.x & 0x01010101u, m.y & 0x01010101u));
+    }
+}
+
+// What one work item needs to know about its place in the problem.
+struct MfmaItem {
+    unsigned long long expert, pair0;
+    unsigned tokens, row_tile;
+};
+
+// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8): every loop below has a fixed
+// trip count, so accumulators never leave registers and no branch sits between matrix
+// instructions.
+template <bool FUSED_UP, unsigned NB>
+__device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
+{
+    const GroupedProblem &pr = a.pr;
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const unsigned li = lane & 15u, kb = lane >> 4;
+    constexpr unsigned kItemRows = FUSED_UP ? 8u * kMfmaWaves : 16u * kMfmaWaves;
+    constexpr unsigned kStagedTokens = NB * 16u;
+    constexpr unsigned kChunks = (kStagedTokens * 16u + kMfmaThreads - 1u) / kMfmaThreads;
+    const unsigned sign_lane = kSignBase + (lane & (kSignReplicas - 1u)) * 16u;
+    const unsigned superblocks = a.width >> 8;
+
+    // ---- activation rows this thread stages: tokens (tid / 16) + 32 j ----
+    const unsigned char *stage_row[kChunks];
+#pragma unroll
+    for (unsigned j = 0; j < kChunks; ++j) {
+        const unsigned token = (tid >> 4) + 32u * j;
+        stage_row[j] = nullptr;
+        if (token < it.tokens) {
+            const unsigned long long ordered = it.pair0 + token;
+            const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+            const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
+            stage_row[j] = (const unsigned char *)pr.activations + arow * pr.act_stride;
+        }
+    }
+    const float *scale_row = nullptr;      // thread t < staged tokens carries token t's block scale
+    if (tid < kStagedTokens && tid < it.tokens) {
+        const unsigned long long ordered = it.pair0 + tid;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
+        scale_row = reinterpret_cast<const float *>((const unsigned char *)pr.activations +
+                                                    arow * pr.act_stride);
+    }
+    // ---- the weight row of this lane: the wave owns one 16-row block ----
+    const unsigned char *weight_row;
+    unsigned out_row_base;
+    if constexpr (FUSED_UP) {
+        out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
+        unsigned row = out_row_base + li;
+        if (row >= a.out_rows) row = a.out_rows - 1u;
+        weight_row = wave < 4u
+            ? pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes
+            : pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes;
+    } else {
+        out_row_base = it.row_tile * kItemRows + wave * 16u;
+        unsigned row = out_row_base + li;
+        if (row >= a.out_rows) row = a.out_rows - 1u;
+        weight_row = pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
+    }
+
+    float acc[NB][4];
+#pragma unroll
+    for (unsigned tb = 0; tb < NB; ++tb)
+#pragma unroll
+        for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
+
+    uint4 staged[kChunks];
+    float staged_scale = 0.0f;
+    uint2 codes[4];
+    unsigned scale16;
+    auto fetch = [&](unsigned sb) {
+#pragma unroll
+        for (unsigned j = 0; j < kChunks; ++j) {
+            staged[j] = make_uint4(0u, 0u, 0u, 0u);
+            if (stage_row[j])
+                __builtin_memcpy(&staged[j], stage_row[j] + (unsigned long long)sb * kQ8KBytes + 4u +
+                                                 16u * (tid & 15u), 16);
+        }
+        staged_scale = scale_row ? scale_row[(unsigned long long)sb * (kQ8KBytes / 4u)] : 0.0f;
+        const unsigned char *block = weight_row + (unsigned long long)sb * 66ull;
+        scale16 = load_u16(block);
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks)
+            codes[ks] = load_u32x2(block + 2u + 8u * (2u * ks + (kb >> 1)));
+    };
+    auto publish = [&](unsigned stage) {
+        const unsigned base = kStageBase + stage * kStageBytes;
+#pragma unroll
+        for (unsigned j = 0; j < kChunks; ++j) {
+            const unsigned token = (tid >> 4) + 32u * j;
+            if (token < kStagedTokens)
+                lds_write_uint4(base + token * kActPitch + 16u * (tid & 15u), staged[j]);
+        }
+        if (tid < kStagedTokens) lds_write_u32(base + kStageActs + 4u * tid, __float_as_uint(staged_scale));
+    };
+
+    __syncthreads();   // every wave is done with the previous item's stages
+    fetch(0u);
+    publish(0u);
+    uint2 now_codes[4];
+    unsigned now_scale16 = scale16;
+#pragma unroll
+    for (unsigned ks = 0; ks < 4u; ++ks) now_codes[ks] = codes[ks];
+    __syncthreads();
+
+    for (unsigned sb = 0; sb < superblocks; ++sb) {
+        const unsigned base = kStageBase + (sb & 1u) * kStageBytes;
+        if (sb + 1u < superblocks) fetch(sb + 1u);
+
+        v4i sum_lo[NB], sum_hi[NB];
+#pragma unroll
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            sum_lo[tb] = v4i{0, 0, 0, 0};
+            sum_hi[tb] = v4i{0, 0, 0, 0};
+        }
+        const unsigned frag_base = base + li * kActPitch + kb * 16u;
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks) {
+            const unsigned grids = now_codes[ks].x >> (16u * (kb & 1u));
+            const unsigned aux = now_codes[ks].y;
+            const unsigned signs = aux >> (14u * (kb & 1u));
+            const unsigned scale_bits = (aux >> 28) << 12;
+            const uint4 l0 = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
+            const uint4 l1 = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
+            const uint4 s0 = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
+            const uint4 s1 = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
+            const v4i a_lo = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
+                                 (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
+            const v4i a_hi = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
+                                 (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
+#pragma unroll
+            for (unsigned tb = 0; tb < NB; ++tb) {
+                const uint4 raw = lds_read_uint4(frag_base + tb * 16u * kActPitch + ks * 64u);
+                const v4i b = v4i{(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w};
+                sum_lo[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, sum_lo[tb], 0, 0, 0);
+                sum_hi[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, sum_hi[tb], 0, 0, 0);
+            }
+        }
+        // ---- exact superblock sums -> fp32 ----
+        float row_scale[4];
+        {
+            const float mine = 0.125f * f16_bits_to_float(now_scale16);
+#pragma unroll
+            for (unsigned r = 0; r < 4u; ++r) row_scale[r] = __shfl(mine, (int)(4u * kb + r), 64);
+        }
+#pragma unroll
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            const float token_scale =
+                __uint_as_float(lds_read_u32(base + kStageActs + 4u * (tb * 16u + li)));
+#pragma unroll
+            for (unsigned r = 0; r < 4u; ++r) {
+                const int total = (sum_hi[tb][r] << 7) + sum_lo[tb][r];
+                acc[tb][r] = __builtin_fmaf(row_scale[r] * token_scale, (float)total, acc[tb][r]);
+            }
+        }
+        if (sb + 1u < superblocks) {
+            publish((sb & 1u) ^ 1u);
+            now_scale16 = scale16;
+#pragma unroll
+            for (unsigned ks = 0; ks < 4u; ++ks) now_codes[ks] = codes[ks];
+        }
+        __syncthreads();
+    }
+
+    // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
+    auto store4 = [&](unsigned token, const float (&value)[4]) {
+        const unsigned long long ordered = it.pair0 + token;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
+        const unsigned row = out_row_base + 4u * kb;
+        const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
+                          finite_f32(value[3]);
+        if (!good) raise_status(a.status, 1);
+        else if (row + 3u < a.out_rows)
+            *reinterpret_cast<float4 *>(pr.out + out_index * a.out_rows + row) =
+                make_float4(value[0], value[1], value[2], value[3]);
+        else
+            for (unsigned r = 0; r < 4u; ++r)
+                if (row + r < a.out_rows) pr.out[out_index * a.out_rows + row + r] = value[r];
+    };
+    if constexpr (FUSED_UP) {
+        // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. They swap token
+        // blocks through LDS (the stages are free after the last barrier): gate waves finish
+        // blocks [0, G), up waves finish blocks [G, NB).
+        constexpr unsigned G = (NB + 1u) / 2u;
+        const bool is_gate = wave < 4u;
+        const unsigned slot = kStageBase + ((wave & 3u) * 2u + (is_gate ? 0u : 1u)) * 4096u;
+        const unsigned peer = kStageBase + ((wave & 3u) * 2u + (is_gate ? 1u : 0u)) * 4096u;
+        if (is_gate) {
+#pragma unroll
+            for (unsigned tb = G; tb < NB; ++tb)
+                lds_write_uint4(slot + ((tb - G) * 64u + lane) * 16u,
+                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
+                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
+        } else {
+#pragma unroll
+            for (unsigned tb = 0; tb < G; ++tb)
+                lds_write_uint4(slot + (tb * 64u + lane) * 16u,
+                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
+                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
+        }
+        __syncthreads();
+        if (is_gate) {
+#pragma unroll
+            for (unsigned tb = 0; tb < G; ++tb) {
+                const unsigned token = tb * 16u + li;
+                const uint4 other = lds_read_uint4(peer + (tb * 64u + lane) * 16u);
+                if (token < it.tokens) {
+                    const unsigned long long source =
+                        pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
+                    const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
+                    const float value[4] = {
+                        swiglu_bf16(acc[tb][0], __uint_as_float(other.x), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][1], __uint_as_float(other.y), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][2], __uint_as_float(other.z), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][3], __uint_as_float(other.w), route_weight, a.limit)};
+                    store4(token, value);
+                }
+            }
+        } else {
+#pragma unroll
+            for (unsigned tb = G; tb < NB; ++tb) {
+                const unsigned token = tb * 16u + li;
+                const uint4 other = lds_read_uint4(peer + ((tb - G) * 64u + lane) * 16u);
+                if (token < it.tokens) {
+                    const unsigned long long source =
+                        pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
+                    const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
+                    const float value[4] = {
+                        swiglu_bf16(__uint_as_float(other.x), acc[tb][0], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.y), acc[tb][1], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.z), acc[tb][2], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.w), acc[tb][3], route_weight, a.limit)};
+                    store4(token, value);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            const unsigned token = tb * 16u + li;
+            if (token < it.tokens) {
+                const float value[4] = {bf16_round(acc[tb][0]), bf16_round(acc[tb][1]),
+                                        bf16_round(acc[tb][2]), bf16_round(acc[tb][3])};
+                store4(token, value);
+            }
+        }
+    }
+}
+
+template <bool FUSED_UP>
+__global__ __launch_bounds__(kMfmaThreads) void mfma_iq2_kernel(MfmaArgs a)
+{
+    extern __shared__ __align__(16) unsigned char mfma_lds[];
+    if (lds_address_of(mfma_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
+        if (threadIdx.x == 0u) raise_status(a.status, 2);
+        return;
+    }
+    const GroupedProblem &pr = a.pr;
+    const unsigned tid = threadIdx.x;
+    const bool fixed = pr.expert_ids == nullptr;
+    const unsigned buckets = fixed ? 1u : (unsigned)pr.counts[0];
+
+    mfma_tables_fill();
+    if (tid == 0u) {
+        // first 128-pair tile of every bucket
+        unsigned cursor = 0u;
+        for (unsigned b = 0; b < buckets && b < 256u; ++b) {
+            lds_write_u32(kTileStartBase + 4u * b, cursor);
+            const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[b];
+            cursor += (unsigned)((n + kTileTokens - 1u) / kTileTokens);
+        }
+        lds_write_u32(kTileStartBase + 4u * (buckets < 256u ? buckets : 256u), cursor);
+    }
+    __syncthreads();
+    if (buckets == 0u || buckets > 256u) {
+        if (tid == 0u && buckets > 256u) raise_status(a.status, 2);
+        return;
+    }
+
+    // weight rows (gate/up row pairs when fused) per work item
+    constexpr unsigned kItemRows = FUSED_UP ? 8u * kMfmaWaves : 16u * kMfmaWaves;
+    const unsigned row_tiles = (a.out_rows + kItemRows - 1u) / kItemRows;
+    const unsigned long long token_tiles = lds_read_u32(kTileStartBase + 4u * buckets);
+    const unsigned long long items = token_tiles * row_tiles;
+
+    for (unsigned long long item = blockIdx.x; item < items; item += gridDim.x) {
+        // ---- which bucket, row tile and token tile ----
+        unsigned low = 0u, high = buckets;
+        while (low + 1u < high) {
+            const unsigned middle = (low + high) >> 1;
+            if ((unsigned long long)lds_read_u32(kTileStartBase + 4u * middle) * row_tiles <= item)
+                low = middle;
+            else
+                high = middle;
+        }
+        const unsigned tile_first = lds_read_u32(kTileStartBase + 4u * low);
+        const unsigned bucket_tiles = lds_read_u32(kTileStartBase + 4u * (low + 1u)) - tile_first;
+        const unsigned long long local = item - (unsigned long long)tile_first * row_tiles;
+        const unsigned token_tile = bucket_tiles ? (unsigned)(local % bucket_tiles) : 0u;
+        const unsigned long long first = fixed ? 0ull : pr.bucket_offsets[low];
+        const unsigned long long population = fixed ? pr.pairs : pr.bucket_populations[low];
+        MfmaItem it;
+        it.expert = fixed ? 0ull : pr.expert_ids[low];
+        it.row_tile = bucket_tiles ? (unsigned)(local / bucket_tiles) : 0u;
+        if (!bucket_tiles || it.expert >= pr.experts || first + population > pr.pairs ||
+            (unsigned long long)token_tile * kTileTokens >= population || it.row_tile >= row_tiles) {
+            if (tid == 0u) raise_status(a.status, 2);
+            continue;
+        }
+        const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
+        it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
+        it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
+        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
+        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
+        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
+        else mfma_item<FUSED_UP, 8u>(a, it);
+    }
+}
+
+static int mfma_grid()
+{
+    static int units = 0;
+    if (!units) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return units;
+}
+
+template <bool FUSED_UP>
+static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
+{
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsBytes) != hipSuccess)
+            (void)hipGetLastError();
+        configured = true;
+    }
+    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), kMfmaThreads, kMfmaLdsBytes, stream>>>(a);
+    return check_launch("moe_rows_mfma");
+}
+
+}  // namespace yvex
+
+using namespace yvex;
+
+extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void *act_q8k,
+                                    const float *route_weights, const uint64_t *order,
+                                    const uint64_t *expert_ids, const uint64_t *bucket_offsets,
+                                    const uint64_t *bucket_populations, const uint64_t *counts,
+                                    uint64_t pairs, uint64_t topk, uint64_t experts, double limit,
+                                    float *intermediate, int *status, yvex_hip_stream stream)
+{
+    if (!w || !w->gate || !w->up || !act_q8k || !intermediate || !status || !pairs || !topk ||
+        !experts || !(limit > 0.0) || (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        return ST_INVALID_ARG;
+    if (w->gate_qtype != QT_IQ2_XXS || w->up_qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
+    if (rc) return rc;
+    if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
+    if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull || w->intermediate % 4u) return ST_BOUNDS;
+    MfmaArgs a{};
+    const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
+    fill_up_problem(a.pr, w, act_q8k, 1, route_weights, wl, pairs, topk, experts, intermediate);
+    a.width = (unsigned)w->hidden;
+    a.out_rows = (unsigned)w->intermediate;
+    a.limit = limit;
+    a.status = status;
+    return launch_mfma<true>(a, as_stream(stream));
+}
+
+extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const void *intermediate_q8k,
+                                      const uint64_t *order, const uint64_t *expert_ids,
+                                      const uint64_t *bucket_offsets,
+                                      const uint64_t *bucket_populations, const uint64_t *counts,
+                                      uint64_t pairs, uint64_t experts, float *pair_outputs,
+                                      int *status, yvex_hip_stream stream)
+{
+    if (!w || !w->down || !intermediate_q8k || !pair_outputs || !status || !pairs || !experts ||
+        (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
+        return ST_INVALID_ARG;
+    if (w->down_qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
+    if (rc) return rc;
+    if (pairs > 0xffffffffull || w->hidden > 0xffffffffull || w->hidden % 4u) return ST_BOUNDS;
+    MfmaArgs a{};
+    const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
+    fill_down_problem(a.pr, w, intermediate_q8k, 1, wl, pairs, experts, pair_outputs);
+    a.width = (unsigned)w->intermediate;
+    a.out_rows = (unsigned)w->hidden;
+    a.limit = 1.0;
+    a.status = status;
+    return launch_mfma<false>(a, as_stream(stream));
+}

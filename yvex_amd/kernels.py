@@ -184,6 +184,25 @@ def moe_down(w: ExpertWeights, intermediate, act_q8, wl, pairs, experts, pair_ou
           _ptr(shared_intermediate), _ptr(shared_outputs), _ptr(status), _stream())
 
 
+def moe_up_rows(w: ExpertWeights, act_q8k, route_weights, wl, pairs, topk, experts, limit,
+                intermediate, status):
+    """Matrix-core form of moe_up; wl None is the single-bucket (shared expert) form."""
+    ptrs = [C.c_void_p(0)] * 5 if wl is None else [
+        _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets), _ptr(wl.bucket_populations),
+        _ptr(wl.counts)]
+    _call("yvex_hip_moe_up_rows", C.byref(w), _ptr(act_q8k), _ptr(route_weights), *ptrs,
+          C.c_uint64(pairs), C.c_uint64(topk), C.c_uint64(experts), C.c_double(limit),
+          _ptr(intermediate), _ptr(status), _stream())
+
+
+def moe_down_rows(w: ExpertWeights, intermediate_q8k, wl, pairs, experts, pair_outputs, status):
+    ptrs = [C.c_void_p(0)] * 5 if wl is None else [
+        _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets), _ptr(wl.bucket_populations),
+        _ptr(wl.counts)]
+    _call("yvex_hip_moe_down_rows", C.byref(w), _ptr(intermediate_q8k), *ptrs, C.c_uint64(pairs),
+          C.c_uint64(experts), _ptr(pair_outputs), _ptr(status), _stream())
+
+
 def moe_reduce_combine(pair_outputs, rows, topk, hidden, shared, routed, combined, status):
     _call("yvex_hip_moe_reduce_combine", _ptr(pair_outputs), C.c_uint64(rows), C.c_uint64(topk),
           C.c_uint64(hidden), _ptr(shared), _ptr(routed), _ptr(combined), _ptr(status), _stream())

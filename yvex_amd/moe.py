@@ -16,7 +16,7 @@ from . import kernels as K
 class MoeLayer:
     def __init__(self, *, hidden, intermediate, experts, topk, qtypes, routed, shared=None,
                  bias=None, scoring=K.SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
-                 act_q8=True, max_rows=64, device="cuda"):
+                 act_q8=True, max_rows=64, device="cuda", matrix_cores=False):
         self.hidden, self.intermediate, self.experts, self.topk = hidden, intermediate, experts, topk
         self.qtypes, self.scoring, self.normalize = qtypes, scoring, normalize
         self.scaling, self.limit, self.act_q8 = scaling, limit, act_q8
@@ -42,6 +42,8 @@ class MoeLayer:
         self.selected = None
         self.weights = None
         self.merge_shared = True
+        # row-batch (prefill-width) kernels on the int8 matrix cores instead of the decode sweeps
+        self.matrix_cores = matrix_cores
 
     def run(self, rows_f32: torch.Tensor, logits: torch.Tensor):
         """Enqueue one batch; returns the combined rows (device tensor, not synchronised)."""
@@ -57,6 +59,8 @@ class MoeLayer:
         self.selected, self.weights = K.moe_route_rows(
             logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st)
         K.worklist_build(self.selected, self.experts, st, self.worklist)
+        if self.matrix_cores:
+            return self._run_rows(acts, rows, pairs)
         merged = self.shared is not None and self.merge_shared
         K.moe_up(self.routed, acts, self.act_q8, self.weights, self.worklist, pairs, self.topk,
                  self.experts, self.limit, self.intermediate_f32, st,
@@ -79,6 +83,23 @@ class MoeLayer:
                    shared_outputs=self.shared_out if merged else None)
         if self.shared is not None and not merged:
             K.moe_down(self.shared, smid, self.act_q8, None, rows, 1, self.shared_out, st)
+        K.moe_reduce_combine(self.pair_outputs, rows, self.topk, self.hidden, self.shared_out,
+                             self.routed_out, self.combined, st)
+        return self.combined[:rows]
+
+    def _run_rows(self, acts, rows, pairs):
+        if not self.act_q8:
+            raise ValueError("the matrix-core kernels take Q8_K activations")
+        st = self.status
+        K.moe_up_rows(self.routed, acts, self.weights, self.worklist, pairs, self.topk, self.experts,
+                      self.limit, self.intermediate_f32, st)
+        K.q8k_quantize(self.intermediate_f32[:pairs], st, self.intermediate_q8)
+        K.moe_down_rows(self.routed, self.intermediate_q8, self.worklist, pairs, self.experts,
+                        self.pair_outputs, st)
+        if self.shared is not None:
+            K.moe_up_rows(self.shared, acts, None, None, rows, 1, 1, self.limit, self.shared_mid, st)
+            K.q8k_quantize(self.shared_mid[:rows], st, self.shared_mid_q8)
+            K.moe_down_rows(self.shared, self.shared_mid_q8, None, rows, 1, self.shared_out, st)
         K.moe_reduce_combine(self.pair_outputs, rows, self.topk, self.hidden, self.shared_out,
                              self.routed_out, self.combined, st)
         return self.combined[:rows]
