@@ -12,8 +12,10 @@
 //       [-120, 63]; both limbs come from one 16-byte LDS lookup keyed by (grid index, s), signs
 //       from a second lookup. Neither limb is ever zero, so negating a byte as (x ^ 0xff) + 1
 //       cannot carry into its neighbour.
-//   B operand (activations): the 128 x 256 int8 block of the current superblock, staged in LDS
-//       (double buffered, 272-byte row pitch: conflict-free 16-byte reads).
+//   B operand (activations): the 128 x 256 int8 block of the current superblock, copied from
+//       global memory straight into LDS (GLOBAL_LOAD_LDS_DWORDX4, no registers in between),
+//       double buffered. 16-byte piece c of token t sits at piece position c ^ (t % 16), so the
+//       16 lanes that read one fragment column together hit 16 different bank groups.
 //   C: per superblock two int32 accumulators per 16 x 16 block; T = 128 * C_hi + C_lo is the
 //       exact integer superblock sum of the reference's primitive
 //       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
@@ -33,7 +35,7 @@ constexpr unsigned kMfmaThreads = 512u;
 constexpr unsigned kMfmaWaves = kMfmaThreads / 64u;
 constexpr unsigned kTileTokens = 128u;
 constexpr unsigned kTokenBlocks = kTileTokens / 16u;
-constexpr unsigned kActPitch = 272u;                       // 256 activation bytes + 16 bytes pad
+constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
 constexpr unsigned kLimbBase = 0u;                          // 4096 entries x 16 bytes
 constexpr unsigned kSignBase = 65536u;                      // 128 entries x 8 replicas x 16 bytes
 constexpr unsigned kSignReplicas = 8u;
@@ -76,6 +78,32 @@ __device__ __forceinline__ unsigned lds_read_u32(unsigned address)
 #else
     (void)address;
     return 0u;
+#endif
+}
+
+// Asynchronous copy global -> LDS (GLOBAL_LOAD_LDS): lane l of the wave writes `bytes` bytes at
+// lds_base + l * bytes; nothing passes through registers. Written as assembly so the compiler
+// does not put a conservative wait in front of every later LDS read: the caller waits with
+// vmcnt(0) (loads retire in order, so the compiler's own counted waits stay correct) before
+// the barrier that publishes the data.
+__device__ __forceinline__ void copy_to_lds_16(const void *global, unsigned lds_base)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(lds_base), "v"(global) : "memory");   // m0 is reserved: the compiler reloads it before any use of its own
+#else
+    (void)global;
+    (void)lds_base;
+#endif
+}
+__device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_base)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :: "s"(lds_base), "v"(global) : "memory");   // m0 is reserved: the compiler reloads it before any use of its own
+#else
+    (void)global;
+    (void)lds_base;
 #endif
 }
 
@@ -132,31 +160,28 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     const unsigned li = lane & 15u, kb = lane >> 4;
     constexpr unsigned kItemRows = FUSED_UP ? 8u * kMfmaWaves : 16u * kMfmaWaves;
     constexpr unsigned kStagedTokens = NB * 16u;
-    constexpr unsigned kChunks = (kStagedTokens * 16u + kMfmaThreads - 1u) / kMfmaThreads;
     const unsigned sign_lane = kSignBase + (lane & (kSignReplicas - 1u)) * 16u;
     const unsigned superblocks = a.width >> 8;
 
-    // ---- activation rows this thread stages: tokens (tid / 16) + 32 j ----
-    const unsigned char *stage_row[kChunks];
-#pragma unroll
-    for (unsigned j = 0; j < kChunks; ++j) {
-        const unsigned token = (tid >> 4) + 32u * j;
-        stage_row[j] = nullptr;
-        if (token < it.tokens) {
-            const unsigned long long ordered = it.pair0 + token;
-            const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
-            const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
-            stage_row[j] = (const unsigned char *)pr.activations + arow * pr.act_stride;
-        }
-    }
-    const float *scale_row = nullptr;      // thread t < staged tokens carries token t's block scale
-    if (tid < kStagedTokens && tid < it.tokens) {
-        const unsigned long long ordered = it.pair0 + tid;
+    // ---- activation rows this lane copies: wave w owns the 4-token groups w, w + 8, ... ----
+    // Lane l of a group moves piece position l % 16 of token 4 g + l / 16; LDS receives the
+    // wave's 64 pieces back to back, so the swizzle is applied on the global side.
+    constexpr unsigned kCopies = (kStagedTokens / 4u + kMfmaWaves - 1u) / kMfmaWaves;
+    auto token_row = [&](unsigned token) {
+        const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
+        const unsigned long long ordered = it.pair0 + live;
         const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
         const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
-        scale_row = reinterpret_cast<const float *>((const unsigned char *)pr.activations +
-                                                    arow * pr.act_stride);
+        return (const unsigned char *)pr.activations + arow * pr.act_stride;
+    };
+    const unsigned char *copy_from[kCopies];
+#pragma unroll
+    for (unsigned j = 0; j < kCopies; ++j) {
+        const unsigned token = 4u * (wave + kMfmaWaves * j) + (lane >> 4);
+        copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
     }
+    // waves 0 and 1 also copy the block scales of tokens 64 w + lane
+    const unsigned char *scale_from = token_row(64u * (wave & 1u) + lane);
     // ---- the weight row of this lane: the wave owns one 16-row block ----
     const unsigned char *weight_row;
     unsigned out_row_base;
@@ -180,39 +205,37 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 #pragma unroll
         for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
 
-    uint4 staged[kChunks];
-    float staged_scale = 0.0f;
     uint2 codes[4];
     unsigned scale16;
-    auto fetch = [&](unsigned sb) {
+    auto copy_activations = [&](unsigned sb, unsigned stage) {
+        const unsigned base = kStageBase + stage * kStageBytes;
 #pragma unroll
-        for (unsigned j = 0; j < kChunks; ++j) {
-            staged[j] = make_uint4(0u, 0u, 0u, 0u);
-            if (stage_row[j])
-                __builtin_memcpy(&staged[j], stage_row[j] + (unsigned long long)sb * kQ8KBytes + 4u +
-                                                 16u * (tid & 15u), 16);
+        for (unsigned j = 0; j < kCopies; ++j) {
+            const unsigned group = wave + kMfmaWaves * j;            // wave-uniform
+            if (group * 4u < kStagedTokens)
+                copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
+                               (unsigned)__builtin_amdgcn_readfirstlane((int)(base + group * 1024u)));
         }
-        staged_scale = scale_row ? scale_row[(unsigned long long)sb * (kQ8KBytes / 4u)] : 0.0f;
+        if (wave * 64u < kStagedTokens)
+            copy_to_lds_4(scale_from + (unsigned long long)sb * kQ8KBytes,
+                          (unsigned)__builtin_amdgcn_readfirstlane((int)(base + kStageActs + wave * 256u)));
+    };
+    auto fetch_codes = [&](unsigned sb) {
         const unsigned char *block = weight_row + (unsigned long long)sb * 66ull;
         scale16 = load_u16(block);
 #pragma unroll
         for (unsigned ks = 0; ks < 4u; ++ks)
             codes[ks] = load_u32x2(block + 2u + 8u * (2u * ks + (kb >> 1)));
     };
-    auto publish = [&](unsigned stage) {
-        const unsigned base = kStageBase + stage * kStageBytes;
+    // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of token 16 tb + li
+    unsigned piece[4];
 #pragma unroll
-        for (unsigned j = 0; j < kChunks; ++j) {
-            const unsigned token = (tid >> 4) + 32u * j;
-            if (token < kStagedTokens)
-                lds_write_uint4(base + token * kActPitch + 16u * (tid & 15u), staged[j]);
-        }
-        if (tid < kStagedTokens) lds_write_u32(base + kStageActs + 4u * tid, __float_as_uint(staged_scale));
-    };
+    for (unsigned ks = 0; ks < 4u; ++ks) piece[ks] = li * kActPitch + (((4u * ks + kb) ^ li) << 4);
 
     __syncthreads();   // every wave is done with the previous item's stages
-    fetch(0u);
-    publish(0u);
+    copy_activations(0u, 0u);
+    fetch_codes(0u);
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the copies above have landed in LDS
     uint2 now_codes[4];
     unsigned now_scale16 = scale16;
 #pragma unroll
@@ -221,7 +244,10 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 
     for (unsigned sb = 0; sb < superblocks; ++sb) {
         const unsigned base = kStageBase + (sb & 1u) * kStageBytes;
-        if (sb + 1u < superblocks) fetch(sb + 1u);
+        if (sb + 1u < superblocks) {
+            copy_activations(sb + 1u, (sb & 1u) ^ 1u);
+            fetch_codes(sb + 1u);
+        }
 
         v4i sum_lo[NB], sum_hi[NB];
 #pragma unroll
@@ -229,28 +255,58 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             sum_lo[tb] = v4i{0, 0, 0, 0};
             sum_hi[tb] = v4i{0, 0, 0, 0};
         }
-        const unsigned frag_base = base + li * kActPitch + kb * 16u;
-#pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) {
+        // Software pipeline over phases (K step, group of up to four token blocks): the
+        // activation fragments of the next phase and the table lookups of the next K step are
+        // requested before the current phase's matrix instructions are issued, so their LDS
+        // latency runs under those instructions.
+        constexpr unsigned kGroups = NB > 4u ? 2u : 1u;      // groups per K step
+        constexpr unsigned kGroupSize = NB / kGroups;
+        constexpr unsigned kPhases = 4u * kGroups;
+        uint4 looked[4];
+        auto lookup = [&](unsigned ks) {
             const unsigned grids = now_codes[ks].x >> (16u * (kb & 1u));
             const unsigned aux = now_codes[ks].y;
             const unsigned signs = aux >> (14u * (kb & 1u));
             const unsigned scale_bits = (aux >> 28) << 12;
-            const uint4 l0 = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
-            const uint4 l1 = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
-            const uint4 s0 = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
-            const uint4 s1 = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
-            const v4i a_lo = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
-                                 (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
-            const v4i a_hi = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
-                                 (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
+            looked[0] = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
+            looked[1] = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
+            looked[2] = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
+            looked[3] = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
+        };
+        v4i a_lo, a_hi;
+        auto weights_from_lookup = [&]() {
+            const uint4 l0 = looked[0], l1 = looked[1], s0 = looked[2], s1 = looked[3];
+            a_lo = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
+                       (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
+            a_hi = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
+                       (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
+        };
+        uint4 frags[2][kGroupSize];
+        auto request = [&](unsigned phase, uint4 (&into)[kGroupSize]) {
+            const unsigned ks = phase / kGroups, group = phase % kGroups;
 #pragma unroll
-            for (unsigned tb = 0; tb < NB; ++tb) {
-                const uint4 raw = lds_read_uint4(frag_base + tb * 16u * kActPitch + ks * 64u);
+            for (unsigned i = 0; i < kGroupSize; ++i)
+                into[i] = lds_read_uint4(base + piece[ks] + (group * kGroupSize + i) * 16u * kActPitch);
+        };
+        lookup(0u);
+        request(0u, frags[0]);
+        weights_from_lookup();
+#pragma unroll
+        for (unsigned phase = 0; phase < kPhases; ++phase) {
+            const unsigned ks = phase / kGroups, group = phase % kGroups;
+            if (phase + 1u < kPhases) request(phase + 1u, frags[(phase + 1u) & 1u]);
+            if (group == 0u && ks + 1u < 4u) lookup(ks + 1u);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (unsigned i = 0; i < kGroupSize; ++i) {
+                const unsigned tb = group * kGroupSize + i;
+                const uint4 raw = frags[phase & 1u][i];
                 const v4i b = v4i{(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w};
                 sum_lo[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, sum_lo[tb], 0, 0, 0);
                 sum_hi[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, sum_hi[tb], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (group == kGroups - 1u && ks + 1u < 4u) weights_from_lookup();
         }
         // ---- exact superblock sums -> fp32 ----
         float row_scale[4];
@@ -270,10 +326,10 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             }
         }
         if (sb + 1u < superblocks) {
-            publish((sb & 1u) ^ 1u);
             now_scale16 = scale16;
 #pragma unroll
             for (unsigned ks = 0; ks < 4u; ++ks) now_codes[ks] = codes[ks];
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the next stage is complete in LDS
         }
         __syncthreads();
     }
@@ -466,6 +522,7 @@ static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
 }  // namespace yvex
 
 using namespace yvex;
+
 
 extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void *act_q8k,
                                     const float *route_weights, const uint64_t *order,
