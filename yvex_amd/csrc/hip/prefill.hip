@@ -31,10 +31,7 @@ namespace yvex {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr unsigned kMfmaThreads = 512u;
-constexpr unsigned kMfmaWaves = kMfmaThreads / 64u;
 constexpr unsigned kTileTokens = 128u;
-constexpr unsigned kTokenBlocks = kTileTokens / 16u;
 constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
 constexpr unsigned kLimbBase = 0u;                          // 4096 entries x 16 bytes
 constexpr unsigned kSignBase = 65536u;                      // 128 entries x 8 replicas x 16 bytes
@@ -149,24 +146,27 @@ struct MfmaItem {
     unsigned tokens, row_tile;
 };
 
-// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8): every loop below has a fixed
-// trip count, so accumulators never leave registers and no branch sits between matrix
-// instructions.
-template <bool FUSED_UP, unsigned NB>
+// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8) for a workgroup whose waves own
+// RB 16-row blocks each (RB = 1: eight waves, two per SIMD; RB = 2: four waves, one per SIMD with
+// the whole register file, each activation fragment feeding twice as many matrix instructions).
+// Every loop below has a fixed trip count, so accumulators never leave registers and no branch
+// sits between matrix instructions.
+template <bool FUSED_UP, unsigned NB, unsigned RB>
 __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
+    constexpr unsigned kWaves = 8u / RB;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned li = lane & 15u, kb = lane >> 4;
-    constexpr unsigned kItemRows = FUSED_UP ? 8u * kMfmaWaves : 16u * kMfmaWaves;
+    constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
     constexpr unsigned kStagedTokens = NB * 16u;
     const unsigned sign_lane = kSignBase + (lane & (kSignReplicas - 1u)) * 16u;
     const unsigned superblocks = a.width >> 8;
 
-    // ---- activation rows this lane copies: wave w owns the 4-token groups w, w + 8, ... ----
+    // ---- activation rows this lane copies: wave w owns the 4-token groups w, w + kWaves, ... ----
     // Lane l of a group moves piece position l % 16 of token 4 g + l / 16; LDS receives the
     // wave's 64 pieces back to back, so the swizzle is applied on the global side.
-    constexpr unsigned kCopies = (kStagedTokens / 4u + kMfmaWaves - 1u) / kMfmaWaves;
+    constexpr unsigned kCopies = (kStagedTokens / 4u + kWaves - 1u) / kWaves;
     auto token_row = [&](unsigned token) {
         const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
         const unsigned long long ordered = it.pair0 + live;
@@ -177,55 +177,65 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     const unsigned char *copy_from[kCopies];
 #pragma unroll
     for (unsigned j = 0; j < kCopies; ++j) {
-        const unsigned token = 4u * (wave + kMfmaWaves * j) + (lane >> 4);
+        const unsigned token = 4u * (wave + kWaves * j) + (lane >> 4);
         copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
     }
     // waves 0 and 1 also copy the block scales of tokens 64 w + lane
     const unsigned char *scale_from = token_row(64u * (wave & 1u) + lane);
-    // ---- the weight row of this lane: the wave owns one 16-row block ----
-    const unsigned char *weight_row;
-    unsigned out_row_base;
-    if constexpr (FUSED_UP) {
-        out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
-        unsigned row = out_row_base + li;
+
+    // ---- the weight rows of this lane, one per row block ----
+    // fused: blocks are (gate, up) of the same 16 rows when RB = 2; with RB = 1 waves 0-3 hold
+    // gate blocks and waves 4-7 the matching up blocks
+    const unsigned char *weight_row[RB];
+    unsigned out_row_base[RB];
+#pragma unroll
+    for (unsigned rb = 0; rb < RB; ++rb) {
+        bool is_up = false;
+        if constexpr (FUSED_UP) {
+            out_row_base[rb] = it.row_tile * kItemRows + (wave & 3u) * 16u;
+            is_up = RB == 2u ? rb == 1u : wave >= 4u;
+        } else {
+            out_row_base[rb] = it.row_tile * kItemRows + (wave * RB + rb) * 16u;
+        }
+        unsigned row = out_row_base[rb] + li;
         if (row >= a.out_rows) row = a.out_rows - 1u;
-        weight_row = wave < 4u
-            ? pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes
-            : pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes;
-    } else {
-        out_row_base = it.row_tile * kItemRows + wave * 16u;
-        unsigned row = out_row_base + li;
-        if (row >= a.out_rows) row = a.out_rows - 1u;
-        weight_row = pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
+        weight_row[rb] = is_up
+            ? pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
+            : pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
     }
 
-    float acc[NB][4];
+    float acc[RB][NB][4];
 #pragma unroll
-    for (unsigned tb = 0; tb < NB; ++tb)
+    for (unsigned rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
+        for (unsigned tb = 0; tb < NB; ++tb)
+#pragma unroll
+            for (unsigned r = 0; r < 4u; ++r) acc[rb][tb][r] = 0.0f;
 
-    uint2 codes[4];
-    unsigned scale16;
+    uint2 codes[RB][4];
+    unsigned scale16[RB];
     auto copy_activations = [&](unsigned sb, unsigned stage) {
         const unsigned base = kStageBase + stage * kStageBytes;
 #pragma unroll
         for (unsigned j = 0; j < kCopies; ++j) {
-            const unsigned group = wave + kMfmaWaves * j;            // wave-uniform
+            const unsigned group = wave + kWaves * j;            // wave-uniform
             if (group * 4u < kStagedTokens)
                 copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
                                (unsigned)__builtin_amdgcn_readfirstlane((int)(base + group * 1024u)));
         }
-        if (wave * 64u < kStagedTokens)
+        if (wave < 2u && wave * 64u < kStagedTokens)
             copy_to_lds_4(scale_from + (unsigned long long)sb * kQ8KBytes,
                           (unsigned)__builtin_amdgcn_readfirstlane((int)(base + kStageActs + wave * 256u)));
     };
     auto fetch_codes = [&](unsigned sb) {
-        const unsigned char *block = weight_row + (unsigned long long)sb * 66ull;
-        scale16 = load_u16(block);
 #pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks)
-            codes[ks] = load_u32x2(block + 2u + 8u * (2u * ks + (kb >> 1)));
+        for (unsigned rb = 0; rb < RB; ++rb) {
+            const unsigned char *block = weight_row[rb] + (unsigned long long)sb * 66ull;
+            scale16[rb] = load_u16(block);
+#pragma unroll
+            for (unsigned ks = 0; ks < 4u; ++ks)
+                codes[rb][ks] = load_u32x2(block + 2u + 8u * (2u * ks + (kb >> 1)));
+        }
     };
     // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of token 16 tb + li
     unsigned piece[4];
@@ -236,10 +246,14 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     copy_activations(0u, 0u);
     fetch_codes(0u);
     __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the copies above have landed in LDS
-    uint2 now_codes[4];
-    unsigned now_scale16 = scale16;
+    uint2 now_codes[RB][4];
+    unsigned now_scale16[RB];
 #pragma unroll
-    for (unsigned ks = 0; ks < 4u; ++ks) now_codes[ks] = codes[ks];
+    for (unsigned rb = 0; rb < RB; ++rb) {
+        now_scale16[rb] = scale16[rb];
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks) now_codes[rb][ks] = codes[rb][ks];
+    }
     __syncthreads();
 
     for (unsigned sb = 0; sb < superblocks; ++sb) {
@@ -249,12 +263,14 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             fetch_codes(sb + 1u);
         }
 
-        v4i sum_lo[NB], sum_hi[NB];
+        v4i sum_lo[RB][NB], sum_hi[RB][NB];
 #pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            sum_lo[tb] = v4i{0, 0, 0, 0};
-            sum_hi[tb] = v4i{0, 0, 0, 0};
-        }
+        for (unsigned rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (unsigned tb = 0; tb < NB; ++tb) {
+                sum_lo[rb][tb] = v4i{0, 0, 0, 0};
+                sum_hi[rb][tb] = v4i{0, 0, 0, 0};
+            }
         // Software pipeline over phases (K step, group of up to four token blocks): the
         // activation fragments of the next phase and the table lookups of the next K step are
         // requested before the current phase's matrix instructions are issued, so their LDS
@@ -262,24 +278,30 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         constexpr unsigned kGroups = NB > 4u ? 2u : 1u;      // groups per K step
         constexpr unsigned kGroupSize = NB / kGroups;
         constexpr unsigned kPhases = 4u * kGroups;
-        uint4 looked[4];
+        uint4 looked[RB][4];
         auto lookup = [&](unsigned ks) {
-            const unsigned grids = now_codes[ks].x >> (16u * (kb & 1u));
-            const unsigned aux = now_codes[ks].y;
-            const unsigned signs = aux >> (14u * (kb & 1u));
-            const unsigned scale_bits = (aux >> 28) << 12;
-            looked[0] = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
-            looked[1] = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
-            looked[2] = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
-            looked[3] = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
+#pragma unroll
+            for (unsigned rb = 0; rb < RB; ++rb) {
+                const unsigned grids = now_codes[rb][ks].x >> (16u * (kb & 1u));
+                const unsigned aux = now_codes[rb][ks].y;
+                const unsigned signs = aux >> (14u * (kb & 1u));
+                const unsigned scale_bits = (aux >> 28) << 12;
+                looked[rb][0] = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
+                looked[rb][1] = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
+                looked[rb][2] = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
+                looked[rb][3] = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
+            }
         };
-        v4i a_lo, a_hi;
+        v4i a_lo[RB], a_hi[RB];
         auto weights_from_lookup = [&]() {
-            const uint4 l0 = looked[0], l1 = looked[1], s0 = looked[2], s1 = looked[3];
-            a_lo = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
-                       (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
-            a_hi = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
-                       (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
+#pragma unroll
+            for (unsigned rb = 0; rb < RB; ++rb) {
+                const uint4 l0 = looked[rb][0], l1 = looked[rb][1], s0 = looked[rb][2], s1 = looked[rb][3];
+                a_lo[rb] = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
+                               (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
+                a_hi[rb] = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
+                               (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
+            }
         };
         uint4 frags[2][kGroupSize];
         auto request = [&](unsigned phase, uint4 (&into)[kGroupSize]) {
@@ -302,44 +324,53 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                 const unsigned tb = group * kGroupSize + i;
                 const uint4 raw = frags[phase & 1u][i];
                 const v4i b = v4i{(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w};
-                sum_lo[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, sum_lo[tb], 0, 0, 0);
-                sum_hi[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, sum_hi[tb], 0, 0, 0);
+#pragma unroll
+                for (unsigned rb = 0; rb < RB; ++rb) {
+                    sum_lo[rb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[rb], b, sum_lo[rb][tb], 0, 0, 0);
+                    sum_hi[rb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[rb], b, sum_hi[rb][tb], 0, 0, 0);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             if (group == kGroups - 1u && ks + 1u < 4u) weights_from_lookup();
         }
         // ---- exact superblock sums -> fp32 ----
-        float row_scale[4];
-        {
-            const float mine = 0.125f * f16_bits_to_float(now_scale16);
+        float row_scale[RB][4];
 #pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) row_scale[r] = __shfl(mine, (int)(4u * kb + r), 64);
+        for (unsigned rb = 0; rb < RB; ++rb) {
+            const float mine = 0.125f * f16_bits_to_float(now_scale16[rb]);
+#pragma unroll
+            for (unsigned r = 0; r < 4u; ++r) row_scale[rb][r] = __shfl(mine, (int)(4u * kb + r), 64);
         }
 #pragma unroll
         for (unsigned tb = 0; tb < NB; ++tb) {
             const float token_scale =
                 __uint_as_float(lds_read_u32(base + kStageActs + 4u * (tb * 16u + li)));
 #pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) {
-                const int total = (sum_hi[tb][r] << 7) + sum_lo[tb][r];
-                acc[tb][r] = __builtin_fmaf(row_scale[r] * token_scale, (float)total, acc[tb][r]);
-            }
+            for (unsigned rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (unsigned r = 0; r < 4u; ++r) {
+                    const int total = (sum_hi[rb][tb][r] << 7) + sum_lo[rb][tb][r];
+                    acc[rb][tb][r] = __builtin_fmaf(row_scale[rb][r] * token_scale, (float)total,
+                                                    acc[rb][tb][r]);
+                }
         }
         if (sb + 1u < superblocks) {
-            now_scale16 = scale16;
 #pragma unroll
-            for (unsigned ks = 0; ks < 4u; ++ks) now_codes[ks] = codes[ks];
+            for (unsigned rb = 0; rb < RB; ++rb) {
+                now_scale16[rb] = scale16[rb];
+#pragma unroll
+                for (unsigned ks = 0; ks < 4u; ++ks) now_codes[rb][ks] = codes[rb][ks];
+            }
             __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the next stage is complete in LDS
         }
         __syncthreads();
     }
 
-    // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
-    auto store4 = [&](unsigned token, const float (&value)[4]) {
+    // ---- publish: the lane holds C rows 4 kb + r of its blocks for tokens tb * 16 + li ----
+    auto store4 = [&](unsigned token, unsigned row, const float (&value)[4]) {
         const unsigned long long ordered = it.pair0 + token;
         const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
         const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
-        const unsigned row = out_row_base + 4u * kb;
         const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
                           finite_f32(value[3]);
         if (!good) raise_status(a.status, 1);
@@ -350,7 +381,24 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             for (unsigned r = 0; r < 4u; ++r)
                 if (row + r < a.out_rows) pr.out[out_index * a.out_rows + row + r] = value[r];
     };
-    if constexpr (FUSED_UP) {
+    auto route_weight_of = [&](unsigned token) {
+        const unsigned long long source = pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
+        return pr.route_weights ? pr.route_weights[source] : 1.0f;
+    };
+    if constexpr (FUSED_UP && RB == 2u) {
+#pragma unroll
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            const unsigned token = tb * 16u + li;
+            if (token < it.tokens) {
+                const float route_weight = route_weight_of(token);
+                const float value[4] = {swiglu_bf16(acc[0][tb][0], acc[RB - 1u][tb][0], route_weight, a.limit),
+                                        swiglu_bf16(acc[0][tb][1], acc[RB - 1u][tb][1], route_weight, a.limit),
+                                        swiglu_bf16(acc[0][tb][2], acc[RB - 1u][tb][2], route_weight, a.limit),
+                                        swiglu_bf16(acc[0][tb][3], acc[RB - 1u][tb][3], route_weight, a.limit)};
+                store4(token, out_row_base[0] + 4u * kb, value);
+            }
+        }
+    } else if constexpr (FUSED_UP) {
         // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. They swap token
         // blocks through LDS (the stages are free after the last barrier): gate waves finish
         // blocks [0, G), up waves finish blocks [G, NB).
@@ -362,14 +410,14 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 #pragma unroll
             for (unsigned tb = G; tb < NB; ++tb)
                 lds_write_uint4(slot + ((tb - G) * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
-                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
+                                make_uint4(__float_as_uint(acc[0][tb][0]), __float_as_uint(acc[0][tb][1]),
+                                           __float_as_uint(acc[0][tb][2]), __float_as_uint(acc[0][tb][3])));
         } else {
 #pragma unroll
             for (unsigned tb = 0; tb < G; ++tb)
                 lds_write_uint4(slot + (tb * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
-                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
+                                make_uint4(__float_as_uint(acc[0][tb][0]), __float_as_uint(acc[0][tb][1]),
+                                           __float_as_uint(acc[0][tb][2]), __float_as_uint(acc[0][tb][3])));
         }
         __syncthreads();
         if (is_gate) {
@@ -378,15 +426,13 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                 const unsigned token = tb * 16u + li;
                 const uint4 other = lds_read_uint4(peer + (tb * 64u + lane) * 16u);
                 if (token < it.tokens) {
-                    const unsigned long long source =
-                        pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
-                    const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
+                    const float route_weight = route_weight_of(token);
                     const float value[4] = {
-                        swiglu_bf16(acc[tb][0], __uint_as_float(other.x), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][1], __uint_as_float(other.y), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][2], __uint_as_float(other.z), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][3], __uint_as_float(other.w), route_weight, a.limit)};
-                    store4(token, value);
+                        swiglu_bf16(acc[0][tb][0], __uint_as_float(other.x), route_weight, a.limit),
+                        swiglu_bf16(acc[0][tb][1], __uint_as_float(other.y), route_weight, a.limit),
+                        swiglu_bf16(acc[0][tb][2], __uint_as_float(other.z), route_weight, a.limit),
+                        swiglu_bf16(acc[0][tb][3], __uint_as_float(other.w), route_weight, a.limit)};
+                    store4(token, out_row_base[0] + 4u * kb, value);
                 }
             }
         } else {
@@ -395,33 +441,34 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                 const unsigned token = tb * 16u + li;
                 const uint4 other = lds_read_uint4(peer + ((tb - G) * 64u + lane) * 16u);
                 if (token < it.tokens) {
-                    const unsigned long long source =
-                        pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
-                    const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
+                    const float route_weight = route_weight_of(token);
                     const float value[4] = {
-                        swiglu_bf16(__uint_as_float(other.x), acc[tb][0], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.y), acc[tb][1], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.z), acc[tb][2], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.w), acc[tb][3], route_weight, a.limit)};
-                    store4(token, value);
+                        swiglu_bf16(__uint_as_float(other.x), acc[0][tb][0], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.y), acc[0][tb][1], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.z), acc[0][tb][2], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.w), acc[0][tb][3], route_weight, a.limit)};
+                    store4(token, out_row_base[0] + 4u * kb, value);
                 }
             }
         }
     } else {
 #pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            const unsigned token = tb * 16u + li;
-            if (token < it.tokens) {
-                const float value[4] = {bf16_round(acc[tb][0]), bf16_round(acc[tb][1]),
-                                        bf16_round(acc[tb][2]), bf16_round(acc[tb][3])};
-                store4(token, value);
+        for (unsigned rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (unsigned tb = 0; tb < NB; ++tb) {
+                const unsigned token = tb * 16u + li;
+                if (token < it.tokens) {
+                    const float value[4] = {bf16_round(acc[rb][tb][0]), bf16_round(acc[rb][tb][1]),
+                                            bf16_round(acc[rb][tb][2]), bf16_round(acc[rb][tb][3])};
+                    store4(token, out_row_base[rb] + 4u * kb, value);
+                }
             }
-        }
     }
 }
 
-template <bool FUSED_UP>
-__global__ __launch_bounds__(kMfmaThreads) void mfma_iq2_kernel(MfmaArgs a)
+template <bool FUSED_UP, unsigned RB>
+__global__ __launch_bounds__(512u / RB) __attribute__((amdgpu_waves_per_eu(1, 3 - RB)))
+void mfma_iq2_kernel(MfmaArgs a)
 {
     extern __shared__ __align__(16) unsigned char mfma_lds[];
     if (lds_address_of(mfma_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
@@ -451,7 +498,7 @@ __global__ __launch_bounds__(kMfmaThreads) void mfma_iq2_kernel(MfmaArgs a)
     }
 
     // weight rows (gate/up row pairs when fused) per work item
-    constexpr unsigned kItemRows = FUSED_UP ? 8u * kMfmaWaves : 16u * kMfmaWaves;
+    constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
     const unsigned row_tiles = (a.out_rows + kItemRows - 1u) / kItemRows;
     const unsigned long long token_tiles = lds_read_u32(kTileStartBase + 4u * buckets);
     const unsigned long long items = token_tiles * row_tiles;
@@ -483,10 +530,10 @@ __global__ __launch_bounds__(kMfmaThreads) void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
-        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
-        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
-        else mfma_item<FUSED_UP, 8u>(a, it);
+        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u, RB>(a, it);
+        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u, RB>(a, it);
+        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u, RB>(a, it);
+        else mfma_item<FUSED_UP, 8u, RB>(a, it);
     }
 }
 
@@ -505,18 +552,37 @@ static int mfma_grid()
     return units;
 }
 
-template <bool FUSED_UP>
-static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
+// Row blocks per wave; see mfma_item. YVEX_MFMA_ROW_BLOCKS=1|2 in the environment overrides the
+// default for experiments.
+static unsigned mfma_row_blocks()
+{
+    static unsigned value = 0u;
+    if (!value) {
+        const char *text = getenv("YVEX_MFMA_ROW_BLOCKS");
+        value = (text && text[0] == '2') ? 2u : 1u;
+    }
+    return value;
+}
+
+template <bool FUSED_UP, unsigned RB>
+static int launch_mfma_rb(const MfmaArgs &a, hipStream_t stream)
 {
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP>,
+        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP, RB>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsBytes) != hipSuccess)
             (void)hipGetLastError();
         configured = true;
     }
-    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), kMfmaThreads, kMfmaLdsBytes, stream>>>(a);
+    mfma_iq2_kernel<FUSED_UP, RB><<<mfma_grid(), 512u / RB, kMfmaLdsBytes, stream>>>(a);
     return check_launch("moe_rows_mfma");
+}
+
+template <bool FUSED_UP>
+static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
+{
+    return mfma_row_blocks() == 2u ? launch_mfma_rb<FUSED_UP, 2u>(a, stream)
+                                   : launch_mfma_rb<FUSED_UP, 1u>(a, stream);
 }
 
 }  // namespace yvex
