@@ -57,6 +57,10 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
     ("Q8_0", 512, 256, 6, 2, 5, True, 0, False),
     ("Q2_K", 768, 256, 6, 2, 5, True, 0, False),
     ("IQ2_XXS", 7168, 2048, 12, 4, 6, True, 1, False),
+    # specialised IQ2_XXS sweeps: four rows per iteration with buckets past four pairs; two rows
+    # per iteration over a down projection whose rows end inside a 16-lane group
+    ("IQ2_XXS", 2048, 2048, 6, 4, 20, True, 1, False),
+    ("IQ2_XXS", 4096, 3072, 4, 2, 5, True, 0, False),
     # row-batch kernels on the matrix cores: tiny buckets, buckets past one 128-pair tile, real widths
     ("IQ2_XXS", 512, 256, 8, 2, 7, True, 0, True),
     ("IQ2_XXS", 768, 512, 4, 2, 300, True, 1, True),

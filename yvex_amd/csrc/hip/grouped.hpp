@@ -115,6 +115,11 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
     p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
 }
 
+// Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16
+// to 64 lanes of 128 columns each.
+bool iq2_sweep_supported(unsigned width);
+int launch_iq2_sweep(const GroupedArgs &a, bool fused, hipStream_t stream);
+
 static inline bool same_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)
 {
     return a->gate_qtype == b->gate_qtype && a->up_qtype == b->up_qtype &&

@@ -564,6 +564,13 @@ static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, hipStream_t
 static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool fused,
                             hipStream_t stream)
 {
+    static int generic_only = -1;   // YVEX_SWEEP_GENERIC=1 keeps the generic kernel (comparison runs)
+    if (generic_only < 0) {
+        const char *text = getenv("YVEX_SWEEP_GENERIC");
+        generic_only = text && text[0] == '1';
+    }
+    if (qtype == QT_IQ2_XXS && q8 && !generic_only && iq2_sweep_supported(a.width))
+        return launch_iq2_sweep(a, fused, stream);
     switch (qtype) {
     case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);
     case QT_Q4_K: return launch_grouped<QT_Q4_K>(a, q8, fused, stream);

@@ -1,0 +1,460 @@
+// Decode-width expert sweeps specialised for IQ2_XXS weights and Q8_K activations on gfx950.
+//
+// Same contract as the generic grouped kernel in moe.hip (src/backend/cuda/moe_kernels.cu:431-582
+// is the reference's counterpart), built around the instruction budget of this one format: at
+// 2.0625 bits per weight the vector ALU, not HBM, is the first limit, so every 32-weight unit is
+// decoded with as few vector instructions as the format allows.
+//
+//   * magnitudes: one 16-byte LDS read returns the eight level bytes of a codebook entry and their
+//     negations; signs: one 8-byte LDS read returns two byte-permute selectors for the 7 stored
+//     sign bits plus parity; V_PERM_B32 then picks +level or -level per byte. Four signed weights
+//     cost one vector instruction after the two reads.
+//   * a sweep serves up to four (row, rank) pairs of a bucket, whose Q8_K columns stay in
+//     registers (128 columns per lane), so an expert's bytes are decoded once for most buckets.
+//   * the exact int32 superblock sum (kernel_primitives.h:287-313) is formed in the lane pair
+//     that shares a superblock, scaled to fp32 as ((0.125 d_w) d_a) T, reduced over the 16 lanes
+//     of a row group with three data-parallel-primitive adds (gate on even lanes, up on odd
+//     lanes, or two pairs of the down projection), and parked in LDS; one pass at the end of the
+//     work item adds the row-group partials, applies the SwiGLU and stores coalesced rows.
+//
+// A work item is (bucket, tile of 16 row iterations, sweep). One workgroup per compute unit
+// stays resident and its waves walk the item list with a stride.
+#include "common.hpp"
+#include "launch.hpp"
+#include "grouped.hpp"
+
+namespace yvex {
+
+#ifndef YVEX_SWEEP_WAVES
+#define YVEX_SWEEP_WAVES 8
+#endif
+constexpr unsigned kSweepWaves = YVEX_SWEEP_WAVES;
+constexpr unsigned kSweepThreads = kSweepWaves * 64u;
+constexpr int kSweepPairs = 4;                 // pairs of one bucket served by one sweep
+constexpr unsigned kSweepIters = 16u;          // weight-row iterations per work item
+
+// LDS map (byte addresses; the dynamic block starts at LDS address 0)
+constexpr unsigned kMagBase = 0u;              // 256 entries x 16 replicas x {+lo, +hi, -lo, -hi}
+constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {selector lo, hi}
+constexpr unsigned kPrefixBase = kSelBase + 128u * 32u * 8u;   // 257 sweep starts, u32
+constexpr unsigned kParkBase = kPrefixBase + 1088u;
+constexpr unsigned kParkBytes = kSweepIters * kSweepPairs * 8u * 4u;   // per wave
+constexpr unsigned kSweepLdsBytes = kParkBase + kSweepWaves * kParkBytes;
+
+__device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) unsigned *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ void lds_store_uint2(unsigned address, uint2 v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) uint2 *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ void lds_store_uint4(unsigned address, uint4 v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) uint4 *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ unsigned lds_load_u32(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const unsigned *>(address);
+#else
+    (void)address;
+    return 0u;
+#endif
+}
+
+__device__ __forceinline__ void sweep_tables_fill()
+{
+    for (unsigned i = threadIdx.x; i < 256u * 16u; i += blockDim.x) {
+        const uint2 m = iq2_magnitude_entry(i >> 4);
+        // byte-wise negation: every level is >= 8, so (x ^ 0xff) + 1 never carries
+        lds_store_uint4(kMagBase + i * 16u,
+                        make_uint4(m.x, m.y, (m.x ^ 0xffffffffu) + 0x01010101u,
+                                   (m.y ^ 0xffffffffu) + 0x01010101u));
+    }
+    for (unsigned i = threadIdx.x; i < 128u * 32u; i += blockDim.x) {
+        const unsigned s7 = i >> 5;
+        const unsigned s = s7 | ((__popc(s7) & 1u) << 7);
+        // selector byte k = k (take +level, source 1) or k + 4 (take -level, source 0)
+        unsigned lo = 0x03020100u, hi = 0x03020100u;
+#pragma unroll
+        for (unsigned l = 0; l < 4u; ++l) {
+            if ((s >> l) & 1u) lo += 4u << (8u * l);
+            if ((s >> (l + 4u)) & 1u) hi += 4u << (8u * l);
+        }
+        lds_store_uint2(kSelBase + i * 8u, make_uint2(lo, hi));
+    }
+}
+
+// A lane's share of one IQ2_XXS weight row: half a superblock, 32 packed bytes plus the scale.
+struct Iq2Half {
+    uint4 lo, hi;
+    unsigned d16;
+    __device__ __forceinline__ void load(const unsigned char *row, unsigned super, unsigned half)
+    {
+        const unsigned char *b = row + super * 66u;
+        d16 = load_u16(b);
+        __builtin_memcpy(&lo, b + 2u + 32u * half, 16);
+        __builtin_memcpy(&hi, b + 18u + 32u * half, 16);
+    }
+};
+
+struct SweepLane {
+    unsigned lanes_per_row, rows_per_iter;
+    unsigned sub, super, half;
+    bool live;
+    unsigned mag_lane;     // (lane % 16) * 16
+    unsigned sel_lane;     // kSelBase + (lane % 32) * 8
+    unsigned park;         // this wave's parking area
+    unsigned park_write;   // + (lane parity) * 16 + (lane / 16) * 4
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+// Exact integer sums of this lane's four units of one weight row against N activation rows.
+template <int N>
+__device__ __forceinline__ void iq2_half_dots(const Iq2Half &c, const SweepLane &g,
+                                              const unsigned (&act)[N][32], int (&total)[N])
+{
+    const unsigned q[8] = {c.lo.x, c.lo.y, c.lo.z, c.lo.w, c.hi.x, c.hi.y, c.hi.z, c.hi.w};
+#pragma unroll
+    for (int p = 0; p < N; ++p) total[p] = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const unsigned grids = q[2 * k], aux = q[2 * k + 1];
+        unsigned w[8];
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            // magnitude address = index byte j << 8 | replica offset
+            const unsigned ma = __builtin_amdgcn_perm(grids, g.mag_lane, 0x0c0c0400u + (j << 8));
+            // selector address = sign field j (7 bits at bit 7j) moved to bit 8 | replica offset
+            const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
+            const unsigned sa = (moved & 0x7f00u) | g.sel_lane;
+            const uint4 m = lds_read_uint4(ma);
+            const uint2 s = lds_read_uint2(sa);
+            w[2 * j] = __builtin_amdgcn_perm(m.z, m.x, s.x);
+            w[2 * j + 1] = __builtin_amdgcn_perm(m.w, m.y, s.y);
+        }
+        const int factor = (int)((aux >> 27) | 1u);   // 2 s + 1: bit 27 is a sign bit, forced to 1
+#pragma unroll
+        for (int p = 0; p < N; ++p) {
+            int d = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = dot4(w[i], act[p][8 * k + i], d);
+            total[p] += __mul24(d, factor);   // |d| <= 32 * 43 * 128 < 2^23
+        }
+    }
+}
+
+// One sweep over the item's weight rows [row_begin, row_end) for N live pairs.
+template <bool FUSED, int N>
+__device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedProblem &pr,
+                                          const SweepLane &g, const unsigned char *gate_e,
+                                          const unsigned char *up_e, unsigned long long first_ordered,
+                                          unsigned row_begin, unsigned row_end)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const bool odd = (lane & 1u) != 0u;
+    // packed values per iteration: (gate, up) of pair v when fused, else pairs (2v, 2v + 1)
+    constexpr int PV = FUSED ? N : (N + 1) / 2;
+
+    // ---- the sweep's activation rows: this lane's 128 columns stay in registers ----
+    unsigned act[N][32];
+    float act_scale[N];
+    float route_weight[N];
+    unsigned long long out_index[N];
+#pragma unroll
+    for (int p = 0; p < N; ++p) {
+        const unsigned long long ordered = first_ordered + p;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
+        route_weight[p] = pr.route_weights ? pr.route_weights[source] : 1.0f;
+        out_index[p] = pr.out_by_source_pair ? source : ordered;
+        const unsigned char *blk = (const unsigned char *)pr.activations + arow * pr.act_stride +
+                                   (unsigned long long)(g.live ? g.super : 0u) * kQ8KBytes;
+        // lanes past the last row group multiply zeros
+        act_scale[p] = g.live ? *reinterpret_cast<const float *>(blk) : 0.0f;
+        const unsigned char *qv = blk + 4u + 128u * g.half;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            uint4 v;
+            __builtin_memcpy(&v, qv + 16 * k, 16);
+            act[p][4 * k] = g.live ? v.x : 0u;
+            act[p][4 * k + 1] = g.live ? v.y : 0u;
+            act[p][4 * k + 2] = g.live ? v.z : 0u;
+            act[p][4 * k + 3] = g.live ? v.w : 0u;
+        }
+    }
+    // the activation scale each lane applies to packed value v
+    float packed_scale[PV];
+#pragma unroll
+    for (int v = 0; v < PV; ++v) {
+        if constexpr (FUSED) packed_scale[v] = act_scale[v];
+        else packed_scale[v] = odd ? (2 * v + 1 < N ? act_scale[2 * v + 1 < N ? 2 * v + 1 : 0] : 0.0f)
+                                   : act_scale[2 * v];
+    }
+
+    const unsigned rows = row_end - row_begin;
+    const unsigned iterations = (rows + g.rows_per_iter - 1u) / g.rows_per_iter;   // <= kSweepIters
+    auto row_pointer = [&](const unsigned char *base, unsigned long long row_bytes, unsigned it) {
+        unsigned local = it * g.rows_per_iter + (g.live ? g.sub : 0u);
+        if (local >= rows) local = 0u;
+        return base + (unsigned long long)(row_begin + local) * row_bytes;
+    };
+    Iq2Half next_gate, next_up;
+    next_gate.load(row_pointer(gate_e, pr.row_bytes, 0u), g.live ? g.super : 0u, g.half);
+    if constexpr (FUSED) next_up.load(row_pointer(up_e, pr.up_row_bytes, 0u), g.live ? g.super : 0u, g.half);
+
+    for (unsigned it = 0; it < iterations; ++it) {
+        const Iq2Half gate = next_gate;
+        Iq2Half up;
+        if constexpr (FUSED) up = next_up;
+        if (it + 1u < iterations) {
+            next_gate.load(row_pointer(gate_e, pr.row_bytes, it + 1u), g.live ? g.super : 0u, g.half);
+            if constexpr (FUSED)
+                next_up.load(row_pointer(up_e, pr.up_row_bytes, it + 1u), g.live ? g.super : 0u, g.half);
+        }
+        int total_gate[N], total_up[N];
+        iq2_half_dots<N>(gate, g, act, total_gate);
+        if constexpr (FUSED) iq2_half_dots<N>(up, g, act, total_up);
+        // the two lanes of a superblock add their halves: exact int32 superblock sums
+#pragma unroll
+        for (int p = 0; p < N; ++p) {
+            total_gate[p] += dpp_move<0xb1, 0xf>(total_gate[p]);
+            if constexpr (FUSED) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
+        }
+        float weight_scale;
+        if constexpr (FUSED) weight_scale = 0.125f * f16_bits_to_float(odd ? up.d16 : gate.d16);
+        else weight_scale = 0.125f * f16_bits_to_float(gate.d16);
+#pragma unroll
+        for (int v = 0; v < PV; ++v) {
+            int t;
+            if constexpr (FUSED) t = odd ? total_up[v] : total_gate[v];
+            else t = odd ? total_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : total_gate[2 * v];
+            float value = weight_scale * packed_scale[v] * (float)t;
+            value = dpp_add<0x4e>(value);     // lanes i and i ^ 2
+            value = dpp_add<0x124>(value);    // + lane i - 4 (row rotate)
+            value = dpp_add<0x128>(value);    // + lanes i - 8, i - 12: all lanes of this parity
+            if ((lane & 15u) < 2u)
+                lds_store_u32(g.park_write + (it * PV + (unsigned)v) * 32u, __float_as_uint(value));
+        }
+    }
+
+    // ---- finish the item: add the row-group partials, SwiGLU or bf16, coalesced stores ----
+    // LDS operations of one wave complete in order, so the partials above are visible here.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const unsigned groups_per_row = 4u / g.rows_per_iter;   // 16-lane groups a weight row spans
+    const unsigned outputs = rows * (unsigned)N;
+    for (unsigned o = lane; o < outputs; o += 64u) {
+        const unsigned p = o / rows, local = o % rows;      // consecutive lanes: consecutive rows
+        const unsigned it = local / g.rows_per_iter, sub = local % g.rows_per_iter;
+        const unsigned v = FUSED ? p : p >> 1, parity = FUSED ? 0u : p & 1u;
+        const unsigned address = g.park + ((it * PV + v) * 2u + parity) * 16u + sub * groups_per_row * 4u;
+        float first = 0.0f, second = 0.0f;
+        for (unsigned k = 0; k < groups_per_row; ++k) {
+            first += __uint_as_float(lds_load_u32(address + 4u * k));
+            if constexpr (FUSED) second += __uint_as_float(lds_load_u32(address + 16u + 4u * k));
+        }
+        float rw = route_weight[0];
+        unsigned long long oi = out_index[0];
+#pragma unroll
+        for (int q = 1; q < N; ++q)
+            if (p == (unsigned)q) {
+                rw = route_weight[q];
+                oi = out_index[q];
+            }
+        const float value = FUSED ? swiglu_bf16(first, second, rw, a.limit) : bf16_round(first);
+        if (!finite_f32(value)) raise_status(a.status, 1);
+        else pr.out[oi * a.out_rows + row_begin + local] = value;
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
+{
+    extern __shared__ __align__(16) unsigned char sweep_lds[];
+    if (lds_address_of(sweep_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
+        if (threadIdx.x == 0u) raise_status(a.status, 2);
+        return;
+    }
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    sweep_tables_fill();
+
+    // ---- sweep numbering of the routed buckets: exclusive prefix of ceil(population / 4) ----
+    const GroupedProblem &routed = a.problem[0];
+    const bool routed_fixed = routed.expert_ids == nullptr;
+    const unsigned buckets = routed_fixed ? 1u : (unsigned)routed.counts[0];
+    if (!routed_fixed && buckets > 256u) {
+        if (tid == 0u) raise_status(a.status, 2);
+        return;
+    }
+    if (!routed_fixed) {
+        // Hillis-Steele scan over 256 slots, two buffers
+        const unsigned scratch = kParkBase;   // the parking areas are free until the first item
+        unsigned mine = 0u;
+        if (tid < 256u) {
+            mine = tid < buckets
+                ? (unsigned)((routed.bucket_populations[tid] + kSweepPairs - 1u) / kSweepPairs) : 0u;
+            lds_store_u32(scratch + 4u * tid, mine);
+        }
+        __syncthreads();
+        unsigned from = scratch, to = scratch + 1024u;
+        for (unsigned step = 1u; step < 256u; step <<= 1) {
+            if (tid < 256u) {
+                unsigned v = lds_load_u32(from + 4u * tid);
+                if (tid >= step) v += lds_load_u32(from + 4u * (tid - step));
+                lds_store_u32(to + 4u * tid, v);
+            }
+            __syncthreads();
+            const unsigned t = from;
+            from = to;
+            to = t;
+        }
+        if (tid < 256u) lds_store_u32(kPrefixBase + 4u * (tid + 1u), lds_load_u32(from + 4u * tid));
+        if (tid == 0u) lds_store_u32(kPrefixBase, 0u);
+    }
+    __syncthreads();
+
+    const unsigned units = a.width >> 5;
+    SweepLane g;
+    g.lanes_per_row = units / 4u;                                  // 16 .. 64, checked on the host
+    g.rows_per_iter = (g.lanes_per_row % 16u) == 0u && 64u % g.lanes_per_row == 0u
+        ? 64u / g.lanes_per_row : 1u;
+    g.sub = lane / g.lanes_per_row;
+    const unsigned seg = lane % g.lanes_per_row;
+    g.live = g.sub < g.rows_per_iter;
+    g.super = seg >> 1;
+    g.half = seg & 1u;
+    g.mag_lane = (lane & 15u) * 16u;
+    g.sel_lane = kSelBase + (lane & 31u) * 8u;
+    g.park = kParkBase + wave * kParkBytes;
+    g.park_write = g.park + (lane & 1u) * 16u + (lane >> 4) * 4u;
+
+    const unsigned item_rows = kSweepIters * g.rows_per_iter;
+    const unsigned tiles = (a.out_rows + item_rows - 1u) / item_rows;
+    const unsigned long long wave_id = (unsigned long long)blockIdx.x * kSweepWaves + wave;
+    const unsigned long long wave_count = (unsigned long long)gridDim.x * kSweepWaves;
+
+    // The shared expert's items come first (their number is known at launch), then the routed
+    // buckets the device-built worklist reports.
+    unsigned long long shift = 0ull;
+    for (int which = (int)a.problems - 1; which >= 0; --which) {
+        const GroupedProblem &pr = a.problem[which];
+        const bool fixed = pr.expert_ids == nullptr;
+        const unsigned long long sweeps = fixed
+            ? (pr.pairs + kSweepPairs - 1u) / kSweepPairs
+            : (unsigned long long)lds_load_u32(kPrefixBase + 4u * buckets);
+        const unsigned long long items = sweeps * tiles;
+        // the second list starts where the first one ended, so no wave runs two short lists
+        unsigned long long item = (wave_id + wave_count - shift) % wave_count;
+        shift = (shift + items) % wave_count;
+        for (; item < items; item += wave_count) {
+            unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
+            unsigned long long local = item, bucket_sweeps = sweeps;
+            if (!fixed) {
+                unsigned low = 0u, high = buckets;   // last bucket whose first item is <= item
+                while (low + 1u < high) {
+                    const unsigned middle = (low + high) >> 1;
+                    if ((unsigned long long)lds_load_u32(kPrefixBase + 4u * middle) * tiles <= item) low = middle;
+                    else high = middle;
+                }
+                const unsigned start = lds_load_u32(kPrefixBase + 4u * low);
+                expert = pr.expert_ids[low];
+                first = pr.bucket_offsets[low];
+                population = pr.bucket_populations[low];
+                local = item - (unsigned long long)start * tiles;
+                bucket_sweeps = lds_load_u32(kPrefixBase + 4u * (low + 1u)) - start;
+            }
+            if (bucket_sweeps == 0ull) {
+                if (lane == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            // the sweeps over one tile are neighbours: they stream the same bytes at the same time
+            const unsigned local32 = (unsigned)local, sweeps32 = (unsigned)bucket_sweeps;
+            const unsigned tile = local32 / sweeps32;
+            const unsigned long long pass = (unsigned long long)(local32 % sweeps32) * kSweepPairs;
+            if (expert >= pr.experts || first + population > pr.pairs || pass >= population ||
+                tile >= tiles) {
+                if (lane == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            const unsigned char *gate_e = pr.gate + expert * pr.expert_bytes;
+            const unsigned char *up_e = FUSED ? pr.up + expert * pr.up_expert_bytes : nullptr;
+            const unsigned row_begin = tile * item_rows;
+            const unsigned row_end = row_begin + item_rows < a.out_rows ? row_begin + item_rows : a.out_rows;
+            const unsigned long long live = population - pass;
+            if (live >= 4ull)
+                iq2_sweep<FUSED, 4>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            else if (live == 3ull)
+                iq2_sweep<FUSED, 3>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            else if (live == 2ull)
+                iq2_sweep<FUSED, 2>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            else
+                iq2_sweep<FUSED, 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+        }
+    }
+}
+
+static int sweep_grid()
+{
+    static int units = 0;
+    if (!units) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return units;
+}
+
+bool iq2_sweep_supported(unsigned width)
+{
+    const unsigned lanes_per_row = width / 128u;
+    return width % 256u == 0u && lanes_per_row >= 16u && lanes_per_row <= 64u;
+}
+
+template <bool FUSED>
+static int launch_iq2_sweep_variant(const GroupedArgs &a, hipStream_t stream)
+{
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void *)iq2_sweep_kernel<FUSED>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSweepLdsBytes) != hipSuccess)
+            (void)hipGetLastError();
+        configured = true;
+    }
+    iq2_sweep_kernel<FUSED><<<sweep_grid(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
+    return check_launch("moe_sweep_iq2");
+}
+
+int launch_iq2_sweep(const GroupedArgs &a, bool fused, hipStream_t stream)
+{
+    return fused ? launch_iq2_sweep_variant<true>(a, stream) : launch_iq2_sweep_variant<false>(a, stream);
+}
+
+}  // namespace yvex
