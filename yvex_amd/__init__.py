@@ -11,7 +11,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libyvex_rocm.so")
+# YVEX_ROCM_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("YVEX_ROCM_LIB") or os.path.join(HERE, "libyvex_rocm.so")
 
 _lib = None
 

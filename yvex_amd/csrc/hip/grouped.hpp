@@ -24,6 +24,7 @@ struct GroupedProblem {
     float *out;                              // [ordered or source pair][out_rows]
     int out_by_source_pair;
     unsigned sweeps;                         // single known bucket: ceil(pairs / kPass), else 0
+    unsigned long long *tickets;             // counts + 4 of the worklist (ticket, finished) or null
 };
 
 struct GroupedArgs {
@@ -35,6 +36,29 @@ struct GroupedArgs {
     double limit;
     int *status;
 };
+
+// The same value from fp32 arithmetic when that provably rounds to the same bfloat16. For
+// |gate| <= 16 the fp32 result is within about 24 units in the last place of the exact one (the
+// rounded product gate * log2(e) and the rounded constant contribute up to 19 of them, exp2,
+// reciprocal, 1 + t and the multiplications the rest), so unless its low 16 bits sit within 64
+// of the rounding midpoint the two roundings agree. Otherwise, and for non-finite or vanishing
+// values, the double path decides.
+__device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weight, double limit);
+__device__ __forceinline__ float swiglu_bf16_fast(float g, float u, float route_weight,
+                                                  double limit, float limit_f32)
+{
+    const float gv = fminf(g, limit_f32);
+    const float uv = fmaxf(-limit_f32, fminf(u, limit_f32));
+    const float t = __builtin_amdgcn_exp2f(-fabsf(gv) * 1.44269504088896340736f);
+    const float r = __builtin_amdgcn_rcpf(1.0f + t);
+    const float silu = gv >= 0.0f ? gv * r : gv * t * r;
+    const float v = silu * uv * route_weight;
+    const unsigned bits = __float_as_uint(v), low = bits & 0xffffu;
+    const bool safe = (double)limit_f32 == limit && finite_f32(v) && fabsf(v) > 1.0e-30f &&
+                      fabsf(gv) <= 16.0f && (low < 0x8000u - 64u || low > 0x8000u + 64u);
+    if (safe) return bf16_round(v);
+    return swiglu_bf16(g, u, route_weight, limit);
+}
 
 // SiLU-gated product in double, as src/graph/moe.c:605-611 orders it.
 __device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weight, double limit)
@@ -86,6 +110,7 @@ static inline void fill_up_problem(GroupedProblem &p, const yvex_hip_expert_weig
     p.out = out;
     p.out_by_source_pair = 0;
     p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
+    p.tickets = wl.expert_ids && wl.counts ? (unsigned long long *)wl.counts + 4 : nullptr;
 }
 
 static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_weights *w,
@@ -113,6 +138,7 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
     p.out = out;
     p.out_by_source_pair = 1;
     p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
+    p.tickets = wl.expert_ids && wl.counts ? (unsigned long long *)wl.counts + 4 : nullptr;
 }
 
 // Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16

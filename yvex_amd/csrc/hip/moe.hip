@@ -162,6 +162,7 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
         counts[1] = maximum;
         counts[2] = cursor;
         counts[3] = sweeps;
+        counts[4] = counts[5] = counts[6] = counts[7] = 0ull;   // tickets of the expert kernels
         if (cursor != pairs) bad = 1u;
     }
     __syncthreads();

@@ -28,17 +28,24 @@ namespace yvex {
 #ifndef YVEX_SWEEP_WAVES
 #define YVEX_SWEEP_WAVES 8
 #endif
+#ifndef YVEX_SWEEP_ITERS
+#define YVEX_SWEEP_ITERS 32
+#endif
+#ifndef YVEX_SWEEP_PAIRS
+#define YVEX_SWEEP_PAIRS 4
+#endif
 constexpr unsigned kSweepWaves = YVEX_SWEEP_WAVES;
 constexpr unsigned kSweepThreads = kSweepWaves * 64u;
-constexpr int kSweepPairs = 4;                 // pairs of one bucket served by one sweep
-constexpr unsigned kSweepIters = 16u;          // weight-row iterations per work item
+constexpr int kSweepPairs = YVEX_SWEEP_PAIRS;  // pairs of one bucket served by one sweep (2..4)
+constexpr unsigned kSweepIters = YVEX_SWEEP_ITERS;          // weight-row iterations per work item
 
 // LDS map (byte addresses; the dynamic block starts at LDS address 0)
 constexpr unsigned kMagBase = 0u;              // 256 entries x 16 replicas x {+lo, +hi, -lo, -hi}
 constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {selector lo, hi}
 constexpr unsigned kPrefixBase = kSelBase + 128u * 32u * 8u;   // 257 sweep starts, u32
+constexpr unsigned kTicketAddress = kPrefixBase + 1056u;   // work-item counter of the workgroup
 constexpr unsigned kParkBase = kPrefixBase + 1088u;
-constexpr unsigned kParkBytes = kSweepIters * kSweepPairs * 8u * 4u;   // per wave
+constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u;   // per wave
 constexpr unsigned kSweepLdsBytes = kParkBase + kSweepWaves * kParkBytes;
 
 __device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
@@ -130,38 +137,68 @@ __device__ __forceinline__ float dpp_add(float v)
     return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
 
-// Exact integer sums of this lane's four units of one weight row against N activation rows.
-template <int N>
-__device__ __forceinline__ void iq2_half_dots(const Iq2Half &c, const SweepLane &g,
-                                              const unsigned (&act)[N][32], int (&total)[N])
+// Exact integer sums of this lane's four units of each of STREAMS weight rows against N
+// activation rows. The work is cut into stages of half a unit (two codebook lookups, two selector
+// lookups, sixteen weights); the LDS reads of stage s + DEPTH are issued before stage s is
+// consumed, so their latency runs under the permutes and dot products of the stages between.
+template <int STREAMS, int N>
+__device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const SweepLane &g,
+                                              const unsigned (&act)[N][32], int (&total)[STREAMS][N])
 {
-    const unsigned q[8] = {c.lo.x, c.lo.y, c.lo.z, c.lo.w, c.hi.x, c.hi.y, c.hi.z, c.hi.w};
+    constexpr int kStages = STREAMS * 8;
+    constexpr int DEPTH = N <= 2 ? 3 : 2;
+    unsigned q[STREAMS][8];
 #pragma unroll
-    for (int p = 0; p < N; ++p) total[p] = 0;
+    for (int w = 0; w < STREAMS; ++w) {
+        q[w][0] = c[w].lo.x; q[w][1] = c[w].lo.y; q[w][2] = c[w].lo.z; q[w][3] = c[w].lo.w;
+        q[w][4] = c[w].hi.x; q[w][5] = c[w].hi.y; q[w][6] = c[w].hi.z; q[w][7] = c[w].hi.w;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const unsigned grids = q[2 * k], aux = q[2 * k + 1];
-        unsigned w[8];
+        for (int p = 0; p < N; ++p) total[w][p] = 0;
+    }
+    uint4 mag[DEPTH + 1][2];
+    uint2 sel[DEPTH + 1][2];
+    auto issue = [&](int stage) {
+        const int w = stage >> 3, k = (stage >> 1) & 3, h = stage & 1, slot = stage % (DEPTH + 1);
+        const unsigned grids = q[w][2 * k], aux = q[w][2 * k + 1];
 #pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
+        for (int jj = 0; jj < 2; ++jj) {
+            const unsigned j = 2u * (unsigned)h + (unsigned)jj;
             // magnitude address = index byte j << 8 | replica offset
             const unsigned ma = __builtin_amdgcn_perm(grids, g.mag_lane, 0x0c0c0400u + (j << 8));
             // selector address = sign field j (7 bits at bit 7j) moved to bit 8 | replica offset
             const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
             const unsigned sa = (moved & 0x7f00u) | g.sel_lane;
-            const uint4 m = lds_read_uint4(ma);
-            const uint2 s = lds_read_uint2(sa);
-            w[2 * j] = __builtin_amdgcn_perm(m.z, m.x, s.x);
-            w[2 * j + 1] = __builtin_amdgcn_perm(m.w, m.y, s.y);
+            mag[slot][jj] = lds_read_uint4(ma);
+            sel[slot][jj] = lds_read_uint2(sa);
         }
-        const int factor = (int)((aux >> 27) | 1u);   // 2 s + 1: bit 27 is a sign bit, forced to 1
+    };
+#pragma unroll
+    for (int stage = 0; stage < DEPTH; ++stage) issue(stage);
+    int d[N];
+#pragma unroll
+    for (int stage = 0; stage < kStages; ++stage) {
+        if (stage + DEPTH < kStages) issue(stage + DEPTH);
+        __builtin_amdgcn_sched_barrier(0);
+        const int w = stage >> 3, k = (stage >> 1) & 3, h = stage & 1, slot = stage % (DEPTH + 1);
+        unsigned weights[4];
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            weights[2 * jj] = __builtin_amdgcn_perm(mag[slot][jj].z, mag[slot][jj].x, sel[slot][jj].x);
+            weights[2 * jj + 1] = __builtin_amdgcn_perm(mag[slot][jj].w, mag[slot][jj].y, sel[slot][jj].y);
+        }
 #pragma unroll
         for (int p = 0; p < N; ++p) {
-            int d = 0;
+            if (h == 0) d[p] = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) d = dot4(w[i], act[p][8 * k + i], d);
-            total[p] += __mul24(d, factor);   // |d| <= 32 * 43 * 128 < 2^23
+            for (int i = 0; i < 4; ++i) d[p] = dot4(weights[i], act[p][8 * k + 4 * h + i], d[p]);
         }
+        if (h == 1) {
+            // 2 s + 1: bit 27 of the word is a sign bit, forced to 1
+            const int factor = (int)((q[w][2 * k + 1] >> 27) | 1u);
+#pragma unroll
+            for (int p = 0; p < N; ++p) total[w][p] += __mul24(d[p], factor);   // |d| < 2^23
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -234,8 +271,22 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
                 next_up.load(row_pointer(up_e, pr.up_row_bytes, it + 1u), g.live ? g.super : 0u, g.half);
         }
         int total_gate[N], total_up[N];
-        iq2_half_dots<N>(gate, g, act, total_gate);
-        if constexpr (FUSED) iq2_half_dots<N>(up, g, act, total_up);
+        if constexpr (FUSED) {
+            const Iq2Half both[2] = {gate, up};
+            int totals[2][N];
+            iq2_half_dots<2, N>(both, g, act, totals);
+#pragma unroll
+            for (int p = 0; p < N; ++p) {
+                total_gate[p] = totals[0][p];
+                total_up[p] = totals[1][p];
+            }
+        } else {
+            const Iq2Half one[1] = {gate};
+            int totals[1][N];
+            iq2_half_dots<1, N>(one, g, act, totals);
+#pragma unroll
+            for (int p = 0; p < N; ++p) total_gate[p] = totals[0][p];
+        }
         // the two lanes of a superblock add their halves: exact int32 superblock sums
 #pragma unroll
         for (int p = 0; p < N; ++p) {
@@ -284,7 +335,8 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
                 rw = route_weight[q];
                 oi = out_index[q];
             }
-        const float value = FUSED ? swiglu_bf16(first, second, rw, a.limit) : bf16_round(first);
+        const float value = FUSED ? swiglu_bf16_fast(first, second, rw, a.limit, (float)a.limit)
+                                  : bf16_round(first);
         if (!finite_f32(value)) raise_status(a.status, 1);
         else pr.out[oi * a.out_rows + row_begin + local] = value;
     }
@@ -301,6 +353,7 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     }
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     sweep_tables_fill();
+    if (tid == 0u) lds_store_u32(kTicketAddress, 0u);
 
     // ---- sweep numbering of the routed buckets: exclusive prefix of ceil(population / 4) ----
     const GroupedProblem &routed = a.problem[0];
@@ -354,66 +407,72 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
 
     const unsigned item_rows = kSweepIters * g.rows_per_iter;
     const unsigned tiles = (a.out_rows + item_rows - 1u) / item_rows;
-    const unsigned long long wave_id = (unsigned long long)blockIdx.x * kSweepWaves + wave;
-    const unsigned long long wave_count = (unsigned long long)gridDim.x * kSweepWaves;
 
-    // The shared expert's items come first (their number is known at launch), then the routed
-    // buckets the device-built worklist reports.
-    unsigned long long shift = 0ull;
-    for (int which = (int)a.problems - 1; which >= 0; --which) {
-        const GroupedProblem &pr = a.problem[which];
-        const bool fixed = pr.expert_ids == nullptr;
-        const unsigned long long sweeps = fixed
-            ? (pr.pairs + kSweepPairs - 1u) / kSweepPairs
-            : (unsigned long long)lds_load_u32(kPrefixBase + 4u * buckets);
-        const unsigned long long items = sweeps * tiles;
-        // the second list starts where the first one ended, so no wave runs two short lists
-        unsigned long long item = (wave_id + wave_count - shift) % wave_count;
-        shift = (shift + items) % wave_count;
-        for (; item < items; item += wave_count) {
-            unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
-            unsigned long long local = item, bucket_sweeps = sweeps;
-            if (!fixed) {
-                unsigned low = 0u, high = buckets;   // last bucket whose first item is <= item
-                while (low + 1u < high) {
-                    const unsigned middle = (low + high) >> 1;
-                    if ((unsigned long long)lds_load_u32(kPrefixBase + 4u * middle) * tiles <= item) low = middle;
-                    else high = middle;
-                }
-                const unsigned start = lds_load_u32(kPrefixBase + 4u * low);
-                expert = pr.expert_ids[low];
-                first = pr.bucket_offsets[low];
-                population = pr.bucket_populations[low];
-                local = item - (unsigned long long)start * tiles;
-                bucket_sweeps = lds_load_u32(kPrefixBase + 4u * (low + 1u)) - start;
+    // Work items are numbered with the shared expert's first (the heaviest: full sweeps), then the
+    // routed buckets in worklist order.
+    const GroupedProblem &extra = a.problem[a.problems > 1u ? 1u : 0u];
+    const unsigned extra_items = a.problems > 1u
+        ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) * tiles : 0u;
+    const unsigned routed_sweeps = routed_fixed
+        ? (unsigned)((routed.pairs + kSweepPairs - 1u) / kSweepPairs)
+        : lds_load_u32(kPrefixBase + 4u * buckets);
+    const unsigned total_items = extra_items + routed_sweeps * tiles;
+    // Workgroup b owns items b, b + grid, b + 2 grid, ...; its waves draw positions in that list
+    // from a counter in LDS, so a wave that met light items takes more of them.
+    auto draw = [&]() -> unsigned {
+        unsigned got = 0u;
+        if (lane == 0u)
+            got = __hip_atomic_fetch_add(
+                reinterpret_cast<__attribute__((address_space(3))) unsigned *>(kTicketAddress), 1u,
+                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return (unsigned)__builtin_amdgcn_readfirstlane((int)got) * gridDim.x + blockIdx.x;
+    };
+    for (unsigned item = draw(); item < total_items; item = draw()) {
+        const bool is_extra = item < extra_items;
+        const GroupedProblem &pr = is_extra ? extra : routed;
+        const bool fixed = is_extra || routed_fixed;
+        unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
+        unsigned local = is_extra ? item : item - extra_items;
+        unsigned bucket_sweeps = is_extra ? extra_items / tiles : routed_sweeps;
+        if (!fixed) {
+            unsigned low = 0u, high = buckets;   // last bucket whose first item is <= local
+            while (low + 1u < high) {
+                const unsigned middle = (low + high) >> 1;
+                if (lds_load_u32(kPrefixBase + 4u * middle) * tiles <= local) low = middle;
+                else high = middle;
             }
-            if (bucket_sweeps == 0ull) {
-                if (lane == 0u) raise_status(a.status, 2);
-                continue;
-            }
-            // the sweeps over one tile are neighbours: they stream the same bytes at the same time
-            const unsigned local32 = (unsigned)local, sweeps32 = (unsigned)bucket_sweeps;
-            const unsigned tile = local32 / sweeps32;
-            const unsigned long long pass = (unsigned long long)(local32 % sweeps32) * kSweepPairs;
-            if (expert >= pr.experts || first + population > pr.pairs || pass >= population ||
-                tile >= tiles) {
-                if (lane == 0u) raise_status(a.status, 2);
-                continue;
-            }
-            const unsigned char *gate_e = pr.gate + expert * pr.expert_bytes;
-            const unsigned char *up_e = FUSED ? pr.up + expert * pr.up_expert_bytes : nullptr;
-            const unsigned row_begin = tile * item_rows;
-            const unsigned row_end = row_begin + item_rows < a.out_rows ? row_begin + item_rows : a.out_rows;
-            const unsigned long long live = population - pass;
-            if (live >= 4ull)
-                iq2_sweep<FUSED, 4>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
-            else if (live == 3ull)
-                iq2_sweep<FUSED, 3>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
-            else if (live == 2ull)
-                iq2_sweep<FUSED, 2>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
-            else
-                iq2_sweep<FUSED, 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            const unsigned start = lds_load_u32(kPrefixBase + 4u * low);
+            expert = pr.expert_ids[low];
+            first = pr.bucket_offsets[low];
+            population = pr.bucket_populations[low];
+            local -= start * tiles;
+            bucket_sweeps = lds_load_u32(kPrefixBase + 4u * (low + 1u)) - start;
         }
+        if (bucket_sweeps == 0u) {
+            if (lane == 0u) raise_status(a.status, 2);
+            continue;
+        }
+        // the sweeps over one tile are neighbours: they stream the same bytes at the same time
+        const unsigned tile = local / bucket_sweeps;
+        const unsigned long long pass = (unsigned long long)(local % bucket_sweeps) * kSweepPairs;
+        if (expert >= pr.experts || first + population > pr.pairs || pass >= population ||
+            tile >= tiles) {
+            if (lane == 0u) raise_status(a.status, 2);
+            continue;
+        }
+        const unsigned char *gate_e = pr.gate + expert * pr.expert_bytes;
+        const unsigned char *up_e = FUSED ? pr.up + expert * pr.up_expert_bytes : nullptr;
+        const unsigned row_begin = tile * item_rows;
+        const unsigned row_end = row_begin + item_rows < a.out_rows ? row_begin + item_rows : a.out_rows;
+        const unsigned long long live = population - pass;
+        if (kSweepPairs >= 4 && live >= 4ull)
+            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+        else if (kSweepPairs >= 3 && live >= 3ull)
+            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+        else if (live >= 2ull)
+            iq2_sweep<FUSED, 2>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+        else
+            iq2_sweep<FUSED, 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
     }
 }
 
