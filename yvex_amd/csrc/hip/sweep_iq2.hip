@@ -31,6 +31,12 @@ namespace yvex {
 #ifndef YVEX_SWEEP_ITERS
 #define YVEX_SWEEP_ITERS 32
 #endif
+#ifndef YVEX_SWEEP_AHEAD_SMALL
+#define YVEX_SWEEP_AHEAD_SMALL 3
+#endif
+#ifndef YVEX_SWEEP_DEPTH_SMALL
+#define YVEX_SWEEP_DEPTH_SMALL 3
+#endif
 #ifndef YVEX_SWEEP_PAIRS
 #define YVEX_SWEEP_PAIRS 4
 #endif
@@ -45,7 +51,8 @@ constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {s
 constexpr unsigned kPrefixBase = kSelBase + 128u * 32u * 8u;   // 257 sweep starts, u32
 constexpr unsigned kTicketAddress = kPrefixBase + 1056u;   // work-item counter of the workgroup
 constexpr unsigned kParkBase = kPrefixBase + 1088u;
-constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u;   // per wave
+constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave: 32 bytes per
+                                                                      // (iteration, packed value), then one spare word per lane
 constexpr unsigned kSweepLdsBytes = kParkBase + kSweepWaves * kParkBytes;
 
 __device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
@@ -112,12 +119,14 @@ __device__ __forceinline__ void sweep_tables_fill()
 struct Iq2Half {
     uint4 lo, hi;
     unsigned d16;
-    __device__ __forceinline__ void load(const unsigned char *row, unsigned super, unsigned half)
+    // rows: wave-uniform address of the iteration's first weight row; scale_at / codes_at: this
+    // lane's byte offsets from it (scalar base + 32-bit lane offset addressing, no vector
+    // arithmetic per load)
+    __device__ __forceinline__ void load(const unsigned char *rows, unsigned scale_at, unsigned codes_at)
     {
-        const unsigned char *b = row + super * 66u;
-        d16 = load_u16(b);
-        __builtin_memcpy(&lo, b + 2u + 32u * half, 16);
-        __builtin_memcpy(&hi, b + 18u + 32u * half, 16);
+        d16 = load_u16(rows + scale_at);
+        __builtin_memcpy(&lo, rows + codes_at, 16);
+        __builtin_memcpy(&hi, rows + codes_at + 16u, 16);
     }
 };
 
@@ -131,6 +140,19 @@ struct SweepLane {
     unsigned park_write;   // + (lane parity) * 16 + (lane / 16) * 4
 };
 
+__device__ __forceinline__ int dot4_from_zero(unsigned a, unsigned b)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    int d;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+#else
+    (void)a;
+    (void)b;
+    return 0;
+#endif
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v)
 {
@@ -138,15 +160,19 @@ __device__ __forceinline__ float dpp_add(float v)
 }
 
 // Exact integer sums of this lane's four units of each of STREAMS weight rows against N
-// activation rows. The work is cut into stages of half a unit (two codebook lookups, two selector
-// lookups, sixteen weights); the LDS reads of stage s + DEPTH are issued before stage s is
-// consumed, so their latency runs under the permutes and dot products of the stages between.
+// activation rows. The work is cut into eight stages of half a unit per stream (two codebook
+// lookups, two selector lookups, sixteen weights); the LDS reads of stage s + DEPTH are issued
+// before stage s is consumed, so their latency runs under the permutes and dot products of the
+// stages between. A stage holds independent dependency chains (one per stream, or the even and
+// odd products of a single stream), because a dependent vector instruction issues only about
+// nine cycles after its producer.
 template <int STREAMS, int N>
 __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const SweepLane &g,
                                               const unsigned (&act)[N][32], int (&total)[STREAMS][N])
 {
-    constexpr int kStages = STREAMS * 8;
-    constexpr int DEPTH = N <= 2 ? 3 : 2;
+    constexpr int kStages = 8;
+    constexpr int DEPTH = STREAMS == 2 ? 1 : 2;
+    constexpr int CHAINS = STREAMS == 2 ? 1 : 2;   // accumulators per (stream, pair)
     unsigned q[STREAMS][8];
 #pragma unroll
     for (int w = 0; w < STREAMS; ++w) {
@@ -155,48 +181,66 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
 #pragma unroll
         for (int p = 0; p < N; ++p) total[w][p] = 0;
     }
-    uint4 mag[DEPTH + 1][2];
-    uint2 sel[DEPTH + 1][2];
+    uint4 mag[DEPTH + 1][STREAMS][2];
+    uint2 sel[DEPTH + 1][STREAMS][2];
     auto issue = [&](int stage) {
-        const int w = stage >> 3, k = (stage >> 1) & 3, h = stage & 1, slot = stage % (DEPTH + 1);
-        const unsigned grids = q[w][2 * k], aux = q[w][2 * k + 1];
+        const int k = stage >> 1, h = stage & 1, slot = stage % (DEPTH + 1);
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            const unsigned j = 2u * (unsigned)h + (unsigned)jj;
-            // magnitude address = index byte j << 8 | replica offset
-            const unsigned ma = __builtin_amdgcn_perm(grids, g.mag_lane, 0x0c0c0400u + (j << 8));
-            // selector address = sign field j (7 bits at bit 7j) moved to bit 8 | replica offset
-            const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
-            const unsigned sa = (moved & 0x7f00u) | g.sel_lane;
-            mag[slot][jj] = lds_read_uint4(ma);
-            sel[slot][jj] = lds_read_uint2(sa);
+        for (int w = 0; w < STREAMS; ++w) {
+            const unsigned grids = q[w][2 * k], aux = q[w][2 * k + 1];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const unsigned j = 2u * (unsigned)h + (unsigned)jj;
+                // magnitude address = index byte j << 8 | replica offset
+                const unsigned ma = __builtin_amdgcn_perm(grids, g.mag_lane, 0x0c0c0400u + (j << 8));
+                // selector address = sign field j (7 bits at bit 7j) moved to bit 8 | replica offset
+                const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
+                const unsigned sa = (moved & 0x7f00u) | g.sel_lane;
+                mag[slot][w][jj] = lds_read_uint4(ma);
+                sel[slot][w][jj] = lds_read_uint2(sa);
+            }
         }
     };
 #pragma unroll
     for (int stage = 0; stage < DEPTH; ++stage) issue(stage);
-    int d[N];
+    int d[STREAMS][N][CHAINS];
 #pragma unroll
     for (int stage = 0; stage < kStages; ++stage) {
         if (stage + DEPTH < kStages) issue(stage + DEPTH);
         __builtin_amdgcn_sched_barrier(0);
-        const int w = stage >> 3, k = (stage >> 1) & 3, h = stage & 1, slot = stage % (DEPTH + 1);
-        unsigned weights[4];
+        const int k = stage >> 1, h = stage & 1, slot = stage % (DEPTH + 1);
+        unsigned weights[STREAMS][4];
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            weights[2 * jj] = __builtin_amdgcn_perm(mag[slot][jj].z, mag[slot][jj].x, sel[slot][jj].x);
-            weights[2 * jj + 1] = __builtin_amdgcn_perm(mag[slot][jj].w, mag[slot][jj].y, sel[slot][jj].y);
-        }
+        for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-        for (int p = 0; p < N; ++p) {
-            if (h == 0) d[p] = 0;
+            for (int w = 0; w < STREAMS; ++w) {
+                weights[w][2 * jj] = __builtin_amdgcn_perm(mag[slot][w][jj].z, mag[slot][w][jj].x, sel[slot][w][jj].x);
+                weights[w][2 * jj + 1] = __builtin_amdgcn_perm(mag[slot][w][jj].w, mag[slot][w][jj].y, sel[slot][w][jj].y);
+            }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) d[p] = dot4(weights[i], act[p][8 * k + 4 * h + i], d[p]);
-        }
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int p = 0; p < N; ++p)
+#pragma unroll
+                for (int w = 0; w < STREAMS; ++w) {
+                    const int chain = i % CHAINS;
+                    const unsigned x = act[p][8 * k + 4 * h + i];
+                    // the first product of a chain starts from the constant zero
+                    if (h == 0 && i < CHAINS) d[w][p][chain] = dot4_from_zero(weights[w][i], x);
+                    else d[w][p][chain] = dot4(weights[w][i], x, d[w][p][chain]);
+                }
         if (h == 1) {
-            // 2 s + 1: bit 27 of the word is a sign bit, forced to 1
-            const int factor = (int)((q[w][2 * k + 1] >> 27) | 1u);
 #pragma unroll
-            for (int p = 0; p < N; ++p) total[w][p] += __mul24(d[p], factor);   // |d| < 2^23
+            for (int w = 0; w < STREAMS; ++w) {
+                // 2 s + 1: bit 27 of the word is a sign bit, forced to 1
+                const int factor = (int)((q[w][2 * k + 1] >> 27) | 1u);
+#pragma unroll
+                for (int p = 0; p < N; ++p) {
+                    int sum = d[w][p][0];
+                    if (CHAINS == 2) sum += d[w][p][1];
+                    total[w][p] += __mul24(sum, factor);   // |sum| < 2^23
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -250,42 +294,54 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
                                    : act_scale[2 * v];
     }
 
-    const unsigned rows = row_end - row_begin;
-    const unsigned iterations = (rows + g.rows_per_iter - 1u) / g.rows_per_iter;   // <= kSweepIters
-    auto row_pointer = [&](const unsigned char *base, unsigned long long row_bytes, unsigned it) {
-        unsigned local = it * g.rows_per_iter + (g.live ? g.sub : 0u);
-        if (local >= rows) local = 0u;
-        return base + (unsigned long long)(row_begin + local) * row_bytes;
+    const unsigned rows = row_end - row_begin;               // a multiple of rows_per_iter
+    const unsigned iterations = rows / g.rows_per_iter;       // <= kSweepIters
+    // wave-uniform row bases advance by a scalar stride; the lane's place inside an iteration's
+    // rows is a constant 32-bit offset
+    const unsigned char *gate_rows = gate_e + (unsigned long long)row_begin * pr.row_bytes;
+    const unsigned char *up_rows = FUSED ? up_e + (unsigned long long)row_begin * pr.up_row_bytes : nullptr;
+    const unsigned long long gate_step = (unsigned long long)g.rows_per_iter * pr.row_bytes;
+    const unsigned long long up_step = (unsigned long long)g.rows_per_iter * pr.up_row_bytes;
+    const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
+    const unsigned gate_scale_at = lane_row * (unsigned)pr.row_bytes + lane_super * 66u;
+    const unsigned gate_codes_at = gate_scale_at + 2u + 32u * g.half;
+    const unsigned up_scale_at = lane_row * (unsigned)pr.up_row_bytes + lane_super * 66u;
+    const unsigned up_codes_at = up_scale_at + 2u + 32u * g.half;
+    // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
+    // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
+    // The loop body is one basic block: every turn requests a row (the last ones clamped to the
+    // final row) and every lane stores (lanes that hold no result write to a spare word), so no
+    // branch sits between a request and the wait that consumes it and the waits stay counted.
+    constexpr int AHEAD = N <= 2 ? YVEX_SWEEP_AHEAD_SMALL : 1;   // AHEAD + 1 is 2 or 4
+    constexpr int STREAMS = FUSED ? 2 : 1;
+    Iq2Half ring[AHEAD + 1][STREAMS];
+    const unsigned last = iterations - 1u;
+    auto request = [&](Iq2Half (&slot)[STREAMS], unsigned it) {
+        const unsigned clamped = it < last ? it : last;
+        slot[0].load(gate_rows + clamped * gate_step, gate_scale_at, gate_codes_at);
+        if constexpr (FUSED) slot[1].load(up_rows + clamped * up_step, up_scale_at, up_codes_at);
     };
-    Iq2Half next_gate, next_up;
-    next_gate.load(row_pointer(gate_e, pr.row_bytes, 0u), g.live ? g.super : 0u, g.half);
-    if constexpr (FUSED) next_up.load(row_pointer(up_e, pr.up_row_bytes, 0u), g.live ? g.super : 0u, g.half);
+#pragma unroll
+    for (int ahead = 0; ahead < AHEAD; ++ahead) request(ring[ahead], (unsigned)ahead);
+    const bool writer = (lane & 15u) < 2u;
+    unsigned park_at = writer ? g.park_write : g.park + kParkBytes - 256u + lane * 4u;
+    const unsigned park_step = writer ? 32u : 0u;
 
-    for (unsigned it = 0; it < iterations; ++it) {
-        const Iq2Half gate = next_gate;
-        Iq2Half up;
-        if constexpr (FUSED) up = next_up;
-        if (it + 1u < iterations) {
-            next_gate.load(row_pointer(gate_e, pr.row_bytes, it + 1u), g.live ? g.super : 0u, g.half);
-            if constexpr (FUSED)
-                next_up.load(row_pointer(up_e, pr.up_row_bytes, it + 1u), g.live ? g.super : 0u, g.half);
-        }
+    for (unsigned it0 = 0; it0 < iterations; it0 += AHEAD + 1) {
+#pragma unroll
+      for (int turn = 0; turn <= AHEAD; ++turn) {
+        const unsigned it = it0 + (unsigned)turn;   // may run past the last row by AHEAD turns
+        request(ring[(turn + AHEAD) % (AHEAD + 1)], it + AHEAD);
+        const Iq2Half (&now)[STREAMS] = ring[turn];
         int total_gate[N], total_up[N];
-        if constexpr (FUSED) {
-            const Iq2Half both[2] = {gate, up};
-            int totals[2][N];
-            iq2_half_dots<2, N>(both, g, act, totals);
+        {
+            int totals[STREAMS][N];
+            iq2_half_dots<STREAMS, N>(now, g, act, totals);
 #pragma unroll
             for (int p = 0; p < N; ++p) {
                 total_gate[p] = totals[0][p];
-                total_up[p] = totals[1][p];
+                total_up[p] = totals[STREAMS - 1][p];
             }
-        } else {
-            const Iq2Half one[1] = {gate};
-            int totals[1][N];
-            iq2_half_dots<1, N>(one, g, act, totals);
-#pragma unroll
-            for (int p = 0; p < N; ++p) total_gate[p] = totals[0][p];
         }
         // the two lanes of a superblock add their halves: exact int32 superblock sums
 #pragma unroll
@@ -294,8 +350,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             if constexpr (FUSED) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
         }
         float weight_scale;
-        if constexpr (FUSED) weight_scale = 0.125f * f16_bits_to_float(odd ? up.d16 : gate.d16);
-        else weight_scale = 0.125f * f16_bits_to_float(gate.d16);
+        weight_scale = 0.125f * f16_bits_to_float(odd ? now[STREAMS - 1].d16 : now[0].d16);
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
             int t;
@@ -305,9 +360,10 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             value = dpp_add<0x4e>(value);     // lanes i and i ^ 2
             value = dpp_add<0x124>(value);    // + lane i - 4 (row rotate)
             value = dpp_add<0x128>(value);    // + lanes i - 8, i - 12: all lanes of this parity
-            if ((lane & 15u) < 2u)
-                lds_store_u32(g.park_write + (it * PV + (unsigned)v) * 32u, __float_as_uint(value));
+            lds_store_u32(park_at, __float_as_uint(value));
+            park_at += park_step;
         }
+      }
     }
 
     // ---- finish the item: add the row-group partials, SwiGLU or bf16, coalesced stores ----
@@ -491,10 +547,13 @@ static int sweep_grid()
     return units;
 }
 
-bool iq2_sweep_supported(unsigned width)
+bool iq2_sweep_supported(unsigned width, unsigned out_rows)
 {
     const unsigned lanes_per_row = width / 128u;
-    return width % 256u == 0u && lanes_per_row >= 16u && lanes_per_row <= 64u;
+    if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
+    const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u
+        ? 64u / lanes_per_row : 1u;
+    return out_rows % rows_per_iter == 0u;   // an iteration never reads past the last row
 }
 
 template <bool FUSED>
