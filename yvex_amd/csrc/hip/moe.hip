@@ -570,7 +570,14 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
         const char *text = getenv("YVEX_SWEEP_GENERIC");
         generic_only = text && text[0] == '1';
     }
-    if (qtype == QT_IQ2_XXS && q8 && !generic_only && iq2_sweep_supported(a.width, a.out_rows))
+    bool aligned = true;   // the specialised sweeps load dwords: bases and strides must allow it
+    for (unsigned i = 0; i < a.problems; ++i) {
+        const GroupedProblem &pr = a.problem[i];
+        aligned = aligned && ((uintptr_t)pr.gate % 4u == 0u) && pr.expert_bytes % 4u == 0u &&
+                  (!pr.up || ((uintptr_t)pr.up % 4u == 0u && pr.up_expert_bytes % 4u == 0u));
+    }
+    if (qtype == QT_IQ2_XXS && q8 && !generic_only && aligned &&
+        iq2_sweep_supported(a.width, a.out_rows))
         return launch_iq2_sweep(a, fused, stream);
     switch (qtype) {
     case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);

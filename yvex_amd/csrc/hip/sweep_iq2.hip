@@ -32,7 +32,7 @@ namespace yvex {
 #define YVEX_SWEEP_ITERS 32
 #endif
 #ifndef YVEX_SWEEP_AHEAD_SMALL
-#define YVEX_SWEEP_AHEAD_SMALL 3
+#define YVEX_SWEEP_AHEAD_SMALL 1
 #endif
 #ifndef YVEX_SWEEP_DEPTH_SMALL
 #define YVEX_SWEEP_DEPTH_SMALL 3
@@ -116,17 +116,23 @@ __device__ __forceinline__ void sweep_tables_fill()
 }
 
 // A lane's share of one IQ2_XXS weight row: half a superblock, 32 packed bytes plus the scale.
+// Superblocks are 66 bytes, so the codes start on a 2-byte boundary, and vector loads that are
+// not dword-aligned run at less than half rate on this part. Every load here is dword-aligned:
+// nine dwords from the aligned address at or below the codes (the ninth only matters when the
+// codes start two bytes in) and the dword that holds the fp16 scale; the consumer shifts the
+// codes into place with byte-align instructions.
 struct Iq2Half {
     uint4 lo, hi;
-    unsigned d16;
-    // rows: wave-uniform address of the iteration's first weight row; scale_at / codes_at: this
-    // lane's byte offsets from it (scalar base + 32-bit lane offset addressing, no vector
-    // arithmetic per load)
-    __device__ __forceinline__ void load(const unsigned char *rows, unsigned scale_at, unsigned codes_at)
+    unsigned tail, scale_word;
+    // rows: wave-uniform address of the iteration's first weight row; the rest are this lane's
+    // byte offsets from it (scalar base + 32-bit lane offset addressing)
+    __device__ __forceinline__ void load(const unsigned char *rows, unsigned codes_at,
+                                         unsigned tail_at, unsigned scale_at)
     {
-        d16 = load_u16(rows + scale_at);
-        __builtin_memcpy(&lo, rows + codes_at, 16);
-        __builtin_memcpy(&hi, rows + codes_at + 16u, 16);
+        lo = *reinterpret_cast<const uint4 *>(rows + codes_at);          // 4-byte aligned
+        hi = *reinterpret_cast<const uint4 *>(rows + codes_at + 16u);
+        tail = *reinterpret_cast<const unsigned *>(rows + tail_at);
+        scale_word = *reinterpret_cast<const unsigned *>(rows + scale_at);
     }
 };
 
@@ -136,6 +142,8 @@ struct SweepLane {
     bool live;
     unsigned mag_lane;     // (lane % 16) * 16
     unsigned sel_lane;     // kSelBase + (lane % 32) * 8
+    unsigned code_shift;   // bytes the codes sit above their aligned load address: 0 or 2
+    unsigned scale_shift;  // bits the fp16 scale sits above its aligned load address: 0 or 16
     unsigned park;         // this wave's parking area
     unsigned park_write;   // + (lane parity) * 16 + (lane / 16) * 4
 };
@@ -176,8 +184,10 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
     unsigned q[STREAMS][8];
 #pragma unroll
     for (int w = 0; w < STREAMS; ++w) {
-        q[w][0] = c[w].lo.x; q[w][1] = c[w].lo.y; q[w][2] = c[w].lo.z; q[w][3] = c[w].lo.w;
-        q[w][4] = c[w].hi.x; q[w][5] = c[w].hi.y; q[w][6] = c[w].hi.z; q[w][7] = c[w].hi.w;
+        const unsigned raw[9] = {c[w].lo.x, c[w].lo.y, c[w].lo.z, c[w].lo.w,
+                                 c[w].hi.x, c[w].hi.y, c[w].hi.z, c[w].hi.w, c[w].tail};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[w][i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], g.code_shift);
 #pragma unroll
         for (int p = 0; p < N; ++p) total[w][p] = 0;
     }
@@ -303,10 +313,13 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned long long gate_step = (unsigned long long)g.rows_per_iter * pr.row_bytes;
     const unsigned long long up_step = (unsigned long long)g.rows_per_iter * pr.up_row_bytes;
     const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
-    const unsigned gate_scale_at = lane_row * (unsigned)pr.row_bytes + lane_super * 66u;
-    const unsigned gate_codes_at = gate_scale_at + 2u + 32u * g.half;
-    const unsigned up_scale_at = lane_row * (unsigned)pr.up_row_bytes + lane_super * 66u;
-    const unsigned up_codes_at = up_scale_at + 2u + 32u * g.half;
+    // (row bases and row strides are multiples of four bytes: checked on the host)
+    const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * 66u;
+    const unsigned up_block = lane_row * (unsigned)pr.up_row_bytes + lane_super * 66u;
+    const unsigned gate_codes_at = (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
+    const unsigned up_codes_at = (up_block + 2u + 32u * g.half) & ~3u;
+    const unsigned tail_step = g.code_shift ? 32u : 0u;   // aligned codes end inside 32 bytes
+    const unsigned gate_scale_at = gate_block & ~3u, up_scale_at = up_block & ~3u;
     // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
     // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
@@ -318,11 +331,18 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned last = iterations - 1u;
     auto request = [&](Iq2Half (&slot)[STREAMS], unsigned it) {
         const unsigned clamped = it < last ? it : last;
-        slot[0].load(gate_rows + clamped * gate_step, gate_scale_at, gate_codes_at);
-        if constexpr (FUSED) slot[1].load(up_rows + clamped * up_step, up_scale_at, up_codes_at);
+        slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_codes_at + tail_step, gate_scale_at);
+        if constexpr (FUSED)
+            slot[1].load(up_rows + clamped * up_step, up_codes_at, up_codes_at + tail_step, up_scale_at);
     };
+    // The first requests are kept in ring order: the loop's first wait is counted against the
+    // loads issued after the slot it consumes, on the entry path and on the back edge alike.
 #pragma unroll
-    for (int ahead = 0; ahead < AHEAD; ++ahead) request(ring[ahead], (unsigned)ahead);
+    for (int ahead = 0; ahead < AHEAD; ++ahead) {
+        __builtin_amdgcn_sched_barrier(0);
+        request(ring[ahead], (unsigned)ahead);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     const bool writer = (lane & 15u) < 2u;
     unsigned park_at = writer ? g.park_write : g.park + kParkBytes - 256u + lane * 4u;
     const unsigned park_step = writer ? 32u : 0u;
@@ -350,7 +370,8 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             if constexpr (FUSED) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
         }
         float weight_scale;
-        weight_scale = 0.125f * f16_bits_to_float(odd ? now[STREAMS - 1].d16 : now[0].d16);
+        weight_scale = 0.125f * f16_bits_to_float(
+            ((odd ? now[STREAMS - 1].scale_word : now[0].scale_word) >> g.scale_shift) & 0xffffu);
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
             int t;
@@ -456,6 +477,10 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     g.live = g.sub < g.rows_per_iter;
     g.super = seg >> 1;
     g.half = seg & 1u;
+    // superblock `super` starts 66 * super bytes into a row whose start is dword-aligned
+    const unsigned block_start = 66u * (g.live ? g.super : 0u);
+    g.code_shift = (block_start + 2u + 32u * g.half) & 3u;
+    g.scale_shift = 8u * (block_start & 3u);
     g.mag_lane = (lane & 15u) * 16u;
     g.sel_lane = kSelBase + (lane & 31u) * 8u;
     g.park = kParkBase + wave * kParkBytes;
@@ -551,6 +576,7 @@ bool iq2_sweep_supported(unsigned width, unsigned out_rows)
 {
     const unsigned lanes_per_row = width / 128u;
     if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
+    if ((width / 256u * 66u) % 4u != 0u) return false;   // rows must start on dword boundaries
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u
         ? 64u / lanes_per_row : 1u;
     return out_rows % rows_per_iter == 0u;   // an iteration never reads past the last row
