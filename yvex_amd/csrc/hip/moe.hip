@@ -113,7 +113,10 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
     __shared__ unsigned bad;
     const unsigned tid = threadIdx.x;
     for (unsigned i = tid; i < experts * words; i += blockDim.x) bitmap[i] = 0u;
-    if (tid == 0u) bad = 0u;
+    if (tid == 0u) {
+        bad = 0u;
+        slot[experts + 1536u] = 0u;   // running maximum of the populations (scan[1536])
+    }
     __syncthreads();
     for (unsigned p = tid; p < pairs; p += blockDim.x) {
         const unsigned long long e = selected[p];
@@ -132,40 +135,72 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
         population[e] = n;
     }
     __syncthreads();
-    if (tid == 0u) {
-        unsigned cursor = 0u, bucket = 0u, maximum = 0u, sweeps = 0u;
-        for (unsigned e = 0; e < experts; ++e) {
-            const unsigned n = population[e];
-            offset[e] = cursor;
-            slot[e] = n ? bucket : 0xffffffffu;
-            if (n) {
-                expert_ids[bucket] = e;
-                bucket_offsets[bucket] = cursor;
-                bucket_populations[bucket] = n;
-                sweep_offsets[bucket] = sweeps;
-                sweeps += (n + (unsigned)kPass - 1u) / (unsigned)kPass;
-                bucket++;
-                maximum = n > maximum ? n : maximum;
-            }
-            cursor += n;
-        }
-        offset[experts] = cursor;
-        bucket_offsets[bucket] = cursor;
-        sweep_offsets[bucket] = sweeps;
-        for (unsigned b = bucket; b < experts; ++b) {
-            expert_ids[b] = 0ull;
-            bucket_populations[b] = 0ull;
-            bucket_offsets[b + 1u] = cursor;
-            sweep_offsets[b + 1u] = sweeps;
-        }
-        counts[0] = bucket;
-        counts[1] = maximum;
-        counts[2] = cursor;
-        counts[3] = sweeps;
-        counts[4] = counts[5] = counts[6] = counts[7] = 0ull;   // tickets of the expert kernels
-        if (cursor != pairs) bad = 1u;
+    // Exclusive prefix sums over the experts (<= 256) of population, sweep count and occupancy,
+    // three Hillis-Steele scans run together in LDS; every expert then publishes its own bucket.
+    unsigned *scan = slot + experts;                       // [2][3][256]
+    if (tid < 256u) {
+        const unsigned n = tid < experts ? population[tid] : 0u;
+        scan[tid] = n;
+        scan[256u + tid] = (n + (unsigned)kPass - 1u) / (unsigned)kPass;
+        scan[512u + tid] = n ? 1u : 0u;
     }
     __syncthreads();
+    unsigned from = 0u, to = 768u;
+    for (unsigned step = 1u; step < 256u; step <<= 1) {
+        if (tid < 768u) {
+            const unsigned lane_in_scan = tid & 255u;
+            unsigned v = scan[from + tid];
+            if (lane_in_scan >= step) v += scan[from + tid - step];
+            scan[to + tid] = v;
+        }
+        __syncthreads();
+        const unsigned t = from;
+        from = to;
+        to = t;
+    }
+    const unsigned total_pairs = scan[from + 255u], total_sweeps = scan[from + 256u + 255u];
+    const unsigned bucket_count = scan[from + 512u + 255u];
+    if (tid < experts) {
+        const unsigned n = population[tid];
+        const unsigned cursor = scan[from + tid] - n;
+        const unsigned sweeps_before = scan[from + 256u + tid] - (n + (unsigned)kPass - 1u) / (unsigned)kPass;
+        const unsigned bucket = scan[from + 512u + tid] - (n ? 1u : 0u);
+        offset[tid] = cursor;
+        if (n) {
+            expert_ids[bucket] = tid;
+            bucket_offsets[bucket] = cursor;
+            bucket_populations[bucket] = n;
+            sweep_offsets[bucket] = sweeps_before;
+        }
+        if (tid >= bucket_count) {                         // unused tail of the bucket arrays
+            expert_ids[tid] = 0ull;
+            bucket_populations[tid] = 0ull;
+            bucket_offsets[tid + 1u] = total_pairs;
+            sweep_offsets[tid + 1u] = total_sweeps;
+        }
+    }
+    if (tid == 0u) {
+        offset[experts] = total_pairs;
+        bucket_offsets[bucket_count] = total_pairs;
+        sweep_offsets[bucket_count] = total_sweeps;
+        counts[0] = bucket_count;
+        counts[2] = total_pairs;
+        counts[3] = total_sweeps;
+        counts[4] = counts[5] = counts[6] = counts[7] = 0ull;   // tickets of the expert kernels
+        if (total_pairs != pairs) bad = 1u;
+    }
+    // largest population: one atomic per wave after a wave-wide maximum
+    {
+        unsigned n = tid < experts ? population[tid] : 0u;
+#pragma unroll
+        for (int offset_lanes = 32; offset_lanes > 0; offset_lanes >>= 1) {
+            const unsigned other = (unsigned)__shfl_xor((int)n, offset_lanes, kWave);
+            n = other > n ? other : n;
+        }
+        if ((tid & 63u) == 0u && tid < 256u) atomicMax(&scan[1536u], n);
+    }
+    __syncthreads();
+    if (tid == 0u) counts[1] = scan[1536u];
     for (unsigned i = tid; i < experts * words; i += blockDim.x) {
         const unsigned e = i / words, w = i % words;
         unsigned bits = bitmap[i];
@@ -622,7 +657,7 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
     const uint64_t rows = pairs / topk;
     if (rows > kWorklistMaxRows) return ST_BOUNDS;
     const uint64_t words = (rows + 31u) / 32u;
-    const size_t lds = (size_t)(experts * words + 3u * experts + 1u) * sizeof(unsigned);
+    const size_t lds = (size_t)(experts * words + 3u * experts + 1u + 1537u) * sizeof(unsigned);
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void *)worklist_kernel,
