@@ -76,12 +76,8 @@ int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t row
  *   expert_ids[experts], bucket_offsets[experts + 1], bucket_populations[experts]
  *   sweep_offsets[experts + 1]  running count of weight sweeps (two pairs per sweep) before each
  *                           bucket: the generic grouped kernels spread sweeps, not buckets, over
- *                           the chip
- *   counts[8]               {bucket_count, maximum_population, pair_count, sweep_count,
- *                           ticket, finished, 0, 0}: words 4 and 5 are the work-item ticket and
- *                           the finished-workgroup count of the expert kernels, zeroed here and
- *                           returned to zero by every kernel that uses them, so kernels that share
- *                           one worklist must run one after the other (one stream) */
+ *                           the chip (the IQ2_XXS sweeps number theirs, four pairs each, on device)
+ *   counts[4]               {bucket_count, maximum_population, pair_count, sweep_count} */
 int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
                             uint64_t experts, uint64_t *order, uint64_t *expert_ids,
                             uint64_t *bucket_offsets, uint64_t *bucket_populations,

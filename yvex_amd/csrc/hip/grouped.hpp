@@ -24,7 +24,6 @@ struct GroupedProblem {
     float *out;                              // [ordered or source pair][out_rows]
     int out_by_source_pair;
     unsigned sweeps;                         // single known bucket: ceil(pairs / kPass), else 0
-    unsigned long long *tickets;             // counts + 4 of the worklist (ticket, finished) or null
 };
 
 struct GroupedArgs {
@@ -110,7 +109,6 @@ static inline void fill_up_problem(GroupedProblem &p, const yvex_hip_expert_weig
     p.out = out;
     p.out_by_source_pair = 0;
     p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
-    p.tickets = wl.expert_ids && wl.counts ? (unsigned long long *)wl.counts + 4 : nullptr;
 }
 
 static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_weights *w,
@@ -138,7 +136,6 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
     p.out = out;
     p.out_by_source_pair = 1;
     p.sweeps = wl.expert_ids ? 0u : (unsigned)((pairs + kPass - 1u) / kPass);
-    p.tickets = wl.expert_ids && wl.counts ? (unsigned long long *)wl.counts + 4 : nullptr;
 }
 
 // Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16
