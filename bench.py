@@ -134,7 +134,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--act", choices=["q8k", "f32"], default="q8k")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=2)
+    ap.add_argument("--cpu-rows", type=int, default=4)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 1 GiB read kernel and a 256 MiB fill kernel, so a "
