@@ -6,12 +6,15 @@
 // V_MFMA_I32_16X16X64_I8. Two waves share a SIMD, so one wave's decode and scaling arithmetic
 // runs under the other's matrix instructions.
 //
-//   A operand (weights): each lane decodes the 16 weights it owns straight into registers. The
+//   A operand (weights): each lane builds the 16 weights it owns straight into registers. The
 //       IQ2_XXS value of one weight is level * sign * (2s+1), up to 43 * 31 = 1333, so it is
 //       split into two int8 limbs, value = 128 * hi + lo with hi in [1, 11] and lo in
-//       [-120, 63]; both limbs come from one 16-byte LDS lookup keyed by (grid index, s), signs
-//       from a second lookup. Neither limb is ever zero, so negating a byte as (x ^ 0xff) + 1
-//       cannot carry into its neighbour.
+//       [-120, 63]. For a given scale there are only three levels, so the six signed limb
+//       values of a group fit two registers and one V_PERM_B32 per four weights picks them:
+//       the selector byte of a weight is its level code (0..2) plus 4 when it is negative.
+//       Three small conflict-free LDS tables feed this: level codes of a codebook entry
+//       (8 bytes), sign selectors of a 7-bit sign field (8 bytes) and the limb words of a
+//       scale (16 bytes).
 //   B operand (activations): the 128 x 256 int8 block of the current superblock, copied from
 //       global memory straight into LDS (GLOBAL_LOAD_LDS_DWORDX4, no registers in between),
 //       double buffered. 16-byte piece c of token t sits at piece position c ^ (t % 16), so the
@@ -33,10 +36,10 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr unsigned kTileTokens = 128u;
 constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
-constexpr unsigned kLimbBase = 0u;                          // 4096 entries x 16 bytes
-constexpr unsigned kSignBase = 65536u;                      // 128 entries x 8 replicas x 16 bytes
-constexpr unsigned kSignReplicas = 8u;
-constexpr unsigned kStageBase = kSignBase + 128u * kSignReplicas * 16u;
+constexpr unsigned kCodeBase = 0u;                          // 256 entries x 32 replicas x 8 bytes
+constexpr unsigned kSelBase = 65536u;                       // 128 entries x 16 replicas x 8 bytes
+constexpr unsigned kLutBase = kSelBase + 128u * 16u * 8u;   // 16 scales x 16 replicas x 16 bytes
+constexpr unsigned kStageBase = kLutBase + 16u * 16u * 16u;
 constexpr unsigned kStageActs = kTileTokens * kActPitch;
 constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per token
 constexpr unsigned kTileStartBase = kStageBase + 2u * kStageBytes;
@@ -104,7 +107,7 @@ __device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_b
 #endif
 }
 
-// Limb pair of one magnitude byte: low limb in bits 0-7, high limb in bits 8-15.
+// Limb pair of one magnitude: low limb in bits 0-7, high limb in bits 8-15.
 __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
 {
     const unsigned magnitude = level * factor;
@@ -114,29 +117,50 @@ __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
     return ((unsigned)lo & 255u) | (hi << 8);
 }
 
+__device__ __forceinline__ void lds_write_uint2(unsigned address, uint2 v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) uint2 *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+
 __device__ __forceinline__ void mfma_tables_fill()
 {
-    for (unsigned index = threadIdx.x; index < 4096u; index += blockDim.x) {
-        const unsigned factor = 2u * (index >> 8) + 1u;
-        const uint2 m = iq2_magnitude_entry(index & 255u);
-        uint4 entry = make_uint4(0u, 0u, 0u, 0u);
+    // level codes: byte l of the entry is 0, 1 or 2 for level 8, 25 or 43 of weight l
+    for (unsigned index = threadIdx.x; index < 256u * 32u; index += blockDim.x) {
+        const uint2 m = iq2_magnitude_entry(index >> 5);
+        uint2 codes = make_uint2(0u, 0u);
 #pragma unroll
         for (unsigned l = 0; l < 4u; ++l) {
-            const unsigned a = iq2_limbs((m.x >> (8u * l)) & 255u, factor);
-            const unsigned b = iq2_limbs((m.y >> (8u * l)) & 255u, factor);
-            entry.x |= (a & 255u) << (8u * l);
-            entry.y |= (b & 255u) << (8u * l);
-            entry.z |= (a >> 8) << (8u * l);
-            entry.w |= (b >> 8) << (8u * l);
+            const unsigned a = (m.x >> (8u * l)) & 255u, b = (m.y >> (8u * l)) & 255u;
+            codes.x |= (a == 8u ? 0u : a == 25u ? 1u : 2u) << (8u * l);
+            codes.y |= (b == 8u ? 0u : b == 25u ? 1u : 2u) << (8u * l);
         }
-        lds_write_uint4(kLimbBase + index * 16u, entry);
+        lds_write_uint2(kCodeBase + index * 8u, codes);
     }
-    // sign entries: replica r of entry e at (e * 8 + r) * 16, a lane reads replica lane % 8, so
-    // the 16 lanes served together spread over all bank groups whatever entries they ask for
-    for (unsigned index = threadIdx.x; index < 128u * kSignReplicas; index += blockDim.x) {
-        const uint2 m = iq2_signmask_entry(index / kSignReplicas);
-        lds_write_uint4(kSignBase + index * 16u,
-                        make_uint4(m.x, m.y, m.x & 0x01010101u, m.y & 0x01010101u));
+    // sign selectors: byte l is 4 when weight l is negative (7 stored bits + parity)
+    for (unsigned index = threadIdx.x; index < 128u * 16u; index += blockDim.x) {
+        const uint2 m = iq2_signmask_entry(index >> 4);
+        lds_write_uint2(kSelBase + index * 8u, make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
+    }
+    // limb words of scale s: {+lo, -lo, +hi, -hi}, byte c = limb of level code c
+    for (unsigned index = threadIdx.x; index < 16u * 16u; index += blockDim.x) {
+        const unsigned factor = 2u * (index >> 4) + 1u;
+        unsigned lo = 0u, hi = 0u;
+        const unsigned levels[3] = {8u, 25u, 43u};
+#pragma unroll
+        for (unsigned c = 0; c < 3u; ++c) {
+            const unsigned pair = iq2_limbs(levels[c], factor);
+            lo |= (pair & 255u) << (8u * c);
+            hi |= (pair >> 8) << (8u * c);
+        }
+        // byte-wise negation: no limb is zero, so (x ^ 0xff) + 1 never carries; byte 3 stays 0
+        const unsigned neg_lo = ((lo ^ 0x00ffffffu) + 0x00010101u) & 0x00ffffffu;
+        const unsigned neg_hi = ((hi ^ 0x00ffffffu) + 0x00010101u) & 0x00ffffffu;
+        lds_write_uint4(kLutBase + index * 16u, make_uint4(lo, neg_lo, hi, neg_hi));
     }
 }
 
@@ -146,21 +170,27 @@ struct MfmaItem {
     unsigned tokens, row_tile;
 };
 
-// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8) for a workgroup whose waves own
-// RB 16-row blocks each (RB = 1: eight waves, two per SIMD; RB = 2: four waves, one per SIMD with
-// the whole register file, each activation fragment feeding twice as many matrix instructions).
-// Every loop below has a fixed trip count, so accumulators never leave registers and no branch
-// sits between matrix instructions.
-template <bool FUSED_UP, unsigned NB, unsigned RB>
+// Twelve aligned bytes that hold one 8-byte group record starting 0 or 2 bytes in.
+struct alignas(4) RawGroup {
+    unsigned x, y, z;
+};
+
+// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8). Eight waves, two per SIMD, each
+// owning one 16-row block. Every loop below has a fixed trip count and the superblock body is one
+// basic block (requests past the end are clamped, not guarded), so accumulators never leave
+// registers and the compiler's wait counts stay exact.
+template <bool FUSED_UP, unsigned NB>
 __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
-    constexpr unsigned kWaves = 8u / RB;
+    constexpr unsigned kWaves = 8u;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned li = lane & 15u, kb = lane >> 4;
     constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
     constexpr unsigned kStagedTokens = NB * 16u;
-    const unsigned sign_lane = kSignBase + (lane & (kSignReplicas - 1u)) * 16u;
+    const unsigned code_lane = kCodeBase + (lane & 31u) * 8u;
+    const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
+    const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
     const unsigned superblocks = a.width >> 8;
 
     // ---- activation rows this lane copies: wave w owns the 4-token groups w, w + kWaves, ... ----
@@ -183,37 +213,40 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     // waves 0 and 1 also copy the block scales of tokens 64 w + lane
     const unsigned char *scale_from = token_row(64u * (wave & 1u) + lane);
 
-    // ---- the weight rows of this lane, one per row block ----
-    // fused: blocks are (gate, up) of the same 16 rows when RB = 2; with RB = 1 waves 0-3 hold
-    // gate blocks and waves 4-7 the matching up blocks
-    const unsigned char *weight_row[RB];
-    unsigned out_row_base[RB];
-#pragma unroll
-    for (unsigned rb = 0; rb < RB; ++rb) {
+    // ---- the weight row of this lane: waves 0-3 hold gate blocks and waves 4-7 the matching up
+    // blocks when the SwiGLU is fused ----
+    unsigned out_row_base;
+    const unsigned char *weight_row;
+    {
         bool is_up = false;
         if constexpr (FUSED_UP) {
-            out_row_base[rb] = it.row_tile * kItemRows + (wave & 3u) * 16u;
-            is_up = RB == 2u ? rb == 1u : wave >= 4u;
+            out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
+            is_up = wave >= 4u;
         } else {
-            out_row_base[rb] = it.row_tile * kItemRows + (wave * RB + rb) * 16u;
+            out_row_base = it.row_tile * kItemRows + wave * 16u;
         }
-        unsigned row = out_row_base[rb] + li;
+        unsigned row = out_row_base + li;
         if (row >= a.out_rows) row = a.out_rows - 1u;
-        weight_row[rb] = is_up
+        weight_row = is_up
             ? pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
             : pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
     }
+    // Superblocks are 66 bytes, so group records start on 2-byte boundaries, and vector loads
+    // that are not dword-aligned run at less than half rate: the lane loads twelve aligned bytes
+    // around each record and shifts them into place. Records of superblock sb start
+    // (row start + 2 sb + 2) mod 4 bytes past a dword, the fp16 scale (row start + 2 sb) mod 4.
+    const unsigned row_misalign = (unsigned)(unsigned long long)weight_row & 3u;
+    const unsigned char *row_aligned = weight_row - row_misalign;
+    const unsigned lane_group = kb >> 1;                      // groups 2 ks + lane_group
 
-    float acc[RB][NB][4];
+    float acc[NB][4];
 #pragma unroll
-    for (unsigned rb = 0; rb < RB; ++rb)
+    for (unsigned tb = 0; tb < NB; ++tb)
 #pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb)
-#pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) acc[rb][tb][r] = 0.0f;
+        for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
 
-    uint2 codes[RB][4];
-    unsigned scale16[RB];
+    RawGroup raw[4];
+    unsigned raw_scale;
     auto copy_activations = [&](unsigned sb, unsigned stage) {
         const unsigned base = kStageBase + stage * kStageBytes;
 #pragma unroll
@@ -228,13 +261,31 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                           (unsigned)__builtin_amdgcn_readfirstlane((int)(base + kStageActs + wave * 256u)));
     };
     auto fetch_codes = [&](unsigned sb) {
+        const unsigned block = row_misalign + sb * 66u;         // from row_aligned
+        raw_scale = *reinterpret_cast<const unsigned *>(row_aligned + (block & ~3u));
 #pragma unroll
-        for (unsigned rb = 0; rb < RB; ++rb) {
-            const unsigned char *block = weight_row[rb] + (unsigned long long)sb * 66ull;
-            scale16[rb] = load_u16(block);
+        for (unsigned ks = 0; ks < 3u; ++ks)
+            raw[ks] = *reinterpret_cast<const RawGroup *>(
+                row_aligned + ((block + 2u + 8u * (2u * ks + lane_group)) & ~3u));
+        // The last record of a superblock may be the last bytes of the tensor: its third dword
+        // is read only when it holds bytes of the record (an aligned dword with a valid byte
+        // lies in a mapped page), otherwise the second dword is read again.
+        const unsigned start = block + 2u + 8u * (6u + lane_group);
+        const unsigned char *at = row_aligned + (start & ~3u);
+        const uint2 head = *reinterpret_cast<const uint2 *>(at);
+        raw[3].x = head.x;
+        raw[3].y = head.y;
+        raw[3].z = *reinterpret_cast<const unsigned *>(at + 4u + 2u * (start & 3u));
+    };
+    uint2 now_codes[4];
+    unsigned now_scale16;
+    auto settle_codes = [&](unsigned sb) {   // the registers fetch_codes(sb) filled -> records
+        const unsigned shift = (row_misalign + 2u * sb + 2u) & 3u;
+        now_scale16 = (raw_scale >> (8u * ((row_misalign + 2u * sb) & 3u))) & 0xffffu;
 #pragma unroll
-            for (unsigned ks = 0; ks < 4u; ++ks)
-                codes[rb][ks] = load_u32x2(block + 2u + 8u * (2u * ks + (kb >> 1)));
+        for (unsigned ks = 0; ks < 4u; ++ks) {
+            now_codes[ks].x = __builtin_amdgcn_alignbyte(raw[ks].y, raw[ks].x, shift);
+            now_codes[ks].y = __builtin_amdgcn_alignbyte(raw[ks].z, raw[ks].y, shift);
         }
     };
     // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of token 16 tb + li
@@ -246,31 +297,22 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     copy_activations(0u, 0u);
     fetch_codes(0u);
     __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the copies above have landed in LDS
-    uint2 now_codes[RB][4];
-    unsigned now_scale16[RB];
-#pragma unroll
-    for (unsigned rb = 0; rb < RB; ++rb) {
-        now_scale16[rb] = scale16[rb];
-#pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) now_codes[rb][ks] = codes[rb][ks];
-    }
+    settle_codes(0u);
     __syncthreads();
 
+    const unsigned last = superblocks - 1u;
     for (unsigned sb = 0; sb < superblocks; ++sb) {
         const unsigned base = kStageBase + (sb & 1u) * kStageBytes;
-        if (sb + 1u < superblocks) {
-            copy_activations(sb + 1u, (sb & 1u) ^ 1u);
-            fetch_codes(sb + 1u);
-        }
+        const unsigned ahead = sb < last ? sb + 1u : last;     // the last turn repeats a request
+        copy_activations(ahead, (sb & 1u) ^ 1u);
+        fetch_codes(ahead);
 
-        v4i sum_lo[RB][NB], sum_hi[RB][NB];
+        v4i sum_lo[NB], sum_hi[NB];
 #pragma unroll
-        for (unsigned rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (unsigned tb = 0; tb < NB; ++tb) {
-                sum_lo[rb][tb] = v4i{0, 0, 0, 0};
-                sum_hi[rb][tb] = v4i{0, 0, 0, 0};
-            }
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            sum_lo[tb] = v4i{0, 0, 0, 0};
+            sum_hi[tb] = v4i{0, 0, 0, 0};
+        }
         // Software pipeline over phases (K step, group of up to four token blocks): the
         // activation fragments of the next phase and the table lookups of the next K step are
         // requested before the current phase's matrix instructions are issued, so their LDS
@@ -278,30 +320,31 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         constexpr unsigned kGroups = NB > 4u ? 2u : 1u;      // groups per K step
         constexpr unsigned kGroupSize = NB / kGroups;
         constexpr unsigned kPhases = 4u * kGroups;
-        uint4 looked[RB][4];
+        uint2 codes_of[2], signs_of[2];
+        uint4 limbs_of;
         auto lookup = [&](unsigned ks) {
-#pragma unroll
-            for (unsigned rb = 0; rb < RB; ++rb) {
-                const unsigned grids = now_codes[rb][ks].x >> (16u * (kb & 1u));
-                const unsigned aux = now_codes[rb][ks].y;
-                const unsigned signs = aux >> (14u * (kb & 1u));
-                const unsigned scale_bits = (aux >> 28) << 12;
-                looked[rb][0] = lds_read_uint4(kLimbBase + (scale_bits | ((grids & 255u) << 4)));
-                looked[rb][1] = lds_read_uint4(kLimbBase + (scale_bits | (((grids >> 8) & 255u) << 4)));
-                looked[rb][2] = lds_read_uint4(sign_lane + ((signs & 127u) << 7));
-                looked[rb][3] = lds_read_uint4(sign_lane + (((signs >> 7) & 127u) << 7));
-            }
+            // the lane's sixteen weights: subgroups 2 (kb & 1) and 2 (kb & 1) + 1 of its group
+            const unsigned grids = now_codes[ks].x >> (16u * (kb & 1u));
+            const unsigned aux = now_codes[ks].y;
+            const unsigned signs = aux >> (14u * (kb & 1u));
+            codes_of[0] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0400u));
+            codes_of[1] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0500u));
+            signs_of[0] = lds_read_uint2(((signs << 7) & 0x3f80u) | sel_lane);
+            signs_of[1] = lds_read_uint2((signs & 0x3f80u) | sel_lane);
+            limbs_of = lds_read_uint4(((aux >> 20) & 0xf00u) | lut_lane);
         };
-        v4i a_lo[RB], a_hi[RB];
+        v4i a_lo, a_hi;
         auto weights_from_lookup = [&]() {
-#pragma unroll
-            for (unsigned rb = 0; rb < RB; ++rb) {
-                const uint4 l0 = looked[rb][0], l1 = looked[rb][1], s0 = looked[rb][2], s1 = looked[rb][3];
-                a_lo[rb] = v4i{(int)((l0.x ^ s0.x) + s0.z), (int)((l0.y ^ s0.y) + s0.w),
-                               (int)((l1.x ^ s1.x) + s1.z), (int)((l1.y ^ s1.y) + s1.w)};
-                a_hi[rb] = v4i{(int)((l0.z ^ s0.x) + s0.z), (int)((l0.w ^ s0.y) + s0.w),
-                               (int)((l1.z ^ s1.x) + s1.z), (int)((l1.w ^ s1.y) + s1.w)};
-            }
+            const unsigned s0 = codes_of[0].x | signs_of[0].x, s1 = codes_of[0].y | signs_of[0].y;
+            const unsigned s2 = codes_of[1].x | signs_of[1].x, s3 = codes_of[1].y | signs_of[1].y;
+            a_lo = v4i{(int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s0),
+                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s1),
+                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s2),
+                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s3)};
+            a_hi = v4i{(int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s0),
+                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s1),
+                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s2),
+                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s3)};
         };
         uint4 frags[2][kGroupSize];
         auto request = [&](unsigned phase, uint4 (&into)[kGroupSize]) {
@@ -322,51 +365,37 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 #pragma unroll
             for (unsigned i = 0; i < kGroupSize; ++i) {
                 const unsigned tb = group * kGroupSize + i;
-                const uint4 raw = frags[phase & 1u][i];
-                const v4i b = v4i{(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w};
-#pragma unroll
-                for (unsigned rb = 0; rb < RB; ++rb) {
-                    sum_lo[rb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[rb], b, sum_lo[rb][tb], 0, 0, 0);
-                    sum_hi[rb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[rb], b, sum_hi[rb][tb], 0, 0, 0);
-                }
+                const uint4 rawb = frags[phase & 1u][i];
+                const v4i b = v4i{(int)rawb.x, (int)rawb.y, (int)rawb.z, (int)rawb.w};
+                sum_lo[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, sum_lo[tb], 0, 0, 0);
+                sum_hi[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, sum_hi[tb], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
             if (group == kGroups - 1u && ks + 1u < 4u) weights_from_lookup();
         }
         // ---- exact superblock sums -> fp32 ----
-        float row_scale[RB][4];
+        float row_scale[4];
+        {
+            const float mine = 0.125f * f16_bits_to_float(now_scale16);
 #pragma unroll
-        for (unsigned rb = 0; rb < RB; ++rb) {
-            const float mine = 0.125f * f16_bits_to_float(now_scale16[rb]);
-#pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) row_scale[rb][r] = __shfl(mine, (int)(4u * kb + r), 64);
+            for (unsigned r = 0; r < 4u; ++r) row_scale[r] = __shfl(mine, (int)(4u * kb + r), 64);
         }
 #pragma unroll
         for (unsigned tb = 0; tb < NB; ++tb) {
             const float token_scale =
                 __uint_as_float(lds_read_u32(base + kStageActs + 4u * (tb * 16u + li)));
 #pragma unroll
-            for (unsigned rb = 0; rb < RB; ++rb)
-#pragma unroll
-                for (unsigned r = 0; r < 4u; ++r) {
-                    const int total = (sum_hi[rb][tb][r] << 7) + sum_lo[rb][tb][r];
-                    acc[rb][tb][r] = __builtin_fmaf(row_scale[rb][r] * token_scale, (float)total,
-                                                    acc[rb][tb][r]);
-                }
-        }
-        if (sb + 1u < superblocks) {
-#pragma unroll
-            for (unsigned rb = 0; rb < RB; ++rb) {
-                now_scale16[rb] = scale16[rb];
-#pragma unroll
-                for (unsigned ks = 0; ks < 4u; ++ks) now_codes[rb][ks] = codes[rb][ks];
+            for (unsigned r = 0; r < 4u; ++r) {
+                const int total = (sum_hi[tb][r] << 7) + sum_lo[tb][r];
+                acc[tb][r] = __builtin_fmaf(row_scale[r] * token_scale, (float)total, acc[tb][r]);
             }
-            __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the next stage is complete in LDS
         }
+        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the next stage is complete in LDS
+        settle_codes(ahead);
         __syncthreads();
     }
 
-    // ---- publish: the lane holds C rows 4 kb + r of its blocks for tokens tb * 16 + li ----
+    // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
     auto store4 = [&](unsigned token, unsigned row, const float (&value)[4]) {
         const unsigned long long ordered = it.pair0 + token;
         const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
@@ -385,20 +414,7 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         const unsigned long long source = pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
         return pr.route_weights ? pr.route_weights[source] : 1.0f;
     };
-    if constexpr (FUSED_UP && RB == 2u) {
-#pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            const unsigned token = tb * 16u + li;
-            if (token < it.tokens) {
-                const float route_weight = route_weight_of(token);
-                const float value[4] = {swiglu_bf16(acc[0][tb][0], acc[RB - 1u][tb][0], route_weight, a.limit),
-                                        swiglu_bf16(acc[0][tb][1], acc[RB - 1u][tb][1], route_weight, a.limit),
-                                        swiglu_bf16(acc[0][tb][2], acc[RB - 1u][tb][2], route_weight, a.limit),
-                                        swiglu_bf16(acc[0][tb][3], acc[RB - 1u][tb][3], route_weight, a.limit)};
-                store4(token, out_row_base[0] + 4u * kb, value);
-            }
-        }
-    } else if constexpr (FUSED_UP) {
+    if constexpr (FUSED_UP) {
         // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. They swap token
         // blocks through LDS (the stages are free after the last barrier): gate waves finish
         // blocks [0, G), up waves finish blocks [G, NB).
@@ -410,14 +426,14 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 #pragma unroll
             for (unsigned tb = G; tb < NB; ++tb)
                 lds_write_uint4(slot + ((tb - G) * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[0][tb][0]), __float_as_uint(acc[0][tb][1]),
-                                           __float_as_uint(acc[0][tb][2]), __float_as_uint(acc[0][tb][3])));
+                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
+                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
         } else {
 #pragma unroll
             for (unsigned tb = 0; tb < G; ++tb)
                 lds_write_uint4(slot + (tb * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[0][tb][0]), __float_as_uint(acc[0][tb][1]),
-                                           __float_as_uint(acc[0][tb][2]), __float_as_uint(acc[0][tb][3])));
+                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
+                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
         }
         __syncthreads();
         if (is_gate) {
@@ -428,11 +444,11 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                 if (token < it.tokens) {
                     const float route_weight = route_weight_of(token);
                     const float value[4] = {
-                        swiglu_bf16(acc[0][tb][0], __uint_as_float(other.x), route_weight, a.limit),
-                        swiglu_bf16(acc[0][tb][1], __uint_as_float(other.y), route_weight, a.limit),
-                        swiglu_bf16(acc[0][tb][2], __uint_as_float(other.z), route_weight, a.limit),
-                        swiglu_bf16(acc[0][tb][3], __uint_as_float(other.w), route_weight, a.limit)};
-                    store4(token, out_row_base[0] + 4u * kb, value);
+                        swiglu_bf16(acc[tb][0], __uint_as_float(other.x), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][1], __uint_as_float(other.y), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][2], __uint_as_float(other.z), route_weight, a.limit),
+                        swiglu_bf16(acc[tb][3], __uint_as_float(other.w), route_weight, a.limit)};
+                    store4(token, out_row_base + 4u * kb, value);
                 }
             }
         } else {
@@ -443,32 +459,29 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                 if (token < it.tokens) {
                     const float route_weight = route_weight_of(token);
                     const float value[4] = {
-                        swiglu_bf16(__uint_as_float(other.x), acc[0][tb][0], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.y), acc[0][tb][1], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.z), acc[0][tb][2], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.w), acc[0][tb][3], route_weight, a.limit)};
-                    store4(token, out_row_base[0] + 4u * kb, value);
+                        swiglu_bf16(__uint_as_float(other.x), acc[tb][0], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.y), acc[tb][1], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.z), acc[tb][2], route_weight, a.limit),
+                        swiglu_bf16(__uint_as_float(other.w), acc[tb][3], route_weight, a.limit)};
+                    store4(token, out_row_base + 4u * kb, value);
                 }
             }
         }
     } else {
 #pragma unroll
-        for (unsigned rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (unsigned tb = 0; tb < NB; ++tb) {
-                const unsigned token = tb * 16u + li;
-                if (token < it.tokens) {
-                    const float value[4] = {bf16_round(acc[rb][tb][0]), bf16_round(acc[rb][tb][1]),
-                                            bf16_round(acc[rb][tb][2]), bf16_round(acc[rb][tb][3])};
-                    store4(token, out_row_base[rb] + 4u * kb, value);
-                }
+        for (unsigned tb = 0; tb < NB; ++tb) {
+            const unsigned token = tb * 16u + li;
+            if (token < it.tokens) {
+                const float value[4] = {bf16_round(acc[tb][0]), bf16_round(acc[tb][1]),
+                                        bf16_round(acc[tb][2]), bf16_round(acc[tb][3])};
+                store4(token, out_row_base + 4u * kb, value);
             }
+        }
     }
 }
 
-template <bool FUSED_UP, unsigned RB>
-__global__ __launch_bounds__(512u / RB) __attribute__((amdgpu_waves_per_eu(1, 3 - RB)))
-void mfma_iq2_kernel(MfmaArgs a)
+template <bool FUSED_UP>
+__global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
 {
     extern __shared__ __align__(16) unsigned char mfma_lds[];
     if (lds_address_of(mfma_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
@@ -530,10 +543,10 @@ void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u, RB>(a, it);
-        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u, RB>(a, it);
-        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u, RB>(a, it);
-        else mfma_item<FUSED_UP, 8u, RB>(a, it);
+        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
+        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
+        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
+        else mfma_item<FUSED_UP, 8u>(a, it);
     }
 }
 
@@ -552,37 +565,18 @@ static int mfma_grid()
     return units;
 }
 
-// Row blocks per wave; see mfma_item. YVEX_MFMA_ROW_BLOCKS=1|2 in the environment overrides the
-// default for experiments.
-static unsigned mfma_row_blocks()
-{
-    static unsigned value = 0u;
-    if (!value) {
-        const char *text = getenv("YVEX_MFMA_ROW_BLOCKS");
-        value = (text && text[0] == '2') ? 2u : 1u;
-    }
-    return value;
-}
-
-template <bool FUSED_UP, unsigned RB>
-static int launch_mfma_rb(const MfmaArgs &a, hipStream_t stream)
+template <bool FUSED_UP>
+static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
 {
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP, RB>,
+        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsBytes) != hipSuccess)
             (void)hipGetLastError();
         configured = true;
     }
-    mfma_iq2_kernel<FUSED_UP, RB><<<mfma_grid(), 512u / RB, kMfmaLdsBytes, stream>>>(a);
+    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), 512u, kMfmaLdsBytes, stream>>>(a);
     return check_launch("moe_rows_mfma");
-}
-
-template <bool FUSED_UP>
-static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
-{
-    return mfma_row_blocks() == 2u ? launch_mfma_rb<FUSED_UP, 2u>(a, stream)
-                                   : launch_mfma_rb<FUSED_UP, 1u>(a, stream);
 }
 
 }  // namespace yvex
