@@ -135,3 +135,60 @@ def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, 
     assert outside.mean() < 2e-2
     terms = np.abs(pair_out.reshape(rows, topk, hidden)).sum(axis=1) + np.abs(shared)
     assert np.all(err[outside] <= 2 * BF16_ULP * terms[outside] + 1e-4)
+
+
+@pytest.mark.parametrize("matrix_cores", [False, True])
+@pytest.mark.parametrize("block", [0, 5])
+def test_expert_kernels_single_superblock_is_bit_exact(gpu, oracle, matrix_cores, block):
+    """With activations that are zero outside one 256-column superblock every output is a single
+    term ((0.125 d_w) d_a) T, so there is no summation order left: the expert kernels (decode
+    sweeps and matrix-core row batches) must equal the CPU path bit for bit, which pins their
+    exact int32 superblock sums T through the real hot path."""
+    from yvex_amd import kernels as K
+    hidden, intermediate, experts, topk, rows = 2048, 2048, 6, 4, 20
+    layer, h = make_layer(oracle, gpu, hidden=hidden, intermediate=intermediate, experts=experts,
+                          topk=topk, rows=rows, qtype="IQ2_XXS", act_q8=True, scoring=1,
+                          matrix_cores=matrix_cores)
+    qt = h["qt"]
+    x = np.zeros_like(h["x"])
+    x[:, 256 * block:256 * (block + 1)] = h["x"][:, 256 * block:256 * (block + 1)]
+    layer.run(dev(x, gpu), dev(h["logits"], gpu))
+    torch.cuda.synchronize()
+    assert int(layer.status.item()) == 0
+    pairs = rows * topk
+    sel = layer.selected.cpu().numpy().reshape(-1)
+    wts = layer.weights.cpu().numpy().reshape(-1)
+    order = layer.worklist.order.cpu().numpy()[:pairs]
+    mid = layer.intermediate_f32.cpu().numpy()[:pairs]
+    gb = oracle.row_bytes(qt, hidden) * intermediate
+    db = oracle.row_bytes(qt, intermediate) * hidden
+    for position in range(pairs):
+        source = int(order[position])
+        row, e = source // topk, int(sel[source])
+        rc, _, want_mid, _ = oracle.moe_expert(
+            (qt, qt, qt), h["gate"][e * gb:(e + 1) * gb], h["up"][e * gb:(e + 1) * gb],
+            h["down"][e * db:(e + 1) * db], hidden, intermediate, x[row], float(wts[source]),
+            act_q8=True)
+        assert rc == 0
+        assert np.array_equal(mid[position], want_mid), f"pair {position}"
+
+    # the down projection on an intermediate with one live superblock per pair
+    crafted = np.zeros((pairs, intermediate), np.float32)
+    crafted[:, 256 * block:256 * (block + 1)] = oracle.Generator(7, "crafted").normal(pairs * 256).reshape(pairs, 256)
+    st = layer.status
+    q = K.q8k_quantize(dev(crafted, gpu), st)
+    if matrix_cores:
+        K.moe_down_rows(layer.routed, q, layer.worklist, pairs, experts, layer.pair_outputs, st)
+    else:
+        K.moe_down(layer.routed, q, True, layer.worklist, pairs, experts, layer.pair_outputs, st)
+    torch.cuda.synchronize()
+    assert int(st.item()) == 0
+    pair_out = layer.pair_outputs.cpu().numpy()[:pairs]
+    q_host = q.cpu().numpy().reshape(pairs, -1)
+    for position in range(pairs):
+        source = int(order[position])
+        e = int(sel[source])
+        raw = oracle.q8_matvec(qt, h["down"][e * db:(e + 1) * db], hidden, intermediate,
+                               q_host[position], 1)[0]
+        want = np.array([oracle.lib().yvo_bf16_round(np.float32(v)) for v in raw], np.float32)
+        assert np.array_equal(pair_out[source], want), f"pair {position}"
