@@ -53,17 +53,43 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
                                           unsigned u, Unit &unit)
 {
     const unsigned sb = u >> 3, g = u & 7u;
+    // Group records and Q8_0 blocks start on 2-byte boundaries, and vector loads that are not
+    // dword-aligned run at under half rate on this part: load the aligned dwords that hold the
+    // bytes and shift them into place. A dword is only read when it holds a byte of the record
+    // (so it lies in a mapped page); rows on odd addresses take the byte-granular path.
     if constexpr (QT == QT_IQ2_XXS) {
-        uint2 packed = load_u32x2(row + sb * 66u + 2u + 8u * g);
+        const unsigned char *p = row + sb * 66u + 2u + 8u * g;
+        uint2 packed;
+        if (((unsigned long long)row & 1ull) == 0ull) {
+            const unsigned shift = (unsigned)(unsigned long long)p & 3u;       // 0 or 2
+            const unsigned char *at = p - shift;
+            const uint2 head = *reinterpret_cast<const uint2 *>(at);
+            const unsigned tail = *reinterpret_cast<const unsigned *>(at + 4u + 2u * shift);
+            packed.x = __builtin_amdgcn_alignbyte(head.y, head.x, shift);
+            packed.y = __builtin_amdgcn_alignbyte(tail, head.y, shift);
+        } else {
+            packed = load_u32x2(p);
+        }
         unit.factor = unit.factor2 = iq2_unit(tables, packed.x, packed.y, unit.w);
         unit.min1 = unit.min2 = 0;
     } else if constexpr (QT == QT_Q8_0) {
         const unsigned char *b = row + u * 34u + 2u;
+        if (((unsigned long long)row & 1ull) == 0ull) {
+            const unsigned shift = (unsigned)(unsigned long long)b & 3u;       // 0 or 2
+            const unsigned char *at = b - shift;
+            const uint4 lo = *reinterpret_cast<const uint4 *>(at);
+            const uint4 hi = *reinterpret_cast<const uint4 *>(at + 16u);
+            const unsigned tail = *reinterpret_cast<const unsigned *>(at + 28u + 2u * shift);
+            const unsigned raw[9] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w, tail};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint2 v = load_u32x2(b + 8 * i);
-            unit.w[2 * i] = v.x;
-            unit.w[2 * i + 1] = v.y;
+            for (int i = 0; i < 8; ++i) unit.w[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint2 v = load_u32x2(b + 8 * i);
+                unit.w[2 * i] = v.x;
+                unit.w[2 * i + 1] = v.y;
+            }
         }
         unit.factor = unit.factor2 = 1;
         unit.min1 = unit.min2 = 0;
