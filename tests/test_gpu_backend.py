@@ -272,6 +272,27 @@ def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, sh
     assert res.kernel_launches >= 8 and res.memory.complete == 1
 
 
+def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle):
+    """Row batches whose buckets average eight pairs or more run the int8 matrix-core kernels
+    (routed and shared expert); the result is the CPU layer's, to the same bar."""
+    case = MoeCase(backend, oracle, qtype="IQ2_XXS", hidden=768, intermediate=512, experts=4, topk=2,
+                   rows=200, scoring=abi.SCORING_SIGMOID)
+    backend.workspace(case.workspace_bytes)
+    rc = case.execute()
+    assert rc == 0, case.err.message
+    want = case.oracle_layer(act_q8=True)
+    assert np.array_equal(case.sel.reshape(case.rows, case.topk), want["selected"])
+    got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+    err = np.abs(got.astype(np.float64) - want["combined"])
+    outside = err > 1e-5 + 1e-3 * np.abs(want["combined"])
+    assert outside.mean() < 2e-2
+    # a one-step bf16 flip of a summed term; terms are of the size of the row's largest outputs
+    row_scale = np.abs(want["combined"]).max(axis=1, keepdims=True) * np.ones_like(want["combined"])
+    assert np.all(err[outside] <= 2 * 2.0 ** -7 * np.abs(want["combined"][outside]) +
+                  2.0 ** -8 * row_scale[outside] + 1e-4)
+    assert case.result.row_expert_pairs == 400 and case.result.completed == 1
+
+
 def test_execute_rows_refusals(backend, oracle):
     b = backend
     case = MoeCase(b, oracle)

@@ -222,7 +222,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     unsigned long long base, pairs, hidden, experts, topk, row_count, launches = 0ull;
     unsigned long long router_address = 0ull, bias_address = 0ull, addresses[6] = {0};
     unsigned long long d2h = 0ull, started, counts[4] = {0};
-    int unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, device_status = 0, rc, defer;
+    int unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
     if (result) memset(result, 0, sizeof(*result));
@@ -322,7 +322,15 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         fill_expert_weights(&shared, &views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
                             &views[YVEX_MOE_WEIGHT_SHARED_DOWN], addresses[3], addresses[4], addresses[5],
                             hidden, layer->shared_intermediate_width);
-    merged = has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
+    /* Row batches whose buckets average eight pairs or more go to the int8 matrix-core kernels
+     * (IQ2_XXS weights, Q8_K activations); below that the decode sweeps, which read an expert's
+     * bytes once per four pairs, are faster. The reference switches its tensor-core kernels on
+     * from 16 input rows (src/backend/cuda/private.h:461-464). */
+    row_batch = routed_q8 && routed.gate_qtype == 16u && routed.up_qtype == 16u &&
+                routed.down_qtype == 16u && pairs >= 8ull * experts;
+    shared_row_batch = row_batch && has_shared && shared_q8 && shared.gate_qtype == 16u &&
+                       shared.up_qtype == 16u && shared.down_qtype == 16u;
+    merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",
                                 "kernel launch failed (test seam)");
@@ -362,6 +370,15 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     if (routed_q8 || (has_shared && shared_q8))
         LAUNCH(yvex_hip_q8k_quantize((const float *)rows->device_rows->data, row_count, hidden, hidden,
                                      (uint8_t *)AT(input_q8), (int *)status, stream), "rocm.moe.rows.q8");
+    if (row_batch)
+        LAUNCH(yvex_hip_moe_up_rows(&routed, AT(input_q8), (const float *)AT(weights),
+                                    (const uint64_t *)AT(order), (const uint64_t *)AT(expert_ids),
+                                    (const uint64_t *)AT(bucket_offsets),
+                                    (const uint64_t *)AT(bucket_populations), (const uint64_t *)AT(counts),
+                                    pairs, topk, experts, layer->activation_limit,
+                                    (float *)AT(intermediate), (int *)status, stream),
+               "rocm.moe.rows.up-matrix");
+    else
     LAUNCH(yvex_hip_moe_up(&routed, routed_q8 ? AT(input_q8) : (void *)rows->device_rows->data, routed_q8,
                            (const float *)AT(weights), (const uint64_t *)AT(order),
                            (const uint64_t *)AT(expert_ids), (const uint64_t *)AT(bucket_offsets),
@@ -370,7 +387,11 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                            (float *)AT(intermediate), merged ? &shared : NULL, merged ? row_count : 0ull,
                            merged ? (float *)AT(shared_intermediate) : NULL, (int *)status, stream),
            "rocm.moe.rows.up");
-    if (has_shared && !merged)
+    if (shared_row_batch)
+        LAUNCH(yvex_hip_moe_up_rows(&shared, AT(input_q8), NULL, NULL, NULL, NULL, NULL, NULL, row_count,
+                                    1ull, 1ull, layer->activation_limit, (float *)AT(shared_intermediate),
+                                    (int *)status, stream), "rocm.moe.rows.shared-up-matrix");
+    else if (has_shared && !merged)
         LAUNCH(yvex_hip_moe_up(&shared, shared_q8 ? AT(input_q8) : (void *)rows->device_rows->data,
                                shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull, 1ull,
                                layer->activation_limit, (float *)AT(shared_intermediate), NULL, 0ull, NULL,
@@ -384,6 +405,13 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                      layer->shared_intermediate_width, layer->shared_intermediate_width,
                                      (uint8_t *)AT(shared_intermediate_q8), (int *)status, stream),
                "rocm.moe.rows.q8-shared-mid");
+    if (row_batch)
+        LAUNCH(yvex_hip_moe_down_rows(&routed, AT(intermediate_q8), (const uint64_t *)AT(order),
+                                      (const uint64_t *)AT(expert_ids), (const uint64_t *)AT(bucket_offsets),
+                                      (const uint64_t *)AT(bucket_populations), (const uint64_t *)AT(counts),
+                                      pairs, experts, (float *)AT(pair_outputs), (int *)status, stream),
+               "rocm.moe.rows.down-matrix");
+    else
     LAUNCH(yvex_hip_moe_down(&routed, routed_q8 ? AT(intermediate_q8) : AT(intermediate), routed_q8,
                              (const uint64_t *)AT(order), (const uint64_t *)AT(expert_ids),
                              (const uint64_t *)AT(bucket_offsets), (const uint64_t *)AT(bucket_populations),
@@ -393,7 +421,11 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                              merged ? (shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate)) : NULL,
                              merged ? (float *)AT(shared_outputs) : NULL, (int *)status, stream),
            "rocm.moe.rows.down");
-    if (has_shared && !merged)
+    if (shared_row_batch)
+        LAUNCH(yvex_hip_moe_down_rows(&shared, AT(shared_intermediate_q8), NULL, NULL, NULL, NULL, NULL,
+                                      row_count, 1ull, (float *)AT(shared_outputs), (int *)status, stream),
+               "rocm.moe.rows.shared-down-matrix");
+    else if (has_shared && !merged)
         LAUNCH(yvex_hip_moe_down(&shared, shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate),
                                  shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull,
                                  (float *)AT(shared_outputs), NULL, 0ull, NULL, NULL, (int *)status, stream),
