@@ -77,6 +77,18 @@ def cpu_baseline(sample_rows: int, threads: int):
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
 
 
+def tile_classes(populations):
+    """128-pair tiles of the row-batch kernels by the number of 16-pair blocks they run with."""
+    out = {"1": 0, "2": 0, "4": 0, "8": 0}
+    for n in populations:
+        full, rest = divmod(int(n), 128)
+        out["8"] += full
+        if rest:
+            blocks = (rest + 15) // 16
+            out["1" if blocks <= 1 else "2" if blocks <= 2 else "4" if blocks <= 4 else "8"] += 1
+    return out
+
+
 def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: int):
     """BASELINE config 4: the same layer over 2048 rows whose top-8 experts follow a Zipf(1.1)
     popularity (Gumbel top-k over log-popularity logits), row-batch kernels on the int8 matrix
@@ -118,6 +130,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
         "int8_TOPs": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12, 2),
         "mfma_peak_frac": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
         "distinct_routed_experts": int(populations.numel()),
+        "token_tiles": tile_classes(populations.cpu().tolist()),
         "max_bucket_population": int(populations.max().item()),
         "roofline": {"bound": "mfma", "kernel": "mfma_iq2_kernel<fused gate/up>",
                      "achieved": round(up_ops / (up_ms * 1e-3) / 1e12, 2), "peak": MFMA_INT8_PEAK_TOPS,

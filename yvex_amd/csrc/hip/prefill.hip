@@ -36,14 +36,23 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr unsigned kTileTokens = 128u;
 constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
-constexpr unsigned kCodeBase = 0u;                          // 256 entries x 32 replicas x 8 bytes
-constexpr unsigned kSelBase = 65536u;                       // 128 entries x 16 replicas x 8 bytes
-constexpr unsigned kLutBase = kSelBase + 128u * 16u * 8u;   // 16 scales x 16 replicas x 16 bytes
+// LDS map. Codebook entry e owns the 256 bytes at 256 e: sixteen replicas of its 8 level codes
+// in the first half; the second half of entries 0-127 holds sixteen replicas of the sign
+// selectors of sign field e.
+constexpr unsigned kCodeBase = 0u;
+constexpr unsigned kSelBase = 128u;
+constexpr unsigned kLutBase = 65536u;                       // 16 scales x 16 replicas x 16 bytes
 constexpr unsigned kStageBase = kLutBase + 16u * 16u * 16u;
 constexpr unsigned kStageActs = kTileTokens * kActPitch;
 constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per token
-constexpr unsigned kTileStartBase = kStageBase + 2u * kStageBytes;
-constexpr unsigned kMfmaLdsBytes = kTileStartBase + 260u * 4u;
+// Weight windows: per wave two slots; a slot holds, for each of the wave's 16 rows, the 80
+// bytes (five 16-byte pieces) around one superblock. Rows 0-11 lie at 80 r, rows 12-15 at
+// 1024 + 80 (r - 12): the two copies that fill a slot each write lane * 16.
+constexpr unsigned kWeightBase = kStageBase + 2u * kStageBytes;
+constexpr unsigned kWeightSlot = 1024u + 4u * 80u;
+constexpr unsigned kTileStartBase = kWeightBase + 8u * 2u * kWeightSlot;
+constexpr unsigned kTrashBase = kTileStartBase + 260u * 4u;   // 256 bytes nobody reads
+constexpr unsigned kMfmaLdsBytes = kTrashBase + 256u;
 
 struct MfmaArgs {
     GroupedProblem pr;
@@ -69,6 +78,17 @@ __device__ __forceinline__ void lds_write_u32(unsigned address, unsigned v)
 #else
     (void)address;
     (void)v;
+#endif
+}
+// One 16-byte LDS read as a vector value (a struct of four words may reach the backend as four
+// scalar loads and come out as two 8-byte reads).
+__device__ __forceinline__ v4i lds_read_v4i(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const v4i *>(address);
+#else
+    (void)address;
+    return v4i{0, 0, 0, 0};
 #endif
 }
 __device__ __forceinline__ unsigned lds_read_u32(unsigned address)
@@ -107,6 +127,20 @@ __device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_b
 #endif
 }
 
+// The same 16-byte copy for lanes 0-19 only (the other lanes neither read nor write).
+__device__ __forceinline__ void copy_to_lds_16_first20(const void *global, unsigned lds_base)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    unsigned long long saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xfffff\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "s"(lds_base), "v"(global) : "memory");
+#else
+    (void)global;
+    (void)lds_base;
+#endif
+}
+
 // Limb pair of one magnitude: low limb in bits 0-7, high limb in bits 8-15.
 __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
 {
@@ -130,8 +164,8 @@ __device__ __forceinline__ void lds_write_uint2(unsigned address, uint2 v)
 __device__ __forceinline__ void mfma_tables_fill()
 {
     // level codes: byte l of the entry is 0, 1 or 2 for level 8, 25 or 43 of weight l
-    for (unsigned index = threadIdx.x; index < 256u * 32u; index += blockDim.x) {
-        const uint2 m = iq2_magnitude_entry(index >> 5);
+    for (unsigned index = threadIdx.x; index < 256u * 16u; index += blockDim.x) {
+        const uint2 m = iq2_magnitude_entry(index >> 4);
         uint2 codes = make_uint2(0u, 0u);
 #pragma unroll
         for (unsigned l = 0; l < 4u; ++l) {
@@ -139,12 +173,13 @@ __device__ __forceinline__ void mfma_tables_fill()
             codes.x |= (a == 8u ? 0u : a == 25u ? 1u : 2u) << (8u * l);
             codes.y |= (b == 8u ? 0u : b == 25u ? 1u : 2u) << (8u * l);
         }
-        lds_write_uint2(kCodeBase + index * 8u, codes);
+        lds_write_uint2(kCodeBase + (index >> 4) * 256u + (index & 15u) * 8u, codes);
     }
     // sign selectors: byte l is 4 when weight l is negative (7 stored bits + parity)
     for (unsigned index = threadIdx.x; index < 128u * 16u; index += blockDim.x) {
         const uint2 m = iq2_signmask_entry(index >> 4);
-        lds_write_uint2(kSelBase + index * 8u, make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
+        lds_write_uint2(kSelBase + (index >> 4) * 256u + (index & 15u) * 8u,
+                        make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
     }
     // limb words of scale s: {+lo, -lo, +hi, -hi}, byte c = limb of level code c
     for (unsigned index = threadIdx.x; index < 16u * 16u; index += blockDim.x) {
@@ -175,28 +210,55 @@ struct alignas(4) RawGroup {
     unsigned x, y, z;
 };
 
+// The lane's four group records and block scale of one superblock of its weight row.
+struct Codes {
+    uint2 c[4];
+    unsigned scale16;
+};
+// Table words of the lane's sixteen weights in one K step.
+struct Lookup {
+    uint2 codes[2], signs[2];
+    uint4 limbs;
+};
+
 // One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8). Eight waves, two per SIMD, each
-// owning one 16-row block. Every loop below has a fixed trip count and the superblock body is one
-// basic block (requests past the end are clamped, not guarded), so accumulators never leave
-// registers and the compiler's wait counts stay exact.
+// owning one 16-row block.
+//
+// The stage in LDS holds 128 "slots" of 256 activation bytes + one scale. An item with fewer than
+// 128 tokens fills them with S consecutive superblocks of its NB * 16 tokens (slot = superblock
+// within the period * NB * 16 + token), so that every period between two barriers carries about
+// the same matrix work and the same copies whatever NB is.
+//
+// A step is one superblock. Its instruction stream is laid out by hand as 4 * NB slots of two
+// matrix instructions (low and high limb of one K step of one token block), and between them,
+// a few vector instructions at a time, everything else: the scaling of the previous token
+// block's integer sums into the fp32 accumulators, the table lookups and byte permutes that
+// build the next superblock's A operands, the LDS reads of the next token block's fragments.
+// The loop body holds D steps back to back in one basic block (requests past the end are
+// clamped, and steps past the end run with a zero row scale), so the compiler's wait counts stay
+// exact and accumulators never leave registers.
 template <bool FUSED_UP, unsigned NB>
 __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
     constexpr unsigned kWaves = 8u;
+    constexpr unsigned S = NB >= 8u ? 1u : NB == 4u ? 2u : 4u;   // superblocks per stage period
+    constexpr unsigned D = S < 2u ? 2u : S;                      // steps per loop turn (even)
+    constexpr unsigned T = NB * 16u;                             // token slots of one superblock
+    constexpr unsigned kStagedSlots = S * T;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned li = lane & 15u, kb = lane >> 4;
     constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
-    constexpr unsigned kStagedTokens = NB * 16u;
-    const unsigned code_lane = kCodeBase + (lane & 31u) * 8u;
+    const unsigned code_lane = kCodeBase + (lane & 15u) * 8u;
     const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
     const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
     const unsigned superblocks = a.width >> 8;
+    const unsigned last = superblocks - 1u;
 
-    // ---- activation rows this lane copies: wave w owns the 4-token groups w, w + kWaves, ... ----
-    // Lane l of a group moves piece position l % 16 of token 4 g + l / 16; LDS receives the
-    // wave's 64 pieces back to back, so the swizzle is applied on the global side.
-    constexpr unsigned kCopies = (kStagedTokens / 4u + kWaves - 1u) / kWaves;
+    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + kWaves, ... ----
+    // Lane l of a group moves piece position l % 16 of slot 4 g + l / 16; LDS receives the wave's
+    // 64 pieces back to back, so the swizzle is applied on the global side.
+    constexpr unsigned kCopies = kStagedSlots / (4u * kWaves);
     auto token_row = [&](unsigned token) {
         const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
         const unsigned long long ordered = it.pair0 + live;
@@ -205,39 +267,165 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         return (const unsigned char *)pr.activations + arow * pr.act_stride;
     };
     const unsigned char *copy_from[kCopies];
+    unsigned copy_step[kCopies];            // superblock of the slot within its period
 #pragma unroll
     for (unsigned j = 0; j < kCopies; ++j) {
-        const unsigned token = 4u * (wave + kWaves * j) + (lane >> 4);
+        const unsigned slot = 4u * (wave + kWaves * j) + (lane >> 4);
+        const unsigned token = slot % T;
+        copy_step[j] = slot / T;
         copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
     }
-    // waves 0 and 1 also copy the block scales of tokens 64 w + lane
-    const unsigned char *scale_from = token_row(64u * (wave & 1u) + lane);
+    // Waves 0 and 1 also copy the 128 slot scales. The other waves run the same instruction on
+    // one address for all lanes (one cache line: next to free) into bytes nobody reads, which is
+    // cheaper than a branch around the copy.
+    const unsigned scale_slot = wave < 2u ? 64u * wave + lane : 0u;
+    const unsigned char *scale_from = token_row(scale_slot % T);
+    const unsigned scale_step = scale_slot / T;
+    const unsigned scale_to = wave < 2u ? kStageActs + wave * 256u : 0xffffffffu;
 
     // ---- the weight row of this lane: waves 0-3 hold gate blocks and waves 4-7 the matching up
     // blocks when the SwiGLU is fused ----
     unsigned out_row_base;
-    const unsigned char *weight_row;
-    {
-        bool is_up = false;
-        if constexpr (FUSED_UP) {
-            out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
-            is_up = wave >= 4u;
-        } else {
-            out_row_base = it.row_tile * kItemRows + wave * 16u;
-        }
-        unsigned row = out_row_base + li;
+    bool is_up = false;
+    if constexpr (FUSED_UP) {
+        out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
+        is_up = wave >= 4u;
+    } else {
+        out_row_base = it.row_tile * kItemRows + wave * 16u;
+    }
+    auto row_pointer = [&](unsigned r) {     // weight row r of the wave's 16
+        unsigned row = out_row_base + r;
         if (row >= a.out_rows) row = a.out_rows - 1u;
-        weight_row = is_up
+        return is_up
             ? pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
             : pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
-    }
-    // Superblocks are 66 bytes, so group records start on 2-byte boundaries, and vector loads
-    // that are not dword-aligned run at less than half rate: the lane loads twelve aligned bytes
-    // around each record and shifts them into place. Records of superblock sb start
-    // (row start + 2 sb + 2) mod 4 bytes past a dword, the fp16 scale (row start + 2 sb) mod 4.
-    const unsigned row_misalign = (unsigned)(unsigned long long)weight_row & 3u;
-    const unsigned char *row_aligned = weight_row - row_misalign;
+    };
+    // Superblocks are 66 bytes, so they start on 2-byte boundaries, and vector loads that are
+    // not dword-aligned run at less than half rate. The wave copies, for each of its rows, the
+    // aligned 68 bytes that hold the superblock into its LDS slot, as five 16-byte pieces (the
+    // fifth one ends with those 68 bytes, so nothing past the dword that holds the superblock's
+    // last byte is touched: an aligned dword with a valid byte lies in a mapped page). Two
+    // copies fill a slot: lanes 0-59 of the first serve rows 0-11, lanes 0-19 of the second
+    // rows 12-15. Every row is fetched once per step by five lanes instead of by all four lane
+    // groups record by record: the memory pipeline's cost per instruction grows with the number
+    // of cache lines it touches.
+    const unsigned row_misalign = (unsigned)(unsigned long long)row_pointer(li) & 3u;   // of the lane's own row
     const unsigned lane_group = kb >> 1;                      // groups 2 ks + lane_group
+    const unsigned char *window_from[2];    // aligned row start + piece offset, of the row this lane copies
+    unsigned window_misalign[2];
+#pragma unroll
+    for (unsigned c = 0; c < 2u; ++c) {
+        const unsigned served = c == 0u ? (lane < 60u ? lane : 0u) : (lane < 20u ? 60u + lane : 60u);
+        const unsigned piece_index = served % 5u;
+        const unsigned char *from = row_pointer(served / 5u);
+        window_misalign[c] = (unsigned)(unsigned long long)from & 3u;
+        window_from[c] = from - window_misalign[c] + (piece_index < 4u ? 16u * piece_index : 52u);
+    }
+    const unsigned weight_slots = kWeightBase + wave * 2u * kWeightSlot;
+    const unsigned row_at = li < 12u ? li * 80u : 1024u + (li - 12u) * 80u;   // of the lane's row in a slot
+    // The copies and loads of a step are issued one piece at a time between its matrix
+    // instructions: a burst of them fills the memory pipeline's queue and holds the wave, and
+    // with it its matrix instructions, until the queue drains.
+    constexpr unsigned kCopyPieces = kCopies + 1u;
+    auto copy_piece = [&](unsigned period, unsigned stage, unsigned j) {
+        const unsigned base = kStageBase + stage * kStageBytes;
+        if (j < kCopies) {
+            unsigned sb = period * S + copy_step[j];
+            sb = sb < last ? sb : last;
+            copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(base + (wave + kWaves * j) * 1024u)));
+        } else {
+            unsigned sb = period * S + scale_step;
+            sb = sb < last ? sb : last;
+            copy_to_lds_4(scale_from + (unsigned long long)sb * kQ8KBytes,
+                          (unsigned)__builtin_amdgcn_readfirstlane(
+                              (int)(scale_to != 0xffffffffu ? base + scale_to : kTrashBase)));
+        }
+    };
+    auto copy_activations = [&](unsigned period, unsigned stage) {
+#pragma unroll
+        for (unsigned j = 0; j < kCopyPieces; ++j) copy_piece(period, stage, j);
+    };
+    constexpr unsigned kFetchPieces = 2u;
+    auto fetch_piece = [&](unsigned slot, unsigned sb, unsigned c) {
+        sb = sb < last ? sb : last;
+        const unsigned char *from = window_from[c] + ((window_misalign[c] + sb * 66u) & ~3u);
+        const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane((int)(weight_slots + slot * kWeightSlot + c * 1024u));
+        if (c == 0u) copy_to_lds_16(from, to);
+        else copy_to_lds_16_first20(from, to);
+    };
+    auto fetch_codes = [&](unsigned slot, unsigned sb) {
+#pragma unroll
+        for (unsigned c = 0; c < kFetchPieces; ++c) fetch_piece(slot, sb, c);
+    };
+    // Records of superblock sb out of the slot fetch_codes(slot, sb) filled. With o = (row start
+    // + 2 sb) mod 4 (0 or 2) the fp16 scale sits o bytes into the window and the record of group
+    // G at o + 2 + 8 G: in dwords 2 G (+1 when o is 2), shifted by 2 bytes when o is 0. Window
+    // dword 16 is the last dword of the fifth piece.
+    auto settle_codes = [&](unsigned slot, unsigned sb) {
+        sb = sb < last ? sb : last;
+        Codes out;
+        const unsigned o = (row_misalign + 2u * sb) & 3u;
+        const unsigned shift = (o + 2u) & 3u;
+        const unsigned row_base = weight_slots + slot * kWeightSlot + row_at;
+        const unsigned first = row_base + 8u * lane_group + (o & 2u) * 2u;    // dword 2 g (+1) of the window
+        out.scale16 = (lds_read_u32(row_base) >> (8u * o)) & 0xffffu;
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks) {
+            unsigned x, y, z;
+            if (ks < 3u) {
+                x = lds_read_u32(first + 16u * ks);
+                y = lds_read_u32(first + 16u * ks + 4u);
+                z = lds_read_u32(first + 16u * ks + 8u);
+            } else {
+                // dwords 12 + 2 g (+1) and the two behind it; 16 lives 12 bytes further on, and
+                // 17 is never part of a record (it is read as 16 and shifted out)
+                const unsigned d0 = 12u + 2u * lane_group + (o >> 1);
+                const unsigned d1 = d0 + 1u, d2 = d0 + 2u < 16u ? d0 + 2u : 16u;
+                x = lds_read_u32(row_base + 4u * d0);
+                y = lds_read_u32(row_base + 4u * d1 + (d1 == 16u ? 12u : 0u));
+                z = lds_read_u32(row_base + 4u * d2 + (d2 == 16u ? 12u : 0u));
+            }
+            out.c[ks].x = __builtin_amdgcn_alignbyte(y, x, shift);
+            out.c[ks].y = __builtin_amdgcn_alignbyte(z, y, shift);
+        }
+        return out;
+    };
+    // the lane's sixteen weights of K step ks: subgroups 2 (kb & 1) and 2 (kb & 1) + 1 of its group
+    auto lookup = [&](const Codes &codes, unsigned ks) {
+        Lookup out;
+        const unsigned grids = codes.c[ks].x >> (16u * (kb & 1u));
+        const unsigned aux = codes.c[ks].y;
+        const unsigned signs = aux >> (14u * (kb & 1u));
+        out.codes[0] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0400u));
+        out.codes[1] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0500u));
+        out.signs[0] = lds_read_uint2(((signs << 8) & 0x7f00u) | sel_lane);
+        out.signs[1] = lds_read_uint2(((signs << 1) & 0x7f00u) | sel_lane);
+        out.limbs = lds_read_uint4(((aux >> 20) & 0xf00u) | lut_lane);
+        return out;
+    };
+    auto weights_from_lookup = [&](const Lookup &lk, v4i &a_lo, v4i &a_hi) {
+        const unsigned s0 = lk.codes[0].x | lk.signs[0].x, s1 = lk.codes[0].y | lk.signs[0].y;
+        const unsigned s2 = lk.codes[1].x | lk.signs[1].x, s3 = lk.codes[1].y | lk.signs[1].y;
+        a_lo = v4i{(int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s0),
+                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s1),
+                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s2),
+                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s3)};
+        a_hi = v4i{(int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s0),
+                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s1),
+                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s2),
+                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s3)};
+    };
+    // fp32 scales of C rows 4 kb + r of superblock sb (zero past the end: such steps add nothing)
+    auto row_scales = [&](const Codes &codes, unsigned sb, float (&out)[4]) {
+        const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(codes.scale16) : 0.0f;
+#pragma unroll
+        for (unsigned r = 0; r < 4u; ++r) out[r] = __shfl(mine, (int)(4u * kb + r), 64);
+    };
+    // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of slot 16 b + li
+    unsigned piece[4];
+#pragma unroll
+    for (unsigned ks = 0; ks < 4u; ++ks) piece[ks] = li * kActPitch + (((4u * ks + kb) ^ li) << 4);
 
     float acc[NB][4];
 #pragma unroll
@@ -245,155 +433,163 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 #pragma unroll
         for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
 
-    RawGroup raw[4];
-    unsigned raw_scale;
-    auto copy_activations = [&](unsigned sb, unsigned stage) {
-        const unsigned base = kStageBase + stage * kStageBytes;
-#pragma unroll
-        for (unsigned j = 0; j < kCopies; ++j) {
-            const unsigned group = wave + kWaves * j;            // wave-uniform
-            if (group * 4u < kStagedTokens)
-                copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
-                               (unsigned)__builtin_amdgcn_readfirstlane((int)(base + group * 1024u)));
-        }
-        if (wave < 2u && wave * 64u < kStagedTokens)
-            copy_to_lds_4(scale_from + (unsigned long long)sb * kQ8KBytes,
-                          (unsigned)__builtin_amdgcn_readfirstlane((int)(base + kStageActs + wave * 256u)));
-    };
-    auto fetch_codes = [&](unsigned sb) {
-        const unsigned block = row_misalign + sb * 66u;         // from row_aligned
-        raw_scale = *reinterpret_cast<const unsigned *>(row_aligned + (block & ~3u));
-#pragma unroll
-        for (unsigned ks = 0; ks < 3u; ++ks)
-            raw[ks] = *reinterpret_cast<const RawGroup *>(
-                row_aligned + ((block + 2u + 8u * (2u * ks + lane_group)) & ~3u));
-        // The last record of a superblock may be the last bytes of the tensor: its third dword
-        // is read only when it holds bytes of the record (an aligned dword with a valid byte
-        // lies in a mapped page), otherwise the second dword is read again.
-        const unsigned start = block + 2u + 8u * (6u + lane_group);
-        const unsigned char *at = row_aligned + (start & ~3u);
-        const uint2 head = *reinterpret_cast<const uint2 *>(at);
-        raw[3].x = head.x;
-        raw[3].y = head.y;
-        raw[3].z = *reinterpret_cast<const unsigned *>(at + 4u + 2u * (start & 3u));
-    };
-    uint2 now_codes[4];
-    unsigned now_scale16;
-    auto settle_codes = [&](unsigned sb) {   // the registers fetch_codes(sb) filled -> records
-        const unsigned shift = (row_misalign + 2u * sb + 2u) & 3u;
-        now_scale16 = (raw_scale >> (8u * ((row_misalign + 2u * sb) & 3u))) & 0xffffu;
+    // ---- pipeline state; every index below is a compile-time constant after unrolling ----
+    // (weight windows: LDS slot x & 1 holds superblock x, copied two steps before its records
+    // are taken out)
+    v4i a_lo[2][4], a_hi[2][4];      // [x & 1]: A operands of superblock x, all four K steps
+    float rs[2][4];                  // [x & 1]: row scales of superblock x
+    v4i frags[4];                    // B fragment of K step ks: re-requested for the next token block
+                                     // as soon as the current one has used it
+    float ts[2];                     // [g & 1]: activation scale of token block g (counted over steps)
+    v4i sum_lo[2], sum_hi[2];        // [g & 1]: its integer sums, scaled one token block later
+    // Fragment addresses: stage base + piece offset live in registers (kept opaque so that the
+    // block offset, under 32 KB, stays the instruction's immediate instead of a separate OR).
+    unsigned piece_at[4];
+    auto enter_stage = [&](unsigned base) {
 #pragma unroll
         for (unsigned ks = 0; ks < 4u; ++ks) {
-            now_codes[ks].x = __builtin_amdgcn_alignbyte(raw[ks].y, raw[ks].x, shift);
-            now_codes[ks].y = __builtin_amdgcn_alignbyte(raw[ks].z, raw[ks].y, shift);
+            piece_at[ks] = base + piece[ks];
+            asm volatile("" : "+v"(piece_at[ks]));
         }
     };
-    // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of token 16 tb + li
-    unsigned piece[4];
-#pragma unroll
-    for (unsigned ks = 0; ks < 4u; ++ks) piece[ks] = li * kActPitch + (((4u * ks + kb) ^ li) << 4);
+    auto request = [&](unsigned block, unsigned ks) {   // block: 16-slot block of the entered stage
+        frags[ks] = lds_read_v4i(piece_at[ks] + block * 16u * kActPitch);
+    };
+    auto request_scale = [&](unsigned base, unsigned block, unsigned g) {
+        ts[g & 1u] = __uint_as_float(lds_read_u32(base + kStageActs + 4u * (block * 16u + li)));
+    };
+    auto stage_of = [&](unsigned step) { return kStageBase + ((step / S) & 1u) * kStageBytes; };
 
     __syncthreads();   // every wave is done with the previous item's stages
     copy_activations(0u, 0u);
-    fetch_codes(0u);
-    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the copies above have landed in LDS
-    settle_codes(0u);
-    __syncthreads();
-
-    const unsigned last = superblocks - 1u;
-    for (unsigned sb = 0; sb < superblocks; ++sb) {
-        const unsigned base = kStageBase + (sb & 1u) * kStageBytes;
-        const unsigned ahead = sb < last ? sb + 1u : last;     // the last turn repeats a request
-        copy_activations(ahead, (sb & 1u) ^ 1u);
-        fetch_codes(ahead);
-
-        v4i sum_lo[NB], sum_hi[NB];
 #pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            sum_lo[tb] = v4i{0, 0, 0, 0};
-            sum_hi[tb] = v4i{0, 0, 0, 0};
-        }
-        // Software pipeline over phases (K step, group of up to four token blocks): the
-        // activation fragments of the next phase and the table lookups of the next K step are
-        // requested before the current phase's matrix instructions are issued, so their LDS
-        // latency runs under those instructions.
-        constexpr unsigned kGroups = NB > 4u ? 2u : 1u;      // groups per K step
-        constexpr unsigned kGroupSize = NB / kGroups;
-        constexpr unsigned kPhases = 4u * kGroups;
-        uint2 codes_of[2], signs_of[2];
-        uint4 limbs_of;
-        auto lookup = [&](unsigned ks) {
-            // the lane's sixteen weights: subgroups 2 (kb & 1) and 2 (kb & 1) + 1 of its group
-            const unsigned grids = now_codes[ks].x >> (16u * (kb & 1u));
-            const unsigned aux = now_codes[ks].y;
-            const unsigned signs = aux >> (14u * (kb & 1u));
-            codes_of[0] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0400u));
-            codes_of[1] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0500u));
-            signs_of[0] = lds_read_uint2(((signs << 7) & 0x3f80u) | sel_lane);
-            signs_of[1] = lds_read_uint2((signs & 0x3f80u) | sel_lane);
-            limbs_of = lds_read_uint4(((aux >> 20) & 0xf00u) | lut_lane);
-        };
-        v4i a_lo, a_hi;
-        auto weights_from_lookup = [&]() {
-            const unsigned s0 = codes_of[0].x | signs_of[0].x, s1 = codes_of[0].y | signs_of[0].y;
-            const unsigned s2 = codes_of[1].x | signs_of[1].x, s3 = codes_of[1].y | signs_of[1].y;
-            a_lo = v4i{(int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s0),
-                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s1),
-                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s2),
-                       (int)__builtin_amdgcn_perm(limbs_of.y, limbs_of.x, s3)};
-            a_hi = v4i{(int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s0),
-                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s1),
-                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s2),
-                       (int)__builtin_amdgcn_perm(limbs_of.w, limbs_of.z, s3)};
-        };
-        uint4 frags[2][kGroupSize];
-        auto request = [&](unsigned phase, uint4 (&into)[kGroupSize]) {
-            const unsigned ks = phase / kGroups, group = phase % kGroups;
-#pragma unroll
-            for (unsigned i = 0; i < kGroupSize; ++i)
-                into[i] = lds_read_uint4(base + piece[ks] + (group * kGroupSize + i) * 16u * kActPitch);
-        };
-        lookup(0u);
-        request(0u, frags[0]);
-        weights_from_lookup();
-#pragma unroll
-        for (unsigned phase = 0; phase < kPhases; ++phase) {
-            const unsigned ks = phase / kGroups, group = phase % kGroups;
-            if (phase + 1u < kPhases) request(phase + 1u, frags[(phase + 1u) & 1u]);
-            if (group == 0u && ks + 1u < 4u) lookup(ks + 1u);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (unsigned i = 0; i < kGroupSize; ++i) {
-                const unsigned tb = group * kGroupSize + i;
-                const uint4 rawb = frags[phase & 1u][i];
-                const v4i b = v4i{(int)rawb.x, (int)rawb.y, (int)rawb.z, (int)rawb.w};
-                sum_lo[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, sum_lo[tb], 0, 0, 0);
-                sum_hi[tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, sum_hi[tb], 0, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (group == kGroups - 1u && ks + 1u < 4u) weights_from_lookup();
-        }
-        // ---- exact superblock sums -> fp32 ----
-        float row_scale[4];
-        {
-            const float mine = 0.125f * f16_bits_to_float(now_scale16);
-#pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) row_scale[r] = __shfl(mine, (int)(4u * kb + r), 64);
-        }
-#pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            const float token_scale =
-                __uint_as_float(lds_read_u32(base + kStageActs + 4u * (tb * 16u + li)));
-#pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) {
-                const int total = (sum_hi[tb][r] << 7) + sum_lo[tb][r];
-                acc[tb][r] = __builtin_fmaf(row_scale[r] * token_scale, (float)total, acc[tb][r]);
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the next stage is complete in LDS
-        settle_codes(ahead);
+    for (unsigned k = 0; k < 2u; ++k) fetch_codes(k, k);
+    {
+        __builtin_amdgcn_s_waitcnt(0x0f70u);   // vmcnt(0): every copy above has landed
+        const Codes first = settle_codes(0u, 0u);
+        // the slot's reads have returned before it is refilled
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        fetch_codes(0u, 2u);
         __syncthreads();
+        enter_stage(stage_of(0u));
+#pragma unroll
+        for (unsigned ks = 0; ks < 3u; ++ks) request(0u, ks);
+        request_scale(stage_of(0u), 0u, 0u);
+        row_scales(first, 0u, rs[0]);
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks) {
+            const Lookup lk = lookup(first, ks);
+            weights_from_lookup(lk, a_lo[0][ks], a_hi[0][ks]);
+        }
     }
+    sum_lo[1] = v4i{0, 0, 0, 0};
+    sum_hi[1] = v4i{0, 0, 0, 0};
+    ts[1] = 0.0f;
+#pragma unroll
+    for (unsigned r = 0; r < 4u; ++r) rs[1][r] = 0.0f;
+
+    // scaling of the integer sums of token block g - 1 into the accumulators, one C row per call
+    auto scale_row = [&](unsigned g_prev, unsigned tb_prev, float row_scale, float token_scale, unsigned r) {
+        const int total = (sum_hi[g_prev & 1u][r] << 7) + sum_lo[g_prev & 1u][r];
+        acc[tb_prev][r] = __builtin_fmaf(row_scale * token_scale, (float)total, acc[tb_prev][r]);
+    };
+
+    const unsigned steps = (superblocks + D - 1u) / D * D;
+    for (unsigned t0 = 0; t0 < steps; t0 += D) {
+#pragma unroll
+        for (unsigned u = 0; u < D; ++u) {
+            const unsigned t = t0 + u;                    // this step's superblock; u == t % D
+            const unsigned base = stage_of(t);
+            // the next superblock's records leave the ring; the one D steps on enters it piece
+            // by piece below, behind this period's copies
+            // (copies are invisible to the compiler's wait counts; they complete in order, so
+            // waiting until only the copies issued after a slot's two are in flight covers it)
+            constexpr unsigned kAfterPeriodStart = 2u + kCopyPieces;
+            if (((u + D - 1u) % D) % S == 0u)
+                __builtin_amdgcn_s_waitcnt(0x0f70u | (kAfterPeriodStart & 15u) | ((kAfterPeriodStart >> 4) << 14));
+            else
+                __builtin_amdgcn_s_waitcnt(0x0f72u);
+            const Codes next = settle_codes((u + 1u) & 1u, t + 1u);
+            constexpr unsigned kSlots = 4u * NB;
+            const unsigned memory_pieces = (u % S == 0u ? kCopyPieces : 0u) + kFetchPieces;
+            float rs_before[4];                           // of the step before this one
+#pragma unroll
+            for (unsigned r = 0; r < 4u; ++r) rs_before[r] = rs[(u + 1u) & 1u][r];
+            row_scales(next, t + 1u, rs[(u + 1u) & 1u]);
+            Lookup lk[4];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (unsigned tb = 0; tb < NB; ++tb) {
+                const unsigned g = u * NB + tb;           // parity of the global token-block count
+                const float ts_before = ts[(g + 1u) & 1u];   // of the token block before this one
+#pragma unroll
+                for (unsigned ks = 0; ks < 4u; ++ks) {
+                    const unsigned q = tb * 4u + ks;
+                    // across a period end the next token block's scale and fragments are
+                    // requested after the barrier instead
+                    const bool next_here = tb + 1u < NB || u % S != S - 1u;
+                    const unsigned next_block = (u % S) * NB + tb + 1u;
+                    if (ks == 0u && next_here) request_scale(base, next_block, g + 1u);
+                    const v4i b = frags[ks];
+                    if (ks == 0u) {
+                        sum_lo[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[u & 1u][0], b, v4i{0, 0, 0, 0}, 0, 0, 0);
+                        sum_hi[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[u & 1u][0], b, v4i{0, 0, 0, 0}, 0, 0, 0);
+                    } else {
+                        sum_lo[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[u & 1u][ks], b, sum_lo[g & 1u], 0, 0, 0);
+                        sum_hi[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[u & 1u][ks], b, sum_hi[g & 1u], 0, 0, 0);
+                    }
+                    // fragment ks - 1 is free now: its next use is one token block on (fragment 3
+                    // of this token block still has to be asked for when ks is 0)
+                    if (ks == 0u) request(next_block - 1u, 3u);
+                    else if (next_here) request(next_block, ks - 1u);
+                    // one C row of the previous token block (the previous step's last one for tb 0)
+                    scale_row(g + 1u, tb ? tb - 1u : NB - 1u, tb ? rs[u & 1u][ks] : rs_before[ks], ts_before, ks);
+                    // this step's copies and loads, spread evenly
+#pragma unroll
+                    for (unsigned v = 0; v < kCopyPieces + kFetchPieces; ++v) {
+                        if (v >= memory_pieces || v * kSlots / memory_pieces != q) continue;
+                        const unsigned first_fetch = memory_pieces - kFetchPieces;
+                        if (v < first_fetch) copy_piece(t / S + 1u, (t / S + 1u) & 1u, v);
+                        else {
+                            // the reads that took this slot's records out have returned
+                            if (v == first_fetch) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                            fetch_piece((u + 1u) & 1u, t + 3u, v - first_fetch);
+                        }
+                    }
+                    // the next superblock's A operands: eight pieces (lookups L, permutes W of the
+                    // four K steps) spread evenly over the slots, every W at least two slots
+                    // behind its L
+#pragma unroll
+                    for (unsigned i = 0; i < 8u; ++i) {
+                        if (i * NB / 2u != q) continue;
+                        unsigned is_w, k;
+                        if (NB >= 8u) {
+                            is_w = i & 1u;
+                            k = i >> 1;
+                        } else {
+                            is_w = (i == 2u || i == 4u || i >= 6u) ? 1u : 0u;
+                            k = is_w ? (i == 2u ? 0u : i == 4u ? 1u : i - 4u) : (i < 2u ? i : (i + 1u) / 2u);
+                        }
+                        if (is_w) weights_from_lookup(lk[k], a_lo[(u + 1u) & 1u][k], a_hi[(u + 1u) & 1u][k]);
+                        else lk[k] = lookup(next, k);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if (u % S == S - 1u) {
+                // the copies of the next period are older than the 2 S window copies issued since
+                __builtin_amdgcn_s_waitcnt(0x0f70u | ((2u * S) & 15u) | (((2u * S) >> 4) << 14));
+                __syncthreads();
+                enter_stage(stage_of(t + 1u));
+#pragma unroll
+                for (unsigned ks = 0; ks < 3u; ++ks) request(0u, ks);
+                request_scale(stage_of(t + 1u), 0u, (u + 1u) * NB);
+            }
+        }
+    }
+    // the last token block of the last step
+#pragma unroll
+    for (unsigned r = 0; r < 4u; ++r) scale_row(D * NB - 1u, NB - 1u, rs[(D - 1u) & 1u][r], ts[(D * NB - 1u) & 1u], r);
 
     // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
     auto store4 = [&](unsigned token, unsigned row, const float (&value)[4]) {
@@ -543,6 +739,10 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
+#ifdef YVEX_ONLY_NB
+        mfma_item<FUSED_UP, YVEX_ONLY_NB>(a, it);
+        continue;
+#endif
         if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
         else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
         else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
