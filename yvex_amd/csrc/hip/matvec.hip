@@ -48,7 +48,12 @@ __device__ float matvec_recover_f64(const unsigned char *row, const float *x,
     return (float)sum;
 }
 
-template <unsigned QT, bool Q8, int T>
+// U: 64-unit chunks of the row whose loads are issued together before the first of them is used.
+// A wave walks one row front to back; with one chunk in flight it waits a full memory latency per
+// chunk (weights, then the activation bytes that go with them), which bounds a long matrix such as
+// an output head well below what the same loads reach when nothing waits on them.
+// EVEN: every row starts on an even address (even base address and even row bytes).
+template <unsigned QT, bool Q8, int T, int U, bool EVEN>
 __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
 {
     __shared__ Iq2Tables tables;
@@ -68,35 +73,45 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     for (int t = 0; t < T; ++t) acc[t] = 0.0f;
 
     // Every lane runs the same trip count so the superblock shuffles below stay converged.
-    for (unsigned base = 0; base < units; base += 64u) {
-        const unsigned u = base + lane;
-        const bool live = u < units;
-        const unsigned uu = live ? u : units - 1u;
-        Unit unit;
-        unit_load<QT>(tables, wrow, uu, unit);
+    for (unsigned base = 0; base < units; base += 64u * U) {
+        Unit unit[U];
+        unsigned uu[U];
+        bool live[U];
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            unsigned long long in = in0 + t;
-            if (in >= a.input_rows) in = a.input_rows - 1ull;   // clamped rows are never written
-            if constexpr (Q8) {
-                const unsigned char *act = (const unsigned char *)a.input + in * act_row_bytes +
-                                           (unsigned long long)(uu >> 3) * kQ8KBytes;
-                UnitSum s = unit_dot_q8<QT>(unit, act, uu & 7u);
-                const float act_scale = *reinterpret_cast<const float *>(act);
-                if constexpr (UnitTraits<QT>::kIntegerCombine) {
-                    if (!live) s.dot = s.min = 0;
-                    s.dot = group_sum_i32<8>(s.dot);
-                    if constexpr (QT != QT_IQ2_XXS) s.min = group_sum_i32<8>(s.min);
-                    if (live && (uu & 7u) == 0u)
-                        acc[t] += super_combine<QT>(wrow + (uu >> 3) * UnitTraits<QT>::kSuperBytes,
-                                                    act_scale, s);
+        for (int j = 0; j < U; ++j) {
+            const unsigned u = base + 64u * j + lane;
+            live[j] = u < units;
+            uu[j] = live[j] ? u : units - 1u;
+            unit_load<QT, EVEN ? 1 : -1>(tables, wrow, uu[j], unit[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (j > 0 && base + 64u * j >= units) break;      // wave-uniform: no chunk here
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                unsigned long long in = in0 + t;
+                if (in >= a.input_rows) in = a.input_rows - 1ull;   // clamped rows are never written
+                if constexpr (Q8) {
+                    const unsigned char *act = (const unsigned char *)a.input + in * act_row_bytes +
+                                               (unsigned long long)(uu[j] >> 3) * kQ8KBytes;
+                    UnitSum s = unit_dot_q8<QT>(unit[j], act, uu[j] & 7u);
+                    const float act_scale = *reinterpret_cast<const float *>(act);
+                    if constexpr (UnitTraits<QT>::kIntegerCombine) {
+                        if (!live[j]) s.dot = s.min = 0;
+                        s.dot = group_sum_i32<8>(s.dot);
+                        if constexpr (QT != QT_IQ2_XXS) s.min = group_sum_i32<8>(s.min);
+                        if (live[j] && (uu[j] & 7u) == 0u)
+                            acc[t] += super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
+                                                        act_scale, s);
+                    } else {
+                        const float v = q8_0_unit_value(wrow, uu[j], act_scale, s.dot);
+                        acc[t] += live[j] ? v : 0.0f;
+                    }
                 } else {
-                    if (live) acc[t] += q8_0_unit_value(wrow, uu, act_scale, s.dot);
+                    const float *x = (const float *)a.input + in * a.input_stride + 32ull * uu[j];
+                    const float v = unit_dot_f32<QT>(unit[j], wrow, uu[j], x);
+                    if (live[j]) acc[t] += v;
                 }
-            } else {
-                const float *x = (const float *)a.input + in * a.input_stride + 32ull * uu;
-                const float v = unit_dot_f32<QT>(unit, wrow, uu, x);
-                if (live) acc[t] += v;
             }
         }
     }
@@ -208,19 +223,30 @@ __global__ __launch_bounds__(256) void gather_kernel(
     else out[index] = value;
 }
 
-template <unsigned QT, bool Q8>
-static int launch_block(const MatvecArgs &a, hipStream_t stream)
+template <unsigned QT, bool Q8, bool EVEN>
+static int launch_block_even(const MatvecArgs &a, hipStream_t stream)
 {
     const unsigned long long grid_x = (a.row_count + 3ull) / 4ull;
     if (grid_x > 0x7fffffffull) return ST_BOUNDS;
     if (a.input_rows == 1ull) {
-        matvec_block_kernel<QT, Q8, 1><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
+        // Q8_K activations against a matrix that takes many rounds of waves: four chunks (8192
+        // columns) in flight; a small matrix is one round and gains nothing from them
+        const bool deep = Q8 && a.row_count * a.row_bytes >= (64ull << 20);
+        if (deep) matvec_block_kernel<QT, Q8, 1, Q8 ? 4 : 1, EVEN><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
+        else matvec_block_kernel<QT, Q8, 1, 1, EVEN><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
     } else {
         const unsigned long long grid_y = (a.input_rows + 3ull) / 4ull;
         if (grid_y > 65535ull) return ST_BOUNDS;
-        matvec_block_kernel<QT, Q8, 4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, stream>>>(a);
+        matvec_block_kernel<QT, Q8, 4, 1, EVEN><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, stream>>>(a);
     }
     return check_launch("matvec");
+}
+
+template <unsigned QT, bool Q8>
+static int launch_block(const MatvecArgs &a, hipStream_t stream)
+{
+    const bool even = (((unsigned long long)a.encoded | a.row_bytes) & 1ull) == 0ull;
+    return even ? launch_block_even<QT, Q8, true>(a, stream) : launch_block_even<QT, Q8, false>(a, stream);
 }
 
 template <unsigned QT>

@@ -48,10 +48,12 @@ struct Unit {
     int min1, min2;  // Q4_K: m (min2 = m); Q2_K: m of each half; else 0
 };
 
-template <unsigned QT>
+// EVEN: 1 = the caller knows the row starts on an even address, 0 = it does not, -1 = look.
+template <unsigned QT, int EVEN = -1>
 __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigned char *row,
                                           unsigned u, Unit &unit)
 {
+    const bool even = EVEN < 0 ? ((unsigned long long)row & 1ull) == 0ull : EVEN != 0;
     const unsigned sb = u >> 3, g = u & 7u;
     // Group records and Q8_0 blocks start on 2-byte boundaries, and vector loads that are not
     // dword-aligned run at under half rate on this part: load the aligned dwords that hold the
@@ -60,7 +62,7 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
     if constexpr (QT == QT_IQ2_XXS) {
         const unsigned char *p = row + sb * 66u + 2u + 8u * g;
         uint2 packed;
-        if (((unsigned long long)row & 1ull) == 0ull) {
+        if (even) {
             const unsigned shift = (unsigned)(unsigned long long)p & 3u;       // 0 or 2
             const unsigned char *at = p - shift;
             const uint2 head = *reinterpret_cast<const uint2 *>(at);
@@ -74,7 +76,7 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
         unit.min1 = unit.min2 = 0;
     } else if constexpr (QT == QT_Q8_0) {
         const unsigned char *b = row + u * 34u + 2u;
-        if (((unsigned long long)row & 1ull) == 0ull) {
+        if (even) {
             const unsigned shift = (unsigned)(unsigned long long)b & 3u;       // 0 or 2
             const unsigned char *at = b - shift;
             const uint4 lo = *reinterpret_cast<const uint4 *>(at);
