@@ -9,7 +9,8 @@ the distinct routed experts hit, divided by the step time.
 
 Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up sweep), timed
 with events on the launch stream; `cpu_baseline` is the CPU oracle timed on the host cores over
-a bounded sample of the same workload.
+a bounded sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8
+matrix cores) and `dense` configs 0-2 and an output head as single matvec launches.
 """
 from __future__ import annotations
 
@@ -75,6 +76,82 @@ def cpu_baseline(sample_rows: int, threads: int):
             "sample": f"{sample_rows} rows x (top-8 + shared) expert FFNs of the same layer shape, "
                       f"scalar C restatement of yvex_quant_cpu_dot/yvex_moe_expert_cpu",
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
+
+
+def dense_leg(torch, K, dev, repeats: int):
+    """BASELINE configs 0-2 and an output head as single matvec launches: random packed bytes with
+    small positive fp16 block scales, 32 distinct weight copies walked in turn (2 for the head) so
+    that no launch finds its weights in cache. Bytes counted: the encoded matrix."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    out = {}
+
+    def run(name, qt, rows, width, inputs, q8, copies=32):
+        total = rows * K.row_bytes(qt, width)
+        if qt == K.IQ2_XXS:
+            w = synth_iq2xxs(torch, copies * rows * width // 256, dev, 5)
+        else:
+            w = torch.randint(0, 256, (copies * total,), dtype=torch.uint8, device=dev, generator=gen)
+            blocks = w.view(-1, 34 if qt == K.Q8_0 else 144)
+            d = (torch.rand(blocks.shape[0], device=dev, generator=gen) * 1e-3 + 1e-4).to(torch.float16)
+            blocks[:, 0:2] = d.view(torch.uint8).reshape(-1, 2)
+            if qt == K.Q4_K:
+                blocks[:, 2:4] = blocks[:, 0:2]
+        x = torch.randn((inputs, width), device=dev, generator=gen)
+        status = K.new_status(dev)
+        act = K.q8k_quantize(x, status) if q8 else x
+        result = torch.empty((inputs, rows), dtype=torch.float32, device=dev)
+        turn = [0]
+
+        def once():
+            i = turn[0] % copies
+            turn[0] += 1
+            K.matvec(w[i * total:(i + 1) * total], qt, rows, width, act, input_q8=q8, input_rows=inputs,
+                     status=status, out=result)
+        for _ in range(copies):
+            once()
+        torch.cuda.synchronize()
+        ms = event_ms(torch, once, repeats)
+        # the same launches replayed from a captured graph: without the host's time per call,
+        # which is what a launch of a few microseconds is otherwise measured by
+        graph_us = None
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(copies):
+                        once()
+                graph.replay()
+                side.synchronize()
+                replays = max(1, repeats // copies)
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record(side)
+                for _ in range(replays):
+                    graph.replay()
+                stop.record(side)
+                stop.synchronize()
+                graph_us = start.elapsed_time(stop) / (replays * copies) * 1e3
+            torch.cuda.current_stream().wait_stream(side)
+        except Exception as error:   # capture refused: keep the eager figure
+            graph_us = None
+            print(f"dense leg: graph capture unavailable ({error})", file=sys.stderr)
+        best_ms = min(ms, graph_us * 1e-3) if graph_us else ms
+        out[name] = {"us": round(ms * 1e3, 2), "graph_us": round(graph_us, 2) if graph_us else None,
+                     "GB_per_s": round(total / (best_ms * 1e-3) / 1e9, 1),
+                     "hbm_peak_frac": round(total / (best_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "matrix_bytes": total, "status": int(status.item())}
+        del w
+
+    run("cfg0_q8_0_4096x4096_f32_b1", K.Q8_0, 4096, 4096, 1, False)
+    run("cfg0_q8_0_4096x4096_q8k_b1", K.Q8_0, 4096, 4096, 1, True)
+    run("cfg1_q4_k_2048x7168_q8k_b1", K.Q4_K, 2048, 7168, 1, True)
+    run("cfg1_q4_k_2048x7168_q8k_b16", K.Q4_K, 2048, 7168, 16, True)
+    run("cfg2_iq2_xxs_7168x2048_f32_b1", K.IQ2_XXS, 7168, 2048, 1, False)
+    run("cfg2_iq2_xxs_7168x2048_q8k_b1", K.IQ2_XXS, 7168, 2048, 1, True)
+    run("head_q8_0_129280x7168_q8k_b1", K.Q8_0, 129280, 7168, 1, True, copies=2)
+    return out
 
 
 def tile_classes(populations):
@@ -149,6 +226,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=4)
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 1 GiB read kernel and a 256 MiB fill kernel, so a "
                          "counter run of this command holds kernels of known HBM traffic")
@@ -261,6 +339,10 @@ def main() -> int:
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)
+    if not args.no_dense:
+        del layer, gate, up, down, shared
+        torch.cuda.empty_cache()
+        out["dense"] = dense_leg(torch, K, dev, 64)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_rows, 1)
         out["cpu_baseline_all_cores"] = cpu_baseline(max(args.cpu_rows, 8), min(16, os.cpu_count() or 1))

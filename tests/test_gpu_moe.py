@@ -65,6 +65,10 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
     ("IQ2_XXS", 512, 256, 8, 2, 7, True, 0, True),
     ("IQ2_XXS", 768, 512, 4, 2, 300, True, 1, True),
     ("IQ2_XXS", 7168, 2048, 12, 4, 10, True, 1, True),
+    # five superblocks per row (steps past the end of a row, rows that start on 2-byte boundaries)
+    # with 32-pair tiles; three superblocks with 64-pair tiles
+    ("IQ2_XXS", 1280, 256, 4, 2, 40, True, 1, True),
+    ("IQ2_XXS", 768, 768, 4, 2, 100, True, 0, True),
 ])
 def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, topk, rows, act_q8,
                              scoring, matrix_cores):
