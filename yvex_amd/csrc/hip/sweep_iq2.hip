@@ -486,18 +486,32 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     g.park = kParkBase + wave * kParkBytes;
     g.park_write = g.park + (lane & 1u) * 16u + (lane >> 4) * 4u;
 
+    // The first part of the weight rows is cut into long items (kSweepIters iterations), the rest
+    // into short ones that come last in the item list: the waves of the grid finish within a short
+    // item of each other instead of a long one, and only the short items pay the fixed cost of an
+    // item (its activation columns, the first requests, the finishing pass) more often.
+#ifndef YVEX_SWEEP_LONG_PERCENT
+#define YVEX_SWEEP_LONG_PERCENT 75
+#endif
+#ifndef YVEX_SWEEP_SHORT_DIV
+#define YVEX_SWEEP_SHORT_DIV 2
+#endif
     const unsigned item_rows = kSweepIters * g.rows_per_iter;
-    const unsigned tiles = (a.out_rows + item_rows - 1u) / item_rows;
+    const unsigned short_rows = item_rows / YVEX_SWEEP_SHORT_DIV;
+    const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * YVEX_SWEEP_LONG_PERCENT / 100u / item_rows);
+    const unsigned long_rows = long_tiles * item_rows;
+    const unsigned short_tiles = (a.out_rows - long_rows + short_rows - 1u) / short_rows;
 
     // Work items are numbered with the shared expert's first (the heaviest: full sweeps), then the
     // routed buckets in worklist order.
     const GroupedProblem &extra = a.problem[a.problems > 1u ? 1u : 0u];
-    const unsigned extra_items = a.problems > 1u
-        ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) * tiles : 0u;
+    const unsigned extra_sweeps = a.problems > 1u
+        ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) : 0u;
     const unsigned routed_sweeps = routed_fixed
         ? (unsigned)((routed.pairs + kSweepPairs - 1u) / kSweepPairs)
         : lds_load_u32(kPrefixBase + 4u * buckets);
-    const unsigned total_items = extra_items + routed_sweeps * tiles;
+    const unsigned total_long = (extra_sweeps + routed_sweeps) * long_tiles;
+    const unsigned total_items = total_long + (extra_sweeps + routed_sweeps) * short_tiles;
     // Workgroup b owns items b, b + grid, b + 2 grid, ...; its waves draw positions in that list
     // from a counter in LDS, so a wave that met light items takes more of them.
     auto draw = [&]() -> unsigned {
@@ -508,13 +522,18 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         return (unsigned)__builtin_amdgcn_readfirstlane((int)got) * gridDim.x + blockIdx.x;
     };
-    for (unsigned item = draw(); item < total_items; item = draw()) {
+    for (unsigned listed = draw(); listed < total_items; listed = draw()) {
+        const bool is_short = listed >= total_long;
+        const unsigned item = is_short ? listed - total_long : listed;   // within its zone of rows
+        const unsigned tiles = is_short ? short_tiles : long_tiles;
+        const unsigned rows_of_item = is_short ? short_rows : item_rows;
+        const unsigned extra_items = extra_sweeps * tiles;
         const bool is_extra = item < extra_items;
         const GroupedProblem &pr = is_extra ? extra : routed;
         const bool fixed = is_extra || routed_fixed;
         unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
         unsigned local = is_extra ? item : item - extra_items;
-        unsigned bucket_sweeps = is_extra ? extra_items / tiles : routed_sweeps;
+        unsigned bucket_sweeps = is_extra ? extra_sweeps : routed_sweeps;
         if (!fixed) {
             unsigned low = 0u, high = buckets;   // last bucket whose first item is <= local
             while (low + 1u < high) {
@@ -543,8 +562,8 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         }
         const unsigned char *gate_e = pr.gate + expert * pr.expert_bytes;
         const unsigned char *up_e = FUSED ? pr.up + expert * pr.up_expert_bytes : nullptr;
-        const unsigned row_begin = tile * item_rows;
-        const unsigned row_end = row_begin + item_rows < a.out_rows ? row_begin + item_rows : a.out_rows;
+        const unsigned row_begin = (is_short ? long_rows : 0u) + tile * rows_of_item;
+        const unsigned row_end = row_begin + rows_of_item < a.out_rows ? row_begin + rows_of_item : a.out_rows;
         const unsigned long long live = population - pass;
         if (kSweepPairs >= 4 && live >= 4ull)
             iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
