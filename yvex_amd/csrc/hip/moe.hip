@@ -186,7 +186,6 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
         counts[0] = bucket_count;
         counts[2] = total_pairs;
         counts[3] = total_sweeps;
-        counts[4] = counts[5] = 0ull;   // work-item counters of the expert kernels
         if (total_pairs != pairs) bad = 1u;
     }
     // largest population: one atomic per wave after a wave-wide maximum

@@ -34,9 +34,6 @@ namespace yvex {
 #ifndef YVEX_SWEEP_AHEAD_SMALL
 #define YVEX_SWEEP_AHEAD_SMALL 1
 #endif
-#ifndef YVEX_SWEEP_DEPTH_SMALL
-#define YVEX_SWEEP_DEPTH_SMALL 3
-#endif
 #ifndef YVEX_SWEEP_PAIRS
 #define YVEX_SWEEP_PAIRS 4
 #endif
@@ -325,7 +322,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
     // final row) and every lane stores (lanes that hold no result write to a spare word), so no
     // branch sits between a request and the wait that consumes it and the waits stay counted.
-    constexpr int AHEAD = N <= 2 ? YVEX_SWEEP_AHEAD_SMALL : 1;   // AHEAD + 1 is 2 or 4
+    constexpr int AHEAD = N <= 2 ? YVEX_SWEEP_AHEAD_SMALL : 1;   // rows requested ahead of the one decoded
     constexpr int STREAMS = FUSED ? 2 : 1;
     Iq2Half ring[AHEAD + 1][STREAMS];
     const unsigned last = iterations - 1u;

@@ -58,7 +58,7 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
     TAKE(bucket_offsets, (experts + 1ull) * sizeof(unsigned long long));
     TAKE(bucket_populations, experts * sizeof(unsigned long long));
     TAKE(sweep_offsets, (experts + 1ull) * sizeof(unsigned long long));
-    TAKE(counts, 8ull * sizeof(unsigned long long));
+    TAKE(counts, 4ull * sizeof(unsigned long long));
     TAKE(intermediate, pairs * routed_i * sizeof(float));
     TAKE(intermediate_q8, pairs * ((routed_i + 255ull) / 256ull) * 292ull);
     TAKE(pair_outputs, pairs * hidden * sizeof(float));

@@ -129,7 +129,7 @@ class Worklist:
         self.bucket_offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
         self.bucket_populations = torch.empty(experts, dtype=torch.int64, device=device)
         self.sweep_offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
-        self.counts = torch.zeros(8, dtype=torch.int64, device=device)
+        self.counts = torch.zeros(4, dtype=torch.int64, device=device)
 
 
 def worklist_build(selected, experts, status, worklist: Worklist | None = None) -> Worklist:
