@@ -327,6 +327,20 @@ int yvex_backend_rocm_encoded_gather(
     unsigned long long selected_rows, yvex_device_tensor *output,
     yvex_backend_rocm_operation_facts *facts, yvex_error *err);
 
+/* ---- greedy selection over logits rows ---------------------------------------------------- */
+
+/* Replaces the select_greedy_rows entry of yvex_backend_sampling_operations
+ * (include/yvex/internal/sampling.h:129-137, src/backend/cuda/sampling.c:284-392): for each of
+ * row_count rows of row_width F32 logits held by a tensor of this backend, the largest value,
+ * the lowest token holding it and the number of tokens holding it, written to host arrays. The
+ * device results live in the attached workspace for the call. Refusals: geometry, ownership,
+ * dtype, unwritten logits -> FORMAT; no workspace -> NOMEM; kernels absent -> UNSUPPORTED; a
+ * non-finite logit, a token outside the row or a zero tie count -> FORMAT, outputs zeroed. */
+int yvex_backend_rocm_select_greedy_rows(
+    yvex_backend *backend, const yvex_device_tensor *logits, unsigned long long row_count,
+    unsigned long long row_width, unsigned int *selected_tokens, float *selected_values,
+    unsigned long long *tie_counts, yvex_backend_rocm_operation_facts *facts, yvex_error *err);
+
 /* ---- MoE row batch: include/yvex/internal/moe.h ------------------------------------------- */
 
 #define YVEX_SHA256_HEX_CAP 65u

@@ -297,6 +297,18 @@ def moe_expert(qtypes, gate, up, down, hidden, intermediate, x, route_weight, li
     return rc, out, mid, raw
 
 
+def argmax_f32(values: np.ndarray):
+    """Per row of a [rows, width] float32 array: status (1 if a row held a non-finite value),
+    tokens u32, values f32, tie counts u64 (kernels.cu:59-110)."""
+    values = np.ascontiguousarray(values, np.float32)
+    rows, width = values.shape
+    tokens = np.zeros(rows, np.uint32)
+    best = np.zeros(rows, np.float32)
+    ties = np.zeros(rows, np.uint64)
+    rc = lib().yvo_argmax_f32(_p(values), C.c_uint64(rows), C.c_uint64(width), _p(tokens), _p(best), _p(ties))
+    return rc, tokens, best, ties
+
+
 def worklist_build(selected: np.ndarray, weights: np.ndarray, topk: int, experts: int):
     selected = np.ascontiguousarray(selected, np.uint64).ravel()
     weights = np.ascontiguousarray(weights, np.float32).ravel()

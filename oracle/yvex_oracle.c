@@ -760,6 +760,40 @@ int yvo_moe_expert(unsigned int gate_qtype, const uint8_t *gate, unsigned int up
     return rc;
 }
 
+/* ---- greedy selection: src/backend/cuda/kernels.cu:59-110 ---- */
+
+int yvo_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
+                   uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts)
+{
+    uint64_t row, index;
+    int status = 0;
+    if (!values || !row_count || !row_width || !selected_tokens || !selected_values || !tie_counts)
+        return YVO_ERR_INVALID_ARG;
+    for (row = 0; row < row_count; ++row) {
+        const float *v = values + row * row_width;
+        float best = -3.402823466e+38F;
+        uint64_t best_index = ~(uint64_t)0, tied = 0;
+        int bad = 0;
+        for (index = 0; index < row_width; ++index) {
+            float value = v[index];
+            if (!isfinite(value)) bad = 1;
+            else if (value > best) best = value, best_index = index, tied = 1;
+            else if (value == best) {
+                if (index < best_index) best_index = index;
+                tied++;
+            }
+        }
+        if (bad) {
+            status = 1;
+            continue;
+        }
+        selected_tokens[row] = (uint32_t)best_index;
+        selected_values[row] = best;
+        tie_counts[row] = tied;
+    }
+    return status;
+}
+
 /* ---- worklist: src/graph/worklist.c:369-441 ---- */
 
 int yvo_worklist_build(const uint64_t *selected_experts, const float *route_weights,

@@ -30,6 +30,10 @@
  *                                                  exact-equality case runtime_moe.c:178-212.
  *   yvo_worklist_build                             properties (stable sort, sums) and the cases of
  *                                                  tests/unit/expert_worklist.c.
+ *   yvo_argmax_f32                                 brute force over small rows (largest value, its
+ *                                                  first position, its multiplicity) and rows built
+ *                                                  with known ties; the reference holds no fixture
+ *                                                  for its selection kernel.
  */
 #ifndef YVEX_ORACLE_H
 #define YVEX_ORACLE_H
@@ -155,6 +159,14 @@ int yvo_worklist_build(const uint64_t *selected_experts, const float *route_weig
                        uint64_t *bucket_populations, uint64_t *source_pairs,
                        uint64_t *source_rows, uint64_t *destination_rows,
                        float *ordered_weights, uint64_t *bucket_count);
+
+/* Greedy selection per row: src/backend/cuda/kernels.cu:59-110 (yvex_argmax_f32). The reference
+ * scans a row with 128 strided threads and merges them in a tree; "larger wins, equal keeps the
+ * lower index and adds the counts" is associative and commutative, so one serial pass gives the
+ * same three numbers. Returns 1 (and leaves that row's outputs untouched) when a row holds a
+ * non-finite value, as the kernel raises status 1. */
+int yvo_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
+                   uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts);
 
 /* MoE layer over a row batch: routing given logits, routed experts in rank order, one shared
  * expert, combined = bf16(routed + shared) (src/runtime/moe.c:596-632).

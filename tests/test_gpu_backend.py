@@ -147,6 +147,43 @@ def test_encoded_gather(backend, oracle):
     assert facts.active_weight_bytes == ids.size * 132
 
 
+def run_greedy(b, logits, rows, width):
+    tokens, best, ties = np.full(rows, 7, np.uint32), np.full(rows, 7, np.float32), np.full(rows, 7, np.uint64)
+    facts, err = abi.OperationFacts(), abi.Error()
+    rc = b.lib.yvex_backend_rocm_select_greedy_rows(b.handle, logits, rows, width, tokens.ctypes.data,
+                                                    best.ctypes.data, ties.ctypes.data, C.byref(facts),
+                                                    C.byref(err))
+    return rc, tokens, best, ties, facts, err
+
+
+def test_select_greedy_rows(backend, oracle):
+    """The sampling table's greedy entry (sampling.c:284-392): results, facts, refusals."""
+    b = backend
+    rows, width = 3, 5000
+    rng = np.random.default_rng(11)
+    values = rng.standard_normal((rows, width)).astype(np.float32)
+    values[1, 4999] = values[1, 12] = 9.0
+    logits = b.f32(values)
+    # no workspace attached: nowhere to put the device results
+    rc, tokens, best, ties, facts, err = run_greedy(b, logits, rows, width)
+    assert rc == abi.NOMEM and not tokens.any() and not ties.any()
+    b.workspace(4096)
+    rc, tokens, best, ties, facts, err = run_greedy(b, logits, rows, width)
+    assert rc == 0, err.message
+    _, want_tokens, want_best, want_ties = oracle.argmax_f32(values)
+    assert np.array_equal(tokens, want_tokens) and np.array_equal(best, want_best)
+    assert np.array_equal(ties, want_ties) and ties[1] == 2 and tokens[1] == 12
+    assert facts.kernel_launches == 1 and facts.download_count == 4
+    assert facts.d2h_bytes == rows * 16 + 4 and facts.activation_bytes == values.nbytes
+    # refusals: rows past the tensor, an unwritten tensor, a non-finite logit (outputs zeroed)
+    assert run_greedy(b, logits, rows + 1, width)[0] == abi.FORMAT
+    assert run_greedy(b, b.empty_f32(width), 1, width)[0] == abi.FORMAT
+    values[2, 77] = np.nan
+    rc, tokens, best, ties, facts, err = run_greedy(b, b.f32(values), rows, width)
+    assert rc == abi.FORMAT and not tokens.any() and not best.any() and not ties.any()
+    assert facts.kernel_launches == 0
+
+
 class MoeCase:
     """One synthetic layer resident on the backend plus everything execute_rows needs."""
 

@@ -187,3 +187,40 @@ def test_worklist_flags_duplicate_expert(gpu):
     K.worklist_build(dev(sel, gpu), 4, status)
     torch.cuda.synchronize()
     assert int(status.item()) == 2
+
+
+@pytest.mark.parametrize("rows,width", [(1, 129280), (5, 1001), (3, 7), (32, 4096), (2, 1)])
+def test_greedy_selection_matches_oracle(gpu, oracle, rows, width):
+    """Largest value, lowest index holding it, tie count: exact (kernels.cu:59-110)."""
+    from yvex_amd import kernels as K
+    rng = np.random.default_rng(rows * 1000 + width)
+    values = rng.standard_normal((rows, width)).astype(np.float32)
+    if width > 4:
+        values[0, width - 1] = values[0, 1] = values[0].max() + 1.0   # a tie at both ends of row 0
+        values[rows - 1] = np.round(values[rows - 1] * 2.0) / 2.0     # many ties in the last row
+    status = K.new_status(gpu)
+    tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
+    status_ok(status)
+    rc, want_tokens, want_best, want_ties = oracle.argmax_f32(values)
+    assert rc == 0
+    assert np.array_equal(tokens.cpu().numpy().astype(np.uint32), want_tokens)
+    assert np.array_equal(best.cpu().numpy(), want_best)
+    assert np.array_equal(ties.cpu().numpy().astype(np.uint64), want_ties)
+
+
+def test_greedy_selection_flags_non_finite(gpu, oracle):
+    from yvex_amd import kernels as K
+    values = np.zeros((3, 515), np.float32)
+    values[0, 17] = 2.0
+    values[1, 300] = np.inf
+    values[2, 2] = values[2, 514] = 1.5
+    status = K.new_status(gpu)
+    tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    rc, want_tokens, want_best, want_ties = oracle.argmax_f32(values)
+    assert rc == 1
+    for row in (0, 2):      # the rows without the bad value publish; the bad row stays as it was
+        assert int(tokens[row]) == want_tokens[row] and float(best[row]) == want_best[row]
+        assert int(ties[row]) == want_ties[row]
+    assert int(ties[1]) == 0

@@ -403,3 +403,26 @@ def test_worklist_properties(oracle):
     bad = sel.copy()
     bad[0, 0] = experts
     assert oracle.worklist_build(bad, w, topk, experts)[0] == oracle.ERR_FORMAT
+
+
+def test_greedy_selection_against_brute_force(oracle):
+    """The serial restatement of the selection kernel (kernels.cu:59-110) against an independent
+    formulation: the maximum, the first position that holds it, the number of positions that
+    hold it. Rows are drawn from a few values so ties are common."""
+    rng = np.random.default_rng(7)
+    for width in (1, 2, 7, 64, 129, 1000):
+        values = rng.integers(-3, 4, size=(9, width)).astype(np.float32) * 0.5
+        values[3] = -3.402823466e+38          # the starting value itself: first index, all tied
+        values[4, width // 2] = 11.0          # a single winner
+        rc, tokens, best, ties = oracle.argmax_f32(values)
+        assert rc == 0
+        for row in range(values.shape[0]):
+            top = values[row].max()
+            where = np.flatnonzero(values[row] == top)
+            assert best[row] == top and tokens[row] == where[0] and ties[row] == where.size
+    # a non-finite value: status 1, that row untouched, the others published
+    values = np.array([[1.0, 2.0, 2.0], [0.0, np.inf, 1.0], [5.0, np.nan, 5.0], [4.0, 1.0, 0.0]], np.float32)
+    rc, tokens, best, ties = oracle.argmax_f32(values)
+    assert rc == 1
+    assert (tokens[0], best[0], ties[0]) == (1, 2.0, 2) and (tokens[3], best[3], ties[3]) == (0, 4.0, 1)
+    assert ties[1] == 0 and ties[2] == 0

@@ -220,11 +220,13 @@ EXPORTS = [
     "yvex_backend_resident_attach", "yvex_backend_resident_detach", "yvex_backend_resident_resolve",
     "yvex_backend_workspace_attach", "yvex_backend_workspace_detach",
     "yvex_backend_workspace_acquire", "yvex_backend_rocm_encoded_matvec",
-    "yvex_backend_rocm_encoded_gather", "yvex_backend_moe_operations_get",
+    "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows",
+    "yvex_backend_moe_operations_get",
     "yvex_expert_worklist_build",
 ]
 KERNEL_EXPORTS = [
     "yvex_hip_q8k_quantize", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
+    "yvex_hip_argmax_f32",
     "yvex_hip_moe_route_rows", "yvex_hip_worklist_build", "yvex_hip_moe_up", "yvex_hip_moe_down",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
     "yvex_hip_moe_reduce_combine", "yvex_hip_stream_read", "yvex_hip_fill_u32",
@@ -281,6 +283,9 @@ def library():
     lib.yvex_backend_rocm_encoded_gather.argtypes = [
         C.c_void_p, C.c_void_p, ULL, C.c_uint, ULL, ULL, ULL, C.c_void_p, ULL,
         C.POINTER(DeviceTensor), C.POINTER(OperationFacts), C.POINTER(Error)]
+    lib.yvex_backend_rocm_select_greedy_rows.argtypes = [
+        C.c_void_p, C.POINTER(DeviceTensor), ULL, ULL, C.c_void_p, C.c_void_p, C.c_void_p,
+        C.POINTER(OperationFacts), C.POINTER(Error)]
     lib.yvex_expert_worklist_build.argtypes = [C.c_void_p, C.c_void_p, ULL, ULL, ULL,
                                                C.POINTER(WorklistStorage),
                                                C.POINTER(WorklistObservation), C.POINTER(Error)]

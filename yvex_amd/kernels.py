@@ -110,6 +110,17 @@ def gather(encoded, qtype, row_count, row_width, row_ids, status):
     return out
 
 
+def argmax_f32(values, status):
+    """Greedy selection per row of a [rows, width] F32 tensor: (tokens u32, values f32, ties u64)."""
+    rows, width = values.shape
+    tokens = torch.zeros(rows, dtype=torch.int32, device=values.device)
+    best = torch.zeros(rows, dtype=torch.float32, device=values.device)
+    ties = torch.zeros(rows, dtype=torch.int64, device=values.device)
+    _call("yvex_hip_argmax_f32", _ptr(values), C.c_uint64(rows), C.c_uint64(width), _ptr(tokens),
+          _ptr(best), _ptr(ties), _ptr(status), _stream())
+    return tokens, best, ties
+
+
 def moe_route_rows(logits, bias, topk, scoring, normalize, scaling, status):
     rows, experts = logits.shape
     selected = torch.empty((rows, topk), dtype=torch.int64, device=logits.device)
