@@ -86,6 +86,39 @@ def dense_leg(torch, K, dev, repeats: int):
     gen.manual_seed(7)
     out = {}
 
+    def eager_and_graph(once, calls):
+        """Average time of once(): launched eagerly (ms) and replayed from a captured graph of
+        `calls` launches (us; None if capture is refused). The graph figure leaves out the host's
+        time per call, which is what a launch of a few microseconds is otherwise measured by."""
+        for _ in range(calls):
+            once()
+        torch.cuda.synchronize()
+        ms = event_ms(torch, once, repeats)
+        graph_us = None
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(calls):
+                        once()
+                graph.replay()
+                side.synchronize()
+                replays = max(1, repeats // calls)
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record(side)
+                for _ in range(replays):
+                    graph.replay()
+                stop.record(side)
+                stop.synchronize()
+                graph_us = start.elapsed_time(stop) / (replays * calls) * 1e3
+            torch.cuda.current_stream().wait_stream(side)
+        except Exception as error:   # capture refused: keep the eager figure
+            graph_us = None
+            print(f"dense leg: graph capture unavailable ({error})", file=sys.stderr)
+        return ms, graph_us
+
     def run(name, qt, rows, width, inputs, q8, copies=32):
         total = rows * K.row_bytes(qt, width)
         if qt == K.IQ2_XXS:
@@ -108,35 +141,7 @@ def dense_leg(torch, K, dev, repeats: int):
             turn[0] += 1
             K.matvec(w[i * total:(i + 1) * total], qt, rows, width, act, input_q8=q8, input_rows=inputs,
                      status=status, out=result)
-        for _ in range(copies):
-            once()
-        torch.cuda.synchronize()
-        ms = event_ms(torch, once, repeats)
-        # the same launches replayed from a captured graph: without the host's time per call,
-        # which is what a launch of a few microseconds is otherwise measured by
-        graph_us = None
-        try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(side):
-                with torch.cuda.graph(graph, stream=side):
-                    for _ in range(copies):
-                        once()
-                graph.replay()
-                side.synchronize()
-                replays = max(1, repeats // copies)
-                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record(side)
-                for _ in range(replays):
-                    graph.replay()
-                stop.record(side)
-                stop.synchronize()
-                graph_us = start.elapsed_time(stop) / (replays * copies) * 1e3
-            torch.cuda.current_stream().wait_stream(side)
-        except Exception as error:   # capture refused: keep the eager figure
-            graph_us = None
-            print(f"dense leg: graph capture unavailable ({error})", file=sys.stderr)
+        ms, graph_us = eager_and_graph(once, copies)
         best_ms = min(ms, graph_us * 1e-3) if graph_us else ms
         out[name] = {"us": round(ms * 1e3, 2), "graph_us": round(graph_us, 2) if graph_us else None,
                      "GB_per_s": round(total / (best_ms * 1e-3) / 1e9, 1),
@@ -154,10 +159,12 @@ def dense_leg(torch, K, dev, repeats: int):
     # greedy selection over one 129 280-entry logits row, left on the device by the head
     logits = torch.randn((1, 129280), device=dev, generator=gen)
     status = K.new_status(dev)
-    K.argmax_f32(logits, status)
+    picked = K.argmax_f32(logits, status)
     torch.cuda.synchronize()
-    ms = event_ms(torch, lambda: K.argmax_f32(logits, status), repeats)
-    out["greedy_selection_1x129280"] = {"us": round(ms * 1e3, 2), "status": int(status.item())}
+    ms, graph_us = eager_and_graph(lambda: K.argmax_f32(logits, status, out=picked), 16)
+    out["greedy_selection_1x129280"] = {"us": round(ms * 1e3, 2),
+                                        "graph_us": round(graph_us, 2) if graph_us else None,
+                                        "status": int(status.item())}
     return out
 
 

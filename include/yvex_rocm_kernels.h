@@ -55,13 +55,16 @@ int yvex_hip_block_dots_i32(const uint8_t *encoded, unsigned int qtype, uint64_t
                             uint64_t input_rows, int32_t *sums, int *status,
                             yvex_hip_stream stream);
 
-/* Replaces yvex_argmax_f32 (kernels.cu:59-110): for each of row_count rows of row_width F32 values
- * the largest value, the lowest index holding it and the number of elements holding it. Values
- * start from -FLT_MAX with no index (token 0xffffffff, ties 0 for a row of smaller values). A
- * non-finite element raises status 1 and its row publishes nothing. row_width < 2^32. */
+/* Replaces yvex_argmax_f32 (kernels.cu:59-110): for each of row_count (<= 65535) rows of
+ * row_width (< 2^32) F32 values the largest value, the lowest index holding it and the number of
+ * elements holding it. A non-finite element raises status 1 and its row publishes nothing.
+ * scratch (8-byte aligned device memory, may be NULL) lets a long row be split over several
+ * workgroups: with at least yvex_hip_argmax_scratch_bytes(row_count, row_width) bytes two
+ * launches share the row among the chip's compute units, without it one workgroup scans a row. */
+uint64_t yvex_hip_argmax_scratch_bytes(uint64_t row_count, uint64_t row_width);
 int yvex_hip_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
                         uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts,
-                        int *status, yvex_hip_stream stream);
+                        void *scratch, uint64_t scratch_bytes, int *status, yvex_hip_stream stream);
 
 /* Replaces yvex_qtype_gather / yvex_encoded_row_decode (kernels.cu:784-830): decode selected
  * rows to F32. row_ids may be NULL (rows 0..selected-1). */

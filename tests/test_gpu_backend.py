@@ -182,6 +182,13 @@ def test_select_greedy_rows(backend, oracle):
     rc, tokens, best, ties, facts, err = run_greedy(b, b.f32(values), rows, width)
     assert rc == abi.FORMAT and not tokens.any() and not best.any() and not ties.any()
     assert facts.kernel_launches == 0
+    # a vocabulary-sized row: shared among workgroups through the workspace (two launches)
+    b.workspace(1 << 16)
+    wide = rng.standard_normal((1, 129280)).astype(np.float32)
+    rc, tokens, best, ties, facts, err = run_greedy(b, b.f32(wide), 1, 129280)
+    assert rc == 0, err.message
+    assert tokens[0] == np.argmax(wide[0]) and best[0] == wide[0].max() and ties[0] == 1
+    assert facts.kernel_launches == 2
 
 
 class MoeCase:

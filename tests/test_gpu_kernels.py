@@ -189,7 +189,7 @@ def test_worklist_flags_duplicate_expert(gpu):
     assert int(status.item()) == 2
 
 
-@pytest.mark.parametrize("rows,width", [(1, 129280), (5, 1001), (3, 7), (32, 4096), (2, 1)])
+@pytest.mark.parametrize("rows,width", [(1, 129280), (5, 1001), (3, 7), (32, 4096), (2, 1), (3, 20001)])
 def test_greedy_selection_matches_oracle(gpu, oracle, rows, width):
     """Largest value, lowest index holding it, tie count: exact (kernels.cu:59-110)."""
     from yvex_amd import kernels as K
@@ -198,14 +198,15 @@ def test_greedy_selection_matches_oracle(gpu, oracle, rows, width):
     if width > 4:
         values[0, width - 1] = values[0, 1] = values[0].max() + 1.0   # a tie at both ends of row 0
         values[rows - 1] = np.round(values[rows - 1] * 2.0) / 2.0     # many ties in the last row
-    status = K.new_status(gpu)
-    tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
-    status_ok(status)
     rc, want_tokens, want_best, want_ties = oracle.argmax_f32(values)
     assert rc == 0
-    assert np.array_equal(tokens.cpu().numpy().astype(np.uint32), want_tokens)
-    assert np.array_equal(best.cpu().numpy(), want_best)
-    assert np.array_equal(ties.cpu().numpy().astype(np.uint64), want_ties)
+    for scratch in (None, False):     # rows split over workgroups (when long), one workgroup per row
+        status = K.new_status(gpu)
+        tokens, best, ties = K.argmax_f32(dev(values, gpu), status, scratch=scratch)
+        status_ok(status)
+        assert np.array_equal(tokens.cpu().numpy().astype(np.uint32), want_tokens)
+        assert np.array_equal(best.cpu().numpy(), want_best)
+        assert np.array_equal(ties.cpu().numpy().astype(np.uint64), want_ties)
 
 
 def test_greedy_selection_flags_non_finite(gpu, oracle):
@@ -224,3 +225,10 @@ def test_greedy_selection_flags_non_finite(gpu, oracle):
         assert int(tokens[row]) == want_tokens[row] and float(best[row]) == want_best[row]
         assert int(ties[row]) == want_ties[row]
     assert int(ties[1]) == 0
+    # a long row shared among workgroups: the status is raised and nothing is published
+    values = np.ones((2, 30000), np.float32)
+    values[1, 29999] = np.nan
+    status = K.new_status(gpu)
+    tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1 and int(ties[0]) == 0 and int(ties[1]) == 0

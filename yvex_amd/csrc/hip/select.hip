@@ -43,51 +43,101 @@ __device__ __forceinline__ void candidate_merge(Candidate &c, const Candidate &o
     }
 }
 
-constexpr unsigned kSelectThreads = 1024u;
-
-__global__ __launch_bounds__(kSelectThreads) void argmax_rows_kernel(
-    const float *values, unsigned long long row_count, unsigned long long row_width,
-    unsigned *selected_tokens, float *selected_values, unsigned long long *tie_counts, int *status)
+// Candidate of the elements [begin, end) of one row, held by thread 0 of the workgroup on return
+// (`ok` false when the span holds a non-finite value). THREADS threads.
+//
+// Two passes without branches, a compare-heavy single pass being bound by the vector ALUs: first
+// the largest finite value of the span (and whether anything is not finite), then, with the span
+// coming from cache, the lowest index and the count of the elements equal to it. Loads are 16
+// bytes over the aligned middle of the span and issued eight at a time.
+template <unsigned THREADS>
+__device__ __forceinline__ Candidate span_candidate(const float *row, unsigned long long begin,
+                                                    unsigned long long end, int *status, bool &ok)
 {
-    __shared__ float best_of[kSelectThreads / 64u];
-    __shared__ unsigned index_of[kSelectThreads / 64u];
-    __shared__ unsigned long long ties_of[kSelectThreads / 64u];
+    __shared__ float best_of[THREADS / 64u];
+    __shared__ unsigned index_of[THREADS / 64u];
+    __shared__ unsigned long long ties_of[THREADS / 64u];
     __shared__ int failed;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const unsigned long long row = blockIdx.x;
-    if (row >= row_count) return;
     if (tid == 0u) failed = 0;
     __syncthreads();
-    const float *v = values + row * row_width;
-    Candidate mine{-3.402823466e+38F, 0xffffffffu, 0ull};
-    bool bad = false;
-    auto look = [&](float value, unsigned index) {
-        if (!finite_f32(value)) bad = true;
-        else candidate_take(mine, value, index);
-    };
-    // 16-byte loads over the aligned middle of the row, scalar loads at its ends
+    const float *v = row + begin;
+    const unsigned long long count_all = end - begin;
     const unsigned long long address = (unsigned long long)v;
     unsigned long long head = ((16ull - (address & 15ull)) & 15ull) / 4ull;
-    if (head > row_width) head = row_width;
-    const unsigned long long quads = (row_width - head) / 4ull;
-    for (unsigned long long i = tid; i < head; i += kSelectThreads) look(v[i], (unsigned)i);
+    if (head > count_all) head = count_all;
+    const unsigned long long quads = (count_all - head) / 4ull;
+    const unsigned long long tail = head + 4ull * quads;
     const float4 *v4 = reinterpret_cast<const float4 *>(v + head);
-    for (unsigned long long q = tid; q < quads; q += kSelectThreads) {
-        const float4 x = v4[q];
-        const unsigned at = (unsigned)(head + 4ull * q);
-        look(x.x, at);
-        look(x.y, at + 1u);
-        look(x.z, at + 2u);
-        look(x.w, at + 3u);
-    }
-    for (unsigned long long i = head + 4ull * quads + tid; i < row_width; i += kSelectThreads)
-        look(v[i], (unsigned)i);
+    constexpr unsigned kBatch = 8u;
+    constexpr float kLowest = -3.402823466e+38F;
 
+    float top = kLowest;
+    bool bad = false;
+    auto rise = [&](float value) {
+        bad |= !finite_f32(value);
+        top = fmaxf(top, value);              // a NaN operand is dropped, an infinity is flagged above
+    };
+    for (unsigned long long i = tid; i < head; i += THREADS) rise(v[i]);
+    for (unsigned long long q0 = 0; q0 < quads; q0 += (unsigned long long)THREADS * kBatch) {
+        float4 x[kBatch];
+#pragma unroll
+        for (unsigned k = 0; k < kBatch; ++k) {
+            const unsigned long long q = q0 + tid + (unsigned long long)k * THREADS;
+            x[k] = v4[q < quads ? q : quads - 1ull];      // a repeated element changes no maximum
+        }
+#pragma unroll
+        for (unsigned k = 0; k < kBatch; ++k) {
+            rise(x[k].x);
+            rise(x[k].y);
+            rise(x[k].z);
+            rise(x[k].w);
+        }
+    }
+    for (unsigned long long i = tail + tid; i < count_all; i += THREADS) rise(v[i]);
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) top = fmaxf(top, __shfl_xor(top, offset, kWave));
+    if (lane == 0u) best_of[wave] = top;
     if (bad) {
         raise_status(status, 1);
         failed = 1;
     }
-    // wave, then workgroup
+    __syncthreads();
+    ok = failed == 0;
+    if (!ok) return Candidate{kLowest, 0xffffffffu, 0ull};
+#pragma unroll
+    for (unsigned w = 0; w < THREADS / 64u; ++w) top = fmaxf(top, best_of[w]);
+    __syncthreads();                          // best_of is reused below
+
+    // (the span's values cannot all lie below the starting value, the lowest finite float: `top`
+    // is a value of the span)
+    Candidate mine{top, 0xffffffffu, 0ull};
+    auto count = [&](float value, unsigned long long index, bool inside) {
+        const bool hit = inside && value == top;
+        const unsigned at = (unsigned)(begin + index);
+        mine.index = hit && at < mine.index ? at : mine.index;
+        mine.ties += hit ? 1ull : 0ull;
+    };
+    for (unsigned long long i = tid; i < head; i += THREADS) count(v[i], i, true);
+    for (unsigned long long q0 = 0; q0 < quads; q0 += (unsigned long long)THREADS * kBatch) {
+        float4 x[kBatch];
+#pragma unroll
+        for (unsigned k = 0; k < kBatch; ++k) {
+            const unsigned long long q = q0 + tid + (unsigned long long)k * THREADS;
+            x[k] = v4[q < quads ? q : quads - 1ull];
+        }
+#pragma unroll
+        for (unsigned k = 0; k < kBatch; ++k) {
+            const unsigned long long q = q0 + tid + (unsigned long long)k * THREADS;
+            const bool inside = q < quads;
+            const unsigned long long at = head + 4ull * q;
+            count(x[k].x, at, inside);
+            count(x[k].y, at + 1ull, inside);
+            count(x[k].z, at + 2ull, inside);
+            count(x[k].w, at + 3ull, inside);
+        }
+    }
+    for (unsigned long long i = tail + tid; i < count_all; i += THREADS) count(v[i], i, true);
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {
         Candidate other;
@@ -102,13 +152,79 @@ __global__ __launch_bounds__(kSelectThreads) void argmax_rows_kernel(
         ties_of[wave] = mine.ties;
     }
     __syncthreads();
-    if (tid == 0u && !failed) {
-        Candidate all{best_of[0], index_of[0], ties_of[0]};
-        for (unsigned w = 1; w < kSelectThreads / 64u; ++w)
+    Candidate all{best_of[0], index_of[0], ties_of[0]};
+    if (tid == 0u)
+        for (unsigned w = 1; w < THREADS / 64u; ++w)
             candidate_merge(all, Candidate{best_of[w], index_of[w], ties_of[w]});
+    return all;
+}
+
+constexpr unsigned kSelectThreads = 1024u;    // one workgroup per row
+constexpr unsigned kSpanThreads = 256u;       // several workgroups per row
+constexpr unsigned kSpanElements = 8192u;
+
+__global__ __launch_bounds__(kSelectThreads) void argmax_rows_kernel(
+    const float *values, unsigned long long row_count, unsigned long long row_width,
+    unsigned *selected_tokens, float *selected_values, unsigned long long *tie_counts, int *status)
+{
+    const unsigned long long row = blockIdx.x;
+    if (row >= row_count) return;
+    bool ok;
+    const Candidate all = span_candidate<kSelectThreads>(values + row * row_width, 0ull, row_width, status, ok);
+    if (threadIdx.x == 0u && ok) {
         selected_tokens[row] = all.index;
         selected_values[row] = all.best;
         tie_counts[row] = all.ties;
+    }
+}
+
+// A long row split over blockIdx.x spans of kSpanElements: partial candidates into scratch
+// ({float best, u32 index, u64 ties} per span), merged by argmax_merge_kernel.
+struct SpanResult {
+    float best;
+    unsigned index;
+    unsigned long long ties;
+};
+
+__global__ __launch_bounds__(kSpanThreads) void argmax_spans_kernel(
+    const float *values, unsigned long long row_count, unsigned long long row_width,
+    SpanResult *partial, int *status)
+{
+    const unsigned long long row = blockIdx.y, span = blockIdx.x;
+    const unsigned long long begin = span * kSpanElements;
+    if (row >= row_count || begin >= row_width) return;
+    const unsigned long long end = begin + kSpanElements < row_width ? begin + kSpanElements : row_width;
+    bool ok;
+    const Candidate all = span_candidate<kSpanThreads>(values + row * row_width, begin, end, status, ok);
+    if (threadIdx.x == 0u)
+        partial[row * gridDim.x + span] = ok ? SpanResult{all.best, all.index, all.ties}
+                                             : SpanResult{-3.402823466e+38F, 0xffffffffu, 0ull};
+}
+
+__global__ __launch_bounds__(64) void argmax_merge_kernel(
+    const SpanResult *partial, unsigned spans, unsigned long long row_count, unsigned *selected_tokens,
+    float *selected_values, unsigned long long *tie_counts, const int *status)
+{
+    const unsigned long long row = blockIdx.x;
+    if (row >= row_count || *status) return;      // a row with a bad value publishes nothing
+    const unsigned lane = threadIdx.x;
+    Candidate mine{-3.402823466e+38F, 0xffffffffu, 0ull};
+    for (unsigned s = lane; s < spans; s += 64u) {
+        const SpanResult r = partial[row * spans + s];
+        candidate_merge(mine, Candidate{r.best, r.index, r.ties});
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        Candidate other;
+        other.best = __shfl_xor(mine.best, offset, kWave);
+        other.index = (unsigned)__shfl_xor((int)mine.index, offset, kWave);
+        other.ties = (unsigned long long)__shfl_xor((long long)mine.ties, offset, kWave);
+        candidate_merge(mine, other);
+    }
+    if (lane == 0u) {
+        selected_tokens[row] = mine.index;
+        selected_values[row] = mine.best;
+        tie_counts[row] = mine.ties;
     }
 }
 
@@ -116,16 +232,36 @@ __global__ __launch_bounds__(kSelectThreads) void argmax_rows_kernel(
 
 using namespace yvex;
 
+extern "C" uint64_t yvex_hip_argmax_scratch_bytes(uint64_t row_count, uint64_t row_width)
+{
+    const uint64_t spans = (row_width + kSpanElements - 1u) / kSpanElements;
+    return spans > 1u ? row_count * spans * sizeof(SpanResult) : 0u;
+}
+
 extern "C" int yvex_hip_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
                                    uint32_t *selected_tokens, float *selected_values,
-                                   uint64_t *tie_counts, int *status, yvex_hip_stream stream)
+                                   uint64_t *tie_counts, void *scratch, uint64_t scratch_bytes,
+                                   int *status, yvex_hip_stream stream)
 {
     if (!values || !row_count || !row_width || !selected_tokens || !selected_values || !tie_counts ||
         !status)
         return ST_INVALID_ARG;
-    if (row_count > 0x7fffffffull || row_width > 0xffffffffull) return ST_BOUNDS;
-    if ((uintptr_t)values & 3u) return ST_INVALID_ARG;
-    argmax_rows_kernel<<<(unsigned)row_count, kSelectThreads, 0, as_stream(stream)>>>(
+    if (row_count > 65535ull || row_width > 0xffffffffull) return ST_BOUNDS;
+    if (((uintptr_t)values & 3u) || ((uintptr_t)scratch & 7u)) return ST_INVALID_ARG;
+    const uint64_t need = yvex_hip_argmax_scratch_bytes(row_count, row_width);
+    hipStream_t s = as_stream(stream);
+    if (need && scratch && scratch_bytes >= need) {
+        const unsigned spans = (unsigned)((row_width + kSpanElements - 1u) / kSpanElements);
+        argmax_spans_kernel<<<dim3(spans, (unsigned)row_count), kSpanThreads, 0, s>>>(
+            values, row_count, row_width, (SpanResult *)scratch, status);
+        int rc = check_launch("argmax_f32.spans");
+        if (rc) return rc;
+        argmax_merge_kernel<<<(unsigned)row_count, 64, 0, s>>>(
+            (const SpanResult *)scratch, spans, row_count, selected_tokens, selected_values,
+            (unsigned long long *)tie_counts, status);
+        return check_launch("argmax_f32.merge");
+    }
+    argmax_rows_kernel<<<(unsigned)row_count, kSelectThreads, 0, s>>>(
         values, row_count, row_width, selected_tokens, selected_values,
         (unsigned long long *)tie_counts, status);
     return check_launch("argmax_f32");

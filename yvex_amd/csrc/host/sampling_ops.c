@@ -28,6 +28,7 @@ int yvex_backend_rocm_select_greedy_rows(
     const char *where = "rocm.sampling.greedy";
     unsigned long long value_count, value_bytes, token_bytes, selected_bytes, tie_bytes;
     unsigned long long temporary_bytes, tokens_device = 0ull, values_device = 0ull, ties_device = 0ull, row;
+    unsigned long long scratch_bytes, scratch_device = 0ull;
     int device_status = 0, rc;
     if (facts) memset(facts, 0, sizeof(*facts));
     if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !logits || !selected_tokens ||
@@ -54,6 +55,11 @@ int yvex_backend_rocm_select_greedy_rows(
         !yvex_backend_workspace_acquire(backend, selected_bytes, 256ull, &values_device))
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                 "greedy row selection needs an attached workspace for its results");
+    /* long rows are shared among the compute units when the workspace has room for the partial
+     * results; otherwise one workgroup scans a row */
+    scratch_bytes = yvex_hip_argmax_scratch_bytes(row_count, row_width);
+    if (scratch_bytes && !yvex_backend_workspace_acquire(backend, scratch_bytes, 256ull, &scratch_device))
+        scratch_bytes = 0ull, scratch_device = 0ull;
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.sampling.greedy.launch",
                                 "kernel launch failed (test seam)");
@@ -62,8 +68,8 @@ int yvex_backend_rocm_select_greedy_rows(
         rc = yvex_rocm_launch_result(
             yvex_hip_argmax_f32((const float *)logits->data, row_count, row_width,
                                 (uint32_t *)(uintptr_t)tokens_device, (float *)(uintptr_t)values_device,
-                                (uint64_t *)(uintptr_t)ties_device, backend->device_status,
-                                backend->stream),
+                                (uint64_t *)(uintptr_t)ties_device, (void *)(uintptr_t)scratch_device,
+                                scratch_bytes, backend->device_status, backend->stream),
             "rocm.sampling.greedy.launch", err);
 #define READ(target_, source_, bytes_)                                                         \
     if (rc == YVEX_OK &&                                                                       \
@@ -86,7 +92,7 @@ int yvex_backend_rocm_select_greedy_rows(
         return rc;
     }
     facts->d2h_bytes = temporary_bytes;
-    facts->kernel_launches = 1ull;
+    facts->kernel_launches = scratch_bytes ? 2ull : 1ull;
     facts->download_count = 4ull;
     facts->stream_synchronizations = 1ull;
     facts->activation_bytes = value_bytes;

@@ -110,14 +110,25 @@ def gather(encoded, qtype, row_count, row_width, row_ids, status):
     return out
 
 
-def argmax_f32(values, status):
-    """Greedy selection per row of a [rows, width] F32 tensor: (tokens u32, values f32, ties u64)."""
+def argmax_f32(values, status, out=None, scratch=None):
+    """Greedy selection per row of a [rows, width] F32 tensor: (tokens u32, values f32, ties u64).
+    scratch: None = allocate what splitting long rows needs, False = one workgroup per row."""
     rows, width = values.shape
-    tokens = torch.zeros(rows, dtype=torch.int32, device=values.device)
-    best = torch.zeros(rows, dtype=torch.float32, device=values.device)
-    ties = torch.zeros(rows, dtype=torch.int64, device=values.device)
+    if out is None:
+        out = (torch.zeros(rows, dtype=torch.int32, device=values.device),
+               torch.zeros(rows, dtype=torch.float32, device=values.device),
+               torch.zeros(rows, dtype=torch.int64, device=values.device))
+    tokens, best, ties = out
+    lib = load_library()
+    lib.yvex_hip_argmax_scratch_bytes.restype = C.c_uint64
+    need = lib.yvex_hip_argmax_scratch_bytes(C.c_uint64(rows), C.c_uint64(width))
+    if scratch is None and need:
+        scratch = torch.empty(need, dtype=torch.uint8, device=values.device)
+    if scratch is False:
+        scratch = None
     _call("yvex_hip_argmax_f32", _ptr(values), C.c_uint64(rows), C.c_uint64(width), _ptr(tokens),
-          _ptr(best), _ptr(ties), _ptr(status), _stream())
+          _ptr(best), _ptr(ties), _ptr(scratch), C.c_uint64(scratch.numel() if scratch is not None else 0),
+          _ptr(status), _stream())
     return tokens, best, ties
 
 
