@@ -50,8 +50,12 @@ constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 
 // 1024 + 80 (r - 12): the two copies that fill a slot each write lane * 16.
 constexpr unsigned kWeightBase = kStageBase + 2u * kStageBytes;
 constexpr unsigned kWeightSlot = 1024u + 4u * 80u;
+// Item numbering: first full 128-pair tile of every bucket (257 words), then per class of last,
+// partial, tile (65-127, 33-64, 17-32, 1-16 pairs) a count and the list of its buckets (u16).
 constexpr unsigned kTileStartBase = kWeightBase + 8u * 2u * kWeightSlot;
-constexpr unsigned kTrashBase = kTileStartBase + 260u * 4u;   // 256 bytes nobody reads
+constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
+constexpr unsigned kClassListBase = kClassCountBase + 16u;
+constexpr unsigned kTrashBase = kClassListBase + 4u * 256u * 2u;   // 256 bytes nobody reads
 constexpr unsigned kMfmaLdsBytes = kTrashBase + 256u;
 
 struct MfmaArgs {
@@ -89,6 +93,24 @@ __device__ __forceinline__ v4i lds_read_v4i(unsigned address)
 #else
     (void)address;
     return v4i{0, 0, 0, 0};
+#endif
+}
+__device__ __forceinline__ void lds_write_u16(unsigned address, unsigned v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) unsigned short *>(address) = (unsigned short)v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ unsigned lds_read_u16(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const unsigned short *>(address);
+#else
+    (void)address;
+    return 0u;
 #endif
 }
 __device__ __forceinline__ unsigned lds_read_u32(unsigned address)
@@ -691,14 +713,23 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
 
     mfma_tables_fill();
     if (tid == 0u) {
-        // first 128-pair tile of every bucket
-        unsigned cursor = 0u;
+        // Full 128-pair tiles come first in the item list, then the partial last tiles by size,
+        // largest first: every workgroup, walking the list with the grid's stride, gets the same
+        // share of each kind of item, and the short items come last.
+        unsigned cursor = 0u, members[4] = {0u, 0u, 0u, 0u};
         for (unsigned b = 0; b < buckets && b < 256u; ++b) {
             lds_write_u32(kTileStartBase + 4u * b, cursor);
             const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[b];
-            cursor += (unsigned)((n + kTileTokens - 1u) / kTileTokens);
+            cursor += (unsigned)(n / kTileTokens);
+            const unsigned rest = (unsigned)(n % kTileTokens);
+            if (rest) {
+                const unsigned c = rest > 64u ? 0u : rest > 32u ? 1u : rest > 16u ? 2u : 3u;
+                lds_write_u16(kClassListBase + (c * 256u + members[c]) * 2u, b);
+                ++members[c];
+            }
         }
         lds_write_u32(kTileStartBase + 4u * (buckets < 256u ? buckets : 256u), cursor);
+        for (unsigned c = 0; c < 4u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
     }
     __syncthreads();
     if (buckets == 0u || buckets > 256u) {
@@ -709,29 +740,57 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
     // weight rows (gate/up row pairs when fused) per work item
     constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
     const unsigned row_tiles = (a.out_rows + kItemRows - 1u) / kItemRows;
-    const unsigned long long token_tiles = lds_read_u32(kTileStartBase + 4u * buckets);
-    const unsigned long long items = token_tiles * row_tiles;
+    const unsigned long long full_items = (unsigned long long)lds_read_u32(kTileStartBase + 4u * buckets) * row_tiles;
+    unsigned members[4];
+    unsigned long long items = full_items;
+    for (unsigned c = 0; c < 4u; ++c) {
+        members[c] = lds_read_u32(kClassCountBase + 4u * c);
+        items += (unsigned long long)members[c] * row_tiles;
+    }
 
     for (unsigned long long item = blockIdx.x; item < items; item += gridDim.x) {
         // ---- which bucket, row tile and token tile ----
-        unsigned low = 0u, high = buckets;
-        while (low + 1u < high) {
-            const unsigned middle = (low + high) >> 1;
-            if ((unsigned long long)lds_read_u32(kTileStartBase + 4u * middle) * row_tiles <= item)
-                low = middle;
-            else
-                high = middle;
-        }
-        const unsigned tile_first = lds_read_u32(kTileStartBase + 4u * low);
-        const unsigned bucket_tiles = lds_read_u32(kTileStartBase + 4u * (low + 1u)) - tile_first;
-        const unsigned long long local = item - (unsigned long long)tile_first * row_tiles;
-        const unsigned token_tile = bucket_tiles ? (unsigned)(local % bucket_tiles) : 0u;
-        const unsigned long long first = fixed ? 0ull : pr.bucket_offsets[low];
-        const unsigned long long population = fixed ? pr.pairs : pr.bucket_populations[low];
+        unsigned bucket, token_tile;
         MfmaItem it;
-        it.expert = fixed ? 0ull : pr.expert_ids[low];
-        it.row_tile = bucket_tiles ? (unsigned)(local / bucket_tiles) : 0u;
-        if (!bucket_tiles || it.expert >= pr.experts || first + population > pr.pairs ||
+        if (item < full_items) {
+            unsigned low = 0u, high = buckets;   // the last bucket whose first full tile is <= item's
+            while (low + 1u < high) {
+                const unsigned middle = (low + high) >> 1;
+                if ((unsigned long long)lds_read_u32(kTileStartBase + 4u * middle) * row_tiles <= item)
+                    low = middle;
+                else
+                    high = middle;
+            }
+            const unsigned tile_first = lds_read_u32(kTileStartBase + 4u * low);
+            const unsigned bucket_tiles = lds_read_u32(kTileStartBase + 4u * (low + 1u)) - tile_first;
+            const unsigned long long local = item - (unsigned long long)tile_first * row_tiles;
+            if (!bucket_tiles) {
+                if (tid == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            bucket = low;
+            token_tile = (unsigned)(local % bucket_tiles);
+            it.row_tile = (unsigned)(local / bucket_tiles);
+        } else {
+            unsigned long long rest = item - full_items;
+            unsigned c = 0u;
+            while (c < 3u && rest >= (unsigned long long)members[c] * row_tiles) {
+                rest -= (unsigned long long)members[c] * row_tiles;
+                ++c;
+            }
+            if (!members[c]) {
+                if (tid == 0u) raise_status(a.status, 2);
+                continue;
+            }
+            bucket = lds_read_u16(kClassListBase + (c * 256u + (unsigned)(rest % members[c])) * 2u);
+            it.row_tile = (unsigned)(rest / members[c]);
+            const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[bucket];
+            token_tile = (unsigned)(n / kTileTokens);
+        }
+        const unsigned long long first = fixed ? 0ull : pr.bucket_offsets[bucket];
+        const unsigned long long population = fixed ? pr.pairs : pr.bucket_populations[bucket];
+        it.expert = fixed ? 0ull : pr.expert_ids[bucket];
+        if (bucket >= buckets || it.expert >= pr.experts || first + population > pr.pairs ||
             (unsigned long long)token_tile * kTileTokens >= population || it.row_tile >= row_tiles) {
             if (tid == 0u) raise_status(a.status, 2);
             continue;
