@@ -56,7 +56,9 @@ constexpr unsigned kTileStartBase = kWeightBase + 8u * 2u * kWeightSlot;
 constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
 constexpr unsigned kClassListBase = kClassCountBase + 16u;
 constexpr unsigned kTrashBase = kClassListBase + 4u * 256u * 2u;   // 256 bytes nobody reads
-constexpr unsigned kMfmaLdsBytes = kTrashBase + 256u;
+// per pair of the item: {output row index, route weight}, read when the item publishes
+constexpr unsigned kPairInfoBase = kTrashBase + 256u;
+constexpr unsigned kMfmaLdsBytes = kPairInfoBase + kTileTokens * 8u;
 
 struct MfmaArgs {
     GroupedProblem pr;
@@ -277,34 +279,6 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     const unsigned superblocks = a.width >> 8;
     const unsigned last = superblocks - 1u;
 
-    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + kWaves, ... ----
-    // Lane l of a group moves piece position l % 16 of slot 4 g + l / 16; LDS receives the wave's
-    // 64 pieces back to back, so the swizzle is applied on the global side.
-    constexpr unsigned kCopies = kStagedSlots / (4u * kWaves);
-    auto token_row = [&](unsigned token) {
-        const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
-        const unsigned long long ordered = it.pair0 + live;
-        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
-        const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
-        return (const unsigned char *)pr.activations + arow * pr.act_stride;
-    };
-    const unsigned char *copy_from[kCopies];
-    unsigned copy_step[kCopies];            // superblock of the slot within its period
-#pragma unroll
-    for (unsigned j = 0; j < kCopies; ++j) {
-        const unsigned slot = 4u * (wave + kWaves * j) + (lane >> 4);
-        const unsigned token = slot % T;
-        copy_step[j] = slot / T;
-        copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
-    }
-    // Waves 0 and 1 also copy the 128 slot scales. The other waves run the same instruction on
-    // one address for all lanes (one cache line: next to free) into bytes nobody reads, which is
-    // cheaper than a branch around the copy.
-    const unsigned scale_slot = wave < 2u ? 64u * wave + lane : 0u;
-    const unsigned char *scale_from = token_row(scale_slot % T);
-    const unsigned scale_step = scale_slot / T;
-    const unsigned scale_to = wave < 2u ? kStageActs + wave * 256u : 0xffffffffu;
-
     // ---- the weight row of this lane: waves 0-3 hold gate blocks and waves 4-7 the matching up
     // blocks when the SwiGLU is fused ----
     unsigned out_row_base;
@@ -345,6 +319,51 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     }
     const unsigned weight_slots = kWeightBase + wave * 2u * kWeightSlot;
     const unsigned row_at = li < 12u ? li * 80u : 1024u + (li - 12u) * 80u;   // of the lane's row in a slot
+    constexpr unsigned kFetchPieces = 2u;
+    auto fetch_piece = [&](unsigned slot, unsigned sb, unsigned c) {
+        sb = sb < last ? sb : last;
+        const unsigned char *from = window_from[c] + ((window_misalign[c] + sb * 66u) & ~3u);
+        const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane((int)(weight_slots + slot * kWeightSlot + c * 1024u));
+        if (c == 0u) copy_to_lds_16(from, to);
+        else copy_to_lds_16_first20(from, to);
+    };
+    auto fetch_codes = [&](unsigned slot, unsigned sb) {
+#pragma unroll
+        for (unsigned c = 0; c < kFetchPieces; ++c) fetch_piece(slot, sb, c);
+    };
+    // The first two superblocks of the weight rows are asked for before anything else: their
+    // trip to HBM runs under the index loads and copies of the activation side below.
+    fetch_codes(0u, 0u);
+    fetch_codes(1u, 1u);
+
+    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + kWaves, ... ----
+    // Lane l of a group moves piece position l % 16 of slot 4 g + l / 16; LDS receives the wave's
+    // 64 pieces back to back, so the swizzle is applied on the global side.
+    constexpr unsigned kCopies = kStagedSlots / (4u * kWaves);
+    auto token_row = [&](unsigned token) {
+        const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
+        const unsigned long long ordered = it.pair0 + live;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
+        return (const unsigned char *)pr.activations + arow * pr.act_stride;
+    };
+    const unsigned char *copy_from[kCopies];
+    unsigned copy_step[kCopies];            // superblock of the slot within its period
+#pragma unroll
+    for (unsigned j = 0; j < kCopies; ++j) {
+        const unsigned slot = 4u * (wave + kWaves * j) + (lane >> 4);
+        const unsigned token = slot % T;
+        copy_step[j] = slot / T;
+        copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
+    }
+    // Waves 0 and 1 also copy the 128 slot scales. The other waves run the same instruction on
+    // one address for all lanes (one cache line: next to free) into bytes nobody reads, which is
+    // cheaper than a branch around the copy.
+    const unsigned scale_slot = wave < 2u ? 64u * wave + lane : 0u;
+    const unsigned char *scale_from = token_row(scale_slot % T);
+    const unsigned scale_step = scale_slot / T;
+    const unsigned scale_to = wave < 2u ? kStageActs + wave * 256u : 0xffffffffu;
+
     // The copies and loads of a step are issued one piece at a time between its matrix
     // instructions: a burst of them fills the memory pipeline's queue and holds the wave, and
     // with it its matrix instructions, until the queue drains.
@@ -367,18 +386,6 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     auto copy_activations = [&](unsigned period, unsigned stage) {
 #pragma unroll
         for (unsigned j = 0; j < kCopyPieces; ++j) copy_piece(period, stage, j);
-    };
-    constexpr unsigned kFetchPieces = 2u;
-    auto fetch_piece = [&](unsigned slot, unsigned sb, unsigned c) {
-        sb = sb < last ? sb : last;
-        const unsigned char *from = window_from[c] + ((window_misalign[c] + sb * 66u) & ~3u);
-        const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane((int)(weight_slots + slot * kWeightSlot + c * 1024u));
-        if (c == 0u) copy_to_lds_16(from, to);
-        else copy_to_lds_16_first20(from, to);
-    };
-    auto fetch_codes = [&](unsigned slot, unsigned sb) {
-#pragma unroll
-        for (unsigned c = 0; c < kFetchPieces; ++c) fetch_piece(slot, sb, c);
     };
     // Records of superblock sb out of the slot fetch_codes(slot, sb) filled. With o = (row start
     // + 2 sb) mod 4 (0 or 2) the fp16 scale sits o bytes into the window and the record of group
@@ -484,8 +491,14 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
 
     __syncthreads();   // every wave is done with the previous item's stages
     copy_activations(0u, 0u);
-#pragma unroll
-    for (unsigned k = 0; k < 2u; ++k) fetch_codes(k, k);
+    // where each pair's results go and its route weight, for the publishing pass
+    if (tid < kTileTokens && tid < it.tokens) {
+        const unsigned long long ordered = it.pair0 + tid;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
+        const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
+        lds_write_uint2(kPairInfoBase + tid * 8u, make_uint2((unsigned)out_index, __float_as_uint(route_weight)));
+    }
     {
         __builtin_amdgcn_s_waitcnt(0x0f70u);   // vmcnt(0): every copy above has landed
         const Codes first = settle_codes(0u, 0u);
@@ -498,11 +511,11 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         for (unsigned ks = 0; ks < 3u; ++ks) request(0u, ks);
         request_scale(stage_of(0u), 0u, 0u);
         row_scales(first, 0u, rs[0]);
+        Lookup lk[4];
 #pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) {
-            const Lookup lk = lookup(first, ks);
-            weights_from_lookup(lk, a_lo[0][ks], a_hi[0][ks]);
-        }
+        for (unsigned ks = 0; ks < 4u; ++ks) lk[ks] = lookup(first, ks);
+#pragma unroll
+        for (unsigned ks = 0; ks < 4u; ++ks) weights_from_lookup(lk[ks], a_lo[0][ks], a_hi[0][ks]);
     }
     sum_lo[1] = v4i{0, 0, 0, 0};
     sum_hi[1] = v4i{0, 0, 0, 0};
@@ -614,10 +627,7 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     for (unsigned r = 0; r < 4u; ++r) scale_row(D * NB - 1u, NB - 1u, rs[(D - 1u) & 1u][r], ts[(D * NB - 1u) & 1u], r);
 
     // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
-    auto store4 = [&](unsigned token, unsigned row, const float (&value)[4]) {
-        const unsigned long long ordered = it.pair0 + token;
-        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
-        const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
+    auto store4 = [&](unsigned long long out_index, unsigned row, const float (&value)[4]) {
         const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
                           finite_f32(value[3]);
         if (!good) raise_status(a.status, 1);
@@ -628,61 +638,37 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             for (unsigned r = 0; r < 4u; ++r)
                 if (row + r < a.out_rows) pr.out[out_index * a.out_rows + row + r] = value[r];
     };
-    auto route_weight_of = [&](unsigned token) {
-        const unsigned long long source = pr.order ? pr.order[it.pair0 + token] : it.pair0 + token;
-        return pr.route_weights ? pr.route_weights[source] : 1.0f;
-    };
     if constexpr (FUSED_UP) {
-        // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. They swap token
-        // blocks through LDS (the stages are free after the last barrier): gate waves finish
-        // blocks [0, G), up waves finish blocks [G, NB).
+        // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. All waves put their
+        // blocks into LDS (the stages are free after the last barrier); gate waves then finish
+        // token blocks [0, G) of their row block, up waves blocks [G, NB), in a loop that is not
+        // unrolled: the activation with its guarded fast path is long, and sixteen copies of it
+        // cost more in registers than they save.
         constexpr unsigned G = (NB + 1u) / 2u;
         const bool is_gate = wave < 4u;
-        const unsigned slot = kStageBase + ((wave & 3u) * 2u + (is_gate ? 0u : 1u)) * 4096u;
-        const unsigned peer = kStageBase + ((wave & 3u) * 2u + (is_gate ? 1u : 0u)) * 4096u;
-        if (is_gate) {
+        const unsigned pair_wave = wave & 3u;
 #pragma unroll
-            for (unsigned tb = G; tb < NB; ++tb)
-                lds_write_uint4(slot + ((tb - G) * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
-                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
-        } else {
-#pragma unroll
-            for (unsigned tb = 0; tb < G; ++tb)
-                lds_write_uint4(slot + (tb * 64u + lane) * 16u,
-                                make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
-                                           __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
-        }
+        for (unsigned tb = 0; tb < NB; ++tb)
+            lds_write_uint4(kStageBase + ((wave * NB + tb) * 64u + lane) * 16u,
+                            make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
+                                       __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
         __syncthreads();
-        if (is_gate) {
-#pragma unroll
-            for (unsigned tb = 0; tb < G; ++tb) {
-                const unsigned token = tb * 16u + li;
-                const uint4 other = lds_read_uint4(peer + (tb * 64u + lane) * 16u);
-                if (token < it.tokens) {
-                    const float route_weight = route_weight_of(token);
-                    const float value[4] = {
-                        swiglu_bf16(acc[tb][0], __uint_as_float(other.x), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][1], __uint_as_float(other.y), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][2], __uint_as_float(other.z), route_weight, a.limit),
-                        swiglu_bf16(acc[tb][3], __uint_as_float(other.w), route_weight, a.limit)};
-                    store4(token, out_row_base + 4u * kb, value);
-                }
-            }
-        } else {
-#pragma unroll
-            for (unsigned tb = G; tb < NB; ++tb) {
-                const unsigned token = tb * 16u + li;
-                const uint4 other = lds_read_uint4(peer + ((tb - G) * 64u + lane) * 16u);
-                if (token < it.tokens) {
-                    const float route_weight = route_weight_of(token);
-                    const float value[4] = {
-                        swiglu_bf16(__uint_as_float(other.x), acc[tb][0], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.y), acc[tb][1], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.z), acc[tb][2], route_weight, a.limit),
-                        swiglu_bf16(__uint_as_float(other.w), acc[tb][3], route_weight, a.limit)};
-                    store4(token, out_row_base + 4u * kb, value);
-                }
+        const unsigned tb_end = is_gate ? G : NB;
+        const float limit_f32 = (float)a.limit;
+#pragma unroll 1
+        for (unsigned tb = is_gate ? 0u : G; tb < tb_end; ++tb) {
+            const unsigned token = tb * 16u + li;
+            const uint4 g = lds_read_uint4(kStageBase + ((pair_wave * NB + tb) * 64u + lane) * 16u);
+            const uint4 u = lds_read_uint4(kStageBase + (((pair_wave + 4u) * NB + tb) * 64u + lane) * 16u);
+            if (token < it.tokens) {
+                const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
+                const float route_weight = __uint_as_float(info.y);
+                const float value[4] = {
+                    swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(u.x), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(u.y), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(u.z), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(u.w), route_weight, a.limit, limit_f32)};
+                store4(info.x, out_row_base + 4u * kb, value);
             }
         }
     } else {
@@ -690,9 +676,10 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         for (unsigned tb = 0; tb < NB; ++tb) {
             const unsigned token = tb * 16u + li;
             if (token < it.tokens) {
+                const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
                 const float value[4] = {bf16_round(acc[tb][0]), bf16_round(acc[tb][1]),
                                         bf16_round(acc[tb][2]), bf16_round(acc[tb][3])};
-                store4(token, out_row_base + 4u * kb, value);
+                store4(info.x, out_row_base + 4u * kb, value);
             }
         }
     }
