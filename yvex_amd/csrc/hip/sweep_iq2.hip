@@ -115,21 +115,24 @@ __device__ __forceinline__ void sweep_tables_fill()
 // A lane's share of one IQ2_XXS weight row: half a superblock, 32 packed bytes plus the scale.
 // Superblocks are 66 bytes, so the codes start on a 2-byte boundary, and vector loads that are
 // not dword-aligned run at less than half rate on this part. Every load here is dword-aligned:
-// nine dwords from the aligned address at or below the codes (the ninth only matters when the
-// codes start two bytes in) and the dword that holds the fp16 scale; the consumer shifts the
-// codes into place with byte-align instructions.
+// eight dwords from the aligned address at or below the codes and a ninth whose place depends on
+// the lane; the consumer shifts the codes into place with byte-align instructions. Each load
+// instruction costs the memory pipeline about two cycles per cache line its lanes touch, so the
+// fp16 scale gets no instruction of its own. Rows start on dword boundaries and superblocks are
+// 66 bytes, so in even superblocks the codes start two bytes into their aligned window: the
+// ninth dword is the end of the codes, and the scale is the low half of the first dword of the
+// superblock's first half. In odd superblocks the codes fill eight aligned dwords exactly and
+// the ninth load fetches the dword whose high half is the scale.
 struct Iq2Half {
     uint4 lo, hi;
-    unsigned tail, scale_word;
+    unsigned tail;
     // rows: wave-uniform address of the iteration's first weight row; the rest are this lane's
     // byte offsets from it (scalar base + 32-bit lane offset addressing)
-    __device__ __forceinline__ void load(const unsigned char *rows, unsigned codes_at,
-                                         unsigned tail_at, unsigned scale_at)
+    __device__ __forceinline__ void load(const unsigned char *rows, unsigned codes_at, unsigned tail_at)
     {
         lo = *reinterpret_cast<const uint4 *>(rows + codes_at);          // 4-byte aligned
         hi = *reinterpret_cast<const uint4 *>(rows + codes_at + 16u);
         tail = *reinterpret_cast<const unsigned *>(rows + tail_at);
-        scale_word = *reinterpret_cast<const unsigned *>(rows + scale_at);
     }
 };
 
@@ -315,8 +318,9 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned up_block = lane_row * (unsigned)pr.up_row_bytes + lane_super * 66u;
     const unsigned gate_codes_at = (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
     const unsigned up_codes_at = (up_block + 2u + 32u * g.half) & ~3u;
-    const unsigned tail_step = g.code_shift ? 32u : 0u;   // aligned codes end inside 32 bytes
-    const unsigned gate_scale_at = gate_block & ~3u, up_scale_at = up_block & ~3u;
+    // ninth dword: the end of the codes where they start two bytes in, else the scale's dword
+    const unsigned gate_tail_at = g.code_shift ? gate_codes_at + 32u : gate_block & ~3u;
+    const unsigned up_tail_at = g.code_shift ? up_codes_at + 32u : up_block & ~3u;
     // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
     // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
@@ -328,9 +332,9 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned last = iterations - 1u;
     auto request = [&](Iq2Half (&slot)[STREAMS], unsigned it) {
         const unsigned clamped = it < last ? it : last;
-        slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_codes_at + tail_step, gate_scale_at);
+        slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at);
         if constexpr (FUSED)
-            slot[1].load(up_rows + clamped * up_step, up_codes_at, up_codes_at + tail_step, up_scale_at);
+            slot[1].load(up_rows + clamped * up_step, up_codes_at, up_tail_at);
     };
     // The first requests are kept in ring order: the loop's first wait is counted against the
     // loads issued after the slot it consumes, on the entry path and on the back edge alike.
@@ -366,9 +370,15 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             total_gate[p] += dpp_move<0xb1, 0xf>(total_gate[p]);
             if constexpr (FUSED) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
         }
-        float weight_scale;
-        weight_scale = 0.125f * f16_bits_to_float(
-            ((odd ? now[STREAMS - 1].scale_word : now[0].scale_word) >> g.scale_shift) & 0xffffu);
+        // The even lane of a pair scales the first stream and the odd lane the last one. An odd
+        // lane holds the second half of its superblock, so where the scale rides in the first
+        // half's codes it comes from the neighbour.
+        const Iq2Half &mine = odd ? now[STREAMS - 1] : now[0];
+        // (the exchange runs in every lane: it reads its neighbour, which must be executing it)
+        const unsigned neighbour_word = (unsigned)dpp_move<0xb1, 0xf>((int)now[STREAMS - 1].lo.x);
+        const unsigned first_word = odd ? neighbour_word : now[0].lo.x;
+        const float weight_scale = 0.125f * f16_bits_to_float(
+            ((g.code_shift ? first_word : mine.tail) >> g.scale_shift) & 0xffffu);
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
             int t;
