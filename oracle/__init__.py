@@ -329,6 +329,65 @@ def worklist_build(selected: np.ndarray, weights: np.ndarray, topk: int, experts
                     source_pairs=sp, source_rows=sr, destination_rows=dr, route_weights=ow)
 
 
+def rms_norm(values: np.ndarray, weights: np.ndarray, epsilon: float):
+    """numeric.c:630-666 on one vector; returns (rc, normalised copy)."""
+    out = np.array(values, np.float32).ravel()
+    weights = np.ascontiguousarray(weights, np.float32).ravel()
+    rc = lib().yvo_rms_norm(_p(out), C.c_uint64(out.size), _p(weights), C.c_double(epsilon))
+    return rc, out
+
+
+def mhc_pre(residual, mixes, scale, base, *, streams, width, iterations, rms_epsilon, mhc_epsilon,
+            post_multiplier):
+    """numeric.c:752-826: (rc, collapsed [t, width], post [t, streams], combination [t, s, s])."""
+    residual = np.ascontiguousarray(residual, np.float32).reshape(-1, streams * width)
+    tokens = residual.shape[0]
+    mixes = np.ascontiguousarray(mixes, np.float32).reshape(tokens, (streams + 2) * streams)
+    scale = np.ascontiguousarray(scale, np.float32).ravel()
+    base = np.ascontiguousarray(base, np.float32).ravel()
+    collapsed = np.zeros((tokens, width), np.float32)
+    post = np.zeros((tokens, streams), np.float32)
+    comb = np.zeros((tokens, streams, streams), np.float32)
+    rc = lib().yvo_mhc_pre(_p(residual), _p(mixes), _p(scale), _p(base), C.c_uint64(tokens),
+                           C.c_uint64(streams), C.c_uint64(width), C.c_uint64(iterations),
+                           C.c_double(rms_epsilon), C.c_double(mhc_epsilon),
+                           C.c_double(post_multiplier), _p(collapsed), _p(post), _p(comb))
+    return rc, collapsed, post, comb
+
+
+def mhc_post(core, residual, post, combination, *, streams, width):
+    """numeric.c:828-877: (rc, envelope output [t, streams * width])."""
+    core = np.ascontiguousarray(core, np.float32).reshape(-1, width)
+    tokens = core.shape[0]
+    residual = np.ascontiguousarray(residual, np.float32).reshape(tokens, streams * width)
+    post = np.ascontiguousarray(post, np.float32).reshape(tokens, streams)
+    combination = np.ascontiguousarray(combination, np.float32).reshape(tokens, streams * streams)
+    out = np.zeros((tokens, streams * width), np.float32)
+    rc = lib().yvo_mhc_post(_p(core), _p(residual), _p(post), _p(combination), C.c_uint64(tokens),
+                            C.c_uint64(streams), C.c_uint64(width), _p(out))
+    return rc, out
+
+
+def moe_ffn_prepare(function_qtype, function, expanded, scale, base, norm, *, streams, width,
+                    iterations, rms_epsilon, mhc_epsilon, post_multiplier):
+    """moe.c:446-495: (rc, normalized [t, width], post [t, streams], combination [t, s, s])."""
+    function = np.ascontiguousarray(function, np.uint8)
+    expanded = np.ascontiguousarray(expanded, np.float32).reshape(-1, streams * width)
+    tokens = expanded.shape[0]
+    scale = np.ascontiguousarray(scale, np.float32).ravel()
+    base = np.ascontiguousarray(base, np.float32).ravel()
+    norm = np.ascontiguousarray(norm, np.float32).ravel()
+    normalized = np.zeros((tokens, width), np.float32)
+    post = np.zeros((tokens, streams), np.float32)
+    comb = np.zeros((tokens, streams, streams), np.float32)
+    rc = lib().yvo_moe_ffn_prepare(C.c_uint(function_qtype), _p(function), _p(expanded), _p(scale),
+                                   _p(base), _p(norm), C.c_uint64(tokens), C.c_uint64(streams),
+                                   C.c_uint64(width), C.c_uint64(iterations), C.c_double(rms_epsilon),
+                                   C.c_double(mhc_epsilon), C.c_double(post_multiplier),
+                                   _p(normalized), _p(post), _p(comb))
+    return rc, normalized, post, comb
+
+
 def moe_layer(*, hidden, intermediate, experts, topk, qtypes, routed, shared, inputs, logits,
               bias=None, scoring=SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
               act_q8=False, threads=1):

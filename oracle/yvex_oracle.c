@@ -794,6 +794,196 @@ int yvo_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
     return status;
 }
 
+/* ---- residual-stream envelope around the expert math ---- */
+
+/* src/graph/numeric.c:630-666: mean of squares in double, one rounding to float per value */
+int yvo_rms_norm(float *values, uint64_t count, const float *weights, double epsilon)
+{
+    double mean = 0.0, inverse;
+    uint64_t i;
+    if (!values || !count || !weights || !isfinite(epsilon) || epsilon <= 0.0)
+        return YVO_ERR_INVALID_ARG;
+    for (i = 0; i < count; ++i) {
+        if (!isfinite(values[i]) || !isfinite(weights[i])) return YVO_ERR_FORMAT;
+        mean += (double)values[i] * (double)values[i];
+    }
+    mean /= (double)count;
+    inverse = 1.0 / sqrt(mean + epsilon);
+    if (!isfinite(inverse)) return YVO_ERR_FORMAT;
+    for (i = 0; i < count; ++i) {
+        double v = (double)values[i] * inverse;
+        v *= (double)weights[i];
+        if (!isfinite(v)) return YVO_ERR_FORMAT;
+        values[i] = (float)v;
+    }
+    return YVO_OK;
+}
+
+/* src/graph/numeric.c:691-702 */
+static double envelope_sigmoid(double value)
+{
+    if (value >= 0.0) return 1.0 / (1.0 + exp(-value));
+    {
+        double direct = exp(value);
+        return direct / (1.0 + direct);
+    }
+}
+
+/* src/graph/numeric.c:704-750: row softmax (+ epsilon), then alternating row and column
+ * normalisations; the first iteration normalises columns only */
+static int envelope_sinkhorn(float *m, uint64_t n, uint64_t iterations, double epsilon)
+{
+    uint64_t r, c, it;
+    for (r = 0; r < n; ++r) {
+        double maximum = -(double)INFINITY, total = 0.0;
+        for (c = 0; c < n; ++c) maximum = fmax(maximum, m[r * n + c]);
+        for (c = 0; c < n; ++c) {
+            double value = exp((double)m[r * n + c] - maximum);
+            m[r * n + c] = (float)value;
+            total += value;
+        }
+        if (!isfinite(total) || total <= 0.0) return 0;
+        for (c = 0; c < n; ++c) m[r * n + c] = (float)((double)m[r * n + c] / total + epsilon);
+    }
+    for (it = 0; it < iterations; ++it) {
+        if (it != 0) {
+            for (r = 0; r < n; ++r) {
+                double total = 0.0;
+                for (c = 0; c < n; ++c) total += m[r * n + c];
+                if (!isfinite(total)) return 0;
+                for (c = 0; c < n; ++c)
+                    m[r * n + c] = (float)((double)m[r * n + c] / (total + epsilon));
+            }
+        }
+        for (c = 0; c < n; ++c) {
+            double total = 0.0;
+            for (r = 0; r < n; ++r) total += m[r * n + c];
+            if (!isfinite(total)) return 0;
+            for (r = 0; r < n; ++r)
+                m[r * n + c] = (float)((double)m[r * n + c] / (total + epsilon));
+        }
+    }
+    return 1;
+}
+
+/* src/graph/numeric.c:752-826 with dense strides */
+int yvo_mhc_pre(const float *residual, const float *mixes, const float *scale, const float *base,
+                uint64_t tokens, uint64_t streams, uint64_t width, uint64_t iterations,
+                double rms_epsilon, double mhc_epsilon, double post_multiplier, float *collapsed,
+                float *post, float *combination)
+{
+    const uint64_t expanded = streams * width, mixing_rows = (streams + 2u) * streams;
+    uint64_t token, stream, target, lane;
+    if (!residual || !mixes || !scale || !base || !collapsed || !post || !combination || !tokens ||
+        !streams || !width || !iterations || !(rms_epsilon > 0.0) || !(mhc_epsilon > 0.0) ||
+        !(post_multiplier > 0.0) || !isfinite(rms_epsilon) || !isfinite(mhc_epsilon) ||
+        !isfinite(post_multiplier))
+        return YVO_ERR_BOUNDS;
+    for (lane = 0; lane < 3u; ++lane)
+        if (!isfinite(scale[lane])) return YVO_ERR_FORMAT;
+    for (lane = 0; lane < mixing_rows; ++lane)
+        if (!isfinite(base[lane])) return YVO_ERR_FORMAT;
+    for (token = 0; token < tokens; ++token) {
+        const float *res = residual + token * expanded;
+        const float *mix = mixes + token * mixing_rows;
+        float *out = collapsed + token * width;
+        float *po = post + token * streams;
+        float *comb = combination + token * streams * streams;
+        double squares = 0.0, inverse;
+        memset(out, 0, (size_t)width * sizeof(*out));
+        for (lane = 0; lane < expanded; ++lane) {
+            if (!isfinite(res[lane])) return YVO_ERR_FORMAT;
+            squares += (double)res[lane] * (double)res[lane];
+        }
+        inverse = 1.0 / sqrt(squares / (double)expanded + rms_epsilon);
+        if (!isfinite(inverse)) return YVO_ERR_FORMAT;
+        for (stream = 0; stream < streams; ++stream) {
+            double pre = envelope_sigmoid((double)mix[stream] * inverse * (double)scale[0] +
+                                          (double)base[stream]);
+            po[stream] = (float)(post_multiplier * envelope_sigmoid(
+                (double)mix[streams + stream] * inverse * (double)scale[1] +
+                (double)base[streams + stream]));
+            for (target = 0; target < streams; ++target) {
+                uint64_t index = 2u * streams + stream * streams + target;
+                comb[stream * streams + target] =
+                    (float)((double)mix[index] * inverse * (double)scale[2] + (double)base[index]);
+            }
+            for (lane = 0; lane < width; ++lane)
+                out[lane] += (float)((pre + mhc_epsilon) * (double)res[stream * width + lane]);
+        }
+        if (!envelope_sinkhorn(comb, streams, iterations, mhc_epsilon)) return YVO_ERR_FORMAT;
+        for (lane = 0; lane < width; ++lane) {
+            if (!isfinite(out[lane])) return YVO_ERR_FORMAT;
+            out[lane] = yvo_bf16_round(out[lane]);
+        }
+    }
+    return YVO_OK;
+}
+
+/* src/graph/numeric.c:828-877 with dense strides: combination rows are sources, columns targets */
+int yvo_mhc_post(const float *core, const float *residual, const float *post,
+                 const float *combination, uint64_t tokens, uint64_t streams, uint64_t width,
+                 float *output)
+{
+    uint64_t token, target, source, lane;
+    if (!core || !residual || !post || !combination || !output || !tokens || !streams || !width)
+        return YVO_ERR_BOUNDS;
+    for (token = 0; token < tokens; ++token) {
+        const float *c = core + token * width, *res = residual + token * streams * width;
+        const float *po = post + token * streams, *comb = combination + token * streams * streams;
+        float *out = output + token * streams * width;
+        for (target = 0; target < streams; ++target)
+            for (lane = 0; lane < width; ++lane) {
+                double value = (double)po[target] * (double)c[lane];
+                for (source = 0; source < streams; ++source)
+                    value += (double)comb[source * streams + target] *
+                             (double)res[source * width + lane];
+                if (!isfinite(value)) return YVO_ERR_FORMAT;
+                out[target * width + lane] = (float)value;
+            }
+        for (lane = 0; lane < streams * width; ++lane) {
+            if (!isfinite(out[lane])) return YVO_ERR_FORMAT;
+            out[lane] = yvo_bf16_round(out[lane]);
+        }
+    }
+    return YVO_OK;
+}
+
+/* src/graph/moe.c:446-495: mixes = function . expanded row through the CPU row dot, ingress,
+ * weighted RMS norm, bf16 publication. scale, base and norm arrive decoded (moe.c:405-428
+ * copies F32, widens BF16 and converts I32). */
+int yvo_moe_ffn_prepare(unsigned int function_qtype, const uint8_t *function,
+                        const float *expanded, const float *scale, const float *base,
+                        const float *norm, uint64_t tokens, uint64_t streams, uint64_t width,
+                        uint64_t iterations, double rms_epsilon, double mhc_epsilon,
+                        double post_multiplier, float *normalized, float *post, float *combination)
+{
+    const uint64_t expanded_width = streams * width, mixing_rows = (streams + 2u) * streams;
+    float mix[64];
+    uint64_t token;
+    int rc;
+    if (!function || !expanded || !norm || !normalized || mixing_rows > 64u || width > 16384u)
+        return YVO_ERR_INVALID_ARG;
+    for (token = 0; token < tokens; ++token) {
+        float *row = normalized + token * width;
+        uint64_t lane;
+        rc = yvo_matvec(function_qtype, function, mixing_rows, expanded_width,
+                        expanded + token * expanded_width, 1, mix);
+        if (rc != YVO_OK) return rc;
+        rc = yvo_mhc_pre(expanded + token * expanded_width, mix, scale, base, 1, streams, width,
+                         iterations, rms_epsilon, mhc_epsilon, post_multiplier, row,
+                         post + token * streams, combination + token * streams * streams);
+        if (rc != YVO_OK) return rc;
+        rc = yvo_rms_norm(row, width, norm, rms_epsilon);
+        if (rc != YVO_OK) return rc;
+        for (lane = 0; lane < width; ++lane) {
+            if (!isfinite(row[lane])) return YVO_ERR_FORMAT;
+            row[lane] = yvo_bf16_round(row[lane]);
+        }
+    }
+    return YVO_OK;
+}
+
 /* ---- worklist: src/graph/worklist.c:369-441 ---- */
 
 int yvo_worklist_build(const uint64_t *selected_experts, const float *route_weights,

@@ -168,6 +168,29 @@ int yvo_worklist_build(const uint64_t *selected_experts, const float *route_weig
 int yvo_argmax_f32(const float *values, uint64_t row_count, uint64_t row_width,
                    uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts);
 
+/* Residual-stream envelope around the expert math (dense strides; tokens x streams x width).
+ * yvo_rms_norm: src/graph/numeric.c:630-666. yvo_mhc_pre: numeric.c:691-826 (sigmoid, Sinkhorn,
+ * ingress; collapsed is bf16-rounded as the compute contract asks). yvo_mhc_post:
+ * numeric.c:828-877. yvo_moe_ffn_prepare: src/graph/moe.c:446-495 (mixes through the CPU row
+ * dot, ingress, weighted RMS norm, bf16 publication) with scale, base and norm already decoded.
+ * Pinned by the reference's own vectors (tests/unit/deepseek_attention.c:2255-2266,2302-2309 and
+ * tests/reference/deepseek_attention.c:2725-2730), by float64 closed forms (doubly-stochastic
+ * combination, einsum egress, sigmoid limits) and by a fixture written from the compiled
+ * reference's yvex_moe_ffn_prepare_cpu. */
+int yvo_rms_norm(float *values, uint64_t count, const float *weights, double epsilon);
+int yvo_mhc_pre(const float *residual, const float *mixes, const float *scale, const float *base,
+                uint64_t tokens, uint64_t streams, uint64_t width, uint64_t iterations,
+                double rms_epsilon, double mhc_epsilon, double post_multiplier, float *collapsed,
+                float *post, float *combination);
+int yvo_mhc_post(const float *core, const float *residual, const float *post,
+                 const float *combination, uint64_t tokens, uint64_t streams, uint64_t width,
+                 float *output);
+int yvo_moe_ffn_prepare(unsigned int function_qtype, const uint8_t *function,
+                        const float *expanded, const float *scale, const float *base,
+                        const float *norm, uint64_t tokens, uint64_t streams, uint64_t width,
+                        uint64_t iterations, double rms_epsilon, double mhc_epsilon,
+                        double post_multiplier, float *normalized, float *post, float *combination);
+
 /* MoE layer over a row batch: routing given logits, routed experts in rank order, one shared
  * expert, combined = bf16(routed + shared) (src/runtime/moe.c:596-632).
  * Weights: routed gate/up/down are expert-major ([experts][rows][row_bytes]).

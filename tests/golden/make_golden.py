@@ -150,6 +150,42 @@ def main():
         out[f"expert_{name}_gate"], out[f"expert_{name}_up"] = gate, up
         out[f"expert_{name}_down"], out[f"expert_{name}_x"] = down, x
         out[f"expert_{name}_out_bits"] = y.view(np.uint32)
+    # residual-stream ingress in front of the experts: mixes, Sinkhorn, weighted RMS norm
+    ref.yvex_moe_ffn_prepare_cpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    for name, streams, width, iterations, tokens in (("wide", 4, 64, 20, 3), ("single", 1, 32, 1, 2)):
+        gen = oracle.Generator(42, f"golden.ingress.{name}")
+        mixing, expanded = (streams + 2) * streams, streams * width
+        function = gen.normal(mixing * expanded, 0.2)
+        scale = gen.normal(3, 0.7)
+        base = gen.normal(mixing, 0.5)
+        norm_bits = ((1.0 + gen.normal(width, 0.2)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        rows = np.round(gen.normal(tokens * expanded) * 64.0) / 64.0     # exact in bf16
+        rows = rows.astype(np.float32).reshape(tokens, expanded)
+        plan = abi.LayerPlan()
+        plan.hidden_width, plan.residual_streams, plan.expanded_width = width, streams, expanded
+        plan.mhc_mixing_rows, plan.mhc_sinkhorn_iterations = mixing, iterations
+        plan.rms_epsilon, plan.mhc_epsilon, plan.mhc_post_multiplier = 1e-6, 1e-6, 2.0
+        job = abi.LayerJob()
+        job.layer = C.pointer(plan)
+        job.weights[abi.W_MHC_FUNCTION] = weight_view(function.view(np.uint8), 0, expanded, mixing)
+        job.weights[abi.W_MHC_SCALE] = weight_view(scale.view(np.uint8), 0, 3, 1)
+        job.weights[abi.W_MHC_BASE] = weight_view(base.view(np.uint8), 0, mixing, 1)
+        job.weights[abi.W_FFN_NORM] = weight_view(norm_bits.view(np.uint8), 30, width, 1)
+        normalized = np.zeros((tokens, width), np.float32)
+        post = np.zeros((tokens, streams), np.float32)
+        comb = np.zeros((tokens, streams * streams), np.float32)
+        for t in range(tokens):
+            err = abi.Error()
+            job.expanded_input = rows[t].ctypes.data
+            rc = ref.yvex_moe_ffn_prepare_cpu(C.byref(job), normalized[t].ctypes.data, post[t].ctypes.data,
+                                              comb[t].ctypes.data, C.byref(err))
+            assert rc == 0, err.message
+        out[f"ingress_{name}_function"], out[f"ingress_{name}_scale"] = function, scale
+        out[f"ingress_{name}_base"], out[f"ingress_{name}_norm_bf16"] = base, norm_bits
+        out[f"ingress_{name}_rows"] = rows
+        out[f"ingress_{name}_normalized_bits"] = normalized.view(np.uint32)
+        out[f"ingress_{name}_post_bits"] = post.view(np.uint32)
+        out[f"ingress_{name}_combination_bits"] = comb.view(np.uint32)
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes")

@@ -426,3 +426,100 @@ def test_greedy_selection_against_brute_force(oracle):
     assert rc == 1
     assert (tokens[0], best[0], ties[0]) == (1, 2.0, 2) and (tokens[3], best[3], ties[3]) == (0, 4.0, 1)
     assert ties[1] == 0 and ties[2] == 0
+
+
+# ---- residual-stream envelope: tests/unit/deepseek_attention.c:2255-2340 ----------------------
+
+def test_envelope_egress_reference_vectors(oracle):
+    """The reference's own known answers for the egress: combination rows are sources and columns
+    are targets (deepseek_attention.c:2263-2266,2302-2309) and the external conformance vector
+    (tests/reference/deepseek_attention.c:2725-2730)."""
+    rc, out = oracle.mhc_post([0.5, -0.25], [1, 2, 3, 4], [0, 0], [1, 2, 3, 4], streams=2, width=2)
+    assert rc == 0 and out.ravel().tolist() == [10.0, 14.0, 14.0, 20.0]
+    rc, out = oracle.mhc_post([0.5, -0.25], [1, 2, 3, 4], [2, 1], [1, 2, 3, 4], streams=2, width=2)
+    assert rc == 0 and out.ravel().tolist() == [11.0, 13.5, 14.5, 19.75]
+
+
+def test_envelope_egress_against_einsum(oracle):
+    rng = np.random.default_rng(3)
+    tokens, streams, width = 5, 4, 48
+    core = rng.standard_normal((tokens, width)).astype(np.float32)
+    res = rng.standard_normal((tokens, streams, width)).astype(np.float32)
+    post = rng.random((tokens, streams)).astype(np.float32)
+    comb = rng.random((tokens, streams, streams)).astype(np.float32)
+    rc, out = oracle.mhc_post(core, res, post, comb, streams=streams, width=width)
+    want = np.einsum("bt,bl->btl", post.astype(np.float64), core.astype(np.float64)) + \
+        np.einsum("bst,bsl->btl", comb.astype(np.float64), res.astype(np.float64))
+    got = out.reshape(tokens, streams, width)
+    assert rc == 0 and np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)   # one bf16 rounding
+    assert np.array_equal(bits(got) & 0xffff, np.zeros_like(bits(got)))                 # bf16 values
+    bad = core.copy()
+    bad[2, 5] = np.inf
+    assert oracle.mhc_post(bad, res, post, comb, streams=streams, width=width)[0] == oracle.ERR_FORMAT
+
+
+def test_envelope_ingress_closed_forms(oracle):
+    """Ingress against what the mathematics fixes: sigmoid gates from an independent float64
+    formula, a combination matrix whose rows and columns sum to one after enough Sinkhorn turns,
+    collapsed rows as the gate-weighted sum of the streams, and the unit test's refusal of
+    non-finite coefficients."""
+    rng = np.random.default_rng(11)
+    tokens, streams, width = 4, 4, 40
+    mixing = (streams + 2) * streams
+    res = (np.round(rng.standard_normal((tokens, streams * width)) * 32) / 32).astype(np.float32)
+    mix = rng.standard_normal((tokens, mixing)).astype(np.float32)
+    scale = np.array([0.5, -0.25, 0.75], np.float32)
+    base = (rng.standard_normal(mixing) * 0.3).astype(np.float32)
+    rc, collapsed, post, comb = oracle.mhc_pre(res, mix, scale, base, streams=streams, width=width,
+                                               iterations=20, rms_epsilon=1e-6, mhc_epsilon=1e-6,
+                                               post_multiplier=2.0)
+    assert rc == 0
+    r64, m64 = res.astype(np.float64), mix.astype(np.float64)
+    inverse = 1.0 / np.sqrt((r64 ** 2).mean(axis=1) + 1e-6)
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    pre = sig(m64[:, :streams] * inverse[:, None] * 0.5 + base[:streams]) + 1e-6
+    want_post = 2.0 * sig(m64[:, streams:2 * streams] * inverse[:, None] * -0.25 + base[streams:2 * streams])
+    assert np.allclose(post, want_post, rtol=1e-6, atol=0)
+    want = np.einsum("bs,bsl->bl", pre, r64.reshape(tokens, streams, width))
+    assert np.all(np.abs(collapsed - want) <= 2.0 ** -8 * np.abs(want) + 1e-6)
+    assert np.allclose(comb.sum(axis=1), 1.0, atol=1e-4) and np.allclose(comb.sum(axis=2), 1.0, atol=1e-4)
+    assert np.all(comb > 0)
+    # one Sinkhorn turn is the row softmax followed by one column normalisation
+    rc, _, _, once = oracle.mhc_pre(res, mix, scale, base, streams=streams, width=width, iterations=1,
+                                    rms_epsilon=1e-6, mhc_epsilon=1e-6, post_multiplier=2.0)
+    raw = m64[:, 2 * streams:].reshape(tokens, streams, streams) * inverse[:, None, None] * 0.75 + \
+        base[2 * streams:].astype(np.float64).reshape(streams, streams)
+    soft = np.exp(raw - raw.max(axis=2, keepdims=True))
+    soft = soft / soft.sum(axis=2, keepdims=True) + 1e-6
+    soft = soft / (soft.sum(axis=1, keepdims=True) + 1e-6)
+    assert rc == 0 and np.allclose(once, soft, rtol=1e-5, atol=1e-7)
+    bad = base.copy()
+    bad[3] = np.nan
+    assert oracle.mhc_pre(res, mix, scale, bad, streams=streams, width=width, iterations=1, rms_epsilon=1e-6,
+                          mhc_epsilon=1e-6, post_multiplier=2.0)[0] == oracle.ERR_FORMAT
+
+
+def test_weighted_rms_norm_closed_form(oracle):
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal(300).astype(np.float32)
+    w = (1.0 + 0.1 * rng.standard_normal(300)).astype(np.float32)
+    rc, out = oracle.rms_norm(v, w, 1e-6)
+    want = v.astype(np.float64) / np.sqrt((v.astype(np.float64) ** 2).mean() + 1e-6) * w
+    assert rc == 0 and np.array_equal(out, want.astype(np.float32))
+    rc, ones = oracle.rms_norm(np.full(8, 3.0, np.float32), np.ones(8, np.float32), 1e-12)
+    assert rc == 0 and np.allclose(ones, 1.0, atol=1e-6)
+
+
+@pytest.mark.parametrize("name,streams,width,iterations", [("wide", 4, 64, 20), ("single", 1, 32, 1)])
+def test_ffn_ingress_matches_reference_fixture(oracle, golden, name, streams, width, iterations):
+    """Bit-for-bit against yvex_moe_ffn_prepare_cpu of the compiled reference (moe.c:446-495):
+    mixes through the CPU row dot, ingress, BF16 norm weights, weighted RMS norm, bf16 round."""
+    norm = (golden[f"ingress_{name}_norm_bf16"].astype(np.uint32) << 16).view(np.float32)
+    rc, normalized, post, comb = oracle.moe_ffn_prepare(
+        oracle.F32, golden[f"ingress_{name}_function"].view(np.uint8), golden[f"ingress_{name}_rows"],
+        golden[f"ingress_{name}_scale"], golden[f"ingress_{name}_base"], norm, streams=streams, width=width,
+        iterations=iterations, rms_epsilon=1e-6, mhc_epsilon=1e-6, post_multiplier=2.0)
+    assert rc == 0
+    assert np.array_equal(bits(normalized), golden[f"ingress_{name}_normalized_bits"])
+    assert np.array_equal(bits(post), golden[f"ingress_{name}_post_bits"])
+    assert np.array_equal(bits(comb).reshape(comb.shape[0], -1), golden[f"ingress_{name}_combination_bits"])
