@@ -166,6 +166,32 @@ int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows, uint64
                                 uint64_t hidden, const float *shared, float *routed,
                                 float *combined, int *status, yvex_hip_stream stream);
 
+/* Residual-stream envelope around the expert math (row_count rows of streams x width F32 values,
+ * streams <= 7 so that (streams + 2) * streams <= 64 mixing rows, width <= 16384).
+ *
+ * yvex_hip_mhc_ingress replaces yvex_residual_mhc_pre followed by yvex_attention_weighted_norm
+ * (src/backend/cuda/kernels.cu:1243-1387 and :867-910; launched from
+ * src/backend/cuda/moe.c:1210-1254) with the arithmetic of src/graph/numeric.c:630-826: the
+ * residual is rounded to bf16 as it is read (the rows themselves are left untouched), gates and
+ * the mixing matrix are formed in double precision from mixes[row, (streams + 2) * streams]
+ * (= function . row), scale[3] and base[(streams + 2) * streams], the collapsed row is
+ * bf16-rounded, normalised with norm[width] and published as bf16 in normalized[row, width];
+ * post[row, streams] and combination[row, streams, streams] are kept for the egress.
+ *
+ * yvex_hip_mhc_egress replaces yvex_residual_mhc_post (kernels.cu:1389-1428,
+ * numeric.c:828-877): output[row, target, lane] = bf16(post[target] * core[row, lane] +
+ * sum over source of combination[source, target] * bf16(rows[row, source, lane])), accumulated
+ * in double in source order. Non-finite values raise status 1 in both. */
+int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const float *scale,
+                         const float *base, const float *norm, uint64_t row_count,
+                         uint64_t streams, uint64_t width, uint64_t iterations,
+                         double rms_epsilon, double mhc_epsilon, double post_multiplier,
+                         float *normalized, float *post, float *combination, int *status,
+                         yvex_hip_stream stream);
+int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,
+                        const float *combination, uint64_t row_count, uint64_t streams,
+                        uint64_t width, float *output, int *status, yvex_hip_stream stream);
+
 /* Bandwidth probe (the reference publishes the same fact at backend start,
  * src/backend/cuda/backend.c:1550): streams `bytes` of device memory through 16-byte loads.
  * Time it with events; `sink` is a 4-byte device word that is practically never written. */

@@ -232,3 +232,88 @@ def test_greedy_selection_flags_non_finite(gpu, oracle):
     tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
     torch.cuda.synchronize()
     assert int(status.item()) == 1 and int(ties[0]) == 0 and int(ties[1]) == 0
+
+
+def envelope_inputs(oracle, tokens, streams, width, name):
+    g = oracle.Generator(42, f"envelope.{name}.{streams}.{width}")
+    mixing = (streams + 2) * streams
+    rows = g.normal(tokens * streams * width).reshape(tokens, streams * width)     # not bf16 values
+    rounded = ((rows.view(np.uint32) + 0x7fff + ((rows.view(np.uint32) >> 16) & 1)) & 0xffff0000).view(np.float32)
+    mixes = g.normal(tokens * mixing).reshape(tokens, mixing) * 3.0
+    scale = np.array([0.5, -0.25, 0.75], np.float32)
+    base = g.normal(mixing, 0.5)
+    norm = (1.0 + g.normal(width, 0.2)).astype(np.float32)
+    return rows, rounded, mixes, scale, base, norm
+
+
+@pytest.mark.parametrize("tokens,streams,width,iterations", [
+    (5, 4, 7168, 20), (3, 1, 512, 1), (2, 7, 200, 3), (33, 4, 256, 20), (1, 2, 16384, 2)])
+def test_envelope_ingress_matches_oracle(gpu, oracle, tokens, streams, width, iterations):
+    """Ingress + weighted RMS norm against numeric.c's order of operations. The kernel rounds the
+    residual to bf16 as the reference's device kernel does, so the oracle is fed the rounded
+    rows. Gates and the mixing matrix come from double-precision exp, whose last bit may differ
+    between the two maths libraries: 1e-6 as the reference's own envelope test allows
+    (tests/unit/deepseek_attention.c:2326-2337); the published row is bf16, so a value on a
+    rounding boundary may move by one bf16 step."""
+    from yvex_amd import kernels as K
+    rows, rounded, mixes, scale, base, norm = envelope_inputs(oracle, tokens, streams, width, "in")
+    kw = dict(streams=streams, width=width, iterations=iterations, rms_epsilon=1e-6, mhc_epsilon=1e-6,
+              post_multiplier=2.0)
+    status = K.new_status(gpu)
+    normalized, post, comb = K.mhc_ingress(dev(rows, gpu), dev(mixes, gpu), dev(scale, gpu), dev(base, gpu),
+                                           dev(norm, gpu), status=status, **kw)
+    status_ok(status)
+    rc, collapsed, want_post, want_comb = oracle.mhc_pre(rounded, mixes, scale, base, **kw)
+    assert rc == 0
+    want = np.zeros_like(collapsed)
+    for t in range(tokens):
+        rc, want[t] = oracle.rms_norm(collapsed[t], norm, 1e-6)
+        assert rc == 0
+    want = ((want.view(np.uint32) + 0x7fff + ((want.view(np.uint32) >> 16) & 1)) & 0xffff0000).view(np.float32)
+    assert_close(post.cpu().numpy(), want_post, rel=1e-6, abs_=1e-6)
+    assert_close(comb.cpu().numpy(), want_comb, rel=1e-6, abs_=1e-6)
+    got = normalized.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32) & 0xffff, np.zeros_like(got.view(np.uint32)))
+    differ = got != want
+    assert differ.mean() < 1e-3
+    assert np.all(np.abs(got[differ] - want[differ]) <= 2.0 ** -7 * np.abs(want[differ]))
+
+
+@pytest.mark.parametrize("tokens,streams,width", [(5, 4, 7168), (3, 1, 512), (2, 7, 200), (64, 4, 300)])
+def test_envelope_egress_bit_exact(gpu, oracle, tokens, streams, width):
+    """Egress is double-precision multiply-adds in a fixed order and one bf16 rounding: bit-exact."""
+    from yvex_amd import kernels as K
+    rows, rounded, _, _, _, _ = envelope_inputs(oracle, tokens, streams, width, "out")
+    g = oracle.Generator(7, f"envelope.core.{streams}.{width}")
+    core = g.normal(tokens * width).reshape(tokens, width)
+    post = np.abs(g.normal(tokens * streams)).reshape(tokens, streams).astype(np.float32)
+    comb = np.abs(g.normal(tokens * streams * streams)).reshape(tokens, streams, streams).astype(np.float32)
+    status = K.new_status(gpu)
+    got = K.mhc_egress(dev(core, gpu), dev(rows, gpu), dev(post, gpu), dev(comb, gpu), streams=streams,
+                       width=width, status=status).cpu().numpy()
+    status_ok(status)
+    rc, want = oracle.mhc_post(core, rounded, post, comb, streams=streams, width=width)
+    assert rc == 0 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_envelope_flags_non_finite(gpu, oracle):
+    from yvex_amd import kernels as K
+    rows, _, mixes, scale, base, norm = envelope_inputs(oracle, 3, 2, 256, "bad")
+    kw = dict(streams=2, width=256, iterations=2, rms_epsilon=1e-6, mhc_epsilon=1e-6, post_multiplier=2.0)
+    for poison in ("rows", "base", "norm"):
+        r, b, n = rows.copy(), base.copy(), norm.copy()
+        {"rows": r, "base": b, "norm": n}[poison].flat[5] = np.inf
+        status = K.new_status(gpu)
+        K.mhc_ingress(dev(r, gpu), dev(mixes, gpu), dev(scale, gpu), dev(b, gpu), dev(n, gpu), status=status, **kw)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 1, poison
+    core = np.ones((3, 256), np.float32)
+    core[1, 7] = np.nan
+    status = K.new_status(gpu)
+    K.mhc_egress(dev(core, gpu), dev(rows, gpu), dev(np.ones((3, 2), np.float32), gpu),
+                 dev(np.ones((3, 2, 2), np.float32), gpu), streams=2, width=256, status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    with pytest.raises(K.KernelError):     # eight streams would need 80 mixing rows
+        K.mhc_egress(dev(core, gpu), dev(rows, gpu), dev(np.ones((3, 8), np.float32), gpu),
+                     dev(np.ones((3, 8, 8), np.float32), gpu), streams=8, width=32, status=status)

@@ -132,6 +132,30 @@ def argmax_f32(values, status, out=None, scratch=None):
     return tokens, best, ties
 
 
+def mhc_ingress(rows, mixes, scale, base, norm, *, streams, width, iterations, rms_epsilon,
+                mhc_epsilon, post_multiplier, status):
+    """Residual-stream ingress + weighted RMS norm: (normalized [n, width], post [n, streams],
+    combination [n, streams, streams])."""
+    count = rows.shape[0]
+    normalized = torch.empty((count, width), dtype=torch.float32, device=rows.device)
+    post = torch.empty((count, streams), dtype=torch.float32, device=rows.device)
+    combination = torch.empty((count, streams, streams), dtype=torch.float32, device=rows.device)
+    _call("yvex_hip_mhc_ingress", _ptr(rows), _ptr(mixes), _ptr(scale), _ptr(base), _ptr(norm),
+          C.c_uint64(count), C.c_uint64(streams), C.c_uint64(width), C.c_uint64(iterations),
+          C.c_double(rms_epsilon), C.c_double(mhc_epsilon), C.c_double(post_multiplier),
+          _ptr(normalized), _ptr(post), _ptr(combination), _ptr(status), _stream())
+    return normalized, post, combination
+
+
+def mhc_egress(core, rows, post, combination, *, streams, width, status):
+    """Residual-stream egress: [n, streams * width] bf16-valued F32 rows."""
+    count = core.shape[0]
+    out = torch.empty((count, streams * width), dtype=torch.float32, device=core.device)
+    _call("yvex_hip_mhc_egress", _ptr(core), _ptr(rows), _ptr(post), _ptr(combination),
+          C.c_uint64(count), C.c_uint64(streams), C.c_uint64(width), _ptr(out), _ptr(status), _stream())
+    return out
+
+
 def moe_route_rows(logits, bias, topk, scoring, normalize, scaling, status):
     rows, experts = logits.shape
     selected = torch.empty((rows, topk), dtype=torch.int64, device=logits.device)
