@@ -159,7 +159,7 @@ def main():
         scale = gen.normal(3, 0.7)
         base = gen.normal(mixing, 0.5)
         norm_bits = ((1.0 + gen.normal(width, 0.2)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-        rows = np.round(gen.normal(tokens * expanded) * 64.0) / 64.0     # exact in bf16
+        rows = np.round(gen.normal(tokens * expanded) * 64.0) / 64.0     # multiples of 1/64
         rows = rows.astype(np.float32).reshape(tokens, expanded)
         plan = abi.LayerPlan()
         plan.hidden_width, plan.residual_streams, plan.expanded_width = width, streams, expanded

@@ -196,8 +196,11 @@ class MoeCase:
 
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
-                 shared=True, family=abi.FAMILY_GFX950, seed=42):
+                 shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20):
         self.b, self.oracle = b, oracle
+        self.streams, self.iterations = streams, iterations
+        expanded = hidden * max(streams, 1)
+        mixing = (streams + 2) * streams
         qt = getattr(oracle, qtype)
         self.qt, self.rows, self.hidden, self.experts, self.topk = qt, rows, hidden, experts, topk
         self.intermediate, self.scoring = intermediate, scoring
@@ -212,6 +215,12 @@ class MoeCase:
             "sup": g.weights(qt, intermediate, hidden),
             "sdown": g.weights(qt, hidden, intermediate),
         }
+        if streams:     # residual-stream envelope: mixing function, scale, base (F32) and BF16 norm weights
+            parts["function"] = g.normal(mixing * expanded, 0.05).view(np.uint8)
+            parts["scale"] = g.normal(3, 0.7).view(np.uint8)
+            parts["base"] = g.normal(mixing, 0.5).view(np.uint8)
+            parts["norm"] = ((1.0 + g.normal(hidden, 0.2)).astype(np.float32).view(np.uint32) >> 16) \
+                .astype(np.uint16).view(np.uint8)
         self.parts = parts
         offsets, cursor = {}, 0
         for name, blob in parts.items():
@@ -221,12 +230,18 @@ class MoeCase:
         for name, blob in parts.items():
             arena[offsets[name]:offsets[name] + blob.nbytes] = blob
         _, host = b.resident(arena)
-        self.x = g.normal(rows * hidden).reshape(rows, hidden)
+        self.x = g.normal(rows * expanded).reshape(rows, expanded)
+        if streams:
+            bits = self.x.view(np.uint32)       # bf16 values, as the CPU path expects of its input
+            self.x = ((bits + 0x7fff + ((bits >> 16) & 1)) & 0xffff0000).view(np.float32)
         self.plan = abi.LayerPlan()
         p = self.plan
         p.schema_version, p.router_class, p.scoring = 1, abi.ROUTER_LEARNED, scoring
-        p.hidden_width = p.expanded_width = hidden
-        p.residual_streams = 1
+        p.hidden_width, p.expanded_width = hidden, expanded
+        p.residual_streams = max(streams, 1)
+        if streams:
+            p.mhc_mixing_rows, p.mhc_sinkhorn_iterations = mixing, iterations
+            p.rms_epsilon, p.mhc_epsilon, p.mhc_post_multiplier = 1e-6, 1e-6, 2.0
         p.routed_experts, p.shared_experts, p.experts_per_token = experts, int(shared), topk
         p.expert_intermediate_width = p.shared_intermediate_width = intermediate
         p.routed_scaling_factor, p.activation_limit = 1.5, 10.0
@@ -250,14 +265,19 @@ class MoeCase:
         view(abi.W_SHARED_GATE, "sgate", qt, hidden, intermediate, rb_h)
         view(abi.W_SHARED_UP, "sup", qt, hidden, intermediate, rb_h)
         view(abi.W_SHARED_DOWN, "sdown", qt, intermediate, hidden, rb_i)
+        if streams:
+            view(abi.W_MHC_FUNCTION, "function", 0, expanded, mixing, expanded * 4, abi.ACT_DEVICE_F32)
+            view(abi.W_MHC_SCALE, "scale", 0, 3, 1, 12, abi.ACT_DEVICE_F32)
+            view(abi.W_MHC_BASE, "base", 0, mixing, 1, mixing * 4, abi.ACT_DEVICE_F32)
+            view(abi.W_FFN_NORM, "norm", 30, hidden, 1, hidden * 2, abi.ACT_DEVICE_F32)
         self.ops = b.lib.yvex_backend_moe_operations_get(b.handle).contents
         need, err = abi.ULL(), abi.Error()
         assert self.ops.workspace_required(C.byref(self.plan), rows, C.byref(need), C.byref(err)) == 0
         self.workspace_bytes = need.value
-        self.rows_in, self.rows_out = b.f32(self.x), b.empty_f32(rows * hidden)
+        self.rows_in, self.rows_out = b.f32(self.x), b.empty_f32(rows * expanded)
         self.batch = abi.RowBatch()
         bt = self.batch
-        bt.schema_version, bt.row_count, bt.row_width, bt.row_stride = 1, rows, hidden, hidden
+        bt.schema_version, bt.row_count, bt.row_width, bt.row_stride = 1, rows, expanded, expanded
         bt.device_rows, bt.device_outputs = self.rows_in, self.rows_out
         bt.provenance, bt.execution_class = abi.BATCH_MULTI_SESSION, 1
         self.sel = np.zeros(rows * topk, np.uint64)
@@ -267,6 +287,11 @@ class MoeCase:
         self.out.combined_rows, self.out.combined_capacity = self.combined.ctypes.data, rows * hidden
         self.out.selected_experts, self.out.selected_weights = self.sel.ctypes.data, self.wts.ctypes.data
         self.out.selection_capacity = rows * topk
+        if streams:
+            self.post = np.zeros((rows, streams), np.float32)
+            self.comb = np.zeros((rows, streams, streams), np.float32)
+            self.out.post_rows, self.out.post_capacity = self.post.ctypes.data, self.post.size
+            self.out.combination_rows, self.out.combination_capacity = self.comb.ctypes.data, self.comb.size
         self.result, self.err = abi.RowBatchResult(), abi.Error()
 
     def execute(self):
@@ -275,15 +300,30 @@ class MoeCase:
 
     def oracle_layer(self, act_q8):
         o, p = self.oracle, self.parts
+        x, ingress = self.x, None
+        if self.streams:      # src/graph/moe.c:446-495 in front, numeric.c:828-877 behind
+            norm = (p["norm"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+            rc, x, post, comb = o.moe_ffn_prepare(
+                o.F32, p["function"], self.x, p["scale"].view(np.float32), p["base"].view(np.float32), norm,
+                streams=self.streams, width=self.hidden, iterations=self.iterations, rms_epsilon=1e-6,
+                mhc_epsilon=1e-6, post_multiplier=2.0)
+            assert rc == 0
+            ingress = (x, post, comb)
         router = p["router"].view(np.float32).reshape(self.experts, self.hidden)
-        logits = o.matvec(o.F32, p["router"], self.experts, self.hidden, self.x)
-        assert np.allclose(logits, self.x @ router.T, rtol=1e-4, atol=1e-5)
+        logits = o.matvec(o.F32, p["router"], self.experts, self.hidden, x)
+        assert np.allclose(logits, x @ router.T, rtol=1e-4, atol=1e-5)
         bias = p["bias"].view(np.float32) if self.plan.requires_correction_bias else None
         shared = (p["sgate"], p["sup"], p["sdown"]) if self.plan.shared_experts else None
-        return o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
+        want = o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
                            topk=self.topk, qtypes=(self.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
-                           shared=shared, inputs=self.x, logits=logits, bias=bias, scoring=self.scoring,
+                           shared=shared, inputs=x, logits=logits, bias=bias, scoring=self.scoring,
                            normalize=True, scaling=1.5, act_q8=act_q8, threads=8)
+        if ingress:
+            want["normalized"], want["post"], want["combination"] = ingress
+            rc, want["envelope"] = o.mhc_post(want["combined"], self.x, ingress[1], ingress[2],
+                                              streams=self.streams, width=self.hidden)
+            assert rc == 0
+        return want
 
 
 @pytest.mark.parametrize("qtype,act,scoring,shared", [
@@ -314,6 +354,46 @@ def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, sh
     assert res.active_weight_per_unique_expert_bytes == per_expert
     assert res.encoded_bytes_read == res.active_weight_base_bytes + per_expert * uniq
     assert res.kernel_launches >= 8 and res.memory.complete == 1
+
+
+@pytest.mark.parametrize("qtype,streams,rows,hidden,iterations", [
+    ("IQ2_XXS", 4, 5, 512, 20), ("IQ2_XXS", 1, 3, 512, 1), ("Q8_0", 2, 7, 256, 3)])
+def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, rows, hidden, iterations):
+    """The layer as the reference's row-batch operation runs it (src/backend/cuda/moe.c:1210-1254,
+    1533-1541): ingress over the expanded rows, weighted norm, routing and experts on the
+    normalised row, egress back onto the streams. The mixes come from the F32-accumulating
+    projection kernel while the CPU accumulates in double (1e-3 rel / 1e-5 abs on the mixes), so
+    gates and the mixing matrix are held to 1e-4 here; given identical mixes the kernel test holds
+    them to 1e-6. The normalised row is bf16: a value that sits on a rounding
+    boundary may land one step away from the CPU's, which moves a router logit by about 1e-4 of
+    its size, so route weights are held to 1e-4 here and the selection must still agree."""
+    case = MoeCase(backend, oracle, qtype=qtype, hidden=hidden, rows=rows, streams=streams,
+                   iterations=iterations)
+    backend.workspace(case.workspace_bytes)
+    assert case.execute() == 0, case.err.message
+    want = case.oracle_layer(act_q8=True)
+    assert np.array_equal(case.sel.reshape(rows, case.topk), want["selected"])
+    assert np.max(np.abs(case.wts.reshape(rows, case.topk) - want["weights"])) <= 1e-4
+    assert np.max(np.abs(case.post - want["post"])) <= 1e-4
+    assert np.max(np.abs(case.comb - want["combination"])) <= 1e-4
+
+    def close_or_one_step(got, ref, steps):
+        err = np.abs(got.astype(np.float64) - ref)
+        outside = err > 1e-5 + 1e-3 * np.abs(ref)
+        assert outside.mean() < 2e-2
+        assert np.all(err[outside] <= steps * 2.0 ** -7 * np.abs(ref[outside]) + 1e-4)
+
+    close_or_one_step(case.combined, want["combined"], 2)
+    expanded = streams * hidden
+    got = backend.read_f32(case.rows_out, rows * expanded).reshape(rows, expanded)
+    assert case.rows_out.contents.is_written == 1
+    assert np.array_equal(got.view(np.uint32) & 0xffff, np.zeros_like(got.view(np.uint32)))
+    # the egress applied to the device's own combined rows is exact
+    rc, replay = oracle.mhc_post(case.combined, case.x, case.post, case.comb, streams=streams, width=hidden)
+    assert rc == 0 and np.array_equal(got.view(np.uint32), replay.view(np.uint32))
+    scale = np.abs(want["envelope"]) + np.abs(want["combined"]).max()
+    assert np.all(np.abs(got - want["envelope"]) <= 2.0 ** -6 * scale)
+    assert case.result.completed == 1 and case.result.kernel_launches >= 14
 
 
 def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle):
@@ -372,10 +452,13 @@ def test_execute_rows_refusals(backend, oracle):
     assert case.execute() == abi.UNSUPPORTED
     for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
         case.job.weights[slot].kernel_family = abi.FAMILY_GFX950
-    # residual mixing envelope and the hash router are outside this backend
+    # mixing rows that disagree with the stream count; expanded rows without mixing rows; hash router
     case.plan.mhc_mixing_rows = 24
-    assert case.execute() == abi.UNSUPPORTED
+    assert case.execute() == abi.BOUNDS
     case.plan.mhc_mixing_rows = 0
+    case.plan.expanded_width = 2 * case.hidden
+    assert case.execute() in (abi.UNSUPPORTED, abi.INVALID_ARG)
+    case.plan.expanded_width = case.hidden
     case.plan.router_class = abi.ROUTER_HASH
     assert case.execute() == abi.UNSUPPORTED
     case.plan.router_class = abi.ROUTER_LEARNED

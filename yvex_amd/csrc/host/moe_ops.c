@@ -29,19 +29,43 @@ typedef struct {
     unsigned long long order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts;
     unsigned long long intermediate, intermediate_q8, pair_outputs;
     unsigned long long shared_intermediate, shared_intermediate_q8, shared_outputs, routed;
+    /* residual-stream envelope (layers whose plan names mixing rows) */
+    unsigned long long mixes, scale, base, norm, normalized, post, combination, combined;
     unsigned long long total;
 } moe_ranges;
 
+/* Layers that carry residual streams run the reference's ingress and egress around the expert
+ * math (src/backend/cuda/moe.c:1210-1254,1533-1541); a plan without mixing rows hands this
+ * backend rows that are already normalised. Geometry as src/graph/numeric.c:668-689 asks. */
+static int moe_envelope(const yvex_moe_layer_plan *layer)
+{
+    return layer->mhc_mixing_rows != 0ull;
+}
+
+static int moe_envelope_geometry(const yvex_moe_layer_plan *layer)
+{
+    unsigned long long streams = layer->residual_streams;
+    return streams >= 1ull && streams <= 7ull && layer->hidden_width <= 16384ull &&
+           layer->expanded_width == streams * layer->hidden_width &&
+           layer->mhc_mixing_rows == (streams + 2ull) * streams &&
+           layer->mhc_sinkhorn_iterations > 0ull && layer->mhc_sinkhorn_iterations <= 0xffffffffull &&
+           isfinite(layer->rms_epsilon) && layer->rms_epsilon > 0.0 &&
+           isfinite(layer->mhc_epsilon) && layer->mhc_epsilon > 0.0 &&
+           isfinite(layer->mhc_post_multiplier) && layer->mhc_post_multiplier > 0.0;
+}
+
 static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows, moe_ranges *r)
 {
-    unsigned long long cursor = 0ull, pairs, hidden, routed_i, shared_i, experts;
+    unsigned long long cursor = 0ull, pairs, hidden, routed_i, shared_i, experts, streams;
     if (!layer || !rows || rows > YVEX_ROCM_MOE_MAX_ROWS || !layer->hidden_width ||
         !layer->routed_experts || layer->routed_experts > 256ull || !layer->experts_per_token ||
         layer->experts_per_token > YVEX_MOE_MAX_SELECTED ||
         layer->experts_per_token > layer->routed_experts || !layer->expert_intermediate_width ||
         layer->hidden_width > (1ull << 20) || layer->expert_intermediate_width > (1ull << 20) ||
-        layer->shared_intermediate_width > (1ull << 20) || layer->shared_experts > 1ull)
+        layer->shared_intermediate_width > (1ull << 20) || layer->shared_experts > 1ull ||
+        (moe_envelope(layer) && !moe_envelope_geometry(layer)))
         return 0;
+    streams = moe_envelope(layer) ? layer->residual_streams : 0ull;
     pairs = rows * layer->experts_per_token;
     hidden = layer->hidden_width;
     routed_i = layer->expert_intermediate_width;
@@ -66,6 +90,16 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
     TAKE(shared_intermediate_q8, rows * ((shared_i + 255ull) / 256ull) * 292ull);
     TAKE(shared_outputs, rows * hidden * sizeof(float));
     TAKE(routed, rows * hidden * sizeof(float));
+    if (streams) {
+        TAKE(mixes, rows * layer->mhc_mixing_rows * sizeof(float));
+        TAKE(scale, 3ull * sizeof(float));
+        TAKE(base, layer->mhc_mixing_rows * sizeof(float));
+        TAKE(norm, hidden * sizeof(float));
+        TAKE(normalized, rows * hidden * sizeof(float));
+        TAKE(post, rows * streams * sizeof(float));
+        TAKE(combination, rows * streams * streams * sizeof(float));
+        TAKE(combined, rows * hidden * sizeof(float));
+    }
 #undef TAKE
     r->total = cursor + ALIGN;   /* slack for aligning the workspace base itself */
     return 1;
@@ -221,8 +255,11 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     moe_ranges ranges;
     unsigned long long base, pairs, hidden, experts, topk, row_count, launches = 0ull;
     unsigned long long router_address = 0ull, bias_address = 0ull, addresses[6] = {0};
+    unsigned long long envelope_addresses[4] = {0}, streams = 0ull, expanded;
     unsigned long long d2h = 0ull, started, counts[4] = {0};
-    int unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
+    const void *activations;
+    void *combined_target;
+    int envelope, unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
     if (result) memset(result, 0, sizeof(*result));
@@ -236,7 +273,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         backend->kind != YVEX_BACKEND_KIND_ROCM ||
         ((job->execution_batch == NULL) != (job->worklist_policy == NULL)) ||
         rows->schema_version != YVEX_MOE_ROW_BATCH_SCHEMA_V1 || !rows->row_count ||
-        rows->row_count > YVEX_ROCM_MOE_MAX_ROWS || rows->row_width != layer->hidden_width ||
+        rows->row_count > YVEX_ROCM_MOE_MAX_ROWS || rows->row_width != layer->expanded_width ||
         rows->row_stride != rows->row_width ||
         !yvex_rocm_tensor_owner_is(backend, rows->device_rows) ||
         !yvex_rocm_tensor_owner_is(backend, rows->device_outputs) ||
@@ -246,11 +283,17 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         rows->device_outputs->bytes < rows->row_count * rows->row_width * sizeof(float))
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
                                 "width-N MoE owners, geometry or admitted width are invalid");
-    if (layer->expanded_width != layer->hidden_width || layer->mhc_mixing_rows ||
+    envelope = moe_envelope(layer);
+    if ((!envelope && layer->expanded_width != layer->hidden_width) ||
         layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE ||
         (layer->scoring != YVEX_MOE_SCORING_SQRT_SOFTPLUS && layer->scoring != YVEX_MOE_SCORING_SIGMOID))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
-                                "residual mixing, hash routing and other scoring policies are outside this backend");
+                                "hash routing, other scoring policies and expanded rows without mixing rows are outside this backend");
+    if (envelope && !moe_envelope_geometry(layer))
+        return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows",
+                                "residual-stream geometry is invalid");
+    streams = envelope ? layer->residual_streams : 0ull;
+    expanded = layer->expanded_width;
     row_count = rows->row_count;
     hidden = layer->hidden_width;
     experts = layer->routed_experts;
@@ -263,7 +306,10 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows", "selection capacity is too small");
     if ((output->combined_rows && output->combined_capacity < row_count * hidden) ||
         (output->routed_rows && output->routed_capacity < row_count * hidden) ||
-        (output->shared_rows && output->shared_capacity < row_count * hidden))
+        (output->shared_rows && output->shared_capacity < row_count * hidden) ||
+        (envelope && output->post_rows && output->post_capacity < row_count * streams) ||
+        (envelope && output->combination_rows &&
+         output->combination_capacity < row_count * streams * streams))
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows", "host output capacity is too small");
     if (job->cancel_requested && job->cancel_requested(job->cancel_context))
         return yvex_rocm_refuse(err, YVEX_ERR_CANCELLED, "rocm.moe.rows",
@@ -302,6 +348,25 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     if (rc == YVEX_OK && has_shared)
         rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], layer->shared_intermediate_width,
                           hidden, &addresses[5], err);
+    if (rc == YVEX_OK && envelope) {
+        /* ingress coefficients: the mixing function is a matrix over the expanded row, the rest
+         * are flat rows of F32, BF16 or I32 values (src/graph/moe.c:405-428) */
+        static const int flat_slots[3] = {YVEX_MOE_WEIGHT_MHC_SCALE, YVEX_MOE_WEIGHT_MHC_BASE,
+                                          YVEX_MOE_WEIGHT_FFN_NORM};
+        const unsigned long long flat_widths[3] = {3ull, layer->mhc_mixing_rows, hidden};
+        int k;
+        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_MHC_FUNCTION], expanded,
+                          layer->mhc_mixing_rows, &envelope_addresses[0], err);
+        for (k = 0; rc == YVEX_OK && k < 3; ++k) {
+            unsigned int q = views[flat_slots[k]].qtype;
+            if (q != 0u && q != 30u && q != 26u)
+                rc = yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.rows",
+                                      "MoE FFN coefficients cannot be decoded");
+            else
+                rc = view_resolve(backend, &views[flat_slots[k]], flat_widths[k], 1ull,
+                                  &envelope_addresses[1 + k], err);
+        }
+    }
     if (rc != YVEX_OK) return rc;
     if (!(layer->activation_limit > 0.0) || !isfinite(layer->activation_limit) ||
         !isfinite(layer->routed_scaling_factor))
@@ -347,10 +412,44 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     LAUNCH(yvex_hip_fill_u32(status, 0u, 1u, stream), "rocm.moe.rows.status");
     if (has_shared && !merged)
         LAUNCH(yvex_hip_fill_u32(AT(shared_outputs), 0u, row_count * hidden, stream), "rocm.moe.rows.zero");
+    activations = rows->device_rows->data;
+    combined_target = rows->device_outputs->data;
+    if (envelope) {
+        /* src/backend/cuda/moe.c:1210-1254: mixes = function . expanded row, coefficients decoded
+         * to F32, then ingress and the weighted norm in one kernel */
+        const yvex_moe_weight_view *function = &views[YVEX_MOE_WEIGHT_MHC_FUNCTION];
+        static const int flat_slots[3] = {YVEX_MOE_WEIGHT_MHC_SCALE, YVEX_MOE_WEIGHT_MHC_BASE,
+                                          YVEX_MOE_WEIGHT_FFN_NORM};
+        void *flat_targets[3];
+        int k;
+        flat_targets[0] = AT(scale);
+        flat_targets[1] = AT(base);
+        flat_targets[2] = AT(norm);
+        LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)envelope_addresses[0], function->qtype,
+                               layer->mhc_mixing_rows, expanded, function->row_bytes,
+                               rows->device_rows->data, 0, row_count, expanded, NULL,
+                               (float *)AT(mixes), layer->mhc_mixing_rows, 0, (int *)status, stream),
+               "rocm.moe.rows.mhc-function");
+        for (k = 0; k < 3; ++k)
+            LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)envelope_addresses[1 + k],
+                                   views[flat_slots[k]].qtype, 1ull, views[flat_slots[k]].row_width,
+                                   views[flat_slots[k]].row_bytes, NULL, 1ull, (float *)flat_targets[k],
+                                   (int *)status, stream), "rocm.moe.rows.mhc-coefficients");
+        LAUNCH(yvex_hip_mhc_ingress((const float *)rows->device_rows->data, (const float *)AT(mixes),
+                                    (const float *)AT(scale), (const float *)AT(base),
+                                    (const float *)AT(norm), row_count, streams, hidden,
+                                    layer->mhc_sinkhorn_iterations, layer->rms_epsilon,
+                                    layer->mhc_epsilon, layer->mhc_post_multiplier,
+                                    (float *)AT(normalized), (float *)AT(post),
+                                    (float *)AT(combination), (int *)status, stream),
+               "rocm.moe.rows.mhc-ingress");
+        activations = AT(normalized);
+        combined_target = AT(combined);
+    }
     /* router: logits = router . row (F32 activations, as src/backend/cuda/moe.c:1259-1284) */
     LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)router_address, views[YVEX_MOE_WEIGHT_ROUTER].qtype,
                            experts, hidden, views[YVEX_MOE_WEIGHT_ROUTER].row_bytes,
-                           rows->device_rows->data, 0, row_count, hidden, NULL, (float *)AT(logits),
+                           activations, 0, row_count, hidden, NULL, (float *)AT(logits),
                            experts, 0, (int *)status, stream), "rocm.moe.rows.router");
     if (layer->requires_correction_bias)
         LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)bias_address, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype,
@@ -368,7 +467,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                    (uint64_t *)AT(sweep_offsets), (uint64_t *)AT(counts), (int *)status,
                                    stream), "rocm.moe.rows.worklist");
     if (routed_q8 || (has_shared && shared_q8))
-        LAUNCH(yvex_hip_q8k_quantize((const float *)rows->device_rows->data, row_count, hidden, hidden,
+        LAUNCH(yvex_hip_q8k_quantize((const float *)activations, row_count, hidden, hidden,
                                      (uint8_t *)AT(input_q8), (int *)status, stream), "rocm.moe.rows.q8");
     if (row_batch)
         LAUNCH(yvex_hip_moe_up_rows(&routed, AT(input_q8), (const float *)AT(weights),
@@ -379,7 +478,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                     (float *)AT(intermediate), (int *)status, stream),
                "rocm.moe.rows.up-matrix");
     else
-    LAUNCH(yvex_hip_moe_up(&routed, routed_q8 ? AT(input_q8) : (void *)rows->device_rows->data, routed_q8,
+    LAUNCH(yvex_hip_moe_up(&routed, routed_q8 ? AT(input_q8) : (void *)(uintptr_t)activations, routed_q8,
                            (const float *)AT(weights), (const uint64_t *)AT(order),
                            (const uint64_t *)AT(expert_ids), (const uint64_t *)AT(bucket_offsets),
                            (const uint64_t *)AT(bucket_populations), (const uint64_t *)AT(sweep_offsets),
@@ -392,7 +491,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                     1ull, 1ull, layer->activation_limit, (float *)AT(shared_intermediate),
                                     (int *)status, stream), "rocm.moe.rows.shared-up-matrix");
     else if (has_shared && !merged)
-        LAUNCH(yvex_hip_moe_up(&shared, shared_q8 ? AT(input_q8) : (void *)rows->device_rows->data,
+        LAUNCH(yvex_hip_moe_up(&shared, shared_q8 ? AT(input_q8) : (void *)(uintptr_t)activations,
                                shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull, 1ull,
                                layer->activation_limit, (float *)AT(shared_intermediate), NULL, 0ull, NULL,
                                (int *)status, stream), "rocm.moe.rows.shared-up");
@@ -434,8 +533,13 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         LAUNCH(yvex_hip_fill_u32(AT(shared_outputs), 0u, row_count * hidden, stream), "rocm.moe.rows.zero");
     LAUNCH(yvex_hip_moe_reduce_combine((const float *)AT(pair_outputs), row_count, topk, hidden,
                                        (const float *)AT(shared_outputs), (float *)AT(routed),
-                                       (float *)rows->device_outputs->data, (int *)status, stream),
+                                       (float *)combined_target, (int *)status, stream),
            "rocm.moe.rows.combine");
+    if (envelope)
+        LAUNCH(yvex_hip_mhc_egress((const float *)AT(combined), (const float *)rows->device_rows->data,
+                                   (const float *)AT(post), (const float *)AT(combination), row_count,
+                                   streams, hidden, (float *)rows->device_outputs->data, (int *)status,
+                                   stream), "rocm.moe.rows.mhc-egress");
     if (rc != YVEX_OK) return rc;
 
     defer = job->device_completion && job->device_completion->defer;
@@ -452,7 +556,11 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                       views[YVEX_MOE_WEIGHT_SHARED_DOWN].encoded_bytes : 0ull);
     result->active_weight_per_unique_expert_bytes =
         routed.gate_expert_bytes + routed.up_expert_bytes + routed.down_expert_bytes;
-    result->memory.activation_bytes = 2ull * row_count * hidden * sizeof(float);
+    if (envelope)
+        result->active_weight_base_bytes += views[YVEX_MOE_WEIGHT_MHC_FUNCTION].encoded_bytes +
+            views[YVEX_MOE_WEIGHT_MHC_SCALE].encoded_bytes + views[YVEX_MOE_WEIGHT_MHC_BASE].encoded_bytes +
+            views[YVEX_MOE_WEIGHT_FFN_NORM].encoded_bytes;
+    result->memory.activation_bytes = 2ull * row_count * expanded * sizeof(float);
     result->memory.temporary_bytes = ranges.total;
     result->memory.measured_operations = 1ull;
     if (defer) {
@@ -492,8 +600,12 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     DOWNLOAD(output->selected_weights, weights, pairs * sizeof(float));
     DOWNLOAD(output->routed_rows, routed, row_count * hidden * sizeof(float));
     DOWNLOAD(output->shared_rows, shared_outputs, row_count * hidden * sizeof(float));
+    if (envelope) {
+        DOWNLOAD(output->post_rows, post, row_count * streams * sizeof(float));
+        DOWNLOAD(output->combination_rows, combination, row_count * streams * streams * sizeof(float));
+    }
     if (rc == YVEX_OK && output->combined_rows) {
-        if (yvex_hip_memcpy_d2h(output->combined_rows, rows->device_outputs->data,
+        if (yvex_hip_memcpy_d2h(output->combined_rows, combined_target,
                                 row_count * hidden * sizeof(float), stream) != 0)
             rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.download", yvex_hip_last_error());
         else { d2h += row_count * hidden * sizeof(float); result->download_count++; }
