@@ -165,6 +165,34 @@ def dense_leg(torch, K, dev, repeats: int):
     out["greedy_selection_1x129280"] = {"us": round(ms * 1e3, 2),
                                         "graph_us": round(graph_us, 2) if graph_us else None,
                                         "status": int(status.item())}
+    # residual-stream ingress and egress around a layer: 4 streams of 7168, decode and prefill rows
+    streams, width, mixing = 4, 7168, 24
+    for rows in (32, 2048):
+        x = torch.randn((rows, streams * width), device=dev, generator=gen)
+        mixes = torch.randn((rows, mixing), device=dev, generator=gen)
+        scale = torch.tensor([0.5, -0.25, 0.75], device=dev)
+        base = torch.randn(mixing, device=dev, generator=gen) * 0.5
+        norm = 1.0 + 0.2 * torch.randn(width, device=dev, generator=gen)
+        kw = dict(streams=streams, width=width, iterations=20, rms_epsilon=1e-6, mhc_epsilon=1e-6,
+                  post_multiplier=2.0)
+        status = K.new_status(dev)
+        held = K.mhc_ingress(x, mixes, scale, base, norm, status=status, **kw)
+        ms, graph_us = eager_and_graph(
+            lambda: K.mhc_ingress(x, mixes, scale, base, norm, status=status, out=held, **kw), 8)
+        best_ms = min(ms, graph_us * 1e-3) if graph_us else ms
+        moved = rows * (streams * width + width) * 4
+        out[f"stream_ingress_{rows}x4x7168"] = {
+            "us": round(ms * 1e3, 2), "graph_us": round(graph_us, 2) if graph_us else None,
+            "GB_per_s": round(moved / (best_ms * 1e-3) / 1e9, 1), "bytes": moved, "status": int(status.item())}
+        spread = K.mhc_egress(held[0], x, held[1], held[2], streams=streams, width=width, status=status)
+        ms, graph_us = eager_and_graph(
+            lambda: K.mhc_egress(held[0], x, held[1], held[2], streams=streams, width=width, status=status,
+                                 out=spread), 8)
+        best_ms = min(ms, graph_us * 1e-3) if graph_us else ms
+        moved = rows * (2 * streams * width + width) * 4
+        out[f"stream_egress_{rows}x4x7168"] = {
+            "us": round(ms * 1e3, 2), "graph_us": round(graph_us, 2) if graph_us else None,
+            "GB_per_s": round(moved / (best_ms * 1e-3) / 1e9, 1), "bytes": moved, "status": int(status.item())}
     return out
 
 

@@ -247,7 +247,8 @@ def envelope_inputs(oracle, tokens, streams, width, name):
 
 
 @pytest.mark.parametrize("tokens,streams,width,iterations", [
-    (5, 4, 7168, 20), (3, 1, 512, 1), (2, 7, 200, 3), (33, 4, 256, 20), (1, 2, 16384, 2)])
+    (5, 4, 7168, 20), (3, 1, 512, 1), (2, 7, 200, 3), (33, 4, 256, 20), (1, 2, 16384, 2), (4, 3, 203, 5),
+    (2, 4, 1028, 4)])
 def test_envelope_ingress_matches_oracle(gpu, oracle, tokens, streams, width, iterations):
     """Ingress + weighted RMS norm against numeric.c's order of operations. The kernel rounds the
     residual to bf16 as the reference's device kernel does, so the oracle is fed the rounded
@@ -279,7 +280,8 @@ def test_envelope_ingress_matches_oracle(gpu, oracle, tokens, streams, width, it
     assert np.all(np.abs(got[differ] - want[differ]) <= 2.0 ** -7 * np.abs(want[differ]))
 
 
-@pytest.mark.parametrize("tokens,streams,width", [(5, 4, 7168), (3, 1, 512), (2, 7, 200), (64, 4, 300)])
+@pytest.mark.parametrize("tokens,streams,width", [(5, 4, 7168), (3, 1, 512), (2, 7, 200), (64, 4, 300),
+                                                  (3, 5, 203)])
 def test_envelope_egress_bit_exact(gpu, oracle, tokens, streams, width):
     """Egress is double-precision multiply-adds in a fixed order and one bf16 rounding: bit-exact."""
     from yvex_amd import kernels as K

@@ -133,13 +133,15 @@ def argmax_f32(values, status, out=None, scratch=None):
 
 
 def mhc_ingress(rows, mixes, scale, base, norm, *, streams, width, iterations, rms_epsilon,
-                mhc_epsilon, post_multiplier, status):
+                mhc_epsilon, post_multiplier, status, out=None):
     """Residual-stream ingress + weighted RMS norm: (normalized [n, width], post [n, streams],
     combination [n, streams, streams])."""
     count = rows.shape[0]
-    normalized = torch.empty((count, width), dtype=torch.float32, device=rows.device)
-    post = torch.empty((count, streams), dtype=torch.float32, device=rows.device)
-    combination = torch.empty((count, streams, streams), dtype=torch.float32, device=rows.device)
+    if out is None:
+        out = (torch.empty((count, width), dtype=torch.float32, device=rows.device),
+               torch.empty((count, streams), dtype=torch.float32, device=rows.device),
+               torch.empty((count, streams, streams), dtype=torch.float32, device=rows.device))
+    normalized, post, combination = out
     _call("yvex_hip_mhc_ingress", _ptr(rows), _ptr(mixes), _ptr(scale), _ptr(base), _ptr(norm),
           C.c_uint64(count), C.c_uint64(streams), C.c_uint64(width), C.c_uint64(iterations),
           C.c_double(rms_epsilon), C.c_double(mhc_epsilon), C.c_double(post_multiplier),
@@ -147,10 +149,11 @@ def mhc_ingress(rows, mixes, scale, base, norm, *, streams, width, iterations, r
     return normalized, post, combination
 
 
-def mhc_egress(core, rows, post, combination, *, streams, width, status):
+def mhc_egress(core, rows, post, combination, *, streams, width, status, out=None):
     """Residual-stream egress: [n, streams * width] bf16-valued F32 rows."""
     count = core.shape[0]
-    out = torch.empty((count, streams * width), dtype=torch.float32, device=core.device)
+    if out is None:
+        out = torch.empty((count, streams * width), dtype=torch.float32, device=core.device)
     _call("yvex_hip_mhc_egress", _ptr(core), _ptr(rows), _ptr(post), _ptr(combination),
           C.c_uint64(count), C.c_uint64(streams), C.c_uint64(width), _ptr(out), _ptr(status), _stream())
     return out
