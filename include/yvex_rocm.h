@@ -554,7 +554,12 @@ typedef struct {
     char execution_identity[YVEX_SHA256_HEX_CAP];
 } yvex_moe_row_batch_result;
 
-/* moe.h:277-297. derived_layout_plan/build take the reference's physical-execution decision;
+/* moe.h:277-297. execute_rows follows src/backend/cuda/moe.c:1826-1923: with mixing rows in the
+ * layer plan it runs the residual-stream ingress (mixing projection, gates, Sinkhorn matrix,
+ * weighted RMS norm; moe.c:1210-1254), the experts on the normalised rows and the egress onto the
+ * streams (moe.c:1533-1541); rows are then row_count x expanded_width. Without mixing rows the
+ * rows are taken as normalised hidden rows and the output is bf16(routed + shared).
+ * derived_layout_plan/build take the reference's physical-execution decision;
  * this backend streams canonical GGUF rows directly and needs no derived layout, so both
  * answer UNSUPPORTED and callers keep layout CANONICAL_ROW / EXPERT_MAJOR. */
 typedef struct {
