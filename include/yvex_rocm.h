@@ -594,6 +594,64 @@ typedef struct {
 /* moe.h:295-296: NULL unless the backend is ROCM and its kernels are loadable. */
 const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend);
 
+/* ---- token-local MoE operation: include/yvex/internal/moe.h:161-166,198-214,308-319 ------------ */
+
+#define YVEX_RUNTIME_DESCRIPTOR_QTYPE_CAP 43u
+#define YVEX_ATTENTION_EVIDENCE_FULL 3      /* include/yvex/internal/graph.h:250-255 */
+
+typedef struct {
+    unsigned long long selected_count;
+    unsigned long long selected_experts[YVEX_MOE_MAX_SELECTED];
+    float router_logits[256], router_scores[256];
+    float selected_weights[YVEX_MOE_MAX_SELECTED];
+} yvex_moe_router_result;
+
+typedef struct {
+    float *combined_output, *post, *combination;
+    unsigned long long combined_capacity, post_capacity, combination_capacity;
+    float *routed_output, *shared_output;
+    unsigned long long routed_capacity, shared_capacity;
+    yvex_moe_router_result router;
+    unsigned long long expert_subviews_accessed, encoded_bytes_read;
+    unsigned long long host_to_device_bytes, device_to_host_bytes, kernel_launches;
+    unsigned long long cache_hits, cache_misses, upload_count, download_count;
+    unsigned long long stream_synchronizations, device_synchronizations, device_to_device_bytes;
+    yvex_execution_memory_facts memory;
+    unsigned long long ingress_ns, routing_ns, routed_ns, shared_ns, post_ns, total_ns;
+    unsigned long long synchronization_ns;
+    unsigned long long qtype_counts[YVEX_RUNTIME_DESCRIPTOR_QTYPE_CAP];
+    char routed_digest[YVEX_SHA256_HEX_CAP], shared_digest[YVEX_SHA256_HEX_CAP];
+    char combined_digest[YVEX_SHA256_HEX_CAP], routing_digest[YVEX_SHA256_HEX_CAP];
+} yvex_moe_layer_result;
+
+/* One row, experts handed over one at a time by a caller that loads them on demand
+ * (src/backend/cuda/moe.c:516-842; the caller is src/runtime/moe.c:647-720).
+ *
+ * begin: uploads job->expanded_input (or copies job->device_input), runs the residual-stream
+ *   ingress and the router, and publishes result->router (logits and scores unless a device
+ *   output is named and evidence is below FULL). When job->device_output is set, evidence is
+ *   below FULL and the three routed matrices are resident, the selected experts run on the
+ *   device at once and the caller adds the shared expert only.
+ * add_expert: intermediate = bf16(silu(min(g, L)) * clamp(u, +-L) * weight) with weight 1 for the
+ *   shared expert, output = bf16(down . intermediate), kept for the rank-ordered sum (at most
+ *   YVEX_MOE_MAX_SELECTED routed experts). Weight views outside the resident arena are uploaded
+ *   to a staging range owned by the execution.
+ * finish: routed = sum in the order added, combined = bf16(routed + shared); with a device
+ *   output the egress writes it; host copies as moe.c:775-803 publishes them.
+ * close: releases the execution (safe on NULL). A kernel status other than zero surfaces as
+ * BACKEND, as moe.c:277-296 reports it. */
+typedef struct yvex_backend_moe_execution yvex_backend_moe_execution;
+int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backend,
+                           const yvex_moe_layer_job *job, yvex_moe_layer_result *result,
+                           yvex_error *err);
+int yvex_backend_moe_add_expert(yvex_backend_moe_execution *execution,
+                                const yvex_moe_weight_view *gate, const yvex_moe_weight_view *up,
+                                const yvex_moe_weight_view *down, float route_weight, int shared,
+                                yvex_error *err);
+int yvex_backend_moe_finish(yvex_backend_moe_execution *execution, yvex_moe_layer_result *result,
+                            yvex_error *err);
+int yvex_backend_moe_close(yvex_backend_moe_execution **execution, yvex_error *err);
+
 /* Largest row batch execute_rows accepts in one call. */
 #define YVEX_ROCM_MOE_MAX_ROWS 4096ull
 

@@ -80,6 +80,12 @@ int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t row
                             double scaling, uint64_t *selected, float *weights, int *status,
                             yvex_hip_stream stream);
 
+/* scores[i] = score(logits[i]) under the layer's scoring policy, as float: what the token-local
+ * operation publishes beside the logits (src/backend/cuda/moe_kernels.cu:29-55,
+ * src/graph/moe.c:497-501). */
+int yvex_hip_moe_route_scores(const float *logits, uint64_t count, int scoring, float *scores,
+                              int *status, yvex_hip_stream stream);
+
 /* Replaces yvex_expert_worklist_build_cuda (moe_kernels.cu:294-402): stable counting sort of
  * the pairs = rows*topk (row, rank) pairs by expert; rows <= 4096 per call. Outputs, all
  * device memory:

@@ -230,6 +230,7 @@ class MoeCase:
         for name, blob in parts.items():
             arena[offsets[name]:offsets[name] + blob.nbytes] = blob
         _, host = b.resident(arena)
+        self.host, self.offsets = host, offsets
         self.x = g.normal(rows * expanded).reshape(rows, expanded)
         if streams:
             bits = self.x.view(np.uint32)       # bf16 values, as the CPU path expects of its input
@@ -488,3 +489,200 @@ def test_execute_rows_deferred_completion(backend, oracle):
     want = case.oracle_layer(act_q8=True)["combined"]
     err_abs = np.abs(got.astype(np.float64) - want)
     assert (err_abs > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
+
+
+# ---- token-local operation: src/backend/cuda/moe.c:516-842 --------------------------------------
+
+class TokenLocal:
+    """begin / add_expert / finish / close over one row of a MoeCase with residual streams."""
+
+    def __init__(self, case, row=0, device=False, evidence=0):
+        self.case, self.b = case, case.b
+        hidden, streams = case.hidden, case.streams
+        self.row = np.ascontiguousarray(case.x[row])
+        self.combined, self.routed = np.zeros(hidden, np.float32), np.zeros(hidden, np.float32)
+        self.shared = np.zeros(hidden, np.float32)
+        self.post, self.comb = np.zeros(streams, np.float32), np.zeros(streams * streams, np.float32)
+        r = self.result = abi.LayerResult()
+        r.combined_output, r.combined_capacity = self.combined.ctypes.data, hidden
+        r.routed_output, r.routed_capacity = self.routed.ctypes.data, hidden
+        r.shared_output, r.shared_capacity = self.shared.ctypes.data, hidden
+        r.post, r.post_capacity = self.post.ctypes.data, streams
+        r.combination, r.combination_capacity = self.comb.ctypes.data, streams * streams
+        self.job = case.job
+        self.job.expanded_input = self.row.ctypes.data
+        self.job.evidence_level = evidence
+        self.device_in = self.device_out = None
+        if device:
+            self.device_in, self.device_out = self.b.f32(self.row), self.b.empty_f32(self.row.size)
+            self.job.device_input = C.cast(self.device_in, C.c_void_p)
+            self.job.device_output = C.cast(self.device_out, C.c_void_p)
+        self.handle, self.err = C.c_void_p(), abi.Error()
+
+    def begin(self):
+        return self.b.lib.yvex_backend_moe_begin(C.byref(self.handle), self.b.handle, C.byref(self.job),
+                                                 C.byref(self.result), C.byref(self.err))
+
+    def expert_views(self, expert=None, outside=False):
+        """Weight views of one routed expert (a slice of the expert-major matrices) or of the
+        shared expert; outside=True points them at a private host copy, away from the arena."""
+        case, keep = self.case, []
+        names = ("gate", "up", "down") if expert is not None else ("sgate", "sup", "sdown")
+        slots = (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN) if expert is not None else \
+            (abi.W_SHARED_GATE, abi.W_SHARED_UP, abi.W_SHARED_DOWN)
+        views = []
+        for name, slot, rows in zip(names, slots, (case.intermediate, case.intermediate, case.hidden)):
+            whole = case.job.weights[slot]
+            v = abi.WeightView()
+            C.memmove(C.byref(v), C.byref(whole), C.sizeof(v))
+            nbytes = whole.row_bytes * rows
+            start = (expert or 0) * nbytes
+            v.row_count, v.encoded_bytes, v.storage_bytes = rows, nbytes, nbytes
+            if outside:
+                copy = np.ascontiguousarray(case.parts[name][start:start + nbytes])
+                keep.append(copy)
+                v.encoded = copy.ctypes.data
+            else:
+                v.encoded = case.host + case.offsets[name] + start
+            views.append(v)
+        return views, keep
+
+    def add(self, views, weight, shared):
+        return self.b.lib.yvex_backend_moe_add_expert(self.handle, C.byref(views[0]), C.byref(views[1]),
+                                                      C.byref(views[2]), C.c_float(weight), int(shared),
+                                                      C.byref(self.err))
+
+    def finish(self):
+        return self.b.lib.yvex_backend_moe_finish(self.handle, C.byref(self.result), C.byref(self.err))
+
+    def close(self):
+        return self.b.lib.yvex_backend_moe_close(C.byref(self.handle), C.byref(self.err))
+
+
+def token_oracle(case, row):
+    """CPU path for one row: ingress, routing, experts on F32 activations in rank order, shared
+    expert, bf16(routed + shared), egress (src/runtime/moe.c:596-645)."""
+    o, p = case.oracle, case.parts
+    norm = (p["norm"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    rc, x, post, comb = o.moe_ffn_prepare(
+        o.F32, p["function"], case.x[row], p["scale"].view(np.float32), p["base"].view(np.float32), norm,
+        streams=case.streams, width=case.hidden, iterations=case.iterations, rms_epsilon=1e-6,
+        mhc_epsilon=1e-6, post_multiplier=2.0)
+    assert rc == 0
+    logits = o.matvec(o.F32, p["router"], case.experts, case.hidden, x)
+    want = o.moe_layer(hidden=case.hidden, intermediate=case.intermediate, experts=case.experts,
+                       topk=case.topk, qtypes=(case.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
+                       shared=(p["sgate"], p["sup"], p["sdown"]), inputs=x, logits=logits,
+                       bias=p["bias"].view(np.float32), scoring=case.scoring, normalize=True, scaling=1.5,
+                       act_q8=False, threads=1)
+    rc, want["envelope"] = o.mhc_post(want["combined"], case.x[row], post, comb, streams=case.streams,
+                                      width=case.hidden)
+    assert rc == 0
+    want.update(logits=logits.ravel(), post=post.ravel(), combination=comb.ravel())
+    return want
+
+
+def to_bf16(values):
+    bits = np.ascontiguousarray(values, np.float32).view(np.uint32)
+    return ((bits + 0x7fff + ((bits >> 16) & 1)) & 0xffff0000).view(np.float32)
+
+
+def rows_close(got, ref, steps=2):
+    err = np.abs(got.astype(np.float64) - ref)
+    outside = err > 1e-5 + 1e-3 * np.abs(ref)
+    return outside.mean() < 2e-2 and np.all(err[outside] <= steps * 2.0 ** -7 * np.abs(ref[outside]) + 1e-4)
+
+
+@pytest.mark.parametrize("qtype,outside", [("IQ2_XXS", False), ("Q8_0", True)])
+def test_token_local_host_publication(backend, oracle, qtype, outside):
+    """The caller's loop of src/runtime/moe.c:647-720: begin publishes logits, scores and the
+    routing; each selected expert is added with its route weight, then the shared expert; finish
+    publishes routed, shared, combined, post and combination. With outside=True the expert views
+    point at host memory outside the arena and travel through the staging range."""
+    case = MoeCase(backend, oracle, qtype=qtype, hidden=512, rows=2, streams=4, iterations=20,
+                   act=abi.ACT_DEVICE_F32)
+    t = TokenLocal(case, row=1)
+    assert t.begin() == 0, t.err.message
+    want = token_oracle(case, 1)
+    router = t.result.router
+    assert router.selected_count == case.topk
+    assert list(router.selected_experts)[:case.topk] == list(want["selected"][0])
+    weights = np.array(list(router.selected_weights)[:case.topk], np.float32)
+    assert np.max(np.abs(weights - want["weights"][0])) <= 1e-4
+    logits = np.array(list(router.router_logits)[:case.experts], np.float32)
+    assert close_to(logits, want["logits"], rel=1e-3, abs_=1e-4)
+    rc, _, _, scores = oracle.moe_route(logits, None, case.topk, case.scoring, True, 1.0)
+    assert np.allclose(np.array(list(router.router_scores)[:case.experts], np.float32), scores, rtol=1e-6)
+    keep = []
+    for rank in range(case.topk):
+        views, held = t.expert_views(int(router.selected_experts[rank]), outside=outside)
+        keep.append(held)
+        assert t.add(views, float(weights[rank]), False) == 0, t.err.message
+    views, held = t.expert_views(None, outside=outside)
+    assert t.add(views, 0.0, True) == 0, t.err.message
+    assert t.finish() == 0, t.err.message
+    assert np.max(np.abs(t.post - want["post"])) <= 1e-4
+    assert np.max(np.abs(t.comb - want["combination"])) <= 1e-4
+    assert rows_close(t.routed, want["routed"][0], 4) and rows_close(t.shared, want["shared"][0])
+    assert rows_close(t.combined, want["combined"][0], 4)
+    assert np.array_equal(t.combined, to_bf16(t.routed + t.shared))      # the combine itself is exact
+    r = t.result
+    assert r.expert_subviews_accessed == 3 * case.topk and r.kernel_launches >= 12
+    assert (r.upload_count > 0) == outside and r.stream_synchronizations == 2
+    # a finished execution takes no more experts and does not finish twice
+    assert t.add(views, 0.0, True) == abi.INVALID_ARG and t.finish() == abi.INVALID_ARG
+    assert t.close() == 0 and not t.handle.value and t.close() == 0
+
+
+def test_token_local_device_output_runs_selected_experts(backend, oracle):
+    """With a device output, evidence below FULL and resident routed matrices, begin runs the
+    selected experts on the device (moe.c:584-672); the caller adds the shared expert only and
+    finish writes the egress into the device output."""
+    case = MoeCase(backend, oracle, qtype="IQ2_XXS", hidden=512, rows=3, streams=4, iterations=20,
+                   act=abi.ACT_DEVICE_F32)
+    t = TokenLocal(case, row=2, device=True)
+    assert t.begin() == 0, t.err.message
+    views, _ = t.expert_views(None)
+    assert t.add(views, 0.0, True) == 0, t.err.message
+    assert t.finish() == 0, t.err.message
+    want = token_oracle(case, 2)
+    router = t.result.router
+    assert list(router.selected_experts)[:case.topk] == list(want["selected"][0])
+    got = backend.read_f32(t.device_out, case.streams * case.hidden)
+    assert t.device_out.contents.is_written == 1
+    scale = np.abs(want["envelope"][0]) + np.abs(want["combined"]).max()
+    assert np.all(np.abs(got - want["envelope"][0]) <= 2.0 ** -6 * scale)
+    assert np.array_equal(got.view(np.uint32) & 0xffff, np.zeros(got.size, np.uint32))
+    assert not t.combined.any()            # host copies are evidence, not published on this path
+    assert t.result.expert_subviews_accessed == 3 * case.topk and t.result.device_to_device_bytes > 0
+    assert t.close() == 0
+
+
+def test_token_local_refusals(backend, oracle):
+    case = MoeCase(backend, oracle, hidden=512, rows=2, streams=2, iterations=2, act=abi.ACT_DEVICE_F32)
+    t = TokenLocal(case)
+    t.result.post_capacity = 1
+    assert t.begin() == abi.INVALID_ARG and not t.handle.value
+    t.result.post_capacity = 2
+    case.plan.mhc_mixing_rows = 9
+    assert t.begin() == abi.BOUNDS
+    case.plan.mhc_mixing_rows = 8
+    case.plan.router_class = abi.ROUTER_HASH
+    assert t.begin() == abi.UNSUPPORTED
+    case.plan.router_class = abi.ROUTER_LEARNED
+    bad = t.row.copy()
+    bad[3] = np.inf
+    t.job.expanded_input = bad.ctypes.data
+    assert t.begin() == abi.BACKEND and not t.handle.value      # kernels flag non-finite input
+    t.job.expanded_input = t.row.ctypes.data
+    assert t.begin() == 0, t.err.message
+    views, _ = t.expert_views(0)
+    views[2].row_count = case.hidden - 1
+    assert t.add(views, 0.5, False) == abi.INVALID_ARG
+    views, _ = t.expert_views(0)
+    views[0].qtype = 2                                           # Q4_0: no device compute
+    assert t.add(views, 0.5, False) == abi.UNSUPPORTED
+    t.result.routed_capacity = 1
+    assert t.finish() == abi.INVALID_ARG
+    t.result.routed_capacity = case.hidden
+    assert t.finish() == 0 and t.close() == 0

@@ -119,6 +119,39 @@ def test_seam_backend_keeps_tensors_and_refuses_compute(seam):
     assert not lib.yvex_backend_moe_operations_get(seam.handle)
 
 
+def test_token_local_operation_without_kernels(seam):
+    """Argument refusals come first (src/backend/cuda/moe.c:523-540), then the missing kernel
+    bundle (moe.c:563-567); close is safe on an execution that never began."""
+    lib = seam.lib
+    plan, job, result, err = abi.LayerPlan(), abi.LayerJob(), abi.LayerResult(), abi.Error()
+    handle = C.c_void_p()
+    job.layer = C.pointer(plan)
+    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+                                      C.byref(err)) == abi.INVALID_ARG
+    plan.hidden_width, plan.residual_streams, plan.expanded_width = 256, 2, 512
+    plan.mhc_mixing_rows, plan.mhc_sinkhorn_iterations = 8, 2
+    plan.rms_epsilon = plan.mhc_epsilon = 1e-6
+    plan.mhc_post_multiplier, plan.activation_limit, plan.routed_scaling_factor = 2.0, 10.0, 1.0
+    plan.routed_experts, plan.experts_per_token, plan.shared_experts = 8, 2, 1
+    plan.expert_intermediate_width = plan.shared_intermediate_width = 256
+    plan.router_class = abi.ROUTER_LEARNED
+    row = np.zeros(512, np.float32)
+    out = [np.zeros(n, np.float32) for n in (256, 256, 256, 2, 4)]
+    job.expanded_input = row.ctypes.data
+    result.combined_output, result.routed_output, result.shared_output = (a.ctypes.data for a in out[:3])
+    result.combined_capacity = result.routed_capacity = result.shared_capacity = 256
+    result.post, result.post_capacity = out[3].ctypes.data, 2
+    result.combination, result.combination_capacity = out[4].ctypes.data, 4
+    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+                                      C.byref(err)) == abi.UNSUPPORTED
+    assert not handle.value and b"kernel" in err.message
+    plan.mhc_mixing_rows = 7
+    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+                                      C.byref(err)) == abi.BOUNDS
+    assert lib.yvex_backend_moe_close(C.byref(handle), C.byref(err)) == 0
+    assert lib.yvex_backend_moe_finish(None, C.byref(result), C.byref(err)) == abi.INVALID_ARG
+
+
 def test_tensor_ownership_and_limits(monkeypatch):
     monkeypatch.setenv("YVEX_TEST_ROCM_NO_DEVICE", "1")
     from backend_helpers import Backend

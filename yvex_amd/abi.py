@@ -146,6 +146,29 @@ class LayerJob(C.Structure):
                 ("worklist_policy", C.POINTER(WorklistPolicy))]
 
 
+class RouterResult(C.Structure):
+    _fields_ = [("selected_count", ULL), ("selected_experts", ULL * 16),
+                ("router_logits", C.c_float * 256), ("router_scores", C.c_float * 256),
+                ("selected_weights", C.c_float * 16)]
+
+
+class LayerResult(C.Structure):
+    _fields_ = [("combined_output", C.c_void_p), ("post", C.c_void_p), ("combination", C.c_void_p),
+                ("combined_capacity", ULL), ("post_capacity", ULL), ("combination_capacity", ULL),
+                ("routed_output", C.c_void_p), ("shared_output", C.c_void_p),
+                ("routed_capacity", ULL), ("shared_capacity", ULL), ("router", RouterResult)] + \
+               [(n, ULL) for n in ("expert_subviews_accessed", "encoded_bytes_read", "host_to_device_bytes",
+                                   "device_to_host_bytes", "kernel_launches", "cache_hits", "cache_misses",
+                                   "upload_count", "download_count", "stream_synchronizations",
+                                   "device_synchronizations", "device_to_device_bytes")] + \
+               [("memory", MemoryFacts)] + \
+               [(n, ULL) for n in ("ingress_ns", "routing_ns", "routed_ns", "shared_ns", "post_ns",
+                                   "total_ns", "synchronization_ns")] + \
+               [("qtype_counts", ULL * 43)] + \
+               [(n, C.c_char * HEX) for n in ("routed_digest", "shared_digest", "combined_digest",
+                                              "routing_digest")]
+
+
 class RowBatch(C.Structure):
     _fields_ = [("schema_version", C.c_uint), ("row_count", ULL), ("row_width", ULL),
                 ("row_stride", ULL), ("expanded_rows", C.c_void_p),
@@ -221,13 +244,14 @@ EXPORTS = [
     "yvex_backend_workspace_attach", "yvex_backend_workspace_detach",
     "yvex_backend_workspace_acquire", "yvex_backend_rocm_encoded_matvec",
     "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows",
-    "yvex_backend_moe_operations_get",
+    "yvex_backend_moe_operations_get", "yvex_backend_moe_begin", "yvex_backend_moe_add_expert",
+    "yvex_backend_moe_finish", "yvex_backend_moe_close",
     "yvex_expert_worklist_build",
 ]
 KERNEL_EXPORTS = [
     "yvex_hip_q8k_quantize", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
     "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes",
-    "yvex_hip_moe_route_rows", "yvex_hip_worklist_build", "yvex_hip_moe_up", "yvex_hip_moe_down",
+    "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_worklist_build", "yvex_hip_moe_up", "yvex_hip_moe_down",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
     "yvex_hip_moe_reduce_combine", "yvex_hip_mhc_ingress", "yvex_hip_mhc_egress",
     "yvex_hip_stream_read", "yvex_hip_fill_u32",
@@ -245,6 +269,12 @@ def library():
     lib.yvex_quant_numeric_capability_at.restype = C.POINTER(NumericCapability)
     lib.yvex_backend_moe_operations_get.restype = C.POINTER(MoeOperations)
     lib.yvex_backend_moe_operations_get.argtypes = [C.c_void_p]
+    lib.yvex_backend_moe_begin.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.POINTER(LayerJob),
+                                           C.POINTER(LayerResult), C.POINTER(Error)]
+    lib.yvex_backend_moe_add_expert.argtypes = [C.c_void_p, C.POINTER(WeightView), C.POINTER(WeightView),
+                                                C.POINTER(WeightView), C.c_float, C.c_int, C.POINTER(Error)]
+    lib.yvex_backend_moe_finish.argtypes = [C.c_void_p, C.POINTER(LayerResult), C.POINTER(Error)]
+    lib.yvex_backend_moe_close.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
     lib.yvex_backend_open.argtypes = [C.POINTER(C.c_void_p), C.POINTER(BackendOptions), C.POINTER(Error)]
     lib.yvex_backend_close_checked.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
     lib.yvex_backend_tensor_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),

@@ -24,6 +24,19 @@ __device__ __forceinline__ double route_score(double v, int scoring)
     return sqrt(softplus);
 }
 
+// The scores alone, as the token-local operation publishes them beside the logits
+// (src/backend/cuda/moe_kernels.cu:29-55).
+__global__ __launch_bounds__(256) void route_scores_kernel(
+    const float *__restrict__ logits, unsigned count, int scoring, float *__restrict__ scores, int *status)
+{
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= count) return;
+    const double s = route_score((double)logits[i], scoring);
+    const float published = (float)s;
+    if (!(s == s) || !finite_f32(published)) raise_status(status, 1);
+    scores[i] = published;
+}
+
 // One wavefront per row; each lane scores four experts (experts <= 256).
 __global__ __launch_bounds__(256) void route_rows_kernel(
     const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long rows,
@@ -641,6 +654,17 @@ extern "C" int yvex_hip_moe_route_rows(const float *logits, const float *bias, u
         logits, bias, rows, (unsigned)experts, (unsigned)topk, scoring, normalize, scaling,
         (unsigned long long *)selected, weights, status);
     return check_launch("moe_route_rows");
+}
+
+extern "C" int yvex_hip_moe_route_scores(const float *logits, uint64_t count, int scoring,
+                                         float *scores, int *status, yvex_hip_stream stream)
+{
+    if (!logits || !scores || !status || !count || count > 0x7fffffffull ||
+        (scoring != YVEX_HIP_SCORING_SQRT_SOFTPLUS && scoring != YVEX_HIP_SCORING_SIGMOID))
+        return ST_INVALID_ARG;
+    route_scores_kernel<<<(unsigned)((count + 255u) / 256u), 256, 0, as_stream(stream)>>>(
+        logits, (unsigned)count, scoring, scores, status);
+    return check_launch("moe_route_scores");
 }
 
 extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,

@@ -42,7 +42,7 @@ static int moe_envelope(const yvex_moe_layer_plan *layer)
     return layer->mhc_mixing_rows != 0ull;
 }
 
-static int moe_envelope_geometry(const yvex_moe_layer_plan *layer)
+int yvex_rocm_moe_envelope_geometry(const yvex_moe_layer_plan *layer)
 {
     unsigned long long streams = layer->residual_streams;
     return streams >= 1ull && streams <= 7ull && layer->hidden_width <= 16384ull &&
@@ -63,7 +63,7 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
         layer->experts_per_token > layer->routed_experts || !layer->expert_intermediate_width ||
         layer->hidden_width > (1ull << 20) || layer->expert_intermediate_width > (1ull << 20) ||
         layer->shared_intermediate_width > (1ull << 20) || layer->shared_experts > 1ull ||
-        (moe_envelope(layer) && !moe_envelope_geometry(layer)))
+        (moe_envelope(layer) && !yvex_rocm_moe_envelope_geometry(layer)))
         return 0;
     streams = moe_envelope(layer) ? layer->residual_streams : 0ull;
     pairs = rows * layer->experts_per_token;
@@ -190,9 +190,9 @@ static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight
 }
 
 /* Check one weight view against the geometry the plan implies and find its device address. */
-static int view_resolve(const yvex_backend *backend, const yvex_moe_weight_view *view,
-                        unsigned long long row_width, unsigned long long row_count,
-                        unsigned long long *device_address, yvex_error *err)
+int yvex_rocm_moe_view_check(const yvex_backend *backend, const yvex_moe_weight_view *view,
+                             unsigned long long row_width, unsigned long long row_count,
+                             unsigned long long *device_address, int *resident, yvex_error *err)
 {
     const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(view->qtype);
     const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(view->qtype);
@@ -206,14 +206,31 @@ static int view_resolve(const yvex_backend *backend, const yvex_moe_weight_view 
         view->row_bytes * row_count != view->encoded_bytes)
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
                                 "MoE weight view geometry disagrees with the layer plan");
+    *resident = 1;
+    *device_address = 0ull;
     if (view->device_address) {
         *device_address = view->device_address;
         return YVEX_OK;
     }
-    if (!view->encoded || !yvex_rocm_resolve(backend, view->encoded, view->encoded_bytes, device_address))
+    if (!view->encoded)
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights", "MoE weight view has no bytes");
+    if (!yvex_rocm_resolve(backend, view->encoded, view->encoded_bytes, device_address)) {
+        *resident = 0;
+        *device_address = 0ull;
+    }
+    return YVEX_OK;
+}
+
+static int view_resolve(const yvex_backend *backend, const yvex_moe_weight_view *view,
+                        unsigned long long row_width, unsigned long long row_count,
+                        unsigned long long *device_address, yvex_error *err)
+{
+    int resident = 0;
+    int rc = yvex_rocm_moe_view_check(backend, view, row_width, row_count, device_address, &resident, err);
+    if (rc == YVEX_OK && !resident)
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
                                 "MoE weight view is not inside the attached resident arena");
-    return YVEX_OK;
+    return rc;
 }
 
 static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weight_view *gate,
@@ -289,7 +306,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         (layer->scoring != YVEX_MOE_SCORING_SQRT_SOFTPLUS && layer->scoring != YVEX_MOE_SCORING_SIGMOID))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
                                 "hash routing, other scoring policies and expanded rows without mixing rows are outside this backend");
-    if (envelope && !moe_envelope_geometry(layer))
+    if (envelope && !yvex_rocm_moe_envelope_geometry(layer))
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows",
                                 "residual-stream geometry is invalid");
     streams = envelope ? layer->residual_streams : 0ull;

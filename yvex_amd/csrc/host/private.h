@@ -48,4 +48,14 @@ int yvex_rocm_status_reset(yvex_backend *backend, const char *where, yvex_error 
 int yvex_rocm_resolve(const yvex_backend *backend, const unsigned char *host,
                       unsigned long long bytes, unsigned long long *device_address);
 
+/* Residual-stream geometry of a layer plan (src/graph/numeric.c:668-689) within this backend's
+ * bounds: at most 7 streams, width at most 16384. */
+int yvex_rocm_moe_envelope_geometry(const yvex_moe_layer_plan *layer);
+/* Check a weight view against the shape the plan implies (FORMAT), its qtype against the device
+ * capability rows (UNSUPPORTED), and find its device address; *resident = 0 when the bytes lie
+ * outside the attached arena and carry no device address (the address is then left 0). */
+int yvex_rocm_moe_view_check(const yvex_backend *backend, const yvex_moe_weight_view *view,
+                             unsigned long long row_width, unsigned long long row_count,
+                             unsigned long long *device_address, int *resident, yvex_error *err);
+
 #endif
