@@ -785,10 +785,6 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-#ifdef YVEX_ONLY_NB
-        mfma_item<FUSED_UP, YVEX_ONLY_NB>(a, it);
-        continue;
-#endif
         if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
         else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
         else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
