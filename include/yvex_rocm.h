@@ -594,6 +594,56 @@ typedef struct {
 /* moe.h:295-296: NULL unless the backend is ROCM and its kernels are loadable. */
 const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend);
 
+/* ---- GGUF tensor directory and resident loading: include/yvex/gguf.h:142-195 ------------------- */
+
+#define YVEX_GGUF_MAX_DIMS 4u
+
+/* include/yvex/gguf.h:142-154 */
+typedef struct {
+    const char *name;
+    unsigned long long name_len;
+    unsigned int rank;
+    unsigned long long dims[YVEX_GGUF_MAX_DIMS];
+    unsigned int ggml_type;
+    const char *ggml_type_name;
+    unsigned long long relative_offset, absolute_offset, storage_bytes, absolute_end_offset;
+    int range_addressable;
+} yvex_gguf_tensor_info;
+
+typedef struct yvex_gguf yvex_gguf;
+
+/* Structural reader with the rules and refusal codes of the reference's yvex_gguf_open
+ * (src/gguf/core.c:1163-1249, :52-79): version 3 only (UNSUPPORTED), bad magic / rank / dimension
+ * / alignment / key grammar / duplicate names (FORMAT), truncation and extents beyond the file
+ * (BOUNDS), qtypes without storage geometry (UNSUPPORTED). It takes a path where the reference
+ * takes its artifact handle. Scalar and string metadata are kept; arrays are walked and dropped. */
+int yvex_gguf_open_path(yvex_gguf **out, const char *path, yvex_error *err);
+void yvex_gguf_close(yvex_gguf *gguf);
+unsigned long long yvex_gguf_metadata_count(const yvex_gguf *gguf);
+int yvex_gguf_metadata_u64(const yvex_gguf *gguf, const char *key, unsigned long long *out);
+int yvex_gguf_metadata_f64(const yvex_gguf *gguf, const char *key, double *out);
+int yvex_gguf_metadata_string(const yvex_gguf *gguf, const char *key, const char **text,
+                              unsigned long long *len);
+unsigned long long yvex_gguf_tensor_count(const yvex_gguf *gguf);
+const yvex_gguf_tensor_info *yvex_gguf_tensor_at(const yvex_gguf *gguf, unsigned long long index);
+const yvex_gguf_tensor_info *yvex_gguf_tensor_find(const yvex_gguf *gguf, const char *name);
+unsigned long long yvex_gguf_tensor_data_offset(const yvex_gguf *gguf);
+unsigned int yvex_gguf_alignment(const yvex_gguf *gguf);
+unsigned long long yvex_gguf_file_size(const yvex_gguf *gguf);
+
+/* The reference's runtime maps an artifact's tensor-data section into the resident arena and
+ * hands the backend borrowed pointers into it (src/runtime/residency.c, contract text
+ * include/yvex/internal/backend.h:283-288). Here: one resident arena of the section's size, the
+ * bytes read from the file into its host shadow, one attach (the upload to HBM). A weight view
+ * of a named tensor is then host_base + relative_offset with rows of dims[0] values; tensors of
+ * rank 3 are expert-major (rows = dims[1] * dims[2]). The view's activation class and kernel
+ * family are the caller's to set. */
+int yvex_backend_rocm_gguf_resident_load(yvex_backend *backend, const yvex_gguf *gguf,
+                                         unsigned long long generation, yvex_device_tensor **arena,
+                                         unsigned char **host_base, yvex_error *err);
+int yvex_backend_rocm_gguf_weight_view(const yvex_gguf *gguf, const unsigned char *host_base,
+                                       const char *name, yvex_moe_weight_view *view, yvex_error *err);
+
 /* ---- token-local MoE operation: include/yvex/internal/moe.h:161-166,198-214,308-319 ------------ */
 
 #define YVEX_RUNTIME_DESCRIPTOR_QTYPE_CAP 43u

@@ -10,6 +10,13 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # PyTorch carries its own copy of the HIP runtime. A process that loads libyvex_rocm.so (and
+    # with it the system's copy) before torch ends up with two runtimes, and the second one finds
+    # no device: torch goes first in every test process, also for tests that never touch it.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
 
 
 @pytest.fixture(scope="session")

@@ -146,6 +146,13 @@ class LayerJob(C.Structure):
                 ("worklist_policy", C.POINTER(WorklistPolicy))]
 
 
+class GgufTensorInfo(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("name_len", ULL), ("rank", C.c_uint), ("dims", ULL * 4),
+                ("ggml_type", C.c_uint), ("ggml_type_name", C.c_char_p), ("relative_offset", ULL),
+                ("absolute_offset", ULL), ("storage_bytes", ULL), ("absolute_end_offset", ULL),
+                ("range_addressable", C.c_int)]
+
+
 class RouterResult(C.Structure):
     _fields_ = [("selected_count", ULL), ("selected_experts", ULL * 16),
                 ("router_logits", C.c_float * 256), ("router_scores", C.c_float * 256),
@@ -247,6 +254,10 @@ EXPORTS = [
     "yvex_backend_moe_operations_get", "yvex_backend_moe_begin", "yvex_backend_moe_add_expert",
     "yvex_backend_moe_finish", "yvex_backend_moe_close",
     "yvex_expert_worklist_build",
+    "yvex_gguf_open_path", "yvex_gguf_close", "yvex_gguf_metadata_count", "yvex_gguf_metadata_u64",
+    "yvex_gguf_metadata_f64", "yvex_gguf_metadata_string", "yvex_gguf_tensor_count", "yvex_gguf_tensor_at",
+    "yvex_gguf_tensor_find", "yvex_gguf_tensor_data_offset", "yvex_gguf_alignment", "yvex_gguf_file_size",
+    "yvex_backend_rocm_gguf_resident_load", "yvex_backend_rocm_gguf_weight_view",
 ]
 KERNEL_EXPORTS = [
     "yvex_hip_q8k_quantize", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
@@ -269,6 +280,27 @@ def library():
     lib.yvex_quant_numeric_capability_at.restype = C.POINTER(NumericCapability)
     lib.yvex_backend_moe_operations_get.restype = C.POINTER(MoeOperations)
     lib.yvex_backend_moe_operations_get.argtypes = [C.c_void_p]
+    lib.yvex_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
+    lib.yvex_gguf_close.argtypes = [C.c_void_p]
+    lib.yvex_gguf_close.restype = None
+    for name in ("yvex_gguf_metadata_count", "yvex_gguf_tensor_count", "yvex_gguf_tensor_data_offset",
+                 "yvex_gguf_file_size"):
+        getattr(lib, name).argtypes = [C.c_void_p]
+        getattr(lib, name).restype = ULL
+    lib.yvex_gguf_alignment.argtypes = [C.c_void_p]
+    lib.yvex_gguf_alignment.restype = C.c_uint
+    lib.yvex_gguf_metadata_u64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(ULL)]
+    lib.yvex_gguf_metadata_f64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
+    lib.yvex_gguf_metadata_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(ULL)]
+    lib.yvex_gguf_tensor_at.argtypes = [C.c_void_p, ULL]
+    lib.yvex_gguf_tensor_at.restype = C.POINTER(GgufTensorInfo)
+    lib.yvex_gguf_tensor_find.argtypes = [C.c_void_p, C.c_char_p]
+    lib.yvex_gguf_tensor_find.restype = C.POINTER(GgufTensorInfo)
+    lib.yvex_backend_rocm_gguf_resident_load.argtypes = [C.c_void_p, C.c_void_p, ULL,
+                                                         C.POINTER(C.POINTER(DeviceTensor)),
+                                                         C.POINTER(C.c_void_p), C.POINTER(Error)]
+    lib.yvex_backend_rocm_gguf_weight_view.argtypes = [C.c_void_p, C.c_void_p, C.c_char_p,
+                                                       C.POINTER(WeightView), C.POINTER(Error)]
     lib.yvex_backend_moe_begin.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.POINTER(LayerJob),
                                            C.POINTER(LayerResult), C.POINTER(Error)]
     lib.yvex_backend_moe_add_expert.argtypes = [C.c_void_p, C.POINTER(WeightView), C.POINTER(WeightView),
