@@ -80,6 +80,18 @@ int yvex_hip_moe_route_rows(const float *logits, const float *bias, uint64_t row
                             double scaling, uint64_t *selected, float *weights, int *status,
                             yvex_hip_stream stream);
 
+/* Hash router of yvex_moe_route_rows (moe_kernels.cu:222-245; CPU rule src/graph/moe.c:539-582):
+ * row r takes the first topk ordinals of row token_ids[r] of an I32 table (table_row_bytes per
+ * row, 4-byte aligned; single_row != 0: the table holds one row that serves every token, as
+ * moe.c:547-549 reads it) and weighs them like the learned router. token_ids[r] >= table_rows,
+ * an ordinal outside [0, experts) or a repeated one raise status 2. */
+int yvex_hip_moe_route_hash_rows(const float *logits, const uint8_t *table,
+                                 const uint32_t *token_ids, uint64_t rows, uint64_t experts,
+                                 uint64_t topk, uint64_t table_rows, uint64_t table_row_bytes,
+                                 int single_row, int scoring, int normalize, double scaling,
+                                 uint64_t *selected, float *weights, int *status,
+                                 yvex_hip_stream stream);
+
 /* scores[i] = score(logits[i]) under the layer's scoring policy, as float: what the token-local
  * operation publishes beside the logits (src/backend/cuda/moe_kernels.cu:29-55,
  * src/graph/moe.c:497-501). */

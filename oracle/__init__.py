@@ -44,7 +44,7 @@ class MoeLayerArgs(C.Structure):
         ("router_bias", C.c_void_p),
         ("scoring", C.c_int), ("normalize", C.c_int), ("act_q8", C.c_int),
         ("scaling", C.c_double), ("activation_limit", C.c_double),
-        ("threads", C.c_uint),
+        ("threads", C.c_uint), ("hash_selected", C.c_void_p),
     ]
 
 
@@ -283,6 +283,20 @@ def moe_route(logits: np.ndarray, bias, topk: int, scoring: int, normalize: bool
     return rc, sel, w, scores
 
 
+def moe_route_hash(logits: np.ndarray, table: np.ndarray, token: int, topk: int, scoring: int,
+                   normalize: bool, scaling: float):
+    """Hash router: table is [rows, columns] int32 (columns >= topk)."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    table = np.ascontiguousarray(table, np.int32).reshape(-1, np.asarray(table).shape[-1])
+    sel, w = np.zeros(topk, np.uint64), np.zeros(topk, np.float32)
+    scores = np.empty(logits.size, np.float32)
+    rc = lib().yvo_moe_route_hash(_p(logits), _p(table), C.c_uint64(table.shape[0]),
+                                  C.c_uint64(table.shape[1] * 4), C.c_uint64(token), C.c_uint64(logits.size),
+                                  C.c_uint64(topk), C.c_int(scoring), C.c_int(int(normalize)),
+                                  C.c_double(scaling), _p(scores), _p(sel), _p(w))
+    return rc, sel, w, scores
+
+
 def moe_expert(qtypes, gate, up, down, hidden, intermediate, x, route_weight, limit=10.0,
                act_q8=False):
     gq, uq, dq = qtypes
@@ -390,7 +404,7 @@ def moe_ffn_prepare(function_qtype, function, expanded, scale, base, norm, *, st
 
 def moe_layer(*, hidden, intermediate, experts, topk, qtypes, routed, shared, inputs, logits,
               bias=None, scoring=SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
-              act_q8=False, threads=1):
+              act_q8=False, threads=1, hash_selected=None):
     inputs = np.ascontiguousarray(inputs, np.float32).reshape(-1, hidden)
     logits = np.ascontiguousarray(logits, np.float32).reshape(-1, experts)
     rows = inputs.shape[0]
@@ -406,6 +420,8 @@ def moe_layer(*, hidden, intermediate, experts, topk, qtypes, routed, shared, in
     a.router_bias = b.ctypes.data if b is not None else None
     a.scoring, a.normalize, a.act_q8 = scoring, int(normalize), int(act_q8)
     a.scaling, a.activation_limit, a.threads = scaling, limit, threads
+    forced = None if hash_selected is None else np.ascontiguousarray(hash_selected, np.int32).reshape(rows, topk)
+    a.hash_selected = forced.ctypes.data if forced is not None else None
     sel = np.empty((rows, topk), np.uint64)
     w = np.empty((rows, topk), np.float32)
     routed_out = np.empty((rows, hidden), np.float32)

@@ -665,9 +665,11 @@ static double score_sigmoid(double v)
     return v >= 0.0 ? 1.0 / (1.0 + exp(-v)) : exp(v) / (1.0 + exp(v));
 }
 
-int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint64_t topk,
-                  int scoring, int normalize, double scaling, float *scores_out,
-                  uint64_t *selected, float *weights)
+/* table_row != NULL is the hash router (moe.c:539-559): the selection comes from the token's
+ * row of expert ordinals and the bias plays no part. */
+static int route_one(const float *logits, const float *bias, const int32_t *table_row,
+                     uint64_t experts, uint64_t topk, int scoring, int normalize, double scaling,
+                     float *scores_out, uint64_t *selected, float *weights)
 {
     float scores[256], biased[256];
     uint64_t e, rank, prior;
@@ -683,7 +685,11 @@ int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint
         biased[e] = (bias ? bias[e] : 0.0f) + scores[e];
         if (scores_out) scores_out[e] = scores[e];
     }
-    for (rank = 0; rank < topk; ++rank) { /* src/graph/moe.c:503-518 */
+    for (rank = 0; table_row && rank < topk; ++rank) {
+        if (table_row[rank] < 0 || (uint64_t)table_row[rank] >= experts) return YVO_ERR_FORMAT;
+        selected[rank] = (uint64_t)table_row[rank];
+    }
+    for (rank = 0; !table_row && rank < topk; ++rank) { /* src/graph/moe.c:503-518 */
         uint64_t best = UINT64_MAX;
         for (e = 0; e < experts; ++e) {
             int used = 0;
@@ -695,6 +701,8 @@ int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint
         selected[rank] = best;
     }
     for (rank = 0; rank < topk; ++rank) {
+        for (prior = 0; prior < rank; ++prior)       /* moe.c:561-566 */
+            if (selected[prior] == selected[rank]) return YVO_ERR_FORMAT;
         weights[rank] = scores[selected[rank]];
         total += weights[rank];
     }
@@ -706,6 +714,25 @@ int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint
         weights[rank] = (float)value;
     }
     return YVO_OK;
+}
+
+int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint64_t topk,
+                  int scoring, int normalize, double scaling, float *scores_out,
+                  uint64_t *selected, float *weights)
+{
+    return route_one(logits, bias, NULL, experts, topk, scoring, normalize, scaling, scores_out,
+                     selected, weights);
+}
+
+int yvo_moe_route_hash(const float *logits, const int32_t *table, uint64_t table_rows,
+                       uint64_t table_row_bytes, uint64_t token, uint64_t experts, uint64_t topk,
+                       int scoring, int normalize, double scaling, float *scores_out,
+                       uint64_t *selected, float *weights)
+{
+    if (!table || table_row_bytes < topk * 4u || (table_row_bytes & 3u)) return YVO_ERR_BOUNDS;
+    if (token >= table_rows) return YVO_ERR_BOUNDS;
+    return route_one(logits, NULL, table + token * (table_row_bytes / 4u), experts, topk, scoring,
+                     normalize, scaling, scores_out, selected, weights);
 }
 
 /* ---- expert FFN: src/graph/moe.c:587-622 ---- */
@@ -1059,8 +1086,9 @@ static void *layer_worker(void *opaque)
         const float *x = s->inputs + row * a->hidden;
         uint64_t *sel = s->selected + row * a->topk;
         float *w = s->weights + row * a->topk;
-        s->rc = yvo_moe_route(s->logits + row * a->experts, a->router_bias, a->experts, a->topk,
-                              a->scoring, a->normalize, a->scaling, NULL, sel, w);
+        s->rc = route_one(s->logits + row * a->experts, a->router_bias,
+                          a->hash_selected ? a->hash_selected + row * a->topk : NULL, a->experts,
+                          a->topk, a->scoring, a->normalize, a->scaling, NULL, sel, w);
         memset(routed, 0, sizeof(float) * a->hidden);
         for (rank = 0; rank < a->topk && s->rc == YVO_OK; ++rank) {
             uint64_t e = sel[rank];

@@ -138,6 +138,13 @@ int yvo_q8_matvec(unsigned int qtype, const uint8_t *encoded, uint64_t row_count
 int yvo_moe_route(const float *logits, const float *bias, uint64_t experts, uint64_t topk,
                   int scoring, int normalize, double scaling, float *scores,
                   uint64_t *selected, float *weights);
+/* Hash router (moe.c:539-559): the token's row of the I32 table names the experts; an ordinal
+ * outside the expert range or a repeated one is FORMAT, a token outside the table is BOUNDS.
+ * Pinned by tests/unit/runtime_moe.c:152-170 and a fixture from the compiled reference. */
+int yvo_moe_route_hash(const float *logits, const int32_t *table, uint64_t table_rows,
+                       uint64_t table_row_bytes, uint64_t token, uint64_t experts, uint64_t topk,
+                       int scoring, int normalize, double scaling, float *scores_out,
+                       uint64_t *selected, float *weights);
 
 /* Expert FFN: src/graph/moe.c:587-622. Weight matrices are encoded rows; gate/up are
  * [intermediate x hidden], down is [hidden x intermediate]. `intermediate_out` (may be NULL)
@@ -204,6 +211,7 @@ typedef struct {
     int scoring, normalize, act_q8;
     double scaling, activation_limit;
     unsigned int threads;
+    const int32_t *hash_selected;   /* [rows][topk] expert ordinals of the hash router, or NULL */
 } yvo_moe_layer_args;
 int yvo_moe_layer(const yvo_moe_layer_args *args, const float *inputs, const float *logits,
                   uint64_t *selected, float *weights, float *routed, float *shared,

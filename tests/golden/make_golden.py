@@ -127,6 +127,23 @@ def main():
     out["route_bias"] = bias
     out["route_selected"] = np.array(sel, np.uint64)
     out["route_weights_bits"] = np.array(wts, np.float32).view(np.uint32)
+    # hash router: the token's row of an I32 table names the experts (same job, same logits)
+    table = np.stack([np.random.default_rng(t).permutation(experts)[:topk] for t in range(8)]).astype(np.int32)
+    plan.router_class, plan.hash_table_rows, plan.hash_table_columns = abi.ROUTER_HASH, 8, topk
+    job.weights[abi.W_ROUTER_TABLE] = weight_view(table.view(np.uint8), 26, topk, 8)
+    job.token_id_present = 1
+    hash_sel, hash_wts = [], []
+    for row, token in zip(xs, (3, 7, 0, 5, 2)):
+        result, err = RouterResult(), abi.Error()
+        job.token_id = token
+        assert ref.yvex_moe_route_cpu(C.byref(job), row.ctypes.data, C.byref(result), C.byref(err)) == 0
+        hash_sel.append(list(result.selected_experts)[:topk])
+        hash_wts.append(list(result.selected_weights)[:topk])
+    out["route_hash_table"] = table
+    out["route_hash_tokens"] = np.array([3, 7, 0, 5, 2], np.uint32)
+    out["route_hash_selected"] = np.array(hash_sel, np.uint64)
+    out["route_hash_weights_bits"] = np.array(hash_wts, np.float32).view(np.uint32)
+    plan.router_class = abi.ROUTER_LEARNED
     # expert FFN on IQ2_XXS and Q8_0 weights
     ref.yvex_moe_expert_cpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                         C.c_float, C.c_void_p, C.c_void_p]

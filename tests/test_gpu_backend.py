@@ -196,7 +196,7 @@ class MoeCase:
 
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
-                 shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20):
+                 shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0):
         self.b, self.oracle = b, oracle
         self.streams, self.iterations = streams, iterations
         expanded = hidden * max(streams, 1)
@@ -215,6 +215,12 @@ class MoeCase:
             "sup": g.weights(qt, intermediate, hidden),
             "sdown": g.weights(qt, hidden, intermediate),
         }
+        self.hash_vocab = hash_vocab
+        if hash_vocab:  # hash router: an I32 table of expert ordinals per token id
+            rng = np.random.default_rng(seed)
+            self.table = np.stack([rng.permutation(experts)[:topk] for _ in range(hash_vocab)]).astype(np.int32)
+            self.tokens = rng.integers(0, hash_vocab, rows).astype(np.uint32)
+            parts["table"] = self.table.view(np.uint8).ravel()
         if streams:     # residual-stream envelope: mixing function, scale, base (F32) and BF16 norm weights
             parts["function"] = g.normal(mixing * expanded, 0.05).view(np.uint8)
             parts["scale"] = g.normal(3, 0.7).view(np.uint8)
@@ -247,6 +253,8 @@ class MoeCase:
         p.expert_intermediate_width = p.shared_intermediate_width = intermediate
         p.routed_scaling_factor, p.activation_limit = 1.5, 10.0
         p.requires_correction_bias, p.normalize_topk_probabilities = int(bias), 1
+        if hash_vocab:
+            p.router_class, p.hash_table_rows, p.hash_table_columns = abi.ROUTER_HASH, hash_vocab, topk
         self.job = abi.LayerJob()
         self.job.layer = C.pointer(self.plan)
         rb_h, rb_i = oracle.row_bytes(qt, hidden), oracle.row_bytes(qt, intermediate)
@@ -266,6 +274,8 @@ class MoeCase:
         view(abi.W_SHARED_GATE, "sgate", qt, hidden, intermediate, rb_h)
         view(abi.W_SHARED_UP, "sup", qt, hidden, intermediate, rb_h)
         view(abi.W_SHARED_DOWN, "sdown", qt, intermediate, hidden, rb_i)
+        if hash_vocab:
+            view(abi.W_ROUTER_TABLE, "table", 26, topk, hash_vocab, topk * 4, abi.ACT_DEVICE_F32)
         if streams:
             view(abi.W_MHC_FUNCTION, "function", 0, expanded, mixing, expanded * 4, abi.ACT_DEVICE_F32)
             view(abi.W_MHC_SCALE, "scale", 0, 3, 1, 12, abi.ACT_DEVICE_F32)
@@ -281,6 +291,8 @@ class MoeCase:
         bt.schema_version, bt.row_count, bt.row_width, bt.row_stride = 1, rows, expanded, expanded
         bt.device_rows, bt.device_outputs = self.rows_in, self.rows_out
         bt.provenance, bt.execution_class = abi.BATCH_MULTI_SESSION, 1
+        if hash_vocab:
+            bt.token_ids, bt.token_ids_present = self.tokens.ctypes.data, 1
         self.sel = np.zeros(rows * topk, np.uint64)
         self.wts = np.zeros(rows * topk, np.float32)
         self.combined = np.zeros((rows, hidden), np.float32)
@@ -318,7 +330,8 @@ class MoeCase:
         want = o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
                            topk=self.topk, qtypes=(self.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
                            shared=shared, inputs=x, logits=logits, bias=bias, scoring=self.scoring,
-                           normalize=True, scaling=1.5, act_q8=act_q8, threads=8)
+                           normalize=True, scaling=1.5, act_q8=act_q8, threads=8,
+                           hash_selected=self.table[self.tokens] if self.hash_vocab else None)
         if ingress:
             want["normalized"], want["post"], want["combination"] = ingress
             rc, want["envelope"] = o.mhc_post(want["combined"], self.x, ingress[1], ingress[2],
@@ -397,6 +410,27 @@ def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, row
     assert case.result.completed == 1 and case.result.kernel_launches >= 14
 
 
+@pytest.mark.parametrize("streams", [0, 4])
+def test_execute_rows_hash_router(backend, oracle, streams):
+    """Hash-routed layers (the reference's first layers route by token id, src/graph/moe.c:539-559):
+    the selection is the token's table row, the rest of the layer is unchanged."""
+    case = MoeCase(backend, oracle, hidden=512, rows=6, streams=streams, iterations=4, hash_vocab=40)
+    backend.workspace(case.workspace_bytes)
+    assert case.execute() == 0, case.err.message
+    want = case.oracle_layer(act_q8=True)
+    assert np.array_equal(case.sel.reshape(6, case.topk), case.table[case.tokens])
+    assert np.array_equal(case.sel.reshape(6, case.topk), want["selected"])
+    assert np.max(np.abs(case.wts.reshape(6, case.topk) - want["weights"])) <= (1e-4 if streams else 1e-6)
+    err = np.abs(case.combined.astype(np.float64) - want["combined"])
+    outside = err > 1e-5 + 1e-3 * np.abs(want["combined"])
+    assert outside.mean() < 2e-2
+    assert np.all(err[outside] <= 2 * 2.0 ** -7 * np.abs(want["combined"][outside]) + 1e-4)
+    # a token outside the table refuses before anything runs; a repeated ordinal is caught on the device
+    case.tokens[2] = 40
+    assert case.execute() == abi.BOUNDS
+    case.tokens[2] = 1
+
+
 def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle):
     """Row batches whose buckets average eight pairs or more run the int8 matrix-core kernels
     (routed and shared expert); the result is the CPU layer's, to the same bar."""
@@ -460,7 +494,9 @@ def test_execute_rows_refusals(backend, oracle):
     case.plan.expanded_width = 2 * case.hidden
     assert case.execute() in (abi.UNSUPPORTED, abi.INVALID_ARG)
     case.plan.expanded_width = case.hidden
-    case.plan.router_class = abi.ROUTER_HASH
+    case.plan.router_class = abi.ROUTER_HASH          # no token ids, no table
+    assert case.execute() == abi.BOUNDS
+    case.plan.router_class = 7
     assert case.execute() == abi.UNSUPPORTED
     case.plan.router_class = abi.ROUTER_LEARNED
     # cancellation is polled before launch
@@ -658,6 +694,22 @@ def test_token_local_device_output_runs_selected_experts(backend, oracle):
     assert t.close() == 0
 
 
+def test_token_local_hash_router(backend, oracle):
+    case = MoeCase(backend, oracle, hidden=512, rows=3, streams=2, iterations=3, act=abi.ACT_DEVICE_F32,
+                   hash_vocab=16)
+    t = TokenLocal(case, row=1)
+    t.job.token_id, t.job.token_id_present = int(case.tokens[1]), 1
+    assert t.begin() == 0, t.err.message
+    assert list(t.result.router.selected_experts)[:case.topk] == list(case.table[case.tokens[1]])
+    rc, _, want_w, _ = oracle.moe_route_hash(
+        np.array(list(t.result.router.router_logits)[:case.experts], np.float32), case.table,
+        int(case.tokens[1]), case.topk, case.scoring, True, 1.5)
+    assert rc == 0 and np.max(np.abs(np.array(list(t.result.router.selected_weights)[:case.topk]) - want_w)) <= 1e-6
+    assert t.close() == 0
+    t.job.token_id = 16
+    assert t.begin() == abi.BOUNDS
+
+
 def test_token_local_refusals(backend, oracle):
     case = MoeCase(backend, oracle, hidden=512, rows=2, streams=2, iterations=2, act=abi.ACT_DEVICE_F32)
     t = TokenLocal(case)
@@ -667,7 +719,9 @@ def test_token_local_refusals(backend, oracle):
     case.plan.mhc_mixing_rows = 9
     assert t.begin() == abi.BOUNDS
     case.plan.mhc_mixing_rows = 8
-    case.plan.router_class = abi.ROUTER_HASH
+    case.plan.router_class = abi.ROUTER_HASH          # no token id
+    assert t.begin() == abi.BOUNDS
+    case.plan.router_class = 7
     assert t.begin() == abi.UNSUPPORTED
     case.plan.router_class = abi.ROUTER_LEARNED
     bad = t.row.copy()

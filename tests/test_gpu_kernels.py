@@ -153,6 +153,46 @@ def test_route_rows(gpu, oracle, scoring):
         assert np.max(np.abs(w[r] - ww)) <= 1e-6
 
 
+@pytest.mark.parametrize("scoring", [0, 1])
+def test_route_hash_rows(gpu, oracle, scoring):
+    """Hash router against the oracle (src/graph/moe.c:539-582): identical selection, weights to
+    1e-6; a repeated ordinal, an ordinal outside the experts and a token outside the table raise
+    the contract status."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(9, f"route.hash.{scoring}")
+    rows, experts, topk, vocab = 37, 256, 6, 50
+    logits = g.normal(rows * experts).reshape(rows, experts) * 2.0
+    rng = np.random.default_rng(2)
+    table = np.stack([rng.permutation(experts)[:8] for _ in range(vocab)]).astype(np.int32)   # 8 columns, 6 used
+    tokens = rng.integers(0, vocab, rows).astype(np.int32)
+    status = K.new_status(gpu)
+    sel, w = K.moe_route_hash_rows(dev(logits, gpu), dev(table, gpu), dev(tokens, gpu), topk, scoring, True, 1.5, status)
+    status_ok(status)
+    sel, w = sel.cpu().numpy(), w.cpu().numpy()
+    for r in range(rows):
+        rc, want_sel, want_w, _ = oracle.moe_route_hash(logits[r], table, int(tokens[r]), topk, scoring, True, 1.5)
+        assert rc == 0 and np.array_equal(sel[r], want_sel.astype(np.int64))
+        assert np.max(np.abs(w[r] - want_w)) <= 1e-6
+    # one row for every token
+    status = K.new_status(gpu)
+    sel1, _ = K.moe_route_hash_rows(dev(logits, gpu), dev(table[7:8], gpu), dev(tokens, gpu), topk, scoring, True,
+                                    1.5, status, table_rows=vocab)
+    status_ok(status)
+    assert np.all(sel1.cpu().numpy() == table[7, :topk])
+    for poison in ("repeat", "range", "token"):
+        t, ids = table.copy(), tokens.copy()
+        if poison == "repeat":
+            t[ids[5], 3] = t[ids[5], 1]
+        elif poison == "range":
+            t[ids[5], 2] = experts
+        else:
+            ids[5] = vocab
+        status = K.new_status(gpu)
+        K.moe_route_hash_rows(dev(logits, gpu), dev(t, gpu), dev(ids, gpu), topk, scoring, True, 1.5, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 2, poison
+
+
 @pytest.mark.parametrize("rows,topk,experts", [(32, 8, 256), (1, 6, 256), (61, 6, 256),
                                                (2048, 8, 256), (5, 2, 4)])
 def test_worklist_matches_stable_sort(gpu, oracle, rows, topk, experts):

@@ -341,6 +341,26 @@ def test_router_matches_reference_fixture(oracle, golden):
         assert np.array_equal(bits(w), golden["route_weights_bits"][r])
 
 
+def test_hash_router_reference_expectations_and_fixture(oracle, golden):
+    """tests/unit/runtime_moe.c:152-170: the token's table row is the selection, a repeated
+    ordinal refuses with FORMAT, a token outside the table with BOUNDS; then the fixture from the
+    compiled reference's yvex_moe_route_cpu, bit for bit."""
+    logits = np.array([1, 2, 2, 0], np.float32)
+    rc, sel, w, _ = oracle.moe_route_hash(logits, np.array([[3, 1]], np.int32), 0, 2, oracle.SQRT_SOFTPLUS, True, 1.5)
+    score = lambda v: math.sqrt(math.log1p(math.exp(v)) if v <= 0 else v + math.log1p(math.exp(-v)))
+    assert rc == 0 and list(sel) == [3, 1]
+    assert abs(w[0] - score(0.0) / (score(0.0) + score(2.0)) * 1.5) < 1e-6
+    assert oracle.moe_route_hash(logits, np.array([[3, 3]], np.int32), 0, 2, 0, True, 1.5)[0] == oracle.ERR_FORMAT
+    assert oracle.moe_route_hash(logits, np.array([[3, 4]], np.int32), 0, 2, 0, True, 1.5)[0] == oracle.ERR_FORMAT
+    assert oracle.moe_route_hash(logits, np.array([[-1, 2]], np.int32), 0, 2, 0, True, 1.5)[0] == oracle.ERR_FORMAT
+    assert oracle.moe_route_hash(logits, np.array([[3, 1]], np.int32), 1, 2, 0, True, 1.5)[0] == oracle.ERR_BOUNDS
+    for r, token in enumerate(golden["route_hash_tokens"]):
+        rc, sel, w, _ = oracle.moe_route_hash(golden["route_logits"][r], golden["route_hash_table"], int(token), 6,
+                                              oracle.SQRT_SOFTPLUS, True, 1.5)
+        assert rc == 0 and np.array_equal(sel, golden["route_hash_selected"][r])
+        assert np.array_equal(bits(w), golden["route_hash_weights_bits"][r])
+
+
 def test_sigmoid_scoring_closed_form(oracle):
     g = oracle.Generator(5, "sigmoid")
     logits = g.normal(256)

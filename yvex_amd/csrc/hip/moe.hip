@@ -100,6 +100,54 @@ __global__ __launch_bounds__(256) void route_rows_kernel(
     }
 }
 
+// Hash router (src/backend/cuda/moe_kernels.cu:222-245, src/graph/moe.c:539-582): a row's experts
+// are the first topk ordinals of its token's row of an I32 table; weights as for the learned
+// router. One wavefront per row, lane r holds rank r. An ordinal outside the expert range, a
+// repeated one or a token outside the table is a contract violation (status 2).
+__global__ __launch_bounds__(256) void route_hash_rows_kernel(
+    const float *__restrict__ logits, const unsigned char *__restrict__ table,
+    const unsigned *__restrict__ token_ids, unsigned long long rows, unsigned experts, unsigned topk,
+    unsigned long long table_rows, unsigned long long table_row_bytes, int single_row, int scoring,
+    int normalize, double scaling, unsigned long long *__restrict__ selected,
+    float *__restrict__ weights, int *status)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const unsigned long long token = token_ids[row];
+    if (token >= table_rows) {
+        if (lane == 0u) raise_status(status, 2);
+        return;
+    }
+    const int *ordinals = reinterpret_cast<const int *>(table + (single_row ? 0ull : token * table_row_bytes));
+    const int mine = lane < topk ? ordinals[lane] : -1;
+    const bool live = lane < topk;
+    bool bad = live && (mine < 0 || (unsigned)mine >= experts);
+    float score = 0.0f;
+    if (live && !bad) {
+        const double s = route_score((double)logits[row * experts + (unsigned)mine], scoring);
+        score = (float)s;
+        if (!(s == s) || !finite_f32(score)) raise_status(status, 1);
+    }
+    double total = 0.0;
+    for (unsigned rank = 0; rank < topk; ++rank) {
+        const int other = __shfl(mine, (int)rank, kWave);
+        bad |= live && rank < lane && other == mine;
+        total += (double)__shfl(score, (int)rank, kWave);      // rank order, in double
+    }
+    if (bad) raise_status(status, 2);
+    if (normalize && !(total > 0.0 && total < 1.0e300)) raise_status(status, 1);
+    if (live) {
+        double value = (double)score;
+        if (normalize) value /= total;
+        value *= scaling;
+        const float w = (float)value;
+        if (!finite_f32(w)) raise_status(status, 1);
+        weights[row * topk + lane] = w;
+        selected[row * topk + lane] = bad ? 0ull : (unsigned long long)mine;
+    }
+}
+
 // ---- worklist -------------------------------------------------------------------------------
 //
 // A row never routes to the same expert twice, so each expert's pairs are a set of rows: one bit
@@ -654,6 +702,28 @@ extern "C" int yvex_hip_moe_route_rows(const float *logits, const float *bias, u
         logits, bias, rows, (unsigned)experts, (unsigned)topk, scoring, normalize, scaling,
         (unsigned long long *)selected, weights, status);
     return check_launch("moe_route_rows");
+}
+
+extern "C" int yvex_hip_moe_route_hash_rows(const float *logits, const uint8_t *table,
+                                            const uint32_t *token_ids, uint64_t rows,
+                                            uint64_t experts, uint64_t topk, uint64_t table_rows,
+                                            uint64_t table_row_bytes, int single_row, int scoring,
+                                            int normalize,
+                                            double scaling, uint64_t *selected, float *weights,
+                                            int *status, yvex_hip_stream stream)
+{
+    if (!logits || !table || !token_ids || !selected || !weights || !status || !rows || !experts ||
+        experts > 256u || !topk || topk > 16u || topk > experts || !table_rows ||
+        ((uintptr_t)table & 3u) ||
+        (scoring != YVEX_HIP_SCORING_SQRT_SOFTPLUS && scoring != YVEX_HIP_SCORING_SIGMOID))
+        return ST_INVALID_ARG;
+    if (table_row_bytes < topk * 4u || (table_row_bytes & 3u)) return ST_BOUNDS;
+    const uint64_t grid = (rows + 3u) / 4u;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    route_hash_rows_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+        logits, table, token_ids, rows, (unsigned)experts, (unsigned)topk, table_rows, table_row_bytes,
+        single_row, scoring, normalize, scaling, (unsigned long long *)selected, weights, status);
+    return check_launch("moe_route_hash_rows");
 }
 
 extern "C" int yvex_hip_moe_route_scores(const float *logits, uint64_t count, int scoring,

@@ -31,6 +31,7 @@ typedef struct {
     unsigned long long shared_intermediate, shared_intermediate_q8, shared_outputs, routed;
     /* residual-stream envelope (layers whose plan names mixing rows) */
     unsigned long long mixes, scale, base, norm, normalized, post, combination, combined;
+    unsigned long long tokens;    /* hash router: the rows' token ids */
     unsigned long long total;
 } moe_ranges;
 
@@ -100,6 +101,7 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
         TAKE(combination, rows * streams * streams * sizeof(float));
         TAKE(combined, rows * hidden * sizeof(float));
     }
+    if (layer->router_class == YVEX_MOE_ROUTER_HASH_TOKEN_ID) TAKE(tokens, rows * sizeof(unsigned int));
 #undef TAKE
     r->total = cursor + ALIGN;   /* slack for aligning the workspace base itself */
     return 1;
@@ -276,7 +278,8 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     unsigned long long d2h = 0ull, started, counts[4] = {0};
     const void *activations;
     void *combined_target;
-    int envelope, unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
+    unsigned long long table_address = 0ull;
+    int envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
     if (result) memset(result, 0, sizeof(*result));
@@ -301,11 +304,12 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
                                 "width-N MoE owners, geometry or admitted width are invalid");
     envelope = moe_envelope(layer);
+    hash_router = layer->router_class == YVEX_MOE_ROUTER_HASH_TOKEN_ID;
     if ((!envelope && layer->expanded_width != layer->hidden_width) ||
-        layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE ||
+        (!hash_router && layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE) ||
         (layer->scoring != YVEX_MOE_SCORING_SQRT_SOFTPLUS && layer->scoring != YVEX_MOE_SCORING_SIGMOID))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
-                                "hash routing, other scoring policies and expanded rows without mixing rows are outside this backend");
+                                "other router classes, other scoring policies and expanded rows without mixing rows are outside this backend");
     if (envelope && !yvex_rocm_moe_envelope_geometry(layer))
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows",
                                 "residual-stream geometry is invalid");
@@ -328,6 +332,19 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         (envelope && output->combination_rows &&
          output->combination_capacity < row_count * streams * streams))
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows", "host output capacity is too small");
+    if (hash_router) {
+        /* src/graph/moe.c:539-549: one in-vocabulary token id per row, an I32 table */
+        const yvex_moe_weight_view *table = &views[YVEX_MOE_WEIGHT_ROUTER_TABLE];
+        unsigned long long r;
+        if (!rows->token_ids || !rows->token_ids_present || !layer->hash_table_rows ||
+            table->qtype != YVEX_GGUF_QTYPE_I32 || table->row_bytes < topk * 4ull || (table->row_bytes & 3ull))
+            return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows",
+                                    "MoE hash router requires one in-vocabulary token ID");
+        for (r = 0ull; r < row_count; ++r)
+            if (rows->token_ids[r] >= layer->hash_table_rows)
+                return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.rows",
+                                        "MoE hash router requires one in-vocabulary token ID");
+    }
     if (job->cancel_requested && job->cancel_requested(job->cancel_context))
         return yvex_rocm_refuse(err, YVEX_ERR_CANCELLED, "rocm.moe.rows",
                                 "width-N MoE was cancelled before launch");
@@ -345,8 +362,15 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     if (rc != YVEX_OK) return rc;
     /* weights: router [experts x hidden], optional bias [1 x experts], expert-major matrices */
     rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER], hidden, experts, &router_address, err);
-    if (rc == YVEX_OK && layer->requires_correction_bias)
+    if (rc == YVEX_OK && !hash_router && layer->requires_correction_bias)
         rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER_BIAS], experts, 1ull, &bias_address, err);
+    if (rc == YVEX_OK && hash_router) {
+        const yvex_moe_weight_view *table = &views[YVEX_MOE_WEIGHT_ROUTER_TABLE];
+        rc = view_resolve(backend, table, table->row_width, table->row_count, &table_address, err);
+        if (rc == YVEX_OK && table->row_count != 1ull && table->row_count < layer->hash_table_rows)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                  "MoE hash table holds fewer rows than the plan names");
+    }
     if (rc == YVEX_OK)
         rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], hidden,
                           experts * layer->expert_intermediate_width, &addresses[0], err);
@@ -468,10 +492,25 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                            experts, hidden, views[YVEX_MOE_WEIGHT_ROUTER].row_bytes,
                            activations, 0, row_count, hidden, NULL, (float *)AT(logits),
                            experts, 0, (int *)status, stream), "rocm.moe.rows.router");
-    if (layer->requires_correction_bias)
+    if (hash_router) {
+        if (rc == YVEX_OK && yvex_hip_memcpy_h2d(AT(tokens), rows->token_ids, row_count * sizeof(unsigned int),
+                                                 stream) != 0)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.token-ids", yvex_hip_last_error());
+        LAUNCH(yvex_hip_moe_route_hash_rows((const float *)AT(logits), (const uint8_t *)(uintptr_t)table_address,
+                                            (const uint32_t *)AT(tokens), row_count, experts, topk,
+                                            layer->hash_table_rows,
+                                            views[YVEX_MOE_WEIGHT_ROUTER_TABLE].row_bytes,
+                                            views[YVEX_MOE_WEIGHT_ROUTER_TABLE].row_count == 1ull,
+                                            (int)layer->scoring, layer->normalize_topk_probabilities,
+                                            layer->routed_scaling_factor, (uint64_t *)AT(selected),
+                                            (float *)AT(weights), (int *)status, stream),
+               "rocm.moe.rows.route");
+    }
+    if (!hash_router && layer->requires_correction_bias)
         LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)bias_address, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype,
                                1ull, experts, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].row_bytes, NULL, 1ull,
                                (float *)AT(bias), (int *)status, stream), "rocm.moe.rows.bias");
+    if (!hash_router)
     LAUNCH(yvex_hip_moe_route_rows((const float *)AT(logits),
                                    layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
                                    row_count, experts, topk, (int)layer->scoring,

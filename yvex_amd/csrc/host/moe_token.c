@@ -26,7 +26,7 @@ struct yvex_backend_moe_execution {
     const yvex_moe_layer_job *job;
     void *block;
     unsigned long long expanded, mixes, scale, base, norm, normalized, post, combination;
-    unsigned long long logits, scores, bias, selected, weights, slot_weights;
+    unsigned long long logits, scores, bias, selected, weights, slot_weights, token;
     unsigned long long order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts;
     unsigned long long intermediate, pair_outputs, shared_output, routed, combined, staging;
     unsigned long long staging_bytes;
@@ -140,6 +140,7 @@ static int plan_ranges(yvex_backend_moe_execution *x, const yvex_moe_layer_plan 
     TAKE(selected, topk * sizeof(unsigned long long));
     TAKE(weights, topk * sizeof(float));
     TAKE(slot_weights, YVEX_MOE_MAX_SELECTED * sizeof(float));
+    TAKE(token, sizeof(unsigned int));
     TAKE(order, topk * sizeof(unsigned long long));
     TAKE(expert_ids, experts * sizeof(unsigned long long));
     TAKE(bucket_offsets, (experts + 1ull) * sizeof(unsigned long long));
@@ -218,7 +219,7 @@ static int prepare_input(yvex_backend_moe_execution *x, yvex_error *err)
     return rc;
 }
 
-/* src/backend/cuda/moe.c:416-514 (learned router only) */
+/* src/backend/cuda/moe.c:416-514 */
 static int route(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, yvex_error *err)
 {
     const yvex_moe_layer_job *job = x->job;
@@ -229,6 +230,7 @@ static int route(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, y
     yvex_hip_stream stream = x->backend->stream;
     int *status = x->backend->device_status;
     int evidence = !job->device_output || job->evidence_level == YVEX_ATTENTION_EVIDENCE_FULL;
+    int hash_router = layer->router_class == YVEX_MOE_ROUTER_HASH_TOKEN_ID;
     int rc = weight_address(x, router, layer->hidden_width, experts, 0ull, &address,
                             "rocm.moe.router-projection", err);
     if (rc == YVEX_OK)
@@ -236,7 +238,7 @@ static int route(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, y
                                          layer->hidden_width, router->row_bytes, AT(normalized), 0, 1ull,
                                          layer->hidden_width, NULL, (float *)AT(logits), experts, 0,
                                          status, stream), "rocm.moe.router-projection", err);
-    if (rc == YVEX_OK && layer->requires_correction_bias) {
+    if (rc == YVEX_OK && !hash_router && layer->requires_correction_bias) {
         if (!flat_qtype(bias->qtype))
             return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.router-bias",
                                     "router bias cannot be decoded");
@@ -250,7 +252,30 @@ static int route(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, y
         rc = launched(x, yvex_hip_moe_route_scores((const float *)AT(logits), experts, (int)layer->scoring,
                                                    (float *)AT(scores), status, stream),
                       "rocm.moe.scores", err);
-    if (rc == YVEX_OK)
+    if (rc == YVEX_OK && hash_router) {
+        /* src/graph/moe.c:539-549 and moe.c:437-456 of the CUDA backend: the token's table row */
+        const yvex_moe_weight_view *table = &job->weights[YVEX_MOE_WEIGHT_ROUTER_TABLE];
+        unsigned int token = job->token_id;
+        if (!job->token_id_present || token >= layer->hash_table_rows || table->qtype != YVEX_GGUF_QTYPE_I32 ||
+            table->row_bytes < topk * 4ull || (table->row_bytes & 3ull) ||
+            (table->row_count != 1ull && table->row_count < layer->hash_table_rows))
+            return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.route",
+                                    "MoE hash router requires one in-vocabulary token ID");
+        rc = weight_address(x, table, table->row_width, table->row_count, 0ull, &address,
+                            "rocm.moe.hash-table", err);
+        if (rc == YVEX_OK) rc = upload(x, AT(token), &token, sizeof(token), "rocm.moe.hash-row", err);
+        if (rc == YVEX_OK)
+            rc = launched(x, yvex_hip_moe_route_hash_rows((const float *)AT(logits),
+                                                          (const uint8_t *)(uintptr_t)address,
+                                                          (const uint32_t *)AT(token), 1ull, experts, topk,
+                                                          layer->hash_table_rows, table->row_bytes,
+                                                          table->row_count == 1ull, (int)layer->scoring,
+                                                          layer->normalize_topk_probabilities,
+                                                          layer->routed_scaling_factor,
+                                                          (uint64_t *)AT(selected), (float *)AT(weights),
+                                                          status, stream), "rocm.moe.route", err);
+    }
+    if (rc == YVEX_OK && !hash_router)
         rc = launched(x, yvex_hip_moe_route_rows((const float *)AT(logits),
                                                  layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
                                                  1ull, experts, topk, (int)layer->scoring,
@@ -386,10 +411,11 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
         layer->expert_intermediate_width > (1ull << 20) || layer->shared_intermediate_width > (1ull << 20))
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.begin",
                                 "MoE layer geometry is outside this backend's bounds");
-    if (layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE ||
+    if ((layer->router_class != YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE &&
+         layer->router_class != YVEX_MOE_ROUTER_HASH_TOKEN_ID) ||
         (layer->scoring != YVEX_MOE_SCORING_SQRT_SOFTPLUS && layer->scoring != YVEX_MOE_SCORING_SIGMOID))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.begin",
-                                "hash routing and other scoring policies are outside this backend");
+                                "other router classes and scoring policies are outside this backend");
     if (!(layer->activation_limit > 0.0) || !isfinite(layer->activation_limit) ||
         !isfinite(layer->routed_scaling_factor))
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.begin",

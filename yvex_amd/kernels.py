@@ -132,6 +132,19 @@ def argmax_f32(values, status, out=None, scratch=None):
     return tokens, best, ties
 
 
+def moe_route_hash_rows(logits, table, token_ids, topk, scoring, normalize, scaling, status, table_rows=None):
+    """Hash router: table is an int32 [rows, columns] tensor, token_ids int32 [n]."""
+    rows, experts = logits.shape
+    selected = torch.zeros((rows, topk), dtype=torch.int64, device=logits.device)
+    weights = torch.zeros((rows, topk), dtype=torch.float32, device=logits.device)
+    single = table.shape[0] == 1 and table_rows is not None
+    _call("yvex_hip_moe_route_hash_rows", _ptr(logits), _ptr(table), _ptr(token_ids), C.c_uint64(rows),
+          C.c_uint64(experts), C.c_uint64(topk), C.c_uint64(table_rows or table.shape[0]),
+          C.c_uint64(table.shape[1] * 4), C.c_int(int(single)), C.c_int(scoring), C.c_int(int(normalize)),
+          C.c_double(scaling), _ptr(selected), _ptr(weights), _ptr(status), _stream())
+    return selected, weights
+
+
 def mhc_ingress(rows, mixes, scale, base, norm, *, streams, width, iterations, rms_epsilon,
                 mhc_epsilon, post_multiplier, status, out=None):
     """Residual-stream ingress + weighted RMS norm: (normalized [n, width], post [n, streams],
