@@ -307,8 +307,10 @@ typedef struct yvex_backend_rocm_operation_facts {
  * Refusals: activation_q8 not 0/1 -> INVALID_ARG; qtype unknown, removed, outside the baseline
  * or without device compute -> UNSUPPORTED (on the host, before any launch); geometry, byte
  * count, ownership, unwritten input, additive aliasing output, resident MISS -> FORMAT; kernels
- * absent -> UNSUPPORTED; non-finite numerics seen on device -> FORMAT. input_tail /
- * input_head_width (the reference's split input for speculation) must be NULL / 0 here. */
+ * absent -> UNSUPPORTED; non-finite numerics seen on device -> FORMAT. With input_tail the rows
+ * are split (the reference's speculation path, qtype.c:256-281, kernels.cu:736-782): row r is
+ * input[r, 0..input_head_width) followed by input_tail[r, ...], every value rounded to bf16, the
+ * Q8 activation policy is ignored, and the attached workspace must hold rows * width floats. */
 int yvex_backend_rocm_encoded_matvec(
     yvex_backend *backend, const unsigned char *resident_encoded,
     unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,

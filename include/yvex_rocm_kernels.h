@@ -55,6 +55,13 @@ int yvex_hip_block_dots_i32(const uint8_t *encoded, unsigned int qtype, uint64_t
                             uint64_t input_rows, int32_t *sums, int *status,
                             yvex_hip_stream stream);
 
+/* The activation side of yvex_qtype_split_matvec (kernels.cu:736-782): out[row] = bf16 values of
+ * head[row, 0..head_width) followed by tail[row, 0..tail_width), so that the split projection is
+ * the ordinary F32-activation projection over out. Non-finite values raise status 1. */
+int yvex_hip_concat_rows_bf16(const float *head, const float *tail, uint64_t rows,
+                              uint64_t head_width, uint64_t tail_width, float *out, int *status,
+                              yvex_hip_stream stream);
+
 /* Replaces yvex_argmax_f32 (kernels.cu:59-110): for each of row_count (<= 65535) rows of
  * row_width (< 2^32) F32 values the largest value, the lowest index holding it and the number of
  * elements holding it. A non-finite element raises status 1 and its row publishes nothing.

@@ -97,6 +97,38 @@ def test_encoded_matvec_additive_and_refusals_on_device(backend, oracle):
     assert run_matvec(b, host, w, 16, rows, width, xt, out, 1, 0)[0] == 0
 
 
+def test_encoded_matvec_split_input(backend, oracle):
+    """The reference's split projection (speculation: src/backend/cuda/qtype.c:256-281,
+    kernels.cu:736-782): a row is head ++ tail, every value rounded to bf16, F32 activations even
+    when the Q8 policy is asked for."""
+    b = backend
+    rows, width, head_width, in_rows = 48, 1024, 384, 3
+    g = oracle.Generator(8, "backend.split")
+    w = g.weights(oracle.Q8_0, rows, width)
+    _, host = b.resident(w)
+    x = g.normal(in_rows * width).reshape(in_rows, width)
+    head, tail = b.f32(x[:, :head_width]), b.f32(x[:, head_width:])
+    out = b.empty_f32(in_rows * rows)
+    facts, err = abi.OperationFacts(), abi.Error()
+
+    def run(tail_tensor, head_w, q8=0):
+        return b.lib.yvex_backend_rocm_encoded_matvec(
+            b.handle, host, w.nbytes, oracle.Q8_0, rows, width, w.nbytes // rows, in_rows, head, tail_tensor,
+            head_w, None, out, q8, C.byref(facts), C.byref(err))
+
+    assert run(tail, head_width) == abi.NOMEM                   # needs the workspace for the joined rows
+    b.workspace(in_rows * width * 4 + 256)
+    bits = x.view(np.uint32)
+    rounded = ((bits + 0x7fff + ((bits >> 16) & 1)) & 0xffff0000).view(np.float32)
+    want = oracle.matvec(oracle.Q8_0, w, rows, width, rounded)
+    for q8 in (0, 1):
+        assert run(tail, head_width, q8) == 0, err.message
+        got = b.read_f32(out, in_rows * rows).reshape(in_rows, rows)
+        assert close_to(got, want) and facts.kernel_launches == 3
+    assert run(tail, 0) == abi.FORMAT and run(None, head_width) == abi.FORMAT
+    assert run(tail, width) == abi.FORMAT and run(out, head_width) == abi.FORMAT
+
+
 def test_launch_and_sync_failure_seams(backend, oracle, monkeypatch):
     b = backend
     rows, width = 8, 256

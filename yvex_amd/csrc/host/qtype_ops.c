@@ -52,26 +52,34 @@ int yvex_backend_rocm_encoded_matvec(
     const char *where = "rocm.encoded-matvec";
     unsigned long long device_address = 0ull, input_bytes, output_bytes, activation_bytes;
     unsigned long long total_bytes, q8_bytes = 0ull, q8_address = 0ull, launches = 0ull;
-    int q8_path, device_status = 0, rc;
+    unsigned long long head_bytes, tail_bytes = 0ull, joined_bytes = 0ull, joined_address = 0ull;
+    const void *activations;
+    int q8_path, device_status = 0, rc, split_input = input_tail != NULL;
     if (facts) memset(facts, 0, sizeof(*facts));
     if (activation_q8 != 0 && activation_q8 != 1)
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.encoded-matvec.activation",
                                 "activation Q8 policy must be explicitly disabled or enabled");
-    if (input_tail || input_head_width)
-        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                                "split head/tail input is not part of this backend");
+    /* split input (speculation): row = head[0..input_head_width) ++ tail, qtype.c:256-281 */
     if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !resident_encoded || !encoded_bytes ||
-        !row_count || !input_rows || !row_width || !row_bytes || !facts || !input || !output)
+        !row_count || !input_rows || !row_width || !row_bytes || !facts || !input || !output ||
+        split_input != (input_head_width != 0ull) || (split_input && input_head_width >= row_width))
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, where,
                                 "resident encoded matvec geometry or ownership is incompatible");
     rc = qtype_admit(qtype, row_width, row_bytes, where, err);
     if (rc != YVEX_OK) return rc;
-    if (!mul_u64(input_rows, row_width, &input_bytes) || !mul_u64(input_bytes, sizeof(float), &input_bytes) ||
+    if (!mul_u64(input_rows, split_input ? input_head_width : row_width, &head_bytes) ||
+        !mul_u64(head_bytes, sizeof(float), &head_bytes) ||
+        (split_input && (!mul_u64(input_rows, row_width - input_head_width, &tail_bytes) ||
+                         !mul_u64(tail_bytes, sizeof(float), &tail_bytes))) ||
+        !mul_u64(input_rows, row_width, &input_bytes) || !mul_u64(input_bytes, sizeof(float), &input_bytes) ||
         !mul_u64(input_rows, row_count, &output_bytes) ||
         !mul_u64(output_bytes, sizeof(float), &output_bytes) ||
         !mul_u64(row_count, row_bytes, &total_bytes) || total_bytes != encoded_bytes ||
         !yvex_rocm_tensor_owner_is(backend, input) || !input->is_written ||
-        input->dtype != YVEX_DTYPE_F32 || input->bytes < input_bytes ||
+        input->dtype != YVEX_DTYPE_F32 || input->bytes < head_bytes ||
+        (split_input && (!yvex_rocm_tensor_owner_is(backend, input_tail) || !input_tail->is_written ||
+                         input_tail->dtype != YVEX_DTYPE_F32 || input_tail->bytes < tail_bytes ||
+                         input_tail == output)) ||
         !yvex_rocm_tensor_owner_is(backend, output) || output->dtype != YVEX_DTYPE_F32 ||
         output->bytes < output_bytes || output == input ||
         (additive && (!yvex_rocm_tensor_owner_is(backend, additive) ||
@@ -81,7 +89,7 @@ int yvex_backend_rocm_encoded_matvec(
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, where,
                                 "resident encoded matvec geometry or ownership is incompatible");
     activation_bytes = input_bytes + output_bytes + (additive ? output_bytes : 0ull);
-    q8_path = activation_q8 && row_width % 256ull == 0ull && q8_eligible(qtype);
+    q8_path = activation_q8 && !split_input && row_width % 256ull == 0ull && q8_eligible(qtype);
     output->is_written = 0;
     rc = yvex_rocm_require_kernels(backend, where, err);
     if (rc != YVEX_OK) return rc;
@@ -93,10 +101,26 @@ int yvex_backend_rocm_encoded_matvec(
             return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                     "Q8 activation needs an attached workspace of rows * width/256 * 292 bytes");
     }
+    if (split_input) {
+        joined_bytes = input_bytes;
+        if (!yvex_backend_workspace_acquire(backend, joined_bytes, 256ull, &joined_address))
+            return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
+                                    "a split input needs an attached workspace of rows * width * 4 bytes");
+    }
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.encoded-matvec.launch",
                                 "kernel launch failed (test seam)");
     rc = yvex_rocm_status_reset(backend, where, err);
+    activations = input->data;
+    if (rc == YVEX_OK && split_input) {
+        rc = yvex_rocm_launch_result(
+            yvex_hip_concat_rows_bf16((const float *)input->data, (const float *)input_tail->data, input_rows,
+                                      input_head_width, row_width - input_head_width,
+                                      (float *)(uintptr_t)joined_address, backend->device_status,
+                                      backend->stream), "rocm.encoded-matvec.split", err);
+        if (rc == YVEX_OK) launches++;
+        activations = (const void *)(uintptr_t)joined_address;
+    }
     if (rc == YVEX_OK && q8_path) {
         rc = yvex_rocm_launch_result(
             yvex_hip_q8k_quantize((const float *)input->data, input_rows, row_width, row_width,
@@ -108,7 +132,7 @@ int yvex_backend_rocm_encoded_matvec(
     if (rc == YVEX_OK) {
         rc = yvex_rocm_launch_result(
             yvex_hip_matvec((const uint8_t *)(uintptr_t)device_address, qtype, row_count, row_width,
-                            row_bytes, q8_path ? (const void *)(uintptr_t)q8_address : (const void *)input->data,
+                            row_bytes, q8_path ? (const void *)(uintptr_t)q8_address : activations,
                             q8_path, input_rows, row_width, additive ? (const float *)additive->data : NULL,
                             (float *)output->data, row_count, 0, backend->device_status, backend->stream),
             "rocm.encoded-matvec.launch", err);
@@ -126,7 +150,7 @@ int yvex_backend_rocm_encoded_matvec(
     facts->stream_synchronizations = 1ull;
     facts->active_weight_bytes = encoded_bytes;
     facts->activation_bytes = activation_bytes;
-    facts->temporary_bytes = sizeof(int) + q8_bytes;
+    facts->temporary_bytes = sizeof(int) + q8_bytes + joined_bytes;
     facts->compulsory_memory_facts_available = 1;
     yvex_error_clear(err);
     return YVEX_OK;
