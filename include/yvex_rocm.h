@@ -343,6 +343,17 @@ int yvex_backend_rocm_select_greedy_rows(
     unsigned long long row_width, unsigned int *selected_tokens, float *selected_values,
     unsigned long long *tie_counts, yvex_backend_rocm_operation_facts *facts, yvex_error *err);
 
+/* The qtype parity probe, yvex_cuda_quant_row_dot (src/backend/cuda/qtype.c:523-700): one encoded
+ * row (host bytes) times one vector (host floats), computed on the device by one thread in double
+ * precision in element order, as src/backend/cuda/kernels.cu:112-124 does, so it equals the CPU
+ * row dot wherever the decoders agree. Refusals: missing or misaligned arguments INVALID_ARG,
+ * qtype without device compute UNSUPPORTED, elements not a whole number of blocks or a byte count
+ * that disagrees BOUNDS, kernels absent UNSUPPORTED. failure is accepted for call compatibility
+ * and left untouched (the reference's record belongs to its quantization pipeline). */
+int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const unsigned char *encoded,
+                            size_t encoded_bytes, const float *vector, unsigned long long elements,
+                            float *out, void *failure, yvex_error *err);
+
 /* ---- MoE row batch: include/yvex/internal/moe.h ------------------------------------------- */
 
 #define YVEX_SHA256_HEX_CAP 65u

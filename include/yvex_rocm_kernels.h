@@ -55,6 +55,11 @@ int yvex_hip_block_dots_i32(const uint8_t *encoded, unsigned int qtype, uint64_t
                             uint64_t input_rows, int32_t *sums, int *status,
                             yvex_hip_stream stream);
 
+/* Replaces yvex_qtype_row_dot (kernels.cu:112-124): out[0] = float(sum over i in order of
+ * double(decode(i)) * double(vector[i])), one thread. */
+int yvex_hip_row_dot(const uint8_t *encoded, unsigned int qtype, const float *vector,
+                     uint64_t elements, float *out, yvex_hip_stream stream);
+
 /* The activation side of yvex_qtype_split_matvec (kernels.cu:736-782): out[row] = bf16 values of
  * head[row, 0..head_width) followed by tail[row, 0..tail_width), so that the split projection is
  * the ordinary F32-activation projection over out. Non-finite values raise status 1. */

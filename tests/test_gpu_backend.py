@@ -97,6 +97,42 @@ def test_encoded_matvec_additive_and_refusals_on_device(backend, oracle):
     assert run_matvec(b, host, w, 16, rows, width, xt, out, 1, 0)[0] == 0
 
 
+@pytest.mark.parametrize("qtype,elements", [("Q8_0", 4096), ("IQ2_XXS", 2048), ("Q4_K", 1024), ("Q2_K", 512),
+                                            ("F32", 333), ("BF16", 77)])
+def test_quant_row_dot_probe(backend, oracle, qtype, elements):
+    """The serial device row dot against the CPU row dot: the reference's bar is
+    1e-6 * (1 + |cpu|) (tests/unit/cuda/quant_qtype.c:118-120); the same order and arithmetic
+    give the same bits here."""
+    qt = {"BF16": 30}.get(qtype) or getattr(oracle, qtype)
+    g = oracle.Generator(4, f"probe.{qtype}")
+    if qtype == "BF16":
+        row = (g.normal(elements).view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        decoded = (row.view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    else:
+        row = g.weights(qt, 1, elements)
+    x = g.normal(elements)
+    out, err = C.c_float(), abi.Error()
+    rc = backend.lib.yvex_rocm_quant_row_dot(backend.handle, qt, row.ctypes.data, row.nbytes, x.ctypes.data,
+                                             elements, C.byref(out), None, C.byref(err))
+    assert rc == 0, err.message
+    if qtype == "BF16":
+        want = np.float32(np.sum(decoded.astype(np.float64) * x.astype(np.float64)))
+        assert abs(out.value - want) <= 1e-6 * (1 + abs(want))
+    elif qtype == "Q4_K":       # outside the reference's CPU path: the oracle's float decode, double sum
+        want = np.float32(np.sum(oracle.decode_rows(qt, row, elements)[0].astype(np.float64) * x.astype(np.float64)))
+        assert abs(out.value - want) <= 1e-6 * (1 + abs(want))
+    else:
+        rc, want = oracle.cpu_dot(qt, row, x)
+        assert rc == 0 and np.float32(out.value).view(np.uint32) == np.float32(want).view(np.uint32)
+    lib, h = backend.lib, backend.handle
+    assert lib.yvex_rocm_quant_row_dot(h, 2, row.ctypes.data, row.nbytes, x.ctypes.data, elements, C.byref(out),
+                                       None, C.byref(err)) == abi.UNSUPPORTED
+    assert lib.yvex_rocm_quant_row_dot(h, qt, row.ctypes.data, row.nbytes + 2, x.ctypes.data, elements,
+                                       C.byref(out), None, C.byref(err)) == abi.BOUNDS
+    assert lib.yvex_rocm_quant_row_dot(h, qt, None, row.nbytes, x.ctypes.data, elements, C.byref(out), None,
+                                       C.byref(err)) == abi.INVALID_ARG
+
+
 def test_encoded_matvec_split_input(backend, oracle):
     """The reference's split projection (speculation: src/backend/cuda/qtype.c:256-281,
     kernels.cu:736-782): a row is head ++ tail, every value rounded to bf16, F32 activations even

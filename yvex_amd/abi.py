@@ -250,7 +250,7 @@ EXPORTS = [
     "yvex_backend_resident_attach", "yvex_backend_resident_detach", "yvex_backend_resident_resolve",
     "yvex_backend_workspace_attach", "yvex_backend_workspace_detach",
     "yvex_backend_workspace_acquire", "yvex_backend_rocm_encoded_matvec",
-    "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows",
+    "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows", "yvex_rocm_quant_row_dot",
     "yvex_backend_moe_operations_get", "yvex_backend_moe_begin", "yvex_backend_moe_add_expert",
     "yvex_backend_moe_finish", "yvex_backend_moe_close",
     "yvex_expert_worklist_build",
@@ -260,7 +260,7 @@ EXPORTS = [
     "yvex_backend_rocm_gguf_resident_load", "yvex_backend_rocm_gguf_weight_view",
 ]
 KERNEL_EXPORTS = [
-    "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
+    "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_row_dot", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
     "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes",
     "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_moe_route_hash_rows", "yvex_hip_worklist_build", "yvex_hip_moe_up", "yvex_hip_moe_down",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
@@ -280,6 +280,8 @@ def library():
     lib.yvex_quant_numeric_capability_at.restype = C.POINTER(NumericCapability)
     lib.yvex_backend_moe_operations_get.restype = C.POINTER(MoeOperations)
     lib.yvex_backend_moe_operations_get.argtypes = [C.c_void_p]
+    lib.yvex_rocm_quant_row_dot.argtypes = [C.c_void_p, C.c_uint, C.c_void_p, C.c_size_t, C.c_void_p, ULL,
+                                            C.POINTER(C.c_float), C.c_void_p, C.POINTER(Error)]
     lib.yvex_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
     lib.yvex_gguf_close.argtypes = [C.c_void_p]
     lib.yvex_gguf_close.restype = None

@@ -205,6 +205,20 @@ __global__ __launch_bounds__(256) void block_dots_kernel(
     }
 }
 
+// Serial double-precision row dot by one thread, element by element: the parity probe of the
+// qtype decoders (src/backend/cuda/kernels.cu:112-124). Same order and arithmetic as the CPU row
+// dot, so the two agree to the last bit wherever the decoders do.
+__global__ void row_dot_serial_kernel(const unsigned char *__restrict__ encoded,
+                                      const float *__restrict__ vector, unsigned long long elements,
+                                      unsigned qtype, float *out)
+{
+    if (blockIdx.x != 0u || threadIdx.x != 0u) return;
+    double sum = 0.0;
+    for (unsigned long long index = 0; index < elements; ++index)
+        sum += (double)qtype_value(encoded, index, qtype) * (double)vector[index];
+    out[0] = (float)sum;
+}
+
 __global__ __launch_bounds__(256) void gather_kernel(
     const unsigned char *encoded, unsigned qtype, unsigned long long row_count,
     unsigned long long row_width, unsigned long long row_bytes, const unsigned *row_ids,
@@ -356,4 +370,15 @@ extern "C" int yvex_hip_gather(const uint8_t *encoded, unsigned int qtype, uint6
     gather_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
         encoded, qtype, row_count, row_width, row_bytes, row_ids, selected, out, status);
     return check_launch("gather");
+}
+
+extern "C" int yvex_hip_row_dot(const uint8_t *encoded, unsigned int qtype, const float *vector,
+                                uint64_t elements, float *out, yvex_hip_stream stream)
+{
+    unsigned block, bytes;
+    if (!encoded || !vector || !out || !elements) return ST_INVALID_ARG;
+    if (!qtype_geometry(qtype, block, bytes)) return ST_UNSUPPORTED;
+    if (elements % block) return ST_BOUNDS;
+    row_dot_serial_kernel<<<1, 1, 0, as_stream(stream)>>>(encoded, vector, elements, qtype, out);
+    return check_launch("row_dot");
 }

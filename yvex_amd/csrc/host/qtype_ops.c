@@ -220,3 +220,63 @@ int yvex_backend_rocm_encoded_gather(
     yvex_error_clear(err);
     return YVEX_OK;
 }
+
+/* src/backend/cuda/qtype.c:523-700: one encoded row times one vector, host pointers in, one float
+ * out, computed on the device by the serial double-precision probe kernel. The device
+ * temporaries live for the call only. */
+int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const unsigned char *encoded,
+                            size_t encoded_bytes, const float *vector, unsigned long long elements,
+                            float *out, void *failure, yvex_error *err)
+{
+    const char *where = "rocm.quant.row_dot";
+    const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(qtype);
+    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(qtype);
+    unsigned long long vector_bytes, weight_offset, total;
+    void *block = NULL;
+    int rc;
+    (void)failure;      /* the reference's failure record belongs to its quantization pipeline */
+    yvex_error_clear(err);
+    if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !encoded || !vector || !out || !elements ||
+        ((uintptr_t)vector & 3u) || ((uintptr_t)out & 3u) ||
+        ((qtype == YVEX_GGUF_QTYPE_F32 || qtype == YVEX_GGUF_QTYPE_I32) && ((uintptr_t)encoded & 3u)) ||
+        ((qtype == 1u || qtype == 30u) && ((uintptr_t)encoded & 1u)))
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, where,
+                                "encoded row, aligned vector/result, and backend are required");
+    if (!capability || !geometry || !capability->device_compute_available)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                                "qtype has no dedicated device numeric contract");
+    if (!geometry->block_size || elements % geometry->block_size)
+        return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, where,
+                                "qtype row does not satisfy canonical block geometry");
+    if (elements / geometry->block_size > ULLONG_MAX / geometry->bytes_per_block ||
+        elements / geometry->block_size * geometry->bytes_per_block != encoded_bytes ||
+        !mul_u64(elements, sizeof(float), &vector_bytes))
+        return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, where, "encoded row byte geometry is inconsistent");
+    rc = yvex_rocm_require_kernels(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    weight_offset = (vector_bytes + 255ull) & ~255ull;
+    total = weight_offset + ((encoded_bytes + 255ull) & ~255ull) + 256ull;
+    if (yvex_hip_malloc(&block, total) != 0)
+        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where, yvex_hip_last_error());
+    {
+        unsigned char *base = (unsigned char *)block;
+        float *device_out = (float *)(base + total - 256ull);
+        if (yvex_hip_memcpy_h2d(base, vector, vector_bytes, backend->stream) != 0 ||
+            yvex_hip_memcpy_h2d(base + weight_offset, encoded, encoded_bytes, backend->stream) != 0)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, where, yvex_hip_last_error());
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_launch_result(yvex_hip_row_dot(base + weight_offset, qtype, (const float *)base,
+                                                          elements, device_out, backend->stream),
+                                         "rocm.quant.row_dot.launch", err);
+        if (rc == YVEX_OK && yvex_hip_memcpy_d2h(out, device_out, sizeof(float), backend->stream) != 0)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, where, yvex_hip_last_error());
+    }
+    if (yvex_hip_free(block) != 0 && rc == YVEX_OK)
+        rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, where, "device temporary cleanup failed");
+    if (rc == YVEX_OK) {
+        backend->memory.h2d_bytes += vector_bytes + encoded_bytes;
+        backend->memory.d2h_bytes += sizeof(float);
+        yvex_error_clear(err);
+    }
+    return rc;
+}
