@@ -693,8 +693,9 @@ typedef struct {
  * begin: uploads job->expanded_input (or copies job->device_input), runs the residual-stream
  *   ingress and the router, and publishes result->router (logits and scores unless a device
  *   output is named and evidence is below FULL). When job->device_output is set, evidence is
- *   below FULL and the three routed matrices are resident, the selected experts run on the
- *   device at once and the caller adds the shared expert only.
+ *   below FULL and the three routed weight views carry a device_address, the selected experts
+ *   run on the device at once and the caller adds the shared expert only (the caller applies
+ *   the same rule, src/runtime/moe.c:654-660).
  * add_expert: intermediate = bf16(silu(min(g, L)) * clamp(u, +-L) * weight) with weight 1 for the
  *   shared expert, output = bf16(down . intermediate), kept for the rank-ordered sum (at most
  *   YVEX_MOE_MAX_SELECTED routed experts). Weight views outside the resident arena are uploaded

@@ -303,8 +303,8 @@ class MoeCase:
         arena = np.zeros(cursor, np.uint8)
         for name, blob in parts.items():
             arena[offsets[name]:offsets[name] + blob.nbytes] = blob
-        _, host = b.resident(arena)
-        self.host, self.offsets = host, offsets
+        arena_tensor, host = b.resident(arena)
+        self.host, self.offsets, self.arena_tensor = host, offsets, arena_tensor
         self.x = g.normal(rows * expanded).reshape(rows, expanded)
         if streams:
             bits = self.x.view(np.uint32)       # bf16 values, as the CPU path expects of its input
@@ -744,6 +744,8 @@ def test_token_local_device_output_runs_selected_experts(backend, oracle):
     finish writes the egress into the device output."""
     case = MoeCase(backend, oracle, qtype="IQ2_XXS", hidden=512, rows=3, streams=4, iterations=20,
                    act=abi.ACT_DEVICE_F32)
+    for slot, name in ((abi.W_ROUTED_GATE, "gate"), (abi.W_ROUTED_UP, "up"), (abi.W_ROUTED_DOWN, "down")):
+        case.job.weights[slot].device_address = case.arena_tensor.contents.data + case.offsets[name]
     t = TokenLocal(case, row=2, device=True)
     assert t.begin() == 0, t.err.message
     views, _ = t.expert_views(None)
@@ -760,6 +762,21 @@ def test_token_local_device_output_runs_selected_experts(backend, oracle):
     assert not t.combined.any()            # host copies are evidence, not published on this path
     assert t.result.expert_subviews_accessed == 3 * case.topk and t.result.device_to_device_bytes > 0
     assert t.close() == 0
+    # without device addresses on the routed views the caller adds the experts itself (the rule of
+    # src/runtime/moe.c:654-660), and the routing is published at begin
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN):
+        case.job.weights[slot].device_address = 0
+    u = TokenLocal(case, row=2, device=True)
+    assert u.begin() == 0, u.err.message
+    assert list(u.result.router.selected_experts)[:case.topk] == list(want["selected"][0])
+    for rank in range(case.topk):
+        views, _ = u.expert_views(int(u.result.router.selected_experts[rank]))
+        assert u.add(views, float(u.result.router.selected_weights[rank]), False) == 0, u.err.message
+    views, _ = u.expert_views(None)
+    assert u.add(views, 0.0, True) == 0 and u.finish() == 0, u.err.message
+    again = backend.read_f32(u.device_out, case.streams * case.hidden)
+    assert np.all(np.abs(again - got) <= 2.0 ** -6 * scale)
+    assert u.close() == 0
 
 
 def test_token_local_hash_router(backend, oracle):

@@ -431,17 +431,12 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
     x->backend = backend;
     x->job = job;
     x->started_ns = now_ns();
-    x->grouped_selected = job->device_output && job->evidence_level != YVEX_ATTENTION_EVIDENCE_FULL;
-    if (x->grouped_selected) {
-        unsigned long long address = 0ull;
-        int slot;
-        for (slot = YVEX_MOE_WEIGHT_ROUTED_GATE; slot <= YVEX_MOE_WEIGHT_ROUTED_DOWN; ++slot)
-            if (!job->weights[slot].device_address &&
-                (!job->weights[slot].encoded ||
-                 !yvex_rocm_resolve(backend, job->weights[slot].encoded, job->weights[slot].encoded_bytes,
-                                    &address)))
-                x->grouped_selected = 0;
-    }
+    /* the caller decides by the same rule whether it still has to add the routed experts
+     * (src/backend/cuda/moe.c:557-561, src/runtime/moe.c:654-660) */
+    x->grouped_selected = job->device_output && job->evidence_level != YVEX_ATTENTION_EVIDENCE_FULL &&
+                          job->weights[YVEX_MOE_WEIGHT_ROUTED_GATE].device_address &&
+                          job->weights[YVEX_MOE_WEIGHT_ROUTED_UP].device_address &&
+                          job->weights[YVEX_MOE_WEIGHT_ROUTED_DOWN].device_address;
     if (!plan_ranges(x, layer)) {
         free(x);
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.begin", "MoE range extent overflowed");
