@@ -247,11 +247,14 @@ static int tensor_storage(unsigned int qtype, const unsigned long long *dims, un
     return YVEX_OK;
 }
 
-static const yvex_gguf *sort_owner;
+typedef struct {
+    const char *name;
+    unsigned long long index;
+} named_index;
+
 static int by_name_compare(const void *a, const void *b)
 {
-    return strcmp(sort_owner->tensors[*(const unsigned long long *)a].name,
-                  sort_owner->tensors[*(const unsigned long long *)b].name);
+    return strcmp(((const named_index *)a)->name, ((const named_index *)b)->name);
 }
 
 static int parse_tensors(yvex_gguf *g, yvex_error *err)
@@ -295,8 +298,17 @@ static int parse_tensors(yvex_gguf *g, yvex_error *err)
         if (t->relative_offset % g->alignment)
             return fail(err, YVEX_ERR_FORMAT, "gguf.tensor.offset", "GGUF tensor relative offset is misaligned");
     }
-    sort_owner = g;
-    qsort(g->by_name, (size_t)g->tensor_count, sizeof(*g->by_name), by_name_compare);
+    {
+        named_index *order = (named_index *)calloc((size_t)(g->tensor_count ? g->tensor_count : 1ull), sizeof(*order));
+        if (!order) return fail(err, YVEX_ERR_NOMEM, "gguf.tensor", "out of host memory");
+        for (i = 0ull; i < g->tensor_count; ++i) {
+            order[i].name = g->tensors[i].name;
+            order[i].index = i;
+        }
+        qsort(order, (size_t)g->tensor_count, sizeof(*order), by_name_compare);
+        for (i = 0ull; i < g->tensor_count; ++i) g->by_name[i] = order[i].index;
+        free(order);
+    }
     for (i = 1ull; i < g->tensor_count; ++i)
         if (!strcmp(g->tensors[g->by_name[i - 1u]].name, g->tensors[g->by_name[i]].name))
             return fail(err, YVEX_ERR_FORMAT, "gguf.tensor.name", "duplicate GGUF tensor name");
