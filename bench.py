@@ -329,11 +329,11 @@ def main() -> int:
     def up_only():
         K.moe_up(layer.routed, acts, layer.act_q8, layer.weights, layer.worklist, pairs, TOPK,
                  EXPERTS, layer.limit, layer.intermediate_f32, layer.status, shared=layer.shared,
-                 shared_rows=ROWS, shared_intermediate=layer.shared_mid)
+                 shared_rows=ROWS, shared_intermediate=layer.last_shared_mid)
 
     def down_only():
         mid = layer.intermediate_q8 if layer.act_q8 else layer.intermediate_f32
-        smid = layer.shared_mid_q8 if layer.act_q8 else layer.shared_mid
+        smid = layer.last_shared_down_input
         K.moe_down(layer.routed, mid, layer.act_q8, layer.worklist, pairs, EXPERTS,
                    layer.pair_outputs, layer.status, shared=layer.shared, shared_rows=ROWS,
                    shared_intermediate=smid, shared_outputs=layer.shared_out)

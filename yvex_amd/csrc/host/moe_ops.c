@@ -32,6 +32,7 @@ typedef struct {
     /* residual-stream envelope (layers whose plan names mixing rows) */
     unsigned long long mixes, scale, base, norm, normalized, post, combination, combined;
     unsigned long long tokens;    /* hash router: the rows' token ids */
+    int joined_intermediates;     /* shared expert's intermediate rows follow the routed pairs' */
     unsigned long long total;
 } moe_ranges;
 
@@ -84,11 +85,26 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
     TAKE(bucket_populations, experts * sizeof(unsigned long long));
     TAKE(sweep_offsets, (experts + 1ull) * sizeof(unsigned long long));
     TAKE(counts, 4ull * sizeof(unsigned long long));
-    TAKE(intermediate, pairs * routed_i * sizeof(float));
-    TAKE(intermediate_q8, pairs * ((routed_i + 255ull) / 256ull) * 292ull);
+    /* With a shared expert of the routed width its intermediate rows are laid right behind the
+     * routed pairs' (F32 and Q8_K alike), so one launch quantizes both. Q8_K rows are read with
+     * 16-byte loads, which the offset must respect. */
+    r->joined_intermediates = shared_i == routed_i && routed_i % 256ull == 0ull &&
+                              (pairs * (routed_i / 256ull) * 292ull) % 16ull == 0ull &&
+                              (pairs * routed_i * sizeof(float)) % 16ull == 0ull;
+    if (r->joined_intermediates) {
+        TAKE(intermediate, (pairs + rows) * routed_i * sizeof(float));
+        TAKE(intermediate_q8, (pairs + rows) * (routed_i / 256ull) * 292ull);
+        r->shared_intermediate = r->intermediate + pairs * routed_i * sizeof(float);
+        r->shared_intermediate_q8 = r->intermediate_q8 + pairs * (routed_i / 256ull) * 292ull;
+    } else {
+        TAKE(intermediate, pairs * routed_i * sizeof(float));
+        TAKE(intermediate_q8, pairs * ((routed_i + 255ull) / 256ull) * 292ull);
+    }
     TAKE(pair_outputs, pairs * hidden * sizeof(float));
-    TAKE(shared_intermediate, rows * shared_i * sizeof(float));
-    TAKE(shared_intermediate_q8, rows * ((shared_i + 255ull) / 256ull) * 292ull);
+    if (!r->joined_intermediates) {
+        TAKE(shared_intermediate, rows * shared_i * sizeof(float));
+        TAKE(shared_intermediate_q8, rows * ((shared_i + 255ull) / 256ull) * 292ull);
+    }
     TAKE(shared_outputs, rows * hidden * sizeof(float));
     TAKE(routed, rows * hidden * sizeof(float));
     if (streams) {
@@ -551,11 +567,16 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull, 1ull,
                                layer->activation_limit, (float *)AT(shared_intermediate), NULL, 0ull, NULL,
                                (int *)status, stream), "rocm.moe.rows.shared-up");
-    if (routed_q8)
+    if (routed_q8 && has_shared && shared_q8 && ranges.joined_intermediates)
+        LAUNCH(yvex_hip_q8k_quantize((const float *)AT(intermediate), pairs + row_count,
+                                     layer->expert_intermediate_width, layer->expert_intermediate_width,
+                                     (uint8_t *)AT(intermediate_q8), (int *)status, stream),
+               "rocm.moe.rows.q8-mid");
+    else if (routed_q8)
         LAUNCH(yvex_hip_q8k_quantize((const float *)AT(intermediate), pairs, layer->expert_intermediate_width,
                                      layer->expert_intermediate_width, (uint8_t *)AT(intermediate_q8),
                                      (int *)status, stream), "rocm.moe.rows.q8-mid");
-    if (has_shared && shared_q8)
+    if (has_shared && shared_q8 && !(routed_q8 && ranges.joined_intermediates))
         LAUNCH(yvex_hip_q8k_quantize((const float *)AT(shared_intermediate), row_count,
                                      layer->shared_intermediate_width, layer->shared_intermediate_width,
                                      (uint8_t *)AT(shared_intermediate_q8), (int *)status, stream),

@@ -31,8 +31,10 @@ class MoeLayer:
         self.status = K.new_status(device)
         self.act_q8_rows = torch.empty(max_rows * (hidden // 256) * 292, **u8)
         self.worklist = K.Worklist(pairs, experts, device)
-        self.intermediate_f32 = torch.empty((pairs, intermediate), **f32)
-        self.intermediate_q8 = torch.empty(pairs * (intermediate // 256) * 292, **u8)
+        # the shared expert's intermediate rows sit right behind the routed pairs' (see run()), so
+        # one launch quantizes both
+        self.intermediate_f32 = torch.empty((pairs + max_rows, intermediate), **f32)
+        self.intermediate_q8 = torch.empty((pairs + max_rows) * (intermediate // 256) * 292, **u8)
         self.pair_outputs = torch.empty((pairs, hidden), **f32)
         self.shared_mid = torch.empty((max_rows, intermediate), **f32)
         self.shared_mid_q8 = torch.empty(max_rows * (intermediate // 256) * 292, **u8)
@@ -62,21 +64,29 @@ class MoeLayer:
         if self.matrix_cores:
             return self._run_rows(acts, rows, pairs)
         merged = self.shared is not None and self.merge_shared
+        row_q8 = (self.intermediate // 256) * 292
+        joined = self.shared is not None and self.act_q8 and (pairs * row_q8) % 16 == 0
+        shared_mid = self.intermediate_f32[pairs:pairs + rows] if joined else self.shared_mid
         K.moe_up(self.routed, acts, self.act_q8, self.weights, self.worklist, pairs, self.topk,
                  self.experts, self.limit, self.intermediate_f32, st,
                  shared=self.shared if merged else None, shared_rows=rows if merged else 0,
-                 shared_intermediate=self.shared_mid if merged else None)
+                 shared_intermediate=shared_mid if merged else None)
         if self.shared is not None and not merged:
             K.moe_up(self.shared, acts, self.act_q8, None, None, rows, 1, 1, self.limit,
-                     self.shared_mid, st)
+                     shared_mid, st)
         if self.act_q8:
-            K.q8k_quantize(self.intermediate_f32[:pairs], st, self.intermediate_q8)
             mid = self.intermediate_q8
-            if self.shared is not None:
-                K.q8k_quantize(self.shared_mid[:rows], st, self.shared_mid_q8)
-            smid = self.shared_mid_q8
+            if joined:
+                K.q8k_quantize(self.intermediate_f32[:pairs + rows], st, self.intermediate_q8)
+                smid = self.intermediate_q8[pairs * row_q8:]
+            else:
+                K.q8k_quantize(self.intermediate_f32[:pairs], st, self.intermediate_q8)
+                if self.shared is not None:
+                    K.q8k_quantize(shared_mid[:rows], st, self.shared_mid_q8)
+                smid = self.shared_mid_q8
         else:
-            mid, smid = self.intermediate_f32, self.shared_mid
+            mid, smid = self.intermediate_f32, shared_mid
+        self.last_shared_mid, self.last_shared_down_input = shared_mid, smid    # for stage-wise callers
         K.moe_down(self.routed, mid, self.act_q8, self.worklist, pairs, self.experts,
                    self.pair_outputs, st, shared=self.shared if merged else None,
                    shared_rows=rows if merged else 0, shared_intermediate=smid if merged else None,
