@@ -78,6 +78,58 @@ def cpu_baseline(sample_rows: int, threads: int):
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
 
 
+def cpu_baseline_reference(sample_rows: int):
+    """The same sample through the reference's own yvex_moe_expert_cpu, compiled from its sources
+    into oracle/_ref (single thread, as the reference runs it). None where that library is absent."""
+    import ctypes as C
+    import numpy as np
+    import oracle
+    from yvex_amd import abi
+    ref = oracle.ref_lib()
+    if ref is None:
+        return None
+    g = oracle.Generator(42, "bench.cpu")
+    experts = 16
+    gate = g.iq2xxs(experts * INTERMEDIATE * HIDDEN // 256)
+    up = g.iq2xxs(experts * INTERMEDIATE * HIDDEN // 256)
+    down = g.iq2xxs(experts * HIDDEN * INTERMEDIATE // 256)
+    shared = tuple(g.iq2xxs(INTERMEDIATE * HIDDEN // 256) for _ in range(3))
+    x = g.normal(sample_rows * HIDDEN).reshape(sample_rows, HIDDEN)
+    logits = g.normal(sample_rows * experts).reshape(sample_rows, experts)
+    plan = abi.LayerPlan()
+    plan.hidden_width, plan.activation_limit = HIDDEN, 10.0
+
+    def views(blobs, expert):
+        out = []
+        for blob, width, rows in zip(blobs, (HIDDEN, HIDDEN, INTERMEDIATE), (INTERMEDIATE, INTERMEDIATE, HIDDEN)):
+            v = abi.WeightView()
+            row_bytes = width // 256 * 66
+            v.qtype, v.row_width, v.row_count, v.row_bytes = oracle.IQ2_XXS, width, rows, row_bytes
+            v.encoded, v.encoded_bytes = blob.ctypes.data + expert * rows * row_bytes, rows * row_bytes
+            out.append(v)
+        return out
+
+    ref.yvex_moe_expert_cpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_float, C.c_void_p, C.c_void_p]
+    y, err = np.zeros(HIDDEN, np.float32), abi.Error()
+    t0 = time.perf_counter()
+    for row in range(sample_rows):
+        rc, selected, weights, _ = oracle.moe_route(logits[row], None, TOPK, oracle.SIGMOID, True, 1.0)
+        work = [(views((gate, up, down), int(e)), float(w)) for e, w in zip(selected, weights)]
+        work.append((views(shared, 0), 1.0))
+        for v, weight in work:
+            rc = ref.yvex_moe_expert_cpu(C.byref(plan), C.byref(v[0]), C.byref(v[1]), C.byref(v[2]),
+                                         x[row].ctypes.data, C.c_float(weight), y.ctypes.data, C.byref(err))
+            if rc != 0:
+                return None
+    seconds = time.perf_counter() - t0
+    touched = sample_rows * (TOPK + 1) * EXPERT_BYTES
+    return {"value": touched / seconds / 1e9, "unit": "GB/s", "cores": 1, "kind": "reference",
+            "sample": f"{sample_rows} rows x (top-8 + shared) expert FFNs of the same layer shape through "
+                      f"yvex_moe_expert_cpu of the reference, compiled from its own sources",
+            "tokens_per_s": sample_rows / seconds, "seconds": seconds}
+
+
 def dense_leg(torch, K, dev, repeats: int):
     """BASELINE configs 0-2 and an output head as single matvec launches: random packed bytes with
     small positive fp16 block scales, 32 distinct weight copies walked in turn (2 for the head) so
@@ -425,7 +477,11 @@ def main() -> int:
         torch.cuda.empty_cache()
         out["dense"] = dense_leg(torch, K, dev, 64)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_rows, 1)
+        port = cpu_baseline(args.cpu_rows, 1)
+        reference = cpu_baseline_reference(args.cpu_rows)
+        out["cpu_baseline"] = reference or port
+        if reference:
+            out["cpu_baseline_port"] = port
         out["cpu_baseline_all_cores"] = cpu_baseline(max(args.cpu_rows, 8), min(16, os.cpu_count() or 1))
     print(json.dumps(out))
     return 0
