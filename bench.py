@@ -28,7 +28,7 @@ MFMA_INT8_PEAK_TOPS = 5000.0
 HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
 EXPERT_BYTES = 3 * 3_784_704   # gate + up + down of one IQ2_XXS expert
 # iq2_sweep_kernel<fused>: FETCH_SIZE 632 787 x 2.000 KiB + WRITE_SIZE 15 782 x 1.000 KiB per launch
-GATE_UP_TRAFFIC_BYTES = int((631_890 * 2.0 + 14_310) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((580_550 * 2.0 + 13_604) * 1024)
 
 
 def synth_iq2xxs(torch, blocks: int, device, seed: int):
@@ -321,6 +321,8 @@ def main() -> int:
     ap.add_argument("--cpu-rows", type=int, default=4)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--alone", action="store_true",
+                    help="also time the two expert sweeps launched alone, back to back")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 1 GiB read kernel and a 256 MiB fill kernel, so a "
                          "counter run of this command holds kernels of known HBM traffic")
@@ -365,10 +367,18 @@ def main() -> int:
     sweeps = int(layer.worklist.counts[3].item())
 
     torch.cuda.synchronize()
+    layer.marks = []          # events around the two expert sweeps of every timed step
     t0 = time.perf_counter()
     step_ms_events = event_ms(torch, lambda: layer.run(x, logits), args.steps)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    marks, layer.marks = layer.marks, None
+
+    def in_step_ms(begin, end):
+        starts = [e for n, e in marks if n == begin]
+        stops = [e for n, e in marks if n == end]
+        spans = sorted(a.elapsed_time(b) for a, b in zip(starts, stops))
+        return sum(spans) / len(spans), spans[len(spans) // 2]
     eager_ms = max(step_ms_events, wall_ms)
     step_ms, launch_mode = eager_ms, "eager launches"
     # The step is eight short launches; replaying them from a captured graph takes the host's
@@ -427,8 +437,13 @@ def main() -> int:
                    layer.pair_outputs, layer.status, shared=layer.shared, shared_rows=ROWS,
                    shared_intermediate=smid, shared_outputs=layer.shared_out)
 
-    up_ms = event_ms(torch, up_only, max(10, args.steps))
-    down_ms = event_ms(torch, down_only, max(10, args.steps))
+    # Launch durations of the two sweeps: inside the timed steps (events before and after the
+    # launch on the launch stream; the first completes when the kernel before it has finished),
+    # and launched alone back to back for comparison.
+    up_ms, up_median_ms = in_step_ms("up_begin", "up_end")
+    down_ms, down_median_ms = in_step_ms("down_begin", "down_end")
+    up_alone_ms = event_ms(torch, up_only, max(10, args.steps)) if args.alone else None
+    down_alone_ms = event_ms(torch, down_only, max(10, args.steps)) if args.alone else None
     up_bytes = (unique + 1) * 2 * 3_784_704   # gate + up of every distinct routed expert and the shared one
     achieved = up_bytes / (up_ms * 1e-3) / 1e9
 
@@ -467,7 +482,10 @@ def main() -> int:
                      # copy kernels of known size in the same runs); null for other settings
                      "traffic": GATE_UP_TRAFFIC_BYTES if (args.act == "q8k" and unique == 158) else None,
                      "launch_ms": round(up_ms, 4), "algorithmic_bytes": up_bytes},
-        "kernels_ms": {"gate_up_sweep": round(up_ms, 4), "down_sweep": round(down_ms, 4)},
+        "kernels_ms": {"gate_up_sweep": round(up_ms, 4), "down_sweep": round(down_ms, 4),
+                       "gate_up_sweep_median": round(up_median_ms, 4), "down_sweep_median": round(down_median_ms, 4),
+                       "gate_up_sweep_alone": round(up_alone_ms, 4) if up_alone_ms else None,
+                       "down_sweep_alone": round(down_alone_ms, 4) if down_alone_ms else None},
     }
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,

@@ -140,7 +140,7 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
 
 // Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16
 // to 64 lanes of 128 columns each.
-bool iq2_sweep_supported(unsigned width, unsigned out_rows);
+bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs);
 int launch_iq2_sweep(const GroupedArgs &a, bool fused, hipStream_t stream);
 
 static inline bool same_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)

@@ -671,8 +671,10 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
         aligned = aligned && ((uintptr_t)pr.gate % 4u == 0u) && pr.expert_bytes % 4u == 0u &&
                   (!pr.up || ((uintptr_t)pr.up % 4u == 0u && pr.up_expert_bytes % 4u == 0u));
     }
+    unsigned long long all_pairs = 0ull;
+    for (unsigned i = 0; i < a.problems; ++i) all_pairs += a.problem[i].pairs;
     if (qtype == QT_IQ2_XXS && q8 && !generic_only && aligned &&
-        iq2_sweep_supported(a.width, a.out_rows))
+        iq2_sweep_supported(a.width, a.out_rows, all_pairs))
         return launch_iq2_sweep(a, fused, stream);
     switch (qtype) {
     case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);

@@ -50,7 +50,13 @@ constexpr unsigned kTicketAddress = kPrefixBase + 1056u;   // work-item counter 
 constexpr unsigned kParkBase = kPrefixBase + 1088u;
 constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave: 32 bytes per
                                                                       // (iteration, packed value), then one spare word per lane
-constexpr unsigned kSweepLdsBytes = kParkBase + kSweepWaves * kParkBytes;
+// Sweeps listed by the number of pairs they serve (4, 3, 2, 1): four class sizes, four class
+// starts (cursors while the list is built) and one word per sweep:
+// {whole problem is one bucket : 1, shared expert's problem : 1, bucket : 14, sweep of the bucket : 16}.
+constexpr unsigned kClassMaxSweeps = 4096u;
+constexpr unsigned kClassCountBase = kParkBase + kSweepWaves * kParkBytes;
+constexpr unsigned kClassListBase = kClassCountBase + 64u;
+constexpr unsigned kSweepLdsBytes = kClassListBase + kClassMaxSweeps * 4u;
 
 __device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
 {
@@ -509,16 +515,80 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     const unsigned long_rows = long_tiles * item_rows;
     const unsigned short_tiles = (a.out_rows - long_rows + short_rows - 1u) / short_rows;
 
-    // Work items are numbered with the shared expert's first (the heaviest: full sweeps), then the
-    // routed buckets in worklist order.
-    const GroupedProblem &extra = a.problem[a.problems > 1u ? 1u : 0u];
-    const unsigned extra_sweeps = a.problems > 1u
-        ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) : 0u;
-    const unsigned routed_sweeps = routed_fixed
-        ? (unsigned)((routed.pairs + kSweepPairs - 1u) / kSweepPairs)
-        : lds_load_u32(kPrefixBase + 4u * buckets);
-    const unsigned total_long = (extra_sweeps + routed_sweeps) * long_tiles;
-    const unsigned total_items = total_long + (extra_sweeps + routed_sweeps) * short_tiles;
+    // Work items: sweeps by class, the ones that serve four pairs first (the shared expert's are
+    // all of that kind), then three, two, one; inside a class sweep by sweep, each over its tiles
+    // (neighbouring items are neighbouring tiles of one expert). A sweep's cost grows with its
+    // pairs and workgroup b owns items b, b + grid, ...: listed by class every workgroup gets the
+    // same share of every kind.
+    unsigned all_sweeps;
+    {
+        const GroupedProblem &extra = a.problem[a.problems > 1u ? 1u : 0u];
+        const unsigned extra_sweeps = a.problems > 1u
+            ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) : 0u;
+        const unsigned routed_sweeps = routed_fixed
+            ? (unsigned)((routed.pairs + kSweepPairs - 1u) / kSweepPairs)
+            : lds_load_u32(kPrefixBase + 4u * buckets);
+        all_sweeps = extra_sweeps + routed_sweeps;
+        if (all_sweeps > kClassMaxSweeps) {          // the launch wrapper bounds the pairs
+            if (tid == 0u) raise_status(a.status, 2);
+            return;
+        }
+        // {pairs served, list word} of sweep s in bucket order (shared expert first)
+        auto describe = [&](unsigned s, unsigned &word) -> unsigned {
+            unsigned long long left;
+            if (s < extra_sweeps) {
+                left = extra.pairs - (unsigned long long)s * kSweepPairs;
+                word = 0xc0000000u | s;
+            } else {
+                const unsigned r = s - extra_sweeps;
+                unsigned low = 0u;
+                unsigned long long population = routed.pairs;
+                if (!routed_fixed) {
+                    unsigned high = buckets;   // last bucket whose first sweep is <= r
+                    while (low + 1u < high) {
+                        const unsigned middle = (low + high) >> 1;
+                        if (lds_load_u32(kPrefixBase + 4u * middle) <= r) low = middle;
+                        else high = middle;
+                    }
+                    population = routed.bucket_populations[low];
+                }
+                const unsigned k = r - (routed_fixed ? 0u : lds_load_u32(kPrefixBase + 4u * low));
+                left = population > (unsigned long long)k * kSweepPairs
+                    ? population - (unsigned long long)k * kSweepPairs : 1ull;
+                word = (routed_fixed ? 0x80000000u : 0u) | (low << 16) | (k & 0xffffu);
+            }
+            return left >= (unsigned long long)kSweepPairs ? (unsigned)kSweepPairs : (unsigned)left;
+        };
+        if (tid < 8u) lds_store_u32(kClassCountBase + 4u * tid, 0u);
+        __syncthreads();
+        for (unsigned s = tid; s < all_sweeps; s += kSweepThreads) {
+            unsigned word;
+            const unsigned n = describe(s, word);
+            __hip_atomic_fetch_add(reinterpret_cast<__attribute__((address_space(3))) unsigned *>(
+                                       kClassCountBase + 4u * (4u - n)), 1u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        __syncthreads();
+        if (tid == 0u) {
+            unsigned start = 0u;
+            for (unsigned c = 0; c < 4u; ++c) {
+                lds_store_u32(kClassCountBase + 16u + 4u * c, start);
+                start += lds_load_u32(kClassCountBase + 4u * c);
+            }
+        }
+        __syncthreads();
+        for (unsigned s = tid; s < all_sweeps; s += kSweepThreads) {
+            unsigned word;
+            const unsigned n = describe(s, word);
+            const unsigned at = __hip_atomic_fetch_add(
+                reinterpret_cast<__attribute__((address_space(3))) unsigned *>(kClassCountBase + 16u + 4u * (4u - n)),
+                1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            lds_store_u32(kClassListBase + 4u * at, word);
+        }
+        __syncthreads();
+    }
+    const unsigned total_long = all_sweeps * long_tiles;
+    const unsigned total_items = total_long + all_sweeps * short_tiles;
     // Workgroup b owns items b, b + grid, b + 2 grid, ...; its waves draw positions in that list
     // from a counter in LDS, so a wave that met light items takes more of them.
     auto draw = [&]() -> unsigned {
@@ -534,36 +604,34 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned item = is_short ? listed - total_long : listed;   // within its zone of rows
         const unsigned tiles = is_short ? short_tiles : long_tiles;
         const unsigned rows_of_item = is_short ? short_rows : item_rows;
-        const unsigned extra_items = extra_sweeps * tiles;
-        const bool is_extra = item < extra_items;
-        const GroupedProblem &pr = is_extra ? extra : routed;
-        const bool fixed = is_extra || routed_fixed;
-        unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
-        unsigned local = is_extra ? item : item - extra_items;
-        unsigned bucket_sweeps = is_extra ? extra_sweeps : routed_sweeps;
-        if (!fixed) {
-            unsigned low = 0u, high = buckets;   // last bucket whose first item is <= local
-            while (low + 1u < high) {
-                const unsigned middle = (low + high) >> 1;
-                if (lds_load_u32(kPrefixBase + 4u * middle) * tiles <= local) low = middle;
-                else high = middle;
+        // class of the item, then (sweep of the class list, tile)
+        unsigned start = 0u, size = 0u, position = item;
+        bool found = false;
+        for (unsigned c = 0; c < 4u && !found; ++c) {
+            size = lds_load_u32(kClassCountBase + 4u * c);
+            if (position < size * tiles) {
+                found = true;
+            } else {
+                position -= size * tiles;
+                start += size;
             }
-            const unsigned start = lds_load_u32(kPrefixBase + 4u * low);
-            expert = pr.expert_ids[low];
-            first = pr.bucket_offsets[low];
-            population = pr.bucket_populations[low];
-            local -= start * tiles;
-            bucket_sweeps = lds_load_u32(kPrefixBase + 4u * (low + 1u)) - start;
         }
-        if (bucket_sweeps == 0u) {
+        if (!found) {
             if (lane == 0u) raise_status(a.status, 2);
             continue;
         }
-        // the sweeps over one tile are neighbours: they stream the same bytes at the same time
-        const unsigned tile = local / bucket_sweeps;
-        const unsigned long long pass = (unsigned long long)(local % bucket_sweeps) * kSweepPairs;
-        if (expert >= pr.experts || first + population > pr.pairs || pass >= population ||
-            tile >= tiles) {
+        const unsigned tile = position % tiles;
+        const unsigned word = lds_load_u32(kClassListBase + 4u * (start + position / tiles));
+        const GroupedProblem &pr = a.problem[(word & 0x40000000u) && a.problems > 1u ? 1u : 0u];
+        unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
+        if (!(word & 0x80000000u)) {
+            const unsigned bucket = (word >> 16) & 0x3fffu;
+            expert = pr.expert_ids[bucket];
+            first = pr.bucket_offsets[bucket];
+            population = pr.bucket_populations[bucket];
+        }
+        const unsigned long long pass = (unsigned long long)(word & 0xffffu) * kSweepPairs;
+        if (expert >= pr.experts || first + population > pr.pairs || pass >= population) {
             if (lane == 0u) raise_status(a.status, 2);
             continue;
         }
@@ -598,8 +666,9 @@ static int sweep_grid()
     return units;
 }
 
-bool iq2_sweep_supported(unsigned width, unsigned out_rows)
+bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs)
 {
+    if (pairs > kClassMaxSweeps) return false;            // every sweep serves at least one pair
     const unsigned lanes_per_row = width / 128u;
     if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
     if ((width / 256u * 66u) % 4u != 0u) return false;   // rows must start on dword boundaries

@@ -46,6 +46,15 @@ class MoeLayer:
         self.merge_shared = True
         # row-batch (prefill-width) kernels on the int8 matrix cores instead of the decode sweeps
         self.matrix_cores = matrix_cores
+        # when a list, run() appends (name, event) marks around the two expert sweeps so a caller
+        # can read their durations inside its own timed steps
+        self.marks = None
+
+    def _mark(self, name):
+        if self.marks is not None:
+            event = torch.cuda.Event(enable_timing=True)
+            event.record()
+            self.marks.append((name, event))
 
     def run(self, rows_f32: torch.Tensor, logits: torch.Tensor):
         """Enqueue one batch; returns the combined rows (device tensor, not synchronised)."""
@@ -67,10 +76,12 @@ class MoeLayer:
         row_q8 = (self.intermediate // 256) * 292
         joined = self.shared is not None and self.act_q8 and (pairs * row_q8) % 16 == 0
         shared_mid = self.intermediate_f32[pairs:pairs + rows] if joined else self.shared_mid
+        self._mark("up_begin")
         K.moe_up(self.routed, acts, self.act_q8, self.weights, self.worklist, pairs, self.topk,
                  self.experts, self.limit, self.intermediate_f32, st,
                  shared=self.shared if merged else None, shared_rows=rows if merged else 0,
                  shared_intermediate=shared_mid if merged else None)
+        self._mark("up_end")
         if self.shared is not None and not merged:
             K.moe_up(self.shared, acts, self.act_q8, None, None, rows, 1, 1, self.limit,
                      shared_mid, st)
@@ -87,10 +98,12 @@ class MoeLayer:
         else:
             mid, smid = self.intermediate_f32, shared_mid
         self.last_shared_mid, self.last_shared_down_input = shared_mid, smid    # for stage-wise callers
+        self._mark("down_begin")
         K.moe_down(self.routed, mid, self.act_q8, self.worklist, pairs, self.experts,
                    self.pair_outputs, st, shared=self.shared if merged else None,
                    shared_rows=rows if merged else 0, shared_intermediate=smid if merged else None,
                    shared_outputs=self.shared_out if merged else None)
+        self._mark("down_end")
         if self.shared is not None and not merged:
             K.moe_down(self.shared, smid, self.act_q8, None, rows, 1, self.shared_out, st)
         K.moe_reduce_combine(self.pair_outputs, rows, self.topk, self.hidden, self.shared_out,
