@@ -55,7 +55,8 @@ constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave
 // {whole problem is one bucket : 1, shared expert's problem : 1, bucket : 14, sweep of the bucket : 16}.
 constexpr unsigned kClassMaxSweeps = 4096u;
 constexpr unsigned kClassCountBase = kParkBase + kSweepWaves * kParkBytes;
-constexpr unsigned kClassListBase = kClassCountBase + 64u;
+constexpr unsigned kClassWaveBase = kClassCountBase + 32u;    // per wave and class: entries of a turn
+constexpr unsigned kClassListBase = kClassCountBase + 32u + kSweepWaves * 16u;
 constexpr unsigned kSweepLdsBytes = kClassListBase + kClassMaxSweeps * 4u;
 
 __device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
@@ -577,15 +578,34 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
             }
         }
         __syncthreads();
-        for (unsigned s = tid; s < all_sweeps; s += kSweepThreads) {
-            unsigned word;
-            const unsigned n = describe(s, word);
-            const unsigned at = __hip_atomic_fetch_add(
-                reinterpret_cast<__attribute__((address_space(3))) unsigned *>(kClassCountBase + 16u + 4u * (4u - n)),
-                1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            lds_store_u32(kClassListBase + 4u * at, word);
+        // Every workgroup must arrive at the same list: a sweep's place in its class is the
+        // number of sweeps of that class before it, counted with ballots inside a wavefront and
+        // per-wavefront totals across the workgroup, a turn of kSweepThreads sweeps at a time.
+        for (unsigned turn = 0; turn < all_sweeps; turn += kSweepThreads) {
+            const unsigned s = turn + tid;
+            unsigned word = 0u;
+            const unsigned mine = s < all_sweeps ? 4u - describe(s, word) : 4u;   // class 0..3, 4: none
+            unsigned rank = 0u;
+#pragma unroll
+            for (unsigned c = 0; c < 4u; ++c) {
+                const unsigned long long members = __ballot(mine == c);
+                if (mine == c) rank = (unsigned)__popcll(members & ((1ull << lane) - 1ull));
+                if (lane == 0u) lds_store_u32(kClassWaveBase + (wave * 4u + c) * 4u, (unsigned)__popcll(members));
+            }
+            __syncthreads();
+            if (mine < 4u) {
+                unsigned at = lds_load_u32(kClassCountBase + 16u + 4u * mine) + rank;
+                for (unsigned w = 0; w < wave; ++w) at += lds_load_u32(kClassWaveBase + (w * 4u + mine) * 4u);
+                lds_store_u32(kClassListBase + 4u * at, word);
+            }
+            __syncthreads();
+            if (tid < 4u) {
+                unsigned total = lds_load_u32(kClassCountBase + 16u + 4u * tid);
+                for (unsigned w = 0; w < kSweepWaves; ++w) total += lds_load_u32(kClassWaveBase + (w * 4u + tid) * 4u);
+                lds_store_u32(kClassCountBase + 16u + 4u * tid, total);
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
     const unsigned total_long = all_sweeps * long_tiles;
     const unsigned total_items = total_long + all_sweeps * short_tiles;
