@@ -28,7 +28,7 @@ MFMA_INT8_PEAK_TOPS = 5000.0
 HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
 EXPERT_BYTES = 3 * 3_784_704   # gate + up + down of one IQ2_XXS expert
 # iq2_sweep_kernel<fused>: FETCH_SIZE 632 787 x 2.000 KiB + WRITE_SIZE 15 782 x 1.000 KiB per launch
-GATE_UP_TRAFFIC_BYTES = int((580_550 * 2.0 + 13_604) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((605_830 * 2.0 + 13_760) * 1024)
 
 
 def synth_iq2xxs(torch, blocks: int, device, seed: int):
