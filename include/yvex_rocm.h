@@ -567,18 +567,75 @@ typedef struct {
     char execution_identity[YVEX_SHA256_HEX_CAP];
 } yvex_moe_row_batch_result;
 
+/* include/yvex/internal/execution.h:56-71,79-84,108-112: the classes a physical-execution
+ * decision names. */
+typedef enum {
+    YVEX_EXECUTION_CONSUMER_EMBEDDING = 0,
+    YVEX_EXECUTION_CONSUMER_ATTENTION_PROJECTION,
+    YVEX_EXECUTION_CONSUMER_ATTENTION_STATE,
+    YVEX_EXECUTION_CONSUMER_MOE_ROUTER,
+    YVEX_EXECUTION_CONSUMER_ROUTED_GATE_UP,
+    YVEX_EXECUTION_CONSUMER_ROUTED_DOWN,
+    YVEX_EXECUTION_CONSUMER_SHARED_EXPERT,
+    YVEX_EXECUTION_CONSUMER_FINAL_NORMALIZATION,
+    YVEX_EXECUTION_CONSUMER_OUTPUT_HEAD,
+    YVEX_EXECUTION_CONSUMER_DRAFT_FEATURE_PROJECTION,
+    YVEX_EXECUTION_CONSUMER_DRAFT_BACKBONE,
+    YVEX_EXECUTION_CONSUMER_MARKOV,
+    YVEX_EXECUTION_CONSUMER_CONFIDENCE,
+    YVEX_EXECUTION_CONSUMER_COUNT
+} yvex_execution_consumer_class;
+
+#define YVEX_EXECUTION_TEXT_CAP 64u
+
+/* include/yvex/internal/execution.h:129-155, field for field (the tensor role and scope, the
+ * placement, sharing, backend-requirement and evidence classes are plain enums there and are
+ * carried as int here: the layout functions never read them). */
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long terminal_tensor_id;
+    int role, scope;
+    unsigned long long layer_index, predictor_index, expert_count;
+    unsigned int canonical_qtype;
+    unsigned long long canonical_row_width, canonical_row_count;
+    unsigned long long encoded_offset, encoded_bytes, alignment;
+    yvex_execution_consumer_class consumer;
+    yvex_execution_layout_class layout;
+    int placement, sharing;
+    yvex_execution_activation_class activation;
+    unsigned long long supported_width_mask, maximum_context, worklist_width_mask;
+    unsigned long long tensor_core_minimum;
+    int required_backend;
+    unsigned int required_compute_major, required_compute_minor;
+    int evidence;
+    yvex_execution_class fallback;
+    int derived_asset_required;
+    char kernel_family[YVEX_EXECUTION_TEXT_CAP];
+    char tensor_core_kernel_family[YVEX_EXECUTION_TEXT_CAP];
+    char terminal_identity[YVEX_SHA256_HEX_CAP];
+    char decision_identity[YVEX_SHA256_HEX_CAP];
+} yvex_physical_execution_decision;
+
 /* moe.h:277-297. execute_rows follows src/backend/cuda/moe.c:1826-1923: with mixing rows in the
  * layer plan it runs the residual-stream ingress (mixing projection, gates, Sinkhorn matrix,
  * weighted RMS norm; moe.c:1210-1254), the experts on the normalised rows and the egress onto the
  * streams (moe.c:1533-1541); rows are then row_count x expanded_width. Without mixing rows the
  * rows are taken as normalised hidden rows and the output is bf16(routed + shared).
- * derived_layout_plan/build take the reference's physical-execution decision;
- * this backend streams canonical GGUF rows directly and needs no derived layout, so both
- * answer UNSUPPORTED and callers keep layout CANONICAL_ROW / EXPERT_MAJOR. */
+ * derived_layout_plan/build replace yvex_cuda_moe_derived_layout_plan/build
+ * (src/backend/cuda/layout.c:95-167): the storage size and the deterministic re-packing of one
+ * routed expert tensor, as host byte work over the caller's buffers. IQ2_XXS: the two scale bytes
+ * of every superblock in block order, then (from the next multiple of 64) its 64 code bytes in
+ * block order. Q2_K: per pair of neighbouring rows of one expert and block, 8 bytes (d, dmin of
+ * the even row, then of the odd row), then from a 64-aligned offset 32 bytes of sub-block scales
+ * (two halves of 16: even row's 8 bytes, odd row's 8 bytes), then from a 64-aligned offset 128
+ * code bytes (the rows' 4-byte words interleaved). Padding is zero. As in the reference, whose
+ * row-batch path refuses a DERIVED_BACKEND view (moe.c:939-958), execute_rows answers UNSUPPORTED
+ * for such views: the sweeps stream canonical rows. */
 typedef struct {
-    int (*derived_layout_plan)(const void *decision, unsigned long long *storage_bytes,
-                               yvex_error *err);
-    int (*derived_layout_build)(const void *decision, const unsigned char *canonical,
+    int (*derived_layout_plan)(const yvex_physical_execution_decision *decision,
+                               unsigned long long *storage_bytes, yvex_error *err);
+    int (*derived_layout_build)(const yvex_physical_execution_decision *decision,
+                                const unsigned char *canonical,
                                 unsigned long long canonical_bytes, unsigned char *derived,
                                 unsigned long long storage_bytes, yvex_error *err);
     int (*workspace_required)(const yvex_moe_layer_plan *layer, unsigned long long row_count,
@@ -588,10 +645,9 @@ typedef struct {
      * src/backend/cuda/moe.c:1826-1923): router projection, scoring and top-k, expert-major
      * worklist, routed experts (gate/up -> clamped SwiGLU -> bf16 -> down -> bf16, summed in rank
      * order), shared expert, combined = bf16(routed + shared) into batch->device_outputs.
-     * batch->device_rows holds the already normalised hidden rows [row_count, hidden_width]:
-     * the residual-mixing envelope around the experts is not part of this build, so a plan with
-     * expanded_width != hidden_width or mhc_mixing_rows != 0 is refused UNSUPPORTED, as is the
-     * hash-token router. Mandatory refusals kept from the reference: row count outside
+     * Without mixing rows batch->device_rows holds the already normalised hidden rows
+     * [row_count, hidden_width]; with them, the residual streams [row_count, expanded_width].
+     * Mandatory refusals kept from the reference: row count outside
      * worklist_policy->supported_width_mask -> UNSUPPORTED before anything is touched
      * (moe.c:1840-1862); gate/up activation or kernel family disagreement -> FORMAT
      * (moe.c:923-928); unknown kernel family -> UNSUPPORTED (moe.c:961-969); workspace missing or
@@ -603,6 +659,15 @@ typedef struct {
     int (*complete_rows)(yvex_backend *backend, int barrier_observed,
                          yvex_moe_row_batch_result *result, yvex_error *err);
 } yvex_backend_moe_operations;
+
+/* The two layout entries of the table above, callable without a backend (they touch no device):
+ * replace yvex_cuda_moe_derived_layout_plan/build, src/backend/cuda/private.h:400-402. */
+int yvex_rocm_moe_derived_layout_plan(const yvex_physical_execution_decision *decision,
+                                      unsigned long long *storage_bytes, yvex_error *err);
+int yvex_rocm_moe_derived_layout_build(const yvex_physical_execution_decision *decision,
+                                       const unsigned char *canonical,
+                                       unsigned long long canonical_bytes, unsigned char *derived,
+                                       unsigned long long storage_bytes, yvex_error *err);
 
 /* moe.h:295-296: NULL unless the backend is ROCM and its kernels are loadable. */
 const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend);

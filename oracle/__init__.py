@@ -432,3 +432,53 @@ def moe_layer(*, hidden, intermediate, experts, topk, qtypes, routed, shared, in
     if rc:
         raise RuntimeError(f"yvo_moe_layer rc={rc}")
     return dict(selected=sel, weights=w, routed=routed_out, shared=shared_out, combined=combined)
+
+
+def _align64(n: int) -> int:
+    return (n + 63) & ~63
+
+
+def derived_layout_plan(qtype: int, row_count: int, row_width: int, expert_count: int) -> int:
+    """Bytes of the derived image of one routed expert tensor (src/backend/cuda/layout.c:23-93).
+
+    numpy restatement; raises ValueError where the reference refuses the geometry."""
+    if expert_count <= 1 or row_count % expert_count or row_width % 256:
+        raise ValueError("incomplete decision")
+    blocks = row_count * (row_width // 256)
+    if qtype == IQ2_XXS:
+        return _align64(2 * blocks) + 64 * blocks
+    if qtype == Q2_K:
+        if (row_count // expert_count) % 2:
+            raise ValueError("odd rows per expert")
+        units = blocks // 2
+        return _align64(_align64(8 * units) + 32 * units) + 128 * units
+    raise ValueError("qtype not admitted")
+
+
+def derived_layout_build(qtype: int, canonical, row_count: int, row_width: int, expert_count: int) -> np.ndarray:
+    """The derived image itself (src/backend/cuda/layout.c:112-167), by reshapes and transposes.
+
+    IQ2_XXS: column 0:2 of the [blocks, 66] byte matrix, then (64-aligned) columns 2:66.
+    Q2_K: [row pair, parity, block, 84] -> per (pair, block): bytes 80:84 of both rows; scale bytes
+    as [half, parity, 8]; code bytes as [word, parity, 4]."""
+    canonical = np.ascontiguousarray(canonical, np.uint8).ravel()
+    total = derived_layout_plan(qtype, row_count, row_width, expert_count)
+    per_row = row_width // 256
+    out = np.zeros(total, np.uint8)
+    if qtype == IQ2_XXS:
+        blocks = canonical.reshape(row_count * per_row, 66)
+        out[:2 * len(blocks)] = blocks[:, :2].ravel()
+        start = _align64(2 * len(blocks))
+        out[start:] = blocks[:, 2:].ravel()
+        return out
+    blocks = canonical.reshape(row_count // 2, 2, per_row, 84)          # [pair, parity, block, byte]
+    units = (row_count // 2) * per_row
+    factors = blocks[..., 80:84].transpose(0, 2, 1, 3)                  # [pair, block, parity, 4]
+    scales = blocks[..., 0:16].reshape(row_count // 2, 2, per_row, 2, 8).transpose(0, 2, 3, 1, 4)
+    codes = blocks[..., 16:80].reshape(row_count // 2, 2, per_row, 16, 4).transpose(0, 2, 3, 1, 4)
+    out[:8 * units] = factors.ravel()
+    second = _align64(8 * units)
+    out[second:second + 32 * units] = scales.ravel()
+    third = _align64(second + 32 * units)
+    out[third:] = codes.ravel()
+    return out

@@ -203,6 +203,27 @@ def main():
         out[f"ingress_{name}_normalized_bits"] = normalized.view(np.uint32)
         out[f"ingress_{name}_post_bits"] = post.view(np.uint32)
         out[f"ingress_{name}_combination_bits"] = comb.view(np.uint32)
+    # ---- derived expert storage: src/backend/cuda/layout.c:95-167 --------------------------------
+    ref.yvex_cuda_moe_derived_layout_plan.argtypes = [C.c_void_p, C.POINTER(abi.ULL), C.c_void_p]
+    ref.yvex_cuda_moe_derived_layout_build.argtypes = [C.c_void_p, C.c_void_p, abi.ULL, C.c_void_p, abi.ULL,
+                                                       C.c_void_p]
+    for name, qtype, block_bytes, experts, rows_per_expert, width in (
+            ("iq2_xxs", oracle.IQ2_XXS, 66, 3, 5, 512), ("q2_k", oracle.Q2_K, 84, 2, 6, 768)):
+        rows = experts * rows_per_expert
+        canonical = oracle.Generator(42, f"golden.layout.{name}").bytes(rows * (width // 256) * block_bytes)
+        decision = abi.ExecutionDecision()
+        decision.expert_count, decision.canonical_qtype = experts, qtype
+        decision.canonical_row_width, decision.canonical_row_count = width, rows
+        decision.encoded_bytes, decision.consumer = canonical.size, abi.CONSUMER_ROUTED_GATE_UP
+        decision.layout, decision.derived_asset_required = abi.LAYOUT_DERIVED, 1
+        storage, err = abi.ULL(), abi.Error()
+        assert ref.yvex_cuda_moe_derived_layout_plan(C.byref(decision), C.byref(storage), C.byref(err)) == 0
+        derived = np.full(storage.value, 0xA5, np.uint8)
+        rc = ref.yvex_cuda_moe_derived_layout_build(C.byref(decision), canonical.ctypes.data, canonical.size,
+                                                    derived.ctypes.data, derived.size, C.byref(err))
+        assert rc == 0, err.message
+        out[f"layout_{name}_shape"] = np.array([qtype, experts, rows, width], np.uint64)
+        out[f"layout_{name}_canonical"], out[f"layout_{name}_derived"] = canonical, derived
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes")

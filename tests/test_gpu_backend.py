@@ -555,6 +555,27 @@ def test_execute_rows_refusals(backend, oracle):
     assert case.execute() == abi.UNSUPPORTED
     for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
         case.job.weights[slot].kernel_family = abi.FAMILY_GFX950
+    # layouts: gate/up must agree and down must be derived exactly when they are (FORMAT); a derived
+    # image is refused by the row-batch path (UNSUPPORTED), src/backend/cuda/moe.c:933-958
+    case.job.weights[abi.W_ROUTED_UP].layout = abi.LAYOUT_CANONICAL_ROW
+    assert case.execute() == abi.FORMAT
+    case.job.weights[abi.W_ROUTED_UP].layout = abi.LAYOUT_EXPERT_MAJOR
+    case.job.weights[abi.W_ROUTED_DOWN].layout = abi.LAYOUT_DERIVED
+    assert case.execute() == abi.FORMAT
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
+        case.job.weights[slot].layout = abi.LAYOUT_DERIVED
+    assert case.execute() == abi.UNSUPPORTED
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN):
+        case.job.weights[slot].layout = abi.LAYOUT_EXPERT_MAJOR
+    # the layout entries of the table answer like the exported functions
+    decision = abi.ExecutionDecision()
+    decision.expert_count, decision.canonical_qtype = 4, 16
+    decision.canonical_row_width, decision.canonical_row_count, decision.encoded_bytes = 512, 8, 8 * 2 * 66
+    decision.consumer, decision.layout, decision.derived_asset_required = (
+        abi.CONSUMER_ROUTED_DOWN, abi.LAYOUT_DERIVED, 1)
+    storage = abi.ULL()
+    assert case.ops.derived_layout_plan(C.byref(decision), C.byref(storage), C.byref(case.err)) == 0
+    assert storage.value == 64 + 16 * 64
     # mixing rows that disagree with the stream count; expanded rows without mixing rows; hash router
     case.plan.mhc_mixing_rows = 24
     assert case.execute() == abi.BOUNDS

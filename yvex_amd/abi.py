@@ -216,10 +216,29 @@ class RowBatchResult(C.Structure):
                                               "execution_identity")]
 
 
+class ExecutionDecision(C.Structure):
+    """yvex_physical_execution_decision, include/yvex/internal/execution.h:129-155."""
+    _fields_ = [("schema_version", C.c_uint), ("terminal_tensor_id", ULL), ("role", C.c_int),
+                ("scope", C.c_int), ("layer_index", ULL), ("predictor_index", ULL), ("expert_count", ULL),
+                ("canonical_qtype", C.c_uint), ("canonical_row_width", ULL), ("canonical_row_count", ULL),
+                ("encoded_offset", ULL), ("encoded_bytes", ULL), ("alignment", ULL),
+                ("consumer", C.c_int), ("layout", C.c_int), ("placement", C.c_int), ("sharing", C.c_int),
+                ("activation", C.c_int), ("supported_width_mask", ULL), ("maximum_context", ULL),
+                ("worklist_width_mask", ULL), ("tensor_core_minimum", ULL), ("required_backend", C.c_int),
+                ("required_compute_major", C.c_uint), ("required_compute_minor", C.c_uint),
+                ("evidence", C.c_int), ("fallback", C.c_int), ("derived_asset_required", C.c_int),
+                ("kernel_family", C.c_char * 64), ("tensor_core_kernel_family", C.c_char * 64),
+                ("terminal_identity", C.c_char * HEX), ("decision_identity", C.c_char * HEX)]
+
+
+CONSUMER_ROUTED_GATE_UP, CONSUMER_ROUTED_DOWN, CONSUMER_SHARED_EXPERT = 4, 5, 6
+
+
 class MoeOperations(C.Structure):
     _fields_ = [
-        ("derived_layout_plan", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(ULL), C.POINTER(Error))),
-        ("derived_layout_build", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, ULL, C.c_void_p, ULL,
+        ("derived_layout_plan", C.CFUNCTYPE(C.c_int, C.POINTER(ExecutionDecision), C.POINTER(ULL),
+                                            C.POINTER(Error))),
+        ("derived_layout_build", C.CFUNCTYPE(C.c_int, C.POINTER(ExecutionDecision), C.c_void_p, ULL, C.c_void_p, ULL,
                                              C.POINTER(Error))),
         ("workspace_required", C.CFUNCTYPE(C.c_int, C.POINTER(LayerPlan), ULL, C.POINTER(ULL),
                                            C.POINTER(Error))),
@@ -253,7 +272,7 @@ EXPORTS = [
     "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows", "yvex_rocm_quant_row_dot",
     "yvex_backend_moe_operations_get", "yvex_backend_moe_begin", "yvex_backend_moe_add_expert",
     "yvex_backend_moe_finish", "yvex_backend_moe_close",
-    "yvex_expert_worklist_build",
+    "yvex_expert_worklist_build", "yvex_rocm_moe_derived_layout_plan", "yvex_rocm_moe_derived_layout_build",
     "yvex_gguf_open_path", "yvex_gguf_close", "yvex_gguf_metadata_count", "yvex_gguf_metadata_u64",
     "yvex_gguf_metadata_f64", "yvex_gguf_metadata_string", "yvex_gguf_tensor_count", "yvex_gguf_tensor_at",
     "yvex_gguf_tensor_find", "yvex_gguf_tensor_data_offset", "yvex_gguf_alignment", "yvex_gguf_file_size",
@@ -282,6 +301,10 @@ def library():
     lib.yvex_backend_moe_operations_get.argtypes = [C.c_void_p]
     lib.yvex_rocm_quant_row_dot.argtypes = [C.c_void_p, C.c_uint, C.c_void_p, C.c_size_t, C.c_void_p, ULL,
                                             C.POINTER(C.c_float), C.c_void_p, C.POINTER(Error)]
+    lib.yvex_rocm_moe_derived_layout_plan.argtypes = [C.POINTER(ExecutionDecision), C.POINTER(ULL),
+                                                      C.POINTER(Error)]
+    lib.yvex_rocm_moe_derived_layout_build.argtypes = [C.POINTER(ExecutionDecision), C.c_void_p, ULL,
+                                                       C.c_void_p, ULL, C.POINTER(Error)]
     lib.yvex_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
     lib.yvex_gguf_close.argtypes = [C.c_void_p]
     lib.yvex_gguf_close.restype = None

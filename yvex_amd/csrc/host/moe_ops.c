@@ -136,23 +136,6 @@ static int moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned lon
     return YVEX_OK;
 }
 
-static int layout_unsupported(const void *decision, unsigned long long *storage_bytes, yvex_error *err)
-{
-    (void)decision;
-    if (storage_bytes) *storage_bytes = 0ull;
-    return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.layout",
-                            "this backend streams canonical rows and defines no derived layout");
-}
-
-static int layout_build_unsupported(const void *decision, const unsigned char *canonical,
-                                    unsigned long long canonical_bytes, unsigned char *derived,
-                                    unsigned long long storage_bytes, yvex_error *err)
-{
-    (void)decision; (void)canonical; (void)canonical_bytes; (void)derived; (void)storage_bytes;
-    return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.layout",
-                            "this backend streams canonical rows and defines no derived layout");
-}
-
 static int q8_eligible(unsigned int qtype)
 {
     return qtype == YVEX_GGUF_QTYPE_Q8_0 || qtype == YVEX_GGUF_QTYPE_Q2_K ||
@@ -187,10 +170,15 @@ static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight
                          strcmp(gate->kernel_family, up->kernel_family) != 0))
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
                                 "compiled MoE gate and up kernel-family decisions disagree");
-    if (gate->layout != up->layout || gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND ||
-        down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)
-        return yvex_rocm_refuse(err, gate->layout != up->layout ? YVEX_ERR_FORMAT : YVEX_ERR_UNSUPPORTED,
-                                "rocm.moe.policy", "compiled routed MoE layouts disagree or are derived");
+    /* moe.c:933-958: layouts must agree (FORMAT); a derived image is not executable by the
+     * row-batch path there either (UNSUPPORTED). */
+    if (gate->layout != up->layout || ((gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND) !=
+                                       (down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)))
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
+                                "compiled routed MoE layouts disagree");
+    if (gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                "the row-batch path executes canonical rows, not a derived image");
     if ((gate_encoded && !family_admitted(gate->kernel_family)) ||
         (down_encoded && !family_admitted(down->kernel_family)))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
@@ -749,7 +737,8 @@ static int moe_complete_rows(yvex_backend *backend, int barrier_observed,
 }
 
 static const yvex_backend_moe_operations moe_operations = {
-    layout_unsupported, layout_build_unsupported, moe_workspace_required, moe_execute_rows,
+    yvex_rocm_moe_derived_layout_plan, yvex_rocm_moe_derived_layout_build, moe_workspace_required,
+    moe_execute_rows,
     moe_complete_rows};
 
 const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend)
