@@ -125,6 +125,20 @@ int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t t
                             uint64_t *sweep_offsets, uint64_t *counts, int *status,
                             yvex_hip_stream stream);
 
+/* A decode batch's preparation in one launch: yvex_hip_moe_route_rows, yvex_hip_worklist_build and
+ * (when values is not NULL) yvex_hip_q8k_quantize of the rows x width input, with the same outputs
+ * bit for bit. One workgroup routes and sorts while the others quantize, so the three launches'
+ * latencies are paid once. For rows <= 128, experts <= 256, topk <= 16
+ * (yvex_hip_moe_prepare_supported), else UNSUPPORTED. The reference launches these steps one by
+ * one (src/backend/cuda/moe.c:1286-1345, 1363-1376). */
+int yvex_hip_moe_prepare_supported(uint64_t rows, uint64_t experts, uint64_t topk);
+int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, uint64_t experts,
+                         uint64_t topk, int scoring, int normalize, double scaling, uint64_t *selected,
+                         float *weights, uint64_t *order, uint64_t *expert_ids, uint64_t *bucket_offsets,
+                         uint64_t *bucket_populations, uint64_t *sweep_offsets, uint64_t *counts,
+                         const float *values, uint64_t width, uint64_t input_stride, uint8_t *encoded,
+                         int *status, yvex_hip_stream stream);
+
 /* Expert matrices of one MoE layer. routed_* are expert-major: expert e starts at
  * base + e * expert_bytes and holds rows * row_bytes canonical GGUF bytes. */
 typedef struct {

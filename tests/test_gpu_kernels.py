@@ -220,6 +220,48 @@ def test_worklist_matches_stable_sort(gpu, oracle, rows, topk, experts):
     assert np.array_equal(wl.order.cpu().numpy().astype(np.uint64), want["source_pairs"])
 
 
+@pytest.mark.parametrize("rows,experts,topk,width,scoring", [
+    (32, 256, 8, 7168, 1), (1, 256, 8, 7168, 0), (128, 64, 6, 512, 0), (17, 200, 16, 1024, 1), (5, 16, 4, 0, 0)])
+def test_fused_preparation_equals_the_three_launches(gpu, oracle, rows, experts, topk, width, scoring):
+    """Routing + worklist + input quantization in one launch: every output bit for bit what the
+    separate launches write, and the oracle's selection."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(5, f"prepare.{rows}.{experts}.{topk}")
+    logits = dev(g.normal(rows * experts).reshape(rows, experts) * 1.5, gpu)
+    bias = dev((g.normal(experts) * 0.05).astype(np.float32), gpu)
+    values = dev(g.normal(rows * width).reshape(rows, width), gpu) if width else None
+    assert K.moe_prepare_supported(rows, experts, topk)
+    assert not K.moe_prepare_supported(129, experts, topk) and not K.moe_prepare_supported(rows, 257, topk)
+    status = K.new_status(gpu)
+    sel, w = K.moe_route_rows(logits, bias, topk, scoring, True, 2.5, status)
+    wl = K.worklist_build(sel, experts, status)
+    q8 = K.q8k_quantize(values, status) if width else None
+    status_ok(status)
+    fused_wl = K.Worklist(rows * topk, experts, gpu)
+    fused_q8 = torch.zeros_like(q8) if width else None
+    fsel, fw = K.moe_prepare(logits, bias, topk, scoring, True, 2.5, status, fused_wl, values, fused_q8)
+    status_ok(status)
+    assert torch.equal(fsel, sel) and torch.equal(fw.view(torch.int32), w.view(torch.int32))
+    n = int(wl.counts[0].item())
+    assert torch.equal(fused_wl.counts, wl.counts)
+    assert torch.equal(fused_wl.order, wl.order)
+    assert torch.equal(fused_wl.expert_ids[:n], wl.expert_ids[:n])
+    assert torch.equal(fused_wl.bucket_populations[:n], wl.bucket_populations[:n])
+    assert torch.equal(fused_wl.bucket_offsets[:n + 1], wl.bucket_offsets[:n + 1])
+    assert torch.equal(fused_wl.sweep_offsets[:n + 1], wl.sweep_offsets[:n + 1])
+    if width:
+        assert torch.equal(fused_q8, q8)
+    rc, want_sel, _, _ = oracle.moe_route(logits[rows - 1].cpu().numpy(), bias.cpu().numpy(), topk, scoring, True, 2.5)
+    assert rc == 0 and np.array_equal(fsel[rows - 1].cpu().numpy().astype(np.uint64), want_sel)
+    # a non-finite logit raises the numeric status from inside the fused launch as well
+    bad = logits.clone()
+    bad[0, 1] = float("nan")
+    status = K.new_status(gpu)
+    K.moe_prepare(bad, bias, topk, scoring, True, 2.5, status, fused_wl, values, fused_q8)
+    torch.cuda.synchronize()
+    assert int(status.item()) != 0
+
+
 def test_worklist_flags_duplicate_expert(gpu):
     from yvex_amd import kernels as K
     sel = np.array([[1, 2], [3, 3]], np.int64)

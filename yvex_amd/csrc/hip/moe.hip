@@ -11,6 +11,7 @@
 #include "launch.hpp"
 #include "units.hpp"
 #include "grouped.hpp"
+#include "q8k.hpp"
 
 namespace yvex {
 
@@ -38,14 +39,12 @@ __global__ __launch_bounds__(256) void route_scores_kernel(
 }
 
 // One wavefront per row; each lane scores four experts (experts <= 256).
-__global__ __launch_bounds__(256) void route_rows_kernel(
-    const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long rows,
+// One row by one wavefront.
+__device__ __forceinline__ void route_row(
+    const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long row, unsigned lane,
     unsigned experts, unsigned topk, int scoring, int normalize, double scaling,
     unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status)
 {
-    const unsigned lane = threadIdx.x & 63u;
-    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
-    if (row >= rows) return;
     float score[4];
     unsigned long long key[4];
 #pragma unroll
@@ -98,6 +97,17 @@ __global__ __launch_bounds__(256) void route_rows_kernel(
         if (!finite_f32(w)) raise_status(status, 1);
         weights[row * topk + lane] = w;
     }
+}
+
+__global__ __launch_bounds__(256) void route_rows_kernel(
+    const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long rows,
+    unsigned experts, unsigned topk, int scoring, int normalize, double scaling,
+    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status)
+{
+    const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    route_row(logits, bias, row, threadIdx.x & 63u, experts, topk, scoring, normalize, scaling, selected,
+              weights, status);
 }
 
 // Hash router (src/backend/cuda/moe_kernels.cu:222-245, src/graph/moe.c:539-582): a row's experts
@@ -156,15 +166,15 @@ __global__ __launch_bounds__(256) void route_hash_rows_kernel(
 
 constexpr unsigned kWorklistMaxRows = 4096u;
 
-__global__ __launch_bounds__(1024) void worklist_kernel(
+// The whole worklist by one workgroup; shared_words is its dynamic LDS (worklist_lds_bytes).
+__device__ __forceinline__ void worklist_block(
     const unsigned long long *__restrict__ selected, unsigned pairs, unsigned topk,
     unsigned experts, unsigned long long *__restrict__ order,
     unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
     unsigned long long *__restrict__ bucket_populations,
     unsigned long long *__restrict__ sweep_offsets, unsigned long long *__restrict__ counts,
-    int *status)
+    int *status, unsigned *shared_words)
 {
-    extern __shared__ unsigned shared_words[];
     const unsigned rows = pairs / topk;
     const unsigned words = (rows + 31u) / 32u;            // bitmap words per expert
     unsigned *bitmap = shared_words;                       // [experts][words]
@@ -280,6 +290,51 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
     }
     __syncthreads();
     if (tid == 0u && bad) raise_status(status, 2);
+}
+
+__global__ __launch_bounds__(1024) void worklist_kernel(
+    const unsigned long long *__restrict__ selected, unsigned pairs, unsigned topk,
+    unsigned experts, unsigned long long *__restrict__ order,
+    unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
+    unsigned long long *__restrict__ bucket_populations,
+    unsigned long long *__restrict__ sweep_offsets, unsigned long long *__restrict__ counts,
+    int *status)
+{
+    extern __shared__ unsigned shared_words[];
+    worklist_block(selected, pairs, topk, experts, order, expert_ids, bucket_offsets, bucket_populations,
+                   sweep_offsets, counts, status, shared_words);
+}
+
+// A decode batch's preparation in one launch instead of three: workgroup 0 routes the rows (one
+// wavefront a row, sixteen at a time) and then builds the worklist from what it wrote; every
+// other workgroup quantizes sixteen Q8_K blocks of the input rows, which depend on neither.
+constexpr unsigned kPrepareMaxRows = 128u;
+
+__global__ __launch_bounds__(1024) void decode_prepare_kernel(
+    const float *__restrict__ logits, const float *__restrict__ bias, unsigned rows, unsigned experts,
+    unsigned topk, int scoring, int normalize, double scaling, unsigned long long *selected,
+    float *__restrict__ weights, unsigned long long *__restrict__ order,
+    unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
+    unsigned long long *__restrict__ bucket_populations, unsigned long long *__restrict__ sweep_offsets,
+    unsigned long long *__restrict__ counts, const float *__restrict__ values, unsigned blocks,
+    unsigned long long input_stride, unsigned char *__restrict__ encoded, int *status)
+{
+    extern __shared__ unsigned shared_words[];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    if (blockIdx.x != 0u) {
+        const unsigned task = (blockIdx.x - 1u) * 16u + wave;
+        if (task >= rows * blocks) return;
+        const unsigned row = task / blocks, block = task % blocks;
+        q8k_quantize_block(values + (unsigned long long)row * input_stride + block * 256u + lane * 4u,
+                           encoded + (unsigned long long)task * kQ8KBytes, lane, status);
+        return;
+    }
+    for (unsigned row = wave; row < rows; row += 16u)
+        route_row(logits, bias, row, lane, experts, topk, scoring, normalize, scaling, selected, weights,
+                  status);
+    __syncthreads();   // the selections written above are read back by other waves below
+    worklist_block(selected, rows * topk, topk, experts, order, expert_ids, bucket_offsets,
+                   bucket_populations, sweep_offsets, counts, status, shared_words);
 }
 
 // ---- grouped expert projections ---------------------------------------------------------------
@@ -739,6 +794,12 @@ extern "C" int yvex_hip_moe_route_scores(const float *logits, uint64_t count, in
     return check_launch("moe_route_scores");
 }
 
+static size_t worklist_lds_bytes(uint64_t experts, uint64_t rows)
+{
+    const uint64_t words = (rows + 31u) / 32u;
+    return (size_t)(experts * words + 3u * experts + 1u + 1537u) * sizeof(unsigned);
+}
+
 extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
                                        uint64_t experts, uint64_t *order, uint64_t *expert_ids,
                                        uint64_t *bucket_offsets, uint64_t *bucket_populations,
@@ -751,8 +812,7 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
         return ST_INVALID_ARG;
     const uint64_t rows = pairs / topk;
     if (rows > kWorklistMaxRows) return ST_BOUNDS;
-    const uint64_t words = (rows + 31u) / 32u;
-    const size_t lds = (size_t)(experts * words + 3u * experts + 1u + 1537u) * sizeof(unsigned);
+    const size_t lds = worklist_lds_bytes(experts, rows);
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void *)worklist_kernel,
@@ -768,6 +828,40 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
         (unsigned long long *)bucket_offsets, (unsigned long long *)bucket_populations,
         (unsigned long long *)sweep_offsets, (unsigned long long *)counts, status);
     return check_launch("worklist_build");
+}
+
+extern "C" int yvex_hip_moe_prepare_supported(uint64_t rows, uint64_t experts, uint64_t topk)
+{
+    return rows != 0u && rows <= kPrepareMaxRows && experts != 0u && experts <= 256u && topk != 0u &&
+           topk <= experts && topk <= 16u;
+}
+
+extern "C" int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, uint64_t experts,
+                                    uint64_t topk, int scoring, int normalize, double scaling,
+                                    uint64_t *selected, float *weights, uint64_t *order,
+                                    uint64_t *expert_ids, uint64_t *bucket_offsets,
+                                    uint64_t *bucket_populations, uint64_t *sweep_offsets, uint64_t *counts,
+                                    const float *values, uint64_t width, uint64_t input_stride,
+                                    uint8_t *encoded, int *status, yvex_hip_stream stream)
+{
+    if (!logits || !selected || !weights || !order || !expert_ids || !bucket_offsets || !bucket_populations ||
+        !sweep_offsets || !counts || !status || (scoring != 0 && scoring != 1))
+        return ST_INVALID_ARG;
+    if (!yvex_hip_moe_prepare_supported(rows, experts, topk)) return ST_UNSUPPORTED;
+    uint64_t tasks = 0u;
+    if (values) {
+        if (!encoded || !width || width % 256u || input_stride < width || width / 256u > 0xffffu)
+            return ST_INVALID_ARG;
+        tasks = rows * (width / 256u);
+    }
+    const size_t lds = worklist_lds_bytes(experts, rows);
+    decode_prepare_kernel<<<(unsigned)(1u + (tasks + 15u) / 16u), 1024, lds, as_stream(stream)>>>(
+        logits, bias, (unsigned)rows, (unsigned)experts, (unsigned)topk, scoring, normalize, scaling,
+        (unsigned long long *)selected, weights, (unsigned long long *)order,
+        (unsigned long long *)expert_ids, (unsigned long long *)bucket_offsets,
+        (unsigned long long *)bucket_populations, (unsigned long long *)sweep_offsets,
+        (unsigned long long *)counts, values, (unsigned)(width / 256u), input_stride, encoded, status);
+    return check_launch("moe_prepare");
 }
 
 extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *activations,

@@ -1,7 +1,6 @@
-// Q8_K activation quantizer for gfx950: one 64-lane wavefront per 256-value block, four values
-// per lane, max-|x| search and the sixteen 16-value sums done with cross-lane shuffles.
-// Behaviour restated from src/backend/cuda/kernels.cu:436-489.
+// Q8_K activation quantizer for gfx950: one 64-lane wavefront per 256-value block (q8k.hpp).
 #include "common.hpp"
+#include "q8k.hpp"
 #include "launch.hpp"
 
 namespace yvex {
@@ -14,44 +13,8 @@ __global__ __launch_bounds__(256) void q8k_quantize_kernel(
     const unsigned long long task = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
     if (task >= rows * blocks) return;
     const unsigned long long row = task / blocks, block = task % blocks;
-    const float *x = values + row * input_stride + block * 256ull + lane * 4u;
-    unsigned char *out = encoded + task * kQ8KBytes;
-    float v[4];
-    unsigned long long key = 0ull;
-    bool bad = false;
-#pragma unroll
-    for (unsigned i = 0; i < 4u; ++i) {
-        v[i] = x[i];
-        const unsigned bits = __float_as_uint(v[i]);
-        bad |= !finite_f32(v[i]);
-        // order by |x|, then by lowest index; the low bit carries the sign of the winner
-        const unsigned long long k = ((unsigned long long)(bits & 0x7fffffffu) << 32) |
-                                     ((unsigned long long)(255u - (lane * 4u + i)) << 1) |
-                                     (bits >> 31);
-        key = k > key ? k : key;
-    }
-    if (bad) raise_status(status, 1);
-#pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) {
-        const unsigned long long other = __shfl_xor(key, offset, kWave);
-        key = other > key ? other : key;
-    }
-    const float magnitude = __uint_as_float((unsigned)(key >> 32));
-    const float signed_max = (key & 1ull) ? -magnitude : magnitude;
-    const float inverse = magnitude == 0.0f ? 0.0f : -127.0f / signed_max;
-    if (lane == 0u) *reinterpret_cast<float *>(out) = inverse == 0.0f ? 0.0f : 1.0f / inverse;
-    unsigned packed = 0u;
-    int sum = 0;
-#pragma unroll
-    for (unsigned i = 0; i < 4u; ++i) {
-        int q = inverse == 0.0f ? 0 : __float2int_rn(inverse * v[i]);
-        q = q > 127 ? 127 : q < -128 ? -128 : q;
-        sum += q;
-        packed |= ((unsigned)q & 255u) << (8u * i);
-    }
-    *reinterpret_cast<unsigned *>(out + 4u + lane * 4u) = packed;
-    sum = group_sum_i32<4>(sum);   // four lanes hold sixteen consecutive values
-    if ((lane & 3u) == 0u) *reinterpret_cast<short *>(out + 260u + (lane >> 2) * 2u) = (short)sum;
+    q8k_quantize_block(values + row * input_stride + block * 256ull + lane * 4u, encoded + task * kQ8KBytes,
+                       lane, status);
 }
 
 // Rows of a split input laid end to end, each value rounded to bf16 as the reference's split

@@ -514,21 +514,38 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
         LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)bias_address, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype,
                                1ull, experts, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].row_bytes, NULL, 1ull,
                                (float *)AT(bias), (int *)status, stream), "rocm.moe.rows.bias");
-    if (!hash_router)
-    LAUNCH(yvex_hip_moe_route_rows((const float *)AT(logits),
-                                   layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
-                                   row_count, experts, topk, (int)layer->scoring,
-                                   layer->normalize_topk_probabilities, layer->routed_scaling_factor,
-                                   (uint64_t *)AT(selected), (float *)AT(weights), (int *)status, stream),
-           "rocm.moe.rows.route");
-    LAUNCH(yvex_hip_worklist_build((const uint64_t *)AT(selected), pairs, topk, experts,
-                                   (uint64_t *)AT(order), (uint64_t *)AT(expert_ids),
-                                   (uint64_t *)AT(bucket_offsets), (uint64_t *)AT(bucket_populations),
-                                   (uint64_t *)AT(sweep_offsets), (uint64_t *)AT(counts), (int *)status,
-                                   stream), "rocm.moe.rows.worklist");
-    if (routed_q8 || (has_shared && shared_q8))
-        LAUNCH(yvex_hip_q8k_quantize((const float *)activations, row_count, hidden, hidden,
-                                     (uint8_t *)AT(input_q8), (int *)status, stream), "rocm.moe.rows.q8");
+    /* a decode-width batch with the learned router: routing, worklist and input quantization
+     * share one launch */
+    const int need_q8 = routed_q8 || (has_shared && shared_q8);
+    if (!hash_router && yvex_hip_moe_prepare_supported(row_count, experts, topk)) {
+        LAUNCH(yvex_hip_moe_prepare((const float *)AT(logits),
+                                    layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                    row_count, experts, topk, (int)layer->scoring,
+                                    layer->normalize_topk_probabilities, layer->routed_scaling_factor,
+                                    (uint64_t *)AT(selected), (float *)AT(weights), (uint64_t *)AT(order),
+                                    (uint64_t *)AT(expert_ids), (uint64_t *)AT(bucket_offsets),
+                                    (uint64_t *)AT(bucket_populations), (uint64_t *)AT(sweep_offsets),
+                                    (uint64_t *)AT(counts), need_q8 ? (const float *)activations : NULL,
+                                    hidden, hidden, need_q8 ? (uint8_t *)AT(input_q8) : NULL,
+                                    (int *)status, stream), "rocm.moe.rows.prepare");
+    } else {
+        if (!hash_router)
+            LAUNCH(yvex_hip_moe_route_rows((const float *)AT(logits),
+                                           layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                           row_count, experts, topk, (int)layer->scoring,
+                                           layer->normalize_topk_probabilities,
+                                           layer->routed_scaling_factor, (uint64_t *)AT(selected),
+                                           (float *)AT(weights), (int *)status, stream),
+                   "rocm.moe.rows.route");
+        LAUNCH(yvex_hip_worklist_build((const uint64_t *)AT(selected), pairs, topk, experts,
+                                       (uint64_t *)AT(order), (uint64_t *)AT(expert_ids),
+                                       (uint64_t *)AT(bucket_offsets), (uint64_t *)AT(bucket_populations),
+                                       (uint64_t *)AT(sweep_offsets), (uint64_t *)AT(counts), (int *)status,
+                                       stream), "rocm.moe.rows.worklist");
+        if (need_q8)
+            LAUNCH(yvex_hip_q8k_quantize((const float *)activations, row_count, hidden, hidden,
+                                         (uint8_t *)AT(input_q8), (int *)status, stream), "rocm.moe.rows.q8");
+    }
     if (row_batch)
         LAUNCH(yvex_hip_moe_up_rows(&routed, AT(input_q8), (const float *)AT(weights),
                                     (const uint64_t *)AT(order), (const uint64_t *)AT(expert_ids),

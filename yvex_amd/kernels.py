@@ -205,6 +205,29 @@ def worklist_build(selected, experts, status, worklist: Worklist | None = None) 
     return wl
 
 
+def moe_prepare_supported(rows: int, experts: int, topk: int) -> bool:
+    fn = load_library().yvex_hip_moe_prepare_supported
+    fn.restype = C.c_int
+    return bool(fn(C.c_uint64(rows), C.c_uint64(experts), C.c_uint64(topk)))
+
+
+def moe_prepare(logits, bias, topk, scoring, normalize, scaling, status, worklist: Worklist,
+                values=None, encoded=None):
+    """Routing, worklist and (with values) the Q8_K quantization of the input rows in one launch."""
+    rows, experts = logits.shape
+    selected = torch.empty((rows, topk), dtype=torch.int64, device=logits.device)
+    weights = torch.empty((rows, topk), dtype=torch.float32, device=logits.device)
+    width = 0 if values is None else values.shape[1]
+    stride = 0 if values is None else values.stride(0)
+    wl = worklist
+    _call("yvex_hip_moe_prepare", _ptr(logits), _ptr(bias), C.c_uint64(rows), C.c_uint64(experts),
+          C.c_uint64(topk), C.c_int(scoring), C.c_int(int(normalize)), C.c_double(scaling), _ptr(selected),
+          _ptr(weights), _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
+          _ptr(wl.bucket_populations), _ptr(wl.sweep_offsets), _ptr(wl.counts), _ptr(values),
+          C.c_uint64(width), C.c_uint64(stride), _ptr(encoded), _ptr(status), _stream())
+    return selected, weights
+
+
 def expert_weights(gate, up, down, qtypes, hidden, intermediate) -> ExpertWeights:
     w = ExpertWeights()
     w.gate, w.up, w.down = gate.data_ptr(), up.data_ptr(), down.data_ptr()

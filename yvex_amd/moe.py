@@ -44,6 +44,8 @@ class MoeLayer:
         self.selected = None
         self.weights = None
         self.merge_shared = True
+        # routing, worklist and input quantization in one launch where the batch is small enough
+        self.fused_prepare = True
         # row-batch (prefill-width) kernels on the int8 matrix cores instead of the decode sweeps
         self.matrix_cores = matrix_cores
         # when a list, run() appends (name, event) marks around the two expert sweeps so a caller
@@ -62,14 +64,17 @@ class MoeLayer:
         assert rows <= self.max_rows
         pairs = rows * self.topk
         st = self.status
-        if self.act_q8:
-            K.q8k_quantize(rows_f32, st, self.act_q8_rows)
-            acts = self.act_q8_rows
+        acts = self.act_q8_rows if self.act_q8 else rows_f32
+        if self.fused_prepare and K.moe_prepare_supported(rows, self.experts, self.topk):
+            self.selected, self.weights = K.moe_prepare(
+                logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st, self.worklist,
+                rows_f32 if self.act_q8 else None, self.act_q8_rows if self.act_q8 else None)
         else:
-            acts = rows_f32
-        self.selected, self.weights = K.moe_route_rows(
-            logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st)
-        K.worklist_build(self.selected, self.experts, st, self.worklist)
+            if self.act_q8:
+                K.q8k_quantize(rows_f32, st, self.act_q8_rows)
+            self.selected, self.weights = K.moe_route_rows(
+                logits, self.bias, self.topk, self.scoring, self.normalize, self.scaling, st)
+            K.worklist_build(self.selected, self.experts, st, self.worklist)
         if self.matrix_cores:
             return self._run_rows(acts, rows, pairs)
         merged = self.shared is not None and self.merge_shared
