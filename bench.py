@@ -321,6 +321,8 @@ def main() -> int:
     ap.add_argument("--cpu-rows", type=int, default=4)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--separate-prepare", action="store_true",
+                    help="launch routing, worklist and input quantization one by one instead of fused")
     ap.add_argument("--alone", action="store_true",
                     help="also time the two expert sweeps launched alone, back to back")
     ap.add_argument("--calibrate", action="store_true",
@@ -355,6 +357,7 @@ def main() -> int:
                      qtypes=(qt, qt, qt), routed=(gate, up, down), shared=shared, bias=None,
                      scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
                      act_q8=args.act == "q8k", max_rows=ROWS, device=dev)
+    layer.fused_prepare = not args.separate_prepare
 
     for _ in range(args.warmup):
         layer.run(x, logits)

@@ -435,7 +435,7 @@ def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, sh
     per_expert = sum(case.parts[n].nbytes for n in ("gate", "up", "down")) // case.experts
     assert res.active_weight_per_unique_expert_bytes == per_expert
     assert res.encoded_bytes_read == res.active_weight_base_bytes + per_expert * uniq
-    assert res.kernel_launches >= 8 and res.memory.complete == 1
+    assert res.kernel_launches >= 6 and res.memory.complete == 1
 
 
 @pytest.mark.parametrize("qtype,streams,rows,hidden,iterations", [

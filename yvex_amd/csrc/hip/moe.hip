@@ -39,6 +39,27 @@ __global__ __launch_bounds__(256) void route_scores_kernel(
 }
 
 // One wavefront per row; each lane scores four experts (experts <= 256).
+// Largest value of the 64 lanes, in every lane: butterflies inside each row of 16 lanes, then the
+// rows' results carried upward (lane 15 into the next row, lane 31 into the upper half) and the
+// last lane read back.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ unsigned dpp_max_u32(unsigned v)
+{
+    const unsigned other = (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROWS, 0xf, false);
+    return other > v ? other : v;
+}
+
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v)
+{
+    v = dpp_max_u32<0xb1, 0xf>(v);    // quad_perm [1, 0, 3, 2]
+    v = dpp_max_u32<0x4e, 0xf>(v);    // quad_perm [2, 3, 0, 1]
+    v = dpp_max_u32<0x141, 0xf>(v);   // row_half_mirror
+    v = dpp_max_u32<0x140, 0xf>(v);   // row_mirror
+    v = dpp_max_u32<0x142, 0xa>(v);   // row_bcast15 into rows 1 and 3
+    v = dpp_max_u32<0x143, 0xc>(v);   // row_bcast31 into rows 2 and 3
+    return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // One row by one wavefront.
 __device__ __forceinline__ void route_row(
     const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long row, unsigned lane,
@@ -70,12 +91,14 @@ __device__ __forceinline__ void route_row(
         unsigned long long best = key[0];
 #pragma unroll
         for (unsigned i = 1; i < 4u; ++i) best = key[i] > best ? key[i] : best;
-#pragma unroll
-        for (int offset = 32; offset > 0; offset >>= 1) {
-            const unsigned long long other = __shfl_xor(best, offset, kWave);
-            best = other > best ? other : best;
-        }
-        const unsigned e = 0xffffffffu - (unsigned)(best & 0xffffffffull);
+        // The wave's best key in two steps that need no cross-lane permutes through LDS: the
+        // largest score word, then the first lane holding it (a lane's ordinals are below the
+        // next lane's, and its own best already is its lowest ordinal with that score).
+        const unsigned top = wave_max_u32((unsigned)(best >> 32));
+        const unsigned long long holders = __ballot((unsigned)(best >> 32) == top);
+        const unsigned winner = (unsigned)__builtin_ctzll(holders);
+        const unsigned e = 0xffffffffu - (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(best & 0xffffffffull),
+                                                                             (int)winner);
         float s = 0.0f;
 #pragma unroll
         for (unsigned i = 0; i < 4u; ++i)
@@ -271,22 +294,16 @@ __device__ __forceinline__ void worklist_block(
     }
     __syncthreads();
     if (tid == 0u) counts[1] = scan[1536u];
-    for (unsigned i = tid; i < experts * words; i += blockDim.x) {
-        const unsigned e = i / words, w = i % words;
-        unsigned bits = bitmap[i];
-        if (!bits) continue;
-        unsigned before = 0u;
-        for (unsigned k = 0; k < w; ++k) before += __popc(bitmap[e * words + k]);
-        while (bits) {
-            const unsigned bit = __ffs(bits) - 1u;
-            bits &= bits - 1u;
-            const unsigned row = w * 32u + bit;
-            unsigned rank = 0u;
-            for (unsigned r = 0; r < topk; ++r)
-                if (selected[row * topk + r] == e) rank = r;
-            order[offset[e] + before] = (unsigned long long)row * topk + rank;
-            before++;
-        }
+    // every pair finds its own place: its bucket's start plus the rows below its own that chose
+    // the same expert (pairs of a bucket stay in row order, which is the stable order)
+    for (unsigned p = tid; p < pairs; p += blockDim.x) {
+        const unsigned long long e = selected[p];
+        if (e >= experts) continue;
+        const unsigned row = p / topk, w = row >> 5;
+        const unsigned *mine = bitmap + (unsigned)e * words;
+        unsigned before = __popc(mine[w] & ((1u << (row & 31u)) - 1u));
+        for (unsigned k = 0; k < w; ++k) before += __popc(mine[k]);
+        order[offset[e] + before] = p;
     }
     __syncthreads();
     if (tid == 0u && bad) raise_status(status, 2);
