@@ -194,7 +194,7 @@ def test_route_hash_rows(gpu, oracle, scoring):
 
 
 @pytest.mark.parametrize("rows,topk,experts", [(32, 8, 256), (1, 6, 256), (61, 6, 256),
-                                               (2048, 8, 256), (5, 2, 4)])
+                                               (2048, 8, 256), (5, 2, 4), (4096, 3, 256)])
 def test_worklist_matches_stable_sort(gpu, oracle, rows, topk, experts):
     from yvex_amd import kernels as K
     rng = np.random.default_rng(rows * 131 + topk)

@@ -196,7 +196,7 @@ __device__ __forceinline__ void worklist_block(
     unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
     unsigned long long *__restrict__ bucket_populations,
     unsigned long long *__restrict__ sweep_offsets, unsigned long long *__restrict__ counts,
-    int *status, unsigned *shared_words)
+    int *status, unsigned *shared_words, bool with_below)
 {
     const unsigned rows = pairs / topk;
     const unsigned words = (rows + 31u) / 32u;            // bitmap words per expert
@@ -223,9 +223,15 @@ __device__ __forceinline__ void worklist_block(
         if (old & (1u << (row & 31u))) bad = 1u;   // duplicate expert inside one row
     }
     __syncthreads();
+    // rows below each bitmap word that chose the expert (16 bits: at most 4096 rows), kept when
+    // the table fits beside the bitmap
+    unsigned short *below = reinterpret_cast<unsigned short *>(slot + experts + 1537u);
     for (unsigned e = tid; e < experts; e += blockDim.x) {
         unsigned n = 0u;
-        for (unsigned w = 0; w < words; ++w) n += __popc(bitmap[e * words + w]);
+        for (unsigned w = 0; w < words; ++w) {
+            if (with_below) below[e * words + w] = (unsigned short)n;
+            n += __popc(bitmap[e * words + w]);
+        }
         population[e] = n;
     }
     __syncthreads();
@@ -302,7 +308,9 @@ __device__ __forceinline__ void worklist_block(
         const unsigned row = p / topk, w = row >> 5;
         const unsigned *mine = bitmap + (unsigned)e * words;
         unsigned before = __popc(mine[w] & ((1u << (row & 31u)) - 1u));
-        for (unsigned k = 0; k < w; ++k) before += __popc(mine[k]);
+        if (with_below) before += below[(unsigned)e * words + w];
+        else
+            for (unsigned k = 0; k < w; ++k) before += __popc(mine[k]);
         order[offset[e] + before] = p;
     }
     __syncthreads();
@@ -315,11 +323,11 @@ __global__ __launch_bounds__(1024) void worklist_kernel(
     unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
     unsigned long long *__restrict__ bucket_populations,
     unsigned long long *__restrict__ sweep_offsets, unsigned long long *__restrict__ counts,
-    int *status)
+    int *status, int with_below)
 {
     extern __shared__ unsigned shared_words[];
     worklist_block(selected, pairs, topk, experts, order, expert_ids, bucket_offsets, bucket_populations,
-                   sweep_offsets, counts, status, shared_words);
+                   sweep_offsets, counts, status, shared_words, with_below != 0);
 }
 
 // A decode batch's preparation in one launch instead of three: workgroup 0 routes the rows (one
@@ -351,7 +359,7 @@ __global__ __launch_bounds__(1024) void decode_prepare_kernel(
                   status);
     __syncthreads();   // the selections written above are read back by other waves below
     worklist_block(selected, rows * topk, topk, experts, order, expert_ids, bucket_offsets,
-                   bucket_populations, sweep_offsets, counts, status, shared_words);
+                   bucket_populations, sweep_offsets, counts, status, shared_words, true);
 }
 
 // ---- grouped expert projections ---------------------------------------------------------------
@@ -811,10 +819,17 @@ extern "C" int yvex_hip_moe_route_scores(const float *logits, uint64_t count, in
     return check_launch("moe_route_scores");
 }
 
-static size_t worklist_lds_bytes(uint64_t experts, uint64_t rows)
+constexpr size_t kWorklistLdsLimit = 160u * 1024u - 64u;
+
+// Dynamic LDS of the worklist workgroup; *with_below says whether the 16-bit table of rows below
+// each bitmap word fits as well.
+static size_t worklist_lds_bytes(uint64_t experts, uint64_t rows, int *with_below)
 {
     const uint64_t words = (rows + 31u) / 32u;
-    return (size_t)(experts * words + 3u * experts + 1u + 1537u) * sizeof(unsigned);
+    const size_t base = (size_t)(experts * words + 3u * experts + 1u + 1537u) * sizeof(unsigned);
+    const size_t table = (size_t)(experts * words) * sizeof(unsigned short);
+    *with_below = base + table <= kWorklistLdsLimit;
+    return *with_below ? base + table : base;
 }
 
 extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs, uint64_t topk,
@@ -829,21 +844,22 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
         return ST_INVALID_ARG;
     const uint64_t rows = pairs / topk;
     if (rows > kWorklistMaxRows) return ST_BOUNDS;
-    const size_t lds = worklist_lds_bytes(experts, rows);
+    int with_below = 0;
+    const size_t lds = worklist_lds_bytes(experts, rows, &with_below);
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void *)worklist_kernel,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) !=
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWorklistLdsLimit) !=
             hipSuccess)
             (void)hipGetLastError();
         configured = true;
     }
-    if (lds > 160u * 1024u - 64u) return ST_BOUNDS;
+    if (lds > kWorklistLdsLimit) return ST_BOUNDS;
     worklist_kernel<<<1, 1024, lds, as_stream(stream)>>>(
         (const unsigned long long *)selected, (unsigned)pairs, (unsigned)topk, (unsigned)experts,
         (unsigned long long *)order, (unsigned long long *)expert_ids,
         (unsigned long long *)bucket_offsets, (unsigned long long *)bucket_populations,
-        (unsigned long long *)sweep_offsets, (unsigned long long *)counts, status);
+        (unsigned long long *)sweep_offsets, (unsigned long long *)counts, status, with_below);
     return check_launch("worklist_build");
 }
 
@@ -871,7 +887,9 @@ extern "C" int yvex_hip_moe_prepare(const float *logits, const float *bias, uint
             return ST_INVALID_ARG;
         tasks = rows * (width / 256u);
     }
-    const size_t lds = worklist_lds_bytes(experts, rows);
+    int with_below = 0;
+    const size_t lds = worklist_lds_bytes(experts, rows, &with_below);   // always fits at these sizes
+    if (!with_below) return ST_BOUNDS;
     decode_prepare_kernel<<<(unsigned)(1u + (tasks + 15u) / 16u), 1024, lds, as_stream(stream)>>>(
         logits, bias, (unsigned)rows, (unsigned)experts, (unsigned)topk, scoring, normalize, scaling,
         (unsigned long long *)selected, weights, (unsigned long long *)order,
