@@ -262,6 +262,42 @@ def test_fused_preparation_equals_the_three_launches(gpu, oracle, rows, experts,
     assert int(status.item()) != 0
 
 
+@pytest.mark.parametrize("rows,topk,hidden,offset", [(5, 3, 8, 0), (32, 8, 7168, 0), (3, 6, 10, 0), (4, 5, 64, 1),
+                                                     (7, 1, 4, 0)])
+def test_reduce_combine_sums_in_rank_order(gpu, oracle, rows, topk, hidden, offset):
+    """routed = the ranks' rows added one after another in fp32 (src/runtime/moe.c:596-632),
+    combined = bf16(routed + shared): exact, for widths and addresses that take the 16-byte path
+    and for those that do not (offset shifts the buffers off 16-byte alignment)."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(3, f"reduce.{rows}.{topk}.{hidden}")
+    pairs = (g.normal(rows * topk * hidden) * 3.0).astype(np.float32).reshape(rows * topk, hidden)
+    shared = g.normal(rows * hidden).astype(np.float32).reshape(rows, hidden)
+
+    def shifted(a):       # a view that starts `offset` floats into a larger allocation
+        t = torch.empty(a.size + offset, dtype=torch.float32, device=gpu)
+        v = t[offset:].view(a.shape)
+        v.copy_(torch.from_numpy(a))
+        return v
+    d_pairs, d_shared = shifted(pairs), shifted(shared)
+    routed, combined = shifted(np.zeros_like(shared)), shifted(np.zeros_like(shared))
+    status = K.new_status(gpu)
+    K.moe_reduce_combine(d_pairs, rows, topk, hidden, d_shared, routed, combined, status)
+    status_ok(status)
+    want = np.zeros((rows, hidden), np.float32)
+    for rank in range(topk):
+        want = (want + pairs.reshape(rows, topk, hidden)[:, rank]).astype(np.float32)
+    assert np.array_equal(routed.cpu().numpy(), want)
+    total = (want + shared).astype(np.float32)
+    want_combined = np.array([oracle.lib().yvo_bf16_round(float(v)) for v in total.ravel()], np.float32)
+    assert np.array_equal(combined.cpu().numpy().ravel(), want_combined)
+    # a non-finite sum raises the numeric status and publishes nothing for that element
+    d_pairs[0, 0] = float("inf")
+    status = K.new_status(gpu)
+    K.moe_reduce_combine(d_pairs, rows, topk, hidden, d_shared, routed, combined, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+
+
 def test_worklist_flags_duplicate_expert(gpu):
     from yvex_amd import kernels as K
     sel = np.array([[1, 2], [3, 3]], np.int64)

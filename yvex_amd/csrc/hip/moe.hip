@@ -674,26 +674,57 @@ __global__ __launch_bounds__(kGroupedThreads) void grouped_kernel(GroupedArgs a)
     }
 }
 
+// LANES columns per thread (4 when the width allows 16-byte accesses); each column's sum runs in
+// rank order, so the result does not depend on LANES.
+template <int LANES>
 __global__ __launch_bounds__(256) void reduce_combine_kernel(
     const float *__restrict__ pair_outputs, unsigned long long rows, unsigned topk,
     unsigned long long hidden, const float *__restrict__ shared, float *__restrict__ routed,
     float *__restrict__ combined, int *status)
 {
-    const unsigned long long index = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    struct alignas(4 * LANES) Pack {
+        float v[LANES];
+    };
+    const unsigned long long index = ((unsigned long long)blockIdx.x * 256ull + threadIdx.x) * LANES;
     if (index >= rows * hidden) return;
     const unsigned long long row = index / hidden, column = index % hidden;
-    float total = 0.0f;
-    for (unsigned rank = 0; rank < topk; ++rank)
-        total += pair_outputs[(row * topk + rank) * hidden + column];   // rank order, fp32
-    if (!finite_f32(total)) {
+    Pack total;
+#pragma unroll
+    for (int i = 0; i < LANES; ++i) total.v[i] = 0.0f;
+    const float *source = pair_outputs + row * topk * hidden + column;
+    unsigned rank = 0;
+    for (; rank + 4u <= topk; rank += 4u) {     // four ranks' loads in flight, added in rank order
+        Pack part[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) part[k] = *reinterpret_cast<const Pack *>(source + (rank + k) * hidden);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int i = 0; i < LANES; ++i) total.v[i] += part[k].v[i];
+    }
+    for (; rank < topk; ++rank) {
+        const Pack part = *reinterpret_cast<const Pack *>(source + rank * hidden);
+#pragma unroll
+        for (int i = 0; i < LANES; ++i) total.v[i] += part.v[i];
+    }
+    bool good = true;
+#pragma unroll
+    for (int i = 0; i < LANES; ++i) good = good && finite_f32(total.v[i]);
+    if (!good) {
         raise_status(status, 1);
         return;
     }
-    if (routed) routed[index] = total;
+    if (routed) *reinterpret_cast<Pack *>(routed + index) = total;
     if (combined && shared) {
-        const float value = bf16_round(total + shared[index]);
-        if (!finite_f32(value)) raise_status(status, 1);
-        else combined[index] = value;
+        const Pack base = *reinterpret_cast<const Pack *>(shared + index);
+        Pack value;
+#pragma unroll
+        for (int i = 0; i < LANES; ++i) {
+            value.v[i] = bf16_round(total.v[i] + base.v[i]);
+            good = good && finite_f32(value.v[i]);
+        }
+        if (!good) raise_status(status, 1);
+        else *reinterpret_cast<Pack *>(combined + index) = value;
     }
 }
 
@@ -990,9 +1021,16 @@ extern "C" int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t r
         (combined && !shared) || topk > 0xffffffffull)
         return ST_INVALID_ARG;
     if (rows > UINT64_MAX / hidden) return ST_BOUNDS;
-    const uint64_t grid = (rows * hidden + 255u) / 256u;
+    const uintptr_t addresses = (uintptr_t)pair_outputs | (uintptr_t)shared | (uintptr_t)routed |
+                                (uintptr_t)combined;
+    const bool quads = hidden % 4u == 0u && addresses % 16u == 0u;
+    const uint64_t grid = (rows * hidden / (quads ? 4u : 1u) + 255u) / 256u;
     if (grid > 0x7fffffffull) return ST_BOUNDS;
-    reduce_combine_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
-        pair_outputs, rows, (unsigned)topk, hidden, shared, routed, combined, status);
+    if (quads)
+        reduce_combine_kernel<4><<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+            pair_outputs, rows, (unsigned)topk, hidden, shared, routed, combined, status);
+    else
+        reduce_combine_kernel<1><<<(unsigned)grid, 256, 0, as_stream(stream)>>>(
+            pair_outputs, rows, (unsigned)topk, hidden, shared, routed, combined, status);
     return check_launch("moe_reduce_combine");
 }
