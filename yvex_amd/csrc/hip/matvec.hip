@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
                             acc[t] += super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
                                                         act_scale, s);
                     } else {
-                        const float v = q8_0_unit_value(wrow, uu[j], act_scale, s.dot);
+                        const float v = q8_0_unit_value(unit[j], act_scale, s.dot);
                         acc[t] += live[j] ? v : 0.0f;
                     }
                 } else {

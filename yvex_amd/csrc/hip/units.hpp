@@ -46,6 +46,7 @@ struct Unit {
     int factor;      // IQ2_XXS 2s+1; Q4_K sc; Q2_K sc of the first 16 values
     int factor2;     // Q2_K sc of the second 16 values (else = factor)
     int min1, min2;  // Q4_K: m (min2 = m); Q2_K: m of each half; else 0
+    unsigned scale_bits;  // Q8_0: the block's fp16 scale, taken from the dwords loaded for the codes
 };
 
 // EVEN: 1 = the caller knows the row starts on an even address, 0 = it does not, -1 = look.
@@ -81,10 +82,17 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
             const unsigned char *at = b - shift;
             const uint4 lo = *reinterpret_cast<const uint4 *>(at);
             const uint4 hi = *reinterpret_cast<const uint4 *>(at + 16u);
-            const unsigned tail = *reinterpret_cast<const unsigned *>(at + 28u + 2u * shift);
+            // Ninth dword: with the codes two bytes into their window it holds their last two
+            // bytes, and the scale is the low half of the first dword; with the codes aligned
+            // the eight dwords are complete and the ninth is the dword before them, whose high
+            // half is the scale (for the first block of a row that dword may lie before the
+            // tensor, so that one block reads its scale on its own).
+            const bool before = shift == 0u && u != 0u;
+            const unsigned tail = *reinterpret_cast<const unsigned *>(shift ? at + 32u : before ? at - 4u : at);
             const unsigned raw[9] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w, tail};
 #pragma unroll
             for (int i = 0; i < 8; ++i) unit.w[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+            unit.scale_bits = shift ? (lo.x & 0xffffu) : before ? (tail >> 16) : (unsigned)load_u16(b - 2u);
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -92,6 +100,7 @@ __device__ __forceinline__ void unit_load(const Iq2Tables &tables, const unsigne
                 unit.w[2 * i] = v.x;
                 unit.w[2 * i + 1] = v.y;
             }
+            unit.scale_bits = load_u16(b - 2u);
         }
         unit.factor = unit.factor2 = 1;
         unit.min1 = unit.min2 = 0;
@@ -325,10 +334,9 @@ __device__ __forceinline__ float super_combine(const unsigned char *super, float
 }
 
 // Q8_0: every unit scales itself (kernel_primitives.h:353-357).
-__device__ __forceinline__ float q8_0_unit_value(const unsigned char *row, unsigned u,
-                                                 float act_scale, int dot)
+__device__ __forceinline__ float q8_0_unit_value(const Unit &unit, float act_scale, int dot)
 {
-    return f16_bits_to_float(load_u16(row + u * 34u)) * act_scale * (float)dot;
+    return f16_bits_to_float((unsigned short)unit.scale_bits) * act_scale * (float)dot;
 }
 
 // Unit against 32 F32 activations. Returns the unit's contribution to the row dot.
@@ -358,6 +366,7 @@ __device__ __forceinline__ float unit_dot_f32(const Unit &unit, const unsigned c
         float gs = f16_bits_to_float(load_u16(b)) * (0.5f + (float)((unit.factor - 1) >> 1)) * 0.25f;
         return gs * (s1 + s2);
     } else if constexpr (QT == QT_Q8_0) {
+        // its own 2-byte load: with F32 activations the scale is needed late and this form measured faster
         return f16_bits_to_float(load_u16(row + u * 34u)) * (s1 + s2);
     } else if constexpr (QT == QT_Q4_K) {
         const unsigned char *b = row + sb * 144u;
