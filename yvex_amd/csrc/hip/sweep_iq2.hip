@@ -48,6 +48,8 @@ constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {s
 constexpr unsigned kPrefixBase = kSelBase + 128u * 32u * 8u;   // 257 sweep starts, u32
 constexpr unsigned kTicketAddress = kPrefixBase + 1056u;   // work-item counter of the workgroup
 constexpr unsigned kParkBase = kPrefixBase + 1088u;
+constexpr unsigned kPopulationBase = kParkBase + 2048u;   // bucket populations while the item list
+                                                          // is built (the parking areas are free then)
 constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave: 32 bytes per
                                                                       // (iteration, packed value), then one spare word per lane
 // Sweeps listed by the number of pairs they serve (4, 3, 2, 1): four class sizes, four class
@@ -443,13 +445,18 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         return;
     }
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    // The bucket count and this thread's bucket population are requested before the tables are
+    // built, so that their round trips to memory run under the table fill instead of after it.
+    const GroupedProblem &routed = a.problem[0];
+    const bool routed_fixed = routed.expert_ids == nullptr;
+    const unsigned buckets = routed_fixed ? 1u : (unsigned)routed.counts[0];
+    unsigned population_here = 0u;
+    if (!routed_fixed && tid < 256u && tid < routed.experts)
+        population_here = (unsigned)routed.bucket_populations[tid];
     sweep_tables_fill();
     if (tid == 0u) lds_store_u32(kTicketAddress, 0u);
 
     // ---- sweep numbering of the routed buckets: exclusive prefix of ceil(population / 4) ----
-    const GroupedProblem &routed = a.problem[0];
-    const bool routed_fixed = routed.expert_ids == nullptr;
-    const unsigned buckets = routed_fixed ? 1u : (unsigned)routed.counts[0];
     if (!routed_fixed && buckets > 256u) {
         if (tid == 0u) raise_status(a.status, 2);
         return;
@@ -459,9 +466,10 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned scratch = kParkBase;   // the parking areas are free until the first item
         unsigned mine = 0u;
         if (tid < 256u) {
-            mine = tid < buckets
-                ? (unsigned)((routed.bucket_populations[tid] + kSweepPairs - 1u) / kSweepPairs) : 0u;
+            if (tid >= buckets) population_here = 0u;
+            mine = (population_here + (unsigned)kSweepPairs - 1u) / (unsigned)kSweepPairs;
             lds_store_u32(scratch + 4u * tid, mine);
+            lds_store_u32(kPopulationBase + 4u * tid, population_here);
         }
         __syncthreads();
         unsigned from = scratch, to = scratch + 1024u;
@@ -551,7 +559,7 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
                         if (lds_load_u32(kPrefixBase + 4u * middle) <= r) low = middle;
                         else high = middle;
                     }
-                    population = routed.bucket_populations[low];
+                    population = lds_load_u32(kPopulationBase + 4u * low);
                 }
                 const unsigned k = r - (routed_fixed ? 0u : lds_load_u32(kPrefixBase + 4u * low));
                 left = population > (unsigned long long)k * kSweepPairs
