@@ -1,0 +1,157 @@
+"""The decode layer at its full size (hidden 7168, 256 routed + 1 shared IQ2_XXS experts of width
+2048, top-8 sigmoid routing, 32 rows, Q8_K activations): properties that do not need the CPU path
+over the whole batch, and the CPU oracle on two of the rows.
+
+  * the same batch twice gives the same bits;
+  * a row's result does not depend on the batch it arrives in (halves of the batch and a single
+    row against the full batch, bit for bit): the sweeps group pairs by expert, four to a sweep,
+    so the grouping changes with the batch while every pair's arithmetic must not;
+  * routing equals the oracle's for every row, and two rows' outputs match the oracle's
+    (src/graph/moe.c:497-622, src/runtime/moe.c:596-645) within the path's tolerance.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
+BF16_STEP = 2.0 ** -7
+
+
+def synthetic_iq2xxs(blocks, device, seed):
+    """Uniform grid / sign / scale bytes with a small positive fp16 block scale."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 66), dtype=torch.uint8, device=device, generator=gen)
+    d = (torch.rand(blocks, device=device, generator=gen) * 3.5e-4 + 1.0e-4).to(torch.float16)
+    raw[:, :2] = d.view(torch.uint8).reshape(blocks, 2)
+    return raw.reshape(-1)
+
+
+@pytest.fixture(scope="module")
+def layer_weights(gpu):
+    blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
+    routed = tuple(synthetic_iq2xxs(blocks, gpu, 1 + i) for i in range(3))
+    shared = tuple(synthetic_iq2xxs(INTERMEDIATE * HIDDEN // 256, gpu, 10 + i) for i in range(3))
+    return routed, shared
+
+
+def within_tolerance(got, want):
+    """1e-3 relative / 1e-5 absolute; beyond it only values one bf16 step apart (a sum that sits
+    on a rounding boundary), and few of them."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    outside = err > 1e-5 + 1e-3 * np.abs(want)
+    assert outside.mean() < 2e-2
+    assert np.all(err[outside] <= BF16_STEP * 1.001 * np.abs(want[outside]))
+
+
+def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
+    from yvex_amd import kernels as K
+    from yvex_amd.moe import MoeLayer
+    routed, shared = layer_weights
+    gen = torch.Generator(device=gpu)
+    gen.manual_seed(42)
+    x = torch.randn((ROWS, HIDDEN), device=gpu, generator=gen)
+    logits = torch.randn((ROWS, EXPERTS), device=gpu, generator=gen)
+    qt = K.IQ2_XXS
+    layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtypes=(qt, qt, qt),
+                     routed=routed, shared=shared, scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
+                     act_q8=True, max_rows=ROWS, device=gpu)
+
+    def run(rows_from, rows_to):
+        out = layer.run(x[rows_from:rows_to].contiguous(), logits[rows_from:rows_to].contiguous())
+        torch.cuda.synchronize()
+        assert int(layer.status.item()) == 0
+        return out[:rows_to - rows_from].clone(), layer.selected.clone(), layer.weights.clone()
+
+    full, selected, weights = run(0, ROWS)
+    again, _, _ = run(0, ROWS)
+    assert torch.equal(full.view(torch.int32), again.view(torch.int32))
+    assert torch.isfinite(full).all() and float(full.abs().max()) > 0.0
+    for lo, hi in ((0, 16), (16, 32), (5, 6), (29, 32)):
+        part, part_selected, _ = run(lo, hi)
+        assert torch.equal(part_selected, selected[lo:hi])
+        assert torch.equal(part.view(torch.int32), full[lo:hi].view(torch.int32)), (lo, hi)
+
+    # routing of every row against the oracle
+    host_logits = logits.cpu().numpy()
+    for r in range(ROWS):
+        rc, want_selected, want_weights, _ = oracle.moe_route(host_logits[r], None, TOPK, oracle.SIGMOID, True, 1.0)
+        assert rc == 0
+        assert np.array_equal(selected[r].cpu().numpy().astype(np.uint64), want_selected)
+        assert np.max(np.abs(weights[r].cpu().numpy() - want_weights)) <= 1e-6
+
+    # two rows through the CPU oracle with the same weights
+    picked = [0, 17]
+    want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                            qtypes=(oracle.IQ2_XXS,) * 3, routed=[t.cpu().numpy() for t in routed],
+                            shared=[t.cpu().numpy() for t in shared], inputs=x[picked].cpu().numpy(),
+                            logits=host_logits[picked], scoring=oracle.SIGMOID, normalize=True, scaling=1.0,
+                            limit=10.0, act_q8=True, threads=16)
+    got = full[picked].cpu().numpy()
+    assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
+    within_tolerance(got, want["combined"])
+
+
+def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
+    """2048 rows through the matrix-core kernels: the same bits twice, the first 32 rows against
+    the decode sweeps' result for them (another summation order: within tolerance), one row
+    against the oracle."""
+    from yvex_amd import kernels as K
+    from yvex_amd.moe import MoeLayer
+    routed, shared = layer_weights
+    rows = 2048
+    gen = torch.Generator(device=gpu)
+    gen.manual_seed(7)
+    x = torch.randn((rows, HIDDEN), device=gpu, generator=gen)
+    logits = torch.randn((rows, EXPERTS), device=gpu, generator=gen)
+    qt = K.IQ2_XXS
+    common = dict(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtypes=(qt, qt, qt),
+                  routed=routed, shared=shared, scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
+                  act_q8=True, device=gpu)
+    wide = MoeLayer(max_rows=rows, matrix_cores=True, **common)
+    first = wide.run(x, logits)[:rows].clone()
+    torch.cuda.synchronize()
+    assert int(wide.status.item()) == 0
+    second = wide.run(x, logits)[:rows].clone()
+    torch.cuda.synchronize()
+    assert torch.equal(first.view(torch.int32), second.view(torch.int32))
+    assert torch.isfinite(first).all()
+    selected = wide.selected.clone()
+    picked = 1000
+    keep = list(range(32)) + [picked]
+    wide_pairs = wide.pair_outputs.view(rows, TOPK, HIDDEN)[keep].cpu().numpy()    # [row, rank, column]
+    wide_shared = wide.shared_out[keep].cpu().numpy()
+    del wide
+
+    def close_by_row(got, want, scale):
+        """Few values beyond the path's tolerance (1e-3 relative / 1e-5 absolute), and those by no
+        more than two bf16 steps at the size of the row's largest terms: an intermediate value
+        that rounds the other way (the SwiGLU product, an expert's output) moves the results it
+        feeds by a step at its own size, whatever their own size is."""
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert (err > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
+        assert np.all(err <= 1e-5 + 1e-3 * np.abs(want) + 2 * BF16_STEP * scale)
+
+    def combined_close(got, want, pairs, shared_rows):
+        scale = np.abs(pairs).max(axis=2).sum(axis=1) + np.abs(shared_rows).max(axis=1)   # per row
+        close_by_row(got, want, scale[:, None])
+
+    narrow = MoeLayer(max_rows=32, **common)
+    sweeps = narrow.run(x[:32].contiguous(), logits[:32].contiguous())[:32].clone()
+    torch.cuda.synchronize()
+    assert int(narrow.status.item()) == 0 and torch.equal(narrow.selected, selected[:32])
+    # expert by expert
+    mine = wide_pairs[:32].reshape(32 * TOPK, HIDDEN)
+    close_by_row(mine, narrow.pair_outputs[:32 * TOPK].cpu().numpy(), np.abs(mine).max(axis=1)[:, None])
+    close_by_row(wide_shared[:32], narrow.shared_out[:32].cpu().numpy(),
+                 np.abs(wide_shared[:32]).max(axis=1)[:, None])
+    combined_close(first[:32].cpu().numpy(), sweeps.cpu().numpy(), wide_pairs[:32], wide_shared[:32])
+    want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                            qtypes=(oracle.IQ2_XXS,) * 3, routed=[t.cpu().numpy() for t in routed],
+                            shared=[t.cpu().numpy() for t in shared], inputs=x[[picked]].cpu().numpy(),
+                            logits=logits[[picked]].cpu().numpy(), scoring=oracle.SIGMOID, normalize=True,
+                            scaling=1.0, limit=10.0, act_q8=True, threads=16)
+    assert np.array_equal(selected[[picked]].cpu().numpy().astype(np.uint64), want["selected"])
+    combined_close(first[[picked]].cpu().numpy(), want["combined"], wide_pairs[32:], wide_shared[32:])
