@@ -100,6 +100,37 @@ def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
     assert_close(got, oracle.matvec(qt, w, rows, width, deq))
 
 
+@pytest.mark.parametrize("qtype,rows,width", [("Q8_0", 9600, 7168), ("IQ2_XXS", 37000, 7168)])
+def test_matvec_output_head_variant(gpu, oracle, qtype, rows, width):
+    """One Q8_K activation row against a matrix of 64 MB or more takes the variant with four
+    chunks of a row in flight (the output-head shape): every 97th row against the oracle's
+    integer path, exactly as the small shapes are checked."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec.head.{qtype}")
+    sample = np.arange(0, rows, 97)
+    distinct = g.weights(qt, len(sample) + 3, width).reshape(len(sample) + 3, -1)
+    row_bytes = distinct.shape[1]
+    assert rows * row_bytes >= 64 << 20
+    w = np.empty((rows, row_bytes), np.uint8)
+    w[:] = distinct[np.arange(rows) % 3 + len(sample)]       # filler rows
+    w[sample] = distinct[:len(sample)]
+    x = g.normal(width).reshape(1, width)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w.ravel(), gpu), qt, rows, width, act, input_q8=True, input_rows=1,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    want = oracle.q8_matvec(qt, np.ascontiguousarray(w[sample]).ravel(), len(sample), width, act_host, 1)
+    assert_close(got[:, sample], want, rel=1e-5, abs_=1e-5)
+    # filler rows repeat with period three: equal weights give equal bits
+    filler = np.setdiff1d(np.arange(rows), sample)
+    for k in range(3):
+        same = got[0, filler[filler % 3 == k]]
+        assert np.all(same.view(np.uint32) == same.view(np.uint32)[0])
+
+
 def test_matvec_additive_and_bf16(gpu, oracle):
     from yvex_amd import kernels as K
     g = oracle.Generator(7, "matvec.additive")
