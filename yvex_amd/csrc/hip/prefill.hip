@@ -1,28 +1,35 @@
 // Row-batch (prefill-width) grouped expert projections on the int8 matrix cores of gfx950.
 //
-// A work item is (bucket, tile of 128 ordered pairs, tile of weight rows). The workgroup's eight
-// waves split the weight rows, 16 each (four gate blocks and the four matching up blocks when the
-// SwiGLU is fused); every wave multiplies its rows by the item's 128 Q8_K activation rows with
-// V_MFMA_I32_16X16X64_I8. Two waves share a SIMD, so one wave's decode and scaling arithmetic
-// runs under the other's matrix instructions.
+// A work item is (bucket, tile of up to 128 ordered pairs, tile of 128 weight rows: 64 gate rows
+// and the 64 matching up rows when the SwiGLU is fused). The workgroup has four waves, one per
+// SIMD; each owns 32 weight rows and multiplies them by all of the item's Q8_K activation rows
+// with V_MFMA_I32_32X32X32_I8, so one activation fragment read from LDS feeds two matrix
+// instructions of 32 passes in total and the decode of a weight is shared by up to 128 tokens.
 //
-//   A operand (weights): each lane builds the 16 weights it owns straight into registers. The
-//       IQ2_XXS value of one weight is level * sign * (2s+1), up to 43 * 31 = 1333, so it is
+//   A operand (weights): built in registers. Lane (r, h) = (lane % 32, lane / 32) owns weight
+//       row r and the groups 4h .. 4h + 3 of the current superblock (128 columns); K chunk m of
+//       the superblock is, for that lane, the 16 weights 16 (m % 2) .. + 15 of group 4h + m / 2.
+//       The order of K inside a matrix instruction is free as long as both operands agree.
+//       The IQ2_XXS value of one weight is level * sign * (2s+1), up to 43 * 31 = 1333, so it is
 //       split into two int8 limbs, value = 128 * hi + lo with hi in [1, 11] and lo in
-//       [-120, 63]. For a given scale there are only three levels, so the six signed limb
-//       values of a group fit two registers and one V_PERM_B32 per four weights picks them:
-//       the selector byte of a weight is its level code (0..2) plus 4 when it is negative.
-//       Three small conflict-free LDS tables feed this: level codes of a codebook entry
-//       (8 bytes), sign selectors of a 7-bit sign field (8 bytes) and the limb words of a
-//       scale (16 bytes).
-//   B operand (activations): the 128 x 256 int8 block of the current superblock, copied from
-//       global memory straight into LDS (GLOBAL_LOAD_LDS_DWORDX4, no registers in between),
-//       double buffered. 16-byte piece c of token t sits at piece position c ^ (t % 16), so the
-//       16 lanes that read one fragment column together hit 16 different bank groups.
-//   C: per superblock two int32 accumulators per 16 x 16 block; T = 128 * C_hi + C_lo is the
-//       exact integer superblock sum of the reference's primitive
+//       [-120, 63], and every K chunk costs two matrix instructions. For one scale there are only
+//       three levels, so the six signed limb values of a group fit two registers and one
+//       V_PERM_B32 per four weights picks them: the selector byte of a weight is its level code
+//       (0..2) plus 4 when it is negative. Three LDS tables feed this: level codes of a codebook
+//       entry (8 bytes, 32 replicas: no two lanes of a half-wave share a bank), sign selectors
+//       of a 7-bit sign field (8 bytes, 16 replicas) and the limb words of a scale (16 bytes,
+//       16 replicas).
+//   B operand (activations): the tile's int8 blocks of one stage period (four superblocks of 32
+//       tokens, two of 64 or one of 128), copied from global memory straight into LDS
+//       (GLOBAL_LOAD_LDS_DWORDX4), double buffered. 16-byte piece c of token t sits at piece
+//       position c ^ (t % 16), so the 16 lanes that read one fragment column together hit 16
+//       different bank groups.
+//   C: per (superblock, 32-token block) two int32 accumulators of 32 x 32; T = 128 * C_hi + C_lo
+//       is the exact integer superblock sum of the reference's primitive
 //       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
 //       ((0.125 * d_w) * d_a) * T and summed over superblocks.
+//   Output: the wave's fp32 sums go through LDS once per item so that every store instruction
+//       writes whole 64-byte runs of an output row.
 //
 // Same inputs, outputs and rounding points as the decode-width sweeps in moe.hip
 // (src/backend/cuda/tensorcore.cu:378-702 is the reference's counterpart, unused there).
@@ -33,32 +40,32 @@
 namespace yvex {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 
+constexpr unsigned kRowWaves = 4u;
+constexpr unsigned kRowThreads = 64u * kRowWaves;
 constexpr unsigned kTileTokens = 128u;
 constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
-// LDS map. Codebook entry e owns the 256 bytes at 256 e: sixteen replicas of its 8 level codes
-// in the first half; the second half of entries 0-127 holds sixteen replicas of the sign
-// selectors of sign field e.
-constexpr unsigned kCodeBase = 0u;
-constexpr unsigned kSelBase = 128u;
-constexpr unsigned kLutBase = 65536u;                       // 16 scales x 16 replicas x 16 bytes
-constexpr unsigned kStageBase = kLutBase + 16u * 16u * 16u;
-constexpr unsigned kStageActs = kTileTokens * kActPitch;
-constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per token
-// Weight windows: per wave two slots; a slot holds, for each of the wave's 16 rows, the 80
-// bytes (five 16-byte pieces) around one superblock. Rows 0-11 lie at 80 r, rows 12-15 at
-// 1024 + 80 (r - 12): the two copies that fill a slot each write lane * 16.
-constexpr unsigned kWeightBase = kStageBase + 2u * kStageBytes;
-constexpr unsigned kWeightSlot = 1024u + 4u * 80u;
+// LDS map (absolute byte offsets; the dynamic allocation starts at 0, checked at kernel start).
+constexpr unsigned kCodeBase = 0u;                          // 256 entries x 32 replicas x 8 bytes
+constexpr unsigned kSelBase = 65536u;                       // 128 sign fields x 16 replicas x 8 bytes
+constexpr unsigned kLutBase = kSelBase + 128u * 16u * 8u;   // 16 scales x 16 replicas x 16 bytes
+constexpr unsigned kRowScaleBase = kLutBase + 16u * 16u * 16u;   // 4 waves x 2 x 32 floats
+constexpr unsigned kPairInfoBase = kRowScaleBase + kRowWaves * 2u * 128u;   // {out row, route weight} x 128
 // Item numbering: first full 128-pair tile of every bucket (257 words), then per class of last,
-// partial, tile (65-127, 33-64, 17-32, 1-16 pairs) a count and the list of its buckets (u16).
-constexpr unsigned kTileStartBase = kWeightBase + 8u * 2u * kWeightSlot;
+// partial, tile (65-127, 33-64, 1-32 pairs) a count and the list of its buckets (u16).
+constexpr unsigned kTileStartBase = kPairInfoBase + kTileTokens * 8u;
 constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
 constexpr unsigned kClassListBase = kClassCountBase + 16u;
-constexpr unsigned kTrashBase = kClassListBase + 4u * 256u * 2u;   // 256 bytes nobody reads
-// per pair of the item: {output row index, route weight}, read when the item publishes
-constexpr unsigned kPairInfoBase = kTrashBase + 256u;
-constexpr unsigned kMfmaLdsBytes = kPairInfoBase + kTileTokens * 8u;
+constexpr unsigned kTrashBase = kClassListBase + 3u * 256u * 2u;   // 256 bytes nobody reads
+constexpr unsigned kStageBase = (kTrashBase + 256u + 255u) & ~255u;
+constexpr unsigned kStageActs = kTileTokens * kActPitch;
+constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per slot
+// the finished tile on its way out: 128 tokens x (128 values + 4 of padding) fp32
+constexpr unsigned kOutPitch = 132u * 4u;
+constexpr unsigned kOutBytes = kTileTokens * kOutPitch;
+constexpr unsigned kMfmaLdsBytes = kStageBase + (2u * kStageBytes > kOutBytes ? 2u * kStageBytes : kOutBytes);
+static_assert(kMfmaLdsBytes <= 160u * 1024u, "one workgroup per compute unit");
 
 struct MfmaArgs {
     GroupedProblem pr;
@@ -77,10 +84,28 @@ __device__ __forceinline__ void lds_write_uint4(unsigned address, uint4 v)
     (void)v;
 #endif
 }
+__device__ __forceinline__ void lds_write_uint2(unsigned address, uint2 v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) uint2 *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
 __device__ __forceinline__ void lds_write_u32(unsigned address, unsigned v)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     *reinterpret_cast<__attribute__((address_space(3))) unsigned *>(address) = v;
+#else
+    (void)address;
+    (void)v;
+#endif
+}
+__device__ __forceinline__ void lds_write_u16(unsigned address, unsigned v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    *reinterpret_cast<__attribute__((address_space(3))) unsigned short *>(address) = (unsigned short)v;
 #else
     (void)address;
     (void)v;
@@ -95,15 +120,6 @@ __device__ __forceinline__ v4i lds_read_v4i(unsigned address)
 #else
     (void)address;
     return v4i{0, 0, 0, 0};
-#endif
-}
-__device__ __forceinline__ void lds_write_u16(unsigned address, unsigned v)
-{
-#if defined(__HIP_DEVICE_COMPILE__)
-    *reinterpret_cast<__attribute__((address_space(3))) unsigned short *>(address) = (unsigned short)v;
-#else
-    (void)address;
-    (void)v;
 #endif
 }
 __device__ __forceinline__ unsigned lds_read_u16(unsigned address)
@@ -127,7 +143,7 @@ __device__ __forceinline__ unsigned lds_read_u32(unsigned address)
 
 // Asynchronous copy global -> LDS (GLOBAL_LOAD_LDS): lane l of the wave writes `bytes` bytes at
 // lds_base + l * bytes; nothing passes through registers. Written as assembly so the compiler
-// does not put a conservative wait in front of every later LDS read: the caller waits with
+// does not put a conservative wait in front of every later LDS read: the kernel waits with
 // vmcnt(0) (loads retire in order, so the compiler's own counted waits stay correct) before
 // the barrier that publishes the data.
 __device__ __forceinline__ void copy_to_lds_16(const void *global, unsigned lds_base)
@@ -151,20 +167,6 @@ __device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_b
 #endif
 }
 
-// The same 16-byte copy for lanes 0-19 only (the other lanes neither read nor write).
-__device__ __forceinline__ void copy_to_lds_16_first20(const void *global, unsigned lds_base)
-{
-#if defined(__HIP_DEVICE_COMPILE__)
-    unsigned long long saved;
-    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xfffff\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-                 "global_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved) : "s"(lds_base), "v"(global) : "memory");
-#else
-    (void)global;
-    (void)lds_base;
-#endif
-}
-
 // Limb pair of one magnitude: low limb in bits 0-7, high limb in bits 8-15.
 __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
 {
@@ -175,21 +177,11 @@ __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
     return ((unsigned)lo & 255u) | (hi << 8);
 }
 
-__device__ __forceinline__ void lds_write_uint2(unsigned address, uint2 v)
-{
-#if defined(__HIP_DEVICE_COMPILE__)
-    *reinterpret_cast<__attribute__((address_space(3))) uint2 *>(address) = v;
-#else
-    (void)address;
-    (void)v;
-#endif
-}
-
 __device__ __forceinline__ void mfma_tables_fill()
 {
     // level codes: byte l of the entry is 0, 1 or 2 for level 8, 25 or 43 of weight l
-    for (unsigned index = threadIdx.x; index < 256u * 16u; index += blockDim.x) {
-        const uint2 m = iq2_magnitude_entry(index >> 4);
+    for (unsigned index = threadIdx.x; index < 256u * 32u; index += blockDim.x) {
+        const uint2 m = iq2_magnitude_entry(index >> 5);
         uint2 codes = make_uint2(0u, 0u);
 #pragma unroll
         for (unsigned l = 0; l < 4u; ++l) {
@@ -197,13 +189,12 @@ __device__ __forceinline__ void mfma_tables_fill()
             codes.x |= (a == 8u ? 0u : a == 25u ? 1u : 2u) << (8u * l);
             codes.y |= (b == 8u ? 0u : b == 25u ? 1u : 2u) << (8u * l);
         }
-        lds_write_uint2(kCodeBase + (index >> 4) * 256u + (index & 15u) * 8u, codes);
+        lds_write_uint2(kCodeBase + index * 8u, codes);
     }
     // sign selectors: byte l is 4 when weight l is negative (7 stored bits + parity)
     for (unsigned index = threadIdx.x; index < 128u * 16u; index += blockDim.x) {
         const uint2 m = iq2_signmask_entry(index >> 4);
-        lds_write_uint2(kSelBase + (index >> 4) * 256u + (index & 15u) * 8u,
-                        make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
+        lds_write_uint2(kSelBase + index * 8u, make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
     }
     // limb words of scale s: {+lo, -lo, +hi, -hi}, byte c = limb of level code c
     for (unsigned index = threadIdx.x; index < 16u * 16u; index += blockDim.x) {
@@ -229,117 +220,120 @@ struct MfmaItem {
     unsigned tokens, row_tile;
 };
 
-// Twelve aligned bytes that hold one 8-byte group record starting 0 or 2 bytes in.
-struct alignas(4) RawGroup {
-    unsigned x, y, z;
+// The aligned dwords around a lane's 32 code bytes of one superblock, and the dword that holds
+// the superblock's fp16 scale.
+struct RawCodes {
+    uint4 x0, x1;
+    unsigned x2, scale_word;
 };
 
-// The lane's four group records and block scale of one superblock of its weight row.
-struct Codes {
-    uint2 c[4];
-    unsigned scale16;
-};
-// Table words of the lane's sixteen weights in one K step.
-struct Lookup {
-    uint2 codes[2], signs[2];
-    uint4 limbs;
+__device__ __forceinline__ uint4 load_uint4_dword_aligned(const unsigned char *p)
+{
+    uint4 v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
+    return v;
+}
+__device__ __forceinline__ unsigned load_u32_aligned(const unsigned char *p)
+{
+    return *reinterpret_cast<const unsigned *>(p);
+}
+
+// Where in the 8 NTB slots of a superblock each piece of the next superblock's decode runs:
+// settle (records out of the loaded dwords, row scale to LDS), then per group g the nine table
+// lookups L(g), the selector words S(g), and per K chunk m the permutes P(m) that overwrite the
+// chunk's operands once the last token block has used them.
+template <unsigned NTB>
+struct DecodePlan {
+    static constexpr unsigned kSlots = 8u * NTB;
+    static constexpr unsigned lookup_slot(unsigned g)
+    {
+        return NTB == 4u ? 1u + 6u * g : NTB == 2u ? 2u * g : g;
+    }
+    static constexpr unsigned select_slot(unsigned g)
+    {
+        return NTB == 4u ? 4u + 6u * g : NTB == 2u ? 2u * g + 2u : g + 2u;
+    }
+    static constexpr unsigned permute_slot(unsigned m)
+    {
+        // after the last token block's matrix instructions on chunk m, and after S(m / 2)
+        const unsigned last_use = kSlots - 8u + m;
+        const unsigned ready = select_slot(m / 2u) + 1u;
+        return last_use > ready ? last_use : ready;
+    }
 };
 
-// One work item with NB live 16-token blocks (NB is 1, 2, 4 or 8). Eight waves, two per SIMD, each
-// owning one 16-row block.
+// One work item with NTB live 32-token blocks (NTB is 1, 2 or 4).
 //
 // The stage in LDS holds 128 "slots" of 256 activation bytes + one scale. An item with fewer than
-// 128 tokens fills them with S consecutive superblocks of its NB * 16 tokens (slot = superblock
-// within the period * NB * 16 + token), so that every period between two barriers carries about
-// the same matrix work and the same copies whatever NB is.
+// 97 tokens fills them with S = 4 / NTB consecutive superblocks of its NTB * 32 tokens (slot =
+// superblock within the period * NTB * 32 + token), so that every period between two barriers
+// carries the same copies and 32 "time slots" of two matrix instructions each.
 //
-// A step is one superblock. Its instruction stream is laid out by hand as 4 * NB slots of two
-// matrix instructions (low and high limb of one K step of one token block), and between them,
-// a few vector instructions at a time, everything else: the scaling of the previous token
-// block's integer sums into the fp32 accumulators, the table lookups and byte permutes that
-// build the next superblock's A operands, the LDS reads of the next token block's fragments.
-// The loop body holds D steps back to back in one basic block (requests past the end are
-// clamped, and steps past the end run with a zero row scale), so the compiler's wait counts stay
-// exact and accumulators never leave registers.
-template <bool FUSED_UP, unsigned NB>
-__device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
+// Time slot (u, tb, m) = superblock u of the period, token block tb, K chunk m. Around its two
+// matrix instructions (low and high limb) the slot carries, a few instructions at a time, the
+// rest of the work: the LDS read of the activation fragment two slots ahead, the scaling of two
+// rows of the previous token block's integer sums into the fp32 accumulators, one piece of the
+// decode of the next superblock's weights, and this period's share of the copies and loads.
+// The loop body is one period in one basic block (requests past the end are clamped, and
+// superblocks past the end run with a zero row scale), so the compiler's wait counts stay exact
+// and accumulators never leave registers.
+template <bool FUSED_UP, unsigned NTB>
+__device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
-    constexpr unsigned kWaves = 8u;
-    constexpr unsigned S = NB >= 8u ? 1u : NB == 4u ? 2u : 4u;   // superblocks per stage period
-    constexpr unsigned D = S < 2u ? 2u : S;                      // steps per loop turn (even)
-    constexpr unsigned T = NB * 16u;                             // token slots of one superblock
-    constexpr unsigned kStagedSlots = S * T;
+    constexpr unsigned S = 4u / NTB;                 // superblocks per stage period
+    constexpr unsigned T = NTB * 32u;                // token slots of one superblock
+    constexpr unsigned kSbSlots = 8u * NTB;
+    constexpr unsigned kPeriodSlots = 32u;
+    constexpr unsigned kBarrierSlot = kPeriodSlots - 3u;
+    using Plan = DecodePlan<NTB>;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const unsigned li = lane & 15u, kb = lane >> 4;
+    const unsigned r = lane & 31u, h = lane >> 5;
     constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
-    const unsigned code_lane = kCodeBase + (lane & 15u) * 8u;
-    const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
-    const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
     const unsigned superblocks = a.width >> 8;
     const unsigned last = superblocks - 1u;
 
-    // ---- the weight row of this lane: waves 0-3 hold gate blocks and waves 4-7 the matching up
-    // blocks when the SwiGLU is fused ----
-    unsigned out_row_base;
-    bool is_up = false;
-    if constexpr (FUSED_UP) {
-        out_row_base = it.row_tile * kItemRows + (wave & 3u) * 16u;
-        is_up = wave >= 4u;
-    } else {
-        out_row_base = it.row_tile * kItemRows + wave * 16u;
-    }
-    auto row_pointer = [&](unsigned r) {     // weight row r of the wave's 16
-        unsigned row = out_row_base + r;
+    // ---- the weight row of this lane: rows 0-15 of a wave are gate rows and rows 16-31 the
+    // matching up rows when the SwiGLU is fused ----
+    const unsigned char *weight_row;
+    {
+        unsigned row;
+        bool is_up = false;
+        if constexpr (FUSED_UP) {
+            row = it.row_tile * kItemRows + wave * 16u + (r & 15u);
+            is_up = r >= 16u;
+        } else {
+            row = it.row_tile * kItemRows + wave * 32u + r;
+        }
         if (row >= a.out_rows) row = a.out_rows - 1u;
-        return is_up
+        weight_row = is_up
             ? pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
             : pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
-    };
-    // Superblocks are 66 bytes, so they start on 2-byte boundaries, and vector loads that are
-    // not dword-aligned run at less than half rate. The wave copies, for each of its rows, the
-    // aligned 68 bytes that hold the superblock into its LDS slot, as five 16-byte pieces (the
-    // fifth one ends with those 68 bytes, so nothing past the dword that holds the superblock's
-    // last byte is touched: an aligned dword with a valid byte lies in a mapped page). Two
-    // copies fill a slot: lanes 0-59 of the first serve rows 0-11, lanes 0-19 of the second
-    // rows 12-15. Every row is fetched once per step by five lanes instead of by all four lane
-    // groups record by record: the memory pipeline's cost per instruction grows with the number
-    // of cache lines it touches.
-    const unsigned row_misalign = (unsigned)(unsigned long long)row_pointer(li) & 3u;   // of the lane's own row
-    const unsigned lane_group = kb >> 1;                      // groups 2 ks + lane_group
-    const unsigned char *window_from[2];    // aligned row start + piece offset, of the row this lane copies
-    unsigned window_misalign[2];
-#pragma unroll
-    for (unsigned c = 0; c < 2u; ++c) {
-        const unsigned served = c == 0u ? (lane < 60u ? lane : 0u) : (lane < 20u ? 60u + lane : 60u);
-        const unsigned piece_index = served % 5u;
-        const unsigned char *from = row_pointer(served / 5u);
-        window_misalign[c] = (unsigned)(unsigned long long)from & 3u;
-        window_from[c] = from - window_misalign[c] + (piece_index < 4u ? 16u * piece_index : 52u);
     }
-    const unsigned weight_slots = kWeightBase + wave * 2u * kWeightSlot;
-    const unsigned row_at = li < 12u ? li * 80u : 1024u + (li - 12u) * 80u;   // of the lane's row in a slot
-    constexpr unsigned kFetchPieces = 2u;
-    auto fetch_piece = [&](unsigned slot, unsigned sb, unsigned c) {
+    // Superblocks are 66 bytes, so the lane's 32 code bytes start on 2-byte boundaries, and vector
+    // loads that are not dword-aligned run at less than half rate: the lane loads the aligned
+    // dwords around them (two 16-byte loads and a ninth dword, which repeats the eighth when the
+    // codes are aligned so that nothing past the dword holding the last code byte is touched)
+    // and shifts the records into place.
+    const unsigned row_misalign = (unsigned)(unsigned long long)weight_row & 3u;
+    const unsigned char *row_aligned = weight_row - row_misalign;
+    const unsigned code_offset = row_misalign + 2u + 32u * h;       // of superblock 0's codes from row_aligned
+    auto load_raw = [&](unsigned sb) {
         sb = sb < last ? sb : last;
-        const unsigned char *from = window_from[c] + ((window_misalign[c] + sb * 66u) & ~3u);
-        const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane((int)(weight_slots + slot * kWeightSlot + c * 1024u));
-        if (c == 0u) copy_to_lds_16(from, to);
-        else copy_to_lds_16_first20(from, to);
+        RawCodes out;
+        const unsigned at = code_offset + sb * 66u;
+        const unsigned char *from = row_aligned + (at & ~3u);
+        out.x0 = load_uint4_dword_aligned(from);
+        out.x1 = load_uint4_dword_aligned(from + 16u);
+        out.x2 = load_u32_aligned(from + ((at & 3u) ? 32u : 28u));
+        out.scale_word = load_u32_aligned(row_aligned + ((row_misalign + sb * 66u) & ~3u));
+        return out;
     };
-    auto fetch_codes = [&](unsigned slot, unsigned sb) {
-#pragma unroll
-        for (unsigned c = 0; c < kFetchPieces; ++c) fetch_piece(slot, sb, c);
-    };
-    // The first two superblocks of the weight rows are asked for before anything else: their
-    // trip to HBM runs under the index loads and copies of the activation side below.
-    fetch_codes(0u, 0u);
-    fetch_codes(1u, 1u);
 
-    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + kWaves, ... ----
+    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + 4, ... ----
     // Lane l of a group moves piece position l % 16 of slot 4 g + l / 16; LDS receives the wave's
     // 64 pieces back to back, so the swizzle is applied on the global side.
-    constexpr unsigned kCopies = kStagedSlots / (4u * kWaves);
+    constexpr unsigned kCopies = kTileTokens / (4u * kRowWaves);
     auto token_row = [&](unsigned token) {
         const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
         const unsigned long long ordered = it.pair0 + live;
@@ -351,22 +345,25 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
     unsigned copy_step[kCopies];            // superblock of the slot within its period
 #pragma unroll
     for (unsigned j = 0; j < kCopies; ++j) {
-        const unsigned slot = 4u * (wave + kWaves * j) + (lane >> 4);
+        const unsigned slot = 4u * (wave + kRowWaves * j) + (lane >> 4);
         const unsigned token = slot % T;
         copy_step[j] = slot / T;
         copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
     }
-    // Waves 0 and 1 also copy the 128 slot scales. The other waves run the same instruction on
-    // one address for all lanes (one cache line: next to free) into bytes nobody reads, which is
-    // cheaper than a branch around the copy.
-    const unsigned scale_slot = wave < 2u ? 64u * wave + lane : 0u;
-    const unsigned char *scale_from = token_row(scale_slot % T);
-    const unsigned scale_step = scale_slot / T;
+    // Waves 0 and 1 also copy the 128 slot scales, laid out [superblock][token % 32][token block]
+    // so that a lane reads the scales of its NTB tokens with one LDS read. The other waves run the
+    // same instruction on one address for all lanes (one cache line: next to free) into bytes
+    // nobody reads, which is cheaper than a branch around the copy.
+    const unsigned char *scale_from;
+    unsigned scale_step;
+    {
+        const unsigned index = wave < 2u ? 64u * wave + lane : 0u;
+        const unsigned within = index % T;
+        scale_step = index / T;
+        scale_from = token_row((within % NTB) * 32u + within / NTB);
+    }
     const unsigned scale_to = wave < 2u ? kStageActs + wave * 256u : 0xffffffffu;
 
-    // The copies and loads of a step are issued one piece at a time between its matrix
-    // instructions: a burst of them fills the memory pipeline's queue and holds the wave, and
-    // with it its matrix instructions, until the queue drains.
     constexpr unsigned kCopyPieces = kCopies + 1u;
     auto copy_piece = [&](unsigned period, unsigned stage, unsigned j) {
         const unsigned base = kStageBase + stage * kStageBytes;
@@ -374,7 +371,7 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             unsigned sb = period * S + copy_step[j];
             sb = sb < last ? sb : last;
             copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
-                           (unsigned)__builtin_amdgcn_readfirstlane((int)(base + (wave + kWaves * j) * 1024u)));
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(base + (wave + kRowWaves * j) * 1024u)));
         } else {
             unsigned sb = period * S + scale_step;
             sb = sb < last ? sb : last;
@@ -383,114 +380,85 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
                               (int)(scale_to != 0xffffffffu ? base + scale_to : kTrashBase)));
         }
     };
-    auto copy_activations = [&](unsigned period, unsigned stage) {
+
+    // ---- decode state of the superblock after the current one ----
+    const unsigned code_lane = kCodeBase + (lane & 31u) * 8u;
+    const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
+    const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
+    const unsigned row_scale_at = kRowScaleBase + wave * 256u;      // + 128 for odd superblocks
+    unsigned grids[4], aux[4];
+    uint2 codes[2][4], signs[2][4];      // [g & 1]: of the groups whose lookups are in flight
+    uint4 limbs[4];                      // limb words per group
+    unsigned sel[4][8];                  // selector words per group
+    v4i a_lo[8], a_hi[8];                // A operands of the current superblock, per K chunk
+
+    // records out of the loaded dwords, and the row's scale into LDS for the lanes that hold
+    // this row's sums (zero past the end: such superblocks add nothing)
+    auto settle = [&](const RawCodes &raw, unsigned sb) {
+        const unsigned clamped = sb < last ? sb : last;
+        const unsigned shift = (code_offset + clamped * 66u) & 3u;
+        const unsigned w[9] = {raw.x0.x, raw.x0.y, raw.x0.z, raw.x0.w, raw.x1.x, raw.x1.y, raw.x1.z, raw.x1.w, raw.x2};
 #pragma unroll
-        for (unsigned j = 0; j < kCopyPieces; ++j) copy_piece(period, stage, j);
-    };
-    // Records of superblock sb out of the slot fetch_codes(slot, sb) filled. With o = (row start
-    // + 2 sb) mod 4 (0 or 2) the fp16 scale sits o bytes into the window and the record of group
-    // G at o + 2 + 8 G: in dwords 2 G (+1 when o is 2), shifted by 2 bytes when o is 0. Window
-    // dword 16 is the last dword of the fifth piece.
-    auto settle_codes = [&](unsigned slot, unsigned sb) {
-        sb = sb < last ? sb : last;
-        Codes out;
-        const unsigned o = (row_misalign + 2u * sb) & 3u;
-        const unsigned shift = (o + 2u) & 3u;
-        const unsigned row_base = weight_slots + slot * kWeightSlot + row_at;
-        const unsigned first = row_base + 8u * lane_group + (o & 2u) * 2u;    // dword 2 g (+1) of the window
-        out.scale16 = (lds_read_u32(row_base) >> (8u * o)) & 0xffffu;
-#pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) {
-            unsigned x, y, z;
-            if (ks < 3u) {
-                x = lds_read_u32(first + 16u * ks);
-                y = lds_read_u32(first + 16u * ks + 4u);
-                z = lds_read_u32(first + 16u * ks + 8u);
-            } else {
-                // dwords 12 + 2 g (+1) and the two behind it; 16 lives 12 bytes further on, and
-                // 17 is never part of a record (it is read as 16 and shifted out)
-                const unsigned d0 = 12u + 2u * lane_group + (o >> 1);
-                const unsigned d1 = d0 + 1u, d2 = d0 + 2u < 16u ? d0 + 2u : 16u;
-                x = lds_read_u32(row_base + 4u * d0);
-                y = lds_read_u32(row_base + 4u * d1 + (d1 == 16u ? 12u : 0u));
-                z = lds_read_u32(row_base + 4u * d2 + (d2 == 16u ? 12u : 0u));
-            }
-            out.c[ks].x = __builtin_amdgcn_alignbyte(y, x, shift);
-            out.c[ks].y = __builtin_amdgcn_alignbyte(z, y, shift);
+        for (unsigned g = 0; g < 4u; ++g) {
+            grids[g] = __builtin_amdgcn_alignbyte(w[2u * g + 1u], w[2u * g], shift);
+            aux[g] = __builtin_amdgcn_alignbyte(w[2u * g + 2u], w[2u * g + 1u], shift);
         }
-        return out;
+        const unsigned scale_shift = ((row_misalign + clamped * 66u) & 3u) * 8u;
+        const unsigned scale16 = (raw.scale_word >> scale_shift) & 0xffffu;
+        const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(scale16) : 0.0f;
+        lds_write_u32(row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
     };
-    // the lane's sixteen weights of K step ks: subgroups 2 (kb & 1) and 2 (kb & 1) + 1 of its group
-    auto lookup = [&](const Codes &codes, unsigned ks) {
-        Lookup out;
-        const unsigned grids = codes.c[ks].x >> (16u * (kb & 1u));
-        const unsigned aux = codes.c[ks].y;
-        const unsigned signs = aux >> (14u * (kb & 1u));
-        out.codes[0] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0400u));
-        out.codes[1] = lds_read_uint2(__builtin_amdgcn_perm(grids, code_lane, 0x0c0c0500u));
-        out.signs[0] = lds_read_uint2(((signs << 8) & 0x7f00u) | sel_lane);
-        out.signs[1] = lds_read_uint2(((signs << 1) & 0x7f00u) | sel_lane);
-        out.limbs = lds_read_uint4(((aux >> 20) & 0xf00u) | lut_lane);
-        return out;
-    };
-    auto weights_from_lookup = [&](const Lookup &lk, v4i &a_lo, v4i &a_hi) {
-        const unsigned s0 = lk.codes[0].x | lk.signs[0].x, s1 = lk.codes[0].y | lk.signs[0].y;
-        const unsigned s2 = lk.codes[1].x | lk.signs[1].x, s3 = lk.codes[1].y | lk.signs[1].y;
-        a_lo = v4i{(int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s0),
-                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s1),
-                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s2),
-                   (int)__builtin_amdgcn_perm(lk.limbs.y, lk.limbs.x, s3)};
-        a_hi = v4i{(int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s0),
-                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s1),
-                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s2),
-                   (int)__builtin_amdgcn_perm(lk.limbs.w, lk.limbs.z, s3)};
-    };
-    // fp32 scales of C rows 4 kb + r of superblock sb (zero past the end: such steps add nothing)
-    auto row_scales = [&](const Codes &codes, unsigned sb, float (&out)[4]) {
-        const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(codes.scale16) : 0.0f;
+    auto lookup = [&](unsigned g) {
 #pragma unroll
-        for (unsigned r = 0; r < 4u; ++r) out[r] = __shfl(mine, (int)(4u * kb + r), 64);
+        for (unsigned j = 0; j < 4u; ++j) {
+            codes[g & 1u][j] = lds_read_uint2(__builtin_amdgcn_perm(grids[g], code_lane, 0x0c0c0400u + (j << 8)));
+            const unsigned field = j == 0u ? aux[g] << 7 : j == 1u ? aux[g] : aux[g] >> (7u * j - 7u);
+            signs[g & 1u][j] = lds_read_uint2((field & 0x3f80u) | sel_lane);
+        }
+        limbs[g] = lds_read_uint4(((aux[g] >> 20) & 0xf00u) | lut_lane);
     };
-    // LDS offsets of this lane's fragment pieces: piece 4 ks + kb of slot 16 b + li
-    unsigned piece[4];
+    auto select = [&](unsigned g) {
 #pragma unroll
-    for (unsigned ks = 0; ks < 4u; ++ks) piece[ks] = li * kActPitch + (((4u * ks + kb) ^ li) << 4);
+        for (unsigned j = 0; j < 4u; ++j) {
+            sel[g][2u * j] = codes[g & 1u][j].x | signs[g & 1u][j].x;
+            sel[g][2u * j + 1u] = codes[g & 1u][j].y | signs[g & 1u][j].y;
+        }
+    };
+    auto permute = [&](unsigned m) {
+        const unsigned g = m >> 1, first = 4u * (m & 1u);
+        a_lo[m] = v4i{(int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first]),
+                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 1u]),
+                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 2u]),
+                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 3u])};
+        a_hi[m] = v4i{(int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first]),
+                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 1u]),
+                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 2u]),
+                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 3u])};
+    };
 
-    float acc[NB][4];
-#pragma unroll
-    for (unsigned tb = 0; tb < NB; ++tb)
-#pragma unroll
-        for (unsigned r = 0; r < 4u; ++r) acc[tb][r] = 0.0f;
-
-    // ---- pipeline state; every index below is a compile-time constant after unrolling ----
-    // (weight windows: LDS slot x & 1 holds superblock x, copied two steps before its records
-    // are taken out)
-    v4i a_lo[2][4], a_hi[2][4];      // [x & 1]: A operands of superblock x, all four K steps
-    float rs[2][4];                  // [x & 1]: row scales of superblock x
-    v4i frags[4];                    // B fragment of K step ks: re-requested for the next token block
-                                     // as soon as the current one has used it
-    float ts[2];                     // [g & 1]: activation scale of token block g (counted over steps)
-    v4i sum_lo[2], sum_hi[2];        // [g & 1]: its integer sums, scaled one token block later
-    // Fragment addresses: stage base + piece offset live in registers (kept opaque so that the
-    // block offset, under 32 KB, stays the instruction's immediate instead of a separate OR).
-    unsigned piece_at[4];
+    // ---- activation fragments: piece 8 h + m of slot r (+ 32 tb + T u) ----
+    unsigned piece_at[8];
     auto enter_stage = [&](unsigned base) {
 #pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) {
-            piece_at[ks] = base + piece[ks];
-            asm volatile("" : "+v"(piece_at[ks]));
+        for (unsigned m = 0; m < 8u; ++m) {
+            // kept opaque so that the slot offset stays the instruction's immediate
+            piece_at[m] = base + r * kActPitch + ((((8u * h) ^ (r & 15u)) ^ m) << 4);
+            asm volatile("" : "+v"(piece_at[m]));
         }
     };
-    auto request = [&](unsigned block, unsigned ks) {   // block: 16-slot block of the entered stage
-        frags[ks] = lds_read_v4i(piece_at[ks] + block * 16u * kActPitch);
-    };
-    auto request_scale = [&](unsigned base, unsigned block, unsigned g) {
-        ts[g & 1u] = __uint_as_float(lds_read_u32(base + kStageActs + 4u * (block * 16u + li)));
-    };
-    auto stage_of = [&](unsigned step) { return kStageBase + ((step / S) & 1u) * kStageBytes; };
+    auto stage_base = [&](unsigned period) { return kStageBase + (period & 1u) * kStageBytes; };
 
-    __syncthreads();   // every wave is done with the previous item's stages
-    copy_activations(0u, 0u);
+    // ---- prologue ----
+    RawCodes raw[S];
+    // The first superblocks of the weight rows are asked for before anything else: their trip to
+    // HBM runs under the index loads and copies of the activation side.
+    RawCodes first_raw = load_raw(0u);
+#pragma unroll
+    for (unsigned x = 1; x <= S; ++x) raw[x % S] = load_raw(x);
+
+    __syncthreads();   // every wave is done with the previous item's stage and output tile
+#pragma unroll
+    for (unsigned j = 0; j < kCopyPieces; ++j) copy_piece(0u, 0u, j);
     // where each pair's results go and its route weight, for the publishing pass
     if (tid < kTileTokens && tid < it.tokens) {
         const unsigned long long ordered = it.pair0 + tid;
@@ -499,134 +467,160 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
         const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
         lds_write_uint2(kPairInfoBase + tid * 8u, make_uint2((unsigned)out_index, __float_as_uint(route_weight)));
     }
-    {
-        __builtin_amdgcn_s_waitcnt(0x0f70u);   // vmcnt(0): every copy above has landed
-        const Codes first = settle_codes(0u, 0u);
-        // the slot's reads have returned before it is refilled
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        fetch_codes(0u, 2u);
-        __syncthreads();
-        enter_stage(stage_of(0u));
+    settle(first_raw, 0u);
 #pragma unroll
-        for (unsigned ks = 0; ks < 3u; ++ks) request(0u, ks);
-        request_scale(stage_of(0u), 0u, 0u);
-        row_scales(first, 0u, rs[0]);
-        Lookup lk[4];
-#pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) lk[ks] = lookup(first, ks);
-#pragma unroll
-        for (unsigned ks = 0; ks < 4u; ++ks) weights_from_lookup(lk[ks], a_lo[0][ks], a_hi[0][ks]);
+    for (unsigned g = 0; g < 4u; ++g) {
+        lookup(g);
+        select(g);
     }
-    sum_lo[1] = v4i{0, 0, 0, 0};
-    sum_hi[1] = v4i{0, 0, 0, 0};
-    ts[1] = 0.0f;
 #pragma unroll
-    for (unsigned r = 0; r < 4u; ++r) rs[1][r] = 0.0f;
+    for (unsigned m = 0; m < 8u; ++m) permute(m);
+    __builtin_amdgcn_s_waitcnt(0x0070u);   // vmcnt(0) lgkmcnt(0): the copies above have landed
+    __syncthreads();
 
-    // scaling of the integer sums of token block g - 1 into the accumulators, one C row per call
-    auto scale_row = [&](unsigned g_prev, unsigned tb_prev, float row_scale, float token_scale, unsigned r) {
-        const int total = (sum_hi[g_prev & 1u][r] << 7) + sum_lo[g_prev & 1u][r];
-        acc[tb_prev][r] = __builtin_fmaf(row_scale * token_scale, (float)total, acc[tb_prev][r]);
+    float acc[NTB][16];
+#pragma unroll
+    for (unsigned tb = 0; tb < NTB; ++tb)
+#pragma unroll
+        for (unsigned i = 0; i < 16u; ++i) acc[tb][i] = 0.0f;
+    float rs[16];                    // row scales of the rows this lane holds sums of
+#pragma unroll
+    for (unsigned i = 0; i < 16u; ++i) rs[i] = 0.0f;
+    float ts[NTB];                   // activation scales of this lane's token per token block
+    float ts_before = 0.0f;          // of the last token block of the superblock before
+#pragma unroll
+    for (unsigned tb = 0; tb < NTB; ++tb) ts[tb] = 0.0f;
+    v16i sum_lo[2], sum_hi[2];       // [phase & 1]: integer sums of a token block, scaled one phase later
+#pragma unroll
+    for (unsigned i = 0; i < 16u; ++i) {
+        sum_lo[1][i] = 0;
+        sum_hi[1][i] = 0;
+    }
+    v4i frag[2];                     // [slot & 1]: re-requested for two slots on as soon as it is used
+    enter_stage(stage_base(0u));
+    frag[0] = lds_read_v4i(piece_at[0]);
+    frag[1] = lds_read_v4i(piece_at[1]);
+
+    auto scale_rows = [&](unsigned parity, unsigned tb_of, float token_scale, unsigned m) {
+#pragma unroll
+        for (unsigned i = 2u * m; i < 2u * m + 2u; ++i) {
+            const int total = (sum_hi[parity][i] << 7) + sum_lo[parity][i];
+            acc[tb_of][i] = __builtin_fmaf(rs[i] * token_scale, (float)total, acc[tb_of][i]);
+        }
     };
 
-    const unsigned steps = (superblocks + D - 1u) / D * D;
-    for (unsigned t0 = 0; t0 < steps; t0 += D) {
+    const unsigned periods = (superblocks + S - 1u) / S;
+    for (unsigned period = 0; period < periods; ++period) {
+        const unsigned base = stage_base(period);
 #pragma unroll
-        for (unsigned u = 0; u < D; ++u) {
-            const unsigned t = t0 + u;                    // this step's superblock; u == t % D
-            const unsigned base = stage_of(t);
-            // the next superblock's records leave the ring; the one D steps on enters it piece
-            // by piece below, behind this period's copies
-            // (copies are invisible to the compiler's wait counts; they complete in order, so
-            // waiting until only the copies issued after a slot's two are in flight covers it)
-            constexpr unsigned kAfterPeriodStart = 2u + kCopyPieces;
-            if (((u + D - 1u) % D) % S == 0u)
-                __builtin_amdgcn_s_waitcnt(0x0f70u | (kAfterPeriodStart & 15u) | ((kAfterPeriodStart >> 4) << 14));
-            else
-                __builtin_amdgcn_s_waitcnt(0x0f72u);
-            const Codes next = settle_codes((u + 1u) & 1u, t + 1u);
-            constexpr unsigned kSlots = 4u * NB;
-            const unsigned memory_pieces = (u % S == 0u ? kCopyPieces : 0u) + kFetchPieces;
-            float rs_before[4];                           // of the step before this one
+        for (unsigned u = 0; u < S; ++u) {
+            const unsigned sb = period * S + u;           // this superblock
 #pragma unroll
-            for (unsigned r = 0; r < 4u; ++r) rs_before[r] = rs[(u + 1u) & 1u][r];
-            row_scales(next, t + 1u, rs[(u + 1u) & 1u]);
-            Lookup lk[4];
-            __builtin_amdgcn_sched_barrier(0);
+            for (unsigned tb = 0; tb < NTB; ++tb) {
+                const unsigned phase = u * NTB + tb;
+                const unsigned parity = phase & 1u;
 #pragma unroll
-            for (unsigned tb = 0; tb < NB; ++tb) {
-                const unsigned g = u * NB + tb;           // parity of the global token-block count
-                const float ts_before = ts[(g + 1u) & 1u];   // of the token block before this one
+                for (unsigned m = 0; m < 8u; ++m) {
+                    const unsigned slot = phase * 8u + m;         // within the period
+                    const unsigned sb_slot = tb * 8u + m;         // within the superblock
+                    // ---- two matrix instructions ----
+                    const v4i b = frag[slot & 1u];
+                    if (m == 0u) {
+                        v16i zero;
 #pragma unroll
-                for (unsigned ks = 0; ks < 4u; ++ks) {
-                    const unsigned q = tb * 4u + ks;
-                    // across a period end the next token block's scale and fragments are
-                    // requested after the barrier instead
-                    const bool next_here = tb + 1u < NB || u % S != S - 1u;
-                    const unsigned next_block = (u % S) * NB + tb + 1u;
-                    if (ks == 0u && next_here) request_scale(base, next_block, g + 1u);
-                    const v4i b = frags[ks];
-                    if (ks == 0u) {
-                        sum_lo[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[u & 1u][0], b, v4i{0, 0, 0, 0}, 0, 0, 0);
-                        sum_hi[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[u & 1u][0], b, v4i{0, 0, 0, 0}, 0, 0, 0);
+                        for (unsigned i = 0; i < 16u; ++i) zero[i] = 0;
+                        sum_lo[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo[0], b, zero, 0, 0, 0);
+                        sum_hi[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi[0], b, zero, 0, 0, 0);
                     } else {
-                        sum_lo[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo[u & 1u][ks], b, sum_lo[g & 1u], 0, 0, 0);
-                        sum_hi[g & 1u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi[u & 1u][ks], b, sum_hi[g & 1u], 0, 0, 0);
+                        sum_lo[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo[m], b, sum_lo[parity], 0, 0, 0);
+                        sum_hi[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi[m], b, sum_hi[parity], 0, 0, 0);
                     }
-                    // fragment ks - 1 is free now: its next use is one token block on (fragment 3
-                    // of this token block still has to be asked for when ks is 0)
-                    if (ks == 0u) request(next_block - 1u, 3u);
-                    else if (next_here) request(next_block, ks - 1u);
-                    // one C row of the previous token block (the previous step's last one for tb 0)
-                    scale_row(g + 1u, tb ? tb - 1u : NB - 1u, tb ? rs[u & 1u][ks] : rs_before[ks], ts_before, ks);
-                    // this step's copies and loads, spread evenly
-#pragma unroll
-                    for (unsigned v = 0; v < kCopyPieces + kFetchPieces; ++v) {
-                        if (v >= memory_pieces || v * kSlots / memory_pieces != q) continue;
-                        const unsigned first_fetch = memory_pieces - kFetchPieces;
-                        if (v < first_fetch) copy_piece(t / S + 1u, (t / S + 1u) & 1u, v);
-                        else {
-                            // the reads that took this slot's records out have returned
-                            if (v == first_fetch) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                            fetch_piece((u + 1u) & 1u, t + 3u, v - first_fetch);
-                        }
-                    }
-                    // the next superblock's A operands: eight pieces (lookups L, permutes W of the
-                    // four K steps) spread evenly over the slots, every W at least two slots
-                    // behind its L
-#pragma unroll
-                    for (unsigned i = 0; i < 8u; ++i) {
-                        if (i * NB / 2u != q) continue;
-                        unsigned is_w, k;
-                        if (NB >= 8u) {
-                            is_w = i & 1u;
-                            k = i >> 1;
+                    // ---- this superblock's token scales at its start ----
+                    if (sb_slot == 0u) {
+                        ts_before = ts[NTB - 1u];
+                        const unsigned at = base + kStageActs + (u * T + r * NTB) * 4u;
+                        if constexpr (NTB == 4u) {
+                            const uint4 v = lds_read_uint4(at);
+                            ts[0] = __uint_as_float(v.x);
+                            ts[1] = __uint_as_float(v.y);
+                            ts[2] = __uint_as_float(v.z);
+                            ts[3] = __uint_as_float(v.w);
+                        } else if constexpr (NTB == 2u) {
+                            const uint2 v = lds_read_uint2(at);
+                            ts[0] = __uint_as_float(v.x);
+                            ts[1] = __uint_as_float(v.y);
                         } else {
-                            is_w = (i == 2u || i == 4u || i >= 6u) ? 1u : 0u;
-                            k = is_w ? (i == 2u ? 0u : i == 4u ? 1u : i - 4u) : (i < 2u ? i : (i + 1u) / 2u);
+                            ts[0] = __uint_as_float(lds_read_u32(at));
                         }
-                        if (is_w) weights_from_lookup(lk[k], a_lo[(u + 1u) & 1u][k], a_hi[(u + 1u) & 1u][k]);
-                        else lk[k] = lookup(next, k);
+                    }
+                    // ---- the fragment two slots on (past the barrier slot the addresses already
+                    // point into the next period's stage) ----
+                    {
+                        const unsigned within = (slot + 2u) % kPeriodSlots;
+                        const unsigned phase_of = within / 8u;
+                        frag[slot & 1u] = lds_read_v4i(piece_at[within % 8u] +
+                                                       ((phase_of / NTB) * T + (phase_of % NTB) * 32u) * kActPitch);
+                    }
+                    // ---- scaling of two rows of the token block before this one ----
+                    scale_rows(parity ^ 1u, tb ? tb - 1u : NTB - 1u, tb ? ts[tb - 1u] : ts_before, m);
+                    // ---- this superblock's share of the decode of the next one ----
+                    if (sb_slot == 0u) settle(raw[(u + 1u) % S], sb + 1u);
+                    if (sb_slot == 1u) raw[(u + 1u) % S] = load_raw(sb + 1u + S);
+#pragma unroll
+                    for (unsigned g = 0; g < 4u; ++g) {
+                        if (sb_slot == Plan::select_slot(g)) select(g);
+                        if (sb_slot == Plan::lookup_slot(g)) lookup(g);
+                    }
+#pragma unroll
+                    for (unsigned k = 0; k < 8u; ++k)
+                        if (sb_slot == Plan::permute_slot(k)) permute(k);
+                    // ---- the row scales of this superblock, once the last sums of the one before
+                    // have been scaled ----
+                    if (sb_slot == 7u) {
+#pragma unroll
+                        for (unsigned q = 0; q < 4u; ++q) {
+                            const uint4 v = lds_read_uint4(row_scale_at + (sb & 1u) * 128u + (8u * q + 4u * h) * 4u);
+                            rs[4u * q] = __uint_as_float(v.x);
+                            rs[4u * q + 1u] = __uint_as_float(v.y);
+                            rs[4u * q + 2u] = __uint_as_float(v.z);
+                            rs[4u * q + 3u] = __uint_as_float(v.w);
+                        }
+                    }
+                    // ---- the next period's copies, one a slot ----
+                    if (slot < kCopyPieces) copy_piece(period + 1u, (period + 1u) & 1u, slot);
+                    if (slot == kBarrierSlot) {
+                        // every activation read of this period has returned and the next period's
+                        // copies have landed: after the barrier nobody reads this stage again
+                        __builtin_amdgcn_s_waitcnt(0x0070u);
+                        __syncthreads();
+                        const unsigned flip = (period & 1u) ? 0u - kStageBytes : kStageBytes;
+#pragma unroll
+                        for (unsigned k = 0; k < 8u; ++k) piece_at[k] += flip;
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            if (u % S == S - 1u) {
-                // the copies of the next period are older than the 2 S window copies issued since
-                __builtin_amdgcn_s_waitcnt(0x0f70u | ((2u * S) & 15u) | (((2u * S) >> 4) << 14));
-                __syncthreads();
-                enter_stage(stage_of(t + 1u));
-#pragma unroll
-                for (unsigned ks = 0; ks < 3u; ++ks) request(0u, ks);
-                request_scale(stage_of(t + 1u), 0u, (u + 1u) * NB);
-            }
         }
     }
-    // the last token block of the last step
+    // the last token block of the last superblock
 #pragma unroll
-    for (unsigned r = 0; r < 4u; ++r) scale_row(D * NB - 1u, NB - 1u, rs[(D - 1u) & 1u][r], ts[(D * NB - 1u) & 1u], r);
+    for (unsigned m = 0; m < 8u; ++m) scale_rows(1u, NTB - 1u, ts[NTB - 1u], m);
 
-    // ---- publish: the lane holds C rows 4 kb + r of its block for tokens tb * 16 + li ----
+    // ---- publish: the lane holds, for tokens 32 tb + r, rows 8 q + 4 h + j of its 32 (j < 4) ----
+    // The tile goes through LDS as [token][value], values 0-63 the gate sums and 64-127 the up
+    // sums of the item's 64 row pairs when fused, else the 128 rows' sums.
+#pragma unroll
+    for (unsigned tb = 0; tb < NTB; ++tb)
+#pragma unroll
+        for (unsigned q = 0; q < 4u; ++q) {
+            unsigned column;
+            if constexpr (FUSED_UP) column = (q >= 2u ? 64u : 0u) + wave * 16u + 8u * (q & 1u) + 4u * h;
+            else column = wave * 32u + 8u * q + 4u * h;
+            lds_write_uint4(kStageBase + (tb * 32u + r) * kOutPitch + column * 4u,
+                            make_uint4(__float_as_uint(acc[tb][4u * q]), __float_as_uint(acc[tb][4u * q + 1u]),
+                                       __float_as_uint(acc[tb][4u * q + 2u]), __float_as_uint(acc[tb][4u * q + 3u])));
+        }
+    __syncthreads();
     auto store4 = [&](unsigned long long out_index, unsigned row, const float (&value)[4]) {
         const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
                           finite_f32(value[3]);
@@ -635,58 +629,38 @@ __device__ __forceinline__ void mfma_item(const MfmaArgs &a, const MfmaItem &it)
             *reinterpret_cast<float4 *>(pr.out + out_index * a.out_rows + row) =
                 make_float4(value[0], value[1], value[2], value[3]);
         else
-            for (unsigned r = 0; r < 4u; ++r)
-                if (row + r < a.out_rows) pr.out[out_index * a.out_rows + row + r] = value[r];
+            for (unsigned j = 0; j < 4u; ++j)
+                if (row + j < a.out_rows) pr.out[out_index * a.out_rows + row + j] = value[j];
     };
-    if constexpr (FUSED_UP) {
-        // Gate wave w and up wave w + 4 hold the two inputs of every SwiGLU. All waves put their
-        // blocks into LDS (the stages are free after the last barrier); gate waves then finish
-        // token blocks [0, G) of their row block, up waves blocks [G, NB), in a loop that is not
-        // unrolled: the activation with its guarded fast path is long, and sixteen copies of it
-        // cost more in registers than they save.
-        constexpr unsigned G = (NB + 1u) / 2u;
-        const bool is_gate = wave < 4u;
-        const unsigned pair_wave = wave & 3u;
-#pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb)
-            lds_write_uint4(kStageBase + ((wave * NB + tb) * 64u + lane) * 16u,
-                            make_uint4(__float_as_uint(acc[tb][0]), __float_as_uint(acc[tb][1]),
-                                       __float_as_uint(acc[tb][2]), __float_as_uint(acc[tb][3])));
-        __syncthreads();
-        const unsigned tb_end = is_gate ? G : NB;
-        const float limit_f32 = (float)a.limit;
+    constexpr unsigned kQuads = kItemRows / 4u;       // groups of four output values per token
+    const float limit_f32 = (float)a.limit;
 #pragma unroll 1
-        for (unsigned tb = is_gate ? 0u : G; tb < tb_end; ++tb) {
-            const unsigned token = tb * 16u + li;
-            const uint4 g = lds_read_uint4(kStageBase + ((pair_wave * NB + tb) * 64u + lane) * 16u);
-            const uint4 u = lds_read_uint4(kStageBase + (((pair_wave + 4u) * NB + tb) * 64u + lane) * 16u);
-            if (token < it.tokens) {
-                const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
-                const float route_weight = __uint_as_float(info.y);
-                const float value[4] = {
-                    swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(u.x), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(u.y), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(u.z), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(u.w), route_weight, a.limit, limit_f32)};
-                store4(info.x, out_row_base + 4u * kb, value);
-            }
-        }
-    } else {
-#pragma unroll
-        for (unsigned tb = 0; tb < NB; ++tb) {
-            const unsigned token = tb * 16u + li;
-            if (token < it.tokens) {
-                const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
-                const float value[4] = {bf16_round(acc[tb][0]), bf16_round(acc[tb][1]),
-                                        bf16_round(acc[tb][2]), bf16_round(acc[tb][3])};
-                store4(info.x, out_row_base + 4u * kb, value);
-            }
+    for (unsigned unit = tid; unit < T * kQuads; unit += kRowThreads) {
+        const unsigned token = unit / kQuads, quad = unit % kQuads;
+        if (token >= it.tokens) break;
+        const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
+        const unsigned row = it.row_tile * kItemRows + 4u * quad;
+        if (row >= a.out_rows) continue;
+        const uint4 g = lds_read_uint4(kStageBase + token * kOutPitch + quad * 16u);
+        if constexpr (FUSED_UP) {
+            const uint4 up = lds_read_uint4(kStageBase + token * kOutPitch + 256u + quad * 16u);
+            const float route_weight = __uint_as_float(info.y);
+            const float value[4] = {
+                swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(up.x), route_weight, a.limit, limit_f32),
+                swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(up.y), route_weight, a.limit, limit_f32),
+                swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(up.z), route_weight, a.limit, limit_f32),
+                swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(up.w), route_weight, a.limit, limit_f32)};
+            store4(info.x, row, value);
+        } else {
+            const float value[4] = {bf16_round(__uint_as_float(g.x)), bf16_round(__uint_as_float(g.y)),
+                                    bf16_round(__uint_as_float(g.z)), bf16_round(__uint_as_float(g.w))};
+            store4(info.x, row, value);
         }
     }
 }
 
 template <bool FUSED_UP>
-__global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
+__global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
 {
     extern __shared__ __align__(16) unsigned char mfma_lds[];
     if (lds_address_of(mfma_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
@@ -703,20 +677,20 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
         // Full 128-pair tiles come first in the item list, then the partial last tiles by size,
         // largest first: every workgroup, walking the list with the grid's stride, gets the same
         // share of each kind of item, and the short items come last.
-        unsigned cursor = 0u, members[4] = {0u, 0u, 0u, 0u};
+        unsigned cursor = 0u, members[3] = {0u, 0u, 0u};
         for (unsigned b = 0; b < buckets && b < 256u; ++b) {
             lds_write_u32(kTileStartBase + 4u * b, cursor);
             const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[b];
             cursor += (unsigned)(n / kTileTokens);
             const unsigned rest = (unsigned)(n % kTileTokens);
             if (rest) {
-                const unsigned c = rest > 64u ? 0u : rest > 32u ? 1u : rest > 16u ? 2u : 3u;
+                const unsigned c = rest > 64u ? 0u : rest > 32u ? 1u : 2u;
                 lds_write_u16(kClassListBase + (c * 256u + members[c]) * 2u, b);
                 ++members[c];
             }
         }
         lds_write_u32(kTileStartBase + 4u * (buckets < 256u ? buckets : 256u), cursor);
-        for (unsigned c = 0; c < 4u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
+        for (unsigned c = 0; c < 3u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
     }
     __syncthreads();
     if (buckets == 0u || buckets > 256u) {
@@ -728,9 +702,9 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
     constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
     const unsigned row_tiles = (a.out_rows + kItemRows - 1u) / kItemRows;
     const unsigned long long full_items = (unsigned long long)lds_read_u32(kTileStartBase + 4u * buckets) * row_tiles;
-    unsigned members[4];
+    unsigned members[3];
     unsigned long long items = full_items;
-    for (unsigned c = 0; c < 4u; ++c) {
+    for (unsigned c = 0; c < 3u; ++c) {
         members[c] = lds_read_u32(kClassCountBase + 4u * c);
         items += (unsigned long long)members[c] * row_tiles;
     }
@@ -761,7 +735,7 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
         } else {
             unsigned long long rest = item - full_items;
             unsigned c = 0u;
-            while (c < 3u && rest >= (unsigned long long)members[c] * row_tiles) {
+            while (c < 2u && rest >= (unsigned long long)members[c] * row_tiles) {
                 rest -= (unsigned long long)members[c] * row_tiles;
                 ++c;
             }
@@ -785,10 +759,9 @@ __global__ __launch_bounds__(512) void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-        if (it.tokens <= 16u) mfma_item<FUSED_UP, 1u>(a, it);
-        else if (it.tokens <= 32u) mfma_item<FUSED_UP, 2u>(a, it);
-        else if (it.tokens <= 64u) mfma_item<FUSED_UP, 4u>(a, it);
-        else mfma_item<FUSED_UP, 8u>(a, it);
+        if (it.tokens <= 32u) rows_item<FUSED_UP, 1u>(a, it);
+        else if (it.tokens <= 64u) rows_item<FUSED_UP, 2u>(a, it);
+        else rows_item<FUSED_UP, 4u>(a, it);
     }
 }
 
@@ -817,7 +790,7 @@ static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
             (void)hipGetLastError();
         configured = true;
     }
-    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), 512u, kMfmaLdsBytes, stream>>>(a);
+    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
     return check_launch("moe_rows_mfma");
 }
 
