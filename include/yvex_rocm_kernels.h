@@ -188,7 +188,7 @@ int yvex_hip_moe_down(const yvex_hip_expert_weights *weights, const void *interm
 /* Row-batch (prefill-width) forms of the two sweeps above on the int8 matrix cores; they replace
  * yvex_moe_grouped_up_tensorcore / _down_tensorcore (tensorcore.cu:378-702). Same inputs,
  * outputs and rounding points as yvex_hip_moe_up / yvex_hip_moe_down with act_q8 = 1; weights
- * must be IQ2_XXS. A work item is 128 ordered pairs of one bucket times a tile of weight rows,
+ * must be IQ2_XXS. A work item is 64 ordered pairs of one bucket times a tile of 256 weight rows,
  * so buckets of any population are served; expert_ids == NULL is the single-bucket form
  * (shared expert: every pair uses expert 0, order may be NULL for the identity). */
 int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *weights, const void *act_q8k,

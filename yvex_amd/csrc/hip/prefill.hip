@@ -1,35 +1,40 @@
 // Row-batch (prefill-width) grouped expert projections on the int8 matrix cores of gfx950.
 //
-// A work item is (bucket, tile of up to 128 ordered pairs, tile of 128 weight rows: 64 gate rows
-// and the 64 matching up rows when the SwiGLU is fused). The workgroup has four waves, one per
+// A work item is (bucket, tile of up to 64 ordered pairs, tile of 256 weight rows: 128 gate rows
+// and the 128 matching up rows when the SwiGLU is fused). The workgroup has eight waves, two per
 // SIMD; each owns 32 weight rows and multiplies them by all of the item's Q8_K activation rows
-// with V_MFMA_I32_32X32X32_I8, so one activation fragment read from LDS feeds two matrix
-// instructions of 32 passes in total and the decode of a weight is shared by up to 128 tokens.
+// with V_MFMA_I32_32X32X32_I8. A wave cannot run vector instructions under its own matrix
+// instruction, the other wave of its SIMD can, so two waves a SIMD is the shape that lets decode
+// and scaling arithmetic overlap the matrix pipe, and 256 registers a wave is what decides the
+// tile: 32 rows x 64 tokens of int32 limb sums and fp32 sums.
 //
-//   A operand (weights): built in registers. Lane (r, h) = (lane % 32, lane / 32) owns weight
-//       row r and the groups 4h .. 4h + 3 of the current superblock (128 columns); K chunk m of
-//       the superblock is, for that lane, the 16 weights 16 (m % 2) .. + 15 of group 4h + m / 2.
-//       The order of K inside a matrix instruction is free as long as both operands agree.
+//   A operand (weights): built in registers, one K chunk (32 columns) ahead of its use. Lane
+//       (r, h) = (lane % 32, lane / 32) owns weight row r and the groups 4h .. 4h + 3 of the
+//       current superblock (128 columns); K chunk m of the superblock is, for that lane, the 16
+//       weights 16 (m % 2) .. + 15 of group 4h + m / 2. The order of K inside a matrix
+//       instruction is free as long as both operands agree.
 //       The IQ2_XXS value of one weight is level * sign * (2s+1), up to 43 * 31 = 1333, so it is
 //       split into two int8 limbs, value = 128 * hi + lo with hi in [1, 11] and lo in
-//       [-120, 63], and every K chunk costs two matrix instructions. For one scale there are only
-//       three levels, so the six signed limb values of a group fit two registers and one
-//       V_PERM_B32 per four weights picks them: the selector byte of a weight is its level code
-//       (0..2) plus 4 when it is negative. Three LDS tables feed this: level codes of a codebook
-//       entry (8 bytes, 32 replicas: no two lanes of a half-wave share a bank), sign selectors
-//       of a 7-bit sign field (8 bytes, 16 replicas) and the limb words of a scale (16 bytes,
-//       16 replicas).
-//   B operand (activations): the tile's int8 blocks of one stage period (four superblocks of 32
-//       tokens, two of 64 or one of 128), copied from global memory straight into LDS
-//       (GLOBAL_LOAD_LDS_DWORDX4), double buffered. 16-byte piece c of token t sits at piece
-//       position c ^ (t % 16), so the 16 lanes that read one fragment column together hit 16
-//       different bank groups.
+//       [-120, 63], and every K chunk costs two matrix instructions per token block. For one
+//       scale there are only three levels, so the six signed limb values of a group fit two
+//       registers and one V_PERM_B32 per four weights picks them: the selector byte of a weight
+//       is its level code (0..2) plus 4 when it is negative. Three LDS tables feed this, sixteen
+//       replicas each so that the lanes of a quarter-wave never share a bank: level codes of a
+//       codebook entry (8 bytes), sign selectors of a 7-bit sign field (8 bytes) and the limb
+//       words of a scale (16 bytes).
+//   Weight bytes: each wave copies, per superblock, the aligned 68 bytes around the superblock of
+//       each of its 32 rows into an LDS window (GLOBAL_LOAD_LDS_DWORDX4, every cache line
+//       fetched once), two superblocks ahead; the lanes take their records out with LDS reads.
+//   B operand (activations): the tile's int8 blocks of one superblock, copied from global memory
+//       straight into LDS, in a ring of stages. 16-byte piece c of token t sits at piece position
+//       c ^ (t % 16), so the 16 lanes that read one fragment column together hit 16 different
+//       bank groups.
 //   C: per (superblock, 32-token block) two int32 accumulators of 32 x 32; T = 128 * C_hi + C_lo
 //       is the exact integer superblock sum of the reference's primitive
 //       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
 //       ((0.125 * d_w) * d_a) * T and summed over superblocks.
-//   Output: the wave's fp32 sums go through LDS once per item so that every store instruction
-//       writes whole 64-byte runs of an output row.
+//   Output: the waves' fp32 sums go through LDS, half a tile at a time, so that every store
+//       instruction writes whole 64-byte runs of an output row.
 //
 // Same inputs, outputs and rounding points as the decode-width sweeps in moe.hip
 // (src/backend/cuda/tensorcore.cu:378-702 is the reference's counterpart, unused there).
@@ -42,29 +47,37 @@ namespace yvex {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr unsigned kRowWaves = 4u;
+constexpr unsigned kRowWaves = 8u;                          // two per SIMD
 constexpr unsigned kRowThreads = 64u * kRowWaves;
-constexpr unsigned kTileTokens = 128u;
+constexpr unsigned kTileTokens = 64u;
 constexpr unsigned kActPitch = 256u;                       // one Q8_K block's int8 payload
 // LDS map (absolute byte offsets; the dynamic allocation starts at 0, checked at kernel start).
-constexpr unsigned kCodeBase = 0u;                          // 256 entries x 32 replicas x 8 bytes
-constexpr unsigned kSelBase = 65536u;                       // 128 sign fields x 16 replicas x 8 bytes
-constexpr unsigned kLutBase = kSelBase + 128u * 16u * 8u;   // 16 scales x 16 replicas x 16 bytes
-constexpr unsigned kRowScaleBase = kLutBase + 16u * 16u * 16u;   // 4 waves x 2 x 32 floats
-constexpr unsigned kPairInfoBase = kRowScaleBase + kRowWaves * 2u * 128u;   // {out row, route weight} x 128
-// Item numbering: first full 128-pair tile of every bucket (257 words), then per class of last,
-// partial, tile (65-127, 33-64, 1-32 pairs) a count and the list of its buckets (u16).
+// Codebook entry e owns the 256 bytes at 256 e: sixteen replicas of its 8 level codes in the
+// first half; the second half of entries 0-127 holds sixteen replicas of the sign selectors of
+// sign field e.
+constexpr unsigned kCodeBase = 0u;
+constexpr unsigned kSelBase = 128u;
+constexpr unsigned kLutBase = 65536u;                       // 16 scales x 16 replicas x 16 bytes
+constexpr unsigned kRowScaleBase = kLutBase + 16u * 16u * 16u;   // 8 waves x 2 x 32 floats
+constexpr unsigned kPairInfoBase = kRowScaleBase + kRowWaves * 2u * 128u;   // {out row, route weight} x 64
+// Item numbering: first full 64-pair tile of every bucket (257 words), then per class of last,
+// partial, tile (33-63, 1-32 pairs) a count and the list of its buckets (u16).
 constexpr unsigned kTileStartBase = kPairInfoBase + kTileTokens * 8u;
 constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
 constexpr unsigned kClassListBase = kClassCountBase + 16u;
-constexpr unsigned kTrashBase = kClassListBase + 3u * 256u * 2u;   // 256 bytes nobody reads
-constexpr unsigned kStageBase = (kTrashBase + 256u + 255u) & ~255u;
-constexpr unsigned kStageActs = kTileTokens * kActPitch;
-constexpr unsigned kStageBytes = kStageActs + kTileTokens * 4u;   // + one fp32 scale per slot
-// the finished tile on its way out: 128 tokens x (128 values + 4 of padding) fp32
+constexpr unsigned kTrashBase = kClassListBase + 2u * 256u * 2u;   // 256 bytes nobody reads
+// Weight windows: per wave two buffers; a buffer holds, for each of the wave's 32 rows, the 80
+// bytes (five 16-byte pieces) around one superblock, rows back to back (three copies of 64, 64
+// and 32 lanes fill it).
+constexpr unsigned kWindowBase = (kTrashBase + 256u + 255u) & ~255u;
+constexpr unsigned kWindowBytes = 32u * 80u;
+constexpr unsigned kStageBase = kWindowBase + kRowWaves * 2u * kWindowBytes;
+// activation stages: a ring of 4 / NTB stages of NTB x 32 slots (256 bytes each) + 64 scales
+constexpr unsigned kStageRingBytes = 128u * kActPitch + 4u * 256u;
+// half of the finished tile on its way out: 64 tokens x (128 values + 4 of padding) fp32
 constexpr unsigned kOutPitch = 132u * 4u;
 constexpr unsigned kOutBytes = kTileTokens * kOutPitch;
-constexpr unsigned kMfmaLdsBytes = kStageBase + (2u * kStageBytes > kOutBytes ? 2u * kStageBytes : kOutBytes);
+constexpr unsigned kMfmaLdsBytes = kStageBase + (kStageRingBytes > kOutBytes ? kStageRingBytes : kOutBytes);
 static_assert(kMfmaLdsBytes <= 160u * 1024u, "one workgroup per compute unit");
 
 struct MfmaArgs {
@@ -180,8 +193,8 @@ __device__ __forceinline__ unsigned iq2_limbs(unsigned level, unsigned factor)
 __device__ __forceinline__ void mfma_tables_fill()
 {
     // level codes: byte l of the entry is 0, 1 or 2 for level 8, 25 or 43 of weight l
-    for (unsigned index = threadIdx.x; index < 256u * 32u; index += blockDim.x) {
-        const uint2 m = iq2_magnitude_entry(index >> 5);
+    for (unsigned index = threadIdx.x; index < 256u * 16u; index += blockDim.x) {
+        const uint2 m = iq2_magnitude_entry(index >> 4);
         uint2 codes = make_uint2(0u, 0u);
 #pragma unroll
         for (unsigned l = 0; l < 4u; ++l) {
@@ -189,12 +202,13 @@ __device__ __forceinline__ void mfma_tables_fill()
             codes.x |= (a == 8u ? 0u : a == 25u ? 1u : 2u) << (8u * l);
             codes.y |= (b == 8u ? 0u : b == 25u ? 1u : 2u) << (8u * l);
         }
-        lds_write_uint2(kCodeBase + index * 8u, codes);
+        lds_write_uint2(kCodeBase + (index >> 4) * 256u + (index & 15u) * 8u, codes);
     }
     // sign selectors: byte l is 4 when weight l is negative (7 stored bits + parity)
     for (unsigned index = threadIdx.x; index < 128u * 16u; index += blockDim.x) {
         const uint2 m = iq2_signmask_entry(index >> 4);
-        lds_write_uint2(kSelBase + index * 8u, make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
+        lds_write_uint2(kSelBase + (index >> 4) * 256u + (index & 15u) * 8u,
+                        make_uint2(m.x & 0x04040404u, m.y & 0x04040404u));
     }
     // limb words of scale s: {+lo, -lo, +hi, -hi}, byte c = limb of level code c
     for (unsigned index = threadIdx.x; index < 16u * 16u; index += blockDim.x) {
@@ -214,126 +228,108 @@ __device__ __forceinline__ void mfma_tables_fill()
     }
 }
 
+// The same 16-byte copy for lanes 0-31 only (the other lanes neither read nor write).
+__device__ __forceinline__ void copy_to_lds_16_first32(const void *global, unsigned lds_base)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    unsigned long long saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "s"(lds_base), "v"(global) : "memory");
+#else
+    (void)global;
+    (void)lds_base;
+#endif
+}
+
 // What one work item needs to know about its place in the problem.
 struct MfmaItem {
     unsigned long long expert, pair0;
     unsigned tokens, row_tile;
 };
 
-// The aligned dwords around a lane's 32 code bytes of one superblock, and the dword that holds
-// the superblock's fp16 scale.
-struct RawCodes {
-    uint4 x0, x1;
-    unsigned x2, scale_word;
-};
-
-__device__ __forceinline__ uint4 load_uint4_dword_aligned(const unsigned char *p)
-{
-    uint4 v;
-    __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
-    return v;
-}
-__device__ __forceinline__ unsigned load_u32_aligned(const unsigned char *p)
-{
-    return *reinterpret_cast<const unsigned *>(p);
-}
-
-// Where in the 8 NTB slots of a superblock each piece of the next superblock's decode runs:
-// settle (records out of the loaded dwords, row scale to LDS), then per group g the nine table
-// lookups L(g), the selector words S(g), and per K chunk m the permutes P(m) that overwrite the
-// chunk's operands once the last token block has used them.
-template <unsigned NTB>
-struct DecodePlan {
-    static constexpr unsigned kSlots = 8u * NTB;
-    static constexpr unsigned lookup_slot(unsigned g)
-    {
-        return NTB == 4u ? 1u + 6u * g : NTB == 2u ? 2u * g : g;
-    }
-    static constexpr unsigned select_slot(unsigned g)
-    {
-        return NTB == 4u ? 4u + 6u * g : NTB == 2u ? 2u * g + 2u : g + 2u;
-    }
-    static constexpr unsigned permute_slot(unsigned m)
-    {
-        // after the last token block's matrix instructions on chunk m, and after S(m / 2)
-        const unsigned last_use = kSlots - 8u + m;
-        const unsigned ready = select_slot(m / 2u) + 1u;
-        return last_use > ready ? last_use : ready;
-    }
-};
-
-// One work item with NTB live 32-token blocks (NTB is 1, 2 or 4).
+// One work item with NTB live 32-token blocks (NTB is 1 or 2).
 //
-// The stage in LDS holds 128 "slots" of 256 activation bytes + one scale. An item with fewer than
-// 97 tokens fills them with S = 4 / NTB consecutive superblocks of its NTB * 32 tokens (slot =
-// superblock within the period * NTB * 32 + token), so that every period between two barriers
-// carries the same copies and 32 "time slots" of two matrix instructions each.
+// Time slot (sb, m) = superblock sb, K chunk m: 2 NTB matrix instructions (low and high limb for
+// every token block) on the chunk's operands, which were built during the slot before: the
+// weights of a superblock are decoded chunk by chunk just ahead of their use, two chunks' worth
+// of operand registers in all. Between the matrix instructions the slot carries the LDS reads of
+// the activation fragments two slots ahead, the table lookups of the chunk two slots ahead,
+// the selector words and permutes of the next chunk, and its share of the copies. After the
+// last chunk the integer sums of the superblock are scaled into the fp32 accumulators. Two waves
+// share a SIMD: while one waits for its own matrix instructions or scales its sums the other's
+// instructions run.
 //
-// Time slot (u, tb, m) = superblock u of the period, token block tb, K chunk m. Around its two
-// matrix instructions (low and high limb) the slot carries, a few instructions at a time, the
-// rest of the work: the LDS read of the activation fragment two slots ahead, the scaling of two
-// rows of the previous token block's integer sums into the fp32 accumulators, one piece of the
-// decode of the next superblock's weights, and this period's share of the copies and loads.
-// The loop body is one period in one basic block (requests past the end are clamped, and
-// superblocks past the end run with a zero row scale), so the compiler's wait counts stay exact
-// and accumulators never leave registers.
+// Everything that comes from memory inside the loop arrives by GLOBAL_LOAD_LDS copies, whose
+// completion the kernel counts by hand (they retire in order):
+//   * activations: a ring of R = 4 / NTB stages of NTB x 32 slots (256 int8 + one scale each);
+//     the copies of superblock sb + R are issued right after the barrier of superblock sb, which
+//     every wave passes once all its reads of that stage have returned;
+//   * weights: per wave two windows holding, for each of its 32 rows, the aligned 80 bytes
+//     around one superblock (five 16-byte pieces a row, the fifth ending with the dword that
+//     holds the superblock's last byte, so nothing behind it is touched). Each cache line of a
+//     row is fetched once; taking the records out of the window is LDS work. Loading the
+//     records lane by lane from global memory touched every row's line four times per
+//     superblock, and the memory pipeline spends about two cycles per line an instruction
+//     touches: with eight waves that was the longest pole of the step.
+// The loop body is one superblock in one basic block (requests past the end are clamped, and
+// superblocks past the end run with a zero row scale), so nothing leaves registers.
 template <bool FUSED_UP, unsigned NTB>
 __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
-    constexpr unsigned S = 4u / NTB;                 // superblocks per stage period
-    constexpr unsigned T = NTB * 32u;                // token slots of one superblock
-    constexpr unsigned kSbSlots = 8u * NTB;
-    constexpr unsigned kPeriodSlots = 32u;
-    constexpr unsigned kBarrierSlot = kPeriodSlots - 3u;
-    using Plan = DecodePlan<NTB>;
+    constexpr unsigned R = 4u / NTB;                 // activation stages
+    constexpr unsigned T = NTB * 32u;                // token slots of one stage
+    constexpr unsigned kStageBytes = T * kActPitch + 256u;
+    constexpr unsigned kBarrierSlot = 5u;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
-    constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
+    constexpr unsigned kItemRows = FUSED_UP ? 128u : 256u;
     const unsigned superblocks = a.width >> 8;
     const unsigned last = superblocks - 1u;
 
-    // ---- the weight row of this lane: rows 0-15 of a wave are gate rows and rows 16-31 the
-    // matching up rows when the SwiGLU is fused ----
-    const unsigned char *weight_row;
-    {
+    // ---- weight rows: rows 0-15 of a wave are gate rows and rows 16-31 the matching up rows
+    // when the SwiGLU is fused ----
+    auto row_pointer = [&](unsigned wave_row) {
         unsigned row;
         bool is_up = false;
         if constexpr (FUSED_UP) {
-            row = it.row_tile * kItemRows + wave * 16u + (r & 15u);
-            is_up = r >= 16u;
+            row = it.row_tile * kItemRows + wave * 16u + (wave_row & 15u);
+            is_up = wave_row >= 16u;
         } else {
-            row = it.row_tile * kItemRows + wave * 32u + r;
+            row = it.row_tile * kItemRows + wave * 32u + wave_row;
         }
         if (row >= a.out_rows) row = a.out_rows - 1u;
-        weight_row = is_up
+        return is_up
             ? pr.up + it.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
             : pr.gate + it.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
+    };
+    // Superblocks are 66 bytes, so they start on 2-byte boundaries, and vector accesses that are
+    // not dword-aligned run at less than half rate: a window starts at the aligned dword that
+    // holds the superblock's first byte. Copy k of a window moves pieces 64 k + lane of the
+    // wave's 160 (row = piece / 5).
+    const unsigned row_misalign = (unsigned)(unsigned long long)row_pointer(r) & 3u;    // of the lane's own row
+    const unsigned char *window_from[3];    // row start + piece offset, of the row this lane copies
+#pragma unroll
+    for (unsigned k = 0; k < 3u; ++k) {
+        const unsigned piece = 64u * k + lane;
+        const unsigned served = piece < 160u ? piece : 159u;
+        const unsigned char *from = row_pointer(served / 5u);
+        window_from[k] = from + (served % 5u < 4u ? 16u * (served % 5u) : 52u);
     }
-    // Superblocks are 66 bytes, so the lane's 32 code bytes start on 2-byte boundaries, and vector
-    // loads that are not dword-aligned run at less than half rate: the lane loads the aligned
-    // dwords around them (two 16-byte loads and a ninth dword, which repeats the eighth when the
-    // codes are aligned so that nothing past the dword holding the last code byte is touched)
-    // and shifts the records into place.
-    const unsigned row_misalign = (unsigned)(unsigned long long)weight_row & 3u;
-    const unsigned char *row_aligned = weight_row - row_misalign;
-    const unsigned code_offset = row_misalign + 2u + 32u * h;       // of superblock 0's codes from row_aligned
-    auto load_raw = [&](unsigned sb) {
+    const unsigned window_base = kWindowBase + wave * 2u * kWindowBytes;
+    auto weight_piece = [&](unsigned sb, unsigned k) {
+        const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane(
+            (int)(window_base + (sb & 1u) * kWindowBytes + k * 1024u));
         sb = sb < last ? sb : last;
-        RawCodes out;
-        const unsigned at = code_offset + sb * 66u;
-        const unsigned char *from = row_aligned + (at & ~3u);
-        out.x0 = load_uint4_dword_aligned(from);
-        out.x1 = load_uint4_dword_aligned(from + 16u);
-        out.x2 = load_u32_aligned(from + ((at & 3u) ? 32u : 28u));
-        out.scale_word = load_u32_aligned(row_aligned + ((row_misalign + sb * 66u) & ~3u));
-        return out;
+        const unsigned char *from = (const unsigned char *)((unsigned long long)(window_from[k] + sb * 66u) & ~3ull);
+        if (k < 2u) copy_to_lds_16(from, to);
+        else copy_to_lds_16_first32(from, to);
     };
 
-    // ---- activation rows this lane copies: wave w owns the 4-slot groups w, w + 4, ... ----
+    // ---- activation rows this lane copies: wave w owns the 4-slot groups w (and w + 8) ----
     // Lane l of a group moves piece position l % 16 of slot 4 g + l / 16; LDS receives the wave's
     // 64 pieces back to back, so the swizzle is applied on the global side.
-    constexpr unsigned kCopies = kTileTokens / (4u * kRowWaves);
     auto token_row = [&](unsigned token) {
         const unsigned live = token < it.tokens ? token : it.tokens - 1u;   // padding repeats a row
         const unsigned long long ordered = it.pair0 + live;
@@ -341,124 +337,120 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
         return (const unsigned char *)pr.activations + arow * pr.act_stride;
     };
-    const unsigned char *copy_from[kCopies];
-    unsigned copy_step[kCopies];            // superblock of the slot within its period
+    const unsigned char *copy_from[NTB];
 #pragma unroll
-    for (unsigned j = 0; j < kCopies; ++j) {
-        const unsigned slot = 4u * (wave + kRowWaves * j) + (lane >> 4);
-        const unsigned token = slot % T;
-        copy_step[j] = slot / T;
+    for (unsigned j = 0; j < NTB; ++j) {
+        const unsigned token = 4u * (wave + kRowWaves * j) + (lane >> 4);
         copy_from[j] = token_row(token) + 4u + 16u * ((lane & 15u) ^ (token & 15u));
     }
-    // Waves 0 and 1 also copy the 128 slot scales, laid out [superblock][token % 32][token block]
-    // so that a lane reads the scales of its NTB tokens with one LDS read. The other waves run the
-    // same instruction on one address for all lanes (one cache line: next to free) into bytes
-    // nobody reads, which is cheaper than a branch around the copy.
+    // Wave 0 also copies the stage's slot scales, laid out [token % 32][token block] so that a lane
+    // reads the scales of its NTB tokens with one LDS read. The other waves run the same
+    // instruction on one address for all lanes (one cache line: next to free) into bytes nobody
+    // reads, which is cheaper than a branch around the copy.
     const unsigned char *scale_from;
-    unsigned scale_step;
     {
-        const unsigned index = wave < 2u ? 64u * wave + lane : 0u;
-        const unsigned within = index % T;
-        scale_step = index / T;
-        scale_from = token_row((within % NTB) * 32u + within / NTB);
+        const unsigned index = wave == 0u ? lane % T : 0u;
+        scale_from = token_row((index % NTB) * 32u + index / NTB);
     }
-    const unsigned scale_to = wave < 2u ? kStageActs + wave * 256u : 0xffffffffu;
-
-    constexpr unsigned kCopyPieces = kCopies + 1u;
-    auto copy_piece = [&](unsigned period, unsigned stage, unsigned j) {
-        const unsigned base = kStageBase + stage * kStageBytes;
-        if (j < kCopies) {
-            unsigned sb = period * S + copy_step[j];
-            sb = sb < last ? sb : last;
+    constexpr unsigned kActPieces = NTB + 1u;
+    auto act_piece = [&](unsigned sb, unsigned j) {
+        const unsigned base = kStageBase + (sb % R) * kStageBytes;
+        sb = sb < last ? sb : last;
+        if (j < NTB) {
             copy_to_lds_16(copy_from[j] + (unsigned long long)sb * kQ8KBytes,
                            (unsigned)__builtin_amdgcn_readfirstlane((int)(base + (wave + kRowWaves * j) * 1024u)));
         } else {
-            unsigned sb = period * S + scale_step;
-            sb = sb < last ? sb : last;
             copy_to_lds_4(scale_from + (unsigned long long)sb * kQ8KBytes,
                           (unsigned)__builtin_amdgcn_readfirstlane(
-                              (int)(scale_to != 0xffffffffu ? base + scale_to : kTrashBase)));
+                              (int)(wave == 0u ? base + T * kActPitch : kTrashBase)));
         }
     };
+    // the copies issued after the barrier of superblock sb: the stage and the window just released
+    constexpr unsigned kRoundPieces = kActPieces + 3u;
+    auto round_piece = [&](unsigned sb, unsigned j) {
+        if (j < kActPieces) act_piece(sb + R, j);
+        else weight_piece(sb + 3u, j - kActPieces);
+    };
 
-    // ---- decode state of the superblock after the current one ----
-    const unsigned code_lane = kCodeBase + (lane & 31u) * 8u;
+    // ---- decode state ----
+    const unsigned code_lane = kCodeBase + (lane & 15u) * 8u;
     const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
     const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
     const unsigned row_scale_at = kRowScaleBase + wave * 256u;      // + 128 for odd superblocks
-    unsigned grids[4], aux[4];
-    uint2 codes[2][4], signs[2][4];      // [g & 1]: of the groups whose lookups are in flight
-    uint4 limbs[4];                      // limb words per group
-    unsigned sel[4][8];                  // selector words per group
-    v4i a_lo[8], a_hi[8];                // A operands of the current superblock, per K chunk
+    const unsigned window_row = window_base + r * 80u;
+    unsigned grids[4], aux[4];           // group records of the superblock being decoded
+    uint2 codes[2][2], signs[2][2];      // [chunk & 1]: table words of the chunk's two subgroups
+    uint4 limbs[2];                      // [group & 1]: limb words of a group
+    v4i a_lo[2], a_hi[2];                // [chunk & 1]: A operands of a K chunk
 
-    // records out of the loaded dwords, and the row's scale into LDS for the lanes that hold
-    // this row's sums (zero past the end: such superblocks add nothing)
-    auto settle = [&](const RawCodes &raw, unsigned sb) {
+    // Records of superblock sb out of its window, and the row's scale into LDS for the lanes that
+    // hold this row's sums (zero past the end: such superblocks add nothing). With o = (row start
+    // + 66 sb) mod 4 (0 or 2) the fp16 scale sits o bytes into the window and the lane's 32 code
+    // bytes at o + 2 + 32 h: in window dwords 8 h + o / 2 onwards, shifted by 2 bytes when o is
+    // 0. Window dword 16 is the last dword of the fifth piece.
+    auto settle = [&](unsigned sb) {
         const unsigned clamped = sb < last ? sb : last;
-        const unsigned shift = (code_offset + clamped * 66u) & 3u;
-        const unsigned w[9] = {raw.x0.x, raw.x0.y, raw.x0.z, raw.x0.w, raw.x1.x, raw.x1.y, raw.x1.z, raw.x1.w, raw.x2};
+        const unsigned o = (row_misalign + 2u * clamped) & 3u;
+        const unsigned at = window_row + (sb & 1u) * kWindowBytes;
+        const unsigned first = at + 32u * h + 2u * o;                   // dword 8 h + o / 2
+        unsigned w[9];
+#pragma unroll
+        for (unsigned i = 0; i < 7u; ++i) w[i] = lds_read_u32(first + 4u * i);
+        // window dword 16 lives 12 bytes further on (it is the last dword of the fifth piece); it
+        // is the eighth of the lane's dwords when h is 1 and o is 2 and the ninth when h is 1 and o
+        // is 0 (the ninth is only part of a record when o is 0)
+        w[7] = lds_read_u32((h && o) ? at + 76u : first + 28u);
+        w[8] = lds_read_u32(h ? at + 76u : first + 32u);
+        const unsigned scale16 = (lds_read_u32(at) >> (8u * o)) & 0xffffu;
+        const unsigned shift = (o + 2u) & 3u;
 #pragma unroll
         for (unsigned g = 0; g < 4u; ++g) {
             grids[g] = __builtin_amdgcn_alignbyte(w[2u * g + 1u], w[2u * g], shift);
             aux[g] = __builtin_amdgcn_alignbyte(w[2u * g + 2u], w[2u * g + 1u], shift);
         }
-        const unsigned scale_shift = ((row_misalign + clamped * 66u) & 3u) * 8u;
-        const unsigned scale16 = (raw.scale_word >> scale_shift) & 0xffffu;
         const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(scale16) : 0.0f;
         lds_write_u32(row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
     };
-    auto lookup = [&](unsigned g) {
+    // table lookups of K chunk c: subgroups 2 (c & 1) and 2 (c & 1) + 1 of group c / 2
+    auto lookup = [&](unsigned c) {
+        const unsigned g = c >> 1;
 #pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
-            codes[g & 1u][j] = lds_read_uint2(__builtin_amdgcn_perm(grids[g], code_lane, 0x0c0c0400u + (j << 8)));
-            const unsigned field = j == 0u ? aux[g] << 7 : j == 1u ? aux[g] : aux[g] >> (7u * j - 7u);
-            signs[g & 1u][j] = lds_read_uint2((field & 0x3f80u) | sel_lane);
+        for (unsigned i = 0; i < 2u; ++i) {
+            const unsigned j = 2u * (c & 1u) + i;
+            codes[c & 1u][i] = lds_read_uint2(__builtin_amdgcn_perm(grids[g], code_lane, 0x0c0c0400u + (j << 8)));
+            const unsigned field = j == 0u ? aux[g] << 8 : j == 1u ? aux[g] << 1 : aux[g] >> (7u * j - 8u);
+            signs[c & 1u][i] = lds_read_uint2((field & 0x7f00u) | sel_lane);
         }
-        limbs[g] = lds_read_uint4(((aux[g] >> 20) & 0xf00u) | lut_lane);
+        if ((c & 1u) == 0u) limbs[g & 1u] = lds_read_uint4(((aux[g] >> 20) & 0xf00u) | lut_lane);
     };
-    auto select = [&](unsigned g) {
-#pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
-            sel[g][2u * j] = codes[g & 1u][j].x | signs[g & 1u][j].x;
-            sel[g][2u * j + 1u] = codes[g & 1u][j].y | signs[g & 1u][j].y;
-        }
-    };
-    auto permute = [&](unsigned m) {
-        const unsigned g = m >> 1, first = 4u * (m & 1u);
-        a_lo[m] = v4i{(int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first]),
-                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 1u]),
-                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 2u]),
-                      (int)__builtin_amdgcn_perm(limbs[g].y, limbs[g].x, sel[g][first + 3u])};
-        a_hi[m] = v4i{(int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first]),
-                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 1u]),
-                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 2u]),
-                      (int)__builtin_amdgcn_perm(limbs[g].w, limbs[g].z, sel[g][first + 3u])};
+    // selector words and permutes of K chunk c
+    auto build = [&](unsigned c) {
+        const uint4 lw = limbs[(c >> 1) & 1u];
+        const unsigned s0 = codes[c & 1u][0].x | signs[c & 1u][0].x, s1 = codes[c & 1u][0].y | signs[c & 1u][0].y;
+        const unsigned s2 = codes[c & 1u][1].x | signs[c & 1u][1].x, s3 = codes[c & 1u][1].y | signs[c & 1u][1].y;
+        a_lo[c & 1u] = v4i{(int)__builtin_amdgcn_perm(lw.y, lw.x, s0), (int)__builtin_amdgcn_perm(lw.y, lw.x, s1),
+                           (int)__builtin_amdgcn_perm(lw.y, lw.x, s2), (int)__builtin_amdgcn_perm(lw.y, lw.x, s3)};
+        a_hi[c & 1u] = v4i{(int)__builtin_amdgcn_perm(lw.w, lw.z, s0), (int)__builtin_amdgcn_perm(lw.w, lw.z, s1),
+                           (int)__builtin_amdgcn_perm(lw.w, lw.z, s2), (int)__builtin_amdgcn_perm(lw.w, lw.z, s3)};
     };
 
-    // ---- activation fragments: piece 8 h + m of slot r (+ 32 tb + T u) ----
-    unsigned piece_at[8];
-    auto enter_stage = [&](unsigned base) {
-#pragma unroll
-        for (unsigned m = 0; m < 8u; ++m) {
-            // kept opaque so that the slot offset stays the instruction's immediate
-            piece_at[m] = base + r * kActPitch + ((((8u * h) ^ (r & 15u)) ^ m) << 4);
-            asm volatile("" : "+v"(piece_at[m]));
-        }
-    };
-    auto stage_base = [&](unsigned period) { return kStageBase + (period & 1u) * kStageBytes; };
+    // ---- activation fragments: piece 8 h + m of slot r (+ 32 tb) of the current stage; stage
+    // bases are multiples of 256, so the piece position is bits 4-7 of the address ----
+    unsigned frag_at = kStageBase + r * kActPitch + (((8u * h) ^ (r & 15u)) << 4);
 
     // ---- prologue ----
-    RawCodes raw[S];
-    // The first superblocks of the weight rows are asked for before anything else: their trip to
-    // HBM runs under the index loads and copies of the activation side.
-    RawCodes first_raw = load_raw(0u);
+    // Copies in flight when the loop starts are those of its own schedule: a round (stage sb + R,
+    // window sb + 3) is issued after the barrier of superblock sb, four pieces in slots 6 and 7 and
+    // the rest at the start of the next superblock, so rounds -(R - 1) .. -1 are issued here
+    // (windows 0 and 1 are needed before them; the rounds before -1 repeat window 1, which keeps
+    // the counts below the same for every superblock).
+    __syncthreads();   // every wave is done with the previous item's stages and output tile
 #pragma unroll
-    for (unsigned x = 1; x <= S; ++x) raw[x % S] = load_raw(x);
-
-    __syncthreads();   // every wave is done with the previous item's stage and output tile
+    for (unsigned k = 0; k < 3u; ++k) weight_piece(0u, k);
 #pragma unroll
-    for (unsigned j = 0; j < kCopyPieces; ++j) copy_piece(0u, 0u, j);
+    for (unsigned j = 0; j < kActPieces; ++j) act_piece(0u, j);
+#pragma unroll
+    for (unsigned k = 0; k < 3u; ++k) weight_piece(1u, k);
     // where each pair's results go and its route weight, for the publishing pass
     if (tid < kTileTokens && tid < it.tokens) {
         const unsigned long long ordered = it.pair0 + tid;
@@ -467,160 +459,157 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
         lds_write_uint2(kPairInfoBase + tid * 8u, make_uint2((unsigned)out_index, __float_as_uint(route_weight)));
     }
-    settle(first_raw, 0u);
+    __builtin_amdgcn_s_waitcnt(0x0f73u);   // vmcnt(3): window 0 and stage 0 have landed
+    settle(0u);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the window's reads have returned before it is refilled
 #pragma unroll
-    for (unsigned g = 0; g < 4u; ++g) {
-        lookup(g);
-        select(g);
+    for (unsigned x = 1; x + 1u < R; ++x) {
+#pragma unroll
+        for (unsigned j = 0; j < kActPieces; ++j) act_piece(x, j);
+#pragma unroll
+        for (unsigned k = 0; k < 3u; ++k) weight_piece(1u, k);
     }
 #pragma unroll
-    for (unsigned m = 0; m < 8u; ++m) permute(m);
-    __builtin_amdgcn_s_waitcnt(0x0070u);   // vmcnt(0) lgkmcnt(0): the copies above have landed
-    __syncthreads();
+    for (unsigned j = 0; j < 4u; ++j) round_piece(0u - 1u, j);
+    lookup(0u);
+    lookup(1u);
+    build(0u);
+    __syncthreads();   // every wave's share of stage 0 has landed
 
     float acc[NTB][16];
 #pragma unroll
     for (unsigned tb = 0; tb < NTB; ++tb)
 #pragma unroll
         for (unsigned i = 0; i < 16u; ++i) acc[tb][i] = 0.0f;
-    float rs[16];                    // row scales of the rows this lane holds sums of
+    v16i sum_lo[NTB], sum_hi[NTB];   // integer sums of the running superblock
+    v4i frag[2][NTB];                // [slot & 1]: re-requested for two slots on as soon as it is used
 #pragma unroll
-    for (unsigned i = 0; i < 16u; ++i) rs[i] = 0.0f;
-    float ts[NTB];                   // activation scales of this lane's token per token block
-    float ts_before = 0.0f;          // of the last token block of the superblock before
-#pragma unroll
-    for (unsigned tb = 0; tb < NTB; ++tb) ts[tb] = 0.0f;
-    v16i sum_lo[2], sum_hi[2];       // [phase & 1]: integer sums of a token block, scaled one phase later
-#pragma unroll
-    for (unsigned i = 0; i < 16u; ++i) {
-        sum_lo[1][i] = 0;
-        sum_hi[1][i] = 0;
+    for (unsigned tb = 0; tb < NTB; ++tb) {
+        frag[0][tb] = lds_read_v4i(frag_at + tb * 32u * kActPitch);
+        frag[1][tb] = lds_read_v4i((frag_at ^ 16u) + tb * 32u * kActPitch);
     }
-    v4i frag[2];                     // [slot & 1]: re-requested for two slots on as soon as it is used
-    enter_stage(stage_base(0u));
-    frag[0] = lds_read_v4i(piece_at[0]);
-    frag[1] = lds_read_v4i(piece_at[1]);
+    // Waits, counted in copies issued later than the one needed:
+    //   * before settle(sb + 1) at slot 5: window sb + 1 belongs to round sb - 2, so one full
+    //     round (sb - 1) may be in flight;
+    //   * at the barrier of superblock sb: stage sb + 1 belongs to round sb + 1 - R, so the
+    //     window of that round and R - 2 full rounds may be in flight.
+    constexpr unsigned kSettleInFlight = kRoundPieces;
+    constexpr unsigned kBarrierInFlight = 3u + (R - 2u) * kRoundPieces;
 
-    auto scale_rows = [&](unsigned parity, unsigned tb_of, float token_scale, unsigned m) {
+    for (unsigned sb = 0; sb < superblocks; ++sb) {
+        float rs[16];                // row scales of the rows this lane holds sums of
+        float ts[NTB];               // activation scales of this lane's token per token block
+        const unsigned stage = kStageBase + (sb % R) * kStageBytes;
 #pragma unroll
-        for (unsigned i = 2u * m; i < 2u * m + 2u; ++i) {
-            const int total = (sum_hi[parity][i] << 7) + sum_lo[parity][i];
-            acc[tb_of][i] = __builtin_fmaf(rs[i] * token_scale, (float)total, acc[tb_of][i]);
-        }
-    };
-
-    const unsigned periods = (superblocks + S - 1u) / S;
-    for (unsigned period = 0; period < periods; ++period) {
-        const unsigned base = stage_base(period);
+        for (unsigned m = 0; m < 8u; ++m) {
+            // ---- 2 NTB matrix instructions with the rest of the slot's work between them, a
+            // few instructions at a time ----
+            auto matrix = [&](unsigned tb, bool high) {
+                const v4i b = frag[m & 1u][tb];
+                v16i zero;
 #pragma unroll
-        for (unsigned u = 0; u < S; ++u) {
-            const unsigned sb = period * S + u;           // this superblock
+                for (unsigned i = 0; i < 16u; ++i) zero[i] = 0;
+                if (!high) sum_lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo[m & 1u], b, m ? sum_lo[tb] : zero, 0, 0, 0);
+                else sum_hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi[m & 1u], b, m ? sum_hi[tb] : zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            const unsigned next_chunk = (m + 1u) & 7u;
+            const uint4 lw = limbs[(next_chunk >> 1) & 1u];
+            unsigned selector[4];
+            matrix(0u, false);
+            // the table lookups of the chunk two slots on
+            lookup((m + 2u) & 7u);
+            __builtin_amdgcn_sched_barrier(0);
+            matrix(0u, true);
+            // selector words and low limbs of the next chunk
+            selector[0] = codes[next_chunk & 1u][0].x | signs[next_chunk & 1u][0].x;
+            selector[1] = codes[next_chunk & 1u][0].y | signs[next_chunk & 1u][0].y;
+            selector[2] = codes[next_chunk & 1u][1].x | signs[next_chunk & 1u][1].x;
+            selector[3] = codes[next_chunk & 1u][1].y | signs[next_chunk & 1u][1].y;
 #pragma unroll
-            for (unsigned tb = 0; tb < NTB; ++tb) {
-                const unsigned phase = u * NTB + tb;
-                const unsigned parity = phase & 1u;
+            for (unsigned i = 0; i < 4u; ++i) a_lo[next_chunk & 1u][i] = (int)__builtin_amdgcn_perm(lw.y, lw.x, selector[i]);
+            if constexpr (NTB == 2u) {
+                __builtin_amdgcn_sched_barrier(0);
+                matrix(1u, false);
+            }
+            // high limbs of the next chunk
 #pragma unroll
-                for (unsigned m = 0; m < 8u; ++m) {
-                    const unsigned slot = phase * 8u + m;         // within the period
-                    const unsigned sb_slot = tb * 8u + m;         // within the superblock
-                    // ---- two matrix instructions ----
-                    const v4i b = frag[slot & 1u];
-                    if (m == 0u) {
-                        v16i zero;
+            for (unsigned i = 0; i < 4u; ++i) a_hi[next_chunk & 1u][i] = (int)__builtin_amdgcn_perm(lw.w, lw.z, selector[i]);
+            if constexpr (NTB == 2u) {
+                __builtin_amdgcn_sched_barrier(0);
+                matrix(1u, true);
+            }
+            // ---- the fragments two slots on (past the barrier slot the addresses already
+            // point into the next superblock's stage) ----
+            {
+                unsigned piece = frag_at ^ (((m + 2u) & 7u) << 4);
+                asm volatile("" : "+v"(piece));   // kept opaque so that the token block offset stays the instruction's immediate
 #pragma unroll
-                        for (unsigned i = 0; i < 16u; ++i) zero[i] = 0;
-                        sum_lo[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo[0], b, zero, 0, 0, 0);
-                        sum_hi[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi[0], b, zero, 0, 0, 0);
-                    } else {
-                        sum_lo[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo[m], b, sum_lo[parity], 0, 0, 0);
-                        sum_hi[parity] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi[m], b, sum_hi[parity], 0, 0, 0);
-                    }
-                    // ---- this superblock's token scales at its start ----
-                    if (sb_slot == 0u) {
-                        ts_before = ts[NTB - 1u];
-                        const unsigned at = base + kStageActs + (u * T + r * NTB) * 4u;
-                        if constexpr (NTB == 4u) {
-                            const uint4 v = lds_read_uint4(at);
-                            ts[0] = __uint_as_float(v.x);
-                            ts[1] = __uint_as_float(v.y);
-                            ts[2] = __uint_as_float(v.z);
-                            ts[3] = __uint_as_float(v.w);
-                        } else if constexpr (NTB == 2u) {
-                            const uint2 v = lds_read_uint2(at);
-                            ts[0] = __uint_as_float(v.x);
-                            ts[1] = __uint_as_float(v.y);
-                        } else {
-                            ts[0] = __uint_as_float(lds_read_u32(at));
-                        }
-                    }
-                    // ---- the fragment two slots on (past the barrier slot the addresses already
-                    // point into the next period's stage) ----
-                    {
-                        const unsigned within = (slot + 2u) % kPeriodSlots;
-                        const unsigned phase_of = within / 8u;
-                        frag[slot & 1u] = lds_read_v4i(piece_at[within % 8u] +
-                                                       ((phase_of / NTB) * T + (phase_of % NTB) * 32u) * kActPitch);
-                    }
-                    // ---- scaling of two rows of the token block before this one ----
-                    scale_rows(parity ^ 1u, tb ? tb - 1u : NTB - 1u, tb ? ts[tb - 1u] : ts_before, m);
-                    // ---- this superblock's share of the decode of the next one ----
-                    if (sb_slot == 0u) settle(raw[(u + 1u) % S], sb + 1u);
-                    if (sb_slot == 1u) raw[(u + 1u) % S] = load_raw(sb + 1u + S);
-#pragma unroll
-                    for (unsigned g = 0; g < 4u; ++g) {
-                        if (sb_slot == Plan::select_slot(g)) select(g);
-                        if (sb_slot == Plan::lookup_slot(g)) lookup(g);
-                    }
-#pragma unroll
-                    for (unsigned k = 0; k < 8u; ++k)
-                        if (sb_slot == Plan::permute_slot(k)) permute(k);
-                    // ---- the row scales of this superblock, once the last sums of the one before
-                    // have been scaled ----
-                    if (sb_slot == 7u) {
-#pragma unroll
-                        for (unsigned q = 0; q < 4u; ++q) {
-                            const uint4 v = lds_read_uint4(row_scale_at + (sb & 1u) * 128u + (8u * q + 4u * h) * 4u);
-                            rs[4u * q] = __uint_as_float(v.x);
-                            rs[4u * q + 1u] = __uint_as_float(v.y);
-                            rs[4u * q + 2u] = __uint_as_float(v.z);
-                            rs[4u * q + 3u] = __uint_as_float(v.w);
-                        }
-                    }
-                    // ---- the next period's copies, one a slot ----
-                    if (slot < kCopyPieces) copy_piece(period + 1u, (period + 1u) & 1u, slot);
-                    if (slot == kBarrierSlot) {
-                        // every activation read of this period has returned and the next period's
-                        // copies have landed: after the barrier nobody reads this stage again
-                        __builtin_amdgcn_s_waitcnt(0x0070u);
-                        __syncthreads();
-                        const unsigned flip = (period & 1u) ? 0u - kStageBytes : kStageBytes;
-#pragma unroll
-                        for (unsigned k = 0; k < 8u; ++k) piece_at[k] += flip;
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                for (unsigned tb = 0; tb < NTB; ++tb) frag[m & 1u][tb] = lds_read_v4i(piece + tb * 32u * kActPitch);
+            }
+            if (m == 5u) {
+                // chunk 7's lookups are on their way: the next superblock's records replace this
+                // one's (its window has landed: see the counts above)
+                __builtin_amdgcn_s_waitcnt(0x0f70u | (kSettleInFlight & 15u) | ((kSettleInFlight >> 4) << 14));
+                settle(sb + 1u);
+            }
+            if (m == 4u) {
+                // this superblock's token scales, while its stage is still held
+                const unsigned at = stage + T * kActPitch + r * NTB * 4u;
+                if constexpr (NTB == 2u) {
+                    const uint2 v = lds_read_uint2(at);
+                    ts[0] = __uint_as_float(v.x);
+                    ts[1] = __uint_as_float(v.y);
+                } else {
+                    ts[0] = __uint_as_float(lds_read_u32(at));
                 }
             }
+            if (m == 6u) {
+                // the row scales of this superblock, for the scaling below
+#pragma unroll
+                for (unsigned q = 0; q < 4u; ++q) {
+                    const uint4 v = lds_read_uint4(row_scale_at + (sb & 1u) * 128u + (8u * q + 4u * h) * 4u);
+                    rs[4u * q] = __uint_as_float(v.x);
+                    rs[4u * q + 1u] = __uint_as_float(v.y);
+                    rs[4u * q + 2u] = __uint_as_float(v.z);
+                    rs[4u * q + 3u] = __uint_as_float(v.w);
+                }
+            }
+            if (m == kBarrierSlot) {
+                // Every read of this superblock's stage and of the next one's window has returned
+                // and this wave's share of the next stage has landed: after the barrier nobody
+                // reads this stage again and the next one is complete.
+                __builtin_amdgcn_s_waitcnt(0x0070u | (kBarrierInFlight & 15u) | ((kBarrierInFlight >> 4) << 14));
+                __syncthreads();
+                const unsigned flip = (sb % R == R - 1u) ? 0u - (R - 1u) * kStageBytes : kStageBytes;
+                frag_at += flip;
+            }
+            // ---- the round of copies into the stage and the window just released: two pieces a
+            // slot behind the barrier, the rest at the start of the next superblock ----
+            if (m > kBarrierSlot) {
+                round_piece(sb, 2u * (m - kBarrierSlot - 1u));
+                round_piece(sb, 2u * (m - kBarrierSlot - 1u) + 1u);
+            }
+            if (m < kRoundPieces - 4u) round_piece(sb - 1u, 4u + m);
+            // ---- the superblock's sums are complete: ((0.125 d_w) d_a) (128 hi + lo) ----
+            if (m == 7u) {
+#pragma unroll
+                for (unsigned tb = 0; tb < NTB; ++tb)
+#pragma unroll
+                    for (unsigned i = 0; i < 16u; ++i) {
+                        const int total = (sum_hi[tb][i] << 7) + sum_lo[tb][i];
+                        acc[tb][i] = __builtin_fmaf(rs[i] * ts[tb], (float)total, acc[tb][i]);
+                    }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
-    // the last token block of the last superblock
-#pragma unroll
-    for (unsigned m = 0; m < 8u; ++m) scale_rows(1u, NTB - 1u, ts[NTB - 1u], m);
+    __builtin_amdgcn_s_waitcnt(0x0070u);   // copies past the end have landed before the tile reuses the stages
 
     // ---- publish: the lane holds, for tokens 32 tb + r, rows 8 q + 4 h + j of its 32 (j < 4) ----
-    // The tile goes through LDS as [token][value], values 0-63 the gate sums and 64-127 the up
-    // sums of the item's 64 row pairs when fused, else the 128 rows' sums.
-#pragma unroll
-    for (unsigned tb = 0; tb < NTB; ++tb)
-#pragma unroll
-        for (unsigned q = 0; q < 4u; ++q) {
-            unsigned column;
-            if constexpr (FUSED_UP) column = (q >= 2u ? 64u : 0u) + wave * 16u + 8u * (q & 1u) + 4u * h;
-            else column = wave * 32u + 8u * q + 4u * h;
-            lds_write_uint4(kStageBase + (tb * 32u + r) * kOutPitch + column * 4u,
-                            make_uint4(__float_as_uint(acc[tb][4u * q]), __float_as_uint(acc[tb][4u * q + 1u]),
-                                       __float_as_uint(acc[tb][4u * q + 2u]), __float_as_uint(acc[tb][4u * q + 3u])));
-        }
-    __syncthreads();
+    // Half of the tile at a time (waves 0-3, then waves 4-7) goes through LDS as [token][value],
+    // values 0-63 the gate sums and 64-127 the up sums of the half's 64 row pairs when fused,
+    // else the 128 rows' sums.
     auto store4 = [&](unsigned long long out_index, unsigned row, const float (&value)[4]) {
         const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
                           finite_f32(value[3]);
@@ -632,29 +621,49 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
             for (unsigned j = 0; j < 4u; ++j)
                 if (row + j < a.out_rows) pr.out[out_index * a.out_rows + row + j] = value[j];
     };
-    constexpr unsigned kQuads = kItemRows / 4u;       // groups of four output values per token
+    constexpr unsigned kHalfRows = kItemRows / 2u;
+    constexpr unsigned kQuads = kHalfRows / 4u;       // groups of four output values per token
     const float limit_f32 = (float)a.limit;
 #pragma unroll 1
-    for (unsigned unit = tid; unit < T * kQuads; unit += kRowThreads) {
-        const unsigned token = unit / kQuads, quad = unit % kQuads;
-        if (token >= it.tokens) break;
-        const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
-        const unsigned row = it.row_tile * kItemRows + 4u * quad;
-        if (row >= a.out_rows) continue;
-        const uint4 g = lds_read_uint4(kStageBase + token * kOutPitch + quad * 16u);
-        if constexpr (FUSED_UP) {
-            const uint4 up = lds_read_uint4(kStageBase + token * kOutPitch + 256u + quad * 16u);
-            const float route_weight = __uint_as_float(info.y);
-            const float value[4] = {
-                swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(up.x), route_weight, a.limit, limit_f32),
-                swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(up.y), route_weight, a.limit, limit_f32),
-                swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(up.z), route_weight, a.limit, limit_f32),
-                swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(up.w), route_weight, a.limit, limit_f32)};
-            store4(info.x, row, value);
-        } else {
-            const float value[4] = {bf16_round(__uint_as_float(g.x)), bf16_round(__uint_as_float(g.y)),
-                                    bf16_round(__uint_as_float(g.z)), bf16_round(__uint_as_float(g.w))};
-            store4(info.x, row, value);
+    for (unsigned half = 0; half < 2u; ++half) {
+        __syncthreads();   // the stage (first half) or the first half's tile is no longer read
+        if ((wave >> 2) == half) {
+            const unsigned w4 = wave & 3u;
+#pragma unroll
+            for (unsigned tb = 0; tb < NTB; ++tb)
+#pragma unroll
+                for (unsigned q = 0; q < 4u; ++q) {
+                    unsigned column;
+                    if constexpr (FUSED_UP) column = (q >= 2u ? 64u : 0u) + w4 * 16u + 8u * (q & 1u) + 4u * h;
+                    else column = w4 * 32u + 8u * q + 4u * h;
+                    lds_write_uint4(kStageBase + (tb * 32u + r) * kOutPitch + column * 4u,
+                                    make_uint4(__float_as_uint(acc[tb][4u * q]), __float_as_uint(acc[tb][4u * q + 1u]),
+                                               __float_as_uint(acc[tb][4u * q + 2u]), __float_as_uint(acc[tb][4u * q + 3u])));
+                }
+        }
+        __syncthreads();
+#pragma unroll 1
+        for (unsigned unit = tid; unit < T * kQuads; unit += kRowThreads) {
+            const unsigned token = unit / kQuads, quad = unit % kQuads;
+            if (token >= it.tokens) break;
+            const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
+            const unsigned row = it.row_tile * kItemRows + half * kHalfRows + 4u * quad;
+            if (row >= a.out_rows) continue;
+            const uint4 g = lds_read_uint4(kStageBase + token * kOutPitch + quad * 16u);
+            if constexpr (FUSED_UP) {
+                const uint4 up = lds_read_uint4(kStageBase + token * kOutPitch + 256u + quad * 16u);
+                const float route_weight = __uint_as_float(info.y);
+                const float value[4] = {
+                    swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(up.x), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(up.y), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(up.z), route_weight, a.limit, limit_f32),
+                    swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(up.w), route_weight, a.limit, limit_f32)};
+                store4(info.x, row, value);
+            } else {
+                const float value[4] = {bf16_round(__uint_as_float(g.x)), bf16_round(__uint_as_float(g.y)),
+                                        bf16_round(__uint_as_float(g.z)), bf16_round(__uint_as_float(g.w))};
+                store4(info.x, row, value);
+            }
         }
     }
 }
@@ -674,23 +683,23 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
 
     mfma_tables_fill();
     if (tid == 0u) {
-        // Full 128-pair tiles come first in the item list, then the partial last tiles by size,
+        // Full 64-pair tiles come first in the item list, then the partial last tiles by size,
         // largest first: every workgroup, walking the list with the grid's stride, gets the same
         // share of each kind of item, and the short items come last.
-        unsigned cursor = 0u, members[3] = {0u, 0u, 0u};
+        unsigned cursor = 0u, members[2] = {0u, 0u};
         for (unsigned b = 0; b < buckets && b < 256u; ++b) {
             lds_write_u32(kTileStartBase + 4u * b, cursor);
             const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[b];
             cursor += (unsigned)(n / kTileTokens);
             const unsigned rest = (unsigned)(n % kTileTokens);
             if (rest) {
-                const unsigned c = rest > 64u ? 0u : rest > 32u ? 1u : 2u;
+                const unsigned c = rest > 32u ? 0u : 1u;
                 lds_write_u16(kClassListBase + (c * 256u + members[c]) * 2u, b);
                 ++members[c];
             }
         }
         lds_write_u32(kTileStartBase + 4u * (buckets < 256u ? buckets : 256u), cursor);
-        for (unsigned c = 0; c < 3u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
+        for (unsigned c = 0; c < 2u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
     }
     __syncthreads();
     if (buckets == 0u || buckets > 256u) {
@@ -699,12 +708,12 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
     }
 
     // weight rows (gate/up row pairs when fused) per work item
-    constexpr unsigned kItemRows = FUSED_UP ? 64u : 128u;
+    constexpr unsigned kItemRows = FUSED_UP ? 128u : 256u;
     const unsigned row_tiles = (a.out_rows + kItemRows - 1u) / kItemRows;
     const unsigned long long full_items = (unsigned long long)lds_read_u32(kTileStartBase + 4u * buckets) * row_tiles;
-    unsigned members[3];
+    unsigned members[2];
     unsigned long long items = full_items;
-    for (unsigned c = 0; c < 3u; ++c) {
+    for (unsigned c = 0; c < 2u; ++c) {
         members[c] = lds_read_u32(kClassCountBase + 4u * c);
         items += (unsigned long long)members[c] * row_tiles;
     }
@@ -735,9 +744,9 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
         } else {
             unsigned long long rest = item - full_items;
             unsigned c = 0u;
-            while (c < 2u && rest >= (unsigned long long)members[c] * row_tiles) {
-                rest -= (unsigned long long)members[c] * row_tiles;
-                ++c;
+            if (rest >= (unsigned long long)members[0] * row_tiles) {
+                rest -= (unsigned long long)members[0] * row_tiles;
+                c = 1u;
             }
             if (!members[c]) {
                 if (tid == 0u) raise_status(a.status, 2);
@@ -760,8 +769,7 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
         if (it.tokens <= 32u) rows_item<FUSED_UP, 1u>(a, it);
-        else if (it.tokens <= 64u) rows_item<FUSED_UP, 2u>(a, it);
-        else rows_item<FUSED_UP, 4u>(a, it);
+        else rows_item<FUSED_UP, 2u>(a, it);
     }
 }
 
