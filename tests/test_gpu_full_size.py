@@ -6,7 +6,7 @@ over the whole batch, and the CPU oracle on two of the rows.
   * a row's result does not depend on the batch it arrives in (halves of the batch and a single
     row against the full batch, bit for bit): the sweeps group pairs by expert, four to a sweep,
     so the grouping changes with the batch while every pair's arithmetic must not;
-  * routing equals the oracle's for every row, and two rows' outputs match the oracle's
+  * routing equals the oracle's for every row, and eight rows' outputs match the oracle's
     (src/graph/moe.c:497-622, src/runtime/moe.c:596-645) within the path's tolerance.
 """
 import numpy as np
@@ -37,12 +37,76 @@ def layer_weights(gpu):
     return routed, shared
 
 
-def within_tolerance(got, want):
+# Measured on MI355X (printed by every run of these tests). Stage by stage, against the oracle fed
+# with the device's own stage input, a value either equals the CPU path's or lies one bf16 step
+# away (the oracle adds a row's 28 superblock terms in double, the kernels in fp32, so the
+# unrounded values differ in their last bits): 1.2e-4 (decode sweeps, 8 rows) and 2.4e-4
+# (matrix-core kernels, 4 rows) of the SwiGLU products, 5.9e-5 and 3.9e-5 of the expert outputs.
+# End to end the fraction beyond 1e-3 relative / 1e-5 absolute depends on the rows looked at: one
+# product that rounds the other way changes its row's Q8_K block and with it, by less than a
+# step, all 7168 outputs of that expert, so a few per cent of them round the other way in turn
+# (decode, 8 rows: 1.7e-5 of the outputs; prefill, 4 rows: 5.1e-2). The stage bounds are two to
+# five times what is measured, the end-to-end ones twice the larger measurement.
+MID_FLIP_BOUND = 6e-4
+OUT_FLIP_BOUND = 1e-4
+DECODE_FLIP_BOUND = 1e-3
+PREFILL_FLIP_BOUND = 1e-1
+
+
+def one_step_or_inside(got, want):
+    """Values that differ are one bf16 step apart, or so small that they lie inside the path's
+    tolerance anyway (sums that cancel to almost nothing)."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    return bool(np.all((err <= BF16_STEP * 1.001 * np.abs(want)) | (err <= 1e-5 + 1e-3 * np.abs(want))))
+
+
+def stage_flip_rates(oracle, layer, routed, x, picked, label):
+    """The picked rows' pairs stage by stage: SwiGLU products against the oracle's, expert outputs
+    against the oracle fed with the device's own products. Differences are single bf16 steps;
+    returns their fractions."""
+    qt = oracle.IQ2_XXS
+    gate, up, down = (t.cpu().numpy() for t in routed)
+    gb = oracle.row_bytes(qt, HIDDEN) * INTERMEDIATE
+    db = oracle.row_bytes(qt, INTERMEDIATE) * HIDDEN
+    sel = layer.selected.cpu().numpy().reshape(-1)
+    wts = layer.weights.cpu().numpy().reshape(-1)
+    order = layer.worklist.order.cpu().numpy()[:sel.size]
+    position_of = np.empty_like(order)
+    position_of[order] = np.arange(order.size)
+    mid_bad = mid_all = out_bad = out_all = 0
+    for row in picked:
+        for rank in range(TOPK):
+            source = row * TOPK + rank
+            e = int(sel[source])
+            mid = layer.intermediate_f32[int(position_of[source])].cpu().numpy()
+            rc, _, want_mid, _ = oracle.moe_expert((qt, qt, qt), gate[e * gb:(e + 1) * gb], up[e * gb:(e + 1) * gb],
+                                                   down[e * db:(e + 1) * db], HIDDEN, INTERMEDIATE,
+                                                   x[row].cpu().numpy(), float(wts[source]), act_q8=True)
+            assert rc == 0
+            differs = mid != want_mid
+            assert one_step_or_inside(mid[differs], want_mid[differs])
+            mid_bad += int(differs.sum())
+            mid_all += mid.size
+            raw = oracle.q8_matvec(qt, down[e * db:(e + 1) * db], HIDDEN, INTERMEDIATE, oracle.q8k_quantize(mid), 1)[0]
+            want_out = np.array([oracle.lib().yvo_bf16_round(np.float32(v)) for v in raw], np.float32)
+            got_out = layer.pair_outputs[source].cpu().numpy()
+            differs = got_out != want_out
+            assert one_step_or_inside(got_out[differs], want_out[differs])
+            out_bad += int(differs.sum())
+            out_all += got_out.size
+    print(f"{label}: {mid_bad} of {mid_all} SwiGLU products ({mid_bad / mid_all:.3e}) and {out_bad} of {out_all} "
+          f"expert outputs ({out_bad / out_all:.3e}) one bf16 step from the oracle's")
+    return mid_bad / mid_all, out_bad / out_all
+
+
+def within_tolerance(got, want, bound, label):
     """1e-3 relative / 1e-5 absolute; beyond it only values one bf16 step apart (a sum that sits
-    on a rounding boundary), and few of them."""
+    on a rounding boundary), and no more of them than `bound`. The measured fraction is printed."""
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     outside = err > 1e-5 + 1e-3 * np.abs(want)
-    assert outside.mean() < 2e-2
+    print(f"{label}: {int(outside.sum())} of {outside.size} outputs beyond 1e-3 / 1e-5 "
+          f"(fraction {outside.mean():.3e}), bit-identical {np.mean(got == want):.4f}")
+    assert outside.mean() < bound
     assert np.all(err[outside] <= BF16_STEP * 1.001 * np.abs(want[outside]))
 
 
@@ -82,8 +146,8 @@ def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
         assert np.array_equal(selected[r].cpu().numpy().astype(np.uint64), want_selected)
         assert np.max(np.abs(weights[r].cpu().numpy() - want_weights)) <= 1e-6
 
-    # two rows through the CPU oracle with the same weights
-    picked = [0, 17]
+    # eight rows through the CPU oracle with the same weights
+    picked = [0, 4, 9, 13, 17, 22, 26, 31]
     want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                             qtypes=(oracle.IQ2_XXS,) * 3, routed=[t.cpu().numpy() for t in routed],
                             shared=[t.cpu().numpy() for t in shared], inputs=x[picked].cpu().numpy(),
@@ -91,13 +155,17 @@ def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
                             limit=10.0, act_q8=True, threads=16)
     got = full[picked].cpu().numpy()
     assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
-    within_tolerance(got, want["combined"])
+    within_tolerance(got, want["combined"], DECODE_FLIP_BOUND, "decode layer, 8 rows against the oracle")
+    full_again, _, _ = run(0, ROWS)     # leaves the whole batch's stage buffers in place
+    mid_rate, out_rate = stage_flip_rates(oracle, layer, routed, x, picked, "decode layer, 8 rows stage by stage")
+    assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
 
 
 def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
-    """2048 rows through the matrix-core kernels: the same bits twice, the first 32 rows against
-    the decode sweeps' result for them (another summation order: within tolerance), one row
-    against the oracle."""
+    """2048 rows whose experts follow a Zipf(1.1) popularity (buckets from a handful of pairs to
+    more than a thousand) through the matrix-core kernels: the same bits twice, the first 32 rows
+    against the decode sweeps' result for them (another summation order: within tolerance), four
+    rows against the oracle."""
     from yvex_amd import kernels as K
     from yvex_amd.moe import MoeLayer
     routed, shared = layer_weights
@@ -105,7 +173,9 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
     gen = torch.Generator(device=gpu)
     gen.manual_seed(7)
     x = torch.randn((rows, HIDDEN), device=gpu, generator=gen)
-    logits = torch.randn((rows, EXPERTS), device=gpu, generator=gen)
+    rank = torch.randperm(EXPERTS, device=gpu, generator=gen).float() + 1.0
+    uniform = torch.rand((rows, EXPERTS), device=gpu, generator=gen).clamp_(1e-9, 1.0 - 1e-9)
+    logits = rank.pow(-1.1).log()[None, :] - (-uniform.log()).log()      # Gumbel top-k over log-popularity
     qt = K.IQ2_XXS
     common = dict(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtypes=(qt, qt, qt),
                   routed=routed, shared=shared, scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
@@ -119,24 +189,34 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
     assert torch.equal(first.view(torch.int32), second.view(torch.int32))
     assert torch.isfinite(first).all()
     selected = wide.selected.clone()
-    picked = 1000
-    keep = list(range(32)) + [picked]
+    picked = [5, 700, 1000, 1900]
+    mid_rate, out_rate = stage_flip_rates(oracle, wide, routed, x, picked, "prefill layer, 4 rows stage by stage")
+    assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
+    keep = list(range(32)) + picked
+    populations = torch.bincount(selected.reshape(-1).long(), minlength=EXPERTS).cpu().numpy()
+    assert populations.max() > 1000 and (populations[populations > 0] < 32).any()
+    print("bucket populations of the experts of the rows checked against the oracle:",
+          [sorted(populations[selected[r].cpu().numpy().astype(np.int64)].tolist()) for r in picked])
     wide_pairs = wide.pair_outputs.view(rows, TOPK, HIDDEN)[keep].cpu().numpy()    # [row, rank, column]
     wide_shared = wide.shared_out[keep].cpu().numpy()
     del wide
 
-    def close_by_row(got, want, scale):
+    def close_by_row(got, want, scale, bound=2e-2, label=None):
         """Few values beyond the path's tolerance (1e-3 relative / 1e-5 absolute), and those by no
         more than two bf16 steps at the size of the row's largest terms: an intermediate value
         that rounds the other way (the SwiGLU product, an expert's output) moves the results it
         feeds by a step at its own size, whatever their own size is."""
         err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-        assert (err > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
+        outside = err > 1e-5 + 1e-3 * np.abs(want)
+        if label:
+            print(f"{label}: {int(outside.sum())} of {outside.size} outputs beyond 1e-3 / 1e-5 "
+                  f"(fraction {outside.mean():.3e}), bit-identical {np.mean(got == want):.4f}")
+        assert outside.mean() < bound
         assert np.all(err <= 1e-5 + 1e-3 * np.abs(want) + 2 * BF16_STEP * scale)
 
-    def combined_close(got, want, pairs, shared_rows):
+    def combined_close(got, want, pairs, shared_rows, bound=2e-2, label=None):
         scale = np.abs(pairs).max(axis=2).sum(axis=1) + np.abs(shared_rows).max(axis=1)   # per row
-        close_by_row(got, want, scale[:, None])
+        close_by_row(got, want, scale[:, None], bound, label)
 
     narrow = MoeLayer(max_rows=32, **common)
     sweeps = narrow.run(x[:32].contiguous(), logits[:32].contiguous())[:32].clone()
@@ -150,8 +230,9 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
     combined_close(first[:32].cpu().numpy(), sweeps.cpu().numpy(), wide_pairs[:32], wide_shared[:32])
     want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                             qtypes=(oracle.IQ2_XXS,) * 3, routed=[t.cpu().numpy() for t in routed],
-                            shared=[t.cpu().numpy() for t in shared], inputs=x[[picked]].cpu().numpy(),
-                            logits=logits[[picked]].cpu().numpy(), scoring=oracle.SIGMOID, normalize=True,
+                            shared=[t.cpu().numpy() for t in shared], inputs=x[picked].cpu().numpy(),
+                            logits=logits[picked].cpu().numpy(), scoring=oracle.SIGMOID, normalize=True,
                             scaling=1.0, limit=10.0, act_q8=True, threads=16)
-    assert np.array_equal(selected[[picked]].cpu().numpy().astype(np.uint64), want["selected"])
-    combined_close(first[[picked]].cpu().numpy(), want["combined"], wide_pairs[32:], wide_shared[32:])
+    assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
+    combined_close(first[picked].cpu().numpy(), want["combined"], wide_pairs[32:], wide_shared[32:],
+                   PREFILL_FLIP_BOUND, "prefill layer, 4 rows against the oracle")

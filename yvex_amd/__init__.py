@@ -11,8 +11,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# YVEX_ROCM_LIB points at another build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("YVEX_ROCM_LIB") or os.path.join(HERE, "libyvex_rocm.so")
+LIB_PATH = os.path.join(HERE, "libyvex_rocm.so")
 
 _lib = None
 

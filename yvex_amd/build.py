@@ -29,7 +29,6 @@ HIP_FLAGS = [
     # keep the compiler from forming packed-FP32 instructions on its own
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-HIP_FLAGS += os.environ.get("YVEX_HIP_EXTRA_FLAGS", "").split()   # e.g. -DNAME for a local experiment
 C_FLAGS = ["-std=c11", "-O2", "-fPIC", "-Wall", "-Wextra", "-ffp-contract=off", "-pthread",
            "-D_POSIX_C_SOURCE=200809L", f"-I{os.path.join(ROOT, 'include')}"]
 

@@ -771,11 +771,6 @@ static int launch_grouped(const GroupedArgs &a, bool q8, bool fused, hipStream_t
 static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool fused,
                             hipStream_t stream)
 {
-    static int generic_only = -1;   // YVEX_SWEEP_GENERIC=1 keeps the generic kernel (comparison runs)
-    if (generic_only < 0) {
-        const char *text = getenv("YVEX_SWEEP_GENERIC");
-        generic_only = text && text[0] == '1';
-    }
     bool aligned = true;   // the specialised sweeps load dwords: bases and strides must allow it
     for (unsigned i = 0; i < a.problems; ++i) {
         const GroupedProblem &pr = a.problem[i];
@@ -784,7 +779,7 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
     }
     unsigned long long all_pairs = 0ull;
     for (unsigned i = 0; i < a.problems; ++i) all_pairs += a.problem[i].pairs;
-    if (qtype == QT_IQ2_XXS && q8 && !generic_only && aligned &&
+    if (qtype == QT_IQ2_XXS && q8 && aligned &&
         iq2_sweep_supported(a.width, a.out_rows, all_pairs))
         return launch_iq2_sweep(a, fused, stream);
     switch (qtype) {
