@@ -259,6 +259,17 @@ int yvex_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes, yvex_hip_str
 int yvex_hip_stream_create(yvex_hip_stream *out);
 int yvex_hip_stream_destroy(yvex_hip_stream stream);
 int yvex_hip_stream_sync(yvex_hip_stream stream);
+/* Launch graphs, the counterpart of yvex_cuda_graph_execute (src/backend/cuda/moe.c:1665-1681):
+ * capture_begin puts the stream in capture mode, the launch wrappers above then record instead
+ * of running, capture_end instantiates the recording (refusing one that holds anything but
+ * kernel nodes, and reporting how many it holds) and capture_abort discards it. A graph is
+ * launched on a stream like a kernel and stays valid while every address it recorded does. */
+typedef void *yvex_hip_graph;
+int yvex_hip_capture_begin(yvex_hip_stream stream);
+int yvex_hip_capture_end(yvex_hip_stream stream, yvex_hip_graph *out, uint64_t *kernel_nodes);
+int yvex_hip_capture_abort(yvex_hip_stream stream);
+int yvex_hip_graph_launch(yvex_hip_graph graph, yvex_hip_stream stream);
+int yvex_hip_graph_destroy(yvex_hip_graph graph);
 /* 1 when the gfx950 code object for the kernels is loadable on the current device. */
 int yvex_hip_kernels_loadable(void);
 const char *yvex_hip_last_error(void);

@@ -616,6 +616,74 @@ def test_execute_rows_deferred_completion(backend, oracle):
     assert (err_abs > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
 
 
+@pytest.mark.parametrize("kwargs", [
+    dict(rows=5),                                                                # decode sweeps
+    dict(rows=3, qtype="Q4_K", shared=False, scoring=abi.SCORING_SIGMOID),       # generic sweeps
+    dict(rows=4, streams=4, hidden=512, iterations=5),                           # residual streams
+    dict(rows=3, hash_vocab=50),                                                 # hash router
+    dict(rows=200, hidden=768, intermediate=512, experts=4, scoring=abi.SCORING_SIGMOID),  # matrix cores
+], ids=["sweep", "generic", "streams", "hash", "matrix"])
+def test_execute_rows_graph_replays_equal_eager(backend, oracle, kwargs):
+    """src/backend/cuda/moe.c:1650-1681: a job that does not ask for eager execution runs as a
+    launch graph keyed on its topology. Here the key's first use runs eagerly, the second is
+    captured, later ones are replayed; every one of them must give the eager bits, also for rows
+    written between replays and with other eager work on the stream in between."""
+    b = backend
+    case = MoeCase(b, oracle, **kwargs)
+    b.workspace(case.workspace_bytes)
+    width = case.x.shape[1]
+    rng = np.random.default_rng(7)
+
+    def run(rows_now, eager):
+        rc = b.lib.yvex_backend_tensor_write(b.handle, case.rows_in, rows_now.ctypes.data, rows_now.nbytes,
+                                             C.byref(b.err))
+        assert rc == 0, b.err.message
+        case.job.eager_execution = int(eager)
+        assert case.execute() == 0, case.err.message
+        facts = (case.result.graph_launches, case.result.graph_captures, case.result.graph_replays)
+        return (b.read_f32(case.rows_out, case.rows * width).copy(), case.combined.copy(),
+                case.sel.copy(), case.wts.copy(), facts, case.result.kernel_launches)
+
+    batches = [case.x] + [np.ascontiguousarray(case.x * s + rng.standard_normal(case.x.shape) * 0.05,
+                                               np.float32) for s in (0.5, -1.0, 2.0, 1.0, 0.25)]
+    if case.streams:      # the CPU path feeds bf16 values; keep the later batches of that kind too
+        batches = [((x.view(np.uint32) + 0x8000) & 0xffff0000).view(np.float32) for x in batches]
+    want = [run(x, eager=True) for x in batches]
+    assert all(w[4] == (0, 0, 0) for w in want)
+    expected_facts = [(0, 0, 0), (1, 1, 0)] + [(1, 0, 1)] * (len(batches) - 2)
+    for step, x in enumerate(batches):
+        got = run(x, eager=False)
+        assert got[4] == expected_facts[step], (step, got[4])
+        assert got[5] == want[step][5]
+        for name, g, w in zip(("rows", "combined", "selected", "weights"), got[:4], want[step][:4]):
+            assert np.array_equal(g.view(np.uint8), w.view(np.uint8)), (step, name)
+        # other work between replays: an eager batch on the same stream
+        run(batches[(step + 1) % len(batches)], eager=True)
+
+
+def test_execute_rows_graph_key_follows_addresses(backend, oracle):
+    """Rows handed over in another tensor are another key: the graph recorded for the first
+    tensor must not be replayed against it."""
+    b = backend
+    case = MoeCase(b, oracle, rows=5)
+    b.workspace(case.workspace_bytes)
+    for _ in range(3):
+        assert case.execute() == 0, case.err.message
+    assert case.result.graph_replays == 1
+    first = b.read_f32(case.rows_out, case.rows * case.hidden).copy()
+    other_in, other_out = b.f32(case.x * 0.5), b.empty_f32(case.rows * case.hidden)
+    case.batch.device_rows, case.batch.device_outputs = other_in, other_out
+    assert case.execute() == 0, case.err.message
+    assert case.result.graph_launches == 0            # first sight of the new key
+    assert case.execute() == 0 and case.result.graph_captures == 1
+    got = b.read_f32(other_out, case.rows * case.hidden)
+    case.job.eager_execution = 1
+    assert case.execute() == 0 and case.result.graph_launches == 0
+    assert np.array_equal(got, b.read_f32(other_out, case.rows * case.hidden))
+    assert np.array_equal(first, b.read_f32(case.rows_out, case.rows * case.hidden))
+    assert not np.array_equal(first, got)
+
+
 # ---- token-local operation: src/backend/cuda/moe.c:516-842 --------------------------------------
 
 class TokenLocal:

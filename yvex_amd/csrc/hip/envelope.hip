@@ -310,16 +310,19 @@ extern "C" int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const
     if (!(rms_epsilon > 0.0) || !(mhc_epsilon > 0.0) || !(post_multiplier > 0.0) ||
         rms_epsilon > 1.0e300 || mhc_epsilon > 1.0e300 || post_multiplier > 1.0e300)
         return ST_INVALID_ARG;
+    static std::once_flag once;
     static bool prepared = false;
-    if (!prepared) {
-        if (hipFuncSetAttribute((const void *)mhc_ingress_kernel<256>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)(kEnvelopeMaxWidth * sizeof(float))) != hipSuccess ||
+    std::call_once(once, [] {
+        prepared =
+            hipFuncSetAttribute((const void *)mhc_ingress_kernel<256>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)(kEnvelopeMaxWidth * sizeof(float))) == hipSuccess &&
             hipFuncSetAttribute((const void *)mhc_ingress_kernel<1024>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)(kEnvelopeMaxWidth * sizeof(float))) != hipSuccess) {
-            set_last_error_text("mhc_ingress: the collapsed row does not fit in LDS");
-            return ST_BACKEND;
-        }
-        prepared = true;
+                                (int)(kEnvelopeMaxWidth * sizeof(float))) == hipSuccess;
+        if (!prepared) (void)hipGetLastError();
+    });
+    if (!prepared) {
+        set_last_error_text("mhc_ingress: the collapsed row does not fit in LDS");
+        return ST_BACKEND;
     }
     const int quads = width % 4u == 0u && !(((uintptr_t)rows | (uintptr_t)norm | (uintptr_t)normalized) & 15u);
     const unsigned lds = (unsigned)(width * sizeof(float));

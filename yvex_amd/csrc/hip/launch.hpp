@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../../include/yvex_rocm_kernels.h"
 
 namespace yvex {
@@ -25,6 +27,20 @@ inline int check_launch(const char *where)
     }
     return ST_OK;
 }
+
+// Compute units of the current device (read once, thread-safe).
+int compute_units();
+
+// Raise a kernel's dynamic LDS limit once per process; safe when several threads launch.
+#define YVEX_ALLOW_DYNAMIC_LDS(kernel, bytes)                                                   \
+    do {                                                                                        \
+        static std::once_flag once_;                                                            \
+        std::call_once(once_, [] {                                                              \
+            if (hipFuncSetAttribute((const void *)(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)(bytes)) != hipSuccess)                                \
+                (void)hipGetLastError();                                                        \
+        });                                                                                     \
+    } while (0)
 
 inline hipStream_t as_stream(yvex_hip_stream s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -728,34 +728,13 @@ __global__ __launch_bounds__(256) void reduce_combine_kernel(
     }
 }
 
-static int grouped_grid()
-{
-    static int units = 0;
-    if (!units) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
-            (void)hipGetLastError();
-            return 256;
-        }
-        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
-    return units;
-}
-
 template <unsigned QT, bool Q8, bool FUSED>
 static int launch_grouped_variant(const GroupedArgs &a, hipStream_t stream)
 {
     const size_t lds = (QT == QT_IQ2_XXS ? kIq2WideBytes : 0u) +
                        (size_t)kGroupedWaves * 2u * kItemRowsMax * kPass * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void *)grouped_kernel<QT, Q8, FUSED>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            (void)hipGetLastError();
-        configured = true;
-    }
-    grouped_kernel<QT, Q8, FUSED><<<grouped_grid(), kGroupedThreads, lds, stream>>>(a);
+    YVEX_ALLOW_DYNAMIC_LDS((grouped_kernel<QT, Q8, FUSED>), lds);
+    grouped_kernel<QT, Q8, FUSED><<<compute_units(), kGroupedThreads, lds, stream>>>(a);
     return check_launch("moe_grouped");
 }
 
@@ -872,14 +851,7 @@ extern "C" int yvex_hip_worklist_build(const uint64_t *selected, uint64_t pairs,
     if (rows > kWorklistMaxRows) return ST_BOUNDS;
     int with_below = 0;
     const size_t lds = worklist_lds_bytes(experts, rows, &with_below);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void *)worklist_kernel,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWorklistLdsLimit) !=
-            hipSuccess)
-            (void)hipGetLastError();
-        configured = true;
-    }
+    YVEX_ALLOW_DYNAMIC_LDS(worklist_kernel, kWorklistLdsLimit);
     if (lds > kWorklistLdsLimit) return ST_BOUNDS;
     worklist_kernel<<<1, 1024, lds, as_stream(stream)>>>(
         (const unsigned long long *)selected, (unsigned)pairs, (unsigned)topk, (unsigned)experts,

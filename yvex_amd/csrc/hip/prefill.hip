@@ -773,32 +773,11 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
     }
 }
 
-static int mfma_grid()
-{
-    static int units = 0;
-    if (!units) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
-            (void)hipGetLastError();
-            return 256;
-        }
-        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
-    return units;
-}
-
 template <bool FUSED_UP>
 static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
 {
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void *)mfma_iq2_kernel<FUSED_UP>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsBytes) != hipSuccess)
-            (void)hipGetLastError();
-        configured = true;
-    }
-    mfma_iq2_kernel<FUSED_UP><<<mfma_grid(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
+    YVEX_ALLOW_DYNAMIC_LDS(mfma_iq2_kernel<FUSED_UP>, kMfmaLdsBytes);
+    mfma_iq2_kernel<FUSED_UP><<<compute_units(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
     return check_launch("moe_rows_mfma");
 }
 

@@ -3,6 +3,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <vector>
+
 #include "launch.hpp"
 
 namespace yvex {
@@ -16,6 +19,23 @@ void set_last_error(const char *where, hipError_t code)
 void set_last_error_text(const char *text)
 {
     snprintf(g_last_error, sizeof(g_last_error), "%s", text);
+}
+
+// Compute units of the current device, read once: persistent kernels size their grids with it.
+int compute_units()
+{
+    static std::once_flag once;
+    static int units = 256;
+    std::call_once(once, [] {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess &&
+            prop.multiProcessorCount > 0)
+            units = prop.multiProcessorCount;
+        else
+            (void)hipGetLastError();
+    });
+    return units;
 }
 
 static int wrap(const char *where, hipError_t code)
@@ -183,6 +203,73 @@ int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream
     if (blocks > 0x7fffffffull) return ST_BOUNDS;
     fill_u32_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>((uint32_t *)dst, value, count);
     return check_launch("fill_u32");
+}
+
+// ---- launch graphs: a captured kernel sequence replayed with one submission ----
+
+int yvex_hip_capture_begin(yvex_hip_stream stream)
+{
+    return wrap("hipStreamBeginCapture",
+                hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+}
+
+int yvex_hip_capture_abort(yvex_hip_stream stream)
+{
+    hipGraph_t graph = nullptr;
+    hipError_t code = hipStreamEndCapture(as_stream(stream), &graph);
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipGetLastError();
+    return code == hipSuccess ? ST_OK : ST_BACKEND;
+}
+
+int yvex_hip_capture_end(yvex_hip_stream stream, yvex_hip_graph *out, uint64_t *kernel_nodes)
+{
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t count = 0;
+    if (!out) return ST_INVALID_ARG;
+    *out = nullptr;
+    if (kernel_nodes) *kernel_nodes = 0;
+    int rc = wrap("hipStreamEndCapture", hipStreamEndCapture(as_stream(stream), &graph));
+    if (rc || !graph) return rc ? rc : ST_BACKEND;
+    // Only kernel nodes are replayed: a memset or copy node would mean a launch wrapper did
+    // something a replay cannot be trusted to repeat.
+    rc = wrap("hipGraphGetNodes", hipGraphGetNodes(graph, nullptr, &count));
+    if (!rc && count) {
+        std::vector<hipGraphNode_t> nodes(count);
+        rc = wrap("hipGraphGetNodes", hipGraphGetNodes(graph, nodes.data(), &count));
+        for (size_t i = 0; !rc && i < count; ++i) {
+            hipGraphNodeType type;
+            rc = wrap("hipGraphNodeGetType", hipGraphNodeGetType(nodes[i], &type));
+            if (!rc && type != hipGraphNodeTypeKernel) {
+                set_last_error_text("launch graph holds a node that is not a kernel");
+                rc = ST_UNSUPPORTED;
+            }
+        }
+    }
+    if (!rc && !count) {
+        set_last_error_text("launch graph is empty");
+        rc = ST_UNSUPPORTED;
+    }
+    if (!rc) rc = wrap("hipGraphInstantiate", hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    (void)hipGraphDestroy(graph);
+    if (rc) return rc;
+    if (kernel_nodes) *kernel_nodes = count;
+    *out = reinterpret_cast<yvex_hip_graph>(exec);
+    return ST_OK;
+}
+
+int yvex_hip_graph_launch(yvex_hip_graph graph, yvex_hip_stream stream)
+{
+    if (!graph) return ST_INVALID_ARG;
+    return wrap("hipGraphLaunch",
+                hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph), as_stream(stream)));
+}
+
+int yvex_hip_graph_destroy(yvex_hip_graph graph)
+{
+    return graph ? wrap("hipGraphExecDestroy", hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph)))
+                 : ST_OK;
 }
 
 }  // extern "C"

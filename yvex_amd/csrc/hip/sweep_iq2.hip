@@ -679,21 +679,6 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     }
 }
 
-static int sweep_grid()
-{
-    static int units = 0;
-    if (!units) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
-            (void)hipGetLastError();
-            return 256;
-        }
-        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
-    return units;
-}
-
 bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs)
 {
     if (pairs > kClassMaxSweeps) return false;            // every sweep serves at least one pair
@@ -708,14 +693,8 @@ bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long p
 template <bool FUSED>
 static int launch_iq2_sweep_variant(const GroupedArgs &a, hipStream_t stream)
 {
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void *)iq2_sweep_kernel<FUSED>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSweepLdsBytes) != hipSuccess)
-            (void)hipGetLastError();
-        configured = true;
-    }
-    iq2_sweep_kernel<FUSED><<<sweep_grid(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
+    YVEX_ALLOW_DYNAMIC_LDS(iq2_sweep_kernel<FUSED>, kSweepLdsBytes);
+    iq2_sweep_kernel<FUSED><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
     return check_launch("moe_sweep_iq2");
 }
 

@@ -156,6 +156,7 @@ int yvex_backend_close_checked(yvex_backend **backend_ref, yvex_error *err)
                                 "resource discharge failed (test seam)");
     }
     if (!backend->host_only) {
+        if (yvex_hip_stream_sync(backend->stream) == 0) yvex_rocm_moe_graphs_release(backend);
         if (yvex_hip_stream_sync(backend->stream) != 0 || yvex_hip_free(backend->device_status) != 0 ||
             yvex_hip_stream_destroy(backend->stream) != 0) {
             backend->status = YVEX_BACKEND_STATUS_FAILED;

@@ -7,6 +7,7 @@
  */
 #include <limits.h>
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 #include <time.h>
 
@@ -268,6 +269,128 @@ static int same_expert_shape(const yvex_hip_expert_weights *a, const yvex_hip_ex
            a->intermediate == b->intermediate;
 }
 
+/* ---- launch graphs -------------------------------------------------------------------------
+ * The launch sequence of a row batch depends only on facts the host knows before the first
+ * kernel: the layer's geometry and policies, the weight views, the row count, and the device
+ * addresses of rows, outputs, weights and workspace. The reference keys a captured graph on the
+ * same topology (src/backend/cuda/moe.c:1545-1643) and replays it unless the job asks for eager
+ * execution (moe.c:1650-1681). Here a key seen for the first time runs eagerly, the second time
+ * it is captured and launched, and from then on it is replayed; sixteen keys are kept, the least
+ * recently used one making room. Everything a kernel argument is computed from is in the key,
+ * so a replay submits exactly the launches the eager sequence would. */
+enum { GRAPH_SLOTS = 16, GRAPH_KEY_WORDS = 176 };
+
+typedef struct {
+    unsigned long long words[GRAPH_KEY_WORDS];
+    unsigned int count;
+    int overflow;
+} graph_key;
+
+typedef struct {
+    graph_key key;
+    yvex_hip_graph graph;              /* NULL: seen once, ran eagerly */
+    unsigned long long launches, last_use;
+    int used;
+} graph_slot;
+
+struct yvex_rocm_moe_graphs {
+    graph_slot slots[GRAPH_SLOTS];
+    unsigned long long clock;
+    int refused;                       /* a capture failed: this backend stays eager */
+};
+
+static void key_word(graph_key *key, unsigned long long value)
+{
+    if (key->count < GRAPH_KEY_WORDS) key->words[key->count++] = value;
+    else key->overflow = 1;
+}
+
+static void key_real(graph_key *key, double value)
+{
+    unsigned long long bits = 0ull;
+    memcpy(&bits, &value, sizeof(bits));
+    key_word(key, bits);
+}
+
+static void key_layer(graph_key *key, const yvex_moe_layer_plan *layer)
+{
+    key_word(key, (unsigned long long)layer->router_class);
+    key_word(key, (unsigned long long)layer->scoring);
+    key_word(key, (unsigned long long)layer->topk_policy);
+    key_word(key, (unsigned long long)layer->activation);
+    key_word(key, layer->hidden_width);
+    key_word(key, layer->residual_streams);
+    key_word(key, layer->expanded_width);
+    key_word(key, layer->mhc_mixing_rows);
+    key_word(key, layer->mhc_sinkhorn_iterations);
+    key_word(key, layer->routed_experts);
+    key_word(key, layer->shared_experts);
+    key_word(key, layer->experts_per_token);
+    key_word(key, layer->expert_intermediate_width);
+    key_word(key, layer->shared_intermediate_width);
+    key_word(key, layer->hash_table_rows);
+    key_word(key, layer->hash_table_columns);
+    key_word(key, layer->correction_bias_width);
+    key_real(key, layer->rms_epsilon);
+    key_real(key, layer->mhc_epsilon);
+    key_real(key, layer->mhc_post_multiplier);
+    key_real(key, layer->routed_scaling_factor);
+    key_real(key, layer->activation_limit);
+    key_word(key, (unsigned long long)layer->requires_token_ids);
+    key_word(key, (unsigned long long)layer->requires_correction_bias);
+    key_word(key, (unsigned long long)layer->normalize_topk_probabilities);
+}
+
+static void key_view(graph_key *key, const yvex_moe_weight_view *view, unsigned long long address)
+{
+    key_word(key, view->qtype);
+    key_word(key, (unsigned long long)view->layout);
+    key_word(key, (unsigned long long)view->activation);
+    key_word(key, view->encoded_bytes);
+    key_word(key, view->row_bytes);
+    key_word(key, view->row_width);
+    key_word(key, view->row_count);
+    key_word(key, address);
+}
+
+static graph_slot *graph_find(struct yvex_rocm_moe_graphs *cache, const graph_key *key)
+{
+    unsigned int i;
+    for (i = 0u; i < GRAPH_SLOTS; ++i)
+        if (cache->slots[i].used && cache->slots[i].key.count == key->count &&
+            !memcmp(cache->slots[i].key.words, key->words, key->count * sizeof(key->words[0])))
+            return &cache->slots[i];
+    return NULL;
+}
+
+static graph_slot *graph_admit(struct yvex_rocm_moe_graphs *cache, const graph_key *key)
+{
+    unsigned int i, oldest = 0u;
+    for (i = 0u; i < GRAPH_SLOTS; ++i) {
+        if (!cache->slots[i].used) { oldest = i; break; }
+        if (cache->slots[i].last_use < cache->slots[oldest].last_use) oldest = i;
+    }
+    if (cache->slots[oldest].used && cache->slots[oldest].graph)
+        (void)yvex_hip_graph_destroy(cache->slots[oldest].graph);
+    memset(&cache->slots[oldest], 0, sizeof(cache->slots[oldest]));
+    cache->slots[oldest].key = *key;
+    cache->slots[oldest].used = 1;
+    return &cache->slots[oldest];
+}
+
+/* Graphs name device addresses: whoever frees or re-attaches what they point into drops them.
+ * The caller has synchronised the stream (or nothing was ever launched). */
+void yvex_rocm_moe_graphs_release(yvex_backend *backend)
+{
+    unsigned int i;
+    if (!backend || !backend->moe_graphs) return;
+    for (i = 0u; i < GRAPH_SLOTS; ++i)
+        if (backend->moe_graphs->slots[i].used && backend->moe_graphs->slots[i].graph)
+            (void)yvex_hip_graph_destroy(backend->moe_graphs->slots[i].graph);
+    free(backend->moe_graphs);
+    backend->moe_graphs = NULL;
+}
+
 static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job,
                             const yvex_moe_row_batch *rows, const yvex_moe_row_batch_output *output,
                             yvex_moe_row_batch_result *result, yvex_error *err)
@@ -286,6 +409,8 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     int envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
+    enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
+    graph_slot *graph_target = NULL;
     if (result) memset(result, 0, sizeof(*result));
     unsupported_width = job && rows && job->worklist_policy &&
                         (rows->row_count >= 64ull ||
@@ -447,9 +572,54 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     status = backend->device_status;
     stream = backend->stream;
 #define AT(field) ((void *)(uintptr_t)(base + ranges.field))
+    /* token ids come from the caller's host buffer on every call, so they travel ahead of the
+     * kernels and never inside a graph */
+    if (hash_router && yvex_hip_memcpy_h2d(AT(tokens), rows->token_ids, row_count * sizeof(unsigned int),
+                                           stream) != 0)
+        return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.token-ids", yvex_hip_last_error());
+    if (!job->eager_execution && !(backend->moe_graphs && backend->moe_graphs->refused)) {
+        graph_key key;
+        unsigned long long slot_address[YVEX_MOE_WEIGHT_COUNT] = {0};
+        int k;
+        slot_address[YVEX_MOE_WEIGHT_FFN_NORM] = envelope_addresses[3];
+        slot_address[YVEX_MOE_WEIGHT_MHC_FUNCTION] = envelope_addresses[0];
+        slot_address[YVEX_MOE_WEIGHT_MHC_BASE] = envelope_addresses[2];
+        slot_address[YVEX_MOE_WEIGHT_MHC_SCALE] = envelope_addresses[1];
+        slot_address[YVEX_MOE_WEIGHT_ROUTER] = router_address;
+        slot_address[YVEX_MOE_WEIGHT_ROUTER_TABLE] = table_address;
+        slot_address[YVEX_MOE_WEIGHT_ROUTER_BIAS] = bias_address;
+        for (k = 0; k < 6; ++k) slot_address[YVEX_MOE_WEIGHT_ROUTED_GATE + k] = addresses[k];
+        key.count = 0u;
+        key.overflow = 0;
+        key_word(&key, row_count);
+        key_word(&key, (unsigned long long)(uintptr_t)status);
+        key_word(&key, (unsigned long long)(uintptr_t)stream);
+        key_word(&key, base);
+        key_word(&key, backend->workspace_bytes);
+        key_word(&key, backend->resident_generation);
+        key_word(&key, (unsigned long long)(uintptr_t)rows->device_rows->data);
+        key_word(&key, (unsigned long long)(uintptr_t)rows->device_outputs->data);
+        key_layer(&key, layer);
+        for (k = 0; k < YVEX_MOE_WEIGHT_COUNT; ++k) key_view(&key, &views[k], slot_address[k]);
+        if (!backend->moe_graphs) backend->moe_graphs = calloc(1u, sizeof(*backend->moe_graphs));
+        if (backend->moe_graphs && !key.overflow) {
+            graph_slot *slot = graph_find(backend->moe_graphs, &key);
+            if (!slot) slot = graph_admit(backend->moe_graphs, &key);   /* first sight: eager */
+            else graph_mode = slot->graph ? GRAPH_REPLAY : GRAPH_CAPTURE;
+            slot->last_use = ++backend->moe_graphs->clock;
+            graph_target = slot;
+        }
+    }
+sequence:
+    rc = YVEX_OK;
+    launches = 0ull;
+    if (graph_mode == GRAPH_CAPTURE && yvex_hip_capture_begin(stream) != 0) {
+        backend->moe_graphs->refused = 1;
+        graph_mode = GRAPH_EAGER;
+    }
 #define LAUNCH(call, where)                                             \
     do {                                                                \
-        if (rc == YVEX_OK) {                                            \
+        if (rc == YVEX_OK && graph_mode != GRAPH_REPLAY) {              \
             rc = yvex_rocm_launch_result((call), (where), err);         \
             if (rc == YVEX_OK) launches++;                              \
         }                                                               \
@@ -497,9 +667,6 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                            activations, 0, row_count, hidden, NULL, (float *)AT(logits),
                            experts, 0, (int *)status, stream), "rocm.moe.rows.router");
     if (hash_router) {
-        if (rc == YVEX_OK && yvex_hip_memcpy_h2d(AT(tokens), rows->token_ids, row_count * sizeof(unsigned int),
-                                                 stream) != 0)
-            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.token-ids", yvex_hip_last_error());
         LAUNCH(yvex_hip_moe_route_hash_rows((const float *)AT(logits), (const uint8_t *)(uintptr_t)table_address,
                                             (const uint32_t *)AT(tokens), row_count, experts, topk,
                                             layer->hash_table_rows,
@@ -622,9 +789,32 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
                                    (const float *)AT(post), (const float *)AT(combination), row_count,
                                    streams, hidden, (float *)rows->device_outputs->data, (int *)status,
                                    stream), "rocm.moe.rows.mhc-egress");
+    if (graph_mode == GRAPH_CAPTURE) {
+        /* a recording that fails, or holds anything but kernels, is dropped for good and the
+         * batch runs eagerly: the stream has executed nothing yet */
+        uint64_t nodes = 0u;
+        if (rc != YVEX_OK) (void)yvex_hip_capture_abort(stream);
+        if (rc != YVEX_OK || yvex_hip_capture_end(stream, &graph_target->graph, &nodes) != 0 ||
+            nodes != launches) {
+            if (graph_target->graph) (void)yvex_hip_graph_destroy(graph_target->graph);
+            graph_target->graph = NULL;
+            backend->moe_graphs->refused = 1;
+            graph_mode = GRAPH_EAGER;
+            goto sequence;
+        }
+        graph_target->launches = launches;
+    }
+    if (graph_mode != GRAPH_EAGER) {
+        launches = graph_target->launches;
+        rc = yvex_rocm_launch_result(yvex_hip_graph_launch(graph_target->graph, stream),
+                                     "rocm.moe.rows.graph", err);
+    }
     if (rc != YVEX_OK) return rc;
 
     defer = job->device_completion && job->device_completion->defer;
+    result->graph_launches = graph_mode != GRAPH_EAGER;
+    result->graph_captures = graph_mode == GRAPH_CAPTURE;
+    result->graph_replays = graph_mode == GRAPH_REPLAY;
     result->schema_version = YVEX_MOE_ROW_BATCH_RESULT_SCHEMA_V4;
     result->execution_class = YVEX_EXECUTION_CLASS_DEVICE_NATIVE;
     result->row_count = row_count;

@@ -31,7 +31,12 @@ struct yvex_backend {
     /* device status word shared by the operations of this backend */
     int *device_status;
     int pending_completion;
+    /* launch graphs of the row-batch MoE operation, keyed on topology and device addresses */
+    struct yvex_rocm_moe_graphs *moe_graphs;
 };
+
+/* Drop every cached launch graph (the stream is idle or was never used). */
+void yvex_rocm_moe_graphs_release(yvex_backend *backend);
 
 int yvex_rocm_refuse(yvex_error *err, yvex_status code, const char *where, const char *message);
 int yvex_rocm_seam(const char *name);
