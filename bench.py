@@ -52,6 +52,33 @@ def event_ms(torch, fn, repeats: int) -> float:
     return start.elapsed_time(stop) / repeats
 
 
+def device_clock(torch, dev):
+    """Clock of the matrix cores under full load, from a launch of known length in cycles
+    (every SIMD runs a chain of dependent 32-cycle matrix instructions), next to the clock the
+    device properties name. Fractions of the matrix-core peak are quoted against the published
+    peak, which assumes the peak engine clock (2.4 GHz): the measured clock says how much of a
+    gap is frequency."""
+    import ctypes as C
+    from yvex_amd import load_library
+    lib = load_library()
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    chain = 100_000
+
+    def once():
+        lib.yvex_hip_clock_probe(C.c_uint64(chain), C.c_void_p(sink.data_ptr()), stream)
+    once()
+    torch.cuda.synchronize()
+    ms = event_ms(torch, once, 3)
+    engine, memory = C.c_int(0), C.c_int(0)
+    lib.yvex_hip_device_clocks(0, C.byref(engine), C.byref(memory))
+    return {"matrix_load_ghz": round(chain * 32 / (ms * 1e6), 3),
+            "device_peak_engine_mhz": round(engine.value / 1e3, 1),
+            "device_peak_memory_mhz": round(memory.value / 1e3, 1),
+            "probe": f"{chain} dependent V_MFMA_I32_32X32X32_I8 per SIMD on every compute unit, "
+                     f"32 cycles each, {round(ms, 3)} ms"}
+
+
 def cpu_baseline(sample_rows: int, threads: int):
     """Time the CPU oracle (reference algorithm: decode to float, double accumulate) on
     `sample_rows` rows of the same layer shape; weights for the experts those rows hit only."""
@@ -128,6 +155,98 @@ def cpu_baseline_reference(sample_rows: int):
             "sample": f"{sample_rows} rows x (top-8 + shared) expert FFNs of the same layer shape through "
                       f"yvex_moe_expert_cpu of the reference, compiled from its own sources",
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
+
+
+class AbiLayer:
+    """The benchmark layer behind include/yvex_rocm.h: a backend of its own, weight views that
+    carry device addresses, backend-owned row tensors and an attached workspace. `step()` is one
+    yvex_backend_moe_operations_get()->execute_rows with deferred completion, `complete()` the
+    phase barrier complete_rows (the reference completes all pending layers of a phase with one
+    call, src/runtime/moe.c:1567-1576)."""
+
+    def __init__(self, torch, routed, shared, router, x_host, rows):
+        import ctypes as C
+        import numpy as np
+        from yvex_amd import abi
+        from yvex_amd.host import Backend
+        self.C, self.abi, self.np, self.rows = C, abi, np, rows
+        self.b = Backend()
+        if not self.b.ok:
+            raise RuntimeError(f"backend open failed: {self.b.err.message.decode()}")
+        self.keep = (routed, shared, router)
+        plan = self.plan = abi.LayerPlan()
+        plan.schema_version, plan.router_class, plan.scoring = 1, abi.ROUTER_LEARNED, abi.SCORING_SIGMOID
+        plan.hidden_width = plan.expanded_width = HIDDEN
+        plan.residual_streams = 1
+        plan.routed_experts, plan.shared_experts, plan.experts_per_token = EXPERTS, 1, TOPK
+        plan.expert_intermediate_width = plan.shared_intermediate_width = INTERMEDIATE
+        plan.routed_scaling_factor, plan.activation_limit = 1.0, 10.0
+        plan.requires_correction_bias, plan.normalize_topk_probabilities = 0, 1
+        job = self.job = abi.LayerJob()
+        job.layer = C.pointer(plan)
+        rb_h, rb_i = HIDDEN // 256 * 66, INTERMEDIATE // 256 * 66
+
+        def view(slot, tensor, qtype, width, count, row_bytes, activation):
+            v = job.weights[slot]
+            v.qtype, v.layout, v.activation = qtype, abi.LAYOUT_EXPERT_MAJOR, activation
+            v.kernel_family = abi.FAMILY_GFX950
+            v.device_address = tensor.data_ptr()
+            v.encoded_bytes = v.storage_bytes = tensor.numel() * tensor.element_size()
+            v.row_bytes, v.row_width, v.row_count = row_bytes, width, count
+
+        enc = abi.ACT_DEVICE_ENCODED
+        view(abi.W_ROUTER, router, 0, HIDDEN, EXPERTS, HIDDEN * 4, abi.ACT_DEVICE_F32)
+        view(abi.W_ROUTED_GATE, routed[0], 16, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
+        view(abi.W_ROUTED_UP, routed[1], 16, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
+        view(abi.W_ROUTED_DOWN, routed[2], 16, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc)
+        view(abi.W_SHARED_GATE, shared[0], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
+        view(abi.W_SHARED_UP, shared[1], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
+        view(abi.W_SHARED_DOWN, shared[2], 16, INTERMEDIATE, HIDDEN, rb_i, enc)
+        self.ops = self.b.lib.yvex_backend_moe_operations_get(self.b.handle).contents
+        need, err = abi.ULL(), abi.Error()
+        if self.ops.workspace_required(C.byref(plan), rows, C.byref(need), C.byref(err)) != 0:
+            raise RuntimeError(err.message.decode())
+        self.b.workspace(need.value)
+        self.rows_in, self.rows_out = self.b.f32(x_host), self.b.empty_f32(rows * HIDDEN)
+        batch = self.batch = abi.RowBatch()
+        batch.schema_version, batch.row_count, batch.row_width, batch.row_stride = 1, rows, HIDDEN, HIDDEN
+        batch.device_rows, batch.device_outputs = self.rows_in, self.rows_out
+        batch.provenance, batch.execution_class = abi.BATCH_MULTI_SESSION, 1
+        self.out = abi.RowBatchOutput()
+        self.result, self.done, self.err = abi.RowBatchResult(), abi.RowBatchResult(), abi.Error()
+        self.deferred = abi.DeviceCompletion(1, None)
+
+    def step(self, defer=True, eager=False):
+        C = self.C
+        self.job.eager_execution = int(eager)
+        self.job.device_completion = C.pointer(self.deferred) if defer else None
+        rc = self.ops.execute_rows(self.b.handle, C.byref(self.job), C.byref(self.batch), C.byref(self.out),
+                                   C.byref(self.result), C.byref(self.err))
+        if rc != 0:
+            raise RuntimeError(f"execute_rows: {self.err.message.decode()}")
+
+    def complete(self):
+        C = self.C
+        if self.ops.complete_rows(self.b.handle, 0, C.byref(self.done), C.byref(self.err)) != 0:
+            raise RuntimeError(f"complete_rows: {self.err.message.decode()}")
+
+    def timed(self, steps, warmup, *, defer=True, eager=False):
+        """Wall-clock ms per step of `steps` execute_rows calls, the backend idle before the
+        first and after the last (complete_rows is the closing synchronisation)."""
+        for _ in range(warmup):
+            self.step(defer, eager)
+        self.complete()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.step(defer, eager)
+        self.complete()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def output(self):
+        return self.b.read_f32(self.rows_out, self.rows * HIDDEN).reshape(self.rows, HIDDEN)
+
+    def close(self):
+        self.b.close()
 
 
 def dense_leg(torch, K, dev, repeats: int):
@@ -249,14 +368,14 @@ def dense_leg(torch, K, dev, repeats: int):
 
 
 def tile_classes(populations):
-    """128-pair tiles of the row-batch kernels by the number of 16-pair blocks they run with."""
-    out = {"1": 0, "2": 0, "4": 0, "8": 0}
+    """Token tiles of the row-batch kernels: full 64-pair tiles, and the partial tile a bucket
+    ends with, by whether it runs with two 32-token blocks or one."""
+    out = {"64": 0, "33-63": 0, "1-32": 0}
     for n in populations:
-        full, rest = divmod(int(n), 128)
-        out["8"] += full
+        full, rest = divmod(int(n), 64)
+        out["64"] += full
         if rest:
-            blocks = (rest + 15) // 16
-            out["1" if blocks <= 1 else "2" if blocks <= 2 else "4" if blocks <= 4 else "8"] += 1
+            out["33-63" if rest > 32 else "1-32"] += 1
     return out
 
 
@@ -270,8 +389,14 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     rank = torch.randperm(EXPERTS, device=dev, generator=gen).float() + 1.0
     popularity = rank.pow(-1.1)
     uniform = torch.rand((rows, EXPERTS), device=dev, generator=gen).clamp_(1e-9, 1.0 - 1e-9)
-    logits = popularity.log()[None, :] - (-uniform.log()).log()
+    wanted = popularity.log()[None, :] - (-uniform.log()).log()
     x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
+    # router weights whose projection of x gives those logits: the minimum-norm solution of
+    # x . router^T = wanted (2048 equations per expert, 7168 unknowns), solved in double
+    xd = x.double()
+    router = (xd.T @ torch.linalg.solve(xd @ xd.T, wanted.double())).T.float().contiguous()
+    logits = K.matvec(router.view(torch.uint8).reshape(-1), K.F32, EXPERTS, HIDDEN, x,
+                      status=K.new_status(dev))
     qt = K.IQ2_XXS
     layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                      qtypes=(qt, qt, qt), routed=weights, shared=shared, bias=None,
@@ -291,6 +416,18 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     down_ms = event_ms(torch, lambda: K.moe_down_rows(
         layer.routed, layer.intermediate_q8, layer.worklist, pairs, EXPERTS, layer.pair_outputs,
         layer.status), steps)
+    # the same step through include/yvex_rocm.h (router projection included)
+    stage_rows = layer.run(x, logits).clone()
+    torch.cuda.synchronize()
+    abi_layer = AbiLayer(torch, weights, shared, router, x.cpu().numpy(), rows)
+    abi_layer.step(defer=False)
+    abi_same = bool((torch.from_numpy(abi_layer.output()) == stage_rows.cpu()).all().item())
+    abi_unique = int(abi_layer.result.unique_experts)
+    abi_eager_ms = abi_layer.timed(steps, warmup, eager=True)
+    abi_graph_ms = abi_layer.timed(steps, max(warmup, 2))
+    abi_layer.close()
+    harness_ms = step_ms
+    step_ms = min(abi_graph_ms, abi_eager_ms)
     pair_ops = 2 * (2 * INTERMEDIATE * HIDDEN + HIDDEN * INTERMEDIATE)
     routed_ops, shared_ops = pair_ops * pairs, pair_ops * rows
     up_ops = 2 * 2 * INTERMEDIATE * HIDDEN * pairs
@@ -298,6 +435,11 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     return {
         "workload": "moe_prefill_iq2xxs: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, Q8_K activations",
         "ms_per_step": round(step_ms, 4), "tokens_per_s": round(rows / (step_ms * 1e-3), 1),
+        "c_abi": {"entry": "yvex_backend_moe_operations_get()->execute_rows + complete_rows",
+                  "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
+                  "rows_identical_to_stage_harness": abi_same,
+                  "distinct_routed_experts": abi_unique},
+        "stage_harness_ms_per_step": round(harness_ms, 4),
         "int8_TOPs": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12, 2),
         "mfma_peak_frac": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
         "distinct_routed_experts": int(populations.numel()),
@@ -308,6 +450,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
                      "unit": "TOP/s", "frac": round(up_ops / (up_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
                      "launch_ms": round(up_ms, 4)},
         "kernels_ms": {"gate_up_rows": round(up_ms, 4), "down_rows": round(down_ms, 4)},
+        "clock_after": device_clock(torch, dev),
     }
 
 
@@ -352,7 +495,10 @@ def main() -> int:
     gen = torch.Generator(device=dev)
     gen.manual_seed(42)
     x = torch.randn((ROWS, HIDDEN), device=dev, generator=gen)
-    logits = torch.randn((ROWS, EXPERTS), device=dev, generator=gen)
+    # router weights (F32, as the model stores them): logits = router . row, unit variance
+    router = torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5
+    logits = K.matvec(router.view(torch.uint8).reshape(-1), K.F32, EXPERTS, HIDDEN, x,
+                      status=K.new_status(dev))
     layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                      qtypes=(qt, qt, qt), routed=(gate, up, down), shared=shared, bias=None,
                      scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
@@ -420,6 +566,31 @@ def main() -> int:
                   file=sys.stderr)
     except Exception as error:       # capture refused: the eager figure stands
         print(f"decode step: graph capture unavailable ({error})", file=sys.stderr)
+    harness_ms, harness_mode = step_ms, launch_mode
+    # The step a caller of include/yvex_rocm.h gets: execute_rows on the backend's own stream
+    # (router projection included), completion deferred to one complete_rows per phase. Its
+    # launch graph is built by the library. This is the headline; the stage harness above only
+    # serves the per-kernel timings.
+    stage_rows = layer.run(x, logits).clone()
+    torch.cuda.synchronize()
+    abi_layer = AbiLayer(torch, (gate, up, down), shared, router, x.cpu().numpy(), ROWS)
+    abi_layer.step(defer=False)
+    abi_unique = int(abi_layer.result.unique_experts)
+    abi_same = bool((torch.from_numpy(abi_layer.output()) == stage_rows.cpu()).all().item())
+    abi_eager_ms = abi_layer.timed(args.steps, args.warmup, eager=True)
+    abi_graph_ms = abi_layer.timed(args.steps, max(args.warmup, 2))
+    graph_facts = (int(abi_layer.result.graph_launches), int(abi_layer.result.graph_replays))
+    abi_sync_ms = abi_layer.timed(args.steps, args.warmup, defer=False)
+    abi_launches = int(abi_layer.result.kernel_launches)
+    abi_layer.close()
+    if abi_unique != unique or not abi_same:
+        print(f"decode step: execute_rows and the stage harness disagree (distinct experts {abi_unique} "
+              f"vs {unique}, identical rows {abi_same})", file=sys.stderr)
+        return 1
+    step_ms = min(abi_graph_ms, abi_eager_ms)
+    launch_mode = ("execute_rows, library launch graph, completion deferred to the phase barrier"
+                   if abi_graph_ms <= abi_eager_ms else
+                   "execute_rows, eager launches, completion deferred to the phase barrier")
     weight_bytes = (unique + 1) * EXPERT_BYTES
     value = weight_bytes / (step_ms * 1e-3) / 1e9
 
@@ -475,8 +646,17 @@ def main() -> int:
                    "max_bucket_population": max_pop, "routed_sweeps": sweeps, "weight_bytes_per_step": weight_bytes},
         "hbm_peak_frac": round(value / HBM_PEAK_GBS, 4),
         "tokens_per_s": round(ROWS / (step_ms * 1e-3), 1),
-        "launch": launch_mode, "eager_ms_per_step": round(eager_ms, 4),
-        "graph_ms_per_step": round(graph_ms, 4) if graph_ms else None,
+        "launch": launch_mode,
+        "c_abi": {"entry": "yvex_backend_moe_operations_get()->execute_rows + complete_rows",
+                  "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
+                  "completed_every_step_ms": round(abi_sync_ms, 4), "kernel_launches": abi_launches,
+                  "graph_launches_replays_last_step": graph_facts,
+                  "rows_identical_to_stage_harness": abi_same},
+        "stage_harness": {"launch": harness_mode, "ms_per_step": round(harness_ms, 4),
+                          "eager_ms_per_step": round(eager_ms, 4),
+                          "graph_ms_per_step": round(graph_ms, 4) if graph_ms else None,
+                          "note": "the same launches from Python with given logits (no router "
+                                  "projection); used for the per-kernel timings only"},
         "roofline": {"bound": "hbm", "kernel": "iq2_sweep_kernel<fused gate/up> (routed + shared)",
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
@@ -490,6 +670,7 @@ def main() -> int:
                        "gate_up_sweep_alone": round(up_alone_ms, 4) if up_alone_ms else None,
                        "down_sweep_alone": round(down_alone_ms, 4) if down_alone_ms else None},
     }
+    out["clock"] = device_clock(torch, dev)
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)

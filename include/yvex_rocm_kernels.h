@@ -241,6 +241,13 @@ int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,
  * Time it with events; `sink` is a 4-byte device word that is practically never written. */
 int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_hip_stream stream);
 
+/* Clock probe, the companion of the bandwidth probe: every SIMD of the device runs `chain`
+ * dependent 32x32x32 int8 matrix instructions (32 shader cycles each), so the launch lasts
+ * chain * 32 cycles; timed with events it gives the clock under matrix-core load, the figure a
+ * fraction of the matrix-core peak has to be read with. `sink` is a device word that is
+ * practically never written. */
+int yvex_hip_clock_probe(uint64_t chain, int *sink, yvex_hip_stream stream);
+
 /* Device-side fill, usable where a captured graph must not hold a memset node. */
 int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream stream);
 
@@ -249,6 +256,8 @@ int yvex_hip_device_count(void);
 int yvex_hip_device_info(int device, char *name, unsigned long name_cap, char *arch,
                          unsigned long arch_cap, uint64_t *total_bytes, uint64_t *free_bytes,
                          int *compute_units);
+/* Peak engine and memory clocks the device reports, in kHz. */
+int yvex_hip_device_clocks(int device, int *engine_khz, int *memory_khz);
 int yvex_hip_malloc(void **out, uint64_t bytes);
 int yvex_hip_free(void *ptr);
 int yvex_hip_host_alloc(void **out, uint64_t bytes);

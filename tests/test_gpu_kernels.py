@@ -77,6 +77,37 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     assert_close(got, want)
 
 
+@pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32)])
+def test_matvec_f32_weights_over_a_row_batch(gpu, oracle, rows, width, inputs):
+    """F32 weight rows against 32 or more F32 input rows (a router or mixing projection over a
+    prefill batch) run on the fp32 matrix cores; ragged edges, the additive operand and the bf16
+    output behave as in the lane-strided kernel (kernels.cu:560-640)."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(42, f"matvec.f32.batch.{rows}.{width}.{inputs}")
+    w = g.weights(oracle.F32, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    got = K.matvec(dev(w, gpu), oracle.F32, rows, width, dev(x, gpu), status=status).cpu().numpy()
+    status_ok(status)
+    want = oracle.matvec(oracle.F32, w, rows, width, x)
+    assert_close(got, want)
+    # against the double-precision product too: a transposed or mis-split operand cannot pass
+    exact = x.astype(np.float64) @ w.view(np.float32).reshape(rows, width).astype(np.float64).T
+    assert np.allclose(got, exact, rtol=1e-4, atol=1e-4)
+    add = g.normal(inputs * rows).reshape(inputs, rows)
+    got = K.matvec(dev(w, gpu), oracle.F32, rows, width, dev(x, gpu), additive=dev(add, gpu),
+                   output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((got.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(got - (want + add)) <= np.abs(want + add) * 2.0 ** -8 + 1e-4)
+    # a non-finite weight is reported, as by the other kernels
+    if rows > 1:
+        poisoned = w.copy()
+        poisoned.view(np.float32)[width + 5] = np.inf
+        K.matvec(dev(poisoned, gpu), oracle.F32, rows, width, dev(x, gpu), status=status)
+        assert int(status.item()) == 1
+
+
 @pytest.mark.parametrize("qtype,rows,width,inputs", [
     ("IQ2_XXS", 67, 2048, 1), ("IQ2_XXS", 9, 7168, 6), ("Q4_K", 33, 7168, 1),
     ("Q4_K", 12, 2048, 16), ("Q8_0", 40, 4096, 2), ("Q2_K", 21, 768, 3)])

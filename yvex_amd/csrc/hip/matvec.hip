@@ -163,6 +163,101 @@ __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsign
     }
 }
 
+__device__ __noinline__ float f32_dot_f64(const float *w, const float *x, unsigned long long width)
+{
+    double exact = 0.0;
+    for (unsigned long long k = 0; k < width; ++k) exact += (double)w[k] * (double)x[k];
+    return (float)exact;
+}
+
+// F32 weight rows against a batch of F32 input rows (a router or mixing projection over a
+// prefill-width batch): a workgroup owns 32 weight rows x 32 input rows on the fp32 matrix cores.
+// Its four waves split the row width into quarters; lane (r, h) of a wave loads four consecutive
+// floats of weight row r and of input row r at offset 8j + 4h, which feed four
+// V_MFMA_F32_32X32X2_F32 (any assignment of k to instructions is valid as long as both operands
+// use the same one). The partial tiles are added in wave order, so the sum is deterministic.
+// Products are exact fp32 products; only the order of the fp32 additions differs from the
+// lane-strided kernel above.
+__global__ __launch_bounds__(256) void matvec_f32_tile_kernel(MatvecArgs a)
+{
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    __shared__ float partial[3][16][64];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned r = lane & 31u, h = lane >> 5;
+    unsigned long long wrow = (unsigned long long)blockIdx.x * 32ull + r;
+    unsigned long long in = (unsigned long long)blockIdx.y * 32ull + r;
+    if (wrow >= a.row_count) wrow = a.row_count - 1ull;      // a ragged edge repeats the last row
+    if (in >= a.input_rows) in = a.input_rows - 1ull;
+    const float *wp = (const float *)(a.encoded + wrow * a.row_bytes);
+    const float *xp = (const float *)a.input + in * a.input_stride;
+    const unsigned long long quarter = a.row_width / 4ull;   // a multiple of 8
+    const unsigned long long begin = wave * quarter + 4u * h;
+    v16f acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    unsigned bad = 0u;
+    const unsigned steps = (unsigned)(quarter / 8ull);
+    wp += begin;
+    xp += begin;
+    // four steps of loads stay in flight ahead of the matrix instructions that use them
+    const unsigned groups = (steps + 3u) / 4u;
+    float4 w[4], x[4];
+#pragma unroll
+    for (unsigned j = 0; j < 4u; ++j) {
+        const unsigned at = 8u * (j < steps ? j : steps - 1u);
+        w[j] = *reinterpret_cast<const float4 *>(wp + at);
+        x[j] = *reinterpret_cast<const float4 *>(xp + at);
+    }
+    for (unsigned group = 0; group < groups; ++group) {
+        float4 wn[4], xn[4];
+        if (group + 1u < groups) {
+#pragma unroll
+            for (unsigned j = 0; j < 4u; ++j) {
+                const unsigned step = 4u * (group + 1u) + j;
+                const unsigned at = 8u * (step < steps ? step : steps - 1u);
+                wn[j] = *reinterpret_cast<const float4 *>(wp + at);
+                xn[j] = *reinterpret_cast<const float4 *>(xp + at);
+            }
+        }
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            if (4u * group + j >= steps) break;
+            bad |= (unsigned)!finite_f32(w[j].x) | (unsigned)!finite_f32(w[j].y) |
+                   (unsigned)!finite_f32(w[j].z) | (unsigned)!finite_f32(w[j].w);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].x, x[j].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].y, x[j].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].z, x[j].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].w, x[j].w, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            w[j] = wn[j];
+            x[j] = xn[j];
+        }
+    }
+    if (bad) raise_status(a.status, 1);
+    if (wave) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) partial[wave - 1u][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wave) return;
+    const unsigned long long out_in = (unsigned long long)blockIdx.y * 32ull + r;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        // accumulator i of lane (r, h): weight row 8 (i / 4) + 4 h + i % 4, input row r
+        const unsigned long long row = (unsigned long long)blockIdx.x * 32ull + 8u * (i >> 2) + 4u * h + (i & 3);
+        float sum = ((acc[i] + partial[0][i][lane]) + partial[1][i][lane]) + partial[2][i][lane];
+        if (row >= a.row_count || out_in >= a.input_rows) continue;
+        if (!finite_f32(sum) && *a.status == 0) {
+            // kernels.cu:616-620: an overflow before opposite terms cancelled is redone in double
+            sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
+                              (const float *)a.input + out_in * a.input_stride, a.row_width);
+        }
+        matvec_publish(a, out_in, row, sum);
+    }
+}
+
 // int32 block sums of the Q8_K path, produced by the same unit code the matvec runs.
 template <unsigned QT>
 __global__ __launch_bounds__(256) void block_dots_kernel(
@@ -295,6 +390,13 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (!input_q8) {
         if (input_stride < row_width) return ST_INVALID_ARG;
         if (!scalar && (((uintptr_t)input & 15u) || (input_stride & 3u))) return ST_INVALID_ARG;
+    }
+    if (qtype == QT_F32 && input_rows >= 32ull && row_width % 32ull == 0ull &&
+        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
+        const unsigned long long grid_x = (row_count + 31ull) / 32ull, grid_y = (input_rows + 31ull) / 32ull;
+        if (grid_x > 0x7fffffffull || grid_y > 65535ull) return ST_BOUNDS;
+        matvec_f32_tile_kernel<<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
+        return check_launch("matvec_f32_tile");
     }
     if (scalar) {
         const unsigned long long grid_x = (row_count + 3ull) / 4ull;

@@ -73,6 +73,20 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4 *__restric
     if (fold == 0x9e3779b9u) *sink = fold;   // practically never true; keeps the loads alive
 }
 
+// A chain of dependent 32x32x32 int8 matrix instructions, one wave per SIMD on every compute
+// unit: each takes 8 passes of 4 cycles and the next cannot start before it, so a launch lasts
+// chain * 32 shader cycles and its duration gives the clock the matrix cores run at under load.
+__global__ __launch_bounds__(256) void clock_probe_kernel(uint64_t chain, int *sink)
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    typedef int v16i __attribute__((ext_vector_type(16)));
+    v4i a = {(int)threadIdx.x, 1, 2, 3}, b = {3, 2, 1, (int)blockIdx.x};
+    v16i acc = {0};
+    for (uint64_t i = 0; i < chain; ++i)
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    if (acc[0] == 0x7fffffff && acc[5] == 0x7ffffffe) *sink = acc[3];   // practically never
+}
+
 __global__ void probe_kernel(int *out)
 {
     if (out) *out = 950;
@@ -113,6 +127,18 @@ int yvex_hip_device_info(int device, char *name, unsigned long name_cap, char *a
     if (rc) return rc;
     if (total_bytes) *total_bytes = total_b;
     if (free_bytes) *free_bytes = free_b;
+    return ST_OK;
+}
+
+int yvex_hip_device_clocks(int device, int *engine_khz, int *memory_khz)
+{
+    int engine = 0, memory = 0;
+    int rc = wrap("hipDeviceGetAttribute", hipDeviceGetAttribute(&engine, hipDeviceAttributeClockRate, device));
+    if (!rc) rc = wrap("hipDeviceGetAttribute",
+                       hipDeviceGetAttribute(&memory, hipDeviceAttributeMemoryClockRate, device));
+    if (rc) return rc;
+    if (engine_khz) *engine_khz = engine;
+    if (memory_khz) *memory_khz = memory;
     return ST_OK;
 }
 
@@ -193,6 +219,13 @@ int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_
     if (!data || !sink || bytes < 16u || ((uintptr_t)data & 15u)) return ST_INVALID_ARG;
     stream_read_kernel<<<256 * 16, 256, 0, as_stream(stream)>>>((const uint4 *)data, bytes / 16u, sink);
     return check_launch("stream_read");
+}
+
+int yvex_hip_clock_probe(uint64_t chain, int *sink, yvex_hip_stream stream)
+{
+    if (!chain || !sink) return ST_INVALID_ARG;
+    clock_probe_kernel<<<compute_units(), 256, 0, as_stream(stream)>>>(chain, sink);
+    return check_launch("clock_probe");
 }
 
 int yvex_hip_fill_u32(void *dst, uint32_t value, uint64_t count, yvex_hip_stream stream)
