@@ -405,13 +405,20 @@ def test_greedy_selection_flags_non_finite(gpu, oracle):
         assert int(tokens[row]) == want_tokens[row] and float(best[row]) == want_best[row]
         assert int(ties[row]) == want_ties[row]
     assert int(ties[1]) == 0
-    # a long row shared among workgroups: the status is raised and nothing is published
+    # long rows shared among workgroups: the status is raised and only the bad row stays silent
     values = np.ones((2, 30000), np.float32)
     values[1, 29999] = np.nan
     status = K.new_status(gpu)
     tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
     torch.cuda.synchronize()
-    assert int(status.item()) == 1 and int(ties[0]) == 0 and int(ties[1]) == 0
+    assert int(status.item()) == 1 and int(ties[1]) == 0
+    assert int(ties[0]) == 30000 and int(tokens[0]) == 0 and float(best[0]) == 1.0
+    # a status another operation left on the shared word does not silence clean rows
+    values[1, 29999] = 3.0
+    status.fill_(2)
+    tokens, best, ties = K.argmax_f32(dev(values, gpu), status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 2 and int(tokens[1]) == 29999 and int(ties[0]) == 30000
 
 
 def envelope_inputs(oracle, tokens, streams, width, name):

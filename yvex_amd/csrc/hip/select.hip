@@ -203,16 +203,21 @@ __global__ __launch_bounds__(kSpanThreads) void argmax_spans_kernel(
 
 __global__ __launch_bounds__(64) void argmax_merge_kernel(
     const SpanResult *partial, unsigned spans, unsigned long long row_count, unsigned *selected_tokens,
-    float *selected_values, unsigned long long *tie_counts, const int *status)
+    float *selected_values, unsigned long long *tie_counts)
 {
     const unsigned long long row = blockIdx.x;
-    if (row >= row_count || *status) return;      // a row with a bad value publishes nothing
+    if (row >= row_count) return;
     const unsigned lane = threadIdx.x;
     Candidate mine{-3.402823466e+38F, 0xffffffffu, 0ull};
+    bool bad = false;         // a span that met a non-finite value counts no element at all
     for (unsigned s = lane; s < spans; s += 64u) {
         const SpanResult r = partial[row * spans + s];
+        if (!r.ties) bad = true;
         candidate_merge(mine, Candidate{r.best, r.index, r.ties});
     }
+    // only the row that holds the bad value publishes nothing, as when one workgroup scans a row;
+    // a status left by other work on the stream does not silence the rows of this launch
+    if (__any(bad)) return;
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {
         Candidate other;
@@ -258,7 +263,7 @@ extern "C" int yvex_hip_argmax_f32(const float *values, uint64_t row_count, uint
         if (rc) return rc;
         argmax_merge_kernel<<<(unsigned)row_count, 64, 0, s>>>(
             (const SpanResult *)scratch, spans, row_count, selected_tokens, selected_values,
-            (unsigned long long *)tie_counts, status);
+            (unsigned long long *)tie_counts);
         return check_launch("argmax_f32.merge");
     }
     argmax_rows_kernel<<<(unsigned)row_count, kSelectThreads, 0, s>>>(
