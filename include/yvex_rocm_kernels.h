@@ -78,6 +78,19 @@ int yvex_hip_argmax_f32(const float *values, uint64_t row_count, uint64_t row_wi
                         uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts,
                         void *scratch, uint64_t scratch_bytes, int *status, yvex_hip_stream stream);
 
+/* yvex_hip_argmax_f32 for callers that cannot allocate device memory (code under graph capture,
+ * serving loops and harnesses that forbid it); it has no counterpart in the reference. The span
+ * results live in a static device array of yvex_hip_argmax_static_capacity() bytes (256 KiB:
+ * 16 384 span results, one per 8192 values of a row) that each device holds until the process
+ * ends, so the call allocates nothing; a batch needing more is refused with BOUNDS and an error
+ * text. Every call on a device shares that device's array: calls that overlap on one device
+ * (different streams or threads) race and must be ordered by the caller. Results are those of
+ * yvex_hip_argmax_f32 given a workspace. */
+uint64_t yvex_hip_argmax_static_capacity(void);
+int yvex_hip_argmax_f32_static(const float *values, uint64_t row_count, uint64_t row_width,
+                               uint32_t *selected_tokens, float *selected_values, uint64_t *tie_counts,
+                               int *status, yvex_hip_stream stream);
+
 /* Replaces yvex_qtype_gather / yvex_encoded_row_decode (kernels.cu:784-830): decode selected
  * rows to F32. row_ids may be NULL (rows 0..selected-1). */
 int yvex_hip_gather(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,

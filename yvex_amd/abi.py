@@ -280,7 +280,8 @@ EXPORTS = [
 ]
 KERNEL_EXPORTS = [
     "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_row_dot", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
-    "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes",
+    "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes", "yvex_hip_argmax_f32_static",
+    "yvex_hip_argmax_static_capacity",
     "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_moe_route_hash_rows", "yvex_hip_worklist_build", "yvex_hip_moe_prepare",
     "yvex_hip_moe_prepare_supported", "yvex_hip_moe_up", "yvex_hip_moe_down",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",

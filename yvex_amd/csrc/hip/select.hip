@@ -233,6 +233,41 @@ __global__ __launch_bounds__(64) void argmax_merge_kernel(
     }
 }
 
+// Span results for callers that cannot allocate: one array per device, held until the process
+// ends. 16 384 span results cover 64 rows of 262 144 values, or one row of 134 million.
+constexpr uint64_t kStaticSpanResults = 16384u;
+constexpr int kStaticDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kStaticSpanResults * sizeof(SpanResult)];
+static std::mutex static_scratch_lock;
+static void *static_scratch_of[kStaticDevices];      // device address of `scratch`, per device
+
+// The device address of this device's copy of the array, looked up once per device with that
+// device current. The array's name is only a host-side handle for this lookup.
+static int static_scratch_address(void **out)
+{
+    int device = -1;
+    hipError_t code = hipGetDevice(&device);
+    if (code != hipSuccess || device < 0 || device >= kStaticDevices) {
+        if (code != hipSuccess) set_last_error("argmax_f32_static: hipGetDevice", code);
+        else set_last_error_text("argmax_f32_static: device ordinal is outside the table");
+        (void)hipGetLastError();
+        return ST_BACKEND;
+    }
+    std::lock_guard<std::mutex> guard(static_scratch_lock);
+    if (!static_scratch_of[device]) {
+        void *address = nullptr;
+        code = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (code != hipSuccess || !address) {
+            set_last_error("argmax_f32_static: hipGetSymbolAddress", code);
+            (void)hipGetLastError();
+            return ST_BACKEND;
+        }
+        static_scratch_of[device] = address;
+    }
+    *out = static_scratch_of[device];
+    return ST_OK;
+}
+
 }  // namespace yvex
 
 using namespace yvex;
@@ -270,4 +305,31 @@ extern "C" int yvex_hip_argmax_f32(const float *values, uint64_t row_count, uint
         values, row_count, row_width, selected_tokens, selected_values,
         (unsigned long long *)tie_counts, status);
     return check_launch("argmax_f32");
+}
+
+extern "C" uint64_t yvex_hip_argmax_static_capacity(void) { return sizeof(scratch); }
+
+extern "C" int yvex_hip_argmax_f32_static(const float *values, uint64_t row_count, uint64_t row_width,
+                                          uint32_t *selected_tokens, float *selected_values,
+                                          uint64_t *tie_counts, int *status, yvex_hip_stream stream)
+{
+    if (!values || !row_count || !row_width || !selected_tokens || !selected_values || !tie_counts ||
+        !status)
+        return ST_INVALID_ARG;
+    if (row_count > 65535ull || row_width > 0xffffffffull) return ST_BOUNDS;
+    const uint64_t need = yvex_hip_argmax_scratch_bytes(row_count, row_width);
+    if (need > sizeof(scratch)) {
+        set_last_error_text("argmax_f32_static: rows x spans exceed the 16384 span results of the "
+                            "static scratch array; use yvex_hip_argmax_f32 with a workspace");
+        return ST_BOUNDS;
+    }
+    void *spans = nullptr;
+    if (need) {
+        const int rc = static_scratch_address(&spans);
+        if (rc) return rc;
+    }
+    // every span result the merge reads is written by the span launch before it: nothing in the
+    // array has to start at zero
+    return yvex_hip_argmax_f32(values, row_count, row_width, selected_tokens, selected_values,
+                               tie_counts, spans, need, status, stream);
 }
