@@ -458,6 +458,36 @@ typedef struct {
     char layer_identity[YVEX_SHA256_HEX_CAP];
 } yvex_moe_layer_plan;
 
+/* execution_batch.h:42-66: who the rows of a batch belong to. The reference seals the identity
+ * fields with SHA-256 (yvex_execution_batch_seal); that seal belongs to its runtime and is not
+ * re-derived here: this backend checks the fields execute_rows compares with the row batch
+ * (schema, row_count, provenance, phase; src/backend/cuda/moe.c:1845-1852). */
+#define YVEX_EXECUTION_BATCH_SCHEMA_V1 1u
+#define YVEX_EXPERT_WORKLIST_POLICY_SCHEMA_V1 1u
+typedef struct {
+    unsigned long long execution_generation, state_generation;
+    char identity[YVEX_SHA256_HEX_CAP];
+} yvex_execution_batch_source;
+typedef struct {
+    unsigned long long source_index, source_row, sequence_position;
+    unsigned long long candidate_ordinal, publication_ordinal;
+    int candidate_present;
+} yvex_execution_batch_row;
+typedef struct {
+    unsigned int schema_version;
+    yvex_execution_batch_provenance provenance;
+    unsigned int phase;
+    unsigned long long row_count, source_count, model_generation;
+    const yvex_execution_batch_source *sources;
+    const yvex_execution_batch_row *rows;
+    char runtime_model_identity[YVEX_SHA256_HEX_CAP];
+    char runtime_binding_identity[YVEX_SHA256_HEX_CAP];
+    char physical_variant_identity[YVEX_SHA256_HEX_CAP];
+    char execution_profile_identity[YVEX_SHA256_HEX_CAP];
+    char operation_identity[YVEX_SHA256_HEX_CAP];
+    char identity[YVEX_SHA256_HEX_CAP];
+} yvex_execution_batch;
+
 /* execution_batch.h:86-93 */
 typedef struct {
     unsigned int schema_version;
@@ -492,9 +522,8 @@ typedef struct {
     void *host;
 } yvex_moe_device_completion;
 
-/* moe.h:182-197. The plan-side identities the reference seals with SHA-256 (execution_batch,
- * compiled profile) belong to its runtime, not to this path: execution_batch stays an opaque
- * pointer whose presence must match worklist_policy's, as moe.c:1845 requires. */
+/* moe.h:182-197. execution_batch and worklist_policy come together or not at all; when present
+ * they are checked against the row batch as moe.c:1845-1852 does (their SHA-256 seals excepted). */
 typedef struct {
     const yvex_moe_layer_plan *layer;
     yvex_moe_weight_view weights[YVEX_MOE_WEIGHT_COUNT];
@@ -508,7 +537,7 @@ typedef struct {
     int evidence_level;
     int eager_execution;
     const yvex_moe_device_completion *device_completion;
-    const void *execution_batch;
+    const yvex_execution_batch *execution_batch;
     const yvex_expert_worklist_policy *worklist_policy;
 } yvex_moe_layer_job;
 

@@ -264,13 +264,16 @@ class MoeCase:
 
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
-                 shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0):
+                 shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
+                 down_qtype=None):
         self.b, self.oracle = b, oracle
         self.streams, self.iterations = streams, iterations
         expanded = hidden * max(streams, 1)
         mixing = (streams + 2) * streams
         qt = getattr(oracle, qtype)
         self.qt, self.rows, self.hidden, self.experts, self.topk = qt, rows, hidden, experts, topk
+        qt_down = getattr(oracle, down_qtype) if down_qtype else qt
+        self.qtypes = (qt, qt, qt_down)
         self.intermediate, self.scoring = intermediate, scoring
         g = oracle.Generator(seed, f"backend.moe.{qtype}.{hidden}.{experts}")
         parts = {
@@ -278,10 +281,10 @@ class MoeCase:
             "bias": (g.normal(experts) * 0.05).astype(np.float32).view(np.uint8),
             "gate": g.weights(qt, experts * intermediate, hidden),
             "up": g.weights(qt, experts * intermediate, hidden),
-            "down": g.weights(qt, experts * hidden, intermediate),
+            "down": g.weights(qt_down, experts * hidden, intermediate),
             "sgate": g.weights(qt, intermediate, hidden),
             "sup": g.weights(qt, intermediate, hidden),
-            "sdown": g.weights(qt, hidden, intermediate),
+            "sdown": g.weights(qt_down, hidden, intermediate),
         }
         self.hash_vocab = hash_vocab
         if hash_vocab:  # hash router: an I32 table of expert ordinals per token id
@@ -325,7 +328,7 @@ class MoeCase:
             p.router_class, p.hash_table_rows, p.hash_table_columns = abi.ROUTER_HASH, hash_vocab, topk
         self.job = abi.LayerJob()
         self.job.layer = C.pointer(self.plan)
-        rb_h, rb_i = oracle.row_bytes(qt, hidden), oracle.row_bytes(qt, intermediate)
+        rb_h, rb_i = oracle.row_bytes(qt, hidden), oracle.row_bytes(qt_down, intermediate)
 
         def view(slot, name, q, width, count, row_bytes, activation=act):
             v = self.job.weights[slot]
@@ -338,10 +341,10 @@ class MoeCase:
         view(abi.W_ROUTER_BIAS, "bias", 0, experts, 1, experts * 4, abi.ACT_DEVICE_F32)
         view(abi.W_ROUTED_GATE, "gate", qt, hidden, experts * intermediate, rb_h)
         view(abi.W_ROUTED_UP, "up", qt, hidden, experts * intermediate, rb_h)
-        view(abi.W_ROUTED_DOWN, "down", qt, intermediate, experts * hidden, rb_i)
+        view(abi.W_ROUTED_DOWN, "down", qt_down, intermediate, experts * hidden, rb_i)
         view(abi.W_SHARED_GATE, "sgate", qt, hidden, intermediate, rb_h)
         view(abi.W_SHARED_UP, "sup", qt, hidden, intermediate, rb_h)
-        view(abi.W_SHARED_DOWN, "sdown", qt, intermediate, hidden, rb_i)
+        view(abi.W_SHARED_DOWN, "sdown", qt_down, intermediate, hidden, rb_i)
         if hash_vocab:
             view(abi.W_ROUTER_TABLE, "table", 26, topk, hash_vocab, topk * 4, abi.ACT_DEVICE_F32)
         if streams:
@@ -396,7 +399,7 @@ class MoeCase:
         bias = p["bias"].view(np.float32) if self.plan.requires_correction_bias else None
         shared = (p["sgate"], p["sup"], p["sdown"]) if self.plan.shared_experts else None
         want = o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
-                           topk=self.topk, qtypes=(self.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
+                           topk=self.topk, qtypes=self.qtypes, routed=(p["gate"], p["up"], p["down"]),
                            shared=shared, inputs=x, logits=logits, bias=bias, scoring=self.scoring,
                            normalize=True, scaling=1.5, act_q8=act_q8, threads=8,
                            hash_selected=self.table[self.tokens] if self.hash_vocab else None)
@@ -531,13 +534,47 @@ def test_execute_rows_refusals(backend, oracle):
     policy.schema_version, policy.supported_width_mask = 1, (1 << 1) | (1 << 4)
     policy.narrow_kernel_family = abi.FAMILY_GFX950
     case.job.worklist_policy = C.pointer(policy)
-    case.job.execution_batch = C.cast(C.pointer(policy), C.c_void_p)
+    batch = abi.ExecutionBatch()
+    batch.schema_version, batch.row_count = 1, case.rows
+    batch.provenance, batch.phase = case.batch.provenance, case.batch.phase
+    case.job.execution_batch = C.pointer(batch)
     sentinel = np.full(case.rows * case.hidden, 7.0, np.float32)
     b.lib.yvex_backend_tensor_write(b.handle, case.rows_out, sentinel.ctypes.data, sentinel.nbytes, None)
     assert case.execute() == abi.UNSUPPORTED
     assert np.array_equal(b.read_f32(case.rows_out, sentinel.size), sentinel)
     policy.supported_width_mask |= 1 << case.rows
     assert case.execute() == 0, case.err.message
+    # src/backend/cuda/moe.c:1845-1852: the batch must describe the rows it comes with
+    for field, wrong in (("row_count", case.rows + 1), ("provenance", abi.BATCH_PREFILL), ("phase", 1),
+                         ("schema_version", 2)):
+        keep = getattr(batch, field)
+        setattr(batch, field, wrong)
+        assert case.execute() == abi.INVALID_ARG, field
+        setattr(batch, field, keep)
+    # src/graph/worklist.c:252-272: width 1 admitted, width 0 and bit 63 not, families consistent
+    good = policy.supported_width_mask
+    for mask in (good & ~2, good | 1, good | (1 << 63)):
+        policy.supported_width_mask = mask
+        assert case.execute() == abi.INVALID_ARG, hex(mask)
+    policy.supported_width_mask = good
+    policy.narrow_kernel_family = b""
+    assert case.execute() == abi.INVALID_ARG
+    policy.narrow_kernel_family = abi.FAMILY_GFX950
+    policy.tensor_core_minimum = 4                      # a minimum needs a family of its own
+    assert case.execute() == abi.INVALID_ARG
+    policy.tensor_core_kernel_family = abi.FAMILY_GFX950
+    assert case.execute() == abi.INVALID_ARG            # ... that differs from the narrow one
+    policy.tensor_core_kernel_family = b"gfx950-int8-matrix-expert-rows"
+    assert case.execute() == 0, case.err.message
+    policy.tensor_core_minimum = 3                      # ... and must be an admitted width
+    assert case.execute() == abi.INVALID_ARG
+    policy.tensor_core_minimum, policy.tensor_core_kernel_family = 0, b""
+    # a profile identity names a compiled batch: without batch and policy it is refused
+    case.job.execution_batch, case.job.worklist_policy = None, None
+    case.batch.execution_profile_identity = b"0" * 64
+    assert case.execute() == abi.INVALID_ARG
+    case.batch.execution_profile_identity = None
+    case.job.execution_batch, case.job.worklist_policy = C.pointer(batch), C.pointer(policy)
     # execution batch and worklist policy must come together
     case.job.execution_batch = None
     assert case.execute() == abi.INVALID_ARG
@@ -764,7 +801,7 @@ def token_oracle(case, row):
     assert rc == 0
     logits = o.matvec(o.F32, p["router"], case.experts, case.hidden, x)
     want = o.moe_layer(hidden=case.hidden, intermediate=case.intermediate, experts=case.experts,
-                       topk=case.topk, qtypes=(case.qt,) * 3, routed=(p["gate"], p["up"], p["down"]),
+                       topk=case.topk, qtypes=case.qtypes, routed=(p["gate"], p["up"], p["down"]),
                        shared=(p["sgate"], p["sup"], p["sdown"]), inputs=x, logits=logits,
                        bias=p["bias"].view(np.float32), scoring=case.scoring, normalize=True, scaling=1.5,
                        act_q8=False, threads=1)
@@ -825,6 +862,50 @@ def test_token_local_host_publication(backend, oracle, qtype, outside):
     # a finished execution takes no more experts and does not finish twice
     assert t.add(views, 0.0, True) == abi.INVALID_ARG and t.finish() == abi.INVALID_ARG
     assert t.close() == 0 and not t.handle.value and t.close() == 0
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+def test_token_local_stages_mixed_qtypes(backend, oracle, workspace):
+    """The reference's own mix of an IQ2_XXS gate/up with a Q2_K down (src/runtime/moe.c:647-720
+    with views outside the arena, staged as src/backend/cuda/moe.c:205-245 does): the down matrix
+    of an expert is larger than its gate, and every projection has a staging range of its own
+    size. With a workspace attached the execution's block comes from it instead of an allocation."""
+    case = MoeCase(backend, oracle, qtype="IQ2_XXS", down_qtype="Q2_K", hidden=512, rows=2, streams=4,
+                   iterations=20, act=abi.ACT_DEVICE_F32)
+    gate, down = case.job.weights[abi.W_ROUTED_GATE], case.job.weights[abi.W_ROUTED_DOWN]
+    assert down.encoded_bytes > gate.encoded_bytes
+    if workspace:
+        backend.workspace(8 << 20)
+    t = TokenLocal(case, row=0)
+    assert t.begin() == 0, t.err.message
+    want = token_oracle(case, 0)
+    router, keep = t.result.router, []
+    weights = np.array(list(router.selected_weights)[:case.topk], np.float32)
+    for rank in range(case.topk):
+        views, held = t.expert_views(int(router.selected_experts[rank]), outside=True)
+        keep.append(held)
+        assert t.add(views, float(weights[rank]), False) == 0, t.err.message
+    views, held = t.expert_views(None, outside=True)
+    assert t.add(views, 0.0, True) == 0, t.err.message
+    assert t.finish() == 0, t.err.message
+    assert rows_close(t.routed, want["routed"][0], 4) and rows_close(t.shared, want["shared"][0])
+    assert rows_close(t.combined, want["combined"][0], 4)
+    assert t.result.upload_count == 3 * (case.topk + 1)
+    # a view larger than the range planned for its projection is refused, not spilled into the next
+    big = abi.WeightView()
+    C.memmove(C.byref(big), C.byref(views[0]), C.sizeof(big))
+    assert t.close() == 0
+    t2 = TokenLocal(case, row=1)
+    assert t2.begin() == 0, t2.err.message
+    wide = np.zeros(case.job.weights[abi.W_SHARED_GATE].encoded_bytes * 2, np.uint8)
+    big.encoded, big.row_count = wide.ctypes.data, views[0].row_count * 2
+    big.encoded_bytes = big.storage_bytes = wide.nbytes
+    up2 = abi.WeightView()
+    C.memmove(C.byref(up2), C.byref(big), C.sizeof(big))
+    down2 = abi.WeightView()
+    C.memmove(C.byref(down2), C.byref(views[2]), C.sizeof(down2))
+    assert t2.add([big, up2, down2], 0.0, True) in (abi.BOUNDS, abi.INVALID_ARG)
+    assert t2.close() == 0
 
 
 def test_token_local_device_output_runs_selected_experts(backend, oracle):

@@ -115,6 +115,15 @@ class WorklistPolicy(C.Structure):
                 ("tensor_core_kernel_family", C.c_char * 64), ("identity", C.c_char * HEX)]
 
 
+class ExecutionBatch(C.Structure):
+    _fields_ = [("schema_version", C.c_uint), ("provenance", C.c_int), ("phase", C.c_uint),
+                ("row_count", ULL), ("source_count", ULL), ("model_generation", ULL),
+                ("sources", C.c_void_p), ("rows", C.c_void_p)] + \
+               [(n, C.c_char * HEX) for n in ("runtime_model_identity", "runtime_binding_identity",
+                                              "physical_variant_identity", "execution_profile_identity",
+                                              "operation_identity", "identity")]
+
+
 class WorklistObservation(C.Structure):
     _fields_ = [("schema_version", C.c_uint), ("worklist_count", ULL), ("pair_count", ULL),
                 ("bucket_count", ULL), ("maximum_bucket_population", ULL),
@@ -142,7 +151,8 @@ class LayerJob(C.Structure):
                 ("device_output", C.c_void_p), ("token_id", C.c_uint), ("token_id_present", C.c_int),
                 ("cancel_requested", CANCEL_FN), ("cancel_context", C.c_void_p),
                 ("evidence_level", C.c_int), ("eager_execution", C.c_int),
-                ("device_completion", C.POINTER(DeviceCompletion)), ("execution_batch", C.c_void_p),
+                ("device_completion", C.POINTER(DeviceCompletion)),
+                ("execution_batch", C.POINTER(ExecutionBatch)),
                 ("worklist_policy", C.POINTER(WorklistPolicy))]
 
 

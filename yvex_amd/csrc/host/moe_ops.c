@@ -391,6 +391,27 @@ void yvex_rocm_moe_graphs_release(yvex_backend *backend)
     backend->moe_graphs = NULL;
 }
 
+/* The structural half of yvex_expert_worklist_policy_seal (src/graph/worklist.c:252-272): width 1
+ * admitted, width 0 and bit 63 not, a narrow family named, and a tensor-core minimum that is an
+ * admitted width below 63 with a family of its own. */
+static int worklist_policy_valid(const yvex_expert_worklist_policy *policy)
+{
+    int tensor_core;
+    if (!policy || policy->schema_version != YVEX_EXPERT_WORKLIST_POLICY_SCHEMA_V1 ||
+        !(policy->supported_width_mask & 2ull) || (policy->supported_width_mask & 1ull) ||
+        (policy->supported_width_mask >> 63u) || !policy->narrow_kernel_family[0])
+        return 0;
+    tensor_core = policy->tensor_core_minimum != 0ull;
+    if (tensor_core != (policy->tensor_core_kernel_family[0] != '\0')) return 0;
+    if (tensor_core &&
+        (policy->tensor_core_minimum >= 63ull ||
+         !(policy->supported_width_mask & (1ull << policy->tensor_core_minimum)) ||
+         !strncmp(policy->narrow_kernel_family, policy->tensor_core_kernel_family,
+                  sizeof(policy->narrow_kernel_family))))
+        return 0;
+    return 1;
+}
+
 static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job,
                             const yvex_moe_row_batch *rows, const yvex_moe_row_batch_output *output,
                             yvex_moe_row_batch_result *result, yvex_error *err)
@@ -412,15 +433,29 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
     graph_slot *graph_target = NULL;
     if (result) memset(result, 0, sizeof(*result));
+    /* src/backend/cuda/moe.c:1840-1852: batch and policy come together, are structurally valid,
+     * describe the same rows, and a profile identity needs both; a width outside the policy's
+     * mask is UNSUPPORTED, the rest INVALID_ARG */
     unsupported_width = job && rows && job->worklist_policy &&
-                        (rows->row_count >= 64ull ||
+                        (rows->row_count >= 63ull ||
                          !(job->worklist_policy->supported_width_mask & (1ull << rows->row_count)));
-    if (unsupported_width)
-        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
-                                "row count is outside the sealed supported width mask");
     if (!backend || !job || !layer || !rows || !output || !result ||
         backend->kind != YVEX_BACKEND_KIND_ROCM ||
         ((job->execution_batch == NULL) != (job->worklist_policy == NULL)) ||
+        (job->execution_batch &&
+         (job->execution_batch->schema_version != YVEX_EXECUTION_BATCH_SCHEMA_V1 ||
+          !worklist_policy_valid(job->worklist_policy) ||
+          job->execution_batch->row_count != rows->row_count ||
+          job->execution_batch->provenance != rows->provenance ||
+          job->execution_batch->phase != rows->phase)) ||
+        (rows->execution_profile_identity && (!job->execution_batch || !job->worklist_policy)) ||
+        unsupported_width)
+        return unsupported_width
+            ? yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.rows",
+                               "row count is outside the sealed supported width mask")
+            : yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.rows",
+                               "width-N MoE owners, execution batch or worklist policy are invalid");
+    if (
         rows->schema_version != YVEX_MOE_ROW_BATCH_SCHEMA_V1 || !rows->row_count ||
         rows->row_count > YVEX_ROCM_MOE_MAX_ROWS || rows->row_width != layer->expanded_width ||
         rows->row_stride != rows->row_width ||

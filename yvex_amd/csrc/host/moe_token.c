@@ -7,9 +7,11 @@
  * combines with the shared expert, rounds to bf16 and, when the job names a device output, runs
  * the egress onto the residual streams.
  *
- * The execution owns one device allocation for all of its ranges; weight views that lie outside
- * the attached resident arena are uploaded into a staging range (the reference does the same,
- * moe.c:205-245). Nothing here computes on tensor data.
+ * All ranges of an execution form one block of device memory: taken from the attached workspace
+ * when it has room (as the reference does, moe.c:565-566), else allocated for the execution.
+ * Weight views that lie outside the attached resident arena are uploaded into staging ranges of
+ * that block (moe.c:205-245), one per projection so that gate, up and down of an expert are on
+ * the device together. Nothing here computes on tensor data.
  */
 #include <limits.h>
 #include <math.h>
@@ -25,11 +27,13 @@ struct yvex_backend_moe_execution {
     yvex_backend *backend;
     const yvex_moe_layer_job *job;
     void *block;
+    int owns_block;                       /* allocated here rather than taken from the workspace */
     unsigned long long expanded, mixes, scale, base, norm, normalized, post, combination;
     unsigned long long logits, scores, bias, selected, weights, slot_weights, token;
     unsigned long long order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts;
     unsigned long long intermediate, pair_outputs, shared_output, routed, combined, staging;
     unsigned long long staging_bytes;
+    unsigned long long stage_offset[3], stage_capacity[3];   /* gate, up, down of one expert */
     unsigned long long routed_added;
     int shared_added, finished, grouped_selected;
     unsigned long long h2d, d2h, d2d, launches, uploads, downloads, direct_weights, subviews;
@@ -77,10 +81,25 @@ static int download(yvex_backend_moe_execution *x, void *dst, const void *src, u
 
 /* Device address of a weight view: resident, or uploaded into the staging range at `offset`
  * (src/backend/cuda/moe.c:226-245). */
+static int weight_address_in(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
+                             unsigned long long row_width, unsigned long long row_count,
+                             unsigned long long offset, unsigned long long capacity,
+                             unsigned long long *address, const char *where, yvex_error *err);
+
+/* A coefficient or router matrix staged alone: the whole staging range is its own. */
 static int weight_address(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
                           unsigned long long row_width, unsigned long long row_count,
                           unsigned long long offset, unsigned long long *address, const char *where,
                           yvex_error *err)
+{
+    return weight_address_in(x, view, row_width, row_count, offset,
+                             offset <= x->staging_bytes ? x->staging_bytes - offset : 0ull, address, where, err);
+}
+
+static int weight_address_in(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
+                             unsigned long long row_width, unsigned long long row_count,
+                             unsigned long long offset, unsigned long long capacity,
+                             unsigned long long *address, const char *where, yvex_error *err)
 {
     int resident = 0;
     int rc = yvex_rocm_moe_view_check(x->backend, view, row_width, row_count, address, &resident, err);
@@ -89,7 +108,7 @@ static int weight_address(yvex_backend_moe_execution *x, const yvex_moe_weight_v
         x->direct_weights++;
         return YVEX_OK;
     }
-    if (offset > x->staging_bytes || view->encoded_bytes > x->staging_bytes - offset)
+    if (offset > x->staging_bytes || capacity > x->staging_bytes - offset || view->encoded_bytes > capacity)
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, where,
                                 "selected MoE encoded weight exceeds its stable staging range");
     rc = upload(x, (unsigned char *)AT(staging) + offset, view->encoded, view->encoded_bytes, where, err);
@@ -122,7 +141,7 @@ static int plan_ranges(yvex_backend_moe_execution *x, const yvex_moe_layer_plan 
     unsigned long long cursor = 0ull, hidden = layer->hidden_width, streams = layer->residual_streams;
     unsigned long long experts = layer->routed_experts, topk = layer->experts_per_token;
     unsigned long long widest = layer->expert_intermediate_width * topk;
-    unsigned long long staging = 0ull, routed_subview;
+    unsigned long long staging = 0ull;
     unsigned int slot;
     if (layer->shared_intermediate_width > widest) widest = layer->shared_intermediate_width;
 #define TAKE(field, bytes) do { x->field = cursor; cursor = align_up(cursor + (bytes)); } while (0)
@@ -152,14 +171,19 @@ static int plan_ranges(yvex_backend_moe_execution *x, const yvex_moe_layer_plan 
     TAKE(shared_output, hidden * sizeof(float));
     TAKE(routed, hidden * sizeof(float));
     TAKE(combined, hidden * sizeof(float));
-    /* staging for views outside the arena: the three matrices of the largest expert, or the
-     * largest ingress / router coefficient matrix (moe.c:552-568 sizes one matrix; the sweeps
-     * here read gate and up together) */
-    routed_subview = x->job->weights[YVEX_MOE_WEIGHT_ROUTED_GATE].encoded_bytes / (experts ? experts : 1ull);
-    for (slot = YVEX_MOE_WEIGHT_SHARED_GATE; slot <= YVEX_MOE_WEIGHT_SHARED_DOWN; ++slot)
-        if (x->job->weights[slot].encoded_bytes > routed_subview)
-            routed_subview = x->job->weights[slot].encoded_bytes;
-    staging = 3ull * align_up(routed_subview);
+    /* staging for views outside the arena: gate, up and down of one expert side by side (the
+     * sweeps read gate and up together), each range as large as the largest expert matrix of its
+     * projection over the routed and the shared slots; or the largest ingress / router
+     * coefficient matrix, staged alone (moe.c:552-568 sizes one matrix at a time) */
+    for (slot = 0u; slot < 3u; ++slot) {
+        unsigned long long part = x->job->weights[YVEX_MOE_WEIGHT_ROUTED_GATE + slot].encoded_bytes /
+                                  (experts ? experts : 1ull);
+        if (x->job->weights[YVEX_MOE_WEIGHT_SHARED_GATE + slot].encoded_bytes > part)
+            part = x->job->weights[YVEX_MOE_WEIGHT_SHARED_GATE + slot].encoded_bytes;
+        x->stage_offset[slot] = staging;
+        x->stage_capacity[slot] = align_up(part);
+        staging += x->stage_capacity[slot];
+    }
     for (slot = 0u; slot <= YVEX_MOE_WEIGHT_ROUTER_BIAS; ++slot)
         if (x->job->weights[slot].encoded_bytes > staging && slot != YVEX_MOE_WEIGHT_ROUTER_TABLE)
             staging = x->job->weights[slot].encoded_bytes;
@@ -442,9 +466,20 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
         return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, "rocm.moe.begin", "MoE range extent overflowed");
     }
     total = x->staging + x->staging_bytes;
-    if (yvex_hip_malloc(&x->block, total) != 0) {
-        free(x);
-        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.begin", yvex_hip_last_error());
+    {
+        /* the attached workspace when it has room (no allocation on the token path), else a
+         * block of the execution's own */
+        unsigned long long base = 0ull;
+        yvex_rocm_workspace_reset(backend);
+        if (backend->workspace_device_tensor &&
+            yvex_backend_workspace_acquire(backend, total, ALIGN, &base)) {
+            x->block = (void *)(uintptr_t)base;
+        } else if (yvex_hip_malloc(&x->block, total) != 0) {
+            free(x);
+            return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.begin", yvex_hip_last_error());
+        } else {
+            x->owns_block = 1;
+        }
     }
     expanded_bytes = layer->expanded_width * sizeof(float);
     rc = launched(x, yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream), "rocm.moe.status", err);
@@ -483,7 +518,7 @@ int yvex_backend_moe_add_expert(yvex_backend_moe_execution *x, const yvex_moe_we
                                 float route_weight, int shared, yvex_error *err)
 {
     const yvex_moe_layer_plan *layer = x && x->job ? x->job->layer : NULL;
-    unsigned long long address[3] = {0}, width, third, started = now_ns();
+    unsigned long long address[3] = {0}, width, started = now_ns();
     yvex_hip_expert_weights w;
     yvex_hip_stream stream;
     float *target;
@@ -500,13 +535,14 @@ int yvex_backend_moe_add_expert(yvex_backend_moe_execution *x, const yvex_moe_we
                                 "MoE expert exceeds the ranges planned at begin");
     stream = x->backend->stream;
     status = x->backend->device_status;
-    third = x->staging_bytes / 3ull & ~(ALIGN - 1ull);
-    rc = weight_address(x, gate, layer->hidden_width, width, 0ull, &address[0], "rocm.moe.expert-gate", err);
+    rc = weight_address_in(x, gate, layer->hidden_width, width, x->stage_offset[0], x->stage_capacity[0],
+                           &address[0], "rocm.moe.expert-gate", err);
     if (rc == YVEX_OK)
-        rc = weight_address(x, up, layer->hidden_width, width, third, &address[1], "rocm.moe.expert-up", err);
+        rc = weight_address_in(x, up, layer->hidden_width, width, x->stage_offset[1], x->stage_capacity[1],
+                               &address[1], "rocm.moe.expert-up", err);
     if (rc == YVEX_OK)
-        rc = weight_address(x, down, width, layer->hidden_width, 2ull * third, &address[2],
-                            "rocm.moe.expert-down", err);
+        rc = weight_address_in(x, down, width, layer->hidden_width, x->stage_offset[2],
+                               x->stage_capacity[2], &address[2], "rocm.moe.expert-down", err);
     if (rc != YVEX_OK) return rc;
     fill_weights(&w, gate, up, down, address, layer->hidden_width, width);
     if (!shared) {
@@ -629,7 +665,7 @@ int yvex_backend_moe_close(yvex_backend_moe_execution **execution, yvex_error *e
         yvex_error_clear(err);
         return YVEX_OK;
     }
-    if ((*execution)->block) {
+    if ((*execution)->block && (*execution)->owns_block) {
         /* kernels of an abandoned execution may still be reading the block */
         (void)yvex_hip_stream_sync((*execution)->backend->stream);
         if (yvex_hip_free((*execution)->block) != 0)
