@@ -160,7 +160,7 @@ def cpu_baseline_reference(sample_rows: int):
 class AbiLayer:
     """The benchmark layer behind include/yvex_rocm.h: a backend of its own, weight views that
     carry device addresses, backend-owned row tensors and an attached workspace. `step()` is one
-    yvex_backend_moe_operations_get()->execute_rows with deferred completion, `complete()` the
+    yvex_rocm_backend_moe_operations_get()->execute_rows with deferred completion, `complete()` the
     phase barrier complete_rows (the reference completes all pending layers of a phase with one
     call, src/runtime/moe.c:1567-1576)."""
 
@@ -202,7 +202,7 @@ class AbiLayer:
         view(abi.W_SHARED_GATE, shared[0], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
         view(abi.W_SHARED_UP, shared[1], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
         view(abi.W_SHARED_DOWN, shared[2], 16, INTERMEDIATE, HIDDEN, rb_i, enc)
-        self.ops = self.b.lib.yvex_backend_moe_operations_get(self.b.handle).contents
+        self.ops = self.b.lib.yvex_rocm_backend_moe_operations_get(self.b.handle).contents
         need, err = abi.ULL(), abi.Error()
         if self.ops.workspace_required(C.byref(plan), rows, C.byref(need), C.byref(err)) != 0:
             raise RuntimeError(err.message.decode())
@@ -435,7 +435,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     return {
         "workload": "moe_prefill_iq2xxs: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, Q8_K activations",
         "ms_per_step": round(step_ms, 4), "tokens_per_s": round(rows / (step_ms * 1e-3), 1),
-        "c_abi": {"entry": "yvex_backend_moe_operations_get()->execute_rows + complete_rows",
+        "c_abi": {"entry": "yvex_rocm_backend_moe_operations_get()->execute_rows + complete_rows",
                   "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
                   "rows_identical_to_stage_harness": abi_same,
                   "distinct_routed_experts": abi_unique},
@@ -647,7 +647,7 @@ def main() -> int:
         "hbm_peak_frac": round(value / HBM_PEAK_GBS, 4),
         "tokens_per_s": round(ROWS / (step_ms * 1e-3), 1),
         "launch": launch_mode,
-        "c_abi": {"entry": "yvex_backend_moe_operations_get()->execute_rows + complete_rows",
+        "c_abi": {"entry": "yvex_rocm_backend_moe_operations_get()->execute_rows + complete_rows",
                   "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
                   "completed_every_step_ms": round(abi_sync_ms, 4), "kernel_launches": abi_launches,
                   "graph_launches_replays_last_step": graph_facts,

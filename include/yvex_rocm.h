@@ -16,6 +16,12 @@
 #ifndef YVEX_ROCM_H
 #define YVEX_ROCM_H
 
+/* The structures, enumerations and constants this header shares with the reference are declared
+ * below with the reference's names and layout (a test compares both, field by field). A
+ * translation unit of the reference itself, which already has them from <yvex/...>, defines
+ * YVEX_ROCM_REFERENCE_TYPES before including this header and gets only the library's own types
+ * and entry points (all named yvex_rocm_*). */
+
 #include <stddef.h>
 #include <stdint.h>
 
@@ -25,6 +31,7 @@ extern "C" {
 
 /* ---- status and error: include/yvex/core.h:13-48 ------------------------------------------ */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef enum {
     YVEX_OK = 0,
     YVEX_ERR = -1,
@@ -47,16 +54,18 @@ typedef struct {
     char where[YVEX_ERROR_WHERE_CAP];
     char message[YVEX_ERROR_MESSAGE_CAP];
 } yvex_error;
+#endif
 
-const char *yvex_status_name(yvex_status status);
-void yvex_error_clear(yvex_error *err);
-void yvex_error_set(yvex_error *err, yvex_status code, const char *where, const char *message);
-int yvex_error_is_set(const yvex_error *err);
-yvex_status yvex_error_code(const yvex_error *err);
+const char *yvex_rocm_status_name(yvex_status status);
+void yvex_rocm_error_clear(yvex_error *err);
+void yvex_rocm_error_set(yvex_error *err, yvex_status code, const char *where, const char *message);
+int yvex_rocm_error_is_set(const yvex_error *err);
+yvex_status yvex_rocm_error_code(const yvex_error *err);
 
 /* ---- qtype identity, geometry and fail-closed admission ----------------------------------- */
 /* include/yvex/qtype.h:19-63, src/gguf/qtype.c:15-104, src/gguf/quant_registry.c:50-117 */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 enum {
     YVEX_GGUF_QTYPE_F32 = 0, YVEX_GGUF_QTYPE_F16 = 1, YVEX_GGUF_QTYPE_Q8_0 = 8,
     YVEX_GGUF_QTYPE_Q2_K = 10, YVEX_GGUF_QTYPE_Q4_K = 12, YVEX_GGUF_QTYPE_Q8_K = 15,
@@ -71,23 +80,24 @@ typedef enum {
     YVEX_GGUF_QTYPE_IDENTITY_OUTSIDE_BASELINE = 3,
     YVEX_GGUF_QTYPE_IDENTITY_UNKNOWN = 4
 } yvex_gguf_qtype_identity_status;
+#endif
 
 typedef struct {
     unsigned int qtype;
     const char *name;
     yvex_gguf_qtype_identity_status identity;
     unsigned int block_size, bytes_per_block;
-} yvex_gguf_qtype_geometry;
+} yvex_rocm_qtype_geometry;
 
 /* Replaces yvex_gguf_qtype_geometry_find (src/gguf/qtype.c:119-124): NULL above ID 42. */
-const yvex_gguf_qtype_geometry *yvex_gguf_qtype_geometry_find(unsigned int qtype);
+const yvex_rocm_qtype_geometry *yvex_rocm_gguf_qtype_geometry_find(unsigned int qtype);
 
 typedef enum {
-    YVEX_QUANT_REFUSAL_NONE = 0,
-    YVEX_QUANT_REFUSAL_ENCODER_UNAVAILABLE,
-    YVEX_QUANT_REFUSAL_REMOVED_IDENTITY,
-    YVEX_QUANT_REFUSAL_OUTSIDE_PINNED_BASELINE
-} yvex_quant_refusal;
+    YVEX_ROCM_QUANT_REFUSAL_NONE = 0,
+    YVEX_ROCM_QUANT_REFUSAL_ENCODER_UNAVAILABLE,
+    YVEX_ROCM_QUANT_REFUSAL_REMOVED_IDENTITY,
+    YVEX_ROCM_QUANT_REFUSAL_OUTSIDE_PINNED_BASELINE
+} yvex_rocm_quant_refusal;
 
 /* One row per qtype ID, index == ID (src/gguf/quant_registry.c:50-103). device_compute is the
  * reference's dedicated_cuda_compute_available restated for this backend. Relative to the
@@ -98,15 +108,16 @@ typedef struct {
     int known, storage_admitted, reference_decoder_available;
     int dedicated_cpu_compute_available, device_compute_available;
     int extension_of_reference;
-    yvex_quant_refusal refusal;
-} yvex_quant_numeric_capability;
+    yvex_rocm_quant_refusal refusal;
+} yvex_rocm_numeric_capability;
 
 /* Replaces yvex_quant_numeric_capability_at (src/gguf/quant_registry.c:114-118). */
-const yvex_quant_numeric_capability *yvex_quant_numeric_capability_at(unsigned int qtype);
+const yvex_rocm_numeric_capability *yvex_rocm_quant_numeric_capability_at(unsigned int qtype);
 
 /* ---- backend object: include/yvex/backend.h:13-152 ----------------------------------------- */
 
-typedef struct yvex_backend yvex_backend;
+typedef struct yvex_rocm_backend yvex_rocm_backend;
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef struct yvex_device_tensor yvex_device_tensor;
 
 typedef enum {
@@ -169,7 +180,7 @@ typedef struct {
 
 /* include/yvex/internal/backend.h:256-269, same fields in the same order. */
 struct yvex_device_tensor {
-    yvex_backend *owner;
+    yvex_rocm_backend *owner;
     unsigned long long owner_id;
     char *name;
     yvex_dtype dtype;
@@ -222,6 +233,7 @@ typedef struct {
     yvex_dtype input_dtype, weight_dtype, output_dtype;
     int context_available, kernel_bundle_available, function_available;
 } yvex_backend_capability_result;
+#endif
 
 /* Replaces yvex_backend_open (src/backend/core.c:176-205) for kind ROCM; every other kind
  * answers UNSUPPORTED. Test seams, read from the environment like the reference's
@@ -231,30 +243,36 @@ typedef struct {
  *   YVEX_TEST_ROCM_BUNDLE_FAILURE=1  a GPU is present but its kernels are treated as absent
  *   YVEX_TEST_ROCM_LAUNCH_FAILURE=1 / _SYNC_FAILURE=1 / _CLEANUP_FAILURE=1
  *                                    the next launch / synchronise / release reports failure */
-int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, yvex_error *err);
+int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *options, yvex_error *err);
+/* For a library that wraps this backend in an object of its own (the reference's struct
+ * yvex_backend with this backend behind `impl`): tensors allocated from now on name `owner` in
+ * their `owner` field, and ownership checks compare against it, so the embedding library's own
+ * checks (src/backend/private.h:95-101) hold on them. No reference counterpart; bound once, before
+ * the first allocation. */
+int yvex_rocm_backend_bind_owner(yvex_rocm_backend *backend, const void *owner, yvex_error *err);
 /* include/yvex/backend.h:142-152: a cleanup failure keeps *backend non-NULL for a retry. */
-int yvex_backend_close_checked(yvex_backend **backend, yvex_error *err);
-yvex_backend_kind yvex_backend_kind_of(const yvex_backend *backend);
-yvex_backend_status yvex_backend_status_of(const yvex_backend *backend);
-int yvex_backend_get_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
+int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend, yvex_error *err);
+yvex_backend_kind yvex_rocm_backend_kind_of(const yvex_rocm_backend *backend);
+yvex_backend_status yvex_rocm_backend_status_of(const yvex_rocm_backend *backend);
+int yvex_rocm_backend_get_memory_stats(const yvex_rocm_backend *backend, yvex_backend_memory_stats *out,
                                   yvex_error *err);
-int yvex_backend_sync(yvex_backend *backend, yvex_error *err);
-int yvex_backend_query_capability(const yvex_backend *backend,
+int yvex_rocm_backend_sync(yvex_rocm_backend *backend, yvex_error *err);
+int yvex_rocm_backend_query_capability(const yvex_rocm_backend *backend,
                                   yvex_backend_operation_variant variant,
                                   yvex_backend_capability_result *out, yvex_error *err);
 
 /* include/yvex/backend.h:177-204 */
-int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+int yvex_rocm_backend_tensor_alloc(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc,
                               yvex_device_tensor **out, yvex_error *err);
-int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor,
+int yvex_rocm_backend_tensor_release(yvex_rocm_backend *backend, yvex_device_tensor **tensor,
                                 yvex_error *err);
-int yvex_backend_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, const void *src,
+int yvex_rocm_backend_tensor_write(yvex_rocm_backend *backend, yvex_device_tensor *tensor, const void *src,
                               unsigned long long len, yvex_error *err);
-int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *tensor, void *dst,
+int yvex_rocm_backend_tensor_read(yvex_rocm_backend *backend, const yvex_device_tensor *tensor, void *dst,
                              unsigned long long len, yvex_error *err);
-int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
+int yvex_rocm_backend_tensor_copy(yvex_rocm_backend *backend, yvex_device_tensor *dst,
                              const yvex_device_tensor *src, yvex_error *err);
-int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_tensor *tensor);
+int yvex_rocm_backend_tensor_owned_by(const yvex_rocm_backend *backend, const yvex_device_tensor *tensor);
 
 /* ---- resident weights: include/yvex/internal/backend.h:270-301, src/backend/residency.c ---- */
 /*
@@ -265,41 +283,43 @@ int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_
  * shadow become visible at the next attach or prefetch. resolve maps a borrowed pointer inside
  * the shadow to device_base + offset exactly as src/backend/residency.c:89-112 does.
  */
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef enum {
     YVEX_BACKEND_RESIDENT_INVALID = -1,
     YVEX_BACKEND_RESIDENT_MISS = 0,
     YVEX_BACKEND_RESIDENT_HIT = 1
 } yvex_backend_resident_result;
+#endif
 
-int yvex_backend_resident_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+int yvex_rocm_backend_resident_alloc(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc,
                                 yvex_device_tensor **out, unsigned char **host, yvex_error *err);
-int yvex_backend_resident_prefetch(yvex_backend *backend, yvex_device_tensor *tensor,
+int yvex_rocm_backend_resident_prefetch(yvex_rocm_backend *backend, yvex_device_tensor *tensor,
                                    unsigned long long *prefetched_bytes, yvex_error *err);
-int yvex_backend_resident_attach(yvex_backend *backend, const unsigned char *host_base,
+int yvex_rocm_backend_resident_attach(yvex_rocm_backend *backend, const unsigned char *host_base,
                                  unsigned long long bytes, const yvex_device_tensor *tensor,
                                  unsigned long long generation, yvex_error *err);
-int yvex_backend_resident_detach(yvex_backend *backend, yvex_error *err);
-int yvex_backend_resident_resolve(const yvex_backend *backend, const unsigned char *host,
+int yvex_rocm_backend_resident_detach(yvex_rocm_backend *backend, yvex_error *err);
+int yvex_rocm_backend_resident_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
                                   unsigned long long bytes, unsigned long long *device_address);
 
 /* include/yvex/internal/backend.h:350-354: bump-allocated device scratch, reset per operation. */
-int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *tensor,
+int yvex_rocm_backend_workspace_attach(yvex_rocm_backend *backend, const yvex_device_tensor *tensor,
                                   unsigned long long bytes, yvex_error *err);
-void yvex_backend_workspace_detach(yvex_backend *backend);
-int yvex_backend_workspace_acquire(yvex_backend *backend, unsigned long long bytes,
+void yvex_rocm_backend_workspace_detach(yvex_rocm_backend *backend);
+int yvex_rocm_backend_workspace_acquire(yvex_rocm_backend *backend, unsigned long long bytes,
                                    unsigned long long alignment,
                                    unsigned long long *device_address);
 
 /* ---- dense projection, output head, gather ------------------------------------------------- */
 
 /* include/yvex/internal/backend.h:325-331 (yvex_backend_cuda_operation_facts). */
-typedef struct yvex_backend_rocm_operation_facts {
+typedef struct yvex_rocm_operation_facts {
     unsigned long long h2d_bytes, d2h_bytes, d2d_bytes, kernel_launches, upload_count;
     unsigned long long download_count, stream_synchronizations, device_synchronizations;
     unsigned long long active_weight_bytes, state_bytes;
     unsigned long long activation_bytes, temporary_bytes, tensor_core_launches;
     int compulsory_memory_facts_available;
-} yvex_backend_rocm_operation_facts;
+} yvex_rocm_operation_facts;
 
 /* Replaces yvex_backend_cuda_encoded_matvec (include/yvex/internal/backend.h:332-337,
  * src/backend/cuda/qtype.c:220-405). output[in, row] = dot(encoded row, input row in)
@@ -311,23 +331,23 @@ typedef struct yvex_backend_rocm_operation_facts {
  * are split (the reference's speculation path, qtype.c:256-281, kernels.cu:736-782): row r is
  * input[r, 0..input_head_width) followed by input_tail[r, ...], every value rounded to bf16, the
  * Q8 activation policy is ignored, and the attached workspace must hold rows * width floats. */
-int yvex_backend_rocm_encoded_matvec(
-    yvex_backend *backend, const unsigned char *resident_encoded,
+int yvex_rocm_encoded_matvec(
+    yvex_rocm_backend *backend, const unsigned char *resident_encoded,
     unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
     unsigned long long row_width, unsigned long long row_bytes, unsigned long long input_rows,
     const yvex_device_tensor *input, const yvex_device_tensor *input_tail,
     unsigned long long input_head_width, const yvex_device_tensor *additive,
-    yvex_device_tensor *output, int activation_q8, yvex_backend_rocm_operation_facts *facts,
+    yvex_device_tensor *output, int activation_q8, yvex_rocm_operation_facts *facts,
     yvex_error *err);
 
 /* Replaces yvex_backend_cuda_encoded_gather (include/yvex/internal/backend.h:338-342,
  * src/backend/cuda/qtype.c:411-521): decode selected rows to F32. row_ids is a host array. */
-int yvex_backend_rocm_encoded_gather(
-    yvex_backend *backend, const unsigned char *resident_encoded,
+int yvex_rocm_encoded_gather(
+    yvex_rocm_backend *backend, const unsigned char *resident_encoded,
     unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
     unsigned long long row_width, unsigned long long row_bytes, const unsigned int *row_ids,
     unsigned long long selected_rows, yvex_device_tensor *output,
-    yvex_backend_rocm_operation_facts *facts, yvex_error *err);
+    yvex_rocm_operation_facts *facts, yvex_error *err);
 
 /* ---- greedy selection over logits rows ---------------------------------------------------- */
 
@@ -338,10 +358,10 @@ int yvex_backend_rocm_encoded_gather(
  * device results live in the attached workspace for the call. Refusals: geometry, ownership,
  * dtype, unwritten logits -> FORMAT; no workspace -> NOMEM; kernels absent -> UNSUPPORTED; a
  * non-finite logit, a token outside the row or a zero tie count -> FORMAT, outputs zeroed. */
-int yvex_backend_rocm_select_greedy_rows(
-    yvex_backend *backend, const yvex_device_tensor *logits, unsigned long long row_count,
+int yvex_rocm_select_greedy_rows(
+    yvex_rocm_backend *backend, const yvex_device_tensor *logits, unsigned long long row_count,
     unsigned long long row_width, unsigned int *selected_tokens, float *selected_values,
-    unsigned long long *tie_counts, yvex_backend_rocm_operation_facts *facts, yvex_error *err);
+    unsigned long long *tie_counts, yvex_rocm_operation_facts *facts, yvex_error *err);
 
 /* The qtype parity probe, yvex_cuda_quant_row_dot (src/backend/cuda/qtype.c:523-700): one encoded
  * row (host bytes) times one vector (host floats), computed on the device by one thread in double
@@ -350,12 +370,13 @@ int yvex_backend_rocm_select_greedy_rows(
  * qtype without device compute UNSUPPORTED, elements not a whole number of blocks or a byte count
  * that disagrees BOUNDS, kernels absent UNSUPPORTED. failure is accepted for call compatibility
  * and left untouched (the reference's record belongs to its quantization pipeline). */
-int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const unsigned char *encoded,
+int yvex_rocm_quant_row_dot(yvex_rocm_backend *backend, unsigned int qtype, const unsigned char *encoded,
                             size_t encoded_bytes, const float *vector, unsigned long long elements,
                             float *out, void *failure, yvex_error *err);
 
 /* ---- MoE row batch: include/yvex/internal/moe.h ------------------------------------------- */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 #define YVEX_SHA256_HEX_CAP 65u
 #define YVEX_MOE_MAX_SELECTED 16u
 #define YVEX_MOE_ROW_BATCH_SCHEMA_V1 1u
@@ -364,8 +385,10 @@ int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const uns
 /* Kernel families this backend admits in a weight view (moe.h:20-23 list the CUDA ones). */
 #define YVEX_MOE_KERNEL_PORTABLE_ENCODED_ROW "portable-encoded-row"
 #define YVEX_MOE_KERNEL_PORTABLE_EXPERT_ROW "portable-expert-row"
+#endif
 #define YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP "gfx950-int8-dot-expert-sweep"
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef enum {
     YVEX_MOE_ROUTER_HASH_TOKEN_ID = 0,
     YVEX_MOE_ROUTER_LEARNED_HIDDEN_STATE
@@ -644,6 +667,7 @@ typedef struct {
     char terminal_identity[YVEX_SHA256_HEX_CAP];
     char decision_identity[YVEX_SHA256_HEX_CAP];
 } yvex_physical_execution_decision;
+#endif
 
 /* moe.h:277-297. execute_rows follows src/backend/cuda/moe.c:1826-1923: with mixing rows in the
  * layer plan it runs the residual-stream ingress (mixing projection, gates, Sinkhorn matrix,
@@ -682,12 +706,12 @@ typedef struct {
      * (moe.c:923-928); unknown kernel family -> UNSUPPORTED (moe.c:961-969); workspace missing or
      * too small -> NOMEM; cancellation -> CANCELLED; non-finite numerics -> FORMAT.
      */
-    int (*execute_rows)(yvex_backend *backend, const yvex_moe_layer_job *job,
+    int (*execute_rows)(yvex_rocm_backend *backend, const yvex_moe_layer_job *job,
                         const yvex_moe_row_batch *batch, const yvex_moe_row_batch_output *output,
                         yvex_moe_row_batch_result *result, yvex_error *err);
-    int (*complete_rows)(yvex_backend *backend, int barrier_observed,
+    int (*complete_rows)(yvex_rocm_backend *backend, int barrier_observed,
                          yvex_moe_row_batch_result *result, yvex_error *err);
-} yvex_backend_moe_operations;
+} yvex_rocm_moe_operations;
 
 /* The two layout entries of the table above, callable without a backend (they touch no device):
  * replace yvex_cuda_moe_derived_layout_plan/build, src/backend/cuda/private.h:400-402. */
@@ -698,11 +722,17 @@ int yvex_rocm_moe_derived_layout_build(const yvex_physical_execution_decision *d
                                        unsigned long long canonical_bytes, unsigned char *derived,
                                        unsigned long long storage_bytes, yvex_error *err);
 
+/* The workspace_required entry of the table below, callable without a backend (it depends on
+ * the layer plan and the row count alone). */
+int yvex_rocm_moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned long long row_count,
+                                     unsigned long long *bytes, yvex_error *err);
+
 /* moe.h:295-296: NULL unless the backend is ROCM and its kernels are loadable. */
-const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend);
+const yvex_rocm_moe_operations *yvex_rocm_backend_moe_operations_get(const yvex_rocm_backend *backend);
 
 /* ---- GGUF tensor directory and resident loading: include/yvex/gguf.h:142-195 ------------------- */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 #define YVEX_GGUF_MAX_DIMS 4u
 
 /* include/yvex/gguf.h:142-154 */
@@ -716,27 +746,28 @@ typedef struct {
     unsigned long long relative_offset, absolute_offset, storage_bytes, absolute_end_offset;
     int range_addressable;
 } yvex_gguf_tensor_info;
+#endif
 
-typedef struct yvex_gguf yvex_gguf;
+typedef struct yvex_rocm_gguf yvex_rocm_gguf;
 
 /* Structural reader with the rules and refusal codes of the reference's yvex_gguf_open
  * (src/gguf/core.c:1163-1249, :52-79): version 3 only (UNSUPPORTED), bad magic / rank / dimension
  * / alignment / key grammar / duplicate names (FORMAT), truncation and extents beyond the file
  * (BOUNDS), qtypes without storage geometry (UNSUPPORTED). It takes a path where the reference
  * takes its artifact handle. Scalar and string metadata are kept; arrays are walked and dropped. */
-int yvex_gguf_open_path(yvex_gguf **out, const char *path, yvex_error *err);
-void yvex_gguf_close(yvex_gguf *gguf);
-unsigned long long yvex_gguf_metadata_count(const yvex_gguf *gguf);
-int yvex_gguf_metadata_u64(const yvex_gguf *gguf, const char *key, unsigned long long *out);
-int yvex_gguf_metadata_f64(const yvex_gguf *gguf, const char *key, double *out);
-int yvex_gguf_metadata_string(const yvex_gguf *gguf, const char *key, const char **text,
+int yvex_rocm_gguf_open_path(yvex_rocm_gguf **out, const char *path, yvex_error *err);
+void yvex_rocm_gguf_close(yvex_rocm_gguf *gguf);
+unsigned long long yvex_rocm_gguf_metadata_count(const yvex_rocm_gguf *gguf);
+int yvex_rocm_gguf_metadata_u64(const yvex_rocm_gguf *gguf, const char *key, unsigned long long *out);
+int yvex_rocm_gguf_metadata_f64(const yvex_rocm_gguf *gguf, const char *key, double *out);
+int yvex_rocm_gguf_metadata_string(const yvex_rocm_gguf *gguf, const char *key, const char **text,
                               unsigned long long *len);
-unsigned long long yvex_gguf_tensor_count(const yvex_gguf *gguf);
-const yvex_gguf_tensor_info *yvex_gguf_tensor_at(const yvex_gguf *gguf, unsigned long long index);
-const yvex_gguf_tensor_info *yvex_gguf_tensor_find(const yvex_gguf *gguf, const char *name);
-unsigned long long yvex_gguf_tensor_data_offset(const yvex_gguf *gguf);
-unsigned int yvex_gguf_alignment(const yvex_gguf *gguf);
-unsigned long long yvex_gguf_file_size(const yvex_gguf *gguf);
+unsigned long long yvex_rocm_gguf_tensor_count(const yvex_rocm_gguf *gguf);
+const yvex_gguf_tensor_info *yvex_rocm_gguf_tensor_at(const yvex_rocm_gguf *gguf, unsigned long long index);
+const yvex_gguf_tensor_info *yvex_rocm_gguf_tensor_find(const yvex_rocm_gguf *gguf, const char *name);
+unsigned long long yvex_rocm_gguf_tensor_data_offset(const yvex_rocm_gguf *gguf);
+unsigned int yvex_rocm_gguf_alignment(const yvex_rocm_gguf *gguf);
+unsigned long long yvex_rocm_gguf_file_size(const yvex_rocm_gguf *gguf);
 
 /* The reference's runtime maps an artifact's tensor-data section into the resident arena and
  * hands the backend borrowed pointers into it (src/runtime/residency.c, contract text
@@ -745,14 +776,15 @@ unsigned long long yvex_gguf_file_size(const yvex_gguf *gguf);
  * of a named tensor is then host_base + relative_offset with rows of dims[0] values; tensors of
  * rank 3 are expert-major (rows = dims[1] * dims[2]). The view's activation class and kernel
  * family are the caller's to set. */
-int yvex_backend_rocm_gguf_resident_load(yvex_backend *backend, const yvex_gguf *gguf,
+int yvex_rocm_gguf_resident_load(yvex_rocm_backend *backend, const yvex_rocm_gguf *gguf,
                                          unsigned long long generation, yvex_device_tensor **arena,
                                          unsigned char **host_base, yvex_error *err);
-int yvex_backend_rocm_gguf_weight_view(const yvex_gguf *gguf, const unsigned char *host_base,
+int yvex_rocm_gguf_weight_view(const yvex_rocm_gguf *gguf, const unsigned char *host_base,
                                        const char *name, yvex_moe_weight_view *view, yvex_error *err);
 
 /* ---- token-local MoE operation: include/yvex/internal/moe.h:161-166,198-214,308-319 ------------ */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 #define YVEX_RUNTIME_DESCRIPTOR_QTYPE_CAP 43u
 #define YVEX_ATTENTION_EVIDENCE_FULL 3      /* include/yvex/internal/graph.h:250-255 */
 
@@ -780,6 +812,7 @@ typedef struct {
     char routed_digest[YVEX_SHA256_HEX_CAP], shared_digest[YVEX_SHA256_HEX_CAP];
     char combined_digest[YVEX_SHA256_HEX_CAP], routing_digest[YVEX_SHA256_HEX_CAP];
 } yvex_moe_layer_result;
+#endif
 
 /* One row, experts handed over one at a time by a caller that loads them on demand
  * (src/backend/cuda/moe.c:516-842; the caller is src/runtime/moe.c:647-720).
@@ -798,35 +831,37 @@ typedef struct {
  *   output the egress writes it; host copies as moe.c:775-803 publishes them.
  * close: releases the execution (safe on NULL). A kernel status other than zero surfaces as
  * BACKEND, as moe.c:277-296 reports it. */
-typedef struct yvex_backend_moe_execution yvex_backend_moe_execution;
-int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backend,
+typedef struct yvex_rocm_moe_execution yvex_rocm_moe_execution;
+int yvex_rocm_backend_moe_begin(yvex_rocm_moe_execution **out, yvex_rocm_backend *backend,
                            const yvex_moe_layer_job *job, yvex_moe_layer_result *result,
                            yvex_error *err);
-int yvex_backend_moe_add_expert(yvex_backend_moe_execution *execution,
+int yvex_rocm_backend_moe_add_expert(yvex_rocm_moe_execution *execution,
                                 const yvex_moe_weight_view *gate, const yvex_moe_weight_view *up,
                                 const yvex_moe_weight_view *down, float route_weight, int shared,
                                 yvex_error *err);
-int yvex_backend_moe_finish(yvex_backend_moe_execution *execution, yvex_moe_layer_result *result,
+int yvex_rocm_backend_moe_finish(yvex_rocm_moe_execution *execution, yvex_moe_layer_result *result,
                             yvex_error *err);
-int yvex_backend_moe_close(yvex_backend_moe_execution **execution, yvex_error *err);
+int yvex_rocm_backend_moe_close(yvex_rocm_moe_execution **execution, yvex_error *err);
 
 /* Largest row batch execute_rows accepts in one call. */
 #define YVEX_ROCM_MOE_MAX_ROWS 4096ull
 
 /* ---- expert worklist on the host: include/yvex/internal/execution_batch.h:95-169 ----------- */
 
+#ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef struct {
     unsigned long long *expert_ids, *bucket_offsets, *bucket_populations;
     unsigned long long *source_pairs, *source_rows, *destination_rows;
     float *route_weights;
     unsigned long long bucket_capacity, pair_capacity;
 } yvex_expert_worklist_storage;
+#endif
 
 /* Replaces the sorting core of yvex_expert_worklist_build (src/graph/worklist.c:369-441):
  * stable counting sort of pairs by expert. bucket_offsets needs bucket_capacity + 1 entries.
  * An expert ordinal >= expert_count or a non-finite weight -> FORMAT; storage too small or
  * pair_count not a multiple of experts_per_row -> INVALID_ARG. */
-int yvex_expert_worklist_build(const unsigned long long *selected_experts,
+int yvex_rocm_expert_worklist_build(const unsigned long long *selected_experts,
                                const float *route_weights, unsigned long long pair_count,
                                unsigned long long experts_per_row,
                                unsigned long long expert_count,

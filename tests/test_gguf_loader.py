@@ -1,5 +1,5 @@
-"""GGUF tensor directory reader and resident loading (yvex_gguf_open_path,
-yvex_backend_rocm_gguf_resident_load, yvex_backend_rocm_gguf_weight_view) against the reference's
+"""GGUF tensor directory reader and resident loading (yvex_rocm_gguf_open_path,
+yvex_rocm_gguf_resident_load, yvex_rocm_gguf_weight_view) against the reference's
 structural rules (src/gguf/core.c:850-1250) — live against the reader compiled from the
 reference's sources where oracle/_ref exists, and against the outcomes written down here from it."""
 import ctypes as C
@@ -43,7 +43,7 @@ def write(tmp_path, name, data):
 
 def open_ours(lib, path):
     handle, err = C.c_void_p(), abi.Error()
-    rc = lib.yvex_gguf_open_path(C.byref(handle), path, C.byref(err))
+    rc = lib.yvex_rocm_gguf_open_path(C.byref(handle), path, C.byref(err))
     return rc, handle, err
 
 
@@ -59,21 +59,21 @@ def open_reference(ref, path):
     return rc, handle, artifact
 
 
-def directory(lib, handle):
-    lib.yvex_gguf_tensor_count.restype = abi.ULL
-    lib.yvex_gguf_tensor_count.argtypes = [C.c_void_p]
-    lib.yvex_gguf_tensor_at.restype = C.POINTER(abi.GgufTensorInfo)
-    lib.yvex_gguf_tensor_at.argtypes = [C.c_void_p, abi.ULL]
-    lib.yvex_gguf_tensor_data_offset.restype = abi.ULL
-    lib.yvex_gguf_tensor_data_offset.argtypes = [C.c_void_p]
-    lib.yvex_gguf_alignment.restype = C.c_uint
-    lib.yvex_gguf_alignment.argtypes = [C.c_void_p]
+def directory(lib, handle, prefix="yvex_rocm_gguf_"):
+    """The tensor directory through one library's reader: ours (yvex_rocm_gguf_*) or the
+    reference's own (yvex_gguf_*), whose accessors have the same signatures."""
+    count, at = getattr(lib, prefix + "tensor_count"), getattr(lib, prefix + "tensor_at")
+    data_offset, alignment = getattr(lib, prefix + "tensor_data_offset"), getattr(lib, prefix + "alignment")
+    count.restype, count.argtypes = abi.ULL, [C.c_void_p]
+    at.restype, at.argtypes = C.POINTER(abi.GgufTensorInfo), [C.c_void_p, abi.ULL]
+    data_offset.restype, data_offset.argtypes = abi.ULL, [C.c_void_p]
+    alignment.restype, alignment.argtypes = C.c_uint, [C.c_void_p]
     rows = []
-    for i in range(lib.yvex_gguf_tensor_count(handle)):
-        t = lib.yvex_gguf_tensor_at(handle, i).contents
+    for i in range(count(handle)):
+        t = at(handle, i).contents
         rows.append((t.name, t.rank, tuple(t.dims[:t.rank]), t.ggml_type, t.relative_offset,
                      t.absolute_offset, t.storage_bytes, t.absolute_end_offset, t.range_addressable))
-    return rows, lib.yvex_gguf_tensor_data_offset(handle), lib.yvex_gguf_alignment(handle)
+    return rows, data_offset(handle), alignment(handle)
 
 
 @pytest.fixture
@@ -89,31 +89,31 @@ def test_directory_of_a_well_formed_file(lib, oracle, tmp_path):
     assert rc == 0, err.message
     rows, data_offset, alignment = directory(lib, handle)
     assert alignment == 64 and data_offset == start and start % 64 == 0
-    assert lib.yvex_gguf_file_size(handle) == len(data) and lib.yvex_gguf_metadata_count(handle) == len(meta)
+    assert lib.yvex_rocm_gguf_file_size(handle) == len(data) and lib.yvex_rocm_gguf_metadata_count(handle) == len(meta)
     for row, (name, dims, qtype, blob), offset in zip(rows, tensors, relative):
         assert row == (name.encode(), len(dims), tuple(dims), qtype, offset, start + offset, len(blob),
                        start + offset + len(blob), 1)
-    found = lib.yvex_gguf_tensor_find(handle, b"output.weight")
+    found = lib.yvex_rocm_gguf_tensor_find(handle, b"output.weight")
     assert found and found.contents.ggml_type == Q8_0 and found.contents.ggml_type_name == b"Q8_0"
-    assert not lib.yvex_gguf_tensor_find(handle, b"output.bias")
+    assert not lib.yvex_rocm_gguf_tensor_find(handle, b"output.bias")
     value, real, text, length = abi.ULL(), C.c_double(), C.c_char_p(), abi.ULL()
-    assert lib.yvex_gguf_metadata_u64(handle, b"deepseek4.expert_count", C.byref(value)) == 0 and value.value == 4
-    assert lib.yvex_gguf_metadata_u64(handle, b"deepseek4.big", C.byref(value)) == 0 and value.value == 1 << 40
-    assert lib.yvex_gguf_metadata_u64(handle, b"deepseek4.flag", C.byref(value)) == 0 and value.value == 1
-    assert lib.yvex_gguf_metadata_u64(handle, b"deepseek4.negative", C.byref(value)) == abi.BOUNDS
-    assert lib.yvex_gguf_metadata_u64(handle, b"general.architecture", C.byref(value)) == abi.FORMAT
-    assert lib.yvex_gguf_metadata_f64(handle, b"deepseek4.rope.scale", C.byref(real)) == 0 and real.value == 0.25
-    assert lib.yvex_gguf_metadata_string(handle, b"general.architecture", C.byref(text), C.byref(length)) == 0
+    assert lib.yvex_rocm_gguf_metadata_u64(handle, b"deepseek4.expert_count", C.byref(value)) == 0 and value.value == 4
+    assert lib.yvex_rocm_gguf_metadata_u64(handle, b"deepseek4.big", C.byref(value)) == 0 and value.value == 1 << 40
+    assert lib.yvex_rocm_gguf_metadata_u64(handle, b"deepseek4.flag", C.byref(value)) == 0 and value.value == 1
+    assert lib.yvex_rocm_gguf_metadata_u64(handle, b"deepseek4.negative", C.byref(value)) == abi.BOUNDS
+    assert lib.yvex_rocm_gguf_metadata_u64(handle, b"general.architecture", C.byref(value)) == abi.FORMAT
+    assert lib.yvex_rocm_gguf_metadata_f64(handle, b"deepseek4.rope.scale", C.byref(real)) == 0 and real.value == 0.25
+    assert lib.yvex_rocm_gguf_metadata_string(handle, b"general.architecture", C.byref(text), C.byref(length)) == 0
     assert text.value == b"deepseek4" and length.value == 9
-    assert lib.yvex_gguf_metadata_string(handle, b"missing.key", C.byref(text), None) == abi.FORMAT
+    assert lib.yvex_rocm_gguf_metadata_string(handle, b"missing.key", C.byref(text), None) == abi.FORMAT
     ref = oracle.ref_lib()
     if ref is not None:      # the reference's own reader sees the same directory
         rc, theirs, artifact = open_reference(ref, path)
         assert rc == 0
-        assert directory(ref, theirs) == (rows, data_offset, alignment)
+        assert directory(ref, theirs, "yvex_gguf_") == (rows, data_offset, alignment)
         ref.yvex_gguf_close(C.c_void_p(theirs.value))
         ref.yvex_artifact_close(C.c_void_p(artifact.value))
-    lib.yvex_gguf_close(handle)
+    lib.yvex_rocm_gguf_close(handle)
 
 
 # (case, expected status): outcomes of the reference's reader (src/gguf/core.c:52-79 maps them)
@@ -157,8 +157,8 @@ def test_refusals_match_the_reference_reader(lib, oracle, tmp_path):
     assert not mismatches
     rc, handle, err = open_ours(lib, os.path.join(str(tmp_path), "absent.gguf").encode())
     assert rc == abi.IO and not handle.value
-    assert lib.yvex_gguf_open_path(None, b"x", None) == abi.INVALID_ARG
-    lib.yvex_gguf_close(None)
+    assert lib.yvex_rocm_gguf_open_path(None, b"x", None) == abi.INVALID_ARG
+    lib.yvex_rocm_gguf_close(None)
 
 
 def test_tensor_beyond_the_file_is_marked_and_not_loadable(lib, oracle, tmp_path):
@@ -172,15 +172,15 @@ def test_tensor_beyond_the_file_is_marked_and_not_loadable(lib, oracle, tmp_path
     ref = oracle.ref_lib()
     if ref is not None:
         theirs_rc, theirs, artifact = open_reference(ref, path)
-        assert theirs_rc == 0 and directory(ref, theirs)[0] == rows
+        assert theirs_rc == 0 and directory(ref, theirs, "yvex_gguf_")[0] == rows
         ref.yvex_gguf_close(C.c_void_p(theirs.value))
         ref.yvex_artifact_close(C.c_void_p(artifact.value))
     view, verr = abi.WeightView(), abi.Error()
     host = (C.c_ubyte * 16)()
-    assert lib.yvex_backend_rocm_gguf_weight_view(handle, host, b"blk.3.ffn_norm.weight", C.byref(view),
+    assert lib.yvex_rocm_gguf_weight_view(handle, host, b"blk.3.ffn_norm.weight", C.byref(view),
                                                   C.byref(verr)) == abi.BOUNDS
-    assert lib.yvex_backend_rocm_gguf_weight_view(handle, host, b"nope", C.byref(view), C.byref(verr)) == abi.FORMAT
-    lib.yvex_gguf_close(handle)
+    assert lib.yvex_rocm_gguf_weight_view(handle, host, b"nope", C.byref(view), C.byref(verr)) == abi.FORMAT
+    lib.yvex_rocm_gguf_close(handle)
 
 
 @pytest.mark.gpu
@@ -197,24 +197,24 @@ def test_tensors_loaded_from_a_file_run_through_the_kernels(gpu, oracle, tmp_pat
     rc, handle, err = open_ours(lib, path)
     assert rc == 0, err.message
     arena, host, lerr = C.POINTER(abi.DeviceTensor)(), C.c_void_p(), abi.Error()
-    assert lib.yvex_backend_rocm_gguf_resident_load(b.handle, handle, 1, C.byref(arena), C.byref(host),
+    assert lib.yvex_rocm_gguf_resident_load(b.handle, handle, 1, C.byref(arena), C.byref(host),
                                                     C.byref(lerr)) == 0, lerr.message
     b.tensors.append(arena)
     assert arena.contents.bytes == len(data) - start
     view = abi.WeightView()
-    assert lib.yvex_backend_rocm_gguf_weight_view(handle, host, b"blk.3.ffn_gate_exps.weight", C.byref(view),
+    assert lib.yvex_rocm_gguf_weight_view(handle, host, b"blk.3.ffn_gate_exps.weight", C.byref(view),
                                                   C.byref(lerr)) == 0
     assert (view.qtype, view.row_width, view.row_count, view.row_bytes) == (IQ2_XXS, 512, 1024, 132)
     assert view.layout == abi.LAYOUT_EXPERT_MAJOR and view.encoded == host.value + relative[0]
     assert view.encoded_bytes == parts["gate"].nbytes
     head = abi.WeightView()
-    assert lib.yvex_backend_rocm_gguf_weight_view(handle, host, b"output.weight", C.byref(head), C.byref(lerr)) == 0
+    assert lib.yvex_rocm_gguf_weight_view(handle, host, b"output.weight", C.byref(head), C.byref(lerr)) == 0
     assert (head.qtype, head.row_width, head.row_count, head.row_bytes) == (Q8_0, 512, 300, 544)
     g = oracle.Generator(3, "gguf.x")
     x = g.normal(2 * 512).reshape(2, 512)
     xin, out = b.f32(x), b.empty_f32(2 * 300)
     facts = abi.OperationFacts()
-    rc = lib.yvex_backend_rocm_encoded_matvec(
+    rc = lib.yvex_rocm_encoded_matvec(
         b.handle, C.c_void_p(head.encoded), abi.ULL(head.encoded_bytes), C.c_uint(head.qtype),
         abi.ULL(head.row_count), abi.ULL(head.row_width), abi.ULL(head.row_bytes), abi.ULL(2), xin, None,
         abi.ULL(0), None, out, 0, C.byref(facts), C.byref(lerr))
@@ -226,12 +226,12 @@ def test_tensors_loaded_from_a_file_run_through_the_kernels(gpu, oracle, tmp_pat
     ids = np.array([2 * 256, 2 * 256 + 255], np.uint32)
     decoded = b.empty_f32(2 * 512)
     b.workspace(4096)       # the gather stages its row identifiers there
-    rc = lib.yvex_backend_rocm_encoded_gather(
+    rc = lib.yvex_rocm_encoded_gather(
         b.handle, C.c_void_p(view.encoded), abi.ULL(view.encoded_bytes), C.c_uint(view.qtype),
         abi.ULL(view.row_count), abi.ULL(view.row_width), abi.ULL(view.row_bytes), ids.ctypes.data, abi.ULL(2),
         decoded, C.byref(facts), C.byref(lerr))
     assert rc == 0, lerr.message
     rows = oracle.decode_rows(oracle.IQ2_XXS, parts["gate"], 512, ids)
     assert np.array_equal(b.read_f32(decoded, 1024).reshape(2, 512), rows)
-    lib.yvex_gguf_close(handle)
+    lib.yvex_rocm_gguf_close(handle)
     assert b.close() == 0

@@ -20,7 +20,7 @@ def backend(gpu):
     from backend_helpers import Backend
     b = Backend()
     assert b.ok, b.err.message
-    assert b.lib.yvex_backend_status_of(b.handle) == abi.STATUS_READY
+    assert b.lib.yvex_rocm_backend_status_of(b.handle) == abi.STATUS_READY
     yield b
     assert b.close() == 0
 
@@ -32,7 +32,7 @@ def close_to(got, want, rel=1e-3, abs_=1e-5):
 
 def run_matvec(b, host, w, qt, rows, width, x_tensor, out, in_rows, q8, additive=None):
     facts, err = abi.OperationFacts(), abi.Error()
-    rc = b.lib.yvex_backend_rocm_encoded_matvec(
+    rc = b.lib.yvex_rocm_encoded_matvec(
         b.handle, host, w.nbytes, qt, rows, width, w.nbytes // rows, in_rows, x_tensor, None, 0,
         additive, out, q8, C.byref(facts), C.byref(err))
     return rc, facts, err
@@ -148,7 +148,7 @@ def test_encoded_matvec_split_input(backend, oracle):
     facts, err = abi.OperationFacts(), abi.Error()
 
     def run(tail_tensor, head_w, q8=0):
-        return b.lib.yvex_backend_rocm_encoded_matvec(
+        return b.lib.yvex_rocm_encoded_matvec(
             b.handle, host, w.nbytes, oracle.Q8_0, rows, width, w.nbytes // rows, in_rows, head, tail_tensor,
             head_w, None, out, q8, C.byref(facts), C.byref(err))
 
@@ -186,13 +186,13 @@ def test_bundle_failure_seam_is_fail_closed(gpu, monkeypatch):
     monkeypatch.setenv("YVEX_TEST_ROCM_BUNDLE_FAILURE", "1")
     from backend_helpers import Backend
     b = Backend()
-    assert b.ok and b.lib.yvex_backend_status_of(b.handle) == abi.STATUS_CONTEXT_READY
+    assert b.ok and b.lib.yvex_rocm_backend_status_of(b.handle) == abi.STATUS_CONTEXT_READY
     t = b.f32(np.arange(4, dtype=np.float32))
     assert np.array_equal(b.read_f32(t, 4), np.arange(4, dtype=np.float32))
     cap = abi.CapabilityResult()
-    b.lib.yvex_backend_query_capability(b.handle, abi.VARIANT_ATTENTION_ENCODED, C.byref(cap), None)
+    b.lib.yvex_rocm_backend_query_capability(b.handle, abi.VARIANT_ATTENTION_ENCODED, C.byref(cap), None)
     assert cap.state == abi.CAP_UNSUPPORTED and cap.reason == abi.REASON_KERNEL_BUNDLE_ABSENT
-    assert not b.lib.yvex_backend_moe_operations_get(b.handle)
+    assert not b.lib.yvex_rocm_backend_moe_operations_get(b.handle)
     assert b.close() == 0
 
 
@@ -205,7 +205,7 @@ def test_encoded_gather(backend, oracle):
     ids = np.array([39, 0, 7, 7], np.uint32)
     out = b.empty_f32(ids.size * width)
     facts, err = abi.OperationFacts(), abi.Error()
-    rc = b.lib.yvex_backend_rocm_encoded_gather(b.handle, host, w.nbytes, 16, rows, width, 132,
+    rc = b.lib.yvex_rocm_encoded_gather(b.handle, host, w.nbytes, 16, rows, width, 132,
                                                 ids.ctypes.data, ids.size, out, C.byref(facts),
                                                 C.byref(err))
     assert rc == 0, err.message
@@ -218,7 +218,7 @@ def test_encoded_gather(backend, oracle):
 def run_greedy(b, logits, rows, width):
     tokens, best, ties = np.full(rows, 7, np.uint32), np.full(rows, 7, np.float32), np.full(rows, 7, np.uint64)
     facts, err = abi.OperationFacts(), abi.Error()
-    rc = b.lib.yvex_backend_rocm_select_greedy_rows(b.handle, logits, rows, width, tokens.ctypes.data,
+    rc = b.lib.yvex_rocm_select_greedy_rows(b.handle, logits, rows, width, tokens.ctypes.data,
                                                     best.ctypes.data, ties.ctypes.data, C.byref(facts),
                                                     C.byref(err))
     return rc, tokens, best, ties, facts, err
@@ -352,7 +352,7 @@ class MoeCase:
             view(abi.W_MHC_SCALE, "scale", 0, 3, 1, 12, abi.ACT_DEVICE_F32)
             view(abi.W_MHC_BASE, "base", 0, mixing, 1, mixing * 4, abi.ACT_DEVICE_F32)
             view(abi.W_FFN_NORM, "norm", 30, hidden, 1, hidden * 2, abi.ACT_DEVICE_F32)
-        self.ops = b.lib.yvex_backend_moe_operations_get(b.handle).contents
+        self.ops = b.lib.yvex_rocm_backend_moe_operations_get(b.handle).contents
         need, err = abi.ULL(), abi.Error()
         assert self.ops.workspace_required(C.byref(self.plan), rows, C.byref(need), C.byref(err)) == 0
         self.workspace_bytes = need.value
@@ -539,7 +539,7 @@ def test_execute_rows_refusals(backend, oracle):
     batch.provenance, batch.phase = case.batch.provenance, case.batch.phase
     case.job.execution_batch = C.pointer(batch)
     sentinel = np.full(case.rows * case.hidden, 7.0, np.float32)
-    b.lib.yvex_backend_tensor_write(b.handle, case.rows_out, sentinel.ctypes.data, sentinel.nbytes, None)
+    b.lib.yvex_rocm_backend_tensor_write(b.handle, case.rows_out, sentinel.ctypes.data, sentinel.nbytes, None)
     assert case.execute() == abi.UNSUPPORTED
     assert np.array_equal(b.read_f32(case.rows_out, sentinel.size), sentinel)
     policy.supported_width_mask |= 1 << case.rows
@@ -672,7 +672,7 @@ def test_execute_rows_graph_replays_equal_eager(backend, oracle, kwargs):
     rng = np.random.default_rng(7)
 
     def run(rows_now, eager):
-        rc = b.lib.yvex_backend_tensor_write(b.handle, case.rows_in, rows_now.ctypes.data, rows_now.nbytes,
+        rc = b.lib.yvex_rocm_backend_tensor_write(b.handle, case.rows_in, rows_now.ctypes.data, rows_now.nbytes,
                                              C.byref(b.err))
         assert rc == 0, b.err.message
         case.job.eager_execution = int(eager)
@@ -750,7 +750,7 @@ class TokenLocal:
         self.handle, self.err = C.c_void_p(), abi.Error()
 
     def begin(self):
-        return self.b.lib.yvex_backend_moe_begin(C.byref(self.handle), self.b.handle, C.byref(self.job),
+        return self.b.lib.yvex_rocm_backend_moe_begin(C.byref(self.handle), self.b.handle, C.byref(self.job),
                                                  C.byref(self.result), C.byref(self.err))
 
     def expert_views(self, expert=None, outside=False):
@@ -778,15 +778,15 @@ class TokenLocal:
         return views, keep
 
     def add(self, views, weight, shared):
-        return self.b.lib.yvex_backend_moe_add_expert(self.handle, C.byref(views[0]), C.byref(views[1]),
+        return self.b.lib.yvex_rocm_backend_moe_add_expert(self.handle, C.byref(views[0]), C.byref(views[1]),
                                                       C.byref(views[2]), C.c_float(weight), int(shared),
                                                       C.byref(self.err))
 
     def finish(self):
-        return self.b.lib.yvex_backend_moe_finish(self.handle, C.byref(self.result), C.byref(self.err))
+        return self.b.lib.yvex_rocm_backend_moe_finish(self.handle, C.byref(self.result), C.byref(self.err))
 
     def close(self):
-        return self.b.lib.yvex_backend_moe_close(C.byref(self.handle), C.byref(self.err))
+        return self.b.lib.yvex_rocm_backend_moe_close(C.byref(self.handle), C.byref(self.err))
 
 
 def token_oracle(case, row):

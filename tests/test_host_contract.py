@@ -46,28 +46,41 @@ def test_header_and_binding_agree_on_symbols():
     assert declared == set(abi.EXPORTS + abi.KERNEL_EXPORTS)
 
 
+def test_library_exports_nothing_else():
+    """Only the declared entry points leave the library, all under its own prefixes: no name of
+    the reference's libyvex (yvex_backend_open, yvex_gguf_*, yvex_error_* ...) is defined, so
+    the two can be linked or loaded together without one interposing on the other."""
+    import subprocess
+    from yvex_amd import LIB_PATH
+    listing = subprocess.run(["nm", "-D", "--defined-only", LIB_PATH], capture_output=True, text=True,
+                             check=True).stdout
+    exported = {line.split()[-1].split("@")[0] for line in listing.splitlines() if line.strip()}
+    assert exported == set(abi.EXPORTS + abi.KERNEL_EXPORTS)
+    assert all(name.startswith(("yvex_rocm_", "yvex_hip_")) for name in exported)
+
+
 def test_status_names(lib):
     names = {0: b"ok", -4: b"format", -5: b"unsupported", -6: b"backend", -7: b"bounds",
              -10: b"invalid-arg", -9: b"cancelled", -2: b"nomem", -8: b"state"}
     for code, name in names.items():
-        assert lib.yvex_status_name(code) == name
+        assert lib.yvex_rocm_status_name(code) == name
 
 
 def test_qtype_geometry_abi(lib):
     expect = {0: (1, 4), 1: (1, 2), 8: (32, 34), 10: (256, 84), 12: (256, 144), 15: (256, 292),
               16: (256, 66), 26: (1, 4), 30: (1, 2), 39: (32, 17)}
     for qtype, (block, nbytes) in expect.items():
-        g = lib.yvex_gguf_qtype_geometry_find(qtype).contents
+        g = lib.yvex_rocm_gguf_qtype_geometry_find(qtype).contents
         assert (g.qtype, g.block_size, g.bytes_per_block) == (qtype, block, nbytes)
-    assert lib.yvex_gguf_qtype_geometry_find(4).contents.identity == 1      # removed
-    assert lib.yvex_gguf_qtype_geometry_find(41).contents.identity == 3     # outside baseline
-    assert not lib.yvex_gguf_qtype_geometry_find(43)
+    assert lib.yvex_rocm_gguf_qtype_geometry_find(4).contents.identity == 1      # removed
+    assert lib.yvex_rocm_gguf_qtype_geometry_find(41).contents.identity == 3     # outside baseline
+    assert not lib.yvex_rocm_gguf_qtype_geometry_find(43)
 
 
 def test_capability_registry_is_total_and_fail_closed(lib, oracle):
     reference_compute = {0, 1, 8, 10, 16, 26, 30, 39}   # src/gguf/quant_registry.c:50-103
     for qtype in range(43):
-        cap = lib.yvex_quant_numeric_capability_at(qtype).contents
+        cap = lib.yvex_rocm_quant_numeric_capability_at(qtype).contents
         assert cap.qtype == qtype and cap.known == 1
         assert bool(cap.dedicated_cpu_compute_available) == (qtype in reference_compute or qtype == 12)
         assert bool(oracle.lib().yvo_qtype_reference_cpu_compute(qtype)) == (qtype in reference_compute)
@@ -79,44 +92,44 @@ def test_capability_registry_is_total_and_fail_closed(lib, oracle):
             assert cap.extension_of_reference == 0
             assert bool(cap.device_compute_available) == (qtype in reference_compute)
     for removed in (4, 5, 31, 32, 33, 36, 37, 38):
-        assert lib.yvex_quant_numeric_capability_at(removed).contents.refusal == 2
+        assert lib.yvex_rocm_quant_numeric_capability_at(removed).contents.refusal == 2
     for outside in (40, 41, 42):
-        assert lib.yvex_quant_numeric_capability_at(outside).contents.refusal == 3
-    assert not lib.yvex_quant_numeric_capability_at(43)
+        assert lib.yvex_rocm_quant_numeric_capability_at(outside).contents.refusal == 3
+    assert not lib.yvex_rocm_quant_numeric_capability_at(43)
 
 
 def test_open_refuses_other_kinds_and_missing_device(lib, monkeypatch):
     monkeypatch.delenv("YVEX_TEST_ROCM_NO_DEVICE", raising=False)
     handle, err = C.c_void_p(), abi.Error()
     opts = abi.BackendOptions(abi.KIND_CUDA, None, 0)
-    assert lib.yvex_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.UNSUPPORTED
+    assert lib.yvex_rocm_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.UNSUPPORTED
     assert not handle.value
     import torch
     if not torch.cuda.is_available():
         opts = abi.BackendOptions(abi.KIND_ROCM, None, 0)
-        assert lib.yvex_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.BACKEND
+        assert lib.yvex_rocm_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.BACKEND
         assert b"device-unavailable" in err.message and not handle.value
     opts = abi.BackendOptions(abi.KIND_ROCM, b"gpu0", 0)
-    assert lib.yvex_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.INVALID_ARG
+    assert lib.yvex_rocm_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == abi.INVALID_ARG
 
 
 def test_seam_backend_keeps_tensors_and_refuses_compute(seam):
     lib = seam.lib
-    assert lib.yvex_backend_kind_of(seam.handle) == abi.KIND_ROCM
-    assert lib.yvex_backend_status_of(seam.handle) == abi.STATUS_CONTEXT_READY
+    assert lib.yvex_rocm_backend_kind_of(seam.handle) == abi.KIND_ROCM
+    assert lib.yvex_rocm_backend_status_of(seam.handle) == abi.STATUS_CONTEXT_READY
     x = np.arange(16, dtype=np.float32)
     t = seam.f32(x)
     assert np.array_equal(seam.read_f32(t, 16), x)
     cap = abi.CapabilityResult()
-    assert lib.yvex_backend_query_capability(seam.handle, abi.VARIANT_TENSOR_ALLOC, C.byref(cap), None) == 0
+    assert lib.yvex_rocm_backend_query_capability(seam.handle, abi.VARIANT_TENSOR_ALLOC, C.byref(cap), None) == 0
     assert cap.state == abi.CAP_SUPPORTED
     for variant in (abi.VARIANT_ATTENTION_ENCODED, abi.VARIANT_QTYPE_ROW_DOT):
-        assert lib.yvex_backend_query_capability(seam.handle, variant, C.byref(cap), None) == 0
+        assert lib.yvex_rocm_backend_query_capability(seam.handle, variant, C.byref(cap), None) == 0
         assert cap.state == abi.CAP_UNSUPPORTED and cap.reason == abi.REASON_KERNEL_BUNDLE_ABSENT
         assert cap.kernel_bundle_available == 0 and cap.context_available == 1
-    assert lib.yvex_backend_query_capability(seam.handle, 9, C.byref(cap), None) == 0
+    assert lib.yvex_rocm_backend_query_capability(seam.handle, 9, C.byref(cap), None) == 0
     assert cap.state == abi.CAP_UNSUPPORTED and cap.reason == abi.REASON_VARIANT_UNSUPPORTED
-    assert not lib.yvex_backend_moe_operations_get(seam.handle)
+    assert not lib.yvex_rocm_backend_moe_operations_get(seam.handle)
 
 
 def test_token_local_operation_without_kernels(seam):
@@ -126,7 +139,7 @@ def test_token_local_operation_without_kernels(seam):
     plan, job, result, err = abi.LayerPlan(), abi.LayerJob(), abi.LayerResult(), abi.Error()
     handle = C.c_void_p()
     job.layer = C.pointer(plan)
-    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+    assert lib.yvex_rocm_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
                                       C.byref(err)) == abi.INVALID_ARG
     plan.hidden_width, plan.residual_streams, plan.expanded_width = 256, 2, 512
     plan.mhc_mixing_rows, plan.mhc_sinkhorn_iterations = 8, 2
@@ -142,14 +155,14 @@ def test_token_local_operation_without_kernels(seam):
     result.combined_capacity = result.routed_capacity = result.shared_capacity = 256
     result.post, result.post_capacity = out[3].ctypes.data, 2
     result.combination, result.combination_capacity = out[4].ctypes.data, 4
-    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+    assert lib.yvex_rocm_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
                                       C.byref(err)) == abi.UNSUPPORTED
     assert not handle.value and b"kernel" in err.message
     plan.mhc_mixing_rows = 7
-    assert lib.yvex_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
+    assert lib.yvex_rocm_backend_moe_begin(C.byref(handle), seam.handle, C.byref(job), C.byref(result),
                                       C.byref(err)) == abi.BOUNDS
-    assert lib.yvex_backend_moe_close(C.byref(handle), C.byref(err)) == 0
-    assert lib.yvex_backend_moe_finish(None, C.byref(result), C.byref(err)) == abi.INVALID_ARG
+    assert lib.yvex_rocm_backend_moe_close(C.byref(handle), C.byref(err)) == 0
+    assert lib.yvex_rocm_backend_moe_finish(None, C.byref(result), C.byref(err)) == abi.INVALID_ARG
 
 
 def test_tensor_ownership_and_limits(monkeypatch):
@@ -160,14 +173,14 @@ def test_tensor_ownership_and_limits(monkeypatch):
     assert rc == abi.NOMEM
     ta = a.f32(np.ones(8, np.float32))
     out = np.empty(8, np.float32)
-    assert b.lib.yvex_backend_tensor_read(b.handle, ta, out.ctypes.data, 32, C.byref(b.err)) == abi.FORMAT
-    assert a.lib.yvex_backend_tensor_read(a.handle, ta, out.ctypes.data, 64, C.byref(a.err)) == abi.BOUNDS
+    assert b.lib.yvex_rocm_backend_tensor_read(b.handle, ta, out.ctypes.data, 32, C.byref(b.err)) == abi.FORMAT
+    assert a.lib.yvex_rocm_backend_tensor_read(a.handle, ta, out.ctypes.data, 64, C.byref(a.err)) == abi.BOUNDS
     rc, unwritten = a.tensor(32)
-    assert a.lib.yvex_backend_tensor_read(a.handle, unwritten, out.ctypes.data, 32, C.byref(a.err)) == abi.STATE
-    assert a.lib.yvex_backend_close_checked(C.byref(a.handle), C.byref(a.err)) == abi.STATE   # live tensors
+    assert a.lib.yvex_rocm_backend_tensor_read(a.handle, unwritten, out.ctypes.data, 32, C.byref(a.err)) == abi.STATE
+    assert a.lib.yvex_rocm_backend_close_checked(C.byref(a.handle), C.byref(a.err)) == abi.STATE   # live tensors
     assert a.handle.value
     stats = abi.MemoryStats()
-    assert a.lib.yvex_backend_get_memory_stats(a.handle, C.byref(stats), None) == 0
+    assert a.lib.yvex_rocm_backend_get_memory_stats(a.handle, C.byref(stats), None) == 0
     assert stats.allocated_bytes == 64 and stats.allocation_count == 2 and stats.h2d_bytes == 32
     assert a.close() == 0 and not a.handle.value
     assert b.close() == 0
@@ -178,10 +191,10 @@ def test_cleanup_failure_keeps_the_owner_for_retry(monkeypatch):
     from backend_helpers import Backend
     b = Backend()
     monkeypatch.setenv("YVEX_TEST_ROCM_CLEANUP_FAILURE", "1")
-    assert b.lib.yvex_backend_close_checked(C.byref(b.handle), C.byref(b.err)) == abi.BACKEND
-    assert b.handle.value and b.lib.yvex_backend_status_of(b.handle) == abi.STATUS_FAILED
+    assert b.lib.yvex_rocm_backend_close_checked(C.byref(b.handle), C.byref(b.err)) == abi.BACKEND
+    assert b.handle.value and b.lib.yvex_rocm_backend_status_of(b.handle) == abi.STATUS_FAILED
     monkeypatch.delenv("YVEX_TEST_ROCM_CLEANUP_FAILURE")
-    assert b.lib.yvex_backend_close_checked(C.byref(b.handle), C.byref(b.err)) == 0
+    assert b.lib.yvex_rocm_backend_close_checked(C.byref(b.handle), C.byref(b.err)) == 0
     assert not b.handle.value
 
 
@@ -190,31 +203,31 @@ def test_resident_resolve_semantics(seam):
     blob = np.arange(4096, dtype=np.uint8)
     arena, host = seam.resident(blob)
     addr = abi.ULL()
-    assert lib.yvex_backend_resident_resolve(seam.handle, host + 100, 50, C.byref(addr)) == abi.RESIDENT_HIT
+    assert lib.yvex_rocm_backend_resident_resolve(seam.handle, host + 100, 50, C.byref(addr)) == abi.RESIDENT_HIT
     assert addr.value == arena.contents.data + 100
-    assert lib.yvex_backend_resident_resolve(seam.handle, host + 4000, 200, C.byref(addr)) == abi.RESIDENT_MISS
-    assert lib.yvex_backend_resident_resolve(seam.handle, host - 1, 4, C.byref(addr)) == abi.RESIDENT_MISS
-    assert lib.yvex_backend_resident_detach(seam.handle, None) == 0
-    assert lib.yvex_backend_resident_resolve(seam.handle, host, 4, C.byref(addr)) == abi.RESIDENT_MISS
+    assert lib.yvex_rocm_backend_resident_resolve(seam.handle, host + 4000, 200, C.byref(addr)) == abi.RESIDENT_MISS
+    assert lib.yvex_rocm_backend_resident_resolve(seam.handle, host - 1, 4, C.byref(addr)) == abi.RESIDENT_MISS
+    assert lib.yvex_rocm_backend_resident_detach(seam.handle, None) == 0
+    assert lib.yvex_rocm_backend_resident_resolve(seam.handle, host, 4, C.byref(addr)) == abi.RESIDENT_MISS
 
 
 def test_workspace_bump_allocation(seam):
     lib = seam.lib
     ws = seam.workspace(4096)
     a, b = abi.ULL(), abi.ULL()
-    assert lib.yvex_backend_workspace_acquire(seam.handle, 100, 256, C.byref(a)) == 1
-    assert lib.yvex_backend_workspace_acquire(seam.handle, 100, 256, C.byref(b)) == 1
+    assert lib.yvex_rocm_backend_workspace_acquire(seam.handle, 100, 256, C.byref(a)) == 1
+    assert lib.yvex_rocm_backend_workspace_acquire(seam.handle, 100, 256, C.byref(b)) == 1
     assert a.value % 256 == 0 and b.value % 256 == 0 and b.value >= a.value + 100
-    assert lib.yvex_backend_workspace_acquire(seam.handle, 8192, 256, C.byref(b)) == 0
-    assert lib.yvex_backend_workspace_acquire(seam.handle, 16, 3, C.byref(b)) == 0     # not a power of two
-    lib.yvex_backend_workspace_detach(seam.handle)
-    assert lib.yvex_backend_workspace_acquire(seam.handle, 16, 16, C.byref(b)) == 0
+    assert lib.yvex_rocm_backend_workspace_acquire(seam.handle, 8192, 256, C.byref(b)) == 0
+    assert lib.yvex_rocm_backend_workspace_acquire(seam.handle, 16, 3, C.byref(b)) == 0     # not a power of two
+    lib.yvex_rocm_backend_workspace_detach(seam.handle)
+    assert lib.yvex_rocm_backend_workspace_acquire(seam.handle, 16, 16, C.byref(b)) == 0
     del ws
 
 
 def matvec(seam, host, nbytes, qtype, rows, width, row_bytes, x, out, additive=None, q8=0, in_rows=1):
     facts, err = abi.OperationFacts(), abi.Error()
-    rc = seam.lib.yvex_backend_rocm_encoded_matvec(
+    rc = seam.lib.yvex_rocm_encoded_matvec(
         seam.handle, host, nbytes, qtype, rows, width, row_bytes, in_rows, x, None, 0, additive, out,
         q8, C.byref(facts), C.byref(err))
     return rc, facts, err
@@ -265,7 +278,7 @@ def test_encoded_gather_refusals(seam, oracle):
     out = seam.empty_f32(2 * width)
     facts, err = abi.OperationFacts(), abi.Error()
     ids = (C.c_uint * 2)(1, 9)
-    call = lambda qt, ids_: seam.lib.yvex_backend_rocm_encoded_gather(
+    call = lambda qt, ids_: seam.lib.yvex_rocm_encoded_gather(
         seam.handle, host, w.nbytes, qt, rows, width, 144, ids_, 2, out, C.byref(facts), C.byref(err))
     assert call(12, ids) == abi.BOUNDS                # row 9 of 8
     assert call(14, (C.c_uint * 2)(1, 2)) == abi.UNSUPPORTED
@@ -286,7 +299,7 @@ def test_host_worklist_matches_oracle_and_refuses(lib, oracle):
         "expert_ids", "bucket_offsets", "bucket_populations", "source_pairs", "source_rows",
         "destination_rows")), rw.ctypes.data, experts, pairs)
     obs, err = abi.WorklistObservation(), abi.Error()
-    rc = lib.yvex_expert_worklist_build(sel.ctypes.data, w.ctypes.data, pairs, topk, experts,
+    rc = lib.yvex_rocm_expert_worklist_build(sel.ctypes.data, w.ctypes.data, pairs, topk, experts,
                                         C.byref(storage), C.byref(obs), C.byref(err))
     assert rc == 0
     orc, want = oracle.worklist_build(sel, w, topk, experts)
@@ -306,12 +319,12 @@ def test_host_worklist_matches_oracle_and_refuses(lib, oracle):
     assert sum(obs.population_histogram) == n
     bad = sel.copy()
     bad[0, 0] = experts
-    assert lib.yvex_expert_worklist_build(bad.ctypes.data, w.ctypes.data, pairs, topk, experts,
+    assert lib.yvex_rocm_expert_worklist_build(bad.ctypes.data, w.ctypes.data, pairs, topk, experts,
                                           C.byref(storage), C.byref(obs), C.byref(err)) == abi.FORMAT
     w2 = w.copy()
     w2[1, 1] = np.inf
-    assert lib.yvex_expert_worklist_build(sel.ctypes.data, w2.ctypes.data, pairs, topk, experts,
+    assert lib.yvex_rocm_expert_worklist_build(sel.ctypes.data, w2.ctypes.data, pairs, topk, experts,
                                           C.byref(storage), C.byref(obs), C.byref(err)) == abi.FORMAT
     storage.pair_capacity = pairs - 1
-    assert lib.yvex_expert_worklist_build(sel.ctypes.data, w.ctypes.data, pairs, topk, experts,
+    assert lib.yvex_rocm_expert_worklist_build(sel.ctypes.data, w.ctypes.data, pairs, topk, experts,
                                           C.byref(storage), C.byref(obs), C.byref(err)) == abi.INVALID_ARG

@@ -269,24 +269,25 @@ class WorklistStorage(C.Structure):
 
 # Every symbol include/yvex_rocm.h declares; the CPU test suite checks the library exports all.
 EXPORTS = [
-    "yvex_status_name", "yvex_error_clear", "yvex_error_set", "yvex_error_is_set", "yvex_error_code",
-    "yvex_gguf_qtype_geometry_find", "yvex_quant_numeric_capability_at",
-    "yvex_backend_open", "yvex_backend_close_checked", "yvex_backend_kind_of",
-    "yvex_backend_status_of", "yvex_backend_get_memory_stats", "yvex_backend_sync",
-    "yvex_backend_query_capability", "yvex_backend_tensor_alloc", "yvex_backend_tensor_release",
-    "yvex_backend_tensor_write", "yvex_backend_tensor_read", "yvex_backend_tensor_copy",
-    "yvex_backend_tensor_owned_by", "yvex_backend_resident_alloc", "yvex_backend_resident_prefetch",
-    "yvex_backend_resident_attach", "yvex_backend_resident_detach", "yvex_backend_resident_resolve",
-    "yvex_backend_workspace_attach", "yvex_backend_workspace_detach",
-    "yvex_backend_workspace_acquire", "yvex_backend_rocm_encoded_matvec",
-    "yvex_backend_rocm_encoded_gather", "yvex_backend_rocm_select_greedy_rows", "yvex_rocm_quant_row_dot",
-    "yvex_backend_moe_operations_get", "yvex_backend_moe_begin", "yvex_backend_moe_add_expert",
-    "yvex_backend_moe_finish", "yvex_backend_moe_close",
-    "yvex_expert_worklist_build", "yvex_rocm_moe_derived_layout_plan", "yvex_rocm_moe_derived_layout_build",
-    "yvex_gguf_open_path", "yvex_gguf_close", "yvex_gguf_metadata_count", "yvex_gguf_metadata_u64",
-    "yvex_gguf_metadata_f64", "yvex_gguf_metadata_string", "yvex_gguf_tensor_count", "yvex_gguf_tensor_at",
-    "yvex_gguf_tensor_find", "yvex_gguf_tensor_data_offset", "yvex_gguf_alignment", "yvex_gguf_file_size",
-    "yvex_backend_rocm_gguf_resident_load", "yvex_backend_rocm_gguf_weight_view",
+    "yvex_rocm_status_name", "yvex_rocm_error_clear", "yvex_rocm_error_set", "yvex_rocm_error_is_set", "yvex_rocm_error_code",
+    "yvex_rocm_gguf_qtype_geometry_find", "yvex_rocm_quant_numeric_capability_at",
+    "yvex_rocm_backend_open", "yvex_rocm_backend_bind_owner", "yvex_rocm_backend_close_checked", "yvex_rocm_backend_kind_of",
+    "yvex_rocm_backend_status_of", "yvex_rocm_backend_get_memory_stats", "yvex_rocm_backend_sync",
+    "yvex_rocm_backend_query_capability", "yvex_rocm_backend_tensor_alloc", "yvex_rocm_backend_tensor_release",
+    "yvex_rocm_backend_tensor_write", "yvex_rocm_backend_tensor_read", "yvex_rocm_backend_tensor_copy",
+    "yvex_rocm_backend_tensor_owned_by", "yvex_rocm_backend_resident_alloc", "yvex_rocm_backend_resident_prefetch",
+    "yvex_rocm_backend_resident_attach", "yvex_rocm_backend_resident_detach", "yvex_rocm_backend_resident_resolve",
+    "yvex_rocm_backend_workspace_attach", "yvex_rocm_backend_workspace_detach",
+    "yvex_rocm_backend_workspace_acquire", "yvex_rocm_encoded_matvec",
+    "yvex_rocm_encoded_gather", "yvex_rocm_select_greedy_rows", "yvex_rocm_quant_row_dot",
+    "yvex_rocm_backend_moe_operations_get", "yvex_rocm_backend_moe_begin", "yvex_rocm_backend_moe_add_expert",
+    "yvex_rocm_backend_moe_finish", "yvex_rocm_backend_moe_close",
+    "yvex_rocm_expert_worklist_build", "yvex_rocm_moe_derived_layout_plan", "yvex_rocm_moe_derived_layout_build",
+    "yvex_rocm_moe_workspace_required",
+    "yvex_rocm_gguf_open_path", "yvex_rocm_gguf_close", "yvex_rocm_gguf_metadata_count", "yvex_rocm_gguf_metadata_u64",
+    "yvex_rocm_gguf_metadata_f64", "yvex_rocm_gguf_metadata_string", "yvex_rocm_gguf_tensor_count", "yvex_rocm_gguf_tensor_at",
+    "yvex_rocm_gguf_tensor_find", "yvex_rocm_gguf_tensor_data_offset", "yvex_rocm_gguf_alignment", "yvex_rocm_gguf_file_size",
+    "yvex_rocm_gguf_resident_load", "yvex_rocm_gguf_weight_view",
 ]
 KERNEL_EXPORTS = [
     "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_row_dot", "yvex_hip_matvec", "yvex_hip_block_dots_i32", "yvex_hip_gather",
@@ -308,87 +309,87 @@ KERNEL_EXPORTS = [
 
 def library():
     lib = load_library()
-    lib.yvex_status_name.restype = C.c_char_p
-    lib.yvex_gguf_qtype_geometry_find.restype = C.POINTER(QtypeGeometry)
-    lib.yvex_quant_numeric_capability_at.restype = C.POINTER(NumericCapability)
-    lib.yvex_backend_moe_operations_get.restype = C.POINTER(MoeOperations)
-    lib.yvex_backend_moe_operations_get.argtypes = [C.c_void_p]
+    lib.yvex_rocm_status_name.restype = C.c_char_p
+    lib.yvex_rocm_gguf_qtype_geometry_find.restype = C.POINTER(QtypeGeometry)
+    lib.yvex_rocm_quant_numeric_capability_at.restype = C.POINTER(NumericCapability)
+    lib.yvex_rocm_backend_moe_operations_get.restype = C.POINTER(MoeOperations)
+    lib.yvex_rocm_backend_moe_operations_get.argtypes = [C.c_void_p]
     lib.yvex_rocm_quant_row_dot.argtypes = [C.c_void_p, C.c_uint, C.c_void_p, C.c_size_t, C.c_void_p, ULL,
                                             C.POINTER(C.c_float), C.c_void_p, C.POINTER(Error)]
     lib.yvex_rocm_moe_derived_layout_plan.argtypes = [C.POINTER(ExecutionDecision), C.POINTER(ULL),
                                                       C.POINTER(Error)]
     lib.yvex_rocm_moe_derived_layout_build.argtypes = [C.POINTER(ExecutionDecision), C.c_void_p, ULL,
                                                        C.c_void_p, ULL, C.POINTER(Error)]
-    lib.yvex_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
-    lib.yvex_gguf_close.argtypes = [C.c_void_p]
-    lib.yvex_gguf_close.restype = None
-    for name in ("yvex_gguf_metadata_count", "yvex_gguf_tensor_count", "yvex_gguf_tensor_data_offset",
-                 "yvex_gguf_file_size"):
+    lib.yvex_rocm_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
+    lib.yvex_rocm_gguf_close.argtypes = [C.c_void_p]
+    lib.yvex_rocm_gguf_close.restype = None
+    for name in ("yvex_rocm_gguf_metadata_count", "yvex_rocm_gguf_tensor_count", "yvex_rocm_gguf_tensor_data_offset",
+                 "yvex_rocm_gguf_file_size"):
         getattr(lib, name).argtypes = [C.c_void_p]
         getattr(lib, name).restype = ULL
-    lib.yvex_gguf_alignment.argtypes = [C.c_void_p]
-    lib.yvex_gguf_alignment.restype = C.c_uint
-    lib.yvex_gguf_metadata_u64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(ULL)]
-    lib.yvex_gguf_metadata_f64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
-    lib.yvex_gguf_metadata_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(ULL)]
-    lib.yvex_gguf_tensor_at.argtypes = [C.c_void_p, ULL]
-    lib.yvex_gguf_tensor_at.restype = C.POINTER(GgufTensorInfo)
-    lib.yvex_gguf_tensor_find.argtypes = [C.c_void_p, C.c_char_p]
-    lib.yvex_gguf_tensor_find.restype = C.POINTER(GgufTensorInfo)
-    lib.yvex_backend_rocm_gguf_resident_load.argtypes = [C.c_void_p, C.c_void_p, ULL,
+    lib.yvex_rocm_gguf_alignment.argtypes = [C.c_void_p]
+    lib.yvex_rocm_gguf_alignment.restype = C.c_uint
+    lib.yvex_rocm_gguf_metadata_u64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(ULL)]
+    lib.yvex_rocm_gguf_metadata_f64.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
+    lib.yvex_rocm_gguf_metadata_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(ULL)]
+    lib.yvex_rocm_gguf_tensor_at.argtypes = [C.c_void_p, ULL]
+    lib.yvex_rocm_gguf_tensor_at.restype = C.POINTER(GgufTensorInfo)
+    lib.yvex_rocm_gguf_tensor_find.argtypes = [C.c_void_p, C.c_char_p]
+    lib.yvex_rocm_gguf_tensor_find.restype = C.POINTER(GgufTensorInfo)
+    lib.yvex_rocm_gguf_resident_load.argtypes = [C.c_void_p, C.c_void_p, ULL,
                                                          C.POINTER(C.POINTER(DeviceTensor)),
                                                          C.POINTER(C.c_void_p), C.POINTER(Error)]
-    lib.yvex_backend_rocm_gguf_weight_view.argtypes = [C.c_void_p, C.c_void_p, C.c_char_p,
+    lib.yvex_rocm_gguf_weight_view.argtypes = [C.c_void_p, C.c_void_p, C.c_char_p,
                                                        C.POINTER(WeightView), C.POINTER(Error)]
-    lib.yvex_backend_moe_begin.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.POINTER(LayerJob),
+    lib.yvex_rocm_backend_moe_begin.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.POINTER(LayerJob),
                                            C.POINTER(LayerResult), C.POINTER(Error)]
-    lib.yvex_backend_moe_add_expert.argtypes = [C.c_void_p, C.POINTER(WeightView), C.POINTER(WeightView),
+    lib.yvex_rocm_backend_moe_add_expert.argtypes = [C.c_void_p, C.POINTER(WeightView), C.POINTER(WeightView),
                                                 C.POINTER(WeightView), C.c_float, C.c_int, C.POINTER(Error)]
-    lib.yvex_backend_moe_finish.argtypes = [C.c_void_p, C.POINTER(LayerResult), C.POINTER(Error)]
-    lib.yvex_backend_moe_close.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
-    lib.yvex_backend_open.argtypes = [C.POINTER(C.c_void_p), C.POINTER(BackendOptions), C.POINTER(Error)]
-    lib.yvex_backend_close_checked.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
-    lib.yvex_backend_tensor_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),
+    lib.yvex_rocm_backend_moe_finish.argtypes = [C.c_void_p, C.POINTER(LayerResult), C.POINTER(Error)]
+    lib.yvex_rocm_backend_moe_close.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
+    lib.yvex_rocm_backend_open.argtypes = [C.POINTER(C.c_void_p), C.POINTER(BackendOptions), C.POINTER(Error)]
+    lib.yvex_rocm_backend_close_checked.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
+    lib.yvex_rocm_backend_tensor_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),
                                               C.POINTER(C.POINTER(DeviceTensor)), C.POINTER(Error)]
-    lib.yvex_backend_tensor_release.argtypes = [C.c_void_p, C.POINTER(C.POINTER(DeviceTensor)),
+    lib.yvex_rocm_backend_tensor_release.argtypes = [C.c_void_p, C.POINTER(C.POINTER(DeviceTensor)),
                                                 C.POINTER(Error)]
-    lib.yvex_backend_tensor_write.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), C.c_void_p, ULL,
+    lib.yvex_rocm_backend_tensor_write.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), C.c_void_p, ULL,
                                               C.POINTER(Error)]
-    lib.yvex_backend_tensor_read.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), C.c_void_p, ULL,
+    lib.yvex_rocm_backend_tensor_read.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), C.c_void_p, ULL,
                                              C.POINTER(Error)]
-    lib.yvex_backend_tensor_copy.argtypes = [C.c_void_p, C.POINTER(DeviceTensor),
+    lib.yvex_rocm_backend_tensor_copy.argtypes = [C.c_void_p, C.POINTER(DeviceTensor),
                                              C.POINTER(DeviceTensor), C.POINTER(Error)]
-    lib.yvex_backend_resident_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),
+    lib.yvex_rocm_backend_resident_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),
                                                 C.POINTER(C.POINTER(DeviceTensor)),
                                                 C.POINTER(C.c_void_p), C.POINTER(Error)]
-    lib.yvex_backend_resident_attach.argtypes = [C.c_void_p, C.c_void_p, ULL, C.POINTER(DeviceTensor),
+    lib.yvex_rocm_backend_resident_attach.argtypes = [C.c_void_p, C.c_void_p, ULL, C.POINTER(DeviceTensor),
                                                  ULL, C.POINTER(Error)]
-    lib.yvex_backend_resident_detach.argtypes = [C.c_void_p, C.POINTER(Error)]
-    lib.yvex_backend_resident_resolve.argtypes = [C.c_void_p, C.c_void_p, ULL, C.POINTER(ULL)]
-    lib.yvex_backend_resident_prefetch.argtypes = [C.c_void_p, C.POINTER(DeviceTensor),
+    lib.yvex_rocm_backend_resident_detach.argtypes = [C.c_void_p, C.POINTER(Error)]
+    lib.yvex_rocm_backend_resident_resolve.argtypes = [C.c_void_p, C.c_void_p, ULL, C.POINTER(ULL)]
+    lib.yvex_rocm_backend_resident_prefetch.argtypes = [C.c_void_p, C.POINTER(DeviceTensor),
                                                    C.POINTER(ULL), C.POINTER(Error)]
-    lib.yvex_backend_workspace_attach.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), ULL,
+    lib.yvex_rocm_backend_workspace_attach.argtypes = [C.c_void_p, C.POINTER(DeviceTensor), ULL,
                                                   C.POINTER(Error)]
-    lib.yvex_backend_workspace_detach.argtypes = [C.c_void_p]
-    lib.yvex_backend_workspace_acquire.argtypes = [C.c_void_p, ULL, ULL, C.POINTER(ULL)]
-    lib.yvex_backend_query_capability.argtypes = [C.c_void_p, C.c_int, C.POINTER(CapabilityResult),
+    lib.yvex_rocm_backend_workspace_detach.argtypes = [C.c_void_p]
+    lib.yvex_rocm_backend_workspace_acquire.argtypes = [C.c_void_p, ULL, ULL, C.POINTER(ULL)]
+    lib.yvex_rocm_backend_query_capability.argtypes = [C.c_void_p, C.c_int, C.POINTER(CapabilityResult),
                                                   C.POINTER(Error)]
-    lib.yvex_backend_get_memory_stats.argtypes = [C.c_void_p, C.POINTER(MemoryStats), C.POINTER(Error)]
-    lib.yvex_backend_sync.argtypes = [C.c_void_p, C.POINTER(Error)]
-    lib.yvex_backend_kind_of.argtypes = [C.c_void_p]
-    lib.yvex_backend_status_of.argtypes = [C.c_void_p]
-    lib.yvex_backend_tensor_owned_by.argtypes = [C.c_void_p, C.POINTER(DeviceTensor)]
-    lib.yvex_backend_rocm_encoded_matvec.argtypes = [
+    lib.yvex_rocm_backend_get_memory_stats.argtypes = [C.c_void_p, C.POINTER(MemoryStats), C.POINTER(Error)]
+    lib.yvex_rocm_backend_sync.argtypes = [C.c_void_p, C.POINTER(Error)]
+    lib.yvex_rocm_backend_kind_of.argtypes = [C.c_void_p]
+    lib.yvex_rocm_backend_status_of.argtypes = [C.c_void_p]
+    lib.yvex_rocm_backend_tensor_owned_by.argtypes = [C.c_void_p, C.POINTER(DeviceTensor)]
+    lib.yvex_rocm_encoded_matvec.argtypes = [
         C.c_void_p, C.c_void_p, ULL, C.c_uint, ULL, ULL, ULL, ULL, C.POINTER(DeviceTensor),
         C.POINTER(DeviceTensor), ULL, C.POINTER(DeviceTensor), C.POINTER(DeviceTensor), C.c_int,
         C.POINTER(OperationFacts), C.POINTER(Error)]
-    lib.yvex_backend_rocm_encoded_gather.argtypes = [
+    lib.yvex_rocm_encoded_gather.argtypes = [
         C.c_void_p, C.c_void_p, ULL, C.c_uint, ULL, ULL, ULL, C.c_void_p, ULL,
         C.POINTER(DeviceTensor), C.POINTER(OperationFacts), C.POINTER(Error)]
-    lib.yvex_backend_rocm_select_greedy_rows.argtypes = [
+    lib.yvex_rocm_select_greedy_rows.argtypes = [
         C.c_void_p, C.POINTER(DeviceTensor), ULL, ULL, C.c_void_p, C.c_void_p, C.c_void_p,
         C.POINTER(OperationFacts), C.POINTER(Error)]
-    lib.yvex_expert_worklist_build.argtypes = [C.c_void_p, C.c_void_p, ULL, ULL, ULL,
+    lib.yvex_rocm_expert_worklist_build.argtypes = [C.c_void_p, C.c_void_p, ULL, ULL, ULL,
                                                C.POINTER(WorklistStorage),
                                                C.POINTER(WorklistObservation), C.POINTER(Error)]
     return lib

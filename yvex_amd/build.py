@@ -65,7 +65,9 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
             if verbose and warnings:
                 print(warnings, file=sys.stderr)
     objs = [t[0] for t in tasks]
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-lm", "-lpthread"])
+    # only the declared entry points leave the library, and its own calls bind inside it
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-lm", "-lpthread",
+          f"-Wl,--version-script={os.path.join(CSRC, 'exports.map')}", "-Wl,-Bsymbolic"])
     return LIB
 
 

@@ -15,7 +15,7 @@ static unsigned long long next_owner_id = 1ull;
 
 int yvex_rocm_refuse(yvex_error *err, yvex_status code, const char *where, const char *message)
 {
-    yvex_error_set(err, code, where, message);
+    yvex_rocm_error_set(err, code, where, message);
     return code;
 }
 
@@ -25,17 +25,18 @@ int yvex_rocm_seam(const char *name)
     return value && value[0] && strcmp(value, "0") != 0;
 }
 
-int yvex_rocm_tensor_owner_is(const yvex_backend *backend, const yvex_device_tensor *tensor)
+int yvex_rocm_tensor_owner_is(const yvex_rocm_backend *backend, const yvex_device_tensor *tensor)
 {
-    return backend && tensor && tensor->owner == backend && tensor->owner_id == backend->owner_id;
+    return backend && tensor && (const void *)tensor->owner == backend->public_owner &&
+           tensor->owner_id == backend->owner_id;
 }
 
-int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_tensor *tensor)
+int yvex_rocm_backend_tensor_owned_by(const yvex_rocm_backend *backend, const yvex_device_tensor *tensor)
 {
     return yvex_rocm_tensor_owner_is(backend, tensor);
 }
 
-void yvex_rocm_workspace_reset(yvex_backend *backend)
+void yvex_rocm_workspace_reset(yvex_rocm_backend *backend)
 {
     if (backend) backend->workspace_cursor = 0ull;
 }
@@ -48,7 +49,7 @@ int yvex_rocm_launch_result(int rc, const char *where, yvex_error *err)
     return yvex_rocm_refuse(err, (yvex_status)rc, where, "kernel launch refused the operand geometry");
 }
 
-int yvex_rocm_require_kernels(const yvex_backend *backend, const char *where, yvex_error *err)
+int yvex_rocm_require_kernels(const yvex_rocm_backend *backend, const char *where, yvex_error *err)
 {
     if (!backend || backend->status == YVEX_BACKEND_STATUS_FAILED)
         return yvex_rocm_refuse(err, YVEX_ERR_STATE, where, "backend is failed or closing");
@@ -58,13 +59,13 @@ int yvex_rocm_require_kernels(const yvex_backend *backend, const char *where, yv
     return YVEX_OK;
 }
 
-int yvex_rocm_status_reset(yvex_backend *backend, const char *where, yvex_error *err)
+int yvex_rocm_status_reset(yvex_rocm_backend *backend, const char *where, yvex_error *err)
 {
     return yvex_rocm_launch_result(yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream),
                                    where, err);
 }
 
-int yvex_rocm_finish(yvex_backend *backend, const char *where, int *device_status, yvex_error *err)
+int yvex_rocm_finish(yvex_rocm_backend *backend, const char *where, int *device_status, yvex_error *err)
 {
     int rc;
     *device_status = 0;
@@ -80,9 +81,9 @@ int yvex_rocm_finish(yvex_backend *backend, const char *where, int *device_statu
     return YVEX_OK;
 }
 
-int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, yvex_error *err)
+int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *options, yvex_error *err)
 {
-    yvex_backend *backend;
+    yvex_rocm_backend *backend;
     int device = 0, host_only;
     if (out) *out = NULL;
     if (!out || !options)
@@ -103,10 +104,11 @@ int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, y
     if (!host_only && device >= yvex_hip_device_count())
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.open",
                                 "no rocm device is available: device-unavailable");
-    backend = (yvex_backend *)calloc(1, sizeof(*backend));
+    backend = (yvex_rocm_backend *)calloc(1, sizeof(*backend));
     if (!backend) return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "backend.open", "out of host memory");
     backend->kind = YVEX_BACKEND_KIND_ROCM;
     backend->owner_id = next_owner_id++;
+    backend->public_owner = backend;
     backend->device_index = device;
     backend->host_only = host_only;
     backend->memory.memory_limit_bytes = options->memory_limit_bytes;
@@ -134,17 +136,17 @@ int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, y
     backend->status = backend->kernels_available ? YVEX_BACKEND_STATUS_READY
                                                  : YVEX_BACKEND_STATUS_CONTEXT_READY;
     *out = backend;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_close_checked(yvex_backend **backend_ref, yvex_error *err)
+int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend_ref, yvex_error *err)
 {
-    yvex_backend *backend = backend_ref ? *backend_ref : NULL;
+    yvex_rocm_backend *backend = backend_ref ? *backend_ref : NULL;
     if (!backend_ref)
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.close", "owner is required");
     if (!backend) {
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
         return YVEX_OK;
     }
     if (backend->live_tensors)
@@ -165,46 +167,58 @@ int yvex_backend_close_checked(yvex_backend **backend_ref, yvex_error *err)
     }
     free(backend);
     *backend_ref = NULL;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-yvex_backend_kind yvex_backend_kind_of(const yvex_backend *backend)
+int yvex_rocm_backend_bind_owner(yvex_rocm_backend *backend, const void *owner, yvex_error *err)
+{
+    if (!backend || !owner)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.bind", "backend and owner are required");
+    if (backend->live_tensors)
+        return yvex_rocm_refuse(err, YVEX_ERR_STATE, "backend.bind",
+                                "the owner is bound before the first tensor is allocated");
+    backend->public_owner = owner;
+    yvex_rocm_error_clear(err);
+    return YVEX_OK;
+}
+
+yvex_backend_kind yvex_rocm_backend_kind_of(const yvex_rocm_backend *backend)
 {
     return backend ? backend->kind : YVEX_BACKEND_KIND_CPU;
 }
 
-yvex_backend_status yvex_backend_status_of(const yvex_backend *backend)
+yvex_backend_status yvex_rocm_backend_status_of(const yvex_rocm_backend *backend)
 {
     return backend ? backend->status : YVEX_BACKEND_STATUS_FAILED;
 }
 
-int yvex_backend_get_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
+int yvex_rocm_backend_get_memory_stats(const yvex_rocm_backend *backend, yvex_backend_memory_stats *out,
                                   yvex_error *err)
 {
     if (!backend || !out)
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.memory", "owner and output required");
     *out = backend->memory;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_sync(yvex_backend *backend, yvex_error *err)
+int yvex_rocm_backend_sync(yvex_rocm_backend *backend, yvex_error *err)
 {
     if (!backend) return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.sync", "owner is required");
     if (backend->host_only) {
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
         return YVEX_OK;
     }
     if (yvex_rocm_seam("YVEX_TEST_ROCM_SYNC_FAILURE") || yvex_hip_stream_sync(backend->stream) != 0) {
         backend->status = YVEX_BACKEND_STATUS_FAILED;
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.sync", "stream synchronisation failed");
     }
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_query_capability(const yvex_backend *backend,
+int yvex_rocm_backend_query_capability(const yvex_rocm_backend *backend,
                                   yvex_backend_operation_variant variant,
                                   yvex_backend_capability_result *out, yvex_error *err)
 {
@@ -237,20 +251,20 @@ int yvex_backend_query_capability(const yvex_backend *backend,
         out->state = YVEX_BACKEND_CAPABILITY_SUPPORTED;
         out->function_available = 1;
     }
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
 /* ---- tensors -------------------------------------------------------------------------------- */
 
-static int memory_can_add(const yvex_backend *backend, unsigned long long bytes)
+static int memory_can_add(const yvex_rocm_backend *backend, unsigned long long bytes)
 {
     const yvex_backend_memory_stats *m = &backend->memory;
     if (bytes > ULLONG_MAX - m->allocated_bytes) return 0;
     return !m->memory_limit_bytes || m->allocated_bytes + bytes <= m->memory_limit_bytes;
 }
 
-static int tensor_create(yvex_backend *backend, const yvex_backend_tensor_desc *desc, int resident,
+static int tensor_create(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc, int resident,
                          yvex_device_tensor **out, const char *where, yvex_error *err)
 {
     yvex_device_tensor *tensor;
@@ -279,7 +293,7 @@ static int tensor_create(yvex_backend *backend, const yvex_backend_tensor_desc *
         free(tensor);
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where, "device allocation failed");
     }
-    tensor->owner = backend;
+    tensor->owner = (yvex_rocm_backend *)backend->public_owner;
     tensor->owner_id = backend->owner_id;
     if (desc->name) {
         size_t n = strlen(desc->name) + 1u;
@@ -302,24 +316,24 @@ static int tensor_create(yvex_backend *backend, const yvex_backend_tensor_desc *
         backend->memory.peak_allocated_bytes = backend->memory.allocated_bytes;
     backend->live_tensors++;
     *out = tensor;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+int yvex_rocm_backend_tensor_alloc(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc,
                               yvex_device_tensor **out, yvex_error *err)
 {
     return tensor_create(backend, desc, 0, out, "backend.tensor.alloc", err);
 }
 
-int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor_ref,
+int yvex_rocm_backend_tensor_release(yvex_rocm_backend *backend, yvex_device_tensor **tensor_ref,
                                 yvex_error *err)
 {
     yvex_device_tensor *tensor = tensor_ref ? *tensor_ref : NULL;
     if (!backend || !tensor_ref)
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.tensor.release", "owner is required");
     if (!tensor) {
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
         return YVEX_OK;
     }
     if (!yvex_rocm_tensor_owner_is(backend, tensor))
@@ -328,8 +342,8 @@ int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tens
     if (yvex_rocm_seam("YVEX_TEST_ROCM_CLEANUP_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.tensor.release",
                                 "release failed (test seam); the owner keeps the tensor");
-    if (backend->resident_device_tensor == tensor) yvex_backend_resident_detach(backend, NULL);
-    if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
+    if (backend->resident_device_tensor == tensor) yvex_rocm_backend_resident_detach(backend, NULL);
+    if (backend->workspace_device_tensor == tensor) yvex_rocm_backend_workspace_detach(backend);
     if (backend->host_only) {
         free(tensor->backend_allocation);
     } else {
@@ -344,11 +358,11 @@ int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tens
     free(tensor->name);
     free(tensor);
     *tensor_ref = NULL;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-static int rw_validate(const char *where, const yvex_backend *backend, const yvex_device_tensor *tensor,
+static int rw_validate(const char *where, const yvex_rocm_backend *backend, const yvex_device_tensor *tensor,
                        const void *host, unsigned long long len, yvex_error *err)
 {
     if (!backend || !tensor || !host)
@@ -362,7 +376,7 @@ static int rw_validate(const char *where, const yvex_backend *backend, const yve
     return YVEX_OK;
 }
 
-int yvex_backend_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, const void *src,
+int yvex_rocm_backend_tensor_write(yvex_rocm_backend *backend, yvex_device_tensor *tensor, const void *src,
                               unsigned long long len, yvex_error *err)
 {
     int rc = rw_validate("backend.tensor.write", backend, tensor, src, len, err);
@@ -372,11 +386,11 @@ int yvex_backend_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor,
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.tensor.write", yvex_hip_last_error());
     backend->memory.h2d_bytes += len;
     tensor->is_written = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *tensor, void *dst,
+int yvex_rocm_backend_tensor_read(yvex_rocm_backend *backend, const yvex_device_tensor *tensor, void *dst,
                              unsigned long long len, yvex_error *err)
 {
     int rc = rw_validate("backend.tensor.read", backend, tensor, dst, len, err);
@@ -387,11 +401,11 @@ int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *te
     else if (yvex_hip_memcpy_d2h(dst, tensor->data, len, backend->stream) != 0)
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.tensor.read", yvex_hip_last_error());
     backend->memory.d2h_bytes += len;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
+int yvex_rocm_backend_tensor_copy(yvex_rocm_backend *backend, yvex_device_tensor *dst,
                              const yvex_device_tensor *src, yvex_error *err)
 {
     if (!backend || !dst || !src)
@@ -405,13 +419,13 @@ int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
              yvex_hip_stream_sync(backend->stream) != 0)
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.tensor.copy", yvex_hip_last_error());
     dst->is_written = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
 /* ---- resident arena -------------------------------------------------------------------------- */
 
-int yvex_backend_resident_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+int yvex_rocm_backend_resident_alloc(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc,
                                 yvex_device_tensor **out, unsigned char **host, yvex_error *err)
 {
     int rc;
@@ -422,7 +436,7 @@ int yvex_backend_resident_alloc(yvex_backend *backend, const yvex_backend_tensor
     return rc;
 }
 
-static int resident_upload(yvex_backend *backend, const yvex_device_tensor *tensor,
+static int resident_upload(yvex_rocm_backend *backend, const yvex_device_tensor *tensor,
                            unsigned long long offset, unsigned long long bytes, const char *where,
                            yvex_error *err)
 {
@@ -433,7 +447,7 @@ static int resident_upload(yvex_backend *backend, const yvex_device_tensor *tens
     return YVEX_OK;
 }
 
-int yvex_backend_resident_prefetch(yvex_backend *backend, yvex_device_tensor *tensor,
+int yvex_rocm_backend_resident_prefetch(yvex_rocm_backend *backend, yvex_device_tensor *tensor,
                                    unsigned long long *prefetched_bytes, yvex_error *err)
 {
     int rc;
@@ -446,11 +460,11 @@ int yvex_backend_resident_prefetch(yvex_backend *backend, yvex_device_tensor *te
     if (rc != YVEX_OK) return rc;
     tensor->is_written = 1;
     *prefetched_bytes = tensor->resident_bytes;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_resident_attach(yvex_backend *backend, const unsigned char *host_base,
+int yvex_rocm_backend_resident_attach(yvex_rocm_backend *backend, const unsigned char *host_base,
                                  unsigned long long bytes, const yvex_device_tensor *tensor,
                                  unsigned long long generation, yvex_error *err)
 {
@@ -474,11 +488,11 @@ int yvex_backend_resident_attach(yvex_backend *backend, const unsigned char *hos
     backend->resident_device_tensor = tensor;
     backend->resident_device_address = (unsigned long long)(uintptr_t)(tensor->data + offset);
     backend->resident_generation = generation;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_resident_detach(yvex_backend *backend, yvex_error *err)
+int yvex_rocm_backend_resident_detach(yvex_rocm_backend *backend, yvex_error *err)
 {
     if (backend) {
         backend->resident_host_base = NULL;
@@ -487,11 +501,11 @@ int yvex_backend_resident_detach(yvex_backend *backend, yvex_error *err)
         backend->resident_device_address = 0ull;
         backend->resident_generation = 0ull;
     }
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_resident_resolve(const yvex_backend *backend, const unsigned char *host,
+int yvex_rocm_backend_resident_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
                                   unsigned long long bytes, unsigned long long *device_address)
 {
     uintptr_t base, pointer;
@@ -511,16 +525,16 @@ int yvex_backend_resident_resolve(const yvex_backend *backend, const unsigned ch
     return YVEX_BACKEND_RESIDENT_HIT;
 }
 
-int yvex_rocm_resolve(const yvex_backend *backend, const unsigned char *host,
+int yvex_rocm_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
                       unsigned long long bytes, unsigned long long *device_address)
 {
-    return yvex_backend_resident_resolve(backend, host, bytes, device_address) ==
+    return yvex_rocm_backend_resident_resolve(backend, host, bytes, device_address) ==
            YVEX_BACKEND_RESIDENT_HIT;
 }
 
 /* ---- workspace -------------------------------------------------------------------------------- */
 
-int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *tensor,
+int yvex_rocm_backend_workspace_attach(yvex_rocm_backend *backend, const yvex_device_tensor *tensor,
                                   unsigned long long bytes, yvex_error *err)
 {
     if (!backend || !tensor || !bytes || !yvex_rocm_tensor_owner_is(backend, tensor) ||
@@ -530,18 +544,18 @@ int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tenso
     backend->workspace_device_tensor = tensor;
     backend->workspace_bytes = bytes;
     backend->workspace_cursor = 0ull;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-void yvex_backend_workspace_detach(yvex_backend *backend)
+void yvex_rocm_backend_workspace_detach(yvex_rocm_backend *backend)
 {
     if (!backend) return;
     backend->workspace_device_tensor = NULL;
     backend->workspace_bytes = backend->workspace_cursor = 0ull;
 }
 
-int yvex_backend_workspace_acquire(yvex_backend *backend, unsigned long long bytes,
+int yvex_rocm_backend_workspace_acquire(yvex_rocm_backend *backend, unsigned long long bytes,
                                    unsigned long long alignment, unsigned long long *device_address)
 {
     unsigned long long base, start;

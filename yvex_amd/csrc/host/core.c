@@ -9,7 +9,7 @@
 
 #include "yvex_rocm.h"
 
-const char *yvex_status_name(yvex_status status)
+const char *yvex_rocm_status_name(yvex_status status)
 {
     switch (status) {
     case YVEX_OK: return "ok";
@@ -28,12 +28,12 @@ const char *yvex_status_name(yvex_status status)
     }
 }
 
-void yvex_error_clear(yvex_error *err)
+void yvex_rocm_error_clear(yvex_error *err)
 {
     if (err) memset(err, 0, sizeof(*err));
 }
 
-void yvex_error_set(yvex_error *err, yvex_status code, const char *where, const char *message)
+void yvex_rocm_error_set(yvex_error *err, yvex_status code, const char *where, const char *message)
 {
     if (!err) return;
     err->code = code;
@@ -41,14 +41,14 @@ void yvex_error_set(yvex_error *err, yvex_status code, const char *where, const 
     snprintf(err->message, sizeof(err->message), "%s", message ? message : "");
 }
 
-int yvex_error_is_set(const yvex_error *err) { return err && err->code != YVEX_OK; }
-yvex_status yvex_error_code(const yvex_error *err) { return err ? err->code : YVEX_OK; }
+int yvex_rocm_error_is_set(const yvex_error *err) { return err && err->code != YVEX_OK; }
+yvex_status yvex_rocm_error_code(const yvex_error *err) { return err ? err->code : YVEX_OK; }
 
 #define ADMIT YVEX_GGUF_QTYPE_IDENTITY_ADMITTED
 #define GONE YVEX_GGUF_QTYPE_IDENTITY_REMOVED
 #define LATER YVEX_GGUF_QTYPE_IDENTITY_OUTSIDE_BASELINE
 
-static const yvex_gguf_qtype_geometry geometry_table[] = {
+static const yvex_rocm_qtype_geometry geometry_table[] = {
     {0, "F32", ADMIT, 1, 4},        {1, "F16", ADMIT, 1, 2},         {2, "Q4_0", ADMIT, 32, 18},
     {3, "Q4_1", ADMIT, 32, 20},     {4, "Q4_2", GONE, 0, 0},         {5, "Q4_3", GONE, 0, 0},
     {6, "Q5_0", ADMIT, 32, 22},     {7, "Q5_1", ADMIT, 32, 24},      {8, "Q8_0", ADMIT, 32, 34},
@@ -66,21 +66,21 @@ static const yvex_gguf_qtype_geometry geometry_table[] = {
     {42, "Q2_0", LATER, 64, 18},
 };
 
-const yvex_gguf_qtype_geometry *yvex_gguf_qtype_geometry_find(unsigned int qtype)
+const yvex_rocm_qtype_geometry *yvex_rocm_gguf_qtype_geometry_find(unsigned int qtype)
 {
     if (qtype > YVEX_GGUF_QTYPE_ABI_UPSTREAM_MAX_ID) return NULL;
     return &geometry_table[qtype];
 }
 
 /* {known, storage, decoder, cpu, device, extension, refusal} per ID. */
-#define FULL(q) {q, 1, 1, 1, 1, 1, 0, YVEX_QUANT_REFUSAL_NONE}
-#define CPU_ONLY(q) {q, 1, 1, 1, 1, 0, 0, YVEX_QUANT_REFUSAL_NONE}
-#define EXTENDED(q) {q, 1, 1, 1, 1, 1, 1, YVEX_QUANT_REFUSAL_NONE}
-#define NO_CODEC(q) {q, 1, 1, 0, 0, 0, 0, YVEX_QUANT_REFUSAL_ENCODER_UNAVAILABLE}
-#define REMOVED(q) {q, 1, 0, 0, 0, 0, 0, YVEX_QUANT_REFUSAL_REMOVED_IDENTITY}
-#define OUTSIDE(q) {q, 1, 0, 0, 0, 0, 0, YVEX_QUANT_REFUSAL_OUTSIDE_PINNED_BASELINE}
+#define FULL(q) {q, 1, 1, 1, 1, 1, 0, YVEX_ROCM_QUANT_REFUSAL_NONE}
+#define CPU_ONLY(q) {q, 1, 1, 1, 1, 0, 0, YVEX_ROCM_QUANT_REFUSAL_NONE}
+#define EXTENDED(q) {q, 1, 1, 1, 1, 1, 1, YVEX_ROCM_QUANT_REFUSAL_NONE}
+#define NO_CODEC(q) {q, 1, 1, 0, 0, 0, 0, YVEX_ROCM_QUANT_REFUSAL_ENCODER_UNAVAILABLE}
+#define REMOVED(q) {q, 1, 0, 0, 0, 0, 0, YVEX_ROCM_QUANT_REFUSAL_REMOVED_IDENTITY}
+#define OUTSIDE(q) {q, 1, 0, 0, 0, 0, 0, YVEX_ROCM_QUANT_REFUSAL_OUTSIDE_PINNED_BASELINE}
 
-static const yvex_quant_numeric_capability capability_table[] = {
+static const yvex_rocm_numeric_capability capability_table[] = {
     FULL(0),      FULL(1),      NO_CODEC(2),  NO_CODEC(3),  REMOVED(4),   REMOVED(5),
     NO_CODEC(6),  NO_CODEC(7),  FULL(8),      NO_CODEC(9),  FULL(10),     NO_CODEC(11),
     EXTENDED(12), NO_CODEC(13), NO_CODEC(14), NO_CODEC(15), FULL(16),     NO_CODEC(17),
@@ -94,7 +94,7 @@ static const yvex_quant_numeric_capability capability_table[] = {
 _Static_assert(sizeof(geometry_table) / sizeof(geometry_table[0]) == 43u, "IDs 0 through 42");
 _Static_assert(sizeof(capability_table) / sizeof(capability_table[0]) == 43u, "IDs 0 through 42");
 
-const yvex_quant_numeric_capability *yvex_quant_numeric_capability_at(unsigned int qtype)
+const yvex_rocm_numeric_capability *yvex_rocm_quant_numeric_capability_at(unsigned int qtype)
 {
     if (qtype >= sizeof(capability_table) / sizeof(capability_table[0])) return NULL;
     return &capability_table[qtype];

@@ -37,7 +37,7 @@ typedef struct {
     char *text;              /* strings (NUL-terminated copy) */
 } gguf_entry;
 
-struct yvex_gguf {
+struct yvex_rocm_gguf {
     FILE *file;
     unsigned long long file_size, cursor;
     unsigned int version, alignment;
@@ -52,7 +52,7 @@ static int fail(yvex_error *err, int code, const char *where, const char *messag
     return yvex_rocm_refuse(err, (yvex_status)code, where, message);
 }
 
-static int take(yvex_gguf *g, void *out, unsigned long long bytes, const char *where, yvex_error *err)
+static int take(yvex_rocm_gguf *g, void *out, unsigned long long bytes, const char *where, yvex_error *err)
 {
     if (bytes > g->file_size - g->cursor) return fail(err, YVEX_ERR_BOUNDS, where, "GGUF input is truncated");
     if (bytes && fread(out, 1u, (size_t)bytes, g->file) != (size_t)bytes)
@@ -61,7 +61,7 @@ static int take(yvex_gguf *g, void *out, unsigned long long bytes, const char *w
     return YVEX_OK;
 }
 
-static int skip(yvex_gguf *g, unsigned long long bytes, const char *where, yvex_error *err)
+static int skip(yvex_rocm_gguf *g, unsigned long long bytes, const char *where, yvex_error *err)
 {
     if (bytes > g->file_size - g->cursor) return fail(err, YVEX_ERR_BOUNDS, where, "GGUF input is truncated");
     if (bytes && fseeko(g->file, (off_t)(g->cursor + bytes), SEEK_SET) != 0)
@@ -77,7 +77,7 @@ static unsigned long long le(const unsigned char *b, unsigned int n)
     return v;
 }
 
-static int take_u32(yvex_gguf *g, unsigned int *out, const char *where, yvex_error *err)
+static int take_u32(yvex_rocm_gguf *g, unsigned int *out, const char *where, yvex_error *err)
 {
     unsigned char b[4];
     int rc = take(g, b, 4u, where, err);
@@ -85,7 +85,7 @@ static int take_u32(yvex_gguf *g, unsigned int *out, const char *where, yvex_err
     return rc;
 }
 
-static int take_u64(yvex_gguf *g, unsigned long long *out, const char *where, yvex_error *err)
+static int take_u64(yvex_rocm_gguf *g, unsigned long long *out, const char *where, yvex_error *err)
 {
     unsigned char b[8];
     int rc = take(g, b, 8u, where, err);
@@ -94,7 +94,7 @@ static int take_u64(yvex_gguf *g, unsigned long long *out, const char *where, yv
 }
 
 /* Length-prefixed string; keep = 0 skips the bytes. Embedded NUL bytes are refused in kept text. */
-static int take_string(yvex_gguf *g, char **out, unsigned long long *len, unsigned long long limit,
+static int take_string(yvex_rocm_gguf *g, char **out, unsigned long long *len, unsigned long long limit,
                        int keep, const char *where, yvex_error *err)
 {
     unsigned long long n;
@@ -128,7 +128,7 @@ static unsigned int scalar_bytes(unsigned int type)
     }
 }
 
-static int walk_array(yvex_gguf *g, unsigned int depth, yvex_error *err)
+static int walk_array(yvex_rocm_gguf *g, unsigned int depth, yvex_error *err)
 {
     unsigned int element;
     unsigned long long count, i;
@@ -175,7 +175,7 @@ static int key_valid(const char *key, unsigned long long len)
     return !segment_start && !previous_underscore;
 }
 
-static int parse_metadata(yvex_gguf *g, yvex_error *err)
+static int parse_metadata(yvex_rocm_gguf *g, yvex_error *err)
 {
     unsigned long long i, j;
     if (g->metadata_count > GGUF_MAX_ENTRIES)
@@ -219,7 +219,7 @@ static int parse_metadata(yvex_gguf *g, yvex_error *err)
     return YVEX_OK;
 }
 
-static const gguf_entry *find_entry(const yvex_gguf *g, const char *key)
+static const gguf_entry *find_entry(const yvex_rocm_gguf *g, const char *key)
 {
     unsigned long long i;
     for (i = 0ull; g && key && i < g->metadata_count; ++i)
@@ -231,7 +231,7 @@ static const gguf_entry *find_entry(const yvex_gguf *g, const char *key)
 static int tensor_storage(unsigned int qtype, const unsigned long long *dims, unsigned int rank,
                           unsigned long long *bytes)
 {
-    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(qtype);
+    const yvex_rocm_qtype_geometry *geometry = yvex_rocm_gguf_qtype_geometry_find(qtype);
     unsigned long long rows = 1ull, row_bytes;
     unsigned int d;
     if (!geometry || !geometry->block_size || !geometry->bytes_per_block) return YVEX_ERR_UNSUPPORTED;
@@ -257,7 +257,7 @@ static int by_name_compare(const void *a, const void *b)
     return strcmp(((const named_index *)a)->name, ((const named_index *)b)->name);
 }
 
-static int parse_tensors(yvex_gguf *g, yvex_error *err)
+static int parse_tensors(yvex_rocm_gguf *g, yvex_error *err)
 {
     unsigned long long i, remainder;
     unsigned int d;
@@ -292,7 +292,7 @@ static int parse_tensors(yvex_gguf *g, yvex_error *err)
                         rc == YVEX_ERR_UNSUPPORTED ? "GGUF tensor qtype has no storage geometry here"
                         : rc == YVEX_ERR_FORMAT ? "GGUF tensor row is not a whole number of blocks"
                                                 : "GGUF tensor storage extent overflows");
-        t->ggml_type_name = yvex_gguf_qtype_geometry_find(t->ggml_type)->name;
+        t->ggml_type_name = yvex_rocm_gguf_qtype_geometry_find(t->ggml_type)->name;
         rc = take_u64(g, &t->relative_offset, "gguf.tensor.offset", err);
         if (rc != YVEX_OK) return rc;
         if (t->relative_offset % g->alignment)
@@ -328,19 +328,19 @@ static int parse_tensors(yvex_gguf *g, yvex_error *err)
     return YVEX_OK;
 }
 
-int yvex_gguf_open_path(yvex_gguf **out, const char *path, yvex_error *err)
+int yvex_rocm_gguf_open_path(yvex_rocm_gguf **out, const char *path, yvex_error *err)
 {
-    yvex_gguf *g;
+    yvex_rocm_gguf *g;
     unsigned char header[24];
     const gguf_entry *alignment;
     int rc;
     if (out) *out = NULL;
-    if (!out || !path) return fail(err, YVEX_ERR_INVALID_ARG, "yvex_gguf_open_path", "output and path are required");
-    g = (yvex_gguf *)calloc(1u, sizeof(*g));
-    if (!g) return fail(err, YVEX_ERR_NOMEM, "yvex_gguf_open_path", "out of host memory");
+    if (!out || !path) return fail(err, YVEX_ERR_INVALID_ARG, "yvex_rocm_gguf_open_path", "output and path are required");
+    g = (yvex_rocm_gguf *)calloc(1u, sizeof(*g));
+    if (!g) return fail(err, YVEX_ERR_NOMEM, "yvex_rocm_gguf_open_path", "out of host memory");
     g->file = fopen(path, "rb");
     if (!g->file || fseeko(g->file, 0, SEEK_END) != 0 || ftello(g->file) < 0 || fseeko(g->file, 0, SEEK_SET) != 0) {
-        rc = fail(err, YVEX_ERR_IO, "yvex_gguf_open_path", "GGUF file cannot be opened");
+        rc = fail(err, YVEX_ERR_IO, "yvex_rocm_gguf_open_path", "GGUF file cannot be opened");
         goto failed;
     }
     fseeko(g->file, 0, SEEK_END);
@@ -350,12 +350,12 @@ int yvex_gguf_open_path(yvex_gguf **out, const char *path, yvex_error *err)
     rc = take(g, header, sizeof(header), "gguf.header", err);
     if (rc != YVEX_OK) goto failed;
     if ((unsigned int)le(header, 4u) != GGUF_MAGIC) {
-        rc = fail(err, YVEX_ERR_FORMAT, "yvex_gguf_open_path", "invalid GGUF magic");
+        rc = fail(err, YVEX_ERR_FORMAT, "yvex_rocm_gguf_open_path", "invalid GGUF magic");
         goto failed;
     }
     g->version = (unsigned int)le(header + 4, 4u);
     if (g->version != GGUF_VERSION) {
-        rc = fail(err, YVEX_ERR_UNSUPPORTED, "yvex_gguf_open_path", "unsupported GGUF container version");
+        rc = fail(err, YVEX_ERR_UNSUPPORTED, "yvex_rocm_gguf_open_path", "unsupported GGUF container version");
         goto failed;
     }
     g->tensor_count = le(header + 8, 8u);
@@ -373,14 +373,14 @@ int yvex_gguf_open_path(yvex_gguf **out, const char *path, yvex_error *err)
     rc = parse_tensors(g, err);
     if (rc != YVEX_OK) goto failed;
     *out = g;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 failed:
-    yvex_gguf_close(g);
+    yvex_rocm_gguf_close(g);
     return rc;
 }
 
-void yvex_gguf_close(yvex_gguf *g)
+void yvex_rocm_gguf_close(yvex_rocm_gguf *g)
 {
     unsigned long long i;
     if (!g) return;
@@ -396,18 +396,18 @@ void yvex_gguf_close(yvex_gguf *g)
     free(g);
 }
 
-unsigned long long yvex_gguf_tensor_count(const yvex_gguf *g) { return g ? g->tensor_count : 0ull; }
-unsigned long long yvex_gguf_metadata_count(const yvex_gguf *g) { return g ? g->metadata_count : 0ull; }
-unsigned long long yvex_gguf_tensor_data_offset(const yvex_gguf *g) { return g ? g->tensor_data_offset : 0ull; }
-unsigned int yvex_gguf_alignment(const yvex_gguf *g) { return g ? g->alignment : 0u; }
-unsigned long long yvex_gguf_file_size(const yvex_gguf *g) { return g ? g->file_size : 0ull; }
+unsigned long long yvex_rocm_gguf_tensor_count(const yvex_rocm_gguf *g) { return g ? g->tensor_count : 0ull; }
+unsigned long long yvex_rocm_gguf_metadata_count(const yvex_rocm_gguf *g) { return g ? g->metadata_count : 0ull; }
+unsigned long long yvex_rocm_gguf_tensor_data_offset(const yvex_rocm_gguf *g) { return g ? g->tensor_data_offset : 0ull; }
+unsigned int yvex_rocm_gguf_alignment(const yvex_rocm_gguf *g) { return g ? g->alignment : 0u; }
+unsigned long long yvex_rocm_gguf_file_size(const yvex_rocm_gguf *g) { return g ? g->file_size : 0ull; }
 
-const yvex_gguf_tensor_info *yvex_gguf_tensor_at(const yvex_gguf *g, unsigned long long index)
+const yvex_gguf_tensor_info *yvex_rocm_gguf_tensor_at(const yvex_rocm_gguf *g, unsigned long long index)
 {
     return g && index < g->tensor_count ? &g->tensors[index] : NULL;
 }
 
-const yvex_gguf_tensor_info *yvex_gguf_tensor_find(const yvex_gguf *g, const char *name)
+const yvex_gguf_tensor_info *yvex_rocm_gguf_tensor_find(const yvex_rocm_gguf *g, const char *name)
 {
     unsigned long long low = 0ull, high;
     if (!g || !name) return NULL;
@@ -422,7 +422,7 @@ const yvex_gguf_tensor_info *yvex_gguf_tensor_find(const yvex_gguf *g, const cha
     return NULL;
 }
 
-int yvex_gguf_metadata_u64(const yvex_gguf *g, const char *key, unsigned long long *out)
+int yvex_rocm_gguf_metadata_u64(const yvex_rocm_gguf *g, const char *key, unsigned long long *out)
 {
     const gguf_entry *e = find_entry(g, key);
     if (!e || !out || e->type == T_STRING || e->type == T_ARRAY || e->type == T_F32 || e->type == T_F64)
@@ -434,7 +434,7 @@ int yvex_gguf_metadata_u64(const yvex_gguf *g, const char *key, unsigned long lo
     return YVEX_OK;
 }
 
-int yvex_gguf_metadata_f64(const yvex_gguf *g, const char *key, double *out)
+int yvex_rocm_gguf_metadata_f64(const yvex_rocm_gguf *g, const char *key, double *out)
 {
     const gguf_entry *e = find_entry(g, key);
     if (!e || !out || (e->type != T_F32 && e->type != T_F64)) return YVEX_ERR_FORMAT;
@@ -442,7 +442,7 @@ int yvex_gguf_metadata_f64(const yvex_gguf *g, const char *key, double *out)
     return YVEX_OK;
 }
 
-int yvex_gguf_metadata_string(const yvex_gguf *g, const char *key, const char **text, unsigned long long *len)
+int yvex_rocm_gguf_metadata_string(const yvex_rocm_gguf *g, const char *key, const char **text, unsigned long long *len)
 {
     const gguf_entry *e = find_entry(g, key);
     if (!e || !text || e->type != T_STRING) return YVEX_ERR_FORMAT;
@@ -453,7 +453,7 @@ int yvex_gguf_metadata_string(const yvex_gguf *g, const char *key, const char **
 
 /* ---- tensor data -> resident arena ---------------------------------------------------------- */
 
-int yvex_backend_rocm_gguf_resident_load(yvex_backend *backend, const yvex_gguf *g,
+int yvex_rocm_gguf_resident_load(yvex_rocm_backend *backend, const yvex_rocm_gguf *g,
                                          unsigned long long generation, yvex_device_tensor **arena,
                                          unsigned char **host_base, yvex_error *err)
 {
@@ -477,7 +477,7 @@ int yvex_backend_rocm_gguf_resident_load(yvex_backend *backend, const yvex_gguf 
     desc.rank = 1u;
     desc.dims[0] = bytes;
     desc.bytes = bytes;
-    rc = yvex_backend_resident_alloc(backend, &desc, arena, &host, err);
+    rc = yvex_rocm_backend_resident_alloc(backend, &desc, arena, &host, err);
     if (rc != YVEX_OK) return rc;
     if (fseeko(g->file, (off_t)g->tensor_data_offset, SEEK_SET) != 0) rc = YVEX_ERR_IO;
     while (rc == YVEX_OK && done < bytes) {
@@ -487,33 +487,33 @@ int yvex_backend_rocm_gguf_resident_load(yvex_backend *backend, const yvex_gguf 
         done += got;
     }
     if (rc != YVEX_OK) {
-        (void)yvex_backend_tensor_release(backend, arena, NULL);
+        (void)yvex_rocm_backend_tensor_release(backend, arena, NULL);
         return fail(err, YVEX_ERR_IO, "rocm.gguf.load", "GGUF tensor data cannot be read");
     }
-    rc = yvex_backend_resident_attach(backend, host, bytes, *arena, generation, err);
+    rc = yvex_rocm_backend_resident_attach(backend, host, bytes, *arena, generation, err);
     if (rc != YVEX_OK) {
-        (void)yvex_backend_tensor_release(backend, arena, NULL);
+        (void)yvex_rocm_backend_tensor_release(backend, arena, NULL);
         return rc;
     }
     *host_base = host;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_rocm_gguf_weight_view(const yvex_gguf *g, const unsigned char *host_base, const char *name,
+int yvex_rocm_gguf_weight_view(const yvex_rocm_gguf *g, const unsigned char *host_base, const char *name,
                                        yvex_moe_weight_view *view, yvex_error *err)
 {
-    const yvex_gguf_tensor_info *t = yvex_gguf_tensor_find(g, name);
-    const yvex_gguf_qtype_geometry *geometry;
-    const yvex_quant_numeric_capability *capability;
+    const yvex_gguf_tensor_info *t = yvex_rocm_gguf_tensor_find(g, name);
+    const yvex_rocm_qtype_geometry *geometry;
+    const yvex_rocm_numeric_capability *capability;
     unsigned long long rows = 1ull;
     unsigned int d;
     if (view) memset(view, 0, sizeof(*view));
     if (!g || !host_base || !name || !view)
         return fail(err, YVEX_ERR_INVALID_ARG, "rocm.gguf.view", "reader, arena base, name and view are required");
     if (!t) return fail(err, YVEX_ERR_FORMAT, "rocm.gguf.view", "GGUF tensor is not in the directory");
-    geometry = yvex_gguf_qtype_geometry_find(t->ggml_type);
-    capability = yvex_quant_numeric_capability_at(t->ggml_type);
+    geometry = yvex_rocm_gguf_qtype_geometry_find(t->ggml_type);
+    capability = yvex_rocm_quant_numeric_capability_at(t->ggml_type);
     if (!geometry || !capability || !capability->device_compute_available)
         return fail(err, YVEX_ERR_UNSUPPORTED, "rocm.gguf.view", "qtype has no device compute on this backend");
     if (!t->range_addressable)
@@ -528,6 +528,6 @@ int yvex_backend_rocm_gguf_weight_view(const yvex_gguf *g, const unsigned char *
     view->row_width = t->dims[0];
     view->row_count = rows;
     view->row_bytes = t->dims[0] / geometry->block_size * geometry->bytes_per_block;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }

@@ -90,7 +90,7 @@ static int layout_sections_of(const yvex_physical_execution_decision *decision, 
         s->total < decision->encoded_bytes)
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, where,
                                 "derived MoE layout differs from canonical geometry");
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
@@ -159,6 +159,6 @@ int yvex_rocm_moe_derived_layout_build(const yvex_physical_execution_decision *d
     memset(derived, 0, (size_t)storage_bytes);
     if (decision->canonical_qtype == YVEX_GGUF_QTYPE_IQ2_XXS) pack_iq2_xxs(&s, canonical, derived);
     else pack_q2_k(&s, decision->expert_count, canonical, derived);
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }

@@ -124,7 +124,7 @@ static int moe_layout(const yvex_moe_layer_plan *layer, unsigned long long rows,
     return 1;
 }
 
-static int moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned long long row_count,
+int yvex_rocm_moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned long long row_count,
                                   unsigned long long *bytes, yvex_error *err)
 {
     moe_ranges ranges;
@@ -133,7 +133,7 @@ static int moe_workspace_required(const yvex_moe_layer_plan *layer, unsigned lon
         return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.moe.workspace",
                                 "MoE layer geometry or row count is outside this backend's bounds");
     *bytes = ranges.total;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
@@ -197,12 +197,12 @@ static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight
 }
 
 /* Check one weight view against the geometry the plan implies and find its device address. */
-int yvex_rocm_moe_view_check(const yvex_backend *backend, const yvex_moe_weight_view *view,
+int yvex_rocm_moe_view_check(const yvex_rocm_backend *backend, const yvex_moe_weight_view *view,
                              unsigned long long row_width, unsigned long long row_count,
                              unsigned long long *device_address, int *resident, yvex_error *err)
 {
-    const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(view->qtype);
-    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(view->qtype);
+    const yvex_rocm_numeric_capability *capability = yvex_rocm_quant_numeric_capability_at(view->qtype);
+    const yvex_rocm_qtype_geometry *geometry = yvex_rocm_gguf_qtype_geometry_find(view->qtype);
     if (!capability || !geometry || !capability->device_compute_available)
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.weights",
                                 "qtype has no device compute on this backend");
@@ -228,7 +228,7 @@ int yvex_rocm_moe_view_check(const yvex_backend *backend, const yvex_moe_weight_
     return YVEX_OK;
 }
 
-static int view_resolve(const yvex_backend *backend, const yvex_moe_weight_view *view,
+static int view_resolve(const yvex_rocm_backend *backend, const yvex_moe_weight_view *view,
                         unsigned long long row_width, unsigned long long row_count,
                         unsigned long long *device_address, yvex_error *err)
 {
@@ -380,7 +380,7 @@ static graph_slot *graph_admit(struct yvex_rocm_moe_graphs *cache, const graph_k
 
 /* Graphs name device addresses: whoever frees or re-attaches what they point into drops them.
  * The caller has synchronised the stream (or nothing was ever launched). */
-void yvex_rocm_moe_graphs_release(yvex_backend *backend)
+void yvex_rocm_moe_graphs_release(yvex_rocm_backend *backend)
 {
     unsigned int i;
     if (!backend || !backend->moe_graphs) return;
@@ -412,7 +412,7 @@ static int worklist_policy_valid(const yvex_expert_worklist_policy *policy)
     return 1;
 }
 
-static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job,
+static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job *job,
                             const yvex_moe_row_batch *rows, const yvex_moe_row_batch_output *output,
                             yvex_moe_row_batch_result *result, yvex_error *err)
 {
@@ -583,7 +583,7 @@ static int moe_execute_rows(yvex_backend *backend, const yvex_moe_layer_job *job
     rows->device_outputs->is_written = 0;
     started = monotonic_ns();
     yvex_rocm_workspace_reset(backend);
-    if (!yvex_backend_workspace_acquire(backend, ranges.total - ALIGN, ALIGN, &base))
+    if (!yvex_rocm_backend_workspace_acquire(backend, ranges.total - ALIGN, ALIGN, &base))
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.rows", "workspace acquisition failed");
     fill_expert_weights(&routed, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], &views[YVEX_MOE_WEIGHT_ROUTED_UP],
                         &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], addresses[0], addresses[1], addresses[2],
@@ -875,7 +875,7 @@ sequence:
         result->device_completion_pending = 1;
         rows->device_outputs->is_written = 1;   /* ordered on the backend stream */
         result->total_ns = monotonic_ns() - started;
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
         return YVEX_OK;
     }
     /* one synchronisation publishes status, worklist facts, routing and optional host copies */
@@ -946,11 +946,11 @@ sequence:
     result->stream_synchronizations = 1ull;
     result->total_ns = monotonic_ns() - started;
     rows->device_outputs->is_written = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-static int moe_complete_rows(yvex_backend *backend, int barrier_observed,
+static int moe_complete_rows(yvex_rocm_backend *backend, int barrier_observed,
                              yvex_moe_row_batch_result *result, yvex_error *err)
 {
     unsigned long long started = 0ull;
@@ -974,16 +974,16 @@ static int moe_complete_rows(yvex_backend *backend, int barrier_observed,
     result->execution_class = YVEX_EXECUTION_CLASS_DEVICE_NATIVE;
     result->stream_synchronizations = barrier_observed ? 0ull : 1ull;
     result->synchronization_ns = started ? monotonic_ns() - started : 0ull;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-static const yvex_backend_moe_operations moe_operations = {
-    yvex_rocm_moe_derived_layout_plan, yvex_rocm_moe_derived_layout_build, moe_workspace_required,
+static const yvex_rocm_moe_operations moe_operations = {
+    yvex_rocm_moe_derived_layout_plan, yvex_rocm_moe_derived_layout_build, yvex_rocm_moe_workspace_required,
     moe_execute_rows,
     moe_complete_rows};
 
-const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_backend *backend)
+const yvex_rocm_moe_operations *yvex_rocm_backend_moe_operations_get(const yvex_rocm_backend *backend)
 {
     if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !backend->kernels_available ||
         backend->status == YVEX_BACKEND_STATUS_FAILED)
@@ -993,7 +993,7 @@ const yvex_backend_moe_operations *yvex_backend_moe_operations_get(const yvex_ba
 
 /* ---- host worklist: src/graph/worklist.c:369-441 ---------------------------------------------- */
 
-int yvex_expert_worklist_build(const unsigned long long *selected_experts,
+int yvex_rocm_expert_worklist_build(const unsigned long long *selected_experts,
                                const float *route_weights, unsigned long long pair_count,
                                unsigned long long experts_per_row, unsigned long long expert_count,
                                const yvex_expert_worklist_storage *storage,
@@ -1043,6 +1043,6 @@ int yvex_expert_worklist_build(const unsigned long long *selected_experts,
     observation->bucket_count = bucket;
     observation->maximum_bucket_population = maximum;
     observation->narrow_pairs = pair_count;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }

@@ -23,8 +23,8 @@
 
 #define ALIGN 256ull
 
-struct yvex_backend_moe_execution {
-    yvex_backend *backend;
+struct yvex_rocm_moe_execution {
+    yvex_rocm_backend *backend;
     const yvex_moe_layer_job *job;
     void *block;
     int owns_block;                       /* allocated here rather than taken from the workspace */
@@ -52,14 +52,14 @@ static unsigned long long align_up(unsigned long long v) { return (v + ALIGN - 1
 
 #define AT(field) ((void *)((unsigned char *)x->block + x->field))
 
-static int launched(yvex_backend_moe_execution *x, int code, const char *where, yvex_error *err)
+static int launched(yvex_rocm_moe_execution *x, int code, const char *where, yvex_error *err)
 {
     int rc = yvex_rocm_launch_result(code, where, err);
     if (rc == YVEX_OK) x->launches++;
     return rc;
 }
 
-static int upload(yvex_backend_moe_execution *x, void *dst, const void *src, unsigned long long bytes,
+static int upload(yvex_rocm_moe_execution *x, void *dst, const void *src, unsigned long long bytes,
                   const char *where, yvex_error *err)
 {
     if (yvex_hip_memcpy_h2d(dst, src, bytes, x->backend->stream) != 0)
@@ -68,7 +68,7 @@ static int upload(yvex_backend_moe_execution *x, void *dst, const void *src, uns
     return YVEX_OK;
 }
 
-static int download(yvex_backend_moe_execution *x, void *dst, const void *src, unsigned long long bytes,
+static int download(yvex_rocm_moe_execution *x, void *dst, const void *src, unsigned long long bytes,
                     const char *where, yvex_error *err)
 {
     if (!dst) return YVEX_OK;
@@ -81,13 +81,13 @@ static int download(yvex_backend_moe_execution *x, void *dst, const void *src, u
 
 /* Device address of a weight view: resident, or uploaded into the staging range at `offset`
  * (src/backend/cuda/moe.c:226-245). */
-static int weight_address_in(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
+static int weight_address_in(yvex_rocm_moe_execution *x, const yvex_moe_weight_view *view,
                              unsigned long long row_width, unsigned long long row_count,
                              unsigned long long offset, unsigned long long capacity,
                              unsigned long long *address, const char *where, yvex_error *err);
 
 /* A coefficient or router matrix staged alone: the whole staging range is its own. */
-static int weight_address(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
+static int weight_address(yvex_rocm_moe_execution *x, const yvex_moe_weight_view *view,
                           unsigned long long row_width, unsigned long long row_count,
                           unsigned long long offset, unsigned long long *address, const char *where,
                           yvex_error *err)
@@ -96,7 +96,7 @@ static int weight_address(yvex_backend_moe_execution *x, const yvex_moe_weight_v
                              offset <= x->staging_bytes ? x->staging_bytes - offset : 0ull, address, where, err);
 }
 
-static int weight_address_in(yvex_backend_moe_execution *x, const yvex_moe_weight_view *view,
+static int weight_address_in(yvex_rocm_moe_execution *x, const yvex_moe_weight_view *view,
                              unsigned long long row_width, unsigned long long row_count,
                              unsigned long long offset, unsigned long long capacity,
                              unsigned long long *address, const char *where, yvex_error *err)
@@ -120,7 +120,7 @@ static int weight_address_in(yvex_backend_moe_execution *x, const yvex_moe_weigh
 }
 
 /* Stream synchronisation and the kernels' status word (moe.c:277-296). */
-static int sync_status(yvex_backend_moe_execution *x, const char *where, yvex_error *err)
+static int sync_status(yvex_rocm_moe_execution *x, const char *where, yvex_error *err)
 {
     int device_status = 0, rc;
     unsigned long long started = now_ns();
@@ -136,7 +136,7 @@ static int sync_status(yvex_backend_moe_execution *x, const char *where, yvex_er
 
 static int flat_qtype(unsigned int qtype) { return qtype == 0u || qtype == 30u || qtype == 26u; }
 
-static int plan_ranges(yvex_backend_moe_execution *x, const yvex_moe_layer_plan *layer)
+static int plan_ranges(yvex_rocm_moe_execution *x, const yvex_moe_layer_plan *layer)
 {
     unsigned long long cursor = 0ull, hidden = layer->hidden_width, streams = layer->residual_streams;
     unsigned long long experts = layer->routed_experts, topk = layer->experts_per_token;
@@ -194,7 +194,7 @@ static int plan_ranges(yvex_backend_moe_execution *x, const yvex_moe_layer_plan 
 }
 
 /* src/backend/cuda/moe.c:372-414 */
-static int prepare_input(yvex_backend_moe_execution *x, yvex_error *err)
+static int prepare_input(yvex_rocm_moe_execution *x, yvex_error *err)
 {
     const yvex_moe_layer_job *job = x->job;
     const yvex_moe_layer_plan *layer = job->layer;
@@ -244,7 +244,7 @@ static int prepare_input(yvex_backend_moe_execution *x, yvex_error *err)
 }
 
 /* src/backend/cuda/moe.c:416-514 */
-static int route(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, yvex_error *err)
+static int route(yvex_rocm_moe_execution *x, yvex_moe_layer_result *result, yvex_error *err)
 {
     const yvex_moe_layer_job *job = x->job;
     const yvex_moe_layer_plan *layer = job->layer;
@@ -348,7 +348,7 @@ static void fill_weights(yvex_hip_expert_weights *w, const yvex_moe_weight_view 
 }
 
 /* The selected experts at once from the resident expert-major matrices (moe.c:584-672). */
-static int add_selected(yvex_backend_moe_execution *x, yvex_error *err)
+static int add_selected(yvex_rocm_moe_execution *x, yvex_error *err)
 {
     const yvex_moe_layer_job *job = x->job;
     const yvex_moe_layer_plan *layer = job->layer;
@@ -404,12 +404,12 @@ static int add_selected(yvex_backend_moe_execution *x, yvex_error *err)
     return rc;
 }
 
-int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backend,
+int yvex_rocm_backend_moe_begin(yvex_rocm_moe_execution **out, yvex_rocm_backend *backend,
                            const yvex_moe_layer_job *job, yvex_moe_layer_result *result,
                            yvex_error *err)
 {
     const yvex_moe_layer_plan *layer = job ? job->layer : NULL;
-    yvex_backend_moe_execution *x;
+    yvex_rocm_moe_execution *x;
     unsigned long long expanded_bytes, total;
     int rc;
     if (out) *out = NULL;
@@ -450,7 +450,7 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
     if (rc != YVEX_OK) return rc;
     if (job->cancel_requested && job->cancel_requested(job->cancel_context))
         return yvex_rocm_refuse(err, YVEX_ERR_CANCELLED, "rocm.moe.begin", "MoE execution was cancelled");
-    x = (yvex_backend_moe_execution *)calloc(1u, sizeof(*x));
+    x = (yvex_rocm_moe_execution *)calloc(1u, sizeof(*x));
     if (!x) return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.begin", "MoE owner allocation failed");
     x->backend = backend;
     x->job = job;
@@ -472,7 +472,7 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
         unsigned long long base = 0ull;
         yvex_rocm_workspace_reset(backend);
         if (backend->workspace_device_tensor &&
-            yvex_backend_workspace_acquire(backend, total, ALIGN, &base)) {
+            yvex_rocm_backend_workspace_acquire(backend, total, ALIGN, &base)) {
             x->block = (void *)(uintptr_t)base;
         } else if (yvex_hip_malloc(&x->block, total) != 0) {
             free(x);
@@ -505,15 +505,15 @@ int yvex_backend_moe_begin(yvex_backend_moe_execution **out, yvex_backend *backe
     }
     if (rc == YVEX_OK && x->grouped_selected) rc = add_selected(x, err);
     if (rc != YVEX_OK) {
-        (void)yvex_backend_moe_close(&x, NULL);
+        (void)yvex_rocm_backend_moe_close(&x, NULL);
         return rc;
     }
     *out = x;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_moe_add_expert(yvex_backend_moe_execution *x, const yvex_moe_weight_view *gate,
+int yvex_rocm_backend_moe_add_expert(yvex_rocm_moe_execution *x, const yvex_moe_weight_view *gate,
                                 const yvex_moe_weight_view *up, const yvex_moe_weight_view *down,
                                 float route_weight, int shared, yvex_error *err)
 {
@@ -573,12 +573,12 @@ int yvex_backend_moe_add_expert(yvex_backend_moe_execution *x, const yvex_moe_we
             x->subviews += 3ull;
             x->routed_ns += now_ns() - started;
         }
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
     }
     return rc;
 }
 
-int yvex_backend_moe_finish(yvex_backend_moe_execution *x, yvex_moe_layer_result *result, yvex_error *err)
+int yvex_rocm_backend_moe_finish(yvex_rocm_moe_execution *x, yvex_moe_layer_result *result, yvex_error *err)
 {
     const yvex_moe_layer_plan *layer = x && x->job ? x->job->layer : NULL;
     unsigned long long hidden, streams;
@@ -655,14 +655,14 @@ int yvex_backend_moe_finish(yvex_backend_moe_execution *x, yvex_moe_layer_result
     x->backend->memory.h2d_bytes += x->h2d;
     x->backend->memory.d2h_bytes += x->d2h - x->synchronizations * sizeof(int);   /* counted by the sync */
     x->finished = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_moe_close(yvex_backend_moe_execution **execution, yvex_error *err)
+int yvex_rocm_backend_moe_close(yvex_rocm_moe_execution **execution, yvex_error *err)
 {
     if (!execution || !*execution) {
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
         return YVEX_OK;
     }
     if ((*execution)->block && (*execution)->owns_block) {
@@ -673,6 +673,6 @@ int yvex_backend_moe_close(yvex_backend_moe_execution **execution, yvex_error *e
     }
     free(*execution);
     *execution = NULL;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }

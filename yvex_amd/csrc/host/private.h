@@ -9,10 +9,13 @@
 #include "yvex_rocm.h"
 #include "yvex_rocm_kernels.h"
 
-struct yvex_backend {
+struct yvex_rocm_backend {
     yvex_backend_kind kind;
     yvex_backend_status status;
     unsigned long long owner_id;
+    /* what this backend's tensors name as their owner: the backend itself, or the object an
+     * embedding library wraps it in (yvex_rocm_backend_bind_owner) */
+    const void *public_owner;
     int device_index;
     int host_only;             /* YVEX_TEST_ROCM_NO_DEVICE: tensors in host memory, no kernels */
     int kernels_available;
@@ -36,21 +39,21 @@ struct yvex_backend {
 };
 
 /* Drop every cached launch graph (the stream is idle or was never used). */
-void yvex_rocm_moe_graphs_release(yvex_backend *backend);
+void yvex_rocm_moe_graphs_release(yvex_rocm_backend *backend);
 
 int yvex_rocm_refuse(yvex_error *err, yvex_status code, const char *where, const char *message);
 int yvex_rocm_seam(const char *name);
-int yvex_rocm_tensor_owner_is(const yvex_backend *backend, const yvex_device_tensor *tensor);
-void yvex_rocm_workspace_reset(yvex_backend *backend);
+int yvex_rocm_tensor_owner_is(const yvex_rocm_backend *backend, const yvex_device_tensor *tensor);
+void yvex_rocm_workspace_reset(yvex_rocm_backend *backend);
 /* Kernels present and the backend healthy, else the typed refusal of a missing bundle. */
-int yvex_rocm_require_kernels(const yvex_backend *backend, const char *where, yvex_error *err);
+int yvex_rocm_require_kernels(const yvex_rocm_backend *backend, const char *where, yvex_error *err);
 /* Map a launch-level return code (negative yvex_status) to an error. */
 int yvex_rocm_launch_result(int rc, const char *where, yvex_error *err);
 /* Stream synchronise + read the device status word (and clear it for the next operation). */
-int yvex_rocm_finish(yvex_backend *backend, const char *where, int *device_status, yvex_error *err);
-int yvex_rocm_status_reset(yvex_backend *backend, const char *where, yvex_error *err);
+int yvex_rocm_finish(yvex_rocm_backend *backend, const char *where, int *device_status, yvex_error *err);
+int yvex_rocm_status_reset(yvex_rocm_backend *backend, const char *where, yvex_error *err);
 /* Resolve a weight view: device_address if given, else the resident arena mapping. */
-int yvex_rocm_resolve(const yvex_backend *backend, const unsigned char *host,
+int yvex_rocm_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
                       unsigned long long bytes, unsigned long long *device_address);
 
 /* Residual-stream geometry of a layer plan (src/graph/numeric.c:668-689) within this backend's
@@ -59,7 +62,7 @@ int yvex_rocm_moe_envelope_geometry(const yvex_moe_layer_plan *layer);
 /* Check a weight view against the shape the plan implies (FORMAT), its qtype against the device
  * capability rows (UNSUPPORTED), and find its device address; *resident = 0 when the bytes lie
  * outside the attached arena and carry no device address (the address is then left 0). */
-int yvex_rocm_moe_view_check(const yvex_backend *backend, const yvex_moe_weight_view *view,
+int yvex_rocm_moe_view_check(const yvex_rocm_backend *backend, const yvex_moe_weight_view *view,
                              unsigned long long row_width, unsigned long long row_count,
                              unsigned long long *device_address, int *resident, yvex_error *err);
 

@@ -20,8 +20,8 @@ static int mul_u64(unsigned long long a, unsigned long long b, unsigned long lon
 static int qtype_admit(unsigned int qtype, unsigned long long row_width, unsigned long long row_bytes,
                        const char *where, yvex_error *err)
 {
-    const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(qtype);
-    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(qtype);
+    const yvex_rocm_numeric_capability *capability = yvex_rocm_quant_numeric_capability_at(qtype);
+    const yvex_rocm_qtype_geometry *geometry = yvex_rocm_gguf_qtype_geometry_find(qtype);
     unsigned long long expected;
     if (!capability || !geometry || !capability->device_compute_available)
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, where,
@@ -40,13 +40,13 @@ static int q8_eligible(unsigned int qtype)
            qtype == YVEX_GGUF_QTYPE_Q4_K || qtype == YVEX_GGUF_QTYPE_IQ2_XXS;
 }
 
-int yvex_backend_rocm_encoded_matvec(
-    yvex_backend *backend, const unsigned char *resident_encoded,
+int yvex_rocm_encoded_matvec(
+    yvex_rocm_backend *backend, const unsigned char *resident_encoded,
     unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
     unsigned long long row_width, unsigned long long row_bytes, unsigned long long input_rows,
     const yvex_device_tensor *input, const yvex_device_tensor *input_tail,
     unsigned long long input_head_width, const yvex_device_tensor *additive,
-    yvex_device_tensor *output, int activation_q8, yvex_backend_rocm_operation_facts *facts,
+    yvex_device_tensor *output, int activation_q8, yvex_rocm_operation_facts *facts,
     yvex_error *err)
 {
     const char *where = "rocm.encoded-matvec";
@@ -97,13 +97,13 @@ int yvex_backend_rocm_encoded_matvec(
     if (q8_path) {
         if (!mul_u64(input_rows * (row_width / 256ull), 292ull, &q8_bytes))
             return yvex_rocm_refuse(err, YVEX_ERR_BOUNDS, where, "Q8 activation workspace exceeds bounds");
-        if (!yvex_backend_workspace_acquire(backend, q8_bytes, 256ull, &q8_address))
+        if (!yvex_rocm_backend_workspace_acquire(backend, q8_bytes, 256ull, &q8_address))
             return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                     "Q8 activation needs an attached workspace of rows * width/256 * 292 bytes");
     }
     if (split_input) {
         joined_bytes = input_bytes;
-        if (!yvex_backend_workspace_acquire(backend, joined_bytes, 256ull, &joined_address))
+        if (!yvex_rocm_backend_workspace_acquire(backend, joined_bytes, 256ull, &joined_address))
             return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                     "a split input needs an attached workspace of rows * width * 4 bytes");
     }
@@ -152,16 +152,16 @@ int yvex_backend_rocm_encoded_matvec(
     facts->activation_bytes = activation_bytes;
     facts->temporary_bytes = sizeof(int) + q8_bytes + joined_bytes;
     facts->compulsory_memory_facts_available = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
-int yvex_backend_rocm_encoded_gather(
-    yvex_backend *backend, const unsigned char *resident_encoded,
+int yvex_rocm_encoded_gather(
+    yvex_rocm_backend *backend, const unsigned char *resident_encoded,
     unsigned long long encoded_bytes, unsigned int qtype, unsigned long long row_count,
     unsigned long long row_width, unsigned long long row_bytes, const unsigned int *row_ids,
     unsigned long long selected_rows, yvex_device_tensor *output,
-    yvex_backend_rocm_operation_facts *facts, yvex_error *err)
+    yvex_rocm_operation_facts *facts, yvex_error *err)
 {
     const char *where = "rocm.encoded-gather";
     unsigned long long device_address = 0ull, output_bytes, total_bytes, ids_address = 0ull, i;
@@ -187,7 +187,7 @@ int yvex_backend_rocm_encoded_gather(
     rc = yvex_rocm_require_kernels(backend, where, err);
     if (rc != YVEX_OK) return rc;
     yvex_rocm_workspace_reset(backend);
-    if (!yvex_backend_workspace_acquire(backend, selected_rows * sizeof(unsigned int), 256ull, &ids_address))
+    if (!yvex_rocm_backend_workspace_acquire(backend, selected_rows * sizeof(unsigned int), 256ull, &ids_address))
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                 "gather needs an attached workspace for the row identifiers");
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
@@ -217,25 +217,25 @@ int yvex_backend_rocm_encoded_gather(
     facts->activation_bytes = output_bytes;
     facts->temporary_bytes = sizeof(int) + selected_rows * sizeof(unsigned int);
     facts->compulsory_memory_facts_available = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }
 
 /* src/backend/cuda/qtype.c:523-700: one encoded row times one vector, host pointers in, one float
  * out, computed on the device by the serial double-precision probe kernel. The device
  * temporaries live for the call only. */
-int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const unsigned char *encoded,
+int yvex_rocm_quant_row_dot(yvex_rocm_backend *backend, unsigned int qtype, const unsigned char *encoded,
                             size_t encoded_bytes, const float *vector, unsigned long long elements,
                             float *out, void *failure, yvex_error *err)
 {
     const char *where = "rocm.quant.row_dot";
-    const yvex_quant_numeric_capability *capability = yvex_quant_numeric_capability_at(qtype);
-    const yvex_gguf_qtype_geometry *geometry = yvex_gguf_qtype_geometry_find(qtype);
+    const yvex_rocm_numeric_capability *capability = yvex_rocm_quant_numeric_capability_at(qtype);
+    const yvex_rocm_qtype_geometry *geometry = yvex_rocm_gguf_qtype_geometry_find(qtype);
     unsigned long long vector_bytes, weight_offset, total;
     void *block = NULL;
     int rc;
     (void)failure;      /* the reference's failure record belongs to its quantization pipeline */
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM || !encoded || !vector || !out || !elements ||
         ((uintptr_t)vector & 3u) || ((uintptr_t)out & 3u) ||
         ((qtype == YVEX_GGUF_QTYPE_F32 || qtype == YVEX_GGUF_QTYPE_I32) && ((uintptr_t)encoded & 3u)) ||
@@ -276,7 +276,7 @@ int yvex_rocm_quant_row_dot(yvex_backend *backend, unsigned int qtype, const uns
     if (rc == YVEX_OK) {
         backend->memory.h2d_bytes += vector_bytes + encoded_bytes;
         backend->memory.d2h_bytes += sizeof(float);
-        yvex_error_clear(err);
+        yvex_rocm_error_clear(err);
     }
     return rc;
 }

@@ -20,10 +20,10 @@ static int mul_u64(unsigned long long a, unsigned long long b, unsigned long lon
     return 1;
 }
 
-int yvex_backend_rocm_select_greedy_rows(
-    yvex_backend *backend, const yvex_device_tensor *logits, unsigned long long row_count,
+int yvex_rocm_select_greedy_rows(
+    yvex_rocm_backend *backend, const yvex_device_tensor *logits, unsigned long long row_count,
     unsigned long long row_width, unsigned int *selected_tokens, float *selected_values,
-    unsigned long long *tie_counts, yvex_backend_rocm_operation_facts *facts, yvex_error *err)
+    unsigned long long *tie_counts, yvex_rocm_operation_facts *facts, yvex_error *err)
 {
     const char *where = "rocm.sampling.greedy";
     unsigned long long value_count, value_bytes, token_bytes, selected_bytes, tie_bytes;
@@ -50,15 +50,15 @@ int yvex_backend_rocm_select_greedy_rows(
     rc = yvex_rocm_require_kernels(backend, where, err);
     if (rc != YVEX_OK) return rc;
     yvex_rocm_workspace_reset(backend);
-    if (!yvex_backend_workspace_acquire(backend, tie_bytes, 256ull, &ties_device) ||
-        !yvex_backend_workspace_acquire(backend, token_bytes, 256ull, &tokens_device) ||
-        !yvex_backend_workspace_acquire(backend, selected_bytes, 256ull, &values_device))
+    if (!yvex_rocm_backend_workspace_acquire(backend, tie_bytes, 256ull, &ties_device) ||
+        !yvex_rocm_backend_workspace_acquire(backend, token_bytes, 256ull, &tokens_device) ||
+        !yvex_rocm_backend_workspace_acquire(backend, selected_bytes, 256ull, &values_device))
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, where,
                                 "greedy row selection needs an attached workspace for its results");
     /* long rows are shared among the compute units when the workspace has room for the partial
      * results; otherwise one workgroup scans a row */
     scratch_bytes = yvex_hip_argmax_scratch_bytes(row_count, row_width);
-    if (scratch_bytes && !yvex_backend_workspace_acquire(backend, scratch_bytes, 256ull, &scratch_device))
+    if (scratch_bytes && !yvex_rocm_backend_workspace_acquire(backend, scratch_bytes, 256ull, &scratch_device))
         scratch_bytes = 0ull, scratch_device = 0ull;
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.sampling.greedy.launch",
@@ -98,6 +98,6 @@ int yvex_backend_rocm_select_greedy_rows(
     facts->activation_bytes = value_bytes;
     facts->temporary_bytes = temporary_bytes;
     facts->compulsory_memory_facts_available = 1;
-    yvex_error_clear(err);
+    yvex_rocm_error_clear(err);
     return YVEX_OK;
 }

@@ -14,7 +14,7 @@ class Backend:
         self.handle = C.c_void_p()
         self.err = abi.Error()
         opts = abi.BackendOptions(abi.KIND_ROCM, None, memory_limit)
-        self.open_rc = self.lib.yvex_backend_open(C.byref(self.handle), C.byref(opts), C.byref(self.err))
+        self.open_rc = self.lib.yvex_rocm_backend_open(C.byref(self.handle), C.byref(opts), C.byref(self.err))
         self.tensors = []
 
     @property
@@ -24,7 +24,7 @@ class Backend:
     def tensor(self, nbytes, dtype=abi.DTYPE_F32, name=b"t"):
         desc = abi.TensorDesc(name, dtype, 1, (abi.ULL * 4)(nbytes, 0, 0, 0), nbytes)
         out = C.POINTER(abi.DeviceTensor)()
-        rc = self.lib.yvex_backend_tensor_alloc(self.handle, C.byref(desc), C.byref(out), C.byref(self.err))
+        rc = self.lib.yvex_rocm_backend_tensor_alloc(self.handle, C.byref(desc), C.byref(out), C.byref(self.err))
         if rc == 0:
             self.tensors.append(out)
         return rc, out
@@ -33,7 +33,7 @@ class Backend:
         array = np.ascontiguousarray(array, np.float32)
         rc, t = self.tensor(array.nbytes)
         assert rc == 0, self.err.message
-        rc = self.lib.yvex_backend_tensor_write(self.handle, t, array.ctypes.data, array.nbytes,
+        rc = self.lib.yvex_rocm_backend_tensor_write(self.handle, t, array.ctypes.data, array.nbytes,
                                                 C.byref(self.err))
         assert rc == 0, self.err.message
         return t
@@ -45,7 +45,7 @@ class Backend:
 
     def read_f32(self, tensor, count):
         out = np.empty(count, np.float32)
-        rc = self.lib.yvex_backend_tensor_read(self.handle, tensor, out.ctypes.data, out.nbytes,
+        rc = self.lib.yvex_rocm_backend_tensor_read(self.handle, tensor, out.ctypes.data, out.nbytes,
                                                C.byref(self.err))
         assert rc == 0, self.err.message
         return out
@@ -56,12 +56,12 @@ class Backend:
         desc = abi.TensorDesc(b"arena", abi.DTYPE_I8, 1, (abi.ULL * 4)(blob.nbytes, 0, 0, 0), blob.nbytes)
         out = C.POINTER(abi.DeviceTensor)()
         host = C.c_void_p()
-        rc = self.lib.yvex_backend_resident_alloc(self.handle, C.byref(desc), C.byref(out),
+        rc = self.lib.yvex_rocm_backend_resident_alloc(self.handle, C.byref(desc), C.byref(out),
                                                   C.byref(host), C.byref(self.err))
         assert rc == 0, self.err.message
         self.tensors.append(out)
         C.memmove(host.value, blob.ctypes.data, blob.nbytes)
-        rc = self.lib.yvex_backend_resident_attach(self.handle, host, blob.nbytes, out, generation,
+        rc = self.lib.yvex_rocm_backend_resident_attach(self.handle, host, blob.nbytes, out, generation,
                                                    C.byref(self.err))
         assert rc == 0, self.err.message
         return out, host.value
@@ -69,15 +69,15 @@ class Backend:
     def workspace(self, nbytes):
         rc, t = self.tensor(nbytes, abi.DTYPE_I8, b"workspace")
         assert rc == 0, self.err.message
-        rc = self.lib.yvex_backend_workspace_attach(self.handle, t, nbytes, C.byref(self.err))
+        rc = self.lib.yvex_rocm_backend_workspace_attach(self.handle, t, nbytes, C.byref(self.err))
         assert rc == 0, self.err.message
         return t
 
     def release_all(self):
         for t in reversed(self.tensors):
-            self.lib.yvex_backend_tensor_release(self.handle, C.byref(t), C.byref(self.err))
+            self.lib.yvex_rocm_backend_tensor_release(self.handle, C.byref(t), C.byref(self.err))
         self.tensors = []
 
     def close(self):
         self.release_all()
-        return self.lib.yvex_backend_close_checked(C.byref(self.handle), C.byref(self.err))
+        return self.lib.yvex_rocm_backend_close_checked(C.byref(self.handle), C.byref(self.err))
