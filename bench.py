@@ -251,8 +251,9 @@ class AbiLayer:
 
 def dense_leg(torch, K, dev, repeats: int):
     """BASELINE configs 0-2 and an output head as single matvec launches: random packed bytes with
-    small positive fp16 block scales, 32 distinct weight copies walked in turn (2 for the head) so
-    that no launch finds its weights in cache. Bytes counted: the encoded matrix."""
+    small positive fp16 block scales, at least 32 distinct weight copies and more than 320 MB of
+    them walked in turn (2 for the head) so that no launch finds its weights in a cache. Bytes
+    counted: the encoded matrix. Batches of 16 rows and more run on the int8 matrix cores."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(7)
     out = {}
@@ -290,8 +291,10 @@ def dense_leg(torch, K, dev, repeats: int):
             print(f"dense leg: graph capture unavailable ({error})", file=sys.stderr)
         return ms, graph_us
 
-    def run(name, qt, rows, width, inputs, q8, copies=32):
+    def run(name, qt, rows, width, inputs, q8, copies=None):
         total = rows * K.row_bytes(qt, width)
+        # enough distinct copies that a launch cannot find its matrix in the 256 MB last-level cache
+        copies = copies or max(32, -(-320_000_000 // total))
         if qt == K.IQ2_XXS:
             w = synth_iq2xxs(torch, copies * rows * width // 256, dev, 5)
         else:
@@ -317,13 +320,18 @@ def dense_leg(torch, K, dev, repeats: int):
         out[name] = {"us": round(ms * 1e3, 2), "graph_us": round(graph_us, 2) if graph_us else None,
                      "GB_per_s": round(total / (best_ms * 1e-3) / 1e9, 1),
                      "hbm_peak_frac": round(total / (best_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "matrix_bytes": total, "status": int(status.item())}
+                     "matrix_bytes": total, "copies": copies, "status": int(status.item())}
+        if inputs >= 16:
+            out[name]["int8_TOPs"] = round(2.0 * rows * width * inputs / (best_ms * 1e-3) / 1e12, 1)
         del w
 
     run("cfg0_q8_0_4096x4096_f32_b1", K.Q8_0, 4096, 4096, 1, False)
     run("cfg0_q8_0_4096x4096_q8k_b1", K.Q8_0, 4096, 4096, 1, True)
     run("cfg1_q4_k_2048x7168_q8k_b1", K.Q4_K, 2048, 7168, 1, True)
     run("cfg1_q4_k_2048x7168_q8k_b16", K.Q4_K, 2048, 7168, 16, True)
+    run("cfg1_q4_k_2048x7168_q8k_b256", K.Q4_K, 2048, 7168, 256, True)
+    run("cfg1_q4_k_2048x7168_q8k_b2048", K.Q4_K, 2048, 7168, 2048, True)
+    run("cfg2_iq2_xxs_7168x2048_q8k_b2048", K.IQ2_XXS, 7168, 2048, 2048, True)
     run("cfg2_iq2_xxs_7168x2048_f32_b1", K.IQ2_XXS, 7168, 2048, 1, False)
     run("cfg2_iq2_xxs_7168x2048_q8k_b1", K.IQ2_XXS, 7168, 2048, 1, True)
     run("head_q8_0_129280x7168_q8k_b1", K.Q8_0, 129280, 7168, 1, True, copies=2)

@@ -131,6 +131,41 @@ def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
     assert_close(got, oracle.matvec(qt, w, rows, width, deq))
 
 
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("IQ2_XXS", 516, 2048, 32), ("IQ2_XXS", 260, 7168, 70), ("IQ2_XXS", 7168, 2048, 33),
+    ("Q4_K", 516, 2048, 16), ("Q4_K", 132, 7168, 70), ("Q4_K", 2048, 7168, 16), ("Q4_K", 36, 512, 200)])
+def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, width, inputs):
+    """From 16 (Q4_K) or 32 (IQ2_XXS) Q8_K input rows on, projections run on the int8 matrix cores
+    (src/backend/cuda/private.h:461-464 turns the tensor-core kernels on at 16). Results are those of the
+    integer path (1e-5 of the oracle's Q8_K product), bf16 output rounds them, and an input-row
+    count below the threshold gives the sweep kernel's values to the same bar."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec.rows.{qtype}.{rows}.{width}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    want = oracle.q8_matvec(qt, w, rows, width, act_host, inputs)
+    assert_close(got, want, rel=1e-5, abs_=1e-5)
+    deq = oracle.q8k_dequantize(act_host).reshape(inputs, width)
+    assert_close(got, oracle.matvec(qt, w, rows, width, deq, threads=8))
+    rounded = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                       output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((rounded.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(rounded - got) <= np.abs(got) * 2.0 ** -8 + 1e-30)
+    # the same rows fifteen at a time take the sweep kernel: same values to the same bar
+    few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=15,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    assert_close(few, got[:15], rel=1e-5, abs_=1e-5)
+
+
 @pytest.mark.parametrize("qtype,rows,width", [("Q8_0", 9600, 7168), ("IQ2_XXS", 37000, 7168)])
 def test_matvec_output_head_variant(gpu, oracle, qtype, rows, width):
     """One Q8_K activation row against a matrix of 64 MB or more takes the variant with four

@@ -42,6 +42,17 @@ int compute_units();
         });                                                                                     \
     } while (0)
 
+// IQ2_XXS rows x Q8_K input rows on the int8 matrix cores as a plain projection (prefill.hip).
+int launch_iq2_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                          uint64_t row_bytes, const void *act_q8k, uint64_t input_rows, float *out,
+                          bool round_bf16, int *status, hipStream_t stream);
+
+// Q4_K rows x Q8_K input rows on the int8 matrix cores (dense_q4k.hip).
+int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                          uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
+                          const float *additive, float *out, uint64_t out_stride, bool output_bf16,
+                          int *status, hipStream_t stream);
+
 inline hipStream_t as_stream(yvex_hip_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
 }  // namespace yvex

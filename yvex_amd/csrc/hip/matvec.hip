@@ -391,6 +391,20 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         if (input_stride < row_width) return ST_INVALID_ARG;
         if (!scalar && (((uintptr_t)input & 15u) || (input_stride & 3u))) return ST_INVALID_ARG;
     }
+    // IQ2_XXS rows against a batch of Q8_K input rows: the int8 matrix-core kernel of the
+    // row-batch expert path, as one bucket that holds every input row (the reference turns its
+    // tensor-core kernels on from 16 input rows, src/backend/cuda/private.h:461-464; measured
+    // here the sweep below stays faster up to 31 rows: 17 us against 22 us for 7168 x 2048 at 16). Same exact
+    // int32 superblock sums and the same fp32 scaling as the sweep below; only the order in
+    // which the superblock terms are added in fp32 differs.
+    if (qtype == QT_IQ2_XXS && input_q8 && input_rows >= 32ull && !additive &&
+        out_stride == row_count && row_count % 4ull == 0ull && !((uintptr_t)encoded & 3u) &&
+        !(row_bytes & 3ull) && row_width / 32ull <= 64ull * 4ull && !((uintptr_t)out & 15u))
+        return launch_iq2_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, out,
+                                     output_bf16 != 0, status, s);
+    if (qtype == QT_Q4_K && input_q8 && input_rows >= 16ull && !((uintptr_t)encoded & 15u))
+        return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
+                                     out, out_stride, output_bf16 != 0, status, s);
     if (qtype == QT_F32 && input_rows >= 32ull && row_width % 32ull == 0ull &&
         !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
         const unsigned long long grid_x = (row_count + 31ull) / 32ull, grid_y = (input_rows + 31ull) / 32ull;

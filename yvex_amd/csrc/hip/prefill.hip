@@ -86,6 +86,7 @@ struct MfmaArgs {
     unsigned out_rows;       // weight rows per expert
     double limit;
     int *status;
+    int plain_output;        // plain projection: outputs stay fp32 instead of being rounded to bf16
 };
 
 __device__ __forceinline__ void lds_write_uint4(unsigned address, uint4 v)
@@ -660,8 +661,12 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
                     swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(up.w), route_weight, a.limit, limit_f32)};
                 store4(info.x, row, value);
             } else {
-                const float value[4] = {bf16_round(__uint_as_float(g.x)), bf16_round(__uint_as_float(g.y)),
-                                        bf16_round(__uint_as_float(g.z)), bf16_round(__uint_as_float(g.w))};
+                float value[4] = {__uint_as_float(g.x), __uint_as_float(g.y), __uint_as_float(g.z),
+                                  __uint_as_float(g.w)};
+                if (!a.plain_output) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) value[k] = bf16_round(value[k]);
+                }
                 store4(info.x, row, value);
             }
         }
@@ -779,6 +784,32 @@ static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
     YVEX_ALLOW_DYNAMIC_LDS(mfma_iq2_kernel<FUSED_UP>, kMfmaLdsBytes);
     mfma_iq2_kernel<FUSED_UP><<<compute_units(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
     return check_launch("moe_rows_mfma");
+}
+
+// A plain projection through the row-batch kernel: every input row in one bucket of expert 0.
+int launch_iq2_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                          uint64_t row_bytes, const void *act_q8k, uint64_t input_rows, float *out,
+                          bool round_bf16, int *status, hipStream_t stream)
+{
+    int rc = check_matrix(QT_IQ2_XXS, row_width, row_bytes);
+    if (rc) return rc;
+    if (input_rows > 0xffffffffull || row_count > 0xffffffffull || row_count % 4u) return ST_BOUNDS;
+    yvex_hip_expert_weights w{};
+    w.down = encoded;
+    w.down_qtype = QT_IQ2_XXS;
+    w.hidden = row_count;
+    w.intermediate = row_width;
+    w.down_row_bytes = row_bytes;
+    w.down_expert_bytes = row_bytes * row_count;
+    MfmaArgs a{};
+    const WorklistView none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    fill_down_problem(a.pr, &w, act_q8k, 1, none, input_rows, 1u, out);
+    a.width = (unsigned)row_width;
+    a.out_rows = (unsigned)row_count;
+    a.limit = 1.0;
+    a.status = status;
+    a.plain_output = round_bf16 ? 0 : 1;
+    return launch_mfma<false>(a, stream);
 }
 
 }  // namespace yvex
