@@ -505,8 +505,7 @@ def main() -> int:
     x = torch.randn((ROWS, HIDDEN), device=dev, generator=gen)
     # router weights (F32, as the model stores them): logits = router . row, unit variance
     router = torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5
-    logits = K.matvec(router.view(torch.uint8).reshape(-1), K.F32, EXPERTS, HIDDEN, x,
-                      status=K.new_status(dev))
+    logits = K.matvec_f32_rows(router, x, K.new_status(dev))     # as execute_rows projects them
     layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                      qtypes=(qt, qt, qt), routed=(gate, up, down), shared=shared, bias=None,
                      scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,

@@ -67,6 +67,18 @@ int yvex_hip_concat_rows_bf16(const float *head, const float *tail, uint64_t row
                               uint64_t head_width, uint64_t tail_width, float *out, int *status,
                               yvex_hip_stream stream);
 
+/* yvex_hip_matvec for F32 weight rows and a decode-width batch of F32 input rows (8 to 255: the
+ * router projection of the MoE row batch, src/backend/cuda/moe.c:1259-1284), given scratch memory:
+ * the row width is split between workgroups so that the whole device takes part, the partial
+ * sums go to scratch and a second launch adds them in split order (deterministic). With NULL or
+ * too little scratch (yvex_hip_matvec_f32_scratch_bytes, 0 when the shape is not split) it is
+ * yvex_hip_matvec. */
+uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64_t row_width, uint64_t input_rows);
+int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t row_width,
+                             const float *input, uint64_t input_rows, uint64_t input_stride,
+                             const float *additive, float *out, uint64_t out_stride, int output_bf16,
+                             void *scratch, uint64_t scratch_bytes, int *status, yvex_hip_stream stream);
+
 /* Replaces yvex_argmax_f32 (kernels.cu:59-110): for each of row_count (<= 65535) rows of
  * row_width (< 2^32) F32 values the largest value, the lowest index holding it and the number of
  * elements holding it. A non-finite element raises status 1 and its row publishes nothing.

@@ -77,7 +77,8 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     assert_close(got, want)
 
 
-@pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32)])
+@pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32),
+                                               (256, 7168, 300), (40, 96, 260), (256, 7168, 8), (3, 256, 9)])
 def test_matvec_f32_weights_over_a_row_batch(gpu, oracle, rows, width, inputs):
     """F32 weight rows against 32 or more F32 input rows (a router or mixing projection over a
     prefill batch) run on the fp32 matrix cores; ragged edges, the additive operand and the bf16
@@ -94,6 +95,14 @@ def test_matvec_f32_weights_over_a_row_batch(gpu, oracle, rows, width, inputs):
     # against the double-precision product too: a transposed or mis-split operand cannot pass
     exact = x.astype(np.float64) @ w.view(np.float32).reshape(rows, width).astype(np.float64).T
     assert np.allclose(got, exact, rtol=1e-4, atol=1e-4)
+    # the same projection with scratch memory (split between workgroups where the shape allows)
+    w_rows = dev(w.view(np.float32).reshape(rows, width), gpu)
+    split = K.matvec_f32_rows(w_rows, dev(x, gpu), status).cpu().numpy()
+    status_ok(status)
+    assert_close(split, want)
+    assert np.allclose(split, exact, rtol=1e-4, atol=1e-4)
+    again = K.matvec_f32_rows(w_rows, dev(x, gpu), status).cpu().numpy()
+    assert np.array_equal(split, again)                # partial sums are added in a fixed order
     add = g.normal(inputs * rows).reshape(inputs, rows)
     got = K.matvec(dev(w, gpu), oracle.F32, rows, width, dev(x, gpu), additive=dev(add, gpu),
                    output_bf16=True, status=status).cpu().numpy()

@@ -49,8 +49,34 @@ def _run(cmd):
     return "\n".join(l for l in proc.stderr.splitlines() if l.strip() and noise not in l)
 
 
+def write_exports_map() -> str:
+    """csrc/exports.map lists exactly the entry points the two public headers declare."""
+    import re
+    names = set()
+    for header in ("yvex_rocm.h", "yvex_rocm_kernels.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(yvex_[a-z0-9_]+)\s*\(", text))
+    lines = ["/* Everything libyvex_rocm.so exports: the entry points include/yvex_rocm.h (yvex_rocm_*)",
+             " * and include/yvex_rocm_kernels.h (yvex_hip_*) declare. No name of the reference's own",
+             " * libyvex is defined here, so both can live in one process or one link. */", "{", "  global:"]
+    row = "   "
+    for name in sorted(names):
+        if len(row) + len(name) + 2 > 100:
+            lines.append(row)
+            row = "   "
+        row += " " + name + ";"
+    lines += [row, "  local: *;", "};", ""]
+    path = os.path.join(CSRC, "exports.map")
+    text = "\n".join(lines)
+    if not os.path.exists(path) or open(path).read() != text:
+        open(path, "w").write(text)
+    return path
+
+
 def build(verbose: bool = False, jobs: int | None = None) -> str:
     os.makedirs(OBJ, exist_ok=True)
+    exports = write_exports_map()
     hip, host = _sources()
     tasks = []
     for src in hip:
@@ -67,7 +93,7 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
     objs = [t[0] for t in tasks]
     # only the declared entry points leave the library, and its own calls bind inside it
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-lm", "-lpthread",
-          f"-Wl,--version-script={os.path.join(CSRC, 'exports.map')}", "-Wl,-Bsymbolic"])
+          f"-Wl,--version-script={exports}", "-Wl,-Bsymbolic"])
     return LIB
 
 

@@ -24,6 +24,7 @@ struct MatvecArgs {
     unsigned long long out_stride;
     int output_bf16;
     int *status;
+    float *parts;            // split projections: [split][input row][weight row] partial sums
 };
 
 __device__ __forceinline__ void matvec_publish(const MatvecArgs &a, unsigned long long in,
@@ -258,6 +259,108 @@ __global__ __launch_bounds__(256) void matvec_f32_tile_kernel(MatvecArgs a)
     }
 }
 
+// The same projection for a decode-width batch (8 to 255 input rows, e.g. the router over 32
+// rows): too few 32 x 32 tiles would leave most compute units idle, so a workgroup of sixteen
+// waves owns 16 weight rows x 16 input rows on V_MFMA_F32_16X16X4_F32 and its waves split the
+// row width sixteen ways. Lane (i, q) loads four consecutive floats of weight row i and of input
+// row i at offset 16 j + 4 q; partial tiles are added in wave order.
+template <unsigned WAVES>
+__global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArgs a)
+{
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    __shared__ float partial[WAVES - 1u][4][64];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned i16 = lane & 15u, q = lane >> 4;
+    unsigned long long wrow = (unsigned long long)blockIdx.x * 16ull + i16;
+    unsigned long long in = (unsigned long long)blockIdx.y * 16ull + i16;
+    if (wrow >= a.row_count) wrow = a.row_count - 1ull;
+    if (in >= a.input_rows) in = a.input_rows - 1ull;
+    // blockIdx.z splits the row width between workgroups (their sums go to a.parts and a second
+    // launch adds them in split order); the waves of a workgroup split its share again
+    const unsigned long long share = a.row_width / ((unsigned long long)gridDim.z * WAVES);   // a multiple of 16
+    const unsigned long long begin = ((unsigned long long)blockIdx.z * WAVES + wave) * share + 4u * q;
+    const float *wp = (const float *)(a.encoded + wrow * a.row_bytes) + begin;
+    const float *xp = (const float *)a.input + in * a.input_stride + begin;
+    const unsigned steps = (unsigned)(share / 16ull);
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned bad = 0u;
+    const unsigned groups = (steps + 3u) / 4u;
+    float4 w[4], x[4];
+#pragma unroll
+    for (unsigned j = 0; j < 4u; ++j) {
+        const unsigned at = 16u * (j < steps ? j : steps - 1u);
+        w[j] = *reinterpret_cast<const float4 *>(wp + at);
+        x[j] = *reinterpret_cast<const float4 *>(xp + at);
+    }
+    for (unsigned group = 0; group < groups; ++group) {
+        float4 wn[4], xn[4];
+        if (group + 1u < groups) {
+#pragma unroll
+            for (unsigned j = 0; j < 4u; ++j) {
+                const unsigned step = 4u * (group + 1u) + j;
+                const unsigned at = 16u * (step < steps ? step : steps - 1u);
+                wn[j] = *reinterpret_cast<const float4 *>(wp + at);
+                xn[j] = *reinterpret_cast<const float4 *>(xp + at);
+            }
+        }
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            if (4u * group + j >= steps) break;
+            bad |= (unsigned)!finite_f32(w[j].x) | (unsigned)!finite_f32(w[j].y) |
+                   (unsigned)!finite_f32(w[j].z) | (unsigned)!finite_f32(w[j].w);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].x, x[j].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].y, x[j].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].z, x[j].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].w, x[j].w, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            w[j] = wn[j];
+            x[j] = xn[j];
+        }
+    }
+    if (bad) raise_status(a.status, 1);
+    if (wave) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) partial[wave - 1u][k][lane] = acc[k];
+    }
+    __syncthreads();
+    if (wave) return;
+    const unsigned long long out_in = (unsigned long long)blockIdx.y * 16ull + i16;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        // accumulator k of lane (i, q): weight row 4 q + k, input row i
+        const unsigned long long row = (unsigned long long)blockIdx.x * 16ull + 4u * q + k;
+        float sum = acc[k];
+#pragma unroll
+        for (unsigned wv = 0; wv + 1u < WAVES; ++wv) sum += partial[wv][k][lane];
+        if (row >= a.row_count || out_in >= a.input_rows) continue;
+        if (a.parts) {
+            a.parts[((unsigned long long)blockIdx.z * a.input_rows + out_in) * a.row_count + row] = sum;
+            continue;
+        }
+        if (!finite_f32(sum) && *a.status == 0)
+            sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
+                              (const float *)a.input + out_in * a.input_stride, a.row_width);
+        matvec_publish(a, out_in, row, sum);
+    }
+}
+
+// Second launch of a split projection: the partial sums of one output added in split order.
+__global__ __launch_bounds__(256) void matvec_f32_join_kernel(MatvecArgs a, unsigned splits)
+{
+    const unsigned long long outputs = a.input_rows * a.row_count;
+    const unsigned long long at = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    if (at >= outputs) return;
+    const unsigned long long in = at / a.row_count, row = at % a.row_count;
+    float sum = a.parts[at];
+    for (unsigned z = 1; z < splits; ++z) sum += a.parts[z * outputs + at];
+    if (!finite_f32(sum) && *a.status == 0)
+        sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
+                          (const float *)a.input + in * a.input_stride, a.row_width);
+    matvec_publish(a, in, row, sum);
+}
+
 // int32 block sums of the Q8_K path, produced by the same unit code the matvec runs.
 template <unsigned QT>
 __global__ __launch_bounds__(256) void block_dots_kernel(
@@ -383,7 +486,7 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (row_width > 0xffffffffull * 32ull) return ST_BOUNDS;
     if (((uintptr_t)input & 3u) || ((uintptr_t)out & 3u)) return ST_INVALID_ARG;
     MatvecArgs a{encoded, row_count, row_width, row_bytes, input, input_rows, input_stride,
-                 additive, out, out_stride, output_bf16, status};
+                 additive, out, out_stride, output_bf16, status, nullptr};
     hipStream_t s = as_stream(stream);
     const bool scalar = qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16 || qtype == QT_I32;
     if (input_q8 && (scalar || row_width % 256u)) return ST_UNSUPPORTED;
@@ -405,6 +508,13 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (qtype == QT_Q4_K && input_q8 && input_rows >= 16ull && !((uintptr_t)encoded & 15u))
         return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
                                      out, out_stride, output_bf16 != 0, status, s);
+    if (qtype == QT_F32 && input_rows >= 8ull && input_rows < 256ull && row_width % 256ull == 0ull &&
+        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
+        const unsigned long long grid_x = (row_count + 15ull) / 16ull, grid_y = (input_rows + 15ull) / 16ull;
+        if (grid_x > 0x7fffffffull) return ST_BOUNDS;
+        matvec_f32_tile16_kernel<16><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
+        return check_launch("matvec_f32_tile16");
+    }
     if (qtype == QT_F32 && input_rows >= 32ull && row_width % 32ull == 0ull &&
         !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
         const unsigned long long grid_x = (row_count + 31ull) / 32ull, grid_y = (input_rows + 31ull) / 32ull;
@@ -497,4 +607,46 @@ extern "C" int yvex_hip_row_dot(const uint8_t *encoded, unsigned int qtype, cons
     if (elements % block) return ST_BOUNDS;
     row_dot_serial_kernel<<<1, 1, 0, as_stream(stream)>>>(encoded, vector, elements, qtype, out);
     return check_launch("row_dot");
+}
+
+// Splits of an F32 projection over a decode-width batch: per-wave shares of 128 columns.
+static unsigned f32_rows_splits(uint64_t row_width, uint64_t input_rows)
+{
+    if (input_rows < 8u || input_rows >= 256u || row_width % 512u) return 0u;
+    const uint64_t splits = row_width / 512u;
+    return splits >= 2u && splits <= 64u ? (unsigned)splits : 0u;
+}
+
+extern "C" uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64_t row_width,
+                                                      uint64_t input_rows)
+{
+    const unsigned splits = f32_rows_splits(row_width, input_rows);
+    return splits ? (uint64_t)splits * input_rows * row_count * sizeof(float) : 0u;
+}
+
+extern "C" int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t row_width,
+                                        const float *input, uint64_t input_rows, uint64_t input_stride,
+                                        const float *additive, float *out, uint64_t out_stride,
+                                        int output_bf16, void *scratch, uint64_t scratch_bytes,
+                                        int *status, yvex_hip_stream stream)
+{
+    const unsigned splits = f32_rows_splits(row_width, input_rows);
+    const uint64_t need = yvex_hip_matvec_f32_scratch_bytes(row_count, row_width, input_rows);
+    if (!splits || !scratch || scratch_bytes < need || ((uintptr_t)scratch & 3u) ||
+        (((uintptr_t)weights | (uintptr_t)input) & 15u) || (input_stride & 3ull) || !weights || !input ||
+        !out || !status || !row_count || out_stride < row_count || input_stride < row_width)
+        return yvex_hip_matvec((const uint8_t *)weights, QT_F32, row_count, row_width, row_width * 4u, input, 0,
+                               input_rows, input_stride, additive, out, out_stride, output_bf16, status,
+                               stream);
+    MatvecArgs a{(const unsigned char *)weights, row_count, row_width, row_width * 4u, input, input_rows,
+                 input_stride, additive, out, out_stride, output_bf16, status, (float *)scratch};
+    hipStream_t s = as_stream(stream);
+    const uint64_t grid_x = (row_count + 15u) / 16u, grid_y = (input_rows + 15u) / 16u;
+    const uint64_t outputs = input_rows * row_count;
+    if (grid_x > 0x7fffffffull || (outputs + 255u) / 256u > 0x7fffffffull) return ST_BOUNDS;
+    matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y, splits), 256, 0, s>>>(a);
+    int rc = check_launch("matvec_f32_rows.parts");
+    if (rc) return rc;
+    matvec_f32_join_kernel<<<(unsigned)((outputs + 255u) / 256u), 256, 0, s>>>(a, splits);
+    return check_launch("matvec_f32_rows.join");
 }

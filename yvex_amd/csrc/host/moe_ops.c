@@ -696,7 +696,18 @@ sequence:
         activations = AT(normalized);
         combined_target = AT(combined);
     }
-    /* router: logits = router . row (F32 activations, as src/backend/cuda/moe.c:1259-1284) */
+    /* router: logits = router . row (F32 activations, as src/backend/cuda/moe.c:1259-1284). F32
+     * router weights over a decode-width batch are split over the whole device; their partial
+     * sums use the pair-output range, which nothing else touches before the down projection. */
+    if (views[YVEX_MOE_WEIGHT_ROUTER].qtype == YVEX_GGUF_QTYPE_F32) {
+        unsigned long long need = yvex_hip_matvec_f32_scratch_bytes(experts, hidden, row_count);
+        int split = need && need <= pairs * hidden * sizeof(float);
+        LAUNCH(yvex_hip_matvec_f32_rows((const float *)(uintptr_t)router_address, experts, hidden,
+                                        (const float *)activations, row_count, hidden, NULL,
+                                        (float *)AT(logits), experts, 0, split ? AT(pair_outputs) : NULL,
+                                        split ? need : 0ull, (int *)status, stream), "rocm.moe.rows.router");
+        if (rc == YVEX_OK && split && graph_mode != GRAPH_REPLAY) launches++;   /* partials, then their sum */
+    } else
     LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)router_address, views[YVEX_MOE_WEIGHT_ROUTER].qtype,
                            experts, hidden, views[YVEX_MOE_WEIGHT_ROUTER].row_bytes,
                            activations, 0, row_count, hidden, NULL, (float *)AT(logits),

@@ -91,6 +91,28 @@ def matvec(encoded, qtype, row_count, row_width, inputs, *, input_q8=False, inpu
     return out
 
 
+def matvec_f32_rows(weights, inputs, status, *, additive=None, output_bf16=False, scratch=None, out=None):
+    """F32 weight rows [rows, width] against F32 input rows with the split-projection scratch:
+    None allocates what yvex_hip_matvec_f32_scratch_bytes asks for, False passes none."""
+    row_count, row_width = weights.shape
+    input_rows = inputs.shape[0]
+    lib = load_library()
+    lib.yvex_hip_matvec_f32_scratch_bytes.restype = C.c_uint64
+    need = lib.yvex_hip_matvec_f32_scratch_bytes(C.c_uint64(row_count), C.c_uint64(row_width),
+                                                 C.c_uint64(input_rows))
+    if scratch is None and need:
+        scratch = torch.empty(need, dtype=torch.uint8, device=weights.device)
+    if scratch is False:
+        scratch = None
+    if out is None:
+        out = torch.empty((input_rows, row_count), dtype=torch.float32, device=weights.device)
+    _call("yvex_hip_matvec_f32_rows", _ptr(weights), C.c_uint64(row_count), C.c_uint64(row_width),
+          _ptr(inputs), C.c_uint64(input_rows), C.c_uint64(inputs.stride(0)), _ptr(additive), _ptr(out),
+          C.c_uint64(row_count), C.c_int(int(output_bf16)), _ptr(scratch),
+          C.c_uint64(scratch.numel() if scratch is not None else 0), _ptr(status), _stream())
+    return out
+
+
 def block_dots_i32(encoded, qtype, row_count, row_width, act_q8, input_rows, status):
     blocks = row_width // 256
     shape = (input_rows, row_count, blocks * 8) if qtype == Q8_0 else (input_rows, row_count, blocks, 2)
