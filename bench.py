@@ -27,8 +27,11 @@ HBM_PEAK_GBS = 8000.0
 MFMA_INT8_PEAK_TOPS = 5000.0
 HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
 EXPERT_BYTES = 3 * 3_784_704   # gate + up + down of one IQ2_XXS expert
-# iq2_sweep_kernel<fused>: FETCH_SIZE 632 787 x 2.000 KiB + WRITE_SIZE 15 782 x 1.000 KiB per launch
-GATE_UP_TRAFFIC_BYTES = int((605_830 * 2.0 + 13_760) * 1024)
+# iq2_sweep_kernel<fused gate/up>, 159 distinct routed experts + the shared one: FETCH_SIZE
+# 609 747 x 2.000 KiB + WRITE_SIZE 13 760 x 1.000 KiB per launch (counter units scaled by a 1 GiB
+# read kernel and a 256 MiB fill kernel in the same runs)
+GATE_UP_TRAFFIC_BYTES = int((609_747 * 2.0 + 13_760) * 1024)
+GATE_UP_TRAFFIC_EXPERTS = 159
 
 
 def synth_iq2xxs(torch, blocks: int, device, seed: int):
@@ -54,7 +57,7 @@ def event_ms(torch, fn, repeats: int) -> float:
 
 def device_clock(torch, dev):
     """Clock of the matrix cores under full load, from a launch of known length in cycles
-    (every SIMD runs a chain of dependent 32-cycle matrix instructions), next to the clock the
+    (every SIMD runs back-to-back 32-cycle matrix instructions on four accumulators), next to the clock the
     device properties name. Fractions of the matrix-core peak are quoted against the published
     peak, which assumes the peak engine clock (2.4 GHz): the measured clock says how much of a
     gap is frequency."""
@@ -75,7 +78,7 @@ def device_clock(torch, dev):
     return {"matrix_load_ghz": round(chain * 32 / (ms * 1e6), 3),
             "device_peak_engine_mhz": round(engine.value / 1e3, 1),
             "device_peak_memory_mhz": round(memory.value / 1e3, 1),
-            "probe": f"{chain} dependent V_MFMA_I32_32X32X32_I8 per SIMD on every compute unit, "
+            "probe": f"{chain} back-to-back V_MFMA_I32_32X32X32_I8 per SIMD on every compute unit, "
                      f"32 cycles each, {round(ms, 3)} ms"}
 
 
@@ -670,7 +673,7 @@ def main() -> int:
                      # HBM bytes per launch of this kernel on this workload from the FETCH_SIZE and
                      # WRITE_SIZE counter runs summarised under profiles/ (scaled by the plain
                      # copy kernels of known size in the same runs); null for other settings
-                     "traffic": GATE_UP_TRAFFIC_BYTES if (args.act == "q8k" and unique == 158) else None,
+                     "traffic": GATE_UP_TRAFFIC_BYTES if (args.act == "q8k" and unique == GATE_UP_TRAFFIC_EXPERTS) else None,
                      "launch_ms": round(up_ms, 4), "algorithmic_bytes": up_bytes},
         "kernels_ms": {"gate_up_sweep": round(up_ms, 4), "down_sweep": round(down_ms, 4),
                        "gate_up_sweep_median": round(up_median_ms, 4), "down_sweep_median": round(down_median_ms, 4),

@@ -266,11 +266,11 @@ int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,
  * Time it with events; `sink` is a 4-byte device word that is practically never written. */
 int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_hip_stream stream);
 
-/* Clock probe, the companion of the bandwidth probe: every SIMD of the device runs `chain`
- * dependent 32x32x32 int8 matrix instructions (32 shader cycles each), so the launch lasts
- * chain * 32 cycles; timed with events it gives the clock under matrix-core load, the figure a
- * fraction of the matrix-core peak has to be read with. `sink` is a device word that is
- * practically never written. */
+/* Clock probe, the companion of the bandwidth probe: every SIMD of the device runs `chain` (a
+ * multiple of 4) 32x32x32 int8 matrix instructions on four accumulators in turn, each taking the
+ * matrix pipe for 32 shader cycles, so the launch lasts chain * 32 cycles; timed with events it
+ * gives the clock under matrix-core load, the figure a fraction of the matrix-core peak has to
+ * be read with. `sink` is a device word that is practically never written. */
 int yvex_hip_clock_probe(uint64_t chain, int *sink, yvex_hip_stream stream);
 
 /* Device-side fill, usable where a captured graph must not hold a memset node. */

@@ -73,18 +73,25 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4 *__restric
     if (fold == 0x9e3779b9u) *sink = fold;   // practically never true; keeps the loads alive
 }
 
-// A chain of dependent 32x32x32 int8 matrix instructions, one wave per SIMD on every compute
-// unit: each takes 8 passes of 4 cycles and the next cannot start before it, so a launch lasts
+// Back-to-back 32x32x32 int8 matrix instructions on four independent accumulators, one wave per
+// SIMD on every compute unit: the matrix pipe takes 8 passes of 4 cycles for each, and with four
+// accumulators in turn no instruction waits for the one before it, so a launch lasts
 // chain * 32 shader cycles and its duration gives the clock the matrix cores run at under load.
+// (A single accumulator would measure the 56-cycle dependent latency instead.)
 __global__ __launch_bounds__(256) void clock_probe_kernel(uint64_t chain, int *sink)
 {
     typedef int v4i __attribute__((ext_vector_type(4)));
     typedef int v16i __attribute__((ext_vector_type(16)));
     v4i a = {(int)threadIdx.x, 1, 2, 3}, b = {3, 2, 1, (int)blockIdx.x};
-    v16i acc = {0};
-    for (uint64_t i = 0; i < chain; ++i)
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
-    if (acc[0] == 0x7fffffff && acc[5] == 0x7ffffffe) *sink = acc[3];   // practically never
+    v16i acc0 = {0}, acc1 = {0}, acc2 = {0}, acc3 = {0};
+    for (uint64_t i = 0; i < chain; i += 4u) {
+        acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc2, 0, 0, 0);
+        acc3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc3, 0, 0, 0);
+    }
+    const int folded = acc0[0] ^ acc1[1] ^ acc2[2] ^ acc3[3];
+    if (folded == 0x7fffffff && acc0[5] == 0x7ffffffe) *sink = folded;   // practically never
 }
 
 __global__ void probe_kernel(int *out)
@@ -223,7 +230,7 @@ int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_
 
 int yvex_hip_clock_probe(uint64_t chain, int *sink, yvex_hip_stream stream)
 {
-    if (!chain || !sink) return ST_INVALID_ARG;
+    if (!chain || (chain & 3u) || !sink) return ST_INVALID_ARG;
     clock_probe_kernel<<<compute_units(), 256, 0, as_stream(stream)>>>(chain, sink);
     return check_launch("clock_probe");
 }
