@@ -25,22 +25,13 @@
 
 namespace yvex {
 
-#ifndef YVEX_SWEEP_WAVES
-#define YVEX_SWEEP_WAVES 8
-#endif
-#ifndef YVEX_SWEEP_ITERS
-#define YVEX_SWEEP_ITERS 32
-#endif
-#ifndef YVEX_SWEEP_AHEAD_SMALL
-#define YVEX_SWEEP_AHEAD_SMALL 1
-#endif
-#ifndef YVEX_SWEEP_PAIRS
-#define YVEX_SWEEP_PAIRS 4
-#endif
-constexpr unsigned kSweepWaves = YVEX_SWEEP_WAVES;
+constexpr unsigned kSweepWaves = 8u;           // two per SIMD: the sweep of four pairs needs their registers
 constexpr unsigned kSweepThreads = kSweepWaves * 64u;
-constexpr int kSweepPairs = YVEX_SWEEP_PAIRS;  // pairs of one bucket served by one sweep (2..4)
-constexpr unsigned kSweepIters = YVEX_SWEEP_ITERS;          // weight-row iterations per work item
+constexpr int kSweepPairs = 4;                 // pairs of one bucket served by one sweep
+constexpr unsigned kSweepIters = 32u;          // weight-row iterations per work item
+constexpr int kSweepAheadSmall = 1;            // rows requested ahead of the one decoded, sweeps of one or two pairs
+constexpr unsigned kSweepLongPercent = 75u;    // share of the weight rows that goes out in full-length items
+constexpr unsigned kSweepShortDiv = 2u;        // the rest goes out in items of 1 / kSweepShortDiv of that length
 
 // LDS map (byte addresses; the dynamic block starts at LDS address 0)
 constexpr unsigned kMagBase = 0u;              // 256 entries x 16 replicas x {+lo, +hi, -lo, -hi}
@@ -335,7 +326,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
     // final row) and every lane stores (lanes that hold no result write to a spare word), so no
     // branch sits between a request and the wait that consumes it and the waits stay counted.
-    constexpr int AHEAD = N <= 2 ? YVEX_SWEEP_AHEAD_SMALL : 1;   // rows requested ahead of the one decoded
+    constexpr int AHEAD = N <= 2 ? kSweepAheadSmall : 1;   // rows requested ahead of the one decoded
     constexpr int STREAMS = FUSED ? 2 : 1;
     Iq2Half ring[AHEAD + 1][STREAMS];
     const unsigned last = iterations - 1u;
@@ -512,15 +503,9 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     // into short ones that come last in the item list: the waves of the grid finish within a short
     // item of each other instead of a long one, and only the short items pay the fixed cost of an
     // item (its activation columns, the first requests, the finishing pass) more often.
-#ifndef YVEX_SWEEP_LONG_PERCENT
-#define YVEX_SWEEP_LONG_PERCENT 75
-#endif
-#ifndef YVEX_SWEEP_SHORT_DIV
-#define YVEX_SWEEP_SHORT_DIV 2
-#endif
     const unsigned item_rows = kSweepIters * g.rows_per_iter;
-    const unsigned short_rows = item_rows / YVEX_SWEEP_SHORT_DIV;
-    const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * YVEX_SWEEP_LONG_PERCENT / 100u / item_rows);
+    const unsigned short_rows = item_rows / kSweepShortDiv;
+    const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * kSweepLongPercent / 100u / item_rows);
     const unsigned long_rows = long_tiles * item_rows;
     const unsigned short_tiles = (a.out_rows - long_rows + short_rows - 1u) / short_rows;
 
