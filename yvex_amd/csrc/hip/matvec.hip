@@ -54,17 +54,26 @@ __device__ float matvec_recover_f64(const unsigned char *row, const float *x,
 // chunk (weights, then the activation bytes that go with them), which bounds a long matrix such as
 // an output head well below what the same loads reach when nothing waits on them.
 // EVEN: every row starts on an even address (even base address and even row bytes).
-template <unsigned QT, bool Q8, int T, int U, bool EVEN>
+// STAGE (one F32 input row): the workgroup copies the input row into LDS once, 16-byte pieces
+// swizzled inside each 128-byte unit, and its four waves read their units from there. A lane owns
+// 32 consecutive values, so read from global memory each of its eight 16-byte loads touches 64
+// different cache lines, which the memory pipeline serves at about two cycles a line.
+template <unsigned QT, bool Q8, int T, int U, bool EVEN, bool STAGE = false>
 __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
 {
     __shared__ Iq2Tables tables;
-    if constexpr (QT == QT_IQ2_XXS) {
-        iq2_tables_fill(tables);
-        __syncthreads();
+    extern __shared__ __align__(16) float4 staged_row[];
+    const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
+    if constexpr (STAGE) {
+        const float4 *source = reinterpret_cast<const float4 *>((const float *)a.input + in0 * a.input_stride);
+        const unsigned pieces = (unsigned)(a.row_width >> 2);
+        for (unsigned p = threadIdx.x; p < pieces; p += 256u)
+            staged_row[(p & ~7u) | ((p ^ (p >> 3)) & 7u)] = source[p];
     }
+    if constexpr (QT == QT_IQ2_XXS) iq2_tables_fill(tables);
+    if constexpr (QT == QT_IQ2_XXS || STAGE) __syncthreads();
     const unsigned lane = threadIdx.x & 63u;
     const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
-    const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
     if (row >= a.row_count) return;
     const unsigned char *wrow = a.encoded + row * a.row_bytes;
     const unsigned units = (unsigned)(a.row_width >> 5);
@@ -108,6 +117,12 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
                         const float v = q8_0_unit_value(unit[j], act_scale, s.dot);
                         acc[t] += live[j] ? v : 0.0f;
                     }
+                } else if constexpr (STAGE) {
+                    float4 x4[8];
+#pragma unroll
+                    for (unsigned i = 0; i < 8u; ++i) x4[i] = staged_row[8u * uu[j] + (i ^ (uu[j] & 7u))];
+                    const float v = unit_dot_f32_values<QT>(unit[j], wrow, uu[j], x4);
+                    if (live[j]) acc[t] += v;
                 } else {
                     const float *x = (const float *)a.input + in * a.input_stride + 32ull * uu[j];
                     const float v = unit_dot_f32<QT>(unit[j], wrow, uu[j], x);
@@ -441,10 +456,16 @@ static int launch_block_even(const MatvecArgs &a, hipStream_t stream)
     const unsigned long long grid_x = (a.row_count + 3ull) / 4ull;
     if (grid_x > 0x7fffffffull) return ST_BOUNDS;
     if (a.input_rows == 1ull) {
-        // Q8_K activations against a matrix that takes many rounds of waves: four chunks (8192
-        // columns) in flight; a small matrix is one round and gains nothing from them
-        const bool deep = Q8 && a.row_count * a.row_bytes >= (64ull << 20);
+        // Q8_K activations: four chunks (8192 columns) in flight for a matrix that takes many
+        // rounds of waves, and for rows of more than one chunk, whose chunks would otherwise each
+        // wait a memory round trip of their own
+        const bool deep = Q8 && (a.row_count * a.row_bytes >= (64ull << 20) || a.row_width > 2048ull);
+        // one F32 input row of up to 12 288 values (48 KB) is staged in LDS
+        const bool stage = !Q8 && a.row_width <= 12288ull && !((uintptr_t)a.input & 15u);
         if (deep) matvec_block_kernel<QT, Q8, 1, Q8 ? 4 : 1, EVEN><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
+        else if (stage)
+            matvec_block_kernel<QT, Q8, 1, 1, EVEN, !Q8><<<dim3((unsigned)grid_x, 1), 256,
+                                                            (size_t)a.row_width * 4u, stream>>>(a);
         else matvec_block_kernel<QT, Q8, 1, 1, EVEN><<<dim3((unsigned)grid_x, 1), 256, 0, stream>>>(a);
     } else {
         const unsigned long long grid_y = (a.input_rows + 3ull) / 4ull;

@@ -341,14 +341,14 @@ __device__ __forceinline__ float q8_0_unit_value(const Unit &unit, float act_sca
 
 // Unit against 32 F32 activations. Returns the unit's contribution to the row dot.
 template <unsigned QT>
-__device__ __forceinline__ float unit_dot_f32(const Unit &unit, const unsigned char *row,
-                                              unsigned u, const float *x)
+__device__ __forceinline__ float unit_dot_f32_values(const Unit &unit, const unsigned char *row,
+                                                     unsigned u, const float4 (&x4)[8])
 {
     const unsigned sb = u >> 3;
     float s1 = 0.0f, s2 = 0.0f, xs1 = 0.0f, xs2 = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const float4 v = *reinterpret_cast<const float4 *>(x + 4 * i);
+        const float4 v = x4[i];
         const unsigned w = unit.w[i];
         float p = 0.0f;
         p = fmaf((float)(signed char)(w & 255u), v.x, p);
@@ -379,6 +379,16 @@ __device__ __forceinline__ float unit_dot_f32(const Unit &unit, const unsigned c
         return (d * (float)unit.factor * s1 - dm * (float)unit.min1 * xs1) +
                (d * (float)unit.factor2 * s2 - dm * (float)unit.min2 * xs2);
     }
+}
+
+template <unsigned QT>
+__device__ __forceinline__ float unit_dot_f32(const Unit &unit, const unsigned char *row,
+                                              unsigned u, const float *x)
+{
+    float4 x4[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x4[i] = *reinterpret_cast<const float4 *>(x + 4 * i);
+    return unit_dot_f32_values<QT>(unit, row, u, x4);
 }
 
 // Partial sums of one decoded unit against 32 F32 activations: halves of 16 values each, and
