@@ -142,12 +142,13 @@ def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
 
 @pytest.mark.parametrize("qtype,rows,width,inputs", [
     ("IQ2_XXS", 516, 2048, 32), ("IQ2_XXS", 260, 7168, 70), ("IQ2_XXS", 7168, 2048, 33),
-    ("Q4_K", 516, 2048, 16), ("Q4_K", 132, 7168, 70), ("Q4_K", 2048, 7168, 16), ("Q4_K", 36, 512, 200)])
+    ("Q4_K", 516, 2048, 16), ("Q4_K", 132, 7168, 70), ("Q4_K", 2048, 7168, 16), ("Q4_K", 36, 512, 200),
+    ("Q4_K", 50, 2304, 17), ("Q4_K", 24, 7168, 32), ("Q4_K", 7, 256, 31)])
 def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, width, inputs):
-    """From 16 (Q4_K) or 32 (IQ2_XXS) Q8_K input rows on, projections run on the int8 matrix cores
+    """From 2 (Q4_K) or 32 (IQ2_XXS) Q8_K input rows on, projections run on the int8 matrix cores
     (src/backend/cuda/private.h:461-464 turns the tensor-core kernels on at 16). Results are those of the
-    integer path (1e-5 of the oracle's Q8_K product), bf16 output rounds them, and an input-row
-    count below the threshold gives the sweep kernel's values to the same bar."""
+    integer path (1e-5 of the oracle's Q8_K product), bf16 output rounds them, and smaller
+    input-row counts (other kernels or tile shapes) give the same values to the same bar."""
     from yvex_amd import kernels as K
     qt = getattr(oracle, qtype)
     g = oracle.Generator(42, f"matvec.rows.{qtype}.{rows}.{width}.{inputs}")
@@ -168,11 +169,12 @@ def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, wid
     status_ok(status)
     assert np.all((rounded.view(np.uint32) & 0xffff) == 0)
     assert np.all(np.abs(rounded - got) <= np.abs(got) * 2.0 ** -8 + 1e-30)
-    # the same rows fifteen at a time take the sweep kernel: same values to the same bar
-    few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=15,
-                   status=status).cpu().numpy()
-    status_ok(status)
-    assert_close(few, got[:15], rel=1e-5, abs_=1e-5)
+    # fewer rows at a time (the sweep kernel, or another tile shape): same values to the same bar
+    for count in (15, 1):
+        few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=count,
+                       status=status).cpu().numpy()
+        status_ok(status)
+        assert_close(few, got[:count], rel=1e-5, abs_=1e-5)
 
 
 @pytest.mark.parametrize("qtype,rows,width", [("Q8_0", 9600, 7168), ("IQ2_XXS", 37000, 7168)])

@@ -258,6 +258,160 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
     }
 }
 
+// The same product for 16 to 32 input rows on V_MFMA_I32_16X16X64_I8: a workgroup owns 16
+// weight rows x 16 or 32 tokens, so a batch of 16 wastes no token slot and twice as many
+// workgroups share the matrix; eight waves (two per SIMD) take every eighth superblock. One K
+// step is a 64-value nibble group, i.e. two sub-blocks, which is fine because the limbs already
+// carry their sub-block's scale. Lane (r, q) holds bytes 16q..16q+15 of weight row r's group as
+// the A operand (q = 0, 1: low nibbles of nibble bytes 16q.., the first sub-block; q = 2, 3:
+// high nibbles of nibble bytes 16(q-2).., the second) and the same positions of token r's
+// activations as the B operand; accumulator i of that lane is weight row 4 q + i against token r.
+template <unsigned NT>
+__global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
+{
+    typedef int v4s __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) float row_scale[8][2][16];
+    __shared__ float partial[7][NT][4][64];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned r = lane & 15u, q = lane >> 4;
+    const unsigned long long row0 = (unsigned long long)blockIdx.x * 16ull;
+    const unsigned long long tok0 = (unsigned long long)blockIdx.y * (16ull * NT);
+    unsigned long long wr = row0 + r;
+    if (wr >= g.row_count) wr = g.row_count - 1ull;
+    const unsigned char *wrow = g.encoded + wr * g.row_bytes;
+    const unsigned char *arow[NT];
+    const unsigned long long act_row_bytes = (unsigned long long)g.blocks * kQ8KBytes;
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt) {
+        unsigned long long t = tok0 + 16ull * nt + r;
+        if (t >= g.input_rows) t = g.input_rows - 1ull;
+        arow[nt] = g.act + t * act_row_bytes;
+    }
+    float acc[NT][4];
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[nt][i] = 0.0f;
+
+    for (unsigned sb = wave; sb < g.blocks; sb += 8u) {
+        const unsigned char *w = wrow + (unsigned long long)sb * 144ull;
+        const unsigned head = *reinterpret_cast<const unsigned *>(w);
+        const uint3 scales = *reinterpret_cast<const uint3 *>(w + 4u);
+        uint4 qs[4];
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j)
+            qs[j] = *reinterpret_cast<const uint4 *>(w + 16u + 32u * j + 16u * (q & 1u));
+        uint4 a[NT][4], bsums[NT][2];
+        float da[NT];
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt) {
+            const unsigned char *ab = arow[nt] + (unsigned long long)sb * kQ8KBytes;
+            da[nt] = *reinterpret_cast<const float *>(ab);
+#pragma unroll
+            for (unsigned j = 0; j < 4u; ++j) {
+                const unsigned *p = reinterpret_cast<const unsigned *>(ab + 4u + 64u * j + 16u * q);
+                a[nt][j] = make_uint4(p[0], p[1], p[2], p[3]);
+            }
+            const unsigned *b = reinterpret_cast<const unsigned *>(ab + 260u);
+            bsums[nt][0] = make_uint4(b[0], b[1], b[2], b[3]);
+            bsums[nt][1] = make_uint4(b[4], b[5], b[6], b[7]);
+        }
+        const unsigned s0 = scales.x, s1 = scales.y, s2 = scales.z;
+        const unsigned sc_pack[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
+        const unsigned mn_pack[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
+        if (q == 0u) {
+            row_scale[wave][0][r] = f16_bits_to_float(head & 0xffffu);
+            row_scale[wave][1][r] = f16_bits_to_float(head >> 16);
+        }
+        v4s lo_sum[NT], hi_sum[NT];
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lo_sum[nt][i] = hi_sum[nt][i] = 0;
+        const unsigned high = q >> 1;                          // this lane decodes the high nibbles
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j) {
+            // sub-block 2 j + high: its scale is byte (2 j + high) of the packed scales
+            const unsigned sc = (sc_pack[j >> 1] >> (16u * (j & 1u) + 8u * high)) & 255u;
+            const unsigned shift = 4u * high;
+            v4i a_lo, a_hi;
+            unsigned lo, hi;
+            limbs(qs[j].x >> shift, sc, lo, hi); a_lo[0] = (int)lo; a_hi[0] = (int)hi;
+            limbs(qs[j].y >> shift, sc, lo, hi); a_lo[1] = (int)lo; a_hi[1] = (int)hi;
+            limbs(qs[j].z >> shift, sc, lo, hi); a_lo[2] = (int)lo; a_hi[2] = (int)hi;
+            limbs(qs[j].w >> shift, sc, lo, hi); a_lo[3] = (int)lo; a_hi[3] = (int)hi;
+#pragma unroll
+            for (unsigned nt = 0; nt < NT; ++nt) {
+                const v4i b = as_v4i(a[nt][j]);
+                lo_sum[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b, lo_sum[nt], 0, 0, 0);
+                hi_sum[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b, hi_sum[nt], 0, 0, 0);
+            }
+        }
+        v4i m_op = {0, 0, 0, 0};
+        if (q == 0u) {
+            m_op[0] = (int)mn_pack[0];
+            m_op[1] = (int)mn_pack[1];
+        }
+        v4s min_lo[NT], min_hi[NT];
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt) {
+            uint2 bl, bh;
+            bsum_limbs(bsums[nt], bl, bh);
+            v4i b_lo = {0, 0, 0, 0}, b_hi = {0, 0, 0, 0};
+            if (q == 0u) {
+                b_lo[0] = (int)bl.x; b_lo[1] = (int)bl.y;
+                b_hi[0] = (int)bh.x; b_hi[1] = (int)bh.y;
+            }
+            const v4s zero = {0, 0, 0, 0};
+            min_lo[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(m_op, b_lo, zero, 0, 0, 0);
+            min_hi[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(m_op, b_hi, zero, 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const float4 d4 = *reinterpret_cast<const float4 *>(&row_scale[wave][0][4u * q]);
+        const float4 m4 = *reinterpret_cast<const float4 *>(&row_scale[wave][1][4u * q]);
+        const float d_of[4] = {d4.x, d4.y, d4.z, d4.w}, dmin_of[4] = {m4.x, m4.y, m4.z, m4.w};
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dot = (hi_sum[nt][i] << 7) + lo_sum[nt][i];
+                const int minimum = (min_hi[nt][i] << 7) + min_lo[nt][i];
+                const float left = (da[nt] * d_of[i]) * (float)dot;
+                const float right = (da[nt] * dmin_of[i]) * (float)minimum;
+                acc[nt][i] += left - right;
+            }
+    }
+
+    if (wave) {
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) partial[wave - 1u][nt][i][lane] = acc[nt][i];
+    }
+    __syncthreads();
+    if (wave) return;
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt) {
+        const unsigned long long token = tok0 + 16ull * nt + r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned long long row = row0 + 4u * q + (unsigned)i;
+            float sum = acc[nt][i];
+#pragma unroll
+            for (unsigned wv = 0; wv < 7u; ++wv) sum += partial[wv][nt][i][lane];
+            if (row >= g.row_count || token >= g.input_rows) continue;
+            const unsigned long long at = token * g.out_stride + row;
+            const float value = g.additive ? sum + g.additive[at] : sum;
+            if (!finite_f32(value)) raise_status(g.status, 1);
+            else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
+        }
+    }
+}
+
 }  // namespace
 
 int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
@@ -274,7 +428,10 @@ int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t r
                    (const unsigned char *)act_q8k, input_rows, additive, out, out_stride,
                    output_bf16 ? 1 : 0, status};
     if (input_rows <= 32u) {
-        dense_q4k_kernel<1><<<dim3((unsigned)row_tiles, 1), 256, 0, stream>>>(g);
+        const uint64_t small_tiles = (row_count + 15u) / 16u;
+        if (small_tiles > 0x7fffffffull) return ST_BOUNDS;
+        if (input_rows <= 16u) dense_q4k16_kernel<1><<<dim3((unsigned)small_tiles, 1), 512, 0, stream>>>(g);
+        else dense_q4k16_kernel<2><<<dim3((unsigned)small_tiles, 1), 512, 0, stream>>>(g);
     } else {
         const uint64_t token_tiles = (input_rows + 63u) / 64u;
         if (token_tiles > 65535ull) return ST_BOUNDS;
