@@ -44,6 +44,17 @@ def synth_iq2xxs(torch, blocks: int, device, seed: int):
     return raw.reshape(-1)
 
 
+def synth_q4k(torch, blocks: int, device, seed: int):
+    """Random Q4_K superblocks: uniform scale, minimum and nibble bytes, small positive fp16 d and dmin."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 144), dtype=torch.uint8, device=device, generator=gen)
+    d = (torch.rand(blocks, device=device, generator=gen) * 1.0e-4 + 2.0e-5).to(torch.float16)
+    raw[:, 0:2] = d.view(torch.uint8).reshape(blocks, 2)
+    raw[:, 2:4] = raw[:, 0:2]
+    return raw.reshape(-1)
+
+
 def event_ms(torch, fn, repeats: int) -> float:
     """Average duration of fn() in ms, measured with events on the current (launch) stream."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -167,7 +178,7 @@ class AbiLayer:
     phase barrier complete_rows (the reference completes all pending layers of a phase with one
     call, src/runtime/moe.c:1567-1576)."""
 
-    def __init__(self, torch, routed, shared, router, x_host, rows):
+    def __init__(self, torch, routed, shared, router, x_host, rows, qtype=16):
         import ctypes as C
         import numpy as np
         from yvex_amd import abi
@@ -187,7 +198,8 @@ class AbiLayer:
         plan.requires_correction_bias, plan.normalize_topk_probabilities = 0, 1
         job = self.job = abi.LayerJob()
         job.layer = C.pointer(plan)
-        rb_h, rb_i = HIDDEN // 256 * 66, INTERMEDIATE // 256 * 66
+        block_bytes = {16: 66, 12: 144}[qtype]
+        rb_h, rb_i = HIDDEN // 256 * block_bytes, INTERMEDIATE // 256 * block_bytes
 
         def view(slot, tensor, qtype, width, count, row_bytes, activation):
             v = job.weights[slot]
@@ -199,12 +211,12 @@ class AbiLayer:
 
         enc = abi.ACT_DEVICE_ENCODED
         view(abi.W_ROUTER, router, 0, HIDDEN, EXPERTS, HIDDEN * 4, abi.ACT_DEVICE_F32)
-        view(abi.W_ROUTED_GATE, routed[0], 16, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
-        view(abi.W_ROUTED_UP, routed[1], 16, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
-        view(abi.W_ROUTED_DOWN, routed[2], 16, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc)
-        view(abi.W_SHARED_GATE, shared[0], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
-        view(abi.W_SHARED_UP, shared[1], 16, HIDDEN, INTERMEDIATE, rb_h, enc)
-        view(abi.W_SHARED_DOWN, shared[2], 16, INTERMEDIATE, HIDDEN, rb_i, enc)
+        view(abi.W_ROUTED_GATE, routed[0], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
+        view(abi.W_ROUTED_UP, routed[1], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc)
+        view(abi.W_ROUTED_DOWN, routed[2], qtype, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc)
+        view(abi.W_SHARED_GATE, shared[0], qtype, HIDDEN, INTERMEDIATE, rb_h, enc)
+        view(abi.W_SHARED_UP, shared[1], qtype, HIDDEN, INTERMEDIATE, rb_h, enc)
+        view(abi.W_SHARED_DOWN, shared[2], qtype, INTERMEDIATE, HIDDEN, rb_i, enc)
         self.ops = self.b.lib.yvex_rocm_backend_moe_operations_get(self.b.handle).contents
         need, err = abi.ULL(), abi.Error()
         if self.ops.workspace_required(C.byref(plan), rows, C.byref(need), C.byref(err)) != 0:
@@ -390,7 +402,7 @@ def tile_classes(populations):
     return out
 
 
-def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: int):
+def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: int, qt=16):
     """BASELINE config 4: the same layer over 2048 rows whose top-8 experts follow a Zipf(1.1)
     popularity (Gumbel top-k over log-popularity logits), row-batch kernels on the int8 matrix
     cores. Ops counted: 2 * (2*I*H + H*I) per (row, expert) pair, routed and shared."""
@@ -408,7 +420,6 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     router = (xd.T @ torch.linalg.solve(xd @ xd.T, wanted.double())).T.float().contiguous()
     logits = K.matvec(router.view(torch.uint8).reshape(-1), K.F32, EXPERTS, HIDDEN, x,
                       status=K.new_status(dev))
-    qt = K.IQ2_XXS
     layer = MoeLayer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                      qtypes=(qt, qt, qt), routed=weights, shared=shared, bias=None,
                      scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0, act_q8=True,
@@ -430,7 +441,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     # the same step through include/yvex_rocm.h (router projection included)
     stage_rows = layer.run(x, logits).clone()
     torch.cuda.synchronize()
-    abi_layer = AbiLayer(torch, weights, shared, router, x.cpu().numpy(), rows)
+    abi_layer = AbiLayer(torch, weights, shared, router, x.cpu().numpy(), rows, qtype=qt)
     abi_layer.step(defer=False)
     abi_same = bool((torch.from_numpy(abi_layer.output()) == stage_rows.cpu()).all().item())
     abi_unique = int(abi_layer.result.unique_experts)
@@ -444,7 +455,8 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     up_ops = 2 * 2 * INTERMEDIATE * HIDDEN * pairs
     populations = layer.worklist.bucket_populations[: int(layer.worklist.counts[0].item())]
     return {
-        "workload": "moe_prefill_iq2xxs: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, Q8_K activations",
+        "workload": f"moe_prefill_{'iq2xxs' if qt == 16 else 'q4k'}: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, "
+                    "Q8_K activations",
         "ms_per_step": round(step_ms, 4), "tokens_per_s": round(rows / (step_ms * 1e-3), 1),
         "c_abi": {"entry": "yvex_rocm_backend_moe_operations_get()->execute_rows + complete_rows",
                   "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
@@ -456,7 +468,8 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
         "distinct_routed_experts": int(populations.numel()),
         "token_tiles": tile_classes(populations.cpu().tolist()),
         "max_bucket_population": int(populations.max().item()),
-        "roofline": {"bound": "mfma", "kernel": "mfma_iq2_kernel<fused gate/up>",
+        "roofline": {"bound": "mfma",
+                     "kernel": "mfma_iq2_kernel<fused gate/up>" if qt == 16 else "grouped_q4k_kernel<fused gate/up>",
                      "achieved": round(up_ops / (up_ms * 1e-3) / 1e12, 2), "peak": MFMA_INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": round(up_ops / (up_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
                      "launch_ms": round(up_ms, 4)},
@@ -684,6 +697,18 @@ def main() -> int:
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)
+    if not args.no_prefill:
+        # config 4's second weight format: the same layer with Q4_K experts (6.3 GB of them)
+        del layer, gate, up, down, shared
+        torch.cuda.empty_cache()
+        q4_blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
+        q4_routed = tuple(synth_q4k(torch, q4_blocks, dev, 21 + i) for i in range(3))
+        q4_shared = tuple(synth_q4k(torch, INTERMEDIATE * HIDDEN // 256, dev, 31 + i) for i in range(3))
+        out["prefill_q4k"] = prefill_leg(torch, K, MoeLayer, q4_routed, q4_shared, dev,
+                                         max(3, args.steps // 10), 2, qt=K.Q4_K)
+        del q4_routed, q4_shared
+        torch.cuda.empty_cache()
+        layer = gate = up = down = shared = None
     if not args.no_dense:
         del layer, gate, up, down, shared
         torch.cuda.empty_cache()

@@ -261,6 +261,30 @@ int yvex_rocm_backend_query_capability(const yvex_rocm_backend *backend,
                                   yvex_backend_operation_variant variant,
                                   yvex_backend_capability_result *out, yvex_error *err);
 
+/* include/yvex/internal/backend.h:174-185,302: what the device sustains, measured at the
+ * caller's request (the reference publishes it in its backend report, src/backend/core.c:1801).
+ * Five samples each of four streaming reads and four device-to-device copies of a 1 GiB working
+ * set (allocated for the probe and released again); the rates are working set x iterations over
+ * the median sample, the copy counting its payload once. A discrete-HBM device has no coherent
+ * host path: those fields stay zero. The identity fields are the reference runtime's SHA-256
+ * seals and stay empty here. */
+#ifndef YVEX_ROCM_REFERENCE_TYPES
+#define YVEX_BACKEND_BANDWIDTH_SCHEMA_V1 1u
+#define YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT 5u
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long working_set_bytes, iterations, sample_count;
+    unsigned long long stream_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long copy_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long coherent_host_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long sustainable_read_bytes_per_second, sustainable_copy_bytes_per_second;
+    unsigned long long sustainable_coherent_host_bytes_per_second;
+    char kernel_bundle_identity[65], identity[65];
+} yvex_backend_bandwidth_evidence;
+#endif
+int yvex_rocm_backend_bandwidth_probe(yvex_rocm_backend *backend, yvex_backend_bandwidth_evidence *out,
+                                      yvex_error *err);
+
 /* include/yvex/backend.h:177-204 */
 int yvex_rocm_backend_tensor_alloc(yvex_rocm_backend *backend, const yvex_backend_tensor_desc *desc,
                               yvex_device_tensor **out, yvex_error *err);

@@ -266,6 +266,12 @@ int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,
  * Time it with events; `sink` is a 4-byte device word that is practically never written. */
 int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_hip_stream stream);
 
+/* One timed sample of the bandwidth probe: `iterations` streaming reads of `bytes` (destination
+ * NULL; `sink` as for yvex_hip_stream_read) or `iterations` device-to-device copies of `bytes`,
+ * bracketed by events on the stream; the call waits for the second event. */
+int yvex_hip_bandwidth_sample(const void *source, void *destination, uint64_t bytes, uint64_t iterations,
+                              uint32_t *sink, uint64_t *elapsed_ns, yvex_hip_stream stream);
+
 /* Clock probe, the companion of the bandwidth probe: every SIMD of the device runs `chain` (a
  * multiple of 4) 32x32x32 int8 matrix instructions on four accumulators in turn, each taking the
  * matrix pipe for 32 shader cycles, so the launch lasts chain * 32 cycles; timed with events it

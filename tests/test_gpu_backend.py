@@ -196,6 +196,27 @@ def test_bundle_failure_seam_is_fail_closed(gpu, monkeypatch):
     assert b.close() == 0
 
 
+def test_bandwidth_probe_publishes_sustainable_rates(backend):
+    """include/yvex/internal/backend.h:174-185: five timed samples of streaming reads and of
+    device-to-device copies; the published rates are the working set over the median sample."""
+    evidence, err = abi.BandwidthEvidence(), abi.Error()
+    rc = backend.lib.yvex_rocm_backend_bandwidth_probe(backend.handle, C.byref(evidence), C.byref(err))
+    assert rc == 0, err.message
+    assert evidence.schema_version == 1 and evidence.sample_count == 5 and evidence.working_set_bytes == 1 << 30
+    reads, copies = sorted(evidence.stream_elapsed_ns), sorted(evidence.copy_elapsed_ns)
+    assert reads[0] > 0 and copies[0] > 0
+    moved = evidence.working_set_bytes * evidence.iterations
+    assert abs(evidence.sustainable_read_bytes_per_second - moved * 1e9 / reads[2]) <= 2
+    assert abs(evidence.sustainable_copy_bytes_per_second - moved * 1e9 / copies[2]) <= 2
+    # an HBM3E part: terabytes a second, and below the 8 TB/s peak
+    assert 1e12 < evidence.sustainable_read_bytes_per_second < 8e12
+    assert 0.5e12 < evidence.sustainable_copy_bytes_per_second < 8e12
+    assert list(evidence.coherent_host_elapsed_ns) == [0] * 5
+    print(f"read {evidence.sustainable_read_bytes_per_second / 1e12:.2f} TB/s, "
+          f"copy {evidence.sustainable_copy_bytes_per_second / 1e12:.2f} TB/s")
+    assert backend.lib.yvex_rocm_backend_bandwidth_probe(backend.handle, None, C.byref(err)) == abi.INVALID_ARG
+
+
 def test_encoded_gather(backend, oracle):
     b = backend
     rows, width = 40, 512
@@ -502,10 +523,11 @@ def test_execute_rows_hash_router(backend, oracle, streams):
     case.tokens[2] = 1
 
 
-def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle):
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q4_K"])
+def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle, qtype):
     """Row batches whose buckets average eight pairs or more run the int8 matrix-core kernels
     (routed and shared expert); the result is the CPU layer's, to the same bar."""
-    case = MoeCase(backend, oracle, qtype="IQ2_XXS", hidden=768, intermediate=512, experts=4, topk=2,
+    case = MoeCase(backend, oracle, qtype=qtype, hidden=768, intermediate=512, experts=4, topk=2,
                    rows=200, scoring=abi.SCORING_SIGMOID)
     backend.workspace(case.workspace_bytes)
     rc = case.execute()

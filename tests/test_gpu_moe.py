@@ -71,6 +71,12 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
     # with 32-pair tiles; three superblocks with 64-pair tiles
     ("IQ2_XXS", 1280, 256, 4, 2, 40, True, 1, True),
     ("IQ2_XXS", 768, 768, 4, 2, 100, True, 0, True),
+    # Q4_K experts on the matrix cores: tiny buckets, buckets of several 32-pair tiles, real
+    # widths, five superblocks a row (the four waves of a tile get two, one, one, one)
+    ("Q4_K", 512, 512, 8, 3, 6, True, 1, True),
+    ("Q4_K", 768, 512, 4, 2, 300, True, 0, True),
+    ("Q4_K", 7168, 2048, 12, 4, 10, True, 1, True),
+    ("Q4_K", 1280, 256, 4, 2, 40, True, 1, True),
 ])
 def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, topk, rows, act_q8,
                              scoring, matrix_cores):

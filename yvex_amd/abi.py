@@ -45,6 +45,15 @@ class MemoryStats(C.Structure):
                                    "peak_allocated_bytes", "memory_limit_bytes")]
 
 
+class BandwidthEvidence(C.Structure):
+    _fields_ = [("schema_version", C.c_uint), ("working_set_bytes", ULL), ("iterations", ULL),
+                ("sample_count", ULL), ("stream_elapsed_ns", ULL * 5), ("copy_elapsed_ns", ULL * 5),
+                ("coherent_host_elapsed_ns", ULL * 5), ("sustainable_read_bytes_per_second", ULL),
+                ("sustainable_copy_bytes_per_second", ULL),
+                ("sustainable_coherent_host_bytes_per_second", ULL),
+                ("kernel_bundle_identity", C.c_char * 65), ("identity", C.c_char * 65)]
+
+
 class TensorDesc(C.Structure):
     _fields_ = [("name", C.c_char_p), ("dtype", C.c_int), ("rank", C.c_uint), ("dims", ULL * 4),
                 ("bytes", ULL)]
@@ -273,7 +282,7 @@ EXPORTS = [
     "yvex_rocm_gguf_qtype_geometry_find", "yvex_rocm_quant_numeric_capability_at",
     "yvex_rocm_backend_open", "yvex_rocm_backend_bind_owner", "yvex_rocm_backend_close_checked", "yvex_rocm_backend_kind_of",
     "yvex_rocm_backend_status_of", "yvex_rocm_backend_get_memory_stats", "yvex_rocm_backend_sync",
-    "yvex_rocm_backend_query_capability", "yvex_rocm_backend_tensor_alloc", "yvex_rocm_backend_tensor_release",
+    "yvex_rocm_backend_query_capability", "yvex_rocm_backend_bandwidth_probe", "yvex_rocm_backend_tensor_alloc", "yvex_rocm_backend_tensor_release",
     "yvex_rocm_backend_tensor_write", "yvex_rocm_backend_tensor_read", "yvex_rocm_backend_tensor_copy",
     "yvex_rocm_backend_tensor_owned_by", "yvex_rocm_backend_resident_alloc", "yvex_rocm_backend_resident_prefetch",
     "yvex_rocm_backend_resident_attach", "yvex_rocm_backend_resident_detach", "yvex_rocm_backend_resident_resolve",
@@ -297,7 +306,7 @@ KERNEL_EXPORTS = [
     "yvex_hip_moe_prepare_supported", "yvex_hip_moe_up", "yvex_hip_moe_down",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
     "yvex_hip_moe_reduce_combine", "yvex_hip_mhc_ingress", "yvex_hip_mhc_egress",
-    "yvex_hip_stream_read", "yvex_hip_clock_probe", "yvex_hip_fill_u32",
+    "yvex_hip_stream_read", "yvex_hip_bandwidth_sample", "yvex_hip_clock_probe", "yvex_hip_fill_u32",
     "yvex_hip_capture_begin", "yvex_hip_capture_end", "yvex_hip_capture_abort", "yvex_hip_graph_launch",
     "yvex_hip_graph_destroy",
     "yvex_hip_device_count", "yvex_hip_device_info", "yvex_hip_device_clocks", "yvex_hip_malloc", "yvex_hip_free",

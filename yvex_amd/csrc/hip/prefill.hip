@@ -827,7 +827,8 @@ extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void
     if (!w || !w->gate || !w->up || !act_q8k || !intermediate || !status || !pairs || !topk ||
         !experts || !(limit > 0.0) || (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
         return ST_INVALID_ARG;
-    if (w->gate_qtype != QT_IQ2_XXS || w->up_qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    if (w->gate_qtype != w->up_qtype || (w->gate_qtype != QT_IQ2_XXS && w->gate_qtype != QT_Q4_K))
+        return ST_UNSUPPORTED;
     int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
     if (rc) return rc;
     if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
@@ -835,6 +836,8 @@ extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void
     MfmaArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
     fill_up_problem(a.pr, w, act_q8k, 1, route_weights, wl, pairs, topk, experts, intermediate);
+    if (w->gate_qtype == QT_Q4_K)
+        return launch_q4k_rows_grouped(a.pr, true, w->hidden, w->intermediate, limit, status, as_stream(stream));
     a.width = (unsigned)w->hidden;
     a.out_rows = (unsigned)w->intermediate;
     a.limit = limit;
@@ -852,13 +855,15 @@ extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const vo
     if (!w || !w->down || !intermediate_q8k || !pair_outputs || !status || !pairs || !experts ||
         (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
         return ST_INVALID_ARG;
-    if (w->down_qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    if (w->down_qtype != QT_IQ2_XXS && w->down_qtype != QT_Q4_K) return ST_UNSUPPORTED;
     int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
     if (rc) return rc;
     if (pairs > 0xffffffffull || w->hidden > 0xffffffffull || w->hidden % 4u) return ST_BOUNDS;
     MfmaArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
     fill_down_problem(a.pr, w, intermediate_q8k, 1, wl, pairs, experts, pair_outputs);
+    if (w->down_qtype == QT_Q4_K)
+        return launch_q4k_rows_grouped(a.pr, false, w->intermediate, w->hidden, 1.0, status, as_stream(stream));
     a.width = (unsigned)w->intermediate;
     a.out_rows = (unsigned)w->hidden;
     a.limit = 1.0;

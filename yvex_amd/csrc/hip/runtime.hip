@@ -228,6 +228,36 @@ int yvex_hip_stream_read(const void *data, uint64_t bytes, uint32_t *sink, yvex_
     return check_launch("stream_read");
 }
 
+int yvex_hip_bandwidth_sample(const void *source, void *destination, uint64_t bytes, uint64_t iterations,
+                              uint32_t *sink, uint64_t *elapsed_ns, yvex_hip_stream stream)
+{
+    if (!source || !elapsed_ns || !iterations || bytes < 16u || ((uintptr_t)source & 15u) ||
+        (!destination && !sink))
+        return ST_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    hipEvent_t begin = nullptr, end = nullptr;
+    int rc = wrap("hipEventCreate", hipEventCreate(&begin));
+    if (!rc) rc = wrap("hipEventCreate", hipEventCreate(&end));
+    if (!rc) rc = wrap("hipEventRecord", hipEventRecord(begin, s));
+    for (uint64_t i = 0; !rc && i < iterations; ++i) {
+        if (destination) {
+            rc = wrap("hipMemcpyAsync(d2d)", hipMemcpyAsync(destination, source, bytes, hipMemcpyDeviceToDevice, s));
+        } else {
+            stream_read_kernel<<<256 * 16, 256, 0, s>>>((const uint4 *)source, bytes / 16u, sink);
+            rc = check_launch("stream_read");
+        }
+    }
+    if (!rc) rc = wrap("hipEventRecord", hipEventRecord(end, s));
+    if (!rc) rc = wrap("hipEventSynchronize", hipEventSynchronize(end));
+    float ms = 0.0f;
+    if (!rc) rc = wrap("hipEventElapsedTime", hipEventElapsedTime(&ms, begin, end));
+    if (begin) (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    if (rc) return rc;
+    *elapsed_ns = (uint64_t)((double)ms * 1.0e6);
+    return ST_OK;
+}
+
 int yvex_hip_clock_probe(uint64_t chain, int *sink, yvex_hip_stream stream)
 {
     if (!chain || (chain & 3u) || !sink) return ST_INVALID_ARG;

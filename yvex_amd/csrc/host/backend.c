@@ -203,6 +203,94 @@ int yvex_rocm_backend_get_memory_stats(const yvex_rocm_backend *backend, yvex_ba
     return YVEX_OK;
 }
 
+static unsigned long long median_of_five(const unsigned long long *values)
+{
+    unsigned long long v[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned int i, j;
+    memcpy(v, values, sizeof(v));
+    for (i = 1u; i < YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT; ++i) {
+        unsigned long long x = v[i];
+        for (j = i; j && v[j - 1u] > x; --j) v[j] = v[j - 1u];
+        v[j] = x;
+    }
+    return v[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT / 2u];
+}
+
+/* src/backend/cuda/backend.c:1386-1640 (cuda_bandwidth_probe) */
+int yvex_rocm_backend_bandwidth_probe(yvex_rocm_backend *backend, yvex_backend_bandwidth_evidence *out,
+                                      yvex_error *err)
+{
+    const unsigned long long working_set = 1ull << 30, iterations = 4ull;
+    void *source = NULL, *destination = NULL;
+    unsigned int sample;
+    int rc;
+    if (out) memset(out, 0, sizeof(*out));
+    if (!backend || !out || backend->kind != YVEX_BACKEND_KIND_ROCM)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.bandwidth", "backend and output are required");
+    rc = yvex_rocm_require_kernels(backend, "rocm.bandwidth", err);
+    if (rc != YVEX_OK) return rc;
+    if (backend->pending_completion)
+        return yvex_rocm_refuse(err, YVEX_ERR_STATE, "rocm.bandwidth",
+                                "a deferred operation is pending on the backend stream");
+    if (yvex_hip_malloc(&source, working_set) != 0 || yvex_hip_malloc(&destination, working_set) != 0) {
+        (void)yvex_hip_free(source);
+        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.bandwidth", yvex_hip_last_error());
+    }
+    rc = yvex_rocm_launch_result(yvex_hip_fill_u32(source, 0x5a5a5a5au, working_set / 4ull, backend->stream),
+                                 "rocm.bandwidth.fill", err);
+    out->schema_version = YVEX_BACKEND_BANDWIDTH_SCHEMA_V1;
+    out->working_set_bytes = working_set;
+    out->iterations = iterations;
+    out->sample_count = YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT;
+    /* one untimed pass of each kind first */
+    if (rc == YVEX_OK) {
+        uint64_t ignored = 0u;
+        rc = yvex_rocm_launch_result(yvex_hip_bandwidth_sample(source, NULL, working_set, 1ull,
+                                                               (uint32_t *)destination, &ignored,
+                                                               backend->stream), "rocm.bandwidth.warmup", err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_launch_result(yvex_hip_bandwidth_sample(source, destination, working_set, 1ull, NULL,
+                                                                   &ignored, backend->stream),
+                                         "rocm.bandwidth.warmup.copy", err);
+    }
+    for (sample = 0u; rc == YVEX_OK && sample < YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT; ++sample) {
+        uint64_t elapsed = 0u;       /* the read kernel's sink is a word of the copy target */
+        rc = yvex_rocm_launch_result(yvex_hip_bandwidth_sample(source, NULL, working_set, iterations,
+                                                               (uint32_t *)destination, &elapsed,
+                                                               backend->stream), "rocm.bandwidth.stream", err);
+        out->stream_elapsed_ns[sample] = elapsed;
+    }
+    for (sample = 0u; rc == YVEX_OK && sample < YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT; ++sample) {
+        uint64_t elapsed = 0u;
+        rc = yvex_rocm_launch_result(yvex_hip_bandwidth_sample(source, destination, working_set, iterations, NULL,
+                                                               &elapsed, backend->stream),
+                                     "rocm.bandwidth.copy", err);
+        out->copy_elapsed_ns[sample] = elapsed;
+    }
+    if (rc == YVEX_OK) {
+        unsigned long long read_ns = median_of_five(out->stream_elapsed_ns);
+        unsigned long long copy_ns = median_of_five(out->copy_elapsed_ns);
+        if (!read_ns || !copy_ns)
+            rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.bandwidth", "a timed sample took no time");
+        else {
+            out->sustainable_read_bytes_per_second =
+                (unsigned long long)((double)working_set * (double)iterations * 1.0e9 / (double)read_ns);
+            out->sustainable_copy_bytes_per_second =
+                (unsigned long long)((double)working_set * (double)iterations * 1.0e9 / (double)copy_ns);
+        }
+    }
+    if (yvex_hip_stream_sync(backend->stream) != 0 && rc == YVEX_OK)
+        rc = yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.bandwidth.sync", yvex_hip_last_error());
+    (void)yvex_hip_free(source);
+    (void)yvex_hip_free(destination);
+    if (rc != YVEX_OK) {
+        memset(out, 0, sizeof(*out));
+        return rc;
+    }
+    yvex_rocm_error_clear(err);
+    return YVEX_OK;
+}
+
 int yvex_rocm_backend_sync(yvex_rocm_backend *backend, yvex_error *err)
 {
     if (!backend) return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "backend.sync", "owner is required");

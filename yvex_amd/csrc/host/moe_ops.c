@@ -262,6 +262,14 @@ static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weigh
     w->down_expert_bytes = down->row_bytes * hidden;
 }
 
+/* Expert weights the matrix-core row-batch kernels take: gate and up of one format, IQ2_XXS (16)
+ * or Q4_K (12); the down matrix may be of the other. */
+static int matrix_core_qtypes(const yvex_hip_expert_weights *w)
+{
+    return w->gate_qtype == w->up_qtype && (w->gate_qtype == 16u || w->gate_qtype == 12u) &&
+           (w->down_qtype == 16u || w->down_qtype == 12u);
+}
+
 static int same_expert_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)
 {
     return a->gate_qtype == b->gate_qtype && a->up_qtype == b->up_qtype &&
@@ -593,13 +601,11 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
                             &views[YVEX_MOE_WEIGHT_SHARED_DOWN], addresses[3], addresses[4], addresses[5],
                             hidden, layer->shared_intermediate_width);
     /* Row batches whose buckets average eight pairs or more go to the int8 matrix-core kernels
-     * (IQ2_XXS weights, Q8_K activations); below that the decode sweeps, which read an expert's
+     * (IQ2_XXS or Q4_K weights, Q8_K activations); below that the decode sweeps, which read an expert's
      * bytes once per four pairs, are faster. The reference switches its tensor-core kernels on
      * from 16 input rows (src/backend/cuda/private.h:461-464). */
-    row_batch = routed_q8 && routed.gate_qtype == 16u && routed.up_qtype == 16u &&
-                routed.down_qtype == 16u && pairs >= 8ull * experts;
-    shared_row_batch = row_batch && has_shared && shared_q8 && shared.gate_qtype == 16u &&
-                       shared.up_qtype == 16u && shared.down_qtype == 16u;
+    row_batch = routed_q8 && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
+    shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",

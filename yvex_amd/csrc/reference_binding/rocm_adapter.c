@@ -94,6 +94,11 @@ static int rocm_memory_stats(const yvex_backend *backend, yvex_backend_memory_st
     return yvex_rocm_backend_get_memory_stats(rocm_of(backend)->backend, out, err);
 }
 
+static int rocm_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_evidence *out, yvex_error *err)
+{
+    return yvex_rocm_backend_bandwidth_probe(rocm_of(backend)->backend, out, err);
+}
+
 static int rocm_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
                              yvex_device_tensor **out, yvex_error *err)
 {
@@ -156,6 +161,7 @@ static int rocm_query_capability(const yvex_backend *backend, yvex_backend_opera
 static const yvex_backend_vtable rocm_vtable = {
     .close = rocm_close,
     .memory_stats = rocm_memory_stats,
+    .bandwidth_probe = rocm_bandwidth_probe,
     .tensor_alloc = rocm_tensor_alloc,
     .resident_alloc = rocm_resident_alloc,
     .resident_prefetch_supported = rocm_resident_prefetch_supported,
