@@ -705,9 +705,15 @@ typedef struct {
  * block order. Q2_K: per pair of neighbouring rows of one expert and block, 8 bytes (d, dmin of
  * the even row, then of the odd row), then from a 64-aligned offset 32 bytes of sub-block scales
  * (two halves of 16: even row's 8 bytes, odd row's 8 bytes), then from a 64-aligned offset 128
- * code bytes (the rows' 4-byte words interleaved). Padding is zero. As in the reference, whose
- * row-batch path refuses a DERIVED_BACKEND view (moe.c:939-958), execute_rows answers UNSUPPORTED
- * for such views: the sweeps stream canonical rows. */
+ * code bytes (the rows' 4-byte words interleaved). Padding is zero. A decision whose
+ * kernel_family is YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP asks for this backend's own image of an
+ * IQ2_XXS tensor instead (routed or shared expert): 72 bytes per superblock in block order, two
+ * records of nine little-endian dwords, one per half superblock {fp16 superblock scale | the four
+ * 4-bit group scales << 16; then per group of 32 weights its four codebook indices and its four
+ * 7-bit sign fields, one to a byte}. The reference's row-batch path refuses every
+ * DERIVED_BACKEND view (moe.c:939-958); execute_rows here runs that one image (IQ2_XXS,
+ * device-encoded activations, the sweep family on gate, up and down) on the decode sweeps and
+ * answers UNSUPPORTED for any other derived view. */
 typedef struct {
     int (*derived_layout_plan)(const yvex_physical_execution_decision *decision,
                                unsigned long long *storage_bytes, yvex_error *err);
@@ -745,6 +751,22 @@ int yvex_rocm_moe_derived_layout_build(const yvex_physical_execution_decision *d
                                        const unsigned char *canonical,
                                        unsigned long long canonical_bytes, unsigned char *derived,
                                        unsigned long long storage_bytes, yvex_error *err);
+
+/* No counterpart in the reference, whose residency step builds derived storage on the host and
+ * uploads it (src/runtime/residency.c:457-600): the image a gfx950-sweep decision asks for, of a
+ * tensor whose canonical bytes are on the device already, built there. decision is what
+ * derived_layout_plan took; canonical_address holds decision->encoded_bytes, image_address
+ * storage_bytes (dword-aligned, no overlap). Synchronous on the backend's stream. A view of the
+ * result carries layout DERIVED_BACKEND, the family YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP,
+ * activation DEVICE_ENCODED, the canonical row geometry and encoded_bytes, storage_bytes, and the
+ * image's device_address (or `encoded` inside the attached arena). execute_rows runs such experts
+ * on the decode sweeps at any batch width; every other operation takes canonical rows
+ * (UNSUPPORTED). */
+int yvex_rocm_moe_sweep_image_build_resident(yvex_rocm_backend *backend,
+                                             const yvex_physical_execution_decision *decision,
+                                             unsigned long long canonical_address,
+                                             unsigned long long image_address,
+                                             unsigned long long storage_bytes, yvex_error *err);
 
 /* The workspace_required entry of the table below, callable without a backend (it depends on
  * the layer plan and the row count alone). */

@@ -165,14 +165,29 @@ int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, 
                          int *status, yvex_hip_stream stream);
 
 /* Expert matrices of one MoE layer. routed_* are expert-major: expert e starts at
- * base + e * expert_bytes and holds rows * row_bytes canonical GGUF bytes. */
+ * base + e * expert_bytes and holds rows * row_bytes canonical GGUF bytes. gate_up_image /
+ * down_image say that those IQ2_XXS matrices are given as the sweep image of
+ * yvex_hip_iq2_sweep_image_build (72 bytes a superblock, row_bytes and expert_bytes counted in
+ * image bytes); only the decode sweeps with Q8_K activations read it. */
 typedef struct {
     const uint8_t *gate, *up, *down;
     unsigned int gate_qtype, up_qtype, down_qtype;
     uint64_t hidden, intermediate;
     uint64_t gate_row_bytes, up_row_bytes, down_row_bytes;
     uint64_t gate_expert_bytes, up_expert_bytes, down_expert_bytes;
+    int gate_up_image, down_image;
 } yvex_hip_expert_weights;
+
+/* The sweep image of IQ2_XXS weights: the backend's own re-packing for the decode sweeps, built
+ * on the device from canonical bytes (`blocks` superblocks of 66 bytes, any alignment) into
+ * `image` (yvex_hip_iq2_sweep_image_bytes(blocks) bytes, dword-aligned), block order kept. Per
+ * superblock two records of nine dwords, one per half: {f16 d | the half's four 4-bit group
+ * scales << 16}, then per group the four codebook bytes and the four 7-bit sign fields one to a
+ * byte. The counterpart of the reference's derived layout (src/backend/cuda/layout.c:95-167) for
+ * this backend's kernels; the canonical bytes stay the authority. */
+uint64_t yvex_hip_iq2_sweep_image_bytes(uint64_t blocks);
+int yvex_hip_iq2_sweep_image_build(const uint8_t *canonical, uint64_t blocks, void *image,
+                                   yvex_hip_stream stream);
 
 /* Replaces yvex_moe_grouped_up_rows (+ _up_tensorcore) (moe_kernels.cu:431-516,
  * tensorcore.cu:527-626): for every ordered pair p of every bucket,

@@ -137,6 +137,55 @@ def test_against_the_compiled_reference(lib, qtype, experts, rows_per_expert, wi
     assert rc == 0 and np.array_equal(derived, expected)
 
 
+def sweep_image_of(canonical):
+    """numpy statement of the expert sweeps' image: per superblock two records of nine dwords."""
+    blocks = canonical.size // 66
+    raw = canonical.reshape(blocks, 66)
+    d = raw[:, 0].astype(np.uint32) | (raw[:, 1].astype(np.uint32) << 8)
+    groups = raw[:, 2:].reshape(blocks, 8, 8)
+    grids = groups[:, :, :4].copy().view(np.uint32).reshape(blocks, 8)
+    aux = groups[:, :, 4:].copy().view(np.uint32).reshape(blocks, 8)
+    image = np.zeros((blocks, 2, 9), np.uint32)
+    for half in range(2):
+        scales = np.zeros(blocks, np.uint32)
+        for j in range(4):
+            a = aux[:, 4 * half + j]
+            image[:, half, 1 + 2 * j] = grids[:, 4 * half + j]
+            image[:, half, 2 + 2 * j] = ((a & 127) | (((a >> 7) & 127) << 8) | (((a >> 14) & 127) << 16)
+                                         | (((a >> 21) & 127) << 24))
+            scales |= (a >> 28) << (4 * j)
+        image[:, half, 0] = d | (scales << 16)
+    return image.view(np.uint8).ravel()
+
+
+@pytest.mark.parametrize("experts,rows,width,consumer", [
+    (4, 8, 512, abi.CONSUMER_ROUTED_GATE_UP), (3, 9, 768, abi.CONSUMER_ROUTED_DOWN),
+    (1, 5, 256, abi.CONSUMER_SHARED_EXPERT)])
+def test_sweep_image_of_the_gfx950_family(lib, experts, rows, width, consumer):
+    """A decision of the gfx950 sweep family gets this backend's own image of an IQ2_XXS tensor
+    (72 bytes a superblock; the shared expert admitted), not the reference's two sections."""
+    d = decision_for(oracle.IQ2_XXS, experts, rows, width, consumer=consumer)
+    d.kernel_family = abi.FAMILY_GFX950
+    rc, storage, err = plan(lib, d)
+    assert rc == 0, err.message
+    assert storage == rows * (width // 256) * 72
+    canonical = oracle.Generator(9, f"layout.sweep.{rows}.{width}").iq2xxs(rows * (width // 256))
+    rc, derived, err = build(lib, d, canonical, storage)
+    assert rc == 0, err.message
+    assert np.array_equal(derived, sweep_image_of(canonical))
+    # and the image decodes to the same weights: scales, code bytes and sign fields are all there
+    records = derived.view(np.uint32).reshape(-1, 2, 9)
+    raw = canonical.reshape(-1, 66)
+    assert np.array_equal(records[:, :, 0] & 0xffff, np.repeat(raw[:, :2].copy().view(np.uint16), 2, 1))
+    # other qtypes have no sweep image; without the family the shared expert has no derived storage
+    q2 = decision_for(oracle.Q2_K, 2, 8, 512)
+    q2.kernel_family = abi.FAMILY_GFX950
+    assert plan(lib, q2)[0] == abi.UNSUPPORTED
+    if consumer == abi.CONSUMER_SHARED_EXPERT:
+        d.kernel_family = b""
+        assert plan(lib, d)[0] == abi.FORMAT
+
+
 def test_refusals(lib):
     good = dict(qtype=oracle.IQ2_XXS, experts=4, rows=8, width=512)
     cases = [

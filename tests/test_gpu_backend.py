@@ -280,13 +280,24 @@ def test_select_greedy_rows(backend, oracle):
     assert facts.kernel_launches == 2
 
 
+def sweep_image_decision(experts, rows, width, consumer):
+    """The decision that asks derived_layout_plan/build for the expert sweeps' image."""
+    d = abi.ExecutionDecision()
+    d.expert_count, d.canonical_qtype = experts, 16
+    d.canonical_row_width, d.canonical_row_count = width, rows
+    d.encoded_bytes = rows * (width // 256) * 66
+    d.consumer, d.layout, d.derived_asset_required = consumer, abi.LAYOUT_DERIVED, 1
+    d.kernel_family = abi.FAMILY_GFX950
+    return d
+
+
 class MoeCase:
     """One synthetic layer resident on the backend plus everything execute_rows needs."""
 
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
                  shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
-                 down_qtype=None):
+                 down_qtype=None, sweep_image=()):
         self.b, self.oracle = b, oracle
         self.streams, self.iterations = streams, iterations
         expanded = hidden * max(streams, 1)
@@ -319,6 +330,27 @@ class MoeCase:
             parts["base"] = g.normal(mixing, 0.5).view(np.uint8)
             parts["norm"] = ((1.0 + g.normal(hidden, 0.2)).astype(np.float32).view(np.uint32) >> 16) \
                 .astype(np.uint16).view(np.uint8)
+        # experts held as the sweeps' image: built by the library's host builder, resident beside
+        # the canonical bytes
+        self.decisions = {}
+        for group, names in (("routed", ("gate", "up", "down")), ("shared", ("sgate", "sup", "sdown"))):
+            if group not in sweep_image:
+                continue
+            for name in names:
+                down = name.endswith("down")
+                decision = sweep_image_decision(
+                    1 if group == "shared" else experts, (hidden if down else intermediate) * (1 if group == "shared" else experts),
+                    intermediate if down else hidden,
+                    abi.CONSUMER_SHARED_EXPERT if group == "shared" else
+                    abi.CONSUMER_ROUTED_DOWN if down else abi.CONSUMER_ROUTED_GATE_UP)
+                storage, err = abi.ULL(), abi.Error()
+                assert b.lib.yvex_rocm_moe_derived_layout_plan(C.byref(decision), C.byref(storage), C.byref(err)) == 0, err.message
+                image = np.full(storage.value, 0xA5, np.uint8)
+                assert b.lib.yvex_rocm_moe_derived_layout_build(
+                    C.byref(decision), parts[name].ctypes.data, parts[name].nbytes, image.ctypes.data,
+                    image.nbytes, C.byref(err)) == 0, err.message
+                parts[name + ".image"] = image
+                self.decisions[name] = decision
         self.parts = parts
         offsets, cursor = {}, 0
         for name, blob in parts.items():
@@ -357,6 +389,9 @@ class MoeCase:
             v.encoded, v.encoded_bytes = host + offsets[name], parts[name].nbytes
             v.storage_bytes = parts[name].nbytes
             v.row_bytes, v.row_width, v.row_count = row_bytes, width, count
+            if name + ".image" in parts:
+                v.layout = abi.LAYOUT_DERIVED
+                v.encoded, v.storage_bytes = host + offsets[name + ".image"], parts[name + ".image"].nbytes
 
         view(abi.W_ROUTER, "router", 0, hidden, experts, hidden * 4, abi.ACT_DEVICE_F32)
         view(abi.W_ROUTER_BIAS, "bias", 0, experts, 1, experts * 4, abi.ACT_DEVICE_F32)
@@ -623,9 +658,16 @@ def test_execute_rows_refusals(backend, oracle):
     assert case.execute() == abi.FORMAT
     for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP):
         case.job.weights[slot].layout = abi.LAYOUT_DERIVED
+    # ... except the expert sweeps' own image (IQ2_XXS, encoded activations, the sweep family on
+    # all three views), whose storage is 72 bytes a superblock: these views still hold canonical bytes
+    assert case.execute() == abi.FORMAT
+    assert b"image" in case.err.message
+    for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN):
+        case.job.weights[slot].kernel_family = abi.FAMILY_PORTABLE_EXPERT_ROW
     assert case.execute() == abi.UNSUPPORTED
     for slot in (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN):
         case.job.weights[slot].layout = abi.LAYOUT_EXPERT_MAJOR
+        case.job.weights[slot].kernel_family = abi.FAMILY_GFX950
     # the layout entries of the table answer like the exported functions
     decision = abi.ExecutionDecision()
     decision.expert_count, decision.canonical_qtype = 4, 16
@@ -673,6 +715,89 @@ def test_execute_rows_deferred_completion(backend, oracle):
     want = case.oracle_layer(act_q8=True)["combined"]
     err_abs = np.abs(got.astype(np.float64) - want)
     assert (err_abs > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
+
+
+@pytest.mark.parametrize("imaged,rows,experts", [
+    (("routed", "shared"), 5, 8), (("routed",), 7, 8), (("shared",), 6, 8), (("routed", "shared"), 40, 4)])
+def test_execute_rows_runs_the_sweep_image(backend, oracle, imaged, rows, experts):
+    """Experts resident as the decode sweeps' image (DERIVED_BACKEND views of the gfx950 sweep
+    family, built by derived_layout_build) give bit for bit what canonical views give on the
+    sweeps; a batch wide enough for the matrix-core kernels stays on the sweeps and agrees with
+    the canonical run (which takes the matrix cores) within the parity bar. No counterpart in the
+    reference, whose row-batch path refuses derived views (src/backend/cuda/moe.c:939-958)."""
+    results = []
+    for image in ((), imaged):
+        case = MoeCase(backend, oracle, hidden=2048, intermediate=2048, experts=experts, rows=rows,
+                       sweep_image=image)
+        backend.workspace(case.workspace_bytes)
+        assert case.execute() == 0, case.err.message
+        results.append((case.combined.copy(), case.sel.copy(), case.wts.copy()))
+        backend.release_all()
+    assert np.array_equal(results[0][1], results[1][1]) and np.array_equal(results[0][2], results[1][2])
+    if rows * 2 < 8 * experts:
+        assert np.array_equal(results[0][0].view(np.uint32), results[1][0].view(np.uint32))
+    else:
+        assert rows_close(results[1][0], results[0][0])
+
+
+def test_sweep_image_built_on_the_device_equals_the_host_builder(backend, oracle):
+    """yvex_rocm_moe_sweep_image_build_resident against derived_layout_build on the same tensor,
+    and its refusals."""
+    case = MoeCase(backend, oracle, hidden=2048, intermediate=2048, experts=4, rows=3, sweep_image=("routed",))
+    lib, decision = backend.lib, case.decisions["down"]
+    want = case.parts["down.image"]
+    base = case.arena_tensor.contents.data
+    rc, target = backend.tensor(want.nbytes, abi.DTYPE_I8, b"image")
+    assert rc == 0
+    err = abi.Error()
+    build = lib.yvex_rocm_moe_sweep_image_build_resident
+    canonical = base + case.offsets["down"]
+    assert build(backend.handle, C.byref(decision), canonical, target.contents.data, want.nbytes,
+                 C.byref(err)) == 0, err.message
+    target.contents.is_written = 1          # written through its address, not through tensor_write
+    got = backend.read_f32(target, want.nbytes // 4).view(np.uint8)
+    assert np.array_equal(got, want)
+    # wrong size, overlapping ranges, a decision for the reference's own image
+    assert build(backend.handle, C.byref(decision), canonical, target.contents.data, want.nbytes - 72,
+                 C.byref(err)) == abi.INVALID_ARG
+    assert build(backend.handle, C.byref(decision), canonical, canonical + 64, want.nbytes,
+                 C.byref(err)) == abi.INVALID_ARG
+    decision.kernel_family = b""
+    assert build(backend.handle, C.byref(decision), canonical, target.contents.data, want.nbytes,
+                 C.byref(err)) == abi.UNSUPPORTED
+    backend.release_all()
+
+
+def test_sweep_image_views_are_checked(backend, oracle):
+    case = MoeCase(backend, oracle, hidden=2048, intermediate=2048, experts=4, rows=3,
+                   sweep_image=("routed", "shared"))
+    backend.workspace(case.workspace_bytes)
+    assert case.execute() == 0, case.err.message
+    routed = (abi.W_ROUTED_GATE, abi.W_ROUTED_UP, abi.W_ROUTED_DOWN)
+    # F32 activations, another qtype, another family: only canonical rows serve those
+    for slot in routed:
+        case.job.weights[slot].activation = abi.ACT_DEVICE_F32
+    assert case.execute() == abi.UNSUPPORTED
+    for slot in routed:
+        case.job.weights[slot].activation = abi.ACT_DEVICE_ENCODED
+        case.job.weights[slot].kernel_family = abi.FAMILY_PORTABLE_EXPERT_ROW
+    assert case.execute() == abi.UNSUPPORTED
+    for slot in routed:
+        case.job.weights[slot].kernel_family = abi.FAMILY_GFX950
+    case.job.weights[abi.W_ROUTED_DOWN].qtype = 12
+    assert case.execute() == abi.UNSUPPORTED
+    case.job.weights[abi.W_ROUTED_DOWN].qtype = 16
+    # storage that is not 72 bytes a superblock, an image outside the arena
+    case.job.weights[abi.W_SHARED_UP].storage_bytes -= 72
+    assert case.execute() == abi.FORMAT
+    case.job.weights[abi.W_SHARED_UP].storage_bytes += 72
+    keep = case.job.weights[abi.W_ROUTED_GATE].encoded
+    outside = np.zeros(case.job.weights[abi.W_ROUTED_GATE].storage_bytes, np.uint8)
+    case.job.weights[abi.W_ROUTED_GATE].encoded = outside.ctypes.data
+    assert case.execute() == abi.FORMAT
+    case.job.weights[abi.W_ROUTED_GATE].encoded = keep
+    assert case.execute() == 0, case.err.message
+    backend.release_all()
 
 
 @pytest.mark.parametrize("kwargs", [

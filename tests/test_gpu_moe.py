@@ -27,7 +27,7 @@ def bf16_flip_report(got, want):
 
 
 def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype, act_q8, scoring,
-               seed=42, shared=True, matrix_cores=False):
+               seed=42, shared=True, matrix_cores=False, sweep_image=False):
     from yvex_amd.moe import MoeLayer
     qt = getattr(oracle, qtype)
     g = oracle.Generator(seed, f"moe.{qtype}.{hidden}.{intermediate}.{experts}")
@@ -45,7 +45,7 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
                      qtypes=(qt, qt, qt), routed=tuple(dev(t, gpu) for t in (gate, up, down)),
                      shared=tuple(dev(t, gpu) for t in sh) if sh else None, bias=dev(bias, gpu),
                      scoring=scoring, normalize=True, scaling=1.5, limit=10.0, act_q8=act_q8,
-                     max_rows=rows, device=gpu, matrix_cores=matrix_cores)
+                     max_rows=rows, device=gpu, matrix_cores=matrix_cores, sweep_image=sweep_image)
     host = dict(qt=qt, gate=gate, up=up, down=down, shared=sh, x=x, logits=logits, bias=bias)
     return layer, host
 
@@ -147,6 +147,52 @@ def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, 
     assert outside.mean() < 2e-2
     terms = np.abs(pair_out.reshape(rows, topk, hidden)).sum(axis=1) + np.abs(shared)
     assert np.all(err[outside] <= 2 * BF16_ULP * terms[outside] + 1e-4)
+
+
+def test_sweep_image_is_the_documented_repacking(gpu, oracle):
+    """The image the device builds from canonical IQ2_XXS bytes, against a numpy statement of the
+    format: per superblock two records of nine dwords {f16 d | four group scales << 16, then per
+    group the codebook bytes and the 7-bit sign fields one to a byte}."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(5, "sweep.image")
+    blocks = 300
+    canonical = g.iq2xxs(blocks)
+    image = K.iq2_sweep_image(dev(canonical, gpu)).cpu().numpy().view(np.uint32).reshape(blocks, 2, 9)
+    raw = canonical.reshape(blocks, 66)
+    d = raw[:, 0].astype(np.uint32) | (raw[:, 1].astype(np.uint32) << 8)
+    groups = raw[:, 2:].reshape(blocks, 8, 8)
+    grids = groups[:, :, :4].copy().view(np.uint32).reshape(blocks, 8)
+    aux = groups[:, :, 4:].copy().view(np.uint32).reshape(blocks, 8)
+    for half in range(2):
+        scales = np.zeros(blocks, np.uint32)
+        for j in range(4):
+            a = aux[:, 4 * half + j]
+            assert np.array_equal(image[:, half, 1 + 2 * j], grids[:, 4 * half + j])
+            signs = (a & 127) | (((a >> 7) & 127) << 8) | (((a >> 14) & 127) << 16) | (((a >> 21) & 127) << 24)
+            assert np.array_equal(image[:, half, 2 + 2 * j], signs)
+            scales |= (a >> 28) << (4 * j)
+        assert np.array_equal(image[:, half, 0], d | (scales << 16))
+
+
+@pytest.mark.parametrize("hidden,intermediate,experts,topk,rows", [
+    (7168, 2048, 12, 4, 6), (2048, 2048, 6, 4, 20), (4096, 3072, 4, 2, 5), (2048, 2048, 200, 8, 40)])
+def test_sweeps_give_the_same_bits_from_the_image(gpu, oracle, hidden, intermediate, experts, topk, rows):
+    """The decode sweeps over the sweep image of the experts (one, two, three, four pairs a sweep,
+    shared expert merged into the launches) publish bit for bit what they publish from canonical
+    bytes: same integer sums, same scaling, same order."""
+    layers = []
+    for image in (False, True):
+        layer, h = make_layer(oracle, gpu, hidden=hidden, intermediate=intermediate, experts=experts,
+                              topk=topk, rows=rows, qtype="IQ2_XXS", act_q8=True, scoring=1,
+                              sweep_image=image)
+        combined = layer.run(dev(h["x"], gpu), dev(h["logits"], gpu)).clone()
+        torch.cuda.synchronize()
+        assert int(layer.status.item()) == 0
+        pairs = rows * topk
+        layers.append((combined.cpu().numpy(), layer.intermediate_f32[:pairs + rows].cpu().numpy().copy(),
+                       layer.pair_outputs[:pairs].cpu().numpy().copy(), layer.shared_out[:rows].cpu().numpy().copy()))
+    for a, b in zip(*layers):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
 @pytest.mark.parametrize("matrix_cores", [False, True])

@@ -292,6 +292,7 @@ EXPORTS = [
     "yvex_rocm_backend_moe_operations_get", "yvex_rocm_backend_moe_begin", "yvex_rocm_backend_moe_add_expert",
     "yvex_rocm_backend_moe_finish", "yvex_rocm_backend_moe_close",
     "yvex_rocm_expert_worklist_build", "yvex_rocm_moe_derived_layout_plan", "yvex_rocm_moe_derived_layout_build",
+    "yvex_rocm_moe_sweep_image_build_resident",
     "yvex_rocm_moe_workspace_required",
     "yvex_rocm_gguf_open_path", "yvex_rocm_gguf_close", "yvex_rocm_gguf_metadata_count", "yvex_rocm_gguf_metadata_u64",
     "yvex_rocm_gguf_metadata_f64", "yvex_rocm_gguf_metadata_string", "yvex_rocm_gguf_tensor_count", "yvex_rocm_gguf_tensor_at",
@@ -303,7 +304,7 @@ KERNEL_EXPORTS = [
     "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes", "yvex_hip_argmax_f32_static",
     "yvex_hip_argmax_static_capacity",
     "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_moe_route_hash_rows", "yvex_hip_worklist_build", "yvex_hip_moe_prepare",
-    "yvex_hip_moe_prepare_supported", "yvex_hip_moe_up", "yvex_hip_moe_down",
+    "yvex_hip_moe_prepare_supported", "yvex_hip_moe_up", "yvex_hip_moe_down", "yvex_hip_iq2_sweep_image_bytes", "yvex_hip_iq2_sweep_image_build",
     "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
     "yvex_hip_moe_reduce_combine", "yvex_hip_mhc_ingress", "yvex_hip_mhc_egress",
     "yvex_hip_stream_read", "yvex_hip_bandwidth_sample", "yvex_hip_clock_probe", "yvex_hip_fill_u32",
@@ -329,6 +330,8 @@ def library():
                                                       C.POINTER(Error)]
     lib.yvex_rocm_moe_derived_layout_build.argtypes = [C.POINTER(ExecutionDecision), C.c_void_p, ULL,
                                                        C.c_void_p, ULL, C.POINTER(Error)]
+    lib.yvex_rocm_moe_sweep_image_build_resident.argtypes = [C.c_void_p, C.POINTER(ExecutionDecision), ULL, ULL,
+                                                             ULL, C.POINTER(Error)]
     lib.yvex_rocm_gguf_open_path.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.POINTER(Error)]
     lib.yvex_rocm_gguf_close.argtypes = [C.c_void_p]
     lib.yvex_rocm_gguf_close.restype = None

@@ -34,6 +34,7 @@ struct GroupedArgs {
     unsigned item_rows;                      // weight rows (row pairs when fused) per work item
     double limit;
     int *status;
+    int image;                               // weights are the IQ2_XXS sweep image (72 B a superblock)
 };
 
 // The same value from fp32 arithmetic when that provably rounds to the same bfloat16. For
@@ -67,6 +68,16 @@ __device__ __forceinline__ float swiglu_bf16(float g, float u, float route_weigh
     const double t = exp(-fabs(gv));
     const double silu = gv >= 0.0 ? gv / (1.0 + t) : gv * t / (1.0 + t);
     return bf16_round((float)(silu * uv * (double)route_weight));
+}
+
+// Geometry of a matrix given as the IQ2_XXS sweep image.
+static inline int check_image_matrix(unsigned qtype, uint64_t width, uint64_t row_bytes, const void *base,
+                                     uint64_t expert_bytes)
+{
+    if (qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    if (!width || width % 256u || width / 256u * 72u != row_bytes) return ST_BOUNDS;
+    if (((uintptr_t)base & 3u) || (expert_bytes & 3u)) return ST_INVALID_ARG;
+    return ST_OK;
 }
 
 static inline int check_matrix(unsigned qtype, uint64_t width, uint64_t row_bytes)
@@ -140,8 +151,8 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
 
 // Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16
 // to 64 lanes of 128 columns each.
-bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs);
-int launch_iq2_sweep(const GroupedArgs &a, bool fused, hipStream_t stream);
+bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs, bool image);
+int launch_iq2_sweep(const GroupedArgs &a, bool fused, bool image, hipStream_t stream);
 
 // Row-batch expert kernels for Q4_K weights on the int8 matrix cores (dense_q4k.hip).
 int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t width, uint64_t out_rows,

@@ -759,8 +759,9 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
     unsigned long long all_pairs = 0ull;
     for (unsigned i = 0; i < a.problems; ++i) all_pairs += a.problem[i].pairs;
     if (qtype == QT_IQ2_XXS && q8 && aligned &&
-        iq2_sweep_supported(a.width, a.out_rows, all_pairs))
-        return launch_iq2_sweep(a, fused, stream);
+        iq2_sweep_supported(a.width, a.out_rows, all_pairs, a.image != 0))
+        return launch_iq2_sweep(a, fused, a.image != 0, stream);
+    if (a.image) return ST_UNSUPPORTED;      // only the specialised sweeps read the image
     switch (qtype) {
     case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);
     case QT_Q4_K: return launch_grouped<QT_Q4_K>(a, q8, fused, stream);
@@ -913,13 +914,18 @@ extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *act
         (shared && (!shared->gate || !shared->up || !shared_rows || !shared_intermediate)))
         return ST_INVALID_ARG;
     if (w->gate_qtype != w->up_qtype) return ST_UNSUPPORTED;
-    int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
+    int rc = w->gate_up_image
+        ? check_image_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes, w->gate, w->gate_expert_bytes)
+        : check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
     if (rc) return rc;
+    if (w->gate_up_image && (!act_q8 || ((uintptr_t)w->up & 3u) || (w->up_expert_bytes & 3u)))
+        return ST_UNSUPPORTED;
     if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
     if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull || shared_rows > 0xffffffffull)
         return ST_BOUNDS;
     if (shared && (!same_shape(w, shared) || shared->gate_row_bytes != w->gate_row_bytes ||
-                   shared->up_row_bytes != w->up_row_bytes))
+                   shared->up_row_bytes != w->up_row_bytes ||
+                   (shared->gate_up_image != 0) != (w->gate_up_image != 0)))
         return ST_UNSUPPORTED;   // launch the shared expert on its own instead
     GroupedArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts};
@@ -937,6 +943,7 @@ extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *act
     a.item_rows = kItemRowsMax;
     a.limit = limit;
     a.status = status;
+    a.image = w->gate_up_image != 0;
     return dispatch_grouped(w->gate_qtype, a, act_q8 != 0, true, as_stream(stream));
 }
 
@@ -955,11 +962,15 @@ extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *i
         (expert_ids && (!bucket_offsets || !bucket_populations || !sweep_offsets || !counts)) ||
         (shared && (!shared->down || !shared_rows || !shared_intermediate || !shared_outputs)))
         return ST_INVALID_ARG;
-    int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
+    int rc = w->down_image
+        ? check_image_matrix(w->down_qtype, w->intermediate, w->down_row_bytes, w->down, w->down_expert_bytes)
+        : check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
     if (rc) return rc;
+    if (w->down_image && !act_q8) return ST_UNSUPPORTED;
     if (pairs > 0xffffffffull || w->hidden > 0xffffffffull || shared_rows > 0xffffffffull)
         return ST_BOUNDS;
-    if (shared && (!same_shape(w, shared) || shared->down_row_bytes != w->down_row_bytes))
+    if (shared && (!same_shape(w, shared) || shared->down_row_bytes != w->down_row_bytes ||
+                   (shared->down_image != 0) != (w->down_image != 0)))
         return ST_UNSUPPORTED;
     GroupedArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts};
@@ -976,6 +987,7 @@ extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *i
     a.item_rows = 64u;
     a.limit = 1.0;
     a.status = status;
+    a.image = w->down_image != 0;
     return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, as_stream(stream));
 }
 

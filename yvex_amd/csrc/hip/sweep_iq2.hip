@@ -19,6 +19,16 @@
 //
 // A work item is (bucket, tile of 16 row iterations, sweep). One workgroup per compute unit
 // stays resident and its waves walk the item list with a stride.
+//
+// IMAGE: the weights come from the backend's own re-packing of the canonical bytes (built once at
+// residency time, the canonical tensor stays the authority), made for this kernel's instruction
+// budget. A superblock is two records of 36 bytes, one per lane of the pair that shares it:
+//     dword 0      f16 d of the superblock | the four 4-bit group scales of this half << 16
+//     dword 1 + 2j the four codebook bytes of group j of this half
+//     dword 2 + 2j its four 7-bit sign fields, one to a byte
+// so every load is dword-aligned with nothing to shift into place, a sign lookup address is one
+// byte permute like a codebook lookup address (the canonical 7-bit fields need a shift and a
+// mask each), and the scale arrives with the lane's own record. 72 bytes against 66.
 #include "common.hpp"
 #include "launch.hpp"
 #include "grouped.hpp"
@@ -174,7 +184,7 @@ __device__ __forceinline__ float dpp_add(float v)
 // stages between. A stage holds independent dependency chains (one per stream, or the even and
 // odd products of a single stream), because a dependent vector instruction issues only about
 // nine cycles after its producer.
-template <int STREAMS, int N>
+template <int STREAMS, int N, bool IMAGE>
 __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const SweepLane &g,
                                               const unsigned (&act)[N][32], int (&total)[STREAMS][N])
 {
@@ -187,7 +197,8 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
         const unsigned raw[9] = {c[w].lo.x, c[w].lo.y, c[w].lo.z, c[w].lo.w,
                                  c[w].hi.x, c[w].hi.y, c[w].hi.z, c[w].hi.w, c[w].tail};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[w][i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], g.code_shift);
+        for (int i = 0; i < 8; ++i)
+            q[w][i] = IMAGE ? raw[i] : __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], g.code_shift);
 #pragma unroll
         for (int p = 0; p < N; ++p) total[w][p] = 0;
     }
@@ -203,9 +214,16 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
                 const unsigned j = 2u * (unsigned)h + (unsigned)jj;
                 // magnitude address = index byte j << 8 | replica offset
                 const unsigned ma = __builtin_amdgcn_perm(grids, g.mag_lane, 0x0c0c0400u + (j << 8));
-                // selector address = sign field j (7 bits at bit 7j) moved to bit 8 | replica offset
-                const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
-                const unsigned sa = (moved & 0x7f00u) | g.sel_lane;
+                // selector address = sign field j moved to bit 8 | replica offset: the image holds
+                // the field in byte j (the table base's third byte comes from the replica word),
+                // the canonical word holds it at bit 7j
+                unsigned sa;
+                if constexpr (IMAGE) {
+                    sa = __builtin_amdgcn_perm(aux, g.sel_lane, 0x0c020400u + (j << 8));
+                } else {
+                    const unsigned moved = 7u * j >= 8u ? aux >> (7u * j - 8u) : aux << (8u - 7u * j);
+                    sa = (moved & 0x7f00u) | g.sel_lane;
+                }
                 mag[slot][w][jj] = lds_read_uint4(ma);
                 sel[slot][w][jj] = lds_read_uint2(sa);
             }
@@ -242,8 +260,10 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
         if (h == 1) {
 #pragma unroll
             for (int w = 0; w < STREAMS; ++w) {
-                // 2 s + 1: bit 27 of the word is a sign bit, forced to 1
-                const int factor = (int)((q[w][2 * k + 1] >> 27) | 1u);
+                // 2 s + 1: bit 27 of the canonical word is a sign bit, forced to 1; the image
+                // keeps the scale of group k in bits 16 + 4k of the record's first dword
+                const int factor = IMAGE ? (int)(((c[w].tail >> (15 + 4 * k)) & 0x1eu) | 1u)
+                                         : (int)((q[w][2 * k + 1] >> 27) | 1u);
 #pragma unroll
                 for (int p = 0; p < N; ++p) {
                     int sum = d[w][p][0];
@@ -257,7 +277,7 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
 }
 
 // One sweep over the item's weight rows [row_begin, row_end) for N live pairs.
-template <bool FUSED, int N>
+template <bool FUSED, int N, bool IMAGE>
 __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedProblem &pr,
                                           const SweepLane &g, const unsigned char *gate_e,
                                           const unsigned char *up_e, unsigned long long first_ordered,
@@ -314,13 +334,16 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned long long up_step = (unsigned long long)g.rows_per_iter * pr.up_row_bytes;
     const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
     // (row bases and row strides are multiples of four bytes: checked on the host)
-    const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * 66u;
-    const unsigned up_block = lane_row * (unsigned)pr.up_row_bytes + lane_super * 66u;
-    const unsigned gate_codes_at = (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
-    const unsigned up_codes_at = (up_block + 2u + 32u * g.half) & ~3u;
+    const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * (IMAGE ? 72u : 66u);
+    const unsigned up_block = lane_row * (unsigned)pr.up_row_bytes + lane_super * (IMAGE ? 72u : 66u);
+    // image: the lane's record is its first dword (scale and group scales) and eight more
+    const unsigned gate_codes_at = IMAGE ? gate_block + 36u * g.half + 4u
+                                         : (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
+    const unsigned up_codes_at = IMAGE ? up_block + 36u * g.half + 4u : (up_block + 2u + 32u * g.half) & ~3u;
     // ninth dword: the end of the codes where they start two bytes in, else the scale's dword
-    const unsigned gate_tail_at = g.code_shift ? gate_codes_at + 32u : gate_block & ~3u;
-    const unsigned up_tail_at = g.code_shift ? up_codes_at + 32u : up_block & ~3u;
+    const unsigned gate_tail_at = IMAGE ? gate_codes_at - 4u
+                                        : g.code_shift ? gate_codes_at + 32u : gate_block & ~3u;
+    const unsigned up_tail_at = IMAGE ? up_codes_at - 4u : g.code_shift ? up_codes_at + 32u : up_block & ~3u;
     // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
     // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
@@ -357,7 +380,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         int total_gate[N], total_up[N];
         {
             int totals[STREAMS][N];
-            iq2_half_dots<STREAMS, N>(now, g, act, totals);
+            iq2_half_dots<STREAMS, N, IMAGE>(now, g, act, totals);
 #pragma unroll
             for (int p = 0; p < N; ++p) {
                 total_gate[p] = totals[0][p];
@@ -374,11 +397,16 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         // lane holds the second half of its superblock, so where the scale rides in the first
         // half's codes it comes from the neighbour.
         const Iq2Half &mine = odd ? now[STREAMS - 1] : now[0];
-        // (the exchange runs in every lane: it reads its neighbour, which must be executing it)
-        const unsigned neighbour_word = (unsigned)dpp_move<0xb1, 0xf>((int)now[STREAMS - 1].lo.x);
-        const unsigned first_word = odd ? neighbour_word : now[0].lo.x;
-        const float weight_scale = 0.125f * f16_bits_to_float(
-            ((g.code_shift ? first_word : mine.tail) >> g.scale_shift) & 0xffffu);
+        float weight_scale;
+        if constexpr (IMAGE) {
+            weight_scale = 0.125f * f16_bits_to_float(mine.tail & 0xffffu);
+        } else {
+            // (the exchange runs in every lane: it reads its neighbour, which must be executing it)
+            const unsigned neighbour_word = (unsigned)dpp_move<0xb1, 0xf>((int)now[STREAMS - 1].lo.x);
+            const unsigned first_word = odd ? neighbour_word : now[0].lo.x;
+            weight_scale = 0.125f * f16_bits_to_float(
+                ((g.code_shift ? first_word : mine.tail) >> g.scale_shift) & 0xffffu);
+        }
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
             int t;
@@ -427,7 +455,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     __builtin_amdgcn_wave_barrier();
 }
 
-template <bool FUSED>
+template <bool FUSED, bool IMAGE>
 __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
 {
     extern __shared__ __align__(16) unsigned char sweep_lds[];
@@ -654,38 +682,80 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned row_end = row_begin + rows_of_item < a.out_rows ? row_begin + rows_of_item : a.out_rows;
         const unsigned long long live = population - pass;
         if (kSweepPairs >= 4 && live >= 4ull)
-            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
         else if (kSweepPairs >= 3 && live >= 3ull)
-            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
         else if (live >= 2ull)
-            iq2_sweep<FUSED, 2>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
         else
-            iq2_sweep<FUSED, 1>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
     }
 }
 
-bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs)
+bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs, bool image)
 {
     if (pairs > kClassMaxSweeps) return false;            // every sweep serves at least one pair
     const unsigned lanes_per_row = width / 128u;
     if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
-    if ((width / 256u * 66u) % 4u != 0u) return false;   // rows must start on dword boundaries
+    if (!image && (width / 256u * 66u) % 4u != 0u) return false;   // rows must start on dword boundaries
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u
         ? 64u / lanes_per_row : 1u;
     return out_rows % rows_per_iter == 0u;   // an iteration never reads past the last row
 }
 
-template <bool FUSED>
+template <bool FUSED, bool IMAGE>
 static int launch_iq2_sweep_variant(const GroupedArgs &a, hipStream_t stream)
 {
-    YVEX_ALLOW_DYNAMIC_LDS(iq2_sweep_kernel<FUSED>, kSweepLdsBytes);
-    iq2_sweep_kernel<FUSED><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
+    YVEX_ALLOW_DYNAMIC_LDS((iq2_sweep_kernel<FUSED, IMAGE>), kSweepLdsBytes);
+    iq2_sweep_kernel<FUSED, IMAGE><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
     return check_launch("moe_sweep_iq2");
 }
 
-int launch_iq2_sweep(const GroupedArgs &a, bool fused, hipStream_t stream)
+int launch_iq2_sweep(const GroupedArgs &a, bool fused, bool image, hipStream_t stream)
 {
-    return fused ? launch_iq2_sweep_variant<true>(a, stream) : launch_iq2_sweep_variant<false>(a, stream);
+    if (image)
+        return fused ? launch_iq2_sweep_variant<true, true>(a, stream)
+                     : launch_iq2_sweep_variant<false, true>(a, stream);
+    return fused ? launch_iq2_sweep_variant<true, false>(a, stream)
+                 : launch_iq2_sweep_variant<false, false>(a, stream);
+}
+
+// ---- the image: canonical IQ2_XXS superblocks re-packed for the sweeps -------------------------
+
+// One thread per half superblock: nine dwords out of the 66 canonical bytes.
+__global__ __launch_bounds__(256) void iq2_sweep_image_kernel(const unsigned char *canonical,
+                                                              unsigned long long blocks, unsigned *image)
+{
+    const unsigned long long at = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    if (at >= 2ull * blocks) return;
+    const unsigned long long block = at >> 1;
+    const unsigned half = (unsigned)(at & 1ull);
+    const unsigned char *b = canonical + block * 66ull;
+    unsigned *record = image + at * 9ull;
+    unsigned scales = 0u;
+#pragma unroll
+    for (unsigned j = 0; j < 4u; ++j) {
+        const unsigned char *group = b + 2u + 8u * (4u * half + j);
+        const unsigned grids = load_u32(group), aux = load_u32(group + 4u);
+        record[1u + 2u * j] = grids;
+        record[2u + 2u * j] = (aux & 127u) | (((aux >> 7) & 127u) << 8) | (((aux >> 14) & 127u) << 16) |
+                              (((aux >> 21) & 127u) << 24);
+        scales |= (aux >> 28) << (4u * j);
+    }
+    record[0] = load_u16(b) | (scales << 16);
 }
 
 }  // namespace yvex
+
+extern "C" uint64_t yvex_hip_iq2_sweep_image_bytes(uint64_t blocks) { return blocks * 72u; }
+
+extern "C" int yvex_hip_iq2_sweep_image_build(const uint8_t *canonical, uint64_t blocks, void *image,
+                                              yvex_hip_stream stream)
+{
+    if (!canonical || !image || !blocks || ((uintptr_t)image & 3u)) return yvex::ST_INVALID_ARG;
+    const uint64_t groups = (2u * blocks + 255u) / 256u;
+    if (groups > 0x7fffffffull) return yvex::ST_BOUNDS;
+    yvex::iq2_sweep_image_kernel<<<(unsigned)groups, 256, 0, yvex::as_stream(stream)>>>(canonical, blocks,
+                                                                                         (unsigned *)image);
+    return yvex::check_launch("iq2_sweep_image");
+}

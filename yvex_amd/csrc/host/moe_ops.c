@@ -153,9 +153,10 @@ static int family_admitted(const char *family)
 /* Activation / kernel-family policy of one expert triple (moe.c:905-990). */
 static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight_view *up,
                          const yvex_moe_weight_view *down, unsigned long long input_width,
-                         unsigned long long intermediate_width, int *act_q8, yvex_error *err)
+                         unsigned long long intermediate_width, int *act_q8, int *image, yvex_error *err)
 {
     int gate_encoded, up_encoded, down_encoded;
+    *image = 0;
     if (gate->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED ||
         up->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED ||
         down->activation > YVEX_EXECUTION_ACTIVATION_DEVICE_ENCODED)
@@ -171,15 +172,25 @@ static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight
                          strcmp(gate->kernel_family, up->kernel_family) != 0))
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
                                 "compiled MoE gate and up kernel-family decisions disagree");
-    /* moe.c:933-958: layouts must agree (FORMAT); a derived image is not executable by the
-     * row-batch path there either (UNSUPPORTED). */
+    /* moe.c:933-958: layouts must agree (FORMAT). The reference's row-batch path executes no
+     * derived image at all (UNSUPPORTED); this one executes the one image its expert sweeps
+     * read: IQ2_XXS tensors, device-encoded activations, the gfx950 sweep family on all three
+     * views. Any other derived view is refused as there. */
     if (gate->layout != up->layout || ((gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND) !=
                                        (down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)))
         return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
                                 "compiled routed MoE layouts disagree");
-    if (gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)
-        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
-                                "the row-batch path executes canonical rows, not a derived image");
+    if (gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND) {
+        if (!gate_encoded || !down_encoded || !down->kernel_family ||
+            strcmp(gate->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
+            strcmp(down->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
+            gate->qtype != YVEX_GGUF_QTYPE_IQ2_XXS || up->qtype != YVEX_GGUF_QTYPE_IQ2_XXS ||
+            down->qtype != YVEX_GGUF_QTYPE_IQ2_XXS)
+            return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                    "the row-batch path executes canonical rows, or the expert sweeps' "
+                                    "image of IQ2_XXS tensors with device-encoded activations");
+        *image = 1;
+    }
     if ((gate_encoded && !family_admitted(gate->kernel_family)) ||
         (down_encoded && !family_admitted(down->kernel_family)))
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
@@ -206,6 +217,9 @@ int yvex_rocm_moe_view_check(const yvex_rocm_backend *backend, const yvex_moe_we
     if (!capability || !geometry || !capability->device_compute_available)
         return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.weights",
                                 "qtype has no device compute on this backend");
+    if (view->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)
+        return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.weights",
+                                "this operation takes canonical rows, not a derived image");
     if (view->row_width != row_width || view->row_count != row_count || !geometry->block_size ||
         row_width % geometry->block_size ||
         row_width / geometry->block_size * geometry->bytes_per_block != view->row_bytes ||
@@ -240,12 +254,50 @@ static int view_resolve(const yvex_rocm_backend *backend, const yvex_moe_weight_
     return rc;
 }
 
+/* A view of the expert sweeps' image (src/runtime/moe.c:297-300 hands a derived binding over the
+ * same way): row geometry and encoded_bytes describe the canonical tensor, `encoded` (or
+ * device_address) and storage_bytes the image, 72 bytes per superblock. */
+static int image_view_resolve(const yvex_rocm_backend *backend, const yvex_moe_weight_view *view,
+                              unsigned long long row_width, unsigned long long row_count,
+                              unsigned long long *device_address, yvex_error *err)
+{
+    unsigned long long blocks;
+    if (view->row_width != row_width || view->row_count != row_count || row_width % 256ull ||
+        view->row_bytes != row_width / 256ull * 66ull ||
+        __builtin_mul_overflow(row_width / 256ull, row_count, &blocks) || blocks > ULLONG_MAX / 72ull ||
+        view->encoded_bytes != blocks * 66ull || view->storage_bytes != blocks * 72ull)
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                "MoE weight image disagrees with the layer plan");
+    if (view->device_address) {
+        *device_address = view->device_address;
+    } else if (!view->encoded ||
+               !yvex_rocm_resolve(backend, view->encoded, view->storage_bytes, device_address)) {
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                "MoE weight image is not inside the attached resident arena");
+    }
+    if (*device_address & 3ull)
+        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.weights",
+                                "MoE weight image must start on a dword boundary");
+    return YVEX_OK;
+}
+
+static int expert_view_resolve(const yvex_rocm_backend *backend, const yvex_moe_weight_view *view, int image,
+                               unsigned long long row_width, unsigned long long row_count,
+                               unsigned long long *device_address, yvex_error *err)
+{
+    return image ? image_view_resolve(backend, view, row_width, row_count, device_address, err)
+                 : view_resolve(backend, view, row_width, row_count, device_address, err);
+}
+
 static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weight_view *gate,
                                 const yvex_moe_weight_view *up, const yvex_moe_weight_view *down,
                                 unsigned long long gate_address, unsigned long long up_address,
                                 unsigned long long down_address, unsigned long long hidden,
-                                unsigned long long intermediate)
+                                unsigned long long intermediate, int image)
 {
+    const unsigned long long gate_row = image ? hidden / 256ull * 72ull : gate->row_bytes;
+    const unsigned long long up_row = image ? hidden / 256ull * 72ull : up->row_bytes;
+    const unsigned long long down_row = image ? intermediate / 256ull * 72ull : down->row_bytes;
     w->gate = (const uint8_t *)(uintptr_t)gate_address;
     w->up = (const uint8_t *)(uintptr_t)up_address;
     w->down = (const uint8_t *)(uintptr_t)down_address;
@@ -254,12 +306,13 @@ static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weigh
     w->down_qtype = down->qtype;
     w->hidden = hidden;
     w->intermediate = intermediate;
-    w->gate_row_bytes = gate->row_bytes;
-    w->up_row_bytes = up->row_bytes;
-    w->down_row_bytes = down->row_bytes;
-    w->gate_expert_bytes = gate->row_bytes * intermediate;
-    w->up_expert_bytes = up->row_bytes * intermediate;
-    w->down_expert_bytes = down->row_bytes * hidden;
+    w->gate_row_bytes = gate_row;
+    w->up_row_bytes = up_row;
+    w->down_row_bytes = down_row;
+    w->gate_expert_bytes = gate_row * intermediate;
+    w->up_expert_bytes = up_row * intermediate;
+    w->down_expert_bytes = down_row * hidden;
+    w->gate_up_image = w->down_image = image;
 }
 
 /* Expert weights the matrix-core row-batch kernels take: gate and up of one format, IQ2_XXS (16)
@@ -274,7 +327,8 @@ static int same_expert_shape(const yvex_hip_expert_weights *a, const yvex_hip_ex
 {
     return a->gate_qtype == b->gate_qtype && a->up_qtype == b->up_qtype &&
            a->down_qtype == b->down_qtype && a->hidden == b->hidden &&
-           a->intermediate == b->intermediate;
+           a->intermediate == b->intermediate && a->gate_up_image == b->gate_up_image &&
+           a->down_image == b->down_image;
 }
 
 /* ---- launch graphs -------------------------------------------------------------------------
@@ -435,7 +489,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     const void *activations;
     void *combined_target;
     unsigned long long table_address = 0ull;
-    int envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
+    int envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
     enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
@@ -526,11 +580,11 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     has_shared = layer->shared_experts == 1ull;
     rc = expert_policy(&views[YVEX_MOE_WEIGHT_ROUTED_GATE], &views[YVEX_MOE_WEIGHT_ROUTED_UP],
                        &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], hidden, layer->expert_intermediate_width,
-                       &routed_q8, err);
+                       &routed_q8, &routed_image, err);
     if (rc == YVEX_OK && has_shared)
         rc = expert_policy(&views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
                            &views[YVEX_MOE_WEIGHT_SHARED_DOWN], hidden, layer->shared_intermediate_width,
-                           &shared_q8, err);
+                           &shared_q8, &shared_image, err);
     if (rc != YVEX_OK) return rc;
     /* weights: router [experts x hidden], optional bias [1 x experts], expert-major matrices */
     rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER], hidden, experts, &router_address, err);
@@ -544,23 +598,23 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
                                   "MoE hash table holds fewer rows than the plan names");
     }
     if (rc == YVEX_OK)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], hidden,
-                          experts * layer->expert_intermediate_width, &addresses[0], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], routed_image, hidden,
+                                 experts * layer->expert_intermediate_width, &addresses[0], err);
     if (rc == YVEX_OK)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_UP], hidden,
-                          experts * layer->expert_intermediate_width, &addresses[1], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_UP], routed_image, hidden,
+                                 experts * layer->expert_intermediate_width, &addresses[1], err);
     if (rc == YVEX_OK)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], layer->expert_intermediate_width,
-                          experts * hidden, &addresses[2], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], routed_image,
+                                 layer->expert_intermediate_width, experts * hidden, &addresses[2], err);
     if (rc == YVEX_OK && has_shared)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_GATE], hidden,
-                          layer->shared_intermediate_width, &addresses[3], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_GATE], shared_image, hidden,
+                                 layer->shared_intermediate_width, &addresses[3], err);
     if (rc == YVEX_OK && has_shared)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_UP], hidden,
-                          layer->shared_intermediate_width, &addresses[4], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_UP], shared_image, hidden,
+                                 layer->shared_intermediate_width, &addresses[4], err);
     if (rc == YVEX_OK && has_shared)
-        rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], layer->shared_intermediate_width,
-                          hidden, &addresses[5], err);
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], shared_image,
+                                 layer->shared_intermediate_width, hidden, &addresses[5], err);
     if (rc == YVEX_OK && envelope) {
         /* ingress coefficients: the mixing function is a matrix over the expanded row, the rest
          * are flat rows of F32, BF16 or I32 values (src/graph/moe.c:405-428) */
@@ -595,17 +649,18 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.moe.rows", "workspace acquisition failed");
     fill_expert_weights(&routed, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], &views[YVEX_MOE_WEIGHT_ROUTED_UP],
                         &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], addresses[0], addresses[1], addresses[2],
-                        hidden, layer->expert_intermediate_width);
+                        hidden, layer->expert_intermediate_width, routed_image);
     if (has_shared)
         fill_expert_weights(&shared, &views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
                             &views[YVEX_MOE_WEIGHT_SHARED_DOWN], addresses[3], addresses[4], addresses[5],
-                            hidden, layer->shared_intermediate_width);
+                            hidden, layer->shared_intermediate_width, shared_image);
     /* Row batches whose buckets average eight pairs or more go to the int8 matrix-core kernels
      * (IQ2_XXS or Q4_K weights, Q8_K activations); below that the decode sweeps, which read an expert's
      * bytes once per four pairs, are faster. The reference switches its tensor-core kernels on
-     * from 16 input rows (src/backend/cuda/private.h:461-464). */
-    row_batch = routed_q8 && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
-    shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
+     * from 16 input rows (src/backend/cuda/private.h:461-464). Only the sweeps read their image:
+     * experts held as one stay on the sweeps at any width. */
+    row_batch = routed_q8 && !routed_image && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
+    shared_row_batch = row_batch && has_shared && shared_q8 && !shared_image && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",

@@ -331,6 +331,7 @@ static void fill_weights(yvex_hip_expert_weights *w, const yvex_moe_weight_view 
                          const unsigned long long address[3], unsigned long long hidden,
                          unsigned long long intermediate)
 {
+    memset(w, 0, sizeof(*w));      /* canonical rows: no sweep image */
     w->gate = (const uint8_t *)(uintptr_t)address[0];
     w->up = (const uint8_t *)(uintptr_t)address[1];
     w->down = (const uint8_t *)(uintptr_t)address[2];

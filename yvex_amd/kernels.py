@@ -34,7 +34,7 @@ class ExpertWeights(C.Structure):
                 ("gate_row_bytes", C.c_uint64), ("up_row_bytes", C.c_uint64),
                 ("down_row_bytes", C.c_uint64),
                 ("gate_expert_bytes", C.c_uint64), ("up_expert_bytes", C.c_uint64),
-                ("down_expert_bytes", C.c_uint64)]
+                ("down_expert_bytes", C.c_uint64), ("gate_up_image", C.c_int), ("down_image", C.c_int)]
 
 
 def row_bytes(qtype: int, width: int) -> int:
@@ -263,6 +263,30 @@ def expert_weights(gate, up, down, qtypes, hidden, intermediate) -> ExpertWeight
     w.down_expert_bytes = w.down_row_bytes * hidden
     w._keep = (gate, up, down)
     return w
+
+
+def iq2_sweep_image(canonical):
+    """The sweep image of canonical IQ2_XXS bytes (a uint8 tensor of whole superblocks)."""
+    blocks = canonical.numel() // 66
+    image = torch.empty(blocks * 72, dtype=torch.uint8, device=canonical.device)
+    _call("yvex_hip_iq2_sweep_image_build", _ptr(canonical), C.c_uint64(blocks), _ptr(image), _stream())
+    return image
+
+
+def expert_weights_image(w: ExpertWeights, hidden, intermediate) -> ExpertWeights:
+    """The same IQ2_XXS experts with all three matrices as sweep images."""
+    gate, up, down = (iq2_sweep_image(t) for t in w._keep)
+    out = ExpertWeights()
+    out.gate, out.up, out.down = gate.data_ptr(), up.data_ptr(), down.data_ptr()
+    out.gate_qtype, out.up_qtype, out.down_qtype = w.gate_qtype, w.up_qtype, w.down_qtype
+    out.hidden, out.intermediate = hidden, intermediate
+    out.gate_row_bytes = out.up_row_bytes = hidden // 256 * 72
+    out.down_row_bytes = intermediate // 256 * 72
+    out.gate_expert_bytes = out.up_expert_bytes = out.gate_row_bytes * intermediate
+    out.down_expert_bytes = out.down_row_bytes * hidden
+    out.gate_up_image = out.down_image = 1
+    out._keep = (gate, up, down)
+    return out
 
 
 def _wl_ptrs(wl):

@@ -16,13 +16,17 @@ from . import kernels as K
 class MoeLayer:
     def __init__(self, *, hidden, intermediate, experts, topk, qtypes, routed, shared=None,
                  bias=None, scoring=K.SQRT_SOFTPLUS, normalize=True, scaling=1.0, limit=10.0,
-                 act_q8=True, max_rows=64, device="cuda", matrix_cores=False):
+                 act_q8=True, max_rows=64, device="cuda", matrix_cores=False, sweep_image=False):
         self.hidden, self.intermediate, self.experts, self.topk = hidden, intermediate, experts, topk
         self.qtypes, self.scoring, self.normalize = qtypes, scoring, normalize
         self.scaling, self.limit, self.act_q8 = scaling, limit, act_q8
         self.device = device
         self.routed = K.expert_weights(*routed, qtypes, hidden, intermediate)
         self.shared = K.expert_weights(*shared, qtypes, hidden, intermediate) if shared else None
+        if sweep_image:      # IQ2_XXS experts re-packed for the decode sweeps (built on the device)
+            self.routed = K.expert_weights_image(self.routed, hidden, intermediate)
+            if self.shared is not None:
+                self.shared = K.expert_weights_image(self.shared, hidden, intermediate)
         self.bias = bias
         self.max_rows = max_rows
         pairs = max_rows * topk
