@@ -11,11 +11,11 @@
 // and the superblock values of a row are added in fp32.
 //
 // A 32-value sub-block is exactly the reduction depth of V_MFMA_I32_32X32X32_I8. The weight
-// operand carries sc_j * nibble (at most 63 * 15 = 945) as two int8 limbs, value = 128 hi + lo
-// with lo in 0..127 and hi in 0..7, so each sub-block costs two matrix instructions per 32
-// tokens and the int32 accumulators run over the whole superblock without rescaling. The
-// minimum term is one more reduction of depth 8 (the m_j against the pair sums of bsums, again in
-// two limbs) through the same instruction.
+// operand carries sc_j * nibble (at most 63 * 15 = 945) as two int8 limbs, value = 8 hi + lo
+// with lo = (sc_j mod 8) * nibble and hi = (sc_j div 8) * nibble, both at most 105, so each
+// sub-block costs two matrix instructions per 32 tokens and the int32 accumulators run over the
+// whole superblock without rescaling. The minimum term is one more reduction of depth 8 (the m_j
+// against the pair sums of bsums, in two limbs of base 128) through the same instruction.
 //
 // A workgroup owns 32 weight rows x 32 or 64 tokens; its four waves take every fourth
 // superblock and their fp32 partial tiles are added in wave order, so results do not depend on
@@ -84,14 +84,18 @@ __device__ __forceinline__ void load_super(const DenseQ4kArgs &g, const unsigned
     (void)g;
 }
 
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
 // Two int8 limbs of sc * nibble for the four nibbles of one dword (already shifted so that the
-// wanted nibble of every byte sits in its low four bits).
+// wanted nibble of every byte sits in its low four bits), value = 8 hi + lo. The 6-bit scale is
+// split as sc = 8 s_hi + s_lo with both parts in 0..7: a limb byte nibble * s is at most 105, so
+// one 16-bit lane multiply scales two bytes at once without a carry from one into the next.
 __device__ __forceinline__ void limbs(unsigned x, unsigned sc, unsigned &lo, unsigned &hi)
 {
-    const unsigned even = (x & 0x000f000fu) * sc;              // bytes 0 and 2, in 16-bit lanes
-    const unsigned odd = ((x >> 8) & 0x000f000fu) * sc;        // bytes 1 and 3
-    lo = (even & 0x007f007fu) | ((odd & 0x007f007fu) << 8);
-    hi = ((even >> 7) & 0x000f000fu) | (((odd >> 7) & 0x000f000fu) << 8);
+    const unsigned nibbles = x & 0x0f0f0f0fu;
+    const unsigned low = (sc & 7u) * 0x00010001u, high = ((sc >> 3) & 7u) * 0x00010001u;
+    lo = __builtin_bit_cast(unsigned, __builtin_bit_cast(u16x2, nibbles) * __builtin_bit_cast(u16x2, low));
+    hi = __builtin_bit_cast(unsigned, __builtin_bit_cast(u16x2, nibbles) * __builtin_bit_cast(u16x2, high));
 }
 
 __device__ __forceinline__ v4i as_v4i(uint4 v)
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
             const float da = cur.act_scale[nt];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int dot = (hi_sum[nt][i] << 7) + lo_sum[nt][i];
+                const int dot = (hi_sum[nt][i] << 3) + lo_sum[nt][i];
                 const int minimum = (min_hi[nt][i] << 7) + min_lo[nt][i];
                 const float left = (da * d_of[i]) * (float)dot;
                 const float right = (da * dmin_of[i]) * (float)minimum;
@@ -379,7 +383,7 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
         for (unsigned nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int dot = (hi_sum[nt][i] << 7) + lo_sum[nt][i];
+                const int dot = (hi_sum[nt][i] << 3) + lo_sum[nt][i];
                 const int minimum = (min_hi[nt][i] << 7) + min_lo[nt][i];
                 const float left = (da[nt] * d_of[i]) * (float)dot;
                 const float right = (da[nt] * dmin_of[i]) * (float)minimum;
@@ -583,7 +587,7 @@ __global__ __launch_bounds__(256) void grouped_q4k_kernel(GroupedQ4kArgs g)
 #pragma unroll
                 for (unsigned k = 0; k < 4u; ++k) {
                     const unsigned i = 4u * q4 + k;
-                    const int dot = (hi_sum[m][i] << 7) + lo_sum[m][i];
+                    const int dot = (hi_sum[m][i] << 3) + lo_sum[m][i];
                     const int minimum = (min_hi[m][i] << 7) + min_lo[m][i];
                     const float left = (da * d_of[k]) * (float)dot;
                     const float right = (da * dmin_of[k]) * (float)minimum;
