@@ -60,7 +60,14 @@ constexpr unsigned kClassMaxSweeps = 4096u;
 constexpr unsigned kClassCountBase = kParkBase + kSweepWaves * kParkBytes;
 constexpr unsigned kClassWaveBase = kClassCountBase + 32u;    // per wave and class: entries of a turn
 constexpr unsigned kClassListBase = kClassCountBase + 32u + kSweepWaves * 16u;
-constexpr unsigned kSweepLdsBytes = kClassListBase + kClassMaxSweeps * 4u;
+// What opens an item without a round trip to memory: expert, first ordered pair and population of
+// every routed bucket, and {source pair, route weight} of every ordered pair when the routed
+// problem has at most kPairCacheMax of them (decode widths; wider batches read them from memory).
+constexpr unsigned kBucketBase = kClassListBase + kClassMaxSweeps * 4u;   // 256 x {expert, first, population}
+constexpr unsigned kPairCacheBase = kBucketBase + 256u * 12u;
+constexpr unsigned kPairCacheMax = 1024u;
+constexpr unsigned kSweepLdsBytes = kPairCacheBase + kPairCacheMax * 8u;
+static_assert(kSweepLdsBytes <= 160u * 1024u, "the sweep's tables, lists and caches must fit the LDS of a compute unit");
 
 __device__ __forceinline__ void lds_store_u32(unsigned address, unsigned v)
 {
@@ -87,6 +94,15 @@ __device__ __forceinline__ void lds_store_uint4(unsigned address, uint4 v)
 #else
     (void)address;
     (void)v;
+#endif
+}
+__device__ __forceinline__ uint2 lds_load_uint2(unsigned address)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<__attribute__((address_space(3))) const uint2 *>(address);
+#else
+    (void)address;
+    return make_uint2(0u, 0u);
 #endif
 }
 __device__ __forceinline__ unsigned lds_load_u32(unsigned address)
@@ -281,7 +297,7 @@ template <bool FUSED, int N, bool IMAGE>
 __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedProblem &pr,
                                           const SweepLane &g, const unsigned char *gate_e,
                                           const unsigned char *up_e, unsigned long long first_ordered,
-                                          unsigned row_begin, unsigned row_end)
+                                          unsigned row_begin, unsigned row_end, bool pairs_in_lds)
 {
     const unsigned lane = threadIdx.x & 63u;
     const bool odd = (lane & 1u) != 0u;
@@ -296,9 +312,16 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 #pragma unroll
     for (int p = 0; p < N; ++p) {
         const unsigned long long ordered = first_ordered + p;
-        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        unsigned long long source;
+        if (pairs_in_lds) {      // wave-uniform
+            const uint2 cached = lds_load_uint2(kPairCacheBase + 8u * (unsigned)ordered);
+            source = cached.x;
+            route_weight[p] = __uint_as_float(cached.y);
+        } else {
+            source = pr.order ? pr.order[ordered] : ordered;
+            route_weight[p] = pr.route_weights ? pr.route_weights[source] : 1.0f;
+        }
         const unsigned long long arow = pr.act_by_ordered_pair ? ordered : source / pr.topk;
-        route_weight[p] = pr.route_weights ? pr.route_weights[source] : 1.0f;
         out_index[p] = pr.out_by_source_pair ? source : ordered;
         const unsigned char *blk = (const unsigned char *)pr.activations + arow * pr.act_stride +
                                    (unsigned long long)(g.live ? g.super : 0u) * kQ8KBytes;
@@ -472,8 +495,36 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     unsigned population_here = 0u;
     if (!routed_fixed && tid < 256u && tid < routed.experts)
         population_here = (unsigned)routed.bucket_populations[tid];
+    // ... and so are the routed buckets' experts and first pairs and the pairs' sources, which
+    // the items will find in LDS
+    unsigned long long expert_here = 0ull, first_here = 0ull;
+    if (!routed_fixed && tid < 256u && tid < routed.experts) {
+        expert_here = routed.expert_ids[tid];
+        first_here = routed.bucket_offsets[tid];
+    }
+    const bool pairs_in_lds = !routed_fixed && routed.order != nullptr && routed.pairs <= kPairCacheMax;
+    static_assert(kPairCacheMax <= 2u * kSweepThreads, "two cached pairs a thread");
+    unsigned long long source_here[2] = {~0ull, ~0ull};
+    if (pairs_in_lds) {
+#pragma unroll
+        for (unsigned k = 0; k < 2u; ++k)
+            if (tid + k * kSweepThreads < routed.pairs) source_here[k] = routed.order[tid + k * kSweepThreads];
+    }
     sweep_tables_fill();
     if (tid == 0u) lds_store_u32(kTicketAddress, 0u);
+    if (pairs_in_lds) {
+        float weight_here[2];
+#pragma unroll
+        for (unsigned k = 0; k < 2u; ++k)   // a source outside the problem reads no weight here; the sweep's own checks refuse it
+            weight_here[k] = routed.route_weights && source_here[k] < routed.pairs
+                ? routed.route_weights[source_here[k]] : 1.0f;
+#pragma unroll
+        for (unsigned k = 0; k < 2u; ++k)
+            if (tid + k * kSweepThreads < routed.pairs)
+                lds_store_uint2(kPairCacheBase + 8u * (tid + k * kSweepThreads),
+                                make_uint2(source_here[k] < 0xffffffffull ? (unsigned)source_here[k] : 0xffffffffu,
+                                           __float_as_uint(weight_here[k])));
+    }
 
     // ---- sweep numbering of the routed buckets: exclusive prefix of ceil(population / 4) ----
     if (!routed_fixed && buckets > 256u) {
@@ -489,6 +540,13 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
             mine = (population_here + (unsigned)kSweepPairs - 1u) / (unsigned)kSweepPairs;
             lds_store_u32(scratch + 4u * tid, mine);
             lds_store_u32(kPopulationBase + 4u * tid, population_here);
+            if (tid < buckets) {
+                // (values past 32 bits fail the item's range check through their low words' sum
+                // only by accident, so they are clamped to a value that always fails it)
+                lds_store_u32(kBucketBase + 12u * tid, expert_here < 0xffffffffull ? (unsigned)expert_here : 0xffffffffu);
+                lds_store_u32(kBucketBase + 12u * tid + 4u, first_here < 0xffffffffull ? (unsigned)first_here : 0xffffffffu);
+                lds_store_u32(kBucketBase + 12u * tid + 8u, population_here);
+            }
         }
         __syncthreads();
         unsigned from = scratch, to = scratch + 1024u;
@@ -665,11 +723,18 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned word = lds_load_u32(kClassListBase + 4u * (start + position / tiles));
         const GroupedProblem &pr = a.problem[(word & 0x40000000u) && a.problems > 1u ? 1u : 0u];
         unsigned long long expert = 0ull, first = 0ull, population = pr.pairs;
+        const bool is_routed = !(word & 0x40000000u);
         if (!(word & 0x80000000u)) {
             const unsigned bucket = (word >> 16) & 0x3fffu;
-            expert = pr.expert_ids[bucket];
-            first = pr.bucket_offsets[bucket];
-            population = pr.bucket_populations[bucket];
+            if (is_routed) {          // the routed problem's buckets were copied at kernel start
+                expert = lds_load_u32(kBucketBase + 12u * bucket);
+                first = lds_load_u32(kBucketBase + 12u * bucket + 4u);
+                population = lds_load_u32(kBucketBase + 12u * bucket + 8u);
+            } else {
+                expert = pr.expert_ids[bucket];
+                first = pr.bucket_offsets[bucket];
+                population = pr.bucket_populations[bucket];
+            }
         }
         const unsigned long long pass = (unsigned long long)(word & 0xffffu) * kSweepPairs;
         if (expert >= pr.experts || first + population > pr.pairs || pass >= population) {
@@ -681,14 +746,15 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned row_begin = (is_short ? long_rows : 0u) + tile * rows_of_item;
         const unsigned row_end = row_begin + rows_of_item < a.out_rows ? row_begin + rows_of_item : a.out_rows;
         const unsigned long long live = population - pass;
+        const bool cached = pairs_in_lds && is_routed;
         if (kSweepPairs >= 4 && live >= 4ull)
-            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (kSweepPairs >= 3 && live >= 3ull)
-            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (live >= 2ull)
-            iq2_sweep<FUSED, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else
-            iq2_sweep<FUSED, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end);
+            iq2_sweep<FUSED, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
     }
 }
 
