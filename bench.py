@@ -492,7 +492,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
         "token_tiles": tile_classes(populations.cpu().tolist()),
         "max_bucket_population": int(populations.max().item()),
         "roofline": {"bound": "mfma",
-                     "kernel": "mfma_iq2_kernel<fused gate/up>" if qt == 16 else "grouped_q4k_kernel<fused gate/up>",
+                     "kernel": "mfma_iq2_kernel<fused gate/up>" if qt == 16 else "rows_q4k_kernel<fused gate/up>",
                      "achieved": round(up_ops / (up_ms * 1e-3) / 1e12, 2), "peak": MFMA_INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": round(up_ops / (up_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
                      "launch_ms": round(up_ms, 4)},

@@ -417,237 +417,7 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
     }
 }
 
-// ---- expert buckets: the row-batch MoE with Q4_K expert weights ---------------------------------
-//
-// The same tile arithmetic over an expert-major worklist (src/backend/cuda/tensorcore.cu:378-702
-// is the reference's counterpart): a workgroup owns (token tile of 32 ordered pairs of one bucket,
-// 32 weight rows of that bucket's expert), its four waves take every fourth superblock. With FUSED
-// the gate and the up matrix are multiplied side by side against the same activation operand and
-// the clamped SwiGLU with the route weight is applied to the summed tiles; otherwise the value is
-// rounded to bf16 as an expert output. Token tiles are numbered bucket by bucket; every
-// workgroup finds its bucket from the bucket populations (at most 256 of them).
-struct GroupedQ4kArgs {
-    GroupedProblem pr;
-    unsigned blocks;         // superblocks per weight row
-    unsigned out_rows;       // weight rows per expert
-    double limit;
-    int *status;
-};
-
-template <bool FUSED>
-__global__ __launch_bounds__(256) void grouped_q4k_kernel(GroupedQ4kArgs g)
-{
-    constexpr unsigned M = FUSED ? 2u : 1u;          // weight matrices multiplied side by side
-    __shared__ __align__(16) float row_scale[4][M][2][32];
-    __shared__ float partial[3][M][16][64];
-    __shared__ unsigned wave_tiles[4];
-    __shared__ unsigned long long found[3];          // expert, first ordered pair of the tile, pairs in it
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned r = lane & 31u, h = lane >> 5;
-    const GroupedProblem &pr = g.pr;
-
-    // which bucket holds token tile blockIdx.y
-    if (threadIdx.x == 0u) found[2] = 0ull;
-    if (!pr.expert_ids) {
-        if (threadIdx.x == 0u) {
-            const unsigned long long first = (unsigned long long)blockIdx.y * 32ull;
-            found[0] = 0ull;
-            found[1] = first;
-            found[2] = first < pr.pairs ? (pr.pairs - first < 32ull ? pr.pairs - first : 32ull) : 0ull;
-        }
-    } else {
-        const unsigned buckets = (unsigned)pr.counts[0];
-        const unsigned long long population = threadIdx.x < buckets ? pr.bucket_populations[threadIdx.x] : 0ull;
-        const unsigned tiles = (unsigned)((population + 31ull) / 32ull);
-        unsigned inclusive = tiles;
-#pragma unroll
-        for (int offset = 1; offset < 64; offset <<= 1) {
-            const unsigned below = __shfl_up(inclusive, offset, kWave);
-            if ((int)lane >= offset) inclusive += below;
-        }
-        if (lane == 63u) wave_tiles[wave] = inclusive;
-        __syncthreads();
-        unsigned before = 0u;
-        for (unsigned w = 0; w < wave; ++w) before += wave_tiles[w];
-        inclusive += before;
-        const unsigned exclusive = inclusive - tiles;
-        if (tiles && blockIdx.y >= exclusive && blockIdx.y < inclusive) {
-            const unsigned long long inside = (unsigned long long)(blockIdx.y - exclusive) * 32ull;
-            found[0] = pr.expert_ids[threadIdx.x];
-            found[1] = pr.bucket_offsets[threadIdx.x] + inside;
-            found[2] = population - inside < 32ull ? population - inside : 32ull;
-        }
-    }
-    __syncthreads();
-    const unsigned long long expert = found[0], first = found[1];
-    const unsigned tokens = (unsigned)found[2];
-    if (!tokens) return;                                   // a tile number past the last bucket
-    if (expert >= pr.experts || first + tokens > pr.pairs) {
-        if (threadIdx.x == 0u) raise_status(g.status, 2);
-        return;
-    }
-
-    // this lane's token: activation row, output place, route weight
-    const unsigned long long ordered = first + (r < tokens ? r : tokens - 1u);
-    const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
-    const unsigned long long act_row = pr.act_by_ordered_pair ? ordered : source / pr.topk;
-    const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
-    const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
-    const unsigned char *arow = (const unsigned char *)pr.activations + act_row * pr.act_stride;
-
-    const unsigned long long row0 = (unsigned long long)blockIdx.x * 32ull;
-    unsigned long long wr = row0 + r;
-    if (wr >= g.out_rows) wr = g.out_rows - 1ull;
-    const unsigned char *wrow[M];
-    wrow[0] = pr.gate + expert * pr.expert_bytes + wr * pr.row_bytes;
-    if constexpr (FUSED) wrow[1] = pr.up + expert * pr.up_expert_bytes + wr * pr.up_row_bytes;
-
-    float acc[M][16];
-#pragma unroll
-    for (unsigned m = 0; m < M; ++m)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
-
-    for (unsigned sb = wave; sb < g.blocks; sb += 4u) {
-        const unsigned char *ab = arow + (unsigned long long)sb * kQ8KBytes;
-        const float da = *reinterpret_cast<const float *>(ab);
-        uint4 a[8], bsums[2];
-#pragma unroll
-        for (unsigned c = 0; c < 8u; ++c) {
-            const unsigned *p = reinterpret_cast<const unsigned *>(ab + 4u + 32u * c + 16u * h);
-            a[c] = make_uint4(p[0], p[1], p[2], p[3]);
-        }
-        {
-            const unsigned *b = reinterpret_cast<const unsigned *>(ab + 260u);
-            bsums[0] = make_uint4(b[0], b[1], b[2], b[3]);
-            bsums[1] = make_uint4(b[4], b[5], b[6], b[7]);
-        }
-        uint2 bl, bh;
-        bsum_limbs(bsums, bl, bh);
-        v4i b_lo = {0, 0, 0, 0}, b_hi = {0, 0, 0, 0};
-        if (h == 0u) {
-            b_lo[0] = (int)bl.x; b_lo[1] = (int)bl.y;
-            b_hi[0] = (int)bh.x; b_hi[1] = (int)bh.y;
-        }
-        v16i lo_sum[M], hi_sum[M], min_lo[M], min_hi[M];
-#pragma unroll
-        for (unsigned m = 0; m < M; ++m) {
-            const unsigned char *w = wrow[m] + (unsigned long long)sb * 144ull;
-            const unsigned head = *reinterpret_cast<const unsigned *>(w);
-            const uint3 scales = *reinterpret_cast<const uint3 *>(w + 4u);
-            uint4 qs[4];
-#pragma unroll
-            for (unsigned j = 0; j < 4u; ++j)
-                qs[j] = *reinterpret_cast<const uint4 *>(w + 16u + 32u * j + 16u * h);
-            const unsigned s0 = scales.x, s1 = scales.y, s2 = scales.z;
-            const unsigned sc_pack[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
-            const unsigned mn_pack[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
-            if (h == 0u) {
-                row_scale[wave][m][0][r] = f16_bits_to_float(head & 0xffffu);
-                row_scale[wave][m][1][r] = f16_bits_to_float(head >> 16);
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) lo_sum[m][i] = hi_sum[m][i] = 0;
-#pragma unroll
-            for (unsigned c = 0; c < 8u; ++c) {
-                const unsigned sc = (sc_pack[c >> 2] >> (8u * (c & 3u))) & 255u;
-                const uint4 q = qs[c >> 1];
-                const unsigned shift = (c & 1u) * 4u;
-                v4i a_lo, a_hi;
-                unsigned lo, hi;
-                limbs(q.x >> shift, sc, lo, hi); a_lo[0] = (int)lo; a_hi[0] = (int)hi;
-                limbs(q.y >> shift, sc, lo, hi); a_lo[1] = (int)lo; a_hi[1] = (int)hi;
-                limbs(q.z >> shift, sc, lo, hi); a_lo[2] = (int)lo; a_hi[2] = (int)hi;
-                limbs(q.w >> shift, sc, lo, hi); a_lo[3] = (int)lo; a_hi[3] = (int)hi;
-                const v4i b = as_v4i(a[c]);
-                lo_sum[m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo, b, lo_sum[m], 0, 0, 0);
-                hi_sum[m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi, b, hi_sum[m], 0, 0, 0);
-            }
-            v4i m_op = {0, 0, 0, 0};
-            if (h == 0u) {
-                m_op[0] = (int)mn_pack[0];
-                m_op[1] = (int)mn_pack[1];
-            }
-            v16i zero;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) zero[i] = 0;
-            min_lo[m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(m_op, b_lo, zero, 0, 0, 0);
-            min_hi[m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(m_op, b_hi, zero, 0, 0, 0);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (unsigned m = 0; m < M; ++m) {
-#pragma unroll
-            for (unsigned q4 = 0; q4 < 4u; ++q4) {
-                const float4 d = *reinterpret_cast<const float4 *>(&row_scale[wave][m][0][8u * q4 + 4u * h]);
-                const float4 mn = *reinterpret_cast<const float4 *>(&row_scale[wave][m][1][8u * q4 + 4u * h]);
-                const float d_of[4] = {d.x, d.y, d.z, d.w}, dmin_of[4] = {mn.x, mn.y, mn.z, mn.w};
-#pragma unroll
-                for (unsigned k = 0; k < 4u; ++k) {
-                    const unsigned i = 4u * q4 + k;
-                    const int dot = (hi_sum[m][i] << 3) + lo_sum[m][i];
-                    const int minimum = (min_hi[m][i] << 7) + min_lo[m][i];
-                    const float left = (da * d_of[k]) * (float)dot;
-                    const float right = (da * dmin_of[k]) * (float)minimum;
-                    acc[m][i] += left - right;
-                }
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-
-    if (wave) {
-#pragma unroll
-        for (unsigned m = 0; m < M; ++m)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) partial[wave - 1u][m][i][lane] = acc[m][i];
-    }
-    __syncthreads();
-    if (wave || r >= tokens) return;
-    const float limit_f32 = (float)g.limit;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const unsigned long long row = row0 + 8u * (i >> 2) + 4u * h + (i & 3);
-        if (row >= g.out_rows) continue;
-        float sum[M];
-#pragma unroll
-        for (unsigned m = 0; m < M; ++m)
-            sum[m] = ((acc[m][i] + partial[0][m][i][lane]) + partial[1][m][i][lane]) + partial[2][m][i][lane];
-        float value;
-        if constexpr (FUSED) value = swiglu_bf16_fast(sum[0], sum[1], route_weight, g.limit, limit_f32);
-        else value = bf16_round(sum[0]);
-        if (!finite_f32(value)) raise_status(g.status, 1);
-        else pr.out[out_index * g.out_rows + row] = value;
-    }
-}
-
 }  // namespace
-
-int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t width, uint64_t out_rows,
-                            double limit, int *status, hipStream_t stream)
-{
-    if (!width || width % 256u || !out_rows) return ST_BOUNDS;
-    if (problem.row_bytes != width / 256u * 144u || (fused && problem.up_row_bytes != problem.row_bytes))
-        return ST_BOUNDS;
-    if (((uintptr_t)problem.gate & 15u) || (fused && ((uintptr_t)problem.up & 15u)) ||
-        ((uintptr_t)problem.activations & 3u) || (problem.expert_bytes & 15u) ||
-        (fused && (problem.up_expert_bytes & 15u)))
-        return ST_INVALID_ARG;
-    if (problem.experts > 256u && problem.expert_ids) return ST_BOUNDS;
-    const uint64_t row_tiles = (out_rows + 31u) / 32u;
-    // token tiles: every bucket may end in a partial tile
-    const uint64_t token_tiles = problem.expert_ids ? (uint64_t)problem.pairs / 32u + problem.experts
-                                                    : ((uint64_t)problem.pairs + 31u) / 32u;
-    if (row_tiles > 0x7fffffffull || token_tiles > 65535ull) return ST_BOUNDS;
-    GroupedQ4kArgs g{problem, (unsigned)(width / 256u), (unsigned)out_rows, limit, status};
-    const dim3 grid((unsigned)row_tiles, (unsigned)token_tiles);
-    if (fused) grouped_q4k_kernel<true><<<grid, 256, 0, stream>>>(g);
-    else grouped_q4k_kernel<false><<<grid, 256, 0, stream>>>(g);
-    return check_launch("moe_rows_q4k");
-}
 
 int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
@@ -670,6 +440,10 @@ int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t r
     } else {
         const uint64_t token_tiles = (input_rows + 63u) / 64u;
         if (token_tiles > 65535ull) return ST_BOUNDS;
+        // enough (128 rows x 64 tokens) tiles for every compute unit: operands staged through LDS
+        if ((row_count + 127u) / 128u * token_tiles >= compute_units())
+            return launch_q4k_rows_staged(encoded, row_count, row_width, row_bytes, act_q8k, input_rows,
+                                          additive, out, out_stride, output_bf16, status, stream);
         dense_q4k_kernel<2><<<dim3((unsigned)row_tiles, (unsigned)token_tiles), 256, 0, stream>>>(g);
     }
     return check_launch("dense_q4k");

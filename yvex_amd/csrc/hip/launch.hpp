@@ -52,6 +52,12 @@ int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t r
                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
                           const float *additive, float *out, uint64_t out_stride, bool output_bf16,
                           int *status, hipStream_t stream);
+// The same product with its operands staged through LDS, for batches that fill every compute
+// unit with (128 rows x 64 tokens) tiles (rows_q4k.hip).
+int launch_q4k_rows_staged(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                          uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
+                          const float *additive, float *out, uint64_t out_stride, bool output_bf16,
+                          int *status, hipStream_t stream);
 
 inline hipStream_t as_stream(yvex_hip_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
