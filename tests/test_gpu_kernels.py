@@ -177,6 +177,42 @@ def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, wid
         assert_close(few, got[:count], rel=1e-5, abs_=1e-5)
 
 
+def test_matvec_q4k_large_batch_stages_operands_in_lds(gpu, oracle):
+    """A Q4_K projection with at least one (128 rows x 64 tokens) tile per compute unit takes the
+    kernel whose operands are staged through LDS: ragged row count (the last tile repeats a row),
+    a last token tile of six rows (one 32-token block), additive rows and bf16 outputs; held to
+    the integer path's bar like the other tile shapes, and equal to the smaller batches' values."""
+    from yvex_amd import kernels as K
+    qt, rows, width, inputs = oracle.Q4_K, 2001, 768, 1030
+    assert (rows + 127) // 128 * ((inputs + 63) // 64) >= 256
+    g = oracle.Generator(42, "matvec.rows.staged.q4k")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    bias = g.normal(inputs * rows).reshape(inputs, rows)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    want = oracle.q8_matvec(qt, w, rows, width, act_host, inputs)
+    assert_close(got, want, rel=1e-5, abs_=1e-5)
+    summed = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                      additive=dev(bias, gpu), status=status).cpu().numpy()
+    status_ok(status)
+    assert np.array_equal(summed, got + bias)
+    rounded = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                       output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((rounded.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(rounded - got) <= np.abs(got) * 2.0 ** -8 + 1e-30)
+    for count in (70, 16):          # the unstaged 32 x 32 tiles, the 16 x 16 tiles
+        few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=count,
+                       status=status).cpu().numpy()
+        status_ok(status)
+        assert_close(few, got[:count], rel=1e-5, abs_=1e-5)
+
+
 @pytest.mark.parametrize("qtype,rows,width", [("Q8_0", 9600, 7168), ("IQ2_XXS", 37000, 7168)])
 def test_matvec_output_head_variant(gpu, oracle, qtype, rows, width):
     """One Q8_K activation row against a matrix of 64 MB or more takes the variant with four
