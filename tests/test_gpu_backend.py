@@ -717,6 +717,28 @@ def test_execute_rows_deferred_completion(backend, oracle):
     assert (err_abs > 1e-5 + 1e-3 * np.abs(want)).mean() < 2e-2
 
 
+def test_deferred_batches_keep_what_an_earlier_one_raised(backend, oracle):
+    """Two batches behind one barrier (src/runtime/moe.c:1567-1576 completes a phase's layers with
+    one call): the first is fed a non-finite row and raises the kernels' status, the second is
+    clean; the barrier still reports the failure, and the phase after it starts clean."""
+    case = MoeCase(backend, oracle, rows=3)
+    backend.workspace(case.workspace_bytes)
+    completion = abi.DeviceCompletion(1, None)
+    case.job.device_completion = C.pointer(completion)
+    clean = case.rows_in
+    bad = case.x.copy()
+    bad[1, 7] = np.inf
+    case.batch.device_rows = backend.f32(bad)
+    assert case.execute() == 0, case.err.message
+    case.batch.device_rows = clean
+    assert case.execute() == 0, case.err.message
+    done, err = abi.RowBatchResult(), abi.Error()
+    assert case.ops.complete_rows(backend.handle, 0, C.byref(done), C.byref(err)) == abi.FORMAT
+    assert case.execute() == 0, case.err.message
+    assert case.ops.complete_rows(backend.handle, 0, C.byref(done), C.byref(err)) == 0, err.message
+    assert done.completed == 1
+
+
 @pytest.mark.parametrize("imaged,rows,experts", [
     (("routed", "shared"), 5, 8), (("routed",), 7, 8), (("shared",), 6, 8), (("routed", "shared"), 40, 4)])
 def test_execute_rows_runs_the_sweep_image(backend, oracle, imaged, rows, experts):

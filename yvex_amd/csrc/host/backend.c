@@ -61,6 +61,9 @@ int yvex_rocm_require_kernels(const yvex_rocm_backend *backend, const char *wher
 
 int yvex_rocm_status_reset(yvex_rocm_backend *backend, const char *where, yvex_error *err)
 {
+    /* row batches whose completion is deferred own the word until their barrier: an operation
+     * that runs between them must not erase what they raised (it then reports it as its own) */
+    if (backend->pending_completion) return YVEX_OK;
     return yvex_rocm_launch_result(yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream),
                                    where, err);
 }

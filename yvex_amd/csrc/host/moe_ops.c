@@ -485,7 +485,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     unsigned long long base, pairs, hidden, experts, topk, row_count, launches = 0ull;
     unsigned long long router_address = 0ull, bias_address = 0ull, addresses[6] = {0};
     unsigned long long envelope_addresses[4] = {0}, streams = 0ull, expanded;
-    unsigned long long d2h = 0ull, started, counts[4] = {0};
+    unsigned long long d2h = 0ull, started, counts[4] = {0}, status_launches = 0ull;
     const void *activations;
     void *combined_target;
     unsigned long long table_address = 0ull;
@@ -673,6 +673,14 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     if (hash_router && yvex_hip_memcpy_h2d(AT(tokens), rows->token_ids, row_count * sizeof(unsigned int),
                                            stream) != 0)
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.token-ids", yvex_hip_last_error());
+    /* The kernels' status word is cleared where a phase starts, not per batch: a batch whose
+     * completion is deferred leaves what it raised for the barrier to find, whatever runs behind
+     * it (the word only ever changes from zero). Like the token ids, outside any graph. */
+    if (!backend->pending_completion) {
+        rc = yvex_rocm_status_reset(backend, "rocm.moe.rows.status", err);
+        if (rc != YVEX_OK) return rc;
+        status_launches = 1ull;
+    }
     if (!job->eager_execution && !(backend->moe_graphs && backend->moe_graphs->refused)) {
         graph_key key;
         unsigned long long slot_address[YVEX_MOE_WEIGHT_COUNT] = {0};
@@ -720,7 +728,6 @@ sequence:
             if (rc == YVEX_OK) launches++;                              \
         }                                                               \
     } while (0)
-    LAUNCH(yvex_hip_fill_u32(status, 0u, 1u, stream), "rocm.moe.rows.status");
     if (has_shared && !merged)
         LAUNCH(yvex_hip_fill_u32(AT(shared_outputs), 0u, row_count * hidden, stream), "rocm.moe.rows.zero");
     activations = rows->device_rows->data;
@@ -926,7 +933,7 @@ sequence:
     result->execution_class = YVEX_EXECUTION_CLASS_DEVICE_NATIVE;
     result->row_count = row_count;
     result->row_expert_pairs = pairs;
-    result->kernel_launches = launches;
+    result->kernel_launches = launches + status_launches;
     result->shared_expert_operations = has_shared ? row_count : 0ull;
     result->grouped_expert_operations = pairs;
     result->active_weight_base_bytes = views[YVEX_MOE_WEIGHT_ROUTER].encoded_bytes +
@@ -1035,6 +1042,7 @@ static int moe_complete_rows(yvex_rocm_backend *backend, int barrier_observed,
     if (!backend->host_only) {
         started = monotonic_ns();
         rc = yvex_rocm_finish(backend, "rocm.moe.rows.phase-sync", &device_status, err);
+        if (rc == YVEX_OK) backend->pending_completion = 0;   /* the barrier was reached: the next phase starts clean */
         if (rc == YVEX_OK && device_status)
             rc = yvex_rocm_refuse(err, device_status == 1 ? YVEX_ERR_FORMAT : YVEX_ERR_BACKEND,
                                   "rocm.moe.complete", "deferred width-N MoE reported a device failure");

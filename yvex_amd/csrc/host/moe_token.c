@@ -483,7 +483,9 @@ int yvex_rocm_backend_moe_begin(yvex_rocm_moe_execution **out, yvex_rocm_backend
         }
     }
     expanded_bytes = layer->expanded_width * sizeof(float);
-    rc = launched(x, yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream), "rocm.moe.status", err);
+    rc = backend->pending_completion   /* deferred row batches own the word until their barrier */
+        ? YVEX_OK
+        : launched(x, yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream), "rocm.moe.status", err);
     if (rc == YVEX_OK)       /* slots never added read as zero in the rank-ordered sum */
         rc = launched(x, yvex_hip_fill_u32(AT(pair_outputs), 0u,
                                            (x->routed - x->pair_outputs) / sizeof(float), backend->stream),

@@ -49,8 +49,9 @@ void yvex_rocm_workspace_reset(yvex_rocm_backend *backend);
 int yvex_rocm_require_kernels(const yvex_rocm_backend *backend, const char *where, yvex_error *err);
 /* Map a launch-level return code (negative yvex_status) to an error. */
 int yvex_rocm_launch_result(int rc, const char *where, yvex_error *err);
-/* Stream synchronise + read the device status word (and clear it for the next operation). */
+/* Stream synchronise + read the device status word. */
 int yvex_rocm_finish(yvex_rocm_backend *backend, const char *where, int *device_status, yvex_error *err);
+/* Clear the status word on the stream, unless deferred row batches are waiting for their barrier. */
 int yvex_rocm_status_reset(yvex_rocm_backend *backend, const char *where, yvex_error *err);
 /* Resolve a weight view: device_address if given, else the resident arena mapping. */
 int yvex_rocm_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
