@@ -60,11 +60,11 @@ def one_step_or_inside(got, want):
     return bool(np.all((err <= BF16_STEP * 1.001 * np.abs(want)) | (err <= 1e-5 + 1e-3 * np.abs(want))))
 
 
-def stage_flip_rates(oracle, layer, routed, x, picked, label):
+def stage_flip_rates(oracle, layer, routed, x, picked, label, qt=None):
     """The picked rows' pairs stage by stage: SwiGLU products against the oracle's, expert outputs
     against the oracle fed with the device's own products. Differences are single bf16 steps;
     returns their fractions."""
-    qt = oracle.IQ2_XXS
+    qt = oracle.IQ2_XXS if qt is None else qt
     gate, up, down = (t.cpu().numpy() for t in routed)
     gb = oracle.row_bytes(qt, HIDDEN) * INTERMEDIATE
     db = oracle.row_bytes(qt, INTERMEDIATE) * HIDDEN
@@ -161,14 +161,31 @@ def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
     assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
 
 
-def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
+def synthetic_q4k(blocks, device, seed):
+    """Uniform scale, minimum and nibble bytes with small positive fp16 d and dmin."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 144), dtype=torch.uint8, device=device, generator=gen)
+    d = (torch.rand(blocks, device=device, generator=gen) * 1.0e-4 + 2.0e-5).to(torch.float16)
+    raw[:, 0:2] = d.view(torch.uint8).reshape(blocks, 2)
+    raw[:, 2:4] = raw[:, 0:2]
+    return raw.reshape(-1)
+
+
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q4_K"])
+def test_prefill_layer_at_full_size(gpu, oracle, layer_weights, qtype):
     """2048 rows whose experts follow a Zipf(1.1) popularity (buckets from a handful of pairs to
-    more than a thousand) through the matrix-core kernels: the same bits twice, the first 32 rows
-    against the decode sweeps' result for them (another summation order: within tolerance), four
-    rows against the oracle."""
+    more than a thousand) through the matrix-core kernels, with IQ2_XXS and with Q4_K experts: the
+    same bits twice, the first 32 rows against the decode sweeps' result for them (another
+    summation order: within tolerance), four rows against the oracle."""
     from yvex_amd import kernels as K
     from yvex_amd.moe import MoeLayer
-    routed, shared = layer_weights
+    if qtype == "IQ2_XXS":
+        routed, shared = layer_weights
+    else:
+        blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
+        routed = tuple(synthetic_q4k(blocks, gpu, 21 + i) for i in range(3))
+        shared = tuple(synthetic_q4k(INTERMEDIATE * HIDDEN // 256, gpu, 31 + i) for i in range(3))
     rows = 2048
     gen = torch.Generator(device=gpu)
     gen.manual_seed(7)
@@ -176,7 +193,7 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
     rank = torch.randperm(EXPERTS, device=gpu, generator=gen).float() + 1.0
     uniform = torch.rand((rows, EXPERTS), device=gpu, generator=gen).clamp_(1e-9, 1.0 - 1e-9)
     logits = rank.pow(-1.1).log()[None, :] - (-uniform.log()).log()      # Gumbel top-k over log-popularity
-    qt = K.IQ2_XXS
+    qt = getattr(K, qtype)
     common = dict(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtypes=(qt, qt, qt),
                   routed=routed, shared=shared, scoring=K.SIGMOID, normalize=True, scaling=1.0, limit=10.0,
                   act_q8=True, device=gpu)
@@ -190,7 +207,8 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
     assert torch.isfinite(first).all()
     selected = wide.selected.clone()
     picked = [5, 700, 1000, 1900]
-    mid_rate, out_rate = stage_flip_rates(oracle, wide, routed, x, picked, "prefill layer, 4 rows stage by stage")
+    mid_rate, out_rate = stage_flip_rates(oracle, wide, routed, x, picked,
+                                          f"prefill layer ({qtype}), 4 rows stage by stage", getattr(oracle, qtype))
     assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
     keep = list(range(32)) + picked
     populations = torch.bincount(selected.reshape(-1).long(), minlength=EXPERTS).cpu().numpy()
@@ -229,10 +247,10 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights):
                  np.abs(wide_shared[:32]).max(axis=1)[:, None])
     combined_close(first[:32].cpu().numpy(), sweeps.cpu().numpy(), wide_pairs[:32], wide_shared[:32])
     want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
-                            qtypes=(oracle.IQ2_XXS,) * 3, routed=[t.cpu().numpy() for t in routed],
+                            qtypes=(getattr(oracle, qtype),) * 3, routed=[t.cpu().numpy() for t in routed],
                             shared=[t.cpu().numpy() for t in shared], inputs=x[picked].cpu().numpy(),
                             logits=logits[picked].cpu().numpy(), scoring=oracle.SIGMOID, normalize=True,
                             scaling=1.0, limit=10.0, act_q8=True, threads=16)
     assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
     combined_close(first[picked].cpu().numpy(), want["combined"], wide_pairs[32:], wide_shared[32:],
-                   PREFILL_FLIP_BOUND, "prefill layer, 4 rows against the oracle")
+                   PREFILL_FLIP_BOUND, f"prefill layer ({qtype}), 4 rows against the oracle")
