@@ -473,6 +473,19 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     abi_layer.close()
     harness_ms = step_ms
     step_ms = min(abi_graph_ms, abi_eager_ms)
+    # IQ2_XXS experts resident as the sweep image only: the matrix-core kernels read it as well
+    image = None
+    if qt == 16:
+        image_layer = AbiLayer(torch, weights, shared, router, x.cpu().numpy(), rows, qtype=qt, sweep_image=True)
+        image_layer.step(defer=False)
+        image_same = bool((torch.from_numpy(image_layer.output()) == stage_rows.cpu()).all().item())
+        image_ms = image_layer.timed(steps, max(warmup, 2))
+        image_layer.close()
+        del image_layer
+        torch.cuda.empty_cache()
+        image = {"graph_ms_per_step": round(image_ms, 4), "rows_identical_to_canonical": image_same}
+        if not image_same:
+            return {"error": "the sweep image and the canonical rows disagree on the matrix-core kernels"}
     pair_ops = 2 * (2 * INTERMEDIATE * HIDDEN + HIDDEN * INTERMEDIATE)
     routed_ops, shared_ops = pair_ops * pairs, pair_ops * rows
     up_ops = 2 * 2 * INTERMEDIATE * HIDDEN * pairs
@@ -485,6 +498,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
                   "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
                   "rows_identical_to_stage_harness": abi_same,
                   "distinct_routed_experts": abi_unique},
+        "c_abi_sweep_image": image,
         "stage_harness_ms_per_step": round(harness_ms, 4),
         "int8_TOPs": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12, 2),
         "mfma_peak_frac": round((routed_ops + shared_ops) / (step_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 4),

@@ -712,8 +712,8 @@ typedef struct {
  * 4-bit group scales << 16; then per group of 32 weights its four codebook indices and its four
  * 7-bit sign fields, one to a byte}. The reference's row-batch path refuses every
  * DERIVED_BACKEND view (moe.c:939-958); execute_rows here runs that one image (IQ2_XXS,
- * device-encoded activations, the sweep family on gate, up and down) on the decode sweeps and
- * answers UNSUPPORTED for any other derived view. */
+ * device-encoded activations, the sweep family on gate, up and down) on the decode sweeps and on
+ * the matrix-core kernels, and answers UNSUPPORTED for any other derived view. */
 typedef struct {
     int (*derived_layout_plan)(const yvex_physical_execution_decision *decision,
                                unsigned long long *storage_bytes, yvex_error *err);
@@ -760,8 +760,9 @@ int yvex_rocm_moe_derived_layout_build(const yvex_physical_execution_decision *d
  * result carries layout DERIVED_BACKEND, the family YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP,
  * activation DEVICE_ENCODED, the canonical row geometry and encoded_bytes, storage_bytes, and the
  * image's device_address (or `encoded` inside the attached arena). execute_rows runs such experts
- * on the decode sweeps at any batch width; every other operation takes canonical rows
- * (UNSUPPORTED). */
+ * on the decode sweeps and, for wide batches, on the matrix-core kernels, both of which read the
+ * image: it can be the only resident form of the experts. Every other operation takes canonical
+ * rows (UNSUPPORTED). */
 int yvex_rocm_moe_sweep_image_build_resident(yvex_rocm_backend *backend,
                                              const yvex_physical_execution_decision *decision,
                                              unsigned long long canonical_address,

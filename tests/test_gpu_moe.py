@@ -174,22 +174,27 @@ def test_sweep_image_is_the_documented_repacking(gpu, oracle):
         assert np.array_equal(image[:, half, 0], d | (scales << 16))
 
 
-@pytest.mark.parametrize("hidden,intermediate,experts,topk,rows", [
-    (7168, 2048, 12, 4, 6), (2048, 2048, 6, 4, 20), (4096, 3072, 4, 2, 5), (2048, 2048, 200, 8, 40)])
-def test_sweeps_give_the_same_bits_from_the_image(gpu, oracle, hidden, intermediate, experts, topk, rows):
-    """The decode sweeps over the sweep image of the experts (one, two, three, four pairs a sweep,
-    shared expert merged into the launches) publish bit for bit what they publish from canonical
+@pytest.mark.parametrize("hidden,intermediate,experts,topk,rows,matrix_cores", [
+    (7168, 2048, 12, 4, 6, False), (2048, 2048, 6, 4, 20, False), (4096, 3072, 4, 2, 5, False),
+    (2048, 2048, 200, 8, 40, False), (2048, 2048, 6, 4, 150, True), (7168, 768, 3, 2, 70, True),
+    (512, 2048, 5, 3, 33, True)])
+def test_kernels_give_the_same_bits_from_the_image(gpu, oracle, hidden, intermediate, experts, topk, rows,
+                                                   matrix_cores):
+    """The decode sweeps (one, two, three, four pairs a sweep, shared expert merged into the
+    launches) and the matrix-core row-batch kernels (token tiles of both sizes, ragged row tiles)
+    over the sweep image of the experts publish bit for bit what they publish from canonical
     bytes: same integer sums, same scaling, same order."""
     layers = []
     for image in (False, True):
         layer, h = make_layer(oracle, gpu, hidden=hidden, intermediate=intermediate, experts=experts,
                               topk=topk, rows=rows, qtype="IQ2_XXS", act_q8=True, scoring=1,
-                              sweep_image=image)
+                              sweep_image=image, matrix_cores=matrix_cores)
         combined = layer.run(dev(h["x"], gpu), dev(h["logits"], gpu)).clone()
         torch.cuda.synchronize()
         assert int(layer.status.item()) == 0
         pairs = rows * topk
-        layers.append((combined.cpu().numpy(), layer.intermediate_f32[:pairs + rows].cpu().numpy().copy(),
+        mids = pairs if matrix_cores else pairs + rows      # the sweeps lay the shared expert's products behind the routed ones
+        layers.append((combined.cpu().numpy(), layer.intermediate_f32[:mids].cpu().numpy().copy(),
                        layer.pair_outputs[:pairs].cpu().numpy().copy(), layer.shared_out[:rows].cpu().numpy().copy()))
     for a, b in zip(*layers):
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32))

@@ -85,6 +85,7 @@ struct MfmaArgs {
     double limit;
     int *status;
     int plain_output;        // plain projection: outputs stay fp32 instead of being rounded to bf16
+    int image;               // weights are the sweep image (72-byte records) instead of canonical bytes
 };
 
 // Limb pair of one magnitude: low limb in bits 0-7, high limb in bits 8-15.
@@ -167,7 +168,7 @@ struct MfmaItem {
 //     touches: with eight waves that was the longest pole of the step.
 // The loop body is one superblock in one basic block (requests past the end are clamped, and
 // superblocks past the end run with a zero row scale), so nothing leaves registers.
-template <bool FUSED_UP, unsigned NTB>
+template <bool FUSED_UP, unsigned NTB, bool IMAGE>
 __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
 {
     const GroupedProblem &pr = a.pr;
@@ -208,14 +209,17 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         const unsigned piece = 64u * k + lane;
         const unsigned served = piece < 160u ? piece : 159u;
         const unsigned char *from = row_pointer(served / 5u);
-        window_from[k] = from + (served % 5u < 4u ? 16u * (served % 5u) : 52u);
+        // (the image's 72-byte records start on dword boundaries: the fifth piece is their last 16 bytes)
+        window_from[k] = from + (served % 5u < 4u ? 16u * (served % 5u) : IMAGE ? 56u : 52u);
     }
     const unsigned window_base = kWindowBase + wave * 2u * kWindowBytes;
     auto weight_piece = [&](unsigned sb, unsigned k) {
         const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane(
             (int)(window_base + (sb & 1u) * kWindowBytes + k * 1024u));
         sb = sb < last ? sb : last;
-        const unsigned char *from = (const unsigned char *)((unsigned long long)(window_from[k] + sb * 66u) & ~3ull);
+        const unsigned char *from = IMAGE
+            ? window_from[k] + sb * 72u
+            : (const unsigned char *)((unsigned long long)(window_from[k] + sb * 66u) & ~3ull);
         if (k < 2u) copy_to_lds_16(from, to);
         else copy_to_lds_16_first32(from, to);
     };
@@ -272,6 +276,7 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
     const unsigned row_scale_at = kRowScaleBase + wave * 256u;      // + 128 for odd superblocks
     const unsigned window_row = window_base + r * 80u;
     unsigned grids[4], aux[4];           // group records of the superblock being decoded
+    unsigned head = 0u;                  // image: fp16 scale | the four group scales of this half << 16
     uint2 codes[2][2], signs[2][2];      // [chunk & 1]: table words of the chunk's two subgroups
     uint4 limbs[2];                      // [group & 1]: limb words of a group
     v4i a_lo[2], a_hi[2];                // [chunk & 1]: A operands of a K chunk
@@ -282,6 +287,21 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
     // bytes at o + 2 + 32 h: in window dwords 8 h + o / 2 onwards, shifted by 2 bytes when o is
     // 0. Window dword 16 is the last dword of the fifth piece.
     auto settle = [&](unsigned sb) {
+        if constexpr (IMAGE) {
+            // The lane's record is nine dwords from byte 36 h of the row's 72; window bytes 64-79
+            // hold record bytes 56-71 (the fifth piece), so bytes from 64 on sit 8 further.
+            const unsigned at = window_row + (sb & 1u) * kWindowBytes;
+            auto place = [&](unsigned byte) { return at + byte + (byte >= 64u ? 8u : 0u); };
+            head = lds_read_u32(place(36u * h));
+#pragma unroll
+            for (unsigned g = 0; g < 4u; ++g) {
+                grids[g] = lds_read_u32(place(36u * h + 4u + 8u * g));
+                aux[g] = lds_read_u32(place(36u * h + 8u + 8u * g));
+            }
+            const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(head & 0xffffu) : 0.0f;
+            lds_write_u32(row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
+            return;
+        }
         const unsigned clamped = sb < last ? sb : last;
         const unsigned o = (row_misalign + 2u * clamped) & 3u;
         const unsigned at = window_row + (sb & 1u) * kWindowBytes;
@@ -311,10 +331,15 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         for (unsigned i = 0; i < 2u; ++i) {
             const unsigned j = 2u * (c & 1u) + i;
             codes[c & 1u][i] = lds_read_uint2(__builtin_amdgcn_perm(grids[g], code_lane, 0x0c0c0400u + (j << 8)));
-            const unsigned field = j == 0u ? aux[g] << 8 : j == 1u ? aux[g] << 1 : aux[g] >> (7u * j - 8u);
-            signs[c & 1u][i] = lds_read_uint2((field & 0x7f00u) | sel_lane);
+            if constexpr (IMAGE) {      // the field has a byte of its own
+                signs[c & 1u][i] = lds_read_uint2(__builtin_amdgcn_perm(aux[g], sel_lane, 0x0c0c0400u + (j << 8)));
+            } else {
+                const unsigned field = j == 0u ? aux[g] << 8 : j == 1u ? aux[g] << 1 : aux[g] >> (7u * j - 8u);
+                signs[c & 1u][i] = lds_read_uint2((field & 0x7f00u) | sel_lane);
+            }
         }
-        if ((c & 1u) == 0u) limbs[g & 1u] = lds_read_uint4(((aux[g] >> 20) & 0xf00u) | lut_lane);
+        if ((c & 1u) == 0u)
+            limbs[g & 1u] = lds_read_uint4((IMAGE ? (head >> (8u + 4u * g)) & 0xf00u : (aux[g] >> 20) & 0xf00u) | lut_lane);
     };
     // selector words and permutes of K chunk c
     auto build = [&](unsigned c) {
@@ -565,7 +590,7 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
     }
 }
 
-template <bool FUSED_UP>
+template <bool FUSED_UP, bool IMAGE>
 __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
 {
     extern __shared__ __align__(16) unsigned char mfma_lds[];
@@ -665,17 +690,24 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
         it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
         it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-        if (it.tokens <= 32u) rows_item<FUSED_UP, 1u>(a, it);
-        else rows_item<FUSED_UP, 2u>(a, it);
+        if (it.tokens <= 32u) rows_item<FUSED_UP, 1u, IMAGE>(a, it);
+        else rows_item<FUSED_UP, 2u, IMAGE>(a, it);
     }
+}
+
+template <bool FUSED_UP, bool IMAGE>
+static int launch_mfma_variant(const MfmaArgs &a, hipStream_t stream)
+{
+    YVEX_ALLOW_DYNAMIC_LDS((mfma_iq2_kernel<FUSED_UP, IMAGE>), kMfmaLdsBytes);
+    mfma_iq2_kernel<FUSED_UP, IMAGE><<<compute_units(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
+    return check_launch("moe_rows_mfma");
 }
 
 template <bool FUSED_UP>
 static int launch_mfma(const MfmaArgs &a, hipStream_t stream)
 {
-    YVEX_ALLOW_DYNAMIC_LDS(mfma_iq2_kernel<FUSED_UP>, kMfmaLdsBytes);
-    mfma_iq2_kernel<FUSED_UP><<<compute_units(), kRowThreads, kMfmaLdsBytes, stream>>>(a);
-    return check_launch("moe_rows_mfma");
+    return a.image ? launch_mfma_variant<FUSED_UP, true>(a, stream)
+                   : launch_mfma_variant<FUSED_UP, false>(a, stream);
 }
 
 // A plain projection through the row-batch kernel: every input row in one bucket of expert 0.
@@ -721,9 +753,12 @@ extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void
         return ST_INVALID_ARG;
     if (w->gate_qtype != w->up_qtype || (w->gate_qtype != QT_IQ2_XXS && w->gate_qtype != QT_Q4_K))
         return ST_UNSUPPORTED;
-    int rc = check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
+    int rc = w->gate_up_image
+        ? check_image_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes, w->gate, w->gate_expert_bytes)
+        : check_matrix(w->gate_qtype, w->hidden, w->gate_row_bytes);
     if (rc) return rc;
     if (w->up_row_bytes != w->gate_row_bytes) return ST_BOUNDS;
+    if (w->gate_up_image && (((uintptr_t)w->up & 3u) || (w->up_expert_bytes & 3u))) return ST_INVALID_ARG;
     if (pairs > 0xffffffffull || w->intermediate > 0xffffffffull || w->intermediate % 4u) return ST_BOUNDS;
     MfmaArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
@@ -734,6 +769,7 @@ extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void
     a.out_rows = (unsigned)w->intermediate;
     a.limit = limit;
     a.status = status;
+    a.image = w->gate_up_image != 0;
     return launch_mfma<true>(a, as_stream(stream));
 }
 
@@ -748,7 +784,9 @@ extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const vo
         (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
         return ST_INVALID_ARG;
     if (w->down_qtype != QT_IQ2_XXS && w->down_qtype != QT_Q4_K) return ST_UNSUPPORTED;
-    int rc = check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
+    int rc = w->down_image
+        ? check_image_matrix(w->down_qtype, w->intermediate, w->down_row_bytes, w->down, w->down_expert_bytes)
+        : check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
     if (rc) return rc;
     if (pairs > 0xffffffffull || w->hidden > 0xffffffffull || w->hidden % 4u) return ST_BOUNDS;
     MfmaArgs a{};
@@ -760,5 +798,6 @@ extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const vo
     a.out_rows = (unsigned)w->hidden;
     a.limit = 1.0;
     a.status = status;
+    a.image = w->down_image != 0;
     return launch_mfma<false>(a, as_stream(stream));
 }

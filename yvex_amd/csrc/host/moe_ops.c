@@ -657,10 +657,10 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     /* Row batches whose buckets average eight pairs or more go to the int8 matrix-core kernels
      * (IQ2_XXS or Q4_K weights, Q8_K activations); below that the decode sweeps, which read an expert's
      * bytes once per four pairs, are faster. The reference switches its tensor-core kernels on
-     * from 16 input rows (src/backend/cuda/private.h:461-464). Only the sweeps read their image:
-     * experts held as one stay on the sweeps at any width. */
-    row_batch = routed_q8 && !routed_image && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
-    shared_row_batch = row_batch && has_shared && shared_q8 && !shared_image && matrix_core_qtypes(&shared);
+     * from 16 input rows (src/backend/cuda/private.h:461-464). Both kernel families read the
+     * sweep image of IQ2_XXS experts as well as canonical bytes. */
+    row_batch = routed_q8 && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
+    shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",
