@@ -603,25 +603,53 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
     const bool fixed = pr.expert_ids == nullptr;
     const unsigned buckets = fixed ? 1u : (unsigned)pr.counts[0];
 
+    // The buckets' populations are requested before the tables are built (one round trip to
+    // memory under the fill instead of one per bucket after it).
+    unsigned long long population_here = 0ull;
+    if (tid < 256u && tid < buckets) population_here = fixed ? pr.pairs : pr.bucket_populations[tid];
     mfma_tables_fill();
-    if (tid == 0u) {
-        // Full 64-pair tiles come first in the item list, then the partial last tiles by size,
-        // largest first: every workgroup, walking the list with the grid's stride, gets the same
-        // share of each kind of item, and the short items come last.
-        unsigned cursor = 0u, members[2] = {0u, 0u};
-        for (unsigned b = 0; b < buckets && b < 256u; ++b) {
-            lds_write_u32(kTileStartBase + 4u * b, cursor);
-            const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[b];
-            cursor += (unsigned)(n / kTileTokens);
-            const unsigned rest = (unsigned)(n % kTileTokens);
-            if (rest) {
-                const unsigned c = rest > 32u ? 0u : 1u;
-                lds_write_u16(kClassListBase + (c * 256u + members[c]) * 2u, b);
-                ++members[c];
-            }
+    // Full 64-pair tiles come first in the item list, then the partial last tiles by size,
+    // largest first: every workgroup, walking the list with the grid's stride, gets the same
+    // share of each kind of item, and the short items come last. Bucket b's first full tile is
+    // the number of full tiles before it (a scan over the 256 bucket slots); its place in its
+    // class of partial tiles (more than 32 pairs, or fewer) is its rank among the buckets of
+    // that class, in bucket order, from ballots and per-wave totals.
+    {
+        const unsigned lane = tid & 63u, wave = tid >> 6;
+        const unsigned full = tid < 256u ? (unsigned)(population_here / kTileTokens) : 0u;
+        const unsigned rest = tid < 256u ? (unsigned)(population_here % kTileTokens) : 0u;
+        const unsigned cls = rest == 0u ? 2u : rest > 32u ? 0u : 1u;
+        unsigned inclusive = full;
+#pragma unroll
+        for (int offset = 1; offset < 64; offset <<= 1) {
+            const unsigned below = (unsigned)__shfl_up((int)inclusive, offset, kWave);
+            if ((int)lane >= offset) inclusive += below;
         }
-        lds_write_u32(kTileStartBase + 4u * (buckets < 256u ? buckets : 256u), cursor);
-        for (unsigned c = 0; c < 2u; ++c) lds_write_u32(kClassCountBase + 4u * c, members[c]);
+        unsigned rank[2];
+#pragma unroll
+        for (unsigned c = 0; c < 2u; ++c) {
+            const unsigned long long members = __ballot(cls == c);
+            rank[c] = (unsigned)__popcll(members & ((1ull << lane) - 1ull));
+            if (lane == 0u && wave < 4u) lds_write_u32(kTrashBase + 16u + (c * 4u + wave) * 4u, (unsigned)__popcll(members));
+        }
+        if (lane == 63u && wave < 4u) lds_write_u32(kTrashBase + wave * 4u, inclusive);
+        __syncthreads();
+        if (tid < 256u) {
+            unsigned before = 0u, class_before[2] = {0u, 0u};
+            for (unsigned w = 0; w < wave; ++w) {
+                before += lds_read_u32(kTrashBase + w * 4u);
+                class_before[0] += lds_read_u32(kTrashBase + 16u + w * 4u);
+                class_before[1] += lds_read_u32(kTrashBase + 16u + (4u + w) * 4u);
+            }
+            lds_write_u32(kTileStartBase + 4u * tid, before + inclusive - full);
+            if (tid == 255u) lds_write_u32(kTileStartBase + 4u * 256u, before + inclusive);
+            if (cls < 2u) lds_write_u16(kClassListBase + (cls * 256u + class_before[cls] + rank[cls]) * 2u, tid);
+        }
+        if (tid < 2u) {
+            unsigned total = 0u;
+            for (unsigned w = 0; w < 4u; ++w) total += lds_read_u32(kTrashBase + 16u + (tid * 4u + w) * 4u);
+            lds_write_u32(kClassCountBase + 4u * tid, total);
+        }
     }
     __syncthreads();
     if (buckets == 0u || buckets > 256u) {
