@@ -46,11 +46,8 @@ constexpr unsigned kSweepShortDiv = 2u;        // the rest goes out in items of 
 // LDS map (byte addresses; the dynamic block starts at LDS address 0)
 constexpr unsigned kMagBase = 0u;              // 256 entries x 16 replicas x {+lo, +hi, -lo, -hi}
 constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {selector lo, hi}
-constexpr unsigned kPrefixBase = kSelBase + 128u * 32u * 8u;   // 257 sweep starts, u32
-constexpr unsigned kTicketAddress = kPrefixBase + 1056u;   // work-item counter of the workgroup
-constexpr unsigned kParkBase = kPrefixBase + 1088u;
-constexpr unsigned kPopulationBase = kParkBase + 2048u;   // bucket populations while the item list
-                                                          // is built (the parking areas are free then)
+constexpr unsigned kTicketAddress = kSelBase + 128u * 32u * 8u;   // work-item counter of the workgroup
+constexpr unsigned kParkBase = kTicketAddress + 32u;
 constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave: 32 bytes per
                                                                       // (iteration, packed value), then one spare word per lane
 // Sweeps listed by the number of pairs they serve (4, 3, 2, 1): four class sizes, four class
@@ -526,45 +523,17 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
                                            __float_as_uint(weight_here[k])));
     }
 
-    // ---- sweep numbering of the routed buckets: exclusive prefix of ceil(population / 4) ----
     if (!routed_fixed && buckets > 256u) {
         if (tid == 0u) raise_status(a.status, 2);
         return;
     }
-    if (!routed_fixed) {
-        // Hillis-Steele scan over 256 slots, two buffers
-        const unsigned scratch = kParkBase;   // the parking areas are free until the first item
-        unsigned mine = 0u;
-        if (tid < 256u) {
-            if (tid >= buckets) population_here = 0u;
-            mine = (population_here + (unsigned)kSweepPairs - 1u) / (unsigned)kSweepPairs;
-            lds_store_u32(scratch + 4u * tid, mine);
-            lds_store_u32(kPopulationBase + 4u * tid, population_here);
-            if (tid < buckets) {
-                // (values past 32 bits fail the item's range check through their low words' sum
-                // only by accident, so they are clamped to a value that always fails it)
-                lds_store_u32(kBucketBase + 12u * tid, expert_here < 0xffffffffull ? (unsigned)expert_here : 0xffffffffu);
-                lds_store_u32(kBucketBase + 12u * tid + 4u, first_here < 0xffffffffull ? (unsigned)first_here : 0xffffffffu);
-                lds_store_u32(kBucketBase + 12u * tid + 8u, population_here);
-            }
-        }
-        __syncthreads();
-        unsigned from = scratch, to = scratch + 1024u;
-        for (unsigned step = 1u; step < 256u; step <<= 1) {
-            if (tid < 256u) {
-                unsigned v = lds_load_u32(from + 4u * tid);
-                if (tid >= step) v += lds_load_u32(from + 4u * (tid - step));
-                lds_store_u32(to + 4u * tid, v);
-            }
-            __syncthreads();
-            const unsigned t = from;
-            from = to;
-            to = t;
-        }
-        if (tid < 256u) lds_store_u32(kPrefixBase + 4u * (tid + 1u), lds_load_u32(from + 4u * tid));
-        if (tid == 0u) lds_store_u32(kPrefixBase, 0u);
+    if (!routed_fixed && tid < buckets) {
+        // (values past 32 bits fail the item's range check through their low words' sum only by
+        // accident, so they are clamped to a value that always fails it)
+        lds_store_u32(kBucketBase + 12u * tid, expert_here < 0xffffffffull ? (unsigned)expert_here : 0xffffffffu);
+        lds_store_u32(kBucketBase + 12u * tid + 4u, first_here < 0xffffffffull ? (unsigned)first_here : 0xffffffffu);
+        lds_store_u32(kBucketBase + 12u * tid + 8u, population_here);
     }
-    __syncthreads();
 
     const unsigned units = a.width >> 5;
     SweepLane g;
@@ -600,91 +569,74 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     // (neighbouring items are neighbouring tiles of one expert). A sweep's cost grows with its
     // pairs and workgroup b owns items b, b + grid, ...: listed by class every workgroup gets the
     // same share of every kind.
+    // Every workgroup must arrive at the same list, so a sweep's place is computed, not drawn:
+    // a bucket of n pairs has n / 4 sweeps of the first class, which start at the number of such
+    // sweeps in the buckets before it (a scan over the bucket slots), and, when n % 4 pairs are
+    // left, one sweep of class 4 - n % 4, whose place is the bucket's rank among the buckets that
+    // have one of that class (ballots and per-wavefront totals). The shared expert's pairs count
+    // as a bucket in front of the routed ones.
+    // list word: {whole problem is one bucket : 1, shared expert's problem : 1, bucket : 14, sweep of the bucket : 16}
+    static_assert(kSweepPairs == 4, "the sweep list has one class per number of pairs served, four of them");
     unsigned all_sweeps;
     {
         const GroupedProblem &extra = a.problem[a.problems > 1u ? 1u : 0u];
-        const unsigned extra_sweeps = a.problems > 1u
-            ? (unsigned)((extra.pairs + kSweepPairs - 1u) / kSweepPairs) : 0u;
-        const unsigned routed_sweeps = routed_fixed
-            ? (unsigned)((routed.pairs + kSweepPairs - 1u) / kSweepPairs)
-            : lds_load_u32(kPrefixBase + 4u * buckets);
-        all_sweeps = extra_sweeps + routed_sweeps;
+        const unsigned extra_pairs = a.problems > 1u ? extra.pairs : 0u;
+        const unsigned extra_full = extra_pairs / 4u, extra_class = extra_pairs % 4u ? 4u - extra_pairs % 4u : 0u;
+        // this thread's slot: bucket tid of the routed problem (or the whole problem as slot 0)
+        unsigned pairs_here = 0u;
+        if (routed_fixed) pairs_here = tid == 0u ? routed.pairs : 0u;
+        else if (tid < buckets) pairs_here = population_here;
+        const unsigned full = pairs_here / 4u;
+        const unsigned cls = pairs_here % 4u ? 4u - pairs_here % 4u : 0u;     // 0: no partial sweep
+        unsigned inclusive = full;
+#pragma unroll
+        for (int offset = 1; offset < 64; offset <<= 1) {
+            const unsigned below = (unsigned)__shfl_up((int)inclusive, offset, kWave);
+            if ((int)lane >= offset) inclusive += below;
+        }
+        unsigned rank[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (unsigned c = 1; c < 4u; ++c) {
+            const unsigned long long members = __ballot(cls == c);
+            rank[c] = (unsigned)__popcll(members & ((1ull << lane) - 1ull));
+            if (lane == 0u) lds_store_u32(kClassWaveBase + (wave * 4u + c) * 4u, (unsigned)__popcll(members));
+        }
+        if (lane == 63u) lds_store_u32(kClassWaveBase + wave * 16u, inclusive);       // class 0: full sweeps of the wave's slots
+        __syncthreads();
+        unsigned before[4] = {0u, 0u, 0u, 0u}, total[4] = {0u, 0u, 0u, 0u};
+        for (unsigned w = 0; w < kSweepWaves; ++w)
+#pragma unroll
+            for (unsigned c = 0; c < 4u; ++c) {
+                const unsigned n = lds_load_u32(kClassWaveBase + (w * 4u + c) * 4u);
+                if (w < wave) before[c] += n;
+                total[c] += n;
+            }
+        total[0] += extra_full;
+        if (extra_class) total[extra_class] += 1u;
+        all_sweeps = total[0] + total[1] + total[2] + total[3];
         if (all_sweeps > kClassMaxSweeps) {          // the launch wrapper bounds the pairs
             if (tid == 0u) raise_status(a.status, 2);
             return;
         }
-        // {pairs served, list word} of sweep s in bucket order (shared expert first)
-        auto describe = [&](unsigned s, unsigned &word) -> unsigned {
-            unsigned long long left;
-            if (s < extra_sweeps) {
-                left = extra.pairs - (unsigned long long)s * kSweepPairs;
-                word = 0xc0000000u | s;
-            } else {
-                const unsigned r = s - extra_sweeps;
-                unsigned low = 0u;
-                unsigned long long population = routed.pairs;
-                if (!routed_fixed) {
-                    unsigned high = buckets;   // last bucket whose first sweep is <= r
-                    while (low + 1u < high) {
-                        const unsigned middle = (low + high) >> 1;
-                        if (lds_load_u32(kPrefixBase + 4u * middle) <= r) low = middle;
-                        else high = middle;
-                    }
-                    population = lds_load_u32(kPopulationBase + 4u * low);
-                }
-                const unsigned k = r - (routed_fixed ? 0u : lds_load_u32(kPrefixBase + 4u * low));
-                left = population > (unsigned long long)k * kSweepPairs
-                    ? population - (unsigned long long)k * kSweepPairs : 1ull;
-                word = (routed_fixed ? 0x80000000u : 0u) | (low << 16) | (k & 0xffffu);
-            }
-            return left >= (unsigned long long)kSweepPairs ? (unsigned)kSweepPairs : (unsigned)left;
-        };
-        if (tid < 8u) lds_store_u32(kClassCountBase + 4u * tid, 0u);
-        __syncthreads();
-        for (unsigned s = tid; s < all_sweeps; s += kSweepThreads) {
-            unsigned word;
-            const unsigned n = describe(s, word);
-            __hip_atomic_fetch_add(reinterpret_cast<__attribute__((address_space(3))) unsigned *>(
-                                       kClassCountBase + 4u * (4u - n)), 1u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        __syncthreads();
-        if (tid == 0u) {
-            unsigned start = 0u;
-            for (unsigned c = 0; c < 4u; ++c) {
-                lds_store_u32(kClassCountBase + 16u + 4u * c, start);
-                start += lds_load_u32(kClassCountBase + 4u * c);
-            }
-        }
-        __syncthreads();
-        // Every workgroup must arrive at the same list: a sweep's place in its class is the
-        // number of sweeps of that class before it, counted with ballots inside a wavefront and
-        // per-wavefront totals across the workgroup, a turn of kSweepThreads sweeps at a time.
-        for (unsigned turn = 0; turn < all_sweeps; turn += kSweepThreads) {
-            const unsigned s = turn + tid;
-            unsigned word = 0u;
-            const unsigned mine = s < all_sweeps ? 4u - describe(s, word) : 4u;   // class 0..3, 4: none
-            unsigned rank = 0u;
+        unsigned start[4];
+        start[0] = 0u;
 #pragma unroll
-            for (unsigned c = 0; c < 4u; ++c) {
-                const unsigned long long members = __ballot(mine == c);
-                if (mine == c) rank = (unsigned)__popcll(members & ((1ull << lane) - 1ull));
-                if (lane == 0u) lds_store_u32(kClassWaveBase + (wave * 4u + c) * 4u, (unsigned)__popcll(members));
-            }
-            __syncthreads();
-            if (mine < 4u) {
-                unsigned at = lds_load_u32(kClassCountBase + 16u + 4u * mine) + rank;
-                for (unsigned w = 0; w < wave; ++w) at += lds_load_u32(kClassWaveBase + (w * 4u + mine) * 4u);
-                lds_store_u32(kClassListBase + 4u * at, word);
-            }
-            __syncthreads();
-            if (tid < 4u) {
-                unsigned total = lds_load_u32(kClassCountBase + 16u + 4u * tid);
-                for (unsigned w = 0; w < kSweepWaves; ++w) total += lds_load_u32(kClassWaveBase + (w * 4u + tid) * 4u);
-                lds_store_u32(kClassCountBase + 16u + 4u * tid, total);
-            }
-            __syncthreads();
+        for (unsigned c = 1; c < 4u; ++c) start[c] = start[c - 1u] + total[c - 1u];
+        const unsigned tag = routed_fixed ? 0x80000000u : tid << 16;
+        {
+            const unsigned at = extra_full + before[0] + inclusive - full;
+            for (unsigned k = 0; k < full; ++k) lds_store_u32(kClassListBase + 4u * (at + k), tag | (k & 0xffffu));
         }
+        if (cls)
+            lds_store_u32(kClassListBase + 4u * (start[cls] + (extra_class == cls ? 1u : 0u) + before[cls] + rank[cls]),
+                          tag | (full & 0xffffu));
+        // the shared expert's sweeps: in front of their classes
+        for (unsigned k = tid; k < extra_full; k += kSweepThreads)
+            lds_store_u32(kClassListBase + 4u * k, 0xc0000000u | (k & 0xffffu));
+        if (tid == 0u && extra_class)
+            lds_store_u32(kClassListBase + 4u * start[extra_class], 0xc0000000u | (extra_full & 0xffffu));
+        if (tid < 4u) lds_store_u32(kClassCountBase + 4u * tid, total[tid]);
+        __syncthreads();
     }
     const unsigned total_long = all_sweeps * long_tiles;
     const unsigned total_items = total_long + all_sweeps * short_tiles;
