@@ -739,6 +739,12 @@ typedef struct {
     int (*execute_rows)(yvex_rocm_backend *backend, const yvex_moe_layer_job *job,
                         const yvex_moe_row_batch *batch, const yvex_moe_row_batch_output *output,
                         yvex_moe_row_batch_result *result, yvex_error *err);
+    /* The barrier of batches whose jobs asked for deferred completion
+     * (job->device_completion->defer; src/runtime/moe.c:1567-1576 closes a phase's layers with one
+     * call): synchronises the backend's stream and reports what any of them raised (non-finite
+     * numerics -> FORMAT, a kernel's contract check -> BACKEND). The kernels' status word is
+     * cleared when a phase starts, not between its batches, so a failure of an early batch is
+     * still there at the barrier; an operation run between deferred batches reports it as its own. */
     int (*complete_rows)(yvex_rocm_backend *backend, int barrier_observed,
                          yvex_moe_row_batch_result *result, yvex_error *err);
 } yvex_rocm_moe_operations;
