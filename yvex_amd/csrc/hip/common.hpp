@@ -50,6 +50,14 @@ __device__ __forceinline__ float bf16_round(float value)
     return __uint_as_float(upper << 16);
 }
 
+// The same rounding without branches, for values that are not NaN (to nearest, ties to even; a
+// value that rounds past the largest finite number becomes infinite, as above).
+__device__ __forceinline__ float bf16_round_number(float value)
+{
+    const unsigned bits = __float_as_uint(value);
+    return __uint_as_float((bits + 0x7fffu + ((bits >> 16) & 1u)) & 0xffff0000u);
+}
+
 __device__ __forceinline__ bool finite_f32(float v)
 {
     return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;

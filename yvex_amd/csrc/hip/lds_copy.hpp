@@ -101,6 +101,17 @@ __device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_b
 #endif
 }
 
+// A workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global
+// load and store the compiler knows to be in flight (a kernel's output stores among them: their
+// acknowledgement takes as long as a load), which a barrier between two users of an LDS region
+// has no need of.
+__device__ __forceinline__ void lds_barrier()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#endif
+}
+
 // The same 16-byte copy for lanes 0-31 only (the other lanes neither read nor write).
 __device__ __forceinline__ void copy_to_lds_16_first32(const void *global, unsigned lds_base)
 {

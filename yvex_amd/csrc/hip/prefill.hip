@@ -72,10 +72,7 @@ constexpr unsigned kWindowBytes = 32u * 80u;
 constexpr unsigned kStageBase = kWindowBase + kRowWaves * 2u * kWindowBytes;
 // activation stages: a ring of 4 / NTB stages of NTB x 32 slots (256 bytes each) + 64 scales
 constexpr unsigned kStageRingBytes = 128u * kActPitch + 4u * 256u;
-// half of the finished tile on its way out: 64 tokens x (128 values + 4 of padding) fp32
-constexpr unsigned kOutPitch = 132u * 4u;
-constexpr unsigned kOutBytes = kTileTokens * kOutPitch;
-constexpr unsigned kMfmaLdsBytes = kStageBase + (kStageRingBytes > kOutBytes ? kStageRingBytes : kOutBytes);
+constexpr unsigned kMfmaLdsBytes = kStageBase + kStageRingBytes;
 static_assert(kMfmaLdsBytes <= 160u * 1024u, "one workgroup per compute unit");
 
 struct MfmaArgs {
@@ -142,6 +139,22 @@ struct MfmaItem {
     unsigned tokens, row_tile;
 };
 
+// A work item whose bucket record has been requested from memory but not looked at yet.
+struct MfmaItemRequest {
+    int state;                      // 0: requested, 1: the lists are inconsistent (skip it), 2: past the last item
+    bool partial;                   // the bucket's last, partial token tile
+    unsigned bucket, token_tile, row_tile;
+    unsigned long long first, population, expert;
+};
+
+// The item a workgroup runs after the current one.
+struct MfmaNextItem {
+    MfmaItem it;
+    int state;                      // as above (0: it holds the item)
+    bool ahead;                     // the current item's last rounds of copies fetch its first two windows
+    long long shift;                // from a weight row of the current item to the same row of this one
+};
+
 // One work item with NTB live 32-token blocks (NTB is 1 or 2).
 //
 // Time slot (sb, m) = superblock sb, K chunk m: 2 NTB matrix instructions (low and high limb for
@@ -168,8 +181,16 @@ struct MfmaItem {
 //     touches: with eight waves that was the longest pole of the step.
 // The loop body is one superblock in one basic block (requests past the end are clamped, and
 // superblocks past the end run with a zero row scale), so nothing leaves registers.
-template <bool FUSED_UP, unsigned NTB, bool IMAGE>
-__device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
+//
+// Between two items of a workgroup: the item that follows is looked up while the first copies of
+// this one are in flight (`request_next` before them, `resolve_next` once they have landed), and
+// when it has the same shape the loop's last rounds of window copies, which have no superblock
+// of this item left to fetch, fetch its first two windows instead (`prefetched` tells the
+// item that they are there). Its first activation stage cannot come early: the publishing pass
+// uses the stages' memory.
+template <bool FUSED_UP, unsigned NTB, bool IMAGE, class Request, class Resolve>
+__device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it, bool prefetched,
+                                          Request &&request_next, Resolve &&resolve_next, MfmaNextItem &next)
 {
     const GroupedProblem &pr = a.pr;
     constexpr unsigned R = 4u / NTB;                 // activation stages
@@ -213,13 +234,19 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         window_from[k] = from + (served % 5u < 4u ? 16u * (served % 5u) : IMAGE ? 56u : 52u);
     }
     const unsigned window_base = kWindowBase + wave * 2u * kWindowBytes;
+    // Windows past the last superblock: windows 0 and 1 of the next item (by parity, so that a
+    // third one repeats the first) when they are fetched ahead, else the last window again.
+    long long ahead_shift = 0;
+    bool ahead = false;
     auto weight_piece = [&](unsigned sb, unsigned k) {
         const unsigned to = (unsigned)__builtin_amdgcn_readfirstlane(
             (int)(window_base + (sb & 1u) * kWindowBytes + k * 1024u));
-        sb = sb < last ? sb : last;
+        const bool past = sb > last;
+        const unsigned record = !past ? sb : ahead ? (sb - superblocks) & 1u : last;
+        const long long offset = (past ? ahead_shift : 0ll) + (long long)(record * (IMAGE ? 72u : 66u));
         const unsigned char *from = IMAGE
-            ? window_from[k] + sb * 72u
-            : (const unsigned char *)((unsigned long long)(window_from[k] + sb * 66u) & ~3ull);
+            ? window_from[k] + offset
+            : (const unsigned char *)((unsigned long long)(window_from[k] + offset) & ~3ull);
         if (k < 2u) copy_to_lds_16(from, to);
         else copy_to_lds_16_first32(from, to);
     };
@@ -249,6 +276,18 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
         const unsigned index = wave == 0u ? lane % T : 0u;
         scale_from = token_row((index % NTB) * 32u + index / NTB);
     }
+    // Where each pair's results go and its route weight, for the publishing pass: requested now,
+    // put into LDS once the previous item's publishing pass is over.
+    const bool info_lane = tid < kTileTokens && tid < it.tokens;
+    unsigned info_out = 0u;
+    float info_weight = 1.0f;
+    if (info_lane) {
+        const unsigned long long ordered = it.pair0 + tid;
+        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
+        info_out = (unsigned)(pr.out_by_source_pair ? source : ordered);
+        if (pr.route_weights) info_weight = pr.route_weights[source];
+    }
+    auto request = request_next();
     constexpr unsigned kActPieces = NTB + 1u;
     auto act_piece = [&](unsigned sb, unsigned j) {
         const unsigned base = kStageBase + (sb % R) * kStageBytes;
@@ -362,22 +401,37 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
     // the rest at the start of the next superblock, so rounds -(R - 1) .. -1 are issued here
     // (windows 0 and 1 are needed before them; the rounds before -1 repeat window 1, which keeps
     // the counts below the same for every superblock).
-    __syncthreads();   // every wave is done with the previous item's stages and output tile
+    lds_barrier();     // every wave is done with the previous item's stages and pair records (its stores may still be on their way)
+    if (prefetched) {      // windows 0 and 1 came with the previous item's last rounds
 #pragma unroll
-    for (unsigned k = 0; k < 3u; ++k) weight_piece(0u, k);
+        for (unsigned j = 0; j < kActPieces; ++j) act_piece(0u, j);
+        __builtin_amdgcn_s_waitcnt(0x0f70u);   // vmcnt(0): stage 0 has landed
+    } else {
 #pragma unroll
-    for (unsigned j = 0; j < kActPieces; ++j) act_piece(0u, j);
+        for (unsigned k = 0; k < 3u; ++k) weight_piece(0u, k);
 #pragma unroll
-    for (unsigned k = 0; k < 3u; ++k) weight_piece(1u, k);
-    // where each pair's results go and its route weight, for the publishing pass
-    if (tid < kTileTokens && tid < it.tokens) {
-        const unsigned long long ordered = it.pair0 + tid;
-        const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
-        const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
-        const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
-        lds_write_uint2(kPairInfoBase + tid * 8u, make_uint2((unsigned)out_index, __float_as_uint(route_weight)));
+        for (unsigned j = 0; j < kActPieces; ++j) act_piece(0u, j);
+#pragma unroll
+        for (unsigned k = 0; k < 3u; ++k) weight_piece(1u, k);
+        __builtin_amdgcn_s_waitcnt(0x0f73u);   // vmcnt(3): window 0 and stage 0 have landed
     }
-    __builtin_amdgcn_s_waitcnt(0x0f73u);   // vmcnt(3): window 0 and stage 0 have landed
+    if (info_lane) lds_write_uint2(kPairInfoBase + tid * 8u, make_uint2(info_out, __float_as_uint(info_weight)));
+    // The next item, and whether its first windows can ride on this item's last rounds: both
+    // items cover whole row tiles of equal geometry (then the same lane copies the same piece of
+    // the same row, one fixed distance on), and the window parity comes out right.
+    resolve_next(request, next);
+    next.ahead = false;
+    next.shift = 0;
+    if (next.state == 0 && superblocks >= 4u && (superblocks & 1u) == 0u &&
+        (!FUSED_UP || (pr.expert_bytes == pr.up_expert_bytes && pr.row_bytes == pr.up_row_bytes)) &&
+        (unsigned long long)(it.row_tile + 1u) * kItemRows <= a.out_rows &&
+        (unsigned long long)(next.it.row_tile + 1u) * kItemRows <= a.out_rows) {
+        next.ahead = true;
+        next.shift = ((long long)next.it.expert - (long long)it.expert) * (long long)pr.expert_bytes +
+                     ((long long)next.it.row_tile - (long long)it.row_tile) * (long long)kItemRows * (long long)pr.row_bytes;
+    }
+    ahead = next.ahead;
+    ahead_shift = next.shift;
     settle(0u);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the window's reads have returned before it is refilled
 #pragma unroll
@@ -522,72 +576,61 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it)
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0x0070u);   // copies past the end have landed before the tile reuses the stages
-
-    // ---- publish: the lane holds, for tokens 32 tb + r, rows 8 q + 4 h + j of its 32 (j < 4) ----
-    // Half of the tile at a time (waves 0-3, then waves 4-7) goes through LDS as [token][value],
-    // values 0-63 the gate sums and 64-127 the up sums of the half's 64 row pairs when fused,
-    // else the 128 rows' sums.
-    auto store4 = [&](unsigned long long out_index, unsigned row, const float (&value)[4]) {
-        const bool good = finite_f32(value[0]) && finite_f32(value[1]) && finite_f32(value[2]) &&
-                          finite_f32(value[3]);
-        if (!good) raise_status(a.status, 1);
-        else if (row + 3u < a.out_rows)
-            *reinterpret_cast<float4 *>(pr.out + out_index * a.out_rows + row) =
-                make_float4(value[0], value[1], value[2], value[3]);
-        else
-            for (unsigned j = 0; j < 4u; ++j)
-                if (row + j < a.out_rows) pr.out[out_index * a.out_rows + row + j] = value[j];
-    };
-    constexpr unsigned kHalfRows = kItemRows / 2u;
-    constexpr unsigned kQuads = kHalfRows / 4u;       // groups of four output values per token
+    // ---- publish: the lane holds, for tokens 32 tb + r, rows 8 q + 4 h + j of its wave's 32
+    // (j < 4): when fused, q 0-1 are gate rows and q 2-3 the matching up rows ----
+    // The values go from the registers straight to memory, 16 bytes a lane: the two halves of a
+    // wave complete 32 bytes of a token's row per store, the four (two) stores of a token block
+    // a whole cache line (half of one), which the L2 merges before it writes them back. No LDS,
+    // no barrier: the stores drain while the next item starts, and copies past the end that are
+    // still in flight land in stages and windows nobody reads before the next item has waited
+    // for copies of its own, which the same wave issues later to the same places.
     const float limit_f32 = (float)a.limit;
-#pragma unroll 1
-    for (unsigned half = 0; half < 2u; ++half) {
-        __syncthreads();   // the stage (first half) or the first half's tile is no longer read
-        if ((wave >> 2) == half) {
-            const unsigned w4 = wave & 3u;
+    const bool whole_quads = (a.out_rows & 3u) == 0u;
+    bool bad = false;
 #pragma unroll
-            for (unsigned tb = 0; tb < NTB; ++tb)
+    for (unsigned tb = 0; tb < NTB; ++tb) {
+        const unsigned token = tb * 32u + r;
+        const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);   // (stale past the item's last token: not used)
+        float *const out_row = pr.out + (unsigned long long)info.x * a.out_rows;
 #pragma unroll
-                for (unsigned q = 0; q < 4u; ++q) {
-                    unsigned column;
-                    if constexpr (FUSED_UP) column = (q >= 2u ? 64u : 0u) + w4 * 16u + 8u * (q & 1u) + 4u * h;
-                    else column = w4 * 32u + 8u * q + 4u * h;
-                    lds_write_uint4(kStageBase + (tb * 32u + r) * kOutPitch + column * 4u,
-                                    make_uint4(__float_as_uint(acc[tb][4u * q]), __float_as_uint(acc[tb][4u * q + 1u]),
-                                               __float_as_uint(acc[tb][4u * q + 2u]), __float_as_uint(acc[tb][4u * q + 3u])));
-                }
-        }
-        __syncthreads();
-#pragma unroll 1
-        for (unsigned unit = tid; unit < T * kQuads; unit += kRowThreads) {
-            const unsigned token = unit / kQuads, quad = unit % kQuads;
-            if (token >= it.tokens) break;
-            const uint2 info = lds_read_uint2(kPairInfoBase + token * 8u);
-            const unsigned row = it.row_tile * kItemRows + half * kHalfRows + 4u * quad;
-            if (row >= a.out_rows) continue;
-            const uint4 g = lds_read_uint4(kStageBase + token * kOutPitch + quad * 16u);
+        for (unsigned q = 0; q < (FUSED_UP ? 2u : 4u); ++q) {
+            const unsigned row = it.row_tile * kItemRows + wave * (FUSED_UP ? 16u : 32u) + 8u * q + 4u * h;
+            float value[4];
+            bool good = true;
             if constexpr (FUSED_UP) {
-                const uint4 up = lds_read_uint4(kStageBase + token * kOutPitch + 256u + quad * 16u);
                 const float route_weight = __uint_as_float(info.y);
-                const float value[4] = {
-                    swiglu_bf16_fast(__uint_as_float(g.x), __uint_as_float(up.x), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.y), __uint_as_float(up.y), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.z), __uint_as_float(up.z), route_weight, a.limit, limit_f32),
-                    swiglu_bf16_fast(__uint_as_float(g.w), __uint_as_float(up.w), route_weight, a.limit, limit_f32)};
-                store4(info.x, row, value);
-            } else {
-                float value[4] = {__uint_as_float(g.x), __uint_as_float(g.y), __uint_as_float(g.z),
-                                  __uint_as_float(g.w)};
-                if (!a.plain_output) {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) value[k] = bf16_round(value[k]);
+                for (unsigned j = 0; j < 4u; ++j)
+                    value[j] = swiglu_bf16_fast(acc[tb][4u * q + j], acc[tb][4u * (q + 2u) + j], route_weight,
+                                                a.limit, limit_f32);
+            } else {
+#pragma unroll
+                for (unsigned j = 0; j < 4u; ++j) {
+                    value[j] = acc[tb][4u * q + j];
+                    good &= finite_f32(value[j]);
+                    if (!a.plain_output) value[j] = bf16_round_number(value[j]);   // (a NaN has just been noted)
                 }
-                store4(info.x, row, value);
+            }
+            good &= finite_f32(value[0]) & finite_f32(value[1]) & finite_f32(value[2]) & finite_f32(value[3]);
+            const bool live = (token < it.tokens) & (row < a.out_rows);
+            bad |= live & !good;
+            if (live & good) {
+                if (whole_quads) {
+                    *reinterpret_cast<float4 *>(out_row + row) = make_float4(value[0], value[1], value[2], value[3]);
+                } else {
+#pragma unroll
+                    for (unsigned j = 0; j < 4u; ++j)
+                        if (row + j < a.out_rows) out_row[row + j] = value[j];
+                }
             }
         }
     }
+    if (bad) raise_status(a.status, 1);
+    // An item with another number of token blocks lays its stages out differently, so that its
+    // copies come from other waves than this item's copies to the same bytes: then this item's
+    // last copies land first (the next item's opening barrier makes that hold for every wave).
+    const unsigned blocks_next = next.state != 0 ? 0u : next.it.tokens <= 32u ? 1u : 2u;
+    if (blocks_next != NTB) __builtin_amdgcn_s_waitcnt(0x0070u);   // vmcnt(0)
 }
 
 template <bool FUSED_UP, bool IMAGE>
@@ -668,10 +711,17 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
         items += (unsigned long long)members[c] * row_tiles;
     }
 
-    for (unsigned long long item = blockIdx.x; item < items; item += gridDim.x) {
-        // ---- which bucket, row tile and token tile ----
-        unsigned bucket, token_tile;
-        MfmaItem it;
+    // ---- which bucket, row tile and token tile an item is: the bucket's record is requested... ----
+    auto request_item = [&](unsigned long long item) {
+        MfmaItemRequest q;
+        q.state = 0;
+        q.partial = false;
+        q.bucket = q.token_tile = q.row_tile = 0u;
+        q.first = q.population = q.expert = 0ull;
+        if (item >= items) {
+            q.state = 2;
+            return q;
+        }
         if (item < full_items) {
             unsigned low = 0u, high = buckets;   // the last bucket whose first full tile is <= item's
             while (low + 1u < high) {
@@ -685,12 +735,12 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
             const unsigned bucket_tiles = lds_read_u32(kTileStartBase + 4u * (low + 1u)) - tile_first;
             const unsigned long long local = item - (unsigned long long)tile_first * row_tiles;
             if (!bucket_tiles) {
-                if (tid == 0u) raise_status(a.status, 2);
-                continue;
+                q.state = 1;
+                return q;
             }
-            bucket = low;
-            token_tile = (unsigned)(local % bucket_tiles);
-            it.row_tile = (unsigned)(local / bucket_tiles);
+            q.bucket = low;
+            q.token_tile = (unsigned)(local % bucket_tiles);
+            q.row_tile = (unsigned)(local / bucket_tiles);
         } else {
             unsigned long long rest = item - full_items;
             unsigned c = 0u;
@@ -699,27 +749,67 @@ __global__ __launch_bounds__(kRowThreads) void mfma_iq2_kernel(MfmaArgs a)
                 c = 1u;
             }
             if (!members[c]) {
-                if (tid == 0u) raise_status(a.status, 2);
-                continue;
+                q.state = 1;
+                return q;
             }
-            bucket = lds_read_u16(kClassListBase + (c * 256u + (unsigned)(rest % members[c])) * 2u);
-            it.row_tile = (unsigned)(rest / members[c]);
-            const unsigned long long n = fixed ? pr.pairs : pr.bucket_populations[bucket];
-            token_tile = (unsigned)(n / kTileTokens);
+            q.bucket = lds_read_u16(kClassListBase + (c * 256u + (unsigned)(rest % members[c])) * 2u);
+            q.row_tile = (unsigned)(rest / members[c]);
+            q.partial = true;               // its token tile is the one after the bucket's full tiles
         }
-        const unsigned long long first = fixed ? 0ull : pr.bucket_offsets[bucket];
-        const unsigned long long population = fixed ? pr.pairs : pr.bucket_populations[bucket];
-        it.expert = fixed ? 0ull : pr.expert_ids[bucket];
-        if (bucket >= buckets || it.expert >= pr.experts || first + population > pr.pairs ||
-            (unsigned long long)token_tile * kTileTokens >= population || it.row_tile >= row_tiles) {
+        if (q.bucket >= buckets) {
+            q.state = 1;
+            return q;
+        }
+        q.first = fixed ? 0ull : pr.bucket_offsets[q.bucket];
+        q.population = fixed ? pr.pairs : pr.bucket_populations[q.bucket];
+        q.expert = fixed ? 0ull : pr.expert_ids[q.bucket];
+        return q;
+    };
+    // ---- ... and looked at later. Every lane holds the same values: the item is kept in scalar
+    // registers. ----
+    auto uniform32 = [](unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); };
+    auto uniform64 = [&](unsigned long long v) {
+        return (unsigned long long)uniform32((unsigned)v) | ((unsigned long long)uniform32((unsigned)(v >> 32)) << 32);
+    };
+    auto resolve_item = [&](const MfmaItemRequest &q, MfmaNextItem &out) {
+        out.ahead = false;
+        out.shift = 0;
+        out.state = (int)uniform32((unsigned)q.state);
+        if (out.state == 2) return;
+        const unsigned long long first = uniform64(q.first), population = uniform64(q.population);
+        const unsigned token_tile = uniform32(q.partial ? (unsigned)(population / kTileTokens) : q.token_tile);
+        out.it.expert = uniform64(q.expert);
+        out.it.row_tile = uniform32(q.row_tile);
+        if (out.state != 0 || out.it.expert >= pr.experts || first + population > pr.pairs ||
+            (unsigned long long)token_tile * kTileTokens >= population || out.it.row_tile >= row_tiles) {
             if (tid == 0u) raise_status(a.status, 2);
-            continue;
+            out.state = 1;
+            return;
         }
         const unsigned long long left = population - (unsigned long long)token_tile * kTileTokens;
-        it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
-        it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
-        if (it.tokens <= 32u) rows_item<FUSED_UP, 1u, IMAGE>(a, it);
-        else rows_item<FUSED_UP, 2u, IMAGE>(a, it);
+        out.it.pair0 = first + (unsigned long long)token_tile * kTileTokens;
+        out.it.tokens = left < kTileTokens ? (unsigned)left : kTileTokens;
+    };
+
+    unsigned long long item = blockIdx.x;
+    MfmaNextItem current;
+    resolve_item(request_item(item), current);
+    bool prefetched = false;
+    while (current.state != 2) {
+        MfmaNextItem next;
+        const unsigned long long following = item + gridDim.x;
+        auto request_next = [&] { return request_item(following); };
+        if (current.state == 0) {
+            if (current.it.tokens <= 32u)
+                rows_item<FUSED_UP, 1u, IMAGE>(a, current.it, prefetched, request_next, resolve_item, next);
+            else
+                rows_item<FUSED_UP, 2u, IMAGE>(a, current.it, prefetched, request_next, resolve_item, next);
+        } else {
+            resolve_item(request_next(), next);
+        }
+        prefetched = current.state == 0 && next.ahead;
+        current = next;
+        item = following;
     }
 }
 
