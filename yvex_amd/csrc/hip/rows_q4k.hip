@@ -291,7 +291,16 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
     }
 
     // ---- publish: lane (token r, half h) holds rows 8 (i / 4) + 4 h + i % 4 of the wave's 32 ----
+    // Four rows at a time, 16 bytes a lane where the output's geometry allows it (the two halves
+    // of a wave then complete 32 bytes of a token's row per store and a token block's stores a
+    // whole cache line, which the L2 merges before writing it back); values that are not finite
+    // are noted and reported once, so that the pass has few branches.
     const float limit_f32 = (float)g.limit;
+    const unsigned long long out_stride = g.plain ? g.out_stride : (unsigned long long)g.out_rows;
+    const bool quads = ((g.out_rows | (unsigned)out_stride) & 3u) == 0u &&
+                       ((unsigned long long)pr.out & 15ull) == 0ull &&
+                       (!(g.plain && g.additive) || ((unsigned long long)g.additive & 15ull) == 0ull);
+    bool bad = false;
 #pragma unroll
     for (unsigned nt = 0; nt < NT; ++nt) {
         const unsigned token = nt * 32u + r;
@@ -300,28 +309,57 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
         const unsigned long long source = pr.order ? pr.order[ordered] : ordered;
         const unsigned long long out_index = pr.out_by_source_pair ? source : ordered;
         const float route_weight = pr.route_weights ? pr.route_weights[source] : 1.0f;
-        constexpr int kValues = FUSED ? 8 : 16;
+        constexpr unsigned kQuads = FUSED ? 2u : 4u;
 #pragma unroll
-        for (int i = 0; i < kValues; ++i) {
-            const unsigned row = row0 + 8u * ((unsigned)i >> 2) + 4u * h + ((unsigned)i & 3u);
+        for (unsigned q4 = 0; q4 < kQuads; ++q4) {
+            const unsigned row = row0 + 8u * q4 + 4u * h;
             if (row >= g.out_rows) continue;
-            float value;
+            const unsigned long long at = out_index * out_stride + row;
+            float value[4];
+            bool fine[4] = {true, true, true, true};
             if constexpr (FUSED) {
-                value = swiglu_bf16_fast(acc[nt][i], acc[nt][i + 8], route_weight, g.limit, limit_f32);
-            } else if (g.plain) {
-                const unsigned long long at = out_index * g.out_stride + row;
-                value = g.additive ? acc[nt][i] + g.additive[at] : acc[nt][i];
-                if (g.output_bf16) value = bf16_round(value);
-                if (!finite_f32(value)) raise_status(g.status, 1);
-                else pr.out[at] = value;
-                continue;
+#pragma unroll
+                for (unsigned k = 0; k < 4u; ++k)
+                    value[k] = swiglu_bf16_fast(acc[nt][4u * q4 + k], acc[nt][4u * q4 + k + 8u], route_weight,
+                                                g.limit, limit_f32);
             } else {
-                value = bf16_round(acc[nt][i]);
+                const bool add = g.plain && g.additive;
+                float extra[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (add) {
+                    if (quads) {
+                        const float4 e = *reinterpret_cast<const float4 *>(g.additive + at);
+                        extra[0] = e.x; extra[1] = e.y; extra[2] = e.z; extra[3] = e.w;
+                    } else {
+#pragma unroll
+                        for (unsigned k = 0; k < 4u; ++k)
+                            if (row + k < g.out_rows) extra[k] = g.additive[at + k];
+                    }
+                }
+                const bool round = g.plain ? g.output_bf16 != 0 : true;
+#pragma unroll
+                for (unsigned k = 0; k < 4u; ++k) {
+                    value[k] = add ? acc[nt][4u * q4 + k] + extra[k] : acc[nt][4u * q4 + k];
+                    fine[k] = finite_f32(value[k]);          // (the rounding below is for numbers)
+                    if (round) value[k] = bf16_round_number(value[k]);
+                }
             }
-            if (!finite_f32(value)) raise_status(g.status, 1);
-            else pr.out[out_index * g.out_rows + row] = value;
+#pragma unroll
+            for (unsigned k = 0; k < 4u; ++k) fine[k] &= finite_f32(value[k]);
+            if (quads & fine[0] & fine[1] & fine[2] & fine[3]) {
+                *reinterpret_cast<float4 *>(pr.out + at) = make_float4(value[0], value[1], value[2], value[3]);
+            } else {
+                // value by value: rows past the last one are not touched, and a value that is
+                // not finite is reported instead of stored
+#pragma unroll
+                for (unsigned k = 0; k < 4u; ++k) {
+                    if (row + k >= g.out_rows) continue;
+                    bad |= !fine[k];
+                    if (fine[k]) pr.out[at + k] = value[k];
+                }
+            }
         }
     }
+    if (bad) raise_status(g.status, 1);
 }
 
 template <bool FUSED>
