@@ -142,6 +142,10 @@ def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
 
 @pytest.mark.parametrize("qtype,rows,width,inputs", [
     ("IQ2_XXS", 516, 2048, 32), ("IQ2_XXS", 260, 7168, 70), ("IQ2_XXS", 7168, 2048, 33),
+    ("IQ2_XXS", 50, 2304, 40), ("IQ2_XXS", 7, 256, 33),
+    # more work items (33 token tiles x 8 row tiles) than workgroups: a workgroup hands over from
+    # one item to the next, whose first weight windows come with the last copies of the one before
+    ("IQ2_XXS", 2048, 1024, 2112),
     ("Q4_K", 516, 2048, 16), ("Q4_K", 132, 7168, 70), ("Q4_K", 2048, 7168, 16), ("Q4_K", 36, 512, 200),
     ("Q4_K", 50, 2304, 17), ("Q4_K", 24, 7168, 32), ("Q4_K", 7, 256, 31)])
 def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, width, inputs):
