@@ -235,36 +235,49 @@ __device__ __forceinline__ void worklist_block(
         population[e] = n;
     }
     __syncthreads();
-    // Exclusive prefix sums over the experts (<= 256) of population, sweep count and occupancy,
-    // three Hillis-Steele scans run together in LDS; every expert then publishes its own bucket.
-    unsigned *scan = slot + experts;                       // [2][3][256]
+    // Inclusive prefix sums over the experts (<= 256: the first four wavefronts) of population,
+    // sweep count and occupancy: a shuffle scan inside each wavefront, the wavefronts' totals
+    // through LDS (one barrier); every expert then publishes its own bucket.
+    unsigned *scan = slot + experts;                       // [4][3] wavefront totals; [1536] running maximum
+    const unsigned n_mine = tid < experts ? population[tid] : 0u;
+    unsigned sum_n = n_mine, sum_sweeps = (n_mine + (unsigned)kPass - 1u) / (unsigned)kPass,
+             sum_used = n_mine ? 1u : 0u;
     if (tid < 256u) {
-        const unsigned n = tid < experts ? population[tid] : 0u;
-        scan[tid] = n;
-        scan[256u + tid] = (n + (unsigned)kPass - 1u) / (unsigned)kPass;
-        scan[512u + tid] = n ? 1u : 0u;
+#pragma unroll
+        for (int step = 1; step < 64; step <<= 1) {
+            const unsigned a = (unsigned)__shfl_up((int)sum_n, step, kWave);
+            const unsigned b = (unsigned)__shfl_up((int)sum_sweeps, step, kWave);
+            const unsigned c = (unsigned)__shfl_up((int)sum_used, step, kWave);
+            if ((int)(tid & 63u) >= step) {
+                sum_n += a;
+                sum_sweeps += b;
+                sum_used += c;
+            }
+        }
+        if ((tid & 63u) == 63u) {
+            scan[3u * (tid >> 6)] = sum_n;
+            scan[3u * (tid >> 6) + 1u] = sum_sweeps;
+            scan[3u * (tid >> 6) + 2u] = sum_used;
+        }
     }
     __syncthreads();
-    unsigned from = 0u, to = 768u;
-    for (unsigned step = 1u; step < 256u; step <<= 1) {
-        if (tid < 768u) {
-            const unsigned lane_in_scan = tid & 255u;
-            unsigned v = scan[from + tid];
-            if (lane_in_scan >= step) v += scan[from + tid - step];
-            scan[to + tid] = v;
+    unsigned total_pairs = 0u, total_sweeps = 0u, bucket_count = 0u;
+    for (unsigned w = 0; w < 4u; ++w) {
+        const unsigned a = scan[3u * w], b = scan[3u * w + 1u], c = scan[3u * w + 2u];
+        if (w < (tid >> 6)) {
+            sum_n += a;
+            sum_sweeps += b;
+            sum_used += c;
         }
-        __syncthreads();
-        const unsigned t = from;
-        from = to;
-        to = t;
+        total_pairs += a;
+        total_sweeps += b;
+        bucket_count += c;
     }
-    const unsigned total_pairs = scan[from + 255u], total_sweeps = scan[from + 256u + 255u];
-    const unsigned bucket_count = scan[from + 512u + 255u];
     if (tid < experts) {
-        const unsigned n = population[tid];
-        const unsigned cursor = scan[from + tid] - n;
-        const unsigned sweeps_before = scan[from + 256u + tid] - (n + (unsigned)kPass - 1u) / (unsigned)kPass;
-        const unsigned bucket = scan[from + 512u + tid] - (n ? 1u : 0u);
+        const unsigned n = n_mine;
+        const unsigned cursor = sum_n - n;
+        const unsigned sweeps_before = sum_sweeps - (n + (unsigned)kPass - 1u) / (unsigned)kPass;
+        const unsigned bucket = sum_used - (n ? 1u : 0u);
         offset[tid] = cursor;
         if (n) {
             expert_ids[bucket] = tid;
