@@ -183,9 +183,9 @@ struct Iq2Tables {
     }
 };
 
-__device__ __forceinline__ uint2 iq2_magnitude_entry(unsigned i)
+// The eight levels of a codebook entry from its sixteen digit bits.
+__device__ __forceinline__ uint2 iq2_magnitude_of_digits(unsigned digits)
 {
-    const unsigned digits = k_iq2_digits[i];
     unsigned lo = 0u, hi = 0u;
 #pragma unroll
     for (unsigned l = 0; l < 4u; ++l) {
@@ -194,6 +194,11 @@ __device__ __forceinline__ uint2 iq2_magnitude_entry(unsigned i)
         hi |= (b == 0u ? 8u : b == 1u ? 25u : 43u) << (8u * l);
     }
     return make_uint2(lo, hi);
+}
+
+__device__ __forceinline__ uint2 iq2_magnitude_entry(unsigned i)
+{
+    return iq2_magnitude_of_digits(k_iq2_digits[i]);
 }
 
 __device__ __forceinline__ uint2 iq2_signmask_entry(unsigned i)

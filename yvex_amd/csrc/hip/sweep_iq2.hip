@@ -114,14 +114,25 @@ __device__ __forceinline__ unsigned lds_load_u32(unsigned address)
 
 __device__ __forceinline__ void sweep_tables_fill()
 {
-    for (unsigned i = threadIdx.x; i < 256u * 16u; i += blockDim.x) {
-        const uint2 m = iq2_magnitude_entry(i >> 4);
+    // (the codebook digits of a thread's entries are requested together: one round trip to
+    // memory, not one per entry)
+    constexpr unsigned kTurns = 256u * 16u / kSweepThreads;
+    static_assert(256u * 16u % kSweepThreads == 0u && 128u * 32u % kSweepThreads == 0u,
+                  "every thread fills the same number of table entries");
+    unsigned digits[kTurns];
+#pragma unroll
+    for (unsigned t = 0; t < kTurns; ++t) digits[t] = k_iq2_digits[(threadIdx.x + t * kSweepThreads) >> 4];
+#pragma unroll
+    for (unsigned t = 0; t < kTurns; ++t) {
+        const unsigned i = threadIdx.x + t * kSweepThreads;
+        const uint2 m = iq2_magnitude_of_digits(digits[t]);
         // byte-wise negation: every level is >= 8, so (x ^ 0xff) + 1 never carries
         lds_store_uint4(kMagBase + i * 16u,
                         make_uint4(m.x, m.y, (m.x ^ 0xffffffffu) + 0x01010101u,
                                    (m.y ^ 0xffffffffu) + 0x01010101u));
     }
-    for (unsigned i = threadIdx.x; i < 128u * 32u; i += blockDim.x) {
+#pragma unroll
+    for (unsigned i = threadIdx.x; i < 128u * 32u; i += kSweepThreads) {
         const unsigned s7 = i >> 5;
         const unsigned s = s7 | ((__popc(s7) & 1u) << 7);
         // selector byte k = k (take +level, source 1) or k + 4 (take -level, source 0)
