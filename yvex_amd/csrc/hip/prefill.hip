@@ -33,8 +33,10 @@
 //       is the exact integer superblock sum of the reference's primitive
 //       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
 //       ((0.125 * d_w) * d_a) * T and summed over superblocks.
-//   Output: the waves' fp32 sums go through LDS, half a tile at a time, so that every store
-//       instruction writes whole 64-byte runs of an output row.
+//   Output: accumulator i of lane (r, h) is token r's sum for row 8 (i / 4) + 4 h + i % 4 of the
+//       wave's 32 (gate sums in the first eight, the matching up sums in the last eight when
+//       fused), so a lane stores four consecutive rows of its token, 16 bytes, straight from its
+//       registers; the stores of a wave complete whole cache lines, which the L2 merges.
 //
 // Same inputs, outputs and rounding points as the decode-width sweeps in moe.hip
 // (src/backend/cuda/tensorcore.cu:378-702 is the reference's counterpart, unused there).
