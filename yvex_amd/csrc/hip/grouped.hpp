@@ -55,8 +55,9 @@ __device__ __forceinline__ float swiglu_bf16_fast(float g, float u, float route_
     const float v = silu * uv * route_weight;
     const unsigned bits = __float_as_uint(v), low = bits & 0xffffu;
     // (one branch: the tests are combined without short circuits)
-    const bool safe = ((double)limit_f32 == limit) & finite_f32(v) & (fabsf(v) > 1.0e-30f) &
-                      (fabsf(gv) <= 16.0f) & ((low < 0x8000u - 64u) | (low > 0x8000u + 64u));
+    const bool finite = finite_f32(v), large = fabsf(v) > 1.0e-30f, inside = fabsf(gv) <= 16.0f;
+    const bool clear = (low < 0x8000u - 64u) | (low > 0x8000u + 64u);
+    const bool safe = ((double)limit_f32 == limit) & finite & large & inside & clear;
     if (safe) return bf16_round_number(v);
     return swiglu_bf16(g, u, route_weight, limit);
 }

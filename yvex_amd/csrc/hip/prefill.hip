@@ -613,7 +613,11 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
                     if (!a.plain_output) value[j] = bf16_round_number(value[j]);   // (a NaN has just been noted)
                 }
             }
-            good &= finite_f32(value[0]) & finite_f32(value[1]) & finite_f32(value[2]) & finite_f32(value[3]);
+#pragma unroll
+            for (unsigned j = 0; j < 4u; ++j) {
+                const bool finite = finite_f32(value[j]);
+                good &= finite;
+            }
             const bool live = (token < it.tokens) & (row < a.out_rows);
             bad |= live & !good;
             if (live & good) {
