@@ -301,16 +301,22 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
 }
 
 // One sweep over the item's weight rows [row_begin, row_end) for N live pairs.
-template <bool FUSED, int N, bool IMAGE>
+// MODE 0: one weight row group (the rows of one iteration) at a time; MODE 1: a gate row group
+// and the matching up row group, SwiGLU in the finishing pass; MODE 2: two consecutive row groups
+// of one matrix, which share the activation columns as gate and up rows do: the fixed cost of an
+// iteration (requests, waits, reduction, loop control) is spent once per two groups.
+template <int MODE, int N, bool IMAGE>
 __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedProblem &pr,
                                           const SweepLane &g, const unsigned char *gate_e,
                                           const unsigned char *up_e, unsigned long long first_ordered,
                                           unsigned row_begin, unsigned row_end, bool pairs_in_lds)
 {
+    constexpr bool FUSED = MODE == 1;
+    constexpr bool TWIN = MODE != 0;     // two streams of weight rows against the same activation columns
     const unsigned lane = threadIdx.x & 63u;
     const bool odd = (lane & 1u) != 0u;
-    // packed values per iteration: (gate, up) of pair v when fused, else pairs (2v, 2v + 1)
-    constexpr int PV = FUSED ? N : (N + 1) / 2;
+    // packed values per iteration: (first, second stream) of pair v with two streams, else pairs (2v, 2v + 1)
+    constexpr int PV = TWIN ? N : (N + 1) / 2;
 
     // ---- the sweep's activation rows: this lane's 128 columns stay in registers ----
     unsigned act[N][32];
@@ -350,23 +356,26 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     float packed_scale[PV];
 #pragma unroll
     for (int v = 0; v < PV; ++v) {
-        if constexpr (FUSED) packed_scale[v] = act_scale[v];
+        if constexpr (TWIN) packed_scale[v] = act_scale[v];
         else packed_scale[v] = odd ? (2 * v + 1 < N ? act_scale[2 * v + 1 < N ? 2 * v + 1 : 0] : 0.0f)
                                    : act_scale[2 * v];
     }
 
-    const unsigned rows = row_end - row_begin;               // a multiple of rows_per_iter
-    const unsigned iterations = rows / g.rows_per_iter;       // <= kSweepIters
+    const unsigned rows_per_turn = MODE == 2 ? 2u * g.rows_per_iter : g.rows_per_iter;
+    const unsigned rows = row_end - row_begin;               // a multiple of rows_per_turn
+    const unsigned iterations = rows / rows_per_turn;         // <= kSweepIters
     // wave-uniform row bases advance by a scalar stride; the lane's place inside an iteration's
     // rows is a constant 32-bit offset
     const unsigned char *gate_rows = gate_e + (unsigned long long)row_begin * pr.row_bytes;
-    const unsigned char *up_rows = FUSED ? up_e + (unsigned long long)row_begin * pr.up_row_bytes : nullptr;
-    const unsigned long long gate_step = (unsigned long long)g.rows_per_iter * pr.row_bytes;
-    const unsigned long long up_step = (unsigned long long)g.rows_per_iter * pr.up_row_bytes;
+    const unsigned long long second_row_bytes = FUSED ? pr.up_row_bytes : pr.row_bytes;
+    const unsigned char *up_rows = FUSED ? up_e + (unsigned long long)row_begin * pr.up_row_bytes
+        : MODE == 2 ? gate_rows + (unsigned long long)g.rows_per_iter * pr.row_bytes : nullptr;
+    const unsigned long long gate_step = (unsigned long long)rows_per_turn * pr.row_bytes;
+    const unsigned long long up_step = (unsigned long long)rows_per_turn * second_row_bytes;
     const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
     // (row bases and row strides are multiples of four bytes: checked on the host)
     const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * (IMAGE ? 72u : 66u);
-    const unsigned up_block = lane_row * (unsigned)pr.up_row_bytes + lane_super * (IMAGE ? 72u : 66u);
+    const unsigned up_block = lane_row * (unsigned)second_row_bytes + lane_super * (IMAGE ? 72u : 66u);
     // image: the lane's record is its first dword (scale and group scales) and eight more
     const unsigned gate_codes_at = IMAGE ? gate_block + 36u * g.half + 4u
                                          : (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
@@ -381,13 +390,13 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     // final row) and every lane stores (lanes that hold no result write to a spare word), so no
     // branch sits between a request and the wait that consumes it and the waits stay counted.
     constexpr int AHEAD = N <= 2 ? kSweepAheadSmall : 1;   // rows requested ahead of the one decoded
-    constexpr int STREAMS = FUSED ? 2 : 1;
+    constexpr int STREAMS = TWIN ? 2 : 1;
     Iq2Half ring[AHEAD + 1][STREAMS];
     const unsigned last = iterations - 1u;
     auto request = [&](Iq2Half (&slot)[STREAMS], unsigned it) {
         const unsigned clamped = it < last ? it : last;
         slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at);
-        if constexpr (FUSED)
+        if constexpr (TWIN)
             slot[1].load(up_rows + clamped * up_step, up_codes_at, up_tail_at);
     };
     // The first requests are kept in ring order: the loop's first wait is counted against the
@@ -422,7 +431,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 #pragma unroll
         for (int p = 0; p < N; ++p) {
             total_gate[p] += dpp_move<0xb1, 0xf>(total_gate[p]);
-            if constexpr (FUSED) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
+            if constexpr (TWIN) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
         }
         // The even lane of a pair scales the first stream and the odd lane the last one. An odd
         // lane holds the second half of its superblock, so where the scale rides in the first
@@ -441,7 +450,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
             int t;
-            if constexpr (FUSED) t = odd ? total_up[v] : total_gate[v];
+            if constexpr (TWIN) t = odd ? total_up[v] : total_gate[v];
             else t = odd ? total_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : total_gate[2 * v];
             float value = weight_scale * packed_scale[v] * (float)t;
             value = dpp_add<0x4e>(value);     // lanes i and i ^ 2
@@ -462,8 +471,10 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned outputs = rows * (unsigned)N;
     for (unsigned o = lane; o < outputs; o += 64u) {
         const unsigned p = o / rows, local = o % rows;      // consecutive lanes: consecutive rows
-        const unsigned it = local / g.rows_per_iter, sub = local % g.rows_per_iter;
-        const unsigned v = FUSED ? p : p >> 1, parity = FUSED ? 0u : p & 1u;
+        // the iteration, which of its two row groups (MODE 2) and the row inside the group
+        const unsigned it = local / rows_per_turn, within = local % rows_per_turn;
+        const unsigned second_group = MODE == 2 ? within / g.rows_per_iter : 0u, sub = within % g.rows_per_iter;
+        const unsigned v = TWIN ? p : p >> 1, parity = TWIN ? second_group : p & 1u;
         const unsigned address = g.park + ((it * PV + v) * 2u + parity) * 16u + sub * groups_per_row * 4u;
         float first = 0.0f, second = 0.0f;
         for (unsigned k = 0; k < groups_per_row; ++k) {
@@ -486,9 +497,10 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     __builtin_amdgcn_wave_barrier();
 }
 
-template <bool FUSED, bool IMAGE>
+template <int MODE, bool IMAGE>
 __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
 {
+    constexpr bool FUSED = MODE == 1;
     extern __shared__ __align__(16) unsigned char sweep_lds[];
     if (lds_address_of(sweep_lds) != 0u) {   // the lookups address LDS by absolute byte offsets
         if (threadIdx.x == 0u) raise_status(a.status, 2);
@@ -569,7 +581,7 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     // into short ones that come last in the item list: the waves of the grid finish within a short
     // item of each other instead of a long one, and only the short items pay the fixed cost of an
     // item (its activation columns, the first requests, the finishing pass) more often.
-    const unsigned item_rows = kSweepIters * g.rows_per_iter;
+    const unsigned item_rows = kSweepIters * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
     const unsigned short_rows = item_rows / kSweepShortDiv;
     const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * kSweepLongPercent / 100u / item_rows);
     const unsigned long_rows = long_tiles * item_rows;
@@ -711,13 +723,13 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned long long live = population - pass;
         const bool cached = pairs_in_lds && is_routed;
         if (kSweepPairs >= 4 && live >= 4ull)
-            iq2_sweep<FUSED, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (kSweepPairs >= 3 && live >= 3ull)
-            iq2_sweep<FUSED, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (live >= 2ull)
-            iq2_sweep<FUSED, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else
-            iq2_sweep<FUSED, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
     }
 }
 
@@ -732,21 +744,28 @@ bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long p
     return out_rows % rows_per_iter == 0u;   // an iteration never reads past the last row
 }
 
-template <bool FUSED, bool IMAGE>
+template <int MODE, bool IMAGE>
 static int launch_iq2_sweep_variant(const GroupedArgs &a, hipStream_t stream)
 {
-    YVEX_ALLOW_DYNAMIC_LDS((iq2_sweep_kernel<FUSED, IMAGE>), kSweepLdsBytes);
-    iq2_sweep_kernel<FUSED, IMAGE><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
+    YVEX_ALLOW_DYNAMIC_LDS((iq2_sweep_kernel<MODE, IMAGE>), kSweepLdsBytes);
+    iq2_sweep_kernel<MODE, IMAGE><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
     return check_launch("moe_sweep_iq2");
 }
 
 int launch_iq2_sweep(const GroupedArgs &a, bool fused, bool image, hipStream_t stream)
 {
+    // a projection that is not fused takes two row groups an iteration where the rows allow it
+    // (every item then holds whole pairs of groups: the short items are half a long one)
+    const unsigned lanes_per_row = a.width / 128u;
+    const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u ? 64u / lanes_per_row : 1u;
+    const int mode = fused ? 1 : a.out_rows % (2u * rows_per_iter) == 0u ? 2 : 0;
     if (image)
-        return fused ? launch_iq2_sweep_variant<true, true>(a, stream)
-                     : launch_iq2_sweep_variant<false, true>(a, stream);
-    return fused ? launch_iq2_sweep_variant<true, false>(a, stream)
-                 : launch_iq2_sweep_variant<false, false>(a, stream);
+        return mode == 1 ? launch_iq2_sweep_variant<1, true>(a, stream)
+             : mode == 2 ? launch_iq2_sweep_variant<2, true>(a, stream)
+                         : launch_iq2_sweep_variant<0, true>(a, stream);
+    return mode == 1 ? launch_iq2_sweep_variant<1, false>(a, stream)
+         : mode == 2 ? launch_iq2_sweep_variant<2, false>(a, stream)
+                     : launch_iq2_sweep_variant<0, false>(a, stream);
 }
 
 // ---- the image: canonical IQ2_XXS superblocks re-packed for the sweeps -------------------------
