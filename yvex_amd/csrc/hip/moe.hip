@@ -383,7 +383,7 @@ __global__ __launch_bounds__(1024) void decode_prepare_kernel(
 // and every sweep serves up to kPass pairs of the bucket.
 
 constexpr int kRowsInFlight = 1;  // weight-row groups a wave decodes back to back
-constexpr int kGroupedThreads = 768;
+constexpr int kGroupedThreads = 512;     // two waves per SIMD: with three, a sweep's activation columns spill out of 168 registers
 constexpr int kGroupedWaves = kGroupedThreads / 64;
 constexpr unsigned kItemRowsMax = 16u;   // gate/up row pairs per item when the SwiGLU is fused
 
