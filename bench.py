@@ -515,6 +515,30 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     }
 
 
+def decode_q4k_leg(torch, K, weights, shared, dev, steps: int, warmup: int):
+    """The headline batch (32 rows, top-8 of 256 + shared) with Q4_K experts, through the C ABI:
+    the decode-width sweeps read Q4_K rows too. Bytes counted: the canonical bytes of the distinct
+    experts hit."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(77)
+    x = torch.randn((ROWS, HIDDEN), device=dev, generator=gen)
+    router = (torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5).contiguous()
+    layer = AbiLayer(torch, weights, shared, router, x.cpu().numpy(), ROWS, qtype=K.Q4_K)
+    layer.step(defer=False)
+    unique = int(layer.result.unique_experts)
+    eager_ms = layer.timed(steps, warmup, eager=True)
+    graph_ms = layer.timed(steps, max(warmup, 2))
+    layer.close()
+    step_ms = min(graph_ms, eager_ms)
+    expert_bytes = 3 * INTERMEDIATE * HIDDEN // 256 * 144
+    read = (unique + 1) * expert_bytes
+    return {"workload": "moe_decode_q4k: 32 rows, top-8 of 256 Q4_K experts + shared, Q8_K activations",
+            "ms_per_step": round(step_ms, 4), "graph_ms_per_step": round(graph_ms, 4),
+            "eager_ms_per_step": round(eager_ms, 4), "distinct_routed_experts": unique,
+            "GB_per_s": round(read / (step_ms * 1e-3) / 1e9, 1),
+            "hbm_peak_frac": round(read / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -800,6 +824,7 @@ def main() -> int:
         q4_shared = tuple(synth_q4k(torch, INTERMEDIATE * HIDDEN // 256, dev, 31 + i) for i in range(3))
         out["prefill_q4k"] = prefill_leg(torch, K, MoeLayer, q4_routed, q4_shared, dev,
                                          max(3, args.steps // 10), 2, qt=K.Q4_K)
+        out["decode_q4k"] = decode_q4k_leg(torch, K, q4_routed, q4_shared, dev, args.steps, args.warmup)
         del q4_routed, q4_shared
         torch.cuda.empty_cache()
         layer = gate = up = down = shared = None

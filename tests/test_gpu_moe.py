@@ -61,6 +61,11 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
     # per iteration over a down projection whose rows end inside a 16-lane group
     ("IQ2_XXS", 2048, 2048, 6, 4, 20, True, 1, False),
     ("IQ2_XXS", 4096, 3072, 4, 2, 5, True, 0, False),
+    # Q4_K rows through the specialised sweeps: four rows per iteration with buckets past four
+    # pairs, real widths (56 lanes a row), two rows per iteration
+    ("Q4_K", 2048, 2048, 6, 4, 20, True, 1, False),
+    ("Q4_K", 7168, 2048, 12, 4, 6, True, 0, False),
+    ("Q4_K", 4096, 3072, 4, 2, 5, True, 0, False),
     # many buckets: more sweeps than one wavefront lists (the class list is built by several)
     ("IQ2_XXS", 2048, 2048, 200, 8, 40, True, 1, False),
     # row-batch kernels on the matrix cores: tiny buckets, buckets past one 128-pair tile, real widths

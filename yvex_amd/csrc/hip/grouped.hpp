@@ -153,8 +153,8 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
 
 // Specialised IQ2_XXS x Q8_K decode sweeps (sweep_iq2.hip): reduction widths whose rows span 16
 // to 64 lanes of 128 columns each.
-bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs, bool image);
-int launch_iq2_sweep(const GroupedArgs &a, bool fused, bool image, hipStream_t stream);
+bool iq2_sweep_supported(unsigned qtype, unsigned width, unsigned out_rows, unsigned long long pairs, bool image);
+int launch_iq2_sweep(const GroupedArgs &a, unsigned qtype, bool fused, bool image, hipStream_t stream);
 
 // Row-batch expert kernels for Q4_K weights on the int8 matrix cores (dense_q4k.hip).
 int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t width, uint64_t out_rows,

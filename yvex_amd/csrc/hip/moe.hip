@@ -771,9 +771,8 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
     }
     unsigned long long all_pairs = 0ull;
     for (unsigned i = 0; i < a.problems; ++i) all_pairs += a.problem[i].pairs;
-    if (qtype == QT_IQ2_XXS && q8 && aligned &&
-        iq2_sweep_supported(a.width, a.out_rows, all_pairs, a.image != 0))
-        return launch_iq2_sweep(a, fused, a.image != 0, stream);
+    if (q8 && aligned && iq2_sweep_supported(qtype, a.width, a.out_rows, all_pairs, a.image != 0))
+        return launch_iq2_sweep(a, qtype, fused, a.image != 0, stream);
     if (a.image) return ST_UNSUPPORTED;      // only the specialised sweeps read the image
     switch (qtype) {
     case QT_IQ2_XXS: return launch_grouped<QT_IQ2_XXS>(a, q8, fused, stream);

@@ -300,12 +300,87 @@ __device__ __forceinline__ void iq2_half_dots(const Iq2Half (&c)[STREAMS], const
     }
 }
 
+// ---- Q4_K rows in the same sweeps ---------------------------------------------------------------
+//
+// A lane's share of one Q4_K weight row: the superblock's 16-byte head (d, dmin, the twelve bytes
+// of 6-bit scales and minimums) and the 64 code bytes of its half (sub-blocks 4 h .. 4 h + 3:
+// two chunks of 32 bytes, low nibbles one sub-block and high nibbles the next). Superblocks are
+// 144 bytes, so every load is 16-byte aligned relative to the row.
+struct Q4kHalf {
+    uint4 head;
+    uint4 q[4];
+    __device__ __forceinline__ void load(const unsigned char *rows, unsigned codes_at, unsigned head_at)
+    {
+        head = *reinterpret_cast<const uint4 *>(rows + head_at);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) q[i] = *reinterpret_cast<const uint4 *>(rows + codes_at + 16u * i);
+    }
+};
+
+template <unsigned QT>
+struct SweepHalf {
+    using type = Iq2Half;
+};
+template <>
+struct SweepHalf<QT_Q4_K> {
+    using type = Q4kHalf;
+};
+
+// Exact integer sums of this lane's four sub-blocks of each of STREAMS weight rows against N
+// activation rows: dot = sum over sub-blocks of scale * (nibbles . activations), minimum = sum of
+// minimum * (sum of the sub-block's activations), the two terms of the reference's primitive
+// (src/backend/cuda/kernel_primitives.h:315-340). No tables: a nibble is a mask away.
+template <int STREAMS, int N>
+__device__ __forceinline__ void q4k_half_dots(const Q4kHalf (&c)[STREAMS], const SweepLane &g,
+                                              const unsigned (&act)[N][32], const int (&act_sums)[N][4],
+                                              int (&dot)[STREAMS][N], int (&minimum)[STREAMS][N])
+{
+#pragma unroll
+    for (int w = 0; w < STREAMS; ++w) {
+        const unsigned s0 = c[w].head.y, s1 = c[w].head.z, s2 = c[w].head.w;
+        // the four scales and the four minimums of this half, one to a byte
+        const unsigned scales = g.half ? ((s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)) : (s0 & 0x3f3f3f3fu);
+        const unsigned minimums = g.half ? (((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u))
+                                         : (s1 & 0x3f3f3f3fu);
+#pragma unroll
+        for (int p = 0; p < N; ++p) {
+            int m = 0;
+#pragma unroll
+            for (int sub = 0; sub < 4; ++sub)
+                m += __mul24((int)((minimums >> (8 * sub)) & 255u), act_sums[p][sub]);   // 63 * 32 * 127 * 4 < 2^23
+            minimum[w][p] = m;
+            dot[w][p] = 0;
+        }
+#pragma unroll
+        for (int chunk = 0; chunk < 2; ++chunk) {
+            const unsigned words[8] = {c[w].q[2 * chunk].x, c[w].q[2 * chunk].y, c[w].q[2 * chunk].z,
+                                       c[w].q[2 * chunk].w, c[w].q[2 * chunk + 1].x, c[w].q[2 * chunk + 1].y,
+                                       c[w].q[2 * chunk + 1].z, c[w].q[2 * chunk + 1].w};
+            int low[N], high[N];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const unsigned lo = words[i] & 0x0f0f0f0fu, hi = (words[i] >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+                for (int p = 0; p < N; ++p) {
+                    low[p] = i == 0 ? dot4_from_zero(lo, act[p][16 * chunk + i]) : dot4(lo, act[p][16 * chunk + i], low[p]);
+                    high[p] = i == 0 ? dot4_from_zero(hi, act[p][16 * chunk + 8 + i])
+                                     : dot4(hi, act[p][16 * chunk + 8 + i], high[p]);
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < N; ++p)   // |sum| <= 15 * 127 * 32 < 2^16
+                dot[w][p] += __mul24(low[p], (int)((scales >> (16 * chunk)) & 255u)) +
+                             __mul24(high[p], (int)((scales >> (16 * chunk + 8)) & 255u));
+        }
+    }
+}
+
 // One sweep over the item's weight rows [row_begin, row_end) for N live pairs.
 // MODE 0: one weight row group (the rows of one iteration) at a time; MODE 1: a gate row group
 // and the matching up row group, SwiGLU in the finishing pass; MODE 2: two consecutive row groups
 // of one matrix, which share the activation columns as gate and up rows do: the fixed cost of an
 // iteration (requests, waits, reduction, loop control) is spent once per two groups.
-template <int MODE, int N, bool IMAGE>
+template <int MODE, int N, bool IMAGE, unsigned QT>
 __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedProblem &pr,
                                           const SweepLane &g, const unsigned char *gate_e,
                                           const unsigned char *up_e, unsigned long long first_ordered,
@@ -313,6 +388,8 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 {
     constexpr bool FUSED = MODE == 1;
     constexpr bool TWIN = MODE != 0;     // two streams of weight rows against the same activation columns
+    constexpr bool Q4 = QT == QT_Q4_K;
+    static_assert(!(Q4 && IMAGE), "the image is a layout of IQ2_XXS rows");
     const unsigned lane = threadIdx.x & 63u;
     const bool odd = (lane & 1u) != 0u;
     // packed values per iteration: (first, second stream) of pair v with two streams, else pairs (2v, 2v + 1)
@@ -320,6 +397,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 
     // ---- the sweep's activation rows: this lane's 128 columns stay in registers ----
     unsigned act[N][32];
+    int act_sums[N][Q4 ? 4 : 1];     // Q4_K: the sums of the activations under each of the lane's four sub-blocks
     float act_scale[N];
     float route_weight[N];
     unsigned long long out_index[N];
@@ -351,6 +429,18 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             act[p][4 * k + 2] = g.live ? v.z : 0u;
             act[p][4 * k + 3] = g.live ? v.w : 0u;
         }
+        if constexpr (Q4) {
+            // the block's sixteen sums of 16 activations follow its 256 values: eight belong to this half
+            uint4 sums;
+            __builtin_memcpy(&sums, blk + 260u + 16u * g.half, 16);
+            const unsigned pairs_of_sums[4] = {sums.x, sums.y, sums.z, sums.w};
+#pragma unroll
+            for (int sub = 0; sub < 4; ++sub)
+                act_sums[p][sub] = g.live ? (int)(short)(pairs_of_sums[sub] & 0xffffu) + (int)(short)(pairs_of_sums[sub] >> 16)
+                                          : 0;
+        } else {
+            act_sums[p][0] = 0;
+        }
     }
     // the activation scale each lane applies to packed value v
     float packed_scale[PV];
@@ -374,16 +464,21 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned long long up_step = (unsigned long long)rows_per_turn * second_row_bytes;
     const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
     // (row bases and row strides are multiples of four bytes: checked on the host)
-    const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * (IMAGE ? 72u : 66u);
-    const unsigned up_block = lane_row * (unsigned)second_row_bytes + lane_super * (IMAGE ? 72u : 66u);
+    constexpr unsigned kSuperBytes = Q4 ? 144u : IMAGE ? 72u : 66u;
+    const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * kSuperBytes;
+    const unsigned up_block = lane_row * (unsigned)second_row_bytes + lane_super * kSuperBytes;
     // image: the lane's record is its first dword (scale and group scales) and eight more
-    const unsigned gate_codes_at = IMAGE ? gate_block + 36u * g.half + 4u
-                                         : (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
-    const unsigned up_codes_at = IMAGE ? up_block + 36u * g.half + 4u : (up_block + 2u + 32u * g.half) & ~3u;
+    // (Q4_K: the half's 64 code bytes behind the 16-byte head, which is the "tail" load)
+    const unsigned gate_codes_at = Q4 ? gate_block + 16u + 64u * g.half
+        : IMAGE ? gate_block + 36u * g.half + 4u
+                : (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
+    const unsigned up_codes_at = Q4 ? up_block + 16u + 64u * g.half
+        : IMAGE ? up_block + 36u * g.half + 4u : (up_block + 2u + 32u * g.half) & ~3u;
     // ninth dword: the end of the codes where they start two bytes in, else the scale's dword
-    const unsigned gate_tail_at = IMAGE ? gate_codes_at - 4u
+    const unsigned gate_tail_at = Q4 ? gate_block : IMAGE ? gate_codes_at - 4u
                                         : g.code_shift ? gate_codes_at + 32u : gate_block & ~3u;
-    const unsigned up_tail_at = IMAGE ? up_codes_at - 4u : g.code_shift ? up_codes_at + 32u : up_block & ~3u;
+    const unsigned up_tail_at = Q4 ? up_block
+        : IMAGE ? up_codes_at - 4u : g.code_shift ? up_codes_at + 32u : up_block & ~3u;
     // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
     // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
     // The loop body is one basic block: every turn requests a row (the last ones clamped to the
@@ -391,9 +486,10 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     // branch sits between a request and the wait that consumes it and the waits stay counted.
     constexpr int AHEAD = N <= 2 ? kSweepAheadSmall : 1;   // rows requested ahead of the one decoded
     constexpr int STREAMS = TWIN ? 2 : 1;
-    Iq2Half ring[AHEAD + 1][STREAMS];
+    using Half = typename SweepHalf<QT>::type;
+    Half ring[AHEAD + 1][STREAMS];
     const unsigned last = iterations - 1u;
-    auto request = [&](Iq2Half (&slot)[STREAMS], unsigned it) {
+    auto request = [&](Half (&slot)[STREAMS], unsigned it) {
         const unsigned clamped = it < last ? it : last;
         slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at);
         if constexpr (TWIN)
@@ -416,15 +512,26 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
       for (int turn = 0; turn <= AHEAD; ++turn) {
         const unsigned it = it0 + (unsigned)turn;   // may run past the last row by AHEAD turns
         request(ring[(turn + AHEAD) % (AHEAD + 1)], it + AHEAD);
-        const Iq2Half (&now)[STREAMS] = ring[turn];
+        const Half (&now)[STREAMS] = ring[turn];
         int total_gate[N], total_up[N];
+        int min_gate[N], min_up[N];          // Q4_K: the sums of the minimum term
         {
-            int totals[STREAMS][N];
-            iq2_half_dots<STREAMS, N, IMAGE>(now, g, act, totals);
+            int totals[STREAMS][N], minimums[STREAMS][N];
+            if constexpr (Q4) {
+                q4k_half_dots<STREAMS, N>(now, g, act, act_sums, totals, minimums);
+            } else {
+                iq2_half_dots<STREAMS, N, IMAGE>(now, g, act, totals);
+#pragma unroll
+                for (int w = 0; w < STREAMS; ++w)
+#pragma unroll
+                    for (int p = 0; p < N; ++p) minimums[w][p] = 0;
+            }
 #pragma unroll
             for (int p = 0; p < N; ++p) {
                 total_gate[p] = totals[0][p];
                 total_up[p] = totals[STREAMS - 1][p];
+                min_gate[p] = minimums[0][p];
+                min_up[p] = minimums[STREAMS - 1][p];
             }
         }
         // the two lanes of a superblock add their halves: exact int32 superblock sums
@@ -432,13 +539,20 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         for (int p = 0; p < N; ++p) {
             total_gate[p] += dpp_move<0xb1, 0xf>(total_gate[p]);
             if constexpr (TWIN) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
+            if constexpr (Q4) {
+                min_gate[p] += dpp_move<0xb1, 0xf>(min_gate[p]);
+                if constexpr (TWIN) min_up[p] += dpp_move<0xb1, 0xf>(min_up[p]);
+            }
         }
         // The even lane of a pair scales the first stream and the odd lane the last one. An odd
         // lane holds the second half of its superblock, so where the scale rides in the first
         // half's codes it comes from the neighbour.
-        const Iq2Half &mine = odd ? now[STREAMS - 1] : now[0];
-        float weight_scale;
-        if constexpr (IMAGE) {
+        const Half &mine = odd ? now[STREAMS - 1] : now[0];
+        float weight_scale, weight_minimum = 0.0f;
+        if constexpr (Q4) {
+            weight_scale = f16_bits_to_float(mine.head.x & 0xffffu);       // d
+            weight_minimum = f16_bits_to_float(mine.head.x >> 16);         // dmin
+        } else if constexpr (IMAGE) {
             weight_scale = 0.125f * f16_bits_to_float(mine.tail & 0xffffu);
         } else {
             // (the exchange runs in every lane: it reads its neighbour, which must be executing it)
@@ -449,10 +563,20 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         }
 #pragma unroll
         for (int v = 0; v < PV; ++v) {
-            int t;
+            int t, m = 0;
             if constexpr (TWIN) t = odd ? total_up[v] : total_gate[v];
             else t = odd ? total_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : total_gate[2 * v];
-            float value = weight_scale * packed_scale[v] * (float)t;
+            float value;
+            if constexpr (Q4) {
+                if constexpr (TWIN) m = odd ? min_up[v] : min_gate[v];
+                else m = odd ? min_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : min_gate[2 * v];
+                // (d_a d) dot - (d_a dmin) minimum, each product rounded: the order of the reference's primitive
+                const float left = packed_scale[v] * weight_scale * (float)t;
+                const float right = packed_scale[v] * weight_minimum * (float)m;
+                value = left - right;
+            } else {
+                value = weight_scale * packed_scale[v] * (float)t;
+            }
             value = dpp_add<0x4e>(value);     // lanes i and i ^ 2
             value = dpp_add<0x124>(value);    // + lane i - 4 (row rotate)
             value = dpp_add<0x128>(value);    // + lanes i - 8, i - 12: all lanes of this parity
@@ -497,7 +621,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int MODE, bool IMAGE>
+template <int MODE, bool IMAGE, unsigned QT>
 __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
 {
     constexpr bool FUSED = MODE == 1;
@@ -530,7 +654,7 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         for (unsigned k = 0; k < 2u; ++k)
             if (tid + k * kSweepThreads < routed.pairs) source_here[k] = routed.order[tid + k * kSweepThreads];
     }
-    sweep_tables_fill();
+    if constexpr (QT == QT_IQ2_XXS) sweep_tables_fill();     // (Q4_K rows need no tables)
     if (tid == 0u) lds_store_u32(kTicketAddress, 0u);
     if (pairs_in_lds) {
         float weight_here[2];
@@ -723,49 +847,57 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         const unsigned long long live = population - pass;
         const bool cached = pairs_in_lds && is_routed;
         if (kSweepPairs >= 4 && live >= 4ull)
-            iq2_sweep<MODE, kSweepPairs >= 4 ? 4 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, kSweepPairs >= 4 ? 4 : 1, IMAGE, QT>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (kSweepPairs >= 3 && live >= 3ull)
-            iq2_sweep<MODE, kSweepPairs >= 3 ? 3 : 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, kSweepPairs >= 3 ? 3 : 1, IMAGE, QT>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else if (live >= 2ull)
-            iq2_sweep<MODE, 2, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, 2, IMAGE, QT>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
         else
-            iq2_sweep<MODE, 1, IMAGE>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
+            iq2_sweep<MODE, 1, IMAGE, QT>(a, pr, g, gate_e, up_e, first + pass, row_begin, row_end, cached);
     }
 }
 
-bool iq2_sweep_supported(unsigned width, unsigned out_rows, unsigned long long pairs, bool image)
+bool iq2_sweep_supported(unsigned qtype, unsigned width, unsigned out_rows, unsigned long long pairs, bool image)
 {
+    if (qtype != QT_IQ2_XXS && qtype != QT_Q4_K) return false;
+    if (image && qtype != QT_IQ2_XXS) return false;
     if (pairs > kClassMaxSweeps) return false;            // every sweep serves at least one pair
     const unsigned lanes_per_row = width / 128u;
     if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
-    if (!image && (width / 256u * 66u) % 4u != 0u) return false;   // rows must start on dword boundaries
+    // IQ2_XXS rows must start on dword boundaries (Q4_K rows are multiples of 144 bytes)
+    if (qtype == QT_IQ2_XXS && !image && (width / 256u * 66u) % 4u != 0u) return false;
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u
         ? 64u / lanes_per_row : 1u;
     return out_rows % rows_per_iter == 0u;   // an iteration never reads past the last row
 }
 
-template <int MODE, bool IMAGE>
+template <int MODE, bool IMAGE, unsigned QT>
 static int launch_iq2_sweep_variant(const GroupedArgs &a, hipStream_t stream)
 {
-    YVEX_ALLOW_DYNAMIC_LDS((iq2_sweep_kernel<MODE, IMAGE>), kSweepLdsBytes);
-    iq2_sweep_kernel<MODE, IMAGE><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
-    return check_launch("moe_sweep_iq2");
+    YVEX_ALLOW_DYNAMIC_LDS((iq2_sweep_kernel<MODE, IMAGE, QT>), kSweepLdsBytes);
+    iq2_sweep_kernel<MODE, IMAGE, QT><<<compute_units(), kSweepThreads, kSweepLdsBytes, stream>>>(a);
+    return check_launch("moe_sweep");
 }
 
-int launch_iq2_sweep(const GroupedArgs &a, bool fused, bool image, hipStream_t stream)
+template <bool IMAGE, unsigned QT>
+static int launch_iq2_sweep_mode(const GroupedArgs &a, int mode, hipStream_t stream)
+{
+    return mode == 1 ? launch_iq2_sweep_variant<1, IMAGE, QT>(a, stream)
+         : mode == 2 ? launch_iq2_sweep_variant<2, IMAGE, QT>(a, stream)
+                     : launch_iq2_sweep_variant<0, IMAGE, QT>(a, stream);
+}
+
+int launch_iq2_sweep(const GroupedArgs &a, unsigned qtype, bool fused, bool image, hipStream_t stream)
 {
     // a projection that is not fused takes two row groups an iteration where the rows allow it
     // (every item then holds whole pairs of groups: the short items are half a long one)
     const unsigned lanes_per_row = a.width / 128u;
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u ? 64u / lanes_per_row : 1u;
     const int mode = fused ? 1 : a.out_rows % (2u * rows_per_iter) == 0u ? 2 : 0;
-    if (image)
-        return mode == 1 ? launch_iq2_sweep_variant<1, true>(a, stream)
-             : mode == 2 ? launch_iq2_sweep_variant<2, true>(a, stream)
-                         : launch_iq2_sweep_variant<0, true>(a, stream);
-    return mode == 1 ? launch_iq2_sweep_variant<1, false>(a, stream)
-         : mode == 2 ? launch_iq2_sweep_variant<2, false>(a, stream)
-                     : launch_iq2_sweep_variant<0, false>(a, stream);
+    if (qtype == QT_Q4_K) return image ? ST_UNSUPPORTED : launch_iq2_sweep_mode<false, QT_Q4_K>(a, mode, stream);
+    if (qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
+    return image ? launch_iq2_sweep_mode<true, QT_IQ2_XXS>(a, mode, stream)
+                 : launch_iq2_sweep_mode<false, QT_IQ2_XXS>(a, mode, stream);
 }
 
 // ---- the image: canonical IQ2_XXS superblocks re-packed for the sweeps -------------------------
