@@ -1,4 +1,6 @@
-// Decode-width expert sweeps specialised for IQ2_XXS weights and Q8_K activations on gfx950.
+// Decode-width expert sweeps specialised for IQ2_XXS (and, with the same item list, streams and
+// finishing pass, Q4_K) weights and Q8_K activations on gfx950. The notes below are about
+// IQ2_XXS; what differs for Q4_K rows stands above `Q4kHalf`.
 //
 // Same contract as the generic grouped kernel in moe.hip (src/backend/cuda/moe_kernels.cu:431-582
 // is the reference's counterpart), built around the instruction budget of this one format: at
@@ -14,11 +16,11 @@
 //   * the exact int32 superblock sum (kernel_primitives.h:287-313) is formed in the lane pair
 //     that shares a superblock, scaled to fp32 as ((0.125 d_w) d_a) T, reduced over the 16 lanes
 //     of a row group with three data-parallel-primitive adds (gate on even lanes, up on odd
-//     lanes, or two pairs of the down projection), and parked in LDS; one pass at the end of the
-//     work item adds the row-group partials, applies the SwiGLU and stores coalesced rows.
+//     lanes, or two row groups of the down projection), and parked in LDS; one pass at the end
+//     of the work item adds the row-group partials, applies the SwiGLU and stores coalesced rows.
 //
-// A work item is (bucket, tile of 16 row iterations, sweep). One workgroup per compute unit
-// stays resident and its waves walk the item list with a stride.
+// A work item is (bucket, tile of up to 32 row iterations, sweep). One workgroup per compute
+// unit stays resident and its waves draw items from the workgroup's share of the list.
 //
 // IMAGE: the weights come from the backend's own re-packing of the canonical bytes (built once at
 // residency time, the canonical tensor stays the authority), made for this kernel's instruction
