@@ -560,7 +560,7 @@ def test_execute_rows_hash_router(backend, oracle, streams):
 
 @pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q4_K"])
 def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle, qtype):
-    """Row batches whose buckets average eight pairs or more run the int8 matrix-core kernels
+    """Row batches whose buckets average six pairs or more run the int8 matrix-core kernels
     (routed and shared expert); the result is the CPU layer's, to the same bar."""
     case = MoeCase(backend, oracle, qtype=qtype, hidden=768, intermediate=512, experts=4, topk=2,
                    rows=200, scoring=abi.SCORING_SIGMOID)

@@ -654,12 +654,15 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
         fill_expert_weights(&shared, &views[YVEX_MOE_WEIGHT_SHARED_GATE], &views[YVEX_MOE_WEIGHT_SHARED_UP],
                             &views[YVEX_MOE_WEIGHT_SHARED_DOWN], addresses[3], addresses[4], addresses[5],
                             hidden, layer->shared_intermediate_width, shared_image);
-    /* Row batches whose buckets average eight pairs or more go to the int8 matrix-core kernels
-     * (IQ2_XXS or Q4_K weights, Q8_K activations); below that the decode sweeps, which read an expert's
-     * bytes once per four pairs, are faster. The reference switches its tensor-core kernels on
-     * from 16 input rows (src/backend/cuda/private.h:461-464). Both kernel families read the
-     * sweep image of IQ2_XXS experts as well as canonical bytes. */
-    row_batch = routed_q8 && matrix_core_qtypes(&routed) && pairs >= 8ull * experts;
+    /* Row batches whose buckets average six pairs or more (four with Q4_K gate and up rows) go to
+     * the int8 matrix-core kernels (IQ2_XXS or Q4_K weights, Q8_K activations); below that the decode
+     * sweeps, which read an expert's bytes once per four pairs, are faster: with 256 experts and
+     * top-8 the two families cross at about 170 rows (IQ2_XXS) and 128 rows (Q4_K). The
+     * reference switches its tensor-core kernels on from 16 input rows
+     * (src/backend/cuda/private.h:461-464). Both kernel families read the sweep image of
+     * IQ2_XXS experts as well as canonical bytes. */
+    row_batch = routed_q8 && matrix_core_qtypes(&routed) &&
+                pairs >= (routed.gate_qtype == 12u ? 4ull : 6ull) * experts;
     shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
