@@ -14,10 +14,13 @@
 //   * a sweep serves up to four (row, rank) pairs of a bucket, whose Q8_K columns stay in
 //     registers (128 columns per lane), so an expert's bytes are decoded once for most buckets.
 //   * the exact int32 superblock sum (kernel_primitives.h:287-313) is formed in the lane pair
-//     that shares a superblock, scaled to fp32 as ((0.125 d_w) d_a) T, reduced over the 16 lanes
-//     of a row group with three data-parallel-primitive adds (gate on even lanes, up on odd
-//     lanes, or two row groups of the down projection), and parked in LDS; one pass at the end
-//     of the work item adds the row-group partials, applies the SwiGLU and stores coalesced rows.
+//     that shares a superblock and scaled to fp32 as ((0.125 d_w) d_a) T (gate on even lanes, up
+//     on odd lanes, or two row groups of the down projection): one float term per superblock,
+//     the same float the CPU path forms. Every lane parks its term in an LDS window; when the
+//     window is full a lane per weight row adds that row's terms in double, in superblock
+//     order, and rounds the sum to float once: the row dot is bit for bit the sum the CPU path
+//     computes (double accumulation over the blocks of a row, src/gguf/quant_compute.c:152-172),
+//     so every value that is rounded to bfloat16 afterwards rounds as it does there.
 //
 // A work item is (bucket, tile of up to 32 row iterations, sweep). One workgroup per compute
 // unit stays resident and its waves draw items from the workgroup's share of the list.
@@ -40,7 +43,7 @@ namespace yvex {
 constexpr unsigned kSweepWaves = 8u;           // two per SIMD: the sweep of four pairs needs their registers
 constexpr unsigned kSweepThreads = kSweepWaves * 64u;
 constexpr int kSweepPairs = 4;                 // pairs of one bucket served by one sweep
-constexpr unsigned kSweepIters = 32u;          // weight-row iterations per work item
+constexpr unsigned kSweepIters = 32u;          // weight-row iterations per work item (at most)
 constexpr int kSweepAheadSmall = 1;            // rows requested ahead of the one decoded, sweeps of one or two pairs
 constexpr unsigned kSweepLongPercent = 75u;    // share of the weight rows that goes out in full-length items
 constexpr unsigned kSweepShortDiv = 2u;        // the rest goes out in items of 1 / kSweepShortDiv of that length
@@ -50,8 +53,15 @@ constexpr unsigned kMagBase = 0u;              // 256 entries x 16 replicas x {+
 constexpr unsigned kSelBase = 65536u;          // 128 entries x 32 replicas x {selector lo, hi}
 constexpr unsigned kTicketAddress = kSelBase + 128u * 32u * 8u;   // work-item counter of the workgroup
 constexpr unsigned kParkBase = kTicketAddress + 32u;
-constexpr unsigned kParkBytes = kSweepIters * 4u * 8u * 4u + 256u;   // per wave: 32 bytes per
-                                                                      // (iteration, packed value), then one spare word per lane
+// Per wave: a window of kWindowLines lines of 64 float terms (one line per iteration and packed
+// value: even lanes' terms in the first 32 words, odd lanes' in the last 32, a weight row's
+// terms next to each other in superblock order), then the (gate, up) row sums of a fused item
+// ([stream][pair][row of the item]) for the SwiGLU pass at its end.
+constexpr unsigned kWindowLines = 16u;
+constexpr unsigned kWindowBytes = kWindowLines * 256u;
+constexpr unsigned kFusedItemRows = 32u;       // weight row pairs per fused work item
+constexpr unsigned kResultBytes = 2u * 4u * kFusedItemRows * 4u;
+constexpr unsigned kParkBytes = kWindowBytes + kResultBytes;
 // Sweeps listed by the number of pairs they serve (4, 3, 2, 1): four class sizes, four class
 // starts (cursors while the list is built) and one word per sweep:
 // {whole problem is one bucket : 1, shared expert's problem : 1, bucket : 14, sweep of the bucket : 16}.
@@ -64,7 +74,7 @@ constexpr unsigned kClassListBase = kClassCountBase + 32u + kSweepWaves * 16u;
 // problem has at most kPairCacheMax of them (decode widths; wider batches read them from memory).
 constexpr unsigned kBucketBase = kClassListBase + kClassMaxSweeps * 4u;   // 256 x {expert, first, population}
 constexpr unsigned kPairCacheBase = kBucketBase + 256u * 12u;
-constexpr unsigned kPairCacheMax = 1024u;
+constexpr unsigned kPairCacheMax = 608u;
 constexpr unsigned kSweepLdsBytes = kPairCacheBase + kPairCacheMax * 8u;
 static_assert(kSweepLdsBytes <= 160u * 1024u, "the sweep's tables, lists and caches must fit the LDS of a compute unit");
 
@@ -180,8 +190,11 @@ struct SweepLane {
     unsigned sel_lane;     // kSelBase + (lane % 32) * 8
     unsigned code_shift;   // bytes the codes sit above their aligned load address: 0 or 2
     unsigned scale_shift;  // bits the fp16 scale sits above its aligned load address: 0 or 16
-    unsigned park;         // this wave's parking area
-    unsigned park_write;   // + (lane parity) * 16 + (lane / 16) * 4
+    unsigned park;         // this wave's term window
+    unsigned term_slot;    // the lane's word inside a line of the window (byte offset)
+    unsigned results;      // the wave's row sums of a fused item
+    unsigned terms;        // superblocks of a weight row: the float terms of one row sum
+    unsigned row_shift;    // log2(rows_per_iter)
 };
 
 __device__ __forceinline__ int dot4_from_zero(unsigned a, unsigned b)
@@ -505,11 +518,67 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         request(ring[ahead], (unsigned)ahead);
     }
     __builtin_amdgcn_sched_barrier(0);
-    const bool writer = (lane & 15u) < 2u;
-    unsigned park_at = writer ? g.park_write : g.park + kParkBytes - 256u + lane * 4u;
-    const unsigned park_step = writer ? 32u : 0u;
 
-    for (unsigned it0 = 0; it0 < iterations; it0 += AHEAD + 1) {
+    // ---- the window's row sums: a lane per (line, parity, row of the iteration) adds that
+    // row's float terms in double, in superblock order, and rounds once ----
+    // A fused item keeps the sums for the SwiGLU pass at its end; a plain projection rounds to
+    // bfloat16 and stores here.
+    const unsigned R = g.rows_per_iter;
+    auto flush = [&](unsigned first_iteration, unsigned count) {
+        // LDS operations of one wave complete in order, so the terms parked above are visible here
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const unsigned sums = (count * (unsigned)PV * 2u) << g.row_shift;
+        const unsigned segment_bytes = 128u >> g.row_shift;       // a row's terms of one parity
+        for (unsigned s = lane; s < sums; s += 64u) {
+            const unsigned line = s >> (g.row_shift + 1u), rest = s & (2u * R - 1u);
+            const unsigned parity = rest >> g.row_shift, group = rest & (R - 1u);
+            const unsigned at = g.park + line * 256u + parity * 128u + group * segment_bytes;
+            double sum = 0.0;
+            unsigned k = 0u;
+            for (; k + 4u <= g.terms; k += 4u) {
+                const uint4 t = lds_read_uint4(at + 4u * k);
+                sum += (double)__uint_as_float(t.x);
+                sum += (double)__uint_as_float(t.y);
+                sum += (double)__uint_as_float(t.z);
+                sum += (double)__uint_as_float(t.w);
+            }
+            for (; k < g.terms; ++k) sum += (double)__uint_as_float(lds_load_u32(at + 4u * k));
+            const float row_sum = (float)sum;
+            const unsigned iteration = first_iteration + line / (unsigned)PV, v = line % (unsigned)PV;
+            if constexpr (FUSED) {
+                const unsigned local = (iteration << g.row_shift) + group;      // < kFusedItemRows
+                lds_store_u32(g.results + ((parity * (unsigned)N + v) * kFusedItemRows + local) * 4u,
+                              __float_as_uint(row_sum));
+            } else {
+                // two row groups an iteration: pair v, group `parity`; one: pairs 2v and 2v + 1
+                const unsigned p = TWIN ? v : 2u * v + parity;
+                const unsigned row = row_begin + (TWIN ? ((2u * iteration + parity) << g.row_shift)
+                                                       : (iteration << g.row_shift)) + group;
+                unsigned long long oi = out_index[0];
+#pragma unroll
+                for (int q = 1; q < N; ++q)
+                    if (p == (unsigned)q) oi = out_index[q];
+                const float value = bf16_round(row_sum);
+                if (p < (unsigned)N) {
+                    if (!finite_f32(value)) raise_status(a.status, 1);
+                    else pr.out[oi * a.out_rows + row] = value;
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    // iterations a window holds (a multiple of the turns of one trip through the loop below)
+    constexpr unsigned kWindowIters = (kWindowLines / (unsigned)PV) / (AHEAD + 1) * (AHEAD + 1);
+    static_assert(kWindowIters >= AHEAD + 1, "a window holds at least one trip's lines");
+
+    for (unsigned window_begin = 0; window_begin < iterations; window_begin += kWindowIters) {
+      const unsigned window_end = window_begin + kWindowIters < iterations ? window_begin + kWindowIters : iterations;
+      unsigned park_at = g.park + g.term_slot;
+      for (unsigned it0 = window_begin; it0 < window_end; it0 += AHEAD + 1) {
 #pragma unroll
       for (int turn = 0; turn <= AHEAD; ++turn) {
         const unsigned it = it0 + (unsigned)turn;   // may run past the last row by AHEAD turns
@@ -579,48 +648,37 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             } else {
                 value = weight_scale * packed_scale[v] * (float)t;
             }
-            value = dpp_add<0x4e>(value);     // lanes i and i ^ 2
-            value = dpp_add<0x124>(value);    // + lane i - 4 (row rotate)
-            value = dpp_add<0x128>(value);    // + lanes i - 8, i - 12: all lanes of this parity
+            // every lane parks its term (lanes past the last row group park zeros nobody adds)
             lds_store_u32(park_at, __float_as_uint(value));
-            park_at += park_step;
+            park_at += 256u;
         }
       }
+      }
+      flush(window_begin, window_end - window_begin);
     }
 
-    // ---- finish the item: add the row-group partials, SwiGLU or bf16, coalesced stores ----
-    // LDS operations of one wave complete in order, so the partials above are visible here.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const unsigned groups_per_row = 4u / g.rows_per_iter;   // 16-lane groups a weight row spans
-    const unsigned outputs = rows * (unsigned)N;
-    for (unsigned o = lane; o < outputs; o += 64u) {
-        const unsigned p = o / rows, local = o % rows;      // consecutive lanes: consecutive rows
-        // the iteration, which of its two row groups (MODE 2) and the row inside the group
-        const unsigned it = local / rows_per_turn, within = local % rows_per_turn;
-        const unsigned second_group = MODE == 2 ? within / g.rows_per_iter : 0u, sub = within % g.rows_per_iter;
-        const unsigned v = TWIN ? p : p >> 1, parity = TWIN ? second_group : p & 1u;
-        const unsigned address = g.park + ((it * PV + v) * 2u + parity) * 16u + sub * groups_per_row * 4u;
-        float first = 0.0f, second = 0.0f;
-        for (unsigned k = 0; k < groups_per_row; ++k) {
-            first += __uint_as_float(lds_load_u32(address + 4u * k));
-            if constexpr (FUSED) second += __uint_as_float(lds_load_u32(address + 16u + 4u * k));
-        }
-        float rw = route_weight[0];
-        unsigned long long oi = out_index[0];
+    // ---- finish a fused item: SwiGLU of the (gate, up) row sums, coalesced stores ----
+    if constexpr (FUSED) {
+        const unsigned outputs = rows * (unsigned)N;
+        for (unsigned o = lane; o < outputs; o += 64u) {
+            const unsigned p = o / rows, local = o % rows;      // consecutive lanes: consecutive rows
+            const float first = __uint_as_float(lds_load_u32(g.results + (p * kFusedItemRows + local) * 4u));
+            const float second = __uint_as_float(
+                lds_load_u32(g.results + (((unsigned)N + p) * kFusedItemRows + local) * 4u));
+            float rw = route_weight[0];
+            unsigned long long oi = out_index[0];
 #pragma unroll
-        for (int q = 1; q < N; ++q)
-            if (p == (unsigned)q) {
-                rw = route_weight[q];
-                oi = out_index[q];
-            }
-        const float value = FUSED ? swiglu_bf16_fast(first, second, rw, a.limit, (float)a.limit)
-                                  : bf16_round(first);
-        if (!finite_f32(value)) raise_status(a.status, 1);
-        else pr.out[oi * a.out_rows + row_begin + local] = value;
+            for (int q = 1; q < N; ++q)
+                if (p == (unsigned)q) {
+                    rw = route_weight[q];
+                    oi = out_index[q];
+                }
+            const float value = swiglu_bf16_fast(first, second, rw, a.limit, (float)a.limit);
+            if (!finite_f32(value)) raise_status(a.status, 1);
+            else pr.out[oi * a.out_rows + row_begin + local] = value;
+        }
+        __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
 }
 
 template <int MODE, bool IMAGE, unsigned QT>
@@ -701,13 +759,21 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     g.mag_lane = (lane & 15u) * 16u;
     g.sel_lane = kSelBase + (lane & 31u) * 8u;
     g.park = kParkBase + wave * kParkBytes;
-    g.park_write = g.park + (lane & 1u) * 16u + (lane >> 4) * 4u;
+    g.results = g.park + kWindowBytes;
+    g.terms = g.lanes_per_row / 2u;
+    g.row_shift = g.rows_per_iter == 4u ? 2u : g.rows_per_iter == 2u ? 1u : 0u;
+    {
+        // a line of the window: parity, then the rows of an iteration, then the row's superblocks
+        const unsigned span = 64u >> g.row_shift;                  // lanes of a weight row's slot
+        g.term_slot = ((lane & 1u) * 32u + (lane / span) * (span / 2u) + (lane % span) / 2u) * 4u;
+    }
 
     // The first part of the weight rows is cut into long items (kSweepIters iterations), the rest
     // into short ones that come last in the item list: the waves of the grid finish within a short
     // item of each other instead of a long one, and only the short items pay the fixed cost of an
     // item (its activation columns, the first requests, the finishing pass) more often.
-    const unsigned item_rows = kSweepIters * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
+    // (a fused item keeps its row sums in LDS until its SwiGLU pass: kFusedItemRows rows)
+    const unsigned item_rows = FUSED ? kFusedItemRows : kSweepIters * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
     const unsigned short_rows = item_rows / kSweepShortDiv;
     const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * kSweepLongPercent / 100u / item_rows);
     const unsigned long_rows = long_tiles * item_rows;
