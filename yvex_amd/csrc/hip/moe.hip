@@ -400,7 +400,7 @@ template <unsigned QT, bool Q8, bool FUSED_UP, int N, typename Tables>
 __device__ __forceinline__ void grouped_sweep(
     const GroupedArgs &a, const GroupedProblem &pr, const Tables &tables, const LaneGeometry &g,
     const unsigned char *gate_e, const unsigned char *up_e, unsigned long long first_ordered,
-    unsigned row_begin, unsigned row_end, float *park)
+    unsigned row_begin, unsigned row_end, float *park, float *terms)
 {
     constexpr int kStreams = FUSED_UP ? 2 : 1;
     constexpr int kRows = Q8 ? kRowsInFlight : 1;
@@ -474,6 +474,7 @@ __device__ __forceinline__ void grouped_sweep(
             for (int w = 0; w < kStreams; ++w) {
                 const LaneChunk<QT> &c = chunk[r][w];
                 int whole_dot[N], whole_min[N];
+                int unit_dots[N][UnitTraits<QT>::kIntegerCombine ? 1 : kUnitsPerLane];   // Q8_0: a dot per 32-value block
 #pragma unroll
                 for (int p = 0; p < N; ++p) {
                     whole_dot[p] = whole_min[p] = 0;
@@ -506,7 +507,7 @@ __device__ __forceinline__ void grouped_sweep(
                                     whole_min[p] += unit.min1 * act_bsum[p][2 * k] +
                                                     unit.min2 * act_bsum[p][2 * k + 1];
                             } else {
-                                sums[r][w][p] += c.unit_value(k, act_scale[p], d);
+                                unit_dots[p][k] = d;
                             }
                         } else {
                             const float *x = reinterpret_cast<const float *>(act_row[p]) +
@@ -528,17 +529,67 @@ __device__ __forceinline__ void grouped_sweep(
                         sums[r][w][p] = (g.seg & 1u) ? 0.0f : v;
                     }
                 }
+                if constexpr (Q8 && !UnitTraits<QT>::kIntegerCombine) {
+                    // Q8_0: the term of a Q8_K block is one chain of eight fused multiply-adds over
+                    // its eight 32-value blocks (kernel_primitives.h:342-359). The even lane of the
+                    // pair runs the first four links, the odd lane goes on from there and holds the
+                    // block's term.
+#pragma unroll
+                    for (int p = 0; p < N; ++p) {
+                        float total = 0.0f;
+#pragma unroll
+                        for (int k = 0; k < kUnitsPerLane; ++k)
+                            total = __builtin_fmaf(c.unit_scale(k) * act_scale[p], (float)unit_dots[p][k], total);
+                        float carried = dpp_move_f32<0xa0, 0xf>(total);     // quad_perm [0,0,2,2]: the even neighbour's
+#pragma unroll
+                        for (int k = 0; k < kUnitsPerLane; ++k)
+                            carried = __builtin_fmaf(c.unit_scale(k) * act_scale[p], (float)unit_dots[p][k], carried);
+                        sums[r][w][p] = (g.seg & 1u) ? carried : 0.0f;
+                    }
+                }
             }
         }
         // ---- sum across the lanes of each row, then publish ----
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
+            if constexpr (Q8) {
+                // One float term per superblock sits in a lane of its pair (the even one; Q8_0: the
+                // odd one). The row's first lane adds them in double, in superblock order, and
+                // rounds once: the row dot of the CPU path (src/gguf/quant_compute.c:152-172 adds a
+                // row's blocks in double).
+                const unsigned lane = threadIdx.x & 63u;
+                constexpr unsigned kTermLane = UnitTraits<QT>::kIntegerCombine ? 0u : 1u;
+                const unsigned blocks = a.width >> 8;
 #pragma unroll
-            for (int w = 0; w < kStreams; ++w)
+                for (int w = 0; w < kStreams; ++w)
 #pragma unroll
-                for (int p = 0; p < N; ++p)
-                    sums[r][w][p] = group_sum_f32_dynamic(row_live[r] ? sums[r][w][p] : 0.0f,
-                                                          g.reduce_width);
+                    for (int p = 0; p < N; ++p)
+                        terms[(w * N + p) * 64 + lane] = row_live[r] ? sums[r][w][p] : 0.0f;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                if (row_live[r] && g.seg == 0u) {
+#pragma unroll
+                    for (int w = 0; w < kStreams; ++w)
+#pragma unroll
+                        for (int p = 0; p < N; ++p) {
+                            double sum = 0.0;
+                            for (unsigned k = 0; k < blocks; ++k)
+                                sum += (double)terms[(w * N + p) * 64 + lane + 2u * k + kTermLane];
+                            sums[r][w][p] = (float)sum;
+                        }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            } else {
+#pragma unroll
+                for (int w = 0; w < kStreams; ++w)
+#pragma unroll
+                    for (int p = 0; p < N; ++p)
+                        sums[r][w][p] = group_sum_f32_dynamic(row_live[r] ? sums[r][w][p] : 0.0f,
+                                                              g.reduce_width);
+            }
             if constexpr (FUSED_UP) {
                 // park (gate, up); the SwiGLU runs once per item with every lane busy
                 const unsigned local = row[r] - row_begin;
@@ -610,6 +661,9 @@ __global__ __launch_bounds__(kGroupedThreads) void grouped_kernel(GroupedArgs a)
     }
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     float *park = reinterpret_cast<float *>(after_tables) + wave * (2u * kItemRowsMax * kPass);
+    // per wave: the float terms of an iteration, one word per (stream, pair, lane)
+    float *terms = reinterpret_cast<float *>(after_tables) + kGroupedWaves * (2u * kItemRowsMax * kPass) +
+                   wave * (2u * kPass * 64u);
 
     const unsigned units = a.width >> 5;                          // multiple of 8
     const unsigned lanes_per_row = units / kUnitsPerLane;         // even, <= 64
@@ -679,10 +733,10 @@ __global__ __launch_bounds__(kGroupedThreads) void grouped_kernel(GroupedArgs a)
                                                                           : a.out_rows;
             if (population - pass >= 2ull)
                 grouped_sweep<QT, Q8, FUSED_UP, 2>(a, pr, tables, g, gate_e, up_e, first + pass,
-                                                   row_begin, row_end, park);
+                                                   row_begin, row_end, park, terms);
             else
                 grouped_sweep<QT, Q8, FUSED_UP, 1>(a, pr, tables, g, gate_e, up_e, first + pass,
-                                                   row_begin, row_end, park);
+                                                   row_begin, row_end, park, terms);
         }
     }
 }
@@ -745,7 +799,8 @@ template <unsigned QT, bool Q8, bool FUSED>
 static int launch_grouped_variant(const GroupedArgs &a, hipStream_t stream)
 {
     const size_t lds = (QT == QT_IQ2_XXS ? kIq2WideBytes : 0u) +
-                       (size_t)kGroupedWaves * 2u * kItemRowsMax * kPass * sizeof(float);
+                       (size_t)kGroupedWaves * 2u * kItemRowsMax * kPass * sizeof(float) +
+                       (size_t)kGroupedWaves * 2u * kPass * 64u * sizeof(float);
     YVEX_ALLOW_DYNAMIC_LDS((grouped_kernel<QT, Q8, FUSED>), lds);
     grouped_kernel<QT, Q8, FUSED><<<compute_units(), kGroupedThreads, lds, stream>>>(a);
     return check_launch("moe_grouped");

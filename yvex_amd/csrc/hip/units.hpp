@@ -273,10 +273,7 @@ struct LaneChunk<QT_Q8_0> {
         unit.factor = unit.factor2 = 1;
         unit.min1 = unit.min2 = 0;
     }
-    __device__ __forceinline__ float unit_value(int k, float act_scale, int dot) const
-    {
-        return f16_bits_to_float(d16[k]) * act_scale * (float)dot;
-    }
+    __device__ __forceinline__ float unit_scale(int k) const { return f16_bits_to_float(d16[k]); }
     __device__ __forceinline__ float combine(float, UnitSum) const { return 0.0f; }
 };
 
