@@ -68,12 +68,19 @@ int yvex_hip_concat_rows_bf16(const float *head, const float *tail, uint64_t row
                               yvex_hip_stream stream);
 
 /* yvex_hip_matvec for F32 weight rows and a decode-width batch of F32 input rows (8 to 255: the
- * router projection of the MoE row batch, src/backend/cuda/moe.c:1259-1284), given scratch memory:
- * the row width is split between workgroups so that the whole device takes part, the partial
- * sums go to scratch and a second launch adds them in split order (deterministic). With NULL or
- * too little scratch (yvex_hip_matvec_f32_scratch_bytes, 0 when the shape is not split) it is
- * yvex_hip_matvec. */
+ * router projection of the MoE row batch, src/backend/cuda/moe.c:1259-1284), given scratch memory
+ * (8-byte aligned): the row width is split between workgroups so that the whole device takes
+ * part, the partial sums (doubles) go to scratch and a second launch adds them in split order
+ * (deterministic). With NULL or too little scratch (yvex_hip_matvec_f32_scratch_bytes, 0 when
+ * the shape is not split) or operands that are not 16-byte aligned it is yvex_hip_matvec;
+ * yvex_hip_matvec_f32_rows_launches says which of the two it will be for given operands (2 or 1
+ * kernel launches). Products and sums run in double and the result is rounded to float once, as
+ * the CPU row dot does (src/gguf/quant_compute.c:152-172). */
 uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64_t row_width, uint64_t input_rows);
+unsigned int yvex_hip_matvec_f32_rows_launches(const float *weights, uint64_t row_count, uint64_t row_width,
+                                               const float *input, uint64_t input_rows,
+                                               uint64_t input_stride, const void *scratch,
+                                               uint64_t scratch_bytes);
 int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t row_width,
                              const float *input, uint64_t input_rows, uint64_t input_stride,
                              const float *additive, float *out, uint64_t out_stride, int output_bf16,

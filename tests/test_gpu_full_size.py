@@ -6,8 +6,10 @@ over the whole batch, and the CPU oracle on two of the rows.
   * a row's result does not depend on the batch it arrives in (halves of the batch and a single
     row against the full batch, bit for bit): the sweeps group pairs by expert, four to a sweep,
     so the grouping changes with the batch while every pair's arithmetic must not;
-  * routing equals the oracle's for every row, and eight rows' outputs match the oracle's
-    (src/graph/moe.c:497-622, src/runtime/moe.c:596-645) within the path's tolerance.
+  * routing equals the oracle's for every row, and eight rows' outputs equal the oracle's
+    (src/graph/moe.c:497-622, src/runtime/moe.c:596-645) bit for bit, stage by stage and end to
+    end: the kernels form the same float term per superblock as the CPU path and add a row's
+    terms in double in block order, so every bfloat16 rounding sees the same value.
 """
 import numpy as np
 import pytest
@@ -16,7 +18,6 @@ import torch
 pytestmark = pytest.mark.gpu
 
 HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
-BF16_STEP = 2.0 ** -7
 
 
 def synthetic_iq2xxs(blocks, device, seed):
@@ -37,33 +38,9 @@ def layer_weights(gpu):
     return routed, shared
 
 
-# Measured on MI355X (printed by every run of these tests). Stage by stage, against the oracle fed
-# with the device's own stage input, a value either equals the CPU path's or lies one bf16 step
-# away (the oracle adds a row's 28 superblock terms in double, the kernels in fp32, so the
-# unrounded values differ in their last bits): 1.2e-4 (decode sweeps, 8 rows) and 2.4e-4
-# (matrix-core kernels, 4 rows) of the SwiGLU products, 5.9e-5 and 3.9e-5 of the expert outputs.
-# End to end the fraction beyond 1e-3 relative / 1e-5 absolute depends on the rows looked at: one
-# product that rounds the other way changes its row's Q8_K block and with it, by less than a
-# step, all 7168 outputs of that expert, so a few per cent of them round the other way in turn
-# (decode, 8 rows: 1.7e-5 of the outputs; prefill, 4 rows: 5.1e-2). The stage bounds are two to
-# five times what is measured, the end-to-end ones twice the larger measurement.
-MID_FLIP_BOUND = 6e-4
-OUT_FLIP_BOUND = 1e-4
-DECODE_FLIP_BOUND = 1e-3
-PREFILL_FLIP_BOUND = 1e-1
-
-
-def one_step_or_inside(got, want):
-    """Values that differ are one bf16 step apart, or so small that they lie inside the path's
-    tolerance anyway (sums that cancel to almost nothing)."""
-    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    return bool(np.all((err <= BF16_STEP * 1.001 * np.abs(want)) | (err <= 1e-5 + 1e-3 * np.abs(want))))
-
-
-def stage_flip_rates(oracle, layer, routed, x, picked, label, qt=None):
+def stage_by_stage(oracle, layer, routed, x, picked, label, qt=None):
     """The picked rows' pairs stage by stage: SwiGLU products against the oracle's, expert outputs
-    against the oracle fed with the device's own products. Differences are single bf16 steps;
-    returns their fractions."""
+    against the oracle fed with the device's own products. Every value must equal the CPU path's."""
     qt = oracle.IQ2_XXS if qt is None else qt
     gate, up, down = (t.cpu().numpy() for t in routed)
     gb = oracle.row_bytes(qt, HIDDEN) * INTERMEDIATE
@@ -83,31 +60,27 @@ def stage_flip_rates(oracle, layer, routed, x, picked, label, qt=None):
                                                    down[e * db:(e + 1) * db], HIDDEN, INTERMEDIATE,
                                                    x[row].cpu().numpy(), float(wts[source]), act_q8=True)
             assert rc == 0
-            differs = mid != want_mid
-            assert one_step_or_inside(mid[differs], want_mid[differs])
-            mid_bad += int(differs.sum())
+            mid_bad += int((mid != want_mid).sum())
             mid_all += mid.size
             raw = oracle.q8_matvec(qt, down[e * db:(e + 1) * db], HIDDEN, INTERMEDIATE, oracle.q8k_quantize(mid), 1)[0]
             want_out = np.array([oracle.lib().yvo_bf16_round(np.float32(v)) for v in raw], np.float32)
             got_out = layer.pair_outputs[source].cpu().numpy()
-            differs = got_out != want_out
-            assert one_step_or_inside(got_out[differs], want_out[differs])
-            out_bad += int(differs.sum())
+            out_bad += int((got_out != want_out).sum())
             out_all += got_out.size
-    print(f"{label}: {mid_bad} of {mid_all} SwiGLU products ({mid_bad / mid_all:.3e}) and {out_bad} of {out_all} "
-          f"expert outputs ({out_bad / out_all:.3e}) one bf16 step from the oracle's")
-    return mid_bad / mid_all, out_bad / out_all
+    print(f"{label}: {mid_bad} of {mid_all} SwiGLU products and {out_bad} of {out_all} expert outputs "
+          f"differ from the oracle's")
+    assert mid_bad == 0 and out_bad == 0
 
 
-def within_tolerance(got, want, bound, label):
-    """1e-3 relative / 1e-5 absolute; beyond it only values one bf16 step apart (a sum that sits
-    on a rounding boundary), and no more of them than `bound`. The measured fraction is printed."""
+def equal_to_oracle(got, want, label):
+    """North star: final fp32 outputs within 1e-3 relative / 1e-5 absolute of the CPU path; the
+    kernels are held to more, every output the CPU path's bit for bit."""
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     outside = err > 1e-5 + 1e-3 * np.abs(want)
-    print(f"{label}: {int(outside.sum())} of {outside.size} outputs beyond 1e-3 / 1e-5 "
-          f"(fraction {outside.mean():.3e}), bit-identical {np.mean(got == want):.4f}")
-    assert outside.mean() < bound
-    assert np.all(err[outside] <= BF16_STEP * 1.001 * np.abs(want[outside]))
+    print(f"{label}: {int(outside.sum())} of {outside.size} outputs beyond 1e-3 / 1e-5, "
+          f"bit-identical {np.mean(got == want):.6f}")
+    assert np.all(err <= 1e-5 + 1e-3 * np.abs(want))
+    assert np.array_equal(got, want)
 
 
 def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
@@ -144,7 +117,7 @@ def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
         rc, want_selected, want_weights, _ = oracle.moe_route(host_logits[r], None, TOPK, oracle.SIGMOID, True, 1.0)
         assert rc == 0
         assert np.array_equal(selected[r].cpu().numpy().astype(np.uint64), want_selected)
-        assert np.max(np.abs(weights[r].cpu().numpy() - want_weights)) <= 1e-6
+        assert np.array_equal(weights[r].cpu().numpy(), want_weights)
 
     # eight rows through the CPU oracle with the same weights
     picked = [0, 4, 9, 13, 17, 22, 26, 31]
@@ -155,10 +128,9 @@ def test_decode_layer_at_full_size(gpu, oracle, layer_weights):
                             limit=10.0, act_q8=True, threads=16)
     got = full[picked].cpu().numpy()
     assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
-    within_tolerance(got, want["combined"], DECODE_FLIP_BOUND, "decode layer, 8 rows against the oracle")
+    equal_to_oracle(got, want["combined"], "decode layer, 8 rows against the oracle")
     full_again, _, _ = run(0, ROWS)     # leaves the whole batch's stage buffers in place
-    mid_rate, out_rate = stage_flip_rates(oracle, layer, routed, x, picked, "decode layer, 8 rows stage by stage")
-    assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
+    stage_by_stage(oracle, layer, routed, x, picked, "decode layer, 8 rows stage by stage")
 
 
 def synthetic_q4k(blocks, device, seed):
@@ -176,8 +148,9 @@ def synthetic_q4k(blocks, device, seed):
 def test_prefill_layer_at_full_size(gpu, oracle, layer_weights, qtype):
     """2048 rows whose experts follow a Zipf(1.1) popularity (buckets from a handful of pairs to
     more than a thousand) through the matrix-core kernels, with IQ2_XXS and with Q4_K experts: the
-    same bits twice, the first 32 rows against the decode sweeps' result for them (another
-    summation order: within tolerance), four rows against the oracle."""
+    same bits twice, the first 32 rows against the decode sweeps' result for them (bit for bit:
+    both add a row's terms as the CPU path does), four rows against the oracle, stage by stage
+    and end to end, for equality."""
     from yvex_amd import kernels as K
     from yvex_amd.moe import MoeLayer
     if qtype == "IQ2_XXS":
@@ -207,9 +180,8 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights, qtype):
     assert torch.isfinite(first).all()
     selected = wide.selected.clone()
     picked = [5, 700, 1000, 1900]
-    mid_rate, out_rate = stage_flip_rates(oracle, wide, routed, x, picked,
-                                          f"prefill layer ({qtype}), 4 rows stage by stage", getattr(oracle, qtype))
-    assert mid_rate < MID_FLIP_BOUND and out_rate < OUT_FLIP_BOUND
+    stage_by_stage(oracle, wide, routed, x, picked, f"prefill layer ({qtype}), 4 rows stage by stage",
+                   getattr(oracle, qtype))
     keep = list(range(32)) + picked
     populations = torch.bincount(selected.reshape(-1).long(), minlength=EXPERTS).cpu().numpy()
     assert populations.max() > 1000 and (populations[populations > 0] < 32).any()
@@ -219,38 +191,20 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights, qtype):
     wide_shared = wide.shared_out[keep].cpu().numpy()
     del wide
 
-    def close_by_row(got, want, scale, bound=2e-2, label=None):
-        """Few values beyond the path's tolerance (1e-3 relative / 1e-5 absolute), and those by no
-        more than two bf16 steps at the size of the row's largest terms: an intermediate value
-        that rounds the other way (the SwiGLU product, an expert's output) moves the results it
-        feeds by a step at its own size, whatever their own size is."""
-        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-        outside = err > 1e-5 + 1e-3 * np.abs(want)
-        if label:
-            print(f"{label}: {int(outside.sum())} of {outside.size} outputs beyond 1e-3 / 1e-5 "
-                  f"(fraction {outside.mean():.3e}), bit-identical {np.mean(got == want):.4f}")
-        assert outside.mean() < bound
-        assert np.all(err <= 1e-5 + 1e-3 * np.abs(want) + 2 * BF16_STEP * scale)
-
-    def combined_close(got, want, pairs, shared_rows, bound=2e-2, label=None):
-        scale = np.abs(pairs).max(axis=2).sum(axis=1) + np.abs(shared_rows).max(axis=1)   # per row
-        close_by_row(got, want, scale[:, None], bound, label)
-
     narrow = MoeLayer(max_rows=32, **common)
     sweeps = narrow.run(x[:32].contiguous(), logits[:32].contiguous())[:32].clone()
     torch.cuda.synchronize()
     assert int(narrow.status.item()) == 0 and torch.equal(narrow.selected, selected[:32])
-    # expert by expert
+    # expert by expert, then the combined rows: the two kernel families agree bit for bit
     mine = wide_pairs[:32].reshape(32 * TOPK, HIDDEN)
-    close_by_row(mine, narrow.pair_outputs[:32 * TOPK].cpu().numpy(), np.abs(mine).max(axis=1)[:, None])
-    close_by_row(wide_shared[:32], narrow.shared_out[:32].cpu().numpy(),
-                 np.abs(wide_shared[:32]).max(axis=1)[:, None])
-    combined_close(first[:32].cpu().numpy(), sweeps.cpu().numpy(), wide_pairs[:32], wide_shared[:32])
+    assert np.array_equal(mine, narrow.pair_outputs[:32 * TOPK].cpu().numpy())
+    assert np.array_equal(wide_shared[:32], narrow.shared_out[:32].cpu().numpy())
+    assert np.array_equal(first[:32].cpu().numpy(), sweeps.cpu().numpy())
     want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
                             qtypes=(getattr(oracle, qtype),) * 3, routed=[t.cpu().numpy() for t in routed],
                             shared=[t.cpu().numpy() for t in shared], inputs=x[picked].cpu().numpy(),
                             logits=logits[picked].cpu().numpy(), scoring=oracle.SIGMOID, normalize=True,
                             scaling=1.0, limit=10.0, act_q8=True, threads=16)
     assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
-    combined_close(first[picked].cpu().numpy(), want["combined"], wide_pairs[32:], wide_shared[32:],
-                   PREFILL_FLIP_BOUND, f"prefill layer ({qtype}), 4 rows against the oracle")
+    equal_to_oracle(first[picked].cpu().numpy(), want["combined"],
+                    f"prefill layer ({qtype}), 4 rows against the oracle")

@@ -101,9 +101,11 @@ def test_moe_layer_stagewise(gpu, oracle, qtype, hidden, intermediate, experts, 
     gb = oracle.row_bytes(qt, hidden) * intermediate
     db = oracle.row_bytes(qt, intermediate) * hidden
 
-    # Q8_K activations through the sweeps: every row sum is the CPU path's bit for bit (same float
-    # term per superblock, added in double in block order), so every stage is compared for equality
-    exact = act_q8 and not matrix_cores
+    # Decode sweeps and matrix-core kernels alike: every row sum is the CPU path's (Q8_K
+    # activations: the same float term per superblock, added in double in block order; F32
+    # activations: the decoder's float weights, products and sums in double), so every stage is
+    # compared for equality
+    exact = True
 
     # routing: identical selection and weights (scores and normalisation run in double on both sides)
     for r in range(rows):

@@ -24,7 +24,7 @@ struct MatvecArgs {
     unsigned long long out_stride;
     int output_bf16;
     int *status;
-    float *parts;            // split projections: [split][input row][weight row] partial sums
+    double *parts;           // split projections: [split][input row][weight row] partial sums
 };
 
 __device__ __forceinline__ void matvec_publish(const MatvecArgs &a, unsigned long long in,
@@ -145,7 +145,11 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     }
 }
 
-// F32 / F16 / BF16 weight rows: lanes stride the row element-wise.
+// F32 / F16 / BF16 weight rows: lanes stride the row element-wise. Products and sums run in
+// double, as the CPU row dot forms them (src/gguf/quant_compute.c:152-172: double(value) *
+// double(x) added in double, rounded to float once); the product of two floats is exact in
+// double, so only the order of the double additions differs from the serial loop, far below
+// what the final rounding to float keeps.
 template <int T>
 __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsigned qtype)
 {
@@ -154,9 +158,9 @@ __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsign
     const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
     if (row >= a.row_count) return;
     const unsigned char *wrow = a.encoded + row * a.row_bytes;
-    float acc[T];
+    double acc[T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    for (int t = 0; t < T; ++t) acc[t] = 0.0;
     for (unsigned long long i = lane; i < a.row_width; i += 64u) {
         const float w = qtype_value(wrow, i, qtype);
         if (!finite_f32(w)) raise_status(a.status, 1);
@@ -164,141 +168,48 @@ __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsign
         for (int t = 0; t < T; ++t) {
             unsigned long long in = in0 + t;
             if (in >= a.input_rows) in = a.input_rows - 1ull;
-            acc[t] = fmaf(w, ((const float *)a.input)[in * a.input_stride + i], acc[t]);
+            acc[t] += (double)w * (double)((const float *)a.input)[in * a.input_stride + i];
         }
     }
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-        float sum = group_sum_f32<64>(acc[t]);
+        double sum = acc[t];
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, kWave);
         const unsigned long long in = in0 + t;
         if (in >= a.input_rows) continue;
-        if (!finite_f32(sum) && *a.status == 0)
-            sum = matvec_recover_f64(wrow, (const float *)a.input + in * a.input_stride,
-                                     a.row_width, qtype);
-        if (lane == 0u) matvec_publish(a, in, row, sum);
+        if (lane == 0u) matvec_publish(a, in, row, (float)sum);
     }
 }
 
-__device__ __noinline__ float f32_dot_f64(const float *w, const float *x, unsigned long long width)
-{
-    double exact = 0.0;
-    for (unsigned long long k = 0; k < width; ++k) exact += (double)w[k] * (double)x[k];
-    return (float)exact;
-}
-
-// F32 weight rows against a batch of F32 input rows (a router or mixing projection over a
-// prefill-width batch): a workgroup owns 32 weight rows x 32 input rows on the fp32 matrix cores.
-// Its four waves split the row width into quarters; lane (r, h) of a wave loads four consecutive
-// floats of weight row r and of input row r at offset 8j + 4h, which feed four
-// V_MFMA_F32_32X32X2_F32 (any assignment of k to instructions is valid as long as both operands
-// use the same one). The partial tiles are added in wave order, so the sum is deterministic.
-// Products are exact fp32 products; only the order of the fp32 additions differs from the
-// lane-strided kernel above.
-__global__ __launch_bounds__(256) void matvec_f32_tile_kernel(MatvecArgs a)
-{
-    typedef float v16f __attribute__((ext_vector_type(16)));
-    __shared__ float partial[3][16][64];
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned r = lane & 31u, h = lane >> 5;
-    unsigned long long wrow = (unsigned long long)blockIdx.x * 32ull + r;
-    unsigned long long in = (unsigned long long)blockIdx.y * 32ull + r;
-    if (wrow >= a.row_count) wrow = a.row_count - 1ull;      // a ragged edge repeats the last row
-    if (in >= a.input_rows) in = a.input_rows - 1ull;
-    const float *wp = (const float *)(a.encoded + wrow * a.row_bytes);
-    const float *xp = (const float *)a.input + in * a.input_stride;
-    const unsigned long long quarter = a.row_width / 4ull;   // a multiple of 8
-    const unsigned long long begin = wave * quarter + 4u * h;
-    v16f acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-    unsigned bad = 0u;
-    const unsigned steps = (unsigned)(quarter / 8ull);
-    wp += begin;
-    xp += begin;
-    // four steps of loads stay in flight ahead of the matrix instructions that use them
-    const unsigned groups = (steps + 3u) / 4u;
-    float4 w[4], x[4];
-#pragma unroll
-    for (unsigned j = 0; j < 4u; ++j) {
-        const unsigned at = 8u * (j < steps ? j : steps - 1u);
-        w[j] = *reinterpret_cast<const float4 *>(wp + at);
-        x[j] = *reinterpret_cast<const float4 *>(xp + at);
-    }
-    for (unsigned group = 0; group < groups; ++group) {
-        float4 wn[4], xn[4];
-        if (group + 1u < groups) {
-#pragma unroll
-            for (unsigned j = 0; j < 4u; ++j) {
-                const unsigned step = 4u * (group + 1u) + j;
-                const unsigned at = 8u * (step < steps ? step : steps - 1u);
-                wn[j] = *reinterpret_cast<const float4 *>(wp + at);
-                xn[j] = *reinterpret_cast<const float4 *>(xp + at);
-            }
-        }
-#pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
-            if (4u * group + j >= steps) break;
-            bad |= (unsigned)!finite_f32(w[j].x) | (unsigned)!finite_f32(w[j].y) |
-                   (unsigned)!finite_f32(w[j].z) | (unsigned)!finite_f32(w[j].w);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].x, x[j].x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].y, x[j].y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].z, x[j].z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].w, x[j].w, acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
-            w[j] = wn[j];
-            x[j] = xn[j];
-        }
-    }
-    if (bad) raise_status(a.status, 1);
-    if (wave) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) partial[wave - 1u][i][lane] = acc[i];
-    }
-    __syncthreads();
-    if (wave) return;
-    const unsigned long long out_in = (unsigned long long)blockIdx.y * 32ull + r;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        // accumulator i of lane (r, h): weight row 8 (i / 4) + 4 h + i % 4, input row r
-        const unsigned long long row = (unsigned long long)blockIdx.x * 32ull + 8u * (i >> 2) + 4u * h + (i & 3);
-        float sum = ((acc[i] + partial[0][i][lane]) + partial[1][i][lane]) + partial[2][i][lane];
-        if (row >= a.row_count || out_in >= a.input_rows) continue;
-        if (!finite_f32(sum) && *a.status == 0) {
-            // kernels.cu:616-620: an overflow before opposite terms cancelled is redone in double
-            sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
-                              (const float *)a.input + out_in * a.input_stride, a.row_width);
-        }
-        matvec_publish(a, out_in, row, sum);
-    }
-}
-
-// The same projection for a decode-width batch (8 to 255 input rows, e.g. the router over 32
-// rows): too few 32 x 32 tiles would leave most compute units idle, so a workgroup of sixteen
-// waves owns 16 weight rows x 16 input rows on V_MFMA_F32_16X16X4_F32 and its waves split the
-// row width sixteen ways. Lane (i, q) loads four consecutive floats of weight row i and of input
-// row i at offset 16 j + 4 q; partial tiles are added in wave order.
+// F32 weight rows against a batch of F32 input rows (a router or mixing projection over a row
+// batch) on the double-precision matrix cores: a workgroup of WAVES waves owns 16 weight rows x
+// 16 input rows on V_MFMA_F64_16X16X4_F64 and its waves split the row width. Lane (i, q) loads
+// four consecutive floats of weight row i and of input row i at offset 16 j + 4 q. A product of
+// two floats is exact in double and the sums run in double, which is how the CPU row dot forms
+// them (src/gguf/quant_compute.c:152-172); only the order of the double additions differs from
+// its serial loop, so the float the sum rounds to is the CPU path's. The partial tiles of the
+// waves (and of the workgroups that split the width: blockIdx.z, joined by a second launch in
+// split order) are doubles, added in a fixed order.
 template <unsigned WAVES>
 __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArgs a)
 {
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    __shared__ float partial[WAVES - 1u][4][64];
+    typedef double v4d __attribute__((ext_vector_type(4)));
+    __shared__ double partial[WAVES - 1u][4][64];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned i16 = lane & 15u, q = lane >> 4;
     unsigned long long wrow = (unsigned long long)blockIdx.x * 16ull + i16;
     unsigned long long in = (unsigned long long)blockIdx.y * 16ull + i16;
-    if (wrow >= a.row_count) wrow = a.row_count - 1ull;
+    if (wrow >= a.row_count) wrow = a.row_count - 1ull;      // a ragged edge repeats the last row
     if (in >= a.input_rows) in = a.input_rows - 1ull;
-    // blockIdx.z splits the row width between workgroups (their sums go to a.parts and a second
-    // launch adds them in split order); the waves of a workgroup split its share again
     const unsigned long long share = a.row_width / ((unsigned long long)gridDim.z * WAVES);   // a multiple of 16
     const unsigned long long begin = ((unsigned long long)blockIdx.z * WAVES + wave) * share + 4u * q;
     const float *wp = (const float *)(a.encoded + wrow * a.row_bytes) + begin;
     const float *xp = (const float *)a.input + in * a.input_stride + begin;
     const unsigned steps = (unsigned)(share / 16ull);
-    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    v4d acc = {0.0, 0.0, 0.0, 0.0};
     unsigned bad = 0u;
+    // four steps of loads stay in flight ahead of the matrix instructions that use them
     const unsigned groups = (steps + 3u) / 4u;
     float4 w[4], x[4];
 #pragma unroll
@@ -323,10 +234,10 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
             if (4u * group + j >= steps) break;
             bad |= (unsigned)!finite_f32(w[j].x) | (unsigned)!finite_f32(w[j].y) |
                    (unsigned)!finite_f32(w[j].z) | (unsigned)!finite_f32(w[j].w);
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].x, x[j].x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].y, x[j].y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].z, x[j].z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j].w, x[j].w, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[j].x, (double)x[j].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[j].y, (double)x[j].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[j].z, (double)x[j].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[j].w, (double)x[j].w, acc, 0, 0, 0);
         }
 #pragma unroll
         for (unsigned j = 0; j < 4u; ++j) {
@@ -344,9 +255,9 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
     const unsigned long long out_in = (unsigned long long)blockIdx.y * 16ull + i16;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        // accumulator k of lane (i, q): weight row 4 q + k, input row i
-        const unsigned long long row = (unsigned long long)blockIdx.x * 16ull + 4u * q + k;
-        float sum = acc[k];
+        // accumulator k of lane (i, q): weight row 4 k + q, input row i
+        const unsigned long long row = (unsigned long long)blockIdx.x * 16ull + 4u * k + q;
+        double sum = acc[k];
 #pragma unroll
         for (unsigned wv = 0; wv + 1u < WAVES; ++wv) sum += partial[wv][k][lane];
         if (row >= a.row_count || out_in >= a.input_rows) continue;
@@ -354,10 +265,7 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
             a.parts[((unsigned long long)blockIdx.z * a.input_rows + out_in) * a.row_count + row] = sum;
             continue;
         }
-        if (!finite_f32(sum) && *a.status == 0)
-            sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
-                              (const float *)a.input + out_in * a.input_stride, a.row_width);
-        matvec_publish(a, out_in, row, sum);
+        matvec_publish(a, out_in, row, (float)sum);
     }
 }
 
@@ -368,12 +276,9 @@ __global__ __launch_bounds__(256) void matvec_f32_join_kernel(MatvecArgs a, unsi
     const unsigned long long at = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
     if (at >= outputs) return;
     const unsigned long long in = at / a.row_count, row = at % a.row_count;
-    float sum = a.parts[at];
+    double sum = a.parts[at];
     for (unsigned z = 1; z < splits; ++z) sum += a.parts[z * outputs + at];
-    if (!finite_f32(sum) && *a.status == 0)
-        sum = f32_dot_f64((const float *)(a.encoded + row * a.row_bytes),
-                          (const float *)a.input + in * a.input_stride, a.row_width);
-    matvec_publish(a, in, row, sum);
+    matvec_publish(a, in, row, (float)sum);
 }
 
 // int32 block sums of the Q8_K path, produced by the same unit code the matvec runs.
@@ -532,19 +437,18 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (qtype == QT_Q4_K && input_q8 && input_rows >= 2ull && !((uintptr_t)encoded & 15u))
         return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
                                      out, out_stride, output_bf16 != 0, status, s);
-    if (qtype == QT_F32 && input_rows >= 8ull && input_rows < 256ull && row_width % 256ull == 0ull &&
-        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
+    // F32 rows against a batch of F32 input rows: 16 x 16 tiles on the double-precision matrix
+    // cores; a small batch offers few tiles, so sixteen waves split the row width, a large one
+    // has tiles enough for four
+    if (qtype == QT_F32 && input_rows >= 8ull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) &&
+        !(input_stride & 3ull) && row_width % (input_rows < 256ull ? 256ull : 64ull) == 0ull) {
         const unsigned long long grid_x = (row_count + 15ull) / 16ull, grid_y = (input_rows + 15ull) / 16ull;
-        if (grid_x > 0x7fffffffull) return ST_BOUNDS;
-        matvec_f32_tile16_kernel<16><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
-        return check_launch("matvec_f32_tile16");
-    }
-    if (qtype == QT_F32 && input_rows >= 32ull && row_width % 32ull == 0ull &&
-        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull)) {
-        const unsigned long long grid_x = (row_count + 31ull) / 32ull, grid_y = (input_rows + 31ull) / 32ull;
         if (grid_x > 0x7fffffffull || grid_y > 65535ull) return ST_BOUNDS;
-        matvec_f32_tile_kernel<<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
-        return check_launch("matvec_f32_tile");
+        if (input_rows < 256ull)
+            matvec_f32_tile16_kernel<16><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
+        else
+            matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
+        return check_launch("matvec_f32_tile16");
     }
     if (scalar) {
         const unsigned long long grid_x = (row_count + 3ull) / 4ull;
@@ -645,7 +549,28 @@ extern "C" uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64
                                                       uint64_t input_rows)
 {
     const unsigned splits = f32_rows_splits(row_width, input_rows);
-    return splits ? (uint64_t)splits * input_rows * row_count * sizeof(float) : 0u;
+    return splits ? (uint64_t)splits * input_rows * row_count * sizeof(double) : 0u;
+}
+
+// Whether the projection runs as partial tiles plus a join (two launches) or as one launch.
+static bool f32_rows_split_applies(const float *weights, uint64_t row_count, uint64_t row_width,
+                                   const float *input, uint64_t input_rows, uint64_t input_stride,
+                                   const void *scratch, uint64_t scratch_bytes)
+{
+    const unsigned splits = f32_rows_splits(row_width, input_rows);
+    const uint64_t need = yvex_hip_matvec_f32_scratch_bytes(row_count, row_width, input_rows);
+    return splits && scratch && scratch_bytes >= need && !((uintptr_t)scratch & 7u) &&
+           !(((uintptr_t)weights | (uintptr_t)input) & 15u) && !(input_stride & 3ull) && weights && input &&
+           row_count && input_stride >= row_width;
+}
+
+extern "C" unsigned int yvex_hip_matvec_f32_rows_launches(const float *weights, uint64_t row_count,
+                                                          uint64_t row_width, const float *input,
+                                                          uint64_t input_rows, uint64_t input_stride,
+                                                          const void *scratch, uint64_t scratch_bytes)
+{
+    return f32_rows_split_applies(weights, row_count, row_width, input, input_rows, input_stride, scratch,
+                                  scratch_bytes) ? 2u : 1u;
 }
 
 extern "C" int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t row_width,
@@ -654,16 +579,14 @@ extern "C" int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count
                                         int output_bf16, void *scratch, uint64_t scratch_bytes,
                                         int *status, yvex_hip_stream stream)
 {
-    const unsigned splits = f32_rows_splits(row_width, input_rows);
-    const uint64_t need = yvex_hip_matvec_f32_scratch_bytes(row_count, row_width, input_rows);
-    if (!splits || !scratch || scratch_bytes < need || ((uintptr_t)scratch & 3u) ||
-        (((uintptr_t)weights | (uintptr_t)input) & 15u) || (input_stride & 3ull) || !weights || !input ||
-        !out || !status || !row_count || out_stride < row_count || input_stride < row_width)
+    if (!f32_rows_split_applies(weights, row_count, row_width, input, input_rows, input_stride, scratch,
+                                scratch_bytes) || !out || !status || out_stride < row_count)
         return yvex_hip_matvec((const uint8_t *)weights, QT_F32, row_count, row_width, row_width * 4u, input, 0,
                                input_rows, input_stride, additive, out, out_stride, output_bf16, status,
                                stream);
+    const unsigned splits = f32_rows_splits(row_width, input_rows);
     MatvecArgs a{(const unsigned char *)weights, row_count, row_width, row_width * 4u, input, input_rows,
-                 input_stride, additive, out, out_stride, output_bf16, status, (float *)scratch};
+                 input_stride, additive, out, out_stride, output_bf16, status, (double *)scratch};
     hipStream_t s = as_stream(stream);
     const uint64_t grid_x = (row_count + 15u) / 16u, grid_y = (input_rows + 15u) / 16u;
     const uint64_t outputs = input_rows * row_count;

@@ -464,6 +464,7 @@ __device__ __forceinline__ void grouped_sweep(
         if (base + stride < row_end) request(base + stride);
 
         float sums[kRows][kStreams][N];
+        double wide[Q8 ? 1 : kRows][Q8 ? 1 : kStreams][Q8 ? 1 : N];   // F32 activations: the lane's sums in double
         unsigned row[kRows];
         bool row_live[kRows];
 #pragma unroll
@@ -479,6 +480,7 @@ __device__ __forceinline__ void grouped_sweep(
                 for (int p = 0; p < N; ++p) {
                     whole_dot[p] = whole_min[p] = 0;
                     sums[r][w][p] = 0.0f;
+                    if constexpr (!Q8) wide[r][w][p] = 0.0;
                 }
 #pragma unroll
                 for (int k = 0; k < kUnitsPerLane; ++k) {
@@ -512,7 +514,7 @@ __device__ __forceinline__ void grouped_sweep(
                         } else {
                             const float *x = reinterpret_cast<const float *>(act_row[p]) +
                                              32ull * (g.unit0 + k);
-                            sums[r][w][p] += chunk_unit_dot_f32<QT>(c, k, unit, x);
+                            wide[r][w][p] = chunk_unit_dot_f64<QT>(c, k, unit, x, wide[r][w][p]);
                         }
                     }
                 }
@@ -583,12 +585,17 @@ __device__ __forceinline__ void grouped_sweep(
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             } else {
+                // F32 activations: the lanes' double sums added in double, rounded once
+                // (the CPU row dot: src/gguf/quant_compute.c:152-172)
 #pragma unroll
                 for (int w = 0; w < kStreams; ++w)
 #pragma unroll
-                    for (int p = 0; p < N; ++p)
-                        sums[r][w][p] = group_sum_f32_dynamic(row_live[r] ? sums[r][w][p] : 0.0f,
-                                                              g.reduce_width);
+                    for (int p = 0; p < N; ++p) {
+                        double sum = row_live[r] ? wide[r][w][p] : 0.0;
+                        for (unsigned offset = g.reduce_width >> 1; offset; offset >>= 1)
+                            sum += __shfl_xor(sum, (int)offset, kWave);
+                        sums[r][w][p] = (float)sum;
+                    }
             }
             if constexpr (FUSED_UP) {
                 // park (gate, up); the SwiGLU runs once per item with every lane busy

@@ -6,7 +6,7 @@
 // with V_MFMA_I32_32X32X32_I8. A wave cannot run vector instructions under its own matrix
 // instruction, the other wave of its SIMD can, so two waves a SIMD is the shape that lets decode
 // and scaling arithmetic overlap the matrix pipe, and 256 registers a wave is what decides the
-// tile: 32 rows x 64 tokens of int32 limb sums and fp32 sums.
+// tile: 32 rows x 64 tokens of int32 limb sums and double-precision row sums.
 //
 //   A operand (weights): built in registers, one K chunk (32 columns) ahead of its use. Lane
 //       (r, h) = (lane % 32, lane / 32) owns weight row r and the groups 4h .. 4h + 3 of the
@@ -31,8 +31,11 @@
 //       bank groups.
 //   C: per (superblock, 32-token block) two int32 accumulators of 32 x 32; T = 128 * C_hi + C_lo
 //       is the exact integer superblock sum of the reference's primitive
-//       (src/backend/cuda/kernel_primitives.h:287-313), scaled into fp32 as
-//       ((0.125 * d_w) * d_a) * T and summed over superblocks.
+//       (src/backend/cuda/kernel_primitives.h:287-313), scaled into the float term
+//       ((0.125 * d_w) * d_a) * T; a row's terms are added in double, in superblock order, and
+//       the sum is rounded to float once, which is what the CPU path computes for a row (double
+//       accumulation over a row's blocks, src/gguf/quant_compute.c:152-172): every value
+//       rounded to bfloat16 afterwards rounds as it does there.
 //   Output: accumulator i of lane (r, h) is token r's sum for row 8 (i / 4) + 4 h + i % 4 of the
 //       wave's 32 (gate sums in the first eight, the matching up sums in the last eight when
 //       fused), so a lane stores four consecutive rows of its token, 16 bytes, straight from its
@@ -165,7 +168,7 @@ struct MfmaNextItem {
 // of operand registers in all. Between the matrix instructions the slot carries the LDS reads of
 // the activation fragments two slots ahead, the table lookups of the chunk two slots ahead,
 // the selector words and permutes of the next chunk, and its share of the copies. After the
-// last chunk the integer sums of the superblock are scaled into the fp32 accumulators. Two waves
+// last chunk the integer sums of the superblock are scaled and added to the row sums. Two waves
 // share a SIMD: while one waits for its own matrix instructions or scales its sums the other's
 // instructions run.
 //
@@ -450,11 +453,11 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
     build(0u);
     __syncthreads();   // every wave's share of stage 0 has landed
 
-    float acc[NTB][16];
+    double acc[NTB][16];            // row sums: float terms added in double, in superblock order
 #pragma unroll
     for (unsigned tb = 0; tb < NTB; ++tb)
 #pragma unroll
-        for (unsigned i = 0; i < 16u; ++i) acc[tb][i] = 0.0f;
+        for (unsigned i = 0; i < 16u; ++i) acc[tb][i] = 0.0;
     v16i sum_lo[NTB], sum_hi[NTB];   // integer sums of the running superblock
     v4i frag[2][NTB];                // [slot & 1]: re-requested for two slots on as soon as it is used
 #pragma unroll
@@ -572,7 +575,8 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
 #pragma unroll
                     for (unsigned i = 0; i < 16u; ++i) {
                         const int total = (sum_hi[tb][i] << 7) + sum_lo[tb][i];
-                        acc[tb][i] = __builtin_fmaf(rs[i] * ts[tb], (float)total, acc[tb][i]);
+                        const float term = rs[i] * ts[tb] * (float)total;    // each product rounded to float
+                        acc[tb][i] += (double)term;
                     }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -603,12 +607,12 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
                 const float route_weight = __uint_as_float(info.y);
 #pragma unroll
                 for (unsigned j = 0; j < 4u; ++j)
-                    value[j] = swiglu_bf16_fast(acc[tb][4u * q + j], acc[tb][4u * (q + 2u) + j], route_weight,
+                    value[j] = swiglu_bf16_fast((float)acc[tb][4u * q + j], (float)acc[tb][4u * (q + 2u) + j], route_weight,
                                                 a.limit, limit_f32);
             } else {
 #pragma unroll
                 for (unsigned j = 0; j < 4u; ++j) {
-                    value[j] = acc[tb][4u * q + j];
+                    value[j] = (float)acc[tb][4u * q + j];
                     good &= finite_f32(value[j]);
                     if (!a.plain_output) value[j] = bf16_round_number(value[j]);   // (a NaN has just been noted)
                 }

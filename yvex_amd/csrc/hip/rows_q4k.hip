@@ -7,7 +7,9 @@
 // sub-block, the int32 accumulators run over the whole superblock, the minimum term is one more
 // K step of depth 8, and
 //     value = (d_a * d) * float(dot) - (d_a * dmin) * float(minimum)
-// is added to the fp32 accumulators superblock by superblock, in superblock order.
+// (a float, every operation rounded) is added to the row sums in double, superblock by
+// superblock, and a sum is rounded to float once when it is published: the row dot the CPU path
+// forms (double accumulation over a row's blocks, src/gguf/quant_compute.c:152-172).
 //
 // What differs is how the operands arrive. A lane that fetches its own 16-byte pieces of a
 // 144-byte weight block and of a 292-byte activation block touches up to 64 cache lines per load
@@ -183,11 +185,11 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
                                                 : kQ4BsumBase + buffer * kQ4Tokens * 32u + 1024u * (wave - 1u))));
     };
 
-    float acc[NT][16];
+    double acc[NT][16];      // row sums: a float term per superblock, added in double in superblock order
 #pragma unroll
     for (unsigned nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0;
 
     __syncthreads();      // the previous tile's reads (none in this kernel: one tile a workgroup) are done
     copies(0u);
@@ -281,7 +283,7 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
                     const int minimum = (min_hi[i] << 7) + min_lo[i];
                     const float left = (da * d_of[k]) * (float)dot;
                     const float right = (da * dmin_of[k]) * (float)minimum;
-                    acc[nt][i] += left - right;
+                    acc[nt][i] += (double)(left - right);
                 }
             }
         }
@@ -320,7 +322,7 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
             if constexpr (FUSED) {
 #pragma unroll
                 for (unsigned k = 0; k < 4u; ++k)
-                    value[k] = swiglu_bf16_fast(acc[nt][4u * q4 + k], acc[nt][4u * q4 + k + 8u], route_weight,
+                    value[k] = swiglu_bf16_fast((float)acc[nt][4u * q4 + k], (float)acc[nt][4u * q4 + k + 8u], route_weight,
                                                 g.limit, limit_f32);
             } else {
                 const bool add = g.plain && g.additive;
@@ -338,7 +340,7 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
                 const bool round = g.plain ? g.output_bf16 != 0 : true;
 #pragma unroll
                 for (unsigned k = 0; k < 4u; ++k) {
-                    value[k] = add ? acc[nt][4u * q4 + k] + extra[k] : acc[nt][4u * q4 + k];
+                    value[k] = add ? (float)acc[nt][4u * q4 + k] + extra[k] : (float)acc[nt][4u * q4 + k];
                     fine[k] = finite_f32(value[k]);          // (the rounding below is for numbers)
                     if (round) value[k] = bf16_round_number(value[k]);
                 }

@@ -438,4 +438,43 @@ __device__ __forceinline__ float chunk_unit_dot_f32(const LaneChunk<QT> &c, int 
     }
 }
 
+// Unit k of a LaneChunk against 32 F32 activations as the CPU row dot forms it
+// (src/gguf/quant_compute.c:152-172): every weight decoded to the float the block decoder gives
+// (src/gguf/quant_block.c:745-881, the float operations in its order), the product with its
+// activation and the running sum in double. `sum` carries the lane's running sum on.
+template <unsigned QT>
+__device__ __forceinline__ double chunk_unit_dot_f64(const LaneChunk<QT> &c, int k, const Unit &unit,
+                                                     const float *x, double sum)
+{
+    float scale1, scale2, minimum1 = 0.0f, minimum2 = 0.0f;
+    if constexpr (QT == QT_IQ2_XXS) {
+        scale1 = scale2 = f16_bits_to_float(c.d16) * (0.5f + (float)((unit.factor - 1) >> 1)) * 0.25f;
+    } else if constexpr (QT == QT_Q8_0) {
+        scale1 = scale2 = f16_bits_to_float(c.d16[k]);
+    } else if constexpr (QT == QT_Q4_K) {
+        scale1 = scale2 = f16_bits_to_float(c.head[0] & 0xffffu) * (float)unit.factor;
+        minimum1 = minimum2 = f16_bits_to_float(c.head[0] >> 16) * (float)unit.min1;
+    } else {
+        scale1 = f16_bits_to_float(c.dd & 0xffffu) * (float)unit.factor;
+        scale2 = f16_bits_to_float(c.dd & 0xffffu) * (float)unit.factor2;
+        minimum1 = f16_bits_to_float(c.dd >> 16) * (float)unit.min1;
+        minimum2 = f16_bits_to_float(c.dd >> 16) * (float)unit.min2;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + 4 * i);
+        const float xs[4] = {v.x, v.y, v.z, v.w};
+        const unsigned w = unit.w[i];
+        const float scale = i < 4 ? scale1 : scale2, minimum = i < 4 ? minimum1 : minimum2;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const float code = (float)(signed char)((w >> (8 * b)) & 255u);
+            float value = scale * code;
+            if constexpr (QT == QT_Q4_K || QT == QT_Q2_K) value = value - minimum;
+            sum += (double)value * (double)xs[b];
+        }
+    }
+    return sum;
+}
+
 }  // namespace yvex

@@ -772,12 +772,17 @@ sequence:
      * sums use the pair-output range, which nothing else touches before the down projection. */
     if (views[YVEX_MOE_WEIGHT_ROUTER].qtype == YVEX_GGUF_QTYPE_F32) {
         unsigned long long need = yvex_hip_matvec_f32_scratch_bytes(experts, hidden, row_count);
-        int split = need && need <= pairs * hidden * sizeof(float);
+        int lend = need && need <= pairs * hidden * sizeof(float);
+        /* (the wrapper says how many launches it makes for these operands: the count below and
+         * the node count of a captured graph must agree) */
+        unsigned int router_launches = yvex_hip_matvec_f32_rows_launches(
+            (const float *)(uintptr_t)router_address, experts, hidden, (const float *)activations, row_count,
+            hidden, lend ? AT(pair_outputs) : NULL, lend ? need : 0ull);
         LAUNCH(yvex_hip_matvec_f32_rows((const float *)(uintptr_t)router_address, experts, hidden,
                                         (const float *)activations, row_count, hidden, NULL,
-                                        (float *)AT(logits), experts, 0, split ? AT(pair_outputs) : NULL,
-                                        split ? need : 0ull, (int *)status, stream), "rocm.moe.rows.router");
-        if (rc == YVEX_OK && split && graph_mode != GRAPH_REPLAY) launches++;   /* partials, then their sum */
+                                        (float *)AT(logits), experts, 0, lend ? AT(pair_outputs) : NULL,
+                                        lend ? need : 0ull, (int *)status, stream), "rocm.moe.rows.router");
+        if (rc == YVEX_OK && router_launches == 2u && graph_mode != GRAPH_REPLAY) launches++;   /* partials, then their sum */
     } else
     LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)router_address, views[YVEX_MOE_WEIGHT_ROUTER].qtype,
                            experts, hidden, views[YVEX_MOE_WEIGHT_ROUTER].row_bytes,
