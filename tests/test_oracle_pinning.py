@@ -543,3 +543,237 @@ def test_ffn_ingress_matches_reference_fixture(oracle, golden, name, streams, wi
     assert np.array_equal(bits(normalized), golden[f"ingress_{name}_normalized_bits"])
     assert np.array_equal(bits(post), golden[f"ingress_{name}_post_bits"])
     assert np.array_equal(bits(comb).reshape(comb.shape[0], -1), golden[f"ingress_{name}_combination_bits"])
+
+
+# ---- the Q8_K-activation path: block floats, row dot, expert, layer ------------------------------
+#
+# The integer block sums are pinned above. What follows pins how they become floats
+# (src/backend/cuda/kernel_primitives.h:312, :336-340, :353-357), how a row's block terms are
+# added (double, block order: the CPU row dot's accumulation, src/gguf/quant_compute.c:152-172),
+# and how route, expert and layer compose (src/graph/moe.c:587-622, src/runtime/moe.c:596-632).
+
+F32 = np.float32
+
+
+def f16_of(oracle, raw16):
+    return F32(oracle.lib().yvo_f16_decode(int(raw16)))
+
+
+def fma32(a, b, c):
+    """float32 fused multiply-add from exact rational arithmetic, correctly rounded once."""
+    from fractions import Fraction
+    exact = Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c))
+    if exact == 0:
+        return F32(0.0)
+    # round the exact value to 24 significant bits, ties to even
+    sign = -1 if exact < 0 else 1
+    mag = abs(exact)
+    e = mag.numerator.bit_length() - mag.denominator.bit_length()
+    if Fraction(2) ** e > mag:
+        e -= 1
+    scaled = mag / Fraction(2) ** (e - 23)          # in [2^23, 2^24)
+    whole = scaled.numerator // scaled.denominator
+    rest = scaled - whole
+    if rest > Fraction(1, 2) or (rest == Fraction(1, 2) and whole & 1):
+        whole += 1
+    return F32(sign * float(Fraction(whole) * Fraction(2) ** (e - 23)))
+
+
+def block_float(oracle, qt, w_block, a_block):
+    return F32(oracle.lib().yvo_block_dot_float(C.c_uint(qt), C.c_void_p(w_block.ctypes.data),
+                                                C.c_void_p(a_block.ctypes.data)))
+
+
+def test_fma32_helper_is_a_fused_multiply_add():
+    # 1 + 2^-24 times itself: the exact product needs 49 bits; rounding the product to float first
+    # loses the term the fused form keeps
+    a = F32(1.0 + 2.0 ** -12)
+    assert fma32(a, a, F32(-1.0)) == F32(2.0 ** -11 + 2.0 ** -24)
+    assert F32(F32(a * a) + F32(-1.0)) != fma32(a, a, F32(-1.0))
+
+
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q4_K", "Q2_K", "Q8_0"])
+def test_block_float_is_the_primitives_order_of_float_operations(oracle, qtype):
+    """One weight superblock against one Q8_K block: the float value is the device primitive's
+    expression evaluated in float32 in its written order. Other plausible orders (scales
+    multiplied first in another grouping, one rounding at the end, 0.25 for 0.125, a product in
+    place of a fused multiply-add) are shown to give different bits on these inputs."""
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(77, f"blockfloat.{qtype}")
+    wb = {"IQ2_XXS": 66, "Q4_K": 144, "Q2_K": 84, "Q8_0": 272}[qtype]
+    orders_seen = set()
+    for trial in range(40):
+        w = g.weights(qt, 1, 256)
+        assert w.size == wb
+        act = oracle.q8k_quantize(g.normal(256) * (1.0 + trial))
+        da = act[:4].copy().view(np.float32)[0]
+        got = block_float(oracle, qt, w, act)
+        sums = oracle.block_dots_i32(qt, w, 1, 256, act, 1)
+        if qtype == "IQ2_XXS":
+            dw = f16_of(oracle, w[:2].copy().view(np.uint16)[0])
+            t = F32(int(sums[0, 0, 0, 0]))
+            want = F32(F32(F32(F32(0.125) * dw) * da) * t)
+            others = [F32(F32(0.125) * F32(dw * F32(da * t))), F32(0.125 * float(dw) * float(da) * float(t)),
+                      F32(F32(F32(F32(0.25) * dw) * da) * t)]
+        elif qtype == "Q8_0":
+            want = F32(0.0)
+            loose = F32(0.0)
+            for b in range(8):
+                d = f16_of(oracle, w[34 * b:34 * b + 2].copy().view(np.uint16)[0])
+                dot = F32(int(sums[0, 0, b]))
+                want = fma32(F32(d * da), dot, want)
+                loose = F32(loose + F32(F32(d * da) * dot))
+            others = [loose]
+        else:
+            head = 0 if qtype == "Q4_K" else 80
+            d = f16_of(oracle, w[head:head + 2].copy().view(np.uint16)[0])
+            dmin = f16_of(oracle, w[head + 2:head + 4].copy().view(np.uint16)[0])
+            dot, minimum = F32(int(sums[0, 0, 0, 0])), F32(int(sums[0, 0, 0, 1]))
+            want = F32(F32(F32(da * d) * dot) - F32(F32(da * dmin) * minimum))
+            others = [F32(float(da) * float(d) * float(dot) - float(da) * float(dmin) * float(minimum)),
+                      F32(da * F32(F32(d * dot) - F32(dmin * minimum)))]
+        assert bits(got) == bits(want), (trial, got, want)
+        for k, other in enumerate(others):
+            if bits(other) != bits(want):
+                orders_seen.add(k)
+    assert orders_seen == set(range(len(others)))      # every alternative was told apart at least once
+
+
+@pytest.mark.parametrize("qtype,width", [("IQ2_XXS", 7168), ("Q4_K", 2048), ("Q2_K", 1024), ("Q8_0", 2048)])
+def test_q8_row_dot_adds_block_floats_in_double_in_block_order(oracle, qtype, width):
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(78, f"rowdot.{qtype}")
+    rows, inputs = 24, 2
+    w = g.weights(qt, rows, width)
+    act = oracle.q8k_quantize(g.normal(inputs * width).reshape(inputs, width))
+    got = oracle.q8_matvec(qt, w, rows, width, act, inputs)
+    blocks = width // 256
+    wb = w.size // (rows * blocks)
+    differs_from_float_sum = 0
+    for i in range(inputs):
+        for r in range(rows):
+            terms = [block_float(oracle, qt, w[(r * blocks + b) * wb:(r * blocks + b + 1) * wb],
+                                 act[(i * blocks + b) * 292:(i * blocks + b + 1) * 292]) for b in range(blocks)]
+            total = 0.0
+            single = F32(0.0)
+            for t in terms:
+                total += float(t)               # Python floats are doubles: one rounded add per block
+                single = F32(single + t)
+            assert bits(got[i, r]).item() == bits(F32(total)).item()
+            differs_from_float_sum += int(bits(single).item() != bits(F32(total)).item())
+    assert differs_from_float_sum > 0          # a float accumulator would have been told apart
+
+
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q8_0", "Q4_K", "Q2_K"])
+def test_q8_matvec_against_the_float_path_on_dequantised_activations(oracle, qtype):
+    """The reference's own bound for its Q8_K-activation kernels (tests/unit/cuda/quant_qtype.c:402,
+    419-421): within 1e-5 (1 + |expected|) of the CPU row dot fed with the dequantised activations.
+    A wrong constant, a dropped minimum term or a transposed operand is orders of magnitude outside."""
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(79, f"q8matvec.{qtype}")
+    rows, width, inputs = 16, 2048, 3
+    w = g.weights(qt, rows, width)
+    act = oracle.q8k_quantize(g.normal(inputs * width).reshape(inputs, width))
+    got = oracle.q8_matvec(qt, w, rows, width, act, inputs)
+    want = oracle.matvec(qt, w, rows, width, oracle.q8k_dequantize(act).reshape(inputs, width))
+    assert got.shape == want.shape == (inputs, rows)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-5 * (1.0 + np.abs(want)))
+    assert np.abs(want).max() > 1e-3
+
+
+def swiglu_reference(oracle, g, u, weight, limit):
+    """src/graph/moe.c:605-611 in Python doubles."""
+    out = np.empty(g.size, np.float32)
+    for i in range(g.size):
+        gv = min(float(g[i]), limit)
+        uv = max(-limit, min(float(u[i]), limit))
+        silu = gv / (1.0 + math.exp(-gv)) if gv >= 0.0 else gv * math.exp(gv) / (1.0 + math.exp(gv))
+        out[i] = oracle.lib().yvo_bf16_round(F32(silu * uv * float(weight)))
+    return out
+
+
+def bf16_rounded(oracle, values):
+    return np.array([oracle.lib().yvo_bf16_round(F32(v)) for v in np.ravel(values)], np.float32).reshape(np.shape(values))
+
+
+def expert_from_pinned_pieces(oracle, qt, gate, up, down, hidden, inter, x, weight, limit):
+    q = oracle.q8k_quantize(x)
+    g = oracle.q8_matvec(qt, gate, inter, hidden, q, 1)[0]
+    u = oracle.q8_matvec(qt, up, inter, hidden, q, 1)[0]
+    h = swiglu_reference(oracle, g, u, weight, limit)
+    out = oracle.q8_matvec(qt, down, hidden, inter, oracle.q8k_quantize(h), 1)[0]
+    return h, bf16_rounded(oracle, out), out
+
+
+@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q8_0"])
+def test_expert_with_q8k_activations_is_the_composition_of_pinned_pieces(oracle, qtype):
+    """yvo_moe_expert(act_q8) against quantize -> gate, up -> clamped SwiGLU with the route weight
+    inside the rounding -> quantize -> down -> bfloat16 built from functions pinned above. The
+    limit is low enough to clamp; a route weight applied after the down projection, an
+    unclamped gate or a float SwiGLU would not give these bits."""
+    qt = getattr(oracle, qtype)
+    hidden, inter = 512, 256
+    g = oracle.Generator(80, f"expert.q8.{qtype}")
+    gate, up = g.weights(qt, inter, hidden), g.weights(qt, inter, hidden)
+    down = g.weights(qt, hidden, inter)
+    x = (g.normal(hidden) * 40.0).astype(np.float32)
+    weight, limit = 0.37, 0.75
+    rc, out, mid, raw = oracle.moe_expert((qt, qt, qt), gate, up, down, hidden, inter, x, weight, limit=limit,
+                                          act_q8=True)
+    assert rc == 0
+    h, want, want_raw = expert_from_pinned_pieces(oracle, qt, gate, up, down, hidden, inter, x, weight, limit)
+    q = oracle.q8k_quantize(x)
+    clamped = np.abs(oracle.q8_matvec(qt, up, inter, hidden, q, 1)[0]) > limit
+    assert clamped.any() and not clamped.all()
+    assert np.array_equal(bits(mid), bits(h))
+    assert np.array_equal(bits(out), bits(want))
+    # the alternatives are different numbers here
+    late = bf16_rounded(oracle, oracle.q8_matvec(
+        qt, down, hidden, inter, oracle.q8k_quantize(swiglu_reference(oracle, *(
+            oracle.q8_matvec(qt, m, inter, hidden, q, 1)[0] for m in (gate, up)), 1.0, limit)), 1)[0] * F32(weight))
+    assert not np.array_equal(bits(late), bits(want))
+
+
+def test_layer_is_route_then_experts_in_rank_order_then_shared(oracle):
+    """yvo_moe_layer against the composition src/runtime/moe.c:596-632 writes: route, one expert per
+    rank added to a float row, the shared expert with weight 1, bfloat16 of the float sum routed +
+    shared. (The experts' outputs are bfloat16 values, a handful of which add exactly in float, so
+    the order of the ranks is not observable on such data.) Plausible slips give other bits here
+    and the test shows that they do: the routed sum rounded to bfloat16 before the shared expert
+    is added, the shared expert weighted like a routed one, the last rounding left out."""
+    qt = oracle.IQ2_XXS
+    hidden, inter, experts, topk, rows = 512, 256, 8, 4, 3
+    g = oracle.Generator(81, "layer.q8")
+    gate, up = g.weights(qt, experts * inter, hidden), g.weights(qt, experts * inter, hidden)
+    down = g.weights(qt, experts * hidden, inter)
+    shared = (g.weights(qt, inter, hidden), g.weights(qt, inter, hidden), g.weights(qt, hidden, inter))
+    x = g.normal(rows * hidden).reshape(rows, hidden)
+    logits = g.normal(rows * experts).reshape(rows, experts)
+    bias = (g.normal(experts) * 0.05).astype(np.float32)
+    got = oracle.moe_layer(hidden=hidden, intermediate=inter, experts=experts, topk=topk, qtypes=(qt, qt, qt),
+                           routed=(gate, up, down), shared=shared, inputs=x, logits=logits, bias=bias,
+                           scoring=oracle.SIGMOID, normalize=True, scaling=1.5, limit=10.0, act_q8=True)
+    gb, db = oracle.row_bytes(qt, hidden) * inter, oracle.row_bytes(qt, inter) * hidden
+    order_matters = 0
+    for r in range(rows):
+        rc, sel, w, _ = oracle.moe_route(logits[r], bias, topk, oracle.SIGMOID, True, 1.5)
+        assert rc == 0 and np.array_equal(sel, got["selected"][r]) and np.array_equal(bits(w), bits(got["weights"][r]))
+        outs = []
+        for rank in range(topk):
+            e = int(sel[rank])
+            _, out, _ = expert_from_pinned_pieces(oracle, qt, gate[e * gb:(e + 1) * gb], up[e * gb:(e + 1) * gb],
+                                                  down[e * db:(e + 1) * db], hidden, inter, x[r], w[rank], 10.0)
+            outs.append(out)
+        routed = np.zeros(hidden, np.float32)
+        for out in outs:
+            routed = (routed + out).astype(np.float32)
+        _, shared_out, _ = expert_from_pinned_pieces(oracle, qt, *shared, hidden, inter, x[r], 1.0, 10.0)
+        assert np.array_equal(bits(got["routed"][r]), bits(routed))
+        assert np.array_equal(bits(got["shared"][r]), bits(shared_out))
+        assert np.array_equal(bits(got["combined"][r]), bits(bf16_rounded(oracle, (routed + shared_out).astype(np.float32))))
+        early = (bf16_rounded(oracle, routed) + shared_out).astype(np.float32)
+        _, weighted_shared, _ = expert_from_pinned_pieces(oracle, qt, *shared, hidden, inter, x[r], w[0], 10.0)
+        order_matters += int(not np.array_equal(bits(bf16_rounded(oracle, early)), bits(got["combined"][r])))
+        order_matters += int(not np.array_equal(bits(weighted_shared), bits(got["shared"][r])))
+        order_matters += int(not np.array_equal(bits((routed + shared_out).astype(np.float32)), bits(got["combined"][r])))
+    assert order_matters == 3 * rows
