@@ -22,12 +22,28 @@
  *                                                  the reference has no CPU entry point for it.
  *   yvo_block_dot_*                                exact integer definitions, numpy int64 brute
  *                                                  force.
+ *   yvo_block_dot_float                            float32 re-evaluation of the device primitive's
+ *                                                  expression step by step (an exact-rational fused
+ *                                                  multiply-add for Q8_0), against which other
+ *                                                  orders of the same operations are shown to differ.
+ *   yvo_q8_row_dot / yvo_q8_matvec                 block floats added in double in block order
+ *                                                  (recomputed in the test; a float accumulator is
+ *                                                  told apart), and the reference's own bound for
+ *                                                  its Q8_K-activation kernels: 1e-5 (1 + |x|) of
+ *                                                  yvo_cpu_dot on the dequantised activations
+ *                                                  (tests/unit/cuda/quant_qtype.c:402,419-421).
  *   yvo_moe_route (sqrt_softplus)                  compiled reference yvex_moe_route_cpu and the
  *                                                  expectations of tests/unit/runtime_moe.c:105-150.
  *   yvo_moe_route (sigmoid)                        PARITY UNPINNED by the reference (not in it);
  *                                                  closed form only.
  *   yvo_moe_expert / yvo_moe_layer                 compiled reference yvex_moe_expert_cpu, the
- *                                                  exact-equality case runtime_moe.c:178-212.
+ *                                                  exact-equality case runtime_moe.c:178-212; with
+ *                                                  Q8_K activations the composition of the pinned
+ *                                                  pieces rebuilt in the test (quantize, row dots,
+ *                                                  double SwiGLU with the clamp active, bfloat16
+ *                                                  roundings, route, float sum over the ranks,
+ *                                                  shared expert), with plausible slips shown to
+ *                                                  give other bits.
  *   yvo_worklist_build                             properties (stable sort, sums) and the cases of
  *                                                  tests/unit/expert_worklist.c.
  *   yvo_argmax_f32                                 brute force over small rows (largest value, its
