@@ -411,6 +411,12 @@ int yvex_rocm_quant_row_dot(yvex_rocm_backend *backend, unsigned int qtype, cons
 #define YVEX_MOE_KERNEL_PORTABLE_EXPERT_ROW "portable-expert-row"
 #endif
 #define YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP "gfx950-int8-dot-expert-sweep"
+/* The family a sealed worklist policy names in tensor_core_kernel_family to admit this backend's
+ * int8 matrix-core expert kernels (the reference names its own, moe.h:22, and refuses any other:
+ * src/backend/cuda/moe.c:937-951). With a policy present the matrix-core regime runs only when
+ * tensor_core_minimum is non-zero and the batch has at least that many rows; execute_rows then
+ * still picks the faster of its two kernel families, which publish the same bits. */
+#define YVEX_MOE_KERNEL_GFX950_MATRIX_CORE_EXPERT "gfx950-int8-matrix-core-expert"
 
 #ifndef YVEX_ROCM_REFERENCE_TYPES
 typedef enum {

@@ -569,6 +569,44 @@ def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle, qty
     assert case.result.row_expert_pairs == 400 and case.result.completed == 1
 
 
+def sealed_policy(case, minimum):
+    """An execution batch and a worklist policy as the runtime seals them for a row batch
+    (src/runtime/moe.c:101-193), the policy with the given tensor-core minimum."""
+    batch, policy = abi.ExecutionBatch(), abi.WorklistPolicy()
+    batch.schema_version, batch.row_count = 1, case.rows
+    batch.provenance, batch.phase = case.batch.provenance, case.batch.phase
+    policy.schema_version = 1
+    policy.supported_width_mask = ((1 << 62) - 1) << 1
+    policy.narrow_kernel_family = abi.FAMILY_GFX950
+    policy.tensor_core_minimum = minimum
+    policy.tensor_core_kernel_family = abi.FAMILY_GFX950_MATRIX_CORE if minimum else b""
+    return batch, policy
+
+
+@pytest.mark.parametrize("minimum,matrix", [(None, True), (0, False), (8, True), (40, False)])
+def test_worklist_policy_decides_the_matrix_core_regime(backend, oracle, minimum, matrix):
+    """src/backend/cuda/moe.c:1341-1361: the tensor-core kernels run only when the sealed policy
+    names a minimum and the batch has that many rows. 36 rows over four experts would take the
+    matrix cores by this backend's own threshold: a policy with minimum 0 keeps them off, one with
+    a minimum above the batch does too, and the published facts say what ran. The rows are the
+    same bits either way."""
+    case = MoeCase(backend, oracle, hidden=512, intermediate=256, experts=4, topk=2, rows=36,
+                   scoring=abi.SCORING_SIGMOID)
+    backend.workspace(case.workspace_bytes)
+    if minimum is not None:
+        batch, policy = sealed_policy(case, minimum)
+        case.job.execution_batch, case.job.worklist_policy = C.pointer(batch), C.pointer(policy)
+    assert case.execute() == 0, case.err.message
+    res = case.result
+    pairs = case.rows * case.topk
+    assert (res.tensor_core_launches > 0) == matrix
+    assert res.worklists.tensor_core_eligible_pairs == (pairs if matrix else 0)
+    assert res.worklists.tensor_core_executed_pairs == (pairs if matrix else 0)
+    assert res.worklists.narrow_pairs == (0 if matrix else pairs)
+    got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+    same_as_cpu(got, case.oracle_layer(act_q8=True)["combined"])
+
+
 def test_execute_rows_refusals(backend, oracle):
     b = backend
     case = MoeCase(b, oracle)
@@ -610,7 +648,9 @@ def test_execute_rows_refusals(backend, oracle):
     assert case.execute() == abi.INVALID_ARG
     policy.tensor_core_kernel_family = abi.FAMILY_GFX950
     assert case.execute() == abi.INVALID_ARG            # ... that differs from the narrow one
-    policy.tensor_core_kernel_family = b"gfx950-int8-matrix-expert-rows"
+    policy.tensor_core_kernel_family = b"sm121-int8-tensorcore-expert"
+    assert case.execute() == abi.UNSUPPORTED            # ... and be this backend's (src/backend/cuda/moe.c:937-951)
+    policy.tensor_core_kernel_family = abi.FAMILY_GFX950_MATRIX_CORE
     assert case.execute() == 0, case.err.message
     policy.tensor_core_minimum = 3                      # ... and must be an admitted width
     assert case.execute() == abi.INVALID_ARG

@@ -208,3 +208,63 @@ def test_prefill_layer_at_full_size(gpu, oracle, layer_weights, qtype):
     assert np.array_equal(selected[picked].cpu().numpy().astype(np.uint64), want["selected"])
     equal_to_oracle(first[picked].cpu().numpy(), want["combined"],
                     f"prefill layer ({qtype}), 4 rows against the oracle")
+
+
+# ---- the same comparisons on the product entry: execute_rows + complete_rows ----------------------
+
+def router_weights(device, seed):
+    """F32 router rows whose projection of N(0, 1) rows gives logits of unit size."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    return torch.randn((EXPERTS, HIDDEN), device=device, generator=gen) * HIDDEN ** -0.5
+
+
+@pytest.mark.parametrize("rows,qtype,sweep_image", [(32, "IQ2_XXS", False), (32, "IQ2_XXS", True),
+                                                    (2048, "IQ2_XXS", False), (2048, "Q4_K", False)])
+def test_execute_rows_at_full_size_equals_the_cpu_layer(gpu, oracle, layer_weights, rows, qtype, sweep_image):
+    """BASELINE configs 3 and 4 through yvex_rocm_backend_moe_operations_get()->execute_rows and
+    complete_rows (the reference's row-batch entry, src/backend/cuda/moe.c:1826-1958), router
+    projection included: 32 rows take the decode sweeps (over canonical bytes and over the sweep
+    image), 2048 rows the matrix-core kernels (IQ2_XXS and Q4_K experts). Picked rows are the CPU
+    layer's bit for bit: router logits from the CPU row dot, then src/graph/moe.c:497-622 and
+    src/runtime/moe.c:596-632 on Q8_K activations. A second call gives the same bits, and the
+    facts say which kernels ran."""
+    from yvex_amd import abi
+    from yvex_amd import kernels as K
+    from yvex_amd.host import RowBatchLayer
+    if qtype == "IQ2_XXS":
+        routed, shared = layer_weights
+    else:
+        blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
+        routed = tuple(synthetic_q4k(blocks, gpu, 21 + i) for i in range(3))
+        shared = tuple(synthetic_q4k(INTERMEDIATE * HIDDEN // 256, gpu, 31 + i) for i in range(3))
+    gen = torch.Generator(device=gpu)
+    gen.manual_seed(rows)
+    x = torch.randn((rows, HIDDEN), device=gpu, generator=gen)
+    router = router_weights(gpu, 5)
+    qt = getattr(K, qtype)
+    layer = RowBatchLayer(torch, routed, shared, router, x.cpu().numpy(), rows, hidden=HIDDEN,
+                          intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtype=qt, sweep_image=sweep_image)
+    try:
+        layer.step(defer=True)
+        layer.complete()
+        assert layer.done.completed == 1
+        first = layer.output().copy()
+        layer.step(defer=False)
+        assert layer.result.completed == 1 and layer.result.row_expert_pairs == rows * TOPK
+        assert np.array_equal(first.view(np.uint32), layer.output().view(np.uint32))
+        matrix_cores = layer.result.tensor_core_launches > 0
+        assert matrix_cores == (rows == 2048)
+    finally:
+        layer.close()
+    assert np.isfinite(first).all() and np.abs(first).max() > 0.0
+    picked = [0, 4, 9, 13, 17, 22, 26, 31] if rows == 32 else [5, 700, 1000, 1900]
+    host_x = x[picked].cpu().numpy()
+    logits = oracle.matvec(oracle.F32, router.cpu().numpy().view(np.uint8).reshape(-1), EXPERTS, HIDDEN, host_x)
+    want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                            qtypes=(getattr(oracle, qtype),) * 3, routed=[t.cpu().numpy() for t in routed],
+                            shared=[t.cpu().numpy() for t in shared], inputs=host_x, logits=logits,
+                            scoring=oracle.SIGMOID, normalize=True, scaling=1.0, limit=10.0, act_q8=True,
+                            threads=16)
+    equal_to_oracle(first[picked], want["combined"],
+                    f"execute_rows, {rows} rows, {qtype}{' (sweep image)' if sweep_image else ''}: picked rows against the oracle")

@@ -27,6 +27,7 @@ W_FFN_NORM, W_MHC_FUNCTION, W_MHC_BASE, W_MHC_SCALE, W_ROUTER, W_ROUTER_TABLE, W
     W_ROUTED_GATE, W_ROUTED_UP, W_ROUTED_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN, W_COUNT = range(14)
 FAMILY_PORTABLE_EXPERT_ROW = b"portable-expert-row"
 FAMILY_GFX950 = b"gfx950-int8-dot-expert-sweep"
+FAMILY_GFX950_MATRIX_CORE = b"gfx950-int8-matrix-core-expert"
 HEX = 65
 ULL = C.c_ulonglong
 

@@ -353,6 +353,7 @@ typedef struct {
     yvex_hip_graph graph;              /* NULL: seen once, ran eagerly */
     unsigned long long launches, last_use;
     int used;
+    int eager_only;                    /* a launch wrapper refused this job while it was recorded */
 } graph_slot;
 
 struct yvex_rocm_moe_graphs {
@@ -489,7 +490,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     const void *activations;
     void *combined_target;
     unsigned long long table_address = 0ull;
-    int envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
+    int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
     void *status;
     yvex_hip_stream stream;
     enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
@@ -586,6 +587,18 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
                            &views[YVEX_MOE_WEIGHT_SHARED_DOWN], hidden, layer->shared_intermediate_width,
                            &shared_q8, &shared_image, err);
     if (rc != YVEX_OK) return rc;
+    /* The sealed worklist policy decides whether the matrix-core regime may run at all
+     * (src/backend/cuda/moe.c:913-951, 1341-1361): a minimum of zero keeps it off, a minimum above
+     * the batch's rows keeps it off for this batch, and a regime named by another family than
+     * this backend's is refused. A job without a policy leaves the choice to the backend. */
+    if (job->worklist_policy && job->worklist_policy->tensor_core_minimum) {
+        if (strcmp(job->worklist_policy->tensor_core_kernel_family, YVEX_MOE_KERNEL_GFX950_MATRIX_CORE_EXPERT) != 0)
+            return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                    "compiled matrix-core MoE worklist regime is unavailable");
+        matrix_allowed = row_count >= job->worklist_policy->tensor_core_minimum;
+    } else if (job->worklist_policy) {
+        matrix_allowed = 0;
+    }
     /* weights: router [experts x hidden], optional bias [1 x experts], expert-major matrices */
     rc = view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTER], hidden, experts, &router_address, err);
     if (rc == YVEX_OK && !hash_router && layer->requires_correction_bias)
@@ -660,8 +673,10 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
      * top-8 the two families cross at about 170 rows (IQ2_XXS) and 128 rows (Q4_K). The
      * reference switches its tensor-core kernels on from 16 input rows
      * (src/backend/cuda/private.h:461-464). Both kernel families read the sweep image of
-     * IQ2_XXS experts as well as canonical bytes. */
-    row_batch = routed_q8 && matrix_core_qtypes(&routed) &&
+     * IQ2_XXS experts as well as canonical bytes, and both publish the same bits (a row's terms
+     * are added in double in block order in either), so the choice is one of speed only; a
+     * sealed worklist policy can keep the matrix-core regime off (matrix_allowed). */
+    row_batch = matrix_allowed && routed_q8 && matrix_core_qtypes(&routed) &&
                 pairs >= (routed.gate_qtype == 12u ? 4ull : 6ull) * experts;
     shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
@@ -699,6 +714,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
         key.count = 0u;
         key.overflow = 0;
         key_word(&key, row_count);
+        key_word(&key, (unsigned long long)row_batch);
         key_word(&key, (unsigned long long)(uintptr_t)status);
         key_word(&key, (unsigned long long)(uintptr_t)stream);
         key_word(&key, base);
@@ -712,7 +728,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
         if (backend->moe_graphs && !key.overflow) {
             graph_slot *slot = graph_find(backend->moe_graphs, &key);
             if (!slot) slot = graph_admit(backend->moe_graphs, &key);   /* first sight: eager */
-            else graph_mode = slot->graph ? GRAPH_REPLAY : GRAPH_CAPTURE;
+            else if (!slot->eager_only) graph_mode = slot->graph ? GRAPH_REPLAY : GRAPH_CAPTURE;
             slot->last_use = ++backend->moe_graphs->clock;
             graph_target = slot;
         }
@@ -915,9 +931,15 @@ sequence:
         /* a recording that fails, or holds anything but kernels, is dropped for good and the
          * batch runs eagerly: the stream has executed nothing yet */
         uint64_t nodes = 0u;
-        if (rc != YVEX_OK) (void)yvex_hip_capture_abort(stream);
-        if (rc != YVEX_OK || yvex_hip_capture_end(stream, &graph_target->graph, &nodes) != 0 ||
-            nodes != launches) {
+        if (rc != YVEX_OK) {
+            /* a launch wrapper refused this job's geometry: the job fails eagerly too, and only
+             * its own slot stops recording; other topologies keep their graphs */
+            (void)yvex_hip_capture_abort(stream);
+            graph_target->eager_only = 1;
+            graph_mode = GRAPH_EAGER;
+            goto sequence;
+        }
+        if (yvex_hip_capture_end(stream, &graph_target->graph, &nodes) != 0 || nodes != launches) {
             if (graph_target->graph) (void)yvex_hip_graph_destroy(graph_target->graph);
             graph_target->graph = NULL;
             backend->moe_graphs->refused = 1;
@@ -931,7 +953,11 @@ sequence:
         rc = yvex_rocm_launch_result(yvex_hip_graph_launch(graph_target->graph, stream),
                                      "rocm.moe.rows.graph", err);
     }
-    if (rc != YVEX_OK) return rc;
+    if (rc != YVEX_OK) {
+        /* a job that fails on first sight is not remembered: its next call is a first sight again */
+        if (graph_target && !graph_target->graph) graph_target->used = 0;
+        return rc;
+    }
 
     defer = job->device_completion && job->device_completion->defer;
     result->graph_launches = graph_mode != GRAPH_EAGER;
@@ -942,6 +968,7 @@ sequence:
     result->row_count = row_count;
     result->row_expert_pairs = pairs;
     result->kernel_launches = launches + status_launches;
+    result->tensor_core_launches = (row_batch ? 2ull : 0ull) + (shared_row_batch ? 2ull : 0ull);
     result->shared_expert_operations = has_shared ? row_count : 0ull;
     result->grouped_expert_operations = pairs;
     result->active_weight_base_bytes = views[YVEX_MOE_WEIGHT_ROUTER].encoded_bytes +
@@ -1019,7 +1046,10 @@ sequence:
     result->worklists.pair_count = counts[2];
     result->worklists.bucket_count = counts[0];
     result->worklists.maximum_bucket_population = counts[1];
-    result->worklists.narrow_pairs = counts[2];
+    /* every pair of a batch runs in one regime (src/graph/worklist.c:407-425 counts per bucket) */
+    result->worklists.tensor_core_eligible_pairs = row_batch ? counts[2] : 0ull;
+    result->worklists.tensor_core_executed_pairs = row_batch ? counts[2] : 0ull;
+    result->worklists.narrow_pairs = row_batch ? 0ull : counts[2];
     result->worklists.width_histogram[row_count < YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP
                                           ? row_count : YVEX_EXPERT_WORKLIST_HISTOGRAM_CAP - 1u] = 1ull;
     result->worklists.provenance_counts[rows->provenance <= YVEX_EXECUTION_BATCH_COMPILED_COMPATIBLE

@@ -81,3 +81,117 @@ class Backend:
     def close(self):
         self.release_all()
         return self.lib.yvex_rocm_backend_close_checked(C.byref(self.handle), C.byref(self.err))
+
+
+class RowBatchLayer:
+    """One MoE layer behind include/yvex_rocm.h: a backend of its own, weight views that
+    carry device addresses, backend-owned row tensors and an attached workspace. `step()` is one
+    yvex_rocm_backend_moe_operations_get()->execute_rows with deferred completion, `complete()` the
+    phase barrier complete_rows (the reference completes all pending layers of a phase with one
+    call, src/runtime/moe.c:1567-1576)."""
+
+    def __init__(self, torch, routed, shared, router, x_host, rows, *, hidden, intermediate, experts, topk,
+                 qtype=16, sweep_image=False, scoring=abi.SCORING_SIGMOID, scaling=1.0, limit=10.0):
+        HIDDEN, INTERMEDIATE, EXPERTS, TOPK = hidden, intermediate, experts, topk
+        self.C, self.abi, self.np, self.rows, self.hidden = C, abi, np, rows, hidden
+        self.b = Backend()
+        if not self.b.ok:
+            raise RuntimeError(f"backend open failed: {self.b.err.message.decode()}")
+        self.keep = (routed, shared, router)
+        plan = self.plan = abi.LayerPlan()
+        plan.schema_version, plan.router_class, plan.scoring = 1, abi.ROUTER_LEARNED, scoring
+        plan.hidden_width = plan.expanded_width = HIDDEN
+        plan.residual_streams = 1
+        plan.routed_experts, plan.shared_experts, plan.experts_per_token = EXPERTS, 1, TOPK
+        plan.expert_intermediate_width = plan.shared_intermediate_width = INTERMEDIATE
+        plan.routed_scaling_factor, plan.activation_limit = scaling, limit
+        plan.requires_correction_bias, plan.normalize_topk_probabilities = 0, 1
+        job = self.job = abi.LayerJob()
+        job.layer = C.pointer(plan)
+        block_bytes = {16: 66, 12: 144}[qtype]
+        rb_h, rb_i = HIDDEN // 256 * block_bytes, INTERMEDIATE // 256 * block_bytes
+
+        self.images = []
+
+        def view(slot, tensor, qtype, width, count, row_bytes, activation, consumer=None):
+            v = job.weights[slot]
+            v.qtype, v.layout, v.activation = qtype, abi.LAYOUT_EXPERT_MAJOR, activation
+            v.kernel_family = abi.FAMILY_GFX950
+            v.device_address = tensor.data_ptr()
+            v.encoded_bytes = v.storage_bytes = tensor.numel() * tensor.element_size()
+            v.row_bytes, v.row_width, v.row_count = row_bytes, width, count
+            if sweep_image and consumer is not None:
+                # the residency step of a caller that keeps its experts as the decode sweeps' image:
+                # plan, allocate, build on the device from the resident canonical bytes
+                d = abi.ExecutionDecision()
+                d.expert_count = 1 if consumer == abi.CONSUMER_SHARED_EXPERT else EXPERTS
+                d.canonical_qtype, d.canonical_row_width, d.canonical_row_count = qtype, width, count
+                d.encoded_bytes = v.encoded_bytes
+                d.consumer, d.layout, d.derived_asset_required = consumer, abi.LAYOUT_DERIVED, 1
+                d.kernel_family = abi.FAMILY_GFX950
+                storage, err = abi.ULL(), abi.Error()
+                if self.b.lib.yvex_rocm_moe_derived_layout_plan(C.byref(d), C.byref(storage), C.byref(err)) != 0:
+                    raise RuntimeError(err.message.decode())
+                image = torch.empty(storage.value, dtype=torch.uint8, device=tensor.device)
+                if self.b.lib.yvex_rocm_moe_sweep_image_build_resident(
+                        self.b.handle, C.byref(d), tensor.data_ptr(), image.data_ptr(), storage.value,
+                        C.byref(err)) != 0:
+                    raise RuntimeError(err.message.decode())
+                self.images.append(image)
+                v.layout, v.device_address, v.storage_bytes = abi.LAYOUT_DERIVED, image.data_ptr(), storage.value
+
+        enc = abi.ACT_DEVICE_ENCODED
+        view(abi.W_ROUTER, router, 0, HIDDEN, EXPERTS, HIDDEN * 4, abi.ACT_DEVICE_F32)
+        gate_up, down_c, shared_c = abi.CONSUMER_ROUTED_GATE_UP, abi.CONSUMER_ROUTED_DOWN, abi.CONSUMER_SHARED_EXPERT
+        view(abi.W_ROUTED_GATE, routed[0], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
+        view(abi.W_ROUTED_UP, routed[1], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
+        view(abi.W_ROUTED_DOWN, routed[2], qtype, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc, down_c)
+        view(abi.W_SHARED_GATE, shared[0], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
+        view(abi.W_SHARED_UP, shared[1], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
+        view(abi.W_SHARED_DOWN, shared[2], qtype, INTERMEDIATE, HIDDEN, rb_i, enc, shared_c)
+        self.ops = self.b.lib.yvex_rocm_backend_moe_operations_get(self.b.handle).contents
+        need, err = abi.ULL(), abi.Error()
+        if self.ops.workspace_required(C.byref(plan), rows, C.byref(need), C.byref(err)) != 0:
+            raise RuntimeError(err.message.decode())
+        self.b.workspace(need.value)
+        self.rows_in, self.rows_out = self.b.f32(x_host), self.b.empty_f32(rows * HIDDEN)
+        batch = self.batch = abi.RowBatch()
+        batch.schema_version, batch.row_count, batch.row_width, batch.row_stride = 1, rows, HIDDEN, HIDDEN
+        batch.device_rows, batch.device_outputs = self.rows_in, self.rows_out
+        batch.provenance, batch.execution_class = abi.BATCH_MULTI_SESSION, 1
+        self.out = abi.RowBatchOutput()
+        self.result, self.done, self.err = abi.RowBatchResult(), abi.RowBatchResult(), abi.Error()
+        self.deferred = abi.DeviceCompletion(1, None)
+
+    def step(self, defer=True, eager=False):
+        C = self.C
+        self.job.eager_execution = int(eager)
+        self.job.device_completion = C.pointer(self.deferred) if defer else None
+        rc = self.ops.execute_rows(self.b.handle, C.byref(self.job), C.byref(self.batch), C.byref(self.out),
+                                   C.byref(self.result), C.byref(self.err))
+        if rc != 0:
+            raise RuntimeError(f"execute_rows: {self.err.message.decode()}")
+
+    def complete(self):
+        C = self.C
+        if self.ops.complete_rows(self.b.handle, 0, C.byref(self.done), C.byref(self.err)) != 0:
+            raise RuntimeError(f"complete_rows: {self.err.message.decode()}")
+
+    def timed(self, steps, warmup, *, defer=True, eager=False):
+        """Wall-clock ms per step of `steps` execute_rows calls, the backend idle before the
+        first and after the last (complete_rows is the closing synchronisation)."""
+        for _ in range(warmup):
+            self.step(defer, eager)
+        self.complete()
+        import time
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.step(defer, eager)
+        self.complete()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def output(self):
+        return self.b.read_f32(self.rows_out, self.rows * self.hidden).reshape(self.rows, self.hidden)
+
+    def close(self):
+        self.b.close()
