@@ -14,6 +14,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libyvex_oracle.so")
 REF_PATH = os.path.join(HERE, "_ref", "libyvex_ref.so")
+REF_BACKEND_PATH = os.path.join(HERE, "_ref", "libyvex_ref_backend.so")
 
 OK, ERR_FORMAT, ERR_UNSUPPORTED, ERR_BOUNDS, ERR_INVALID_ARG = 0, -4, -5, -7, -10
 F32, F16, Q8_0, Q2_K, Q4_K, Q8_K, IQ2_XXS, I32, BF16, MXFP4 = 0, 1, 8, 10, 12, 15, 16, 26, 30, 39
@@ -32,6 +33,11 @@ def build(force: bool = False) -> None:
         subprocess.run(["make", "-C", HERE, "oracle"], check=True, capture_output=True)
     if os.path.isdir("/root/reference/src/gguf") and (force or not os.path.exists(REF_PATH)):
         subprocess.run(["make", "-C", HERE, "ref"], check=True, capture_output=True)
+    rocm_lib = os.path.join(os.path.dirname(HERE), "yvex_amd", "libyvex_rocm.so")
+    if os.path.isdir("/root/reference/src/backend") and os.path.exists(rocm_lib) and (
+            force or not os.path.exists(REF_BACKEND_PATH) or
+            os.path.getmtime(REF_BACKEND_PATH) < os.path.getmtime(rocm_lib)):
+        subprocess.run(["make", "-C", HERE, "ref_backend"], check=True, capture_output=True)
 
 
 class MoeLayerArgs(C.Structure):
@@ -85,6 +91,18 @@ def lib() -> C.CDLL:
         L.yvo_rng_seed.argtypes = [C.c_void_p, C.c_uint64, C.c_char_p]
         _lib = L
     return _lib
+
+
+def ref_backend_lib():
+    """The reference's generic backend code (src/backend/core.c, residency.c) linked with the ROCm
+    adapter and libyvex_rocm.so, or None where it cannot exist. Load torch first in a process
+    that will use the GPU (it carries its own copy of the HIP runtime)."""
+    if not os.path.exists(REF_BACKEND_PATH):
+        if os.path.isdir("/root/reference/src/backend"):
+            build()
+        if not os.path.exists(REF_BACKEND_PATH):
+            return None
+    return C.CDLL(REF_BACKEND_PATH)
 
 
 def ref_lib():

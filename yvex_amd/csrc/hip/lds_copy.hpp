@@ -75,6 +75,13 @@ __device__ __forceinline__ unsigned lds_read_u32(unsigned address)
 #endif
 }
 
+// The copies below write m0. The compiler reserves m0 and reloads it before every use of its
+// own, but it may merge two of its own loads of the same value across code that sits between
+// them; naming m0 as written by the assembly keeps it from doing that across a copy. It answers
+// the clobber with a diagnostic about reserved registers, silenced here.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+
 // Asynchronous copy global -> LDS (GLOBAL_LOAD_LDS): lane l of the wave writes `bytes` bytes at
 // lds_base + l * bytes; nothing passes through registers. Written as assembly so the compiler
 // does not put a conservative wait in front of every later LDS read: the kernel waits with
@@ -84,7 +91,7 @@ __device__ __forceinline__ void copy_to_lds_16(const void *global, unsigned lds_
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :: "s"(lds_base), "v"(global) : "memory");   // m0 is reserved: the compiler reloads it before any use of its own
+                 :: "s"(lds_base), "v"(global) : "memory", "m0");   // (m0 named: a value the compiler keeps there is reloaded)
 #else
     (void)global;
     (void)lds_base;
@@ -94,7 +101,7 @@ __device__ __forceinline__ void copy_to_lds_4(const void *global, unsigned lds_b
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-                 :: "s"(lds_base), "v"(global) : "memory");   // m0 is reserved: the compiler reloads it before any use of its own
+                 :: "s"(lds_base), "v"(global) : "memory", "m0");   // (m0 named: a value the compiler keeps there is reloaded)
 #else
     (void)global;
     (void)lds_base;
@@ -119,11 +126,13 @@ __device__ __forceinline__ void copy_to_lds_16_first32(const void *global, unsig
     unsigned long long saved;
     asm volatile("s_mov_b64 %0, exec\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved) : "s"(lds_base), "v"(global) : "memory");
+                 : "=&s"(saved) : "s"(lds_base), "v"(global) : "memory", "m0");
 #else
     (void)global;
     (void)lds_base;
 #endif
 }
+
+#pragma clang diagnostic pop
 
 }  // namespace yvex
