@@ -250,6 +250,16 @@ int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *
  * checks (src/backend/private.h:95-101) hold on them. No reference counterpart; bound once, before
  * the first allocation. */
 int yvex_rocm_backend_bind_owner(yvex_rocm_backend *backend, const void *owner, yvex_error *err);
+/* yvex_backend_open_shared_cuda (include/yvex/internal/backend.h:254-255,
+ * src/backend/cuda/backend.c:1913-2000): session-local state that borrows one owning backend's
+ * device and resident arena. The child has a stream, a device status word, memory accounting
+ * under its own limit, tensors, a workspace and launch graphs of its own, so sessions that share
+ * one set of resident weights each run their own row batches; attaching the owner's arena to a
+ * child (yvex_rocm_backend_resident_attach with the owner's resident tensor, the same host base
+ * and generation the owner attached) uploads nothing. The owner must itself be an owning
+ * backend (INVALID_ARG otherwise) and refuses to close while a child is open (STATE). */
+int yvex_rocm_backend_open_shared(yvex_rocm_backend **out, yvex_rocm_backend *context_owner,
+                                  unsigned long long memory_limit_bytes, yvex_error *err);
 /* include/yvex/backend.h:142-152: a cleanup failure keeps *backend non-NULL for a retry. */
 int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend, yvex_error *err);
 yvex_backend_kind yvex_rocm_backend_kind_of(const yvex_rocm_backend *backend);

@@ -307,7 +307,9 @@ class MoeCase:
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
                  shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
-                 down_qtype=None, sweep_image=()):
+                 down_qtype=None, sweep_image=(), arena_from=None):
+        """arena_from: a MoeCase of the same layer on the owning backend of `b` (a shared session):
+        its published arena is attached instead of another copy being made resident."""
         self.b, self.oracle = b, oracle
         self.streams, self.iterations = streams, iterations
         expanded = hidden * max(streams, 1)
@@ -369,8 +371,12 @@ class MoeCase:
         arena = np.zeros(cursor, np.uint8)
         for name, blob in parts.items():
             arena[offsets[name]:offsets[name] + blob.nbytes] = blob
-        arena_tensor, host = b.resident(arena)
-        self.host, self.offsets, self.arena_tensor = host, offsets, arena_tensor
+        if arena_from is None:
+            arena_tensor, host = b.resident(arena)
+        else:
+            arena_tensor, host = arena_from.arena_tensor, arena_from.host
+            assert b.attach_shared_arena(arena_tensor, host, arena.nbytes) == 0, b.err.message
+        self.host, self.offsets, self.arena_tensor, self.arena_bytes = host, offsets, arena_tensor, arena.nbytes
         self.x = g.normal(rows * expanded).reshape(rows, expanded)
         if streams:
             bits = self.x.view(np.uint32)       # bf16 values, as the CPU path expects of its input
@@ -605,6 +611,49 @@ def test_worklist_policy_decides_the_matrix_core_regime(backend, oracle, minimum
     assert res.worklists.narrow_pairs == (0 if matrix else pairs)
     got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
     same_as_cpu(got, case.oracle_layer(act_q8=True)["combined"])
+
+
+def test_shared_sessions_run_row_batches_against_one_arena(backend, oracle):
+    """Sessions that share one set of resident weights (yvex_backend_open_shared_cuda,
+    include/yvex/internal/backend.h:254-255; the runtime opens one per session and attaches the
+    model-owned arena, src/runtime/residency.c:1463-1469): two children of one owning backend
+    attach its arena without another upload and issue row batches in turn, each on its own
+    stream, workspace and launch graphs. Their rows are bit for bit the owner's own."""
+    from yvex_amd.host import Backend
+    owner_case = MoeCase(backend, oracle, rows=7, scoring=abi.SCORING_SIGMOID)
+    backend.workspace(owner_case.workspace_bytes)
+    assert owner_case.execute() == 0, owner_case.err.message
+    want = backend.read_f32(owner_case.rows_out, 7 * owner_case.hidden).reshape(7, owner_case.hidden).copy()
+    same_as_cpu(want, owner_case.oracle_layer(act_q8=True)["combined"])
+    children = [Backend(shared_with=backend), Backend(shared_with=backend)]
+    try:
+        assert all(c.ok for c in children)
+        # a shared session is not an owner, and the arena must be the one the owner attached
+        grandchild = Backend(shared_with=children[0])
+        assert grandchild.open_rc == abi.INVALID_ARG and not grandchild.handle.value
+        assert children[0].attach_shared_arena(owner_case.arena_tensor, owner_case.host, owner_case.arena_bytes,
+                                               generation=2) == abi.STATE
+        cases = [MoeCase(children[0], oracle, rows=7, scoring=abi.SCORING_SIGMOID, arena_from=owner_case),
+                 MoeCase(children[1], oracle, rows=5, scoring=abi.SCORING_SIGMOID, arena_from=owner_case)]
+        for child, case in zip(children, cases):
+            child.workspace(case.workspace_bytes)
+            stats = abi.MemoryStats()
+            assert child.lib.yvex_rocm_backend_get_memory_stats(child.handle, C.byref(stats), C.byref(child.err)) == 0
+            assert stats.h2d_bytes < owner_case.arena_bytes        # rows only: the arena was not uploaded again
+        for turn in range(4):       # first sight, recording, two replays, interleaved
+            for case in cases:
+                assert case.execute() == 0, case.err.message
+                got = case.b.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+                assert np.array_equal(got.view(np.uint32), want[:case.rows].view(np.uint32)), turn
+        assert cases[0].result.graph_replays == 1 and cases[1].result.graph_replays == 1
+        # the owner keeps working beside them
+        assert owner_case.execute() == 0, owner_case.err.message
+        again = backend.read_f32(owner_case.rows_out, 7 * owner_case.hidden).reshape(7, owner_case.hidden)
+        assert np.array_equal(again.view(np.uint32), want.view(np.uint32))
+    finally:
+        for child in children:
+            if child.handle.value:
+                assert child.close() == 0, child.err.message
 
 
 def test_execute_rows_refusals(backend, oracle):

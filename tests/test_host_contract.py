@@ -328,3 +328,39 @@ def test_host_worklist_matches_oracle_and_refuses(lib, oracle):
     storage.pair_capacity = pairs - 1
     assert lib.yvex_rocm_expert_worklist_build(sel.ctypes.data, w.ctypes.data, pairs, topk, experts,
                                           C.byref(storage), C.byref(obs), C.byref(err)) == abi.INVALID_ARG
+
+
+
+def test_shared_sessions_borrow_the_owner(monkeypatch):
+    """yvex_backend_open_shared_cuda's contract (src/backend/cuda/backend.c:1913-2000,
+    src/backend/residency.c:47-57, src/backend/core.c:251-343) on the host-only backend: a child
+    needs an owning backend, attaches the arena its owner published (same base and generation,
+    the owner's device address, no copy), keeps tensors and a workspace of its own, and the
+    owner does not close while a child is open."""
+    monkeypatch.setenv("YVEX_TEST_ROCM_NO_DEVICE", "1")
+    from yvex_amd.host import Backend
+    owner = Backend()
+    assert owner.ok
+    blob = np.arange(4096, dtype=np.uint8)
+    arena, host = owner.resident(blob, generation=5)
+    child = Backend(shared_with=owner, memory_limit=1 << 20)
+    assert child.ok and child.lib.yvex_rocm_backend_kind_of(child.handle) == abi.KIND_ROCM
+    assert Backend(shared_with=child).open_rc == abi.INVALID_ARG
+    # the owner's arena: wrong generation, wrong base, then the matching attach
+    assert child.attach_shared_arena(arena, host, blob.nbytes, generation=4) == abi.STATE
+    assert child.attach_shared_arena(arena, host + 256, blob.nbytes - 256, generation=5) == abi.STATE
+    assert child.attach_shared_arena(arena, host, blob.nbytes, generation=5) == 0, child.err.message
+    assert child.attach_shared_arena(arena, host, blob.nbytes, generation=5) == abi.STATE      # already attached
+    mine, theirs = abi.ULL(), abi.ULL()
+    for b, out in ((owner, theirs), (child, mine)):
+        assert b.lib.yvex_rocm_backend_resident_resolve(b.handle, C.c_void_p(host + 100), 50, C.byref(out)) == abi.RESIDENT_HIT
+    assert mine.value == theirs.value
+    # tensors belong to the session that allocated them, under its own limit
+    rc, t = child.tensor(1024)
+    assert rc == 0 and t.contents.owner == child.handle.value
+    assert child.tensor(2 << 20)[0] == abi.NOMEM
+    assert owner.lib.yvex_rocm_backend_tensor_write(owner.handle, t, blob.ctypes.data, 1024, C.byref(owner.err)) != 0
+    # the owner waits for its sessions
+    assert owner.close() == abi.STATE and owner.handle.value
+    assert child.close() == 0, child.err.message
+    assert owner.close() == 0, owner.err.message

@@ -32,6 +32,7 @@ def binding(oracle):
         pytest.skip("the reference tree is not here and oracle/_ref/libyvex_ref_backend.so was not shipped")
     P, ULL = C.c_void_p, C.c_ulonglong
     lib.yvex_backend_open_rocm_impl.argtypes = [C.POINTER(P), C.c_char_p, ULL, P]
+    lib.yvex_backend_open_shared_rocm.argtypes = [C.POINTER(P), P, ULL, P]
     lib.yvex_backend_close_checked.argtypes = [C.POINTER(P), P]
     lib.yvex_backend_kind_of.argtypes = [P]
     lib.yvex_backend_status_of.argtypes = [P]
@@ -59,9 +60,12 @@ def binding(oracle):
 class Reference:
     """A backend opened by the adapter, used through the reference's generic entry points."""
 
-    def __init__(self, lib):
+    def __init__(self, lib, shared_with=None):
         self.lib, self.handle, self.err = lib, C.c_void_p(), abi.Error()
-        rc = lib.yvex_backend_open_rocm_impl(C.byref(self.handle), None, 0, C.byref(self.err))
+        if shared_with is None:
+            rc = lib.yvex_backend_open_rocm_impl(C.byref(self.handle), None, 0, C.byref(self.err))
+        else:
+            rc = lib.yvex_backend_open_shared_rocm(C.byref(self.handle), shared_with.handle, 0, C.byref(self.err))
         assert rc == 0, self.err.message
         assert lib.yvex_backend_kind_of(self.handle) == abi.KIND_ROCM
 
@@ -156,6 +160,36 @@ def run_sequence(lib, oracle, with_gpu):
             assert rc == abi.UNSUPPORTED and b"kernel" in ref.err.message.lower()
             assert out.contents.is_written == 0
             assert not lib.yvex_backend_rocm_moe_operations_get(ref.handle)
+        # a shared session (yvex_backend_open_shared_cuda's counterpart in the adapter): the
+        # reference's generic attach gives it the owner's arena (src/backend/residency.c:47-57),
+        # the adapter carries that over, and the owner cannot close under it
+        session = Reference(lib, shared_with=ref)
+        assert lib.yvex_backend_resident_attach(session.handle, mapped, encoded.nbytes, resident, 17,
+                                                session.e()) == 0, session.err.message
+        assert lib.yvex_backend_resident_resolve(session.handle, inner, row_bytes, C.byref(device)) == abi.RESIDENT_HIT
+        assert device.value == base + 3 * row_bytes
+        s_in = session.tensor(b"session-input", abi.DTYPE_F32, WIDTH * 4, WIDTH)
+        s_out = session.tensor(b"session-output", abi.DTYPE_F32, ROWS * 4, ROWS)
+        assert lib.yvex_backend_tensor_write(session.handle, s_in, x.ctypes.data, x.nbytes, session.e()) == 0
+        rc = lib.yvex_backend_rocm_encoded_matvec(session.handle, mapped, encoded.nbytes, qt, ROWS, WIDTH, row_bytes,
+                                                  1, s_in, None, 0, None, s_out, 0, C.byref(facts), session.e())
+        if with_gpu:
+            assert rc == 0, session.err.message
+            got = np.empty(ROWS, np.float32)
+            assert lib.yvex_backend_tensor_read(session.handle, s_out, got.ctypes.data, got.nbytes, session.e()) == 0
+            want = oracle.matvec(qt, encoded, ROWS, WIDTH, x)[0]
+            assert np.all(np.abs(got - want) <= 1e-5 + 1e-3 * np.abs(want))
+        else:
+            assert rc == abi.UNSUPPORTED
+        # the owner's input belongs to the owner, not to the session
+        assert lib.yvex_backend_rocm_encoded_matvec(session.handle, mapped, encoded.nbytes, qt, ROWS, WIDTH, row_bytes,
+                                                    1, inp, None, 0, None, s_out, 0, C.byref(facts),
+                                                    session.e()) == abi.FORMAT
+        for t in (s_in, s_out):
+            assert lib.yvex_backend_tensor_release(session.handle, C.byref(t), session.e()) == 0
+        # src/backend/core.c:610-634: while a session is open the owner releases nothing it may borrow
+        assert lib.yvex_backend_tensor_release(ref.handle, C.byref(resident), ref.e()) == abi.STATE and resident
+        session.close()
         # a tensor of another backend is refused by the ownership check behind the adapter
         other = Reference(lib)
         foreign = other.tensor(b"foreign", abi.DTYPE_F32, WIDTH * 4, WIDTH)

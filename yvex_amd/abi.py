@@ -281,7 +281,7 @@ class WorklistStorage(C.Structure):
 EXPORTS = [
     "yvex_rocm_status_name", "yvex_rocm_error_clear", "yvex_rocm_error_set", "yvex_rocm_error_is_set", "yvex_rocm_error_code",
     "yvex_rocm_gguf_qtype_geometry_find", "yvex_rocm_quant_numeric_capability_at",
-    "yvex_rocm_backend_open", "yvex_rocm_backend_bind_owner", "yvex_rocm_backend_close_checked", "yvex_rocm_backend_kind_of",
+    "yvex_rocm_backend_open", "yvex_rocm_backend_bind_owner", "yvex_rocm_backend_close_checked", "yvex_rocm_backend_open_shared", "yvex_rocm_backend_kind_of",
     "yvex_rocm_backend_status_of", "yvex_rocm_backend_get_memory_stats", "yvex_rocm_backend_sync",
     "yvex_rocm_backend_query_capability", "yvex_rocm_backend_bandwidth_probe", "yvex_rocm_backend_tensor_alloc", "yvex_rocm_backend_tensor_release",
     "yvex_rocm_backend_tensor_write", "yvex_rocm_backend_tensor_read", "yvex_rocm_backend_tensor_copy",
@@ -362,6 +362,7 @@ def library():
     lib.yvex_rocm_backend_moe_close.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
     lib.yvex_rocm_backend_open.argtypes = [C.POINTER(C.c_void_p), C.POINTER(BackendOptions), C.POINTER(Error)]
     lib.yvex_rocm_backend_close_checked.argtypes = [C.POINTER(C.c_void_p), C.POINTER(Error)]
+    lib.yvex_rocm_backend_open_shared.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, ULL, C.POINTER(Error)]
     lib.yvex_rocm_backend_tensor_alloc.argtypes = [C.c_void_p, C.POINTER(TensorDesc),
                                               C.POINTER(C.POINTER(DeviceTensor)), C.POINTER(Error)]
     lib.yvex_rocm_backend_tensor_release.argtypes = [C.c_void_p, C.POINTER(C.POINTER(DeviceTensor)),

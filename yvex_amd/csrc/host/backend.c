@@ -138,6 +138,57 @@ int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *
     }
     backend->status = backend->kernels_available ? YVEX_BACKEND_STATUS_READY
                                                  : YVEX_BACKEND_STATUS_CONTEXT_READY;
+    backend->resource_owner = backend;
+    *out = backend;
+    yvex_rocm_error_clear(err);
+    return YVEX_OK;
+}
+
+/* Session-local state that borrows one owning backend's device and resident arena
+ * (yvex_backend_open_shared_cuda, src/backend/cuda/backend.c:1913-2000): a stream, a status word,
+ * memory accounting under its own limit, tensors, a workspace and launch graphs of its own. The
+ * owner's arena is attached to the child without another upload (yvex_rocm_backend_resident_attach).
+ * The owner refuses to close while a child is open. One caller at a time per backend, as ever;
+ * different backends of one owner may run from different threads. */
+int yvex_rocm_backend_open_shared(yvex_rocm_backend **out, yvex_rocm_backend *context_owner,
+                                  unsigned long long memory_limit_bytes, yvex_error *err)
+{
+    yvex_rocm_backend *backend;
+    if (out) *out = NULL;
+    if (!out || !context_owner || context_owner->kind != YVEX_BACKEND_KIND_ROCM ||
+        context_owner->resource_owner != context_owner)
+        return yvex_rocm_refuse(err, YVEX_ERR_INVALID_ARG, "rocm.shared.open",
+                                "one owning rocm backend is required");
+    if (context_owner->status == YVEX_BACKEND_STATUS_FAILED)
+        return yvex_rocm_refuse(err, YVEX_ERR_STATE, "rocm.shared.open",
+                                "owning rocm backend became unavailable");
+    backend = (yvex_rocm_backend *)calloc(1, sizeof(*backend));
+    if (!backend)
+        return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.shared.open", "shared rocm session allocation failed");
+    backend->kind = YVEX_BACKEND_KIND_ROCM;
+    backend->owner_id = next_owner_id++;
+    backend->public_owner = backend;
+    backend->device_index = context_owner->device_index;
+    backend->host_only = context_owner->host_only;
+    backend->memory.memory_limit_bytes = memory_limit_bytes;
+    if (!backend->host_only) {
+        void *status_word = NULL;
+        if (yvex_hip_stream_create(&backend->stream) != 0 || yvex_hip_malloc(&status_word, 256u) != 0) {
+            if (backend->stream) yvex_hip_stream_destroy(backend->stream);
+            free(backend);
+            return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.shared.open", yvex_hip_last_error());
+        }
+        backend->device_status = (int *)status_word;
+        backend->kernels_available = context_owner->kernels_available;
+        if (backend->kernels_available &&
+            (yvex_hip_fill_u32(backend->device_status, 0u, 1u, backend->stream) != 0 ||
+             yvex_hip_stream_sync(backend->stream) != 0))
+            backend->kernels_available = 0;
+    }
+    backend->status = backend->kernels_available ? YVEX_BACKEND_STATUS_READY
+                                                 : YVEX_BACKEND_STATUS_CONTEXT_READY;
+    backend->resource_owner = context_owner;
+    __atomic_add_fetch(&context_owner->shared_children, 1ull, __ATOMIC_ACQ_REL);
     *out = backend;
     yvex_rocm_error_clear(err);
     return YVEX_OK;
@@ -155,6 +206,9 @@ int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend_ref, yvex_error 
     if (backend->live_tensors)
         return yvex_rocm_refuse(err, YVEX_ERR_STATE, "backend.close",
                                 "backend still owns live tensors");
+    if (__atomic_load_n(&backend->shared_children, __ATOMIC_ACQUIRE))
+        return yvex_rocm_refuse(err, YVEX_ERR_STATE, "backend.close",
+                                "backend still serves shared sessions");
     if (yvex_rocm_seam("YVEX_TEST_ROCM_CLEANUP_FAILURE")) {
         backend->status = YVEX_BACKEND_STATUS_FAILED;   /* owner kept for a checked retry */
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.close",
@@ -168,6 +222,8 @@ int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend_ref, yvex_error 
             return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.close", yvex_hip_last_error());
         }
     }
+    if (backend->resource_owner && backend->resource_owner != backend)
+        __atomic_sub_fetch(&backend->resource_owner->shared_children, 1ull, __ATOMIC_ACQ_REL);
     free(backend);
     *backend_ref = NULL;
     yvex_rocm_error_clear(err);
@@ -561,6 +617,26 @@ int yvex_rocm_backend_resident_attach(yvex_rocm_backend *backend, const unsigned
 {
     unsigned long long offset;
     int rc;
+    if (backend && backend->resource_owner && backend->resource_owner != backend && host_base && bytes &&
+        tensor && generation && yvex_rocm_tensor_owner_is(backend->resource_owner, tensor)) {
+        /* a shared session attaches the arena its owner has published (src/backend/residency.c:47-57:
+         * same base, same generation, the owner's device address): nothing is uploaded again */
+        const yvex_rocm_backend *owner = backend->resource_owner;
+        if (backend->resident_host_base)
+            return yvex_rocm_refuse(err, YVEX_ERR_STATE, "backend.resident.attach",
+                                    "backend residency mapping is already attached");
+        if (owner->resident_host_base != host_base || owner->resident_host_bytes < bytes ||
+            owner->resident_generation != generation || !owner->resident_device_address)
+            return yvex_rocm_refuse(err, YVEX_ERR_STATE, "backend.resident.attach",
+                                    "the owning backend has no matching resident arena attached");
+        backend->resident_host_base = host_base;
+        backend->resident_host_bytes = bytes;
+        backend->resident_device_tensor = tensor;
+        backend->resident_device_address = owner->resident_device_address;
+        backend->resident_generation = generation;
+        yvex_rocm_error_clear(err);
+        return YVEX_OK;
+    }
     if (!backend || !host_base || !bytes || !tensor || !generation ||
         !yvex_rocm_tensor_owner_is(backend, tensor) || !tensor->host_data ||
         host_base < tensor->host_data)

@@ -36,6 +36,12 @@ struct yvex_rocm_backend {
     int pending_completion;
     /* launch graphs of the row-batch MoE operation, keyed on topology and device addresses */
     struct yvex_rocm_moe_graphs *moe_graphs;
+    /* shared sessions (src/backend/cuda/backend.c:1913-2000): a child borrows the device and the
+     * resident arena of `resource_owner` (itself for an owning backend) and keeps a stream, a
+     * status word, tensors, a workspace and launch graphs of its own; an owner counts its
+     * children and does not close while one is open */
+    struct yvex_rocm_backend *resource_owner;
+    unsigned long long shared_children;
 };
 
 /* Drop every cached launch graph (the stream is idle or was never used). */

@@ -17,6 +17,7 @@
  * a changed attachment over to the library before an operation runs. The library publishes a
  * resident arena to HBM at attach, so the first operation after a new generation pays the upload.
  */
+#include <stdatomic.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -49,6 +50,11 @@ static int rocm_follow(yvex_backend *backend, yvex_error *err)
     if (!impl) {
         yvex_error_set(err, YVEX_ERR_INVALID_ARG, "rocm.adapter", "a ROCm backend is required");
         return YVEX_ERR_INVALID_ARG;
+    }
+    /* a shared session attaches what its owner has published: the owner goes first */
+    if (backend->resource_owner && backend->resource_owner != backend) {
+        rc = rocm_follow(backend->resource_owner, err);
+        if (rc != YVEX_OK) return rc;
     }
     if (impl->resident_generation != backend->resident_generation ||
         impl->resident_tensor != backend->resident_device_tensor) {
@@ -213,7 +219,67 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
     backend->status = yvex_rocm_backend_status_of(impl->backend);
     backend->vtable = &rocm_vtable;
     backend->impl = impl;
+    backend->resource_owner = backend;
+    backend->tensor_id_next = 1ull;
     backend->stats.memory_limit_bytes = memory_limit_bytes;
+    *out = backend;
+    return YVEX_OK;
+}
+
+/* The ROCm counterpart of yvex_backend_open_shared_cuda (include/yvex/internal/backend.h:254-255,
+ * src/backend/cuda/backend.c:1913-2000): session-local state that borrows one model-owned backend.
+ * The lease on the owner is the child count in its lifecycle word, which the reference's
+ * yvex_backend_close_checked releases (src/backend/core.c:283-343). */
+int yvex_backend_open_shared_rocm(yvex_backend **out, yvex_backend *context_owner,
+                                  unsigned long long memory_limit_bytes, yvex_error *err)
+{
+    yvex_backend *backend;
+    rocm_impl *impl, *owner_impl = rocm_of(context_owner);
+    unsigned long long observed;
+    int rc;
+    if (out) *out = NULL;
+    if (!out || !owner_impl || context_owner->resource_owner != context_owner) {
+        yvex_error_set(err, YVEX_ERR_INVALID_ARG, "rocm.shared.open", "one owning ROCm backend is required");
+        return YVEX_ERR_INVALID_ARG;
+    }
+    backend = (yvex_backend *)calloc(1u, sizeof(*backend));
+    impl = (rocm_impl *)calloc(1u, sizeof(*impl));
+    if (!backend || !impl) {
+        free(backend);
+        free(impl);
+        yvex_error_set(err, YVEX_ERR_NOMEM, "rocm.shared.open", "shared ROCm session allocation failed");
+        return YVEX_ERR_NOMEM;
+    }
+    observed = atomic_load_explicit(&context_owner->lifecycle, memory_order_acquire);
+    for (;;) {
+        if (observed & YVEX_BACKEND_LIFECYCLE_CLOSING) {
+            free(backend);
+            free(impl);
+            yvex_error_set(err, YVEX_ERR_STATE, "rocm.shared.open", "owning ROCm backend is closing");
+            return YVEX_ERR_STATE;
+        }
+        if (atomic_compare_exchange_weak_explicit(&context_owner->lifecycle, &observed, observed + 1ull,
+                                                  memory_order_acq_rel, memory_order_acquire))
+            break;
+    }
+    rc = yvex_rocm_backend_open_shared(&impl->backend, owner_impl->backend, memory_limit_bytes, err);
+    if (rc == YVEX_OK) rc = yvex_rocm_backend_bind_owner(impl->backend, backend, err);
+    if (rc != YVEX_OK) {
+        if (impl->backend) (void)yvex_rocm_backend_close_checked(&impl->backend, NULL);
+        atomic_fetch_sub_explicit(&context_owner->lifecycle, 1ull, memory_order_acq_rel);
+        free(impl);
+        free(backend);
+        return rc;
+    }
+    backend->kind = YVEX_BACKEND_KIND_ROCM;
+    backend->status = yvex_rocm_backend_status_of(impl->backend);
+    backend->vtable = &rocm_vtable;
+    backend->impl = impl;
+    backend->resource_owner = context_owner;
+    backend->shared_owner_registered = 1;
+    backend->tensor_id_next = 1ull;
+    backend->stats.memory_limit_bytes = memory_limit_bytes;
+    backend->device_info = context_owner->device_info;
     *out = backend;
     return YVEX_OK;
 }

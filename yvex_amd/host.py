@@ -9,13 +9,24 @@ from . import abi
 
 
 class Backend:
-    def __init__(self, memory_limit=0):
+    def __init__(self, memory_limit=0, shared_with=None):
+        """An owning backend, or (shared_with = an owning Backend) a session that borrows its
+        device and resident arena (yvex_rocm_backend_open_shared)."""
         self.lib = abi.library()
         self.handle = C.c_void_p()
         self.err = abi.Error()
-        opts = abi.BackendOptions(abi.KIND_ROCM, None, memory_limit)
-        self.open_rc = self.lib.yvex_rocm_backend_open(C.byref(self.handle), C.byref(opts), C.byref(self.err))
+        if shared_with is None:
+            opts = abi.BackendOptions(abi.KIND_ROCM, None, memory_limit)
+            self.open_rc = self.lib.yvex_rocm_backend_open(C.byref(self.handle), C.byref(opts), C.byref(self.err))
+        else:
+            self.open_rc = self.lib.yvex_rocm_backend_open_shared(C.byref(self.handle), shared_with.handle,
+                                                                  memory_limit, C.byref(self.err))
         self.tensors = []
+
+    def attach_shared_arena(self, owner_tensor, host_base, nbytes, generation=1):
+        """Attach the arena the owning backend has published: nothing is uploaded again."""
+        return self.lib.yvex_rocm_backend_resident_attach(self.handle, C.c_void_p(host_base), nbytes, owner_tensor,
+                                                          generation, C.byref(self.err))
 
     @property
     def ok(self):
