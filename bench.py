@@ -173,6 +173,48 @@ def cpu_baseline_reference(sample_rows: int):
             "tokens_per_s": sample_rows / seconds, "seconds": seconds}
 
 
+def cpu_baseline_dense():
+    """BASELINE configs 0-2 on the host: one pass of the whole matrix against one F32 input row
+    through the reference's own yvex_quant_cpu_dot (compiled from its sources into oracle/_ref;
+    one core, row by row, as src/graph/core.c:1131-1166 calls it), or through the C restatement
+    where the reference has no codec (Q4_K) or its library is absent. A batch of b rows costs b
+    such passes on the CPU path: it has no batched form."""
+    import ctypes as C
+    import numpy as np
+    import oracle
+    ref = oracle.ref_lib()
+    if ref is not None:
+        ref.yvex_quant_cpu_dot.argtypes = [C.c_uint, C.c_void_p, C.c_size_t, C.c_void_p, C.c_ulonglong,
+                                           C.c_void_p, C.c_void_p, C.c_void_p]
+    out = {}
+    g = oracle.Generator(42, "bench.cpu.dense")
+    for name, qt, rows, width in (("cfg0_q8_0_4096x4096", oracle.Q8_0, 4096, 4096),
+                                  ("cfg1_q4_k_2048x7168", oracle.Q4_K, 2048, 7168),
+                                  ("cfg2_iq2_xxs_7168x2048", oracle.IQ2_XXS, 7168, 2048)):
+        w = g.weights(qt, rows, width)
+        x = g.normal(width)
+        row_bytes = oracle.row_bytes(qt, width)
+        use_ref = ref is not None and qt != oracle.Q4_K
+        t0 = time.perf_counter()
+        if use_ref:
+            y, failure, err = C.c_float(), (C.c_ubyte * 512)(), (C.c_ubyte * 512)()
+            base = w.ctypes.data
+            for r in range(rows):
+                if ref.yvex_quant_cpu_dot(qt, base + r * row_bytes, row_bytes, x.ctypes.data, width, C.byref(y),
+                                          failure, err) != 0:
+                    use_ref = False
+                    break
+        if not use_ref:
+            t0 = time.perf_counter()
+            oracle.matvec(qt, w, rows, width, x)
+        seconds = time.perf_counter() - t0
+        out[name] = {"ms": round(seconds * 1e3, 3), "GB_per_s": round(w.nbytes / seconds / 1e9, 4),
+                     "cores": 1, "kind": "reference" if use_ref else "port",
+                     "sample": "the whole matrix against one F32 input row"
+                               + ("" if use_ref or qt != oracle.Q4_K else " (the reference refuses Q4_K: C restatement)")}
+    return out
+
+
 def AbiLayer(torch, routed, shared, router, x_host, rows, qtype=16, sweep_image=False):
     """The benchmark layer behind include/yvex_rocm.h (yvex_amd.host.RowBatchLayer at this
     benchmark's shape)."""
@@ -733,6 +775,21 @@ def main() -> int:
         if reference:
             out["cpu_baseline_port"] = port
         out["cpu_baseline_all_cores"] = cpu_baseline(max(args.cpu_rows, 8), min(16, os.cpu_count() or 1))
+        # The CPU path runs a prefill row exactly as a decode row (top-8 + shared expert FFNs, an
+        # expert's bytes decoded again for every row: src/runtime/moe.c:596-632 has no batched
+        # form), so the sample above is a sample of the prefill batch too, extrapolated linearly.
+        base = out["cpu_baseline"]
+        pair_ops = 2 * (2 * INTERMEDIATE * HIDDEN + HIDDEN * INTERMEDIATE)
+        for leg in ("prefill", "prefill_q4k"):
+            if isinstance(out.get(leg), dict) and "error" not in out[leg]:
+                out[leg]["cpu_baseline"] = {
+                    "value": round(pair_ops * (TOPK + 1) * base["tokens_per_s"] / 1e12, 6), "unit": "TOP/s",
+                    "tokens_per_s": round(base["tokens_per_s"], 4), "cores": base["cores"], "kind": base["kind"],
+                    "sample": base["sample"] + " (IQ2_XXS experts); a 2048-row batch is 2048 such rows, "
+                              "extrapolated linearly",
+                    "extrapolated_step_seconds": round(2048 / base["tokens_per_s"], 1)}
+        if isinstance(out.get("dense"), dict):
+            out["dense"]["cpu_baseline"] = cpu_baseline_dense()
     print(json.dumps(out))
     return 0
 
