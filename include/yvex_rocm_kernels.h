@@ -316,6 +316,9 @@ int yvex_hip_free(void *ptr);
 int yvex_hip_host_alloc(void **out, uint64_t bytes);
 int yvex_hip_host_free(void *ptr);
 int yvex_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
+/* The same copy queued on the stream without waiting for it: `src` is pinned host memory
+ * (yvex_hip_host_alloc) that stays untouched until the stream has passed the copy. */
+int yvex_hip_memcpy_h2d_queued(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
 int yvex_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
 int yvex_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream);
 int yvex_hip_stream_create(yvex_hip_stream *out);

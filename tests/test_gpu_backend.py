@@ -816,6 +816,31 @@ def test_deferred_batches_keep_what_an_earlier_one_raised(backend, oracle):
     assert done.completed == 1
 
 
+def test_deferred_hash_routed_batches_keep_their_own_token_ids(backend, oracle):
+    """Two hash-routed batches behind one barrier, the caller's token buffer rewritten as soon as
+    each call returns: the ids travel through the backend's pinned memory, so each batch routes by
+    the ids it was given although neither call waited for the stream."""
+    case = MoeCase(backend, oracle, hidden=512, rows=6, iterations=4, hash_vocab=40)
+    backend.workspace(case.workspace_bytes)
+    completion = abi.DeviceCompletion(1, None)
+    case.job.device_completion = C.pointer(completion)
+    first = case.tokens.copy()
+    second = ((first + 7) % 40).astype(np.uint32)
+    outputs = [case.rows_out, backend.empty_f32(case.rows * case.hidden)]
+    for ids, out in zip((first, second), outputs):
+        case.tokens[:] = ids
+        case.batch.device_outputs = out
+        assert case.execute() == 0, case.err.message
+        assert case.result.device_completion_pending == 1
+        case.tokens[:] = 39 - ids          # the caller reuses its buffer at once
+    done, err = abi.RowBatchResult(), abi.Error()
+    assert case.ops.complete_rows(backend.handle, 0, C.byref(done), C.byref(err)) == 0, err.message
+    for ids, out in zip((first, second), outputs):
+        case.tokens[:] = ids
+        got = backend.read_f32(out, case.rows * case.hidden).reshape(case.rows, case.hidden)
+        same_as_cpu(got, case.oracle_layer(act_q8=True)["combined"])
+
+
 @pytest.mark.parametrize("imaged,rows,experts", [
     (("routed", "shared"), 5, 8), (("routed",), 7, 8), (("shared",), 6, 8), (("routed", "shared"), 40, 4)])
 def test_execute_rows_runs_the_sweep_image(backend, oracle, imaged, rows, experts):

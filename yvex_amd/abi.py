@@ -312,7 +312,7 @@ KERNEL_EXPORTS = [
     "yvex_hip_capture_begin", "yvex_hip_capture_end", "yvex_hip_capture_abort", "yvex_hip_graph_launch",
     "yvex_hip_graph_destroy",
     "yvex_hip_device_count", "yvex_hip_device_info", "yvex_hip_device_clocks", "yvex_hip_malloc", "yvex_hip_free",
-    "yvex_hip_host_alloc", "yvex_hip_host_free", "yvex_hip_memcpy_h2d", "yvex_hip_memcpy_d2h",
+    "yvex_hip_host_alloc", "yvex_hip_host_free", "yvex_hip_memcpy_h2d", "yvex_hip_memcpy_h2d_queued", "yvex_hip_memcpy_d2h",
     "yvex_hip_memcpy_d2d", "yvex_hip_stream_create", "yvex_hip_stream_destroy",
     "yvex_hip_stream_sync", "yvex_hip_kernels_loadable", "yvex_hip_last_error",
 ]

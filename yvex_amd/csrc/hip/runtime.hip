@@ -190,6 +190,12 @@ int yvex_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes, yvex_hip_str
                   hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
     return rc ? rc : wrap("hipStreamSynchronize", hipStreamSynchronize(as_stream(stream)));
 }
+int yvex_hip_memcpy_h2d_queued(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream)
+{
+    if (!bytes) return ST_OK;
+    return wrap("hipMemcpyAsync(h2d)",
+                hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+}
 int yvex_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes, yvex_hip_stream stream)
 {
     if (!bytes) return ST_OK;

@@ -84,6 +84,36 @@ int yvex_rocm_finish(yvex_rocm_backend *backend, const char *where, int *device_
     return YVEX_OK;
 }
 
+int yvex_rocm_upload_queued(yvex_rocm_backend *backend, void *device, const void *host,
+                            unsigned long long bytes)
+{
+    const unsigned long long piece = (bytes + 63ull) & ~63ull;
+    if (!bytes) return 0;
+    /* nothing deferred: every earlier copy out of the staging memory has been waited for */
+    if (!backend->pending_completion) backend->token_staging_cursor = 0ull;
+    if (backend->token_staging_cursor == 0ull && backend->token_staging_bytes < piece) {
+        unsigned long long want = piece < (64ull << 10) ? (64ull << 10) : piece * 2ull;
+        void *fresh = NULL;
+        if (yvex_hip_stream_sync(backend->stream) != 0) return -1;
+        if (backend->token_staging) (void)yvex_hip_host_free(backend->token_staging);
+        backend->token_staging = NULL;
+        backend->token_staging_bytes = 0ull;
+        if (yvex_hip_host_alloc(&fresh, want) == 0) {
+            backend->token_staging = (unsigned char *)fresh;
+            backend->token_staging_bytes = want;
+        }
+    }
+    if (!backend->token_staging ||
+        backend->token_staging_bytes - backend->token_staging_cursor < piece)
+        return yvex_hip_memcpy_h2d(device, host, bytes, backend->stream);   /* waits for the copy */
+    memcpy(backend->token_staging + backend->token_staging_cursor, host, (size_t)bytes);
+    if (yvex_hip_memcpy_h2d_queued(device, backend->token_staging + backend->token_staging_cursor, bytes,
+                                   backend->stream) != 0)
+        return -1;
+    backend->token_staging_cursor += piece;
+    return 0;
+}
+
 int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *options, yvex_error *err)
 {
     yvex_rocm_backend *backend;
@@ -216,7 +246,12 @@ int yvex_rocm_backend_close_checked(yvex_rocm_backend **backend_ref, yvex_error 
     }
     if (!backend->host_only) {
         if (yvex_hip_stream_sync(backend->stream) == 0) yvex_rocm_moe_graphs_release(backend);
-        if (yvex_hip_stream_sync(backend->stream) != 0 || yvex_hip_free(backend->device_status) != 0 ||
+        if (yvex_hip_stream_sync(backend->stream) == 0 && yvex_hip_host_free(backend->token_staging) == 0) {
+            backend->token_staging = NULL;
+            backend->token_staging_bytes = 0ull;
+        }
+        if (yvex_hip_stream_sync(backend->stream) != 0 || backend->token_staging ||
+            yvex_hip_free(backend->device_status) != 0 ||
             yvex_hip_stream_destroy(backend->stream) != 0) {
             backend->status = YVEX_BACKEND_STATUS_FAILED;
             return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "backend.close", yvex_hip_last_error());

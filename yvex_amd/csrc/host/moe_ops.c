@@ -687,9 +687,10 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     stream = backend->stream;
 #define AT(field) ((void *)(uintptr_t)(base + ranges.field))
     /* token ids come from the caller's host buffer on every call, so they travel ahead of the
-     * kernels and never inside a graph */
-    if (hash_router && yvex_hip_memcpy_h2d(AT(tokens), rows->token_ids, row_count * sizeof(unsigned int),
-                                           stream) != 0)
+     * kernels and never inside a graph; they pass through pinned memory of the backend, so a
+     * deferred batch queues the copy and returns without waiting for the stream */
+    if (hash_router && yvex_rocm_upload_queued(backend, AT(tokens), rows->token_ids,
+                                               row_count * sizeof(unsigned int)) != 0)
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.token-ids", yvex_hip_last_error());
     /* The kernels' status word is cleared where a phase starts, not per batch: a batch whose
      * completion is deferred leaves what it raised for the barrier to find, whatever runs behind

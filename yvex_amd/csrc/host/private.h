@@ -42,6 +42,11 @@ struct yvex_rocm_backend {
      * children and does not close while one is open */
     struct yvex_rocm_backend *resource_owner;
     unsigned long long shared_children;
+    /* pinned host memory the token ids of hash-routed row batches are copied through, so that the
+     * upload is queued on the stream instead of waited for; deferred batches each take a fresh
+     * piece, and the cursor returns to the start once nothing is pending on the stream */
+    unsigned char *token_staging;
+    unsigned long long token_staging_bytes, token_staging_cursor;
 };
 
 /* Drop every cached launch graph (the stream is idle or was never used). */
@@ -60,6 +65,10 @@ int yvex_rocm_finish(yvex_rocm_backend *backend, const char *where, int *device_
 /* Clear the status word on the stream, unless deferred row batches are waiting for their barrier. */
 int yvex_rocm_status_reset(yvex_rocm_backend *backend, const char *where, yvex_error *err);
 /* Resolve a weight view: device_address if given, else the resident arena mapping. */
+/* Queue `bytes` of caller-owned host memory for upload to `device` on the backend's stream; the
+ * caller's buffer may be reused as soon as this returns. */
+int yvex_rocm_upload_queued(yvex_rocm_backend *backend, void *device, const void *host,
+                            unsigned long long bytes);
 int yvex_rocm_resolve(const yvex_rocm_backend *backend, const unsigned char *host,
                       unsigned long long bytes, unsigned long long *device_address);
 
