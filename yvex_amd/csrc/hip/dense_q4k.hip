@@ -8,7 +8,8 @@
 //     dot     = sum_j sc_j * sum_{i in sub-block j} nibble_i * a_i        (int32, exact)
 //     minimum = sum_j m_j  * (bsums[2j] + bsums[2j+1])                    (int32, exact)
 //     value   = (d_a * d) * float(dot) - (d_a * dmin) * float(minimum)    (two products, one subtraction)
-// and the superblock values of a row are added in fp32.
+// and the superblock values of a row are added in double and rounded to float once, as the
+// CPU path adds a row's blocks (src/gguf/quant_compute.c:152-172).
 //
 // A 32-value sub-block is exactly the reduction depth of V_MFMA_I32_32X32X32_I8. The weight
 // operand carries sc_j * nibble (at most 63 * 15 = 945) as two int8 limbs, value = 8 hi + lo
@@ -18,7 +19,7 @@
 // against the pair sums of bsums, in two limbs of base 128) through the same instruction.
 //
 // A workgroup owns 32 weight rows x 32 or 64 tokens; its four waves take every fourth
-// superblock and their fp32 partial tiles are added in wave order, so results do not depend on
+// superblock and their double-precision partial tiles are added in wave order, so results do not depend on
 // timing. Lane (r, h) of a wave holds bytes 16h..16h+15 of weight row r's sub-block as the A
 // operand and the same bytes of token r's activations as the B operand; accumulator i of that
 // lane is weight row 8 (i / 4) + 4 h + i % 4 against token r.
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
 {
     // per wave: d and dmin of its 32 rows for the superblock in hand; then the partial tiles
     __shared__ __align__(16) float row_scale[4][2][32];
-    __shared__ float partial[3][NT][16][64];
+    __shared__ double partial[3][NT][16][64];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
     const unsigned long long row0 = (unsigned long long)blockIdx.x * 32ull;
@@ -140,11 +141,11 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
         if (t >= g.input_rows) t = g.input_rows - 1ull;
         arow[nt] = g.act + t * act_row_bytes;
     }
-    float acc[NT][16];
+    double acc[NT][16];
 #pragma unroll
     for (unsigned nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0;
 
     SuperInputs<NT> cur;
     if (wave < g.blocks) load_super<NT>(g, wrow, arow, wave, h, cur);
@@ -232,7 +233,7 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
                 const int minimum = (min_hi[nt][i] << 7) + min_lo[nt][i];
                 const float left = (da * d_of[i]) * (float)dot;
                 const float right = (da * dmin_of[i]) * (float)minimum;
-                acc[nt][i] += left - right;
+                acc[nt][i] += (double)(left - right);
             }
         }
         cur = nxt;
@@ -252,8 +253,8 @@ __global__ __launch_bounds__(256) void dense_q4k_kernel(DenseQ4kArgs g)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const unsigned long long row = row0 + 8u * (i >> 2) + 4u * h + (i & 3);
-            const float sum = ((acc[nt][i] + partial[0][nt][i][lane]) + partial[1][nt][i][lane]) +
-                              partial[2][nt][i][lane];
+            const float sum = (float)(((acc[nt][i] + partial[0][nt][i][lane]) + partial[1][nt][i][lane]) +
+                                      partial[2][nt][i][lane]);
             if (row >= g.row_count || token >= g.input_rows) continue;
             const unsigned long long at = token * g.out_stride + row;
             const float value = g.additive ? sum + g.additive[at] : sum;
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
 {
     typedef int v4s __attribute__((ext_vector_type(4)));
     __shared__ __align__(16) float row_scale[8][2][16];
-    __shared__ float partial[7][NT][4][64];
+    __shared__ double partial[7][NT][4][64];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned r = lane & 15u, q = lane >> 4;
     const unsigned long long row0 = (unsigned long long)blockIdx.x * 16ull;
@@ -292,11 +293,11 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
         if (t >= g.input_rows) t = g.input_rows - 1ull;
         arow[nt] = g.act + t * act_row_bytes;
     }
-    float acc[NT][4];
+    double acc[NT][4];
 #pragma unroll
     for (unsigned nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[nt][i] = 0.0f;
+        for (int i = 0; i < 4; ++i) acc[nt][i] = 0.0;
 
     for (unsigned sb = wave; sb < g.blocks; sb += 8u) {
         const unsigned char *w = wrow + (unsigned long long)sb * 144ull;
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
                 const int minimum = (min_hi[nt][i] << 7) + min_lo[nt][i];
                 const float left = (da[nt] * d_of[i]) * (float)dot;
                 const float right = (da[nt] * dmin_of[i]) * (float)minimum;
-                acc[nt][i] += left - right;
+                acc[nt][i] += (double)(left - right);
             }
     }
 
@@ -405,9 +406,10 @@ __global__ __launch_bounds__(512) void dense_q4k16_kernel(DenseQ4kArgs g)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const unsigned long long row = row0 + 4u * q + (unsigned)i;
-            float sum = acc[nt][i];
+            double wide = acc[nt][i];
 #pragma unroll
-            for (unsigned wv = 0; wv < 7u; ++wv) sum += partial[wv][nt][i][lane];
+            for (unsigned wv = 0; wv < 7u; ++wv) wide += partial[wv][nt][i][lane];
+            const float sum = (float)wide;
             if (row >= g.row_count || token >= g.input_rows) continue;
             const unsigned long long at = token * g.out_stride + row;
             const float value = g.additive ? sum + g.additive[at] : sum;

@@ -8,6 +8,7 @@
 //
 // Behaviour restated from src/backend/cuda/kernels.cu:529-626 (matvec), :784-830 (gather) and
 // src/backend/cuda/kernel_primitives.h:218-255,566-596 (row dots).
+#include <type_traits>
 #include "common.hpp"
 #include "launch.hpp"
 #include "units.hpp"
@@ -78,9 +79,17 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     const unsigned char *wrow = a.encoded + row * a.row_bytes;
     const unsigned units = (unsigned)(a.row_width >> 5);
     const unsigned long long act_row_bytes = (a.row_width >> 8) * kQ8KBytes;
-    float acc[T];
+    // Q8_K activations against superblock formats: a superblock's float term is formed in the
+    // order of the reference's device primitive and the terms of a row are added in double and
+    // rounded once, as the CPU path adds a row's blocks (src/gguf/quant_compute.c:152-172): the
+    // result is that path's, bit for bit. Q8_0 rows (a term per 32 values, not chained through
+    // the eight of a superblock as the primitive chains them) and F32 activations keep float
+    // partial sums, inside the tolerance of the dense projections.
+    constexpr bool kWide = Q8 && UnitTraits<QT>::kIntegerCombine;
+    using Sum = typename std::conditional<kWide, double, float>::type;
+    Sum acc[T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    for (int t = 0; t < T; ++t) acc[t] = (Sum)0;
 
     // Every lane runs the same trip count so the superblock shuffles below stay converged.
     for (unsigned base = 0; base < units; base += 64u * U) {
@@ -111,11 +120,11 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
                         s.dot = group_sum_i32<8>(s.dot);
                         if constexpr (QT != QT_IQ2_XXS) s.min = group_sum_i32<8>(s.min);
                         if (live[j] && (uu[j] & 7u) == 0u)
-                            acc[t] += super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
-                                                        act_scale, s);
+                            acc[t] += (Sum)super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
+                                                             act_scale, s);
                     } else {
                         const float v = q8_0_unit_value(unit[j], act_scale, s.dot);
-                        acc[t] += live[j] ? v : 0.0f;
+                        acc[t] += (Sum)(live[j] ? v : 0.0f);
                     }
                 } else if constexpr (STAGE) {
                     float4 x4[8];
@@ -133,7 +142,15 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     }
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-        float sum = group_sum_f32<64>(acc[t]);
+        float sum;
+        if constexpr (kWide) {
+            double wide = acc[t];
+#pragma unroll
+            for (int offset = 32; offset > 0; offset >>= 1) wide += __shfl_xor(wide, offset, kWave);
+            sum = (float)wide;
+        } else {
+            sum = group_sum_f32<64>(acc[t]);
+        }
         const unsigned long long in = in0 + t;
         if (in >= a.input_rows) continue;
         if constexpr (!Q8) {
@@ -424,8 +441,8 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     // row-batch expert path, as one bucket that holds every input row (the reference turns its
     // tensor-core kernels on from 16 input rows, src/backend/cuda/private.h:461-464; measured
     // here the sweep below stays faster up to 31 rows: 17 us against 22 us for 7168 x 2048 at 16). Same exact
-    // int32 superblock sums and the same fp32 scaling as the sweep below; only the order in
-    // which the superblock terms are added in fp32 differs.
+    // int32 superblock sums and the same float terms as the sweep below, added in double in
+    // superblock order there and here: the same bits.
     if (qtype == QT_IQ2_XXS && input_q8 && input_rows >= 32ull && !additive &&
         out_stride == row_count && row_count % 4ull == 0ull && !((uintptr_t)encoded & 3u) &&
         !(row_bytes & 3ull) && row_width / 32ull <= 64ull * 4ull && !((uintptr_t)out & 15u))
