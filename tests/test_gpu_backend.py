@@ -845,6 +845,24 @@ def test_deferred_hash_routed_batches_keep_their_own_token_ids(backend, oracle):
         same_as_cpu(got, case.oracle_layer(act_q8=True)["combined"])
 
 
+@pytest.mark.parametrize("hidden,intermediate,rows", [(3072, 2048, 5), (2048, 4096, 6), (4096, 3072, 3)])
+def test_sweep_image_at_other_widths(backend, oracle, hidden, intermediate, rows):
+    """Image sweeps at widths where a wavefront holds one row and lanes are left over (3072: 24
+    of 64 lanes hold columns), two rows (4096) or four (2048), in both projections: the CPU
+    layer's bits, and the canonical views' bits."""
+    results = []
+    for image in ((), ("routed", "shared")):
+        case = MoeCase(backend, oracle, hidden=hidden, intermediate=intermediate, experts=8, rows=rows,
+                       sweep_image=image)
+        backend.workspace(case.workspace_bytes)
+        assert case.execute() == 0, case.err.message
+        results.append(case.combined.copy())
+        if image:
+            same_as_cpu(case.combined, case.oracle_layer(act_q8=True)["combined"])
+        backend.release_all()
+    assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32))
+
+
 @pytest.mark.parametrize("imaged,rows,experts", [
     (("routed", "shared"), 5, 8), (("routed",), 7, 8), (("shared",), 6, 8), (("routed", "shared"), 40, 4)])
 def test_execute_rows_runs_the_sweep_image(backend, oracle, imaged, rows, experts):
