@@ -409,6 +409,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
     abi_layer.close()
     harness_ms = step_ms
     step_ms = min(abi_graph_ms, abi_eager_ms)
+    residency = "canonical bytes"
     # IQ2_XXS experts resident as the sweep image only: the matrix-core kernels read it as well
     image = None
     if qt == 16:
@@ -422,6 +423,11 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
         image = {"graph_ms_per_step": round(image_ms, 4), "rows_identical_to_canonical": image_same}
         if not image_same:
             return {"error": "the sweep image and the canonical rows disagree on the matrix-core kernels"}
+        # as for the decode step, the faster residency is the leg's figure (same rows bit for bit;
+        # the operations counted do not depend on it)
+        if image_ms < step_ms:
+            step_ms, residency = image_ms, "sweep image"
+
     pair_ops = 2 * (2 * INTERMEDIATE * HIDDEN + HIDDEN * INTERMEDIATE)
     routed_ops, shared_ops = pair_ops * pairs, pair_ops * rows
     up_ops = 2 * 2 * INTERMEDIATE * HIDDEN * pairs
@@ -430,6 +436,7 @@ def prefill_leg(torch, K, MoeLayer, weights, shared, dev, steps: int, warmup: in
         "workload": f"moe_prefill_{'iq2xxs' if qt == 16 else 'q4k'}: 2048 rows, Zipf(1.1) top-8 of 256 experts + shared, "
                     "Q8_K activations",
         "ms_per_step": round(step_ms, 4), "tokens_per_s": round(rows / (step_ms * 1e-3), 1),
+        "residency": residency,
         "c_abi": {"entry": "yvex_rocm_backend_moe_operations_get()->execute_rows + complete_rows",
                   "graph_ms_per_step": round(abi_graph_ms, 4), "eager_ms_per_step": round(abi_eager_ms, 4),
                   "rows_identical_to_stage_harness": abi_same,
