@@ -24,7 +24,9 @@
 //       words of a scale (16 bytes).
 //   Weight bytes: each wave copies, per superblock, the aligned 68 bytes around the superblock of
 //       each of its 32 rows into an LDS window (GLOBAL_LOAD_LDS_DWORDX4, every cache line
-//       fetched once), two superblocks ahead; the lanes take their records out with LDS reads.
+//       fetched once), two superblocks ahead; the lanes take their records out with LDS reads
+//       (canonical bytes: dword reads of rows 80 bytes apart, four lanes to a bank; the image:
+//       three 16-byte reads from a piece-major window, no two lanes of sixteen on one bank).
 //   B operand (activations): the tile's int8 blocks of one superblock, copied from global memory
 //       straight into LDS, in a ring of stages. 16-byte piece c of token t sits at piece position
 //       c ^ (t % 16), so the 16 lanes that read one fragment column together hit 16 different
@@ -69,11 +71,13 @@ constexpr unsigned kTileStartBase = kPairInfoBase + kTileTokens * 8u;
 constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
 constexpr unsigned kClassListBase = kClassCountBase + 16u;
 constexpr unsigned kTrashBase = kClassListBase + 2u * 256u * 2u;   // 256 bytes nobody reads
-// Weight windows: per wave two buffers; a buffer holds, for each of the wave's 32 rows, the 80
-// bytes (five 16-byte pieces) around one superblock, rows back to back (three copies of 64, 64
-// and 32 lanes fill it).
+// Weight windows: per wave two buffers. Canonical bytes: a buffer holds, for each of the wave's
+// 32 rows, the 80 bytes (five 16-byte pieces) around one superblock, rows back to back (three
+// copies of 64, 64 and 32 lanes fill it). Image: six pieces a row, piece-major (piece p of row r
+// at slot 32 p + r): the three pieces a lane's record lies in are three conflict-free 16-byte
+// reads (three full copies fill it).
 constexpr unsigned kWindowBase = (kTrashBase + 256u + 255u) & ~255u;
-constexpr unsigned kWindowBytes = 32u * 80u;
+constexpr unsigned kWindowBytes = 32u * 96u;
 constexpr unsigned kStageBase = kWindowBase + kRowWaves * 2u * kWindowBytes;
 // activation stages: a ring of 4 / NTB stages of NTB x 32 slots (256 bytes each) + 64 scales
 constexpr unsigned kStageRingBytes = 128u * kActPitch + 4u * 256u;
@@ -179,7 +183,8 @@ struct MfmaNextItem {
 //     every wave passes once all its reads of that stage have returned;
 //   * weights: per wave two windows holding, for each of its 32 rows, the aligned 80 bytes
 //     around one superblock (five 16-byte pieces a row, the fifth ending with the dword that
-//     holds the superblock's last byte, so nothing behind it is touched). Each cache line of a
+//     holds the superblock's last byte, so nothing behind it is touched; the image: six pieces
+//     a row, the three that hold each lane record, stored piece-major). Each cache line of a
 //     row is fetched once; taking the records out of the window is LDS work. Loading the
 //     records lane by lane from global memory touched every row's line four times per
 //     superblock, and the memory pipeline spends about two cycles per line an instruction
@@ -232,11 +237,18 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
     const unsigned char *window_from[3];    // row start + piece offset, of the row this lane copies
 #pragma unroll
     for (unsigned k = 0; k < 3u; ++k) {
-        const unsigned piece = 64u * k + lane;
-        const unsigned served = piece < 160u ? piece : 159u;
-        const unsigned char *from = row_pointer(served / 5u);
-        // (the image's 72-byte records start on dword boundaries: the fifth piece is their last 16 bytes)
-        window_from[k] = from + (served % 5u < 4u ? 16u * (served % 5u) : IMAGE ? 56u : 52u);
+        if constexpr (IMAGE) {
+            // The 72-byte record of a row's superblock is two lane records of 36 bytes (dword
+            // aligned): bytes 0-35 lie in the pieces at 0, 16 and 32, bytes 36-71 in the pieces at
+            // 36, 52 and 56 (the last one ends with the record, so nothing behind it is touched).
+            const unsigned piece = 2u * k + (lane >> 5);        // slot 64 k + lane = 32 piece + row
+            const unsigned at = piece < 3u ? 16u * piece : piece == 3u ? 36u : piece == 4u ? 52u : 56u;
+            window_from[k] = row_pointer(lane & 31u) + at;
+        } else {
+            const unsigned piece = 64u * k + lane;
+            const unsigned served = piece < 160u ? piece : 159u;
+            window_from[k] = row_pointer(served / 5u) + (served % 5u < 4u ? 16u * (served % 5u) : 52u);
+        }
     }
     const unsigned window_base = kWindowBase + wave * 2u * kWindowBytes;
     // Windows past the last superblock: windows 0 and 1 of the next item (by parity, so that a
@@ -252,7 +264,7 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
         const unsigned char *from = IMAGE
             ? window_from[k] + offset
             : (const unsigned char *)((unsigned long long)(window_from[k] + offset) & ~3ull);
-        if (k < 2u) copy_to_lds_16(from, to);
+        if (IMAGE || k < 2u) copy_to_lds_16(from, to);
         else copy_to_lds_16_first32(from, to);
     };
 
@@ -332,16 +344,19 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
     // 0. Window dword 16 is the last dword of the fifth piece.
     auto settle = [&](unsigned sb) {
         if constexpr (IMAGE) {
-            // The lane's record is nine dwords from byte 36 h of the row's 72; window bytes 64-79
-            // hold record bytes 56-71 (the fifth piece), so bytes from 64 on sit 8 further.
-            const unsigned at = window_row + (sb & 1u) * kWindowBytes;
-            auto place = [&](unsigned byte) { return at + byte + (byte >= 64u ? 8u : 0u); };
-            head = lds_read_u32(place(36u * h));
-#pragma unroll
-            for (unsigned g = 0; g < 4u; ++g) {
-                grids[g] = lds_read_u32(place(36u * h + 4u + 8u * g));
-                aux[g] = lds_read_u32(place(36u * h + 8u + 8u * g));
-            }
+            // The lane's record is nine dwords: pieces 3 h and 3 h + 1 whole, and of piece 3 h + 2
+            // the first dword (bytes 32-35 of the row's 72) or the last (bytes 68-71).
+            const unsigned at = window_base + (sb & 1u) * kWindowBytes + (3u * h * 32u + r) * 16u;
+            const v4i first = lds_read_v4i(at), second = lds_read_v4i(at + 512u), third = lds_read_v4i(at + 1024u);
+            head = (unsigned)first[0];
+            grids[0] = (unsigned)first[1];
+            aux[0] = (unsigned)first[2];
+            grids[1] = (unsigned)first[3];
+            aux[1] = (unsigned)second[0];
+            grids[2] = (unsigned)second[1];
+            aux[2] = (unsigned)second[2];
+            grids[3] = (unsigned)second[3];
+            aux[3] = (unsigned)(h ? third[3] : third[0]);
             const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(head & 0xffffu) : 0.0f;
             lds_write_u32(row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
             return;
