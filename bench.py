@@ -8,10 +8,13 @@ single-token rows, Q8_K device activations) over synthetic inputs already reside
 the distinct routed experts hit, divided by the step time.
 
 Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up sweep), timed
-with events on the launch stream; `cpu_baseline` is the CPU oracle timed on the host cores over
-a bounded sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8
-matrix cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, and `dense`
-configs 0-2 and an output head as single matvec launches.
+with events on the launch stream; `cpu_baseline` is the reference's own CPU expert path
+(compiled from its sources; the C restatement beside it) timed on the host cores over a bounded
+sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8 matrix
+cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, and `dense` configs
+0-2 and an output head as single matvec launches; the prefill legs and the dense configs carry a
+CPU baseline of their own (the same sample extrapolated per row; the reference's row dot over
+the whole matrix).
 """
 from __future__ import annotations
 
