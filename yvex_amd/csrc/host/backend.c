@@ -140,7 +140,7 @@ int yvex_rocm_backend_open(yvex_rocm_backend **out, const yvex_backend_options *
     backend = (yvex_rocm_backend *)calloc(1, sizeof(*backend));
     if (!backend) return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "backend.open", "out of host memory");
     backend->kind = YVEX_BACKEND_KIND_ROCM;
-    backend->owner_id = next_owner_id++;
+    backend->owner_id = __atomic_fetch_add(&next_owner_id, 1ull, __ATOMIC_RELAXED);   /* sessions may be opened from several threads */
     backend->public_owner = backend;
     backend->device_index = device;
     backend->host_only = host_only;
@@ -196,7 +196,7 @@ int yvex_rocm_backend_open_shared(yvex_rocm_backend **out, yvex_rocm_backend *co
     if (!backend)
         return yvex_rocm_refuse(err, YVEX_ERR_NOMEM, "rocm.shared.open", "shared rocm session allocation failed");
     backend->kind = YVEX_BACKEND_KIND_ROCM;
-    backend->owner_id = next_owner_id++;
+    backend->owner_id = __atomic_fetch_add(&next_owner_id, 1ull, __ATOMIC_RELAXED);   /* sessions may be opened from several threads */
     backend->public_owner = backend;
     backend->device_index = context_owner->device_index;
     backend->host_only = context_owner->host_only;
