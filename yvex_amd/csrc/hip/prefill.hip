@@ -24,9 +24,9 @@
 //       words of a scale (16 bytes).
 //   Weight bytes: each wave copies, per superblock, the aligned 68 bytes around the superblock of
 //       each of its 32 rows into an LDS window (GLOBAL_LOAD_LDS_DWORDX4, every cache line
-//       fetched once), two superblocks ahead; the lanes take their records out with LDS reads
-//       (canonical bytes: dword reads of rows 80 bytes apart, four lanes to a bank; the image:
-//       three 16-byte reads from a piece-major window, no two lanes of sixteen on one bank).
+//       fetched once), two superblocks ahead; the lanes take their records out with three
+//       16-byte LDS reads from a piece-major window (no two lanes of sixteen on one bank; dword
+//       reads of rows 80 bytes apart put four lanes on a bank).
 //   B operand (activations): the tile's int8 blocks of one superblock, copied from global memory
 //       straight into LDS, in a ring of stages. 16-byte piece c of token t sits at piece position
 //       c ^ (t % 16), so the 16 lanes that read one fragment column together hit 16 different
@@ -71,11 +71,11 @@ constexpr unsigned kTileStartBase = kPairInfoBase + kTileTokens * 8u;
 constexpr unsigned kClassCountBase = kTileStartBase + 260u * 4u;
 constexpr unsigned kClassListBase = kClassCountBase + 16u;
 constexpr unsigned kTrashBase = kClassListBase + 2u * 256u * 2u;   // 256 bytes nobody reads
-// Weight windows: per wave two buffers. Canonical bytes: a buffer holds, for each of the wave's
-// 32 rows, the 80 bytes (five 16-byte pieces) around one superblock, rows back to back (three
-// copies of 64, 64 and 32 lanes fill it). Image: six pieces a row, piece-major (piece p of row r
-// at slot 32 p + r): the three pieces a lane's record lies in are three conflict-free 16-byte
-// reads (three full copies fill it).
+// Weight windows: per wave two buffers of six 16-byte pieces for each of the wave's 32 rows,
+// piece-major (piece p of row r at slot 32 p + r; three full copies fill a buffer): the pieces a
+// lane's record lies in are three conflict-free 16-byte reads. Canonical bytes: the aligned 68
+// bytes around a superblock (pieces at 0, 16, 32, 48 and 52, the sixth repeats the fifth); the
+// image: the two 36-byte lane records (pieces at 0, 16, 32 and at 36, 52, 56).
 constexpr unsigned kWindowBase = (kTrashBase + 256u + 255u) & ~255u;
 constexpr unsigned kWindowBytes = 32u * 96u;
 constexpr unsigned kStageBase = kWindowBase + kRowWaves * 2u * kWindowBytes;
@@ -181,10 +181,10 @@ struct MfmaNextItem {
 //   * activations: a ring of R = 4 / NTB stages of NTB x 32 slots (256 int8 + one scale each);
 //     the copies of superblock sb + R are issued right after the barrier of superblock sb, which
 //     every wave passes once all its reads of that stage have returned;
-//   * weights: per wave two windows holding, for each of its 32 rows, the aligned 80 bytes
+//   * weights: per wave two windows holding, for each of its 32 rows, the aligned 68 bytes
 //     around one superblock (five 16-byte pieces a row, the fifth ending with the dword that
-//     holds the superblock's last byte, so nothing behind it is touched; the image: six pieces
-//     a row, the three that hold each lane record, stored piece-major). Each cache line of a
+//     holds the superblock's last byte, so nothing behind it is touched; the image: the three
+//     pieces that hold each of the two lane records), stored piece-major. Each cache line of a
 //     row is fetched once; taking the records out of the window is LDS work. Loading the
 //     records lane by lane from global memory touched every row's line four times per
 //     superblock, and the memory pipeline spends about two cycles per line an instruction
@@ -245,9 +245,11 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
             const unsigned at = piece < 3u ? 16u * piece : piece == 3u ? 36u : piece == 4u ? 52u : 56u;
             window_from[k] = row_pointer(lane & 31u) + at;
         } else {
-            const unsigned piece = 64u * k + lane;
-            const unsigned served = piece < 160u ? piece : 159u;
-            window_from[k] = row_pointer(served / 5u) + (served % 5u < 4u ? 16u * (served % 5u) : 52u);
+            // The aligned 68 bytes around a superblock lie in the pieces at 0, 16, 32, 48 and 52
+            // (the last ends with the dword that holds the superblock's last byte); the sixth slot
+            // repeats the fifth.
+            const unsigned piece = 2u * k + (lane >> 5);
+            window_from[k] = row_pointer(lane & 31u) + (piece < 4u ? 16u * piece : 52u);
         }
     }
     const unsigned window_base = kWindowBase + wave * 2u * kWindowBytes;
@@ -264,8 +266,7 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
         const unsigned char *from = IMAGE
             ? window_from[k] + offset
             : (const unsigned char *)((unsigned long long)(window_from[k] + offset) & ~3ull);
-        if (IMAGE || k < 2u) copy_to_lds_16(from, to);
-        else copy_to_lds_16_first32(from, to);
+        copy_to_lds_16(from, to);
     };
 
     // ---- activation rows this lane copies: wave w owns the 4-slot groups w (and w + 8) ----
@@ -330,7 +331,6 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
     const unsigned sel_lane = kSelBase + (lane & 15u) * 8u;
     const unsigned lut_lane = kLutBase + (lane & 15u) * 16u;
     const unsigned row_scale_at = kRowScaleBase + wave * 256u;      // + 128 for odd superblocks
-    const unsigned window_row = window_base + r * 80u;
     unsigned grids[4], aux[4];           // group records of the superblock being decoded
     unsigned head = 0u;                  // image: fp16 scale | the four group scales of this half << 16
     uint2 codes[2][2], signs[2][2];      // [chunk & 1]: table words of the chunk's two subgroups
@@ -340,8 +340,8 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
     // Records of superblock sb out of its window, and the row's scale into LDS for the lanes that
     // hold this row's sums (zero past the end: such superblocks add nothing). With o = (row start
     // + 66 sb) mod 4 (0 or 2) the fp16 scale sits o bytes into the window and the lane's 32 code
-    // bytes at o + 2 + 32 h: in window dwords 8 h + o / 2 onwards, shifted by 2 bytes when o is
-    // 0. Window dword 16 is the last dword of the fifth piece.
+    // bytes at o + 2 + 32 h: in aligned dwords 8 h + o / 2 onwards, shifted by 2 bytes when o is
+    // 0. Aligned dword 16 is the last dword of the fifth piece.
     auto settle = [&](unsigned sb) {
         if constexpr (IMAGE) {
             // The lane's record is nine dwords: pieces 3 h and 3 h + 1 whole, and of piece 3 h + 2
@@ -363,17 +363,21 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
         }
         const unsigned clamped = sb < last ? sb : last;
         const unsigned o = (row_misalign + 2u * clamped) & 3u;
-        const unsigned at = window_row + (sb & 1u) * kWindowBytes;
-        const unsigned first = at + 32u * h + 2u * o;                   // dword 8 h + o / 2
+        // Aligned dwords 8 h .. 8 h + 8 of the window: pieces 2 h and 2 h + 1 whole, and the dword
+        // behind them (the first of piece 2, or the last of the fifth piece, which is aligned
+        // dword 16). The lane's nine dwords start at dword 8 h + o / 2 of the window.
+        const unsigned at = window_base + (sb & 1u) * kWindowBytes + (2u * h * 32u + r) * 16u;
+        const v4i first = lds_read_v4i(at), second = lds_read_v4i(at + 512u), third = lds_read_v4i(at + 1024u);
+        const unsigned d[9] = {(unsigned)first[0], (unsigned)first[1], (unsigned)first[2], (unsigned)first[3],
+                               (unsigned)second[0], (unsigned)second[1], (unsigned)second[2], (unsigned)second[3],
+                               (unsigned)(h ? third[3] : third[0])};
         unsigned w[9];
 #pragma unroll
-        for (unsigned i = 0; i < 7u; ++i) w[i] = lds_read_u32(first + 4u * i);
-        // window dword 16 lives 12 bytes further on (it is the last dword of the fifth piece); it
-        // is the eighth of the lane's dwords when h is 1 and o is 2 and the ninth when h is 1 and o
-        // is 0 (the ninth is only part of a record when o is 0)
-        w[7] = lds_read_u32((h && o) ? at + 76u : first + 28u);
-        w[8] = lds_read_u32(h ? at + 76u : first + 32u);
-        const unsigned scale16 = (lds_read_u32(at) >> (8u * o)) & 0xffffu;
+        for (unsigned i = 0; i < 8u; ++i) w[i] = o ? d[i + 1u] : d[i];
+        w[8] = d[8];           // (the ninth is only part of a record when o is 0)
+        // the fp16 scale sits o bytes into the window: in the first dword of the first half's lanes,
+        // which are the ones that publish it
+        const unsigned scale16 = ((unsigned)first[0] >> (8u * o)) & 0xffffu;
         const unsigned shift = (o + 2u) & 3u;
 #pragma unroll
         for (unsigned g = 0; g < 4u; ++g) {
@@ -381,7 +385,7 @@ __device__ __forceinline__ void rows_item(const MfmaArgs &a, const MfmaItem &it,
             aux[g] = __builtin_amdgcn_alignbyte(w[2u * g + 2u], w[2u * g + 1u], shift);
         }
         const float mine = sb < superblocks ? 0.125f * f16_bits_to_float(scale16) : 0.0f;
-        lds_write_u32(row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
+        lds_write_u32(h ? kTrashBase : row_scale_at + (sb & 1u) * 128u + r * 4u, __float_as_uint(mine));
     };
     // table lookups of K chunk c: subgroups 2 (c & 1) and 2 (c & 1) + 1 of group c / 2
     auto lookup = [&](unsigned c) {
