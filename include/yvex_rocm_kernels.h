@@ -85,6 +85,18 @@ int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t 
                              const float *input, uint64_t input_rows, uint64_t input_stride,
                              const float *additive, float *out, uint64_t out_stride, int output_bf16,
                              void *scratch, uint64_t scratch_bytes, int *status, yvex_hip_stream stream);
+/* The split form of yvex_hip_matvec_f32_rows for the router's logits, which also publishes the
+ * router's score of every logit (scores, dense [input row][weight row]; the float that the
+ * double-precision score of src/graph/moe.c:497-537 rounds to, as yvex_hip_moe_route_scores
+ * publishes it): the second launch's many workgroups compute them, so that the routing launch
+ * that follows (yvex_hip_moe_prepare_scored) has none left. UNSUPPORTED where
+ * yvex_hip_matvec_f32_rows_launches says 1 for the operands. A logit whose score is not finite
+ * raises status 1. */
+int yvex_hip_matvec_f32_rows_scored(const float *weights, uint64_t row_count, uint64_t row_width,
+                                    const float *input, uint64_t input_rows, uint64_t input_stride,
+                                    float *out, uint64_t out_stride, float *scores, int scoring,
+                                    void *scratch, uint64_t scratch_bytes, int *status,
+                                    yvex_hip_stream stream);
 
 /* Replaces yvex_argmax_f32 (kernels.cu:59-110): for each of row_count (<= 65535) rows of
  * row_width (< 2^32) F32 values the largest value, the lowest index holding it and the number of
@@ -170,6 +182,15 @@ int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, 
                          uint64_t *bucket_populations, uint64_t *sweep_offsets, uint64_t *counts,
                          const float *values, uint64_t width, uint64_t input_stride, uint8_t *encoded,
                          int *status, yvex_hip_stream stream);
+/* yvex_hip_moe_prepare over scores that yvex_hip_matvec_f32_rows_scored has published
+ * (rows x experts floats) in place of the logits: same outputs bit for bit. */
+int yvex_hip_moe_prepare_scored(const float *scores, const float *bias, uint64_t rows, uint64_t experts,
+                                uint64_t topk, int normalize, double scaling, uint64_t *selected,
+                                float *weights, uint64_t *order, uint64_t *expert_ids,
+                                uint64_t *bucket_offsets, uint64_t *bucket_populations,
+                                uint64_t *sweep_offsets, uint64_t *counts, const float *values,
+                                uint64_t width, uint64_t input_stride, uint8_t *encoded, int *status,
+                                yvex_hip_stream stream);
 
 /* Expert matrices of one MoE layer. routed_* are expert-major: expert e starts at
  * base + e * expert_bytes and holds rows * row_bytes canonical GGUF bytes. gate_up_image /

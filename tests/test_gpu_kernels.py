@@ -420,6 +420,57 @@ def test_fused_preparation_equals_the_three_launches(gpu, oracle, rows, experts,
     assert int(status.item()) != 0
 
 
+@pytest.mark.parametrize("rows,experts,topk,width,scoring", [
+    (32, 256, 8, 7168, 1), (32, 256, 8, 7168, 0), (8, 64, 6, 1024, 0), (100, 200, 16, 2048, 1)])
+def test_scored_projection_and_preparation_equal_the_plain_pair(gpu, oracle, rows, experts, topk, width,
+                                                                scoring):
+    """The router projection that publishes the scores beside the logits, and the preparation
+    that starts from them: logits, selection, route weights, worklist and quantized input bit
+    for bit what the projection and the preparation over logits write; the scores are the
+    oracle's (src/graph/moe.c:497-537)."""
+    from yvex_amd import kernels as K
+    g = oracle.Generator(9, f"scored.{rows}.{experts}.{topk}.{scoring}")
+    router = dev(g.normal(experts * width).reshape(experts, width) * 0.05, gpu)
+    values = dev(g.normal(rows * width).reshape(rows, width), gpu)
+    bias = dev((g.normal(experts) * 0.05).astype(np.float32), gpu)
+    status = K.new_status(gpu)
+    logits = K.matvec_f32_rows(router, values, status)
+    wl = K.Worklist(rows * topk, experts, gpu)
+    q8 = torch.zeros(rows * (width // 256) * 292, dtype=torch.uint8, device=gpu)
+    sel, w = K.moe_prepare(logits, bias, topk, scoring, True, 2.5, status, wl, values, q8)
+    status_ok(status)
+    got_logits, scores = K.matvec_f32_rows_scored(router, values, scoring, status)
+    got_wl = K.Worklist(rows * topk, experts, gpu)
+    got_q8 = torch.zeros_like(q8)
+    got_sel, got_w = K.moe_prepare_scored(scores, bias, topk, True, 2.5, status, got_wl, values, got_q8)
+    status_ok(status)
+    assert torch.equal(got_logits.view(torch.int32), logits.view(torch.int32))
+    assert torch.equal(got_sel, sel) and torch.equal(got_w.view(torch.int32), w.view(torch.int32))
+    n = int(wl.counts[0].item())
+    assert torch.equal(got_wl.counts, wl.counts) and torch.equal(got_wl.order, wl.order)
+    assert torch.equal(got_wl.expert_ids[:n], wl.expert_ids[:n])
+    assert torch.equal(got_wl.bucket_offsets[:n + 1], wl.bucket_offsets[:n + 1])
+    assert torch.equal(got_wl.bucket_populations[:n], wl.bucket_populations[:n])
+    assert torch.equal(got_wl.sweep_offsets[:n + 1], wl.sweep_offsets[:n + 1])
+    assert torch.equal(got_q8, q8)
+    for row in (0, rows - 1):
+        rc, want_sel, want_w, want_scores = oracle.moe_route(logits[row].cpu().numpy(), bias.cpu().numpy(), topk,
+                                                             scoring, True, 2.5)
+        assert rc == 0 and np.array_equal(got_sel[row].cpu().numpy().astype(np.uint64), want_sel)
+        np.testing.assert_allclose(scores[row].cpu().numpy(), want_scores, rtol=2e-7, atol=0)
+        np.testing.assert_allclose(got_w[row].cpu().numpy(), want_w, rtol=1e-6, atol=0)
+    # a shape the projection does not split is refused, not run some other way
+    with pytest.raises(K.KernelError):
+        K.matvec_f32_rows_scored(router[:, :256].contiguous(), values[:, :256].contiguous(), scoring, status)
+    # an input that makes a logit non-finite raises the numeric status from the join
+    bad = values.clone()
+    bad[0, 3] = float("inf")
+    status = K.new_status(gpu)
+    K.matvec_f32_rows_scored(router, bad, scoring, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) != 0
+
+
 @pytest.mark.parametrize("rows,topk,hidden,offset", [(5, 3, 8, 0), (32, 8, 7168, 0), (3, 6, 10, 0), (4, 5, 64, 1),
                                                      (7, 1, 4, 0)])
 def test_reduce_combine_sums_in_rank_order(gpu, oracle, rows, topk, hidden, offset):

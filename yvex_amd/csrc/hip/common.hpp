@@ -63,6 +63,16 @@ __device__ __forceinline__ bool finite_f32(float v)
     return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;
 }
 
+// Router score of a logit in double (src/graph/moe.c:497-537): sigmoid, or the square root of the
+// softplus. `sigmoid` is YVEX_HIP_SCORING_SIGMOID of the launch-level header.
+__device__ __forceinline__ double route_score(double v, int scoring)
+{
+    if (scoring == 1)
+        return v >= 0.0 ? 1.0 / (1.0 + exp(-v)) : exp(v) / (1.0 + exp(v));
+    const double softplus = v > 0.0 ? v + log1p(exp(-v)) : log1p(exp(v));
+    return sqrt(softplus);
+}
+
 __device__ __forceinline__ unsigned load_u16(const unsigned char *p)
 {
     unsigned short v;

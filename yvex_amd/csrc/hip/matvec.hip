@@ -26,6 +26,8 @@ struct MatvecArgs {
     int output_bf16;
     int *status;
     double *parts;           // split projections: [split][input row][weight row] partial sums
+    float *scores;           // join of a split projection: the router scores of the outputs as well
+    int scoring;
 };
 
 __device__ __forceinline__ void matvec_publish(const MatvecArgs &a, unsigned long long in,
@@ -296,6 +298,14 @@ __global__ __launch_bounds__(256) void matvec_f32_join_kernel(MatvecArgs a, unsi
     double sum = a.parts[at];
     for (unsigned z = 1; z < splits; ++z) sum += a.parts[z * outputs + at];
     matvec_publish(a, in, row, (float)sum);
+    if (a.scores) {
+        // the router's score of this logit: the routing launch behind this one then has no
+        // double-precision exponentials left in its one workgroup
+        const double s = route_score((double)(float)sum, a.scoring);
+        const float published = (float)s;
+        if (!(s == s) || !finite_f32(published)) raise_status(a.status, 1);
+        a.scores[in * a.row_count + row] = published;
+    }
 }
 
 // int32 block sums of the Q8_K path, produced by the same unit code the matvec runs.
@@ -429,7 +439,7 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (row_width > 0xffffffffull * 32ull) return ST_BOUNDS;
     if (((uintptr_t)input & 3u) || ((uintptr_t)out & 3u)) return ST_INVALID_ARG;
     MatvecArgs a{encoded, row_count, row_width, row_bytes, input, input_rows, input_stride,
-                 additive, out, out_stride, output_bf16, status, nullptr};
+                 additive, out, out_stride, output_bf16, status, nullptr, nullptr, 0};
     hipStream_t s = as_stream(stream);
     const bool scalar = qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16 || qtype == QT_I32;
     if (input_q8 && (scalar || row_width % 256u)) return ST_UNSUPPORTED;
@@ -590,6 +600,8 @@ extern "C" unsigned int yvex_hip_matvec_f32_rows_launches(const float *weights, 
                                   scratch_bytes) ? 2u : 1u;
 }
 
+static int launch_f32_rows_split(const MatvecArgs &a, yvex_hip_stream stream);
+
 extern "C" int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count, uint64_t row_width,
                                         const float *input, uint64_t input_rows, uint64_t input_stride,
                                         const float *additive, float *out, uint64_t out_stride,
@@ -601,9 +613,36 @@ extern "C" int yvex_hip_matvec_f32_rows(const float *weights, uint64_t row_count
         return yvex_hip_matvec((const uint8_t *)weights, QT_F32, row_count, row_width, row_width * 4u, input, 0,
                                input_rows, input_stride, additive, out, out_stride, output_bf16, status,
                                stream);
-    const unsigned splits = f32_rows_splits(row_width, input_rows);
     MatvecArgs a{(const unsigned char *)weights, row_count, row_width, row_width * 4u, input, input_rows,
-                 input_stride, additive, out, out_stride, output_bf16, status, (double *)scratch};
+                 input_stride, additive, out, out_stride, output_bf16, status, (double *)scratch, nullptr, 0};
+    return launch_f32_rows_split(a, stream);
+}
+
+// The split projection with the router's score of every output published beside it
+// (`scores`, dense [input row][weight row]): the scores are computed by the join's many
+// workgroups instead of the routing launch's one. Only where the split applies (two launches,
+// as yvex_hip_matvec_f32_rows_launches says); anything else is refused.
+extern "C" int yvex_hip_matvec_f32_rows_scored(const float *weights, uint64_t row_count, uint64_t row_width,
+                                               const float *input, uint64_t input_rows,
+                                               uint64_t input_stride, float *out, uint64_t out_stride,
+                                               float *scores, int scoring, void *scratch,
+                                               uint64_t scratch_bytes, int *status, yvex_hip_stream stream)
+{
+    if (!out || !scores || !status || out_stride < row_count || (scoring != 0 && scoring != 1) ||
+        ((uintptr_t)out & 3u) || ((uintptr_t)scores & 3u))
+        return ST_INVALID_ARG;
+    if (!f32_rows_split_applies(weights, row_count, row_width, input, input_rows, input_stride, scratch,
+                                scratch_bytes))
+        return ST_UNSUPPORTED;
+    MatvecArgs a{(const unsigned char *)weights, row_count, row_width, row_width * 4u, input, input_rows,
+                 input_stride, nullptr, out, out_stride, 0, status, (double *)scratch, scores, scoring};
+    return launch_f32_rows_split(a, stream);
+}
+
+static int launch_f32_rows_split(const MatvecArgs &a, yvex_hip_stream stream)
+{
+    const uint64_t row_count = a.row_count, input_rows = a.input_rows;
+    const unsigned splits = f32_rows_splits(a.row_width, input_rows);
     hipStream_t s = as_stream(stream);
     const uint64_t grid_x = (row_count + 15u) / 16u, grid_y = (input_rows + 15u) / 16u;
     const uint64_t outputs = input_rows * row_count;

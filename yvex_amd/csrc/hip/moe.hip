@@ -17,14 +17,6 @@ namespace yvex {
 
 // ---- routing --------------------------------------------------------------------------------
 
-__device__ __forceinline__ double route_score(double v, int scoring)
-{
-    if (scoring == YVEX_HIP_SCORING_SIGMOID)
-        return v >= 0.0 ? 1.0 / (1.0 + exp(-v)) : exp(v) / (1.0 + exp(v));
-    const double softplus = v > 0.0 ? v + log1p(exp(-v)) : log1p(exp(v));
-    return sqrt(softplus);
-}
-
 // The scores alone, as the token-local operation publishes them beside the logits
 // (src/backend/cuda/moe_kernels.cu:29-55).
 __global__ __launch_bounds__(256) void route_scores_kernel(
@@ -61,10 +53,13 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v)
 }
 
 // One row by one wavefront.
+// `scores`: the rows' scores as a launch before this one has published them (the float a
+// double-precision score rounds to, what is computed here otherwise); `logits` is then not read.
 __device__ __forceinline__ void route_row(
     const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long row, unsigned lane,
     unsigned experts, unsigned topk, int scoring, int normalize, double scaling,
-    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status)
+    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status,
+    const float *__restrict__ scores = nullptr)
 {
     float score[4];
     unsigned long long key[4];
@@ -74,10 +69,14 @@ __device__ __forceinline__ void route_row(
         score[i] = 0.0f;
         key[i] = 0ull;
         if (e < experts) {
-            const double s = route_score((double)logits[row * experts + e], scoring);
-            score[i] = (float)s;
+            if (scores) {
+                score[i] = scores[row * experts + e];
+            } else {
+                const double s = route_score((double)logits[row * experts + e], scoring);
+                score[i] = (float)s;      // (a NaN stays a NaN)
+            }
             float biased = (bias ? bias[e] : 0.0f) + score[i];
-            if (!(s == s) || !finite_f32(score[i]) || !finite_f32(biased)) raise_status(status, 1);
+            if (!finite_f32(score[i]) || !finite_f32(biased)) raise_status(status, 1);
             biased += 0.0f;   // -0 and +0 must compare equal
             const unsigned bits = __float_as_uint(biased);
             const unsigned sortable = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
@@ -355,7 +354,8 @@ __global__ __launch_bounds__(1024) void decode_prepare_kernel(
     unsigned long long *__restrict__ expert_ids, unsigned long long *__restrict__ bucket_offsets,
     unsigned long long *__restrict__ bucket_populations, unsigned long long *__restrict__ sweep_offsets,
     unsigned long long *__restrict__ counts, const float *__restrict__ values, unsigned blocks,
-    unsigned long long input_stride, unsigned char *__restrict__ encoded, int *status)
+    unsigned long long input_stride, unsigned char *__restrict__ encoded, int *status,
+    const float *__restrict__ scores)
 {
     extern __shared__ unsigned shared_words[];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(1024) void decode_prepare_kernel(
     }
     for (unsigned row = wave; row < rows; row += 16u)
         route_row(logits, bias, row, lane, experts, topk, scoring, normalize, scaling, selected, weights,
-                  status);
+                  status, scores);
     __syncthreads();   // the selections written above are read back by other waves below
     worklist_block(selected, rows * topk, topk, experts, order, expert_ids, bucket_offsets,
                    bucket_populations, sweep_offsets, counts, status, shared_words, true);
@@ -942,16 +942,15 @@ extern "C" int yvex_hip_moe_prepare_supported(uint64_t rows, uint64_t experts, u
            topk <= experts && topk <= 16u;
 }
 
-extern "C" int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, uint64_t experts,
-                                    uint64_t topk, int scoring, int normalize, double scaling,
-                                    uint64_t *selected, float *weights, uint64_t *order,
-                                    uint64_t *expert_ids, uint64_t *bucket_offsets,
-                                    uint64_t *bucket_populations, uint64_t *sweep_offsets, uint64_t *counts,
-                                    const float *values, uint64_t width, uint64_t input_stride,
-                                    uint8_t *encoded, int *status, yvex_hip_stream stream)
+static int launch_moe_prepare(const float *logits, const float *scores, const float *bias, uint64_t rows,
+                              uint64_t experts, uint64_t topk, int scoring, int normalize, double scaling,
+                              uint64_t *selected, float *weights, uint64_t *order, uint64_t *expert_ids,
+                              uint64_t *bucket_offsets, uint64_t *bucket_populations, uint64_t *sweep_offsets,
+                              uint64_t *counts, const float *values, uint64_t width, uint64_t input_stride,
+                              uint8_t *encoded, int *status, yvex_hip_stream stream)
 {
-    if (!logits || !selected || !weights || !order || !expert_ids || !bucket_offsets || !bucket_populations ||
-        !sweep_offsets || !counts || !status || (scoring != 0 && scoring != 1))
+    if ((!logits && !scores) || !selected || !weights || !order || !expert_ids || !bucket_offsets ||
+        !bucket_populations || !sweep_offsets || !counts || !status || (scoring != 0 && scoring != 1))
         return ST_INVALID_ARG;
     if (!yvex_hip_moe_prepare_supported(rows, experts, topk)) return ST_UNSUPPORTED;
     uint64_t tasks = 0u;
@@ -968,8 +967,37 @@ extern "C" int yvex_hip_moe_prepare(const float *logits, const float *bias, uint
         (unsigned long long *)selected, weights, (unsigned long long *)order,
         (unsigned long long *)expert_ids, (unsigned long long *)bucket_offsets,
         (unsigned long long *)bucket_populations, (unsigned long long *)sweep_offsets,
-        (unsigned long long *)counts, values, (unsigned)(width / 256u), input_stride, encoded, status);
+        (unsigned long long *)counts, values, (unsigned)(width / 256u), input_stride, encoded, status, scores);
     return check_launch("moe_prepare");
+}
+
+extern "C" int yvex_hip_moe_prepare(const float *logits, const float *bias, uint64_t rows, uint64_t experts,
+                                    uint64_t topk, int scoring, int normalize, double scaling,
+                                    uint64_t *selected, float *weights, uint64_t *order,
+                                    uint64_t *expert_ids, uint64_t *bucket_offsets,
+                                    uint64_t *bucket_populations, uint64_t *sweep_offsets, uint64_t *counts,
+                                    const float *values, uint64_t width, uint64_t input_stride,
+                                    uint8_t *encoded, int *status, yvex_hip_stream stream)
+{
+    if (!logits) return ST_INVALID_ARG;
+    return launch_moe_prepare(logits, nullptr, bias, rows, experts, topk, scoring, normalize, scaling, selected,
+                              weights, order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets,
+                              counts, values, width, input_stride, encoded, status, stream);
+}
+
+extern "C" int yvex_hip_moe_prepare_scored(const float *scores, const float *bias, uint64_t rows,
+                                           uint64_t experts, uint64_t topk, int normalize, double scaling,
+                                           uint64_t *selected, float *weights, uint64_t *order,
+                                           uint64_t *expert_ids, uint64_t *bucket_offsets,
+                                           uint64_t *bucket_populations, uint64_t *sweep_offsets,
+                                           uint64_t *counts, const float *values, uint64_t width,
+                                           uint64_t input_stride, uint8_t *encoded, int *status,
+                                           yvex_hip_stream stream)
+{
+    if (!scores) return ST_INVALID_ARG;
+    return launch_moe_prepare(nullptr, scores, bias, rows, experts, topk, 0, normalize, scaling, selected, weights,
+                              order, expert_ids, bucket_offsets, bucket_populations, sweep_offsets, counts,
+                              values, width, input_stride, encoded, status, stream);
 }
 
 extern "C" int yvex_hip_moe_up(const yvex_hip_expert_weights *w, const void *activations,

@@ -490,7 +490,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     const void *activations;
     void *combined_target;
     unsigned long long table_address = 0ull;
-    int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer;
+    int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer, scored = 0;
     void *status;
     yvex_hip_stream stream;
     enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
@@ -795,6 +795,19 @@ sequence:
         unsigned int router_launches = yvex_hip_matvec_f32_rows_launches(
             (const float *)(uintptr_t)router_address, experts, hidden, (const float *)activations, row_count,
             hidden, lend ? AT(pair_outputs) : NULL, lend ? need : 0ull);
+        /* the split projection's second launch publishes the learned router's scores as well
+         * (into the combine's output range, which nothing reads or writes before the combine):
+         * the preparation launch, whose one routing workgroup everything behind it waits for,
+         * then starts from them */
+        scored = router_launches == 2u && !hash_router && hidden >= experts &&
+                 yvex_hip_moe_prepare_supported(row_count, experts, topk);
+        if (scored)
+            LAUNCH(yvex_hip_matvec_f32_rows_scored((const float *)(uintptr_t)router_address, experts, hidden,
+                                                   (const float *)activations, row_count, hidden,
+                                                   (float *)AT(logits), experts, (float *)AT(routed),
+                                                   (int)layer->scoring, AT(pair_outputs), need,
+                                                   (int *)status, stream), "rocm.moe.rows.router");
+        else
         LAUNCH(yvex_hip_matvec_f32_rows((const float *)(uintptr_t)router_address, experts, hidden,
                                         (const float *)activations, row_count, hidden, NULL,
                                         (float *)AT(logits), experts, 0, lend ? AT(pair_outputs) : NULL,
@@ -823,7 +836,19 @@ sequence:
     /* a decode-width batch with the learned router: routing, worklist and input quantization
      * share one launch */
     const int need_q8 = routed_q8 || (has_shared && shared_q8);
-    if (!hash_router && yvex_hip_moe_prepare_supported(row_count, experts, topk)) {
+    if (scored) {
+        LAUNCH(yvex_hip_moe_prepare_scored((const float *)AT(routed),
+                                           layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                           row_count, experts, topk, layer->normalize_topk_probabilities,
+                                           layer->routed_scaling_factor, (uint64_t *)AT(selected),
+                                           (float *)AT(weights), (uint64_t *)AT(order),
+                                           (uint64_t *)AT(expert_ids), (uint64_t *)AT(bucket_offsets),
+                                           (uint64_t *)AT(bucket_populations),
+                                           (uint64_t *)AT(sweep_offsets), (uint64_t *)AT(counts),
+                                           need_q8 ? (const float *)activations : NULL, hidden, hidden,
+                                           need_q8 ? (uint8_t *)AT(input_q8) : NULL, (int *)status, stream),
+               "rocm.moe.rows.prepare");
+    } else if (!hash_router && yvex_hip_moe_prepare_supported(row_count, experts, topk)) {
         LAUNCH(yvex_hip_moe_prepare((const float *)AT(logits),
                                     layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
                                     row_count, experts, topk, (int)layer->scoring,

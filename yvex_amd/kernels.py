@@ -113,6 +113,24 @@ def matvec_f32_rows(weights, inputs, status, *, additive=None, output_bf16=False
     return out
 
 
+def matvec_f32_rows_scored(weights, inputs, scoring, status):
+    """The split router projection with the scores beside the logits: (logits, scores)."""
+    row_count, row_width = weights.shape
+    input_rows = inputs.shape[0]
+    lib = load_library()
+    lib.yvex_hip_matvec_f32_scratch_bytes.restype = C.c_uint64
+    need = lib.yvex_hip_matvec_f32_scratch_bytes(C.c_uint64(row_count), C.c_uint64(row_width),
+                                                 C.c_uint64(input_rows))
+    scratch = torch.empty(max(need, 8), dtype=torch.uint8, device=weights.device)
+    out = torch.empty((input_rows, row_count), dtype=torch.float32, device=weights.device)
+    scores = torch.empty((input_rows, row_count), dtype=torch.float32, device=weights.device)
+    _call("yvex_hip_matvec_f32_rows_scored", _ptr(weights), C.c_uint64(row_count), C.c_uint64(row_width),
+          _ptr(inputs), C.c_uint64(input_rows), C.c_uint64(inputs.stride(0)), _ptr(out),
+          C.c_uint64(row_count), _ptr(scores), C.c_int(scoring), _ptr(scratch), C.c_uint64(need),
+          _ptr(status), _stream())
+    return out, scores
+
+
 def block_dots_i32(encoded, qtype, row_count, row_width, act_q8, input_rows, status):
     blocks = row_width // 256
     shape = (input_rows, row_count, blocks * 8) if qtype == Q8_0 else (input_rows, row_count, blocks, 2)
@@ -244,6 +262,23 @@ def moe_prepare(logits, bias, topk, scoring, normalize, scaling, status, worklis
     wl = worklist
     _call("yvex_hip_moe_prepare", _ptr(logits), _ptr(bias), C.c_uint64(rows), C.c_uint64(experts),
           C.c_uint64(topk), C.c_int(scoring), C.c_int(int(normalize)), C.c_double(scaling), _ptr(selected),
+          _ptr(weights), _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
+          _ptr(wl.bucket_populations), _ptr(wl.sweep_offsets), _ptr(wl.counts), _ptr(values),
+          C.c_uint64(width), C.c_uint64(stride), _ptr(encoded), _ptr(status), _stream())
+    return selected, weights
+
+
+def moe_prepare_scored(scores, bias, topk, normalize, scaling, status, worklist: Worklist,
+                       values=None, encoded=None):
+    """moe_prepare over scores published by matvec_f32_rows_scored."""
+    rows, experts = scores.shape
+    selected = torch.empty((rows, topk), dtype=torch.int64, device=scores.device)
+    weights = torch.empty((rows, topk), dtype=torch.float32, device=scores.device)
+    width = 0 if values is None else values.shape[1]
+    stride = 0 if values is None else values.stride(0)
+    wl = worklist
+    _call("yvex_hip_moe_prepare_scored", _ptr(scores), _ptr(bias), C.c_uint64(rows), C.c_uint64(experts),
+          C.c_uint64(topk), C.c_int(int(normalize)), C.c_double(scaling), _ptr(selected),
           _ptr(weights), _ptr(wl.order), _ptr(wl.expert_ids), _ptr(wl.bucket_offsets),
           _ptr(wl.bucket_populations), _ptr(wl.sweep_offsets), _ptr(wl.counts), _ptr(values),
           C.c_uint64(width), C.c_uint64(stride), _ptr(encoded), _ptr(status), _stream())
