@@ -151,6 +151,46 @@ def test_matvec_q8k_activations(gpu, oracle, qtype, rows, width, inputs):
 
 
 @pytest.mark.parametrize("qtype,rows,width,inputs", [
+    # lanes a row: 8 (and fewer superblocks than lanes), 16, 32, 64; row counts that leave lanes
+    # and waves without a row; a row of more than 8192 columns (several passes of the wave)
+    ("IQ2_XXS", 67, 512, 1), ("IQ2_XXS", 7168, 2048, 1), ("IQ2_XXS", 41, 4096, 1), ("IQ2_XXS", 2048, 7168, 1),
+    ("IQ2_XXS", 5, 16384, 1), ("Q4_K", 2048, 7168, 1), ("Q4_K", 19, 1024, 1), ("Q4_K", 3, 24576, 1),
+    ("Q2_K", 77, 2048, 1), ("Q2_K", 9, 7168, 1),
+    # a few input rows over weights decoded once
+    ("IQ2_XXS", 7168, 2048, 2), ("IQ2_XXS", 35, 2048, 31), ("IQ2_XXS", 130, 7168, 12), ("IQ2_XXS", 10, 768, 5),
+    ("Q4_K", 2048, 7168, 3), ("Q4_K", 21, 512, 2), ("Q2_K", 33, 4096, 7)])
+def test_matvec_q8k_one_round_trip_kernels(gpu, oracle, qtype, rows, width, inputs):
+    """One (or a few) Q8_K input rows against superblock-format rows run through the kernels
+    that ask for all of a lane's bytes at once: the oracle's Q8_K product bit for bit, with the
+    additive rows and the bf16 rounding of the other kernels, and the same bits from weights on
+    a 2-byte boundary, which take the general kernel."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(43, f"matvec.row.{qtype}.{rows}.{width}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    add = g.normal(inputs * rows).reshape(inputs, rows)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    want = oracle.q8_matvec(qt, w, rows, width, oracle.q8k_quantize(x), inputs)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    summed = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                      additive=dev(add, gpu), output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((summed.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(summed - (got + add)) <= np.abs(got + add) * 2.0 ** -8 + 1e-30)
+    shifted = torch.zeros(w.size + 2, dtype=torch.uint8, device=gpu)
+    shifted[2:] = dev(w, gpu)
+    moved = K.matvec(shifted[2:], qt, rows, width, act, input_q8=True, input_rows=inputs,
+                     status=status).cpu().numpy()
+    status_ok(status)
+    assert np.array_equal(moved.view(np.uint32), got.view(np.uint32))
+
+
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
     ("IQ2_XXS", 516, 2048, 32), ("IQ2_XXS", 260, 7168, 70), ("IQ2_XXS", 7168, 2048, 33),
     ("IQ2_XXS", 50, 2304, 40), ("IQ2_XXS", 7, 256, 33),
     # more work items (33 token tiles x 8 row tiles) than workgroups: a workgroup hands over from

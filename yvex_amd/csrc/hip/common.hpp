@@ -157,6 +157,30 @@ __device__ __forceinline__ float group_sum_f32(float v)
     return v;
 }
 
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move_f64(double v)
+{
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, ROW_MASK, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, ROW_MASK, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+
+// Double-precision sum over aligned groups of WIDTH lanes, valid in the LAST lane of every group
+// (the other lanes hold partial sums).
+template <int WIDTH>
+__device__ __forceinline__ double group_sum_f64_last(double v)
+{
+    static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 ||
+                  WIDTH == 32 || WIDTH == 64, "power of two up to the wave");
+    if constexpr (WIDTH >= 2) v += dpp_move_f64<0xb1, 0xf>(v);
+    if constexpr (WIDTH >= 4) v += dpp_move_f64<0x4e, 0xf>(v);
+    if constexpr (WIDTH >= 8) v += dpp_move_f64<0x141, 0xf>(v);
+    if constexpr (WIDTH >= 16) v += dpp_move_f64<0x140, 0xf>(v);
+    if constexpr (WIDTH >= 32) v += dpp_move_f64<0x142, 0xa>(v);   // rows 1 and 3 take rows 0 and 2
+    if constexpr (WIDTH == 64) v += dpp_move_f64<0x143, 0xc>(v);   // rows 2 and 3 take row 1
+    return v;
+}
+
 // Same with the width known only at run time (wave-uniform).
 __device__ __forceinline__ float group_sum_f32_dynamic(float v, unsigned width)
 {

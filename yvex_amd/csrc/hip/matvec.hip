@@ -164,6 +164,209 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     }
 }
 
+// A unit against 32 int8 activations held in registers; `sums` = the two 16-value sums of the
+// activations as Q8_K stores them (low and high half of the dword).
+template <unsigned QT>
+__device__ __forceinline__ UnitSum unit_dot_regs(const Unit &unit, const unsigned *a, unsigned sums)
+{
+    const int first = (int)(short)(sums & 0xffffu), second = (int)(short)(sums >> 16);
+    UnitSum out;
+    if constexpr (QT == QT_Q2_K) {
+        int d1 = 0, d2 = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            d1 = dot4(unit.w[i], a[i], d1);
+            d2 = dot4(unit.w[4 + i], a[4 + i], d2);
+        }
+        out.dot = unit.factor * d1 + unit.factor2 * d2;
+        out.min = unit.min1 * first + unit.min2 * second;
+    } else {
+        int d = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d = dot4(unit.w[i], a[i], d);
+        out.dot = unit.factor * d;
+        out.min = QT == QT_Q4_K ? unit.min1 * (first + second) : 0;
+    }
+    return out;
+}
+
+// One Q8_K input row against superblock-format weight rows, for matrices of a few megabytes
+// whose launch is over before the memory system is busy: what counts is the number of memory
+// round trips a wave waits for one after another. A lane owns half a superblock (four units)
+// of its weight row and L lanes share the row, so a wave holds 64 / L rows; every byte the lane
+// needs (weight record, superblock header, activation bytes, their scale and sums) is asked for
+// by loads that depend on nothing, issued together, and (IQ2_XXS) the codebook tables are
+// built in LDS while those are in flight: one round trip, where the general kernel above
+// waits for several in turn (unit after unit, then the header for the lane that combines).
+// The float term of a superblock and the double-precision row sum are the general kernel's.
+template <unsigned QT, int L>
+__global__ __launch_bounds__(256) void dense_row_q8k_kernel(MatvecArgs a)
+{
+    __shared__ Iq2Tables tables;
+    constexpr unsigned kRows = 64u / L;
+    const unsigned lane = threadIdx.x & 63u, slot = lane % L;
+    unsigned long long row = ((unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6)) * kRows + lane / L;
+    const bool row_live = row < a.row_count;
+    if (!row_live) row = a.row_count - 1ull;          // (no early exit: the barrier below)
+    const unsigned char *wrow = a.encoded + row * a.row_bytes;
+    const unsigned halves = (unsigned)(a.row_width >> 7);
+    // (asked for ahead of the weight bytes: loads come back in order, and the tables are to be
+    // built while the weight bytes are on their way, not after them)
+    unsigned digits = 0u;
+    if constexpr (QT == QT_IQ2_XXS) digits = k_iq2_digits[threadIdx.x];
+    double acc = 0.0;
+    for (unsigned base = 0; base < halves; base += L) {
+        // a superblock's two lanes are live or clamped together (halves and L are even)
+        const bool live = base + slot < halves;
+        const unsigned hs = live ? base + slot : halves - 1u;
+        const unsigned sb = hs >> 1, half = hs & 1u;
+        LaneChunk<QT> chunk;
+        if constexpr (QT == QT_IQ2_XXS) {
+            // the 32 record bytes start on a 2-byte boundary: aligned dwords, shifted into place
+            const unsigned char *b = wrow + sb * 66u;
+            const unsigned char *p = b + 2u + 32u * half;
+            const unsigned shift = (unsigned)(unsigned long long)p & 3u;       // 0 or 2
+            const unsigned *at = reinterpret_cast<const unsigned *>(p - shift);
+            unsigned raw[9];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) raw[i] = at[i];
+            raw[8] = at[shift ? 8 : 0];                   // (aligned records end with the eighth)
+            const unsigned head = *reinterpret_cast<const unsigned *>(b - ((unsigned long long)b & 2ull));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) chunk.q[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+            chunk.d16 = ((unsigned long long)b & 2ull) ? head >> 16 : head & 0xffffu;
+        } else {
+            chunk.load(wrow, 8u * sb + 4u * half);
+        }
+        const unsigned char *block = (const unsigned char *)a.input + (unsigned long long)sb * kQ8KBytes;
+        const unsigned *values = reinterpret_cast<const unsigned *>(block + 4u + 128u * half);
+        unsigned act[32], sums[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 32; ++i) act[i] = values[i];
+        if constexpr (QT != QT_IQ2_XXS) {
+            const unsigned *s = reinterpret_cast<const unsigned *>(block + 260u + 16u * half);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sums[i] = s[i];
+        }
+        const float act_scale = *reinterpret_cast<const float *>(block);
+        if constexpr (QT == QT_IQ2_XXS) {
+            if (base == 0u) {                             // (the same trip for every thread)
+                asm volatile("" : "+v"(digits));          // (the entry is not to be worked out, and waited for, ahead of the loads above)
+                tables.magnitudes[threadIdx.x] = iq2_magnitude_of_digits(digits);   // 256 threads, 256 entries
+                if (threadIdx.x < 128u) tables.signmask[threadIdx.x] = iq2_signmask_entry(threadIdx.x);
+                __syncthreads();
+            }
+        }
+        UnitSum total{0, 0};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            Unit unit;
+            chunk.decode(tables, k, 8u * sb + 4u * half, unit);
+            const UnitSum s = unit_dot_regs<QT>(unit, act + 8 * k, sums[k]);
+            total.dot += s.dot;
+            total.min += s.min;
+        }
+        total.dot += dpp_move<0xb1, 0xf>(total.dot);      // the superblock's other half
+        if constexpr (QT != QT_IQ2_XXS) total.min += dpp_move<0xb1, 0xf>(total.min);
+        const float term = chunk.combine(act_scale, total);
+        if (live && half == 0u) acc += (double)term;
+    }
+    acc = group_sum_f64_last<L>(acc);
+    if (row_live && slot == (unsigned)L - 1u) matvec_publish(a, 0ull, row, (float)acc);
+}
+
+// The same for a few Q8_K input rows (rows of up to 8192 columns, which L lanes hold whole): the
+// lane's four units are decoded once and stay in registers, and the input rows go by one after
+// another, the next one's bytes asked for before the current one is multiplied.
+struct RowActs {
+    unsigned values[32];
+    unsigned sums[4];
+    float scale;
+};
+
+template <unsigned QT>
+__device__ __forceinline__ void row_acts_load(RowActs &r, const unsigned char *block, unsigned half)
+{
+    const unsigned *values = reinterpret_cast<const unsigned *>(block + 4u + 128u * half);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) r.values[i] = values[i];
+    if constexpr (QT != QT_IQ2_XXS) {
+        const unsigned *s = reinterpret_cast<const unsigned *>(block + 260u + 16u * half);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.sums[i] = s[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.sums[i] = 0u;
+    }
+    r.scale = *reinterpret_cast<const float *>(block);
+}
+
+template <unsigned QT, int L>
+__global__ __launch_bounds__(256) void dense_fewrows_q8k_kernel(MatvecArgs a)
+{
+    __shared__ Iq2Tables tables;
+    constexpr unsigned kRows = 64u / L;
+    const unsigned lane = threadIdx.x & 63u, slot = lane % L;
+    unsigned long long row = ((unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6)) * kRows + lane / L;
+    const bool row_live = row < a.row_count;
+    if (!row_live) row = a.row_count - 1ull;
+    const unsigned char *wrow = a.encoded + row * a.row_bytes;
+    const unsigned halves = (unsigned)(a.row_width >> 7);             // <= L
+    const unsigned long long act_row_bytes = (a.row_width >> 8) * kQ8KBytes;
+    unsigned digits = 0u;
+    if constexpr (QT == QT_IQ2_XXS) digits = k_iq2_digits[threadIdx.x];
+    const bool live = slot < halves;
+    const unsigned hs = live ? slot : halves - 1u;
+    const unsigned sb = hs >> 1, half = hs & 1u;
+    LaneChunk<QT> chunk;
+    if constexpr (QT == QT_IQ2_XXS) {
+        const unsigned char *b = wrow + sb * 66u;
+        const unsigned char *p = b + 2u + 32u * half;
+        const unsigned shift = (unsigned)(unsigned long long)p & 3u;
+        const unsigned *at = reinterpret_cast<const unsigned *>(p - shift);
+        unsigned raw[9];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) raw[i] = at[i];
+        raw[8] = at[shift ? 8 : 0];
+        const unsigned head = *reinterpret_cast<const unsigned *>(b - ((unsigned long long)b & 2ull));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) chunk.q[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+        chunk.d16 = ((unsigned long long)b & 2ull) ? head >> 16 : head & 0xffffu;
+    } else {
+        chunk.load(wrow, 8u * sb + 4u * half);
+    }
+    const unsigned char *block = (const unsigned char *)a.input + (unsigned long long)sb * kQ8KBytes;
+    RowActs current;
+    row_acts_load<QT>(current, block, half);
+    if constexpr (QT == QT_IQ2_XXS) {
+        asm volatile("" : "+v"(digits));
+        tables.magnitudes[threadIdx.x] = iq2_magnitude_of_digits(digits);
+        if (threadIdx.x < 128u) tables.signmask[threadIdx.x] = iq2_signmask_entry(threadIdx.x);
+        __syncthreads();
+    }
+    Unit units[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) chunk.decode(tables, k, 8u * sb + 4u * half, units[k]);
+    for (unsigned long long in = 0; in < a.input_rows; ++in) {
+        RowActs next;
+        const unsigned long long ahead = in + 1ull < a.input_rows ? in + 1ull : in;
+        row_acts_load<QT>(next, block + ahead * act_row_bytes, half);
+        UnitSum total{0, 0};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const UnitSum s = unit_dot_regs<QT>(units[k], current.values + 8 * k, current.sums[k]);
+            total.dot += s.dot;
+            total.min += s.min;
+        }
+        total.dot += dpp_move<0xb1, 0xf>(total.dot);
+        if constexpr (QT != QT_IQ2_XXS) total.min += dpp_move<0xb1, 0xf>(total.min);
+        const float term = chunk.combine(current.scale, total);
+        const double sum = group_sum_f64_last<L>(live && half == 0u ? (double)term : 0.0);
+        if (row_live && slot == (unsigned)L - 1u) matvec_publish(a, in, row, (float)sum);
+        current = next;
+    }
+}
+
 // F32 / F16 / BF16 weight rows: lanes stride the row element-wise. Products and sums run in
 // double, as the CPU row dot forms them (src/gguf/quant_compute.c:152-172: double(value) *
 // double(x) added in double, rounded to float once); the product of two floats is exact in
@@ -407,9 +610,72 @@ static int launch_block_even(const MatvecArgs &a, hipStream_t stream)
     return check_launch("matvec");
 }
 
+template <unsigned QT, int L>
+static int launch_dense_row(const MatvecArgs &a, hipStream_t stream)
+{
+    const unsigned long long grid = (a.row_count + 4ull * (64u / L) - 1ull) / (4ull * (64u / L));
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    dense_row_q8k_kernel<QT, L><<<(unsigned)grid, 256, 0, stream>>>(a);
+    return check_launch("matvec.row");
+}
+
+// One Q8_K input row against superblock-format rows on dword boundaries: the row kernel, whatever
+// the size of the matrix (a 470 MB Q4_K matrix streams at 4.8 TB/s through it, at 2.4 TB/s
+// through the general kernel, whose lanes wait for the superblock header on their own).
+template <unsigned QT>
+static bool dense_row_applies(const MatvecArgs &a)
+{
+    return UnitTraits<QT>::kIntegerCombine && a.input_rows == 1ull &&
+           !((unsigned long long)a.encoded & 3ull) && !(a.row_bytes & 3ull);
+}
+
+template <unsigned QT, int L>
+static int launch_dense_fewrows(const MatvecArgs &a, hipStream_t stream)
+{
+    const unsigned long long grid = (a.row_count + 4ull * (64u / L) - 1ull) / (4ull * (64u / L));
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    dense_fewrows_q8k_kernel<QT, L><<<(unsigned)grid, 256, 0, stream>>>(a);
+    return check_launch("matvec.fewrows");
+}
+
+template <unsigned QT>
+static bool dense_fewrows_applies(const MatvecArgs &a)
+{
+    // (measured against the general kernel on 2048 x 7168 and 7168 x 2048 matrices: ahead up to
+    // a dozen input rows, and at any number below 32 where a row is 2048 columns or fewer)
+    return UnitTraits<QT>::kIntegerCombine && a.input_rows >= 2ull && a.input_rows < 32ull &&
+           (a.input_rows <= 12ull || a.row_width <= 2048ull) &&
+           a.row_width <= 8192ull && a.row_count * a.row_bytes < (64ull << 20) &&
+           !((unsigned long long)a.encoded & 3ull) && !(a.row_bytes & 3ull);
+}
+
+template <unsigned QT>
+static int launch_dense_fewrows_width(const MatvecArgs &a, hipStream_t stream)
+{
+    const unsigned long long halves = a.row_width >> 7;
+    if (halves <= 8ull) return launch_dense_fewrows<QT, 8>(a, stream);
+    if (halves <= 16ull) return launch_dense_fewrows<QT, 16>(a, stream);
+    if (halves <= 32ull) return launch_dense_fewrows<QT, 32>(a, stream);
+    return launch_dense_fewrows<QT, 64>(a, stream);
+}
+
+template <unsigned QT>
+static int launch_dense_row_width(const MatvecArgs &a, hipStream_t stream)
+{
+    const unsigned long long halves = a.row_width >> 7;
+    if (halves <= 8ull) return launch_dense_row<QT, 8>(a, stream);
+    if (halves <= 16ull) return launch_dense_row<QT, 16>(a, stream);
+    if (halves <= 32ull) return launch_dense_row<QT, 32>(a, stream);
+    return launch_dense_row<QT, 64>(a, stream);
+}
+
 template <unsigned QT, bool Q8>
 static int launch_block(const MatvecArgs &a, hipStream_t stream)
 {
+    if constexpr (Q8 && UnitTraits<QT>::kIntegerCombine) {
+        if (dense_row_applies<QT>(a)) return launch_dense_row_width<QT>(a, stream);
+        if (dense_fewrows_applies<QT>(a)) return launch_dense_fewrows_width<QT>(a, stream);
+    }
     const bool even = (((unsigned long long)a.encoded | a.row_bytes) & 1ull) == 0ull;
     return even ? launch_block_even<QT, Q8, true>(a, stream) : launch_block_even<QT, Q8, false>(a, stream);
 }
@@ -459,9 +725,11 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         return launch_iq2_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, out,
                                      output_bf16 != 0, status, s);
     // Q4_K rows against two or more Q8_K input rows: matrix cores (the reference's threshold is 16
-    // input rows; here the 16-token tiles beat the sweep below from two rows on, 10.5 us against
-    // 12.2 us at 2 and 19.7 us at 15 rows for 2048 x 7168)
-    if (qtype == QT_Q4_K && input_q8 && input_rows >= 2ull && !((uintptr_t)encoded & 15u))
+    // input rows; here the 16-token tiles beat the general kernel below from two rows on, 10.5 us
+    // against 12.2 us at 2 and 19.7 us at 15 rows for 2048 x 7168; the few-rows kernel, where it
+    // applies, is ahead of both at two and three rows: 6.0 and 7.1 us against 8.6)
+    if (qtype == QT_Q4_K && input_q8 && input_rows >= 2ull && !((uintptr_t)encoded & 15u) &&
+        !(input_rows < 4ull && dense_fewrows_applies<QT_Q4_K>(a)))
         return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
                                      out, out_stride, output_bf16 != 0, status, s);
     // F32 rows against a batch of F32 input rows: 16 x 16 tiles on the double-precision matrix

@@ -181,24 +181,23 @@ struct LaneChunk<QT_Q4_K> {
             q[4 * i] = v.x; q[4 * i + 1] = v.y; q[4 * i + 2] = v.z; q[4 * i + 3] = v.w;
         }
     }
-    __device__ __forceinline__ unsigned scale_byte(unsigned i) const
-    {
-        return (head[1u + (i >> 2)] >> (8u * (i & 3u))) & 255u;
-    }
+    // Unit k of the lane's four (unit0 is a multiple of four: the lane owns the first or the
+    // second half of the superblock). The 6-bit scale and minimum of unit g are, for g < 4, the
+    // low bits of scale bytes g and g + 4, and for g >= 4 the nibbles of byte g + 4 with the top
+    // bits of bytes g - 4 and g (public ggml block_q4_K). With k a constant every byte sits at a
+    // fixed place of the header words, and which half the lane owns is a select, not a branch
+    // over an indexed array.
     template <typename Tables>
     __device__ __forceinline__ void decode(const Tables &, int k, unsigned unit0, Unit &unit) const
     {
-        const unsigned g = (unit0 & 7u) + (unsigned)k, shift = (g & 1u) * 4u;
+        const bool second = (unit0 & 4u) != 0u;
+        const unsigned shift = ((unsigned)k & 1u) * 4u;
 #pragma unroll
         for (int i = 0; i < 8; ++i) unit.w[i] = (q[8 * (k >> 1) + i] >> shift) & 0x0f0f0f0fu;
-        unsigned sc, mn;
-        if (g < 4u) {
-            sc = scale_byte(g) & 63u;
-            mn = scale_byte(g + 4u) & 63u;
-        } else {
-            sc = (scale_byte(g + 4u) & 15u) | ((scale_byte(g - 4u) >> 6) << 4);
-            mn = (scale_byte(g + 4u) >> 4) | ((scale_byte(g) >> 6) << 4);
-        }
+        const unsigned s0 = (head[1] >> (8u * k)) & 255u, s1 = (head[2] >> (8u * k)) & 255u,
+                       s2 = (head[3] >> (8u * k)) & 255u;
+        const unsigned sc = second ? (s2 & 15u) | ((s0 >> 6) << 4) : s0 & 63u;
+        const unsigned mn = second ? (s2 >> 4) | ((s1 >> 6) << 4) : s1 & 63u;
         unit.factor = unit.factor2 = (int)sc;
         unit.min1 = unit.min2 = (int)mn;
     }
