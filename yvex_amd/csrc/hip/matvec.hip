@@ -190,6 +190,33 @@ __device__ __forceinline__ UnitSum unit_dot_regs(const Unit &unit, const unsigne
     return out;
 }
 
+// A lane's half superblock (units 4 half .. 4 half + 3 of superblock sb) of a weight row that
+// starts on a dword boundary. The 32 record bytes of an IQ2_XXS half start on a 2-byte boundary,
+// and vector loads that are not dword-aligned run at less than half rate: the aligned dwords
+// that hold them are loaded and shifted into place, and the superblock's fp16 scale comes out
+// of the aligned dword that holds it (never a byte outside the row's own or its neighbours').
+template <unsigned QT>
+__device__ __forceinline__ void half_superblock_load(LaneChunk<QT> &chunk, const unsigned char *wrow,
+                                                     unsigned sb, unsigned half)
+{
+    if constexpr (QT == QT_IQ2_XXS) {
+        const unsigned char *b = wrow + sb * 66u;
+        const unsigned char *p = b + 2u + 32u * half;
+        const unsigned shift = (unsigned)(unsigned long long)p & 3u;       // 0 or 2
+        const unsigned *at = reinterpret_cast<const unsigned *>(p - shift);
+        unsigned raw[9];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) raw[i] = at[i];
+        raw[8] = at[shift ? 8 : 0];                       // (aligned records end with the eighth)
+        const unsigned head = *reinterpret_cast<const unsigned *>(b - ((unsigned long long)b & 2ull));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) chunk.q[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+        chunk.d16 = ((unsigned long long)b & 2ull) ? head >> 16 : head & 0xffffu;
+    } else {
+        chunk.load(wrow, 8u * sb + 4u * half);
+    }
+}
+
 // One Q8_K input row against superblock-format weight rows, for matrices of a few megabytes
 // whose launch is over before the memory system is busy: what counts is the number of memory
 // round trips a wave waits for one after another. A lane owns half a superblock (four units)
@@ -221,23 +248,7 @@ __global__ __launch_bounds__(256) void dense_row_q8k_kernel(MatvecArgs a)
         const unsigned hs = live ? base + slot : halves - 1u;
         const unsigned sb = hs >> 1, half = hs & 1u;
         LaneChunk<QT> chunk;
-        if constexpr (QT == QT_IQ2_XXS) {
-            // the 32 record bytes start on a 2-byte boundary: aligned dwords, shifted into place
-            const unsigned char *b = wrow + sb * 66u;
-            const unsigned char *p = b + 2u + 32u * half;
-            const unsigned shift = (unsigned)(unsigned long long)p & 3u;       // 0 or 2
-            const unsigned *at = reinterpret_cast<const unsigned *>(p - shift);
-            unsigned raw[9];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) raw[i] = at[i];
-            raw[8] = at[shift ? 8 : 0];                   // (aligned records end with the eighth)
-            const unsigned head = *reinterpret_cast<const unsigned *>(b - ((unsigned long long)b & 2ull));
-#pragma unroll
-            for (int i = 0; i < 8; ++i) chunk.q[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
-            chunk.d16 = ((unsigned long long)b & 2ull) ? head >> 16 : head & 0xffffu;
-        } else {
-            chunk.load(wrow, 8u * sb + 4u * half);
-        }
+        half_superblock_load<QT>(chunk, wrow, sb, half);
         const unsigned char *block = (const unsigned char *)a.input + (unsigned long long)sb * kQ8KBytes;
         const unsigned *values = reinterpret_cast<const unsigned *>(block + 4u + 128u * half);
         unsigned act[32], sums[4] = {0u, 0u, 0u, 0u};
@@ -319,22 +330,7 @@ __global__ __launch_bounds__(256) void dense_fewrows_q8k_kernel(MatvecArgs a)
     const unsigned hs = live ? slot : halves - 1u;
     const unsigned sb = hs >> 1, half = hs & 1u;
     LaneChunk<QT> chunk;
-    if constexpr (QT == QT_IQ2_XXS) {
-        const unsigned char *b = wrow + sb * 66u;
-        const unsigned char *p = b + 2u + 32u * half;
-        const unsigned shift = (unsigned)(unsigned long long)p & 3u;
-        const unsigned *at = reinterpret_cast<const unsigned *>(p - shift);
-        unsigned raw[9];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) raw[i] = at[i];
-        raw[8] = at[shift ? 8 : 0];
-        const unsigned head = *reinterpret_cast<const unsigned *>(b - ((unsigned long long)b & 2ull));
-#pragma unroll
-        for (int i = 0; i < 8; ++i) chunk.q[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
-        chunk.d16 = ((unsigned long long)b & 2ull) ? head >> 16 : head & 0xffffu;
-    } else {
-        chunk.load(wrow, 8u * sb + 4u * half);
-    }
+    half_superblock_load<QT>(chunk, wrow, sb, half);
     const unsigned char *block = (const unsigned char *)a.input + (unsigned long long)sb * kQ8KBytes;
     RowActs current;
     row_acts_load<QT>(current, block, half);
