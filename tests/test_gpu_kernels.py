@@ -88,10 +88,15 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
 
 
 @pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32),
-                                               (256, 7168, 300), (40, 96, 260), (256, 7168, 8), (3, 256, 9)])
+                                               (256, 7168, 300), (40, 96, 260), (256, 7168, 8), (3, 256, 9),
+                                               (45, 448, 257), (32, 64, 256),
+                                               # enough (32 rows x 64 input rows) blocks for the device and
+                                               # 128-column chunks: the kernel with operands staged in LDS,
+                                               # ragged on both sides
+                                               (250, 256, 1570), (256, 384, 2048)])
 def test_matvec_f32_weights_over_a_row_batch(gpu, oracle, rows, width, inputs):
-    """F32 weight rows against 32 or more F32 input rows (a router or mixing projection over a
-    prefill batch) run on the fp32 matrix cores; ragged edges, the additive operand and the bf16
+    """F32 weight rows against 8 or more F32 input rows (a router or mixing projection over a
+    row batch) run on the double-precision matrix cores; ragged edges, the additive operand and the bf16
     output behave as in the lane-strided kernel (kernels.cu:560-640)."""
     from yvex_amd import kernels as K
     g = oracle.Generator(42, f"matvec.f32.batch.{rows}.{width}.{inputs}")

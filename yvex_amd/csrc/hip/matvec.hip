@@ -487,6 +487,107 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
     }
 }
 
+// The same product for a batch of 256 input rows or more (the router projection of a prefill
+// batch): with one 16 x 16 tile a workgroup every wave loads its own operands, four bytes for
+// every matrix-core flop, and the launch runs at what the caches deliver (33 TFLOP/s where the
+// instruction alone sustains 75). Here a workgroup of eight waves (two a SIMD, so that one
+// multiplies while the other waits) owns 32 weight rows x 64 input rows and stages 128 columns
+// of both in LDS (a 528-byte pitch keeps the sixteen rows that one 16-byte read phase touches
+// on sixteen different bank groups), the next chunk's loads in flight while the current one is
+// multiplied; wave w multiplies the 16-row half w % 2 of the weight block by input rows
+// 16 (w / 2) .. + 15. Sums and rounding as above.
+constexpr unsigned kF32BlockColumns = 128u, kF32BlockPitch = kF32BlockColumns * 4u + 16u;
+constexpr unsigned kF32BlockWeightRows = 32u, kF32BlockInputRows = 64u;
+constexpr unsigned kF32BlockLdsBytes = 2u * (kF32BlockWeightRows + kF32BlockInputRows) * kF32BlockPitch;
+
+__global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
+{
+    typedef double v4d __attribute__((ext_vector_type(4)));
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    constexpr unsigned kRows = kF32BlockWeightRows + kF32BlockInputRows;
+    constexpr unsigned kPieces = kF32BlockColumns / 4u;                   // 16-byte pieces a row
+    constexpr unsigned kHeld = kRows * kPieces / 512u;
+    extern __shared__ __align__(16) unsigned char staged[];               // [2][kRows * kF32BlockPitch]
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned i16 = lane & 15u, q = lane >> 4;
+    // staging: piece p = threadIdx.x + 512 j of the chunk is columns 4 (p % 32) .. + 3 of staged
+    // row p / 32 (weight rows first, then input rows); 32 lanes read one row's 512 bytes
+    const float *source[kHeld];
+    unsigned target[kHeld];
+#pragma unroll
+    for (unsigned j = 0; j < kHeld; ++j) {
+        const unsigned p = threadIdx.x + 512u * j, row = p / kPieces, piece = p % kPieces;
+        if (row < kF32BlockWeightRows) {
+            unsigned long long wrow = (unsigned long long)blockIdx.x * kF32BlockWeightRows + row;
+            if (wrow >= a.row_count) wrow = a.row_count - 1ull;          // a ragged edge repeats the last row
+            source[j] = (const float *)(a.encoded + wrow * a.row_bytes) + 4u * piece;
+        } else {
+            unsigned long long in = (unsigned long long)blockIdx.y * kF32BlockInputRows + (row - kF32BlockWeightRows);
+            if (in >= a.input_rows) in = a.input_rows - 1ull;
+            source[j] = (const float *)a.input + in * a.input_stride + 4u * piece;
+        }
+        target[j] = row * kF32BlockPitch + 16u * piece;
+    }
+    const unsigned chunks = (unsigned)(a.row_width / kF32BlockColumns);
+    v4f held[kHeld];
+    unsigned bad = 0u;
+#pragma unroll
+    for (unsigned j = 0; j < kHeld; ++j) held[j] = *reinterpret_cast<const v4f *>(source[j]);
+#pragma unroll
+    for (unsigned j = 0; j < kHeld; ++j) {
+        if (512u * (j + 1u) <= kF32BlockWeightRows * kPieces)
+            bad |= (unsigned)!finite_f32(held[j][0]) | (unsigned)!finite_f32(held[j][1]) |
+                   (unsigned)!finite_f32(held[j][2]) | (unsigned)!finite_f32(held[j][3]);
+        *reinterpret_cast<v4f *>(&staged[target[j]]) = held[j];
+    }
+    __syncthreads();
+    v4d acc = {0.0, 0.0, 0.0, 0.0};
+    const unsigned weight_at = (16u * (wave & 1u) + i16) * kF32BlockPitch + 16u * q;
+    const unsigned input_at = (kF32BlockWeightRows + 16u * (wave >> 1) + i16) * kF32BlockPitch + 16u * q;
+    for (unsigned chunk = 0; chunk < chunks; ++chunk) {
+        // (the last turn asks for its own chunk again and stages it where nobody reads it: no
+        // branch around the loads, whose registers would otherwise be kept in scratch memory)
+        const unsigned ahead = chunk + 1u < chunks ? chunk + 1u : chunk;
+#pragma unroll
+        for (unsigned j = 0; j < kHeld; ++j)
+            held[j] = *reinterpret_cast<const v4f *>(source[j] + (unsigned long long)ahead * kF32BlockColumns);
+        const unsigned char *now = staged + (chunk & 1u) * (kRows * kF32BlockPitch);
+        unsigned char *next = staged + ((chunk + 1u) & 1u) * (kRows * kF32BlockPitch);
+#pragma unroll
+        for (unsigned step = 0; step < kF32BlockColumns / 16u; ++step) {
+            if (step == kF32BlockColumns / 32u) {
+                // half way: the loads have had four steps to arrive, and the stores have four
+                // more to land before the barrier
+#pragma unroll
+                for (unsigned j = 0; j < kHeld; ++j) {
+                    // (the weight rows are the first pieces: a non-finite weight is reported by
+                    // the thread that stages it, once, not by the sixteen lanes that multiply it)
+                    if (512u * (j + 1u) <= kF32BlockWeightRows * kPieces)
+                        bad |= (unsigned)!finite_f32(held[j][0]) | (unsigned)!finite_f32(held[j][1]) |
+                               (unsigned)!finite_f32(held[j][2]) | (unsigned)!finite_f32(held[j][3]);
+                    *reinterpret_cast<v4f *>(next + target[j]) = held[j];
+                }
+            }
+            const v4f x = *reinterpret_cast<const v4f *>(now + input_at + 64u * step);
+            const v4f w = *reinterpret_cast<const v4f *>(now + weight_at + 64u * step);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[0], (double)x[0], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[1], (double)x[1], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[2], (double)x[2], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)w[3], (double)x[3], acc, 0, 0, 0);
+        }
+        // the next chunk is complete, and nobody reads this one any more when it is overwritten
+        __syncthreads();
+    }
+    if (bad) raise_status(a.status, 1);
+    const unsigned long long in = (unsigned long long)blockIdx.y * kF32BlockInputRows + 16u * (wave >> 1) + i16;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        // accumulator k of lane (i, q): weight row 4 k + q of the tile, input row i
+        const unsigned long long row = (unsigned long long)blockIdx.x * kF32BlockWeightRows + 16u * (wave & 1u) + 4u * k + q;
+        if (row < a.row_count && in < a.input_rows) matvec_publish(a, in, row, (float)acc[k]);
+    }
+}
+
 // Second launch of a split projection: the partial sums of one output added in split order.
 __global__ __launch_bounds__(256) void matvec_f32_join_kernel(MatvecArgs a, unsigned splits)
 {
@@ -735,10 +836,22 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         !(input_stride & 3ull) && row_width % (input_rows < 256ull ? 256ull : 64ull) == 0ull) {
         const unsigned long long grid_x = (row_count + 15ull) / 16ull, grid_y = (input_rows + 15ull) / 16ull;
         if (grid_x > 0x7fffffffull || grid_y > 65535ull) return ST_BOUNDS;
-        if (input_rows < 256ull)
+        if (input_rows < 256ull) {
             matvec_f32_tile16_kernel<16><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
-        else
+        } else if (row_width % kF32BlockColumns == 0ull &&
+                   (row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows *
+                       ((input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows) >= 3ull * compute_units() / 4ull) {
+            // (a block a compute unit or close to it: the staged kernel walks the row width
+            // chunk by chunk, 3 us each, and is behind the small tiles on a grid that leaves
+            // most of the device idle: 161 us against 46 us for 256 rows by 256)
+            const unsigned long long block_y = (input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows;
+            if (block_y > 65535ull) return ST_BOUNDS;
+            YVEX_ALLOW_DYNAMIC_LDS(matvec_f32_block_kernel, kF32BlockLdsBytes);
+            matvec_f32_block_kernel<<<dim3((unsigned)((row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows),
+                                           (unsigned)block_y), 512, kF32BlockLdsBytes, s>>>(a);
+        } else {
             matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
+        }
         return check_launch("matvec_f32_tile16");
     }
     if (scalar) {
