@@ -32,11 +32,11 @@ MFMA_INT8_PEAK_TOPS = 5000.0
 HIDDEN, INTERMEDIATE, EXPERTS, TOPK, ROWS = 7168, 2048, 256, 8, 32
 EXPERT_BYTES = 3 * 3_784_704   # gate + up + down of one IQ2_XXS expert
 # iq2_sweep_kernel<fused gate/up>, 159 distinct routed experts + the shared one: FETCH_SIZE
-# 616 679 x 2.000 KiB + WRITE_SIZE 15 776 x 1.000 KiB per launch (counter units scaled by a 1 GiB
+# 616 664 x 2.000 KiB + WRITE_SIZE 15 776 x 1.000 KiB per launch (counter units scaled by a 1 GiB
 # read kernel and a 256 MiB fill kernel in the same runs)
-GATE_UP_TRAFFIC_BYTES = int((616_679 * 2.0 + 15_776) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((616_664 * 2.0 + 15_776) * 1024)
 GATE_UP_TRAFFIC_EXPERTS = 159
-GATE_UP_IMAGE_TRAFFIC_BYTES = int((664_053 * 2.0 + 18_176) * 1024)   # the same launch over the sweep image
+GATE_UP_IMAGE_TRAFFIC_BYTES = int((664_027 * 2.0 + 18_176) * 1024)   # the same launch over the sweep image
 
 
 def synth_iq2xxs(torch, blocks: int, device, seed: int):
