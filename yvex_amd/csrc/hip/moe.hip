@@ -52,14 +52,33 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v)
     return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
 }
 
-// One row by one wavefront.
-// `scores`: the rows' scores as a launch before this one has published them (the float a
-// double-precision score rounds to, what is computed here otherwise); `logits` is then not read.
+// What a lane reads of one row: the logits (or the scores a launch before this one has
+// published: the float a double-precision score rounds to, what route_row works out from a logit
+// otherwise) and the correction biases of experts 4 lane .. 4 lane + 3. The loads depend on
+// nothing and sit under no condition on the lane (a lane past the last expert reads the last
+// one's again), so a caller can ask for a row's values while it routes the row before: under
+// `if (e < experts)` they were issued, and waited for, one expert after another.
+struct RouteInputs {
+    float value[4], bias[4];
+};
+
+__device__ __forceinline__ void route_inputs_load(RouteInputs &in, const float *__restrict__ values,
+                                                  const float *__restrict__ bias, unsigned long long row,
+                                                  unsigned lane, unsigned experts)
+{
+#pragma unroll
+    for (unsigned i = 0; i < 4u; ++i) {
+        const unsigned e = lane * 4u + i < experts ? lane * 4u + i : experts - 1u;
+        in.value[i] = values[row * experts + e];
+        in.bias[i] = bias ? bias[e] : 0.0f;
+    }
+}
+
+// One row by one wavefront. `published`: in.value holds scores, not logits.
 __device__ __forceinline__ void route_row(
-    const float *__restrict__ logits, const float *__restrict__ bias, unsigned long long row, unsigned lane,
+    const RouteInputs &in, bool published, unsigned long long row, unsigned lane,
     unsigned experts, unsigned topk, int scoring, int normalize, double scaling,
-    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status,
-    const float *__restrict__ scores = nullptr)
+    unsigned long long *__restrict__ selected, float *__restrict__ weights, int *status)
 {
     float score[4];
     unsigned long long key[4];
@@ -69,13 +88,13 @@ __device__ __forceinline__ void route_row(
         score[i] = 0.0f;
         key[i] = 0ull;
         if (e < experts) {
-            if (scores) {
-                score[i] = scores[row * experts + e];
+            if (published) {
+                score[i] = in.value[i];
             } else {
-                const double s = route_score((double)logits[row * experts + e], scoring);
+                const double s = route_score((double)in.value[i], scoring);
                 score[i] = (float)s;      // (a NaN stays a NaN)
             }
-            float biased = (bias ? bias[e] : 0.0f) + score[i];
+            float biased = in.bias[i] + score[i];
             if (!finite_f32(score[i]) || !finite_f32(biased)) raise_status(status, 1);
             biased += 0.0f;   // -0 and +0 must compare equal
             const unsigned bits = __float_as_uint(biased);
@@ -105,7 +124,8 @@ __device__ __forceinline__ void route_row(
                 s = score[i];
                 key[i] = 0ull;
             }
-        s = __shfl(s, (int)(e >> 2), kWave);
+        // (the winner's ordinal is the same in every lane: a lane read, no permute through LDS)
+        s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), (int)(e >> 2)));
         total += (double)s;                 // rank order, in double (src/graph/moe.c:566-574)
         if (lane == rank) picked_score = s;
         if (lane == 0u) selected[row * topk + rank] = e;
@@ -128,7 +148,9 @@ __global__ __launch_bounds__(256) void route_rows_kernel(
 {
     const unsigned long long row = (unsigned long long)blockIdx.x * 4ull + (threadIdx.x >> 6);
     if (row >= rows) return;
-    route_row(logits, bias, row, threadIdx.x & 63u, experts, topk, scoring, normalize, scaling, selected,
+    RouteInputs in;
+    route_inputs_load(in, logits, bias, row, threadIdx.x & 63u, experts);
+    route_row(in, false, row, threadIdx.x & 63u, experts, topk, scoring, normalize, scaling, selected,
               weights, status);
 }
 
@@ -367,9 +389,17 @@ __global__ __launch_bounds__(1024) void decode_prepare_kernel(
                            encoded + (unsigned long long)task * kQ8KBytes, lane, status);
         return;
     }
-    for (unsigned row = wave; row < rows; row += 16u)
-        route_row(logits, bias, row, lane, experts, topk, scoring, normalize, scaling, selected, weights,
-                  status, scores);
+    // a wave's rows one after another, the next row's values on their way while this one is routed
+    const float *values_in = scores ? scores : logits;
+    RouteInputs current;
+    if (wave < rows) route_inputs_load(current, values_in, bias, wave, lane, experts);
+    for (unsigned row = wave; row < rows; row += 16u) {
+        RouteInputs next;
+        route_inputs_load(next, values_in, bias, row + 16u < rows ? row + 16u : row, lane, experts);
+        route_row(current, scores != nullptr, row, lane, experts, topk, scoring, normalize, scaling, selected,
+                  weights, status);
+        current = next;
+    }
     __syncthreads();   // the selections written above are read back by other waves below
     worklist_block(selected, rows * topk, topk, experts, order, expert_ids, bucket_offsets,
                    bucket_populations, sweep_offsets, counts, status, shared_words, true);
