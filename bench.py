@@ -11,7 +11,8 @@ Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up 
 with events on the launch stream; `cpu_baseline` is the reference's own CPU expert path
 (compiled from its sources; the C restatement beside it) timed on the host cores over a bounded
 sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8 matrix
-cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, and `dense` configs
+cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `decode_envelope` the
+headline step with four residual streams around the layer, and `dense` configs
 0-2 and an output head as single matvec launches; the prefill legs and the dense configs carry a
 CPU baseline of their own (the same sample extrapolated per row; the reference's row dot over
 the whole matrix).
@@ -485,6 +486,35 @@ def decode_q4k_leg(torch, K, weights, shared, dev, steps: int, warmup: int):
             "hbm_peak_frac": round(read / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def envelope_leg(torch, routed, shared, router, dev, steps: int, warmup: int):
+    """The headline step for a layer with residual streams around it (four streams of 7168, 24
+    mixing rows, 20 Sinkhorn iterations; src/backend/cuda/moe.c:1210-1254, 1533-1541), through the
+    same execute_rows over the sweep image: mixing projection, ingress with the weighted norm,
+    the layer, egress."""
+    from yvex_amd.host import RowBatchLayer
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(43)
+    streams, mixing = 4, 24
+    x = torch.randn((ROWS, streams * HIDDEN), device=dev, generator=gen)
+    envelope = dict(streams=streams, iterations=20,
+                    function=torch.randn((mixing, streams * HIDDEN), device=dev, generator=gen) / (streams * HIDDEN) ** 0.5,
+                    scale=torch.tensor([0.5, -0.25, 0.75], device=dev),
+                    base=torch.randn(mixing, device=dev, generator=gen) * 0.5,
+                    norm=(1.0 + 0.2 * torch.randn(HIDDEN, device=dev, generator=gen)).to(torch.bfloat16))
+    layer = RowBatchLayer(torch, routed, shared, router, x.cpu().numpy(), ROWS, hidden=HIDDEN,
+                          intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, sweep_image=True,
+                          envelope=envelope)
+    layer.step(defer=False)
+    launches = int(layer.result.kernel_launches)
+    eager_ms = layer.timed(steps, warmup, eager=True)
+    graph_ms = layer.timed(steps, max(warmup, 2))
+    layer.close()
+    return {"workload": "the decode step with 4 residual streams of 7168 around the layer (24 mixing rows, "
+                        "20 Sinkhorn iterations), sweep image",
+            "ms_per_step": round(min(graph_ms, eager_ms), 4), "graph_ms_per_step": round(graph_ms, 4),
+            "eager_ms_per_step": round(eager_ms, 4), "kernel_launches": launches}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -758,6 +788,8 @@ def main() -> int:
                        "down_sweep_alone": round(down_alone_ms, 4) if down_alone_ms else None},
     }
     out["clock"] = device_clock(torch, dev)
+    if not args.no_dense:
+        out["decode_envelope"] = envelope_leg(torch, (gate, up, down), shared, router, dev, args.steps, args.warmup)
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)

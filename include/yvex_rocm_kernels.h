@@ -300,6 +300,16 @@ int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const float *sca
                          double rms_epsilon, double mhc_epsilon, double post_multiplier,
                          float *normalized, float *post, float *combination, int *status,
                          yvex_hip_stream stream);
+/* yvex_hip_mhc_ingress with scale, base and norm as the layer stores them (F32 or BF16 values;
+ * UNSUPPORTED for anything else), decoded inside the launch: the reference decodes each
+ * into an F32 buffer with a launch of its own first (src/backend/cuda/moe.c:1226-1240). Same
+ * outputs and status. */
+int yvex_hip_mhc_ingress_encoded(const float *rows, const float *mixes, const void *scale,
+                                 unsigned int scale_qtype, const void *base, unsigned int base_qtype,
+                                 const void *norm, unsigned int norm_qtype, uint64_t row_count,
+                                 uint64_t streams, uint64_t width, uint64_t iterations, double rms_epsilon,
+                                 double mhc_epsilon, double post_multiplier, float *normalized, float *post,
+                                 float *combination, int *status, yvex_hip_stream stream);
 int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,
                         const float *combination, uint64_t row_count, uint64_t streams,
                         uint64_t width, float *output, int *status, yvex_hip_stream stream);

@@ -311,7 +311,7 @@ class MoeCase:
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
                  shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
-                 down_qtype=None, sweep_image=(), arena_from=None):
+                 down_qtype=None, sweep_image=(), arena_from=None, norm_qtype="BF16"):
         """arena_from: a MoeCase of the same layer on the owning backend of `b` (a shared session):
         its published arena is attached instead of another copy being made resident."""
         self.b, self.oracle = b, oracle
@@ -344,8 +344,16 @@ class MoeCase:
             parts["function"] = g.normal(mixing * expanded, 0.05).view(np.uint8)
             parts["scale"] = g.normal(3, 0.7).view(np.uint8)
             parts["base"] = g.normal(mixing, 0.5).view(np.uint8)
-            parts["norm"] = ((1.0 + g.normal(hidden, 0.2)).astype(np.float32).view(np.uint32) >> 16) \
-                .astype(np.uint16).view(np.uint8)
+            # norm weights as BF16 or F32 values (the ingress decodes them itself) or as I32 values
+            # (a decode launch in front of it)
+            self.norm_qt = getattr(oracle, norm_qtype)
+            values = (1.0 + g.normal(hidden, 0.2)).astype(np.float32)
+            if norm_qtype == "BF16":
+                parts["norm"] = (values.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+            elif norm_qtype == "F32":
+                parts["norm"] = values.view(np.uint8)
+            else:
+                parts["norm"] = np.rint(values * 2.0).astype(np.int32).view(np.uint8)
         # experts held as the sweeps' image: built by the library's host builder, resident beside
         # the canonical bytes
         self.decisions = {}
@@ -427,7 +435,8 @@ class MoeCase:
             view(abi.W_MHC_FUNCTION, "function", 0, expanded, mixing, expanded * 4, abi.ACT_DEVICE_F32)
             view(abi.W_MHC_SCALE, "scale", 0, 3, 1, 12, abi.ACT_DEVICE_F32)
             view(abi.W_MHC_BASE, "base", 0, mixing, 1, mixing * 4, abi.ACT_DEVICE_F32)
-            view(abi.W_FFN_NORM, "norm", 30, hidden, 1, hidden * 2, abi.ACT_DEVICE_F32)
+            view(abi.W_FFN_NORM, "norm", self.norm_qt, hidden, 1, oracle.row_bytes(self.norm_qt, hidden),
+                 abi.ACT_DEVICE_F32)
         self.ops = b.lib.yvex_rocm_backend_moe_operations_get(b.handle).contents
         need, err = abi.ULL(), abi.Error()
         assert self.ops.workspace_required(C.byref(self.plan), rows, C.byref(need), C.byref(err)) == 0
@@ -462,7 +471,7 @@ class MoeCase:
         o, p = self.oracle, self.parts
         x, ingress = self.x, None
         if self.streams:      # src/graph/moe.c:446-495 in front, numeric.c:828-877 behind
-            norm = (p["norm"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+            norm = o.decode_rows(self.norm_qt, p["norm"], self.hidden)[0]
             rc, x, post, comb = o.moe_ffn_prepare(
                 o.F32, p["function"], self.x, p["scale"].view(np.float32), p["base"].view(np.float32), norm,
                 streams=self.streams, width=self.hidden, iterations=self.iterations, rms_epsilon=1e-6,
@@ -514,9 +523,11 @@ def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, sh
     assert res.kernel_launches >= 6 and res.memory.complete == 1
 
 
-@pytest.mark.parametrize("qtype,streams,rows,hidden,iterations", [
-    ("IQ2_XXS", 4, 5, 512, 20), ("IQ2_XXS", 1, 3, 512, 1), ("Q8_0", 2, 7, 256, 3)])
-def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, rows, hidden, iterations):
+@pytest.mark.parametrize("qtype,streams,rows,hidden,iterations,norm_qtype", [
+    ("IQ2_XXS", 4, 5, 512, 20, "BF16"), ("IQ2_XXS", 1, 3, 512, 1, "F32"), ("Q8_0", 2, 7, 256, 3, "I32"),
+    ("IQ2_XXS", 4, 12, 512, 20, "BF16")])
+def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, rows, hidden, iterations,
+                                            norm_qtype):
     """The layer as the reference's row-batch operation runs it (src/backend/cuda/moe.c:1210-1254,
     1533-1541): ingress over the expanded rows, weighted norm, routing and experts on the
     normalised row, egress back onto the streams. The mixes come from the F32-accumulating
@@ -524,7 +535,7 @@ def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, row
     matrix differ from the CPU's only by what two maths libraries' double exp differ (1e-6), the
     normalised row, the routing and the layer's combined rows are the CPU path's."""
     case = MoeCase(backend, oracle, qtype=qtype, hidden=hidden, rows=rows, streams=streams,
-                   iterations=iterations)
+                   iterations=iterations, norm_qtype=norm_qtype)
     backend.workspace(case.workspace_bytes)
     assert case.execute() == 0, case.err.message
     want = case.oracle_layer(act_q8=True)
@@ -542,7 +553,9 @@ def test_execute_rows_with_residual_streams(backend, oracle, qtype, streams, row
     assert rc == 0 and np.array_equal(got.view(np.uint32), replay.view(np.uint32))
     scale = np.abs(want["envelope"]) + np.abs(want["combined"]).max()
     assert np.all(np.abs(got - want["envelope"]) <= 2.0 ** -6 * scale)
-    assert case.result.completed == 1 and case.result.kernel_launches >= 14
+    # mixing projection, ingress (which decodes scale, base and norm itself) and egress on top of
+    # the layer's own launches
+    assert case.result.completed == 1 and case.result.kernel_launches >= 11
 
 
 @pytest.mark.parametrize("streams", [0, 4])
@@ -1083,7 +1096,7 @@ def token_oracle(case, row):
     """CPU path for one row: ingress, routing, experts on F32 activations in rank order, shared
     expert, bf16(routed + shared), egress (src/runtime/moe.c:596-645)."""
     o, p = case.oracle, case.parts
-    norm = (p["norm"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    norm = o.decode_rows(case.norm_qt, p["norm"], case.hidden)[0]
     rc, x, post, comb = o.moe_ffn_prepare(
         o.F32, p["function"], case.x[row], p["scale"].view(np.float32), p["base"].view(np.float32), norm,
         streams=case.streams, width=case.hidden, iterations=case.iterations, rms_epsilon=1e-6,

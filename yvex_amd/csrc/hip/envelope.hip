@@ -55,18 +55,38 @@ __device__ __forceinline__ float4 bf16_round4(float4 v)
     return make_float4(bf16_round(v.x), bf16_round(v.y), bf16_round(v.z), bf16_round(v.w));
 }
 
+// A coefficient vector (scale, base, norm) as the layer stores it, F32 or BF16 values, decoded
+// where they are used (the reference decodes them into F32 buffers with launches of their own,
+// src/backend/cuda/moe.c:1226-1240; the decoded value is the same float).
+__device__ __forceinline__ float coefficient(const void *values, unsigned qtype, unsigned index)
+{
+    if (qtype == QT_F32) return static_cast<const float *>(values)[index];
+    return __uint_as_float((unsigned)static_cast<const unsigned short *>(values)[index] << 16);
+}
+
+// Four consecutive coefficients from a 16-byte (F32) or 8-byte (BF16) aligned address.
+__device__ __forceinline__ float4 coefficient4(const void *values, unsigned qtype, unsigned quad)
+{
+    if (qtype == QT_F32) return static_cast<const float4 *>(values)[quad];
+    const uint2 v = static_cast<const uint2 *>(values)[quad];
+    return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                       __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+
 // One workgroup per row. The row is read twice (mean square, then the gated sum of the streams);
 // both passes keep four 16-byte loads per thread in flight, because a row is a short stream and
 // a loop that waits for each load in turn spends its time on latency; long rows take 1024
 // threads for the same reason. Rows whose width is not a multiple of four take the scalar loops.
 template <unsigned THREADS>
 __global__ __launch_bounds__(THREADS) void mhc_ingress_kernel(
-    const float *__restrict__ rows, const float *__restrict__ mixes, const float *__restrict__ scale,
-    const float *__restrict__ base, const float *__restrict__ norm, unsigned streams, unsigned width,
+    const float *__restrict__ rows, const float *__restrict__ mixes, const void *__restrict__ scale_values,
+    const void *__restrict__ base_values, const void *__restrict__ norm, unsigned scale_qtype,
+    unsigned base_qtype, unsigned norm_qtype, unsigned streams, unsigned width,
     unsigned iterations, double rms_epsilon, double mhc_epsilon, double post_multiplier,
     float *__restrict__ normalized, float *__restrict__ post, float *__restrict__ combination,
     int quads, int *status)
 {
+    __shared__ float base[64], scale[3];      // (streams + 2) * streams <= 63 mixing rows
     extern __shared__ __align__(16) float collapsed[];   // width values
     __shared__ double slots[THREADS / 64u];
     __shared__ double gate[8];
@@ -108,8 +128,15 @@ __global__ __launch_bounds__(THREADS) void mhc_ingress_kernel(
             squares += (double)v * (double)v;
         }
     }
-    if (tid < mixing_rows) bad |= !finite_f32(base[tid]) || !finite_f32(mix[tid]);
-    if (tid < 3u) bad |= !finite_f32(scale[tid]);
+    if (tid < mixing_rows) {
+        base[tid] = coefficient(base_values, base_qtype, tid);
+        bad |= !finite_f32(base[tid]) || !finite_f32(mix[tid]);
+    }
+    if (tid < 3u) {
+        scale[tid] = coefficient(scale_values, scale_qtype, tid);
+        bad |= !finite_f32(scale[tid]);
+    }
+    // (the barriers inside the sum publish base and scale to the threads that read them below)
     const double inverse = 1.0 / sqrt(workgroup_sum<THREADS / 64u>(squares, slots) / (double)expanded + rms_epsilon);
     bad |= !finite_f64(inverse);
 
@@ -206,11 +233,10 @@ __global__ __launch_bounds__(THREADS) void mhc_ingress_kernel(
     const double norm_inverse = 1.0 / sqrt(mean + rms_epsilon);
     bad |= !finite_f64(norm_inverse);
     if (quads && streams <= kBatch) {
-        const float4 *norm4 = reinterpret_cast<const float4 *>(norm);
         float4 *out4 = reinterpret_cast<float4 *>(normalized + row * width);
         const unsigned count = width >> 2;
         for (unsigned at = tid; at < count; at += THREADS) {
-            const float4 w = norm4[at], v = reinterpret_cast<const float4 *>(collapsed)[at];
+            const float4 w = coefficient4(norm, norm_qtype, at), v = reinterpret_cast<const float4 *>(collapsed)[at];
             const float in_lane[4] = {v.x, v.y, v.z, v.w}, weight[4] = {w.x, w.y, w.z, w.w};
             float value[4];
 #pragma unroll
@@ -224,7 +250,7 @@ __global__ __launch_bounds__(THREADS) void mhc_ingress_kernel(
         }
     } else {
         for (unsigned lane = tid; lane < width; lane += THREADS) {
-            const float weight = norm[lane];
+            const float weight = coefficient(norm, norm_qtype, lane);
             double v = (double)collapsed[lane] * norm_inverse;
             v *= (double)weight;
             const float value = (float)v;
@@ -296,15 +322,21 @@ static bool envelope_shape_ok(uint64_t row_count, uint64_t streams, uint64_t wid
            row_count <= 0x7fffffffull / ((width + kEnvelopeThreads - 1u) / kEnvelopeThreads);
 }
 
-extern "C" int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const float *scale,
-                                    const float *base, const float *norm, uint64_t row_count,
-                                    uint64_t streams, uint64_t width, uint64_t iterations,
-                                    double rms_epsilon, double mhc_epsilon, double post_multiplier,
-                                    float *normalized, float *post, float *combination, int *status,
-                                    yvex_hip_stream stream)
+static int launch_mhc_ingress(const float *rows, const float *mixes, const void *scale, unsigned scale_qtype,
+                              const void *base, unsigned base_qtype, const void *norm, unsigned norm_qtype,
+                              uint64_t row_count, uint64_t streams, uint64_t width, uint64_t iterations,
+                              double rms_epsilon, double mhc_epsilon, double post_multiplier,
+                              float *normalized, float *post, float *combination, int *status,
+                              yvex_hip_stream stream)
 {
     if (!rows || !mixes || !scale || !base || !norm || !normalized || !post || !combination || !status)
         return ST_INVALID_ARG;
+    const unsigned qtypes[3] = {scale_qtype, base_qtype, norm_qtype};
+    const void *const vectors[3] = {scale, base, norm};
+    for (int k = 0; k < 3; ++k) {
+        if (qtypes[k] != QT_F32 && qtypes[k] != QT_BF16) return ST_UNSUPPORTED;
+        if ((uintptr_t)vectors[k] & (qtypes[k] == QT_F32 ? 3u : 1u)) return ST_INVALID_ARG;
+    }
     if (!envelope_shape_ok(row_count, streams, width) || !iterations || iterations > 0xffffffffull)
         return ST_BOUNDS;
     if (!(rms_epsilon > 0.0) || !(mhc_epsilon > 0.0) || !(post_multiplier > 0.0) ||
@@ -324,17 +356,46 @@ extern "C" int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const
         set_last_error_text("mhc_ingress: the collapsed row does not fit in LDS");
         return ST_BACKEND;
     }
-    const int quads = width % 4u == 0u && !(((uintptr_t)rows | (uintptr_t)norm | (uintptr_t)normalized) & 15u);
+    const int quads = width % 4u == 0u && !(((uintptr_t)rows | (uintptr_t)normalized) & 15u) &&
+                      !((uintptr_t)norm & (norm_qtype == QT_F32 ? 15u : 7u));
     const unsigned lds = (unsigned)(width * sizeof(float));
     if (streams * width >= 8192u)
         mhc_ingress_kernel<1024><<<(unsigned)row_count, 1024, lds, as_stream(stream)>>>(
-            rows, mixes, scale, base, norm, (unsigned)streams, (unsigned)width, (unsigned)iterations,
-            rms_epsilon, mhc_epsilon, post_multiplier, normalized, post, combination, quads, status);
+            rows, mixes, scale, base, norm, scale_qtype, base_qtype, norm_qtype, (unsigned)streams,
+            (unsigned)width, (unsigned)iterations, rms_epsilon, mhc_epsilon, post_multiplier, normalized, post,
+            combination, quads, status);
     else
         mhc_ingress_kernel<256><<<(unsigned)row_count, 256, lds, as_stream(stream)>>>(
-            rows, mixes, scale, base, norm, (unsigned)streams, (unsigned)width, (unsigned)iterations,
-            rms_epsilon, mhc_epsilon, post_multiplier, normalized, post, combination, quads, status);
+            rows, mixes, scale, base, norm, scale_qtype, base_qtype, norm_qtype, (unsigned)streams,
+            (unsigned)width, (unsigned)iterations, rms_epsilon, mhc_epsilon, post_multiplier, normalized, post,
+            combination, quads, status);
     return check_launch("mhc_ingress");
+}
+
+extern "C" int yvex_hip_mhc_ingress(const float *rows, const float *mixes, const float *scale,
+                                    const float *base, const float *norm, uint64_t row_count,
+                                    uint64_t streams, uint64_t width, uint64_t iterations,
+                                    double rms_epsilon, double mhc_epsilon, double post_multiplier,
+                                    float *normalized, float *post, float *combination, int *status,
+                                    yvex_hip_stream stream)
+{
+    return launch_mhc_ingress(rows, mixes, scale, QT_F32, base, QT_F32, norm, QT_F32, row_count, streams, width,
+                              iterations, rms_epsilon, mhc_epsilon, post_multiplier, normalized, post,
+                              combination, status, stream);
+}
+
+extern "C" int yvex_hip_mhc_ingress_encoded(const float *rows, const float *mixes, const void *scale,
+                                            unsigned int scale_qtype, const void *base,
+                                            unsigned int base_qtype, const void *norm,
+                                            unsigned int norm_qtype, uint64_t row_count, uint64_t streams,
+                                            uint64_t width, uint64_t iterations, double rms_epsilon,
+                                            double mhc_epsilon, double post_multiplier, float *normalized,
+                                            float *post, float *combination, int *status,
+                                            yvex_hip_stream stream)
+{
+    return launch_mhc_ingress(rows, mixes, scale, scale_qtype, base, base_qtype, norm, norm_qtype, row_count,
+                              streams, width, iterations, rms_epsilon, mhc_epsilon, post_multiplier, normalized,
+                              post, combination, status, stream);
 }
 
 extern "C" int yvex_hip_mhc_egress(const float *core, const float *rows, const float *post,

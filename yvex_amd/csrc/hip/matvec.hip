@@ -944,9 +944,15 @@ extern "C" int yvex_hip_row_dot(const uint8_t *encoded, unsigned int qtype, cons
 // Splits of an F32 projection over a decode-width batch: per-wave shares of 128 columns.
 static unsigned f32_rows_splits(uint64_t row_width, uint64_t input_rows)
 {
-    if (input_rows < 8u || input_rows >= 256u || row_width % 512u) return 0u;
-    const uint64_t splits = row_width / 512u;
-    return splits >= 2u && splits <= 64u ? (unsigned)splits : 0u;
+    if (input_rows < 8u || input_rows >= 256u || row_width % 128u) return 0u;
+    // 512 columns a split (128 a wave) where that gives 2 to 64 splits; a wider row takes the
+    // most splits up to 64 that leave every wave a multiple of 16 columns
+    if (row_width % 512u == 0u && row_width / 512u >= 2u && row_width / 512u <= 64u)
+        return (unsigned)(row_width / 512u);
+    if (row_width < 64u * 512u) return 0u;
+    for (unsigned splits = 64u; splits >= 2u; --splits)
+        if (row_width % (64ull * splits) == 0u) return splits;
+    return 0u;
 }
 
 extern "C" uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64_t row_width,

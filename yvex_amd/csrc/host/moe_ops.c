@@ -759,15 +759,56 @@ sequence:
         static const int flat_slots[3] = {YVEX_MOE_WEIGHT_MHC_SCALE, YVEX_MOE_WEIGHT_MHC_BASE,
                                           YVEX_MOE_WEIGHT_FFN_NORM};
         void *flat_targets[3];
-        int k;
+        int k, fused_coefficients;
         flat_targets[0] = AT(scale);
         flat_targets[1] = AT(base);
         flat_targets[2] = AT(norm);
+        /* F32 mixing rows over a decode-width batch: two dozen weight rows are four tiles, so the
+         * row width is split over the whole device like the router's, the partial sums in the
+         * pair-output range (116 us unsplit for 24 x 28672 against 32 rows, 11 us split) */
+        if (function->qtype == YVEX_GGUF_QTYPE_F32) {
+            unsigned long long need = yvex_hip_matvec_f32_scratch_bytes(layer->mhc_mixing_rows, expanded, row_count);
+            int lend = need && need <= pairs * hidden * sizeof(float);
+            unsigned int mixing_launches = yvex_hip_matvec_f32_rows_launches(
+                (const float *)(uintptr_t)envelope_addresses[0], layer->mhc_mixing_rows, expanded,
+                (const float *)rows->device_rows->data, row_count, expanded, lend ? AT(pair_outputs) : NULL,
+                lend ? need : 0ull);
+            LAUNCH(yvex_hip_matvec_f32_rows((const float *)(uintptr_t)envelope_addresses[0],
+                                            layer->mhc_mixing_rows, expanded,
+                                            (const float *)rows->device_rows->data, row_count, expanded, NULL,
+                                            (float *)AT(mixes), layer->mhc_mixing_rows, 0,
+                                            lend ? AT(pair_outputs) : NULL, lend ? need : 0ull, (int *)status,
+                                            stream), "rocm.moe.rows.mhc-function");
+            if (rc == YVEX_OK && mixing_launches == 2u && graph_mode != GRAPH_REPLAY) launches++;
+        } else
         LAUNCH(yvex_hip_matvec((const uint8_t *)(uintptr_t)envelope_addresses[0], function->qtype,
                                layer->mhc_mixing_rows, expanded, function->row_bytes,
                                rows->device_rows->data, 0, row_count, expanded, NULL,
                                (float *)AT(mixes), layer->mhc_mixing_rows, 0, (int *)status, stream),
                "rocm.moe.rows.mhc-function");
+        /* coefficient vectors stored as F32 or BF16 values are decoded by the ingress itself;
+         * I32 ones go through the decode launches first */
+        fused_coefficients = 1;
+        for (k = 0; k < 3; ++k) {
+            unsigned int q = views[flat_slots[k]].qtype;
+            if (q == YVEX_GGUF_QTYPE_F32) fused_coefficients &= !(envelope_addresses[1 + k] & 3ull);
+            else if (q == YVEX_GGUF_QTYPE_BF16) fused_coefficients &= !(envelope_addresses[1 + k] & 1ull);
+            else fused_coefficients = 0;
+        }
+        if (fused_coefficients)
+            LAUNCH(yvex_hip_mhc_ingress_encoded((const float *)rows->device_rows->data, (const float *)AT(mixes),
+                                                (const void *)(uintptr_t)envelope_addresses[1],
+                                                views[flat_slots[0]].qtype,
+                                                (const void *)(uintptr_t)envelope_addresses[2],
+                                                views[flat_slots[1]].qtype,
+                                                (const void *)(uintptr_t)envelope_addresses[3],
+                                                views[flat_slots[2]].qtype, row_count, streams, hidden,
+                                                layer->mhc_sinkhorn_iterations, layer->rms_epsilon,
+                                                layer->mhc_epsilon, layer->mhc_post_multiplier,
+                                                (float *)AT(normalized), (float *)AT(post),
+                                                (float *)AT(combination), (int *)status, stream),
+                   "rocm.moe.rows.mhc-ingress");
+        else {
         for (k = 0; k < 3; ++k)
             LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)envelope_addresses[1 + k],
                                    views[flat_slots[k]].qtype, 1ull, views[flat_slots[k]].row_width,
@@ -781,6 +822,7 @@ sequence:
                                     (float *)AT(normalized), (float *)AT(post),
                                     (float *)AT(combination), (int *)status, stream),
                "rocm.moe.rows.mhc-ingress");
+        }
         activations = AT(normalized);
         combined_target = AT(combined);
     }

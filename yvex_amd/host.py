@@ -102,7 +102,12 @@ class RowBatchLayer:
     call, src/runtime/moe.c:1567-1576)."""
 
     def __init__(self, torch, routed, shared, router, x_host, rows, *, hidden, intermediate, experts, topk,
-                 qtype=16, sweep_image=False, scoring=abi.SCORING_SIGMOID, scaling=1.0, limit=10.0):
+                 qtype=16, sweep_image=False, scoring=abi.SCORING_SIGMOID, scaling=1.0, limit=10.0,
+                 envelope=None):
+        """envelope: None, or the residual-stream weights around the layer as device tensors,
+        dict(streams, iterations, function [F32 (streams + 2) * streams x streams * hidden], scale
+        [F32 3], base [F32 (streams + 2) * streams], norm [BF16 hidden]); x_host then holds
+        streams * hidden values a row and so does the output."""
         HIDDEN, INTERMEDIATE, EXPERTS, TOPK = hidden, intermediate, experts, topk
         self.C, self.abi, self.np, self.rows, self.hidden = C, abi, np, rows, hidden
         self.b = Backend()
@@ -113,6 +118,13 @@ class RowBatchLayer:
         plan.schema_version, plan.router_class, plan.scoring = 1, abi.ROUTER_LEARNED, scoring
         plan.hidden_width = plan.expanded_width = HIDDEN
         plan.residual_streams = 1
+        streams = envelope["streams"] if envelope else 0
+        expanded = streams * HIDDEN if envelope else HIDDEN
+        if envelope:
+            plan.residual_streams, plan.expanded_width = streams, expanded
+            plan.mhc_mixing_rows, plan.mhc_sinkhorn_iterations = (streams + 2) * streams, envelope["iterations"]
+            plan.rms_epsilon, plan.mhc_epsilon, plan.mhc_post_multiplier = 1e-6, 1e-6, 2.0
+            self.keep += tuple(envelope[k] for k in ("function", "scale", "base", "norm"))
         plan.routed_experts, plan.shared_experts, plan.experts_per_token = EXPERTS, 1, TOPK
         plan.expert_intermediate_width = plan.shared_intermediate_width = INTERMEDIATE
         plan.routed_scaling_factor, plan.activation_limit = scaling, limit
@@ -160,14 +172,22 @@ class RowBatchLayer:
         view(abi.W_SHARED_GATE, shared[0], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
         view(abi.W_SHARED_UP, shared[1], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
         view(abi.W_SHARED_DOWN, shared[2], qtype, INTERMEDIATE, HIDDEN, rb_i, enc, shared_c)
+        if envelope:
+            mixing = (streams + 2) * streams
+            f32 = abi.ACT_DEVICE_F32
+            view(abi.W_MHC_FUNCTION, envelope["function"], 0, expanded, mixing, expanded * 4, f32)
+            view(abi.W_MHC_SCALE, envelope["scale"], 0, 3, 1, 12, f32)
+            view(abi.W_MHC_BASE, envelope["base"], 0, mixing, 1, mixing * 4, f32)
+            view(abi.W_FFN_NORM, envelope["norm"], 30, HIDDEN, 1, HIDDEN * 2, f32)
         self.ops = self.b.lib.yvex_rocm_backend_moe_operations_get(self.b.handle).contents
         need, err = abi.ULL(), abi.Error()
         if self.ops.workspace_required(C.byref(plan), rows, C.byref(need), C.byref(err)) != 0:
             raise RuntimeError(err.message.decode())
         self.b.workspace(need.value)
-        self.rows_in, self.rows_out = self.b.f32(x_host), self.b.empty_f32(rows * HIDDEN)
+        self.width = expanded
+        self.rows_in, self.rows_out = self.b.f32(x_host), self.b.empty_f32(rows * expanded)
         batch = self.batch = abi.RowBatch()
-        batch.schema_version, batch.row_count, batch.row_width, batch.row_stride = 1, rows, HIDDEN, HIDDEN
+        batch.schema_version, batch.row_count, batch.row_width, batch.row_stride = 1, rows, expanded, expanded
         batch.device_rows, batch.device_outputs = self.rows_in, self.rows_out
         batch.provenance, batch.execution_class = abi.BATCH_MULTI_SESSION, 1
         self.out = abi.RowBatchOutput()
@@ -202,7 +222,7 @@ class RowBatchLayer:
         return (time.perf_counter() - t0) * 1e3 / steps
 
     def output(self):
-        return self.b.read_f32(self.rows_out, self.rows * self.hidden).reshape(self.rows, self.hidden)
+        return self.b.read_f32(self.rows_out, self.rows * self.width).reshape(self.rows, self.width)
 
     def close(self):
         self.b.close()
