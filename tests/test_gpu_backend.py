@@ -311,7 +311,7 @@ class MoeCase:
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
                  shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
-                 down_qtype=None, sweep_image=(), arena_from=None, norm_qtype="BF16"):
+                 down_qtype=None, sweep_image=(), arena_from=None, norm_qtype="BF16", bias_qtype="F32"):
         """arena_from: a MoeCase of the same layer on the owning backend of `b` (a shared session):
         its published arena is attached instead of another copy being made resident."""
         self.b, self.oracle = b, oracle
@@ -334,6 +334,13 @@ class MoeCase:
             "sup": g.weights(qt, intermediate, hidden),
             "sdown": g.weights(qt_down, hidden, intermediate),
         }
+        # the correction bias as F32 values (read where they lie) or as BF16 values (decoded into
+        # the workspace first)
+        self.bias_qt = getattr(oracle, bias_qtype)
+        self.bias_values = parts["bias"].view(np.float32)
+        if bias_qtype == "BF16":
+            parts["bias"] = (self.bias_values.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+            self.bias_values = (parts["bias"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
         self.hash_vocab = hash_vocab
         if hash_vocab:  # hash router: an I32 table of expert ordinals per token id
             rng = np.random.default_rng(seed)
@@ -422,7 +429,8 @@ class MoeCase:
                 v.encoded, v.storage_bytes = host + offsets[name + ".image"], parts[name + ".image"].nbytes
 
         view(abi.W_ROUTER, "router", 0, hidden, experts, hidden * 4, abi.ACT_DEVICE_F32)
-        view(abi.W_ROUTER_BIAS, "bias", 0, experts, 1, experts * 4, abi.ACT_DEVICE_F32)
+        view(abi.W_ROUTER_BIAS, "bias", self.bias_qt, experts, 1, oracle.row_bytes(self.bias_qt, experts),
+             abi.ACT_DEVICE_F32)
         view(abi.W_ROUTED_GATE, "gate", qt, hidden, experts * intermediate, rb_h)
         view(abi.W_ROUTED_UP, "up", qt, hidden, experts * intermediate, rb_h)
         view(abi.W_ROUTED_DOWN, "down", qt_down, intermediate, experts * hidden, rb_i)
@@ -481,7 +489,7 @@ class MoeCase:
         router = p["router"].view(np.float32).reshape(self.experts, self.hidden)
         logits = o.matvec(o.F32, p["router"], self.experts, self.hidden, x)
         assert np.allclose(logits, x @ router.T, rtol=1e-4, atol=1e-5)
-        bias = p["bias"].view(np.float32) if self.plan.requires_correction_bias else None
+        bias = self.bias_values if self.plan.requires_correction_bias else None
         shared = (p["sgate"], p["sup"], p["sdown"]) if self.plan.shared_experts else None
         want = o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
                            topk=self.topk, qtypes=self.qtypes, routed=(p["gate"], p["up"], p["down"]),
@@ -496,13 +504,13 @@ class MoeCase:
         return want
 
 
-@pytest.mark.parametrize("qtype,act,scoring,shared", [
-    ("IQ2_XXS", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True),
-    ("IQ2_XXS", abi.ACT_DEVICE_F32, abi.SCORING_SIGMOID, True),
-    ("Q4_K", abi.ACT_DEVICE_ENCODED, abi.SCORING_SIGMOID, False),
-    ("Q8_0", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True)])
-def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, shared):
-    case = MoeCase(backend, oracle, qtype=qtype, act=act, scoring=scoring, shared=shared)
+@pytest.mark.parametrize("qtype,act,scoring,shared,bias_qtype", [
+    ("IQ2_XXS", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True, "F32"),
+    ("IQ2_XXS", abi.ACT_DEVICE_F32, abi.SCORING_SIGMOID, True, "F32"),
+    ("Q4_K", abi.ACT_DEVICE_ENCODED, abi.SCORING_SIGMOID, False, "BF16"),
+    ("Q8_0", abi.ACT_DEVICE_ENCODED, abi.SCORING_SQRT_SOFTPLUS, True, "F32")])
+def test_execute_rows_matches_cpu_layer(backend, oracle, qtype, act, scoring, shared, bias_qtype):
+    case = MoeCase(backend, oracle, qtype=qtype, act=act, scoring=scoring, shared=shared, bias_qtype=bias_qtype)
     backend.workspace(case.workspace_bytes)
     rc = case.execute()
     assert rc == 0, case.err.message
@@ -1106,7 +1114,7 @@ def token_oracle(case, row):
     want = o.moe_layer(hidden=case.hidden, intermediate=case.intermediate, experts=case.experts,
                        topk=case.topk, qtypes=case.qtypes, routed=(p["gate"], p["up"], p["down"]),
                        shared=(p["sgate"], p["sup"], p["sdown"]), inputs=x, logits=logits,
-                       bias=p["bias"].view(np.float32), scoring=case.scoring, normalize=True, scaling=1.5,
+                       bias=case.bias_values, scoring=case.scoring, normalize=True, scaling=1.5,
                        act_q8=False, threads=1)
     rc, want["envelope"] = o.mhc_post(want["combined"], case.x[row], post, comb, streams=case.streams,
                                       width=case.hidden)

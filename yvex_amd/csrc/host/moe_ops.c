@@ -488,6 +488,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     unsigned long long envelope_addresses[4] = {0}, streams = 0ull, expanded;
     unsigned long long d2h = 0ull, started, counts[4] = {0}, status_launches = 0ull;
     const void *activations;
+    const float *bias_rows;
     void *combined_target;
     unsigned long long table_address = 0ull;
     int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer, scored = 0;
@@ -871,7 +872,13 @@ sequence:
                                             (float *)AT(weights), (int *)status, stream),
                "rocm.moe.rows.route");
     }
+    /* a correction bias stored as F32 values is read where it lies; any other encoding is
+     * decoded into the workspace first */
+    bias_rows = NULL;
     if (!hash_router && layer->requires_correction_bias)
+        bias_rows = views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype == YVEX_GGUF_QTYPE_F32 && !(bias_address & 3ull)
+                        ? (const float *)(uintptr_t)bias_address : (const float *)AT(bias);
+    if (bias_rows && bias_rows == (const float *)AT(bias))
         LAUNCH(yvex_hip_gather((const uint8_t *)(uintptr_t)bias_address, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].qtype,
                                1ull, experts, views[YVEX_MOE_WEIGHT_ROUTER_BIAS].row_bytes, NULL, 1ull,
                                (float *)AT(bias), (int *)status, stream), "rocm.moe.rows.bias");
@@ -880,7 +887,7 @@ sequence:
     const int need_q8 = routed_q8 || (has_shared && shared_q8);
     if (scored) {
         LAUNCH(yvex_hip_moe_prepare_scored((const float *)AT(routed),
-                                           layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                           bias_rows,
                                            row_count, experts, topk, layer->normalize_topk_probabilities,
                                            layer->routed_scaling_factor, (uint64_t *)AT(selected),
                                            (float *)AT(weights), (uint64_t *)AT(order),
@@ -892,7 +899,7 @@ sequence:
                "rocm.moe.rows.prepare");
     } else if (!hash_router && yvex_hip_moe_prepare_supported(row_count, experts, topk)) {
         LAUNCH(yvex_hip_moe_prepare((const float *)AT(logits),
-                                    layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                    bias_rows,
                                     row_count, experts, topk, (int)layer->scoring,
                                     layer->normalize_topk_probabilities, layer->routed_scaling_factor,
                                     (uint64_t *)AT(selected), (float *)AT(weights), (uint64_t *)AT(order),
@@ -904,7 +911,7 @@ sequence:
     } else {
         if (!hash_router)
             LAUNCH(yvex_hip_moe_route_rows((const float *)AT(logits),
-                                           layer->requires_correction_bias ? (const float *)AT(bias) : NULL,
+                                           bias_rows,
                                            row_count, experts, topk, (int)layer->scoring,
                                            layer->normalize_topk_probabilities,
                                            layer->routed_scaling_factor, (uint64_t *)AT(selected),
