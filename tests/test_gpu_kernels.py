@@ -90,6 +90,8 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
 @pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32),
                                                (256, 7168, 300), (40, 96, 260), (256, 7168, 8), (3, 256, 9),
                                                (45, 448, 257), (32, 64, 256),
+                                               # fewer than eight input rows: a workgroup a weight row
+                                               (256, 7168, 1), (24, 28672, 5), (7, 100, 3), (9, 4096, 2), (5, 30, 2),
                                                # enough (32 rows x 64 input rows) blocks for the device and
                                                # 128-column chunks: the kernel with operands staged in LDS,
                                                # ragged on both sides

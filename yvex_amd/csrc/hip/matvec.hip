@@ -400,6 +400,74 @@ __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsign
     }
 }
 
+// F32 weight rows against fewer than eight F32 input rows (the router and mixing projections of a
+// batch of one to seven tokens): the lane-strided kernel above walks a row one load at a time, a
+// wave a row, and a 256 x 7168 router took 90 us of memory round trips. Here a workgroup owns
+// one weight row, its 256 threads take 16-byte pieces of it side by side (a 4 KB stretch a
+// step), DEPTH steps of weight and input loads are in flight before the first product, and the
+// four waves' double-precision sums are joined through LDS in wave order. Products and sums in
+// double as above.
+template <int T, int DEPTH>
+__global__ __launch_bounds__(256) void matvec_f32_few_kernel(MatvecArgs a)
+{
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    __shared__ double partial[3][T];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned long long row = blockIdx.x, in0 = (unsigned long long)blockIdx.y * T;
+    const v4f *w4 = reinterpret_cast<const v4f *>(a.encoded + row * a.row_bytes);
+    const v4f *x4[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const unsigned long long in = in0 + t < a.input_rows ? in0 + t : a.input_rows - 1ull;   // clamped rows are never written
+        x4[t] = reinterpret_cast<const v4f *>((const float *)a.input + in * a.input_stride);
+    }
+    const unsigned quads = (unsigned)(a.row_width >> 2);
+    double acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0;
+    unsigned bad = 0u;
+    for (unsigned first = threadIdx.x; first < quads; first += 256u * DEPTH) {
+        v4f w[DEPTH], x[T][DEPTH];
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            const unsigned at = first + 256u * u < quads ? first + 256u * u : first;
+            w[u] = w4[at];
+#pragma unroll
+            for (int t = 0; t < T; ++t) x[t][u] = x4[t][at];
+        }
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            // (a step past the end repeated the first one: its inputs count as zeros. A branch
+            // here would pull each step's loads behind it, one wait a step)
+            const bool live = first + 256u * u < quads;
+            bad |= (unsigned)!finite_f32(w[u][0]) | (unsigned)!finite_f32(w[u][1]) | (unsigned)!finite_f32(w[u][2]) |
+                   (unsigned)!finite_f32(w[u][3]);
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                if (!live) x[t][u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[t] += (double)w[u][c] * (double)x[t][u][c];
+        }
+    }
+    if (bad) raise_status(a.status, 1);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) acc[t] += __shfl_xor(acc[t], offset, kWave);
+        if (wave && lane == 0u) partial[wave - 1u][t] = acc[t];
+    }
+    __syncthreads();
+    if (threadIdx.x != 0u) return;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (in0 + t >= a.input_rows) continue;
+        const double sum = acc[t] + partial[0][t] + partial[1][t] + partial[2][t];
+        matvec_publish(a, in0 + t, row, (float)sum);
+    }
+}
+
 // F32 weight rows against a batch of F32 input rows (a router or mixing projection over a row
 // batch) on the double-precision matrix cores: a workgroup of WAVES waves owns 16 weight rows x
 // 16 input rows on V_MFMA_F64_16X16X4_F64 and its waves split the row width. Lane (i, q) loads
@@ -853,6 +921,16 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
             matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
         }
         return check_launch("matvec_f32_tile16");
+    }
+    if (qtype == QT_F32 && input_rows < 8ull && row_width % 4ull == 0ull && row_count <= 0x7fffffffull &&
+        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) && !(row_bytes & 15ull)) {
+        if (input_rows == 1ull)
+            matvec_f32_few_kernel<1, 8><<<dim3((unsigned)row_count, 1), 256, 0, s>>>(a);
+        else if (input_rows == 2ull)
+            matvec_f32_few_kernel<2, 8><<<dim3((unsigned)row_count, 1), 256, 0, s>>>(a);
+        else
+            matvec_f32_few_kernel<4, 4><<<dim3((unsigned)row_count, (unsigned)((input_rows + 3ull) / 4ull)), 256, 0, s>>>(a);
+        return check_launch("matvec_f32_few");
     }
     if (scalar) {
         const unsigned long long grid_x = (row_count + 3ull) / 4ull;

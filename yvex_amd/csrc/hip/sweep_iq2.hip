@@ -773,11 +773,6 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
     // item of each other instead of a long one, and only the short items pay the fixed cost of an
     // item (its activation columns, the first requests, the finishing pass) more often.
     // (a fused item keeps its row sums in LDS until its SwiGLU pass: kFusedItemRows rows)
-    const unsigned item_rows = FUSED ? kFusedItemRows : kSweepIters * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
-    const unsigned short_rows = item_rows / kSweepShortDiv;
-    const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * kSweepLongPercent / 100u / item_rows);
-    const unsigned long_rows = long_tiles * item_rows;
-    const unsigned short_tiles = (a.out_rows - long_rows + short_rows - 1u) / short_rows;
 
     // Work items: sweeps by class, the ones that serve four pairs first (the shared expert's are
     // all of that kind), then three, two, one; inside a class sweep by sweep, each over its tiles
@@ -853,6 +848,18 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
         if (tid < 4u) lds_store_u32(kClassCountBase + 4u * tid, total[tid]);
         __syncthreads();
     }
+    // A batch of a few rows has few sweeps: its items are made shorter (down to four iterations)
+    // until every wave of the grid has one, which matters more there than an item's fixed cost.
+    unsigned item_rows = FUSED ? kFusedItemRows : kSweepIters * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
+    {
+        const unsigned least = 4u * g.rows_per_iter * (MODE == 2 ? 2u : 1u);
+        const unsigned waves = gridDim.x * kSweepWaves;
+        while (item_rows / 2u >= least && all_sweeps * (a.out_rows / item_rows) < waves) item_rows /= 2u;
+    }
+    const unsigned short_rows = item_rows / kSweepShortDiv;
+    const unsigned long_tiles = (unsigned)((unsigned long long)a.out_rows * kSweepLongPercent / 100u / item_rows);
+    const unsigned long_rows = long_tiles * item_rows;
+    const unsigned short_tiles = (a.out_rows - long_rows + short_rows - 1u) / short_rows;
     const unsigned total_long = all_sweeps * long_tiles;
     const unsigned total_items = total_long + all_sweeps * short_tiles;
     // Workgroup b owns items b, b + grid, b + 2 grid, ...; its waves draw positions in that list
