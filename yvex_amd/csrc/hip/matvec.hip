@@ -1019,10 +1019,19 @@ extern "C" int yvex_hip_row_dot(const uint8_t *encoded, unsigned int qtype, cons
     return check_launch("row_dot");
 }
 
-// Splits of an F32 projection over a decode-width batch: per-wave shares of 128 columns.
-static unsigned f32_rows_splits(uint64_t row_width, uint64_t input_rows)
+// Splits of an F32 projection over a decode-width batch: per-wave shares of 128 columns. A larger
+// batch against a few weight rows (the mixing projection of a prefill batch: 24 rows) is split
+// too, as often as brings its 16 x 16 tiles to about two thousand.
+static unsigned f32_rows_splits(uint64_t row_count, uint64_t row_width, uint64_t input_rows)
 {
-    if (input_rows < 8u || input_rows >= 256u || row_width % 128u) return 0u;
+    if (input_rows < 8u || row_width % 128u) return 0u;
+    if (input_rows >= 256u) {
+        const uint64_t tiles = (row_count + 15u) / 16u * ((input_rows + 15u) / 16u);
+        if (tiles >= 1024u) return 0u;
+        for (unsigned splits = (unsigned)(2048u / tiles < 16u ? 2048u / tiles : 16u); splits >= 2u; --splits)
+            if (row_width % (64ull * splits) == 0u) return splits;
+        return 0u;
+    }
     // 512 columns a split (128 a wave) where that gives 2 to 64 splits; a wider row takes the
     // most splits up to 64 that leave every wave a multiple of 16 columns
     if (row_width % 512u == 0u && row_width / 512u >= 2u && row_width / 512u <= 64u)
@@ -1036,7 +1045,7 @@ static unsigned f32_rows_splits(uint64_t row_width, uint64_t input_rows)
 extern "C" uint64_t yvex_hip_matvec_f32_scratch_bytes(uint64_t row_count, uint64_t row_width,
                                                       uint64_t input_rows)
 {
-    const unsigned splits = f32_rows_splits(row_width, input_rows);
+    const unsigned splits = f32_rows_splits(row_count, row_width, input_rows);
     return splits ? (uint64_t)splits * input_rows * row_count * sizeof(double) : 0u;
 }
 
@@ -1045,7 +1054,7 @@ static bool f32_rows_split_applies(const float *weights, uint64_t row_count, uin
                                    const float *input, uint64_t input_rows, uint64_t input_stride,
                                    const void *scratch, uint64_t scratch_bytes)
 {
-    const unsigned splits = f32_rows_splits(row_width, input_rows);
+    const unsigned splits = f32_rows_splits(row_count, row_width, input_rows);
     const uint64_t need = yvex_hip_matvec_f32_scratch_bytes(row_count, row_width, input_rows);
     return splits && scratch && scratch_bytes >= need && !((uintptr_t)scratch & 7u) &&
            !(((uintptr_t)weights | (uintptr_t)input) & 15u) && !(input_stride & 3ull) && weights && input &&
@@ -1103,11 +1112,11 @@ extern "C" int yvex_hip_matvec_f32_rows_scored(const float *weights, uint64_t ro
 static int launch_f32_rows_split(const MatvecArgs &a, yvex_hip_stream stream)
 {
     const uint64_t row_count = a.row_count, input_rows = a.input_rows;
-    const unsigned splits = f32_rows_splits(a.row_width, input_rows);
+    const unsigned splits = f32_rows_splits(row_count, a.row_width, input_rows);
     hipStream_t s = as_stream(stream);
     const uint64_t grid_x = (row_count + 15u) / 16u, grid_y = (input_rows + 15u) / 16u;
     const uint64_t outputs = input_rows * row_count;
-    if (grid_x > 0x7fffffffull || (outputs + 255u) / 256u > 0x7fffffffull) return ST_BOUNDS;
+    if (grid_x > 0x7fffffffull || grid_y > 65535ull || (outputs + 255u) / 256u > 0x7fffffffull) return ST_BOUNDS;
     matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y, splits), 256, 0, s>>>(a);
     int rc = check_launch("matvec_f32_rows.parts");
     if (rc) return rc;
