@@ -12,7 +12,8 @@ with events on the launch stream; `cpu_baseline` is the reference's own CPU expe
 (compiled from its sources; the C restatement beside it) timed on the host cores over a bounded
 sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8 matrix
 cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `decode_envelope` the
-headline step with four residual streams around the layer, and `dense` configs
+headline step with four residual streams around the layer, `decode_small_batches` the headline
+layer at 1 to 16 rows, and `dense` configs
 0-2 and an output head as single matvec launches; the prefill legs and the dense configs carry a
 CPU baseline of their own (the same sample extrapolated per row; the reference's row dot over
 the whole matrix).
@@ -515,6 +516,27 @@ def envelope_leg(torch, routed, shared, router, dev, steps: int, warmup: int):
             "eager_ms_per_step": round(eager_ms, 4), "kernel_launches": launches}
 
 
+def small_batches_leg(torch, routed, shared, router, dev, steps: int, warmup: int):
+    """The headline layer at other decode widths (1, 4, 8 and 16 rows) through the same
+    execute_rows over the sweep image: step time and GB/s of the distinct experts' canonical bytes."""
+    from yvex_amd.host import RowBatchLayer
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(44)
+    out = {}
+    for rows in (1, 4, 8, 16):
+        x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
+        layer = RowBatchLayer(torch, routed, shared, router, x.cpu().numpy(), rows, hidden=HIDDEN,
+                              intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, sweep_image=True)
+        layer.step(defer=False)
+        unique = int(layer.result.unique_experts)
+        layer.timed(steps, warmup)
+        ms = min(layer.timed(steps, max(warmup, 2)), layer.timed(steps, warmup, eager=True))
+        layer.close()
+        out[f"rows_{rows}"] = {"us_per_step": round(ms * 1e3, 1), "distinct_routed_experts": unique,
+                               "GB_per_s": round((unique + 1) * EXPERT_BYTES / (ms * 1e-3) / 1e9, 1)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -790,6 +812,8 @@ def main() -> int:
     out["clock"] = device_clock(torch, dev)
     if not args.no_dense:
         out["decode_envelope"] = envelope_leg(torch, (gate, up, down), shared, router, dev, args.steps, args.warmup)
+        out["decode_small_batches"] = small_batches_leg(torch, (gate, up, down), shared, router, dev,
+                                                        args.steps, args.warmup)
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)
