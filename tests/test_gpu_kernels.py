@@ -87,11 +87,51 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     assert_close(got, want)
 
 
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("F16", 300, 4096, 1), ("BF16", 70, 7168, 1), ("F16", 33, 1000, 2), ("BF16", 9, 264, 5), ("F16", 5, 8, 7),
+    ("F16", 4100, 264, 1), ("BF16", 4097, 136, 3),      # many rows: a wave a row
+    ("BF16", 40, 100, 3),       # rows that are not whole 16-byte pieces: the lane-strided kernel
+    ("F16", 12, 512, 9)])       # eight input rows or more: the lane-strided kernel too
+def test_matvec_sixteen_bit_weights(gpu, oracle, qtype, rows, width, inputs):
+    """F16 and BF16 weight rows against F32 input rows (projections and output heads kept in
+    16-bit floats; src/gguf/quant_compute.c:152-172 forms double products and a double sum):
+    the CPU path's float, which is the float of the exact double-precision product up to the
+    order of the additions."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec16.{qtype}.{rows}.{width}.{inputs}")
+    values = g.normal(rows * width).reshape(rows, width).astype(np.float32)
+    if qtype == "F16":
+        encoded = values.astype(np.float16)
+        decoded = encoded.astype(np.float32)
+    else:
+        encoded = (values.view(np.uint32) >> 16).astype(np.uint16)
+        decoded = (encoded.astype(np.uint32) << 16).view(np.float32)
+    w = np.ascontiguousarray(encoded).view(np.uint8).ravel()
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    got = K.matvec(dev(w, gpu), qt, rows, width, dev(x, gpu), status=status).cpu().numpy()
+    status_ok(status)
+    assert_close(got, oracle.matvec(qt, w, rows, width, x))
+    exact = (x.astype(np.float64) @ decoded.astype(np.float64).T).astype(np.float32)
+    assert np.mean(got.view(np.uint32) != exact.view(np.uint32)) < 1e-3      # (sums that sit on a rounding boundary)
+    assert np.allclose(got, exact, rtol=1e-6, atol=1e-6)
+    # a weight that is not finite is reported
+    if rows > 1:
+        poisoned = encoded.copy()
+        poisoned.view(np.uint16).reshape(-1)[width + 3] = 0x7c00 if qtype == "F16" else 0x7f80
+        K.matvec(dev(np.ascontiguousarray(poisoned).view(np.uint8).ravel(), gpu), qt, rows, width, dev(x, gpu),
+                 status=status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 1
+
+
 @pytest.mark.parametrize("rows,width,inputs", [(256, 7168, 64), (50, 512, 45), (24, 28672, 33), (1, 32, 32),
                                                (256, 7168, 300), (40, 96, 260), (256, 7168, 8), (3, 256, 9),
                                                (45, 448, 257), (32, 64, 256),
                                                # fewer than eight input rows: a workgroup a weight row
                                                (256, 7168, 1), (24, 28672, 5), (7, 100, 3), (9, 4096, 2), (5, 30, 2),
+                                               (4100, 132, 2),
                                                # enough (32 rows x 64 input rows) blocks for the device and
                                                # 128-column chunks: the kernel with operands staged in LDS,
                                                # ragged on both sides

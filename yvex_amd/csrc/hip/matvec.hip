@@ -400,55 +400,88 @@ __global__ __launch_bounds__(256) void matvec_scalar_kernel(MatvecArgs a, unsign
     }
 }
 
-// F32 weight rows against fewer than eight F32 input rows (the router and mixing projections of a
-// batch of one to seven tokens): the lane-strided kernel above walks a row one load at a time, a
-// wave a row, and a 256 x 7168 router took 90 us of memory round trips. Here a workgroup owns
+// F32, F16 or BF16 weight rows against fewer than eight F32 input rows (the router and mixing
+// projections of a batch of one to seven tokens; a projection or an output head kept in 16-bit
+// floats): the lane-strided kernel above walks a row one load at a time, a wave a row: a
+// 256 x 7168 F32 router took 90 us of memory round trips, a 129 280 x 7168 F16 head streamed at
+// 1.1 TB/s. Here a workgroup owns
 // one weight row, its 256 threads take 16-byte pieces of it side by side (a 4 KB stretch a
 // step), DEPTH steps of weight and input loads are in flight before the first product, and the
 // four waves' double-precision sums are joined through LDS in wave order. Products and sums in
 // double as above.
-template <int T, int DEPTH>
-__global__ __launch_bounds__(256) void matvec_f32_few_kernel(MatvecArgs a)
+// WAVE_ROW: a wave a weight row (four rows a workgroup, no barrier) for matrices of many rows,
+// where the device is full either way and a workgroup a row is a launch and a barrier a row.
+template <unsigned QT, int T, int DEPTH, bool WAVE_ROW>
+__global__ __launch_bounds__(256) void matvec_scalar_few_kernel(MatvecArgs a)
 {
+    constexpr unsigned kSpan = WAVE_ROW ? 64u : 256u;       // threads that share a row
     typedef float v4f __attribute__((ext_vector_type(4)));
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    constexpr int kColumns = QT == QT_F32 ? 4 : 8;           // weights in a 16-byte piece
+    constexpr int kInputs = kColumns / 4;                    // 16-byte pieces of an input row beside it
     __shared__ double partial[3][T];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned long long row = blockIdx.x, in0 = (unsigned long long)blockIdx.y * T;
-    const v4f *w4 = reinterpret_cast<const v4f *>(a.encoded + row * a.row_bytes);
+    const unsigned long long row = WAVE_ROW ? (unsigned long long)blockIdx.x * 4ull + wave : blockIdx.x;
+    const unsigned long long in0 = (unsigned long long)blockIdx.y * T;
+    if (WAVE_ROW && row >= a.row_count) return;
+    const unsigned self = WAVE_ROW ? lane : threadIdx.x;
+    const v4u *w4 = reinterpret_cast<const v4u *>(a.encoded + row * a.row_bytes);
     const v4f *x4[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         const unsigned long long in = in0 + t < a.input_rows ? in0 + t : a.input_rows - 1ull;   // clamped rows are never written
         x4[t] = reinterpret_cast<const v4f *>((const float *)a.input + in * a.input_stride);
     }
-    const unsigned quads = (unsigned)(a.row_width >> 2);
+    const unsigned pieces = (unsigned)(a.row_width / kColumns);
     double acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.0;
     unsigned bad = 0u;
-    for (unsigned first = threadIdx.x; first < quads; first += 256u * DEPTH) {
-        v4f w[DEPTH], x[T][DEPTH];
+    for (unsigned base = 0; base < pieces; base += kSpan * DEPTH) {
+        const unsigned first = base + self;
+        // steps of this turn that hold a piece for some thread (the same for the whole
+        // workgroup: a step with none is not loaded at all, a short row costs what it holds)
+        const unsigned steps = (pieces - base + kSpan - 1u) / kSpan;
+        v4u raw[DEPTH];
+        v4f x[T][DEPTH][kInputs];
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
-            const unsigned at = first + 256u * u < quads ? first + 256u * u : first;
-            w[u] = w4[at];
+            if ((unsigned)u < steps) {
+                const unsigned at = first + kSpan * u < pieces ? first + kSpan * u : pieces - 1u;
+                raw[u] = w4[at];
 #pragma unroll
-            for (int t = 0; t < T; ++t) x[t][u] = x4[t][at];
+                for (int t = 0; t < T; ++t)
+#pragma unroll
+                    for (int j = 0; j < kInputs; ++j) x[t][u][j] = x4[t][at * kInputs + j];
+            } else {
+                raw[u] = v4u{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int t = 0; t < T; ++t)
+#pragma unroll
+                    for (int j = 0; j < kInputs; ++j) x[t][u][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            }
         }
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
-            // (a step past the end repeated the first one: its inputs count as zeros. A branch
-            // here would pull each step's loads behind it, one wait a step)
-            const bool live = first + 256u * u < quads;
-            bad |= (unsigned)!finite_f32(w[u][0]) | (unsigned)!finite_f32(w[u][1]) | (unsigned)!finite_f32(w[u][2]) |
-                   (unsigned)!finite_f32(w[u][3]);
+            // (a thread past the end of the row repeated the last piece: its inputs count as
+            // zeros. A branch here would pull each step's loads behind it, one wait a step)
+            const bool live = first + kSpan * u < pieces;
+            float w[kColumns];
+#pragma unroll
+            for (int c = 0; c < kColumns; ++c) {
+                if constexpr (QT == QT_F32) {
+                    w[c] = __uint_as_float(raw[u][c]);
+                } else {
+                    const unsigned bits = (raw[u][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+                    w[c] = QT == QT_BF16 ? __uint_as_float(bits << 16) : f16_bits_to_float(bits);
+                }
+                bad |= (unsigned)!finite_f32(w[c]);
+            }
 #pragma unroll
             for (int t = 0; t < T; ++t)
-                if (!live) x[t][u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int t = 0; t < T; ++t)
-#pragma unroll
-                for (int c = 0; c < 4; ++c) acc[t] += (double)w[u][c] * (double)x[t][u][c];
+                for (int c = 0; c < kColumns; ++c)
+                    acc[t] += (double)w[c] * (double)(live ? x[t][u][c >> 2][c & 3] : 0.0f);
         }
     }
     if (bad) raise_status(a.status, 1);
@@ -456,7 +489,14 @@ __global__ __launch_bounds__(256) void matvec_f32_few_kernel(MatvecArgs a)
     for (int t = 0; t < T; ++t) {
 #pragma unroll
         for (int offset = 32; offset > 0; offset >>= 1) acc[t] += __shfl_xor(acc[t], offset, kWave);
-        if (wave && lane == 0u) partial[wave - 1u][t] = acc[t];
+        if (!WAVE_ROW && wave && lane == 0u) partial[wave - 1u][t] = acc[t];
+    }
+    if constexpr (WAVE_ROW) {
+        if (lane != 0u) return;
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+            if (in0 + t < a.input_rows) matvec_publish(a, in0 + t, row, (float)acc[t]);
+        return;
     }
     __syncthreads();
     if (threadIdx.x != 0u) return;
@@ -466,6 +506,27 @@ __global__ __launch_bounds__(256) void matvec_f32_few_kernel(MatvecArgs a)
         const double sum = acc[t] + partial[0][t] + partial[1][t] + partial[2][t];
         matvec_publish(a, in0 + t, row, (float)sum);
     }
+}
+
+template <unsigned QT, bool WAVE_ROW>
+static int launch_scalar_few_rows(const MatvecArgs &a, hipStream_t s)
+{
+    const unsigned long long grid_x = WAVE_ROW ? (a.row_count + 3ull) / 4ull : a.row_count;
+    if (a.input_rows == 1ull)
+        matvec_scalar_few_kernel<QT, 1, 8, WAVE_ROW><<<dim3((unsigned)grid_x, 1), 256, 0, s>>>(a);
+    else if (a.input_rows == 2ull)
+        matvec_scalar_few_kernel<QT, 2, 8, WAVE_ROW><<<dim3((unsigned)grid_x, 1), 256, 0, s>>>(a);
+    else
+        matvec_scalar_few_kernel<QT, 4, 4, WAVE_ROW><<<dim3((unsigned)grid_x, (unsigned)((a.input_rows + 3ull) / 4ull)),
+                                                       256, 0, s>>>(a);
+    return check_launch("matvec_scalar_few");
+}
+
+template <unsigned QT>
+static int launch_scalar_few(const MatvecArgs &a, hipStream_t s)
+{
+    // (sixteen waves a compute unit either way from 4096 rows on)
+    return a.row_count >= 4096ull ? launch_scalar_few_rows<QT, true>(a, s) : launch_scalar_few_rows<QT, false>(a, s);
 }
 
 // F32 weight rows against a batch of F32 input rows (a router or mixing projection over a row
@@ -922,15 +983,11 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         }
         return check_launch("matvec_f32_tile16");
     }
-    if (qtype == QT_F32 && input_rows < 8ull && row_width % 4ull == 0ull && row_count <= 0x7fffffffull &&
-        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) && !(row_bytes & 15ull)) {
-        if (input_rows == 1ull)
-            matvec_f32_few_kernel<1, 8><<<dim3((unsigned)row_count, 1), 256, 0, s>>>(a);
-        else if (input_rows == 2ull)
-            matvec_f32_few_kernel<2, 8><<<dim3((unsigned)row_count, 1), 256, 0, s>>>(a);
-        else
-            matvec_f32_few_kernel<4, 4><<<dim3((unsigned)row_count, (unsigned)((input_rows + 3ull) / 4ull)), 256, 0, s>>>(a);
-        return check_launch("matvec_f32_few");
+    if ((qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16) && input_rows < 8ull &&
+        row_count <= 0x7fffffffull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
+        !(row_bytes & 15ull)) {      // (whole 16-byte pieces a row: a multiple of 4 or 8 columns)
+        if (qtype == QT_F32) return launch_scalar_few<QT_F32>(a, s);
+        return qtype == QT_F16 ? launch_scalar_few<QT_F16>(a, s) : launch_scalar_few<QT_BF16>(a, s);
     }
     if (scalar) {
         const unsigned long long grid_x = (row_count + 3ull) / 4ull;
