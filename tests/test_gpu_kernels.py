@@ -91,7 +91,7 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     ("F16", 300, 4096, 1), ("BF16", 70, 7168, 1), ("F16", 33, 1000, 2), ("BF16", 9, 264, 5), ("F16", 5, 8, 7),
     ("F16", 4100, 264, 1), ("BF16", 4097, 136, 3),      # many rows: a wave a row
     ("BF16", 40, 100, 3),       # rows that are not whole 16-byte pieces: the lane-strided kernel
-    ("F16", 12, 512, 9)])       # eight input rows or more: the lane-strided kernel too
+    ("F16", 12, 512, 9), ("BF16", 40, 1024, 70)])       # eight input rows and more
 def test_matvec_sixteen_bit_weights(gpu, oracle, qtype, rows, width, inputs):
     """F16 and BF16 weight rows against F32 input rows (projections and output heads kept in
     16-bit floats; src/gguf/quant_compute.c:152-172 forms double products and a double sum):

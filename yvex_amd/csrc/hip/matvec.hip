@@ -983,7 +983,10 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         }
         return check_launch("matvec_f32_tile16");
     }
-    if ((qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16) && input_rows < 8ull &&
+    // (F32 rows go to the matrix cores from eight input rows on; 16-bit rows have no other fast
+    // kernel and stay here, four input rows a workgroup)
+    if (((qtype == QT_F32 && input_rows < 8ull) ||
+         ((qtype == QT_F16 || qtype == QT_BF16) && (input_rows + 3ull) / 4ull <= 65535ull)) &&
         row_count <= 0x7fffffffull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
         !(row_bytes & 15ull)) {      // (whole 16-byte pieces a row: a multiple of 4 or 8 columns)
         if (qtype == QT_F32) return launch_scalar_few<QT_F32>(a, s);
