@@ -306,6 +306,8 @@ def dense_leg(torch, K, dev, repeats: int):
 
     run("cfg0_q8_0_4096x4096_f32_b1", K.Q8_0, 4096, 4096, 1, False)
     run("cfg0_q8_0_4096x4096_q8k_b1", K.Q8_0, 4096, 4096, 1, True)
+    run("cfg0_q8_0_4096x4096_q8k_b16", K.Q8_0, 4096, 4096, 16, True)
+    run("cfg0_q8_0_4096x4096_q8k_b2048", K.Q8_0, 4096, 4096, 2048, True)
     run("cfg1_q4_k_2048x7168_q8k_b1", K.Q4_K, 2048, 7168, 1, True)
     run("cfg1_q4_k_2048x7168_q8k_b16", K.Q4_K, 2048, 7168, 16, True)
     run("cfg1_q4_k_2048x7168_q8k_b256", K.Q4_K, 2048, 7168, 256, True)

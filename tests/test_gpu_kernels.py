@@ -278,6 +278,41 @@ def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, wid
         assert np.array_equal(few.view(np.uint32), got[:count].view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,width,inputs", [(516, 4096, 16), (40, 256, 33), (4096, 4096, 70), (33, 2304, 64),
+                                               (7, 512, 200)])
+def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, inputs):
+    """Q8_0 rows against 16 or more Q8_K input rows (the reference's tensor-core threshold,
+    src/backend/cuda/private.h:461-464): the oracle's Q8_K product within the tolerance of the
+    Q8_0 dense rows (a float term per block, float row sums), ragged on both sides, with the
+    additive operand and the bf16 rounding, and the smaller batches' lane-strided kernel beside it."""
+    from yvex_amd import kernels as K
+    qt = oracle.Q8_0
+    g = oracle.Generator(42, f"matvec.q8_0.rows.{rows}.{width}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    add = g.normal(inputs * rows).reshape(inputs, rows)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    want = oracle.q8_matvec(qt, w, rows, width, act_host, inputs)
+    assert_q8_product(got, want, "Q8_0")
+    deq = oracle.q8k_dequantize(act_host).reshape(inputs, width)
+    assert_close(got, oracle.matvec(qt, w, rows, width, deq, threads=8))
+    summed = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                      additive=dev(add, gpu), output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((summed.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(summed - (got + add)) <= np.abs(got + add) * 2.0 ** -8 + 1e-30)
+    few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=15,
+                   status=status).cpu().numpy()          # below the threshold: the lane-strided kernel
+    status_ok(status)
+    assert_q8_product(few, want[:15], "Q8_0")
+    assert np.allclose(few, got[:15], rtol=2e-5, atol=1e-6)
+
+
 def test_matvec_q4k_large_batch_stages_operands_in_lds(gpu, oracle):
     """A Q4_K projection with at least one (128 rows x 64 tokens) tile per compute unit takes the
     kernel whose operands are staged through LDS: ragged row count (the last tile repeats a row),

@@ -1,0 +1,226 @@
+// Q8_0 weight rows against a batch of Q8_K input rows on the int8 matrix cores: the dense
+// projection at prefill width (the reference turns its tensor-core kernels on from 16 input rows
+// for every format that takes Q8 activations, src/backend/cuda/private.h:461-464,
+// src/backend/cuda/qtype.c:252-255).
+//
+// Arithmetic per 32-value block, as the lane-strided kernel and the reference's primitive form it
+// (src/backend/cuda/kernel_primitives.h:353-357):
+//     dot   = sum_i q_i * a_i                       (int32, exact: one K step of V_MFMA_I32_32X32X32_I8)
+//     value = (d_block * d_a) * float(dot)          (two float products)
+// and the values of a row are added in float. Here the eight blocks under one input scale are
+// added as d_block * float(dot) and the sum is multiplied by d_a once: float sums in another
+// order, inside the 1e-5 the format's dense rows are held to. A block has a scale of its own, so
+// every matrix instruction starts from zero and its sixteen results a lane are converted, scaled
+// and added on the vector ALU.
+//
+// A workgroup owns 32 weight rows x 32 or 64 input rows; its four waves take every fourth
+// superblock (eight blocks, 272 bytes a row) and their partial tiles are added in wave order, so
+// results do not depend on timing. Lane (r, h) holds bytes 16 h .. 16 h + 15 of weight row r's
+// block as the A operand and the same bytes of input row r's block as the B operand; accumulator
+// i of that lane is weight row 8 (i / 4) + 4 h + i % 4 against input row r. Blocks start on 2-byte
+// boundaries (34 bytes each): the codes of an even block are read as five aligned dwords and
+// shifted into place, those of an odd block are dword-aligned as they lie.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace yvex {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct DenseQ80Args {
+    const unsigned char *encoded;
+    unsigned long long row_count, row_bytes;
+    unsigned blocks;                         // superblocks (256 columns) per row
+    const unsigned char *act;                // Q8_K rows, blocks * 292 bytes each
+    unsigned long long input_rows;
+    const float *additive;
+    float *out;
+    unsigned long long out_stride;
+    int output_bf16;
+    int *status;
+};
+
+// What a lane needs of one superblock: its half of the eight blocks' codes, their scales, and
+// its half of NT input rows' blocks.
+template <unsigned NT>
+struct Q80Inputs {
+    uint4 codes[8];         // even blocks: the aligned window two bytes in front of the codes
+    unsigned tail[4];       // even blocks: the dword behind the window
+    uint4 a[NT][8];
+    float act_scale[NT];
+};
+
+template <unsigned NT>
+__device__ __forceinline__ void q80_load(const unsigned char *wrow, const unsigned char *const (&arow)[NT],
+                                         unsigned sb, unsigned h, Q80Inputs<NT> &in)
+{
+    const unsigned char *w = wrow + (unsigned long long)sb * 272ull;     // dword-aligned
+#pragma unroll
+    for (unsigned c = 0; c < 8u; ++c) {
+        // block c starts at 34 c: two bytes past a dword boundary when c is odd
+        const unsigned codes = 34u * c + 2u + 16u * h;
+        if (c % 2u == 0u) {
+            const unsigned *p = reinterpret_cast<const unsigned *>(w + codes - 2u);
+            in.codes[c] = make_uint4(p[0], p[1], p[2], p[3]);
+            in.tail[c / 2u] = p[4];
+        } else {
+            const unsigned *p = reinterpret_cast<const unsigned *>(w + codes);
+            in.codes[c] = make_uint4(p[0], p[1], p[2], p[3]);
+        }
+    }
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt) {
+        const unsigned char *a = arow[nt] + (unsigned long long)sb * kQ8KBytes;
+        in.act_scale[nt] = *reinterpret_cast<const float *>(a);
+#pragma unroll
+        for (unsigned c = 0; c < 8u; ++c) {
+            const unsigned *p = reinterpret_cast<const unsigned *>(a + 4u + 32u * c + 16u * h);
+            in.a[nt][c] = make_uint4(p[0], p[1], p[2], p[3]);
+        }
+    }
+}
+
+template <unsigned NT>
+__global__ __launch_bounds__(256) void dense_q8_0_kernel(DenseQ80Args g)
+{
+    // per wave: the scales of its 32 rows' eight blocks of the superblock in hand; then the partial tiles
+    __shared__ __align__(16) float block_scale[4][8][32];
+    __shared__ float partial[3][NT][16][64];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned r = lane & 31u, h = lane >> 5;
+    const unsigned long long row0 = (unsigned long long)blockIdx.x * 32ull;
+    const unsigned long long tok0 = (unsigned long long)blockIdx.y * (32ull * NT);
+    unsigned long long wr = row0 + r;
+    if (wr >= g.row_count) wr = g.row_count - 1ull;              // a ragged edge repeats the last row
+    const unsigned char *wrow = g.encoded + wr * g.row_bytes;
+    const unsigned char *arow[NT];
+    const unsigned long long act_row_bytes = (unsigned long long)g.blocks * kQ8KBytes;
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt) {
+        unsigned long long t = tok0 + 32ull * nt + r;
+        if (t >= g.input_rows) t = g.input_rows - 1ull;
+        arow[nt] = g.act + t * act_row_bytes;
+    }
+    float acc[NT][16];
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+
+    Q80Inputs<NT> cur;
+    q80_load<NT>(wrow, arow, wave < g.blocks ? wave : 0u, h, cur);
+    for (unsigned sb = wave; sb < g.blocks; sb += 4u) {
+        // the next superblock's bytes travel while this one is worked on
+        Q80Inputs<NT> nxt;
+        q80_load<NT>(wrow, arow, sb + 4u < g.blocks ? sb + 4u : sb, h, nxt);
+
+        // The scales lie in the windows already: an even block's in front of its codes (the low
+        // half of the first dword of the lane with h = 0), an odd block's behind the codes of the
+        // block before it (the high half of the tail dword of the lane with h = 1).
+#pragma unroll
+        for (unsigned j = 0; j < 4u; ++j)
+            block_scale[wave][2u * j + h][r] =
+                f16_bits_to_float(h ? cur.tail[j] >> 16 : cur.codes[2u * j].x & 0xffffu);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float within[NT][16];       // the superblock's sum before the input row's scale
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) within[nt][i] = 0.0f;
+#pragma unroll
+        for (unsigned c = 0; c < 8u; ++c) {
+            v4i a;
+            if (c % 2u == 0u) {
+                const uint4 q = cur.codes[c];
+                a[0] = (int)__builtin_amdgcn_alignbyte(q.y, q.x, 2u);
+                a[1] = (int)__builtin_amdgcn_alignbyte(q.z, q.y, 2u);
+                a[2] = (int)__builtin_amdgcn_alignbyte(q.w, q.z, 2u);
+                a[3] = (int)__builtin_amdgcn_alignbyte(cur.tail[c / 2u], q.w, 2u);
+            } else {
+                a[0] = (int)cur.codes[c].x; a[1] = (int)cur.codes[c].y;
+                a[2] = (int)cur.codes[c].z; a[3] = (int)cur.codes[c].w;
+            }
+            // the scales of the sixteen rows this lane accumulates
+            float d_of[16];
+#pragma unroll
+            for (unsigned q4 = 0; q4 < 4u; ++q4) {
+                const float4 d = *reinterpret_cast<const float4 *>(&block_scale[wave][c][8u * q4 + 4u * h]);
+                d_of[4u * q4] = d.x; d_of[4u * q4 + 1u] = d.y; d_of[4u * q4 + 2u] = d.z; d_of[4u * q4 + 3u] = d.w;
+            }
+#pragma unroll
+            for (unsigned nt = 0; nt < NT; ++nt) {
+                v16i zero;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) zero[i] = 0;
+                const v4i b = {(int)cur.a[nt][c].x, (int)cur.a[nt][c].y, (int)cur.a[nt][c].z, (int)cur.a[nt][c].w};
+                const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) within[nt][i] += d_of[i] * (float)dot[i];
+            }
+        }
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nt][i] += cur.act_scale[nt] * within[nt][i];
+        // (the next superblock's scales are not written before every lane has read these)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        cur = nxt;
+    }
+
+    if (wave) {
+#pragma unroll
+        for (unsigned nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) partial[wave - 1u][nt][i][lane] = acc[nt][i];
+    }
+    __syncthreads();
+    if (wave) return;
+#pragma unroll
+    for (unsigned nt = 0; nt < NT; ++nt) {
+        const unsigned long long token = tok0 + 32ull * nt + r;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const unsigned long long row = row0 + 8u * (i >> 2) + 4u * h + (i & 3);
+            const float sum = ((acc[nt][i] + partial[0][nt][i][lane]) + partial[1][nt][i][lane]) +
+                              partial[2][nt][i][lane];
+            if (row >= g.row_count || token >= g.input_rows) continue;
+            const unsigned long long at = token * g.out_stride + row;
+            const float value = g.additive ? sum + g.additive[at] : sum;
+            if (!finite_f32(value)) raise_status(g.status, 1);
+            else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
+        }
+    }
+}
+
+}  // namespace
+
+int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
+                           const float *additive, float *out, uint64_t out_stride, bool output_bf16,
+                           int *status, hipStream_t stream)
+{
+    if (!row_count || !input_rows || row_width % 256u || row_width / 32u * 34u != row_bytes)
+        return ST_BOUNDS;
+    if (((uintptr_t)encoded & 3u) || ((uintptr_t)act_q8k & 3u)) return ST_INVALID_ARG;
+    const uint64_t row_tiles = (row_count + 31u) / 32u;
+    if (row_tiles > 0x7fffffffull || row_width / 256u > 0xffffffffull) return ST_BOUNDS;
+    DenseQ80Args g{encoded, row_count, row_bytes, (unsigned)(row_width / 256u),
+                   (const unsigned char *)act_q8k, input_rows, additive, out, out_stride,
+                   output_bf16 ? 1 : 0, status};
+    if (input_rows <= 32u) {
+        dense_q8_0_kernel<1><<<dim3((unsigned)row_tiles, 1), 256, 0, stream>>>(g);
+    } else {
+        const uint64_t token_tiles = (input_rows + 63u) / 64u;
+        if (token_tiles > 65535ull) return ST_BOUNDS;
+        dense_q8_0_kernel<2><<<dim3((unsigned)row_tiles, (unsigned)token_tiles), 256, 0, stream>>>(g);
+    }
+    return check_launch("dense_q8_0");
+}
+
+}  // namespace yvex

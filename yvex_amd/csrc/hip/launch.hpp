@@ -47,6 +47,12 @@ int launch_iq2_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t r
                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows, float *out,
                           bool round_bf16, int *status, hipStream_t stream);
 
+// Q8_0 rows x Q8_K input rows on the int8 matrix cores (dense_q8_0.hip).
+int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,
+                           const float *additive, float *out, uint64_t out_stride, bool output_bf16,
+                           int *status, hipStream_t stream);
+
 // Q4_K rows x Q8_K input rows on the int8 matrix cores (dense_q4k.hip).
 int launch_q4k_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
                           uint64_t row_bytes, const void *act_q8k, uint64_t input_rows,

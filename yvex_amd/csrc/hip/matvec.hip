@@ -958,6 +958,11 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         !(input_rows < 4ull && dense_fewrows_applies<QT_Q4_K>(a)))
         return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
                                      out, out_stride, output_bf16 != 0, status, s);
+    // Q8_0 rows against a batch of Q8_K input rows: matrix cores from the reference's threshold on
+    // (src/backend/cuda/private.h:461-464); below it the lane-strided kernel
+    if (qtype == QT_Q8_0 && input_q8 && input_rows >= 16ull && !((uintptr_t)encoded & 3u))
+        return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive, out,
+                                      out_stride, output_bf16 != 0, status, s);
     // F32 rows against a batch of F32 input rows: 16 x 16 tiles on the double-precision matrix
     // cores; a small batch offers few tiles, so sixteen waves split the row width, a large one
     // has tiles enough for four
