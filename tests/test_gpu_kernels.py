@@ -313,6 +313,44 @@ def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, in
     assert np.allclose(few, got[:15], rtol=2e-5, atol=1e-6)
 
 
+def test_matvec_q8_0_large_batch_stages_operands_in_lds(gpu, oracle):
+    """A Q8_0 projection with at least one (128 rows x 64 input rows) tile per compute unit takes
+    the kernel whose operands pass through LDS: ragged row count (the last tile repeats a row), a
+    last tile of six input rows, several superblocks a row (both LDS buffers), additive rows and
+    bf16 outputs; the oracle's product within the format's tolerance, and the unstaged kernels
+    beside it."""
+    from yvex_amd import kernels as K
+    qt, rows, width, inputs = oracle.Q8_0, 2001, 1280, 1030
+    assert (rows + 127) // 128 * ((inputs + 63) // 64) >= 256
+    g = oracle.Generator(42, "matvec.rows.staged.q8_0")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    bias = g.normal(inputs * rows).reshape(inputs, rows)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                   status=status).cpu().numpy()
+    status_ok(status)
+    act_host = oracle.q8k_quantize(x)
+    want = oracle.q8_matvec(qt, w, rows, width, act_host, inputs)
+    assert_q8_product(got, want, "Q8_0")
+    summed = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                      additive=dev(bias, gpu), status=status).cpu().numpy()
+    status_ok(status)
+    assert np.array_equal(summed, got + bias)
+    rounded = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs,
+                       output_bf16=True, status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((rounded.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(rounded - got) <= np.abs(got) * 2.0 ** -8 + 1e-30)
+    for count in (70, 16, 3):       # the unstaged tiles (float sums in another order), the lane-strided kernel
+        few = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=count,
+                       status=status).cpu().numpy()
+        status_ok(status)
+        assert_q8_product(few, want[:count], "Q8_0")
+        assert np.allclose(few, got[:count], rtol=2e-5, atol=2e-6)
+
+
 def test_matvec_q4k_large_batch_stages_operands_in_lds(gpu, oracle):
     """A Q4_K projection with at least one (128 rows x 64 tokens) tile per compute unit takes the
     kernel whose operands are staged through LDS: ragged row count (the last tile repeats a row),

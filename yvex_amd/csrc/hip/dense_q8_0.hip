@@ -22,13 +22,11 @@
 // shifted into place, those of an odd block are dword-aligned as they lie.
 #include "common.hpp"
 #include "launch.hpp"
+#include "lds_copy.hpp"
 
 namespace yvex {
 
 namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct DenseQ80Args {
     const unsigned char *encoded;
@@ -198,6 +196,159 @@ __global__ __launch_bounds__(256) void dense_q8_0_kernel(DenseQ80Args g)
     }
 }
 
+// The same product for batches that offer every compute unit a tile of 128 weight rows x 64
+// input rows: the operands of one superblock pass through LDS. GLOBAL_LOAD_LDS instructions whose
+// lanes walk consecutive 16-byte pieces of consecutive rows (a dozen cache lines an instruction
+// where the kernel above touches up to 64) fill the other of two buffers while this one is
+// multiplied; one barrier per superblock. A weight row keeps its 272 bytes and an input row's 256
+// codes get the same pitch, its scale (the row's first 16 bytes) as a seventeenth piece behind
+// them, so the 16-byte operand reads of 16 lanes fall on 16 different bank groups. The window of
+// a block's codes is not 16-byte aligned in its row: a lane reads the two aligned pieces around
+// it and picks its dwords (the offsets are compile-time constants).
+//
+// Eight waves, two per SIMD, each 32 weight rows x 32 input rows over the whole row width: no
+// partial tiles. Here the input rows are the A operand and the weight rows the B operand, so lane
+// (r, h) holds weight row r against input rows 8 (i / 4) + 4 h + i % 4: the block's scale is one
+// value a lane (read from the row's bytes in LDS) and the input rows' scales, needed once a
+// superblock, are sixteen broadcast reads.
+constexpr unsigned kStagedThreads = 512u, kStagedRows = 128u, kStagedTokens = 64u, kStagedPitch = 272u;
+constexpr unsigned kStagedWeightBytes = kStagedRows * kStagedPitch;                 // one buffer
+constexpr unsigned kStagedActBytes = kStagedTokens * kStagedPitch;
+constexpr unsigned kStagedWeightBase = 0u;                                          // [buffer]
+constexpr unsigned kStagedActBase = kStagedWeightBase + 2u * kStagedWeightBytes;    // [buffer]
+constexpr unsigned kStagedLdsBytes = kStagedActBase + 2u * kStagedActBytes;
+
+__device__ __forceinline__ uint4 read16(unsigned address)
+{
+    const v4i v = lds_read_v4i(address);
+    return make_uint4((unsigned)v[0], (unsigned)v[1], (unsigned)v[2], (unsigned)v[3]);
+}
+
+__global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(DenseQ80Args g)
+{
+    extern __shared__ __align__(16) unsigned char dense_q8_0_lds[];
+    if (lds_address_of(dense_q8_0_lds) != 0u) {   // operands are addressed by absolute LDS offsets
+        if (threadIdx.x == 0u) raise_status(g.status, 2);
+        return;
+    }
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const unsigned r = lane & 31u, h = lane >> 5;
+    const unsigned row_block = wave & 3u, token_block = wave >> 2;
+    const unsigned long long row0 = (unsigned long long)blockIdx.x * kStagedRows;
+    const unsigned long long tok0 = (unsigned long long)blockIdx.y * kStagedTokens;
+    const unsigned rows_here = (unsigned)(g.row_count - row0 < kStagedRows ? g.row_count - row0 : kStagedRows);
+    const unsigned toks_here = (unsigned)(g.input_rows - tok0 < kStagedTokens ? g.input_rows - tok0 : kStagedTokens);
+    const unsigned long long act_row_bytes = (unsigned long long)g.blocks * kQ8KBytes;
+
+    // ---- copy sources (a ragged edge repeats the tile's last row) ----
+    // weights: piece q = tid + 512 k of the tile's 128 x 17; input rows: piece q of 64 x 17, the
+    // seventeenth being the 16 bytes at the row's start
+    const unsigned char *weight_from[5], *act_from[3];
+#pragma unroll
+    for (unsigned k = 0; k < 5u; ++k) {
+        unsigned q = tid + 512u * k;
+        if (q >= kStagedRows * 17u) q = kStagedRows * 17u - 1u;            // (waves that do not copy this round)
+        const unsigned row = q / 17u, piece = q - row * 17u;
+        weight_from[k] = g.encoded + (row0 + (row < rows_here ? row : rows_here - 1u)) * g.row_bytes + 16u * piece;
+    }
+#pragma unroll
+    for (unsigned k = 0; k < 3u; ++k) {
+        unsigned q = tid + 512u * k;
+        if (q >= kStagedTokens * 17u) q = kStagedTokens * 17u - 1u;
+        const unsigned token = q / 17u, piece = q - token * 17u;
+        act_from[k] = g.act + (tok0 + (token < toks_here ? token : toks_here - 1u)) * act_row_bytes +
+                      (piece < 16u ? 4u + 16u * piece : 0u);
+    }
+    const unsigned last_block = g.blocks - 1u;
+    auto copies = [&](unsigned sb) {
+        const unsigned buffer = sb & 1u;
+        const unsigned clamped = sb < last_block ? sb : last_block;
+        const unsigned long long w_at = (unsigned long long)clamped * 272ull;
+        const unsigned long long a_at = (unsigned long long)clamped * kQ8KBytes;
+        const unsigned w_to = kStagedWeightBase + buffer * kStagedWeightBytes + 1024u * wave;
+        const unsigned a_to = kStagedActBase + buffer * kStagedActBytes + 1024u * wave;
+#pragma unroll
+        for (unsigned k = 0; k < 4u; ++k)
+            copy_to_lds_16(weight_from[k] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 8192u * k)));
+        if (wave < 2u)
+            copy_to_lds_16(weight_from[4] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 32768u)));
+#pragma unroll
+        for (unsigned k = 0; k < 2u; ++k)
+            copy_to_lds_16(act_from[k] + a_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 8192u * k)));
+        if (wave == 0u)
+            copy_to_lds_16(act_from[2] + a_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16384u)));
+    };
+
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+    copies(0u);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (unsigned sb = 0; sb < g.blocks; ++sb) {
+        const unsigned buffer = sb & 1u;
+        if (sb + 1u < g.blocks) copies(sb + 1u);
+        const unsigned w_row = kStagedWeightBase + buffer * kStagedWeightBytes + (32u * row_block + r) * kStagedPitch;
+        const unsigned a_tile = kStagedActBase + buffer * kStagedActBytes + 32u * token_block * kStagedPitch;
+
+        float within[16];           // the superblock's sum before the input rows' scales
+#pragma unroll
+        for (int i = 0; i < 16; ++i) within[i] = 0.0f;
+#pragma unroll
+        for (unsigned c = 0; c < 8u; ++c) {
+            const unsigned start = c % 2u == 0u ? 34u * c : 34u * c + 2u;      // the lane's window: + 16 h
+            const unsigned at = (start & 15u) / 4u;
+            const uint4 lo = read16(w_row + 16u * h + (start & ~15u));
+            // (an even block's window is 20 bytes, an odd block's 16: only block 7's fits one piece)
+            const uint4 hi = c % 2u == 0u || (start & 15u) ? read16(w_row + 16u * h + (start & ~15u) + 16u) : lo;
+            const float d_w = f16_bits_to_float(lds_read_u16(w_row + 34u * c));
+            const v4i tokens = lds_read_v4i(a_tile + r * kStagedPitch + 16u * (2u * c + h));
+            const unsigned q[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            v4i codes;
+            if (c % 2u == 0u) {
+#pragma unroll
+                for (unsigned j = 0; j < 4u; ++j)
+                    codes[j] = (int)__builtin_amdgcn_alignbyte(q[at + j + 1u], q[at + j], 2u);
+            } else {
+#pragma unroll
+                for (unsigned j = 0; j < 4u; ++j) codes[j] = (int)q[at + j];
+            }
+            v16i zero;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) zero[i] = 0;
+            const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(tokens, codes, zero, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w, (float)dot[i], within[i]);
+        }
+#pragma unroll
+        for (unsigned i = 0; i < 16u; ++i) {
+            const unsigned token = 8u * (i >> 2) + 4u * h + (i & 3u);
+            const float d_a = __uint_as_float(lds_read_u32(a_tile + token * kStagedPitch + 256u));
+            acc[i] = __builtin_fmaf(d_a, within[i], acc[i]);
+        }
+        // the next superblock's copies have landed and every wave is done with this one's buffers
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // lane (r, h): weight row r of the wave's 32 against sixteen input rows; a store instruction
+    // writes 32 consecutive floats of two output rows
+    const unsigned long long row = row0 + 32u * row_block + r;
+    if (row >= g.row_count) return;
+    bool bad = false;
+#pragma unroll
+    for (unsigned i = 0; i < 16u; ++i) {
+        const unsigned long long token = tok0 + 32u * token_block + 8u * (i >> 2) + 4u * h + (i & 3u);
+        if (token >= g.input_rows) continue;
+        const unsigned long long at = token * g.out_stride + row;
+        const float value = g.additive ? acc[i] + g.additive[at] : acc[i];
+        if (!finite_f32(value)) bad = true;
+        else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
+    }
+    if (bad) raise_status(g.status, 1);
+}
+
 }  // namespace
 
 int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
@@ -213,6 +364,15 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
     DenseQ80Args g{encoded, row_count, row_bytes, (unsigned)(row_width / 256u),
                    (const unsigned char *)act_q8k, input_rows, additive, out, out_stride,
                    output_bf16 ? 1 : 0, status};
+    const uint64_t staged_row_tiles = (row_count + kStagedRows - 1u) / kStagedRows;
+    const uint64_t staged_token_tiles = (input_rows + kStagedTokens - 1u) / kStagedTokens;
+    if (!((uintptr_t)encoded & 15u) && staged_row_tiles * staged_token_tiles >= (uint64_t)compute_units() &&
+        staged_token_tiles <= 65535ull) {
+        YVEX_ALLOW_DYNAMIC_LDS(dense_q8_0_staged_kernel, kStagedLdsBytes);
+        dense_q8_0_staged_kernel<<<dim3((unsigned)staged_row_tiles, (unsigned)staged_token_tiles), kStagedThreads,
+                                   kStagedLdsBytes, stream>>>(g);
+        return check_launch("dense_q8_0_staged");
+    }
     if (input_rows <= 32u) {
         dense_q8_0_kernel<1><<<dim3((unsigned)row_tiles, 1), 256, 0, stream>>>(g);
     } else {
