@@ -295,31 +295,53 @@ __global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(Dense
         float within[16];           // the superblock's sum before the input rows' scales
 #pragma unroll
         for (int i = 0; i < 16; ++i) within[i] = 0.0f;
+        // Three stages in flight, or a wave would run its LDS reads, its matrix instruction and the
+        // scaling of the results one after the other: in step k the operands of block k are
+        // read, block k - 1 is multiplied and the results of block k - 2 are scaled (vector
+        // instructions that issue while the matrix pipe works).
+        uint4 lo[2], hi[2];
+        v4i tokens[2];
+        unsigned scale_bits[2];
+        v16i dot[2];
+        float d_w[2];
 #pragma unroll
-        for (unsigned c = 0; c < 8u; ++c) {
-            const unsigned start = c % 2u == 0u ? 34u * c : 34u * c + 2u;      // the lane's window: + 16 h
-            const unsigned at = (start & 15u) / 4u;
-            const uint4 lo = read16(w_row + 16u * h + (start & ~15u));
-            // (an even block's window is 20 bytes, an odd block's 16: only block 7's fits one piece)
-            const uint4 hi = c % 2u == 0u || (start & 15u) ? read16(w_row + 16u * h + (start & ~15u) + 16u) : lo;
-            const float d_w = f16_bits_to_float(lds_read_u16(w_row + 34u * c));
-            const v4i tokens = lds_read_v4i(a_tile + r * kStagedPitch + 16u * (2u * c + h));
-            const unsigned q[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            v4i codes;
-            if (c % 2u == 0u) {
-#pragma unroll
-                for (unsigned j = 0; j < 4u; ++j)
-                    codes[j] = (int)__builtin_amdgcn_alignbyte(q[at + j + 1u], q[at + j], 2u);
-            } else {
-#pragma unroll
-                for (unsigned j = 0; j < 4u; ++j) codes[j] = (int)q[at + j];
+        for (unsigned k = 0; k < 10u; ++k) {
+            if (k < 8u) {
+                const unsigned c = k, slot = c % 2u;
+                const unsigned start = c % 2u == 0u ? 34u * c : 34u * c + 2u;      // the lane's window: + 16 h
+                lo[slot] = read16(w_row + 16u * h + (start & ~15u));
+                // (an even block's window is 20 bytes, an odd block's 16: only block 7's fits one piece)
+                hi[slot] = c % 2u == 0u || (start & 15u) ? read16(w_row + 16u * h + (start & ~15u) + 16u) : lo[slot];
+                scale_bits[slot] = lds_read_u16(w_row + 34u * c);
+                tokens[slot] = lds_read_v4i(a_tile + r * kStagedPitch + 16u * (2u * c + h));
             }
-            v16i zero;
+            if (k >= 1u && k < 9u) {
+                const unsigned c = k - 1u, slot = c % 2u;
+                const unsigned start = c % 2u == 0u ? 34u * c : 34u * c + 2u;
+                const unsigned at = (start & 15u) / 4u;
+                const unsigned q[8] = {lo[slot].x, lo[slot].y, lo[slot].z, lo[slot].w,
+                                       hi[slot].x, hi[slot].y, hi[slot].z, hi[slot].w};
+                v4i codes;
+                if (c % 2u == 0u) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) zero[i] = 0;
-            const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(tokens, codes, zero, 0, 0, 0);
+                    for (unsigned j = 0; j < 4u; ++j)
+                        codes[j] = (int)__builtin_amdgcn_alignbyte(q[at + j + 1u], q[at + j], 2u);
+                } else {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w, (float)dot[i], within[i]);
+                    for (unsigned j = 0; j < 4u; ++j) codes[j] = (int)q[at + j];
+                }
+                v16i zero;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) zero[i] = 0;
+                dot[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(tokens[slot], codes, zero, 0, 0, 0);
+                d_w[slot] = f16_bits_to_float(scale_bits[slot]);
+            }
+            if (k >= 2u) {
+                const unsigned slot = k % 2u;           // block k - 2
+#pragma unroll
+                for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w[slot], (float)dot[slot][i], within[i]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (unsigned i = 0; i < 16u; ++i) {
