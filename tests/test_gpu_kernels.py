@@ -313,16 +313,17 @@ def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, in
     assert np.allclose(few, got[:15], rtol=2e-5, atol=1e-6)
 
 
-def test_matvec_q8_0_large_batch_stages_operands_in_lds(gpu, oracle):
-    """A Q8_0 projection with at least one (128 rows x 64 input rows) tile per compute unit takes
-    the kernel whose operands pass through LDS: ragged row count (the last tile repeats a row), a
-    last tile of six input rows, several superblocks a row (both LDS buffers), additive rows and
-    bf16 outputs; the oracle's product within the format's tolerance, and the unstaged kernels
-    beside it."""
+@pytest.mark.parametrize("rows,width,inputs", [(2001, 1280, 1030), (4100, 512, 250)])
+def test_matvec_q8_0_large_batch_stages_operands_in_lds(gpu, oracle, rows, width, inputs):
+    """A Q8_0 projection with more unstaged tiles than one round of workgroups takes the kernel
+    whose operands pass through LDS, on tiles of 128 weight rows (the first case) or 64 (the
+    second): ragged row count (the last tile repeats a row), a ragged last tile of input rows,
+    several superblocks a row (both LDS buffers), additive rows and bf16 outputs; the oracle's
+    product within the format's tolerance, and the unstaged kernels beside it."""
     from yvex_amd import kernels as K
-    qt, rows, width, inputs = oracle.Q8_0, 2001, 1280, 1030
-    assert (rows + 127) // 128 * ((inputs + 63) // 64) >= 256
-    g = oracle.Generator(42, "matvec.rows.staged.q8_0")
+    qt = oracle.Q8_0
+    assert (rows + 31) // 32 * ((inputs + 63) // 64) > 256
+    g = oracle.Generator(42, f"matvec.rows.staged.q8_0.{rows}")
     w = g.weights(qt, rows, width)
     x = g.normal(inputs * width).reshape(inputs, width)
     bias = g.normal(inputs * rows).reshape(inputs, rows)

@@ -211,12 +211,16 @@ __global__ __launch_bounds__(256) void dense_q8_0_kernel(DenseQ80Args g)
 // (r, h) holds weight row r against input rows 8 (i / 4) + 4 h + i % 4: the block's scale is one
 // value a lane (read from the row's bytes in LDS) and the input rows' scales, needed once a
 // superblock, are sixteen broadcast reads.
-constexpr unsigned kStagedThreads = 512u, kStagedRows = 128u, kStagedTokens = 64u, kStagedPitch = 272u;
-constexpr unsigned kStagedWeightBytes = kStagedRows * kStagedPitch;                 // one buffer
-constexpr unsigned kStagedActBytes = kStagedTokens * kStagedPitch;
-constexpr unsigned kStagedWeightBase = 0u;                                          // [buffer]
-constexpr unsigned kStagedActBase = kStagedWeightBase + 2u * kStagedWeightBytes;    // [buffer]
-constexpr unsigned kStagedLdsBytes = kStagedActBase + 2u * kStagedActBytes;
+//
+// ROW_BLOCKS = 4: the tile above (512 lanes, 104 KB of LDS, a workgroup a compute unit);
+// ROW_BLOCKS = 2: 64 weight rows, four waves, 70 KB, two workgroups a compute unit, for batches
+// that have too few of the large tiles.
+constexpr unsigned kStagedTokens = 64u, kStagedPitch = 272u;
+constexpr unsigned kStagedActBytes = kStagedTokens * kStagedPitch;                  // one buffer
+constexpr unsigned staged_lds_bytes(unsigned row_blocks)
+{
+    return 2u * (32u * row_blocks * kStagedPitch + kStagedActBytes);
+}
 
 __device__ __forceinline__ uint4 read16(unsigned address)
 {
@@ -224,8 +228,18 @@ __device__ __forceinline__ uint4 read16(unsigned address)
     return make_uint4((unsigned)v[0], (unsigned)v[1], (unsigned)v[2], (unsigned)v[3]);
 }
 
-__global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(DenseQ80Args g)
+template <unsigned ROW_BLOCKS>
+__global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(DenseQ80Args g)
 {
+    constexpr unsigned kStagedThreads = 128u * ROW_BLOCKS, kStagedRows = 32u * ROW_BLOCKS;
+    constexpr unsigned kStagedWeightBytes = kStagedRows * kStagedPitch;                 // one buffer
+    constexpr unsigned kStagedWeightBase = 0u;                                          // [buffer]
+    constexpr unsigned kStagedActBase = kStagedWeightBase + 2u * kStagedWeightBytes;    // [buffer]
+    constexpr unsigned kWeightRounds = kStagedRows * 17u / kStagedThreads;              // full rounds of copies
+    constexpr unsigned kWeightRest = (kStagedRows * 17u - kWeightRounds * kStagedThreads) / 64u;   // waves of the last
+    constexpr unsigned kActRounds = kStagedTokens * 17u / kStagedThreads;
+    constexpr unsigned kActRest = (kStagedTokens * 17u - kActRounds * kStagedThreads) / 64u;
+    static_assert(kWeightRounds + 1u <= 5u && kActRounds + 1u <= 5u, "copy sources");
     extern __shared__ __align__(16) unsigned char dense_q8_0_lds[];
     if (lds_address_of(dense_q8_0_lds) != 0u) {   // operands are addressed by absolute LDS offsets
         if (threadIdx.x == 0u) raise_status(g.status, 2);
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(Dense
     }
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
-    const unsigned row_block = wave & 3u, token_block = wave >> 2;
+    const unsigned row_block = wave % ROW_BLOCKS, token_block = wave / ROW_BLOCKS;
     const unsigned long long row0 = (unsigned long long)blockIdx.x * kStagedRows;
     const unsigned long long tok0 = (unsigned long long)blockIdx.y * kStagedTokens;
     const unsigned rows_here = (unsigned)(g.row_count - row0 < kStagedRows ? g.row_count - row0 : kStagedRows);
@@ -241,19 +255,19 @@ __global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(Dense
     const unsigned long long act_row_bytes = (unsigned long long)g.blocks * kQ8KBytes;
 
     // ---- copy sources (a ragged edge repeats the tile's last row) ----
-    // weights: piece q = tid + 512 k of the tile's 128 x 17; input rows: piece q of 64 x 17, the
-    // seventeenth being the 16 bytes at the row's start
-    const unsigned char *weight_from[5], *act_from[3];
+    // weights: piece q = tid + threads * k of the tile's rows x 17; input rows: piece q of 64 x 17,
+    // the seventeenth being the 16 bytes at the row's start
+    const unsigned char *weight_from[kWeightRounds + 1u], *act_from[kActRounds + 1u];
 #pragma unroll
-    for (unsigned k = 0; k < 5u; ++k) {
-        unsigned q = tid + 512u * k;
+    for (unsigned k = 0; k < kWeightRounds + 1u; ++k) {
+        unsigned q = tid + kStagedThreads * k;
         if (q >= kStagedRows * 17u) q = kStagedRows * 17u - 1u;            // (waves that do not copy this round)
         const unsigned row = q / 17u, piece = q - row * 17u;
         weight_from[k] = g.encoded + (row0 + (row < rows_here ? row : rows_here - 1u)) * g.row_bytes + 16u * piece;
     }
 #pragma unroll
-    for (unsigned k = 0; k < 3u; ++k) {
-        unsigned q = tid + 512u * k;
+    for (unsigned k = 0; k < kActRounds + 1u; ++k) {
+        unsigned q = tid + kStagedThreads * k;
         if (q >= kStagedTokens * 17u) q = kStagedTokens * 17u - 1u;
         const unsigned token = q / 17u, piece = q - token * 17u;
         act_from[k] = g.act + (tok0 + (token < toks_here ? token : toks_here - 1u)) * act_row_bytes +
@@ -268,15 +282,19 @@ __global__ __launch_bounds__(kStagedThreads) void dense_q8_0_staged_kernel(Dense
         const unsigned w_to = kStagedWeightBase + buffer * kStagedWeightBytes + 1024u * wave;
         const unsigned a_to = kStagedActBase + buffer * kStagedActBytes + 1024u * wave;
 #pragma unroll
-        for (unsigned k = 0; k < 4u; ++k)
-            copy_to_lds_16(weight_from[k] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 8192u * k)));
-        if (wave < 2u)
-            copy_to_lds_16(weight_from[4] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 32768u)));
+        for (unsigned k = 0; k < kWeightRounds; ++k)
+            copy_to_lds_16(weight_from[k] + w_at,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 16u * kStagedThreads * k)));
+        if (wave < kWeightRest)
+            copy_to_lds_16(weight_from[kWeightRounds] + w_at,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 16u * kStagedThreads * kWeightRounds)));
 #pragma unroll
-        for (unsigned k = 0; k < 2u; ++k)
-            copy_to_lds_16(act_from[k] + a_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 8192u * k)));
-        if (wave == 0u)
-            copy_to_lds_16(act_from[2] + a_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16384u)));
+        for (unsigned k = 0; k < kActRounds; ++k)
+            copy_to_lds_16(act_from[k] + a_at,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16u * kStagedThreads * k)));
+        if (wave < kActRest)
+            copy_to_lds_16(act_from[kActRounds] + a_at,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16u * kStagedThreads * kActRounds)));
     };
 
     float acc[16];
@@ -386,14 +404,32 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
     DenseQ80Args g{encoded, row_count, row_bytes, (unsigned)(row_width / 256u),
                    (const unsigned char *)act_q8k, input_rows, additive, out, out_stride,
                    output_bf16 ? 1 : 0, status};
-    const uint64_t staged_row_tiles = (row_count + kStagedRows - 1u) / kStagedRows;
-    const uint64_t staged_token_tiles = (input_rows + kStagedTokens - 1u) / kStagedTokens;
-    if (!((uintptr_t)encoded & 15u) && staged_row_tiles * staged_token_tiles >= (uint64_t)compute_units() &&
-        staged_token_tiles <= 65535ull) {
-        YVEX_ALLOW_DYNAMIC_LDS(dense_q8_0_staged_kernel, kStagedLdsBytes);
-        dense_q8_0_staged_kernel<<<dim3((unsigned)staged_row_tiles, (unsigned)staged_token_tiles), kStagedThreads,
-                                   kStagedLdsBytes, stream>>>(g);
-        return check_launch("dense_q8_0_staged");
+    // Which tiles: a pass over the row width costs a workgroup about the same whatever the device's
+    // load (measured at 16 superblocks a row, microseconds: 17 or 25 unstaged with one or two
+    // blocks of input rows, 29 on the 64-row staged tile and 43 once two of them share a compute
+    // unit, 35 on the 128-row tile), so the choice is the number of rounds each shape needs.
+    const uint64_t token_tiles64 = (input_rows + kStagedTokens - 1u) / kStagedTokens;
+    const uint64_t tall = (row_count + 127u) / 128u * token_tiles64, low = (row_count + 63u) / 64u * token_tiles64;
+    const uint64_t units = (uint64_t)compute_units();
+    if (!((uintptr_t)encoded & 15u) && token_tiles64 <= 65535ull && units) {
+        const uint64_t plain = input_rows <= 32u ? row_tiles : row_tiles * token_tiles64;
+        const double plain_cost = input_rows <= 32u ? 17.0 * (double)((plain + 2u * units - 1u) / (2u * units))
+                                                    : 25.0 * (double)((plain + units - 1u) / units);
+        const double low_share = 43.0 * (double)low / (double)(2u * units);
+        const double low_cost = low <= units ? 29.0 : (low_share > 43.0 ? low_share : 43.0);
+        const double tall_cost = 35.0 * (double)((tall + units - 1u) / units);
+        if (tall_cost < plain_cost && tall_cost <= low_cost) {
+            YVEX_ALLOW_DYNAMIC_LDS(dense_q8_0_staged_kernel<4u>, staged_lds_bytes(4u));
+            dense_q8_0_staged_kernel<4u><<<dim3((unsigned)((row_count + 127u) / 128u), (unsigned)token_tiles64), 512,
+                                          staged_lds_bytes(4u), stream>>>(g);
+            return check_launch("dense_q8_0_staged");
+        }
+        if (low_cost < plain_cost) {
+            YVEX_ALLOW_DYNAMIC_LDS(dense_q8_0_staged_kernel<2u>, staged_lds_bytes(2u));
+            dense_q8_0_staged_kernel<2u><<<dim3((unsigned)((row_count + 63u) / 64u), (unsigned)token_tiles64), 256,
+                                          staged_lds_bytes(2u), stream>>>(g);
+            return check_launch("dense_q8_0_staged");
+        }
     }
     if (input_rows <= 32u) {
         dense_q8_0_kernel<1><<<dim3((unsigned)row_tiles, 1), 256, 0, stream>>>(g);
