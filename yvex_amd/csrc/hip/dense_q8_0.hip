@@ -8,16 +8,17 @@
 //     dot   = sum_i q_i * a_i                       (int32, exact: one K step of V_MFMA_I32_32X32X32_I8)
 //     value = (d_block * d_a) * float(dot)          (two float products)
 // and the values of a row are added in float. Here the eight blocks under one input scale are
-// added as d_block * float(dot) and the sum is multiplied by d_a once: float sums in another
-// order, inside the 1e-5 the format's dense rows are held to. A block has a scale of its own, so
+// added as fma(d_block, float(dot), sum) and the sum enters the row's with fma(d_a, sum, row):
+// float sums in another order and with fewer roundings, inside the 1e-5 the format's dense rows
+// are held to. A block has a scale of its own, so
 // every matrix instruction starts from zero and its sixteen results a lane are converted, scaled
 // and added on the vector ALU.
 //
-// A workgroup owns 32 weight rows x 32 or 64 input rows; its four waves take every fourth
-// superblock (eight blocks, 272 bytes a row) and their partial tiles are added in wave order, so
-// results do not depend on timing. Lane (r, h) holds bytes 16 h .. 16 h + 15 of weight row r's
-// block as the A operand and the same bytes of input row r's block as the B operand; accumulator
-// i of that lane is weight row 8 (i / 4) + 4 h + i % 4 against input row r. Blocks start on 2-byte
+// A workgroup owns 32 weight rows x 32 input rows; its four waves take every fourth superblock
+// (eight blocks, 272 bytes a row) and their partial tiles are added in wave order, so results do
+// not depend on timing. The input rows are the A operand and the weight rows the B operand: lane (r, h) holds bytes 16 h .. 16 h + 15 of input row r's block and
+// of weight row r's block, and accumulator i of that lane is weight row r against input row
+// 8 (i / 4) + 4 h + i % 4, so a block's scale is one value a lane. Blocks start on 2-byte
 // boundaries (34 bytes each): the codes of an even block are read as five aligned dwords and
 // shifted into place, those of an odd block are dword-aligned as they lie.
 #include "common.hpp"
@@ -41,19 +42,17 @@ struct DenseQ80Args {
     int *status;
 };
 
-// What a lane needs of one superblock: its half of the eight blocks' codes, their scales, and
-// its half of NT input rows' blocks.
-template <unsigned NT>
+// What a lane needs of one superblock: its half of the eight blocks' codes (their scales lie in
+// the same windows) and its half of one input row's blocks.
 struct Q80Inputs {
     uint4 codes[8];         // even blocks: the aligned window two bytes in front of the codes
     unsigned tail[4];       // even blocks: the dword behind the window
-    uint4 a[NT][8];
-    float act_scale[NT];
+    uint4 a[8];
+    float act_scale;
 };
 
-template <unsigned NT>
-__device__ __forceinline__ void q80_load(const unsigned char *wrow, const unsigned char *const (&arow)[NT],
-                                         unsigned sb, unsigned h, Q80Inputs<NT> &in)
+__device__ __forceinline__ void q80_load(const unsigned char *wrow, const unsigned char *arow, unsigned sb,
+                                         unsigned h, Q80Inputs &in)
 {
     const unsigned char *w = wrow + (unsigned long long)sb * 272ull;     // dword-aligned
 #pragma unroll
@@ -69,102 +68,102 @@ __device__ __forceinline__ void q80_load(const unsigned char *wrow, const unsign
             in.codes[c] = make_uint4(p[0], p[1], p[2], p[3]);
         }
     }
+    const unsigned char *a = arow + (unsigned long long)sb * kQ8KBytes;
+    in.act_scale = *reinterpret_cast<const float *>(a);
 #pragma unroll
-    for (unsigned nt = 0; nt < NT; ++nt) {
-        const unsigned char *a = arow[nt] + (unsigned long long)sb * kQ8KBytes;
-        in.act_scale[nt] = *reinterpret_cast<const float *>(a);
-#pragma unroll
-        for (unsigned c = 0; c < 8u; ++c) {
-            const unsigned *p = reinterpret_cast<const unsigned *>(a + 4u + 32u * c + 16u * h);
-            in.a[nt][c] = make_uint4(p[0], p[1], p[2], p[3]);
-        }
+    for (unsigned c = 0; c < 8u; ++c) {
+        const unsigned *p = reinterpret_cast<const unsigned *>(a + 4u + 32u * c + 16u * h);
+        in.a[c] = make_uint4(p[0], p[1], p[2], p[3]);
     }
 }
 
-template <unsigned NT>
-__global__ __launch_bounds__(256) void dense_q8_0_kernel(DenseQ80Args g)
+constexpr unsigned kPlainWaves = 4u;
+
+__global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Args g)
 {
-    // per wave: the scales of its 32 rows' eight blocks of the superblock in hand; then the partial tiles
-    __shared__ __align__(16) float block_scale[4][8][32];
-    __shared__ float partial[3][NT][16][64];
+    // per wave: the scales of the input rows whose blocks its lanes hold; then the partial tiles
+    __shared__ __align__(16) float row_scale[kPlainWaves][32];
+    __shared__ float partial[kPlainWaves - 1u][16][64];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
     const unsigned long long row0 = (unsigned long long)blockIdx.x * 32ull;
-    const unsigned long long tok0 = (unsigned long long)blockIdx.y * (32ull * NT);
+    const unsigned long long tok0 = (unsigned long long)blockIdx.y * 32ull;
     unsigned long long wr = row0 + r;
     if (wr >= g.row_count) wr = g.row_count - 1ull;              // a ragged edge repeats the last row
     const unsigned char *wrow = g.encoded + wr * g.row_bytes;
-    const unsigned char *arow[NT];
-    const unsigned long long act_row_bytes = (unsigned long long)g.blocks * kQ8KBytes;
+    unsigned long long t = tok0 + r;
+    if (t >= g.input_rows) t = g.input_rows - 1ull;
+    const unsigned char *arow = g.act + t * ((unsigned long long)g.blocks * kQ8KBytes);
+    float acc[16];
 #pragma unroll
-    for (unsigned nt = 0; nt < NT; ++nt) {
-        unsigned long long t = tok0 + 32ull * nt + r;
-        if (t >= g.input_rows) t = g.input_rows - 1ull;
-        arow[nt] = g.act + t * act_row_bytes;
-    }
-    float acc[NT][16];
-#pragma unroll
-    for (unsigned nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-    Q80Inputs<NT> cur;
-    q80_load<NT>(wrow, arow, wave < g.blocks ? wave : 0u, h, cur);
-    for (unsigned sb = wave; sb < g.blocks; sb += 4u) {
+    Q80Inputs cur;
+    q80_load(wrow, arow, wave < g.blocks ? wave : 0u, h, cur);
+    for (unsigned sb = wave; sb < g.blocks; sb += kPlainWaves) {
         // the next superblock's bytes travel while this one is worked on
-        Q80Inputs<NT> nxt;
-        q80_load<NT>(wrow, arow, sb + 4u < g.blocks ? sb + 4u : sb, h, nxt);
+        Q80Inputs nxt;
+        q80_load(wrow, arow, sb + kPlainWaves < g.blocks ? sb + kPlainWaves : sb, h, nxt);
 
-        // The scales lie in the windows already: an even block's in front of its codes (the low
-        // half of the first dword of the lane with h = 0), an odd block's behind the codes of the
-        // block before it (the high half of the tail dword of the lane with h = 1).
+        // The block scales lie in the windows already: an even block's in front of its codes (the
+        // low half of the first dword of the lane with h = 0), an odd block's behind the codes of
+        // the block before it (the high half of the tail dword of the lane with h = 1). Each half
+        // packs its four and takes the other half's from the lane 32 away.
+        unsigned mine[2], theirs[2];
 #pragma unroll
-        for (unsigned j = 0; j < 4u; ++j)
-            block_scale[wave][2u * j + h][r] =
-                f16_bits_to_float(h ? cur.tail[j] >> 16 : cur.codes[2u * j].x & 0xffffu);
+        for (unsigned j = 0; j < 2u; ++j) {
+            const unsigned first = h ? cur.tail[2u * j] >> 16 : cur.codes[4u * j].x & 0xffffu;
+            const unsigned second = h ? cur.tail[2u * j + 1u] >> 16 : cur.codes[4u * j + 2u].x & 0xffffu;
+            mine[j] = first | (second << 16);
+            theirs[j] = (unsigned)__shfl_xor((int)mine[j], 32, 64);
+        }
+        float d_w[8];
+#pragma unroll
+        for (unsigned c = 0; c < 8u; ++c) {
+            const unsigned pack = (c % 2u == h) ? mine[c / 4u] : theirs[c / 4u];     // blocks c with c % 2 == h are mine
+            d_w[c] = f16_bits_to_float((c / 2u) % 2u ? pack >> 16 : pack & 0xffffu);
+        }
+        // the input rows' scales to the lanes that hold their sums
+        row_scale[wave][r] = cur.act_scale;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float within[NT][16];       // the superblock's sum before the input row's scale
+
+        float within[16];       // the superblock's sum before the input rows' scales
 #pragma unroll
-        for (unsigned nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) within[nt][i] = 0.0f;
+        for (int i = 0; i < 16; ++i) within[i] = 0.0f;
 #pragma unroll
         for (unsigned c = 0; c < 8u; ++c) {
-            v4i a;
+            v4i codes;
             if (c % 2u == 0u) {
                 const uint4 q = cur.codes[c];
-                a[0] = (int)__builtin_amdgcn_alignbyte(q.y, q.x, 2u);
-                a[1] = (int)__builtin_amdgcn_alignbyte(q.z, q.y, 2u);
-                a[2] = (int)__builtin_amdgcn_alignbyte(q.w, q.z, 2u);
-                a[3] = (int)__builtin_amdgcn_alignbyte(cur.tail[c / 2u], q.w, 2u);
+                codes[0] = (int)__builtin_amdgcn_alignbyte(q.y, q.x, 2u);
+                codes[1] = (int)__builtin_amdgcn_alignbyte(q.z, q.y, 2u);
+                codes[2] = (int)__builtin_amdgcn_alignbyte(q.w, q.z, 2u);
+                codes[3] = (int)__builtin_amdgcn_alignbyte(cur.tail[c / 2u], q.w, 2u);
             } else {
-                a[0] = (int)cur.codes[c].x; a[1] = (int)cur.codes[c].y;
-                a[2] = (int)cur.codes[c].z; a[3] = (int)cur.codes[c].w;
+                codes[0] = (int)cur.codes[c].x; codes[1] = (int)cur.codes[c].y;
+                codes[2] = (int)cur.codes[c].z; codes[3] = (int)cur.codes[c].w;
             }
-            // the scales of the sixteen rows this lane accumulates
-            float d_of[16];
+            v16i zero;
 #pragma unroll
-            for (unsigned q4 = 0; q4 < 4u; ++q4) {
-                const float4 d = *reinterpret_cast<const float4 *>(&block_scale[wave][c][8u * q4 + 4u * h]);
-                d_of[4u * q4] = d.x; d_of[4u * q4 + 1u] = d.y; d_of[4u * q4 + 2u] = d.z; d_of[4u * q4 + 3u] = d.w;
-            }
+            for (int i = 0; i < 16; ++i) zero[i] = 0;
+            const v4i tokens = {(int)cur.a[c].x, (int)cur.a[c].y, (int)cur.a[c].z, (int)cur.a[c].w};
+            const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(tokens, codes, zero, 0, 0, 0);
 #pragma unroll
-            for (unsigned nt = 0; nt < NT; ++nt) {
-                v16i zero;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) zero[i] = 0;
-                const v4i b = {(int)cur.a[nt][c].x, (int)cur.a[nt][c].y, (int)cur.a[nt][c].z, (int)cur.a[nt][c].w};
-                const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 16; ++i) within[nt][i] += d_of[i] * (float)dot[i];
-            }
+            for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w[c], (float)dot[i], within[i]);
+            // (left alone the scheduler issues the matrix instructions of all blocks first and
+            // keeps their results)
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (unsigned nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[nt][i] += cur.act_scale[nt] * within[nt][i];
+        for (unsigned q4 = 0; q4 < 4u; ++q4) {
+            const float4 d = *reinterpret_cast<const float4 *>(&row_scale[wave][8u * q4 + 4u * h]);
+            acc[4u * q4] = __builtin_fmaf(d.x, within[4u * q4], acc[4u * q4]);
+            acc[4u * q4 + 1u] = __builtin_fmaf(d.y, within[4u * q4 + 1u], acc[4u * q4 + 1u]);
+            acc[4u * q4 + 2u] = __builtin_fmaf(d.z, within[4u * q4 + 2u], acc[4u * q4 + 2u]);
+            acc[4u * q4 + 3u] = __builtin_fmaf(d.w, within[4u * q4 + 3u], acc[4u * q4 + 3u]);
+        }
         // (the next superblock's scales are not written before every lane has read these)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -173,26 +172,24 @@ __global__ __launch_bounds__(256) void dense_q8_0_kernel(DenseQ80Args g)
 
     if (wave) {
 #pragma unroll
-        for (unsigned nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) partial[wave - 1u][nt][i][lane] = acc[nt][i];
+        for (int i = 0; i < 16; ++i) partial[wave - 1u][i][lane] = acc[i];
     }
     __syncthreads();
     if (wave) return;
+    // lane (r, h): weight row r against sixteen input rows; a store instruction writes 32
+    // consecutive floats of two output rows
+    const unsigned long long row = row0 + r;
 #pragma unroll
-    for (unsigned nt = 0; nt < NT; ++nt) {
-        const unsigned long long token = tok0 + 32ull * nt + r;
+    for (int i = 0; i < 16; ++i) {
+        const unsigned long long token = tok0 + 8u * (i >> 2) + 4u * h + (i & 3);
+        float sum = acc[i];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const unsigned long long row = row0 + 8u * (i >> 2) + 4u * h + (i & 3);
-            const float sum = ((acc[nt][i] + partial[0][nt][i][lane]) + partial[1][nt][i][lane]) +
-                              partial[2][nt][i][lane];
-            if (row >= g.row_count || token >= g.input_rows) continue;
-            const unsigned long long at = token * g.out_stride + row;
-            const float value = g.additive ? sum + g.additive[at] : sum;
-            if (!finite_f32(value)) raise_status(g.status, 1);
-            else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
-        }
+        for (unsigned w = 0; w + 1u < kPlainWaves; ++w) sum += partial[w][i][lane];
+        if (row >= g.row_count || token >= g.input_rows) continue;
+        const unsigned long long at = token * g.out_stride + row;
+        const float value = g.additive ? sum + g.additive[at] : sum;
+        if (!finite_f32(value)) raise_status(g.status, 1);
+        else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
     }
 }
 
@@ -405,16 +402,17 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
                    (const unsigned char *)act_q8k, input_rows, additive, out, out_stride,
                    output_bf16 ? 1 : 0, status};
     // Which tiles: a pass over the row width costs a workgroup about the same whatever the device's
-    // load (measured at 16 superblocks a row, microseconds: 17 or 25 unstaged with one or two
-    // blocks of input rows, 29 on the 64-row staged tile and 43 once two of them share a compute
-    // unit, 35 on the 128-row tile), so the choice is the number of rounds each shape needs.
+    // load (measured at 16 superblocks a row, microseconds: 17 unstaged and 27 once two such
+    // workgroups share a compute unit, 29 on the 64-row staged tile and 43 once two of them share
+    // a compute unit, 35 on the 128-row tile), so the choice is the number of rounds each shape needs.
+    const uint64_t token_tiles32 = (input_rows + 31u) / 32u;
     const uint64_t token_tiles64 = (input_rows + kStagedTokens - 1u) / kStagedTokens;
-    const uint64_t tall = (row_count + 127u) / 128u * token_tiles64, low = (row_count + 63u) / 64u * token_tiles64;
+    if (token_tiles32 > 65535ull) return ST_BOUNDS;
     const uint64_t units = (uint64_t)compute_units();
-    if (!((uintptr_t)encoded & 15u) && token_tiles64 <= 65535ull && units) {
-        const uint64_t plain = input_rows <= 32u ? row_tiles : row_tiles * token_tiles64;
-        const double plain_cost = input_rows <= 32u ? 17.0 * (double)((plain + 2u * units - 1u) / (2u * units))
-                                                    : 25.0 * (double)((plain + units - 1u) / units);
+    if (!((uintptr_t)encoded & 15u) && units) {
+        const uint64_t plain = row_tiles * token_tiles32;
+        const uint64_t tall = (row_count + 127u) / 128u * token_tiles64, low = (row_count + 63u) / 64u * token_tiles64;
+        const double plain_cost = plain <= units ? 17.0 : 27.0 * (double)((plain + 2u * units - 1u) / (2u * units));
         const double low_share = 43.0 * (double)low / (double)(2u * units);
         const double low_cost = low <= units ? 29.0 : (low_share > 43.0 ? low_share : 43.0);
         const double tall_cost = 35.0 * (double)((tall + units - 1u) / units);
@@ -431,13 +429,7 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
             return check_launch("dense_q8_0_staged");
         }
     }
-    if (input_rows <= 32u) {
-        dense_q8_0_kernel<1><<<dim3((unsigned)row_tiles, 1), 256, 0, stream>>>(g);
-    } else {
-        const uint64_t token_tiles = (input_rows + 63u) / 64u;
-        if (token_tiles > 65535ull) return ST_BOUNDS;
-        dense_q8_0_kernel<2><<<dim3((unsigned)row_tiles, (unsigned)token_tiles), 256, 0, stream>>>(g);
-    }
+    dense_q8_0_kernel<<<dim3((unsigned)row_tiles, (unsigned)token_tiles32), 64 * kPlainWaves, 0, stream>>>(g);
     return check_launch("dense_q8_0");
 }
 
