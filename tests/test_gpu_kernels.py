@@ -244,7 +244,10 @@ def test_matvec_q8k_one_round_trip_kernels(gpu, oracle, qtype, rows, width, inpu
     # one item to the next, whose first weight windows come with the last copies of the one before
     ("IQ2_XXS", 2048, 1024, 2112),
     ("Q4_K", 516, 2048, 16), ("Q4_K", 132, 7168, 70), ("Q4_K", 2048, 7168, 16), ("Q4_K", 36, 512, 200),
-    ("Q4_K", 50, 2304, 17), ("Q4_K", 24, 7168, 32), ("Q4_K", 7, 256, 31)])
+    ("Q4_K", 50, 2304, 17), ("Q4_K", 24, 7168, 32), ("Q4_K", 7, 256, 31),
+    # Q4_K tile shapes by the number of workgroups: 16 x 32 tiles in several token tiles (the
+    # cases of 70 and 200 rows above), 32 x 32 tiles, 32 x 64 tiles
+    ("Q4_K", 2048, 512, 70), ("Q4_K", 2048, 256, 200)])
 def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, width, inputs):
     """From 2 (Q4_K) or 32 (IQ2_XXS) Q8_K input rows on, projections run on the int8 matrix cores
     (src/backend/cuda/private.h:461-464 turns the tensor-core kernels on at 16). Results are the
