@@ -355,6 +355,36 @@ def test_matvec_q8_0_large_batch_stages_operands_in_lds(gpu, oracle, rows, width
         assert np.allclose(few, got[:count], rtol=2e-5, atol=2e-6)
 
 
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("Q8_0", 130, 512, 3), ("Q8_0", 130, 512, 20), ("Q8_0", 1030, 256, 70), ("Q8_0", 2001, 256, 1030),
+    ("Q4_K", 130, 512, 3), ("Q4_K", 130, 512, 20), ("Q4_K", 2048, 256, 70), ("Q4_K", 2048, 256, 200),
+    ("Q4_K", 2001, 256, 1030), ("IQ2_XXS", 132, 512, 3), ("IQ2_XXS", 132, 512, 40), ("F32", 50, 256, 9)])
+def test_matvec_writes_rows_of_a_wider_output(gpu, oracle, qtype, rows, width, inputs):
+    """Every kernel behind yvex_hip_matvec honours the output stride (the additive operand shares
+    it): results land in the first `rows` columns of a wider buffer, bit for bit what the dense
+    output holds, and the columns behind them keep what they held."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec.stride.{qtype}.{rows}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    add = g.normal(inputs * (rows + 12)).reshape(inputs, rows + 12)
+    status = K.new_status(gpu)
+    q8 = qtype != "F32"
+    act = K.q8k_quantize(dev(x, gpu), status) if q8 else dev(x, gpu)
+    wide_add = dev(add, gpu)
+    dense_add = wide_add[:, :rows].contiguous()
+    for additive in (None, (dense_add, wide_add)):
+        dense = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=q8, input_rows=inputs,
+                         additive=additive[0] if additive else None, status=status)
+        wide = torch.full((inputs, rows + 12), -7.25, dtype=torch.float32, device=gpu)
+        K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=q8, input_rows=inputs,
+                 additive=additive[1] if additive else None, status=status, out=wide)
+        status_ok(status)
+        assert torch.equal(wide[:, :rows].contiguous().view(torch.int32), dense.view(torch.int32))
+        assert bool((wide[:, rows:] == -7.25).all())
+
+
 def test_matvec_q4k_large_batch_stages_operands_in_lds(gpu, oracle):
     """A Q4_K projection with at least one (128 rows x 64 tokens) tile per compute unit takes the
     kernel whose operands are staged through LDS: ragged row count (the last tile repeats a row),

@@ -84,10 +84,11 @@ def matvec(encoded, qtype, row_count, row_width, inputs, *, input_q8=False, inpu
     if out is None:
         out = torch.empty((input_rows, row_count), dtype=torch.float32, device=encoded.device)
     stride = row_width if input_q8 else inputs.stride(0)
+    out_stride = out.stride(0) if out.dim() == 2 else row_count      # `additive` shares the output's stride
     _call("yvex_hip_matvec", _ptr(encoded), C.c_uint(qtype), C.c_uint64(row_count),
           C.c_uint64(row_width), C.c_uint64(row_bytes(qtype, row_width)), _ptr(inputs),
           C.c_int(int(input_q8)), C.c_uint64(input_rows), C.c_uint64(stride), _ptr(additive),
-          _ptr(out), C.c_uint64(row_count), C.c_int(int(output_bf16)), _ptr(status), _stream())
+          _ptr(out), C.c_uint64(out_stride), C.c_int(int(output_bf16)), _ptr(status), _stream())
     return out
 
 
