@@ -385,6 +385,39 @@ def test_matvec_writes_rows_of_a_wider_output(gpu, oracle, qtype, rows, width, i
         assert bool((wide[:, rows:] == -7.25).all())
 
 
+@pytest.mark.parametrize("qtype,rows,width,inputs", [
+    ("Q8_0", 130, 512, 20), ("Q8_0", 1030, 256, 70), ("Q8_0", 2001, 256, 1030),
+    ("Q4_K", 130, 512, 20), ("Q4_K", 2048, 256, 70), ("Q4_K", 2048, 256, 200), ("Q4_K", 2001, 256, 1030),
+    ("IQ2_XXS", 132, 512, 40)])
+def test_matvec_row_batch_flags_non_finite(gpu, oracle, qtype, rows, width, inputs):
+    """A block scale that is infinite makes every sum of its weight row non-finite: the
+    matrix-core kernels raise the numeric status, publish no value that is not finite (a kernel
+    may hold back the stores that share an instruction with one: the row's neighbours in its
+    32-row tile) and leave the other tiles' results what they are with clean weights."""
+    from yvex_amd import kernels as K
+    qt = getattr(oracle, qtype)
+    g = oracle.Generator(42, f"matvec.poison.{qtype}.{rows}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    clean = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs, status=status)
+    status_ok(status)
+    row_bytes = oracle.row_bytes(qt, width)
+    bad_row = rows - 3
+    poisoned = w.copy()
+    poisoned[bad_row * row_bytes:bad_row * row_bytes + 2] = (0x00, 0x7c)         # the first block's fp16 scale
+    out = torch.full((inputs, rows), -7.25, dtype=torch.float32, device=gpu)
+    K.matvec(dev(poisoned, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs, status=status, out=out)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    keep = torch.ones(rows, dtype=torch.bool, device=gpu)
+    keep[bad_row // 32 * 32:bad_row // 32 * 32 + 32] = False
+    assert torch.equal(out[:, keep].contiguous().view(torch.int32), clean[:, keep].contiguous().view(torch.int32))
+    assert bool((out[:, bad_row] == -7.25).all())
+    assert bool(torch.isfinite(out).all())
+
+
 def test_matvec_q4k_large_batch_stages_operands_in_lds(gpu, oracle):
     """A Q4_K projection with at least one (128 rows x 64 tokens) tile per compute unit takes the
     kernel whose operands are staged through LDS: ragged row count (the last tile repeats a row),
