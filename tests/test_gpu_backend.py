@@ -584,15 +584,19 @@ def test_execute_rows_hash_router(backend, oracle, streams):
     case.tokens[2] = 1
 
 
-@pytest.mark.parametrize("qtype", ["IQ2_XXS", "Q4_K"])
-def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle, qtype):
+@pytest.mark.parametrize("qtype,down_qtype", [("IQ2_XXS", None), ("Q4_K", None), ("IQ2_XXS", "Q2_K"),
+                                              ("Q4_K", "Q2_K"), ("IQ2_XXS", "Q4_K")])
+def test_execute_rows_large_batch_takes_matrix_core_kernels(backend, oracle, qtype, down_qtype):
     """Row batches whose buckets average six pairs or more run the int8 matrix-core kernels
-    (routed and shared expert); the result is the CPU layer's, bit for bit."""
-    case = MoeCase(backend, oracle, qtype=qtype, hidden=768, intermediate=512, experts=4, topk=2,
-                   rows=200, scoring=abi.SCORING_SIGMOID)
+    (routed and shared expert); the result is the CPU layer's, bit for bit. IQ2_XXS gate and up
+    rows with Q2_K down rows is the pairing the reference's tensor-core kernels serve
+    (src/backend/cuda/tensorcore.cu:563-564, 660)."""
+    case = MoeCase(backend, oracle, qtype=qtype, down_qtype=down_qtype, hidden=768, intermediate=512, experts=4,
+                   topk=2, rows=200, scoring=abi.SCORING_SIGMOID)
     backend.workspace(case.workspace_bytes)
     rc = case.execute()
     assert rc == 0, case.err.message
+    assert case.result.tensor_core_launches > 0
     want = case.oracle_layer(act_q8=True)
     assert np.array_equal(case.sel.reshape(case.rows, case.topk), want["selected"])
     got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)

@@ -156,9 +156,10 @@ static inline void fill_down_problem(GroupedProblem &p, const yvex_hip_expert_we
 bool iq2_sweep_supported(unsigned qtype, unsigned width, unsigned out_rows, unsigned long long pairs, bool image);
 int launch_iq2_sweep(const GroupedArgs &a, unsigned qtype, bool fused, bool image, hipStream_t stream);
 
-// Row-batch expert kernels for Q4_K weights on the int8 matrix cores (dense_q4k.hip).
-int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t width, uint64_t out_rows,
-                            double limit, int *status, hipStream_t stream);
+// Row-batch expert kernels on the int8 matrix cores (rows_q4k.hip): Q4_K weights, fused gate/up
+// or a plain projection; Q2_K weights, a plain projection (the down experts).
+int launch_q4k_rows_grouped(const GroupedProblem &problem, unsigned qtype, bool fused, uint64_t width,
+                            uint64_t out_rows, double limit, int *status, hipStream_t stream);
 
 static inline bool same_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)
 {

@@ -911,7 +911,7 @@ extern "C" int yvex_hip_moe_up_rows(const yvex_hip_expert_weights *w, const void
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
     fill_up_problem(a.pr, w, act_q8k, 1, route_weights, wl, pairs, topk, experts, intermediate);
     if (w->gate_qtype == QT_Q4_K)
-        return launch_q4k_rows_grouped(a.pr, true, w->hidden, w->intermediate, limit, status, as_stream(stream));
+        return launch_q4k_rows_grouped(a.pr, QT_Q4_K, true, w->hidden, w->intermediate, limit, status, as_stream(stream));
     a.width = (unsigned)w->hidden;
     a.out_rows = (unsigned)w->intermediate;
     a.limit = limit;
@@ -930,7 +930,7 @@ extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const vo
     if (!w || !w->down || !intermediate_q8k || !pair_outputs || !status || !pairs || !experts ||
         (expert_ids && (!bucket_offsets || !bucket_populations || !counts)))
         return ST_INVALID_ARG;
-    if (w->down_qtype != QT_IQ2_XXS && w->down_qtype != QT_Q4_K) return ST_UNSUPPORTED;
+    if (w->down_qtype != QT_IQ2_XXS && w->down_qtype != QT_Q4_K && w->down_qtype != QT_Q2_K) return ST_UNSUPPORTED;
     int rc = w->down_image
         ? check_image_matrix(w->down_qtype, w->intermediate, w->down_row_bytes, w->down, w->down_expert_bytes)
         : check_matrix(w->down_qtype, w->intermediate, w->down_row_bytes);
@@ -939,8 +939,9 @@ extern "C" int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *w, const vo
     MfmaArgs a{};
     const WorklistView wl{order, expert_ids, bucket_offsets, bucket_populations, nullptr, counts};
     fill_down_problem(a.pr, w, intermediate_q8k, 1, wl, pairs, experts, pair_outputs);
-    if (w->down_qtype == QT_Q4_K)
-        return launch_q4k_rows_grouped(a.pr, false, w->intermediate, w->hidden, 1.0, status, as_stream(stream));
+    if (w->down_qtype == QT_Q4_K || w->down_qtype == QT_Q2_K)
+        return launch_q4k_rows_grouped(a.pr, w->down_qtype, false, w->intermediate, w->hidden, 1.0, status,
+                                       as_stream(stream));
     a.width = (unsigned)w->intermediate;
     a.out_rows = (unsigned)w->hidden;
     a.limit = 1.0;

@@ -99,15 +99,35 @@ __device__ __forceinline__ void q4k_bsum_limbs(const uint4 (&b)[2], uint2 &lo, u
     hi = make_uint2(u[0], u[1]);
 }
 
+// The sixteen int16 block sums as two int8 limbs (value = 128 hi + lo, lo in 0..127), in order.
+__device__ __forceinline__ void q2k_bsum_limbs(const uint4 (&b)[2], v4i &lo, v4i &hi)
+{
+    const unsigned w[8] = {b[0].x, b[0].y, b[0].z, b[0].w, b[1].x, b[1].y, b[1].z, b[1].w};
+#pragma unroll
+    for (unsigned i = 0; i < 4u; ++i) {
+        unsigned l = 0u, u = 0u;
+#pragma unroll
+        for (unsigned k = 0; k < 4u; ++k) {
+            const unsigned word = w[2u * i + k / 2u];
+            const int sum = k % 2u ? (int)word >> 16 : (int)(short)(word & 0xffffu);
+            l |= ((unsigned)sum & 127u) << (8u * k);
+            u |= ((unsigned)(sum >> 7) & 255u) << (8u * k);
+        }
+        lo[i] = (int)l;
+        hi[i] = (int)u;
+    }
+}
+
 struct Q4Tile {
     unsigned long long expert, first;
     unsigned tokens;
 };
 
 // One (token tile, row tile) with NT live 32-token blocks.
-template <bool FUSED, unsigned NT>
+template <unsigned QT, bool FUSED, unsigned NT>
 __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile &tile)
 {
+    static_assert(QT == QT_Q4_K || (QT == QT_Q2_K && !FUSED), "Q4_K rows, or Q2_K rows of a plain projection");
     const GroupedProblem &pr = g.pr;
     const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
@@ -125,20 +145,26 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
     };
 
     // ---- copy sources ----
-    // weights: piece p = lane + 64 k of this wave's 288 (row p / 9, 16-byte piece p % 9)
-    const unsigned char *weight_from[5];
+    // Q4_K weights: piece p = lane + 64 k of this wave's 288 (row p / 9, 16-byte piece p % 9).
+    // Q2_K weights: dword p = lane + 64 k of this wave's 672 (row p / 21, dword p % 21: superblocks
+    // of 84 bytes are dword-aligned, not more); the eleventh round's upper half repeats the last
+    // dword into padding behind the rows.
+    constexpr unsigned kRounds = QT == QT_Q2_K ? 11u : 5u;
+    constexpr unsigned kPieces = QT == QT_Q2_K ? 21u : 9u, kPieceBytes = QT == QT_Q2_K ? 4u : 16u;
+    constexpr unsigned kSuperblockBytes = QT == QT_Q2_K ? 84u : 144u;
+    const unsigned char *weight_from[kRounds];
 #pragma unroll
-    for (unsigned k = 0; k < 5u; ++k) {
+    for (unsigned k = 0; k < kRounds; ++k) {
         const unsigned piece = lane + 64u * k;
-        const unsigned served = piece < 288u ? piece : 287u;
-        const unsigned wave_row = served / 9u;
+        const unsigned served = piece < 32u * kPieces ? piece : 32u * kPieces - 1u;
+        const unsigned wave_row = served / kPieces;
         unsigned row = row0 + (FUSED ? (wave_row & 15u) : wave_row);
         if (row >= g.out_rows) row = g.out_rows - 1u;        // a ragged edge repeats the last row
         const bool is_up = FUSED && wave_row >= 16u;
         const unsigned char *base = is_up
             ? pr.up + tile.expert * pr.up_expert_bytes + (unsigned long long)row * pr.up_row_bytes
             : pr.gate + tile.expert * pr.expert_bytes + (unsigned long long)row * pr.row_bytes;
-        weight_from[k] = base + 16u * (served % 9u);
+        weight_from[k] = base + kPieceBytes * (served % kPieces);
     }
     // activations: position q = tid + 256 k of the tile's 1024 (token q / 16, position q % 16
     // holds piece position ^ (token % 16))
@@ -161,13 +187,19 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
     auto copies = [&](unsigned sb) {
         const unsigned buffer = sb & 1u;
         const unsigned clamped = sb < last_block ? sb : last_block;
-        const unsigned long long w_at = (unsigned long long)clamped * 144ull;
+        const unsigned long long w_at = (unsigned long long)clamped * kSuperblockBytes;
         const unsigned long long a_at = (unsigned long long)clamped * kQ8KBytes;
         const unsigned w_to = weight_base + buffer * kQ4WeightBytes;
+        if constexpr (QT == QT_Q2_K) {
 #pragma unroll
-        for (unsigned k = 0; k < 4u; ++k)
-            copy_to_lds_16(weight_from[k] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 1024u * k)));
-        copy_to_lds_16_first32(weight_from[4] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 4096u)));
+            for (unsigned k = 0; k < kRounds; ++k)
+                copy_to_lds_4(weight_from[k] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 256u * k)));
+        } else {
+#pragma unroll
+            for (unsigned k = 0; k < 4u; ++k)
+                copy_to_lds_16(weight_from[k] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 1024u * k)));
+            copy_to_lds_16_first32(weight_from[4] + w_at, (unsigned)__builtin_amdgcn_readfirstlane((int)(w_to + 4096u)));
+        }
 #pragma unroll
         for (unsigned k = 0; k < 2u * NT; ++k)
             copy_to_lds_16(act_from[k] + a_at,
@@ -202,49 +234,88 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
         if (sb + 1u < g.blocks) copies(sb + 1u);
 
         // ---- this lane's weight row of the superblock ----
-        const unsigned w_at = weight_base + buffer * kQ4WeightBytes + r * 144u;
-        const uint4 head = read16(w_at);             // d | dmin << 16, then the 12 scale bytes
-        const unsigned s0 = head.y, s1 = head.z, s2 = head.w;
-        const unsigned sc_pack[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
-        const unsigned mn_pack[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
-        if (h == 0u) {
-            lds_write_u32(row_scale_at + 4u * r, __float_as_uint(f16_bits_to_float(head.x & 0xffffu)));
-            lds_write_u32(row_scale_at + 128u + 4u * r, __float_as_uint(f16_bits_to_float(head.x >> 16)));
-        }
+        const unsigned w_at = weight_base + buffer * kQ4WeightBytes + r * kSuperblockBytes;
         const unsigned a_at = kQ4ActBase + buffer * kQ4Tokens * 256u + r * 256u;
-
-        v16i lo_sum[NT], hi_sum[NT];
+        v16i lo_sum[NT], hi_sum[NT];     // Q2_K: one limb, lo_sum alone
 #pragma unroll
         for (unsigned nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) lo_sum[nt][i] = hi_sum[nt][i] = 0;
+        v4i m_op = {0, 0, 0, 0};         // the minimums of the row's sub-blocks, on the h = 0 half
+        if constexpr (QT == QT_Q2_K) {
+            // Public ggml block_q2_K (src/backend/cuda/kernel_primitives.h:314-341 is the product):
+            // sixteen bytes (scale | minimum << 4) of the 16-value sub-blocks, 64 bytes of 2-bit
+            // codes (byte l of half p holds values 128 p + 32 s + l at bit 2 s), fp16 d and dmin.
+            // K step c = 4 p + s is the sub-blocks 2 c and 2 c + 1: lane (r, h) scales the sixteen
+            // codes of sub-block 2 c + h (at most 3 * 15 = 45, one int8 limb), so one matrix
+            // instruction per step and token block.
+            const unsigned scale_words[4] = {lds_read_u32(w_at), lds_read_u32(w_at + 4u), lds_read_u32(w_at + 8u),
+                                             lds_read_u32(w_at + 12u)};
+            const unsigned dd = lds_read_u32(w_at + 80u);
+            if (h == 0u) {
+                lds_write_u32(row_scale_at + 4u * r, __float_as_uint(f16_bits_to_float(dd & 0xffffu)));
+                lds_write_u32(row_scale_at + 128u + 4u * r, __float_as_uint(f16_bits_to_float(dd >> 16)));
 #pragma unroll
-        for (unsigned j = 0; j < 4u; ++j) {
-            const uint4 q = read16(w_at + 16u + 32u * j + 16u * h);
+                for (unsigned i = 0; i < 4u; ++i) m_op[i] = (int)((scale_words[i] >> 4) & 0x0f0f0f0fu);
+            }
 #pragma unroll
-            for (unsigned half = 0; half < 2u; ++half) {
-                const unsigned c = 2u * j + half;
-                const unsigned sc = (sc_pack[c >> 2] >> (8u * (c & 3u))) & 255u;
-                const unsigned shift = 4u * half;
-                v4i a_lo, a_hi;
-                unsigned lo, hi;
-                q4k_limbs(q.x >> shift, sc, lo, hi); a_lo[0] = (int)lo; a_hi[0] = (int)hi;
-                q4k_limbs(q.y >> shift, sc, lo, hi); a_lo[1] = (int)lo; a_hi[1] = (int)hi;
-                q4k_limbs(q.z >> shift, sc, lo, hi); a_lo[2] = (int)lo; a_hi[2] = (int)hi;
-                q4k_limbs(q.w >> shift, sc, lo, hi); a_lo[3] = (int)lo; a_hi[3] = (int)hi;
+            for (unsigned p = 0; p < 2u; ++p) {
+                unsigned q[4];
 #pragma unroll
-                for (unsigned nt = 0; nt < NT; ++nt) {
-                    const v4i b = lds_read_v4i(a_at + nt * 32u * 256u + 16u * ((2u * c + h) ^ (r & 15u)));
-                    lo_sum[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo, b, lo_sum[nt], 0, 0, 0);
-                    hi_sum[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi, b, hi_sum[nt], 0, 0, 0);
+                for (unsigned i = 0; i < 4u; ++i) q[i] = lds_read_u32(w_at + 16u + 32u * p + 16u * h + 4u * i);
+#pragma unroll
+                for (unsigned sft = 0; sft < 4u; ++sft) {
+                    const unsigned c = 4u * p + sft;
+                    // scale byte 2 c + h: word c / 2, byte (2 c) % 4 + h
+                    const unsigned sc = (scale_words[c >> 1] >> (8u * ((2u * c) & 3u) + 8u * h)) & 15u;
+                    const u16x2 twice = __builtin_bit_cast(u16x2, sc * 0x00010001u);
+                    v4i a;
+#pragma unroll
+                    for (unsigned i = 0; i < 4u; ++i)
+                        // two bytes a 16-bit lane: (code * sc) stays inside its byte
+                        a[i] = (int)__builtin_bit_cast(unsigned,
+                                                       __builtin_bit_cast(u16x2, (q[i] >> (2u * sft)) & 0x03030303u) * twice);
+#pragma unroll
+                    for (unsigned nt = 0; nt < NT; ++nt) {
+                        const v4i b = lds_read_v4i(a_at + nt * 32u * 256u + 16u * ((2u * c + h) ^ (r & 15u)));
+                        lo_sum[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, lo_sum[nt], 0, 0, 0);
+                    }
                 }
             }
-        }
-        // minimum term: m_j (bytes 0..7 of the h = 0 half, zeros elsewhere) against the pair sums
-        v4i m_op = {0, 0, 0, 0};
-        if (h == 0u) {
-            m_op[0] = (int)mn_pack[0];
-            m_op[1] = (int)mn_pack[1];
+        } else {
+            const uint4 head = read16(w_at);             // d | dmin << 16, then the 12 scale bytes
+            const unsigned s0 = head.y, s1 = head.z, s2 = head.w;
+            const unsigned sc_pack[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
+            const unsigned mn_pack[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
+            if (h == 0u) {
+                lds_write_u32(row_scale_at + 4u * r, __float_as_uint(f16_bits_to_float(head.x & 0xffffu)));
+                lds_write_u32(row_scale_at + 128u + 4u * r, __float_as_uint(f16_bits_to_float(head.x >> 16)));
+                // minimum term: m_j (bytes 0..7 of the h = 0 half, zeros elsewhere) against the pair sums
+                m_op[0] = (int)mn_pack[0];
+                m_op[1] = (int)mn_pack[1];
+            }
+#pragma unroll
+            for (unsigned j = 0; j < 4u; ++j) {
+                const uint4 q = read16(w_at + 16u + 32u * j + 16u * h);
+#pragma unroll
+                for (unsigned half = 0; half < 2u; ++half) {
+                    const unsigned c = 2u * j + half;
+                    const unsigned sc = (sc_pack[c >> 2] >> (8u * (c & 3u))) & 255u;
+                    const unsigned shift = 4u * half;
+                    v4i a_lo, a_hi;
+                    unsigned lo, hi;
+                    q4k_limbs(q.x >> shift, sc, lo, hi); a_lo[0] = (int)lo; a_hi[0] = (int)hi;
+                    q4k_limbs(q.y >> shift, sc, lo, hi); a_lo[1] = (int)lo; a_hi[1] = (int)hi;
+                    q4k_limbs(q.z >> shift, sc, lo, hi); a_lo[2] = (int)lo; a_hi[2] = (int)hi;
+                    q4k_limbs(q.w >> shift, sc, lo, hi); a_lo[3] = (int)lo; a_hi[3] = (int)hi;
+#pragma unroll
+                    for (unsigned nt = 0; nt < NT; ++nt) {
+                        const v4i b = lds_read_v4i(a_at + nt * 32u * 256u + 16u * ((2u * c + h) ^ (r & 15u)));
+                        lo_sum[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_lo, b, lo_sum[nt], 0, 0, 0);
+                        hi_sum[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_hi, b, hi_sum[nt], 0, 0, 0);
+                    }
+                }
+            }
         }
         // d and dmin of the sixteen rows this lane accumulates (written above by the wave itself)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -258,10 +329,14 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
             if (h == 0u) {
                 const unsigned at = kQ4BsumBase + buffer * kQ4Tokens * 32u + 32u * token;
                 const uint4 bsums[2] = {read16(at), read16(at + 16u)};
-                uint2 bl, bh;
-                q4k_bsum_limbs(bsums, bl, bh);
-                b_lo[0] = (int)bl.x; b_lo[1] = (int)bl.y;
-                b_hi[0] = (int)bh.x; b_hi[1] = (int)bh.y;
+                if constexpr (QT == QT_Q2_K) {
+                    q2k_bsum_limbs(bsums, b_lo, b_hi);       // a minimum per 16 values: the sums as they are
+                } else {
+                    uint2 bl, bh;
+                    q4k_bsum_limbs(bsums, bl, bh);
+                    b_lo[0] = (int)bl.x; b_lo[1] = (int)bl.y;
+                    b_hi[0] = (int)bh.x; b_hi[1] = (int)bh.y;
+                }
             }
             v16i zero;
 #pragma unroll
@@ -279,7 +354,7 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
 #pragma unroll
                 for (unsigned k = 0; k < 4u; ++k) {
                     const unsigned i = 4u * q4 + k;
-                    const int dot = (hi_sum[nt][i] << 3) + lo_sum[nt][i];
+                    const int dot = QT == QT_Q2_K ? lo_sum[nt][i] : (hi_sum[nt][i] << 3) + lo_sum[nt][i];
                     const int minimum = (min_hi[i] << 7) + min_lo[i];
                     const float left = (da * d_of[k]) * (float)dot;
                     const float right = (da * dmin_of[k]) * (float)minimum;
@@ -364,7 +439,7 @@ __device__ __forceinline__ void rows_q4k_tile(const RowsQ4kArgs &g, const Q4Tile
     if (bad) raise_status(g.status, 1);
 }
 
-template <bool FUSED>
+template <unsigned QT, bool FUSED>
 __global__ __launch_bounds__(kQ4Threads, 2) void rows_q4k_kernel(RowsQ4kArgs g)
 {
     extern __shared__ __align__(16) unsigned char rows_q4k_lds[];
@@ -423,28 +498,32 @@ __global__ __launch_bounds__(kQ4Threads, 2) void rows_q4k_kernel(RowsQ4kArgs g)
         if (threadIdx.x == 0u) raise_status(g.status, 2);
         return;
     }
-    if (tile.tokens > 32u) rows_q4k_tile<FUSED, 2u>(g, tile);
-    else rows_q4k_tile<FUSED, 1u>(g, tile);
+    if (tile.tokens > 32u) rows_q4k_tile<QT, FUSED, 2u>(g, tile);
+    else rows_q4k_tile<QT, FUSED, 1u>(g, tile);
 }
 
-template <bool FUSED>
+template <unsigned QT, bool FUSED>
 int launch_rows_q4k(const RowsQ4kArgs &g, dim3 grid, hipStream_t stream)
 {
-    YVEX_ALLOW_DYNAMIC_LDS((rows_q4k_kernel<FUSED>), kQ4LdsBytes);
-    rows_q4k_kernel<FUSED><<<grid, kQ4Threads, kQ4LdsBytes, stream>>>(g);
+    YVEX_ALLOW_DYNAMIC_LDS((rows_q4k_kernel<QT, FUSED>), kQ4LdsBytes);
+    rows_q4k_kernel<QT, FUSED><<<grid, kQ4Threads, kQ4LdsBytes, stream>>>(g);
     return check_launch("rows_q4k");
 }
 
 }  // namespace
 
-int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t width, uint64_t out_rows,
-                            double limit, int *status, hipStream_t stream)
+int launch_q4k_rows_grouped(const GroupedProblem &problem, unsigned qtype, bool fused, uint64_t width,
+                            uint64_t out_rows, double limit, int *status, hipStream_t stream)
 {
+    if (qtype != QT_Q4_K && !(qtype == QT_Q2_K && !fused)) return ST_UNSUPPORTED;
     if (!width || width % 256u || !out_rows || out_rows > 0x7fffffffull) return ST_BOUNDS;
-    if (problem.row_bytes != width / 256u * 144u || (fused && problem.up_row_bytes != problem.row_bytes))
+    const uint64_t superblock = qtype == QT_Q2_K ? 84u : 144u;
+    // (Q4_K rows are copied in 16-byte pieces, Q2_K rows in dwords)
+    const uintptr_t misaligned = qtype == QT_Q2_K ? 3u : 15u;
+    if (problem.row_bytes != width / 256u * superblock || (fused && problem.up_row_bytes != problem.row_bytes))
         return ST_BOUNDS;
-    if (((uintptr_t)problem.gate & 15u) || (fused && ((uintptr_t)problem.up & 15u)) ||
-        ((uintptr_t)problem.activations & 3u) || (problem.expert_bytes & 15u) ||
+    if (((uintptr_t)problem.gate & misaligned) || (fused && ((uintptr_t)problem.up & 15u)) ||
+        ((uintptr_t)problem.activations & 3u) || (problem.expert_bytes & misaligned) ||
         (fused && (problem.up_expert_bytes & 15u)) || (problem.act_stride & 3u))
         return ST_INVALID_ARG;
     if (problem.experts > 256u && problem.expert_ids) return ST_BOUNDS;
@@ -455,7 +534,8 @@ int launch_q4k_rows_grouped(const GroupedProblem &problem, bool fused, uint64_t 
     if (row_tiles > 0x7fffffffull || token_tiles > 65535ull) return ST_BOUNDS;
     RowsQ4kArgs g{problem, (unsigned)(width / 256u), (unsigned)out_rows, limit, status, 0, 0, nullptr, 0ull};
     const dim3 grid((unsigned)row_tiles, (unsigned)token_tiles);
-    return fused ? launch_rows_q4k<true>(g, grid, stream) : launch_rows_q4k<false>(g, grid, stream);
+    if (qtype == QT_Q2_K) return launch_rows_q4k<QT_Q2_K, false>(g, grid, stream);
+    return fused ? launch_rows_q4k<QT_Q4_K, true>(g, grid, stream) : launch_rows_q4k<QT_Q4_K, false>(g, grid, stream);
 }
 
 // A plain projection of many input rows: one bucket that holds them all, outputs left in fp32
@@ -484,7 +564,7 @@ int launch_q4k_rows_staged(const uint8_t *encoded, uint64_t row_count, uint64_t 
     if (token_tiles > 65535ull) return ST_BOUNDS;
     RowsQ4kArgs g{problem, (unsigned)(row_width / 256u), (unsigned)row_count, 0.0, status, 1, output_bf16 ? 1 : 0,
                   additive, out_stride};
-    return launch_rows_q4k<false>(g, dim3((unsigned)row_tiles, (unsigned)token_tiles), stream);
+    return launch_rows_q4k<QT_Q4_K, false>(g, dim3((unsigned)row_tiles, (unsigned)token_tiles), stream);
 }
 
 }  // namespace yvex

@@ -316,11 +316,13 @@ static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weigh
 }
 
 /* Expert weights the matrix-core row-batch kernels take: gate and up of one format, IQ2_XXS (16)
- * or Q4_K (12); the down matrix may be of the other. */
+ * or Q4_K (12); the down matrix of either or Q2_K (10), the pairing the reference's own
+ * tensor-core kernels serve (IQ2_XXS gate and up, src/backend/cuda/tensorcore.cu:563-564; Q2_K
+ * down, tensorcore.cu:660). */
 static int matrix_core_qtypes(const yvex_hip_expert_weights *w)
 {
     return w->gate_qtype == w->up_qtype && (w->gate_qtype == 16u || w->gate_qtype == 12u) &&
-           (w->down_qtype == 16u || w->down_qtype == 12u);
+           (w->down_qtype == 16u || w->down_qtype == 12u || w->down_qtype == 10u);
 }
 
 static int same_expert_shape(const yvex_hip_expert_weights *a, const yvex_hip_expert_weights *b)

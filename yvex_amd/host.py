@@ -103,7 +103,7 @@ class RowBatchLayer:
 
     def __init__(self, torch, routed, shared, router, x_host, rows, *, hidden, intermediate, experts, topk,
                  qtype=16, sweep_image=False, scoring=abi.SCORING_SIGMOID, scaling=1.0, limit=10.0,
-                 envelope=None):
+                 envelope=None, down_qtype=None):
         """envelope: None, or the residual-stream weights around the layer as device tensors,
         dict(streams, iterations, function [F32 (streams + 2) * streams x streams * hidden], scale
         [F32 3], base [F32 (streams + 2) * streams], norm [BF16 hidden]); x_host then holds
@@ -131,8 +131,10 @@ class RowBatchLayer:
         plan.requires_correction_bias, plan.normalize_topk_probabilities = 0, 1
         job = self.job = abi.LayerJob()
         job.layer = C.pointer(plan)
-        block_bytes = {16: 66, 12: 144}[qtype]
-        rb_h, rb_i = HIDDEN // 256 * block_bytes, INTERMEDIATE // 256 * block_bytes
+        # down_qtype: the down projections' format where it differs from the gate and up projections'
+        down_qtype = qtype if down_qtype is None else down_qtype
+        block_bytes = {16: 66, 12: 144, 10: 84}
+        rb_h, rb_i = HIDDEN // 256 * block_bytes[qtype], INTERMEDIATE // 256 * block_bytes[down_qtype]
 
         self.images = []
 
@@ -168,10 +170,10 @@ class RowBatchLayer:
         gate_up, down_c, shared_c = abi.CONSUMER_ROUTED_GATE_UP, abi.CONSUMER_ROUTED_DOWN, abi.CONSUMER_SHARED_EXPERT
         view(abi.W_ROUTED_GATE, routed[0], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
         view(abi.W_ROUTED_UP, routed[1], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
-        view(abi.W_ROUTED_DOWN, routed[2], qtype, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc, down_c)
+        view(abi.W_ROUTED_DOWN, routed[2], down_qtype, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc, down_c)
         view(abi.W_SHARED_GATE, shared[0], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
         view(abi.W_SHARED_UP, shared[1], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
-        view(abi.W_SHARED_DOWN, shared[2], qtype, INTERMEDIATE, HIDDEN, rb_i, enc, shared_c)
+        view(abi.W_SHARED_DOWN, shared[2], down_qtype, INTERMEDIATE, HIDDEN, rb_i, enc, shared_c)
         if envelope:
             mixing = (streams + 2) * streams
             f32 = abi.ACT_DEVICE_F32
