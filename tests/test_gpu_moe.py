@@ -66,6 +66,10 @@ def make_layer(oracle, gpu, *, hidden, intermediate, experts, topk, rows, qtype,
     ("Q4_K", 2048, 2048, 6, 4, 20, True, 1, False),
     ("Q4_K", 7168, 2048, 12, 4, 6, True, 0, False),
     ("Q4_K", 4096, 3072, 4, 2, 5, True, 0, False),
+    # Q2_K rows: the down projection through the specialised sweeps (gate and up rows of this
+    # format take the generic kernel), buckets past four pairs, one and four rows an iteration
+    ("Q2_K", 2048, 2048, 6, 4, 20, True, 1, False),
+    ("Q2_K", 4096, 3072, 4, 2, 5, True, 0, False),
     # many buckets: more sweeps than one wavefront lists (the class list is built by several)
     ("IQ2_XXS", 2048, 2048, 200, 8, 40, True, 1, False),
     # row-batch kernels on the matrix cores: tiny buckets, buckets past one 128-pair tile, real widths

@@ -863,7 +863,9 @@ static int dispatch_grouped(unsigned qtype, const GroupedArgs &a, bool q8, bool 
     }
     unsigned long long all_pairs = 0ull;
     for (unsigned i = 0; i < a.problems; ++i) all_pairs += a.problem[i].pairs;
-    if (q8 && aligned && iq2_sweep_supported(qtype, a.width, a.out_rows, all_pairs, a.image != 0))
+    // (Q2_K rows have the sweeps for a plain projection, the down experts, only)
+    if (q8 && aligned && !(qtype == QT_Q2_K && fused) &&
+        iq2_sweep_supported(qtype, a.width, a.out_rows, all_pairs, a.image != 0))
         return launch_iq2_sweep(a, qtype, fused, a.image != 0, stream);
     if (a.image) return ST_UNSUPPORTED;      // only the specialised sweeps read the image
     switch (qtype) {

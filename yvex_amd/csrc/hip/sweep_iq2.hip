@@ -332,6 +332,26 @@ struct Q4kHalf {
     }
 };
 
+// ---- Q2_K rows in the same sweeps (the down experts of the reference's model file) --------------
+//
+// A lane's share of one Q2_K weight row (public ggml block_q2_K, 84 bytes: sixteen bytes
+// scale | minimum << 4 of the 16-value sub-blocks, 64 bytes of 2-bit codes, fp16 d and dmin): the
+// 32 code bytes of its half (byte l holds the values 32 s + l of the half at bit 2 s), the half's
+// eight scale bytes and the dword of d and dmin. Superblocks are dword-aligned, not more.
+struct Q2kHalf {
+    uint4 q[2];
+    uint2 scales;
+    unsigned dd;
+    __device__ __forceinline__ void load(const unsigned char *rows, unsigned codes_at, unsigned scales_at,
+                                         unsigned dd_at)
+    {
+        q[0] = *reinterpret_cast<const uint4 *>(rows + codes_at);
+        q[1] = *reinterpret_cast<const uint4 *>(rows + codes_at + 16u);
+        scales = *reinterpret_cast<const uint2 *>(rows + scales_at);
+        dd = *reinterpret_cast<const unsigned *>(rows + dd_at);
+    }
+};
+
 template <unsigned QT>
 struct SweepHalf {
     using type = Iq2Half;
@@ -340,6 +360,56 @@ template <>
 struct SweepHalf<QT_Q4_K> {
     using type = Q4kHalf;
 };
+template <>
+struct SweepHalf<QT_Q2_K> {
+    using type = Q2kHalf;
+};
+
+// Exact integer sums of this lane's eight Q2_K sub-blocks of each of STREAMS weight rows against N
+// activation rows: dot = sum over sub-blocks of scale * (codes . activations), minimum = sum of
+// minimum * (sum of the sub-block's sixteen activations), the two terms of the reference's
+// primitive (src/backend/cuda/kernel_primitives.h:314-341). A code is a shift and a mask away.
+template <int STREAMS, int N>
+__device__ __forceinline__ void q2k_half_dots(const Q2kHalf (&c)[STREAMS], const unsigned (&act)[N][32],
+                                              const int (&act_sums)[N][8], int (&dot)[STREAMS][N],
+                                              int (&minimum)[STREAMS][N])
+{
+#pragma unroll
+    for (int w = 0; w < STREAMS; ++w) {
+        const unsigned packed[2] = {c[w].scales.x, c[w].scales.y};
+        const unsigned words[8] = {c[w].q[0].x, c[w].q[0].y, c[w].q[0].z, c[w].q[0].w,
+                                   c[w].q[1].x, c[w].q[1].y, c[w].q[1].z, c[w].q[1].w};
+#pragma unroll
+        for (int p = 0; p < N; ++p) {
+            int m = 0;
+#pragma unroll
+            for (int sub = 0; sub < 8; ++sub)       // 15 * 16 * 128 * 8 < 2^23
+                m += __mul24((int)((packed[sub >> 2] >> (8 * (sub & 3) + 4)) & 15u), act_sums[p][sub]);
+            minimum[w][p] = m;
+            dot[w][p] = 0;
+        }
+#pragma unroll
+        for (int shift = 0; shift < 4; ++shift) {
+            int first[N], second[N];     // sub-blocks 2 shift (bytes 0-15) and 2 shift + 1 (bytes 16-31)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const unsigned codes = (words[i] >> (2 * shift)) & 0x03030303u;
+#pragma unroll
+                for (int p = 0; p < N; ++p) {
+                    if (i < 4) first[p] = i == 0 ? dot4_from_zero(codes, act[p][8 * shift + i])
+                                                  : dot4(codes, act[p][8 * shift + i], first[p]);
+                    else second[p] = i == 4 ? dot4_from_zero(codes, act[p][8 * shift + i])
+                                            : dot4(codes, act[p][8 * shift + i], second[p]);
+                }
+            }
+            const int sc_first = (int)((packed[shift >> 1] >> (16 * (shift & 1))) & 15u);
+            const int sc_second = (int)((packed[shift >> 1] >> (16 * (shift & 1) + 8)) & 15u);
+#pragma unroll
+            for (int p = 0; p < N; ++p)   // |sum| <= 3 * 128 * 16 < 2^13
+                dot[w][p] += __mul24(first[p], sc_first) + __mul24(second[p], sc_second);
+        }
+    }
+}
 
 // Exact integer sums of this lane's four sub-blocks of each of STREAMS weight rows against N
 // activation rows: dot = sum over sub-blocks of scale * (nibbles . activations), minimum = sum of
@@ -403,8 +473,9 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 {
     constexpr bool FUSED = MODE == 1;
     constexpr bool TWIN = MODE != 0;     // two streams of weight rows against the same activation columns
-    constexpr bool Q4 = QT == QT_Q4_K;
-    static_assert(!(Q4 && IMAGE), "the image is a layout of IQ2_XXS rows");
+    constexpr bool Q4 = QT == QT_Q4_K, Q2 = QT == QT_Q2_K;
+    constexpr bool KQ = Q4 || Q2;        // formats with a minimum term
+    static_assert(!(KQ && IMAGE), "the image is a layout of IQ2_XXS rows");
     const unsigned lane = threadIdx.x & 63u;
     const bool odd = (lane & 1u) != 0u;
     // packed values per iteration: (first, second stream) of pair v with two streams, else pairs (2v, 2v + 1)
@@ -412,7 +483,8 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
 
     // ---- the sweep's activation rows: this lane's 128 columns stay in registers ----
     unsigned act[N][32];
-    int act_sums[N][Q4 ? 4 : 1];     // Q4_K: the sums of the activations under each of the lane's four sub-blocks
+    // the sums of the activations under each of the lane's sub-blocks: four of 32 (Q4_K), eight of 16 (Q2_K)
+    int act_sums[N][Q4 ? 4 : Q2 ? 8 : 1];
     float act_scale[N];
     float route_weight[N];
     unsigned long long out_index[N];
@@ -453,6 +525,14 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             for (int sub = 0; sub < 4; ++sub)
                 act_sums[p][sub] = g.live ? (int)(short)(pairs_of_sums[sub] & 0xffffu) + (int)(short)(pairs_of_sums[sub] >> 16)
                                           : 0;
+        } else if constexpr (Q2) {
+            uint4 sums;
+            __builtin_memcpy(&sums, blk + 260u + 16u * g.half, 16);
+            const unsigned pairs_of_sums[4] = {sums.x, sums.y, sums.z, sums.w};
+#pragma unroll
+            for (int sub = 0; sub < 8; ++sub)
+                act_sums[p][sub] = !g.live ? 0 : sub % 2 ? (int)pairs_of_sums[sub / 2] >> 16
+                                                         : (int)(short)(pairs_of_sums[sub / 2] & 0xffffu);
         } else {
             act_sums[p][0] = 0;
         }
@@ -479,20 +559,23 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned long long up_step = (unsigned long long)rows_per_turn * second_row_bytes;
     const unsigned lane_row = g.live ? g.sub : 0u, lane_super = g.live ? g.super : 0u;
     // (row bases and row strides are multiples of four bytes: checked on the host)
-    constexpr unsigned kSuperBytes = Q4 ? 144u : IMAGE ? 72u : 66u;
+    constexpr unsigned kSuperBytes = Q4 ? 144u : Q2 ? 84u : IMAGE ? 72u : 66u;
     const unsigned gate_block = lane_row * (unsigned)pr.row_bytes + lane_super * kSuperBytes;
     const unsigned up_block = lane_row * (unsigned)second_row_bytes + lane_super * kSuperBytes;
     // image: the lane's record is its first dword (scale and group scales) and eight more
     // (Q4_K: the half's 64 code bytes behind the 16-byte head, which is the "tail" load)
+    // (Q2_K: the half's 32 code bytes behind the sixteen scale bytes; "tail" is the half's eight scale bytes)
     const unsigned gate_codes_at = Q4 ? gate_block + 16u + 64u * g.half
+        : Q2 ? gate_block + 16u + 32u * g.half
         : IMAGE ? gate_block + 36u * g.half + 4u
                 : (gate_block + 2u + 32u * g.half) & ~3u;   // + code_shift = codes
     const unsigned up_codes_at = Q4 ? up_block + 16u + 64u * g.half
+        : Q2 ? up_block + 16u + 32u * g.half
         : IMAGE ? up_block + 36u * g.half + 4u : (up_block + 2u + 32u * g.half) & ~3u;
     // ninth dword: the end of the codes where they start two bytes in, else the scale's dword
-    const unsigned gate_tail_at = Q4 ? gate_block : IMAGE ? gate_codes_at - 4u
+    const unsigned gate_tail_at = Q4 ? gate_block : Q2 ? gate_block + 8u * g.half : IMAGE ? gate_codes_at - 4u
                                         : g.code_shift ? gate_codes_at + 32u : gate_block & ~3u;
-    const unsigned up_tail_at = Q4 ? up_block
+    const unsigned up_tail_at = Q4 ? up_block : Q2 ? up_block + 8u * g.half
         : IMAGE ? up_codes_at - 4u : g.code_shift ? up_codes_at + 32u : up_block & ~3u;
     // Ring of packed rows: the bytes of iteration it + AHEAD are requested before iteration it is
     // decoded, so about AHEAD iterations of arithmetic cover the HBM latency.
@@ -506,9 +589,15 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
     const unsigned last = iterations - 1u;
     auto request = [&](Half (&slot)[STREAMS], unsigned it) {
         const unsigned clamped = it < last ? it : last;
-        slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at);
-        if constexpr (TWIN)
-            slot[1].load(up_rows + clamped * up_step, up_codes_at, up_tail_at);
+        if constexpr (Q2) {
+            slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at, gate_block + 80u);
+            if constexpr (TWIN)
+                slot[1].load(up_rows + clamped * up_step, up_codes_at, up_tail_at, up_block + 80u);
+        } else {
+            slot[0].load(gate_rows + clamped * gate_step, gate_codes_at, gate_tail_at);
+            if constexpr (TWIN)
+                slot[1].load(up_rows + clamped * up_step, up_codes_at, up_tail_at);
+        }
     };
     // The first requests are kept in ring order: the loop's first wait is counted against the
     // loads issued after the slot it consumes, on the entry path and on the back edge alike.
@@ -590,6 +679,8 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             int totals[STREAMS][N], minimums[STREAMS][N];
             if constexpr (Q4) {
                 q4k_half_dots<STREAMS, N>(now, g, act, act_sums, totals, minimums);
+            } else if constexpr (Q2) {
+                q2k_half_dots<STREAMS, N>(now, act, act_sums, totals, minimums);
             } else {
                 iq2_half_dots<STREAMS, N, IMAGE>(now, g, act, totals);
 #pragma unroll
@@ -610,7 +701,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         for (int p = 0; p < N; ++p) {
             total_gate[p] += dpp_move<0xb1, 0xf>(total_gate[p]);
             if constexpr (TWIN) total_up[p] += dpp_move<0xb1, 0xf>(total_up[p]);
-            if constexpr (Q4) {
+            if constexpr (KQ) {
                 min_gate[p] += dpp_move<0xb1, 0xf>(min_gate[p]);
                 if constexpr (TWIN) min_up[p] += dpp_move<0xb1, 0xf>(min_up[p]);
             }
@@ -623,6 +714,9 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
         if constexpr (Q4) {
             weight_scale = f16_bits_to_float(mine.head.x & 0xffffu);       // d
             weight_minimum = f16_bits_to_float(mine.head.x >> 16);         // dmin
+        } else if constexpr (Q2) {
+            weight_scale = f16_bits_to_float(mine.dd & 0xffffu);
+            weight_minimum = f16_bits_to_float(mine.dd >> 16);
         } else if constexpr (IMAGE) {
             weight_scale = 0.125f * f16_bits_to_float(mine.tail & 0xffffu);
         } else {
@@ -638,7 +732,7 @@ __device__ __forceinline__ void iq2_sweep(const GroupedArgs &a, const GroupedPro
             if constexpr (TWIN) t = odd ? total_up[v] : total_gate[v];
             else t = odd ? total_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : total_gate[2 * v];
             float value;
-            if constexpr (Q4) {
+            if constexpr (KQ) {
                 if constexpr (TWIN) m = odd ? min_up[v] : min_gate[v];
                 else m = odd ? min_gate[2 * v + 1 < N ? 2 * v + 1 : 2 * v] : min_gate[2 * v];
                 // (d_a d) dot - (d_a dmin) minimum, each product rounded: the order of the reference's primitive
@@ -934,12 +1028,12 @@ __global__ __launch_bounds__(kSweepThreads) void iq2_sweep_kernel(GroupedArgs a)
 
 bool iq2_sweep_supported(unsigned qtype, unsigned width, unsigned out_rows, unsigned long long pairs, bool image)
 {
-    if (qtype != QT_IQ2_XXS && qtype != QT_Q4_K) return false;
+    if (qtype != QT_IQ2_XXS && qtype != QT_Q4_K && qtype != QT_Q2_K) return false;
     if (image && qtype != QT_IQ2_XXS) return false;
     if (pairs > kClassMaxSweeps) return false;            // every sweep serves at least one pair
     const unsigned lanes_per_row = width / 128u;
     if (width % 256u != 0u || lanes_per_row < 16u || lanes_per_row > 64u) return false;
-    // IQ2_XXS rows must start on dword boundaries (Q4_K rows are multiples of 144 bytes)
+    // IQ2_XXS rows must start on dword boundaries (Q4_K rows are multiples of 144 bytes, Q2_K rows of 84)
     if (qtype == QT_IQ2_XXS && !image && (width / 256u * 66u) % 4u != 0u) return false;
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u
         ? 64u / lanes_per_row : 1u;
@@ -970,6 +1064,11 @@ int launch_iq2_sweep(const GroupedArgs &a, unsigned qtype, bool fused, bool imag
     const unsigned rows_per_iter = lanes_per_row % 16u == 0u && 64u % lanes_per_row == 0u ? 64u / lanes_per_row : 1u;
     const int mode = fused ? 1 : a.out_rows % (2u * rows_per_iter) == 0u ? 2 : 0;
     if (qtype == QT_Q4_K) return image ? ST_UNSUPPORTED : launch_iq2_sweep_mode<false, QT_Q4_K>(a, mode, stream);
+    if (qtype == QT_Q2_K) {      // the down experts: a plain projection
+        if (image || fused) return ST_UNSUPPORTED;
+        return mode == 2 ? launch_iq2_sweep_variant<2, false, QT_Q2_K>(a, stream)
+                         : launch_iq2_sweep_variant<0, false, QT_Q2_K>(a, stream);
+    }
     if (qtype != QT_IQ2_XXS) return ST_UNSUPPORTED;
     return image ? launch_iq2_sweep_mode<true, QT_IQ2_XXS>(a, mode, stream)
                  : launch_iq2_sweep_mode<false, QT_IQ2_XXS>(a, mode, stream);
