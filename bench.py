@@ -11,7 +11,8 @@ Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up 
 with events on the launch stream; `cpu_baseline` is the reference's own CPU expert path
 (compiled from its sources; the C restatement beside it) timed on the host cores over a bounded
 sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8 matrix
-cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `decode_envelope` the
+cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `q2k_down` both batches
+with the reference's own pairing of IQ2_XXS gate/up and Q2_K down experts, `decode_envelope` the
 headline step with four residual streams around the layer, `decode_small_batches` the headline
 layer at 1 to 16 rows, and `dense` configs
 0-2 and an output head as single matvec launches; the prefill legs and the dense configs carry a
@@ -489,6 +490,52 @@ def decode_q4k_leg(torch, K, weights, shared, dev, steps: int, warmup: int):
             "hbm_peak_frac": round(read / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def synth_q2k(torch, blocks: int, device, seed: int):
+    """Q2_K superblocks (84 bytes): random scale/minimum bytes and 2-bit codes, small positive fp16
+    d and dmin behind them."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 84), dtype=torch.uint8, device=device, generator=gen)
+    scales = (torch.rand((blocks, 2), device=device, generator=gen) * 1e-3 + 1e-4).to(torch.float16)
+    raw[:, 80:84] = scales.view(torch.uint8).reshape(-1, 4)
+    return raw.reshape(-1)
+
+
+def q2k_down_leg(torch, gate, up, shared, dev, steps: int, warmup: int):
+    """The pairing of the reference's model file (IQ2_XXS gate and up experts, Q2_K down experts:
+    src/backend/cuda/tensorcore.cu:563-564, 660) through the C ABI over canonical bytes: the
+    headline batch of 32 rows (decode sweeps) and 2048 rows (matrix cores). Bytes counted: the
+    canonical bytes of the distinct experts hit."""
+    from yvex_amd.host import RowBatchLayer
+    blocks = INTERMEDIATE * HIDDEN // 256
+    down = synth_q2k(torch, EXPERTS * blocks, dev, 41)
+    shared_down = synth_q2k(torch, blocks, dev, 42)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(78)
+    router = (torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5).contiguous()
+    out = {"workload": "IQ2_XXS gate/up experts with Q2_K down experts, top-8 of 256 + shared, Q8_K activations, "
+                       "canonical bytes"}
+    for rows, count in ((ROWS, steps), (2048, max(3, steps // 10))):
+        x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
+        layer = RowBatchLayer(torch, (gate, up, down), (shared[0], shared[1], shared_down), router, x.cpu().numpy(),
+                              rows, hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
+                              qtype=16, down_qtype=10)
+        layer.step(defer=False)
+        unique = int(layer.result.unique_experts)
+        matrix = int(layer.result.tensor_core_launches)
+        ms = min(layer.timed(count, max(warmup, 2)), layer.timed(count, warmup, eager=True))
+        layer.close()
+        read = (unique + 1) * blocks * (2 * 66 + 84)
+        leg = {"ms_per_step": round(ms, 4), "distinct_routed_experts": unique, "matrix_core_launches": matrix,
+               "GB_per_s": round(read / (ms * 1e-3) / 1e9, 1)}
+        if rows > ROWS:
+            ops = 2 * 3 * INTERMEDIATE * HIDDEN * rows * (TOPK + 1)
+            leg["int8_TOPs"] = round(ops / (ms * 1e-3) / 1e12, 2)
+            leg["tokens_per_s"] = round(rows / (ms * 1e-3), 1)
+        out[f"rows_{rows}"] = leg
+    return out
+
+
 def envelope_leg(torch, routed, shared, router, dev, steps: int, warmup: int):
     """The headline step for a layer with residual streams around it (four streams of 7168, 24
     mixing rows, 20 Sinkhorn iterations; src/backend/cuda/moe.c:1210-1254, 1533-1541), through the
@@ -819,6 +866,7 @@ def main() -> int:
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)
+        out["q2k_down"] = q2k_down_leg(torch, gate, up, shared, dev, args.steps, args.warmup)
     if not args.no_prefill:
         # config 4's second weight format: the same layer with Q4_K experts (6.3 GB of them)
         del layer, gate, up, down, shared
