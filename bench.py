@@ -503,9 +503,10 @@ def synth_q2k(torch, blocks: int, device, seed: int):
 
 def q2k_down_leg(torch, gate, up, shared, dev, steps: int, warmup: int):
     """The pairing of the reference's model file (IQ2_XXS gate and up experts, Q2_K down experts:
-    src/backend/cuda/tensorcore.cu:563-564, 660) through the C ABI over canonical bytes: the
-    headline batch of 32 rows (decode sweeps) and 2048 rows (matrix cores). Bytes counted: the
-    canonical bytes of the distinct experts hit."""
+    src/backend/cuda/tensorcore.cu:563-564, 660) through the C ABI, gate and up experts resident as
+    the sweeps' image and the down experts as canonical rows (they have no image): the headline
+    batch of 32 rows (decode sweeps) and 2048 rows (matrix cores). Bytes counted: the canonical
+    bytes of the distinct experts hit."""
     from yvex_amd.host import RowBatchLayer
     blocks = INTERMEDIATE * HIDDEN // 256
     down = synth_q2k(torch, EXPERTS * blocks, dev, 41)
@@ -513,13 +514,13 @@ def q2k_down_leg(torch, gate, up, shared, dev, steps: int, warmup: int):
     gen = torch.Generator(device=dev)
     gen.manual_seed(78)
     router = (torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5).contiguous()
-    out = {"workload": "IQ2_XXS gate/up experts with Q2_K down experts, top-8 of 256 + shared, Q8_K activations, "
-                       "canonical bytes"}
+    out = {"workload": "IQ2_XXS gate/up experts (sweep image) with Q2_K down experts (canonical rows), top-8 of "
+                       "256 + shared, Q8_K activations"}
     for rows, count in ((ROWS, steps), (2048, max(3, steps // 10))):
         x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
         layer = RowBatchLayer(torch, (gate, up, down), (shared[0], shared[1], shared_down), router, x.cpu().numpy(),
                               rows, hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
-                              qtype=16, down_qtype=10)
+                              qtype=16, down_qtype=10, sweep_image=True)
         layer.step(defer=False)
         unique = int(layer.result.unique_experts)
         matrix = int(layer.result.tensor_core_launches)

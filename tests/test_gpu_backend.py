@@ -369,6 +369,8 @@ class MoeCase:
                 continue
             for name in names:
                 down = name.endswith("down")
+                if down and qt_down != oracle.IQ2_XXS:
+                    continue        # (down rows of another format are read as they lie)
                 decision = sweep_image_decision(
                     1 if group == "shared" else experts, (hidden if down else intermediate) * (1 if group == "shared" else experts),
                     intermediate if down else hidden,
@@ -584,17 +586,22 @@ def test_execute_rows_hash_router(backend, oracle, streams):
     case.tokens[2] = 1
 
 
-@pytest.mark.parametrize("qtype,hidden,intermediate,experts,topk,rows", [
-    ("IQ2_XXS", 2048, 2048, 16, 4, 20),     # four rows an iteration, buckets past four pairs (two sweeps)
-    ("IQ2_XXS", 4096, 3072, 4, 2, 5),       # 24 lanes a row: one row an iteration
-    ("Q4_K", 2048, 4096, 5, 2, 3),          # 32 lanes a row: two rows an iteration
-    ("IQ2_XXS", 7168, 2048, 12, 4, 6)])     # the benchmark layer's widths
-def test_execute_rows_with_q2k_down_experts(backend, oracle, qtype, hidden, intermediate, experts, topk, rows):
+@pytest.mark.parametrize("qtype,hidden,intermediate,experts,topk,rows,image", [
+    ("IQ2_XXS", 2048, 2048, 16, 4, 20, ()),    # four rows an iteration, buckets past four pairs (two sweeps)
+    ("IQ2_XXS", 4096, 3072, 4, 2, 5, ()),      # 24 lanes a row: one row an iteration
+    ("Q4_K", 2048, 4096, 5, 2, 3, ()),         # 32 lanes a row: two rows an iteration
+    ("IQ2_XXS", 7168, 2048, 12, 4, 6, ()),     # the benchmark layer's widths
+    # gate and up rows as the sweeps' image beside canonical Q2_K down rows, which have no image:
+    # the one pairing of layouts that need not agree; decode width and matrix-core width
+    ("IQ2_XXS", 2048, 2048, 16, 4, 20, ("routed", "shared")),
+    ("IQ2_XXS", 2048, 2048, 4, 2, 60, ("routed", "shared"))])
+def test_execute_rows_with_q2k_down_experts(backend, oracle, qtype, hidden, intermediate, experts, topk, rows,
+                                            image):
     """The pairing of the reference's model file, IQ2_XXS gate and up experts with Q2_K down
     experts (src/backend/cuda/tensorcore.cu:563-564, 660), at decode width: the down projection
     runs the specialised sweeps over Q2_K rows, and the result is the CPU layer's bit for bit."""
     case = MoeCase(backend, oracle, qtype=qtype, down_qtype="Q2_K", hidden=hidden, intermediate=intermediate,
-                   experts=experts, topk=topk, rows=rows, scoring=abi.SCORING_SIGMOID)
+                   experts=experts, topk=topk, rows=rows, scoring=abi.SCORING_SIGMOID, sweep_image=image)
     backend.workspace(case.workspace_bytes)
     rc = case.execute()
     assert rc == 0, case.err.message
@@ -602,7 +609,7 @@ def test_execute_rows_with_q2k_down_experts(backend, oracle, qtype, hidden, inte
     assert np.array_equal(case.sel.reshape(case.rows, case.topk), want["selected"])
     got = backend.read_f32(case.rows_out, case.rows * case.hidden).reshape(case.rows, case.hidden)
     same_as_cpu(got, want["combined"])
-    assert case.result.completed == 1 and case.result.tensor_core_launches == 0
+    assert case.result.completed == 1 and (case.result.tensor_core_launches > 0) == (rows == 60)
 
 
 @pytest.mark.parametrize("qtype,down_qtype", [("IQ2_XXS", None), ("Q4_K", None), ("IQ2_XXS", "Q2_K"),

@@ -176,20 +176,27 @@ static int expert_policy(const yvex_moe_weight_view *gate, const yvex_moe_weight
      * derived image at all (UNSUPPORTED); this one executes the one image its expert sweeps
      * read: IQ2_XXS tensors, device-encoded activations, the gfx950 sweep family on all three
      * views. Any other derived view is refused as there. */
-    if (gate->layout != up->layout || ((gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND) !=
-                                       (down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND)))
-        return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
-                                "compiled routed MoE layouts disagree");
-    if (gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND) {
-        if (!gate_encoded || !down_encoded || !down->kernel_family ||
-            strcmp(gate->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
-            strcmp(down->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
-            gate->qtype != YVEX_GGUF_QTYPE_IQ2_XXS || up->qtype != YVEX_GGUF_QTYPE_IQ2_XXS ||
-            down->qtype != YVEX_GGUF_QTYPE_IQ2_XXS)
-            return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
-                                    "the row-batch path executes canonical rows, or the expert sweeps' "
-                                    "image of IQ2_XXS tensors with device-encoded activations");
-        *image = 1;
+    /* One exception to the agreement: Q2_K down rows have no image (the sweeps read them as they
+     * lie), so canonical Q2_K down rows beside imaged IQ2_XXS gate and up rows are admitted, the
+     * pairing of the reference's model file. *image: bit 0 gate and up, bit 1 down. */
+    {
+        const int gate_derived = gate->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND;
+        const int down_derived = down->layout == YVEX_EXECUTION_LAYOUT_DERIVED_BACKEND;
+        const int q2k_down_as_it_lies = gate_derived && !down_derived && down->qtype == YVEX_GGUF_QTYPE_Q2_K;
+        if (gate->layout != up->layout || (gate_derived != down_derived && !q2k_down_as_it_lies))
+            return yvex_rocm_refuse(err, YVEX_ERR_FORMAT, "rocm.moe.policy",
+                                    "compiled routed MoE layouts disagree");
+        if (gate_derived) {
+            if (!gate_encoded || !down_encoded || !down->kernel_family ||
+                strcmp(gate->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
+                strcmp(down->kernel_family, YVEX_MOE_KERNEL_GFX950_EXPERT_SWEEP) != 0 ||
+                gate->qtype != YVEX_GGUF_QTYPE_IQ2_XXS || up->qtype != YVEX_GGUF_QTYPE_IQ2_XXS ||
+                (down_derived && down->qtype != YVEX_GGUF_QTYPE_IQ2_XXS))
+                return yvex_rocm_refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.moe.policy",
+                                        "the row-batch path executes canonical rows, or the expert sweeps' "
+                                        "image of IQ2_XXS tensors with device-encoded activations");
+            *image = down_derived ? 3 : 1;
+        }
     }
     if ((gate_encoded && !family_admitted(gate->kernel_family)) ||
         (down_encoded && !family_admitted(down->kernel_family)))
@@ -295,9 +302,10 @@ static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weigh
                                 unsigned long long down_address, unsigned long long hidden,
                                 unsigned long long intermediate, int image)
 {
-    const unsigned long long gate_row = image ? hidden / 256ull * 72ull : gate->row_bytes;
-    const unsigned long long up_row = image ? hidden / 256ull * 72ull : up->row_bytes;
-    const unsigned long long down_row = image ? intermediate / 256ull * 72ull : down->row_bytes;
+    /* image: bit 0 the gate and up matrices, bit 1 the down matrix */
+    const unsigned long long gate_row = (image & 1) ? hidden / 256ull * 72ull : gate->row_bytes;
+    const unsigned long long up_row = (image & 1) ? hidden / 256ull * 72ull : up->row_bytes;
+    const unsigned long long down_row = (image & 2) ? intermediate / 256ull * 72ull : down->row_bytes;
     w->gate = (const uint8_t *)(uintptr_t)gate_address;
     w->up = (const uint8_t *)(uintptr_t)up_address;
     w->down = (const uint8_t *)(uintptr_t)down_address;
@@ -312,7 +320,8 @@ static void fill_expert_weights(yvex_hip_expert_weights *w, const yvex_moe_weigh
     w->gate_expert_bytes = gate_row * intermediate;
     w->up_expert_bytes = up_row * intermediate;
     w->down_expert_bytes = down_row * hidden;
-    w->gate_up_image = w->down_image = image;
+    w->gate_up_image = image & 1;
+    w->down_image = (image >> 1) & 1;
 }
 
 /* Expert weights the matrix-core row-batch kernels take: gate and up of one format, IQ2_XXS (16)
@@ -614,22 +623,22 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
                                   "MoE hash table holds fewer rows than the plan names");
     }
     if (rc == YVEX_OK)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], routed_image, hidden,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_GATE], routed_image & 1, hidden,
                                  experts * layer->expert_intermediate_width, &addresses[0], err);
     if (rc == YVEX_OK)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_UP], routed_image, hidden,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_UP], routed_image & 1, hidden,
                                  experts * layer->expert_intermediate_width, &addresses[1], err);
     if (rc == YVEX_OK)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], routed_image,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_ROUTED_DOWN], (routed_image >> 1) & 1,
                                  layer->expert_intermediate_width, experts * hidden, &addresses[2], err);
     if (rc == YVEX_OK && has_shared)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_GATE], shared_image, hidden,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_GATE], shared_image & 1, hidden,
                                  layer->shared_intermediate_width, &addresses[3], err);
     if (rc == YVEX_OK && has_shared)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_UP], shared_image, hidden,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_UP], shared_image & 1, hidden,
                                  layer->shared_intermediate_width, &addresses[4], err);
     if (rc == YVEX_OK && has_shared)
-        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], shared_image,
+        rc = expert_view_resolve(backend, &views[YVEX_MOE_WEIGHT_SHARED_DOWN], (shared_image >> 1) & 1,
                                  layer->shared_intermediate_width, hidden, &addresses[5], err);
     if (rc == YVEX_OK && envelope) {
         /* ingress coefficients: the mixing function is a matrix over the expanded row, the rest

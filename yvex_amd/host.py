@@ -145,7 +145,7 @@ class RowBatchLayer:
             v.device_address = tensor.data_ptr()
             v.encoded_bytes = v.storage_bytes = tensor.numel() * tensor.element_size()
             v.row_bytes, v.row_width, v.row_count = row_bytes, width, count
-            if sweep_image and consumer is not None:
+            if sweep_image and consumer is not None and qtype == 16:     # (only IQ2_XXS tensors have an image)
                 # the residency step of a caller that keeps its experts as the decode sweeps' image:
                 # plan, allocate, build on the device from the resident canonical bytes
                 d = abi.ExecutionDecision()
