@@ -729,7 +729,9 @@ typedef struct {
  * 7-bit sign fields, one to a byte}. The reference's row-batch path refuses every
  * DERIVED_BACKEND view (moe.c:939-958); execute_rows here runs that one image (IQ2_XXS,
  * device-encoded activations, the sweep family on gate, up and down) on the decode sweeps and on
- * the matrix-core kernels, and answers UNSUPPORTED for any other derived view. */
+ * the matrix-core kernels, and answers UNSUPPORTED for any other derived view. Q2_K down rows
+ * have no image: canonical Q2_K down rows beside imaged IQ2_XXS gate and up rows are admitted,
+ * the one pairing of layouts that need not agree. */
 typedef struct {
     int (*derived_layout_plan)(const yvex_physical_execution_decision *decision,
                                unsigned long long *storage_bytes, yvex_error *err);
