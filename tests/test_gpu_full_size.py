@@ -219,8 +219,21 @@ def router_weights(device, seed):
     return torch.randn((EXPERTS, HIDDEN), device=device, generator=gen) * HIDDEN ** -0.5
 
 
+def synthetic_q2k(blocks, device, seed):
+    """Q2_K superblocks (84 bytes): random scale | minimum << 4 bytes and 2-bit codes, small positive
+    fp16 d and dmin behind them."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 84), dtype=torch.uint8, device=device, generator=gen)
+    scales = (torch.rand((blocks, 2), device=device, generator=gen) * 1e-3 + 1e-4).to(torch.float16)
+    raw[:, 80:84] = scales.view(torch.uint8).reshape(-1, 4)
+    return raw.reshape(-1)
+
+
 @pytest.mark.parametrize("rows,qtype,sweep_image", [(32, "IQ2_XXS", False), (32, "IQ2_XXS", True),
-                                                    (2048, "IQ2_XXS", False), (2048, "Q4_K", False)])
+                                                    (2048, "IQ2_XXS", False), (2048, "Q4_K", False),
+                                                    # the pairing of the reference's model file: Q2_K down experts
+                                                    (32, "IQ2_XXS+Q2_K", True), (2048, "IQ2_XXS+Q2_K", False)])
 def test_execute_rows_at_full_size_equals_the_cpu_layer(gpu, oracle, layer_weights, rows, qtype, sweep_image):
     """BASELINE configs 3 and 4 through yvex_rocm_backend_moe_operations_get()->execute_rows and
     complete_rows (the reference's row-batch entry, src/backend/cuda/moe.c:1826-1958), router
@@ -232,8 +245,14 @@ def test_execute_rows_at_full_size_equals_the_cpu_layer(gpu, oracle, layer_weigh
     from yvex_amd import abi
     from yvex_amd import kernels as K
     from yvex_amd.host import RowBatchLayer
+    down_qtype = None
     if qtype == "IQ2_XXS":
         routed, shared = layer_weights
+    elif qtype == "IQ2_XXS+Q2_K":
+        qtype, down_qtype = "IQ2_XXS", "Q2_K"
+        routed, shared = layer_weights
+        routed = routed[:2] + (synthetic_q2k(EXPERTS * INTERMEDIATE * HIDDEN // 256, gpu, 41),)
+        shared = shared[:2] + (synthetic_q2k(INTERMEDIATE * HIDDEN // 256, gpu, 42),)
     else:
         blocks = EXPERTS * INTERMEDIATE * HIDDEN // 256
         routed = tuple(synthetic_q4k(blocks, gpu, 21 + i) for i in range(3))
@@ -244,7 +263,8 @@ def test_execute_rows_at_full_size_equals_the_cpu_layer(gpu, oracle, layer_weigh
     router = router_weights(gpu, 5)
     qt = getattr(K, qtype)
     layer = RowBatchLayer(torch, routed, shared, router, x.cpu().numpy(), rows, hidden=HIDDEN,
-                          intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtype=qt, sweep_image=sweep_image)
+                          intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK, qtype=qt, sweep_image=sweep_image,
+                          down_qtype=getattr(K, down_qtype) if down_qtype else None)
     try:
         layer.step(defer=True)
         layer.complete()
@@ -262,9 +282,11 @@ def test_execute_rows_at_full_size_equals_the_cpu_layer(gpu, oracle, layer_weigh
     host_x = x[picked].cpu().numpy()
     logits = oracle.matvec(oracle.F32, router.cpu().numpy().view(np.uint8).reshape(-1), EXPERTS, HIDDEN, host_x)
     want = oracle.moe_layer(hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
-                            qtypes=(getattr(oracle, qtype),) * 3, routed=[t.cpu().numpy() for t in routed],
+                            qtypes=(getattr(oracle, qtype),) * 2 + (getattr(oracle, down_qtype or qtype),),
+                            routed=[t.cpu().numpy() for t in routed],
                             shared=[t.cpu().numpy() for t in shared], inputs=host_x, logits=logits,
                             scoring=oracle.SIGMOID, normalize=True, scaling=1.0, limit=10.0, act_q8=True,
                             threads=16)
     equal_to_oracle(first[picked], want["combined"],
-                    f"execute_rows, {rows} rows, {qtype}{' (sweep image)' if sweep_image else ''}: picked rows against the oracle")
+                    f"execute_rows, {rows} rows, {qtype}{' + Q2_K down' if down_qtype else ''}"
+                    f"{' (sweep image)' if sweep_image else ''}: picked rows against the oracle")
