@@ -91,7 +91,11 @@ def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     ("F16", 300, 4096, 1), ("BF16", 70, 7168, 1), ("F16", 33, 1000, 2), ("BF16", 9, 264, 5), ("F16", 5, 8, 7),
     ("F16", 4100, 264, 1), ("BF16", 4097, 136, 3),      # many rows: a wave a row
     ("BF16", 40, 100, 3),       # rows that are not whole 16-byte pieces: the lane-strided kernel
-    ("F16", 12, 512, 9), ("BF16", 40, 1024, 70)])       # eight input rows and more
+    # eight input rows and more: the double-precision matrix cores (sixteen waves a tile, four
+    # waves a tile from 256 input rows, staged blocks once there is one a compute unit); a row
+    # width they do not take stays on the kernel above
+    ("F16", 12, 512, 9), ("BF16", 40, 1024, 70), ("BF16", 70, 512, 300), ("F16", 1030, 256, 520),
+    ("BF16", 2100, 128, 1000), ("F16", 20, 264, 30)])
 def test_matvec_sixteen_bit_weights(gpu, oracle, qtype, rows, width, inputs):
     """F16 and BF16 weight rows against F32 input rows (projections and output heads kept in
     16-bit floats; src/gguf/quant_compute.c:152-172 forms double products and a double sum):

@@ -538,7 +538,24 @@ static int launch_scalar_few(const MatvecArgs &a, hipStream_t s)
 // its serial loop, so the float the sum rounds to is the CPU path's. The partial tiles of the
 // waves (and of the workgroups that split the width: blockIdx.z, joined by a second launch in
 // split order) are doubles, added in a fixed order.
-template <unsigned WAVES>
+// Four consecutive weights of a row of F32, F16 or BF16 values as floats (exact conversions).
+template <unsigned QT>
+__device__ __forceinline__ float4 scalar_weights4(const unsigned char *row, unsigned long long column)
+{
+    if constexpr (QT == QT_F32) {
+        return *reinterpret_cast<const float4 *>(row + 4ull * column);
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(row + 2ull * column);
+        if constexpr (QT == QT_F16)
+            return make_float4(f16_bits_to_float(v.x & 0xffffu), f16_bits_to_float(v.x >> 16),
+                               f16_bits_to_float(v.y & 0xffffu), f16_bits_to_float(v.y >> 16));
+        else
+            return make_float4(bf16_bits_to_float(v.x & 0xffffu), bf16_bits_to_float(v.x >> 16),
+                               bf16_bits_to_float(v.y & 0xffffu), bf16_bits_to_float(v.y >> 16));
+    }
+}
+
+template <unsigned WAVES, unsigned QT = QT_F32>
 __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArgs a)
 {
     typedef double v4d __attribute__((ext_vector_type(4)));
@@ -551,7 +568,7 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
     if (in >= a.input_rows) in = a.input_rows - 1ull;
     const unsigned long long share = a.row_width / ((unsigned long long)gridDim.z * WAVES);   // a multiple of 16
     const unsigned long long begin = ((unsigned long long)blockIdx.z * WAVES + wave) * share + 4u * q;
-    const float *wp = (const float *)(a.encoded + wrow * a.row_bytes) + begin;
+    const unsigned char *wp = a.encoded + wrow * a.row_bytes;       // columns from `begin` on
     const float *xp = (const float *)a.input + in * a.input_stride + begin;
     const unsigned steps = (unsigned)(share / 16ull);
     v4d acc = {0.0, 0.0, 0.0, 0.0};
@@ -562,7 +579,7 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
 #pragma unroll
     for (unsigned j = 0; j < 4u; ++j) {
         const unsigned at = 16u * (j < steps ? j : steps - 1u);
-        w[j] = *reinterpret_cast<const float4 *>(wp + at);
+        w[j] = scalar_weights4<QT>(wp, begin + at);
         x[j] = *reinterpret_cast<const float4 *>(xp + at);
     }
     for (unsigned group = 0; group < groups; ++group) {
@@ -572,7 +589,7 @@ __global__ __launch_bounds__(WAVES * 64) void matvec_f32_tile16_kernel(MatvecArg
             for (unsigned j = 0; j < 4u; ++j) {
                 const unsigned step = 4u * (group + 1u) + j;
                 const unsigned at = 16u * (step < steps ? step : steps - 1u);
-                wn[j] = *reinterpret_cast<const float4 *>(wp + at);
+                wn[j] = scalar_weights4<QT>(wp, begin + at);
                 xn[j] = *reinterpret_cast<const float4 *>(xp + at);
             }
         }
@@ -629,6 +646,7 @@ constexpr unsigned kF32BlockColumns = 128u, kF32BlockPitch = kF32BlockColumns * 
 constexpr unsigned kF32BlockWeightRows = 32u, kF32BlockInputRows = 64u;
 constexpr unsigned kF32BlockLdsBytes = 2u * (kF32BlockWeightRows + kF32BlockInputRows) * kF32BlockPitch;
 
+template <unsigned QT>
 __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
 {
     typedef double v4d __attribute__((ext_vector_type(4)));
@@ -641,7 +659,7 @@ __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
     const unsigned i16 = lane & 15u, q = lane >> 4;
     // staging: piece p = threadIdx.x + 512 j of the chunk is columns 4 (p % 32) .. + 3 of staged
     // row p / 32 (weight rows first, then input rows); 32 lanes read one row's 512 bytes
-    const float *source[kHeld];
+    const unsigned char *source[kHeld];       // (weight rows: F32, F16 or BF16 values; input rows: F32)
     unsigned target[kHeld];
 #pragma unroll
     for (unsigned j = 0; j < kHeld; ++j) {
@@ -649,19 +667,27 @@ __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
         if (row < kF32BlockWeightRows) {
             unsigned long long wrow = (unsigned long long)blockIdx.x * kF32BlockWeightRows + row;
             if (wrow >= a.row_count) wrow = a.row_count - 1ull;          // a ragged edge repeats the last row
-            source[j] = (const float *)(a.encoded + wrow * a.row_bytes) + 4u * piece;
+            source[j] = a.encoded + wrow * a.row_bytes + (QT == QT_F32 ? 16u : 8u) * piece;
         } else {
             unsigned long long in = (unsigned long long)blockIdx.y * kF32BlockInputRows + (row - kF32BlockWeightRows);
             if (in >= a.input_rows) in = a.input_rows - 1ull;
-            source[j] = (const float *)a.input + in * a.input_stride + 4u * piece;
+            source[j] = (const unsigned char *)((const float *)a.input + in * a.input_stride + 4u * piece);
         }
         target[j] = row * kF32BlockPitch + 16u * piece;
     }
     const unsigned chunks = (unsigned)(a.row_width / kF32BlockColumns);
     v4f held[kHeld];
     unsigned bad = 0u;
+    // piece j of this thread is a piece of a weight row for the first two j, of an input row after
+    auto fetch = [&](unsigned j, unsigned chunk) -> v4f {
+        if (512u * (j + 1u) <= kF32BlockWeightRows * kPieces) {
+            const float4 w = scalar_weights4<QT>(source[j], (unsigned long long)chunk * kF32BlockColumns);
+            return v4f{w.x, w.y, w.z, w.w};
+        }
+        return *reinterpret_cast<const v4f *>(source[j] + (unsigned long long)chunk * kF32BlockColumns * 4ull);
+    };
 #pragma unroll
-    for (unsigned j = 0; j < kHeld; ++j) held[j] = *reinterpret_cast<const v4f *>(source[j]);
+    for (unsigned j = 0; j < kHeld; ++j) held[j] = fetch(j, 0u);
 #pragma unroll
     for (unsigned j = 0; j < kHeld; ++j) {
         if (512u * (j + 1u) <= kF32BlockWeightRows * kPieces)
@@ -679,7 +705,7 @@ __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
         const unsigned ahead = chunk + 1u < chunks ? chunk + 1u : chunk;
 #pragma unroll
         for (unsigned j = 0; j < kHeld; ++j)
-            held[j] = *reinterpret_cast<const v4f *>(source[j] + (unsigned long long)ahead * kF32BlockColumns);
+            held[j] = fetch(j, ahead);
         const unsigned char *now = staged + (chunk & 1u) * (kRows * kF32BlockPitch);
         unsigned char *next = staged + ((chunk + 1u) & 1u) * (kRows * kF32BlockPitch);
 #pragma unroll
@@ -916,6 +942,33 @@ static int launch_block_q(const MatvecArgs &a, bool q8, hipStream_t stream)
 
 using namespace yvex;
 
+// Rows of F32, F16 or BF16 values against eight or more F32 input rows: 16 x 16 tiles on the
+// double-precision matrix cores; a small batch offers few tiles, so sixteen waves split the row
+// width, a large one has tiles enough for four, or for the staged kernel.
+template <unsigned QT>
+static int launch_scalar_rows(const MatvecArgs &a, hipStream_t s)
+{
+    const unsigned long long grid_x = (a.row_count + 15ull) / 16ull, grid_y = (a.input_rows + 15ull) / 16ull;
+    if (grid_x > 0x7fffffffull || grid_y > 65535ull) return ST_BOUNDS;
+    if (a.input_rows < 256ull) {
+        matvec_f32_tile16_kernel<16, QT><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
+    } else if (a.row_width % kF32BlockColumns == 0ull &&
+               (a.row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows *
+                   ((a.input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows) >= 3ull * compute_units() / 4ull) {
+        // (a block a compute unit or close to it: the staged kernel walks the row width
+        // chunk by chunk, 3 us each, and is behind the small tiles on a grid that leaves
+        // most of the device idle: 161 us against 46 us for 256 rows by 256)
+        const unsigned long long block_y = (a.input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows;
+        if (block_y > 65535ull) return ST_BOUNDS;
+        YVEX_ALLOW_DYNAMIC_LDS(matvec_f32_block_kernel<QT>, kF32BlockLdsBytes);
+        matvec_f32_block_kernel<QT><<<dim3((unsigned)((a.row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows),
+                                       (unsigned)block_y), 512, kF32BlockLdsBytes, s>>>(a);
+    } else {
+        matvec_f32_tile16_kernel<4, QT><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
+    }
+    return check_launch("matvec_f32_tile16");
+}
+
 extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint64_t row_count,
                                uint64_t row_width, uint64_t row_bytes, const void *input,
                                int input_q8, uint64_t input_rows, uint64_t input_stride,
@@ -963,33 +1016,15 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
     if (qtype == QT_Q8_0 && input_q8 && input_rows >= 16ull && !((uintptr_t)encoded & 3u))
         return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive, out,
                                       out_stride, output_bf16 != 0, status, s);
-    // F32 rows against a batch of F32 input rows: 16 x 16 tiles on the double-precision matrix
-    // cores; a small batch offers few tiles, so sixteen waves split the row width, a large one
-    // has tiles enough for four
-    if (qtype == QT_F32 && input_rows >= 8ull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) &&
-        !(input_stride & 3ull) && row_width % (input_rows < 256ull ? 256ull : 64ull) == 0ull) {
-        const unsigned long long grid_x = (row_count + 15ull) / 16ull, grid_y = (input_rows + 15ull) / 16ull;
-        if (grid_x > 0x7fffffffull || grid_y > 65535ull) return ST_BOUNDS;
-        if (input_rows < 256ull) {
-            matvec_f32_tile16_kernel<16><<<dim3((unsigned)grid_x, (unsigned)grid_y), 1024, 0, s>>>(a);
-        } else if (row_width % kF32BlockColumns == 0ull &&
-                   (row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows *
-                       ((input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows) >= 3ull * compute_units() / 4ull) {
-            // (a block a compute unit or close to it: the staged kernel walks the row width
-            // chunk by chunk, 3 us each, and is behind the small tiles on a grid that leaves
-            // most of the device idle: 161 us against 46 us for 256 rows by 256)
-            const unsigned long long block_y = (input_rows + kF32BlockInputRows - 1ull) / kF32BlockInputRows;
-            if (block_y > 65535ull) return ST_BOUNDS;
-            YVEX_ALLOW_DYNAMIC_LDS(matvec_f32_block_kernel, kF32BlockLdsBytes);
-            matvec_f32_block_kernel<<<dim3((unsigned)((row_count + kF32BlockWeightRows - 1ull) / kF32BlockWeightRows),
-                                           (unsigned)block_y), 512, kF32BlockLdsBytes, s>>>(a);
-        } else {
-            matvec_f32_tile16_kernel<4><<<dim3((unsigned)grid_x, (unsigned)grid_y), 256, 0, s>>>(a);
-        }
-        return check_launch("matvec_f32_tile16");
-    }
-    // (F32 rows go to the matrix cores from eight input rows on; 16-bit rows have no other fast
-    // kernel and stay here, four input rows a workgroup)
+    // F32 rows against a batch of F32 input rows: the double-precision matrix cores; rows of F16
+    // and BF16 values take the same kernels (the conversion to double is exact for them as well)
+    if ((qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16) && input_rows >= 8ull &&
+        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
+        row_width % (input_rows < 256ull ? 256ull : 64ull) == 0ull)
+        return qtype == QT_F32 ? launch_scalar_rows<QT_F32>(a, s)
+             : qtype == QT_F16 ? launch_scalar_rows<QT_F16>(a, s) : launch_scalar_rows<QT_BF16>(a, s);
+    // (fewer than eight input rows, or a row width the matrix-core kernels do not take: 16-bit
+    // rows have no other fast kernel and stay here at any number of input rows, four a workgroup)
     if (((qtype == QT_F32 && input_rows < 8ull) ||
          ((qtype == QT_F16 || qtype == QT_BF16) && (input_rows + 3ull) / 4ull <= 65535ull)) &&
         row_count <= 0x7fffffffull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
