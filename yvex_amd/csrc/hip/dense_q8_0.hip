@@ -3,16 +3,14 @@
 // for every format that takes Q8 activations, src/backend/cuda/private.h:461-464,
 // src/backend/cuda/qtype.c:252-255).
 //
-// Arithmetic per 32-value block, as the lane-strided kernel and the reference's primitive form it
-// (src/backend/cuda/kernel_primitives.h:353-357):
-//     dot   = sum_i q_i * a_i                       (int32, exact: one K step of V_MFMA_I32_32X32X32_I8)
-//     value = (d_block * d_a) * float(dot)          (two float products)
-// and the values of a row are added in float. Here the eight blocks under one input scale are
-// added as fma(d_block, float(dot), sum) and the sum enters the row's with fma(d_a, sum, row):
-// float sums in another order and with fewer roundings, inside the 1e-5 the format's dense rows
-// are held to. A block has a scale of its own, so
-// every matrix instruction starts from zero and its sixteen results a lane are converted, scaled
-// and added on the vector ALU.
+// Arithmetic, as the reference's primitive forms it for one 256-value superblock
+// (src/backend/cuda/kernel_primitives.h:342-359) and the CPU path adds a row's superblocks
+// (src/gguf/quant_compute.c:152-172):
+//     dot_b = sum_i q_i * a_i                              (int32, exact: one K step of V_MFMA_I32_32X32X32_I8)
+//     total = fmaf(d_b * d_a, float(dot_b), total)         b = 0 .. 7 in order, floats, from zero
+//     row  += double(total)                                superblock by superblock, rounded to float once
+// A block has a scale of its own, so every matrix instruction starts from zero and its sixteen
+// results a lane are converted, scaled and chained on the vector ALU (three instructions each).
 //
 // A workgroup owns 32 weight rows x 32 input rows; its four waves take every fourth superblock
 // (eight blocks, 272 bytes a row) and their partial tiles are added in wave order, so results do
@@ -83,7 +81,7 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
 {
     // per wave: the scales of the input rows whose blocks its lanes hold; then the partial tiles
     __shared__ __align__(16) float row_scale[kPlainWaves][32];
-    __shared__ float partial[kPlainWaves - 1u][16][64];
+    __shared__ double partial[kPlainWaves - 1u][16][64];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned r = lane & 31u, h = lane >> 5;
     const unsigned long long row0 = (unsigned long long)blockIdx.x * 32ull;
@@ -94,9 +92,9 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
     unsigned long long t = tok0 + r;
     if (t >= g.input_rows) t = g.input_rows - 1ull;
     const unsigned char *arow = g.act + t * ((unsigned long long)g.blocks * kQ8KBytes);
-    float acc[16];
+    double acc[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0;
 
     Q80Inputs cur;
     q80_load(wrow, arow, wave < g.blocks ? wave : 0u, h, cur);
@@ -129,9 +127,14 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        float within[16];       // the superblock's sum before the input rows' scales
+        float d_a[16], total[16];       // the input rows' scales; the superblock's chain of eight terms
 #pragma unroll
-        for (int i = 0; i < 16; ++i) within[i] = 0.0f;
+        for (unsigned q4 = 0; q4 < 4u; ++q4) {
+            const float4 d = *reinterpret_cast<const float4 *>(&row_scale[wave][8u * q4 + 4u * h]);
+            d_a[4u * q4] = d.x; d_a[4u * q4 + 1u] = d.y; d_a[4u * q4 + 2u] = d.z; d_a[4u * q4 + 3u] = d.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) total[i] = 0.0f;
 #pragma unroll
         for (unsigned c = 0; c < 8u; ++c) {
             v4i codes;
@@ -151,19 +154,13 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
             const v4i tokens = {(int)cur.a[c].x, (int)cur.a[c].y, (int)cur.a[c].z, (int)cur.a[c].w};
             const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(tokens, codes, zero, 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w[c], (float)dot[i], within[i]);
+            for (int i = 0; i < 16; ++i) total[i] = __builtin_fmaf(d_w[c] * d_a[i], (float)dot[i], total[i]);
             // (left alone the scheduler issues the matrix instructions of all blocks first and
             // keeps their results)
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (unsigned q4 = 0; q4 < 4u; ++q4) {
-            const float4 d = *reinterpret_cast<const float4 *>(&row_scale[wave][8u * q4 + 4u * h]);
-            acc[4u * q4] = __builtin_fmaf(d.x, within[4u * q4], acc[4u * q4]);
-            acc[4u * q4 + 1u] = __builtin_fmaf(d.y, within[4u * q4 + 1u], acc[4u * q4 + 1u]);
-            acc[4u * q4 + 2u] = __builtin_fmaf(d.z, within[4u * q4 + 2u], acc[4u * q4 + 2u]);
-            acc[4u * q4 + 3u] = __builtin_fmaf(d.w, within[4u * q4 + 3u], acc[4u * q4 + 3u]);
-        }
+        for (int i = 0; i < 16; ++i) acc[i] += (double)total[i];
         // (the next superblock's scales are not written before every lane has read these)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -182,9 +179,10 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const unsigned long long token = tok0 + 8u * (i >> 2) + 4u * h + (i & 3);
-        float sum = acc[i];
+        double wide = acc[i];
 #pragma unroll
-        for (unsigned w = 0; w + 1u < kPlainWaves; ++w) sum += partial[w][i][lane];
+        for (unsigned w = 0; w + 1u < kPlainWaves; ++w) wide += partial[w][i][lane];
+        const float sum = (float)wide;
         if (row >= g.row_count || token >= g.input_rows) continue;
         const unsigned long long at = token * g.out_stride + row;
         const float value = g.additive ? sum + g.additive[at] : sum;
@@ -294,9 +292,9 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
                            (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16u * kStagedThreads * kActRounds)));
     };
 
-    float acc[16];
+    double acc[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0;
 
     copies(0u);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -307,9 +305,13 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
         const unsigned w_row = kStagedWeightBase + buffer * kStagedWeightBytes + (32u * row_block + r) * kStagedPitch;
         const unsigned a_tile = kStagedActBase + buffer * kStagedActBytes + 32u * token_block * kStagedPitch;
 
-        float within[16];           // the superblock's sum before the input rows' scales
+        float d_a[16], total[16];   // the input rows' scales; the superblock's chain of eight terms
 #pragma unroll
-        for (int i = 0; i < 16; ++i) within[i] = 0.0f;
+        for (unsigned i = 0; i < 16u; ++i) {
+            const unsigned token = 8u * (i >> 2) + 4u * h + (i & 3u);
+            d_a[i] = __uint_as_float(lds_read_u32(a_tile + token * kStagedPitch + 256u));
+            total[i] = 0.0f;
+        }
         // Three stages in flight, or a wave would run its LDS reads, its matrix instruction and the
         // scaling of the results one after the other: in step k the operands of block k are
         // read, block k - 1 is multiplied and the results of block k - 2 are scaled (vector
@@ -354,16 +356,13 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
             if (k >= 2u) {
                 const unsigned slot = k % 2u;           // block k - 2
 #pragma unroll
-                for (int i = 0; i < 16; ++i) within[i] = __builtin_fmaf(d_w[slot], (float)dot[slot][i], within[i]);
+                for (int i = 0; i < 16; ++i)
+                    total[i] = __builtin_fmaf(d_w[slot] * d_a[i], (float)dot[slot][i], total[i]);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (unsigned i = 0; i < 16u; ++i) {
-            const unsigned token = 8u * (i >> 2) + 4u * h + (i & 3u);
-            const float d_a = __uint_as_float(lds_read_u32(a_tile + token * kStagedPitch + 256u));
-            acc[i] = __builtin_fmaf(d_a, within[i], acc[i]);
-        }
+        for (int i = 0; i < 16; ++i) acc[i] += (double)total[i];
         // the next superblock's copies have landed and every wave is done with this one's buffers
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -379,7 +378,8 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
         const unsigned long long token = tok0 + 32u * token_block + 8u * (i >> 2) + 4u * h + (i & 3u);
         if (token >= g.input_rows) continue;
         const unsigned long long at = token * g.out_stride + row;
-        const float value = g.additive ? acc[i] + g.additive[at] : acc[i];
+        const float sum = (float)acc[i];
+        const float value = g.additive ? sum + g.additive[at] : sum;
         if (!finite_f32(value)) bad = true;
         else g.out[at] = g.output_bf16 ? bf16_round(value) : value;
     }

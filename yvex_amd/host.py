@@ -103,7 +103,7 @@ class RowBatchLayer:
 
     def __init__(self, torch, routed, shared, router, x_host, rows, *, hidden, intermediate, experts, topk,
                  qtype=16, sweep_image=False, scoring=abi.SCORING_SIGMOID, scaling=1.0, limit=10.0,
-                 envelope=None, down_qtype=None):
+                 envelope=None, down_qtype=None, shared_qtype=None):
         """envelope: None, or the residual-stream weights around the layer as device tensors,
         dict(streams, iterations, function [F32 (streams + 2) * streams x streams * hidden], scale
         [F32 3], base [F32 (streams + 2) * streams], norm [BF16 hidden]); x_host then holds
@@ -133,8 +133,12 @@ class RowBatchLayer:
         job.layer = C.pointer(plan)
         # down_qtype: the down projections' format where it differs from the gate and up projections'
         down_qtype = qtype if down_qtype is None else down_qtype
-        block_bytes = {16: 66, 12: 144, 10: 84}
+        # shared_qtype: the format of all three matrices of the shared expert where it differs
+        block_bytes = {16: 66, 12: 144, 10: 84, 8: 272}
         rb_h, rb_i = HIDDEN // 256 * block_bytes[qtype], INTERMEDIATE // 256 * block_bytes[down_qtype]
+        sq_gate = qtype if shared_qtype is None else shared_qtype
+        sq_down = down_qtype if shared_qtype is None else shared_qtype
+        srb_h, srb_i = HIDDEN // 256 * block_bytes[sq_gate], INTERMEDIATE // 256 * block_bytes[sq_down]
 
         self.images = []
 
@@ -171,9 +175,9 @@ class RowBatchLayer:
         view(abi.W_ROUTED_GATE, routed[0], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
         view(abi.W_ROUTED_UP, routed[1], qtype, HIDDEN, EXPERTS * INTERMEDIATE, rb_h, enc, gate_up)
         view(abi.W_ROUTED_DOWN, routed[2], down_qtype, INTERMEDIATE, EXPERTS * HIDDEN, rb_i, enc, down_c)
-        view(abi.W_SHARED_GATE, shared[0], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
-        view(abi.W_SHARED_UP, shared[1], qtype, HIDDEN, INTERMEDIATE, rb_h, enc, shared_c)
-        view(abi.W_SHARED_DOWN, shared[2], down_qtype, INTERMEDIATE, HIDDEN, rb_i, enc, shared_c)
+        view(abi.W_SHARED_GATE, shared[0], sq_gate, HIDDEN, INTERMEDIATE, srb_h, enc, shared_c)
+        view(abi.W_SHARED_UP, shared[1], sq_gate, HIDDEN, INTERMEDIATE, srb_h, enc, shared_c)
+        view(abi.W_SHARED_DOWN, shared[2], sq_down, INTERMEDIATE, HIDDEN, srb_i, enc, shared_c)
         if envelope:
             mixing = (streams + 2) * streams
             f32 = abi.ACT_DEVICE_F32
