@@ -11,8 +11,9 @@ Prints ONE JSON line. `roofline` covers the dominant kernel (the routed gate/up 
 with events on the launch stream; `cpu_baseline` is the reference's own CPU expert path
 (compiled from its sources; the C restatement beside it) timed on the host cores over a bounded
 sample of the same workload. `prefill` holds BASELINE config 4 (2048 rows on the int8 matrix
-cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `q2k_down` both batches
-with the reference's own pairing of IQ2_XXS gate/up and Q2_K down experts, `decode_envelope` the
+cores), `prefill_q4k` and `decode_q4k` the same batches with Q4_K experts, `model_file_layer` both
+batches with the formats of the reference's model file (IQ2_XXS gate/up and Q2_K down routed experts,
+a Q8_0 shared expert), `decode_envelope` the
 headline step with four residual streams around the layer, `decode_small_batches` the headline
 layer at 1 to 16 rows, and `dense` configs
 0-2 and an output head as single matvec launches; the prefill legs and the dense configs carry a
@@ -501,32 +502,43 @@ def synth_q2k(torch, blocks: int, device, seed: int):
     return raw.reshape(-1)
 
 
-def q2k_down_leg(torch, gate, up, shared, dev, steps: int, warmup: int):
-    """The pairing of the reference's model file (IQ2_XXS gate and up experts, Q2_K down experts:
-    src/backend/cuda/tensorcore.cu:563-564, 660) through the C ABI, gate and up experts resident as
-    the sweeps' image and the down experts as canonical rows (they have no image): the headline
-    batch of 32 rows (decode sweeps) and 2048 rows (matrix cores). Bytes counted: the canonical
-    bytes of the distinct experts hit."""
+def synth_q8_0(torch, blocks: int, device, seed: int):
+    """Q8_0 blocks (34 bytes): a small positive fp16 scale, then 32 random int8 codes."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    raw = torch.randint(0, 256, (blocks, 34), dtype=torch.uint8, device=device, generator=gen)
+    scales = (torch.rand(blocks, device=device, generator=gen) * 1e-3 + 1e-4).to(torch.float16)
+    raw[:, 0:2] = scales.view(torch.uint8).reshape(-1, 2)
+    return raw.reshape(-1)
+
+
+def model_file_layer_leg(torch, gate, up, dev, steps: int, warmup: int):
+    """The formats of the reference's model file (src/graph/families/deepseek_v4.c:1550-1575: routed
+    experts with IQ2_XXS gate and up and Q2_K down matrices, everything else Q8_0, the shared
+    expert with it) through the C ABI, the routed gate and up experts resident as the sweeps'
+    image and the rest as canonical rows: the headline batch of 32 rows (decode sweeps, the shared
+    expert as dense projections) and 2048 rows (matrix cores). Bytes counted: the canonical bytes
+    of the distinct experts hit and of the shared expert."""
     from yvex_amd.host import RowBatchLayer
     blocks = INTERMEDIATE * HIDDEN // 256
     down = synth_q2k(torch, EXPERTS * blocks, dev, 41)
-    shared_down = synth_q2k(torch, blocks, dev, 42)
+    shared = tuple(synth_q8_0(torch, blocks * 8, dev, 42 + i) for i in range(3))
     gen = torch.Generator(device=dev)
     gen.manual_seed(78)
     router = (torch.randn((EXPERTS, HIDDEN), device=dev, generator=gen) / HIDDEN ** 0.5).contiguous()
-    out = {"workload": "IQ2_XXS gate/up experts (sweep image) with Q2_K down experts (canonical rows), top-8 of "
-                       "256 + shared, Q8_K activations"}
+    out = {"workload": "routed experts IQ2_XXS gate/up (sweep image) + Q2_K down, Q8_0 shared expert, top-8 of 256, "
+                       "Q8_K activations"}
     for rows, count in ((ROWS, steps), (2048, max(3, steps // 10))):
         x = torch.randn((rows, HIDDEN), device=dev, generator=gen)
-        layer = RowBatchLayer(torch, (gate, up, down), (shared[0], shared[1], shared_down), router, x.cpu().numpy(),
+        layer = RowBatchLayer(torch, (gate, up, down), shared, router, x.cpu().numpy(),
                               rows, hidden=HIDDEN, intermediate=INTERMEDIATE, experts=EXPERTS, topk=TOPK,
-                              qtype=16, down_qtype=10, sweep_image=True)
+                              qtype=16, down_qtype=10, shared_qtype=8, sweep_image=True)
         layer.step(defer=False)
         unique = int(layer.result.unique_experts)
         matrix = int(layer.result.tensor_core_launches)
         ms = min(layer.timed(count, max(warmup, 2)), layer.timed(count, warmup, eager=True))
         layer.close()
-        read = (unique + 1) * blocks * (2 * 66 + 84)
+        read = unique * blocks * (2 * 66 + 84) + 3 * blocks * 8 * 34
         leg = {"ms_per_step": round(ms, 4), "distinct_routed_experts": unique, "matrix_core_launches": matrix,
                "GB_per_s": round(read / (ms * 1e-3) / 1e9, 1)}
         if rows > ROWS:
@@ -867,7 +879,7 @@ def main() -> int:
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, K, MoeLayer, (gate, up, down), shared, dev,
                                      max(3, args.steps // 10), 2)
-        out["q2k_down"] = q2k_down_leg(torch, gate, up, shared, dev, args.steps, args.warmup)
+        out["model_file_layer"] = model_file_layer_leg(torch, gate, up, dev, args.steps, args.warmup)
     if not args.no_prefill:
         # config 4's second weight format: the same layer with Q4_K experts (6.3 GB of them)
         del layer, gate, up, down, shared

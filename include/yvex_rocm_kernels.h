@@ -271,6 +271,14 @@ int yvex_hip_moe_down_rows(const yvex_hip_expert_weights *weights, const void *i
                            const uint64_t *counts, uint64_t pairs, uint64_t experts,
                            float *pair_outputs, int *status, yvex_hip_stream stream);
 
+/* The SwiGLU stage of an expert whose gate and up projections ran as dense projections (a shared
+ * expert of a format the expert kernels do not take): out[i] = bf16(silu(min(gate[i], limit)) *
+ * clamp(up[i], -limit, limit)), the value yvex_moe_grouped_up_rows forms with a route weight of
+ * one (moe_kernels.cu:431-516, src/graph/moe.c:605-611). out may be gate or up. A product that is
+ * not finite raises status 1 and is not stored. */
+int yvex_hip_moe_swiglu_rows(const float *gate, const float *up, uint64_t count, double limit,
+                             float *out, int *status, yvex_hip_stream stream);
+
 /* Replaces yvex_moe_reduce_rows + yvex_moe_combine_rows (moe_kernels.cu:584-616):
  * routed[row, c] = sum over rank (in rank order, fp32) of pair_outputs[row*topk+rank, c];
  * combined[row, c] = bf16(routed + shared) when shared != NULL and combined != NULL. */

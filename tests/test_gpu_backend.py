@@ -311,7 +311,8 @@ class MoeCase:
     def __init__(self, b, oracle, *, qtype="IQ2_XXS", hidden=512, intermediate=256, experts=8, topk=2,
                  rows=5, act=abi.ACT_DEVICE_ENCODED, scoring=abi.SCORING_SQRT_SOFTPLUS, bias=True,
                  shared=True, family=abi.FAMILY_GFX950, seed=42, streams=0, iterations=20, hash_vocab=0,
-                 down_qtype=None, sweep_image=(), arena_from=None, norm_qtype="BF16", bias_qtype="F32"):
+                 down_qtype=None, sweep_image=(), arena_from=None, norm_qtype="BF16", bias_qtype="F32",
+                 shared_qtype=None):
         """arena_from: a MoeCase of the same layer on the owning backend of `b` (a shared session):
         its published arena is attached instead of another copy being made resident."""
         self.b, self.oracle = b, oracle
@@ -322,6 +323,10 @@ class MoeCase:
         self.qt, self.rows, self.hidden, self.experts, self.topk = qt, rows, hidden, experts, topk
         qt_down = getattr(oracle, down_qtype) if down_qtype else qt
         self.qtypes = (qt, qt, qt_down)
+        # the shared expert's three matrices in a format of their own (the reference's model file
+        # keeps it in Q8_0)
+        qs = getattr(oracle, shared_qtype) if shared_qtype else None
+        self.shared_qtypes = (qs, qs, qs) if shared_qtype else self.qtypes
         self.intermediate, self.scoring = intermediate, scoring
         g = oracle.Generator(seed, f"backend.moe.{qtype}.{hidden}.{experts}")
         parts = {
@@ -330,9 +335,9 @@ class MoeCase:
             "gate": g.weights(qt, experts * intermediate, hidden),
             "up": g.weights(qt, experts * intermediate, hidden),
             "down": g.weights(qt_down, experts * hidden, intermediate),
-            "sgate": g.weights(qt, intermediate, hidden),
-            "sup": g.weights(qt, intermediate, hidden),
-            "sdown": g.weights(qt_down, hidden, intermediate),
+            "sgate": g.weights(self.shared_qtypes[0], intermediate, hidden),
+            "sup": g.weights(self.shared_qtypes[1], intermediate, hidden),
+            "sdown": g.weights(self.shared_qtypes[2], hidden, intermediate),
         }
         # the correction bias as F32 values (read where they lie) or as BF16 values (decoded into
         # the workspace first)
@@ -436,9 +441,10 @@ class MoeCase:
         view(abi.W_ROUTED_GATE, "gate", qt, hidden, experts * intermediate, rb_h)
         view(abi.W_ROUTED_UP, "up", qt, hidden, experts * intermediate, rb_h)
         view(abi.W_ROUTED_DOWN, "down", qt_down, intermediate, experts * hidden, rb_i)
-        view(abi.W_SHARED_GATE, "sgate", qt, hidden, intermediate, rb_h)
-        view(abi.W_SHARED_UP, "sup", qt, hidden, intermediate, rb_h)
-        view(abi.W_SHARED_DOWN, "sdown", qt_down, intermediate, hidden, rb_i)
+        sq = self.shared_qtypes
+        view(abi.W_SHARED_GATE, "sgate", sq[0], hidden, intermediate, oracle.row_bytes(sq[0], hidden))
+        view(abi.W_SHARED_UP, "sup", sq[1], hidden, intermediate, oracle.row_bytes(sq[1], hidden))
+        view(abi.W_SHARED_DOWN, "sdown", sq[2], intermediate, hidden, oracle.row_bytes(sq[2], intermediate))
         if hash_vocab:
             view(abi.W_ROUTER_TABLE, "table", 26, topk, hash_vocab, topk * 4, abi.ACT_DEVICE_F32)
         if streams:
@@ -493,11 +499,25 @@ class MoeCase:
         assert np.allclose(logits, x @ router.T, rtol=1e-4, atol=1e-5)
         bias = self.bias_values if self.plan.requires_correction_bias else None
         shared = (p["sgate"], p["sup"], p["sdown"]) if self.plan.shared_experts else None
+        own_format = shared is not None and self.shared_qtypes != self.qtypes
         want = o.moe_layer(hidden=self.hidden, intermediate=self.intermediate, experts=self.experts,
                            topk=self.topk, qtypes=self.qtypes, routed=(p["gate"], p["up"], p["down"]),
-                           shared=shared, inputs=x, logits=logits, bias=bias, scoring=self.scoring,
-                           normalize=True, scaling=1.5, act_q8=act_q8, threads=8,
+                           shared=None if own_format else shared, inputs=x, logits=logits, bias=bias,
+                           scoring=self.scoring, normalize=True, scaling=1.5, act_q8=act_q8, threads=8,
                            hash_selected=self.table[self.tokens] if self.hash_vocab else None)
+        if own_format:
+            # the layer's own composition (src/runtime/moe.c:596-632) with the shared expert run in
+            # its format: route weight one, combined = bf16(routed + shared)
+            rows = np.ascontiguousarray(x, np.float32).reshape(-1, self.hidden)
+            outs = []
+            for row in rows:
+                rc, out, _, _ = o.moe_expert(self.shared_qtypes, *shared, self.hidden, self.intermediate, row, 1.0,
+                                             act_q8=act_q8)
+                assert rc == 0
+                outs.append(out)
+            want["shared"] = np.stack(outs)
+            bits = (want["routed"] + want["shared"]).astype(np.float32).view(np.uint32)
+            want["combined"] = ((bits + 0x7fff + ((bits >> 16) & 1)) & 0xffff0000).view(np.float32)
         if ingress:
             want["normalized"], want["post"], want["combination"] = ingress
             rc, want["envelope"] = o.mhc_post(want["combined"], self.x, ingress[1], ingress[2],
@@ -595,13 +615,17 @@ def test_execute_rows_hash_router(backend, oracle, streams):
     # the one pairing of layouts that need not agree; decode width and matrix-core width
     ("IQ2_XXS", 2048, 2048, 16, 4, 20, ("routed", "shared")),
     ("IQ2_XXS", 2048, 2048, 4, 2, 60, ("routed", "shared"))])
+@pytest.mark.parametrize("shared_qtype", [None, "Q8_0"])
 def test_execute_rows_with_q2k_down_experts(backend, oracle, qtype, hidden, intermediate, experts, topk, rows,
-                                            image):
+                                            image, shared_qtype):
     """The pairing of the reference's model file, IQ2_XXS gate and up experts with Q2_K down
     experts (src/backend/cuda/tensorcore.cu:563-564, 660), at decode width: the down projection
     runs the specialised sweeps over Q2_K rows, and the result is the CPU layer's bit for bit."""
+    if shared_qtype:        # (a Q8_0 shared expert, the model file's: dense projections from 16 rows on)
+        image = tuple(group for group in image if group != "shared")
     case = MoeCase(backend, oracle, qtype=qtype, down_qtype="Q2_K", hidden=hidden, intermediate=intermediate,
-                   experts=experts, topk=topk, rows=rows, scoring=abi.SCORING_SIGMOID, sweep_image=image)
+                   experts=experts, topk=topk, rows=rows, scoring=abi.SCORING_SIGMOID, sweep_image=image,
+                   shared_qtype=shared_qtype)
     backend.workspace(case.workspace_bytes)
     rc = case.execute()
     assert rc == 0, case.err.message

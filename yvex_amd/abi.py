@@ -306,7 +306,7 @@ KERNEL_EXPORTS = [
     "yvex_hip_argmax_static_capacity",
     "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_moe_route_hash_rows", "yvex_hip_worklist_build", "yvex_hip_moe_prepare", "yvex_hip_moe_prepare_scored",
     "yvex_hip_moe_prepare_supported", "yvex_hip_moe_up", "yvex_hip_moe_down", "yvex_hip_iq2_sweep_image_bytes", "yvex_hip_iq2_sweep_image_build",
-    "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows",
+    "yvex_hip_moe_up_rows", "yvex_hip_moe_down_rows", "yvex_hip_moe_swiglu_rows",
     "yvex_hip_moe_reduce_combine", "yvex_hip_mhc_ingress", "yvex_hip_mhc_ingress_encoded", "yvex_hip_mhc_egress",
     "yvex_hip_stream_read", "yvex_hip_bandwidth_sample", "yvex_hip_clock_probe", "yvex_hip_fill_u32",
     "yvex_hip_capture_begin", "yvex_hip_capture_end", "yvex_hip_capture_abort", "yvex_hip_graph_launch",

@@ -1125,6 +1125,29 @@ extern "C" int yvex_hip_moe_down(const yvex_hip_expert_weights *w, const void *i
     return dispatch_grouped(w->down_qtype, a, act_q8 != 0, false, as_stream(stream));
 }
 
+// The clamped SiLU-gated products of given gate and up sums (src/graph/moe.c:605-611), rounded
+// to bfloat16 as the fused kernels round them; out may be either input.
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float *gate, const float *up,
+                                                          unsigned long long count, double limit, float *out,
+                                                          int *status)
+{
+    const unsigned long long at = (unsigned long long)blockIdx.x * 256ull + threadIdx.x;
+    if (at >= count) return;
+    const float value = swiglu_bf16_fast(gate[at], up[at], 1.0f, limit, (float)limit);
+    if (!finite_f32(value)) raise_status(status, 1);
+    else out[at] = value;
+}
+
+extern "C" int yvex_hip_moe_swiglu_rows(const float *gate, const float *up, uint64_t count, double limit,
+                                        float *out, int *status, yvex_hip_stream stream)
+{
+    if (!gate || !up || !out || !status || !count || !(limit > 0.0)) return ST_INVALID_ARG;
+    const uint64_t grid = (count + 255u) / 256u;
+    if (grid > 0x7fffffffull) return ST_BOUNDS;
+    swiglu_rows_kernel<<<(unsigned)grid, 256, 0, as_stream(stream)>>>(gate, up, count, limit, out, status);
+    return check_launch("moe_swiglu_rows");
+}
+
 extern "C" int yvex_hip_moe_reduce_combine(const float *pair_outputs, uint64_t rows,
                                            uint64_t topk, uint64_t hidden, const float *shared,
                                            float *routed, float *combined, int *status,

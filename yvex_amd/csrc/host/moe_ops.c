@@ -502,7 +502,7 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     const float *bias_rows;
     void *combined_target;
     unsigned long long table_address = 0ull;
-    int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, device_status = 0, rc, defer, scored = 0;
+    int matrix_allowed = 1, envelope, hash_router, unsupported_width, routed_q8 = 0, shared_q8 = 0, routed_image = 0, shared_image = 0, has_shared, merged, row_batch, shared_row_batch, shared_dense, device_status = 0, rc, defer, scored = 0;
     void *status;
     yvex_hip_stream stream;
     enum { GRAPH_EAGER = 0, GRAPH_CAPTURE, GRAPH_REPLAY } graph_mode = GRAPH_EAGER;
@@ -692,6 +692,15 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
                 pairs >= (routed.gate_qtype == 12u ? 4ull : 6ull) * experts;
     shared_row_batch = row_batch && has_shared && shared_q8 && matrix_core_qtypes(&shared);
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
+    /* A Q8_0 shared expert (the format the reference's model file keeps it in, its default for every
+     * tensor outside the routed experts: src/graph/families/deepseek_v4.c:1550-1557) is three dense
+     * projections of every row, and from 16 rows on the dense Q8_0 kernels give the CPU path's bits
+     * on the matrix cores: gate and up sums, the SwiGLU stage, quantization, down. The up sums
+     * borrow the pair-output range, which nothing uses between the router and the routed down
+     * projection. */
+    shared_dense = has_shared && shared_q8 && !merged && !shared_row_batch && !shared_image &&
+                   shared.gate_qtype == 8u && shared.up_qtype == 8u && shared.down_qtype == 8u &&
+                   row_count >= 16ull && layer->shared_intermediate_width <= topk * hidden;
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",
                                 "kernel launch failed (test seam)");
@@ -958,7 +967,20 @@ sequence:
         LAUNCH(yvex_hip_moe_up_rows(&shared, AT(input_q8), NULL, NULL, NULL, NULL, NULL, NULL, row_count,
                                     1ull, 1ull, layer->activation_limit, (float *)AT(shared_intermediate),
                                     (int *)status, stream), "rocm.moe.rows.shared-up-matrix");
-    else if (has_shared && !merged)
+    else if (shared_dense) {
+        LAUNCH(yvex_hip_matvec(shared.gate, shared.gate_qtype, layer->shared_intermediate_width, hidden,
+                               shared.gate_row_bytes, AT(input_q8), 1, row_count, hidden, NULL,
+                               (float *)AT(shared_intermediate), layer->shared_intermediate_width, 0,
+                               (int *)status, stream), "rocm.moe.rows.shared-gate-dense");
+        LAUNCH(yvex_hip_matvec(shared.up, shared.up_qtype, layer->shared_intermediate_width, hidden,
+                               shared.up_row_bytes, AT(input_q8), 1, row_count, hidden, NULL,
+                               (float *)AT(pair_outputs), layer->shared_intermediate_width, 0,
+                               (int *)status, stream), "rocm.moe.rows.shared-up-dense");
+        LAUNCH(yvex_hip_moe_swiglu_rows((const float *)AT(shared_intermediate), (const float *)AT(pair_outputs),
+                                        row_count * layer->shared_intermediate_width, layer->activation_limit,
+                                        (float *)AT(shared_intermediate), (int *)status, stream),
+               "rocm.moe.rows.shared-swiglu");
+    } else if (has_shared && !merged)
         LAUNCH(yvex_hip_moe_up(&shared, shared_q8 ? AT(input_q8) : (void *)(uintptr_t)activations,
                                shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull, 1ull,
                                layer->activation_limit, (float *)AT(shared_intermediate), NULL, 0ull, NULL,
@@ -997,6 +1019,11 @@ sequence:
         LAUNCH(yvex_hip_moe_down_rows(&shared, AT(shared_intermediate_q8), NULL, NULL, NULL, NULL, NULL,
                                       row_count, 1ull, (float *)AT(shared_outputs), (int *)status, stream),
                "rocm.moe.rows.shared-down-matrix");
+    else if (shared_dense)
+        LAUNCH(yvex_hip_matvec(shared.down, shared.down_qtype, hidden, layer->shared_intermediate_width,
+                               shared.down_row_bytes, AT(shared_intermediate_q8), 1, row_count,
+                               layer->shared_intermediate_width, NULL, (float *)AT(shared_outputs), hidden, 1,
+                               (int *)status, stream), "rocm.moe.rows.shared-down-dense");
     else if (has_shared && !merged)
         LAUNCH(yvex_hip_moe_down(&shared, shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate),
                                  shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull,
