@@ -321,6 +321,33 @@ def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, in
     assert np.allclose(few, got[:15], rtol=2e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("rows,width,inputs", [(130, 512, 1), (33, 2304, 5), (2048, 7168, 3), (40, 256, 15)])
+def test_matvec_q8_0_exact_at_few_rows(gpu, oracle, rows, width, inputs):
+    """yvex_hip_matvec_q8_0_exact below 16 input rows (a shared expert run as dense projections at
+    decode width): the oracle's Q8_K product bit for bit, where yvex_hip_matvec's faster kernel is
+    held to 1e-5; additive rows and the bf16 rounding on top."""
+    from yvex_amd import kernels as K
+    qt = oracle.Q8_0
+    g = oracle.Generator(42, f"matvec.q8_0.exact.{rows}.{width}.{inputs}")
+    w = g.weights(qt, rows, width)
+    x = g.normal(inputs * width).reshape(inputs, width)
+    add = g.normal(inputs * rows).reshape(inputs, rows)
+    status = K.new_status(gpu)
+    act = K.q8k_quantize(dev(x, gpu), status)
+    got = K.matvec_q8_0_exact(dev(w, gpu), rows, width, act, inputs, status=status).cpu().numpy()
+    status_ok(status)
+    want = oracle.q8_matvec(qt, w, rows, width, oracle.q8k_quantize(x), inputs)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    summed = K.matvec_q8_0_exact(dev(w, gpu), rows, width, act, inputs, additive=dev(add, gpu), output_bf16=True,
+                                 status=status).cpu().numpy()
+    status_ok(status)
+    assert np.all((summed.view(np.uint32) & 0xffff) == 0)
+    assert np.all(np.abs(summed - (got + add)) <= np.abs(got + add) * 2.0 ** -8 + 1e-30)
+    fast = K.matvec(dev(w, gpu), qt, rows, width, act, input_q8=True, input_rows=inputs, status=status).cpu().numpy()
+    status_ok(status)
+    assert_q8_product(fast, want, "Q8_0")
+
+
 @pytest.mark.parametrize("rows,width,inputs", [(2001, 1280, 1030), (4100, 512, 250)])
 def test_matvec_q8_0_large_batch_stages_operands_in_lds(gpu, oracle, rows, width, inputs):
     """A Q8_0 projection with more unstaged tiles than one round of workgroups takes the kernel

@@ -942,6 +942,18 @@ static int launch_block_q(const MatvecArgs &a, bool q8, hipStream_t stream)
 
 using namespace yvex;
 
+extern "C" int yvex_hip_matvec_q8_0_exact(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
+                                          uint64_t row_bytes, const void *input_q8k, uint64_t input_rows,
+                                          const float *additive, float *out, uint64_t out_stride,
+                                          int output_bf16, int *status, yvex_hip_stream stream)
+{
+    if (!encoded || !input_q8k || !out || !status || !row_count || !row_width || !input_rows ||
+        out_stride < row_count || (((uintptr_t)input_q8k | (uintptr_t)out) & 3u))
+        return ST_INVALID_ARG;
+    return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input_q8k, input_rows, additive, out,
+                                  out_stride, output_bf16 != 0, status, as_stream(stream));
+}
+
 // Rows of F32, F16 or BF16 values against eight or more F32 input rows: 16 x 16 tiles on the
 // double-precision matrix cores; a small batch offers few tiles, so sixteen waves split the row
 // width, a large one has tiles enough for four, or for the staged kernel.
