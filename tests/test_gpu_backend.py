@@ -1026,7 +1026,9 @@ def test_sweep_image_views_are_checked(backend, oracle):
     dict(rows=4, streams=4, hidden=512, iterations=5),                           # residual streams
     dict(rows=3, hash_vocab=50),                                                 # hash router
     dict(rows=200, hidden=768, intermediate=512, experts=4, scoring=abi.SCORING_SIGMOID),  # matrix cores
-], ids=["sweep", "generic", "streams", "hash", "matrix"])
+    # the model file's formats: Q2_K down sweeps, the Q8_0 shared expert as dense projections
+    dict(rows=7, hidden=2048, intermediate=2048, experts=8, down_qtype="Q2_K", shared_qtype="Q8_0"),
+], ids=["sweep", "generic", "streams", "hash", "matrix", "model-file-formats"])
 def test_execute_rows_graph_replays_equal_eager(backend, oracle, kwargs):
     """src/backend/cuda/moe.c:1650-1681: a job that does not ask for eager execution runs as a
     launch graph keyed on its topology. Here the key's first use runs eagerly, the second is
