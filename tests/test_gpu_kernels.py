@@ -73,7 +73,10 @@ def test_integer_block_dots_bit_exact(gpu, oracle, qtype, rows, width, inputs):
 @pytest.mark.parametrize("qtype,rows,width,inputs", [
     ("IQ2_XXS", 67, 2048, 1), ("IQ2_XXS", 9, 7168, 5), ("Q4_K", 33, 2048, 1),
     ("Q4_K", 10, 7168, 16), ("Q8_0", 64, 4096, 1), ("Q8_0", 13, 96, 3), ("Q2_K", 21, 768, 2),
-    ("F32", 17, 100, 3)])
+    ("F32", 17, 100, 3),
+    # Q8_0 rows against eight and more F32 rows: the double-precision matrix cores (16 x 16 tiles,
+    # sixteen and four waves a tile, staged blocks); a width they do not take stays lane-strided
+    ("Q8_0", 70, 512, 9), ("Q8_0", 33, 1024, 300), ("Q8_0", 2100, 256, 1000), ("Q8_0", 20, 96, 30)])
 def test_matvec_f32_activations(gpu, oracle, qtype, rows, width, inputs):
     from yvex_amd import kernels as K
     qt = getattr(oracle, qtype)

@@ -538,12 +538,22 @@ static int launch_scalar_few(const MatvecArgs &a, hipStream_t s)
 // its serial loop, so the float the sum rounds to is the CPU path's. The partial tiles of the
 // waves (and of the workgroups that split the width: blockIdx.z, joined by a second launch in
 // split order) are doubles, added in a fixed order.
-// Four consecutive weights of a row of F32, F16 or BF16 values as floats (exact conversions).
+// Four consecutive weights (column a multiple of four) of a row of F32, F16 or BF16 values, or of
+// Q8_0 blocks (scale times code, exact in float: the value the CPU decoder forms,
+// src/gguf/quant_block.c:715-881), as floats.
 template <unsigned QT>
 __device__ __forceinline__ float4 scalar_weights4(const unsigned char *row, unsigned long long column)
 {
     if constexpr (QT == QT_F32) {
         return *reinterpret_cast<const float4 *>(row + 4ull * column);
+    } else if constexpr (QT == QT_Q8_0) {
+        const unsigned char *block = row + 34ull * (column >> 5);
+        const float d = f16_bits_to_float(*reinterpret_cast<const unsigned short *>(block));
+        const unsigned char *codes = block + 2u + (unsigned)(column & 31ull);      // on a 2-byte boundary
+        const unsigned lo = *reinterpret_cast<const unsigned short *>(codes);
+        const unsigned hi = *reinterpret_cast<const unsigned short *>(codes + 2);
+        return make_float4(d * (float)(signed char)(lo & 255u), d * (float)(signed char)(lo >> 8),
+                           d * (float)(signed char)(hi & 255u), d * (float)(signed char)(hi >> 8));
     } else {
         const uint2 v = *reinterpret_cast<const uint2 *>(row + 2ull * column);
         if constexpr (QT == QT_F16)
@@ -667,7 +677,7 @@ __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
         if (row < kF32BlockWeightRows) {
             unsigned long long wrow = (unsigned long long)blockIdx.x * kF32BlockWeightRows + row;
             if (wrow >= a.row_count) wrow = a.row_count - 1ull;          // a ragged edge repeats the last row
-            source[j] = a.encoded + wrow * a.row_bytes + (QT == QT_F32 ? 16u : 8u) * piece;
+            source[j] = a.encoded + wrow * a.row_bytes;       // (a weight row: columns from 4 * piece on)
         } else {
             unsigned long long in = (unsigned long long)blockIdx.y * kF32BlockInputRows + (row - kF32BlockWeightRows);
             if (in >= a.input_rows) in = a.input_rows - 1ull;
@@ -681,7 +691,8 @@ __global__ __launch_bounds__(512) void matvec_f32_block_kernel(MatvecArgs a)
     // piece j of this thread is a piece of a weight row for the first two j, of an input row after
     auto fetch = [&](unsigned j, unsigned chunk) -> v4f {
         if (512u * (j + 1u) <= kF32BlockWeightRows * kPieces) {
-            const float4 w = scalar_weights4<QT>(source[j], (unsigned long long)chunk * kF32BlockColumns);
+            const unsigned piece = (threadIdx.x + 512u * j) % kPieces;
+            const float4 w = scalar_weights4<QT>(source[j], (unsigned long long)chunk * kF32BlockColumns + 4u * piece);
             return v4f{w.x, w.y, w.z, w.w};
         }
         return *reinterpret_cast<const v4f *>(source[j] + (unsigned long long)chunk * kF32BlockColumns * 4ull);
@@ -1029,12 +1040,16 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive, out,
                                       out_stride, output_bf16 != 0, status, s);
     // F32 rows against a batch of F32 input rows: the double-precision matrix cores; rows of F16
-    // and BF16 values take the same kernels (the conversion to double is exact for them as well)
-    if ((qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16) && input_rows >= 8ull &&
-        !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
+    // and BF16 values take the same kernels (the conversion to double is exact for them as well),
+    // and so do Q8_0 rows against F32 input rows (a caller that switched the Q8 activation policy
+    // off: the decoded weight, scale times code, is exact in float; 4096 x 4096 by 2048 rows 20.9 ms
+    // on the lane-strided kernel)
+    if ((qtype == QT_F32 || qtype == QT_F16 || qtype == QT_BF16 || (qtype == QT_Q8_0 && !input_q8)) &&
+        input_rows >= 8ull && !(((uintptr_t)encoded | (uintptr_t)input) & 15u) && !(input_stride & 3ull) &&
         row_width % (input_rows < 256ull ? 256ull : 64ull) == 0ull)
         return qtype == QT_F32 ? launch_scalar_rows<QT_F32>(a, s)
-             : qtype == QT_F16 ? launch_scalar_rows<QT_F16>(a, s) : launch_scalar_rows<QT_BF16>(a, s);
+             : qtype == QT_F16 ? launch_scalar_rows<QT_F16>(a, s)
+             : qtype == QT_BF16 ? launch_scalar_rows<QT_BF16>(a, s) : launch_scalar_rows<QT_Q8_0>(a, s);
     // (fewer than eight input rows, or a row width the matrix-core kernels do not take: 16-bit
     // rows have no other fast kernel and stay here at any number of input rows, four a workgroup)
     if (((qtype == QT_F32 && input_rows < 8ull) ||
