@@ -1,4 +1,4 @@
-// Q4_K expert weights against a row batch of Q8_K activations on the int8 matrix cores, operands
+// Q4_K (and Q2_K) expert weights against a row batch of Q8_K activations on the int8 matrix cores, operands
 // staged through LDS (src/backend/cuda/tensorcore.cu:378-702 is the reference's counterpart, for
 // its own formats).
 //
@@ -30,6 +30,13 @@
 //     rows on 16 different bank groups).
 // One barrier per superblock publishes the next superblock's copies and retires the reads of
 // the buffer they will overwrite.
+//
+// Q2_K weight rows (a plain projection: the down experts of the reference's model file, whose own
+// tensor-core down kernel serves this format only, src/backend/cuda/tensorcore.cu:628-702) run
+// through the same tiles, copies and publication. Their operand is simpler: a 2-bit code times its
+// sub-block's 4-bit scale is at most 45, one int8 limb, so a K step (two 16-value sub-blocks) is
+// one matrix instruction a token block; the minimum term is a K step of depth 16 against the
+// Q8_K block's sixteen sums; rows are copied as dwords (84-byte superblocks), pitch 21 dwords.
 #include "common.hpp"
 #include "launch.hpp"
 #include "grouped.hpp"

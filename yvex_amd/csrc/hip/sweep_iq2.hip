@@ -1,6 +1,7 @@
 // Decode-width expert sweeps specialised for IQ2_XXS (and, with the same item list, streams and
-// finishing pass, Q4_K) weights and Q8_K activations on gfx950. The notes below are about
-// IQ2_XXS; what differs for Q4_K rows stands above `Q4kHalf`.
+// finishing pass, Q4_K rows and the Q2_K rows of a down projection) weights and Q8_K activations
+// on gfx950. The notes below are about IQ2_XXS; what differs for Q4_K rows stands above
+// `Q4kHalf`, for Q2_K rows above `Q2kHalf`.
 //
 // Same contract as the generic grouped kernel in moe.hip (src/backend/cuda/moe_kernels.cu:431-582
 // is the reference's counterpart), built around the instruction budget of this one format: at
