@@ -318,6 +318,7 @@ def dense_leg(torch, K, dev, repeats: int):
     run("cfg2_iq2_xxs_7168x2048_f32_b1", K.IQ2_XXS, 7168, 2048, 1, False)
     run("cfg2_iq2_xxs_7168x2048_q8k_b1", K.IQ2_XXS, 7168, 2048, 1, True)
     run("head_q8_0_129280x7168_q8k_b1", K.Q8_0, 129280, 7168, 1, True, copies=2)
+    run("head_q8_0_129280x7168_q8k_b32", K.Q8_0, 129280, 7168, 32, True, copies=2)
     # greedy selection over one 129 280-entry logits row, left on the device by the head
     logits = torch.randn((1, 129280), device=dev, generator=gen)
     status = K.new_status(dev)

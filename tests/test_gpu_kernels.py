@@ -520,6 +520,17 @@ def test_matvec_output_head_variant(gpu, oracle, qtype, rows, width):
     for k in range(3):
         same = got[0, filler[filler % 3 == k]]
         assert np.all(same.view(np.uint32) == same.view(np.uint32)[0])
+    if qtype == "Q8_0":
+        # a few rows against a Q8_0 matrix this large go to the matrix cores (the lane-strided
+        # kernel would read the matrix once per input row): the oracle's bits
+        few = g.normal(5 * width).reshape(5, width)
+        act = K.q8k_quantize(dev(few, gpu), status)
+        got = K.matvec(dev(w.ravel(), gpu), qt, rows, width, act, input_q8=True, input_rows=5,
+                       status=status).cpu().numpy()
+        status_ok(status)
+        want = oracle.q8_matvec(qt, np.ascontiguousarray(w[sample]).ravel(), len(sample), width,
+                                oracle.q8k_quantize(few), 5)
+        assert np.array_equal(np.ascontiguousarray(got[:, sample]).view(np.uint32), want.view(np.uint32))
 
 
 def test_matvec_additive_and_bf16(gpu, oracle):

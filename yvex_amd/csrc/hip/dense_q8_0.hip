@@ -210,11 +210,13 @@ __global__ __launch_bounds__(64 * kPlainWaves) void dense_q8_0_kernel(DenseQ80Ar
 // ROW_BLOCKS = 4: the tile above (512 lanes, 104 KB of LDS, a workgroup a compute unit);
 // ROW_BLOCKS = 2: 64 weight rows, four waves, 70 KB, two workgroups a compute unit, for batches
 // that have too few of the large tiles.
-constexpr unsigned kStagedTokens = 64u, kStagedPitch = 272u;
-constexpr unsigned kStagedActBytes = kStagedTokens * kStagedPitch;                  // one buffer
-constexpr unsigned staged_lds_bytes(unsigned row_blocks)
+// TOKEN_BLOCKS = 1 (with ROW_BLOCKS = 8: 256 weight rows x 32 input rows, 153 KB): batches of up to
+// 32 input rows against a matrix too large for the caches, an output head at decode width, where
+// the second block of input rows would be padding and half of every wave's work with it.
+constexpr unsigned kStagedPitch = 272u;
+constexpr unsigned staged_lds_bytes(unsigned row_blocks, unsigned token_blocks = 2u)
 {
-    return 2u * (32u * row_blocks * kStagedPitch + kStagedActBytes);
+    return 2u * (32u * row_blocks + 32u * token_blocks) * kStagedPitch;
 }
 
 __device__ __forceinline__ uint4 read16(unsigned address)
@@ -223,10 +225,12 @@ __device__ __forceinline__ uint4 read16(unsigned address)
     return make_uint4((unsigned)v[0], (unsigned)v[1], (unsigned)v[2], (unsigned)v[3]);
 }
 
-template <unsigned ROW_BLOCKS>
-__global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(DenseQ80Args g)
+template <unsigned ROW_BLOCKS, unsigned TOKEN_BLOCKS = 2u>
+__global__ __launch_bounds__(64 * ROW_BLOCKS * TOKEN_BLOCKS) void dense_q8_0_staged_kernel(DenseQ80Args g)
 {
-    constexpr unsigned kStagedThreads = 128u * ROW_BLOCKS, kStagedRows = 32u * ROW_BLOCKS;
+    constexpr unsigned kStagedThreads = 64u * ROW_BLOCKS * TOKEN_BLOCKS, kStagedRows = 32u * ROW_BLOCKS;
+    constexpr unsigned kStagedTokens = 32u * TOKEN_BLOCKS;
+    constexpr unsigned kStagedActBytes = kStagedTokens * kStagedPitch;                  // one buffer
     constexpr unsigned kStagedWeightBytes = kStagedRows * kStagedPitch;                 // one buffer
     constexpr unsigned kStagedWeightBase = 0u;                                          // [buffer]
     constexpr unsigned kStagedActBase = kStagedWeightBase + 2u * kStagedWeightBytes;    // [buffer]
@@ -234,7 +238,9 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
     constexpr unsigned kWeightRest = (kStagedRows * 17u - kWeightRounds * kStagedThreads) / 64u;   // waves of the last
     constexpr unsigned kActRounds = kStagedTokens * 17u / kStagedThreads;
     constexpr unsigned kActRest = (kStagedTokens * 17u - kActRounds * kStagedThreads) / 64u;
-    static_assert(kWeightRounds + 1u <= 5u && kActRounds + 1u <= 5u, "copy sources");
+    constexpr unsigned kActTail = (kStagedTokens * 17u - kActRounds * kStagedThreads) % 64u;    // lanes of one more wave
+    static_assert((kStagedRows * 17u) % 64u == 0u && (kActTail == 0u || kActTail == 32u), "whole or half waves copy");
+    static_assert(kWeightRounds + 1u <= 10u && kActRounds + 1u <= 5u, "copy sources");
     extern __shared__ __align__(16) unsigned char dense_q8_0_lds[];
     if (lds_address_of(dense_q8_0_lds) != 0u) {   // operands are addressed by absolute LDS offsets
         if (threadIdx.x == 0u) raise_status(g.status, 2);
@@ -290,6 +296,9 @@ __global__ __launch_bounds__(128 * ROW_BLOCKS) void dense_q8_0_staged_kernel(Den
         if (wave < kActRest)
             copy_to_lds_16(act_from[kActRounds] + a_at,
                            (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16u * kStagedThreads * kActRounds)));
+        else if (kActTail && wave == kActRest)
+            copy_to_lds_16_first32(act_from[kActRounds] + a_at,
+                                   (unsigned)__builtin_amdgcn_readfirstlane((int)(a_to + 16u * kStagedThreads * kActRounds)));
     };
 
     double acc[16];
@@ -406,9 +415,17 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
     // workgroups share a compute unit, 29 on the 64-row staged tile and 43 once two of them share
     // a compute unit, 35 on the 128-row tile), so the choice is the number of rounds each shape needs.
     const uint64_t token_tiles32 = (input_rows + 31u) / 32u;
-    const uint64_t token_tiles64 = (input_rows + kStagedTokens - 1u) / kStagedTokens;
+    const uint64_t token_tiles64 = (input_rows + 63u) / 64u;
     if (token_tiles32 > 65535ull) return ST_BOUNDS;
     const uint64_t units = (uint64_t)compute_units();
+    // up to 32 input rows against a matrix too large for the caches (an output head at decode
+    // width, 129 280 x 7168: 306 us on the 128 x 64 tiles, half of them padding; memory time 173 us)
+    if (!((uintptr_t)encoded & 15u) && input_rows <= 32u && row_count * row_bytes >= (64ull << 20)) {
+        YVEX_ALLOW_DYNAMIC_LDS((dense_q8_0_staged_kernel<8u, 1u>), staged_lds_bytes(8u, 1u));
+        dense_q8_0_staged_kernel<8u, 1u><<<dim3((unsigned)((row_count + 255u) / 256u), 1), 512, staged_lds_bytes(8u, 1u),
+                                           stream>>>(g);
+        return check_launch("dense_q8_0_staged");
+    }
     if (!((uintptr_t)encoded & 15u) && units) {
         const uint64_t plain = row_tiles * token_tiles32;
         const uint64_t tall = (row_count + 127u) / 128u * token_tiles64, low = (row_count + 63u) / 64u * token_tiles64;

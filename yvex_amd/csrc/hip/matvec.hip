@@ -1035,8 +1035,12 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
         return launch_q4k_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive,
                                      out, out_stride, output_bf16 != 0, status, s);
     // Q8_0 rows against a batch of Q8_K input rows: matrix cores from the reference's threshold on
-    // (src/backend/cuda/private.h:461-464); below it the lane-strided kernel
-    if (qtype == QT_Q8_0 && input_q8 && input_rows >= 16ull && !((uintptr_t)encoded & 3u))
+    // (src/backend/cuda/private.h:461-464); below it the lane-strided kernel, which reads the
+    // matrix once per input row: fine while the matrix stays in the caches, but an output head of
+    // 129 280 x 7168 takes 171 us for one row, 336 for two and 1.5 ms for fifteen where the matrix
+    // cores take 290 us for up to 32, so a matrix of 64 MB or more goes there from two rows on
+    if (qtype == QT_Q8_0 && input_q8 && !((uintptr_t)encoded & 3u) &&
+        (input_rows >= 16ull || (input_rows >= 2ull && row_count * row_bytes >= (64ull << 20))))
         return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive, out,
                                       out_stride, output_bf16 != 0, status, s);
     // F32 rows against a batch of F32 input rows: the double-precision matrix cores; rows of F16
