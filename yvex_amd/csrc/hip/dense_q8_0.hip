@@ -418,9 +418,10 @@ int launch_q8_0_rows_dense(const uint8_t *encoded, uint64_t row_count, uint64_t 
     const uint64_t token_tiles64 = (input_rows + 63u) / 64u;
     if (token_tiles32 > 65535ull) return ST_BOUNDS;
     const uint64_t units = (uint64_t)compute_units();
-    // up to 32 input rows against a matrix too large for the caches (an output head at decode
-    // width, 129 280 x 7168: 306 us on the 128 x 64 tiles, half of them padding; memory time 173 us)
-    if (!((uintptr_t)encoded & 15u) && input_rows <= 32u && row_count * row_bytes >= (64ull << 20)) {
+    // up to 32 input rows against a matrix with a 256-row tile for every compute unit (an output
+    // head at decode width, 129 280 x 7168: 306 us on the 128 x 64 tiles, half of them padding;
+    // memory time 173 us)
+    if (!((uintptr_t)encoded & 15u) && input_rows <= 32u && units && (row_count + 255u) / 256u >= units) {
         YVEX_ALLOW_DYNAMIC_LDS((dense_q8_0_staged_kernel<8u, 1u>), staged_lds_bytes(8u, 1u));
         dense_q8_0_staged_kernel<8u, 1u><<<dim3((unsigned)((row_count + 255u) / 256u), 1), 512, staged_lds_bytes(8u, 1u),
                                            stream>>>(g);

@@ -1036,11 +1036,15 @@ extern "C" int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint6
                                      out, out_stride, output_bf16 != 0, status, s);
     // Q8_0 rows against a batch of Q8_K input rows: matrix cores from the reference's threshold on
     // (src/backend/cuda/private.h:461-464); below it the lane-strided kernel, which reads the
-    // matrix once per input row: fine while the matrix stays in the caches, but an output head of
-    // 129 280 x 7168 takes 171 us for one row, 336 for two and 1.5 ms for fifteen where the matrix
-    // cores take 290 us for up to 32, so a matrix of 64 MB or more goes there from two rows on
+    // matrix once per input row: fine while the matrix stays in the caches (4096 x 4096, 18 MB:
+    // 10 us up to four rows, 12.5 at eight, 19 at fifteen; the matrix cores 13.5 us throughout),
+    // but 7168 x 7168 (55 MB) takes 15 us for one row, 21 for two and 66 for fifteen where the
+    // matrix cores take 18.5, and an output head of 129 280 x 7168 171 us for one row, 336 for two
+    // and 1.5 ms for fifteen where they take 200 to 235
+    const unsigned long long matrix_bytes = row_count * row_bytes;
     if (qtype == QT_Q8_0 && input_q8 && !((uintptr_t)encoded & 3u) &&
-        (input_rows >= 16ull || (input_rows >= 2ull && row_count * row_bytes >= (64ull << 20))))
+        (input_rows >= 16ull || (input_rows >= 2ull && matrix_bytes >= (32ull << 20)) ||
+         (input_rows >= 12ull && matrix_bytes >= (8ull << 20))))
         return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input, input_rows, additive, out,
                                       out_stride, output_bf16 != 0, status, s);
     // F32 rows against a batch of F32 input rows: the double-precision matrix cores; rows of F16
