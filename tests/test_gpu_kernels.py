@@ -289,7 +289,10 @@ def test_matvec_q8k_row_batch_runs_on_matrix_cores(gpu, oracle, qtype, rows, wid
 
 
 @pytest.mark.parametrize("rows,width,inputs", [(516, 4096, 16), (40, 256, 33), (4096, 4096, 70), (33, 2304, 64),
-                                               (7, 512, 200)])
+                                               (7, 512, 200),
+                                               # a 256-row tile for every compute unit and up to 32 input rows:
+                                               # the 256 x 32 staged shape (ragged last tile, two superblocks)
+                                               (65700, 512, 20), (65536, 256, 32)])
 def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, inputs):
     """Q8_0 rows against 16 or more Q8_K input rows (the reference's tensor-core threshold,
     src/backend/cuda/private.h:461-464): the oracle's Q8_K product bit for bit (the chain of eight
@@ -324,7 +327,8 @@ def test_matvec_q8_0_row_batch_runs_on_matrix_cores(gpu, oracle, rows, width, in
     assert np.allclose(few, got[:15], rtol=2e-5, atol=1e-6)
 
 
-@pytest.mark.parametrize("rows,width,inputs", [(130, 512, 1), (33, 2304, 5), (2048, 7168, 3), (40, 256, 15)])
+@pytest.mark.parametrize("rows,width,inputs", [(130, 512, 1), (33, 2304, 5), (2048, 7168, 3), (40, 256, 15),
+                                               (65700, 256, 3)])
 def test_matvec_q8_0_exact_at_few_rows(gpu, oracle, rows, width, inputs):
     """yvex_hip_matvec_q8_0_exact below 16 input rows (a shared expert run as dense projections at
     decode width): the oracle's Q8_K product bit for bit, where yvex_hip_matvec's faster kernel is
