@@ -45,16 +45,6 @@ int yvex_hip_matvec(const uint8_t *encoded, unsigned int qtype, uint64_t row_cou
                     float *out, uint64_t out_stride, int output_bf16, int *status,
                     yvex_hip_stream stream);
 
-/* The same product for Q8_0 rows against Q8_K input rows with the CPU path's bits at any number
- * of input rows (kernel_primitives.h:342-359 per superblock, superblocks added in double,
- * src/gguf/quant_compute.c:152-172): the matrix-core kernels yvex_hip_matvec takes from 16 input
- * rows on, here also below that, where yvex_hip_matvec prefers a faster kernel that keeps float
- * partial sums. For callers that need those bits, such as a shared expert run as dense
- * projections. encoded on a 4-byte boundary, row_width % 256 == 0. */
-int yvex_hip_matvec_q8_0_exact(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
-                               uint64_t row_bytes, const void *input_q8k, uint64_t input_rows,
-                               const float *additive, float *out, uint64_t out_stride, int output_bf16,
-                               int *status, yvex_hip_stream stream);
 
 /* Verification twin of the integer hot loop (kernel_primitives.h:287-359): writes the int32
  * block sums the Q8_K matvec accumulates, before any float scaling.

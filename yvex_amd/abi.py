@@ -301,7 +301,7 @@ EXPORTS = [
     "yvex_rocm_gguf_resident_load", "yvex_rocm_gguf_weight_view",
 ]
 KERNEL_EXPORTS = [
-    "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_row_dot", "yvex_hip_matvec", "yvex_hip_matvec_f32_rows", "yvex_hip_matvec_f32_scratch_bytes", "yvex_hip_matvec_f32_rows_launches", "yvex_hip_matvec_f32_rows_scored", "yvex_hip_matvec_q8_0_exact", "yvex_hip_block_dots_i32", "yvex_hip_gather",
+    "yvex_hip_q8k_quantize", "yvex_hip_concat_rows_bf16", "yvex_hip_row_dot", "yvex_hip_matvec", "yvex_hip_matvec_f32_rows", "yvex_hip_matvec_f32_scratch_bytes", "yvex_hip_matvec_f32_rows_launches", "yvex_hip_matvec_f32_rows_scored", "yvex_hip_block_dots_i32", "yvex_hip_gather",
     "yvex_hip_argmax_f32", "yvex_hip_argmax_scratch_bytes", "yvex_hip_argmax_f32_static",
     "yvex_hip_argmax_static_capacity",
     "yvex_hip_moe_route_rows", "yvex_hip_moe_route_scores", "yvex_hip_moe_route_hash_rows", "yvex_hip_worklist_build", "yvex_hip_moe_prepare", "yvex_hip_moe_prepare_scored",

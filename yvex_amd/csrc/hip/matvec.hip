@@ -84,10 +84,11 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
     // Q8_K activations against superblock formats: a superblock's float term is formed in the
     // order of the reference's device primitive and the terms of a row are added in double and
     // rounded once, as the CPU path adds a row's blocks (src/gguf/quant_compute.c:152-172): the
-    // result is that path's, bit for bit. Q8_0 rows (a term per 32 values, not chained through
-    // the eight of a superblock as the primitive chains them) and F32 activations keep float
-    // partial sums, inside the tolerance of the dense projections.
-    constexpr bool kWide = Q8 && UnitTraits<QT>::kIntegerCombine;
+    // result is that path's, bit for bit. Q8_0 rows chain their eight terms of a superblock as
+    // the primitive chains them (total = fmaf(d_b * d_a, float(dot_b), total), b = 0 .. 7, from
+    // zero: kernel_primitives.h:342-359) across the eight lanes that hold the superblock's blocks.
+    // F32 activations keep float partial sums, inside the tolerance of the dense projections.
+    constexpr bool kWide = Q8 && (UnitTraits<QT>::kIntegerCombine || QT == QT_Q8_0);
     using Sum = typename std::conditional<kWide, double, float>::type;
     Sum acc[T];
 #pragma unroll
@@ -125,8 +126,21 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
                             acc[t] += (Sum)super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
                                                              act_scale, s);
                     } else {
-                        const float v = q8_0_unit_value(unit[j], act_scale, s.dot);
-                        acc[t] += (Sum)(live[j] ? v : 0.0f);
+                        // lane b of a group of eight holds block b: after step k the lanes up to
+                        // k hold the chain through their block, after seven the last lane holds
+                        // the superblock's total (units past the row's end belong to no superblock:
+                        // a row is whole superblocks)
+                        const float scale = f16_bits_to_float((unsigned short)unit[j].scale_bits) * act_scale;
+                        const float value = (float)s.dot;
+                        const bool first = (lane & 7u) == 0u;
+                        float total = __builtin_fmaf(scale, value, 0.0f);
+#pragma unroll
+                        for (int step = 0; step < 7; ++step) {
+                            const float before = __int_as_float(
+                                __builtin_amdgcn_update_dpp(0, __float_as_int(total), 0x111, 0xf, 0xf, false));   // row_shr:1
+                            total = __builtin_fmaf(scale, value, first ? 0.0f : before);
+                        }
+                        acc[t] += (Sum)(live[j] && (lane & 7u) == 7u ? total : 0.0f);
                     }
                 } else if constexpr (STAGE) {
                     float4 x4[8];
@@ -952,18 +966,6 @@ static int launch_block_q(const MatvecArgs &a, bool q8, hipStream_t stream)
 }  // namespace yvex
 
 using namespace yvex;
-
-extern "C" int yvex_hip_matvec_q8_0_exact(const uint8_t *encoded, uint64_t row_count, uint64_t row_width,
-                                          uint64_t row_bytes, const void *input_q8k, uint64_t input_rows,
-                                          const float *additive, float *out, uint64_t out_stride,
-                                          int output_bf16, int *status, yvex_hip_stream stream)
-{
-    if (!encoded || !input_q8k || !out || !status || !row_count || !row_width || !input_rows ||
-        out_stride < row_count || (((uintptr_t)input_q8k | (uintptr_t)out) & 3u))
-        return ST_INVALID_ARG;
-    return launch_q8_0_rows_dense(encoded, row_count, row_width, row_bytes, input_q8k, input_rows, additive, out,
-                                  out_stride, output_bf16 != 0, status, as_stream(stream));
-}
 
 // Rows of F32, F16 or BF16 values against eight or more F32 input rows: 16 x 16 tiles on the
 // double-precision matrix cores; a small batch offers few tiles, so sixteen waves split the row

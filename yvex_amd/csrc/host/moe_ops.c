@@ -694,14 +694,13 @@ static int moe_execute_rows(yvex_rocm_backend *backend, const yvex_moe_layer_job
     merged = !row_batch && has_shared && shared_q8 == routed_q8 && same_expert_shape(&routed, &shared);
     /* A Q8_0 shared expert (the format the reference's model file keeps it in, its default for every
      * tensor outside the routed experts: src/graph/families/deepseek_v4.c:1550-1557) is three dense
-     * projections of every row, and the Q8_0 matrix-core kernels give the CPU path's bits at any
-     * number of rows: gate and up sums, the SwiGLU stage, quantization, down. The up sums
+     * projections of every row, and the dense Q8_0 kernels give the CPU path's bits at any number of
+     * rows: gate and up sums, the SwiGLU stage, quantization, down. The up sums
      * borrow the pair-output range, which nothing uses between the router and the routed down
      * projection. */
     shared_dense = has_shared && shared_q8 && !merged && !shared_row_batch && !shared_image &&
                    shared.gate_qtype == 8u && shared.up_qtype == 8u && shared.down_qtype == 8u &&
-                   layer->shared_intermediate_width <= topk * hidden &&
-                   !(((uintptr_t)shared.gate | (uintptr_t)shared.up | (uintptr_t)shared.down) & 3u);
+                   layer->shared_intermediate_width <= topk * hidden;
     if (yvex_rocm_seam("YVEX_TEST_ROCM_LAUNCH_FAILURE"))
         return yvex_rocm_refuse(err, YVEX_ERR_BACKEND, "rocm.moe.rows.launch",
                                 "kernel launch failed (test seam)");
@@ -969,14 +968,14 @@ sequence:
                                     1ull, 1ull, layer->activation_limit, (float *)AT(shared_intermediate),
                                     (int *)status, stream), "rocm.moe.rows.shared-up-matrix");
     else if (shared_dense) {
-        LAUNCH(yvex_hip_matvec_q8_0_exact(shared.gate, layer->shared_intermediate_width, hidden,
-                                          shared.gate_row_bytes, AT(input_q8), row_count, NULL,
-                                          (float *)AT(shared_intermediate), layer->shared_intermediate_width, 0,
-                                          (int *)status, stream), "rocm.moe.rows.shared-gate-dense");
-        LAUNCH(yvex_hip_matvec_q8_0_exact(shared.up, layer->shared_intermediate_width, hidden,
-                                          shared.up_row_bytes, AT(input_q8), row_count, NULL,
-                                          (float *)AT(pair_outputs), layer->shared_intermediate_width, 0,
-                                          (int *)status, stream), "rocm.moe.rows.shared-up-dense");
+        LAUNCH(yvex_hip_matvec(shared.gate, shared.gate_qtype, layer->shared_intermediate_width, hidden,
+                               shared.gate_row_bytes, AT(input_q8), 1, row_count, hidden, NULL,
+                               (float *)AT(shared_intermediate), layer->shared_intermediate_width, 0,
+                               (int *)status, stream), "rocm.moe.rows.shared-gate-dense");
+        LAUNCH(yvex_hip_matvec(shared.up, shared.up_qtype, layer->shared_intermediate_width, hidden,
+                               shared.up_row_bytes, AT(input_q8), 1, row_count, hidden, NULL,
+                               (float *)AT(pair_outputs), layer->shared_intermediate_width, 0,
+                               (int *)status, stream), "rocm.moe.rows.shared-up-dense");
         LAUNCH(yvex_hip_moe_swiglu_rows((const float *)AT(shared_intermediate), (const float *)AT(pair_outputs),
                                         row_count * layer->shared_intermediate_width, layer->activation_limit,
                                         (float *)AT(shared_intermediate), (int *)status, stream),
@@ -1021,10 +1020,10 @@ sequence:
                                       row_count, 1ull, (float *)AT(shared_outputs), (int *)status, stream),
                "rocm.moe.rows.shared-down-matrix");
     else if (shared_dense)
-        LAUNCH(yvex_hip_matvec_q8_0_exact(shared.down, hidden, layer->shared_intermediate_width,
-                                          shared.down_row_bytes, AT(shared_intermediate_q8), row_count, NULL,
-                                          (float *)AT(shared_outputs), hidden, 1, (int *)status, stream),
-               "rocm.moe.rows.shared-down-dense");
+        LAUNCH(yvex_hip_matvec(shared.down, shared.down_qtype, hidden, layer->shared_intermediate_width,
+                               shared.down_row_bytes, AT(shared_intermediate_q8), 1, row_count,
+                               layer->shared_intermediate_width, NULL, (float *)AT(shared_outputs), hidden, 1,
+                               (int *)status, stream), "rocm.moe.rows.shared-down-dense");
     else if (has_shared && !merged)
         LAUNCH(yvex_hip_moe_down(&shared, shared_q8 ? AT(shared_intermediate_q8) : AT(shared_intermediate),
                                  shared_q8, NULL, NULL, NULL, NULL, NULL, NULL, row_count, 1ull,

@@ -92,17 +92,6 @@ def matvec(encoded, qtype, row_count, row_width, inputs, *, input_q8=False, inpu
     return out
 
 
-def matvec_q8_0_exact(encoded, row_count, row_width, inputs_q8k, input_rows, *, additive=None, output_bf16=False,
-                      status=None, out=None):
-    """Q8_0 rows against Q8_K input rows with the CPU path's bits at any number of input rows."""
-    if out is None:
-        out = torch.empty((input_rows, row_count), dtype=torch.float32, device=encoded.device)
-    _call("yvex_hip_matvec_q8_0_exact", _ptr(encoded), C.c_uint64(row_count), C.c_uint64(row_width),
-          C.c_uint64(row_bytes(Q8_0, row_width)), _ptr(inputs_q8k), C.c_uint64(input_rows), _ptr(additive),
-          _ptr(out), C.c_uint64(out.stride(0)), C.c_int(int(output_bf16)), _ptr(status), _stream())
-    return out
-
-
 def matvec_f32_rows(weights, inputs, status, *, additive=None, output_bf16=False, scratch=None, out=None):
     """F32 weight rows [rows, width] against F32 input rows with the split-projection scratch:
     None allocates what yvex_hip_matvec_f32_scratch_bytes asks for, False passes none."""
