@@ -126,19 +126,20 @@ __global__ __launch_bounds__(256) void matvec_block_kernel(MatvecArgs a)
                             acc[t] += (Sum)super_combine<QT>(wrow + (uu[j] >> 3) * UnitTraits<QT>::kSuperBytes,
                                                              act_scale, s);
                     } else {
-                        // lane b of a group of eight holds block b: after step k the lanes up to
-                        // k hold the chain through their block, after seven the last lane holds
-                        // the superblock's total (units past the row's end belong to no superblock:
-                        // a row is whole superblocks)
+                        // lane b of a group of eight holds block b. The start gives lane 0 its
+                        // chain (block 0 onto zero); step k gives lane k the chain through block k
+                        // from lane k - 1's value of the step before, so after seven steps the last
+                        // lane holds the superblock's total. What a lane holds after its own step
+                        // is read by nobody and may be anything (units past the row's end belong
+                        // to no superblock: a row is whole superblocks)
                         const float scale = f16_bits_to_float((unsigned short)unit[j].scale_bits) * act_scale;
                         const float value = (float)s.dot;
-                        const bool first = (lane & 7u) == 0u;
                         float total = __builtin_fmaf(scale, value, 0.0f);
 #pragma unroll
-                        for (int step = 0; step < 7; ++step) {
+                        for (int step = 1; step < 8; ++step) {
                             const float before = __int_as_float(
                                 __builtin_amdgcn_update_dpp(0, __float_as_int(total), 0x111, 0xf, 0xf, false));   // row_shr:1
-                            total = __builtin_fmaf(scale, value, first ? 0.0f : before);
+                            total = __builtin_fmaf(scale, value, before);
                         }
                         acc[t] += (Sum)(live[j] && (lane & 7u) == 7u ? total : 0.0f);
                     }
